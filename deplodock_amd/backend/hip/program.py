@@ -1,0 +1,676 @@
+"""Program runtime: buffers, scratch slab, launches, graphs and event timing.
+
+Takes a lowered ``Graph[HipOp + InputOp + ConstantOp]`` and runs it on the
+current HIP device through ``libemmy_hip.so``.  Same responsibilities as the
+reference's ``program.py`` (emmy/compiler/backend/cuda/program.py: ``_compile``
+:177-226, ``_allocate`` :340-364, ``_launch`` :394-424, ``CompiledProgram``
+:614-1090, ``benchmark_program`` :1152-1325) with two deliberate differences:
+device memory is PyTorch-ROCm tensors (the launcher only borrows their
+pointers), and inputs that already live on the device are used in place.
+"""
+
+from __future__ import annotations
+
+import contextlib
+import fcntl
+import logging
+import math
+import statistics
+import time
+from dataclasses import dataclass, field
+
+import numpy as np
+
+from deplodock_amd import config
+from deplodock_amd.backend import BenchmarkResult, LaunchTime, RunResult
+from deplodock_amd.backend.hip import hiprtc, launcher
+from deplodock_amd.backend.hip.launcher import PackedArgs
+from deplodock_amd.dtype import BF16, DType, bf16_bits_from_f32, to_torch
+from deplodock_amd.graph import Graph, Node
+from deplodock_amd.ir.base import ConstantOp, InputOp
+from deplodock_amd.ir.hip import HipOp, resolve_dim
+
+logger = logging.getLogger(__name__)
+
+_STATIC_LDS_CAP = 64 * 1024  # per-workgroup LDS available without opting in
+_KERNEL_TIMEOUT_MS = 1000.0  # per-window watchdog
+_WARMUP_TARGET_MS = 10.0  # keep warming until this much device time has run
+_BATCH_TARGET_MS = 1.0  # launches per event window are sized to cover this
+_AUTO_BUDGET_MS = 100.0
+_AUTO_MAX_ITERS = 20000
+_SLAB_ALIGN = 256
+
+
+class HungKernelError(RuntimeError):
+    """An event window did not complete within the watchdog budget."""
+
+
+class GraphCaptureError(RuntimeError):
+    """Capturing launches into a HIP graph failed; timing falls back to plain launches."""
+
+
+@contextlib.contextmanager
+def gpu_lock():
+    """Cross-process device lock (``EMMY_GPU_LOCK``; emmy/compiler/backend/gpu_lock.py)."""
+    path = config.gpu_lock_path()
+    try:
+        fh = open(path, "a+")
+    except OSError:
+        yield
+        return
+    try:
+        fcntl.flock(fh, fcntl.LOCK_EX)
+        yield
+    finally:
+        fcntl.flock(fh, fcntl.LOCK_UN)
+        fh.close()
+
+
+# ---------------------------------------------------------------------------
+# Compile: kernels + buffer plan + launch list
+# ---------------------------------------------------------------------------
+
+
+@dataclass
+class _Buffer:
+    name: str
+    shape: tuple
+    dtype: DType
+    role: str  # input | constant | output | scratch
+
+    def resolve_shape(self, sym_values: dict[str, int]) -> tuple[int, ...]:
+        return tuple(int(d) if not isinstance(d, str) else int(sym_values[d]) for d in self.shape)
+
+
+@dataclass
+class _Launch:
+    node_id: str
+    kernel_name: str
+    arg_names: tuple[str, ...]
+    grid: tuple
+    block: tuple
+    lds_bytes: int
+    zero_outputs: tuple[str, ...]
+    runtime_args: tuple[str, ...] = ()
+    algo_bytes: int = 0
+    algo_flops: int = 0
+
+
+@dataclass
+class _Compiled:
+    bufs: list[_Buffer]
+    buf_by_name: dict[str, _Buffer]
+    constants: dict[str, float]
+    kernels: dict[str, hiprtc.LoadedKernel]
+    launches: list[_Launch]
+    symbolic_bindings: dict[str, tuple[str, int]] = field(default_factory=dict)
+
+
+_ZERO_KERNEL_NAME = "emh_zero_words"
+_ZERO_KERNEL_SRC = r"""
+extern "C" __global__ __launch_bounds__(256) void emh_zero_words(unsigned int* __restrict__ p, int n) {
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) p[i] = 0u;
+}
+"""
+
+
+def _launches(graph: Graph) -> list[Node]:
+    nodes = []
+    for nid in graph.topological_order():
+        node = graph.nodes[nid]
+        if isinstance(node.op, (InputOp, ConstantOp)):
+            continue
+        if not isinstance(node.op, HipOp):
+            raise TypeError(f"HipBackend: node {nid!r} has non-HipOp {type(node.op).__name__!r}; lowering must produce Graph[HipOp].")
+        nodes.append(node)
+    return nodes
+
+
+def _buffers(graph: Graph) -> list[_Buffer]:
+    return [_Buffer(nid, tuple(graph.nodes[nid].output.shape), graph.nodes[nid].output.dtype, graph.node_role(nid)) for nid in graph.topological_order()]
+
+
+def _symbolic_bindings(graph: Graph) -> dict[str, tuple[str, int]]:
+    out: dict[str, tuple[str, int]] = {}
+    for nid in graph.inputs:
+        for i, d in enumerate(graph.nodes[nid].output.shape):
+            if isinstance(d, str) and d not in out:
+                out[d] = (nid, i)
+    return out
+
+
+def _compile(graph: Graph) -> _Compiled:
+    bufs = _buffers(graph)
+    kernels: dict[str, hiprtc.LoadedKernel] = {}
+    seen_source: dict[str, str] = {}
+    launches: list[_Launch] = []
+    need_zero = False
+    for node in _launches(graph):
+        op: HipOp = node.op
+        kname = op.kernel_name
+        if kname not in kernels:
+            prev = seen_source.get(kname)
+            if prev is not None and prev != op.kernel_source:
+                raise ValueError(f"kernel name {kname!r} used by two distinct sources")
+            seen_source[kname] = op.kernel_source
+            kernels[kname] = hiprtc.load_function(op.kernel_source, kname)
+        elif seen_source[kname] != op.kernel_source:
+            raise ValueError(f"kernel name {kname!r} used by two distinct sources")
+        need_zero = need_zero or bool(op.zero_outputs)
+        launches.append(
+            _Launch(
+                node_id=node.id,
+                kernel_name=kname,
+                arg_names=tuple(op.arg_order),
+                grid=op.grid,
+                block=op.block,
+                lds_bytes=op.lds_bytes,
+                zero_outputs=tuple(op.zero_outputs),
+                runtime_args=tuple(op.runtime_args),
+                algo_bytes=op.algo_bytes,
+                algo_flops=op.algo_flops,
+            )
+        )
+    if need_zero:
+        kernels[_ZERO_KERNEL_NAME] = hiprtc.load_function(_ZERO_KERNEL_SRC, _ZERO_KERNEL_NAME)
+    constants = {nid: float(op.value) for nid, op in graph.constant_ops() if op.value is not None}
+    return _Compiled(bufs, {b.name: b for b in bufs}, constants, kernels, launches, _symbolic_bindings(graph))
+
+
+# ---------------------------------------------------------------------------
+# Scratch planning (role of the reference's backend/cuda/_planner.py)
+# ---------------------------------------------------------------------------
+
+
+def compute_live_intervals(names: list[str], launches: list[_Launch]) -> dict[str, tuple[int, int]]:
+    """``name -> (first launch index that touches it, last one)``."""
+    out: dict[str, tuple[int, int]] = {}
+    wanted = set(names)
+    for i, ln in enumerate(launches):
+        for n in (*ln.arg_names, *ln.zero_outputs):
+            if n in wanted:
+                lo, hi = out.get(n, (i, i))
+                out[n] = (min(lo, i), max(hi, i))
+    for n in names:
+        out.setdefault(n, (0, max(len(launches) - 1, 0)))
+    return out
+
+
+def plan_offsets(intervals: dict[str, tuple[int, int]], sizes: dict[str, int], align: int = _SLAB_ALIGN) -> tuple[dict[str, int], int]:
+    """Greedy first-fit: buffers whose live intervals overlap never share bytes.
+    Largest first; each lands at the lowest aligned offset free for its interval."""
+    placed: list[tuple[int, int, int, int]] = []  # (offset, end, lo, hi)
+    offsets: dict[str, int] = {}
+    total = 0
+    for name in sorted(sizes, key=lambda n: (-sizes[n], n)):
+        size = -(-sizes[name] // align) * align
+        lo, hi = intervals[name]
+        conflicts = sorted((o, e) for o, e, plo, phi in placed if not (phi < lo or hi < plo))
+        off = 0
+        for o, e in conflicts:
+            if off + size <= o:
+                break
+            off = max(off, e)
+        offsets[name] = off
+        placed.append((off, off + size, lo, hi))
+        total = max(total, off + size)
+    return offsets, total
+
+
+# ---------------------------------------------------------------------------
+# Buffer materialization
+# ---------------------------------------------------------------------------
+
+
+def _torch():
+    import torch
+
+    return torch
+
+
+def _device():
+    torch = _torch()
+    if not torch.cuda.is_available():
+        raise launcher.LauncherError("no HIP device is visible: the HIP backend cannot run (there is no CPU fallback)")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _to_device(src, buf: _Buffer, shape: tuple[int, ...]):
+    """Host array / tensor → device tensor of ``buf``'s dtype.  A device tensor
+    that already matches is used in place (no copy)."""
+    torch = _torch()
+    want = to_torch(buf.dtype)
+    if isinstance(src, torch.Tensor):
+        t = src
+        if t.dtype != want:
+            raise TypeError(f"buffer {buf.name!r}: expected {want}, got {t.dtype}")
+        t = t.reshape(shape)
+        if not t.is_cuda:
+            t = t.contiguous().to(_device())
+        elif not t.is_contiguous():
+            t = t.contiguous()
+        return t
+    arr = np.asarray(src)
+    if buf.dtype is BF16:
+        if arr.dtype != np.uint16:
+            arr = bf16_bits_from_f32(np.asarray(arr, dtype=np.float32))
+        arr = np.ascontiguousarray(arr).reshape(shape)
+        return torch.from_numpy(arr.view(np.int16)).to(_device()).view(torch.bfloat16)
+    arr = np.ascontiguousarray(arr, dtype=buf.dtype.np).reshape(shape)
+    return torch.from_numpy(arr).to(_device())
+
+
+def _materialize(buf: _Buffer, shape: tuple[int, ...], src, constants: dict[str, float]):
+    torch = _torch()
+    if src is not None:
+        return _to_device(src, buf, shape)
+    want = to_torch(buf.dtype)
+    if buf.role == "constant":
+        if buf.name not in constants:
+            raise KeyError(f"constant {buf.name!r} has no static value and was not supplied in input_data")
+        return torch.full(shape, constants[buf.name], dtype=want, device=_device())
+    if buf.role == "input":
+        # Deterministic pseudo-random fill for un-supplied inputs, values in
+        # [-0.5, 0.5] (same recipe as emmy/compiler/backend/cuda/program.py:265-276).
+        n = int(np.prod(shape)) if shape else 1
+        idx = np.arange(n, dtype=np.int64)
+        vals = (0.01 * ((idx.astype(np.float32) * 7 + 13) % 101 - 50)).astype(np.float32)
+        return torch.from_numpy(vals.reshape(shape)).to(_device()).to(want)
+    return torch.zeros(shape, dtype=want, device=_device())
+
+
+def _resolve_symbolic(compiled: _Compiled, input_data: dict) -> dict[str, int]:
+    env: dict[str, int] = {}
+    for name, (buf, dim) in compiled.symbolic_bindings.items():
+        arr = input_data.get(buf)
+        if arr is None:
+            raise ValueError(f"symbolic dim {name!r} reads from input {buf!r}.shape[{dim}] but no array was supplied")
+        env[name] = int(arr.shape[dim])
+    return env
+
+
+def _host(t, dtype: DType) -> np.ndarray:
+    """Device tensor → host ndarray (bf16 as uint16 bit patterns)."""
+    torch = _torch()
+    if dtype is BF16:
+        return t.view(torch.int16).cpu().numpy().view(np.uint16)
+    return t.cpu().numpy()
+
+
+# ---------------------------------------------------------------------------
+# CompiledProgram
+# ---------------------------------------------------------------------------
+
+
+class CompiledProgram:
+    """A compiled graph bound to device buffers, ready to launch repeatedly.
+
+    Scratch buffers are typed views into one liveness-planned slab that lives
+    as long as the program, so pointers baked into argument packs and captured
+    graphs stay valid across replays (program.py:281-337)."""
+
+    def __init__(self, compiled: _Compiled, arrays: dict, sym_values: dict[str, int], slab, slab_bytes: int, naive_bytes: int):
+        self.lib = launcher.load()
+        self.compiled = compiled
+        self.arrays = arrays
+        self.sym_values = sym_values
+        self._slab = slab
+        self.slab_bytes = slab_bytes
+        self.naive_scratch_bytes = naive_bytes
+        self._packs: list[tuple[PackedArgs, tuple, tuple, list[tuple[PackedArgs, int]]]] = []
+        self._stream: int | None = None  # private stream for capture / timing
+        self._launch_graphs: dict[int, int] = {}
+        self._launch_graph_sizes: list[int] | None = None
+        self._program_graph: int | None = None
+        self._events: list[int] = []
+        self._build_packs()
+
+    # -- construction ---------------------------------------------------------
+    @classmethod
+    def build(cls, graph: Graph, input_data: dict | None = None, compile_timeout_s: float | None = None) -> CompiledProgram:
+        t0 = time.perf_counter()
+        compiled = _compile(graph)
+        input_data = dict(input_data or {})
+        sym_values = _resolve_symbolic(compiled, input_data)
+        torch = _torch()
+        arrays: dict = {}
+        for buf in compiled.bufs:
+            if buf.role == "scratch":
+                continue
+            shape = buf.resolve_shape(sym_values) or (1,)
+            arrays[buf.name] = _materialize(buf, shape, input_data.get(buf.name), compiled.constants)
+        sizes = {}
+        for buf in compiled.bufs:
+            if buf.role == "scratch":
+                shape = buf.resolve_shape(sym_values) or (1,)
+                sizes[buf.name] = max(1, int(np.prod(shape))) * buf.dtype.nbytes
+        intervals = compute_live_intervals(list(sizes), compiled.launches)
+        offsets, total = plan_offsets(intervals, sizes)
+        slab = torch.zeros(max(total, _SLAB_ALIGN), dtype=torch.uint8, device=_device())
+        for buf in compiled.bufs:
+            if buf.role == "scratch":
+                shape = buf.resolve_shape(sym_values) or (1,)
+                off = offsets[buf.name]
+                arrays[buf.name] = slab[off : off + sizes[buf.name]].view(to_torch(buf.dtype)).view(shape)
+        prog = cls(compiled, arrays, sym_values, slab, total, sum(sizes.values()))
+        # Uploads ran on torch's stream; timing and capture use a private one.
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        if compile_timeout_s is not None and elapsed > compile_timeout_s:
+            raise RuntimeError(f"benchmark compile stage exceeded {compile_timeout_s:.1f}s ({elapsed:.1f}s) — variant marked bench_fail")
+        return prog
+
+    def _build_packs(self) -> None:
+        self._packs = []
+        for ln in self.compiled.launches:
+            ptrs = []
+            for name in ln.arg_names:
+                t = self.arrays[name]
+                ptr = t.data_ptr()
+                if ptr % 16:
+                    raise ValueError(f"buffer {name!r} is not 16-byte aligned (vector loads require it)")
+                ptrs.append(ptr)
+            ints = [self.sym_values[n] for n in ln.runtime_args]
+            pack = PackedArgs(ptrs, ints)
+            grid = tuple(resolve_dim(s, self.sym_values) for s in ln.grid)
+            block = tuple(resolve_dim(s, self.sym_values) for s in ln.block)
+            zero_packs = []
+            for z in ln.zero_outputs:
+                t = self.arrays[z]
+                nbytes = t.numel() * t.element_size()
+                if nbytes % 4:
+                    raise ValueError(f"zero_outputs buffer {z!r} is not a whole number of 32-bit words")
+                zero_packs.append((PackedArgs([t.data_ptr()], [nbytes // 4]), nbytes // 4))
+            if ln.lds_bytes > _STATIC_LDS_CAP:
+                self.lib.func_set_dynamic_lds(self.compiled.kernels[ln.kernel_name].fn, ln.lds_bytes)
+            self._packs.append((pack, grid, block, zero_packs))
+
+    # -- launching ----------------------------------------------------------------
+    def _torch_stream(self) -> int:
+        return int(_torch().cuda.current_stream().cuda_stream)
+
+    def launch_one(self, i: int, stream: int | None) -> None:
+        ln = self.compiled.launches[i]
+        pack, grid, block, zero_packs = self._packs[i]
+        for zp, words in zero_packs:
+            zgrid = (max(1, min(1024, -(-words // 256))), 1, 1)
+            self.lib.launch(self.compiled.kernels[_ZERO_KERNEL_NAME].fn, zgrid, (256, 1, 1), 0, stream, zp)
+        self.lib.launch(self.compiled.kernels[ln.kernel_name].fn, grid, block, ln.lds_bytes, stream, pack)
+
+    def run(self, stream: int | None = None) -> None:
+        """Issue every launch once, in program order, on ``stream`` (default: torch's current stream)."""
+        s = self._torch_stream() if stream is None else stream
+        for i in range(len(self.compiled.launches)):
+            self.launch_one(i, s)
+
+    def outputs(self) -> dict[str, np.ndarray]:
+        _torch().cuda.synchronize()
+        return {b.name: _host(self.arrays[b.name], b.dtype) for b in self.compiled.bufs if b.role == "output"}
+
+    def output_tensors(self) -> dict:
+        return {b.name: self.arrays[b.name] for b in self.compiled.bufs if b.role == "output"}
+
+    # -- timing -----------------------------------------------------------------------
+    def _ensure_stream(self) -> int:
+        if self._stream is None:
+            self._stream = self.lib.stream_create()
+        return self._stream
+
+    def _event(self) -> int:
+        e = self.lib.event_create()
+        self._events.append(e)
+        return e
+
+    def _wait_for_event(self, event: int, what: str) -> None:
+        """Poll instead of blocking so a hung kernel raises instead of stalling (program.py:574-611)."""
+        deadline = time.perf_counter() + _KERNEL_TIMEOUT_MS / 1000.0
+        while not self.lib.event_query(event):
+            if time.perf_counter() > deadline:
+                raise HungKernelError(f"{what} did not finish within {_KERNEL_TIMEOUT_MS:.0f} ms")
+            time.sleep(0)
+
+    def _elapsed(self, start: int, stop: int, what: str) -> float:
+        ms = self.lib.event_elapsed_ms(start, stop)
+        if not ms > 0.0:
+            raise RuntimeError(f"{what} reported {ms:.3f}ms elapsed — degenerate launch, variant marked bench_fail")
+        return ms
+
+    def iter_once(self, batch_sizes: list[int], pre_iter=None) -> list[float]:
+        """One benchmark iteration: for each launch, one event window around
+        ``batch_sizes[i]`` back-to-back issues (a graph replay when captured).
+        Returns per-launch ms normalised to one issue."""
+        stream = self._ensure_stream()
+        if pre_iter is not None:
+            pre_iter(max(batch_sizes) if batch_sizes else 1)
+        out: list[float] = []
+        if not hasattr(self, "_win"):
+            self._win = (self._event(), self._event())
+        start, stop = self._win
+        for i, ln in enumerate(self.compiled.launches):
+            self.lib.event_record(start, stream)
+            g = self._launch_graphs.get(i) if self._launch_graph_sizes == batch_sizes else None
+            if g is not None:
+                self.lib.graph_launch(g, stream)
+            else:
+                for _ in range(batch_sizes[i]):
+                    self.launch_one(i, stream)
+            self.lib.event_record(stop, stream)
+            self._wait_for_event(stop, f"kernel {ln.kernel_name!r}")
+            out.append(self._elapsed(start, stop, f"kernel {ln.kernel_name!r}") / batch_sizes[i])
+        return out
+
+    def capture_launch_graphs(self, batch_sizes: list[int]) -> None:
+        """Capture each launch's batch into its own graph; no-op when already captured at these sizes."""
+        if self._launch_graph_sizes == batch_sizes:
+            return
+        self._drop_launch_graphs()
+        stream = self._ensure_stream()
+        self.lib.stream_synchronize(stream)
+        try:
+            for i in range(len(self.compiled.launches)):
+                self.lib.graph_begin_capture(stream)
+                try:
+                    for _ in range(batch_sizes[i]):
+                        self.launch_one(i, stream)
+                finally:
+                    g = self.lib.graph_end_capture(stream)
+                self._launch_graphs[i] = g
+        except launcher.LauncherError as exc:
+            self._drop_launch_graphs()
+            raise GraphCaptureError(f"graph capture failed: {exc}") from exc
+        self._launch_graph_sizes = list(batch_sizes)
+
+    def _drop_launch_graphs(self) -> None:
+        for g in self._launch_graphs.values():
+            self.lib.graph_destroy(g)
+        self._launch_graphs = {}
+        self._launch_graph_sizes = None
+
+    def capture_program_graph(self) -> None:
+        """One graph holding every launch in program order."""
+        if self._program_graph is not None:
+            return
+        stream = self._ensure_stream()
+        self.lib.stream_synchronize(stream)
+        try:
+            self.lib.graph_begin_capture(stream)
+            try:
+                self.run(stream)
+            finally:
+                g = self.lib.graph_end_capture(stream)
+        except launcher.LauncherError as exc:
+            raise GraphCaptureError(f"whole-program graph capture failed: {exc}") from exc
+        self._program_graph = g
+
+    def replay_program(self, stream: int | None = None) -> None:
+        if self._program_graph is None:
+            self.capture_program_graph()
+        self.lib.graph_launch(self._program_graph, self._ensure_stream() if stream is None else stream)
+
+    def time_program_window(self, replays: int) -> float:
+        """ms per whole-program replay over one event window of ``replays`` replays."""
+        stream = self._ensure_stream()
+        if not hasattr(self, "_win"):
+            self._win = (self._event(), self._event())
+        start, stop = self._win
+        self.lib.event_record(start, stream)
+        for _ in range(replays):
+            self.lib.graph_launch(self._program_graph, stream)
+        self.lib.event_record(stop, stream)
+        self._wait_for_event(stop, "whole-program graph")
+        return self._elapsed(start, stop, "whole-program graph") / replays
+
+    def close(self) -> None:
+        self._drop_launch_graphs()
+        if self._program_graph is not None:
+            self.lib.graph_destroy(self._program_graph)
+            self._program_graph = None
+        for e in self._events:
+            self.lib.event_destroy(e)
+        self._events = []
+        if hasattr(self, "_win"):
+            del self._win
+        if self._stream is not None:
+            self.lib.stream_synchronize(self._stream)
+            self.lib.stream_destroy(self._stream)
+            self._stream = None
+
+
+# ---------------------------------------------------------------------------
+# Entry points
+# ---------------------------------------------------------------------------
+
+
+def run_program(graph: Graph, input_data: dict | None = None, pre_run=None) -> tuple[RunResult, object]:
+    """Compile, allocate, launch once and fetch outputs — all inside the GPU lock (program.py:1098-1119)."""
+    with gpu_lock():
+        prog = CompiledProgram.build(graph, input_data)
+        try:
+            pre_result = pre_run() if pre_run is not None else None
+            torch = _torch()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            prog.run()
+            torch.cuda.synchronize()
+            elapsed = (time.perf_counter() - t0) * 1000.0
+            outputs = prog.outputs()
+        finally:
+            prog.close()
+    return RunResult(outputs=outputs, time_ms=elapsed), pre_result
+
+
+def _resolve_iter_budget(num_iters) -> tuple[float, int, bool]:
+    if isinstance(num_iters, str):
+        if num_iters != "auto":
+            raise ValueError(f"num_iters must be int or 'auto', got {num_iters!r}")
+        return (_AUTO_BUDGET_MS, _AUTO_MAX_ITERS, True)
+    return (float("inf"), int(num_iters), False)
+
+
+def _calibrate_batch_sizes(iter_dts: list[float]) -> list[int]:
+    return [max(1, int(round(_BATCH_TARGET_MS / dt))) if 0 < dt < _BATCH_TARGET_MS else 1 for dt in iter_dts]
+
+
+def _samples_to_result(samples: list[list[float]], launches: list[_Launch], *, captured: bool, e2e_samples: list[float]) -> BenchmarkResult:
+    per_launch = []
+    for i, ln in enumerate(launches):
+        s = samples[i]
+        per_launch.append(LaunchTime(idx=i, kernel_name=ln.kernel_name, time_ms=statistics.median(s) if s else 0.0, samples=tuple(s)))
+    total = sum(p.time_ms for p in per_launch)
+    mins = sum(min(samples[i]) for i in range(len(launches)) if samples[i])
+    maxs = sum(max(samples[i]) for i in range(len(launches)) if samples[i])
+    return BenchmarkResult(
+        time_ms=total,
+        min_ms=mins,
+        max_ms=maxs,
+        num_launches=len(launches),
+        per_launch=per_launch,
+        captured=captured,
+        e2e_ms=statistics.median(e2e_samples) if e2e_samples else None,
+        e2e_min_ms=min(e2e_samples) if e2e_samples else None,
+    )
+
+
+def benchmark_program(
+    graph: Graph,
+    input_data: dict | None = None,
+    warmup: int = 5,
+    num_iters=20,
+    on_iter=None,
+    compile_timeout_s: float | None = None,
+    run_timeout_s: float | None = None,
+    capture_graphs: bool = True,
+) -> BenchmarkResult:
+    """Time the program's launches with device events (program.py:1152-1325).
+
+    One loop covers warm-up and measurement.  After ``warmup`` iterations the
+    per-launch batch sizes are calibrated so each event window spans about
+    ``_BATCH_TARGET_MS`` and, when ``capture_graphs`` holds, each batch is
+    captured into a graph so windows hold dense device work.  Warm-up is
+    extended until ``_WARMUP_TARGET_MS`` of device time has run.  Reported
+    per-launch time is the median of measured windows; a multi-launch program
+    also gets whole-program graph windows (``e2e_ms``).  Budgets: the per-window
+    watchdog (``HungKernelError``), ``run_timeout_s`` of accumulated device time,
+    and zero-elapsed windows raise ``RuntimeError`` (bench_fail)."""
+    target_total_ms, max_measured, auto = _resolve_iter_budget(num_iters)
+    with gpu_lock():
+        prog = CompiledProgram.build(graph, input_data, compile_timeout_s=compile_timeout_s)
+        try:
+            n = len(prog.compiled.launches)
+            batch_sizes = [1] * n
+            samples: list[list[float]] = [[] for _ in range(n)]
+            measure_e2e = n > 1
+            e2e_samples: list[float] = []
+            e2e_replays = 0
+            iters_run = measured = 0
+            cumulative_ms = total_ms = 0.0
+
+            def try_capture(sizes: list[int]) -> bool:
+                try:
+                    prog.capture_launch_graphs(sizes)
+                except GraphCaptureError as exc:
+                    logger.warning("[hip] %s — continuing with uncaptured (dispatch-inclusive) timing", exc)
+                    return False
+                return True
+
+            if capture_graphs and warmup == 0:
+                capture_graphs = try_capture(batch_sizes)
+            while True:
+                dts = prog.iter_once(batch_sizes, pre_iter=on_iter)
+                iters_run += 1
+                total_ms += sum(dts[i] * batch_sizes[i] for i in range(n))
+                if run_timeout_s is not None and total_ms > run_timeout_s * 1000.0:
+                    raise RuntimeError(f"benchmark run stage exceeded {run_timeout_s:.1f}s of GPU time — variant marked bench_fail")
+                if iters_run == warmup:
+                    batch_sizes = _calibrate_batch_sizes(dts)
+                    if capture_graphs:
+                        capture_graphs = try_capture(batch_sizes)
+                    if total_ms < _WARMUP_TARGET_MS:
+                        per_iter = sum(dts[i] * batch_sizes[i] for i in range(n))
+                        if per_iter > 0:
+                            warmup += int(math.ceil((_WARMUP_TARGET_MS - total_ms) / per_iter))
+                if iters_run <= warmup:
+                    continue
+                for i in range(n):
+                    samples[i].append(dts[i])
+                cumulative_ms += sum(dts[i] * batch_sizes[i] for i in range(n))
+                measured += 1
+                if measure_e2e and capture_graphs:
+                    if e2e_replays == 0:
+                        try:
+                            prog.capture_program_graph()
+                        except GraphCaptureError as exc:
+                            logger.warning("[hip] %s — skipping whole-program e2e timing", exc)
+                            measure_e2e = False
+                        else:
+                            it = sum(dts)
+                            e2e_replays = max(1, int(round(_BATCH_TARGET_MS / it))) if 0 < it < _BATCH_TARGET_MS else 1
+                    if measure_e2e:
+                        dt = prog.time_program_window(e2e_replays)
+                        e2e_samples.append(dt)
+                        total_ms += dt * e2e_replays
+                if measured >= max_measured or (auto and cumulative_ms >= target_total_ms):
+                    break
+            return _samples_to_result(samples, prog.compiled.launches, captured=capture_graphs, e2e_samples=e2e_samples)
+        finally:
+            prog.close()

@@ -1,0 +1,234 @@
+"""Row-reduction emitter: fused statistic(s) + projection kernels for gfx950.
+
+Covers what the reference builds from ``_tile_reduce_axis`` / ``emit_combine``
+(emmy/compiler/pipeline/passes/lowering/kernel/_factor.py:467-521, 652-746)
+plus ``WarpShuffle`` / ``TreeHalve`` (emmy/compiler/ir/kernel/ir.py:569-702),
+designed for wave64 instead of translated:
+
+* ``coop`` lanes own one row.  Each lane keeps its slice of the row **resident
+  in registers** (16-byte vector loads, lane-interleaved so every wave-load is
+  one contiguous run), so the row is read from HBM exactly once however many
+  statistics are taken — the reference's cooperative form re-reads the row per
+  pass (``StridedLoop`` per statistic, _factor.py:652-746).
+* Lane partials combine with DPP / swizzle / permlane butterflies only
+  (``prelude.WAVE_REDUCE``).  Rows wider than one wave add a single LDS
+  hand-off of ``coop/64`` partials per statistic — never a log-tree of
+  barriers.
+* A statistic's pre-map may replace the resident element (``Stat.keep``):
+  softmax stores ``exp(x - max)`` once and the projection only scales it.
+"""
+
+from __future__ import annotations
+
+from deplodock_amd.context import Context
+from deplodock_amd.dtype import BF16, F16, F32, DType
+from deplodock_amd.emit import prelude
+from deplodock_amd.emit.errors import LoweringError
+from deplodock_amd.ir import expr as E
+from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.tile import RowReduce
+
+_MAX_RESIDENT = 64  # fp32 row elements a lane may keep in registers
+
+_VEC_T = {
+    ("f32", 4): "f32x4",
+    ("f32", 2): "f32x2",
+    ("f32", 1): "float",
+    ("bf16", 8): "bf16x8",
+    ("bf16", 4): "bf16x4",
+    ("bf16", 2): "bf16x2",
+    ("bf16", 1): "__bf16",
+    ("f16", 8): "f16x8",
+    ("f16", 4): "f16x4",
+    ("f16", 2): "f16x2",
+    ("f16", 1): "_Float16",
+}
+
+
+def pick_vec(cols: int, dtypes: list[DType], strides: list[int]) -> int:
+    """Widest element count per access such that the widest dtype moves 16 bytes
+    and every row start stays aligned."""
+    v = 16 // max(d.nbytes for d in dtypes)
+    while v > 1 and (cols % v or any(s % v for s in strides)):
+        v //= 2
+    return v
+
+
+def _load_vec(ptr: str, idx: str, dt: DType, v: int, dst: str, nontemporal: bool) -> list[str]:
+    """Lines that load ``v`` elements of ``dt`` at vector index ``idx`` into ``float dst[v]``."""
+    vt = _VEC_T[(dt.name, v)]
+    addr = f"((const {vt}*)({ptr}))[{idx}]" if v > 1 else f"({ptr})[{idx}]"
+    if nontemporal:
+        addr = f"__builtin_nontemporal_load(&{addr})"
+    if v == 1:
+        return [f"{dst}[0] = (float){addr};"]
+    lines = [f"{{ {vt} t_ = {addr};"]
+    if dt is F32:
+        lines += [f"  {dst}[{j}] = t_[{j}];" for j in range(v)]
+    else:
+        lines += [f"  {dst}[{j}] = (float)t_[{j}];" for j in range(v)]
+    lines.append("}")
+    return lines
+
+
+def _store_vec(ptr: str, idx: str, dt: DType, v: int, src: str, nontemporal: bool) -> list[str]:
+    vt = _VEC_T[(dt.name, v)]
+    cast = "" if dt is F32 else f"({dt.c_name})"
+    if v == 1:
+        tgt = f"({ptr})[{idx}]"
+        val = f"{cast}{src}[0]"
+        return [f"__builtin_nontemporal_store({val}, &{tgt});" if nontemporal else f"{tgt} = {val};"]
+    lines = [f"{{ {vt} t_;"]
+    lines += [f"  t_[{j}] = {cast}{src}[{j}];" for j in range(v)]
+    tgt = f"(({vt}*)({ptr}))[{idx}]"
+    lines.append(f"  __builtin_nontemporal_store(t_, &{tgt});" if nontemporal else f"  {tgt} = t_;")
+    lines.append("}")
+    return lines
+
+
+def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context(), *, nontemporal: bool = False) -> HipOp:
+    """Render ``body`` (schedule already stamped on ``body.reduce``) to a HipOp."""
+    plan = body.reduce
+    L = plan.coop
+    if plan.cta != 1:
+        raise LoweringError("row reduce: cross-workgroup split (g<n>) is not defined for a projected row")
+    stride_in = body.row_stride_in if body.row_stride_in is not None else body.cols
+    stride_out = body.row_stride_out if body.row_stride_out is not None else body.cols
+    col_dts = [dt for _, dt in body.col_operands]
+    V = pick_vec(body.cols, [body.x_dtype, body.out_dtype, *col_dts], [stride_in, stride_out])
+    C = body.cols // V  # vector chunks per row
+    NV = -(-C // L)  # chunks per lane
+    if NV * V > _MAX_RESIDENT:
+        raise LoweringError(
+            f"row reduce: {body.cols} columns over {L} lanes needs {NV * V} resident elements per lane "
+            f"(> {_MAX_RESIDENT}); widen REDUCE b<n>"
+        )
+    masked = C % L != 0
+    T = max(L, min(256, ctx.max_threads_per_block))
+    if body.rows_per_block is not None:
+        T = L * body.rows_per_block
+    if T > ctx.max_threads_per_block or T % L:
+        raise LoweringError(f"row reduce: {T} threads per workgroup is not launchable")
+    R = T // L
+    # Do not spread fewer rows than one workgroup holds over idle lanes.
+    while R > 1 and R > body.rows and T > ctx.wave_size:
+        R //= 2
+        T = L * R
+    grid = -(-body.rows // R)
+    row_guard = body.rows % R != 0
+    NW = max(1, L // ctx.wave_size)  # waves per row
+    W = min(L, ctx.wave_size)  # butterfly width
+
+    stat_names = [s.name for s in body.stats]
+    known = {"x", *stat_names, *(n for n, _ in body.col_operands)}
+    for s_i, st in enumerate(body.stats):
+        unknown = E.variables(st.pre) - ({"x"} | set(stat_names[:s_i]))
+        if unknown:
+            raise LoweringError(f"stat {st.name!r}: pre-map uses unknown names {sorted(unknown)}")
+    unknown = E.variables(body.project) - known
+    if unknown:
+        raise LoweringError(f"projection uses unknown names {sorted(unknown)}")
+
+    params = [f"const {body.x_dtype.c_name}* __restrict__ x"]
+    params += [f"const {dt.c_name}* __restrict__ c{ci}" for ci, (_, dt) in enumerate(body.col_operands)]
+    params.append(f"{body.out_dtype.c_name}* __restrict__ out")
+
+    o: list[str] = []
+    a = o.append
+    a(f"// {name}: rows={body.rows} cols={body.cols} REDUCE={plan.spell() or 'serial'} vec={V} rows/wg={R}")
+    a(f'extern "C" __global__ __launch_bounds__({T}) void {name}({", ".join(params)}) {{')
+    a(f"  const int lane = threadIdx.x % {L};")
+    a(f"  const int rib = threadIdx.x / {L};")
+    a(f"  long row = (long)blockIdx.x * {R} + rib;")
+    if row_guard:
+        a(f"  const bool row_ok = row < {body.rows}L;")
+        a(f"  if (!row_ok) row = {body.rows - 1}L;")
+    a(f"  const {body.x_dtype.c_name}* xr = x + row * {stride_in}L;")
+    a(f"  float xv[{NV}][{V}];")
+    if masked:
+        a(f"  bool ok[{NV}];")
+    for i in range(NV):
+        idx = f"{i * L} + lane"
+        if masked and (i + 1) * L > C:
+            a(f"  ok[{i}] = ({idx}) < {C};")
+            a(f"  if (ok[{i}]) {{")
+            o.extend("    " + ln for ln in _load_vec("xr", idx, body.x_dtype, V, f"xv[{i}]", nontemporal))
+            a("  } else {")
+            a(f"    for (int j = 0; j < {V}; ++j) xv[{i}][j] = 0.0f;")
+            a("  }")
+        else:
+            if masked:
+                a(f"  ok[{i}] = true;")
+            o.extend("  " + ln for ln in _load_vec("xr", idx, body.x_dtype, V, f"xv[{i}]", nontemporal))
+
+    if NW > 1:
+        a(f"  __shared__ float emh_part[{len(body.stats)}][{R}][{NW}];")
+        a(f"  const int wave_in_row = lane / {ctx.wave_size};")
+
+    env_base = {s: f"s_{s}" for s in stat_names}
+    for s_i, st in enumerate(body.stats):
+        mono = prelude.MONOID_STRUCT[st.monoid]
+        nacc = max(1, min(plan.reg, NV * V))
+        a(f"  float acc_{st.name}[{nacc}];")
+        a(f"  for (int r = 0; r < {nacc}; ++r) acc_{st.name}[r] = {mono}::identity();")
+        e_idx = 0
+        for i in range(NV):
+            guard = f"if (ok[{i}]) " if masked and (i + 1) * L > C else ""
+            a(f"  {guard}{{")
+            for j in range(V):
+                env = dict(env_base, x=f"xv[{i}][{j}]")
+                val = E.render(st.pre, env)
+                r = e_idx % nacc
+                if st.keep:
+                    a(f"    xv[{i}][{j}] = {val};")
+                    val = f"xv[{i}][{j}]"
+                a(f"    acc_{st.name}[{r}] = {mono}::op(acc_{st.name}[{r}], {val});")
+                e_idx += 1
+            a("  }")
+        a(f"  float s_{st.name} = acc_{st.name}[0];")
+        for r in range(1, nacc):
+            a(f"  s_{st.name} = {mono}::op(s_{st.name}, acc_{st.name}[{r}]);")
+        a(f"  s_{st.name} = emh_wave_reduce<{mono}, {W}>(s_{st.name});")
+        if NW > 1:
+            a(f"  if ((lane % {ctx.wave_size}) == 0) emh_part[{s_i}][rib][wave_in_row] = s_{st.name};")
+            a("  __syncthreads();")
+            a(f"  s_{st.name} = emh_part[{s_i}][rib][0];")
+            for w in range(1, NW):
+                a(f"  s_{st.name} = {mono}::op(s_{st.name}, emh_part[{s_i}][rib][{w}]);")
+
+    a(f"  {body.out_dtype.c_name}* orow = out + row * {stride_out}L;")
+    if row_guard:
+        a("  if (row_ok) {")
+    for i in range(NV):
+        idx = f"{i * L} + lane"
+        guard = f"if (ok[{i}]) " if masked and (i + 1) * L > C else ""
+        a(f"  {guard}{{")
+        a(f"    float y[{V}];")
+        for ci, (_, dt) in enumerate(body.col_operands):
+            a(f"    float cv{ci}[{V}];")
+            o.extend("    " + ln for ln in _load_vec(f"c{ci}", idx, dt, V, f"cv{ci}", False))
+        for j in range(V):
+            env = dict(env_base, x=f"xv[{i}][{j}]")
+            env.update({n: f"cv{ci}[{j}]" for ci, (n, _) in enumerate(body.col_operands)})
+            a(f"    y[{j}] = {E.render(body.project, env)};")
+        o.extend("    " + ln for ln in _store_vec("orow", idx, body.out_dtype, V, "y", nontemporal))
+        a("  }")
+    if row_guard:
+        a("  }")
+    a("}")
+
+    source = prelude.header(prelude.WAVE_REDUCE) + "\n".join(o) + "\n"
+    return HipOp(
+        kernel_source=source,
+        kernel_name=name,
+        arg_order=(body.x, *(n for n, _ in body.col_operands), body.out),
+        grid=((grid,), (1,), (1,)),
+        block=((T,), (1,), (1,)),
+        lds_bytes=0,
+        comment=f"row_reduce rows={body.rows} cols={body.cols} REDUCE={plan.spell()}",
+        algo_bytes=body.algo_bytes(),
+        knobs={"REDUCE": plan.spell(), "VEC": V, "NT": int(nontemporal)},
+    )
+
+
+__all__ = ["emit_row_reduce", "pick_vec", "BF16", "F16"]

@@ -1,0 +1,206 @@
+"""Scalar expression trees used inside kernel bodies (projections, epilogues).
+
+A small counterpart of the reference's elementwise vocabulary
+(emmy/compiler/ir/elementwise.py:36-78, intrinsic spellings
+emmy/compiler/ir/kernel/render.py:374-384).  An expression renders to HIP C
+(``render``) and evaluates on numpy arrays (``evaluate``) so kernel bodies can
+be checked on the host without a GPU.
+
+All arithmetic is fp32.  ``Round(bf16)`` marks a point where the value is
+rounded to a storage type and widened again — this is how a fused kernel
+reproduces the rounding points of an eager bf16 module.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+
+from deplodock_amd.dtype import bf16_bits_from_f32, f32_from_bf16_bits
+
+
+class Expr:
+    def __add__(self, o):
+        return Bin("add", self, wrap(o))
+
+    def __radd__(self, o):
+        return Bin("add", wrap(o), self)
+
+    def __sub__(self, o):
+        return Bin("sub", self, wrap(o))
+
+    def __rsub__(self, o):
+        return Bin("sub", wrap(o), self)
+
+    def __mul__(self, o):
+        return Bin("mul", self, wrap(o))
+
+    def __rmul__(self, o):
+        return Bin("mul", wrap(o), self)
+
+    def __truediv__(self, o):
+        return Bin("div", self, wrap(o))
+
+    def __neg__(self):
+        return Un("neg", self)
+
+
+@dataclass(frozen=True, eq=False)
+class Var(Expr):
+    name: str
+
+
+@dataclass(frozen=True, eq=False)
+class Const(Expr):
+    value: float
+
+
+@dataclass(frozen=True, eq=False)
+class Un(Expr):
+    op: str  # neg | exp | rsqrt | sqrt | rcp | sigmoid | silu | abs | tanh
+    a: Expr
+
+
+@dataclass(frozen=True, eq=False)
+class Bin(Expr):
+    op: str  # add | sub | mul | div | max | min
+    a: Expr
+    b: Expr
+
+
+@dataclass(frozen=True, eq=False)
+class Round(Expr):
+    """Round to ``dtype`` storage precision ("bf16" | "f16") and widen back to fp32."""
+
+    dtype: str
+    a: Expr
+
+
+def wrap(v) -> Expr:
+    if isinstance(v, Expr):
+        return v
+    return Const(float(v))
+
+
+def float_literal(v: float) -> str:
+    """An fp32 literal that round-trips exactly (hex float)."""
+    f = float(np.float32(v))
+    if f != f:
+        return "__builtin_nanf(\"\")"
+    if f in (float("inf"), float("-inf")):
+        return "__builtin_inff()" if f > 0 else "(-__builtin_inff())"
+    return f"{f.hex()}f"
+
+
+_UN_C = {
+    "neg": "(-({a}))",
+    "exp": "expf({a})",
+    "exp2": "exp2f({a})",
+    "fast_exp2": "__builtin_amdgcn_exp2f({a})",
+    "rsqrt": "rsqrtf({a})",
+    "sqrt": "sqrtf({a})",
+    "rcp": "(1.0f / ({a}))",
+    "abs": "fabsf({a})",
+    "tanh": "tanhf({a})",
+    # x * 1/(1+e^-x): the reference's SiLU decomposition
+    # (emmy/compiler/pipeline/passes/frontend/decomposition/020_silu.py).
+    "sigmoid": "(1.0f / (1.0f + expf(-({a}))))",
+    "silu": "(({a}) / (1.0f + expf(-({a}))))",
+}
+_BIN_C = {
+    "add": "(({a}) + ({b}))",
+    "sub": "(({a}) - ({b}))",
+    "mul": "(({a}) * ({b}))",
+    "div": "(({a}) / ({b}))",
+    "max": "fmaxf({a}, {b})",
+    "min": "fminf({a}, {b})",
+}
+_ROUND_C = {"bf16": "emh_round_bf16({a})", "f16": "((float)(_Float16)({a}))"}
+
+
+def render(e: Expr, env: dict[str, str]) -> str:
+    """HIP C text of ``e``; ``env`` maps variable names to C expressions."""
+    if isinstance(e, Var):
+        return env[e.name]
+    if isinstance(e, Const):
+        return float_literal(e.value)
+    if isinstance(e, Un):
+        return _UN_C[e.op].format(a=render(e.a, env))
+    if isinstance(e, Bin):
+        return _BIN_C[e.op].format(a=render(e.a, env), b=render(e.b, env))
+    if isinstance(e, Round):
+        return _ROUND_C[e.dtype].format(a=render(e.a, env))
+    raise TypeError(f"cannot render {type(e).__name__}")
+
+
+def evaluate(e: Expr, env: dict[str, np.ndarray]) -> np.ndarray:
+    """Numpy fp32 evaluation with the same rounding points as the device code."""
+    f32 = np.float32
+    if isinstance(e, Var):
+        return np.asarray(env[e.name], dtype=f32)
+    if isinstance(e, Const):
+        return f32(e.value)
+    if isinstance(e, Round):
+        a = np.asarray(evaluate(e.a, env), dtype=f32)
+        if e.dtype == "bf16":
+            return f32_from_bf16_bits(bf16_bits_from_f32(a)).reshape(a.shape)
+        return a.astype(np.float16).astype(f32)
+    if isinstance(e, Un):
+        a = np.asarray(evaluate(e.a, env), dtype=f32)
+        with np.errstate(over="ignore", divide="ignore", invalid="ignore"):
+            return {
+                "neg": lambda: -a,
+                "exp": lambda: np.exp(a),
+                "exp2": lambda: np.exp2(a),
+                "fast_exp2": lambda: np.exp2(a),
+                "rsqrt": lambda: (f32(1) / np.sqrt(a)).astype(f32),
+                "sqrt": lambda: np.sqrt(a),
+                "rcp": lambda: (f32(1) / a).astype(f32),
+                "abs": lambda: np.abs(a),
+                "tanh": lambda: np.tanh(a),
+                "sigmoid": lambda: (f32(1) / (f32(1) + np.exp(-a))).astype(f32),
+                "silu": lambda: (a / (f32(1) + np.exp(-a))).astype(f32),
+            }[e.op]().astype(f32)
+    if isinstance(e, Bin):
+        a = np.asarray(evaluate(e.a, env), dtype=f32)
+        b = np.asarray(evaluate(e.b, env), dtype=f32)
+        with np.errstate(over="ignore", divide="ignore", invalid="ignore"):
+            return {
+                "add": lambda: a + b,
+                "sub": lambda: a - b,
+                "mul": lambda: a * b,
+                "div": lambda: a / b,
+                "max": lambda: np.maximum(a, b),
+                "min": lambda: np.minimum(a, b),
+            }[e.op]().astype(f32)
+    raise TypeError(f"cannot evaluate {type(e).__name__}")
+
+
+def variables(e: Expr) -> set[str]:
+    if isinstance(e, Var):
+        return {e.name}
+    if isinstance(e, Const):
+        return set()
+    if isinstance(e, (Un, Round)):
+        return variables(e.a)
+    if isinstance(e, Bin):
+        return variables(e.a) | variables(e.b)
+    raise TypeError(type(e).__name__)
+
+
+def pretty(e: Expr) -> str:
+    if isinstance(e, Var):
+        return e.name
+    if isinstance(e, Const):
+        return repr(float(np.float32(e.value)))
+    if isinstance(e, Un):
+        return f"{e.op}({pretty(e.a)})"
+    if isinstance(e, Round):
+        return f"{e.dtype}({pretty(e.a)})"
+    if isinstance(e, Bin):
+        sym = {"add": "+", "sub": "-", "mul": "*", "div": "/"}.get(e.op)
+        if sym:
+            return f"({pretty(e.a)} {sym} {pretty(e.b)})"
+        return f"{e.op}({pretty(e.a)}, {pretty(e.b)})"
+    raise TypeError(type(e).__name__)

@@ -1,0 +1,186 @@
+"""Tile IR — one scheduled kernel per ``TileOp``.
+
+The input contract of the gfx950 lowering, playing the role of the
+reference's ``TileOp`` (emmy/compiler/ir/tile/ir.py:424-459) whose body is a
+``Map`` (:392), ``Reduction`` (:89) or ``Contraction`` (:196) with the schedule
+plans stamped on it (``ReducePlan`` / ``TilePlan`` / ``Stage``).  The emitters
+apply a stamped plan verbatim and decide nothing.
+
+Buffers are named by graph node id.  Element-wise pieces (statistic
+pre-maps, projections, epilogues) are ``ir.expr`` trees over named scalars.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+from deplodock_amd.dtype import DType
+from deplodock_amd.ir.base import Op
+from deplodock_amd.ir.expr import Expr
+from deplodock_amd.ir.schedule import ReducePlan, Stage, TilePlan
+
+
+@dataclass(frozen=True)
+class Stat:
+    """One row statistic: ``name = monoid over columns of pre(x, earlier stats)``."""
+
+    name: str
+    monoid: str  # "sum" | "max" | "min"
+    pre: Expr  # over Var("x") and earlier stat names
+    keep: bool = False  # the pre-mapped value replaces the resident element ``x``
+
+
+@dataclass
+class RowReduce:
+    """``Map(source=Reduction)``: per-row statistics followed by a projection.
+
+    ``x`` is ``[rows, cols]`` with the reduce axis innermost and contiguous and
+    ``row_stride_*`` elements between rows.  ``project`` is evaluated per
+    element over ``x``, the statistics, and the per-column operands
+    (``col_operands``: vectors of length ``cols`` such as a norm weight).
+    RMSNorm is ``stats=(ss = sum x*x)``, ``project = x * rsqrt(ss/cols + eps) * w``
+    (emmy/compiler/ir/frontend/ir.py:309-312); softmax is ``m = max x``,
+    ``d = sum exp(x - m)``, ``project = exp(x - m) / d`` (:354-358)."""
+
+    rows: int
+    cols: int
+    x: str
+    x_dtype: DType
+    out: str
+    out_dtype: DType
+    stats: tuple[Stat, ...]
+    project: Expr
+    col_operands: tuple[tuple[str, DType], ...] = ()
+    row_stride_in: int | None = None
+    row_stride_out: int | None = None
+    reduce: ReducePlan = field(default_factory=ReducePlan)
+    rows_per_block: int | None = None  # derived from the plan when None
+
+    def algo_bytes(self) -> int:
+        b = self.rows * self.cols * (self.x_dtype.nbytes + self.out_dtype.nbytes)
+        for _, dt in self.col_operands:
+            b += self.cols * dt.nbytes
+        return b
+
+
+@dataclass
+class Contraction:
+    """``out[m, n] = epilogue(sum_k a[m, k] * b[n, k])`` — both operands
+    K-contiguous (the reference's ``b_trans`` layout for ``nn.Linear`` weights,
+    emmy/compiler/ir/tile/ir.py:325).  ``epilogue`` is an expression over
+    ``acc`` and the names in ``epilogue_operands`` (``[m, n]`` tensors such as a
+    residual).  With ``gate_pair`` the weight holds two stacked matrices
+    ``[2n, k]`` and the epilogue sees ``acc`` (rows ``0..n``) and ``acc2`` (rows
+    ``n..2n``) — the SwiGLU gate/up pair computed in one pass over ``a``."""
+
+    m: int
+    n: int
+    k: int
+    a: str
+    b: str
+    out: str
+    in_dtype: DType
+    out_dtype: DType
+    epilogue: Expr | None = None
+    epilogue_operands: tuple[tuple[str, DType], ...] = ()
+    gate_pair: bool = False
+    tile: TilePlan | None = None
+    stage: Stage | None = None
+    reduce: ReducePlan = field(default_factory=ReducePlan)  # split-K
+    lda: int | None = None
+    ldb: int | None = None
+    ldo: int | None = None
+
+    def algo_flops(self) -> int:
+        return 2 * self.m * self.n * self.k * (2 if self.gate_pair else 1)
+
+    def algo_bytes(self) -> int:
+        nb = self.n * (2 if self.gate_pair else 1)
+        b = (self.m * self.k + nb * self.k) * self.in_dtype.nbytes + self.m * self.n * self.out_dtype.nbytes
+        for _, dt in self.epilogue_operands:
+            b += self.m * self.n * dt.nbytes
+        return b
+
+
+@dataclass
+class Flash:
+    """Fused attention ``softmax(q k^T * scale + causal) v`` with grouped KV
+    heads (``kv head = q head // group``), streamed over keys with the online
+    (m, l, O) carrier (emmy/compiler/pipeline/passes/lowering/kernel/_twist.py:229-363).
+
+    Tensors are addressed as ``base + b*stride_b + h*stride_h + s*stride_s + d``
+    (``d`` contiguous), so ``[B,H,S,D]`` and ``[B,S,H,D]`` both fit."""
+
+    batch: int
+    q_heads: int
+    kv_heads: int
+    q_len: int
+    kv_len: int
+    head_dim: int
+    q: str
+    k: str
+    v: str
+    out: str
+    dtype: DType
+    scale: float
+    causal: bool
+    q_strides: tuple[int, int, int]  # (batch, head, seq) in elements
+    k_strides: tuple[int, int, int]
+    v_strides: tuple[int, int, int]
+    o_strides: tuple[int, int, int]
+    block_q: int = 128
+    block_kv: int = 64
+    waves: int = 4
+
+    def algo_flops(self) -> int:
+        if self.causal and self.q_len == self.kv_len:
+            pairs = self.q_len * (self.q_len + 1) // 2
+        else:
+            pairs = self.q_len * self.kv_len
+        return 4 * self.batch * self.q_heads * self.head_dim * pairs
+
+    def algo_bytes(self) -> int:
+        e = self.dtype.nbytes
+        q = self.batch * self.q_heads * self.q_len * self.head_dim
+        kv = self.batch * self.kv_heads * self.kv_len * self.head_dim
+        return (2 * q + 2 * kv) * e
+
+
+@dataclass
+class MapOperand:
+    """One pointwise input.  ``index`` names the addressing scheme:
+    ``"flat"`` (same linear index as the output) or ``"row"`` / ``"col"``
+    broadcasts described by the owning ``Map``."""
+
+    name: str
+    dtype: DType
+    index: str = "flat"
+
+
+@dataclass
+class Map:
+    """Pointwise kernel: ``out[i] = expr(operands[i])`` over ``numel`` cells."""
+
+    numel: int
+    operands: tuple[MapOperand, ...]
+    expr: Expr
+    out: str
+    out_dtype: DType
+    inner: int = 1  # extent of the innermost axis, for "col" broadcasts
+
+    def algo_bytes(self) -> int:
+        b = self.numel * self.out_dtype.nbytes
+        for o in self.operands:
+            b += (self.numel if o.index == "flat" else self.inner) * o.dtype.nbytes
+        return b
+
+
+@dataclass
+class TileOp(Op):
+    """One kernel: a name plus a scheduled body."""
+
+    name: str = ""
+    body: object = None
+
+    def pretty_body(self) -> str:
+        return f"{self.name}: {self.body!r}"
