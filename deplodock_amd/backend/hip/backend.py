@@ -1,0 +1,129 @@
+"""HIP backend: ``Graph`` → lowered ``Graph[HipOp]`` → hipRTC → MI355X.
+
+Same call surface as the reference's ``CudaBackend``
+(emmy/compiler/backend/cuda/backend.py:59-237): the compiled artifact is the
+lowered graph itself; ``run`` returns host arrays; ``benchmark_async`` is the
+single benchmarking entry point.  Differences that follow from the platform:
+constants traced from a module are bound automatically from the traced
+parameter values unless ``input_data`` overrides them, and tensors may be
+passed as device ``torch.Tensor`` objects, in which case they are used in place.
+"""
+
+from __future__ import annotations
+
+from deplodock_amd import config
+from deplodock_amd.backend import Backend, BenchmarkResult, RunResult
+from deplodock_amd.context import Context
+from deplodock_amd.graph import Graph
+from deplodock_amd.pipeline import HIP_PASSES, Pipeline
+
+
+class HipBackend(Backend):
+    name = "hip"
+
+    def __init__(
+        self,
+        *,
+        debug: bool | None = None,
+        dump=None,
+        bench_wall_timeout_s: float | None = None,
+        bench_compile_timeout_s: float = 30.0,
+        bench_run_timeout_s: float = 10.0,
+        tune_db=None,
+        device_id: int | None = None,
+        context: Context | None = None,
+    ) -> None:
+        self.debug = config.debug_enabled() if debug is None else debug
+        self.dump = dump
+        self.bench_wall_timeout_s = bench_wall_timeout_s
+        self.bench_compile_timeout_s = bench_compile_timeout_s
+        self.bench_run_timeout_s = bench_run_timeout_s
+        self.tune_db = tune_db
+        self.device_id = device_id
+        self.context = context or Context()
+
+    # -- compile ------------------------------------------------------------
+    def compile(self, graph: Graph) -> Graph:
+        """Lower ``Graph`` → ``Graph[TileOp]`` → ``Graph[HipOp]`` (needs no GPU)."""
+        return Pipeline.build(HIP_PASSES, self.context).run(graph, dump_dir=self.dump)
+
+    # -- binding ------------------------------------------------------------
+    @staticmethod
+    def bind(compiled: Graph, input_data: dict | None) -> dict:
+        """``input_data`` completed with the traced parameter values of every
+        constant it does not override (stacked constants are assembled here)."""
+        from deplodock_amd.passes.fuse import StackedConstant
+
+        data = dict(input_data or {})
+        traced = getattr(compiled, "constant_values", {})
+        for nid, _op in compiled.constant_ops():
+            if nid in data:
+                continue
+            stacked = compiled.nodes[nid].hints.get("stacked")
+            if isinstance(stacked, StackedConstant):
+                import torch
+
+                parts = [data[p] if p in data else traced[p] for p in stacked.parts]
+                data[nid] = torch.cat([p if isinstance(p, torch.Tensor) else torch.as_tensor(p) for p in parts], dim=0).contiguous()
+            elif nid in traced:
+                data[nid] = traced[nid]
+        return data
+
+    # -- run ------------------------------------------------------------------
+    def run(self, compiled: Graph, *, input_data: dict | None = None, pre_run=None) -> tuple[RunResult, object]:
+        from deplodock_amd.backend.hip.program import run_program
+
+        self._select_device()
+        result, pre = run_program(compiled, input_data=self.bind(compiled, input_data), pre_run=pre_run)
+        outputs = {}
+        for name, vals in result.outputs.items():
+            outputs[name] = vals
+            for alias, shape in compiled.nodes[name].hints.get("output_alias", []):
+                outputs[alias] = vals.reshape(shape)
+        return RunResult(outputs=outputs, time_ms=result.time_ms), pre
+
+    def program(self, compiled: Graph, input_data: dict | None = None):
+        """A persistent :class:`CompiledProgram` bound to device buffers (for serving loops)."""
+        from deplodock_amd.backend.hip.program import CompiledProgram
+
+        self._select_device()
+        return CompiledProgram.build(compiled, self.bind(compiled, input_data))
+
+    # -- benchmark --------------------------------------------------------------
+    async def benchmark_async(
+        self,
+        compiled: Graph,
+        *,
+        warmup: int = 5,
+        num_iters=20,
+        on_iter=None,
+        nvcc_flags: str | None = None,
+        capture_graphs: bool = True,
+        input_data: dict | None = None,
+    ) -> BenchmarkResult:
+        """Event-timed benchmark (backend.py:179-237).  ``nvcc_flags`` keeps the
+        reference's keyword; here it re-points ``EMMY_HIPRTC_FLAGS`` for this one
+        compile."""
+        return self.benchmark(compiled, warmup=warmup, num_iters=num_iters, on_iter=on_iter, hiprtc_flags=nvcc_flags, capture_graphs=capture_graphs, input_data=input_data)
+
+    def benchmark(self, compiled: Graph, *, warmup: int = 5, num_iters=20, on_iter=None, hiprtc_flags: str | None = None, capture_graphs: bool = True, input_data: dict | None = None) -> BenchmarkResult:
+        from deplodock_amd.backend.hip.program import benchmark_program
+
+        self._select_device()
+        with config.hiprtc_flags_override(hiprtc_flags):
+            return benchmark_program(
+                compiled,
+                input_data=self.bind(compiled, input_data),
+                warmup=warmup,
+                num_iters=num_iters,
+                on_iter=on_iter,
+                compile_timeout_s=self.bench_compile_timeout_s,
+                run_timeout_s=self.bench_run_timeout_s,
+                capture_graphs=capture_graphs,
+            )
+
+    def _select_device(self) -> None:
+        if self.device_id is not None:
+            import torch
+
+            torch.cuda.set_device(self.device_id)

@@ -1,0 +1,448 @@
+"""MFMA contraction emitter: ``out[m, n] = epilogue(sum_k a[m, k] * b[n, k])``.
+
+Replaces the reference's warp-MMA contraction (``_MmaOps``, ``_contract_kloop``
+and ``_staged`` in emmy/compiler/pipeline/passes/lowering/kernel/_atom.py:397-715,
+the cp.async ring of _stage.py:400-450, ``LdmatrixLoad`` / ``MmaSyncPtx`` /
+``RegStore`` in emmy/compiler/ir/kernel/ir.py:1076-1529).  The design is for
+CDNA4, not a translation:
+
+* **Operand roles are swapped** relative to the math: the weight tile (rows =
+  output features ``n``) feeds the MFMA *A* port and the activation tile (rows
+  = ``m``) the *B* port, so the fp32 accumulator fragment holds, per lane, four
+  *consecutive n* of one output row ``m``.  The epilogue therefore packs and
+  stores 8-byte bf16x4 runs straight from registers — no shared-memory
+  transpose, no 2-byte scatter.
+* Both operands are K-contiguous in memory, which is exactly what an MFMA lane
+  wants (8 consecutive k of one row = one 16-byte chunk), so LDS holds plain
+  row-major slabs and fragments are single ``ds_read_b128``.
+* LDS slabs are XOR-swizzled at 16-byte granularity so the 16 rows a quarter
+  wave reads of one k-chunk land in 16 distinct 16-byte bank groups (64 banks).
+* ``STAGE=d<n>/sync`` software-pipelines global → VGPR → LDS one slab ahead
+  with one barrier per slab; ``STAGE=d<n>/dl`` issues global loads that write
+  LDS directly (no VGPR hop), ``n - 1`` slabs ahead.
+* Workgroup ids are remapped so the 8 XCDs (hardware round-robins consecutive
+  ids over them) each own a compact block of output tiles and keep their
+  operand rows in their own L2.
+"""
+
+from __future__ import annotations
+
+from deplodock_amd.context import Context
+from deplodock_amd.dtype import BF16, F16, F32
+from deplodock_amd.emit import prelude
+from deplodock_amd.emit.errors import LoweringError
+from deplodock_amd.ir import expr as E
+from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.schedule import Stage
+from deplodock_amd.ir.tile import Contraction
+
+_FRAG_T = {"bf16": "bf16x8", "f16": "f16x8"}
+_PACK4_T = {"bf16": "bf16x4", "f16": "f16x4", "f32": "f32x4"}
+
+
+def xcd_block(tiles_m: int, tiles_n: int, tile_m: int, tile_n: int, xcds: int) -> tuple[int, int]:
+    """Shape ``(gm, gn)`` of the tile block one XCD owns: ``gm*gn`` as close to
+    ``tiles/xcds`` as the grid allows, minimising operand rows touched
+    (``gm*tile_m + gn*tile_n``) so the block's working set fits its L2."""
+    per = max(1, (tiles_m * tiles_n) // xcds)
+    best = None
+    for gm in range(1, tiles_m + 1):
+        if tiles_m % gm:
+            continue
+        gn = max(1, min(tiles_n, per // gm))
+        while gn > 1 and tiles_n % gn:
+            gn -= 1
+        if gm * gn > per and not (gm == 1 and gn == 1):
+            continue
+        cost = (gm * tile_m + gn * tile_n, -(gm * gn))
+        if best is None or (-(gm * gn), cost[0]) < (-(best[0] * best[1]), best[2]):
+            best = (gm, gn, cost[0])
+    return (best[0], best[1]) if best else (1, 1)
+
+
+def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> HipOp:
+    plan = body.tile
+    if plan is None:
+        raise LoweringError("contraction: no TilePlan stamped")
+    if body.in_dtype.name not in _FRAG_T or plan.atom.dtype != body.in_dtype.name:
+        raise LoweringError(f"contraction: atom {plan.atom.name} does not take {body.in_dtype} operands")
+    stage = body.stage or Stage(depth=2, transport="sync")
+    if body.reduce.cta != 1:
+        raise LoweringError("contraction: split-K is lowered by emit_contraction_splitk")
+    M, N, K = body.m, body.n, body.k
+    lda = body.lda or K
+    ldb = body.ldb or K
+    ldo = body.ldo or N
+    AM = plan.atom.m  # 32 or 16 (square atoms)
+    KG = 64 // AM  # lane groups along k
+    KSTEP = plan.atom.k  # k per MFMA
+    ACC = plan.atom.acc_per_lane
+    WM, WN = plan.units
+    FM, FN = plan.regs
+    TM, TN = plan.tile_m, plan.tile_n
+    BK = plan.bk_elems
+    T = plan.block_threads
+    if K % BK:
+        raise LoweringError(f"contraction: K={K} is not a multiple of the slab depth {BK}")
+    if BK % 8 or BK > 128:
+        raise LoweringError(f"contraction: slab depth {BK} must be a multiple of 8 and at most 128")
+    if lda % 8 or ldb % 8 or ldo % 4 or body.a_offset % 8 or body.b_offset % 8 or body.out_offset % 8:
+        raise LoweringError("contraction: leading dimensions must keep 16-byte operand / 8-byte output alignment")
+    CPR = BK // 8  # 16-byte chunks per slab row
+    if CPR & (CPR - 1):
+        raise LoweringError(f"contraction: slab depth {BK} must give a power-of-two chunk count")
+    RPL = max(1, 16 // CPR)  # slab rows per 256-byte bank line
+    gate = body.gate_pair
+    NB = 2 if gate else 1  # weight matrices consumed per pass
+    a_chunks = TM * CPR
+    b_chunks = TN * CPR * NB
+    if a_chunks % T or b_chunks % T:
+        raise LoweringError(f"contraction: tile {TM}x{TN}x{BK} does not divide over {T} threads")
+    A_PER_T, B_PER_T = a_chunks // T, b_chunks // T
+    slab_bytes = (TM + TN * NB) * BK * 2
+    depth = max(2, stage.depth)
+    lds_bytes = slab_bytes * depth
+    if lds_bytes > ctx.lds_bytes_per_cu:
+        raise LoweringError(f"contraction: {lds_bytes} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
+    acc_regs = FM * FN * ACC * NB
+    if acc_regs > 384:
+        raise LoweringError(f"contraction: {acc_regs} accumulator registers per lane exceed the register file")
+    tiles_m, tiles_n = -(-M // TM), -(-N // TN)
+    n_tiles = tiles_m * tiles_n
+    gm, gn = xcd_block(tiles_m, tiles_n, TM, TN, ctx.xcds)
+    KT = K // BK
+    m_guard = M % TM != 0
+    n_guard = N % TN != 0
+    dl = stage.transport == "dl"
+    if dl and (a_chunks % 64 or b_chunks % 64):
+        raise LoweringError("contraction: direct-to-LDS staging needs whole-wave chunk counts")
+
+    frag_t = _FRAG_T[body.in_dtype.name]
+    in_c = body.in_dtype.c_name
+    out_c = body.out_dtype.c_name
+    epi_names = [n for n, _ in body.epilogue_operands]
+    epi = body.epilogue if body.epilogue is not None else E.Var("acc")
+    allowed = {"acc"} | ({"acc2"} if gate else set())
+    unknown = E.variables(epi) - allowed
+    if unknown:
+        raise LoweringError(f"contraction epilogue uses unknown names {sorted(unknown)} (operands belong in `post`)")
+
+    params = [f"const {in_c}* __restrict__ A", f"const {in_c}* __restrict__ B"]
+    params += [f"const {dt.c_name}* __restrict__ e{i}" for i, (_, dt) in enumerate(body.epilogue_operands)]
+    params.append(f"{out_c}* __restrict__ O")
+
+    D = dict(
+        name=name, T=T, M=M, N=N, K=K, LDA=lda, LDB=ldb, LDO=ldo, TM=TM, TN=TN, BK=BK, WM=WM, WN=WN, FM=FM, FN=FN,
+        AM=AM, KG=KG, KSTEP=KSTEP, ACC=ACC, CPR=CPR, RPL=RPL, NB=NB, A_PER_T=A_PER_T, B_PER_T=B_PER_T,
+        SLAB=slab_bytes, DEPTH=depth, KT=KT, TILES_M=tiles_m, TILES_N=tiles_n, NTILES=n_tiles, GM=gm, GN=gn,
+        XCDS=ctx.xcds, frag_t=frag_t, in_c=in_c, out_c=out_c, params=", ".join(params), builtin=plan.atom.builtin,
+        acc_t="f32x16" if ACC == 16 else "f32x4", G=ACC // 4,
+    )  # fmt: skip
+
+    o: list[str] = []
+    a = o.append
+    a(f"// {name}: M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()} xcd-block={gm}x{gn}")
+    for k_, v_ in D.items():
+        if isinstance(v_, int):
+            a(f"#define {k_} {v_}")
+    a(r"""
+EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
+""")
+    a(f'extern "C" __global__ __launch_bounds__({T}) void {name}({D["params"]}) {{')
+    a(r"""  extern __shared__ __attribute__((aligned(16))) unsigned char emh_lds[];
+  // ---- tile ownership: consecutive workgroup ids rotate over the XCDs ----
+  const int bid = blockIdx.x;
+  const int xcd = bid % XCDS;
+  const int slot = bid / XCDS;
+  constexpr int PER_BLOCK = GM * GN;
+  constexpr int BLOCKS_N = TILES_N / GN;
+  constexpr int NBLOCKS = (TILES_M / GM) * BLOCKS_N;
+  int tm, tn;
+  {
+    // XCD x owns tile blocks x, x+XCDS, ...; `slot` walks the tiles of those blocks.
+    const int blk = xcd + (slot / PER_BLOCK) * XCDS;
+    const int in_blk = slot % PER_BLOCK;
+    if (blk < NBLOCKS) {
+      tm = (blk / BLOCKS_N) * GM + in_blk / GN;
+      tn = (blk % BLOCKS_N) * GN + in_blk % GN;
+    } else {
+      return;  // padding workgroup of a launch rounded up to whole XCD rounds
+    }
+  }
+  const int m0 = tm * TM, n0 = tn * TN;
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int wm = wave / WN, wn = wave % WN;
+  const int lr = lane % AM, lk = lane / AM;  // fragment row, k-group
+""")
+    # ---- staging ------------------------------------------------------------
+    a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];")
+    a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
+    a(r"""  #pragma unroll
+  for (int i = 0; i < A_PER_T; ++i) {
+    const int q = tid + i * T;""")
+    if dl:
+        a("    const int row = q / CPR, c = emh_swz(row, q % CPR);  // lane order fixes the LDS slot; pick the chunk that belongs there")
+        a("    la[i] = q * 16;")
+    else:
+        a("    const int row = q / CPR, c = q % CPR;")
+        a("    la[i] = row * (BK * 2) + emh_swz(row, c) * 16;")
+    a(f"    int gr = m0 + row;{' if (gr > M - 1) gr = M - 1;' if m_guard else ''}")
+    a(f"    ga[i] = A + {body.a_offset}L + (long)gr * LDA + c * 8;")
+    a("  }")
+    a(r"""  #pragma unroll
+  for (int i = 0; i < B_PER_T; ++i) {
+    const int q = tid + i * T;""")
+    if dl:
+        a("    const int row = q / CPR, c = emh_swz(row, q % CPR);")
+        a("    lb[i] = TM * BK * 2 + q * 16;")
+    else:
+        a("    const int row = q / CPR, c = q % CPR;")
+        a("    lb[i] = TM * BK * 2 + row * (BK * 2) + emh_swz(row, c) * 16;")
+    if gate:
+        a("    int gr = (row < TN) ? (n0 + row) : (N + n0 + row - TN);  // second half of the slab: the paired matrix")
+        if n_guard:
+            a("    { const int lim = (row < TN) ? (N - 1) : (2 * N - 1); if (gr > lim) gr = lim; }")
+    else:
+        a(f"    int gr = n0 + row;{' if (gr > N - 1) gr = N - 1;' if n_guard else ''}")
+    a(f"    gb[i] = B + {body.b_offset}L + (long)gr * LDB + c * 8;")
+    a("  }")
+
+    a(f"  {D['acc_t']} acc[NB][FM][FN];")
+    a(r"""  #pragma unroll
+  for (int h = 0; h < NB; ++h)
+  #pragma unroll
+  for (int i = 0; i < FM; ++i)
+  #pragma unroll
+  for (int j = 0; j < FN; ++j)
+  #pragma unroll
+  for (int r = 0; r < ACC; ++r) acc[h][i][j][r] = 0.0f;
+""")
+    frag_decl = f"  {frag_t} fw[2][NB][FN], fx[2][FM];"
+    a(frag_decl)
+    a(r"""  // Fragments are double-buffered in registers: the reads for step s+1 are
+  // issued before the MFMAs of step s and complete in their shadow.  The
+  // sched_barriers pin that order (the scheduler otherwise sinks the reads to
+  // just before their use).
+  #define EMH_READ(P, buf, kk) { \
+    const unsigned char* sA_ = emh_lds + (buf) * SLAB; \
+    const unsigned char* sB_ = sA_ + TM * BK * 2; \
+    const int c_ = (kk) * KG + lk; \
+    _Pragma("unroll") for (int h = 0; h < NB; ++h) \
+    _Pragma("unroll") for (int j = 0; j < FN; ++j) { \
+      const int row_ = h * TN + (wn * FN + j) * AM + lr; \
+      fw[P][h][j] = *(const FRAG_T*)(sB_ + row_ * (BK * 2) + emh_swz(row_, c_) * 16); } \
+    _Pragma("unroll") for (int i = 0; i < FM; ++i) { \
+      const int row_ = (wm * FM + i) * AM + lr; \
+      fx[P][i] = *(const FRAG_T*)(sA_ + row_ * (BK * 2) + emh_swz(row_, c_) * 16); } \
+    __builtin_amdgcn_sched_barrier(0); }
+  #define EMH_MMA(P) { \
+    _Pragma("unroll") for (int h = 0; h < NB; ++h) \
+    _Pragma("unroll") for (int i = 0; i < FM; ++i) \
+    _Pragma("unroll") for (int j = 0; j < FN; ++j) \
+      acc[h][i][j] = BUILTIN(fw[P][h][j], fx[P][i], acc[h][i][j], 0, 0, 0); \
+    __builtin_amdgcn_sched_barrier(0); }
+""".replace("FRAG_T", frag_t).replace("BUILTIN", plan.atom.builtin))
+    KS = BK // KSTEP
+    if not dl:
+        # global -> VGPR -> LDS, one slab ahead, one barrier per slab.
+        a(r"""  u32x4 ra[A_PER_T], rb[B_PER_T];
+  #define EMH_GLOAD(kt) { \
+    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) ra[i] = *(const u32x4*)(ga[i] + (kt) * BK); \
+    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[i] = *(const u32x4*)(gb[i] + (kt) * BK); }
+  #define EMH_LSTORE(buf) { \
+    unsigned char* s_ = emh_lds + (buf) * SLAB; \
+    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) *(u32x4*)(s_ + la[i]) = ra[i]; \
+    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[i]; }
+  EMH_GLOAD(0);
+  EMH_LSTORE(0);
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const int cur = kt % DEPTH;
+    if (kt + 1 < KT) EMH_GLOAD(kt + 1);
+    EMH_READ(0, cur, 0);""")
+        for kk in range(KS):
+            if kk + 1 < KS:
+                a(f"    EMH_READ({(kk + 1) & 1}, cur, {kk + 1});")
+            a(f"    EMH_MMA({kk & 1});")
+        a(r"""    if (kt + 1 < KT) EMH_LSTORE((kt + 1) % DEPTH);
+    __syncthreads();
+  }""")
+    else:
+        if KS % 2:
+            raise LoweringError(f"contraction: direct-to-LDS pipeline needs an even number of MFMA steps per slab (BK={BK}, step={KSTEP})")
+        loads_per_slab = A_PER_T + B_PER_T
+        if (depth - 1) * loads_per_slab > 63:
+            raise LoweringError("contraction: too many loads in flight for the 6-bit vmcnt counter; lower STAGE depth")
+        a(r"""  // Each wave-level direct-to-LDS load fills 64 consecutive 16-byte LDS slots
+  // (slot = lane); the per-lane *global* address selects which chunk lands there.
+  #define EMH_DLOAD(kt, buf) { \
+    unsigned char* s_ = emh_lds + (buf) * SLAB; \
+    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) \
+      __builtin_amdgcn_global_load_lds((const void*)(ga[i] + (kt) * BK), (__attribute__((address_space(3))) void*)(s_ + la[i] - lane * 16), 16, 0, 0); \
+    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) \
+      __builtin_amdgcn_global_load_lds((const void*)(gb[i] + (kt) * BK), (__attribute__((address_space(3))) void*)(s_ + lb[i] - lane * 16), 16, 0, 0); }
+  // A plain s_barrier is used on purpose: a workgroup fence would drain every
+  // outstanding direct-to-LDS load and serialise the pipeline.  Loads retire in
+  // issue order, so "at most n outstanding" means the older slabs have landed.
+  #define EMH_SLAB_SYNC(n) { \
+    __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM_LGKM0(n)); \
+    asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
+  #pragma unroll
+  for (int p = 0; p < DEPTH; ++p) if (p < KT) EMH_DLOAD(p, p);""")
+        first_younger = min(depth - 1, KT - 1) * loads_per_slab
+        a(f"  EMH_SLAB_SYNC({first_younger});")
+        a("  EMH_READ(0, 0, 0);")
+
+        def slab_steps(kt: str, static_kt: int | None) -> None:
+            """MFMA steps of slab ``kt``.  With ``static_kt`` the hand-over to the
+            next slab is resolved at emit time (tail); otherwise it is the
+            steady state, where every condition holds and the body is branch-free
+            (so the wait-count pass can see that only the newest reads are pending)."""
+            a(f"    {{ const int cur = ({kt}) % DEPTH;")
+            for kk in range(KS):
+                P = kk & 1
+                if kk + 1 < KS:
+                    a(f"    EMH_READ({P ^ 1}, cur, {kk + 1});")
+                elif static_kt is None:
+                    a(f"    EMH_SLAB_SYNC({(depth - 2) * loads_per_slab});")
+                    a(f"    EMH_DLOAD(({kt}) + DEPTH, cur);")
+                    a(f"    EMH_READ({P ^ 1}, (({kt}) + 1) % DEPTH, 0);")
+                elif static_kt + 1 < KT:
+                    younger = min(KT - static_kt - 2, depth - 2)
+                    a(f"    EMH_SLAB_SYNC({younger * loads_per_slab});")
+                    if static_kt + depth < KT:
+                        a(f"    EMH_DLOAD({static_kt + depth}, cur);")
+                    a(f"    EMH_READ({P ^ 1}, {(static_kt + 1) % depth}, 0);")
+                a(f"    EMH_MMA({P});")
+            a("    }")
+
+        steady = max(0, KT - depth)
+        if steady:
+            a(f"  for (int kt = 0; kt < {steady}; ++kt) {{")
+            slab_steps("kt", None)
+            a("  }")
+        for kt_s in range(steady, KT):
+            slab_steps(str(kt_s), kt_s)
+
+    # ---- epilogue ------------------------------------------------------------------
+    esz = body.out_dtype.nbytes
+    EPC = 16 // esz  # output elements per 16-byte chunk
+    c_stride = TN * esz + 16
+    staged = (N % EPC == 0) and (TN % EPC == 0) and (TM * c_stride <= ctx.lds_bytes_per_cu) and ((TM * (TN // EPC)) % T == 0)
+    vt4 = _PACK4_T[body.out_dtype.name]
+    cast = "" if body.out_dtype is F32 else f"({out_c})"
+    post = body.post if body.post is not None else E.Var("y")
+    unknown = E.variables(post) - ({"y"} | set(epi_names))
+    if unknown:
+        raise LoweringError(f"contraction post-epilogue uses unknown names {sorted(unknown)}")
+    a(r"""  // Accumulator lane layout: column (l % AM) is the output row m; the registers
+  // of group g hold four consecutive n starting at g*4*KG + (l / AM)*4.""")
+    if staged:
+        lds_bytes = max(lds_bytes, TM * c_stride)
+        a(f"  constexpr int CSTRIDE = {c_stride};")
+        a("  __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM_LGKM0(0));" if dl else "")
+        a("  __syncthreads();  // every wave is done with the operand slabs; reuse them for the output tile")
+        a(r"""  #pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int ml = (wm * FM + i) * AM + lr;
+    #pragma unroll
+    for (int j = 0; j < FN; ++j)
+    #pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int nl = (wn * FN + j) * AM + g * 4 * KG + lk * 4;""")
+        a(f"      {vt4} yo;")
+        for r in range(4):
+            env = {"acc": f"acc[0][i][j][g * 4 + {r}]"}
+            if gate:
+                env["acc2"] = f"acc[1][i][j][g * 4 + {r}]"
+            a(f"      yo[{r}] = {cast}({E.render(epi, env)});")
+        a(f"      *({vt4}*)(emh_lds + ml * CSTRIDE + nl * {esz}) = yo;")
+        a("    }")
+        a("  }")
+        a("  __syncthreads();")
+        vt_chunk = {("bf16"): "bf16x8", "f16": "f16x8", "f32": "f32x4"}[body.out_dtype.name]
+        a(f"  constexpr int CPRC = TN / {EPC};  // 16-byte chunks per output-tile row")
+        a(r"""  #pragma unroll
+  for (int it = 0; it < (TM * CPRC) / T; ++it) {
+    const int q = tid + it * T;
+    const int row = q / CPRC, cc = q % CPRC;""")
+        a(f"    const int m = m0 + row, n = n0 + cc * {EPC};")
+        conds = []
+        if m_guard:
+            conds.append("m < M")
+        if n_guard:
+            conds.append("n < N")
+        a(f"    if ({' && '.join(conds) if conds else 'true'}) {{")
+        a(f"      {vt_chunk} v = *(const {vt_chunk}*)(emh_lds + row * CSTRIDE + cc * 16);")
+        if body.post is not None:
+            for i, (_, dt) in enumerate(body.epilogue_operands):
+                if dt.nbytes != esz:
+                    raise LoweringError("contraction: post-epilogue operands must have the output dtype")
+                a(f"      const {vt_chunk} ev{i} = *(const {vt_chunk}*)(e{i} + (long)m * LDO + n);")
+            for r in range(EPC):
+                env = {"y": f"(float)v[{r}]"}
+                for i, (n_, _) in enumerate(body.epilogue_operands):
+                    env[n_] = f"(float)ev{i}[{r}]"
+                a(f"      v[{r}] = {cast}({E.render(post, env)});")
+        a(f"      *({vt_chunk}*)(O + {body.out_offset}L + (long)m * LDO + n) = v;")
+        a("    }")
+        a("  }")
+    else:
+        a(r"""  #pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int m = m0 + (wm * FM + i) * AM + lr;""")
+        if m_guard:
+            a("    if (m >= M) continue;")
+        a(r"""    #pragma unroll
+    for (int j = 0; j < FN; ++j)
+    #pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int n = n0 + (wn * FN + j) * AM + g * 4 * KG + lk * 4;""")
+        if n_guard:
+            a("      if (n >= N) continue;  // N and tile widths are multiples of 4: a run is all in or all out")
+        for i, (_, dt) in enumerate(body.epilogue_operands):
+            vt = _PACK4_T[dt.name]
+            a(f"      const {vt} ev{i} = *(const {vt}*)(e{i} + (long)m * LDO + n);")
+        a(f"      {vt4} yo;")
+        for r in range(4):
+            env = {"acc": f"acc[0][i][j][g * 4 + {r}]"}
+            if gate:
+                env["acc2"] = f"acc[1][i][j][g * 4 + {r}]"
+            pre = E.render(epi, env)
+            if body.post is not None:
+                env2 = {"y": f"(float){cast}({pre})"}
+                for i, (n_, _) in enumerate(body.epilogue_operands):
+                    env2[n_] = f"(float)ev{i}[{r}]"
+                pre = E.render(post, env2)
+            a(f"      yo[{r}] = {cast}({pre});")
+        a(f"      *({vt4}*)(O + {body.out_offset}L + (long)m * LDO + n) = yo;")
+        a("    }")
+        a("  }")
+    a("}")
+
+    vm_macro = r"""
+// s_waitcnt immediate: vmcnt <= n and lgkmcnt == 0 (gfx9 encoding: vmcnt[3:0] in
+// bits 3:0, vmcnt[5:4] in bits 15:14; expcnt left at its maximum, lgkmcnt = 0).
+#define EMH_WAIT_VM_LGKM0(n) ((((n) & 0xF) | ((((n) >> 4) & 0x3) << 14)) | 0x0070)
+"""
+    source = prelude.header(vm_macro) + "\n".join(o) + "\n"
+    if N % 4 or TN % 4:
+        raise LoweringError("contraction: N must be a multiple of 4 (8-byte output runs)")
+    n_blocks = (tiles_m // gm) * (tiles_n // gn)
+    rounds = -(-n_blocks // ctx.xcds)
+    grid = rounds * ctx.xcds * gm * gn
+    return HipOp(
+        kernel_source=source,
+        kernel_name=name,
+        arg_order=(body.a, body.b, *(body.operand_buffers.get(n, n) for n in epi_names), body.out),
+        grid=((grid,), (1,), (1,)),
+        block=((T,), (1,), (1,)),
+        lds_bytes=lds_bytes,
+        comment=f"contraction M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()}",
+        algo_bytes=body.algo_bytes(),
+        algo_flops=body.algo_flops(),
+        knobs={"TILE": plan.spell(), "STAGE": stage.spell()},
+    )
+
+
+__all__ = ["emit_contraction", "xcd_block", "BF16", "F16"]

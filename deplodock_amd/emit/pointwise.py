@@ -1,0 +1,64 @@
+"""Pointwise map emitter: ``out[i] = expr(operands[i])`` over a flat index space.
+
+The per-cell ``Tile`` of the reference (one thread per output cell,
+emmy/compiler/ir/kernel/ir.py:159-297; degenerate arm of ``_bind``,
+passes/lowering/kernel/_factor.py:329-398) with 16-byte vector accesses and a
+grid sized to the index space.
+"""
+
+from __future__ import annotations
+
+from deplodock_amd.context import Context
+from deplodock_amd.emit import prelude
+from deplodock_amd.emit.errors import LoweringError
+from deplodock_amd.emit.reduce import _load_vec, _store_vec
+from deplodock_amd.ir import expr as E
+from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.tile import Map
+
+_T = 256
+
+
+def emit_map(body: Map, name: str, ctx: Context = Context()) -> HipOp:
+    names = [o.name for o in body.operands]
+    unknown = E.variables(body.expr) - set(names)
+    if unknown:
+        raise LoweringError(f"map expression uses unknown names {sorted(unknown)}")
+    dts = [body.out_dtype, *(o.dtype for o in body.operands)]
+    V = 16 // max(d.nbytes for d in dts)
+    offs = [body.operand_offsets.get(o.name, 0) for o in body.operands]
+    while V > 1 and (body.numel % V or body.inner % V or any(off % V for off in offs)):
+        V //= 2
+    chunks = body.numel // V
+    grid = max(1, -(-chunks // _T))
+    params = [f"const {o.dtype.c_name}* __restrict__ p{i}" for i, o in enumerate(body.operands)]
+    params.append(f"{body.out_dtype.c_name}* __restrict__ out")
+    o: list[str] = []
+    a = o.append
+    a(f"// {name}: numel={body.numel} vec={V}")
+    a(f'extern "C" __global__ __launch_bounds__({_T}) void {name}({", ".join(params)}) {{')
+    a(f"  const long c = (long)blockIdx.x * {_T} + threadIdx.x;")
+    a(f"  if (c >= {chunks}L) return;")
+    for i, op in enumerate(body.operands):
+        a(f"  float v{i}[{V}];")
+        if op.index == "flat":
+            o.extend("  " + ln for ln in _load_vec(f"p{i} + {offs[i]}L", "c", op.dtype, V, f"v{i}", False))
+        elif op.index == "col":
+            o.extend("  " + ln for ln in _load_vec(f"p{i} + {offs[i]}L", f"(c % {body.inner // V}L)", op.dtype, V, f"v{i}", False))
+        else:
+            raise LoweringError(f"map operand index scheme {op.index!r} is not supported")
+    a(f"  float y[{V}];")
+    for j in range(V):
+        env = {op.name: f"v{i}[{j}]" for i, op in enumerate(body.operands)}
+        a(f"  y[{j}] = {E.render(body.expr, env)};")
+    o.extend("  " + ln for ln in _store_vec("out", "c", body.out_dtype, V, "y", False))
+    a("}")
+    return HipOp(
+        kernel_source=prelude.header() + "\n".join(o) + "\n",
+        kernel_name=name,
+        arg_order=(*(body.operand_buffers.get(n, n) for n in names), body.out),
+        grid=((grid,), (1,), (1,)),
+        block=((_T,), (1,), (1,)),
+        comment=f"map numel={body.numel}",
+        algo_bytes=body.algo_bytes(),
+    )

@@ -26,7 +26,7 @@ from deplodock_amd.emit import prelude
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
-from deplodock_amd.ir.tile import RowReduce
+from deplodock_amd.ir.tile import RowAddr, RowReduce
 
 _MAX_RESIDENT = 64  # fp32 row elements a lane may keep in registers
 
@@ -45,13 +45,21 @@ _VEC_T = {
 }
 
 
-def pick_vec(cols: int, dtypes: list[DType], strides: list[int]) -> int:
+def pick_vec(cols: int, dtypes: list[DType], addrs: list[RowAddr]) -> int:
     """Widest element count per access such that the widest dtype moves 16 bytes
     and every row start stays aligned."""
     v = 16 // max(d.nbytes for d in dtypes)
-    while v > 1 and (cols % v or any(s % v for s in strides)):
+    while v > 1 and cols % v:
         v //= 2
+    for a in addrs:
+        v = a.max_vec(v)
     return v
+
+
+def _row_offset(addr: RowAddr, row: str) -> str:
+    if addr.div == 1:
+        return f"{addr.offset}L + {row} * {addr.stride_hi}L"
+    return f"{addr.offset}L + ({row} / {addr.div}) * {addr.stride_hi}L + ({row} % {addr.div}) * {addr.stride_lo}L"
 
 
 def _load_vec(ptr: str, idx: str, dt: DType, v: int, dst: str, nontemporal: bool) -> list[str]:
@@ -86,17 +94,27 @@ def _store_vec(ptr: str, idx: str, dt: DType, v: int, src: str, nontemporal: boo
     return lines
 
 
-def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context(), *, nontemporal: bool = False) -> HipOp:
+def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> HipOp:
     """Render ``body`` (schedule already stamped on ``body.reduce``) to a HipOp."""
     plan = body.reduce
     L = plan.coop
+    nontemporal = body.nontemporal
     if plan.cta != 1:
         raise LoweringError("row reduce: cross-workgroup split (g<n>) is not defined for a projected row")
-    stride_in = body.row_stride_in if body.row_stride_in is not None else body.cols
-    stride_out = body.row_stride_out if body.row_stride_out is not None else body.cols
+    x_addr = body.x_addr or RowAddr.uniform(body.cols)
+    out_addr = body.out_addr or RowAddr.uniform(body.cols)
     col_dts = [dt for _, dt in body.col_operands]
-    V = pick_vec(body.cols, [body.x_dtype, body.out_dtype, *col_dts], [stride_in, stride_out])
+    row_dts = [ro.dtype for ro in body.row_operands]
+    V = pick_vec(body.cols, [body.x_dtype, body.out_dtype, *col_dts, *row_dts], [x_addr, out_addr])
+    for ro in body.row_operands:
+        while V > 1 and ro.offset % V:
+            V //= 2
     C = body.cols // V  # vector chunks per row
+    if body.rotate is not None:
+        if C % 2:
+            raise LoweringError("row reduce: rotate-half needs an even number of vector chunks per row")
+        if (C // 2) % L:
+            raise LoweringError(f"row reduce: rotate-half keeps both halves in one lane, which needs REDUCE b<n> with n dividing {C // 2}")
     NV = -(-C // L)  # chunks per lane
     if NV * V > _MAX_RESIDENT:
         raise LoweringError(
@@ -120,17 +138,22 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context(), *, non
     W = min(L, ctx.wave_size)  # butterfly width
 
     stat_names = [s.name for s in body.stats]
-    known = {"x", *stat_names, *(n for n, _ in body.col_operands)}
+    operand_names = [n for n, _ in body.col_operands] + [ro.name for ro in body.row_operands]
     for s_i, st in enumerate(body.stats):
         unknown = E.variables(st.pre) - ({"x"} | set(stat_names[:s_i]))
         if unknown:
             raise LoweringError(f"stat {st.name!r}: pre-map uses unknown names {sorted(unknown)}")
-    unknown = E.variables(body.project) - known
+    unknown = E.variables(body.project) - ({"x"} | set(stat_names) | set(operand_names))
     if unknown:
         raise LoweringError(f"projection uses unknown names {sorted(unknown)}")
+    if body.rotate is not None:
+        unknown = E.variables(body.rotate.expr) - ({"y", "yr"} | set(stat_names) | set(operand_names))
+        if unknown:
+            raise LoweringError(f"rotate-half expression uses unknown names {sorted(unknown)}")
 
     params = [f"const {body.x_dtype.c_name}* __restrict__ x"]
     params += [f"const {dt.c_name}* __restrict__ c{ci}" for ci, (_, dt) in enumerate(body.col_operands)]
+    params += [f"const {ro.dtype.c_name}* __restrict__ r{ri}" for ri, ro in enumerate(body.row_operands)]
     params.append(f"{body.out_dtype.c_name}* __restrict__ out")
 
     o: list[str] = []
@@ -143,7 +166,7 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context(), *, non
     if row_guard:
         a(f"  const bool row_ok = row < {body.rows}L;")
         a(f"  if (!row_ok) row = {body.rows - 1}L;")
-    a(f"  const {body.x_dtype.c_name}* xr = x + row * {stride_in}L;")
+    a(f"  const {body.x_dtype.c_name}* xr = x + ({_row_offset(x_addr, 'row')});")
     a(f"  float xv[{NV}][{V}];")
     if masked:
         a(f"  bool ok[{NV}];")
@@ -161,7 +184,7 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context(), *, non
                 a(f"  ok[{i}] = true;")
             o.extend("  " + ln for ln in _load_vec("xr", idx, body.x_dtype, V, f"xv[{i}]", nontemporal))
 
-    if NW > 1:
+    if NW > 1 and body.stats:
         a(f"  __shared__ float emh_part[{len(body.stats)}][{R}][{NW}];")
         a(f"  const int wave_in_row = lane / {ctx.wave_size};")
 
@@ -196,23 +219,68 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context(), *, non
             for w in range(1, NW):
                 a(f"  s_{st.name} = {mono}::op(s_{st.name}, emh_part[{s_i}][rib][{w}]);")
 
-    a(f"  {body.out_dtype.c_name}* orow = out + row * {stride_out}L;")
+    a(f"  {body.out_dtype.c_name}* orow = out + ({_row_offset(out_addr, 'row')});")
+    for ri, ro in enumerate(body.row_operands):
+        a(f"  const {ro.dtype.c_name}* rrow{ri} = r{ri} + {ro.offset}L + ((row / {ro.div}) % {ro.mod}) * {body.cols}L;")
+
+    def operand_loads(i: int, indent: str) -> None:
+        idx = f"{i * L} + lane"
+        for ci, (_, dt) in enumerate(body.col_operands):
+            a(f"{indent}float cv{ci}[{V}];")
+            o.extend(indent + ln for ln in _load_vec(f"c{ci}", idx, dt, V, f"cv{ci}", False))
+        for ri, ro in enumerate(body.row_operands):
+            a(f"{indent}float rv{ri}[{V}];")
+            o.extend(indent + ln for ln in _load_vec(f"rrow{ri}", idx, ro.dtype, V, f"rv{ri}", False))
+
+    def operand_env(j: int) -> dict[str, str]:
+        env = {n: f"cv{ci}[{j}]" for ci, (n, _) in enumerate(body.col_operands)}
+        env.update({ro.name: f"rv{ri}[{j}]" for ri, ro in enumerate(body.row_operands)})
+        return env
+
     if row_guard:
         a("  if (row_ok) {")
-    for i in range(NV):
-        idx = f"{i * L} + lane"
-        guard = f"if (ok[{i}]) " if masked and (i + 1) * L > C else ""
-        a(f"  {guard}{{")
-        a(f"    float y[{V}];")
-        for ci, (_, dt) in enumerate(body.col_operands):
-            a(f"    float cv{ci}[{V}];")
-            o.extend("    " + ln for ln in _load_vec(f"c{ci}", idx, dt, V, f"cv{ci}", False))
-        for j in range(V):
-            env = dict(env_base, x=f"xv[{i}][{j}]")
-            env.update({n: f"cv{ci}[{j}]" for ci, (n, _) in enumerate(body.col_operands)})
-            a(f"    y[{j}] = {E.render(body.project, env)};")
-        o.extend("    " + ln for ln in _store_vec("orow", idx, body.out_dtype, V, "y", nontemporal))
-        a("  }")
+    if body.rotate is None:
+        for i in range(NV):
+            idx = f"{i * L} + lane"
+            guard = f"if (ok[{i}]) " if masked and (i + 1) * L > C else ""
+            a(f"  {guard}{{")
+            a(f"    float y[{V}];")
+            operand_loads(i, "    ")
+            for j in range(V):
+                env = dict(env_base, x=f"xv[{i}][{j}]", **operand_env(j))
+                a(f"    y[{j}] = {E.render(body.project, env)};")
+            o.extend("    " + ln for ln in _store_vec("orow", idx, body.out_dtype, V, "y", nontemporal))
+            a("  }")
+    else:
+        # Phase 1: project the whole resident row; phase 2: combine each element
+        # with its half-rotated partner, which lives in the same lane (the lane
+        # count divides half the chunks), NV/2 chunks away.
+        half = NV // 2
+        a(f"  float yv[{NV}][{V}];")
+        for i in range(NV):
+            a("  {")
+            for ci, (_, dt) in enumerate(body.col_operands):
+                a(f"    float cv{ci}[{V}];")
+                o.extend("    " + ln for ln in _load_vec(f"c{ci}", f"{i * L} + lane", dt, V, f"cv{ci}", False))
+            for j in range(V):
+                env = dict(env_base, x=f"xv[{i}][{j}]")
+                env.update({n: f"cv{ci}[{j}]" for ci, (n, _) in enumerate(body.col_operands)})
+                a(f"    yv[{i}][{j}] = {E.render(body.project, env)};")
+            a("  }")
+        for i in range(NV):
+            idx = f"{i * L} + lane"
+            a("  {")
+            a(f"    float y[{V}];")
+            for ri, ro in enumerate(body.row_operands):
+                a(f"    float rv{ri}[{V}];")
+                o.extend("    " + ln for ln in _load_vec(f"rrow{ri}", idx, ro.dtype, V, f"rv{ri}", False))
+            for j in range(V):
+                partner = f"(-yv[{i + half}][{j}])" if i < half else f"yv[{i - half}][{j}]"
+                env = dict(env_base, y=f"yv[{i}][{j}]", yr=partner)
+                env.update({ro.name: f"rv{ri}[{j}]" for ri, ro in enumerate(body.row_operands)})
+                a(f"    y[{j}] = {E.render(body.rotate.expr, env)};")
+            o.extend("    " + ln for ln in _store_vec("orow", idx, body.out_dtype, V, "y", nontemporal))
+            a("  }")
     if row_guard:
         a("  }")
     a("}")
@@ -221,7 +289,12 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context(), *, non
     return HipOp(
         kernel_source=source,
         kernel_name=name,
-        arg_order=(body.x, *(n for n, _ in body.col_operands), body.out),
+        arg_order=(
+            body.x,
+            *(body.operand_buffers.get(n, n) for n, _ in body.col_operands),
+            *(body.operand_buffers.get(ro.name, ro.name) for ro in body.row_operands),
+            body.out,
+        ),
         grid=((grid,), (1,), (1,)),
         block=((T,), (1,), (1,)),
         lds_bytes=0,

@@ -263,8 +263,8 @@ class Stage:
             else:
                 raise ScheduleError(f"STAGE: cannot parse {tok!r} (expect d<depth> / sync|dl / ring / p<reg_depth>)")
         st = cls(**kw)
-        if not 1 <= st.depth <= 4:
-            raise ScheduleError(f"STAGE: depth must be 1..4, got {st.depth}")
+        if not 1 <= st.depth <= 8:
+            raise ScheduleError(f"STAGE: depth must be 1..8, got {st.depth}")
         return st
 
     def spell(self) -> str:

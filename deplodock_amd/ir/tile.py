@@ -30,17 +30,62 @@ class Stat:
     keep: bool = False  # the pre-mapped value replaces the resident element ``x``
 
 
+@dataclass(frozen=True)
+class RowAddr:
+    """Element offset of row ``r``: ``offset + (r // div) * stride_hi + (r % div) * stride_lo``.
+    ``div == 1`` is the plain ``offset + r * stride_hi``; the two-level form walks
+    e.g. the heads of a ``[tokens, heads * head_dim]`` buffer as rows."""
+
+    offset: int = 0
+    div: int = 1
+    stride_hi: int = 0
+    stride_lo: int = 0
+
+    @classmethod
+    def uniform(cls, stride: int, offset: int = 0) -> RowAddr:
+        return cls(offset=offset, div=1, stride_hi=stride, stride_lo=0)
+
+    def max_vec(self, v: int) -> int:
+        """Largest power-of-two vector width <= ``v`` every row start is aligned to."""
+        while v > 1 and (self.offset % v or self.stride_hi % v or (self.div > 1 and self.stride_lo % v)):
+            v //= 2
+        return v
+
+
+@dataclass(frozen=True)
+class RowOperand:
+    """A per-(row-group, column) table such as RoPE ``cos`` / ``sin`` ``[positions, cols]``:
+    row ``r`` reads table row ``(r // div) % mod``."""
+
+    name: str
+    dtype: DType
+    div: int = 1
+    mod: int = 1
+    offset: int = 0
+
+
+@dataclass(frozen=True)
+class RotateHalf:
+    """Second projection phase for rotary embeddings.  With ``y`` the projected
+    row and ``yr`` its signed half-rotation (``-y[c + cols/2]`` for the first
+    half, ``y[c - cols/2]`` for the second; the reference traces it as
+    ``cat(neg(slice_hi), slice_lo)``), the output is ``expr(y, yr, row operands)``."""
+
+    expr: Expr
+
+
 @dataclass
 class RowReduce:
     """``Map(source=Reduction)``: per-row statistics followed by a projection.
 
-    ``x`` is ``[rows, cols]`` with the reduce axis innermost and contiguous and
-    ``row_stride_*`` elements between rows.  ``project`` is evaluated per
+    ``x`` is ``[rows, cols]`` with the reduce axis innermost and contiguous;
+    ``x_addr`` / ``out_addr`` place the rows.  ``project`` is evaluated per
     element over ``x``, the statistics, and the per-column operands
     (``col_operands``: vectors of length ``cols`` such as a norm weight).
     RMSNorm is ``stats=(ss = sum x*x)``, ``project = x * rsqrt(ss/cols + eps) * w``
     (emmy/compiler/ir/frontend/ir.py:309-312); softmax is ``m = max x``,
-    ``d = sum exp(x - m)``, ``project = exp(x - m) / d`` (:354-358)."""
+    ``d = sum exp(x - m)``, ``project = exp(x - m) / d`` (:354-358).  ``stats``
+    may be empty (a pure row-wise map)."""
 
     rows: int
     cols: int
@@ -51,15 +96,22 @@ class RowReduce:
     stats: tuple[Stat, ...]
     project: Expr
     col_operands: tuple[tuple[str, DType], ...] = ()
-    row_stride_in: int | None = None
-    row_stride_out: int | None = None
+    row_operands: tuple[RowOperand, ...] = ()
+    rotate: RotateHalf | None = None
+    x_addr: RowAddr | None = None
+    out_addr: RowAddr | None = None
     reduce: ReducePlan = field(default_factory=ReducePlan)
     rows_per_block: int | None = None  # derived from the plan when None
+    nontemporal: bool = False
+    # expression name -> buffer (graph node id) for col/row operands; identity when absent
+    operand_buffers: dict = field(default_factory=dict)
 
     def algo_bytes(self) -> int:
         b = self.rows * self.cols * (self.x_dtype.nbytes + self.out_dtype.nbytes)
         for _, dt in self.col_operands:
             b += self.cols * dt.nbytes
+        for ro in self.row_operands:
+            b += ro.mod * self.cols * ro.dtype.nbytes
         return b
 
 
@@ -71,7 +123,13 @@ class Contraction:
     ``acc`` and the names in ``epilogue_operands`` (``[m, n]`` tensors such as a
     residual).  With ``gate_pair`` the weight holds two stacked matrices
     ``[2n, k]`` and the epilogue sees ``acc`` (rows ``0..n``) and ``acc2`` (rows
-    ``n..2n``) — the SwiGLU gate/up pair computed in one pass over ``a``."""
+    ``n..2n``) — the SwiGLU gate/up pair computed in one pass over ``a``.
+
+    The element-wise tail has two phases so a fused kernel can reproduce the
+    rounding points of an eager module: ``epilogue`` maps the fp32 accumulator(s)
+    (names ``acc``, ``acc2``) and is rounded to ``out_dtype``; ``post`` then maps
+    that value (name ``y``) together with ``epilogue_operands`` (``[m, n]``
+    tensors of ``out_dtype`` such as a residual) and is rounded again."""
 
     m: int
     n: int
@@ -82,6 +140,7 @@ class Contraction:
     in_dtype: DType
     out_dtype: DType
     epilogue: Expr | None = None
+    post: Expr | None = None
     epilogue_operands: tuple[tuple[str, DType], ...] = ()
     gate_pair: bool = False
     tile: TilePlan | None = None
@@ -90,6 +149,10 @@ class Contraction:
     lda: int | None = None
     ldb: int | None = None
     ldo: int | None = None
+    a_offset: int = 0
+    b_offset: int = 0
+    out_offset: int = 0
+    operand_buffers: dict = field(default_factory=dict)  # epilogue operand name -> buffer id
 
     def algo_flops(self) -> int:
         return 2 * self.m * self.n * self.k * (2 if self.gate_pair else 1)
@@ -128,6 +191,10 @@ class Flash:
     k_strides: tuple[int, int, int]
     v_strides: tuple[int, int, int]
     o_strides: tuple[int, int, int]
+    q_offset: int = 0
+    k_offset: int = 0
+    v_offset: int = 0
+    o_offset: int = 0
     block_q: int = 128
     block_kv: int = 64
     waves: int = 4
@@ -167,6 +234,8 @@ class Map:
     out: str
     out_dtype: DType
     inner: int = 1  # extent of the innermost axis, for "col" broadcasts
+    operand_buffers: dict = field(default_factory=dict)  # operand name -> buffer id
+    operand_offsets: dict = field(default_factory=dict)  # operand name -> element offset
 
     def algo_bytes(self) -> int:
         b = self.numel * self.out_dtype.nbytes

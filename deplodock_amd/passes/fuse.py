@@ -1,0 +1,616 @@
+"""Frontend graph → graph of tile kernels (which ops become one kernel).
+
+Decides the kernel boundaries.  The reference reaches the same boundaries by
+decomposing frontend ops to primitives and re-fusing loops
+(emmy/compiler/pipeline/passes/frontend/decomposition/*, passes/loop/fusion/010_merge_loop_ops.py:48-183,
+recognizers passes/lowering/tile/010_recognize.py, _flash.py:478-571, _softmax.py:35-123);
+here recognizers match the traced ops directly, walking back from each value
+that must exist in memory:
+
+* ``add(residual, linear)``                       → contraction with a residual post-epilogue
+* ``silu(linear(x, Wg)) * linear(x, Wu)``          → one gate/up contraction (weights stacked at bind time)
+* ``linear``                                      → contraction
+* RMSNorm, as one op or as the traced primitive chain
+  ``w * bf16(f32(x) * rsqrt(mean(f32(x)^2) + eps))`` → row reduce
+* rotary embedding ``t*cos + cat(-t_hi, t_lo)*sin`` → fused into the norm that feeds it, or a row map
+* ``softmax``                                     → row reduce with the (max, sum-exp) carrier
+* ``scaled_dot_product_attention``                → flash kernel addressing q/k/v/out through strides
+* anything else element-wise                       → pointwise map
+
+Layout ops never become kernels (``passes.views``).  The over-fusion the
+reference reports for whole-model traces (four mega-kernels holding 97 % of the
+forward, plans/qwen3-embedding-06b-tune-findings.md:42-57) is avoided by
+construction: a reduction never absorbs a following contraction.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+
+from deplodock_amd.dtype import BF16, F16, F32, DType
+from deplodock_amd.graph import Graph, Node, Tensor
+from deplodock_amd.ir import expr as E
+from deplodock_amd.ir import frontend as F
+from deplodock_amd.ir.base import ConstantOp, InputOp
+from deplodock_amd.ir.tile import Contraction, Flash, Map, MapOperand, RotateHalf, RowAddr, RowOperand, RowReduce, Stat, TileOp
+from deplodock_amd.passes.views import LAYOUT_OPS, NotViewable, View, apply_layout, contiguous_strides, resolve_view
+
+
+class FusionError(NotImplementedError):
+    """No kernel recognizer covers a traced op (or its layout needs a copy this build lacks)."""
+
+
+def _round(dtype: DType, e: E.Expr) -> E.Expr:
+    """Round to ``dtype`` storage and widen again (identity for fp32)."""
+    return e if dtype is F32 else E.Round(dtype.name, e)
+
+
+@dataclass
+class StackedConstant:
+    """A constant the runtime assembles at bind time by stacking other constants
+    along dim 0 (the reference folds such layout work into ``ConstantOp.load_ops``,
+    emmy/compiler/ir/base.py:118-160)."""
+
+    parts: tuple[str, ...]
+
+
+@dataclass
+class _Ctx:
+    g: Graph
+    out: Graph
+    done: dict[str, str] = field(default_factory=dict)  # frontend node id -> lowered buffer id
+    names: dict[str, int] = field(default_factory=dict)
+
+    def kname(self, label: str) -> str:
+        """Kernel label; the lowering appends a hash of the rendered body, so
+        identical kernels (e.g. the k and v projections) share one name."""
+        return f"k_{label}"
+
+    def single_use(self, nid: str) -> bool:
+        return len(self.g.consumers(nid)) == 1 and nid not in self.g.outputs
+
+    def producer(self, nid: str) -> Node:
+        return self.g.nodes[nid]
+
+
+def _is(node: Node, cls, **attrs) -> bool:
+    return isinstance(node.op, cls) and all(getattr(node.op, k) == v for k, v in attrs.items())
+
+
+def _peel_layout(g: Graph, nid: str) -> str:
+    """Follow layout ops back to the node that owns the memory."""
+    while isinstance(g.nodes[nid].op, LAYOUT_OPS):
+        nid = g.nodes[nid].inputs[0]
+    return nid
+
+
+# ---------------------------------------------------------------------------
+# Recognizers (each returns True when it emitted a kernel for ``nid``)
+# ---------------------------------------------------------------------------
+
+
+def _need(c: _Ctx, nid: str) -> View:
+    """Make sure the value of frontend node ``nid`` exists in memory; return how
+    to address it.  Honours a producer that stored its result in another memory
+    order than its logical shape (rope, sdpa): the layout chain between that
+    producer and ``nid`` is replayed on top of the stored layout."""
+    g = c.g
+    chain = []
+    cur = nid
+    while isinstance(g.nodes[cur].op, LAYOUT_OPS):
+        chain.append(cur)
+        cur = g.nodes[cur].inputs[0]
+    _materialize(c, cur)
+    base = c.done[cur]
+    hint = c.out.nodes[base].hints.get("logical_view")
+    if hint is not None:
+        shape, strides = hint
+        v = View(base, 0, tuple(shape), tuple(strides), g.nodes[cur].output.dtype)
+    else:
+        shape = tuple(int(d) for d in g.nodes[cur].output.shape)
+        v = View(base, 0, shape, contiguous_strides(shape), g.nodes[cur].output.dtype)
+    for lid in reversed(chain):
+        v = apply_layout(v, g.nodes[lid].op, tuple(int(d) for d in g.nodes[lid].output.shape), lid)
+    return v
+
+
+def _materialize(c: _Ctx, nid: str) -> None:
+    if nid in c.done:
+        return
+    node = c.g.nodes[nid]
+    if isinstance(node.op, (InputOp, ConstantOp)):
+        t = node.output
+        if isinstance(node.op, InputOp):
+            c.out.add_input(nid, t.shape, t.dtype)
+        else:
+            c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
+        c.done[nid] = nid
+        return
+    for rec in (_rec_linear_residual, _rec_gate_up, _rec_linear, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_pointwise):
+        if rec(c, nid):
+            return
+    raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
+
+
+def _emit(c: _Ctx, nid: str, body, label: str, inputs: list[str], shape=None, dtype=None) -> None:
+    node = c.g.nodes[nid]
+    t = Tensor(nid, shape if shape is not None else node.output.shape, dtype or node.output.dtype)
+    c.out.add_node(TileOp(name=c.kname(label), body=body), list(dict.fromkeys(inputs)), t, nid)
+    c.done[nid] = nid
+
+
+def _matrix(view: View, what: str) -> tuple[int, int, int]:
+    """``view`` as a row-major matrix ``[rows, cols]``: returns ``(rows, cols, ld)``."""
+    if view.strides[-1] != 1 and view.shape[-1] != 1:
+        raise FusionError(f"{what}: innermost dimension must be contiguous")
+    lead = view.collapse_leading(1)
+    if lead is None:
+        raise FusionError(f"{what}: leading dimensions do not collapse to one stride")
+    rows, ld = lead
+    return rows, view.shape[-1], (ld if rows > 1 else view.shape[-1])
+
+
+def _linear_parts(c: _Ctx, nid: str):
+    node = c.g.nodes[nid]
+    if node.op.has_bias:
+        raise FusionError("linear with bias is not supported yet")
+    x = _need(c, node.inputs[0])
+    w = _need(c, node.inputs[1])
+    m, k, lda = _matrix(x, "linear input")
+    n, k2, ldb = _matrix(w, "linear weight")
+    if k != k2:
+        raise FusionError("linear: inner dimensions differ")
+    return x, w, m, n, k, lda, ldb
+
+
+def _rec_linear(c: _Ctx, nid: str) -> bool:
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.LinearOp):
+        return False
+    x, w, m, n, k, lda, ldb = _linear_parts(c, nid)
+    body = Contraction(m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset)
+    _emit(c, nid, body, "linear", [x.base, w.base])
+    return True
+
+
+def _rec_linear_residual(c: _Ctx, nid: str) -> bool:
+    node = c.g.nodes[nid]
+    if not (_is(node, F.ElementwiseOp, fn="add") and len(node.inputs) == 2):
+        return False
+    for li, ri in ((0, 1), (1, 0)):
+        lin_id, res_id = node.inputs[li], node.inputs[ri]
+        lin = c.g.nodes[lin_id]
+        if not (isinstance(lin.op, F.LinearOp) and c.single_use(lin_id) and not lin.op.has_bias):
+            continue
+        if c.g.nodes[res_id].output.shape != node.output.shape or c.g.nodes[res_id].output.dtype != node.output.dtype:
+            continue
+        res = _need(c, res_id)
+        if not res.is_contiguous() or res.offset:
+            continue
+        x, w, m, n, k, lda, ldb = _linear_parts(c, lin_id)
+        od = node.output.dtype
+        body = Contraction(
+            m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=od, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset,
+            post=E.Var("y") + E.Var("res"), epilogue_operands=(("res", od),),
+        )  # fmt: skip
+        body.operand_buffers = {"res": res.base}
+        _emit(c, nid, body, "linear_add", [x.base, w.base, res.base])
+        return True
+    return False
+
+
+def _rec_gate_up(c: _Ctx, nid: str) -> bool:
+    node = c.g.nodes[nid]
+    if not (_is(node, F.ElementwiseOp, fn="mul") and len(node.inputs) == 2):
+        return False
+    for si, ui in ((0, 1), (1, 0)):
+        silu = c.g.nodes[node.inputs[si]]
+        up = c.g.nodes[node.inputs[ui]]
+        if not (_is(silu, F.ElementwiseOp, fn="silu") and c.single_use(silu.id) and isinstance(up.op, F.LinearOp) and c.single_use(up.id)):
+            continue
+        gate = c.g.nodes[silu.inputs[0]]
+        if not (isinstance(gate.op, F.LinearOp) and c.single_use(gate.id)) or gate.op.has_bias or up.op.has_bias:
+            continue
+        if gate.inputs[0] != up.inputs[0]:
+            continue
+        wg, wu = c.g.nodes[gate.inputs[1]], c.g.nodes[up.inputs[1]]
+        if not (isinstance(wg.op, ConstantOp) and isinstance(wu.op, ConstantOp)) or wg.output.shape != wu.output.shape:
+            continue
+        x = _need(c, gate.inputs[0])
+        m, k, lda = _matrix(x, "gate/up input")
+        n = int(wg.output.shape[0])
+        stacked = f"{wg.id}__{wu.id}"
+        if stacked not in c.out.nodes:
+            c.out.add_constant(stacked, (2 * n, k), wg.output.dtype)
+            c.out.nodes[stacked].hints["stacked"] = StackedConstant((wg.id, wu.id))
+        od = node.output.dtype
+        epi = _round(od, E.Un("silu", _round(od, E.Var("acc")))) * _round(od, E.Var("acc2"))
+        body = Contraction(m=m, n=n, k=k, a=x.base, b=stacked, out=nid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset, epilogue=epi, gate_pair=True)
+        _emit(c, nid, body, "linear_silu_mul", [x.base, stacked])
+        return True
+    return False
+
+
+@dataclass
+class _RmsMatch:
+    x: str  # frontend node holding the row values (before any f32 cast)
+    weight: str | None
+    eps: float
+    inner: DType  # dtype the normalised value is rounded to before the weight multiply
+    cols: int
+
+
+def _match_rms_chain(c: _Ctx, nid: str) -> _RmsMatch | None:
+    """``w * cast(f32(x) * rsqrt(mean(f32(x)^2, -1, keepdim) + eps))`` as traced from HF-style RMSNorm."""
+    g = c.g
+    node = g.nodes[nid]
+    weight = None
+    cur = node
+    if _is(cur, F.ElementwiseOp, fn="mul") and len(cur.inputs) == 2:
+        a, b = (g.nodes[i] for i in cur.inputs)
+        cand = [(a, b), (b, a)]
+        for wnode, other in cand:
+            if len(wnode.output.shape) == 1 and wnode.output.shape[0] == cur.output.shape[-1] and isinstance(g.nodes[_peel_layout(g, wnode.id)].op, (ConstantOp, InputOp)):
+                weight, cur = wnode.id, other
+                break
+    inner = cur.output.dtype
+    if isinstance(cur.op, F.CastOp):
+        cur = g.nodes[cur.inputs[0]]
+    if not (_is(cur, F.ElementwiseOp, fn="mul") and len(cur.inputs) == 2):
+        return None
+    a, b = (g.nodes[i] for i in cur.inputs)
+    for xs, rs in ((a, b), (b, a)):
+        if not _is(rs, F.ElementwiseOp, fn="rsqrt"):
+            continue
+        add = g.nodes[rs.inputs[0]]
+        if not (_is(add, F.ElementwiseOp, fn="add") and add.op.scalar is not None):
+            continue
+        mean = g.nodes[add.inputs[0]]
+        rank = len(g.nodes[mean.inputs[0]].output.shape) if mean.inputs else 0
+        if not (isinstance(mean.op, F.MeanOp) and mean.op.keepdim and mean.op.axis == rank - 1):
+            continue
+        pw = g.nodes[mean.inputs[0]]
+        if not (_is(pw, F.ElementwiseOp, fn="pow") and pw.op.scalar == 2.0):
+            continue
+        if pw.inputs[0] != xs.id:
+            continue
+        src = xs
+        if isinstance(src.op, F.CastOp):
+            src = g.nodes[src.inputs[0]]
+        return _RmsMatch(x=src.id, weight=weight, eps=float(add.op.scalar), inner=inner, cols=int(node.output.shape[-1]))
+    return None
+
+
+def _rms_body(c: _Ctx, nid: str, m: _RmsMatch, out_dtype: DType):
+    xv = _need(c, m.x)
+    if xv.strides[-1] != 1:
+        raise FusionError("rms_norm: the normalised axis must be contiguous")
+    rows, x_addr = _row_addr(xv)
+    x = E.Var("x")
+    norm = x * E.Un("rsqrt", E.Var("ss") / float(m.cols) + m.eps)
+    col_ops: tuple = ()
+    inputs = [xv.base]
+    if m.weight is not None:
+        wv = _need(c, m.weight)
+        if not wv.is_contiguous() or wv.offset:
+            raise FusionError("rms_norm: weight must be a plain vector")
+        project = E.Var("w") * _round(m.inner, norm)
+        col_ops = (("w", wv.dtype),)
+        inputs.append(wv.base)
+    else:
+        project = norm
+    body = RowReduce(rows=rows, cols=m.cols, x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=out_dtype, stats=(Stat("ss", "sum", x * x),), project=project, col_operands=col_ops, x_addr=x_addr)
+    body.operand_buffers = {"w": inputs[1]} if m.weight is not None else {}
+    return body, inputs, xv
+
+
+def _row_addr(v: View) -> tuple[int, RowAddr]:
+    """Rows of ``v`` (all dims but the last) as a ``RowAddr``; one- or two-level."""
+    lead = v.collapse_leading(1)
+    if lead is not None:
+        rows, stride = lead
+        return rows, RowAddr.uniform(stride if rows > 1 else v.shape[-1], v.offset)
+    dims = [(n, s) for n, s in zip(v.shape[:-1], v.strides[:-1]) if n != 1]
+    # split into (outer run, inner run), each uniformly strided
+    for cut in range(1, len(dims)):
+        hi, lo = dims[:cut], dims[cut:]
+
+        def run(ds):
+            count, stride = ds[-1]
+            for n, s in reversed(ds[:-1]):
+                if s != stride * count:
+                    return None
+                count *= n
+            return count, stride
+
+        rh, rl = run(hi), run(lo)
+        if rh and rl:
+            return rh[0] * rl[0], RowAddr(offset=v.offset, div=rl[0], stride_hi=rh[1], stride_lo=rl[1])
+    raise FusionError("row kernel: rows are not addressable with two strides")
+
+
+def _rec_rms_chain(c: _Ctx, nid: str) -> bool:
+    m = _match_rms_chain(c, nid)
+    if m is None:
+        return False
+    node = c.g.nodes[nid]
+    body, inputs, _ = _rms_body(c, nid, m, node.output.dtype)
+    _emit(c, nid, body, "rms_norm_reduce", inputs)
+    return True
+
+
+def _rec_rms_op(c: _Ctx, nid: str) -> bool:
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.RmsNormOp):
+        return False
+    m = _RmsMatch(x=node.inputs[0], weight=node.inputs[1] if node.op.has_weight else None, eps=node.op.eps, inner=F32, cols=int(node.output.shape[-1]))
+    # nn.RMSNorm computes in the input dtype's fp32 upcast and rounds once at the end.
+    body, inputs, _ = _rms_body(c, nid, m, node.output.dtype)
+    if m.weight is not None:
+        x = E.Var("x")
+        body.project = x * E.Un("rsqrt", E.Var("ss") / float(m.cols) + m.eps) * E.Var("w")
+    _emit(c, nid, body, "rms_norm_reduce", inputs)
+    return True
+
+
+def _rec_softmax(c: _Ctx, nid: str) -> bool:
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.SoftmaxOp):
+        return False
+    if node.op.axis != len(node.output.shape) - 1:
+        raise FusionError("softmax over a non-innermost axis is not supported")
+    xv = _need(c, node.inputs[0])
+    if xv.strides[-1] != 1:
+        raise FusionError("softmax: the reduced axis must be contiguous")
+    rows, x_addr = _row_addr(xv)
+    x = E.Var("x")
+    stats = (Stat("m", "max", x), Stat("d", "sum", E.Un("exp", x - E.Var("m")), keep=True))
+    body = RowReduce(rows=rows, cols=int(node.output.shape[-1]), x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=node.output.dtype, stats=stats, project=x * E.Un("rcp", E.Var("d")), x_addr=x_addr)
+    _emit(c, nid, body, "softmax_reduce", [xv.base])
+    return True
+
+
+def _match_rope(c: _Ctx, nid: str):
+    """``t*cos + cat(neg(t[..., h:]), t[..., :h]) * sin`` → ``(t, cos, sin)`` node ids."""
+    g = c.g
+    node = g.nodes[nid]
+    if not (_is(node, F.ElementwiseOp, fn="add") and len(node.inputs) == 2):
+        return None
+    for ai, bi in ((0, 1), (1, 0)):
+        ma, mb = g.nodes[node.inputs[ai]], g.nodes[node.inputs[bi]]
+        if not (_is(ma, F.ElementwiseOp, fn="mul") and _is(mb, F.ElementwiseOp, fn="mul") and len(ma.inputs) == 2 and len(mb.inputs) == 2):
+            continue
+        for ci, si in ((0, 1), (1, 0)):
+            cat = g.nodes[mb.inputs[ci]]
+            sin = mb.inputs[si]
+            if not (isinstance(cat.op, F.CatOp) and len(cat.inputs) == 2 and cat.op.dim == len(cat.output.shape) - 1):
+                continue
+            neg, lo = g.nodes[cat.inputs[0]], g.nodes[cat.inputs[1]]
+            if not (_is(neg, F.ElementwiseOp, fn="neg") and isinstance(lo.op, F.SliceOp)):
+                continue
+            hi = g.nodes[neg.inputs[0]]
+            if not isinstance(hi.op, F.SliceOp):
+                continue
+            t = lo.inputs[0]
+            d = int(g.nodes[t].output.shape[-1])
+            last = len(g.nodes[t].output.shape) - 1
+            if hi.inputs[0] != t or lo.op.dim != last or hi.op.dim != last:
+                continue
+            if (lo.op.start, lo.op.end, hi.op.start, hi.op.end) != (0, d // 2, d // 2, d):
+                continue
+            for ti, co in ((0, 1), (1, 0)):
+                if ma.inputs[ti] == t:
+                    return t, ma.inputs[co], sin
+    return None
+
+
+def _rec_rope(c: _Ctx, nid: str) -> bool:
+    hit = _match_rope(c, nid)
+    if hit is None:
+        return False
+    t_id, cos_id, sin_id = hit
+    g = c.g
+    node = g.nodes[nid]
+    od = node.output.dtype
+    d = int(node.output.shape[-1])
+    # The rotated tensor, viewed through its layout ops, and what produced it.
+    t_view_shape = tuple(int(v) for v in g.nodes[t_id].output.shape)
+    src_id = _peel_layout(g, t_id)
+    rms = _match_rms_chain(c, src_id)
+    fuse_norm = rms is not None and rms.cols == d and all(cons in _rope_internal(g, t_id, nid) or isinstance(g.nodes[cons].op, LAYOUT_OPS) for cons in g.consumers(src_id))
+    # cos / sin tables: [.., positions, d] broadcast over the head axis.
+    cos_v, sin_v = _need(c, cos_id), _need(c, sin_id)
+    rot_expr = _round(od, _round(od, E.Var("y") * E.Var("cos")) + _round(od, E.Var("yr") * E.Var("sin")))
+
+    # Address rows of the *output* in the memory order of the rotated operand
+    # (so the kernel is a row map whatever transposes the trace applied).
+    tv = resolve_view(g, t_id)
+    if tv.strides[-1] != 1:
+        raise FusionError("rope: the rotated axis must be contiguous")
+    # memory-order dims of t (excluding the last): sort by stride descending
+    order = sorted(range(len(tv.shape) - 1), key=lambda i: -tv.strides[i] if tv.shape[i] > 1 else 0)
+    order = [i for i in order if tv.shape[i] > 1]
+    mem_shape = tuple(tv.shape[i] for i in order)
+    rows = 1
+    for n in mem_shape:
+        rows *= n
+    # position axis = the axis of t that cos varies over
+    cos_shape = tuple(int(v) for v in g.nodes[cos_id].output.shape)
+    pos_axes = [i for i in range(len(cos_shape) - 1) if cos_shape[i] > 1]
+    if len(pos_axes) > 1 or cos_shape[-1] != d:
+        raise FusionError("rope: cos/sin must vary over one position axis")
+    if not (cos_v.strides[-1] == 1 and sin_v.strides[-1] == 1):
+        raise FusionError("rope: cos/sin must be contiguous along the rotated axis")
+    if pos_axes:
+        pa = pos_axes[0]
+        if pa not in order or cos_v.strides[pa] != d or sin_v.strides[pa] != d:
+            raise FusionError("rope: unsupported cos/sin layout")
+        k = order.index(pa)
+        div = 1
+        for n in mem_shape[k + 1 :]:
+            div *= n
+        mod = mem_shape[k]
+        if any(mem_shape[i] > 1 for i in range(k)):
+            # batch axes outside the position axis: positions repeat per batch element
+            pass
+    else:
+        div, mod = 1, 1
+    row_ops = (RowOperand("cos", cos_v.dtype, div=div, mod=mod, offset=cos_v.offset), RowOperand("sin", sin_v.dtype, div=div, mod=mod, offset=sin_v.offset))
+
+    # Output buffer: rows in t's memory order; the logical result is a view of it.
+    out_mem_shape = (*mem_shape, d)
+    if fuse_norm:
+        body, inputs, xv = _rms_body(c, nid, rms, od)
+        if (body.rows, body.cols) != (rows, d):
+            raise FusionError("rope: norm rows do not match the rotated tensor")
+    else:
+        xv = _need(c, t_id)
+        rows2, x_addr = _row_addr(View(xv.base, xv.offset, tuple(tv.shape[i] for i in order) + (d,), tuple(tv.strides[i] for i in order) + (1,), xv.dtype))
+        body = RowReduce(rows=rows2, cols=d, x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=od, stats=(), project=E.Var("x"), x_addr=x_addr)
+        body.operand_buffers = {}
+        inputs = [xv.base]
+    body.row_operands = row_ops
+    body.rotate = RotateHalf(rot_expr)
+    body.operand_buffers.update({"cos": cos_v.base, "sin": sin_v.base})
+    inputs += [cos_v.base, sin_v.base]
+    _emit(c, nid, body, "rms_norm_rope" if fuse_norm else "rope", inputs, shape=out_mem_shape)
+    # Record how the logical (traced) shape maps onto the memory-order buffer.
+    strides_mem = contiguous_strides(out_mem_shape)
+    logical_strides = [0] * len(t_view_shape)
+    for pos, i in enumerate(order):
+        logical_strides[i] = strides_mem[pos]
+    logical_strides[-1] = 1
+    c.out.nodes[nid].hints["logical_view"] = (t_view_shape, tuple(logical_strides))
+    return True
+
+
+def _rope_internal(g: Graph, t_id: str, add_id: str) -> set[str]:
+    """Node ids that belong to the rope expression rooted at ``add_id`` (for single-use checks)."""
+    seen: set[str] = set()
+    stack = [add_id]
+    while stack:
+        n = stack.pop()
+        if n in seen or n == t_id:
+            continue
+        seen.add(n)
+        stack.extend(g.nodes[n].inputs)
+    seen.add(t_id)
+    return seen
+
+
+def _rec_sdpa(c: _Ctx, nid: str) -> bool:
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.SdpaOp):
+        return False
+    q, k, v = (_need_logical(c, i) for i in node.inputs)
+    if len(q.shape) != 4:
+        raise FusionError("sdpa: expected [batch, heads, seq, head_dim] operands")
+    B, Hq, Sq, D = q.shape
+    _, Hkv, Skv, _ = k.shape
+    if Hq != Hkv and not node.op.enable_gqa:
+        raise FusionError("sdpa: grouped heads need enable_gqa=True")
+    for t in (q, k, v):
+        if t.strides[-1] != 1:
+            raise FusionError("sdpa: head_dim must be contiguous")
+    # If the only consumer transposes to [B, S, H, D] (and flattens), write that layout directly.
+    out_id, o_shape, o_strides = nid, (B, Hq, Sq, D), (Hq * Sq * D, Sq * D, D)
+    cons = c.g.consumers(nid)
+    if len(cons) == 1 and nid not in c.g.outputs and _is(c.g.nodes[cons[0]], F.TransposeOp, dim0=1, dim1=2):
+        o_shape, o_strides = (B, Sq, Hq, D), (Sq * Hq * D, D, Hq * D)
+    scale = node.op.scale if node.op.scale is not None else 1.0 / math.sqrt(D)
+    body = Flash(
+        batch=B, q_heads=Hq, kv_heads=Hkv, q_len=Sq, kv_len=Skv, head_dim=D, q=q.base, k=k.base, v=v.base, out=out_id, dtype=q.dtype,
+        scale=float(scale), causal=node.op.is_causal, q_strides=q.strides[:3], k_strides=k.strides[:3], v_strides=v.strides[:3], o_strides=o_strides,
+        q_offset=q.offset, k_offset=k.offset, v_offset=v.offset,
+    )  # fmt: skip
+    _emit(c, nid, body, "sdpa_reduce", [q.base, k.base, v.base], shape=o_shape)
+    if o_shape != (B, Hq, Sq, D):
+        c.out.nodes[nid].hints["logical_view"] = ((B, Hq, Sq, D), (o_strides[0], o_strides[1], o_strides[2], 1))
+    return True
+
+
+def _need_logical(c: _Ctx, nid: str) -> View:
+    return _need(c, nid)
+
+
+_POINTWISE_FN = {"add": "add", "sub": "sub", "mul": "mul", "div": "div", "maximum": "max", "minimum": "min"}
+_POINTWISE_UN = {"neg": "neg", "rsqrt": "rsqrt", "sqrt": "sqrt", "exp": "exp", "silu": "silu", "sigmoid": "sigmoid", "tanh": "tanh", "abs": "abs", "reciprocal": "rcp"}
+
+
+def _rec_pointwise(c: _Ctx, nid: str) -> bool:
+    """Fallback: one element-wise op (or cast / copy) as a flat map over contiguous, same-shape operands."""
+    node = c.g.nodes[nid]
+    op = node.op
+    od = node.output.dtype
+    shape = tuple(int(d) for d in node.output.shape)
+    if isinstance(op, (F.CastOp, F.ContiguousOp)):
+        views = [_need_logical(c, node.inputs[0])]
+        expr = E.Var("a0")
+    elif isinstance(op, F.ElementwiseOp):
+        views = [_need_logical(c, i) for i in node.inputs]
+        vars_ = [E.Var(f"a{i}") for i in range(len(views))]
+        if op.fn in _POINTWISE_UN and len(vars_) == 1:
+            expr = E.Un(_POINTWISE_UN[op.fn], vars_[0])
+        elif op.fn == "pow" and op.scalar == 2.0:
+            expr = vars_[0] * vars_[0]
+        elif op.fn in _POINTWISE_FN:
+            if op.scalar is not None:
+                a, b = (E.Const(op.scalar), vars_[0]) if op.scalar_first else (vars_[0], E.Const(op.scalar))
+            else:
+                a, b = vars_
+            expr = E.Bin(_POINTWISE_FN[op.fn], a, b)
+        else:
+            raise FusionError(f"element-wise op {op.fn!r} is not supported")
+    else:
+        return False
+    operands = []
+    for i, v in enumerate(views):
+        if v.shape == shape and v.is_contiguous():
+            operands.append(MapOperand(f"a{i}", v.dtype, "flat"))
+        elif len(v.shape) >= 1 and v.shape[-1] == shape[-1] and all(d == 1 for d in v.shape[:-1]) and v.strides[-1] == 1:
+            operands.append(MapOperand(f"a{i}", v.dtype, "col"))
+        else:
+            raise FusionError(f"pointwise operand {i} of {nid!r} needs general broadcasting (shape {v.shape} strides {v.strides})")
+    numel = 1
+    for d in shape:
+        numel *= d
+    body = Map(numel=numel, operands=tuple(operands), expr=_round(od, expr) if od is not F32 else expr, out=nid, out_dtype=od, inner=shape[-1] if shape else 1)
+    body.operand_buffers = {f"a{i}": v.base for i, v in enumerate(views)}
+    body.operand_offsets = {f"a{i}": v.offset for i, v in enumerate(views)}
+    _emit(c, nid, body, f"pointwise_{type(op).__name__.lower().removesuffix('op')}", [v.base for v in views])
+    return True
+
+
+# ---------------------------------------------------------------------------
+# Driver
+# ---------------------------------------------------------------------------
+
+
+def fuse(g: Graph) -> Graph:
+    """Lower a frontend ``Graph`` to ``Graph[TileOp + InputOp + ConstantOp]``."""
+    out = Graph()
+    out.constant_values = dict(getattr(g, "constant_values", {}))
+    c = _Ctx(g=g, out=out)
+    # Inputs first, in their traced order, so positional binding stays stable.
+    for nid in g.inputs:
+        _materialize(c, nid)
+    final_outputs = []
+    for oid in g.outputs:
+        v = _need_logical(c, oid)
+        shape = tuple(int(d) for d in g.nodes[oid].output.shape)
+        if not (v.offset == 0 and v.shape == shape and v.is_contiguous()) and not _same_memory(v, shape):
+            raise FusionError(f"graph output {oid!r} is a strided view; a final copy kernel is not implemented")
+        final_outputs.append(v.base)
+        if v.base != oid:
+            out.nodes[v.base].hints.setdefault("output_alias", []).append((oid, shape))
+    out.outputs = final_outputs
+    return out
+
+
+def _same_memory(v: View, shape: tuple[int, ...]) -> bool:
+    """True when ``v`` enumerates its buffer in plain row-major order (e.g. a reshape of a contiguous buffer)."""
+    return v.offset == 0 and v.strides == contiguous_strides(v.shape)
+
+
+__all__ = ["fuse", "FusionError", "StackedConstant", "BF16", "F16"]

@@ -1,0 +1,54 @@
+"""``Graph[TileOp]`` → ``Graph[HipOp]``: render every scheduled tile to gfx950 source.
+
+Counterpart of the reference's last two pass directories
+(emmy/compiler/pipeline/__init__.py:46-47: ``lowering/kernel`` then
+``lowering/cuda``; 010_lower_kernelop.py renders a KernelOp to a CudaOp).
+Kernel names follow the reference's rule ``k_<label>_<hash[:6]>``
+(provenance.py:246-252) with the hash taken over the rendered body.
+"""
+
+from __future__ import annotations
+
+import hashlib
+
+from deplodock_amd.context import Context
+from deplodock_amd.emit.contraction import emit_contraction
+from deplodock_amd.emit.flash import emit_flash
+from deplodock_amd.emit.pointwise import emit_map
+from deplodock_amd.emit.reduce import emit_row_reduce
+from deplodock_amd.graph import Graph
+from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.tile import Contraction, Flash, Map, RowReduce, TileOp
+
+_PLACEHOLDER = "EMH_KERNEL_NAME_"
+
+
+def lower_tile(op: TileOp, ctx: Context) -> HipOp:
+    body = op.body
+    if isinstance(body, RowReduce):
+        hip = emit_row_reduce(body, _PLACEHOLDER, ctx)
+    elif isinstance(body, Contraction):
+        hip = emit_contraction(body, _PLACEHOLDER, ctx)
+    elif isinstance(body, Flash):
+        hip = emit_flash(body, _PLACEHOLDER, ctx)
+    elif isinstance(body, Map):
+        hip = emit_map(body, _PLACEHOLDER, ctx)
+    else:
+        raise TypeError(f"unknown tile body {type(body).__name__}")
+    label = op.name.split("__")[0]
+    digest = hashlib.sha1(hip.kernel_source.encode()).hexdigest()[:6]
+    name = f"{label}_{digest}"
+    hip.kernel_source = hip.kernel_source.replace(_PLACEHOLDER, name)
+    hip.kernel_name = name
+    hip.source = op
+    hip.knobs = {**op.knobs, **hip.knobs}
+    return hip
+
+
+def lower(graph: Graph, ctx: Context | None = None) -> Graph:
+    """Replace every ``TileOp`` by its ``HipOp`` (in place) and return the graph."""
+    ctx = ctx or Context()
+    for node in graph.nodes.values():
+        if isinstance(node.op, TileOp):
+            node.op = lower_tile(node.op, ctx)
+    return graph

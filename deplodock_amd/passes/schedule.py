@@ -1,0 +1,214 @@
+"""Schedule selection for gfx950: stamp ``ReducePlan`` / ``TilePlan`` / ``Stage`` on each tile.
+
+Plays the role of the reference's ``_schedule`` (emmy/compiler/pipeline/passes/lowering/tile/_schedule.py:
+``_pick_coop`` :104-117, contraction rows :382-419, ``schedule`` :819-899) with the
+constants re-derived for 256 CUs, wave64 and 160 KB of LDS:
+
+* ``EMMY_REDUCE`` / ``EMMY_TILE`` / ``EMMY_STAGE`` (or ``EMMY_KNOBS``) pins are
+  authoritative.  A pin that does not parse or cannot be realised degrades to the
+  heuristic pick and the *resolved* spelling is stamped on the op's ``knobs``
+  (_schedule.py:755-761, 813-815).
+* Row reductions: the reference refuses cooperation above 256 free rows
+  (``_FREE_CAP``) and falls back to one thread per row; here every row kernel
+  is cooperative and coalesced, and the lane count per row follows the row
+  length so the row stays register-resident.
+* Contractions: the tile is chosen so the launch fills the CUs (>= one workgroup
+  per CU where the problem allows) before it is chosen for operand reuse; the
+  candidates and their measured ranking live in ``TILE_CANDIDATES``.
+"""
+
+from __future__ import annotations
+
+import logging
+
+from deplodock_amd import config
+from deplodock_amd.context import Context
+from deplodock_amd.graph import Graph
+from deplodock_amd.ir.schedule import ATOMS, ReducePlan, ScheduleError, Stage, TilePlan
+from deplodock_amd.ir.tile import Contraction, Flash, Map, RowReduce, TileOp
+
+logger = logging.getLogger(__name__)
+
+# (tile_m, tile_n, waves_m, waves_n, atom, bk) — ordered by measured throughput on
+# MI355X for large bf16 problems (first fit that fills the machine wins).
+TILE_CANDIDATES: tuple[tuple[int, int, int, int, str, int], ...] = (
+    (128, 192, 4, 2, "mfma_16x16x32_bf16", 2),
+    (128, 128, 2, 2, "mfma_32x32x16_bf16", 4),
+    (128, 96, 4, 1, "mfma_32x32x16_bf16", 4),
+    (64, 128, 2, 2, "mfma_32x32x16_bf16", 4),
+    (64, 64, 2, 2, "mfma_16x16x32_bf16", 2),
+    (32, 64, 1, 2, "mfma_16x16x32_bf16", 2),
+    (16, 64, 1, 4, "mfma_16x16x32_bf16", 2),
+)
+
+
+def _pin(name: str) -> str | None:
+    return config.knob_raw(name)
+
+
+def pick_coop(cols: int, elem_bytes: int, rows: int, ctx: Context, *, rotate: bool = False) -> int:
+    """Lanes that share one row.  A lane keeps at most 32 row elements resident;
+    up to 256 lanes are used as long as each still issues two 16-byte loads."""
+    vec = max(1, 16 // elem_bytes)
+    chunks = max(1, cols // vec) if cols % vec == 0 else cols
+    if rotate:
+        lanes = 1
+        while lanes * 2 <= 64 and (chunks // 2) % (lanes * 2) == 0 and chunks // (lanes * 2) >= 2:
+            lanes *= 2
+        return lanes
+    lanes = 1
+    while lanes < 1024 and cols > lanes * 32:
+        lanes *= 2
+    # Bandwidth-bound rows run fastest with two 16-byte loads per lane in flight
+    # and many waves per CU (measured on 2048-wide fp32 rows: b256 beats b64 by 10 %).
+    while lanes < 256 and chunks >= lanes * 4:
+        lanes *= 2
+    # Few rows: spread each row over more lanes so more CUs take part.
+    while lanes < 256 and rows * lanes < ctx.compute_units * 64 and chunks >= lanes * 2:
+        lanes *= 2
+    return min(lanes, 1024)
+
+
+def _pow2_floor(v: int) -> int:
+    p = 1
+    while p * 2 <= v:
+        p *= 2
+    return p
+
+
+def schedule_row_reduce(body: RowReduce, ctx: Context) -> dict:
+    pinned = _pin("REDUCE")
+    plan = None
+    if pinned is not None:
+        try:
+            plan = ReducePlan.parse(pinned)
+            if plan.cta != 1:
+                raise ScheduleError("cross-workgroup split does not apply to a projected row")
+            if body.rotate is not None:
+                vec = 16 // max(body.x_dtype.nbytes, body.out_dtype.nbytes)
+                if (body.cols // vec // 2) % plan.coop:
+                    raise ScheduleError("rotate-half needs both halves of a row in one lane")
+        except ScheduleError as exc:
+            logger.warning("EMMY_REDUCE=%r ignored: %s", pinned, exc)
+            plan = None
+    if plan is None:
+        eb = max(body.x_dtype.nbytes, body.out_dtype.nbytes)
+        plan = ReducePlan(coop=pick_coop(body.cols, eb, body.rows, ctx, rotate=body.rotate is not None))
+    body.reduce = plan
+    nt = _pin("NT")
+    if nt is not None:
+        body.nontemporal = nt.strip().lower() in ("1", "true", "yes", "on")
+    else:
+        # Streaming rows far larger than the caches: bypass-style accesses measured ~10 % faster.
+        body.nontemporal = body.algo_bytes() > 256 * 1024 * 1024
+    return {"REDUCE": plan.spell(), "NT": int(body.nontemporal)}
+
+
+def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context) -> TilePlan:
+    """First candidate (in measured-throughput order) whose launch covers the
+    CUs, else the one that launches the most workgroups."""
+    best = None
+    for tm, tn, wm, wn, atom_name, bk in TILE_CANDIDATES:
+        atom = ATOMS[atom_name]
+        if tm % (wm * atom.m) or tn % (wn * atom.n):
+            continue
+        fm, fn = tm // (wm * atom.m), tn // (wn * atom.n)
+        if fm * fn * atom.acc_per_lane * (2 if gate_pair else 1) > 256:
+            continue
+        while bk > 1 and k % (bk * atom.k):
+            bk //= 2
+        if k % (bk * atom.k):
+            continue
+        threads = wm * wn * 64
+        cpr = bk * atom.k // 8
+        if (tm * cpr) % threads or (tn * cpr * (2 if gate_pair else 1)) % threads:
+            continue
+        plan = TilePlan(atom=atom, units=(wm, wn), regs=(fm, fn), bk=bk)
+        groups = -(-m // tm) * -(-n // tn)
+        # penalise tiles that mostly hang over the edge of a small problem
+        waste = (-(-m // tm) * tm * -(-n // tn) * tn) / float(m * n)
+        if groups >= ctx.compute_units and waste < 1.5:
+            return plan
+        score = (min(groups, ctx.compute_units) / waste, tm * tn)
+        if best is None or score > best[0]:
+            best = (score, plan)
+    if best is None:
+        raise ScheduleError(f"no MFMA tile fits M={m} N={n} K={k}")
+    return best[1]
+
+
+def schedule_contraction(body: Contraction, ctx: Context) -> dict:
+    pinned = _pin("TILE")
+    plan = None
+    if pinned:
+        try:
+            plan = TilePlan.parse(pinned)
+            if plan.atom.dtype != body.in_dtype.name:
+                raise ScheduleError(f"atom {plan.atom.name} does not take {body.in_dtype} operands")
+            if body.k % plan.bk_elems:
+                raise ScheduleError(f"K={body.k} is not a multiple of the slab depth {plan.bk_elems}")
+        except ScheduleError as exc:
+            logger.warning("EMMY_TILE=%r ignored: %s", pinned, exc)
+            plan = None
+    if plan is None:
+        atom_dtype = body.in_dtype.name
+        plan = pick_tile(body.m, body.n, body.k, body.gate_pair, ctx)
+        if plan.atom.dtype != atom_dtype:
+            plan = TilePlan(atom=ATOMS[plan.atom.name.replace("bf16", atom_dtype)], units=plan.units, regs=plan.regs, bk=plan.bk)
+    body.tile = plan
+    stage = None
+    pinned_stage = _pin("STAGE")
+    if pinned_stage:
+        try:
+            stage = Stage.parse(pinned_stage)
+            if stage is not None and stage.transport == "dl" and (plan.bk_elems // plan.atom.k) % 2:
+                raise ScheduleError("direct-to-LDS staging needs an even number of MFMA steps per slab")
+        except ScheduleError as exc:
+            logger.warning("EMMY_STAGE=%r ignored: %s", pinned_stage, exc)
+            stage = None
+    if stage is None:
+        stage = Stage(depth=2, transport="sync")
+    body.stage = stage
+    return {"TILE": plan.spell(), "STAGE": stage.spell()}
+
+
+def schedule_flash(body: Flash, ctx: Context) -> dict:
+    pinned = _pin("FLASH")
+    if pinned:
+        try:
+            for tok in pinned.split("/"):
+                if tok.startswith("w"):
+                    body.waves = int(tok[1:])
+                elif tok.startswith("kv"):
+                    body.block_kv = int(tok[2:])
+                else:
+                    raise ScheduleError(f"cannot parse {tok!r} (expect w<waves> / kv<keys>)")
+        except (ValueError, ScheduleError) as exc:
+            logger.warning("EMMY_FLASH=%r ignored: %s", pinned, exc)
+    else:
+        # Short sequences: shrink the query block until the launch covers the CUs.
+        heads = body.batch * body.q_heads
+        while body.waves > 1 and heads * -(-body.q_len // (32 * body.waves)) < ctx.compute_units:
+            body.waves //= 2
+    return {"FLASH": f"w{body.waves}/kv{body.block_kv}"}
+
+
+def schedule(graph: Graph, ctx: Context | None = None) -> Graph:
+    """Stamp a plan on every ``TileOp`` in ``graph`` (in place) and return it."""
+    ctx = ctx or Context()
+    for node in graph.nodes.values():
+        op = node.op
+        if not isinstance(op, TileOp):
+            continue
+        body = op.body
+        if isinstance(body, RowReduce):
+            op.knobs.update(schedule_row_reduce(body, ctx))
+        elif isinstance(body, Contraction):
+            op.knobs.update(schedule_contraction(body, ctx))
+        elif isinstance(body, Flash):
+            op.knobs.update(schedule_flash(body, ctx))
+        elif isinstance(body, Map):
+            pass
+        else:
+            raise TypeError(f"unknown tile body {type(body).__name__}")
+    return graph

@@ -1,0 +1,214 @@
+"""``torch.export`` → frontend ``Graph`` (one node per ATen call).
+
+Mirrors the reference tracer's contract (emmy/compiler/trace/torch.py:52-135):
+``trace_module(module, example_inputs, kwargs=...)`` returns a ``Graph`` whose
+inputs are the user inputs, whose constants are the module's parameters and
+buffers (values kept on ``graph.constant_values``), and whose nodes carry the
+traced shapes and dtypes — the graph dtype *is* the traced dtype.  SDPA's
+``is_causal`` / ``scale`` / ``enable_gqa`` are captured as attributes (:559-583).
+"""
+
+from __future__ import annotations
+
+import operator
+
+from deplodock_amd import dtype as dt
+from deplodock_amd.graph import Graph, Tensor
+from deplodock_amd.ir import frontend as F
+
+
+class TraceError(NotImplementedError):
+    """The module uses an ATen op this tracer does not know."""
+
+
+def _shape(val) -> tuple[int, ...]:
+    return tuple(int(d) for d in val.shape)
+
+
+def _norm_dim(d: int, rank: int) -> int:
+    return d if d >= 0 else d + rank
+
+
+def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dynamic_shapes=None) -> Graph:
+    """Trace ``module(*example_inputs, **kwargs)`` into a frontend ``Graph``."""
+    import torch
+
+    if dynamic_shapes is not None:
+        raise TraceError("symbolic shapes are not supported by this tracer yet: trace at the concrete shape")
+    module = module.eval()
+    with torch.no_grad():
+        ep = torch.export.export(module, tuple(example_inputs), kwargs=kwargs or {}, strict=False)
+    sig = ep.graph_signature
+    kinds = {s.arg.name: s for s in sig.input_specs}
+    state = {}
+    state.update(dict(ep.state_dict))
+    state.update(dict(getattr(ep, "constants", {}) or {}))
+
+    g = Graph()
+    g.constant_values = {}
+    env: dict[str, str] = {}  # fx node name -> graph node id
+
+    def out_tensor(node) -> Tensor:
+        val = node.meta["val"]
+        return Tensor(node.name, _shape(val), dt.from_torch(val.dtype))
+
+    def add(node, op, inputs) -> None:
+        env[node.name] = g.add_node(op, [env[i.name] for i in inputs], out_tensor(node), node.name)
+
+    aten = torch.ops.aten
+    for node in ep.graph.nodes:
+        if node.op == "placeholder":
+            spec = kinds[node.name]
+            val = node.meta["val"]
+            if spec.kind.name == "USER_INPUT":
+                env[node.name] = g.add_input(node.name, _shape(val), dt.from_torch(val.dtype))
+            else:
+                nid = g.add_constant(node.name, _shape(val), dt.from_torch(val.dtype), source_path=spec.target)
+                g.constant_values[nid] = state[spec.target].detach()
+                env[node.name] = nid
+            continue
+        if node.op == "output":
+            outs = node.args[0]
+            outs = outs if isinstance(outs, (tuple, list)) else (outs,)
+            g.outputs = [env[o.name] for o in outs if o is not None]
+            continue
+        if node.op != "call_function":
+            raise TraceError(f"unsupported fx node kind {node.op!r}")
+        t = node.target
+        a = node.args
+        kw = node.kwargs
+        rank_in = len(a[0].meta["val"].shape) if a and hasattr(a[0], "meta") and hasattr(a[0].meta.get("val"), "shape") else 0
+
+        if t in (aten._assert_tensor_metadata.default,):
+            continue
+        if t is operator.getitem:
+            raise TraceError("tuple-valued ops are not supported")
+        if t == aten.rms_norm.default:
+            x, _shape_arg, w, eps = (list(a) + [None, None])[:4]
+            add(node, F.RmsNormOp(eps=float(eps if eps is not None else 1e-6), has_weight=w is not None), [x] + ([w] if w is not None else []))
+        elif t in (aten.softmax.int, aten._softmax.default):
+            add(node, F.SoftmaxOp(axis=_norm_dim(int(a[1]), rank_in)), [a[0]])
+        elif t == aten.linear.default:
+            ins = [a[0], a[1]] + ([a[2]] if len(a) > 2 and a[2] is not None else [])
+            add(node, F.LinearOp(has_bias=len(ins) == 3), ins)
+        elif t == aten.scaled_dot_product_attention.default:
+            mask = a[3] if len(a) > 3 else kw.get("attn_mask")
+            if mask is not None:
+                raise TraceError("scaled_dot_product_attention with an explicit mask is not supported")
+            dropout = a[4] if len(a) > 4 else kw.get("dropout_p", 0.0)
+            if dropout:
+                raise TraceError("attention dropout is not supported")
+            causal = bool(a[5] if len(a) > 5 else kw.get("is_causal", False))
+            scale = kw.get("scale")
+            add(node, F.SdpaOp(is_causal=causal, scale=None if scale is None else float(scale), enable_gqa=bool(kw.get("enable_gqa", False))), [a[0], a[1], a[2]])
+        elif t in (aten.to.dtype, aten._to_copy.default, aten.to.dtype_layout):
+            target = a[1] if len(a) > 1 and isinstance(a[1], torch.dtype) else kw.get("dtype")
+            add(node, F.CastOp(dtype=dt.from_torch(target)), [a[0]])
+        elif t in (aten.mean.dim, aten.sum.dim_IntList):
+            dims = a[1] if isinstance(a[1], (list, tuple)) else [a[1]]
+            if len(dims) != 1:
+                raise TraceError("multi-axis reductions are not supported")
+            keep = bool(a[2]) if len(a) > 2 else bool(kw.get("keepdim", False))
+            cls = F.MeanOp if t == aten.mean.dim else F.SumOp
+            add(node, cls(axis=_norm_dim(int(dims[0]), rank_in), keepdim=keep), [a[0]])
+        elif t in (aten.view.default, aten.reshape.default, aten._unsafe_view.default):
+            add(node, F.ViewOp(shape=_shape(node.meta["val"])), [a[0]])
+        elif t == aten.flatten.using_ints:
+            add(node, F.ViewOp(shape=_shape(node.meta["val"])), [a[0]])
+        elif t == aten.transpose.int:
+            add(node, F.TransposeOp(dim0=_norm_dim(int(a[1]), rank_in), dim1=_norm_dim(int(a[2]), rank_in)), [a[0]])
+        elif t == aten.permute.default:
+            add(node, F.PermuteOp(dims=tuple(_norm_dim(int(d), rank_in) for d in a[1])), [a[0]])
+        elif t == aten.unsqueeze.default:
+            add(node, F.UnsqueezeOp(dim=_norm_dim(int(a[1]), rank_in + 1)), [a[0]])
+        elif t == aten.squeeze.dim:
+            add(node, F.SqueezeOp(dim=_norm_dim(int(a[1]), rank_in)), [a[0]])
+        elif t == aten.slice.Tensor:
+            dim = _norm_dim(int(a[1]) if len(a) > 1 else 0, rank_in)
+            size = int(a[0].meta["val"].shape[dim])
+            start = int(a[2]) if len(a) > 2 and a[2] is not None else 0
+            end = int(a[3]) if len(a) > 3 and a[3] is not None else size
+            step = int(a[4]) if len(a) > 4 else 1
+            start = max(0, start + size if start < 0 else start)
+            end = min(size, end + size if end < 0 else end)
+            add(node, F.SliceOp(dim=dim, start=start, end=end, step=step), [a[0]])
+        elif t == aten.cat.default:
+            tensors = list(a[0])
+            dim = _norm_dim(int(a[1]) if len(a) > 1 else 0, len(tensors[0].meta["val"].shape))
+            add(node, F.CatOp(dim=dim), tensors)
+        elif t in (aten.contiguous.default, aten.clone.default, aten.alias.default, aten.detach.default):
+            add(node, F.ContiguousOp(), [a[0]])
+        elif t in _UNARY:
+            add(node, F.ElementwiseOp(fn=_UNARY[t]), [a[0]])
+        elif t in _BINARY:
+            fn = _BINARY[t]
+            lhs, rhs = a[0], a[1]
+            lt, rt = hasattr(lhs, "meta"), hasattr(rhs, "meta")
+            if lt and rt:
+                add(node, F.ElementwiseOp(fn=fn), [lhs, rhs])
+            elif lt:
+                add(node, F.ElementwiseOp(fn=fn, scalar=float(rhs)), [lhs])
+            elif rt:
+                add(node, F.ElementwiseOp(fn=fn, scalar=float(lhs), scalar_first=True), [rhs])
+            else:
+                raise TraceError(f"{t}: no tensor operand")
+        else:
+            raise TraceError(f"unsupported ATen op {t} (node {node.name})")
+    return g
+
+
+def _tables():
+    import torch
+
+    aten = torch.ops.aten
+    unary = {
+        aten.neg.default: "neg",
+        aten.rsqrt.default: "rsqrt",
+        aten.sqrt.default: "sqrt",
+        aten.exp.default: "exp",
+        aten.silu.default: "silu",
+        aten.sigmoid.default: "sigmoid",
+        aten.tanh.default: "tanh",
+        aten.abs.default: "abs",
+        aten.reciprocal.default: "reciprocal",
+    }
+    binary = {
+        aten.add.Tensor: "add",
+        aten.add.Scalar: "add",
+        aten.sub.Tensor: "sub",
+        aten.sub.Scalar: "sub",
+        aten.mul.Tensor: "mul",
+        aten.mul.Scalar: "mul",
+        aten.div.Tensor: "div",
+        aten.div.Scalar: "div",
+        aten.pow.Tensor_Scalar: "pow",
+        aten.maximum.default: "maximum",
+        aten.minimum.default: "minimum",
+    }
+    return unary, binary
+
+
+class _Lazy(dict):
+    """ATen-target tables built on first use (keeps ``import`` torch-free)."""
+
+    def __init__(self, idx: int):
+        super().__init__()
+        self._idx = idx
+        self._ready = False
+
+    def _fill(self) -> None:
+        if not self._ready:
+            self.update(_tables()[self._idx])
+            self._ready = True
+
+    def __contains__(self, k) -> bool:
+        self._fill()
+        return dict.__contains__(self, k)
+
+    def __getitem__(self, k):
+        self._fill()
+        return dict.__getitem__(self, k)
+
+
+_UNARY = _Lazy(0)
+_BINARY = _Lazy(1)
