@@ -141,22 +141,18 @@ def _symbolic_bindings(graph: Graph) -> dict[str, tuple[str, int]]:
 
 def _compile(graph: Graph) -> _Compiled:
     bufs = _buffers(graph)
-    kernels: dict[str, hiprtc.LoadedKernel] = {}
-    seen_source: dict[str, str] = {}
     launches: list[_Launch] = []
-    need_zero = False
+    sources: dict[str, str] = {}
+    # Pass 1 — validate the whole graph before anything touches the device.
     for node in _launches(graph):
         op: HipOp = node.op
         kname = op.kernel_name
-        if kname not in kernels:
-            prev = seen_source.get(kname)
-            if prev is not None and prev != op.kernel_source:
-                raise ValueError(f"kernel name {kname!r} used by two distinct sources")
-            seen_source[kname] = op.kernel_source
-            kernels[kname] = hiprtc.load_function(op.kernel_source, kname)
-        elif seen_source[kname] != op.kernel_source:
+        if sources.setdefault(kname, op.kernel_source) != op.kernel_source:
             raise ValueError(f"kernel name {kname!r} used by two distinct sources")
-        need_zero = need_zero or bool(op.zero_outputs)
+        known = {b.name for b in bufs}
+        for arg in (*op.arg_order, *op.zero_outputs):
+            if arg not in known:
+                raise KeyError(f"kernel {kname!r} references unknown buffer {arg!r}")
         launches.append(
             _Launch(
                 node_id=node.id,
@@ -171,8 +167,10 @@ def _compile(graph: Graph) -> _Compiled:
                 algo_flops=op.algo_flops,
             )
         )
-    if need_zero:
-        kernels[_ZERO_KERNEL_NAME] = hiprtc.load_function(_ZERO_KERNEL_SRC, _ZERO_KERNEL_NAME)
+    if any(ln.zero_outputs for ln in launches):
+        sources[_ZERO_KERNEL_NAME] = _ZERO_KERNEL_SRC
+    # Pass 2 — compile (cached) and load.
+    kernels = {name: hiprtc.load_function(src, name) for name, src in sources.items()}
     constants = {nid: float(op.value) for nid, op in graph.constant_ops() if op.value is not None}
     return _Compiled(bufs, {b.name: b for b in bufs}, constants, kernels, launches, _symbolic_bindings(graph))
 

@@ -84,6 +84,8 @@ def schedule_row_reduce(body: RowReduce, ctx: Context) -> dict:
             plan = ReducePlan.parse(pinned)
             if plan.cta != 1:
                 raise ScheduleError("cross-workgroup split does not apply to a projected row")
+            if -(-body.cols // plan.coop) > 64:
+                raise ScheduleError(f"{body.cols} columns over {plan.coop} lanes do not fit the register-resident row")
             if body.rotate is not None:
                 vec = 16 // max(body.x_dtype.nbytes, body.out_dtype.nbytes)
                 if (body.cols // vec // 2) % plan.coop:

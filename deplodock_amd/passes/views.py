@@ -32,7 +32,9 @@ class View:
         return n
 
     def is_contiguous(self) -> bool:
-        return self.strides == contiguous_strides(self.shape) or self.numel <= 1
+        """Row-major dense; the stride of a size-1 dimension is irrelevant."""
+        want = contiguous_strides(self.shape)
+        return all(n == 1 or s == w for n, s, w in zip(self.shape, self.strides, want))
 
     def collapse_leading(self, keep: int) -> tuple[int, int] | None:
         """If all but the last ``keep`` dims form one uniformly strided run,

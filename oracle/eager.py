@@ -1,0 +1,180 @@
+"""The prescribed oracle: PyTorch eager on the same module and seeded inputs.
+
+TEST INFRASTRUCTURE ONLY (see ``oracle/__init__.py``).  Holds the seeded input
+recipes of the five benchmark configurations (generated on the CPU so every
+machine sees identical bits), the modules they run through, and the tolerance
+checker.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+from torch import nn
+
+FP32_RTOL = 1e-5
+BF16_RTOL = 2e-2
+
+
+@dataclass
+class Case:
+    name: str
+    module: nn.Module
+    inputs: tuple
+    rtol: float
+    atol: float
+    algo_bytes: int = 0
+    algo_flops: int = 0
+
+
+class Sdpa(nn.Module):
+    def __init__(self, causal: bool = True):
+        super().__init__()
+        self.causal = causal
+
+    def forward(self, q, k, v):
+        return nn.functional.scaled_dot_product_attention(q, k, v, is_causal=self.causal, enable_gqa=True)
+
+
+def rms_norm_case(rows: int = 32, cols: int = 2048, seed: int = 0) -> Case:
+    """C1: ``nn.RMSNorm(2048, eps=1e-6)`` on fp32 ``[1, rows, cols]`` ~N(0,1), weight ~N(1, 0.1)."""
+    torch.manual_seed(seed)
+    x = torch.randn(1, rows, cols)
+    m = nn.RMSNorm(cols, eps=1e-6)
+    with torch.no_grad():
+        m.weight.copy_(1 + 0.1 * torch.randn(cols))
+    return Case(f"rms_norm_{rows}x{cols}", m.eval(), (x,), FP32_RTOL, 1e-6, algo_bytes=(2 * rows * cols + cols) * 4)
+
+
+def softmax_case(shape=(1, 28, 2048, 2048), seed: int = 0) -> Case:
+    """C2: ``nn.Softmax(-1)`` on fp32 ~N(0, 2).  The absolute floor covers outputs
+    near zero, where a pure relative bound is ill-posed."""
+    torch.manual_seed(seed)
+    x = 2 * torch.randn(*shape)
+    return Case("softmax_" + "x".join(map(str, shape)), nn.Softmax(dim=-1).eval(), (x,), FP32_RTOL, 1e-9, algo_bytes=2 * x.numel() * 4)
+
+
+def linear_case(m: int = 2048, k: int = 1024, n: int = 3072, seed: int = 0) -> Case:
+    """C3: ``nn.Linear(k, n, bias=False)`` bf16, x ~N(0,1), W ~N(0, 0.02)."""
+    torch.manual_seed(seed)
+    x = torch.randn(m, k).bfloat16()
+    lin = nn.Linear(k, n, bias=False)
+    with torch.no_grad():
+        lin.weight.copy_(0.02 * torch.randn(n, k))
+    return Case(f"linear_{m}x{k}x{n}", lin.bfloat16().eval(), (x,), BF16_RTOL, 2e-2, algo_bytes=(m * k + n * k + m * n) * 2, algo_flops=2 * m * n * k)
+
+
+def sdpa_case(b: int = 1, hq: int = 16, hkv: int = 8, s: int = 2048, d: int = 128, causal: bool = True, seed: int = 0) -> Case:
+    """C4: causal GQA attention, bf16 ~N(0,1), scale 1/sqrt(d)."""
+    torch.manual_seed(seed)
+    q = torch.randn(b, hq, s, d).bfloat16()
+    k = torch.randn(b, hkv, s, d).bfloat16()
+    v = torch.randn(b, hkv, s, d).bfloat16()
+    pairs = s * (s + 1) // 2 if causal else s * s
+    return Case(
+        f"sdpa_{b}x{hq}x{hkv}x{s}x{d}", Sdpa(causal).eval(), (q, k, v), BF16_RTOL, 2e-2,
+        algo_bytes=(2 * b * hq * s * d + 2 * b * hkv * s * d) * 2, algo_flops=4 * b * hq * d * pairs,
+    )  # fmt: skip
+
+
+class Qwen3Block(nn.Module):
+    """Wraps ``transformers``' ``Qwen3DecoderLayer`` (built from a local config,
+    no download) so it takes ``(x, cos, sin)`` and returns the hidden state."""
+
+    def __init__(self, layer):
+        super().__init__()
+        self.l = layer
+
+    def forward(self, x, cos, sin):
+        out = self.l(x, position_embeddings=(cos, sin), attention_mask=None)
+        return out[0] if isinstance(out, tuple) else out
+
+
+def qwen3_block_case(seq: int = 512, seed: int = 0, dtype=torch.bfloat16) -> Case:
+    """C5: one Qwen3-0.6B-architecture decoder block, weights ~N(0, 0.02), norm
+    weights 1, x ~N(0,1), positions 0..seq-1, RoPE theta 1e6."""
+    from transformers import Qwen3Config
+    from transformers.models.qwen3.modeling_qwen3 import Qwen3DecoderLayer, Qwen3RotaryEmbedding
+
+    cfg = Qwen3Config(
+        hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128, intermediate_size=3072,
+        rms_norm_eps=1e-6, rope_theta=1e6, num_hidden_layers=1, vocab_size=1024, max_position_embeddings=max(4096, seq),
+    )  # fmt: skip
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(seed)
+    layer = Qwen3DecoderLayer(cfg, 0)
+    with torch.no_grad():
+        for name, p in layer.named_parameters():
+            if "norm" in name:
+                p.fill_(1.0)
+            else:
+                p.copy_(0.02 * torch.randn_like(p))
+    x = torch.randn(1, seq, 1024)
+    cos, sin = Qwen3RotaryEmbedding(cfg)(x, torch.arange(seq)[None])
+    h, hq, hkv, d, inter = 1024, 16, 8, 128, 3072
+    flops = 2 * seq * h * (hq * d + 2 * hkv * d) + 2 * seq * hq * d * h + 3 * 2 * seq * h * inter + 4 * hq * d * (seq * (seq + 1) // 2)
+    wbytes = (h * (hq * d + 2 * hkv * d) + hq * d * h + 3 * h * inter) * 2
+    return Case(
+        f"qwen3_block_s{seq}", Qwen3Block(layer).to(dtype).eval(), (x.to(dtype), cos.to(dtype), sin.to(dtype)),
+        BF16_RTOL if dtype is torch.bfloat16 else 1e-4, 4e-2 if dtype is torch.bfloat16 else 1e-4, algo_bytes=wbytes, algo_flops=flops,
+    )  # fmt: skip
+
+
+def block_weights(case: Case) -> dict:
+    """Parameter arrays of a :func:`qwen3_block_case` keyed the way ``emmy_ops.qwen3_block`` wants."""
+    sd = {k: v.float().numpy() for k, v in case.module.state_dict().items()}
+    pick = lambda frag: next(v for k, v in sd.items() if frag in k)  # noqa: E731
+    return {
+        "input_layernorm": pick("input_layernorm"), "post_attention_layernorm": pick("post_attention_layernorm"),
+        "q_proj": pick("q_proj"), "k_proj": pick("k_proj"), "v_proj": pick("v_proj"), "o_proj": pick("o_proj"),
+        "q_norm": pick("q_norm"), "k_norm": pick("k_norm"), "gate_proj": pick("gate_proj"), "up_proj": pick("up_proj"), "down_proj": pick("down_proj"),
+    }  # fmt: skip
+
+
+def run_eager(case: Case, device: str = "cpu") -> torch.Tensor:
+    m = case.module.to(device)
+    with torch.no_grad():
+        out = m(*(t.to(device) for t in case.inputs))
+    return out
+
+
+def assert_close(actual: torch.Tensor, expected: torch.Tensor, rtol: float, atol: float, what: str = "") -> None:
+    a, e = actual.detach().float().cpu(), expected.detach().float().cpu()
+    if a.shape != e.shape:
+        raise AssertionError(f"{what}: shape {tuple(a.shape)} != {tuple(e.shape)}")
+    err = (a - e).abs()
+    bound = atol + rtol * e.abs()
+    bad = err > bound
+    if bool(bad.any()) or not bool(torch.isfinite(a).all()):
+        idx = int(torch.argmax(err - bound))
+        raise AssertionError(
+            f"{what}: {int(bad.sum())}/{a.numel()} elements outside atol={atol} rtol={rtol}; "
+            f"worst |diff|={float(err.flatten()[idx]):.3e} at flat index {idx} (expected {float(e.flatten()[idx]):.6e}, got {float(a.flatten()[idx]):.6e})"
+        )
+
+
+def time_eager_cpu(case: Case, *, threads: int, warmup: int = 1, iters: int = 3) -> float:
+    """Median seconds per forward of ``case`` on ``threads`` host cores."""
+    import statistics
+    import time
+
+    old = torch.get_num_threads()
+    torch.set_num_threads(threads)
+    try:
+        m = case.module.cpu()
+        with torch.no_grad():
+            for _ in range(warmup):
+                m(*case.inputs)
+            samples = []
+            for _ in range(iters):
+                t0 = time.perf_counter()
+                m(*case.inputs)
+                samples.append(time.perf_counter() - t0)
+    finally:
+        torch.set_num_threads(old)
+    return statistics.median(samples)
+
+
+__all__ = ["Case", "rms_norm_case", "softmax_case", "linear_case", "sdpa_case", "qwen3_block_case", "run_eager", "assert_close", "time_eager_cpu", "block_weights", "math"]

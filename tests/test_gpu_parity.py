@@ -1,0 +1,224 @@
+"""Parity of the HIP path with the oracle (PyTorch eager on the same module and
+seeded inputs), through the public backend API and therefore through the C-ABI
+library.  Tolerances: fp32 rtol 1e-5 (plus a stated absolute floor), bf16 rtol
+2e-2 with fp32 accumulation."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+from deplodock_amd import HipBackend, trace_module
+from deplodock_amd.backend.hip import program
+from deplodock_amd.dtype import BF16, F32
+from deplodock_amd.graph import Graph, Tensor
+from deplodock_amd.ir import expr as E
+from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.schedule import ReducePlan
+from deplodock_amd.ir.tile import RowReduce, Stat, TileOp
+from deplodock_amd.passes.lower import lower
+from oracle import eager
+from oracle import emmy_ops as O
+
+pytestmark = pytest.mark.gpu
+
+
+def run_case(case, device, **env):
+    """Trace → compile → run on the device; returns (our output tensor, eager-on-GPU output)."""
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    names = compiled.inputs
+    prog = be.program(compiled, {n: t.to(device) for n, t in zip(names, case.inputs)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = eager.run_eager(case, device)
+    return ours.reshape(want.shape), want, compiled
+
+
+# -- C1 ---------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("rows", [32, 32768])
+def test_c1_rms_norm(device, rows):
+    case = eager.rms_norm_case(rows=rows)
+    ours, want, _ = run_case(case, device)
+    eager.assert_close(ours, want, case.rtol, case.atol, "rms_norm vs eager (GPU)")
+    if rows == 32:
+        eager.assert_close(ours, eager.run_eager(case, "cpu"), case.rtol, case.atol, "rms_norm vs eager (CPU)")
+    # size-independent property: rows of y / w have unit RMS
+    w = case.module.weight.detach().to(device)
+    rms = ((ours / w).double().pow(2).mean(-1)).sqrt()
+    assert float((rms - 1).abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("coop", ["b16", "b64", "b128", "b256", "b1024"])
+def test_c1_every_cooperative_width(device, coop, monkeypatch):
+    monkeypatch.setenv("EMMY_REDUCE", coop)
+    case = eager.rms_norm_case(rows=37, cols=1024, seed=1)
+    ours, want, compiled = run_case(case, device)
+    assert [n.op.knobs["REDUCE"] for n in compiled.nodes.values() if isinstance(n.op, HipOp)] == [coop]
+    eager.assert_close(ours, want, case.rtol, case.atol, f"rms_norm {coop}")
+
+
+def test_reference_recipe_rms_sum_variant(device, golden):
+    """``x * rsqrt(sum(x^2) + eps) * w`` — the graph the reference's own e2e tests build
+    (tests/compiler/e2e/test_accuracy.py:184-212), as a hand-written tile."""
+    x = E.Var("x")
+    body = RowReduce(rows=8, cols=64, x="X", x_dtype=F32, out="out", out_dtype=F32, stats=(Stat("ss", "sum", x * x),),
+                     project=x * E.Un("rsqrt", E.Var("ss") + 1e-6) * E.Var("w"), col_operands=(("w", F32),), reduce=ReducePlan(coop=16))  # fmt: skip
+    g = Graph()
+    g.add_input("X", (8, 64))
+    g.add_input("w", (64,))
+    g.add_node(TileOp(name="k_rms_sum", body=body), ["X", "w"], Tensor("out", (8, 64), F32))
+    g.outputs = ["out"]
+    res, _ = HipBackend().run(lower(g), input_data={"X": golden["rms_sum_x"], "w": golden["rms_sum_w"]})
+    np.testing.assert_allclose(res.outputs["out"], golden["rms_sum_y"], rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(res.outputs["out"], O.rms_norm_sum(golden["rms_sum_x"], golden["rms_sum_w"], 1e-6), rtol=1e-5, atol=1e-7)
+
+
+# -- C2 ---------------------------------------------------------------------------
+
+
+def test_c2_softmax_full_size(device):
+    case = eager.softmax_case()
+    ours, want, _ = run_case(case, device)
+    eager.assert_close(ours, want, case.rtol, case.atol, "softmax vs eager (GPU)")
+    assert float((ours.double().sum(-1) - 1).abs().max()) < 1e-5  # rows sum to one
+    sl = (0, 3, slice(100, 164))
+    cpu = torch.softmax(case.inputs[0][sl], -1)
+    eager.assert_close(ours[sl], cpu, case.rtol, case.atol, "softmax slice vs eager (CPU)")
+
+
+@pytest.mark.parametrize("shape", [(4, 8), (4, 2048), (3, 5, 1000), (7, 7), (1, 2050), (130, 16384), (2, 3, 1)])
+def test_c2_softmax_ragged_and_small(device, shape, golden):
+    case = eager.softmax_case(shape=shape, seed=2)
+    ours, want, _ = run_case(case, device)
+    eager.assert_close(ours, want, case.rtol, case.atol, f"softmax {shape}")
+    eager.assert_close(ours, torch.from_numpy(O.softmax(case.inputs[0].numpy())).float(), case.rtol, case.atol, f"softmax {shape} vs numpy restatement")
+
+
+def test_c2_softmax_golden_and_extremes(device, golden):
+    for key in ("4x8", "4x2048"):
+        m = nn.Softmax(dim=-1)
+        x = torch.from_numpy(golden[f"softmax_{key}_x"])
+        ours, _, _ = run_case(eager.Case("g", m, (x,), 1e-5, 1e-9), device)
+        np.testing.assert_allclose(ours.cpu().numpy(), golden[f"softmax_{key}_y"], rtol=1e-5, atol=1e-9)
+    # large magnitudes and a fully dominated row stay finite and exact
+    x = torch.tensor([[1e4, 1e4 - 1, -1e4, 0.0] * 16, [-80.0] * 63 + [80.0]], dtype=torch.float32)
+    ours, want, _ = run_case(eager.Case("x", nn.Softmax(dim=-1), (x,), 1e-5, 1e-30), device)
+    eager.assert_close(ours, want, 1e-5, 1e-30, "softmax extremes")
+
+
+# -- C3 ---------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("m", [1, 16, 128, 2048])
+def test_c3_linear(device, m):
+    case = eager.linear_case(m=m)
+    ours, want, _ = run_case(case, device)
+    eager.assert_close(ours, want, case.rtol, case.atol, f"linear M={m} vs eager (GPU)")
+    # fp32-accumulated then rounded once: must sit within one bf16 ulp of the exact product
+    x, w = case.inputs[0][: min(m, 8)].double(), case.module.weight.detach().double().cpu()
+    exact = x @ w.T
+    eager.assert_close(ours[: min(m, 8)], exact, 2 ** -7, 1e-3, f"linear M={m} vs float64")
+
+
+@pytest.mark.parametrize(
+    "tile,stage",
+    [
+        ("a:mfma_32x32x16_bf16/w2x2/f2x3/k4", "d2/sync"),
+        ("a:mfma_32x32x16_bf16/w2x2/f2x3/k4", "d3/dl"),
+        ("a:mfma_32x32x16_bf16/w2x2/f2x3/k2", "d4/dl"),
+        ("a:mfma_16x16x32_bf16/w4x2/f2x6/k2", "d2/sync"),
+        ("a:mfma_16x16x32_bf16/w2x2/f2x2/k2", "d2/dl"),
+        ("a:mfma_32x32x16_bf16/w1x4/f2x1/k2", "d2/sync"),
+    ],
+)
+@pytest.mark.parametrize("shape", [(2048, 1024, 3072), (200, 128, 388), (129, 256, 72)])
+def test_c3_linear_every_tier(device, tile, stage, shape, monkeypatch):
+    monkeypatch.setenv("EMMY_TILE", tile)
+    monkeypatch.setenv("EMMY_STAGE", stage)
+    m, k, n = shape
+    case = eager.linear_case(m=m, k=k, n=n, seed=4)
+    ours, want, compiled = run_case(case, device)
+    knobs = [n_.op.knobs for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)][0]
+    assert knobs["TILE"] == tile
+    eager.assert_close(ours, want, case.rtol, case.atol, f"linear {shape} {tile} {stage}")
+
+
+def test_c3_golden(device, golden):
+    case = eager.linear_case(32, 128, 96)
+    ours, _, _ = run_case(case, device)
+    want = torch.from_numpy(golden["c3_y_bits"].view(np.int16).copy()).view(torch.bfloat16).float()
+    eager.assert_close(ours, want, 2e-2, 2e-2, "linear golden")
+
+
+# -- C4 ---------------------------------------------------------------------------
+
+
+def test_c4_sdpa_full_size(device):
+    case = eager.sdpa_case()
+    ours, want, _ = run_case(case, device)
+    eager.assert_close(ours, want, case.rtol, case.atol, "sdpa vs eager (GPU)")
+    q, k, v = (t.to(device).float() for t in case.inputs)
+    exact = nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+    eager.assert_close(ours, exact, case.rtol, case.atol, "sdpa vs fp32 eager")
+    # size-independent property: attention rows sum to one, so V = 1 gives O = 1
+    ones = eager.Case("ones", case.module, (case.inputs[0], case.inputs[1], torch.ones_like(case.inputs[2])), 2e-2, 2e-2)
+    o1, _, _ = run_case(ones, device)
+    assert float((o1.float() - 1).abs().max()) <= 2 ** -7
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("dims", [(1, 2, 1, 128, 128), (2, 4, 2, 200, 200), (1, 4, 4, 96, 160), (1, 6, 2, 33, 33), (1, 2, 2, 1, 70)])
+def test_c4_sdpa_shapes_against_streaming_restatement(device, causal, dims):
+    b, hq, hkv, sq, skv = dims
+    torch.manual_seed(6)
+    q = torch.randn(b, hq, sq, 128).bfloat16()
+    k = torch.randn(b, hkv, skv, 128).bfloat16()
+    v = torch.randn(b, hkv, skv, 128).bfloat16()
+    case = eager.Case("s", eager.Sdpa(causal), (q, k, v), 2e-2, 2e-2)
+    ours, want, _ = run_case(case, device)
+    eager.assert_close(ours, want, 2e-2, 2e-2, f"sdpa {dims} causal={causal} vs eager")
+    ref = O.flash_attention(q.float().numpy(), k.float().numpy(), v.float().numpy(), is_causal=causal, scale=128 ** -0.5, block_kv=64)
+    eager.assert_close(ours, torch.from_numpy(ref).float(), 2e-2, 2e-2, f"sdpa {dims} causal={causal} vs streaming restatement")
+
+
+def test_c4_golden(device, golden):
+    ours, _, _ = run_case(eager.sdpa_case(1, 4, 2, 96, 128), device)
+    want = torch.from_numpy(golden["c4_y_bits"].view(np.int16).copy()).view(torch.bfloat16).float()
+    eager.assert_close(ours, want, 2e-2, 2e-2, "sdpa golden")
+
+
+# -- C5 ---------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("seq", [32, 64, 512])
+def test_c5_qwen3_block(device, seq, golden):
+    case = eager.qwen3_block_case(seq=seq)
+    ours, want, compiled = run_case(case, device)
+    eager.assert_close(ours, want, case.rtol, case.atol, f"block S={seq} vs eager (GPU)")
+    assert sum(isinstance(n.op, HipOp) for n in compiled.nodes.values()) == 11
+    if seq == 32:
+        gold = torch.from_numpy(golden["c5_y_bits"].view(np.int16).copy()).view(torch.bfloat16).float()
+        eager.assert_close(ours, gold.reshape(ours.shape), case.rtol, case.atol, "block golden (CPU eager bf16)")
+        eager.assert_close(ours, torch.from_numpy(golden["c5_y_f32"]).reshape(ours.shape), 2e-2, 6e-2, "block vs fp32 eager")
+
+
+def test_run_api_returns_host_arrays_with_bf16_as_bits(device):
+    case = eager.linear_case(m=16)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    marker = []
+    res, pre = be.run(compiled, input_data={compiled.inputs[0]: case.inputs[0].view(torch.int16).numpy().view(np.uint16)}, pre_run=lambda: marker.append(1) or "pre")
+    assert pre == "pre" and marker == [1]
+    out = res.outputs[compiled.outputs[0]]
+    assert out.dtype == np.uint16 and out.shape == (16, 3072)
+    want = eager.run_eager(case, device).float().cpu()
+    eager.assert_close(torch.from_numpy(O.from_bf16_bits(out)), want, 2e-2, 2e-2, "run() output")

@@ -1,0 +1,133 @@
+"""Runtime behaviour on the device: graph replays, event timing, the watchdog,
+zeroed accumulation targets — all through the C-ABI library."""
+
+from __future__ import annotations
+
+import asyncio
+
+import numpy as np
+import pytest
+import torch
+
+from deplodock_amd import HipBackend, trace_module
+from deplodock_amd.backend.hip import launcher, program
+from deplodock_amd.dtype import F32
+from deplodock_amd.graph import Graph, Tensor
+from deplodock_amd.ir.hip import HipOp
+from oracle import eager
+
+pytestmark = pytest.mark.gpu
+
+
+def test_device_is_gfx950(launcher_lib, device):
+    props = launcher_lib.device_props(0)
+    assert props["arch"].startswith("gfx950") and props["wavefront_size"] == 64 and props["compute_units"] == 256
+
+
+def test_graph_replays_match_eager_every_time(device):
+    """A captured whole-program graph is replayed several times with eager work and
+    synchronisations in between; every replay must reproduce the eager result."""
+    case = eager.qwen3_block_case(seq=64)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    want = eager.run_eager(case, device)
+    prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, case.inputs)})
+    try:
+        out = prog.output_tensors()[compiled.outputs[0]]
+        prog.capture_program_graph()
+        for i in range(4):
+            out.zero_()
+            torch.cuda.synchronize()
+            prog.replay_program()
+            prog.lib.stream_synchronize(prog._ensure_stream())
+            eager.assert_close(out.reshape(want.shape), want, case.rtol, case.atol, f"replay {i}")
+            _ = (torch.randn(256, 256, device=device) @ torch.randn(256, 256, device=device)).sum().item()  # eager work between replays
+    finally:
+        prog.close()
+
+
+def test_zero_outputs_are_cleared_before_each_launch_also_in_graphs(device):
+    src = 'extern "C" __global__ void k_acc(const float* x, float* y) { atomicAdd(&y[threadIdx.x % 4], x[threadIdx.x]); }'
+    g = Graph()
+    g.add_input("x", (64,), F32)
+    op = HipOp(kernel_source=src, kernel_name="k_acc", arg_order=("x", "y"), grid=((1,), (1,), (1,)), block=((64,), (1,), (1,)), zero_outputs=("y",))
+    g.add_node(op, ["x"], Tensor("y", (4,), F32), "y")
+    g.outputs = ["y"]
+    x = torch.arange(64, dtype=torch.float32)
+    want = x.reshape(16, 4).sum(0)
+    prog = program.CompiledProgram.build(g, {"x": x})
+    try:
+        for _ in range(3):
+            prog.run()
+        torch.cuda.synchronize()
+        torch.testing.assert_close(prog.output_tensors()["y"].cpu(), want)
+        prog.capture_program_graph()
+        for _ in range(3):
+            prog.replay_program()
+            prog.lib.stream_synchronize(prog._ensure_stream())
+            torch.testing.assert_close(prog.output_tensors()["y"].cpu(), want)
+    finally:
+        prog.close()
+
+
+def test_benchmark_reports_event_times_and_e2e(device):
+    case = eager.qwen3_block_case(seq=64)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    calls = []
+    res = asyncio.run(be.benchmark_async(compiled, warmup=2, num_iters=5, on_iter=lambda b: calls.append(b)))
+    assert res.num_launches == 11 and len(res.per_launch) == 11 and res.captured
+    assert all(p.time_ms > 0 and len(p.samples) == 5 for p in res.per_launch)
+    assert res.e2e_ms is not None and res.e2e_min_ms <= res.e2e_ms
+    assert 0 < res.min_ms <= res.time_ms <= res.max_ms
+    assert len(calls) >= 7 and all(b >= 1 for b in calls)
+    single = be.benchmark(be.compile(trace_module(*(lambda c: (c.module, c.inputs))(eager.rms_norm_case()))), warmup=1, num_iters=3)
+    assert single.e2e_ms is None and single.num_launches == 1  # the solo window is the program time
+
+
+def test_watchdog_raises_instead_of_stalling(device, monkeypatch):
+    """Forced from the host: with a negative budget the poll gives up while the
+    (perfectly healthy, ~150 us) kernel is still running; the kernel still finishes."""
+    case = eager.softmax_case()
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    prog = be.program(compiled, {compiled.inputs[0]: case.inputs[0].to(device)})
+    monkeypatch.setattr(program, "_KERNEL_TIMEOUT_MS", -1.0)
+    try:
+        with pytest.raises(program.HungKernelError):
+            prog.iter_once([64])
+    finally:
+        monkeypatch.undo()
+        prog.close()  # drains the stream: every wave exits normally
+    torch.cuda.synchronize()
+
+
+def test_run_budget_marks_bench_fail(device):
+    case = eager.softmax_case(shape=(64, 2048))
+    be = HipBackend(bench_run_timeout_s=1e-9)
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    with pytest.raises(RuntimeError, match="bench_fail"):
+        be.benchmark(compiled, warmup=1, num_iters=3)
+
+
+def test_misaligned_device_tensor_is_rejected(device):
+    case = eager.rms_norm_case(rows=4, cols=64)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    base = torch.randn(4 * 64 + 1, device=device)
+    with pytest.raises(ValueError, match="16-byte aligned"):
+        be.program(compiled, {compiled.inputs[0]: base[1:].reshape(1, 4, 64)})
+
+
+def test_launch_errors_surface_as_exceptions(launcher_lib, device):
+    from deplodock_amd.backend.hip import hiprtc
+    from deplodock_amd.backend.hip.launcher import PackedArgs
+
+    k = hiprtc.load_function('extern "C" __global__ void k_one(float* x) { x[threadIdx.x] = 1.0f; }', "k_one")
+    buf = torch.zeros(64, device=device)
+    with pytest.raises(launcher.LauncherError, match="1024"):
+        launcher_lib.launch(k.fn, (1, 1, 1), (2048, 1, 1), 0, None, PackedArgs([buf.data_ptr()]))
+    launcher_lib.launch(k.fn, (1, 1, 1), (64, 1, 1), 0, None, PackedArgs([buf.data_ptr()]))
+    torch.cuda.synchronize()
+    assert float(buf.sum()) == 64.0
+    np.testing.assert_equal(launcher_lib.func_attributes(k.fn)["private_bytes"], 0)

@@ -1,0 +1,135 @@
+"""Compile-only checks (no GPU): tracing, kernel boundaries, knob pins, source structure,
+and hipRTC cross-compilation of every kernel the five configurations need."""
+
+from __future__ import annotations
+
+import re
+
+import pytest
+import torch
+from torch import nn
+
+from deplodock_amd import HipBackend, trace_module
+from deplodock_amd.backend.hip import hiprtc
+from deplodock_amd.ir.hip import HipOp
+from oracle import eager
+
+
+def kernels(compiled):
+    return [compiled.nodes[n].op for n in compiled.topological_order() if isinstance(compiled.nodes[n].op, HipOp)]
+
+
+def compile_case(case):
+    return HipBackend().compile(trace_module(case.module, case.inputs))
+
+
+def test_rms_norm_is_one_fused_reduce_kernel(launcher_lib):
+    ks = kernels(compile_case(eager.rms_norm_case()))
+    assert len(ks) == 1
+    k = ks[0]
+    assert re.fullmatch(r"k_rms_norm_reduce_[0-9a-f]{6}", k.kernel_name)
+    assert k.knobs["REDUCE"] == "b256" and k.grid[0] == (32,) and k.block[0] == (256,)
+    src = k.kernel_source
+    assert "emh_wave_reduce<EmhSum, 64>" in src and "rsqrtf" in src
+    assert "__shfl" not in src  # wave combine is DPP / swizzle, not a bpermute butterfly
+    assert src.count("__syncthreads") == 1  # one LDS hand-off for the 4 waves of a row, no tree
+    assert k.algo_bytes == 532480
+    hiprtc.compile_to_hsaco(src, k.kernel_name)
+
+
+def test_softmax_is_one_kernel_with_row_resident_single_read(launcher_lib):
+    ks = kernels(compile_case(eager.softmax_case()))
+    assert len(ks) == 1
+    k = ks[0]
+    assert k.kernel_name.startswith("k_softmax_reduce_")
+    assert k.algo_bytes == 939524096
+    src = k.kernel_source
+    assert src.count("expf(") == len(re.findall(r"xv\[\d+\]\[\d+\] = expf", src))  # exp evaluated once per element, kept resident
+    assert "EmhMax" in src and "EmhSum" in src
+    hiprtc.compile_to_hsaco(src, k.kernel_name)
+
+
+@pytest.mark.parametrize("m", [1, 16, 128, 2048])
+def test_linear_is_one_mfma_kernel(launcher_lib, m):
+    ks = kernels(compile_case(eager.linear_case(m=m)))
+    assert len(ks) == 1
+    k = ks[0]
+    assert k.kernel_name.startswith("k_linear_")
+    assert "__builtin_amdgcn_mfma_f32_" in k.kernel_source
+    assert k.algo_flops == 2 * m * 3072 * 1024
+    hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+
+
+def test_sdpa_is_one_flash_kernel(launcher_lib):
+    ks = kernels(compile_case(eager.sdpa_case()))
+    assert len(ks) == 1
+    k = ks[0]
+    assert k.kernel_name.startswith("k_sdpa_reduce_")
+    assert k.algo_flops == 17188257792
+    assert "#define GROUP 2" in k.kernel_source and "#define CAUSAL 1" in k.kernel_source
+    assert "flash_pv_smem" not in k.kernel_source  # P stays in registers
+    hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+
+
+def test_qwen3_block_kernel_boundaries(launcher_lib):
+    compiled = compile_case(eager.qwen3_block_case(seq=64))
+    names = [re.sub(r"_[0-9a-f]{6}$", "", k.kernel_name) for k in kernels(compiled)]
+    assert names == [
+        "k_rms_norm_reduce", "k_linear", "k_rms_norm_rope", "k_linear", "k_rms_norm_rope", "k_linear",
+        "k_sdpa_reduce", "k_linear_add", "k_rms_norm_reduce", "k_linear_silu_mul", "k_linear_add",
+    ]  # fmt: skip
+    for k in kernels(compiled):
+        hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+    # layout ops produced no kernels and no buffers
+    assert not any("transpose" in n or "view" in n or "slice" in n for n in compiled.nodes)
+    # the gate and up weights are stacked into one constant the runtime assembles
+    stacked = [n for n in compiled.nodes.values() if n.hints.get("stacked")]
+    assert len(stacked) == 1 and stacked[0].output.shape == (6144, 1024)
+    data = HipBackend.bind(compiled, {})
+    assert data[stacked[0].id].shape == (6144, 1024)
+
+
+def test_reduce_pin_is_authoritative_and_bad_pin_degrades(launcher_lib, monkeypatch):
+    case = eager.rms_norm_case()
+    monkeypatch.setenv("EMMY_REDUCE", "b64")
+    k = kernels(compile_case(case))[0]
+    assert k.knobs["REDUCE"] == "b64" and k.block[0] == (256,) and k.grid[0] == (8,)
+    assert "__syncthreads" not in k.kernel_source  # one wave per row: no LDS at all
+    monkeypatch.setenv("EMMY_REDUCE", "b100")
+    assert kernels(compile_case(case))[0].knobs["REDUCE"] == "b256"  # resolved spelling is stamped
+    monkeypatch.setenv("EMMY_REDUCE", "b16")  # 2048 columns over 16 lanes cannot stay register-resident
+    assert kernels(compile_case(case))[0].knobs["REDUCE"] == "b256"
+
+
+def test_tile_and_stage_pins(launcher_lib, monkeypatch):
+    case = eager.linear_case()
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x2/f2x3/k4")
+    monkeypatch.setenv("EMMY_STAGE", "d3/cp")
+    k = kernels(compile_case(case))[0]
+    assert k.knobs["TILE"] == "a:mfma_32x32x16_bf16/w2x2/f2x3/k4" and k.knobs["STAGE"] == "d3/dl"
+    assert "__builtin_amdgcn_global_load_lds" in k.kernel_source and k.lds_bytes == 3 * (128 + 192) * 64 * 2
+    assert k.grid[0] == (256,)
+    hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+    monkeypatch.setenv("EMMY_TILE", "a:mma_m16n8k16_bf16/w2x2/f4x8/k2")  # an NVIDIA pin degrades to the gfx950 pick
+    monkeypatch.setenv("EMMY_STAGE", "d2/tma")
+    k = kernels(compile_case(case))[0]
+    assert "mfma" in k.knobs["TILE"] and k.knobs["STAGE"] == "d2/sync"
+
+
+def test_unsupported_op_raises_not_silently_falls_back():
+    class Weird(nn.Module):
+        def forward(self, x):
+            return torch.cumsum(x, -1)
+
+    with pytest.raises(NotImplementedError):
+        trace_module(Weird(), (torch.randn(4, 4),))
+
+
+def test_cache_is_content_addressed(launcher_lib, tmp_path, monkeypatch):
+    monkeypatch.setenv("EMMY_HSACO_CACHE", str(tmp_path))
+    src = 'extern "C" __global__ void k(float* x) { x[threadIdx.x] = 2.0f; }'
+    p1 = hiprtc.compile_to_hsaco(src, "k")
+    assert p1.parent == tmp_path and hiprtc.compile_to_hsaco(src, "k") == p1
+    monkeypatch.setenv("EMMY_HIPRTC_FLAGS", "-O1")
+    assert hiprtc.compile_to_hsaco(src, "k") != p1  # flags are part of the key
+    assert not list(tmp_path.glob("*.tmp"))

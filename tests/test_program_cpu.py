@@ -1,0 +1,66 @@
+"""Runtime contract checks that need no device: graph validation happens before
+anything is loaded (mirrors the hand-written-CudaOp tests of the reference,
+tests/compiler/backend/test_program.py:74-101)."""
+
+from __future__ import annotations
+
+import pytest
+
+from deplodock_amd.backend.hip import program
+from deplodock_amd.dtype import F32
+from deplodock_amd.graph import Graph, Tensor
+from deplodock_amd.ir.base import Op
+from deplodock_amd.ir.hip import HipOp
+
+SRC = 'extern "C" __global__ void k(const float* x, float* y) { y[threadIdx.x] = x[threadIdx.x]; }'
+
+
+def graph_with(ops):
+    g = Graph()
+    g.add_input("x", (64,), F32)
+    prev = "x"
+    for i, op in enumerate(ops):
+        nid = f"y{i}"
+        if isinstance(op, HipOp) and not op.arg_order:
+            op.arg_order = (prev, nid)
+        g.add_node(op, [prev], Tensor(nid, (64,), F32), nid)
+        prev = nid
+    g.outputs = [prev]
+    return g
+
+
+def test_non_hip_node_is_a_type_error():
+    with pytest.raises(TypeError, match="non-HipOp"):
+        program._compile(graph_with([Op()]))
+
+
+def test_duplicate_kernel_name_with_other_source_is_rejected():
+    a = HipOp(kernel_source=SRC, kernel_name="k", block=((64,), (1,), (1,)))
+    b = HipOp(kernel_source=SRC.replace("x[threadIdx.x]", "2.0f * x[threadIdx.x]"), kernel_name="k", block=((64,), (1,), (1,)))
+    with pytest.raises(ValueError, match="two distinct sources"):
+        program._compile(graph_with([a, b]))
+
+
+def test_unknown_buffer_is_rejected():
+    a = HipOp(kernel_source=SRC, kernel_name="k", arg_order=("x", "nope"))
+    with pytest.raises(KeyError, match="unknown buffer"):
+        program._compile(graph_with([a]))
+
+
+def test_batch_calibration_and_iter_budget():
+    assert program._calibrate_batch_sizes([0.002, 0.5, 3.0, 0.0]) == [500, 2, 1, 1]
+    assert program._resolve_iter_budget(20) == (float("inf"), 20, False)
+    assert program._resolve_iter_budget("auto")[2] is True
+    with pytest.raises(ValueError):
+        program._resolve_iter_budget("many")
+
+
+def test_no_device_means_a_loud_error_not_a_fallback():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a device is present")
+    from deplodock_amd.backend.hip.launcher import LauncherError
+
+    with pytest.raises(LauncherError, match="no CPU fallback"):
+        program._device()
