@@ -284,8 +284,13 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   // A plain s_barrier is used on purpose: a workgroup fence would drain every
   // outstanding direct-to-LDS load and serialise the pipeline.  Loads retire in
   // issue order, so "at most n outstanding" means the older slabs have landed.
+  // vmcnt reaching its target does not yet make direct-to-LDS data visible to
+  // other waves (measured: stale fragment reads right after the barrier); an LDS
+  // read of this wave queues behind its own DMA writes, so waiting for it orders
+  // them before the barrier.
   #define EMH_SLAB_SYNC(n) { \
     __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM_LGKM0(n)); \
+    { const unsigned d_ = *(volatile unsigned*)(emh_lds + tid * 4); asm volatile("s_waitcnt lgkmcnt(0)" :: "v"(d_) : "memory"); } \
     asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
   #pragma unroll
   for (int p = 0; p < DEPTH; ++p) if (p < KT) EMH_DLOAD(p, p);""")

@@ -20,14 +20,19 @@ kernel is laid out for CDNA4:
   the 16 keys of an MFMA step that is applied identically to the ``V`` operand
   (a contraction does not care in which order its terms are summed).  The
   reference round-trips ``P`` through shared memory (``flash_pv_smem``, _twist.py:324-330).
-* ``V`` stays ``[key][d]`` in LDS; the A operand is gathered with 8-byte reads of
-  four consecutive ``d`` and a register transpose, which assigns output rows
-  ``d = 4*m + T`` to MFMA tile ``T`` — again a fixed permutation, undone when
-  storing.
-* One workgroup = ``waves`` waves x 32 query rows; K/V blocks of 64 keys are
-  staged in LDS (K XOR-swizzled for conflict-free 16-byte fragment reads) and
-  prefetched through registers one block ahead.  Causal workgroups stop at the
-  diagonal and are launched heaviest-first.
+* ``V`` stays ``[key][d]`` in LDS; its operand fragments come from the gfx950
+  transposing LDS read (``ds_read_b64_tr_b16``): two reads per fragment, no
+  register shuffling.
+* One workgroup = ``waves`` groups of 32 query rows x ``kv_split`` wave groups that
+  share those rows and split the key blocks between them, so each SIMD hosts
+  several waves whose MFMA, LDS and softmax phases overlap in hardware; the
+  groups' ``(m, l, O)`` are merged through LDS at the end.  K/V blocks are staged
+  with direct-to-LDS loads one step ahead (K XOR-swizzled for conflict-free
+  16-byte fragment reads, V swizzled for the transposing reads).
+* The exponentials are taken against a reference maximum that is only raised
+  when a row outgrows it by 2^8, which makes the accumulator rescale rare; the
+  score scale is folded into the exponent's fma.  Causal workgroups stop at the
+  diagonal, mask only diagonal blocks, and are launched heaviest-first.
 """
 
 from __future__ import annotations
@@ -41,29 +46,40 @@ from deplodock_amd.ir.expr import float_literal
 from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.ir.tile import Flash
 
+# The key range of a workgroup's query rows is split over KVS wave groups.  Group g
+# owns key blocks g, g+KVS, ...; the groups hold the same query rows, so every
+# SIMD hosts KVS waves whose MFMA, LDS and softmax phases interleave in hardware.
+# Each group keeps its own (m, l, O); they are merged through LDS at the end with
+# the same exp-family combine the streaming loop uses.  KVS = 1 is the plain form.
 _SRC = r"""
 EMH_DEV int emh_kswz(int row, int c) { return c ^ (row % CPR); }
+// V keeps [key][d] order; its 16-byte chunks are XOR-swizzled in groups of four
+// so the four consecutive key rows one transposing read touches sit in four
+// different bank quarters.
+EMH_DEV int emh_vswz(int row, int c) { return c ^ ((row % 4) << 2); }
 EMH_DEV float emh_xor32(float v) { return __shfl_xor(v, 32, 64); }
+typedef short emh_s16x4 __attribute__((ext_vector_type(4)));
+#define KBYTES (BKV * D * 2)
+#define WQ (NT / 64 / KVS)           /* waves (32-row groups) per key-split group */
+#define STEP_BYTES (KVS * 2 * KBYTES)  /* one step: K and V block of every group */
 
 extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q, const ELT* __restrict__ Kp,
                                                       const ELT* __restrict__ Vp, ELT* __restrict__ Op) {
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * 2 * BKV * D * 2];  // [buf][K|V][key][d]
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // [2 buffers][group][K | V][key][d]
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int grp = wave / WQ, wq = wave % WQ;
   const int lq = lane % 32, lh = lane / 32;
-  // Heaviest (latest) query blocks first: causal work grows with the block index.
   const int qb = (QBLOCKS - 1) - (int)(blockIdx.x % QBLOCKS);
   const int head = (blockIdx.x / QBLOCKS) % HQ;
   const int batch = blockIdx.x / (QBLOCKS * HQ);
   const int kvh = head / GROUP;
-  const int q0 = qb * BQ;            // first query row of the workgroup
-  const int qw0 = q0 + wave * 32;    // first query row of this wave
-  const int qrow = qw0 + lq;         // this lane's query row
+  const int q0 = qb * BQ;
+  const int qw0 = q0 + wq * 32;
+  const int qrow = qw0 + lq;
   const ELT* qbase = Q + Q_OFF + (long)batch * Q_SB + (long)head * Q_SH;
   const ELT* kbase = Kp + K_OFF + (long)batch * K_SB + (long)kvh * K_SH;
   const ELT* vbase = Vp + V_OFF + (long)batch * V_SB + (long)kvh * V_SH;
 
-  // Q fragments (B operand of S^T = K Q^T): lane (q = l%32, h = l/32) holds
-  // q[qrow][16*kk + 8*h .. +8] for every k-step kk.
   FRAG qf[D / 16];
   {
     const int qr = qrow < SQ ? qrow : SQ - 1;
@@ -71,102 +87,131 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
     #pragma unroll
     for (int kk = 0; kk < D / 16; ++kk) qf[kk] = *(const FRAG*)(qp + 16 * kk);
   }
-
-  // Number of key blocks this workgroup visits.
   int ntiles = (SKV + BKV - 1) / BKV;
   if (CAUSAL) {
-    const int lim = (q0 + BQ - 1 < SQ - 1 ? q0 + BQ - 1 : SQ - 1) / BKV + 1;  // last block touching the diagonal
+    const int lim = (q0 + BQ - 1 < SQ - 1 ? q0 + BQ - 1 : SQ - 1) / BKV + 1;
     if (lim < ntiles) ntiles = lim;
   }
+  const int nsteps = (ntiles + KVS - 1) / KVS;
 
-  // Staging: K and V blocks are BKV x D elements = BKV*D/8 16-byte chunks each.
-  constexpr int CHUNKS = BKV * D / 8;
-  constexpr int PER_T = CHUNKS / NT;
-  u32x4 rk[PER_T], rv[PER_T];
-  #define EMH_GLOAD(jt) { \
+  // Direct-to-LDS staging.  A step holds KVS key blocks; their K and V chunks
+  // (16 bytes each) are dealt over all threads.  Every wave-level load fills 64
+  // consecutive LDS slots, so for K the XOR swizzle is applied by choosing which
+  // global chunk each lane fetches.
+  constexpr int CHUNKS = BKV * D / 8;          // per block, per operand
+  constexpr int PER_T = KVS * CHUNKS / NT;     // chunks per thread, per operand
+  // Chunk q = tid + i*NT of a step: block g = q / CHUNKS, row (q % CHUNKS) / CPR,
+  // slot q % CPR = tid % CPR.  CHUNKS is a multiple of NT, so g and the row offset
+  // of iteration i are compile-time; with 256 or more threads the row offset is a
+  // multiple of 16 and the swizzled chunk choice is the same for every i.
+  const int st_row = tid / CPR, st_pos = tid % CPR;
+  const ELT* gk_lane = kbase + (long)st_row * K_SS;
+  const ELT* gv_lane = vbase + (long)st_row * V_SS;
+  const int dst_lane = (tid - lane) * 16;
+  #define EMH_STAGE(st, buf) { \
+    unsigned char* sb_ = lds + (buf) * STEP_BYTES + dst_lane; \
     _Pragma("unroll") for (int i = 0; i < PER_T; ++i) { \
-      const int q_ = tid + i * NT; const int row_ = q_ / CPR, c_ = q_ % CPR; \
-      int kr_ = (jt) * BKV + row_; if (kr_ > SKV - 1) kr_ = SKV - 1; \
-      rk[i] = *(const u32x4*)(kbase + (long)kr_ * K_SS + c_ * 8); \
-      rv[i] = *(const u32x4*)(vbase + (long)kr_ * V_SS + c_ * 8); } }
-  #define EMH_LSTORE(buf) { \
-    unsigned char* sk_ = lds + (buf) * (2 * BKV * D * 2); unsigned char* sv_ = sk_ + BKV * D * 2; \
-    _Pragma("unroll") for (int i = 0; i < PER_T; ++i) { \
-      const int q_ = tid + i * NT; const int row_ = q_ / CPR, c_ = q_ % CPR; \
-      *(u32x4*)(sk_ + row_ * (D * 2) + emh_kswz(row_, c_) * 16) = rk[i]; \
-      *(u32x4*)(sv_ + row_ * (D * 2) + c_ * 16) = rv[i]; } }
+      const int g_ = (i * NT) / CHUNKS, ro_ = ((i * NT) % CHUNKS) / CPR; \
+      long krow_ = (long)((st) * KVS + g_) * BKV + ro_; \
+      if (SKV % (KVS * BKV) != 0) { const long lim_ = SKV - 1 - st_row; if (krow_ > lim_) krow_ = lim_; } \
+      const int kc_ = emh_kswz(st_row + ro_ % CPR, st_pos), vc_ = emh_vswz(st_row + ro_ % 4, st_pos); \
+      unsigned char* dk_ = sb_ + g_ * 2 * KBYTES + ((i * NT) % CHUNKS) * 16; \
+      __builtin_amdgcn_global_load_lds((const void*)(gk_lane + krow_ * K_SS + kc_ * 8), (__attribute__((address_space(3))) void*)dk_, 16, 0, 0); \
+      __builtin_amdgcn_global_load_lds((const void*)(gv_lane + krow_ * V_SS + vc_ * 8), (__attribute__((address_space(3))) void*)(dk_ + KBYTES), 16, 0, 0); } }
+
+  // Publishing direct-to-LDS data: vmcnt reaching zero does not yet mean the
+  // data is visible to other waves' LDS reads (measured: stale reads right after
+  // the barrier).  An LDS read of this wave queues behind its own DMA writes, so
+  // waiting for that read orders them before the barrier.
+  #define EMH_DMA_FENCE() { \
+    __builtin_amdgcn_s_waitcnt(0x0070); /* vmcnt(0) lgkmcnt(0) */ \
+    const unsigned d_ = *(volatile unsigned*)(lds + tid * 4); \
+    asm volatile("s_waitcnt lgkmcnt(0)" :: "v"(d_) : "memory"); }
 
   f32x16 oacc[D / 32];
   #pragma unroll
   for (int t = 0; t < D / 32; ++t)
   #pragma unroll
   for (int r = 0; r < 16; ++r) oacc[t][r] = 0.0f;
-  float m_run = -1.0e30f, l_run = 0.0f;
+  float m_ref = -1.0e30f, l_run = 0.0f;
 
-  EMH_GLOAD(0);
-  EMH_LSTORE(0);
+  // ds_read_b64_tr_b16: within 16 lanes, lane i receives element (i % 4) of the
+  // 8-byte chunks addressed by lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12.  Lane i
+  // therefore points at key row (i / 4) and d-chunk 4*(i % 4) of its half tile,
+  // and receives four consecutive keys of its own d = 32*T + (l % 32): the V
+  // operand fragment of an MFMA step is two such reads and no shuffling.
+  const int i16 = lane % 16, q4 = i16 / 4;
+  const int v_lane = (4 * lh + q4) * (D * 2) + ((lane % 32) / 16) * 32 + (i16 % 4) * 8;
+  int v_tile[4];
+  #pragma unroll
+  for (int T = 0; T < 4; ++T) v_tile[T] = v_lane + ((T ^ q4) * 64);
+
+  EMH_STAGE(0, 0);
+  EMH_DMA_FENCE();
   __syncthreads();
 
-  for (int jt = 0; jt < ntiles; ++jt) {
-    const int cur = jt & 1;
-    if (jt + 1 < ntiles) EMH_GLOAD(jt + 1);
+  for (int st = 0; st < nsteps; ++st) {
+    if (st + 1 < nsteps) EMH_STAGE(st + 1, (st + 1) & 1);
+    const int jt = st * KVS + grp;
     const int k0 = jt * BKV;
-    // A wave whose rows all lie above this key block has nothing to add (causal).
-    const bool active = !CAUSAL || (k0 <= qw0 + 31);
+    const bool active = (jt < ntiles) && (!CAUSAL || (k0 <= qw0 + 31));
     if (active) {
-      const unsigned char* sK = lds + cur * (2 * BKV * D * 2);
-      const unsigned char* sV = sK + BKV * D * 2;
-      // ---- S^T = K Q^T for BKV/32 sub-blocks of 32 keys ----
+      const unsigned char* sK = lds + (st & 1) * STEP_BYTES + grp * 2 * KBYTES;
+      const unsigned char* sV = sK + KBYTES;
       f32x16 sacc[BKV / 32];
       #pragma unroll
       for (int u = 0; u < BKV / 32; ++u) {
         #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[u][r] = 0.0f;
+        // All fragments of a 32-key sub-block are fetched before its MFMAs, so the
+        // LDS latency is paid once per sub-block rather than once per MFMA pair.
         const int krow = u * 32 + lq;
+        FRAG kf[D / 16];
         #pragma unroll
-        for (int kk = 0; kk < D / 16; ++kk) {
-          const FRAG kf = *(const FRAG*)(sK + krow * (D * 2) + emh_kswz(krow, kk * 2 + lh) * 16);
-          sacc[u] = MFMA(kf, qf[kk], sacc[u], 0, 0, 0);
-        }
+        for (int kk = 0; kk < D / 16; ++kk) kf[kk] = *(const FRAG*)(sK + krow * (D * 2) + emh_kswz(krow, kk * 2 + lh) * 16);
+        __builtin_amdgcn_sched_barrier(0);
+        #pragma unroll
+        for (int kk = 0; kk < D / 16; ++kk) sacc[u] = MFMA(kf[kk], qf[kk], sacc[u], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      // ---- scale (log2 domain), mask, running max ----
-      // Register r of sub-block u is key k0 + 32u + 8*(r/4) + 4*lh + r%4 for query qrow.
-      const bool need_mask = (CAUSAL && (k0 + BKV - 1 > qw0)) || (k0 + BKV > SKV);
       float mx = -1.0e30f;
-      #pragma unroll
-      for (int u = 0; u < BKV / 32; ++u)
-      #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float s = sacc[u][r] * SCALE_LOG2;
-        if (need_mask) {
+      if ((CAUSAL && (k0 + BKV - 1 > qw0)) || (k0 + BKV > SKV)) {
+        #pragma unroll
+        for (int u = 0; u < BKV / 32; ++u)
+        #pragma unroll
+        for (int r = 0; r < 16; ++r) {
           const int key = k0 + 32 * u + 8 * (r / 4) + 4 * lh + (r % 4);
-          if ((CAUSAL && key > qrow) || key >= SKV) s = -1.0e30f;
+          if ((CAUSAL && key > qrow) || key >= SKV) sacc[u][r] = -1.0e30f;
+          mx = fmaxf(mx, sacc[u][r]);
         }
-        sacc[u][r] = s;
-        mx = fmaxf(mx, s);
+      } else {
+        #pragma unroll
+        for (int u = 0; u < BKV / 32; ++u)
+        #pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[u][r]);
       }
-      mx = fmaxf(mx, emh_xor32(mx));  // the other half of this query's keys lives in lane l^32
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = EXP2(m_run - m_new);
-      m_run = m_new;
+      mx *= SCALE_LOG2;
+      mx = fmaxf(mx, emh_xor32(mx));
+      if (__any(mx > m_ref + RESCALE_SLACK)) {
+        const float m_new = fmaxf(m_ref, mx);
+        const float alpha = EXP2(m_ref - m_new);
+        m_ref = m_new;
+        l_run *= alpha;
+        #pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+        #pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+      }
       float psum = 0.0f;
       #pragma unroll
       for (int u = 0; u < BKV / 32; ++u)
       #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float p = EXP2(sacc[u][r] - m_new);
+        const float p = EXP2(__builtin_fmaf(sacc[u][r], SCALE_LOG2, -m_ref));
         sacc[u][r] = p;
         psum += p;
       }
-      l_run = l_run * alpha + psum;  // per-lane partial over this lane's keys; halves meet at the end
-      #pragma unroll
-      for (int t = 0; t < D / 32; ++t)
-      #pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
-      // ---- O^T += V^T P^T ----
-      // MFMA step (u, s) contracts 16 keys.  Operand slot (h, t) of that step is
-      // key 32u + 16s + 4h + t (t < 4) or 32u + 16s + 8 + 4h + (t - 4): exactly the
-      // keys whose probabilities this lane already holds in sacc[u][8s .. 8s+7].
+      l_run += psum;
       #pragma unroll
       for (int u = 0; u < BKV / 32; ++u)
       #pragma unroll
@@ -174,54 +219,68 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         FRAG pf;
         #pragma unroll
         for (int t = 0; t < 8; ++t) pf[t] = (ELT)sacc[u][8 * s + t];
-        // Gather V: for each of the 8 keys, 4 consecutive d (= 4*lq .. 4*lq+3) per 32-wide tile group.
         #pragma unroll
-        for (int dg = 0; dg < D / 128 + (D % 128 ? 1 : 0); ++dg) {
-          u32x2 vr[8];
-          #pragma unroll
-          for (int t = 0; t < 8; ++t) {
-            const int key = 32 * u + 16 * s + 4 * lh + (t < 4 ? t : t + 4);
-            vr[t] = *(const u32x2*)(sV + key * (D * 2) + dg * 256 + lq * 8);
-          }
-          // Register transpose 8 keys x 4 d -> 4 fragments of 8 keys.
-          #pragma unroll
-          for (int T = 0; T < 4; ++T) {
-            if (dg * 4 + T >= D / 32) continue;
-            u32x4 av;
-            #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-              const unsigned lo = vr[2 * w][T / 2], hi = vr[2 * w + 1][T / 2];
-              av[w] = (T % 2 == 0) ? __builtin_amdgcn_perm(hi, lo, 0x05040100u) : __builtin_amdgcn_perm(hi, lo, 0x07060302u);
-            }
-            oacc[dg * 4 + T] = MFMA(__builtin_bit_cast(FRAG, av), pf, oacc[dg * 4 + T], 0, 0, 0);
-          }
+        for (int dg = 0; dg < D / 128; ++dg)
+        #pragma unroll
+        for (int T = 0; T < 4; ++T) {
+          const unsigned char* vp = sV + (32 * u + 16 * s) * (D * 2) + dg * 256 + v_tile[T];
+          const emh_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) emh_s16x4*)(vp));
+          const emh_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) emh_s16x4*)(vp + 8 * (D * 2)));
+          const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+          u32x4 av;
+          av[0] = l2[0]; av[1] = l2[1]; av[2] = h2[0]; av[3] = h2[1];
+          oacc[dg * 4 + T] = MFMA(__builtin_bit_cast(FRAG, av), pf, oacc[dg * 4 + T], 0, 0, 0);
         }
       }
     }
-    if (jt + 1 < ntiles) EMH_LSTORE((jt + 1) & 1);
+    EMH_DMA_FENCE();  // the next step's blocks (they had this whole step to land)
     __syncthreads();
   }
 
-  // ---- close: O / l, undo the d permutation, store ----
-  const float l_tot = l_run + emh_xor32(l_run);
-  const float inv = 1.0f / l_tot;
-  if (qrow < SQ) {
-    ELT* op = Op + O_OFF + (long)batch * O_SB + (long)head * O_SH + (long)qrow * O_SS;
-    // Tile T = 4*dg + Tl, register r = 4*i + j holds d = 128*dg + 4*(8*i + 4*lh + j) + Tl.
-    #pragma unroll
-    for (int dg = 0; dg < D / 128 + (D % 128 ? 1 : 0); ++dg)
-    #pragma unroll
-    for (int i = 0; i < 4; ++i)
-    #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      PACK4 y;
+  // ---- merge the key-split groups: group g > 0 parks (m, l, O) in LDS ----
+  float* park = (float*)lds;  // [wq][66][64 lanes]; the staging buffers are free after the last barrier
+  #pragma unroll 1
+  for (int g = 1; g < KVS; ++g) {
+    if (grp == g) {
+      float* pw = park + wq * (D / 32 * 16 + 2) * 64 + lane;
+      pw[0] = m_ref;
+      pw[64] = l_run;
       #pragma unroll
-      for (int Tl = 0; Tl < 4; ++Tl) {
-        const int T = dg * 4 + Tl;
-        y[Tl] = (T < D / 32) ? (ELT)(oacc[T < D / 32 ? T : 0][4 * i + j] * inv) : (ELT)0.0f;
+      for (int t = 0; t < D / 32; ++t)
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) pw[(2 + t * 16 + r) * 64] = oacc[t][r];
+    }
+    __syncthreads();
+    if (grp == 0) {
+      const float* pw = park + wq * (D / 32 * 16 + 2) * 64 + lane;
+      const float m_o = pw[0], l_o = pw[64];
+      const float m_new = fmaxf(m_ref, m_o);
+      const float a_s = EXP2(m_ref - m_new), a_o = EXP2(m_o - m_new);
+      m_ref = m_new;
+      l_run = l_run * a_s + l_o * a_o;
+      #pragma unroll
+      for (int t = 0; t < D / 32; ++t)
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[t][r] = oacc[t][r] * a_s + pw[(2 + t * 16 + r) * 64] * a_o;
+    }
+    __syncthreads();
+  }
+
+  if (grp == 0) {
+    const float l_tot = l_run + emh_xor32(l_run);
+    const float inv = 1.0f / l_tot;
+    if (qrow < SQ) {
+      ELT* op = Op + O_OFF + (long)batch * O_SB + (long)head * O_SH + (long)qrow * O_SS;
+      // Register r = 4*i + j of tile T is d = 32*T + 8*i + 4*lh + j.
+      #pragma unroll
+      for (int T = 0; T < D / 32; ++T)
+      #pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        PACK4 y;
+        #pragma unroll
+        for (int j = 0; j < 4; ++j) y[j] = (ELT)(oacc[T][4 * i + j] * inv);
+        *(PACK4*)(op + 32 * T + 8 * i + 4 * lh) = y;
       }
-      const int d = 128 * dg + 4 * (8 * i + 4 * lh + j);
-      if (d < D) *(PACK4*)(op + d) = y;
     }
   }
 }
@@ -237,16 +296,19 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     if body.q_heads % body.kv_heads:
         raise LoweringError("flash: q heads must be a multiple of kv heads")
     waves = body.waves
+    kvs = body.kv_split
     BQ = 32 * waves
     BKV = body.block_kv
     if BKV % 32 or BKV < 32:
         raise LoweringError("flash: key block must be a multiple of 32")
-    NT = waves * 64
+    NT = waves * kvs * 64
+    if NT > ctx.max_threads_per_block:
+        raise LoweringError(f"flash: {waves} x {kvs} waves exceed {ctx.max_threads_per_block} threads")
     if (BKV * D // 8) % NT:
-        raise LoweringError("flash: key block does not divide over the workgroup's threads")
-    lds = 2 * 2 * BKV * D * 2
-    if lds > ctx.static_lds_cap:
-        raise LoweringError(f"flash: {lds} B of LDS exceeds the static cap {ctx.static_lds_cap}")
+        raise LoweringError("flash: a key block's 16-byte chunks must be a multiple of the workgroup's threads")
+    lds = max(2 * kvs * 2 * BKV * D * 2, waves * (D // 32 * 16 + 2) * 64 * 4 if kvs > 1 else 0)
+    if lds > ctx.lds_bytes_per_cu:
+        raise LoweringError(f"flash: {lds} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
     for st in (body.q_strides, body.k_strides, body.v_strides):
         if st[2] % 8:
             raise LoweringError("flash: sequence strides must keep 16-byte row alignment")
@@ -260,6 +322,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "D": D,
         "BQ": BQ,
         "BKV": BKV,
+        "KVS": kvs,
         "CPR": D // 8,
         "SQ": body.q_len,
         "SKV": body.kv_len,
@@ -279,6 +342,9 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         # 2^x straight on the transcendental unit; inputs are <= 0 and the result
         # feeds a 16-bit operand, so the fast form loses nothing that survives.
         "EXP2": "__builtin_amdgcn_exp2f",
+        # log2-domain slack before the accumulators are rescaled to a new maximum:
+        # probabilities stay below 2^8, far inside fp32 / bf16 range.
+        "RESCALE_SLACK": "8.0f",
     }  # fmt: skip
     head = f"// {name}: B={body.batch} Hq={body.q_heads} Hkv={body.kv_heads} Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal}\n"
     head += "".join(f"#define {k} {v}\n" for k, v in defs.items())
@@ -290,9 +356,9 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         arg_order=(body.q, body.k, body.v, body.out),
         grid=((grid,), (1,), (1,)),
         block=((NT,), (1,), (1,)),
-        lds_bytes=0,
+        lds_bytes=lds,
         comment=f"flash Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} bkv={BKV}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
-        knobs={"FLASH": f"w{waves}/kv{BKV}"},
+        knobs={"FLASH": f"w{waves}/kv{BKV}" + (f"/s{kvs}" if kvs > 1 else "")},
     )

@@ -197,7 +197,8 @@ class Flash:
     o_offset: int = 0
     block_q: int = 128
     block_kv: int = 64
-    waves: int = 4
+    waves: int = 4  # 32-row query groups per workgroup
+    kv_split: int = 1  # wave groups that split the key blocks of a query group between them
 
     def algo_flops(self) -> int:
         if self.causal and self.q_len == self.kv_len:

@@ -190,6 +190,28 @@ def test_c4_sdpa_shapes_against_streaming_restatement(device, causal, dims):
     eager.assert_close(ours, torch.from_numpy(ref).float(), 2e-2, 2e-2, f"sdpa {dims} causal={causal} vs streaming restatement")
 
 
+@pytest.mark.parametrize("pin", ["w4/kv64/s1", "w4/kv64/s2", "w2/kv64/s2", "w4/kv32/s2", "w1/kv32/s4", "w2/kv64/s4"])
+def test_c4_every_workgroup_shape(device, pin, monkeypatch):
+    """Key-split groups, direct-to-LDS staging and the final (m, l, O) merge: the first
+    key blocks are consumed right after they are staged, so every launch is checked."""
+    monkeypatch.setenv("EMMY_FLASH", pin)
+    case = eager.sdpa_case(b=1, hq=8, hkv=4, s=320, d=128, seed=9)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    assert [n.op.knobs["FLASH"] for n in compiled.nodes.values() if isinstance(n.op, HipOp)] == [pin]
+    want = eager.run_eager(case, device)
+    prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, case.inputs)})
+    try:
+        out = prog.output_tensors()[compiled.outputs[0]]
+        for rep in range(10):
+            out.zero_()
+            prog.run()
+            torch.cuda.synchronize()
+            eager.assert_close(out.reshape(want.shape), want, case.rtol, case.atol, f"sdpa {pin} launch {rep}")
+    finally:
+        prog.close()
+
+
 def test_c4_golden(device, golden):
     ours, _, _ = run_case(eager.sdpa_case(1, 4, 2, 96, 128), device)
     want = torch.from_numpy(golden["c4_y_bits"].view(np.int16).copy()).view(torch.bfloat16).float()
