@@ -360,5 +360,5 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         comment=f"flash Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} bkv={BKV}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
-        knobs={"FLASH": f"w{waves}/kv{BKV}" + (f"/s{kvs}" if kvs > 1 else "")},
+        knobs={"FLASH": f"w{waves}/kv{BKV}/s{kvs}"},
     )

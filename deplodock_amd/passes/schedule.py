@@ -194,6 +194,8 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
             chunks = body.block_kv * body.head_dim // 8
             if body.waves < 1 or body.kv_split < 1 or body.block_kv % 32 or chunks % (body.waves * body.kv_split * 64):
                 raise ScheduleError("unrealisable workgroup shape")
+            if 2 * body.kv_split * 2 * body.block_kv * body.head_dim * 2 > ctx.lds_bytes_per_cu:
+                raise ScheduleError("the double-buffered K/V blocks of all key-split groups exceed the LDS")
         except (ValueError, ScheduleError) as exc:
             logger.warning("EMMY_FLASH=%r ignored: %s", pinned, exc)
             pinned = None

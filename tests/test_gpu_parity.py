@@ -190,7 +190,7 @@ def test_c4_sdpa_shapes_against_streaming_restatement(device, causal, dims):
     eager.assert_close(ours, torch.from_numpy(ref).float(), 2e-2, 2e-2, f"sdpa {dims} causal={causal} vs streaming restatement")
 
 
-@pytest.mark.parametrize("pin", ["w4/kv64/s1", "w4/kv64/s2", "w2/kv64/s2", "w4/kv32/s2", "w1/kv32/s4", "w2/kv64/s4"])
+@pytest.mark.parametrize("pin", ["w4/kv64/s1", "w4/kv64/s2", "w2/kv64/s2", "w4/kv32/s2", "w1/kv32/s4", "w2/kv32/s4"])
 def test_c4_every_workgroup_shape(device, pin, monkeypatch):
     """Key-split groups, direct-to-LDS staging and the final (m, l, O) merge: the first
     key blocks are consumed right after they are staged, so every launch is checked."""

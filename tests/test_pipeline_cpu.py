@@ -116,6 +116,20 @@ def test_tile_and_stage_pins(launcher_lib, monkeypatch):
     assert "mfma" in k.knobs["TILE"] and k.knobs["STAGE"] == "d2/sync"
 
 
+def test_flash_pin_grammar_and_degrade(launcher_lib, monkeypatch):
+    case = eager.sdpa_case(1, 8, 4, 320, 128)
+    default = kernels(compile_case(case))[0].knobs["FLASH"]
+    assert default == "w1/kv64/s2"  # few heads, short sequence: one 32-row group per workgroup to cover the CUs
+    assert kernels(compile_case(eager.sdpa_case()))[0].knobs["FLASH"] == "w4/kv64/s2"
+    monkeypatch.setenv("EMMY_FLASH", "w2/kv32/s4")
+    k = kernels(compile_case(case))[0]
+    assert k.knobs["FLASH"] == "w2/kv32/s4" and k.block[0] == (512,) and k.lds_bytes == 2 * 4 * 2 * 32 * 128 * 2
+    monkeypatch.setenv("EMMY_FLASH", "w2/kv64/s4")  # 256 KiB of staging does not fit: degrade to the default pick
+    assert kernels(compile_case(case))[0].knobs["FLASH"] == default
+    monkeypatch.setenv("EMMY_FLASH", "w3/zz")
+    assert kernels(compile_case(case))[0].knobs["FLASH"] == default
+
+
 def test_unsupported_op_raises_not_silently_falls_back():
     class Weird(nn.Module):
         def forward(self, x):
