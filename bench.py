@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the emitted-kernel hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-table] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-table] [--no-cpu] [--only TEXT]
 
 A *step* is one pass of the headline kernel — the emitted ``nn.Softmax(-1)``
 row reduction over fp32 ``[1, 28, 2048, 2048]`` (the configuration the
@@ -114,7 +114,7 @@ def _cpu_baseline() -> dict:
     }
 
 
-def _table(device) -> list[dict]:
+def _table(device, only: str | None = None) -> list[dict]:
     """Per-kernel µs / achieved rate / fraction of peak for every configuration."""
     import torch
 
@@ -124,7 +124,10 @@ def _table(device) -> list[dict]:
     be = HipBackend(device_id=0)
     rows: list[dict] = []
 
-    def bench(case, label: str, bound: str, check: bool = True) -> None:
+    def bench(make_case, label: str, bound: str, check: bool = True) -> None:
+        if only is not None and only not in label:
+            return
+        case = make_case()
         compiled = be.compile(trace_module(case.module, case.inputs))
         data = {n: t.to(device) for n, t in zip(compiled.inputs, case.inputs)}
         if check:
@@ -151,14 +154,14 @@ def _table(device) -> list[dict]:
             row.update(bound="mfma", achieved=round(tf, 1), unit="TFLOP/s", frac=round(tf / MFMA_BF16_PEAK_TFLOPS, 4))
         rows.append(row)
 
-    bench(eager.rms_norm_case(), "C1 rms_norm fp32 [1,32,2048]", "hbm")
-    bench(eager.rms_norm_case(rows=32768), "C1x rms_norm fp32 [1,32768,2048]", "hbm")
-    bench(eager.softmax_case(), "C2 softmax fp32 [1,28,2048,2048]", "hbm")
+    bench(eager.rms_norm_case, "C1 rms_norm fp32 [1,32,2048]", "hbm")
+    bench(lambda: eager.rms_norm_case(rows=32768), "C1x rms_norm fp32 [1,32768,2048]", "hbm")
+    bench(eager.softmax_case, "C2 softmax fp32 [1,28,2048,2048]", "hbm")
     for m in (1, 16, 128):
-        bench(eager.linear_case(m=m), f"C3 linear bf16 M={m} K=1024 N=3072", "hbm")
-    bench(eager.linear_case(m=2048), "C3 linear bf16 M=2048 K=1024 N=3072", "mfma")
-    bench(eager.sdpa_case(), "C4 causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
-    bench(eager.qwen3_block_case(seq=512), "C5 qwen3-0.6B block bf16 S=512", "mfma")
+        bench(lambda m=m: eager.linear_case(m=m), f"C3 linear bf16 M={m} K=1024 N=3072", "hbm")
+    bench(lambda: eager.linear_case(m=2048), "C3 linear bf16 M=2048 K=1024 N=3072", "mfma")
+    bench(eager.sdpa_case, "C4 causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
+    bench(lambda: eager.qwen3_block_case(seq=512), "C5 qwen3-0.6B block bf16 S=512", "mfma")
     return rows
 
 
@@ -169,6 +172,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-table", action="store_true", help="skip the per-configuration kernel table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--only", default=None, metavar="TEXT", help="restrict the kernel table to configurations whose label contains TEXT (e.g. 'M=2048', 'C4')")
     ap.add_argument("--copy-probe", action="store_true", help="also run a plain 469762048-byte device copy 5 times (counter calibration under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -219,7 +223,7 @@ def main() -> int:
     }
     out["cpu_baseline"] = None if args.no_cpu else _cpu_baseline()
     if not args.no_table:
-        out["kernels"] = _table(device)
+        out["kernels"] = _table(device, args.only)
     print(json.dumps(out))
     return 0
 

@@ -1,0 +1,202 @@
+"""``run``: compile an inline expression, execute it on the GPU, check it
+against eager PyTorch on the same device, and (``--bench``) time both.
+
+The shape of the reference's ``emmy run [--bench] --code`` (emmy/commands/run.py:
+137-260 for the flow, :1423-1500 for the accuracy verdict, :470-603 and
+:1718-1728 for the two tables).  The accuracy gate here is the tighter one this
+backend is held to: fp32 within rtol 1e-5 (absolute floor 1e-5 of the output's
+peak), bf16/fp16 within rtol 2e-2.
+"""
+
+from __future__ import annotations
+
+import statistics
+import sys
+from pathlib import Path
+
+from deplodock_amd.commands.compile import add_common_args, apply_common_args, trace_from_args
+from deplodock_amd.commands.table import render_table
+
+HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+TOLERANCES = {"float32": (1e-5, 1e-5), "bfloat16": (2e-2, 2e-2), "float16": (2e-2, 2e-2)}
+
+
+def register_run_command(subparsers) -> None:
+    p = subparsers.add_parser("run", help="Compile + run an inline torch expression on the MI355X backend")
+    add_common_args(p)
+    p.add_argument("--bench", "-b", action="store_true", help="Time eager PyTorch and the emitted kernels and print a comparison table.")
+    p.add_argument("--warmup", type=int, default=10, help="Warmup iterations for --bench (default: 10).")
+    p.add_argument("--iters", type=int, default=100, help="Measurement iterations for --bench (default: 100).")
+    p.add_argument("--ab", action="append", default=None, metavar="KNOBS", help="Also compile + bench a variant with these knobs pinned ('K1=V1,K2=V2'); repeatable; needs --bench.")
+    p.set_defaults(func=handle_run)
+
+
+def check_accuracy(ours, want) -> tuple[bool, str]:
+    """Compare one output with eager's; ``(ok, one-line verdict)``."""
+    import torch
+
+    rtol, atol_rel = TOLERANCES.get(str(want.dtype).replace("torch.", ""), (1e-5, 1e-5))
+    a = ours.reshape(want.shape).to(torch.float64)
+    b = want.to(torch.float64)
+    peak = float(b.abs().max()) if b.numel() else 0.0
+    atol = atol_rel * max(peak, 1.0)
+    err = (a - b).abs()
+    bad = err > (atol + rtol * b.abs())
+    finite = bool(torch.isfinite(a).all()) or not bool(torch.isfinite(b).all())
+    max_err = float(err.max()) if err.numel() else 0.0
+    ok = finite and not bool(bad.any())
+    return ok, f"max |err| {max_err:.3e} (peak {peak:.3e}, rtol {rtol:g}, atol {atol:.1e}), {int(bad.sum())} of {b.numel()} outside"
+
+
+def _eager_us(module, args, kwargs, warmup: int, iters: int) -> tuple[float, float]:
+    """Median and min µs of eager PyTorch on the current device (event pairs per call)."""
+    import torch
+
+    with torch.no_grad():
+        for _ in range(max(1, warmup)):
+            module(*args, **kwargs)
+        torch.cuda.synchronize()
+        samples = []
+        for _ in range(iters):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            module(*args, **kwargs)
+            e1.record()
+            e1.synchronize()
+            samples.append(e0.elapsed_time(e1) * 1e3)
+    return statistics.median(samples), min(samples)
+
+
+def _to_device(obj, device):
+    import torch
+
+    if isinstance(obj, torch.Tensor):
+        return obj.to(device)
+    if isinstance(obj, (tuple, list)):
+        return type(obj)(_to_device(o, device) for o in obj)
+    if isinstance(obj, dict):
+        return {k: _to_device(v, device) for k, v in obj.items()}
+    return obj
+
+
+def _flatten_tensors(obj) -> list:
+    import torch
+
+    if isinstance(obj, torch.Tensor):
+        return [obj]
+    if isinstance(obj, (tuple, list)):
+        return [t for o in obj for t in _flatten_tensors(o)]
+    if isinstance(obj, dict):
+        return [t for o in obj.values() for t in _flatten_tensors(o)]
+    return []
+
+
+def kernel_rows(compiled, bench) -> list[list[str]]:
+    """One row per launch: geometry, time, achieved rate against the MI355X peak that bounds it."""
+    from deplodock_amd.ir.hip import HipOp, resolve_dim
+
+    ops = [compiled.nodes[n].op for n in compiled.topological_order() if isinstance(compiled.nodes[n].op, HipOp)]
+    times = {lt.idx: (min(lt.samples) if lt.samples else lt.time_ms) * 1e3 for lt in (bench.per_launch or [])}
+    total = sum(times.values()) or 1.0
+    rows = []
+    for i, op in enumerate(ops):
+        us = times.get(i)
+        grid = "x".join(str(resolve_dim(d, {})) for d in op.grid)
+        block = "x".join(str(resolve_dim(d, {})) for d in op.block)
+        rate = frac = "-"
+        if us:
+            gbps = op.algo_bytes / (us * 1e-6) / 1e9
+            tfs = op.algo_flops / (us * 1e-6) / 1e12
+            if op.algo_flops and tfs / MFMA_BF16_PEAK_TFLOPS > gbps / HBM_PEAK_GBPS:
+                rate, frac = f"{tfs:.1f} TFLOP/s", f"{100 * tfs / MFMA_BF16_PEAK_TFLOPS:.1f}% mfma"
+            else:
+                rate, frac = f"{gbps:.0f} GB/s", f"{100 * gbps / HBM_PEAK_GBPS:.1f}% hbm"
+        knobs = " ".join(f"{k}={v}" for k, v in op.knobs.items())
+        rows.append([str(i), op.kernel_name, grid, block, str(op.lds_bytes), f"{us:.2f}" if us else "-", f"{100 * us / total:.0f}" if us else "-", rate, frac, knobs])
+    return rows
+
+
+def handle_run(args) -> None:
+    import torch
+
+    from deplodock_amd.backend.hip.backend import HipBackend
+
+    apply_common_args(args)
+    if args.ab and not args.bench:
+        print("error: --ab requires --bench", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("error: no HIP device visible; this backend has no CPU execution path", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(0)
+    graph, prog = trace_from_args(args)
+    be = HipBackend(dump=Path(args.dump_dir) if args.dump_dir else None, device_id=0)
+    compiled = be.compile(graph)
+
+    module = prog.module.to(device).eval()
+    d_args = _to_device(prog.args, device)
+    d_kwargs = _to_device(prog.kwargs, device)
+    flat_inputs = _flatten_tensors(d_args) + _flatten_tensors(d_kwargs)
+    if len(flat_inputs) != len(compiled.inputs):
+        print(f"error: traced graph has {len(compiled.inputs)} inputs but the expression supplies {len(flat_inputs)} tensors", file=sys.stderr)
+        sys.exit(2)
+    data = dict(zip(compiled.inputs, flat_inputs))
+    # parameters were traced on the host; bind the device copies eager uses
+    with torch.no_grad():
+        want = _flatten_tensors(module(*d_args, **d_kwargs))
+    program = be.program(compiled, data)
+    try:
+        program.run()
+        torch.cuda.synchronize()
+        outs = program.output_tensors()
+        ok_all = True
+        for name, w in zip(compiled.outputs, want):
+            ok, line = check_accuracy(outs[name], w)
+            ok_all &= ok
+            print(f"{'PASS' if ok else 'FAIL'}  {name}: {line}")
+    finally:
+        program.close()
+    if not ok_all:
+        sys.exit(1)
+    if not args.bench:
+        return
+
+    eager_med, eager_min = _eager_us(module, d_args, d_kwargs, args.warmup, args.iters)
+    res = be.benchmark(compiled, input_data=data, warmup=args.warmup, num_iters=args.iters)
+    ours_min = (res.e2e_min_ms if res.e2e_ms is not None else (res.min_ms or res.time_ms)) * 1e3
+    ours_med = (res.e2e_ms if res.e2e_ms is not None else res.time_ms) * 1e3
+    rows = [["Eager PyTorch", f"{eager_med:.1f}", f"{eager_min:.1f}", "1.00x"], ["emmy (hip)", f"{ours_med:.1f}", f"{ours_min:.1f}", f"{eager_min / ours_min:.2f}x"]]
+    variants = []
+    for spec in args.ab or []:
+        import os
+
+        from deplodock_amd import config
+
+        old = os.environ.get(config.KNOBS)
+        os.environ[config.KNOBS] = spec
+        try:
+            c2 = be.compile(graph)
+            r2 = be.benchmark(c2, input_data=data, warmup=args.warmup, num_iters=args.iters)
+        finally:
+            if old is None:
+                os.environ.pop(config.KNOBS, None)
+            else:
+                os.environ[config.KNOBS] = old
+        m2 = (r2.e2e_min_ms if r2.e2e_ms is not None else (r2.min_ms or r2.time_ms)) * 1e3
+        d2 = (r2.e2e_ms if r2.e2e_ms is not None else r2.time_ms) * 1e3
+        rows.append([f"emmy [{spec}]", f"{d2:.1f}", f"{m2:.1f}", f"{eager_min / m2:.2f}x"])
+        variants.append((spec, c2, r2))
+    print()
+    for line in render_table(["Backend", "Latency (us)", "min (us)", "vs Eager"], rows, "lrrr"):
+        print(line)
+    headers = ["#", "Kernel", "Grid", "Block", "LDS", "us", "%", "Rate", "of peak", "Knobs"]
+    print()
+    for line in render_table(headers, kernel_rows(compiled, res), "llllrrrrrl"):
+        print(line)
+    for spec, c2, r2 in variants:
+        print(f"\n[{spec}]")
+        for line in render_table(headers, kernel_rows(c2, r2), "llllrrrrrl"):
+            print(line)

@@ -1,0 +1,106 @@
+"""Command-line front end: the ``--code`` grammar and the ``compile`` / ``run`` commands."""
+
+import pytest
+import torch
+
+from deplodock_amd.cli import main
+from deplodock_amd.commands.code import CodeError, parse_inline, slugify
+
+
+def test_module_call_keeps_parameters_as_constants():
+    p = parse_inline("nn.RMSNorm(64)(torch.randn(2, 4, 64))")
+    assert isinstance(p.module, torch.nn.RMSNorm)
+    assert [tuple(a.shape) for a in p.args] == [(2, 4, 64)]
+    assert p.slug == "nn-rmsnorm-64"
+
+
+def test_module_call_with_preamble_and_kwargs():
+    p = parse_inline("m = nn.Softmax(dim=-1); x = torch.randn(3, 8); m(x)")
+    assert isinstance(p.module, torch.nn.Softmax)
+    assert tuple(p.args[0].shape) == (3, 8)
+
+
+def test_expression_lifts_inline_and_named_tensors():
+    p = parse_inline("w = torch.randn(8); torch.exp(torch.randn(4, 8)) * w + torch.ones(8)")
+    assert set(p.input_names) == {"w", "x0", "x1"}
+    want = torch.exp(p.args[p.input_names.index("x0")]) * p.args[p.input_names.index("w")] + 1.0
+    got = p.module(*p.args)
+    assert torch.allclose(got, want)
+
+
+def test_single_inline_tensor_is_named_x():
+    p = parse_inline("torch.softmax(torch.randn(4, 16), -1)")
+    assert p.input_names == ("x",)
+
+
+@pytest.mark.parametrize("bad", ["x = 1", "def f(:", "1 + 2"])
+def test_rejects_unusable_code(bad):
+    with pytest.raises(CodeError):
+        parse_inline(bad)
+
+
+def test_slugify():
+    assert slugify("torch.nn.RMSNorm(2048)") == "torch-nn-rmsnorm-2048"
+    assert slugify("***") == "code"
+
+
+def test_compile_prints_one_kernel_per_launch(capsys):
+    main(["compile", "-c", "nn.RMSNorm(2048)(torch.randn(1,32,2048))"])
+    out = capsys.readouterr().out
+    assert out.count('extern "C" __global__') == 1
+    assert "k_rms_norm_reduce" in out and "REDUCE=b256" in out
+
+
+def test_compile_torch_stage_and_output_file(tmp_path, capsys):
+    dst = tmp_path / "g.txt"
+    main(["compile", "--ir", "torch", "-o", str(dst), "-c", "torch.softmax(torch.randn(4,128), -1)"])
+    assert capsys.readouterr().out == ""
+    assert "SoftmaxOp" in dst.read_text()
+
+
+def test_compile_knob_pin_reaches_the_schedule(capsys, monkeypatch):
+    monkeypatch.delenv("EMMY_KNOBS", raising=False)
+    main(["compile", "--knobs", "REDUCE=b64", "-c", "nn.RMSNorm(1024)(torch.randn(8,1024))"])
+    monkeypatch.delenv("EMMY_KNOBS", raising=False)
+    assert "REDUCE=b64" in capsys.readouterr().out
+
+
+def test_compile_without_code_exits_2(capsys):
+    with pytest.raises(SystemExit) as e:
+        main(["compile"])
+    assert e.value.code == 2
+
+
+def test_run_ab_requires_bench():
+    with pytest.raises(SystemExit) as e:
+        main(["run", "--ab", "REDUCE=b64", "-c", "torch.softmax(torch.randn(4,128), -1)"])
+    assert e.value.code == 2
+
+
+def test_accuracy_verdict_flags_a_wrong_output():
+    from deplodock_amd.commands.run import check_accuracy
+
+    want = torch.randn(64, 64)
+    ok, _ = check_accuracy(want.clone(), want)
+    assert ok
+    bad = want.clone()
+    bad[3, 5] += 1e-2
+    ok, line = check_accuracy(bad, want)
+    assert not ok and "1 of 4096" in line
+    ok, _ = check_accuracy(torch.full_like(want, float("nan")), want)
+    assert not ok
+
+
+@pytest.mark.gpu
+def test_run_checks_against_eager_and_benches(capsys):
+    main(["run", "--bench", "--iters", "10", "--warmup", "2", "--ab", "REDUCE=b128", "-c", "nn.RMSNorm(2048)(torch.randn(1,32,2048))"])
+    out = capsys.readouterr().out
+    assert out.startswith("PASS")
+    assert "Eager PyTorch" in out and "emmy (hip)" in out and "emmy [REDUCE=b128]" in out
+    assert "k_rms_norm_reduce" in out and "% hbm" in out
+
+
+@pytest.mark.gpu
+def test_run_multi_kernel_expression(capsys):
+    main(["run", "-c", "x = torch.randn(64, 512); torch.softmax(x * 0.5, -1)"])
+    assert capsys.readouterr().out.count("PASS") == 1
