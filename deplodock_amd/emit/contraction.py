@@ -84,8 +84,8 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     T = plan.block_threads
     if K % BK:
         raise LoweringError(f"contraction: K={K} is not a multiple of the slab depth {BK}")
-    if BK % 8 or BK > 128:
-        raise LoweringError(f"contraction: slab depth {BK} must be a multiple of 8 and at most 128")
+    if BK % 8 or BK > 256:
+        raise LoweringError(f"contraction: slab depth {BK} must be a multiple of 8 and at most 256")
     if lda % 8 or ldb % 8 or ldo % 4 or body.a_offset % 8 or body.b_offset % 8 or body.out_offset % 8:
         raise LoweringError("contraction: leading dimensions must keep 16-byte operand / 8-byte output alignment")
     CPR = BK // 8  # 16-byte chunks per slab row

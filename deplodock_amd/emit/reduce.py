@@ -256,15 +256,22 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
         # with its half-rotated partner, which lives in the same lane (the lane
         # count divides half the chunks), NV/2 chunks away.
         half = NV // 2
+        in_project = E.variables(body.project)
+        in_rotate = E.variables(body.rotate.expr)
         a(f"  float yv[{NV}][{V}];")
         for i in range(NV):
             a("  {")
             for ci, (_, dt) in enumerate(body.col_operands):
                 a(f"    float cv{ci}[{V}];")
                 o.extend("    " + ln for ln in _load_vec(f"c{ci}", f"{i * L} + lane", dt, V, f"cv{ci}", False))
+            for ri, ro in enumerate(body.row_operands):
+                if ro.name in in_project:
+                    a(f"    float rv{ri}[{V}];")
+                    o.extend("    " + ln for ln in _load_vec(f"rrow{ri}", f"{i * L} + lane", ro.dtype, V, f"rv{ri}", False))
             for j in range(V):
                 env = dict(env_base, x=f"xv[{i}][{j}]")
                 env.update({n: f"cv{ci}[{j}]" for ci, (n, _) in enumerate(body.col_operands)})
+                env.update({ro.name: f"rv{ri}[{j}]" for ri, ro in enumerate(body.row_operands) if ro.name in in_project})
                 a(f"    yv[{i}][{j}] = {E.render(body.project, env)};")
             a("  }")
         for i in range(NV):
@@ -272,12 +279,13 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
             a("  {")
             a(f"    float y[{V}];")
             for ri, ro in enumerate(body.row_operands):
-                a(f"    float rv{ri}[{V}];")
-                o.extend("    " + ln for ln in _load_vec(f"rrow{ri}", idx, ro.dtype, V, f"rv{ri}", False))
+                if ro.name in in_rotate:
+                    a(f"    float rv{ri}[{V}];")
+                    o.extend("    " + ln for ln in _load_vec(f"rrow{ri}", idx, ro.dtype, V, f"rv{ri}", False))
             for j in range(V):
                 partner = f"(-yv[{i + half}][{j}])" if i < half else f"yv[{i - half}][{j}]"
                 env = dict(env_base, y=f"yv[{i}][{j}]", yr=partner)
-                env.update({ro.name: f"rv{ri}[{j}]" for ri, ro in enumerate(body.row_operands)})
+                env.update({ro.name: f"rv{ri}[{j}]" for ri, ro in enumerate(body.row_operands) if ro.name in in_rotate})
                 a(f"    y[{j}] = {E.render(body.rotate.expr, env)};")
             o.extend("    " + ln for ln in _store_vec("orow", idx, body.out_dtype, V, "y", nontemporal))
             a("  }")

@@ -61,6 +61,9 @@ class _Ctx:
     out: Graph
     done: dict[str, str] = field(default_factory=dict)  # frontend node id -> lowered buffer id
     names: dict[str, int] = field(default_factory=dict)
+    # frontend node id -> (offset, shape, strides) of its value inside ``done[id]``
+    # when it is a window of a wider buffer (column slice of a merged projection)
+    windows: dict[str, tuple[int, tuple[int, ...], tuple[int, ...]]] = field(default_factory=dict)
 
     def kname(self, label: str) -> str:
         """Kernel label; the lowering appends a hash of the rendered body, so
@@ -104,7 +107,10 @@ def _need(c: _Ctx, nid: str) -> View:
     _materialize(c, cur)
     base = c.done[cur]
     hint = c.out.nodes[base].hints.get("logical_view")
-    if hint is not None:
+    if cur in c.windows:
+        offset, shape, strides = c.windows[cur]
+        v = View(base, offset, shape, strides, g.nodes[cur].output.dtype)
+    elif hint is not None:
         shape, strides = hint
         v = View(base, 0, tuple(shape), tuple(strides), g.nodes[cur].output.dtype)
     else:
@@ -127,7 +133,7 @@ def _materialize(c: _Ctx, nid: str) -> None:
             c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
         c.done[nid] = nid
         return
-    for rec in (_rec_linear_residual, _rec_gate_up, _rec_linear, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_pointwise):
+    for rec in (_rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_pointwise):
         if rec(c, nid):
             return
     raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
@@ -171,6 +177,67 @@ def _rec_linear(c: _Ctx, nid: str) -> bool:
     x, w, m, n, k, lda, ldb = _linear_parts(c, nid)
     body = Contraction(m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset)
     _emit(c, nid, body, "linear", [x.base, w.base])
+    return True
+
+
+def _plain_projection(c: _Ctx, nid: str) -> bool:
+    """A bias-free linear over a constant weight whose result only feeds layout ops
+    (so no other recognizer wants to absorb it) and is not a graph output."""
+    g = c.g
+    node = g.nodes[nid]
+    if not isinstance(node.op, F.LinearOp) or node.op.has_bias or nid in g.outputs or nid in c.done:
+        return False
+    if not isinstance(g.nodes[node.inputs[1]].op, ConstantOp) or len(g.nodes[node.inputs[1]].output.shape) != 2:
+        return False
+    cons = g.consumers(nid)
+    return bool(cons) and all(isinstance(g.nodes[x].op, LAYOUT_OPS) for x in cons)
+
+
+def _rec_linear_siblings(c: _Ctx, nid: str) -> bool:
+    """Projections of one activation (q/k/v) as a single contraction over the
+    stacked weights; each projection becomes a column window of the wide result."""
+    g = c.g
+    if not _plain_projection(c, nid):
+        return False
+    node = g.nodes[nid]
+    x_id = node.inputs[0]
+    w0 = g.nodes[node.inputs[1]].output
+    group = [
+        sid
+        for sid in g.topological_order()
+        if _plain_projection(c, sid)
+        and g.nodes[sid].inputs[0] == x_id
+        and g.nodes[sid].output.dtype == node.output.dtype
+        and g.nodes[g.nodes[sid].inputs[1]].output.dtype == w0.dtype
+        and g.nodes[g.nodes[sid].inputs[1]].output.shape[1] == w0.shape[1]
+        and g.nodes[sid].output.shape[:-1] == node.output.shape[:-1]
+    ]
+    if len(group) < 2:
+        return False
+    x = _need(c, x_id)
+    m, k, lda = _matrix(x, "linear input")
+    if k != int(w0.shape[1]):
+        raise FusionError("linear: inner dimensions differ")
+    weights = [g.nodes[sid].inputs[1] for sid in group]
+    widths = [int(g.nodes[w].output.shape[0]) for w in weights]
+    if any(n % 8 for n in widths):
+        return False  # column windows must stay 16-byte aligned for the consumers' vector loads
+    n_total = sum(widths)
+    stacked = "__".join(weights)
+    if stacked not in c.out.nodes:
+        c.out.add_constant(stacked, (n_total, k), w0.dtype)
+        c.out.nodes[stacked].hints["stacked"] = StackedConstant(tuple(weights))
+    fid = "__".join(group)
+    od = node.output.dtype
+    body = Contraction(m=m, n=n_total, k=k, a=x.base, b=stacked, out=fid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset)
+    c.out.add_node(TileOp(name=c.kname("linear"), body=body), list(dict.fromkeys([x.base, stacked])), Tensor(fid, (m, n_total), od), fid)
+    col = 0
+    for sid, n in zip(group, widths):
+        shape = tuple(int(d) for d in g.nodes[sid].output.shape)
+        lead = contiguous_strides(shape[:-1] + (1,))[:-1]
+        c.done[sid] = fid
+        c.windows[sid] = (col, shape, tuple(s * n_total for s in lead) + (1,))
+        col += n
     return True
 
 
@@ -405,83 +472,183 @@ def _match_rope(c: _Ctx, nid: str):
     return None
 
 
-def _rec_rope(c: _Ctx, nid: str) -> bool:
+@dataclass
+class _RopePlan:
+    """What ``_rec_rope`` needs to know about one rotary-embedding expression."""
+
+    t_id: str
+    cos_id: str
+    sin_id: str
+    d: int
+    od: DType
+    t_view_shape: tuple[int, ...]
+    order: list[int]  # dims of the rotated tensor (minus the last) in memory order
+    mem_shape: tuple[int, ...]
+    rows: int
+    div: int  # cos/sin table row of memory row r is (r // div) % mod
+    mod: int
+    rms: _RmsMatch | None  # the norm feeding the rotation when it can be fused in
+
+
+def _plan_rope(c: _Ctx, nid: str) -> _RopePlan | None:
     hit = _match_rope(c, nid)
     if hit is None:
-        return False
+        return None
     t_id, cos_id, sin_id = hit
     g = c.g
     node = g.nodes[nid]
-    od = node.output.dtype
     d = int(node.output.shape[-1])
-    # The rotated tensor, viewed through its layout ops, and what produced it.
-    t_view_shape = tuple(int(v) for v in g.nodes[t_id].output.shape)
     src_id = _peel_layout(g, t_id)
     rms = _match_rms_chain(c, src_id)
     fuse_norm = rms is not None and rms.cols == d and all(cons in _rope_internal(g, t_id, nid) or isinstance(g.nodes[cons].op, LAYOUT_OPS) for cons in g.consumers(src_id))
-    # cos / sin tables: [.., positions, d] broadcast over the head axis.
-    cos_v, sin_v = _need(c, cos_id), _need(c, sin_id)
-    rot_expr = _round(od, _round(od, E.Var("y") * E.Var("cos")) + _round(od, E.Var("yr") * E.Var("sin")))
-
     # Address rows of the *output* in the memory order of the rotated operand
     # (so the kernel is a row map whatever transposes the trace applied).
     tv = resolve_view(g, t_id)
     if tv.strides[-1] != 1:
         raise FusionError("rope: the rotated axis must be contiguous")
-    # memory-order dims of t (excluding the last): sort by stride descending
     order = sorted(range(len(tv.shape) - 1), key=lambda i: -tv.strides[i] if tv.shape[i] > 1 else 0)
     order = [i for i in order if tv.shape[i] > 1]
     mem_shape = tuple(tv.shape[i] for i in order)
     rows = 1
     for n in mem_shape:
         rows *= n
-    # position axis = the axis of t that cos varies over
+    # position axis = the axis of t that cos varies over; tables are [.., positions, d]
     cos_shape = tuple(int(v) for v in g.nodes[cos_id].output.shape)
     pos_axes = [i for i in range(len(cos_shape) - 1) if cos_shape[i] > 1]
     if len(pos_axes) > 1 or cos_shape[-1] != d:
         raise FusionError("rope: cos/sin must vary over one position axis")
-    if not (cos_v.strides[-1] == 1 and sin_v.strides[-1] == 1):
-        raise FusionError("rope: cos/sin must be contiguous along the rotated axis")
     if pos_axes:
         pa = pos_axes[0]
-        if pa not in order or cos_v.strides[pa] != d or sin_v.strides[pa] != d:
+        if pa not in order:
             raise FusionError("rope: unsupported cos/sin layout")
         k = order.index(pa)
         div = 1
         for n in mem_shape[k + 1 :]:
             div *= n
         mod = mem_shape[k]
-        if any(mem_shape[i] > 1 for i in range(k)):
-            # batch axes outside the position axis: positions repeat per batch element
-            pass
     else:
         div, mod = 1, 1
-    row_ops = (RowOperand("cos", cos_v.dtype, div=div, mod=mod, offset=cos_v.offset), RowOperand("sin", sin_v.dtype, div=div, mod=mod, offset=sin_v.offset))
+    return _RopePlan(t_id, cos_id, sin_id, d, node.output.dtype, tuple(int(v) for v in g.nodes[t_id].output.shape), order, mem_shape, rows, div, mod, rms if fuse_norm else None)
 
+
+def _rope_tables(c: _Ctx, p: _RopePlan, div: int) -> tuple[tuple[RowOperand, RowOperand], View, View]:
+    cos_v, sin_v = _need(c, p.cos_id), _need(c, p.sin_id)
+    if not (cos_v.strides[-1] == 1 and sin_v.strides[-1] == 1):
+        raise FusionError("rope: cos/sin must be contiguous along the rotated axis")
+    if p.mod > 1:
+        pa = [i for i in range(len(cos_v.shape) - 1) if cos_v.shape[i] > 1][0]
+        if cos_v.strides[pa] != p.d or sin_v.strides[pa] != p.d:
+            raise FusionError("rope: unsupported cos/sin layout")
+    ops = (RowOperand("cos", cos_v.dtype, div=div, mod=p.mod, offset=cos_v.offset), RowOperand("sin", sin_v.dtype, div=div, mod=p.mod, offset=sin_v.offset))
+    return ops, cos_v, sin_v
+
+
+def _rope_expr(od: DType) -> E.Expr:
+    return _round(od, _round(od, E.Var("y") * E.Var("cos")) + _round(od, E.Var("yr") * E.Var("sin")))
+
+
+def _logical_strides(p: _RopePlan, mem_strides: tuple[int, ...]) -> tuple[int, ...]:
+    """Strides of the traced (logical) shape over a buffer whose rows follow
+    ``p.order``; ``mem_strides`` are the strides of those memory-order dims."""
+    out = [0] * len(p.t_view_shape)
+    for pos, i in enumerate(p.order):
+        out[i] = mem_strides[pos]
+    out[-1] = 1
+    return tuple(out)
+
+
+def _rec_rope_pair(c: _Ctx, nid: str) -> bool:
+    """Query and key head-norm + rotary embedding as one launch.  Applies when
+    both read adjacent head ranges of one merged projection buffer
+    (``[tokens, (q heads + k heads + ...) * d]``): the heads of both are walked
+    as rows of one kernel, the two norm weights are stacked per head, and each
+    result is a window of the ``[tokens, q heads + k heads, d]`` output."""
+    g = c.g
+    p = _plan_rope(c, nid)
+    if p is None or p.rms is None or p.rms.weight is None or len(p.mem_shape) != 2 or p.mod != p.mem_shape[0]:
+        return False
+    partner = None
+    for oid in g.topological_order():
+        if oid == nid or oid in c.done or not _is(g.nodes[oid], F.ElementwiseOp, fn="add"):
+            continue
+        q = _plan_rope(c, oid)
+        if q is None or q.rms is None or q.rms.weight is None:
+            continue
+        if (q.cos_id, q.sin_id, q.d, q.od, q.mod, q.order, q.rms.eps, q.rms.inner) == (p.cos_id, p.sin_id, p.d, p.od, p.mod, p.order, p.rms.eps, p.rms.inner) and len(q.mem_shape) == 2:
+            partner = (oid, q)
+            break
+    if partner is None:
+        return False
+    oid, q = partner
+    xa, xb = _need(c, p.rms.x), _need(c, q.rms.x)
+    if xa.base != xb.base or xa.dtype != xb.dtype:
+        return False
+    plans = [(nid, p, xa), (oid, q, xb)]
+    plans.sort(key=lambda t: t[2].offset)
+    (id0, p0, x0), (id1, p1, x1) = plans
+    try:
+        (rows0, a0), (rows1, a1) = _row_addr(x0), _row_addr(x1)
+    except FusionError:
+        return False
+    h0, h1 = p0.mem_shape[1], p1.mem_shape[1]
+    d = p.d
+    if not (a0.div == h0 and a1.div == h1 and a0.stride_lo == d and a1.stride_lo == d and a0.stride_hi == a1.stride_hi and a1.offset == a0.offset + h0 * d and (h0 + h1) * d <= a0.stride_hi):
+        return False
+    w0, w1 = _need(c, p0.rms.weight), _need(c, p1.rms.weight)
+    if not (isinstance(g.nodes[p0.rms.weight].op, ConstantOp) and isinstance(g.nodes[p1.rms.weight].op, ConstantOp) and w0.dtype == w1.dtype):
+        return False
+    heads = h0 + h1
+    tokens = p0.mem_shape[0]
+    stacked = f"{p0.rms.weight}__x{h0}__{p1.rms.weight}__x{h1}"
+    if stacked not in c.out.nodes:
+        c.out.add_constant(stacked, (heads * d,), w0.dtype)
+        c.out.nodes[stacked].hints["stacked"] = StackedConstant((p0.rms.weight,) * h0 + (p1.rms.weight,) * h1)
+    od = p.od
+    x = E.Var("x")
+    norm = x * E.Un("rsqrt", E.Var("ss") / float(d) + p.rms.eps)
+    tables, cos_v, sin_v = _rope_tables(c, p, div=heads)
+    fid = f"{id0}__{id1}"
+    body = RowReduce(
+        rows=tokens * heads, cols=d, x=x0.base, x_dtype=x0.dtype, out=fid, out_dtype=od, stats=(Stat("ss", "sum", x * x),),
+        project=E.Var("w") * _round(p.rms.inner, norm), x_addr=RowAddr(offset=a0.offset, div=heads, stride_hi=a0.stride_hi, stride_lo=d),
+        row_operands=(RowOperand("w", w0.dtype, div=1, mod=heads, offset=0), *tables),
+    )  # fmt: skip
+    body.rotate = RotateHalf(_rope_expr(od))
+    body.operand_buffers = {"w": stacked, "cos": cos_v.base, "sin": sin_v.base}
+    c.out.add_node(TileOp(name=c.kname("rms_norm_rope"), body=body), list(dict.fromkeys([x0.base, stacked, cos_v.base, sin_v.base])), Tensor(fid, (tokens, heads, d), od), fid)
+    for rid, rp, first in ((id0, p0, 0), (id1, p1, h0)):
+        c.done[rid] = fid
+        c.windows[rid] = (first * d, rp.t_view_shape, _logical_strides(rp, (heads * d, d)))
+    return True
+
+
+def _rec_rope(c: _Ctx, nid: str) -> bool:
+    p = _plan_rope(c, nid)
+    if p is None:
+        return False
+    g = c.g
+    od, d = p.od, p.d
+    row_ops, cos_v, sin_v = _rope_tables(c, p, div=p.div)
     # Output buffer: rows in t's memory order; the logical result is a view of it.
-    out_mem_shape = (*mem_shape, d)
-    if fuse_norm:
-        body, inputs, xv = _rms_body(c, nid, rms, od)
-        if (body.rows, body.cols) != (rows, d):
+    out_mem_shape = (*p.mem_shape, d)
+    if p.rms is not None:
+        body, inputs, xv = _rms_body(c, nid, p.rms, od)
+        if (body.rows, body.cols) != (p.rows, d):
             raise FusionError("rope: norm rows do not match the rotated tensor")
     else:
-        xv = _need(c, t_id)
-        rows2, x_addr = _row_addr(View(xv.base, xv.offset, tuple(tv.shape[i] for i in order) + (d,), tuple(tv.strides[i] for i in order) + (1,), xv.dtype))
+        tv = resolve_view(g, p.t_id)
+        xv = _need(c, p.t_id)
+        rows2, x_addr = _row_addr(View(xv.base, xv.offset, tuple(tv.shape[i] for i in p.order) + (d,), tuple(tv.strides[i] for i in p.order) + (1,), xv.dtype))
         body = RowReduce(rows=rows2, cols=d, x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=od, stats=(), project=E.Var("x"), x_addr=x_addr)
         body.operand_buffers = {}
         inputs = [xv.base]
     body.row_operands = row_ops
-    body.rotate = RotateHalf(rot_expr)
+    body.rotate = RotateHalf(_rope_expr(od))
     body.operand_buffers.update({"cos": cos_v.base, "sin": sin_v.base})
     inputs += [cos_v.base, sin_v.base]
-    _emit(c, nid, body, "rms_norm_rope" if fuse_norm else "rope", inputs, shape=out_mem_shape)
+    _emit(c, nid, body, "rms_norm_rope" if p.rms is not None else "rope", inputs, shape=out_mem_shape)
     # Record how the logical (traced) shape maps onto the memory-order buffer.
-    strides_mem = contiguous_strides(out_mem_shape)
-    logical_strides = [0] * len(t_view_shape)
-    for pos, i in enumerate(order):
-        logical_strides[i] = strides_mem[pos]
-    logical_strides[-1] = 1
-    c.out.nodes[nid].hints["logical_view"] = (t_view_shape, tuple(logical_strides))
+    c.out.nodes[nid].hints["logical_view"] = (p.t_view_shape, _logical_strides(p, contiguous_strides(out_mem_shape)[:-1]))
     return True
 
 

@@ -30,16 +30,24 @@ from deplodock_amd.ir.tile import Contraction, Flash, Map, RowReduce, TileOp
 logger = logging.getLogger(__name__)
 
 # (tile_m, tile_n, waves_m, waves_n, atom, bk) — ordered by measured throughput on
-# MI355X for large bf16 problems (first fit that fills the machine wins).
+# MI355X (first fit that fills the machine wins).  The large tiles are ranked on a
+# compute-bound 2048x3072x1024 problem; the small ones on 512-row and decode-size
+# problems timed with operands rotating through more memory than the L2s hold,
+# where a step of the k loop costs one L2-miss round trip whatever its size: deep
+# slabs (256 elements) and 4-8 waves per workgroup won every such shape.
 TILE_CANDIDATES: tuple[tuple[int, int, int, int, str, int], ...] = (
     (128, 192, 4, 2, "mfma_16x16x32_bf16", 2),
     (128, 128, 2, 2, "mfma_32x32x16_bf16", 4),
     (128, 96, 4, 1, "mfma_32x32x16_bf16", 4),
-    (64, 128, 2, 2, "mfma_32x32x16_bf16", 4),
-    (64, 64, 2, 2, "mfma_16x16x32_bf16", 2),
-    (32, 64, 1, 2, "mfma_16x16x32_bf16", 2),
-    (16, 64, 1, 4, "mfma_16x16x32_bf16", 2),
+    (64, 128, 2, 4, "mfma_16x16x32_bf16", 4),
+    (64, 64, 2, 2, "mfma_16x16x32_bf16", 4),
+    (32, 64, 1, 4, "mfma_16x16x32_bf16", 8),
+    (16, 16, 1, 1, "mfma_16x16x32_bf16", 8),
 )
+
+# A launch "fills the machine" from this fraction of the CUs on: 192 workgroups of
+# a 64x128 tile beat 384 of a 64x64 tile on the gate/up shape (12.1 vs 16.1 us).
+_FILL_FRACTION = 0.75
 
 
 def _pin(name: str) -> str | None:
@@ -117,7 +125,8 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context) -> TilePlan
         fm, fn = tm // (wm * atom.m), tn // (wn * atom.n)
         if fm * fn * atom.acc_per_lane * (2 if gate_pair else 1) > 256:
             continue
-        while bk > 1 and k % (bk * atom.k):
+        nb = 2 if gate_pair else 1
+        while bk > 1 and (k % (bk * atom.k) or 2 * (tm + tn * nb) * bk * atom.k * 2 > ctx.lds_bytes_per_cu):
             bk //= 2
         if k % (bk * atom.k):
             continue
@@ -129,7 +138,7 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context) -> TilePlan
         groups = -(-m // tm) * -(-n // tn)
         # penalise tiles that mostly hang over the edge of a small problem
         waste = (-(-m // tm) * tm * -(-n // tn) * tn) / float(m * n)
-        if groups >= ctx.compute_units and waste < 1.5:
+        if groups >= _FILL_FRACTION * ctx.compute_units and waste < 1.5:
             return plan
         score = (min(groups, ctx.compute_units) / waste, tm * tn)
         if best is None or score > best[0]:

@@ -75,18 +75,34 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
     compiled = compile_case(eager.qwen3_block_case(seq=64))
     names = [re.sub(r"_[0-9a-f]{6}$", "", k.kernel_name) for k in kernels(compiled)]
     assert names == [
-        "k_rms_norm_reduce", "k_linear", "k_rms_norm_rope", "k_linear", "k_rms_norm_rope", "k_linear",
+        "k_rms_norm_reduce", "k_linear", "k_rms_norm_rope",
         "k_sdpa_reduce", "k_linear_add", "k_rms_norm_reduce", "k_linear_silu_mul", "k_linear_add",
     ]  # fmt: skip
+    # q, k and v projections are one contraction over the stacked weights; each
+    # projection is a column window of its [tokens, 2048 + 1024 + 1024] result
+    qkv = kernels(compiled)[1]
+    assert "N=4096" in qkv.comment and qkv.algo_flops == 2 * 64 * 4096 * 1024
     for k in kernels(compiled):
         hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
     # layout ops produced no kernels and no buffers
     assert not any("transpose" in n or "view" in n or "slice" in n for n in compiled.nodes)
-    # the gate and up weights are stacked into one constant the runtime assembles
-    stacked = [n for n in compiled.nodes.values() if n.hints.get("stacked")]
-    assert len(stacked) == 1 and stacked[0].output.shape == (6144, 1024)
+    # the query and key head norms + rotary embeddings are one launch over the
+    # 16 + 8 heads of every token, with the two norm weights stacked per head
+    rope = kernels(compiled)[2]
+    assert "rows=1536 cols=128" in rope.comment and "(row / 24) * 4096L + (row % 24) * 128L" in rope.kernel_source
+    # q/k/v and gate/up weights are stacked into constants the runtime assembles
+    stacked = sorted((n for n in compiled.nodes.values() if n.hints.get("stacked") and len(n.output.shape) == 2), key=lambda n: n.output.shape[0])
+    assert [n.output.shape for n in stacked] == [(4096, 1024), (6144, 1024)]
     data = HipBackend.bind(compiled, {})
-    assert data[stacked[0].id].shape == (6144, 1024)
+    assert [tuple(data[n.id].shape) for n in stacked] == [(4096, 1024), (6144, 1024)]
+    traced = compiled.constant_values
+    (norm_w,) = [n for n in compiled.nodes.values() if n.hints.get("stacked") and len(n.output.shape) == 1]
+    assert tuple(data[norm_w.id].shape) == (24 * 128,)
+    assert (data[norm_w.id][15 * 128 : 16 * 128] == traced["p_l_self_attn_q_norm_weight"]).all()
+    assert (data[norm_w.id][16 * 128 : 17 * 128] == traced["p_l_self_attn_k_norm_weight"]).all()
+    parts = stacked[0].hints["stacked"].parts
+    assert [p.split("_proj")[0][-1] for p in parts] == ["q", "k", "v"]
+    assert (data[stacked[0].id][2048:3072] == traced[parts[1]]).all()
 
 
 def test_reduce_pin_is_authoritative_and_bad_pin_degrades(launcher_lib, monkeypatch):
