@@ -69,16 +69,22 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int grp = wave / WQ, wq = wave % WQ;
   const int lq = lane % 32, lh = lane / 32;
-  const int qb = (QBLOCKS - 1) - (int)(blockIdx.x % QBLOCKS);
-  const int head = (blockIdx.x / QBLOCKS) % HQ;
-  const int batch = blockIdx.x / (QBLOCKS * HQ);
+  // PAIR: a workgroup takes query block b from the heavy end and then its
+  // mirror from the light end, so under a causal mask every workgroup streams
+  // the same number of key blocks (QBLOCKS + 1) whatever b is.
+  const int slot = (int)(blockIdx.x % QSLOTS);
+  const int head = (blockIdx.x / QSLOTS) % HQ;
+  const int batch = blockIdx.x / (QSLOTS * HQ);
   const int kvh = head / GROUP;
-  const int q0 = qb * BQ;
-  const int qw0 = q0 + wq * 32;
-  const int qrow = qw0 + lq;
   const ELT* qbase = Q + Q_OFF + (long)batch * Q_SB + (long)head * Q_SH;
   const ELT* kbase = Kp + K_OFF + (long)batch * K_SB + (long)kvh * K_SH;
   const ELT* vbase = Vp + V_OFF + (long)batch * V_SB + (long)kvh * V_SH;
+  #pragma unroll 1
+  for (int pass = 0; pass < (PAIR ? 2 : 1); ++pass) {
+  const int qb = pass == 0 ? (QBLOCKS - 1) - slot : slot;
+  const int q0 = qb * BQ;
+  const int qw0 = q0 + wq * 32;
+  const int qrow = qw0 + lq;
 
   FRAG qf[D / 16];
   {
@@ -283,6 +289,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       }
     }
   }
+  if (PAIR) __syncthreads();  // the staging buffers are rewritten by the next pass
+  }
 }
 """
 
@@ -315,6 +323,10 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     if body.o_strides[2] % 4 or any(o % 8 for o in (body.q_offset, body.k_offset, body.v_offset)) or body.o_offset % 4:
         raise LoweringError("flash: offsets / output stride break vector alignment")
     qblocks = -(-body.q_len // BQ)
+    pair = bool(body.pair)
+    if pair and not (body.causal and qblocks % 2 == 0):
+        raise LoweringError("flash: pairing mirrored query blocks needs a causal mask and an even block count")
+    qslots = qblocks // 2 if pair else qblocks
     bf16 = body.dtype.name == "bf16"
     defs = {
         "KNAME": name,
@@ -329,6 +341,8 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "HQ": body.q_heads,
         "GROUP": body.q_heads // body.kv_heads,
         "QBLOCKS": qblocks,
+        "QSLOTS": qslots,
+        "PAIR": 1 if pair else 0,
         "CAUSAL": 1 if body.causal else 0,
         "SCALE_LOG2": float_literal(body.scale * math.log2(math.e)),
         "Q_SB": body.q_strides[0], "Q_SH": body.q_strides[1], "Q_SS": body.q_strides[2], "Q_OFF": body.q_offset,
@@ -349,7 +363,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     head = f"// {name}: B={body.batch} Hq={body.q_heads} Hkv={body.kv_heads} Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal}\n"
     head += "".join(f"#define {k} {v}\n" for k, v in defs.items())
     source = prelude.header() + head + _SRC
-    grid = qblocks * body.q_heads * body.batch
+    grid = qslots * body.q_heads * body.batch
     return HipOp(
         kernel_source=source,
         kernel_name=name,
@@ -357,8 +371,8 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         grid=((grid,), (1,), (1,)),
         block=((NT,), (1,), (1,)),
         lds_bytes=lds,
-        comment=f"flash Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} bkv={BKV}",
+        comment=f"flash Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} bkv={BKV} split={kvs} pair={int(pair)}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
-        knobs={"FLASH": f"w{waves}/kv{BKV}/s{kvs}"},
+        knobs={"FLASH": f"w{waves}/kv{BKV}/s{kvs}" + ("/p" if pair else "")},
     )

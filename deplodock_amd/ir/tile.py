@@ -199,6 +199,7 @@ class Flash:
     block_kv: int = 64
     waves: int = 4  # 32-row query groups per workgroup
     kv_split: int = 1  # wave groups that split the key blocks of a query group between them
+    pair: bool = False  # causal only: a workgroup takes query block b and its mirror QBLOCKS-1-b
 
     def algo_flops(self) -> int:
         if self.causal and self.q_len == self.kv_len:

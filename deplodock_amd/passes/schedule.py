@@ -184,37 +184,51 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
 
 
 def schedule_flash(body: Flash, ctx: Context) -> dict:
-    """``EMMY_FLASH=w<row groups>/kv<keys per block>/s<key split>``.  Default: four
-    32-row groups x two key-split wave groups (8 waves, two per SIMD; measured
-    41.5 us vs 62.7 us unsplit on the S=2048 causal shape), with the row groups
-    halved until the launch covers the CUs."""
+    """``EMMY_FLASH=w<row groups>/kv<keys per block>/s<key split>[/p]``.
+
+    Default: four 32-row groups x two key-split wave groups (8 waves, two per
+    SIMD; measured 41.5 us vs 62.7 us unsplit on the S=2048 causal shape), with the
+    row groups halved until the launch covers the CUs.  A causal self-attention
+    whose mirrored query-block pairs (``/p``: block b then block n-1-b in one
+    workgroup, equal key work for every workgroup) still cover the CUs takes
+    ``w2/kv32/s4/p`` instead: 36.6 us on the same shape, where unpaired
+    workgroups wait for the one that owns the last rows."""
     pinned = _pin("FLASH")
     if pinned:
         try:
+            body.pair = False
             for tok in pinned.split("/"):
-                if tok.startswith("w"):
+                if tok == "p":
+                    body.pair = True
+                elif tok.startswith("w"):
                     body.waves = int(tok[1:])
                 elif tok.startswith("kv"):
                     body.block_kv = int(tok[2:])
                 elif tok.startswith("s"):
                     body.kv_split = int(tok[1:])
                 else:
-                    raise ScheduleError(f"cannot parse {tok!r} (expect w<groups> / kv<keys> / s<split>)")
+                    raise ScheduleError(f"cannot parse {tok!r} (expect w<groups> / kv<keys> / s<split> / p)")
             chunks = body.block_kv * body.head_dim // 8
             if body.waves < 1 or body.kv_split < 1 or body.block_kv % 32 or chunks % (body.waves * body.kv_split * 64):
                 raise ScheduleError("unrealisable workgroup shape")
             if 2 * body.kv_split * 2 * body.block_kv * body.head_dim * 2 > ctx.lds_bytes_per_cu:
                 raise ScheduleError("the double-buffered K/V blocks of all key-split groups exceed the LDS")
+            if body.pair and not (body.causal and -(-body.q_len // (32 * body.waves)) % 2 == 0):
+                raise ScheduleError("pairing mirrored query blocks needs a causal mask and an even block count")
         except (ValueError, ScheduleError) as exc:
             logger.warning("EMMY_FLASH=%r ignored: %s", pinned, exc)
             pinned = None
     if not pinned:
-        body.waves, body.block_kv = 4, 64
         heads = body.batch * body.q_heads
-        while body.waves > 1 and heads * -(-body.q_len // (32 * body.waves)) < ctx.compute_units:
-            body.waves //= 2
-        body.kv_split = 2 if -(-body.kv_len // body.block_kv) >= 2 else 1
-    return {"FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}"}
+        blocks64 = -(-body.q_len // 64)
+        if body.causal and body.q_len == body.kv_len and blocks64 % 2 == 0 and heads * blocks64 // 2 >= _FILL_FRACTION * ctx.compute_units and body.head_dim == 128:
+            body.waves, body.block_kv, body.kv_split, body.pair = 2, 32, 4, True
+        else:
+            body.waves, body.block_kv, body.pair = 4, 64, False
+            while body.waves > 1 and heads * -(-body.q_len // (32 * body.waves)) < ctx.compute_units:
+                body.waves //= 2
+            body.kv_split = 2 if -(-body.kv_len // body.block_kv) >= 2 else 1
+    return {"FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "")}
 
 
 def schedule(graph: Graph, ctx: Context | None = None) -> Graph:

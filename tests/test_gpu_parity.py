@@ -212,6 +212,28 @@ def test_c4_every_workgroup_shape(device, pin, monkeypatch):
         prog.close()
 
 
+@pytest.mark.parametrize("pin", ["w2/kv32/s4/p", "w1/kv64/s2/p", "w4/kv64/s2/p", "w2/kv64/s1/p"])
+def test_c4_mirrored_query_block_pairs(device, pin, monkeypatch):
+    """A workgroup that takes query block b and then block n-1-b reuses its LDS and
+    registers for the second block: both halves of every pair are checked, on repeated launches."""
+    monkeypatch.setenv("EMMY_FLASH", pin)
+    case = eager.sdpa_case(b=2, hq=4, hkv=2, s=512, d=128, seed=11)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    assert [n.op.knobs["FLASH"] for n in compiled.nodes.values() if isinstance(n.op, HipOp)] == [pin]
+    want = eager.run_eager(case, device)
+    prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, case.inputs)})
+    try:
+        out = prog.output_tensors()[compiled.outputs[0]]
+        for rep in range(5):
+            out.zero_()
+            prog.run()
+            torch.cuda.synchronize()
+            eager.assert_close(out.reshape(want.shape), want, case.rtol, case.atol, f"sdpa {pin} launch {rep}")
+    finally:
+        prog.close()
+
+
 def test_c4_golden(device, golden):
     ours, _, _ = run_case(eager.sdpa_case(1, 4, 2, 96, 128), device)
     want = torch.from_numpy(golden["c4_y_bits"].view(np.int16).copy()).view(torch.bfloat16).float()

@@ -136,7 +136,11 @@ def test_flash_pin_grammar_and_degrade(launcher_lib, monkeypatch):
     case = eager.sdpa_case(1, 8, 4, 320, 128)
     default = kernels(compile_case(case))[0].knobs["FLASH"]
     assert default == "w1/kv64/s2"  # few heads, short sequence: one 32-row group per workgroup to cover the CUs
-    assert kernels(compile_case(eager.sdpa_case()))[0].knobs["FLASH"] == "w4/kv64/s2"
+    # long causal self-attention: mirrored query-block pairs, so every workgroup streams the same number of keys
+    big = kernels(compile_case(eager.sdpa_case()))[0]
+    assert big.knobs["FLASH"] == "w2/kv32/s4/p" and big.grid[0] == (16 * 32 // 2,) and "#define PAIR 1" in big.kernel_source
+    monkeypatch.setenv("EMMY_FLASH", "w4/kv64/s2/p")  # 320 rows = 3 blocks of 128: no mirror for the middle one
+    assert kernels(compile_case(case))[0].knobs["FLASH"] == default
     monkeypatch.setenv("EMMY_FLASH", "w2/kv32/s4")
     k = kernels(compile_case(case))[0]
     assert k.knobs["FLASH"] == "w2/kv32/s4" and k.block[0] == (512,) and k.lds_bytes == 2 * 4 * 2 * 32 * 128 * 2
