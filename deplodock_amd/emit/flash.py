@@ -243,12 +243,13 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
     __syncthreads();
   }
 
-  // ---- merge the key-split groups: group g > 0 parks (m, l, O) in LDS ----
-  float* park = (float*)lds;  // [wq][66][64 lanes]; the staging buffers are free after the last barrier
+  // ---- merge the key-split groups pairwise through LDS: in round r, group g with
+  // g % 2^(r+1) == 2^r parks (m, l, O) and group g - 2^r folds it in ----
+  float* park = (float*)lds;  // [slot][wq][66][64 lanes]; the staging buffers are free after the last barrier
   #pragma unroll 1
-  for (int g = 1; g < KVS; ++g) {
-    if (grp == g) {
-      float* pw = park + wq * (D / 32 * 16 + 2) * 64 + lane;
+  for (int sft = 1; sft < KVS; sft *= 2) {
+    float* pw = park + ((grp / (2 * sft)) * WQ + wq) * (D / 32 * 16 + 2) * 64 + lane;
+    if (grp % (2 * sft) == sft) {
       pw[0] = m_ref;
       pw[64] = l_run;
       #pragma unroll
@@ -257,8 +258,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       for (int r = 0; r < 16; ++r) pw[(2 + t * 16 + r) * 64] = oacc[t][r];
     }
     __syncthreads();
-    if (grp == 0) {
-      const float* pw = park + wq * (D / 32 * 16 + 2) * 64 + lane;
+    if (grp % (2 * sft) == 0 && grp + sft < KVS) {
       const float m_o = pw[0], l_o = pw[64];
       const float m_new = fmaxf(m_ref, m_o);
       const float a_s = EXP2(m_ref - m_new), a_o = EXP2(m_o - m_new);
@@ -314,7 +314,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         raise LoweringError(f"flash: {waves} x {kvs} waves exceed {ctx.max_threads_per_block} threads")
     if (BKV * D // 8) % NT:
         raise LoweringError("flash: a key block's 16-byte chunks must be a multiple of the workgroup's threads")
-    lds = max(2 * kvs * 2 * BKV * D * 2, waves * (D // 32 * 16 + 2) * 64 * 4 if kvs > 1 else 0)
+    lds = max(2 * kvs * 2 * BKV * D * 2, ((kvs + 1) // 2) * waves * (D // 32 * 16 + 2) * 64 * 4 if kvs > 1 else 0)
     if lds > ctx.lds_bytes_per_cu:
         raise LoweringError(f"flash: {lds} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
     for st in (body.q_strides, body.k_strides, body.v_strides):
