@@ -72,9 +72,14 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   // PAIR: a workgroup takes query block b from the heavy end and then its
   // mirror from the light end, so under a causal mask every workgroup streams
   // the same number of key blocks (QBLOCKS + 1) whatever b is.
-  const int slot = (int)(blockIdx.x % QSLOTS);
-  const int head = (blockIdx.x / QSLOTS) % HQ;
-  const int batch = blockIdx.x / (QSLOTS * HQ);
+  // Workgroup ids go round-robin over the XCDs, each with its own L2.  Consecutive
+  // logical ids (the query blocks of one head, then the next head of the same KV
+  // group) are dealt to one XCD, so a KV head's keys and values are fetched from
+  // HBM by one L2 instead of by all of them.
+  const int bid = GRID % XCDS == 0 ? (int)(blockIdx.x % XCDS) * (GRID / XCDS) + (int)(blockIdx.x / XCDS) : (int)blockIdx.x;
+  const int slot = bid % QSLOTS;
+  const int head = (bid / QSLOTS) % HQ;
+  const int batch = bid / (QSLOTS * HQ);
   const int kvh = head / GROUP;
   const ELT* qbase = Q + Q_OFF + (long)batch * Q_SB + (long)head * Q_SH;
   const ELT* kbase = Kp + K_OFF + (long)batch * K_SB + (long)kvh * K_SH;
@@ -362,8 +367,9 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     }  # fmt: skip
     head = f"// {name}: B={body.batch} Hq={body.q_heads} Hkv={body.kv_heads} Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal}\n"
     head += "".join(f"#define {k} {v}\n" for k, v in defs.items())
-    source = prelude.header() + head + _SRC
     grid = qslots * body.q_heads * body.batch
+    head += f"#define GRID {grid}\n#define XCDS {ctx.xcds}\n"
+    source = prelude.header() + head + _SRC
     return HipOp(
         kernel_source=source,
         kernel_name=name,
