@@ -118,7 +118,7 @@ def _cpu_baseline() -> dict:
     }
 
 
-def _table(device, only: str | None = None) -> list[dict]:
+def _table(device, only: str | None = None, extended: bool = False) -> list[dict]:
     """Per-kernel µs / achieved rate / fraction of peak for every configuration."""
     import torch
 
@@ -210,7 +210,11 @@ def _table(device, only: str | None = None) -> list[dict]:
     for m in (1, 16, 128):
         bench(lambda m=m: eager.linear_case(m=m), f"C3 linear bf16 M={m} K=1024 N=3072", "hbm", cold=True)
     bench(lambda: eager.linear_case(m=2048), "C3 linear bf16 M=2048 K=1024 N=3072", "mfma")
+    if extended:
+        bench(lambda: eager.linear_case(m=4096, k=4096, n=4096), "C3x linear bf16 M=4096 K=4096 N=4096", "mfma")
     bench(eager.sdpa_case, "C4 causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
+    if extended:
+        bench(lambda: eager.sdpa_case(causal=False), "C4x non-causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
     bench(lambda: eager.qwen3_block_case(seq=512), "C5 qwen3-0.6B block bf16 S=512", "mfma")
     return rows
 
@@ -223,6 +227,7 @@ def main() -> int:
     ap.add_argument("--no-table", action="store_true", help="skip the per-configuration kernel table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default=None, metavar="TEXT", help="restrict the kernel table to configurations whose label contains TEXT (e.g. 'M=2048', 'C4')")
+    ap.add_argument("--extended", action="store_true", help="add machine-filling variants to the kernel table (4096^3 linear, non-causal attention)")
     ap.add_argument("--copy-probe", action="store_true", help="also run a plain 469762048-byte device copy 5 times (counter calibration under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -273,7 +278,7 @@ def main() -> int:
     }
     out["cpu_baseline"] = None if args.no_cpu else _cpu_baseline()
     if not args.no_table:
-        out["kernels"] = _table(device, args.only)
+        out["kernels"] = _table(device, args.only, args.extended)
     print(json.dumps(out))
     return 0
 

@@ -104,3 +104,14 @@ def test_run_checks_against_eager_and_benches(capsys):
 def test_run_multi_kernel_expression(capsys):
     main(["run", "-c", "x = torch.randn(64, 512); torch.softmax(x * 0.5, -1)"])
     assert capsys.readouterr().out.count("PASS") == 1
+
+
+def test_microbench_kernels_compile_for_gfx950():
+    from deplodock_amd.backend.hip import hiprtc
+    from deplodock_amd.commands.microbench import _kernel_source
+
+    for k, kind, mfma in ((0, "fma", True), (8, "exp", True), (4, "fma", False)):
+        name = f"k_coissue_test_{k}_{kind}_{int(mfma)}"
+        src = _kernel_source(name, k, kind, 256, mfma)
+        assert src.count("__builtin_amdgcn_mfma_f32_32x32x16_bf16") == (2 if mfma else 0)
+        assert hiprtc.compile_to_hsaco(src, name).stat().st_size > 0
