@@ -11,6 +11,8 @@ passed as device ``torch.Tensor`` objects, in which case they are used in place.
 
 from __future__ import annotations
 
+from collections import OrderedDict
+
 from deplodock_amd import config
 from deplodock_amd.backend import Backend, BenchmarkResult, RunResult
 from deplodock_amd.context import Context
@@ -44,8 +46,49 @@ class HipBackend(Backend):
 
     # -- compile ------------------------------------------------------------
     def compile(self, graph: Graph) -> Graph:
-        """Lower ``Graph`` → ``Graph[TileOp]`` → ``Graph[HipOp]`` (needs no GPU)."""
-        return Pipeline.build(HIP_PASSES, self.context).run(graph, dump_dir=self.dump)
+        """Lower ``Graph`` → ``Graph[TileOp]`` → ``Graph[HipOp]`` (needs no GPU).
+
+        A graph traced with ``dynamic_shapes`` is lowered at its example sizes; the
+        result remembers how to re-trace (``compiled.dynamic``) and ``run`` /
+        ``program`` / ``benchmark`` pick — building on first use — the variant that
+        matches the shapes of the inputs they are given."""
+        compiled = Pipeline.build(HIP_PASSES, self.context).run(graph, dump_dir=self.dump)
+        spec = getattr(graph, "dynamic", None)
+        if spec is not None:
+            compiled.dynamic = spec
+            compiled.variants = OrderedDict({tuple(sorted(spec.hints.items())): compiled})
+        return compiled
+
+    #: distinct size combinations kept per dynamically shaped graph
+    VARIANT_CACHE = 8
+
+    def variant(self, compiled: Graph, input_data: dict | None) -> Graph:
+        """The lowering of ``compiled``'s module at the sizes ``input_data`` has."""
+        spec = getattr(compiled, "dynamic", None)
+        if spec is None or not input_data:
+            return compiled
+        shapes = []
+        for nid, axes in zip(compiled.inputs, spec.input_axes):
+            if nid not in input_data:
+                if axes:
+                    return compiled  # benchmark-style call with synthetic inputs: the traced sizes
+                shapes.append(compiled.nodes[nid].output.shape)
+                continue
+            shapes.append(tuple(input_data[nid].shape))
+        env = spec.env_of(shapes)
+        key = tuple(sorted(env.items()))
+        cache = compiled.variants
+        if key in cache:
+            cache.move_to_end(key)
+            return cache[key]
+        g = Pipeline.build(HIP_PASSES, self.context).run(spec.retrace(env), dump_dir=self.dump)
+        if g.inputs != compiled.inputs or g.outputs != compiled.outputs:
+            raise ValueError("re-tracing at another size changed the graph's inputs or outputs")
+        g.dynamic, g.variants = spec, cache
+        cache[key] = g
+        while len(cache) > self.VARIANT_CACHE:
+            cache.popitem(last=False)
+        return g
 
     # -- binding ------------------------------------------------------------
     @staticmethod
@@ -74,6 +117,7 @@ class HipBackend(Backend):
         from deplodock_amd.backend.hip.program import run_program
 
         self._select_device()
+        compiled = self.variant(compiled, input_data)
         result, pre = run_program(compiled, input_data=self.bind(compiled, input_data), pre_run=pre_run)
         outputs = {}
         for name, vals in result.outputs.items():
@@ -87,6 +131,7 @@ class HipBackend(Backend):
         from deplodock_amd.backend.hip.program import CompiledProgram
 
         self._select_device()
+        compiled = self.variant(compiled, input_data)
         return CompiledProgram.build(compiled, self.bind(compiled, input_data))
 
     # -- benchmark --------------------------------------------------------------
@@ -110,6 +155,7 @@ class HipBackend(Backend):
         from deplodock_amd.backend.hip.program import benchmark_program
 
         self._select_device()
+        compiled = self.variant(compiled, input_data)
         with config.hiprtc_flags_override(hiprtc_flags):
             return benchmark_program(
                 compiled,

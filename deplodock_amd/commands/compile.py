@@ -23,6 +23,14 @@ def add_common_args(parser) -> None:
     parser.add_argument("--knobs", default=None, help="Pin scheduling knobs for this invocation, 'K1=V1,K2=V2' (the EMMY_KNOBS grammar), e.g. 'TILE=a:mfma_32x32x16_bf16/w2x2/f2x3/k4'.")
     parser.add_argument("--hiprtc-flags", default=None, help="Extra hipRTC options (space separated); same as EMMY_HIPRTC_FLAGS.")
     parser.add_argument("--seed", type=int, default=0, help="torch RNG seed applied before the expression is evaluated (default 0).")
+    parser.add_argument(
+        "--dynamic",
+        action="append",
+        default=None,
+        metavar="NAME@INPUT:AXIS",
+        help="Let axis AXIS of forward argument INPUT vary at run time under the name NAME (repeatable), e.g. 'seq_len@x:1'. "
+        "Kernels stay specialised per size: another size re-traces and re-lowers on first use.",
+    )
     parser.add_argument("-v", "--verbose", action="count", default=0)
 
 
@@ -52,7 +60,23 @@ def trace_from_args(args):
     except CodeError as e:
         print(f"error: {e}", file=sys.stderr)
         sys.exit(2)
-    return trace_module(prog.module, prog.args, kwargs=prog.kwargs or None), prog
+    return trace_module(prog.module, prog.args, kwargs=prog.kwargs or None, dynamic_shapes=parse_dynamic(args.dynamic)), prog
+
+
+def parse_dynamic(specs: list[str] | None) -> dict | None:
+    """``NAME@INPUT:AXIS`` strings → ``{INPUT: {AXIS: NAME}}``."""
+    if not specs:
+        return None
+    out: dict[str, dict[int, str]] = {}
+    for spec in specs:
+        try:
+            name, rest = spec.split("@", 1)
+            arg, axis = rest.rsplit(":", 1)
+            out.setdefault(arg, {})[int(axis)] = name
+        except ValueError:
+            print(f"error: --dynamic expects NAME@INPUT:AXIS, got {spec!r}", file=sys.stderr)
+            sys.exit(2)
+    return out
 
 
 def register_compile_command(subparsers) -> None:

@@ -29,6 +29,7 @@ def register_run_command(subparsers) -> None:
     p.add_argument("--bench", "-b", action="store_true", help="Time eager PyTorch and the emitted kernels and print a comparison table.")
     p.add_argument("--warmup", type=int, default=10, help="Warmup iterations for --bench (default: 10).")
     p.add_argument("--iters", type=int, default=100, help="Measurement iterations for --bench (default: 100).")
+    p.add_argument("--at", action="append", default=None, metavar="NAME=SIZE", help="With --dynamic: also run and check the expression with symbolic axis NAME at SIZE (repeatable).")
     p.add_argument("--ab", action="append", default=None, metavar="KNOBS", help="Also compile + bench a variant with these knobs pinned ('K1=V1,K2=V2'); repeatable; needs --bench.")
     p.set_defaults(func=handle_run)
 
@@ -118,6 +119,57 @@ def kernel_rows(compiled, bench) -> list[list[str]]:
     return rows
 
 
+def _run_at(be, compiled, module, d_args, d_kwargs, spec: str) -> bool:
+    """Re-run the expression with one symbolic axis resized (random data) and check it against eager."""
+    import torch
+
+    dyn = getattr(compiled, "dynamic", None)
+    try:
+        name, size = spec.split("=", 1)
+        size = int(size)
+    except ValueError:
+        print(f"error: --at expects NAME=SIZE, got {spec!r}", file=sys.stderr)
+        sys.exit(2)
+    if dyn is None or name not in dyn.hints:
+        print(f"error: --at {spec}: {name!r} is not a --dynamic axis of this expression", file=sys.stderr)
+        sys.exit(2)
+    flat = _flatten_tensors(d_args) + _flatten_tensors(d_kwargs)
+    resized = []
+    for t, axes in zip(flat, dyn.input_axes):
+        shape = list(t.shape)
+        for axis, sym in axes.items():
+            if sym == name:
+                shape[axis] = size
+        resized.append(torch.randn(shape, device=t.device).to(t.dtype) if tuple(shape) != tuple(t.shape) else t)
+    it = iter(resized)
+
+    def rebuild(obj):
+        if isinstance(obj, torch.Tensor):
+            return next(it)
+        if isinstance(obj, (tuple, list)):
+            return type(obj)(rebuild(o) for o in obj)
+        if isinstance(obj, dict):
+            return {k: rebuild(v) for k, v in obj.items()}
+        return obj
+
+    n_args, n_kwargs = rebuild(d_args), rebuild(d_kwargs)
+    with torch.no_grad():
+        want = _flatten_tensors(module(*n_args, **n_kwargs))
+    program = be.program(compiled, dict(zip(compiled.inputs, resized)))
+    try:
+        program.run()
+        torch.cuda.synchronize()
+        outs = program.output_tensors()
+        ok_all = True
+        for out_name, w in zip(compiled.outputs, want):
+            ok, line = check_accuracy(outs[out_name], w)
+            ok_all &= ok
+            print(f"{'PASS' if ok else 'FAIL'}  {out_name} at {name}={size}: {line}")
+        return ok_all
+    finally:
+        program.close()
+
+
 def handle_run(args) -> None:
     import torch
 
@@ -159,6 +211,8 @@ def handle_run(args) -> None:
             print(f"{'PASS' if ok else 'FAIL'}  {name}: {line}")
     finally:
         program.close()
+    for spec in args.at or []:
+        ok_all &= _run_at(be, compiled, module, d_args, d_kwargs, spec)
     if not ok_all:
         sys.exit(1)
     if not args.bench:

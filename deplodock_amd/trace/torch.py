@@ -11,6 +11,7 @@ traced shapes and dtypes — the graph dtype *is* the traced dtype.  SDPA's
 from __future__ import annotations
 
 import operator
+from dataclasses import dataclass
 
 from deplodock_amd import dtype as dt
 from deplodock_amd.graph import Graph, Tensor
@@ -29,12 +30,128 @@ def _norm_dim(d: int, rank: int) -> int:
     return d if d >= 0 else d + rank
 
 
+@dataclass
+class DynamicSpec:
+    """How to re-trace a module at other sizes of its symbolic axes.
+
+    The reference marks axes symbolic (``dynamic_shapes={"x": {1: Dim("seq_len")}}``,
+    emmy/compiler/trace/torch.py:52-135) and carries the symbol into the kernels as
+    a runtime ``int``.  Here kernels stay shape-specialised: the graph remembers
+    the module and which axes of which inputs are symbolic, and the backend
+    re-traces and re-lowers per distinct size, keeping the results in an LRU (as
+    the reference keeps one captured graph per symbolic key,
+    emmy/compiler/backend/cuda/program.py:843-907)."""
+
+    module: object
+    example_inputs: tuple
+    kwargs: dict
+    input_axes: list  # per flattened tensor input (= graph input order): {axis: symbol name}
+    hints: dict  # symbol name -> size it was traced at
+
+    def env_of(self, shapes: list) -> dict:
+        """Symbol sizes implied by the shapes of the graph inputs (in graph input order)."""
+        env: dict[str, int] = {}
+        for axes, shape in zip(self.input_axes, shapes):
+            for axis, sym in axes.items():
+                size = int(shape[axis])
+                if env.setdefault(sym, size) != size:
+                    raise ValueError(f"inputs disagree on the size of {sym!r}: {env[sym]} vs {size}")
+        for sym in self.hints:
+            env.setdefault(sym, self.hints[sym])
+        return env
+
+    def retrace(self, env: dict) -> Graph:
+        """The graph of the same module with the symbolic axes at ``env`` sizes."""
+        import torch
+        from torch.utils import _pytree as pytree
+
+        leaves, tree = pytree.tree_flatten((tuple(self.example_inputs), dict(self.kwargs)))
+        out = []
+        t_i = 0
+        for leaf in leaves:
+            if not isinstance(leaf, torch.Tensor):
+                out.append(leaf)
+                continue
+            axes = self.input_axes[t_i]
+            t_i += 1
+            if not axes:
+                out.append(leaf)
+                continue
+            shape = list(leaf.shape)
+            for axis, sym in axes.items():
+                shape[axis] = int(env[sym])
+            out.append(torch.zeros(shape, dtype=leaf.dtype))  # tracing reads shapes and dtypes only
+        args, kwargs = pytree.tree_unflatten(out, tree)
+        g = trace_module(self.module, args, kwargs=kwargs or None)
+        g.dynamic = DynamicSpec(self.module, self.example_inputs, self.kwargs, self.input_axes, self.hints)
+        return g
+
+
+def _dim_name(d) -> str:
+    return d if isinstance(d, str) else getattr(d, "__name__", None) or str(d)
+
+
+def _flatten_dynamic(module, example_inputs: tuple, kwargs: dict, dynamic_shapes: dict) -> tuple[list, dict]:
+    """Per flattened tensor input: ``{axis: symbol}``; plus the traced size of every symbol."""
+    import inspect
+
+    import torch
+    from torch.utils import _pytree as pytree
+
+    params = [p for p in inspect.signature(module.forward).parameters]
+    by_arg: dict[str, object] = {}
+    for i, v in enumerate(example_inputs):
+        by_arg[params[i] if i < len(params) else f"arg{i}"] = v
+    by_arg.update(kwargs)
+    unknown = set(dynamic_shapes) - set(by_arg)
+    if unknown:
+        raise TraceError(f"dynamic_shapes names {sorted(unknown)} are not arguments of forward({', '.join(params)})")
+
+    def spec_leaves(value, spec) -> list:
+        if isinstance(value, torch.Tensor):
+            return [dict(spec or {})]
+        if isinstance(value, (tuple, list)):
+            subs = spec if isinstance(spec, (tuple, list)) else [None] * len(value)
+            return [x for v, s in zip(value, subs) for x in spec_leaves(v, s)]
+        if isinstance(value, dict):
+            return [x for k, v in value.items() for x in spec_leaves(v, (spec or {}).get(k))]
+        return []
+
+    order = list(range(len(example_inputs)))
+    input_axes: list = []
+    for i in order:
+        name = params[i] if i < len(params) else f"arg{i}"
+        input_axes += spec_leaves(example_inputs[i], dynamic_shapes.get(name))
+    for k, v in kwargs.items():
+        input_axes += spec_leaves(v, dynamic_shapes.get(k))
+    leaves = [x for x in pytree.tree_flatten((tuple(example_inputs), dict(kwargs)))[0] if isinstance(x, torch.Tensor)]
+    hints: dict[str, int] = {}
+    named: list = []
+    for leaf, axes in zip(leaves, input_axes):
+        fixed = {}
+        for axis, d in axes.items():
+            sym = _dim_name(d)
+            ax = int(axis) % leaf.dim()
+            fixed[ax] = sym
+            if hints.setdefault(sym, int(leaf.shape[ax])) != int(leaf.shape[ax]):
+                raise TraceError(f"example inputs disagree on the size of {sym!r}")
+        named.append(fixed)
+    return named, hints
+
+
 def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dynamic_shapes=None) -> Graph:
-    """Trace ``module(*example_inputs, **kwargs)`` into a frontend ``Graph``."""
+    """Trace ``module(*example_inputs, **kwargs)`` into a frontend ``Graph``.
+
+    ``dynamic_shapes`` (``{forward-arg name: {axis: Dim or name}}``) marks axes whose
+    size may differ at run time; the graph is traced at the example sizes and
+    carries a :class:`DynamicSpec` on ``graph.dynamic``."""
     import torch
 
-    if dynamic_shapes is not None:
-        raise TraceError("symbolic shapes are not supported by this tracer yet: trace at the concrete shape")
+    if dynamic_shapes:
+        input_axes, hints = _flatten_dynamic(module, tuple(example_inputs), dict(kwargs or {}), dynamic_shapes)
+        g = trace_module(module, example_inputs, kwargs=kwargs)
+        g.dynamic = DynamicSpec(module, tuple(example_inputs), dict(kwargs or {}), input_axes, hints)
+        return g
     module = module.eval()
     with torch.no_grad():
         ep = torch.export.export(module, tuple(example_inputs), kwargs=kwargs or {}, strict=False)

@@ -115,3 +115,19 @@ def test_microbench_kernels_compile_for_gfx950():
         src = _kernel_source(name, k, kind, 256, mfma)
         assert src.count("__builtin_amdgcn_mfma_f32_32x32x16_bf16") == (2 if mfma else 0)
         assert hiprtc.compile_to_hsaco(src, name).stat().st_size > 0
+
+
+def test_dynamic_flag_grammar():
+    from deplodock_amd.commands.compile import parse_dynamic
+
+    assert parse_dynamic(None) is None
+    assert parse_dynamic(["seq_len@x:1", "b@x:0", "seq_len@cos:1"]) == {"x": {1: "seq_len", 0: "b"}, "cos": {1: "seq_len"}}
+    with pytest.raises(SystemExit):
+        parse_dynamic(["seq_len-x-1"])
+
+
+@pytest.mark.gpu
+def test_run_dynamic_axis_at_other_sizes(capsys):
+    main(["run", "--dynamic", "rows@input:1", "--at", "rows=48", "--at", "rows=7", "-c", "nn.Softmax(-1)(torch.randn(2, 32, 512))"])
+    out = capsys.readouterr().out
+    assert out.count("PASS") == 3 and "at rows=48" in out and "at rows=7" in out

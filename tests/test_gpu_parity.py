@@ -266,3 +266,23 @@ def test_run_api_returns_host_arrays_with_bf16_as_bits(device):
     assert out.dtype == np.uint16 and out.shape == (16, 3072)
     want = eager.run_eager(case, device).float().cpu()
     eager.assert_close(torch.from_numpy(O.from_bf16_bits(out)), want, 2e-2, 2e-2, "run() output")
+
+
+def test_c5_block_dynamic_seq_len(device):
+    """One compile with a symbolic ``seq_len``; runs at other lengths go through the per-size variants."""
+    case = eager.qwen3_block_case(seq=64)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs, dynamic_shapes={"x": {1: "seq_len"}, "cos": {1: "seq_len"}, "sin": {1: "seq_len"}}))
+    for seq in (64, 96, 32):
+        other = eager.qwen3_block_case(seq=seq)
+        data = {n: t.to(device) for n, t in zip(compiled.inputs, other.inputs)}
+        prog = be.program(compiled, data)
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            ours = prog.output_tensors()[compiled.outputs[0]]
+            want = eager.run_eager(other, device)
+            eager.assert_close(ours.reshape(want.shape), want, other.rtol, other.atol, f"block with seq_len={seq} through a seq_len=64 compile")
+        finally:
+            prog.close()
+    assert len(compiled.variants) == 3

@@ -167,3 +167,31 @@ def test_cache_is_content_addressed(launcher_lib, tmp_path, monkeypatch):
     monkeypatch.setenv("EMMY_HIPRTC_FLAGS", "-O1")
     assert hiprtc.compile_to_hsaco(src, "k") != p1  # flags are part of the key
     assert not list(tmp_path.glob("*.tmp"))
+
+
+def test_dynamic_shapes_are_specialised_per_size(launcher_lib):
+    """``dynamic_shapes`` marks axes; the backend re-traces and re-lowers per distinct size and keeps an LRU."""
+    case = eager.qwen3_block_case(seq=64)
+    g = trace_module(case.module, case.inputs, dynamic_shapes={"x": {1: "seq_len"}, "cos": {1: "seq_len"}, "sin": {1: "seq_len"}})
+    assert g.dynamic.hints == {"seq_len": 64} and g.dynamic.input_axes == [{1: "seq_len"}] * 3
+    be = HipBackend()
+    compiled = be.compile(g)
+    assert be.variant(compiled, None) is compiled
+
+    def inputs_at(s):
+        return {n: torch.zeros([s if i == 1 else d for i, d in enumerate(t.shape)], dtype=t.dtype) for n, t in zip(compiled.inputs, case.inputs)}
+
+    assert be.variant(compiled, inputs_at(64)) is compiled
+    v96 = be.variant(compiled, inputs_at(96))
+    assert v96 is not compiled and be.variant(compiled, inputs_at(96)) is v96
+    assert v96.nodes[v96.outputs[0]].output.shape[-2:] == (96, 1024) or 96 in v96.nodes[v96.outputs[0]].output.shape
+    assert v96.inputs == compiled.inputs and v96.outputs == compiled.outputs
+    for s in range(1, 12):
+        be.variant(compiled, inputs_at(32 * s + 32))
+    assert len(compiled.variants) == HipBackend.VARIANT_CACHE
+    bad = inputs_at(96)
+    bad[compiled.inputs[1]] = torch.zeros(1, 80, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="disagree"):
+        be.variant(compiled, bad)
+    with pytest.raises(NotImplementedError, match="not arguments"):
+        trace_module(case.module, case.inputs, dynamic_shapes={"nope": {1: "s"}})
