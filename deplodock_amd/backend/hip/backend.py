@@ -40,9 +40,17 @@ class HipBackend(Backend):
         self.bench_wall_timeout_s = bench_wall_timeout_s
         self.bench_compile_timeout_s = bench_compile_timeout_s
         self.bench_run_timeout_s = bench_run_timeout_s
-        self.tune_db = tune_db
         self.device_id = device_id
         self.context = context or Context()
+        # ``tune_db``: None = heuristics only; "auto" = the per-user database; a path; or an open TuneDB.
+        if tune_db is not None:
+            from dataclasses import replace
+
+            from deplodock_amd.tune import TuneDB
+
+            tune_db = tune_db if isinstance(tune_db, TuneDB) else TuneDB(tune_db, arch=self.context.arch)
+            self.context = replace(self.context, tune_db=tune_db)
+        self.tune_db = tune_db
 
     # -- compile ------------------------------------------------------------
     def compile(self, graph: Graph) -> Graph:

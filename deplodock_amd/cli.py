@@ -9,11 +9,13 @@ def build_parser() -> argparse.ArgumentParser:
     from deplodock_amd.commands.compile import register_compile_command
     from deplodock_amd.commands.microbench import register_microbench_command
     from deplodock_amd.commands.run import register_run_command
+    from deplodock_amd.commands.tune import register_tune_command
 
     parser = argparse.ArgumentParser(prog="deplodock_amd", description="MI355X kernel backend: compile / run inline torch expressions")
     sub = parser.add_subparsers(dest="command", required=True)
     register_compile_command(sub)
     register_run_command(sub)
+    register_tune_command(sub)
     register_microbench_command(sub)
     return parser
 

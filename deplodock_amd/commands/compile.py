@@ -31,6 +31,7 @@ def add_common_args(parser) -> None:
         help="Let axis AXIS of forward argument INPUT vary at run time under the name NAME (repeatable), e.g. 'seq_len@x:1'. "
         "Kernels stay specialised per size: another size re-traces and re-lowers on first use.",
     )
+    parser.add_argument("--tune-db", default=None, help="Consult this tune database (path, or 'auto' for the per-user default) for knob pins the environment does not set.")
     parser.add_argument("-v", "--verbose", action="count", default=0)
 
 
@@ -98,7 +99,7 @@ def handle_compile(args) -> None:
     if args.ir == "torch":
         text = graph.pretty_print() + "\n"
     else:
-        compiled = HipBackend(dump=Path(args.dump_dir) if args.dump_dir else None).compile(graph)
+        compiled = HipBackend(dump=Path(args.dump_dir) if args.dump_dir else None, tune_db=getattr(args, "tune_db", None)).compile(graph)
         text = format_kernels(compiled)
         if args.hsaco:
             from deplodock_amd.backend.hip import hiprtc

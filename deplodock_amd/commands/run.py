@@ -185,7 +185,7 @@ def handle_run(args) -> None:
     device = torch.device("cuda:0")
     torch.cuda.set_device(0)
     graph, prog = trace_from_args(args)
-    be = HipBackend(dump=Path(args.dump_dir) if args.dump_dir else None, device_id=0)
+    be = HipBackend(dump=Path(args.dump_dir) if args.dump_dir else None, device_id=0, tune_db=getattr(args, "tune_db", None))
     compiled = be.compile(graph)
 
     module = prog.module.to(device).eval()

@@ -29,6 +29,7 @@ class Context:
     l2_bytes_per_xcd: int = 4 * 1024 * 1024
     backend_name: str = "hip"
     compile_flags: str = ""
+    tune_db: object = None  # a ``deplodock_amd.tune.TuneDB`` the schedule consults for pins, or None
 
     @property
     def cus_per_xcd(self) -> int:

@@ -51,8 +51,21 @@ TILE_CANDIDATES: tuple[tuple[int, int, int, int, str, int], ...] = (
 _FILL_FRACTION = 0.75
 
 
-def _pin(name: str) -> str | None:
-    return config.knob_raw(name)
+def _pin(name: str, tuned: dict | None = None) -> str | None:
+    """The value knob ``name`` is pinned to: the environment first, then the tune database's entry for this kernel."""
+    raw = config.knob_raw(name)
+    if raw is None and tuned:
+        raw = tuned.get(name)
+    return raw
+
+
+def _tuned(body, ctx: Context) -> dict:
+    db = getattr(ctx, "tune_db", None)
+    if db is None:
+        return {}
+    from deplodock_amd.tune import shape_key
+
+    return db.lookup(shape_key(body))
 
 
 def pick_coop(cols: int, elem_bytes: int, rows: int, ctx: Context, *, rotate: bool = False) -> int:
@@ -86,7 +99,8 @@ def _pow2_floor(v: int) -> int:
 
 
 def schedule_row_reduce(body: RowReduce, ctx: Context) -> dict:
-    pinned = _pin("REDUCE")
+    tuned = _tuned(body, ctx)
+    pinned = _pin("REDUCE", tuned)
     plan = None
     if pinned is not None:
         try:
@@ -106,7 +120,7 @@ def schedule_row_reduce(body: RowReduce, ctx: Context) -> dict:
         eb = max(body.x_dtype.nbytes, body.out_dtype.nbytes)
         plan = ReducePlan(coop=pick_coop(body.cols, eb, body.rows, ctx, rotate=body.rotate is not None))
     body.reduce = plan
-    nt = _pin("NT")
+    nt = _pin("NT", tuned)
     if nt is not None:
         body.nontemporal = nt.strip().lower() in ("1", "true", "yes", "on")
     else:
@@ -149,8 +163,32 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context) -> TilePlan
     return best[1]
 
 
+def _check_tile(plan: TilePlan, body: Contraction, ctx: Context, depth: int, dl: bool = False) -> None:
+    """The emitter's shape constraints, checked at schedule time so that an
+    unrealisable pin degrades for the one kernel it does not fit instead of
+    failing the whole lowering."""
+    bk = plan.bk_elems
+    cpr = bk // 8
+    nb = 2 if body.gate_pair else 1
+    threads = plan.block_threads
+    if bk % 8 or bk > 256 or cpr & (cpr - 1):
+        raise ScheduleError(f"slab depth {bk} must be a power-of-two number of 16-byte chunks, at most 256 elements")
+    a_chunks, b_chunks = plan.tile_m * cpr, plan.tile_n * cpr * nb
+    if a_chunks % threads or b_chunks % threads:
+        raise ScheduleError(f"tile {plan.tile_m}x{plan.tile_n}x{bk} does not divide over {threads} threads")
+    if dl and (a_chunks % 64 or b_chunks % 64):
+        raise ScheduleError("direct-to-LDS staging needs whole-wave chunk counts")
+    if (plan.tile_m + plan.tile_n * nb) * bk * 2 * depth > ctx.lds_bytes_per_cu:
+        raise ScheduleError("slabs exceed the LDS")
+    if plan.regs[0] * plan.regs[1] * plan.atom.acc_per_lane * nb > 384:
+        raise ScheduleError("accumulators exceed the register file")
+    if threads > ctx.max_threads_per_block:
+        raise ScheduleError(f"{threads} threads per workgroup is not launchable")
+
+
 def schedule_contraction(body: Contraction, ctx: Context) -> dict:
-    pinned = _pin("TILE")
+    tuned = _tuned(body, ctx)
+    pinned = _pin("TILE", tuned)
     plan = None
     if pinned:
         try:
@@ -159,6 +197,7 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
                 raise ScheduleError(f"atom {plan.atom.name} does not take {body.in_dtype} operands")
             if body.k % plan.bk_elems:
                 raise ScheduleError(f"K={body.k} is not a multiple of the slab depth {plan.bk_elems}")
+            _check_tile(plan, body, ctx, depth=2)
         except ScheduleError as exc:
             logger.warning("EMMY_TILE=%r ignored: %s", pinned, exc)
             plan = None
@@ -169,12 +208,14 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
             plan = TilePlan(atom=ATOMS[plan.atom.name.replace("bf16", atom_dtype)], units=plan.units, regs=plan.regs, bk=plan.bk)
     body.tile = plan
     stage = None
-    pinned_stage = _pin("STAGE")
+    pinned_stage = _pin("STAGE", tuned)
     if pinned_stage:
         try:
             stage = Stage.parse(pinned_stage)
             if stage is not None and stage.transport == "dl" and (plan.bk_elems // plan.atom.k) % 2:
                 raise ScheduleError("direct-to-LDS staging needs an even number of MFMA steps per slab")
+            if stage is not None:
+                _check_tile(plan, body, ctx, depth=max(2, stage.depth), dl=stage.transport == "dl")
         except ScheduleError as exc:
             logger.warning("EMMY_STAGE=%r ignored: %s", pinned_stage, exc)
             stage = None
@@ -194,7 +235,7 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
     workgroup, equal key work for every workgroup) still cover the CUs takes
     ``w2/kv32/s4/p`` instead: 36.6 us on the same shape, where unpaired
     workgroups wait for the one that owns the last rows."""
-    pinned = _pin("FLASH")
+    pinned = _pin("FLASH", _tuned(body, ctx))
     if pinned:
         try:
             body.pair = False

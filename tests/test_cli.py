@@ -131,3 +131,13 @@ def test_run_dynamic_axis_at_other_sizes(capsys):
     main(["run", "--dynamic", "rows@input:1", "--at", "rows=48", "--at", "rows=7", "-c", "nn.Softmax(-1)(torch.randn(2, 32, 512))"])
     out = capsys.readouterr().out
     assert out.count("PASS") == 3 and "at rows=48" in out and "at rows=7" in out
+
+
+@pytest.mark.gpu
+def test_tune_command_fills_a_database_run_then_uses(tmp_path, capsys):
+    db = tmp_path / "tune.db"
+    main(["tune", "--db", str(db), "--rounds", "4", "--iters", "3", "--warmup", "1", "-c", "nn.RMSNorm(1024)(torch.randn(512, 1024))"])
+    out = capsys.readouterr().out
+    assert "row_reduce/r512/c1024" in out and f"database: {db}" in out
+    main(["run", "--tune-db", str(db), "-c", "nn.RMSNorm(1024)(torch.randn(512, 1024))"])
+    assert capsys.readouterr().out.startswith("PASS")
