@@ -85,6 +85,7 @@ def register_compile_command(subparsers) -> None:
     add_common_args(p)
     p.add_argument("--output", "-o", help="Write the kernel sources here instead of stdout")
     p.add_argument("--ir", choices=["torch", "hip"], default="hip", help="Stage to print: the traced graph or the emitted kernels (default).")
+    p.add_argument("--json", default=None, metavar="PATH", help="Also write the selected stage as a JSON graph (a reproducer `run --ir PATH` replays on random data).")
     p.add_argument("--hsaco", action="store_true", help="Also compile each kernel with hipRTC for gfx950 and report code-object sizes.")
     p.set_defaults(func=handle_compile)
 
@@ -96,11 +97,13 @@ def handle_compile(args) -> None:
 
     apply_common_args(args)
     graph, _prog = trace_from_args(args)
+    staged = graph
     if args.ir == "torch":
         text = graph.pretty_print() + "\n"
     else:
         compiled = HipBackend(dump=Path(args.dump_dir) if args.dump_dir else None, tune_db=getattr(args, "tune_db", None)).compile(graph)
         text = format_kernels(compiled)
+        staged = compiled
         if args.hsaco:
             from deplodock_amd.backend.hip import hiprtc
 
@@ -111,6 +114,10 @@ def handle_compile(args) -> None:
                     seen.add(op.kernel_name)
                     path = hiprtc.compile_to_hsaco(op.kernel_source, op.kernel_name)
                     print(f"// {op.kernel_name}: {path.stat().st_size} bytes of gfx950 code object ({path.name})", file=sys.stderr)
+    if args.json:
+        from deplodock_amd import serialize
+
+        serialize.save(staged, args.json)
     if args.output:
         Path(args.output).write_text(text)
     else:

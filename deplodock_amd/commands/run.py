@@ -29,6 +29,7 @@ def register_run_command(subparsers) -> None:
     p.add_argument("--bench", "-b", action="store_true", help="Time eager PyTorch and the emitted kernels and print a comparison table.")
     p.add_argument("--warmup", type=int, default=10, help="Warmup iterations for --bench (default: 10).")
     p.add_argument("--iters", type=int, default=100, help="Measurement iterations for --bench (default: 100).")
+    p.add_argument("--ir", default=None, metavar="PATH", help="Replay a JSON graph written by `compile --json` (traced or lowered stage) on seeded random data; no eager check (there is no module to compare with).")
     p.add_argument("--at", action="append", default=None, metavar="NAME=SIZE", help="With --dynamic: also run and check the expression with symbolic axis NAME at SIZE (repeatable).")
     p.add_argument("--ab", action="append", default=None, metavar="KNOBS", help="Also compile + bench a variant with these knobs pinned ('K1=V1,K2=V2'); repeatable; needs --bench.")
     p.set_defaults(func=handle_run)
@@ -170,6 +171,39 @@ def _run_at(be, compiled, module, d_args, d_kwargs, spec: str) -> bool:
         program.close()
 
 
+def _run_ir(args, device) -> None:
+    """``run --ir``: load a JSON graph, lower it if it is a traced one, run it on random data."""
+    import torch
+
+    from deplodock_amd import serialize
+    from deplodock_amd.backend.hip.backend import HipBackend
+    from deplodock_amd.ir.hip import HipOp
+
+    graph = serialize.load(args.ir)
+    be = HipBackend(dump=Path(args.dump_dir) if args.dump_dir else None, device_id=0, tune_db=getattr(args, "tune_db", None))
+    compiled = graph if any(isinstance(n.op, HipOp) for n in graph.nodes.values()) else be.compile(graph)
+    data = serialize.random_inputs(compiled, seed=args.seed, device=device)
+    program = be.program(compiled, data)
+    try:
+        program.run()
+        torch.cuda.synchronize()
+        for name, t in program.output_tensors().items():
+            if name in compiled.outputs:
+                f = t.float()
+                finite = bool(torch.isfinite(f).all())
+                print(f"{'RAN ' if finite else 'FAIL'}  {name}: shape {tuple(t.shape)} mean {float(f.mean()):.6g} max |y| {float(f.abs().max()):.6g}{'' if finite else ' (non-finite values)'}")
+                if not finite:
+                    sys.exit(1)
+    finally:
+        program.close()
+    if args.bench:
+        res = be.benchmark(compiled, input_data=data, warmup=args.warmup, num_iters=args.iters)
+        us = (res.e2e_ms if res.e2e_ms is not None else res.time_ms) * 1e3
+        print(f"\nprogram: {us:.1f} us over {res.num_launches} launch(es)\n")
+        for line in render_table(["#", "Kernel", "Grid", "Block", "LDS", "us", "%", "Rate", "of peak", "Knobs"], kernel_rows(compiled, res), "llllrrrrrl"):
+            print(line)
+
+
 def handle_run(args) -> None:
     import torch
 
@@ -184,6 +218,9 @@ def handle_run(args) -> None:
         sys.exit(1)
     device = torch.device("cuda:0")
     torch.cuda.set_device(0)
+    if args.ir:
+        _run_ir(args, device)
+        return
     graph, prog = trace_from_args(args)
     be = HipBackend(dump=Path(args.dump_dir) if args.dump_dir else None, device_id=0, tune_db=getattr(args, "tune_db", None))
     compiled = be.compile(graph)

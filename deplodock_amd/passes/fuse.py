@@ -594,14 +594,15 @@ def _rec_rope_pair(c: _Ctx, nid: str) -> bool:
     d = p.d
     if not (a0.div == h0 and a1.div == h1 and a0.stride_lo == d and a1.stride_lo == d and a0.stride_hi == a1.stride_hi and a1.offset == a0.offset + h0 * d and (h0 + h1) * d <= a0.stride_hi):
         return False
-    w0, w1 = _need(c, p0.rms.weight), _need(c, p1.rms.weight)
-    if not (isinstance(g.nodes[p0.rms.weight].op, ConstantOp) and isinstance(g.nodes[p1.rms.weight].op, ConstantOp) and w0.dtype == w1.dtype):
+    # the two weights are only read through their stacked copy: they get no buffers of their own
+    w0, w1 = g.nodes[p0.rms.weight], g.nodes[p1.rms.weight]
+    if not (isinstance(w0.op, ConstantOp) and isinstance(w1.op, ConstantOp) and w0.output.dtype == w1.output.dtype and tuple(w0.output.shape) == tuple(w1.output.shape) == (d,)):
         return False
     heads = h0 + h1
     tokens = p0.mem_shape[0]
     stacked = f"{p0.rms.weight}__x{h0}__{p1.rms.weight}__x{h1}"
     if stacked not in c.out.nodes:
-        c.out.add_constant(stacked, (heads * d,), w0.dtype)
+        c.out.add_constant(stacked, (heads * d,), w0.output.dtype)
         c.out.nodes[stacked].hints["stacked"] = StackedConstant((p0.rms.weight,) * h0 + (p1.rms.weight,) * h1)
     od = p.od
     x = E.Var("x")
@@ -611,7 +612,7 @@ def _rec_rope_pair(c: _Ctx, nid: str) -> bool:
     body = RowReduce(
         rows=tokens * heads, cols=d, x=x0.base, x_dtype=x0.dtype, out=fid, out_dtype=od, stats=(Stat("ss", "sum", x * x),),
         project=E.Var("w") * _round(p.rms.inner, norm), x_addr=RowAddr(offset=a0.offset, div=heads, stride_hi=a0.stride_hi, stride_lo=d),
-        row_operands=(RowOperand("w", w0.dtype, div=1, mod=heads, offset=0), *tables),
+        row_operands=(RowOperand("w", w0.output.dtype, div=1, mod=heads, offset=0), *tables),
     )  # fmt: skip
     body.rotate = RotateHalf(_rope_expr(od))
     body.operand_buffers = {"w": stacked, "cos": cos_v.base, "sin": sin_v.base}
