@@ -127,7 +127,20 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     if unknown:
         raise LoweringError(f"contraction epilogue uses unknown names {sorted(unknown)} (operands belong in `post`)")
 
+    pro = body.a_prologue
+    if pro is not None:
+        if dl:
+            raise LoweringError("contraction: a row prologue transforms the operand in registers; it needs STAGE .../sync")
+        if body.in_dtype.nbytes != 2 or (pro.weight is not None and pro.weight_dtype.nbytes != 2):
+            raise LoweringError("contraction: the row prologue is written for 16-bit operands")
+        bad = (E.variables(pro.stat_pre) - {"x"}) | (E.variables(pro.project) - ({"x", "ss"} | ({"w"} if pro.weight else set())))
+        if bad:
+            raise LoweringError(f"contraction: row prologue uses unknown names {sorted(bad)}")
+        if CPR > 64:
+            raise LoweringError("contraction: a row's slab chunks must sit in one wave for the prologue's row sum")
     params = [f"const {in_c}* __restrict__ A", f"const {in_c}* __restrict__ B"]
+    if pro is not None and pro.weight is not None:
+        params.append(f"const {pro.weight_dtype.c_name}* __restrict__ NW")
     params += [f"const {dt.c_name}* __restrict__ e{i}" for i, (_, dt) in enumerate(body.epilogue_operands)]
     params.append(f"{out_c}* __restrict__ O")
 
@@ -175,7 +188,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   const int lr = lane % AM, lk = lane / AM;  // fragment row, k-group
 """)
     # ---- staging ------------------------------------------------------------
-    a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];")
+    a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else ""))
     a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
     a(r"""  #pragma unroll
   for (int i = 0; i < A_PER_T; ++i) {
@@ -188,6 +201,8 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         a("    la[i] = row * (BK * 2) + emh_swz(row, c) * 16;")
     a(f"    int gr = m0 + row;{' if (gr > M - 1) gr = M - 1;' if m_guard else ''}")
     a(f"    ga[i] = A + {body.a_offset}L + (long)gr * LDA + c * 8;")
+    if pro is not None:
+        a("    ca[i] = c * 8;")
     a("  }")
     a(r"""  #pragma unroll
   for (int i = 0; i < B_PER_T; ++i) {
@@ -245,15 +260,53 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     KS = BK // KSTEP
     if not dl:
         # global -> VGPR -> LDS, one slab ahead, one barrier per slab.
-        a(r"""  u32x4 ra[A_PER_T], rb[B_PER_T];
+        if pro is not None:
+            # Row statistic over the full k extent of this thread's rows: the chunks of
+            # a row's slab sit in CPR consecutive lanes, so a lane sums its own chunk
+            # column over all slabs and a butterfly over those lanes finishes the row.
+            unroll = max(1, min(KT, 32 // max(1, A_PER_T)))
+            a("  float ss[A_PER_T];")
+            a("  #pragma unroll")
+            a("  for (int i = 0; i < A_PER_T; ++i) ss[i] = 0.0f;")
+            a(f"  #pragma unroll {unroll}")
+            a("  for (int kt = 0; kt < KT; ++kt) {")
+            a("    #pragma unroll")
+            a("    for (int i = 0; i < A_PER_T; ++i) {")
+            a(f"      const {frag_t} xv = *(const {frag_t}*)(ga[i] + kt * BK);")
+            a("      #pragma unroll")
+            a("      for (int e = 0; e < 8; ++e) { const float x_ = (float)xv[e]; ss[i] += " + E.render(pro.stat_pre, {"x": "x_"}) + "; }")
+            a("    }")
+            a("  }")
+            a("  #pragma unroll")
+            a("  for (int i = 0; i < A_PER_T; ++i)")
+            a("  #pragma unroll")
+            a("  for (int msk = 1; msk < CPR; msk *= 2) ss[i] += __shfl_xor(ss[i], msk, 64);")
+            wdecl = f" {frag_t} rw[A_PER_T];" if pro.weight is not None else ""
+            a(f"  u32x4 ra[A_PER_T], rb[B_PER_T];{wdecl}")
+            wload = " rw[i] = *(const FRAG_T*)(NW + (kt) * BK + ca[i]);".replace("FRAG_T", frag_t) if pro.weight is not None else ""
+            a("  #define EMH_GLOAD(kt) { \\")
+            a(f'    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) {{ ra[i] = *(const u32x4*)(ga[i] + (kt) * BK);{wload} }} \\')
+            a('    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[i] = *(const u32x4*)(gb[i] + (kt) * BK); }')
+            env = {"x": "(float)xv_[e]", "ss": "ss[i]"}
+            if pro.weight is not None:
+                env["w"] = "(float)rw[i][e]"
+            a("  #define EMH_LSTORE(buf) { \\")
+            a("    unsigned char* s_ = emh_lds + (buf) * SLAB; \\")
+            a('    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) { \\')
+            a(f"      {frag_t} xv_ = __builtin_bit_cast({frag_t}, ra[i]); \\")
+            a(f'      _Pragma("unroll") for (int e = 0; e < 8; ++e) xv_[e] = ({in_c})({E.render(pro.project, env)}); \\')
+            a(f"      *({frag_t}*)(s_ + la[i]) = xv_; }} \\")
+            a('    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[i]; }')
+        else:
+            a(r"""  u32x4 ra[A_PER_T], rb[B_PER_T];
   #define EMH_GLOAD(kt) { \
     _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) ra[i] = *(const u32x4*)(ga[i] + (kt) * BK); \
     _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[i] = *(const u32x4*)(gb[i] + (kt) * BK); }
   #define EMH_LSTORE(buf) { \
     unsigned char* s_ = emh_lds + (buf) * SLAB; \
     _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) *(u32x4*)(s_ + la[i]) = ra[i]; \
-    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[i]; }
-  EMH_GLOAD(0);
+    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[i]; }""")
+        a(r"""  EMH_GLOAD(0);
   EMH_LSTORE(0);
   __syncthreads();
   for (int kt = 0; kt < KT; ++kt) {
@@ -439,11 +492,11 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     return HipOp(
         kernel_source=source,
         kernel_name=name,
-        arg_order=(body.a, body.b, *(body.operand_buffers.get(n, n) for n in epi_names), body.out),
+        arg_order=(body.a, body.b, *((pro.weight,) if pro is not None and pro.weight is not None else ()), *(body.operand_buffers.get(n, n) for n in epi_names), body.out),
         grid=((grid,), (1,), (1,)),
         block=((T,), (1,), (1,)),
         lds_bytes=lds_bytes,
-        comment=f"contraction M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()}",
+        comment=f"contraction M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()}" + (" a=row-normalised" if pro is not None else ""),
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
         knobs={"TILE": plan.spell(), "STAGE": stage.spell()},

@@ -115,6 +115,22 @@ class RowReduce:
         return b
 
 
+@dataclass(frozen=True)
+class RowPrologue:
+    """A row-wise normalisation applied to the ``a`` operand on its way into the
+    contraction, so ``norm -> linear`` is one launch: every workgroup first
+    folds ``stat_pre(x)`` over the full ``k`` extent of its rows (name ``ss``),
+    then maps each element with ``project`` (names ``x``, ``ss`` and, when
+    ``weight`` is set, ``w`` — a length-``k`` vector) while staging the slab.
+    ``project`` carries the producer's own rounding points, so the operand the
+    MFMAs see is bit-for-bit what the separate kernel would have written."""
+
+    stat_pre: Expr
+    project: Expr
+    weight: str | None = None
+    weight_dtype: DType | None = None
+
+
 @dataclass
 class Contraction:
     """``out[m, n] = epilogue(sum_k a[m, k] * b[n, k])`` — both operands
@@ -153,6 +169,7 @@ class Contraction:
     b_offset: int = 0
     out_offset: int = 0
     operand_buffers: dict = field(default_factory=dict)  # epilogue operand name -> buffer id
+    a_prologue: RowPrologue | None = None
 
     def algo_flops(self) -> int:
         return 2 * self.m * self.n * self.k * (2 if self.gate_pair else 1)
@@ -162,6 +179,8 @@ class Contraction:
         b = (self.m * self.k + nb * self.k) * self.in_dtype.nbytes + self.m * self.n * self.out_dtype.nbytes
         for _, dt in self.epilogue_operands:
             b += self.m * self.n * dt.nbytes
+        if self.a_prologue is not None and self.a_prologue.weight is not None:
+            b += self.k * self.a_prologue.weight_dtype.nbytes
         return b
 
 

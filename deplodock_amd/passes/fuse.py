@@ -33,7 +33,7 @@ from deplodock_amd.graph import Graph, Node, Tensor
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir import frontend as F
 from deplodock_amd.ir.base import ConstantOp, InputOp
-from deplodock_amd.ir.tile import Contraction, Flash, Map, MapOperand, RotateHalf, RowAddr, RowOperand, RowReduce, Stat, TileOp
+from deplodock_amd.ir.tile import Contraction, Flash, Map, MapOperand, RotateHalf, RowAddr, RowOperand, RowPrologue, RowReduce, Stat, TileOp
 from deplodock_amd.passes.views import LAYOUT_OPS, NotViewable, View, apply_layout, contiguous_strides, resolve_view
 
 
@@ -157,26 +157,59 @@ def _matrix(view: View, what: str) -> tuple[int, int, int]:
     return rows, view.shape[-1], (ld if rows > 1 else view.shape[-1])
 
 
+def _a_operand(c: _Ctx, x_id: str, absorbers: set[str]) -> tuple[View, RowPrologue | None, list[str]]:
+    """The ``a`` operand of a contraction: ``(view, prologue, extra input buffers)``.
+
+    When ``x_id`` is a row RMSNorm of 16-bit rows that nothing but the
+    contractions in ``absorbers`` reads, the norm is not materialised: the view
+    is the norm's *input* and the prologue carries its statistic and projection
+    (with the producer's rounding points), so ``norm -> linear`` is one launch."""
+    g = c.g
+    node = g.nodes[x_id]
+    if x_id not in c.done and x_id not in g.outputs and not (set(g.consumers(x_id)) - absorbers):
+        m = None
+        if isinstance(node.op, F.RmsNormOp):
+            m = _RmsMatch(x=node.inputs[0], weight=node.inputs[1] if node.op.has_weight else None, eps=node.op.eps, inner=F32, cols=int(node.output.shape[-1]))
+        elif len(node.output.shape) >= 2:
+            m = _match_rms_chain(c, x_id)
+        if m is not None and node.output.dtype.nbytes == 2:
+            try:
+                body, inputs, xv = _rms_body(c, x_id, m, node.output.dtype)
+            except FusionError:
+                body = None
+            if body is not None and isinstance(node.op, F.RmsNormOp) and m.weight is not None:
+                body.project = E.Var("x") * E.Un("rsqrt", E.Var("ss") / float(m.cols) + m.eps) * E.Var("w")
+            if body is not None and xv.dtype == node.output.dtype and body.x_addr.div == 1 and body.x_addr.stride_hi % 8 == 0 and body.x_addr.offset % 8 == 0:
+                wbuf = body.operand_buffers.get("w")
+                wdt = body.col_operands[0][1] if body.col_operands else None
+                if wbuf is None or wdt.nbytes == 2:
+                    shape = tuple(int(d) for d in node.output.shape)
+                    view = View(xv.base, body.x_addr.offset, (body.rows, m.cols), (body.x_addr.stride_hi, 1), xv.dtype)
+                    del shape
+                    return view, RowPrologue(stat_pre=body.stats[0].pre, project=body.project, weight=wbuf, weight_dtype=wdt), ([wbuf] if wbuf else [])
+    return _need(c, x_id), None, []
+
+
 def _linear_parts(c: _Ctx, nid: str):
     node = c.g.nodes[nid]
     if node.op.has_bias:
         raise FusionError("linear with bias is not supported yet")
-    x = _need(c, node.inputs[0])
+    x, pro, extra = _a_operand(c, node.inputs[0], {nid})
     w = _need(c, node.inputs[1])
     m, k, lda = _matrix(x, "linear input")
     n, k2, ldb = _matrix(w, "linear weight")
     if k != k2:
         raise FusionError("linear: inner dimensions differ")
-    return x, w, m, n, k, lda, ldb
+    return x, w, m, n, k, lda, ldb, pro, extra
 
 
 def _rec_linear(c: _Ctx, nid: str) -> bool:
     node = c.g.nodes[nid]
     if not isinstance(node.op, F.LinearOp):
         return False
-    x, w, m, n, k, lda, ldb = _linear_parts(c, nid)
-    body = Contraction(m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset)
-    _emit(c, nid, body, "linear", [x.base, w.base])
+    x, w, m, n, k, lda, ldb, pro, extra = _linear_parts(c, nid)
+    body = Contraction(m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset, a_prologue=pro)
+    _emit(c, nid, body, "rms_norm_linear" if pro else "linear", [x.base, w.base, *extra])
     return True
 
 
@@ -214,7 +247,7 @@ def _rec_linear_siblings(c: _Ctx, nid: str) -> bool:
     ]
     if len(group) < 2:
         return False
-    x = _need(c, x_id)
+    x, pro, extra = _a_operand(c, x_id, set(group))
     m, k, lda = _matrix(x, "linear input")
     if k != int(w0.shape[1]):
         raise FusionError("linear: inner dimensions differ")
@@ -229,8 +262,8 @@ def _rec_linear_siblings(c: _Ctx, nid: str) -> bool:
         c.out.nodes[stacked].hints["stacked"] = StackedConstant(tuple(weights))
     fid = "__".join(group)
     od = node.output.dtype
-    body = Contraction(m=m, n=n_total, k=k, a=x.base, b=stacked, out=fid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset)
-    c.out.add_node(TileOp(name=c.kname("linear"), body=body), list(dict.fromkeys([x.base, stacked])), Tensor(fid, (m, n_total), od), fid)
+    body = Contraction(m=m, n=n_total, k=k, a=x.base, b=stacked, out=fid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset, a_prologue=pro)
+    c.out.add_node(TileOp(name=c.kname("rms_norm_linear" if pro else "linear"), body=body), list(dict.fromkeys([x.base, stacked, *extra])), Tensor(fid, (m, n_total), od), fid)
     col = 0
     for sid, n in zip(group, widths):
         shape = tuple(int(d) for d in g.nodes[sid].output.shape)
@@ -255,14 +288,14 @@ def _rec_linear_residual(c: _Ctx, nid: str) -> bool:
         res = _need(c, res_id)
         if not res.is_contiguous() or res.offset:
             continue
-        x, w, m, n, k, lda, ldb = _linear_parts(c, lin_id)
+        x, w, m, n, k, lda, ldb, pro, extra = _linear_parts(c, lin_id)
         od = node.output.dtype
         body = Contraction(
             m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=od, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset,
-            post=E.Var("y") + E.Var("res"), epilogue_operands=(("res", od),),
+            post=E.Var("y") + E.Var("res"), epilogue_operands=(("res", od),), a_prologue=pro,
         )  # fmt: skip
         body.operand_buffers = {"res": res.base}
-        _emit(c, nid, body, "linear_add", [x.base, w.base, res.base])
+        _emit(c, nid, body, "rms_norm_linear_add" if pro else "linear_add", [x.base, w.base, *extra, res.base])
         return True
     return False
 
@@ -284,7 +317,7 @@ def _rec_gate_up(c: _Ctx, nid: str) -> bool:
         wg, wu = c.g.nodes[gate.inputs[1]], c.g.nodes[up.inputs[1]]
         if not (isinstance(wg.op, ConstantOp) and isinstance(wu.op, ConstantOp)) or wg.output.shape != wu.output.shape:
             continue
-        x = _need(c, gate.inputs[0])
+        x, pro, extra = _a_operand(c, gate.inputs[0], {gate.id, up.id})
         m, k, lda = _matrix(x, "gate/up input")
         n = int(wg.output.shape[0])
         stacked = f"{wg.id}__{wu.id}"
@@ -293,8 +326,8 @@ def _rec_gate_up(c: _Ctx, nid: str) -> bool:
             c.out.nodes[stacked].hints["stacked"] = StackedConstant((wg.id, wu.id))
         od = node.output.dtype
         epi = _round(od, E.Un("silu", _round(od, E.Var("acc")))) * _round(od, E.Var("acc2"))
-        body = Contraction(m=m, n=n, k=k, a=x.base, b=stacked, out=nid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset, epilogue=epi, gate_pair=True)
-        _emit(c, nid, body, "linear_silu_mul", [x.base, stacked])
+        body = Contraction(m=m, n=n, k=k, a=x.base, b=stacked, out=nid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset, epilogue=epi, gate_pair=True, a_prologue=pro)
+        _emit(c, nid, body, "rms_norm_linear_silu_mul" if pro else "linear_silu_mul", [x.base, stacked, *extra])
         return True
     return False
 

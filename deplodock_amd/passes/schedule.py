@@ -219,6 +219,9 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
         except ScheduleError as exc:
             logger.warning("EMMY_STAGE=%r ignored: %s", pinned_stage, exc)
             stage = None
+    if stage is not None and body.a_prologue is not None and stage.transport != "sync":
+        logger.warning("STAGE=%s ignored: the row-normalised operand is transformed in registers (sync staging only)", stage.spell())
+        stage = None
     if stage is None:
         stage = Stage(depth=2, transport="sync")
     body.stage = stage

@@ -75,12 +75,18 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
     compiled = compile_case(eager.qwen3_block_case(seq=64))
     names = [re.sub(r"_[0-9a-f]{6}$", "", k.kernel_name) for k in kernels(compiled)]
     assert names == [
-        "k_rms_norm_reduce", "k_linear", "k_rms_norm_rope",
-        "k_sdpa_reduce", "k_linear_add", "k_rms_norm_reduce", "k_linear_silu_mul", "k_linear_add",
+        "k_rms_norm_linear", "k_rms_norm_rope",
+        "k_sdpa_reduce", "k_linear_add", "k_rms_norm_linear_silu_mul", "k_linear_add",
     ]  # fmt: skip
+    # the two layer norms are prologues of the contractions that read them: the row
+    # statistic is folded over the workgroup's rows before the k loop and the
+    # projection (with the norm's own rounding points) is applied while staging
+    first = kernels(compiled)[0]
+    assert "a=row-normalised" in first.comment and first.arg_order[0] == compiled.inputs[0]
+    assert "__shfl_xor(ss[i], msk, 64)" in first.kernel_source and "emh_round_bf16" in first.kernel_source
     # q, k and v projections are one contraction over the stacked weights; each
     # projection is a column window of its [tokens, 2048 + 1024 + 1024] result
-    qkv = kernels(compiled)[1]
+    qkv = kernels(compiled)[0]
     assert "N=4096" in qkv.comment and qkv.algo_flops == 2 * 64 * 4096 * 1024
     for k in kernels(compiled):
         hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
@@ -88,7 +94,7 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
     assert not any("transpose" in n or "view" in n or "slice" in n for n in compiled.nodes)
     # the query and key head norms + rotary embeddings are one launch over the
     # 16 + 8 heads of every token, with the two norm weights stacked per head
-    rope = kernels(compiled)[2]
+    rope = kernels(compiled)[1]
     assert "rows=1536 cols=128" in rope.comment and "(row / 24) * 4096L + (row % 24) * 128L" in rope.kernel_source
     # q/k/v and gate/up weights are stacked into constants the runtime assembles
     stacked = sorted((n for n in compiled.nodes.values() if n.hints.get("stacked") and len(n.output.shape) == 2), key=lambda n: n.output.shape[0])

@@ -33,10 +33,11 @@ def test_shape_keys_separate_what_the_schedule_depends_on(launcher_lib):
 
     block = fuse(trace_module(*(lambda c: (c.module, c.inputs))(eager.qwen3_block_case(seq=64))))
     keys = [shape_key(n.op.body) for n in block.nodes.values() if hasattr(n.op, "body")]
-    assert len(keys) == 8 and len(set(keys)) == 7  # the two 1024-wide norms share a key
+    assert len(keys) == 6 and len(set(keys)) == 6
     fams = {k.split("/")[0] for k in keys}
     assert fams == set(FAMILY_KNOBS)
-    assert "contraction/m64/n4096/k1024/bf16>bf16/g0/p0" in keys and "contraction/m64/n3072/k1024/bf16>bf16/g1/p0" in keys
+    assert "contraction/m64/n4096/k1024/bf16>bf16/g0/p0/a1" in keys and "contraction/m64/n3072/k1024/bf16>bf16/g1/p0/a1" in keys
+    assert "contraction/m64/n1024/k2048/bf16>bf16/g0/p1/a0" in keys
     assert any(k.startswith("flash/b1/hq16/hkv8/sq64/skv64/d128/c1") for k in keys)
 
 
@@ -49,7 +50,7 @@ def test_schedule_takes_pins_from_the_db_and_env_wins(tmp_path, monkeypatch, lau
     db = TuneDB(tmp_path / "t.db")
     tuned = "a:mfma_16x16x32_bf16/w2x2/f2x2/k4"
     assert tuned != default
-    db.store("contraction/m128/n3072/k1024/bf16>bf16/g0/p0", {"TILE": tuned, "STAGE": "d3/dl"}, 1.0)
+    db.store("contraction/m128/n3072/k1024/bf16>bf16/g0/p0/a0", {"TILE": tuned, "STAGE": "d3/dl"}, 1.0)
     k = kernels(HipBackend(tune_db=db).compile(graph))[0]
     assert k.knobs["TILE"] == tuned and k.knobs["STAGE"] == "d3/dl"
     # another shape is not affected
@@ -60,7 +61,7 @@ def test_schedule_takes_pins_from_the_db_and_env_wins(tmp_path, monkeypatch, lau
     assert kernels(HipBackend(tune_db=db).compile(graph))[0].knobs["TILE"] == "a:mfma_16x16x32_bf16/w1x2/f2x2/k4"
     monkeypatch.delenv("EMMY_TILE")
     # a stored pin the emitter could not realise degrades to the heuristic pick
-    db.store("contraction/m128/n3072/k1024/bf16>bf16/g0/p0", {"TILE": "a:mfma_32x32x16_bf16/w4x4/f8x8/k4"}, 0.5)
+    db.store("contraction/m128/n3072/k1024/bf16>bf16/g0/p0/a0", {"TILE": "a:mfma_32x32x16_bf16/w4x4/f8x8/k4"}, 0.5)
     assert kernels(HipBackend(tune_db=db).compile(graph))[0].knobs["TILE"] == default
     # path form of the constructor argument
     assert kernels(HipBackend(tune_db=str(tmp_path / "t.db")).compile(graph))[0].knobs["TILE"] == default
