@@ -122,7 +122,9 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     out_c = body.out_dtype.c_name
     epi_names = [n for n, _ in body.epilogue_operands]
     epi = body.epilogue if body.epilogue is not None else E.Var("acc")
-    allowed = {"acc"} | ({"acc2"} if gate else set())
+    allowed = {"acc"} | ({"acc2"} if gate else set()) | ({"bias"} if body.bias is not None else set())
+    if body.bias is not None and gate:
+        raise LoweringError("contraction: a bias on a gate/up pair is not supported")
     unknown = E.variables(epi) - allowed
     if unknown:
         raise LoweringError(f"contraction epilogue uses unknown names {sorted(unknown)} (operands belong in `post`)")
@@ -141,6 +143,8 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     params = [f"const {in_c}* __restrict__ A", f"const {in_c}* __restrict__ B"]
     if pro is not None and pro.weight is not None:
         params.append(f"const {pro.weight_dtype.c_name}* __restrict__ NW")
+    if body.bias is not None:
+        params.append(f"const {body.bias_dtype.c_name}* __restrict__ BIAS")
     params += [f"const {dt.c_name}* __restrict__ e{i}" for i, (_, dt) in enumerate(body.epilogue_operands)]
     params.append(f"{out_c}* __restrict__ O")
 
@@ -408,11 +412,17 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     #pragma unroll
     for (int g = 0; g < G; ++g) {
       const int nl = (wn * FN + j) * AM + g * 4 * KG + lk * 4;""")
+        if body.bias is not None:
+            bt4 = _PACK4_T[body.bias_dtype.name]
+            clamp = f"(n0 + nl < N ? n0 + nl : N - 4)" if n_guard else "(n0 + nl)"
+            a(f"      const {bt4} bv = *(const {bt4}*)(BIAS + {clamp});")
         a(f"      {vt4} yo;")
         for r in range(4):
             env = {"acc": f"acc[0][i][j][g * 4 + {r}]"}
             if gate:
                 env["acc2"] = f"acc[1][i][j][g * 4 + {r}]"
+            if body.bias is not None:
+                env["bias"] = f"(float)bv[{r}]"
             a(f"      yo[{r}] = {cast}({E.render(epi, env)});")
         a(f"      *({vt4}*)(emh_lds + ml * CSTRIDE + nl * {esz}) = yo;")
         a("    }")
@@ -461,11 +471,16 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         for i, (_, dt) in enumerate(body.epilogue_operands):
             vt = _PACK4_T[dt.name]
             a(f"      const {vt} ev{i} = *(const {vt}*)(e{i} + (long)m * LDO + n);")
+        if body.bias is not None:
+            bt4 = _PACK4_T[body.bias_dtype.name]
+            a(f"      const {bt4} bv = *(const {bt4}*)(BIAS + n);")
         a(f"      {vt4} yo;")
         for r in range(4):
             env = {"acc": f"acc[0][i][j][g * 4 + {r}]"}
             if gate:
                 env["acc2"] = f"acc[1][i][j][g * 4 + {r}]"
+            if body.bias is not None:
+                env["bias"] = f"(float)bv[{r}]"
             pre = E.render(epi, env)
             if body.post is not None:
                 env2 = {"y": f"(float){cast}({pre})"}
@@ -492,7 +507,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     return HipOp(
         kernel_source=source,
         kernel_name=name,
-        arg_order=(body.a, body.b, *((pro.weight,) if pro is not None and pro.weight is not None else ()), *(body.operand_buffers.get(n, n) for n in epi_names), body.out),
+        arg_order=(body.a, body.b, *((pro.weight,) if pro is not None and pro.weight is not None else ()), *((body.bias,) if body.bias is not None else ()), *(body.operand_buffers.get(n, n) for n in epi_names), body.out),
         grid=((grid,), (1,), (1,)),
         block=((T,), (1,), (1,)),
         lds_bytes=lds_bytes,

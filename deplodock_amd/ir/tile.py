@@ -170,6 +170,8 @@ class Contraction:
     out_offset: int = 0
     operand_buffers: dict = field(default_factory=dict)  # epilogue operand name -> buffer id
     a_prologue: RowPrologue | None = None
+    bias: str | None = None  # length-n vector the epilogue may name ``bias`` (added to the fp32 accumulator)
+    bias_dtype: DType | None = None
 
     def algo_flops(self) -> int:
         return 2 * self.m * self.n * self.k * (2 if self.gate_pair else 1)
@@ -181,6 +183,8 @@ class Contraction:
             b += self.m * self.n * dt.nbytes
         if self.a_prologue is not None and self.a_prologue.weight is not None:
             b += self.k * self.a_prologue.weight_dtype.nbytes
+        if self.bias is not None:
+            b += self.n * self.bias_dtype.nbytes
         return b
 
 

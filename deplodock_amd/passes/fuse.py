@@ -192,8 +192,6 @@ def _a_operand(c: _Ctx, x_id: str, absorbers: set[str]) -> tuple[View, RowProlog
 
 def _linear_parts(c: _Ctx, nid: str):
     node = c.g.nodes[nid]
-    if node.op.has_bias:
-        raise FusionError("linear with bias is not supported yet")
     x, pro, extra = _a_operand(c, node.inputs[0], {nid})
     w = _need(c, node.inputs[1])
     m, k, lda = _matrix(x, "linear input")
@@ -203,13 +201,26 @@ def _linear_parts(c: _Ctx, nid: str):
     return x, w, m, n, k, lda, ldb, pro, extra
 
 
+def _bias_of(c: _Ctx, nid: str, n: int) -> dict:
+    """Contraction keyword arguments that add the linear's bias to the fp32
+    accumulator before the single rounding to the output type."""
+    node = c.g.nodes[nid]
+    if not node.op.has_bias:
+        return {}
+    b = _need(c, node.inputs[2])
+    if b.numel != n or not b.is_contiguous() or b.offset % 4 or n % 4:
+        raise FusionError("linear: the bias must be a dense length-n vector (n a multiple of 4)")
+    return {"bias": b.base, "bias_dtype": b.dtype, "epilogue": E.Var("acc") + E.Var("bias")}
+
+
 def _rec_linear(c: _Ctx, nid: str) -> bool:
     node = c.g.nodes[nid]
     if not isinstance(node.op, F.LinearOp):
         return False
     x, w, m, n, k, lda, ldb, pro, extra = _linear_parts(c, nid)
-    body = Contraction(m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset, a_prologue=pro)
-    _emit(c, nid, body, "rms_norm_linear" if pro else "linear", [x.base, w.base, *extra])
+    bias = _bias_of(c, nid, n)
+    body = Contraction(m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset, a_prologue=pro, **bias)
+    _emit(c, nid, body, "rms_norm_linear" if pro else "linear", [x.base, w.base, *extra, *([bias["bias"]] if bias else [])])
     return True
 
 
@@ -281,7 +292,7 @@ def _rec_linear_residual(c: _Ctx, nid: str) -> bool:
     for li, ri in ((0, 1), (1, 0)):
         lin_id, res_id = node.inputs[li], node.inputs[ri]
         lin = c.g.nodes[lin_id]
-        if not (isinstance(lin.op, F.LinearOp) and c.single_use(lin_id) and not lin.op.has_bias):
+        if not (isinstance(lin.op, F.LinearOp) and c.single_use(lin_id)):
             continue
         if c.g.nodes[res_id].output.shape != node.output.shape or c.g.nodes[res_id].output.dtype != node.output.dtype:
             continue
@@ -292,10 +303,10 @@ def _rec_linear_residual(c: _Ctx, nid: str) -> bool:
         od = node.output.dtype
         body = Contraction(
             m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=od, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset,
-            post=E.Var("y") + E.Var("res"), epilogue_operands=(("res", od),), a_prologue=pro,
+            post=E.Var("y") + E.Var("res"), epilogue_operands=(("res", od),), a_prologue=pro, **(bias := _bias_of(c, lin_id, n)),
         )  # fmt: skip
         body.operand_buffers = {"res": res.base}
-        _emit(c, nid, body, "rms_norm_linear_add" if pro else "linear_add", [x.base, w.base, *extra, res.base])
+        _emit(c, nid, body, "rms_norm_linear_add" if pro else "linear_add", [x.base, w.base, *extra, *([bias["bias"]] if bias else []), res.base])
         return True
     return False
 

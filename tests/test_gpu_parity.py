@@ -365,3 +365,54 @@ def test_row_norm_with_a_second_reader_stays_a_kernel(device):
         eager.assert_close(outs[compiled.outputs[1]].reshape(want_h.shape), want_h, 2e-2, 2e-2, "shared norm")
     finally:
         prog.close()
+
+
+@pytest.mark.parametrize("m,k,n,dtype", [(128, 512, 768, torch.bfloat16), (100, 512, 260, torch.bfloat16), (16, 1024, 3072, torch.float16), (2048, 1024, 3072, torch.bfloat16)])
+def test_linear_with_bias(device, m, k, n, dtype):
+    """``nn.Linear``'s default has a bias: it is added to the fp32 accumulator before the one rounding."""
+    torch.manual_seed(5)
+    mod = nn.Linear(k, n).to(dtype).eval()
+    with torch.no_grad():
+        mod.bias.copy_(torch.randn(n))
+    x = torch.randn(m, k).to(dtype)
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, (x,)))
+    assert sum(isinstance(n_.op, HipOp) for n_ in compiled.nodes.values()) == 1
+    prog = be.program(compiled, {compiled.inputs[0]: x.to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]]
+        want = (x.to(device).float() @ mod.weight.to(device).float().T + mod.bias.to(device).float()).to(dtype)
+        eager.assert_close(ours.reshape(want.shape), want, 2e-2, 2e-2, f"linear+bias {m}x{k}x{n} vs fp32-accumulated reference")
+        with torch.no_grad():
+            eager.assert_close(ours.reshape(want.shape), mod.to(device)(x.to(device)), 2e-2, 2e-2, f"linear+bias {m}x{k}x{n} vs eager")
+    finally:
+        prog.close()
+
+
+def test_residual_linear_with_bias(device):
+    class Res(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = nn.Linear(256, 256)
+
+        def forward(self, x):
+            return x + self.lin(x)
+
+    torch.manual_seed(6)
+    mod = Res().bfloat16().eval()
+    x = torch.randn(192, 256).bfloat16()
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, (x,)))
+    ops = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+    assert len(ops) == 1 and ops[0].kernel_name.startswith("k_linear_add")
+    prog = be.program(compiled, {compiled.inputs[0]: x.to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        with torch.no_grad():
+            want = mod.to(device)(x.to(device))
+        eager.assert_close(prog.output_tensors()[compiled.outputs[0]].reshape(want.shape), want, 2e-2, 2e-2, "x + linear(x) with bias")
+    finally:
+        prog.close()
