@@ -27,7 +27,8 @@ def emit_map(body: Map, name: str, ctx: Context = Context()) -> HipOp:
     dts = [body.out_dtype, *(o.dtype for o in body.operands)]
     V = 16 // max(d.nbytes for d in dts)
     offs = [body.operand_offsets.get(o.name, 0) for o in body.operands]
-    while V > 1 and (body.numel % V or body.inner % V or any(off % V for off in offs)):
+    kinds = {o.index for o in body.operands}
+    while V > 1 and (body.numel % V or ((kinds & {"col", "row"}) and body.inner % V) or any(off % V for off, o in zip(offs, body.operands) if o.index in ("flat", "col"))):
         V //= 2
     chunks = body.numel // V
     grid = max(1, -(-chunks // _T))
@@ -45,6 +46,11 @@ def emit_map(body: Map, name: str, ctx: Context = Context()) -> HipOp:
             o.extend("  " + ln for ln in _load_vec(f"p{i} + {offs[i]}L", "c", op.dtype, V, f"v{i}", False))
         elif op.index == "col":
             o.extend("  " + ln for ln in _load_vec(f"p{i} + {offs[i]}L", f"(c % {body.inner // V}L)", op.dtype, V, f"v{i}", False))
+        elif op.index == "row":
+            # one value per output row: a vector chunk never straddles rows (inner % V == 0)
+            a(f"  {{ const float s_ = (float)p{i}[{offs[i]}L + (c * {V}L) / {body.inner}L]; for (int j = 0; j < {V}; ++j) v{i}[j] = s_; }}")
+        elif op.index == "scalar":
+            a(f"  {{ const float s_ = (float)p{i}[{offs[i]}L]; for (int j = 0; j < {V}; ++j) v{i}[j] = s_; }}")
         else:
             raise LoweringError(f"map operand index scheme {op.index!r} is not supported")
     a(f"  float y[{V}];")

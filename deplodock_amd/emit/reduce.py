@@ -219,6 +219,25 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
             for w in range(1, NW):
                 a(f"  s_{st.name} = {mono}::op(s_{st.name}, emh_part[{s_i}][rib][{w}]);")
 
+    if body.scalar_out:
+        # plain row reduction: every lane holds the statistics; one of them stores the row's value
+        bad = E.variables(body.project) - set(stat_names)
+        if bad or body.rotate is not None or body.col_operands or body.row_operands:
+            raise LoweringError(f"row reduce: a one-value-per-row output maps the statistics only (got {sorted(bad)})")
+        cast_ = "" if body.out_dtype.name == "f32" else f"({body.out_dtype.c_name})"
+        a(f"  if (lane == 0{' && row_ok' if row_guard else ''}) out[row] = {cast_}({E.render(body.project, env_base)});")
+        a("}")
+        return HipOp(
+            kernel_source=prelude.header(prelude.WAVE_REDUCE) + "\n".join(o) + "\n",
+            kernel_name=name,
+            arg_order=(body.x, body.out),
+            grid=((grid,), (1,), (1,)),
+            block=((T,), (1,), (1,)),
+            lds_bytes=0,
+            comment=f"row_reduce rows={body.rows} cols={body.cols} REDUCE={plan.spell()} one value per row",
+            algo_bytes=body.algo_bytes(),
+            knobs={"REDUCE": plan.spell(), "VEC": V, "NT": int(nontemporal)},
+        )
     a(f"  {body.out_dtype.c_name}* orow = out + ({_row_offset(out_addr, 'row')});")
     for ri, ro in enumerate(body.row_operands):
         a(f"  const {ro.dtype.c_name}* rrow{ri} = r{ri} + {ro.offset}L + ((row / {ro.div}) % {ro.mod}) * {body.cols}L;")

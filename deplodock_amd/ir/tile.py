@@ -85,7 +85,8 @@ class RowReduce:
     RMSNorm is ``stats=(ss = sum x*x)``, ``project = x * rsqrt(ss/cols + eps) * w``
     (emmy/compiler/ir/frontend/ir.py:309-312); softmax is ``m = max x``,
     ``d = sum exp(x - m)``, ``project = exp(x - m) / d`` (:354-358).  ``stats``
-    may be empty (a pure row-wise map)."""
+    may be empty (a pure row-wise map).  With ``scalar_out`` the kernel is a plain
+    row reduction (``sum`` / ``mean`` over the last axis): one value per row."""
 
     rows: int
     cols: int
@@ -103,11 +104,12 @@ class RowReduce:
     reduce: ReducePlan = field(default_factory=ReducePlan)
     rows_per_block: int | None = None  # derived from the plan when None
     nontemporal: bool = False
+    scalar_out: bool = False  # the output is one value per row: ``project`` over the statistics only
     # expression name -> buffer (graph node id) for col/row operands; identity when absent
     operand_buffers: dict = field(default_factory=dict)
 
     def algo_bytes(self) -> int:
-        b = self.rows * self.cols * (self.x_dtype.nbytes + self.out_dtype.nbytes)
+        b = self.rows * self.cols * self.x_dtype.nbytes + self.rows * (1 if self.scalar_out else self.cols) * self.out_dtype.nbytes
         for _, dt in self.col_operands:
             b += self.cols * dt.nbytes
         for ro in self.row_operands:
@@ -241,8 +243,8 @@ class Flash:
 @dataclass
 class MapOperand:
     """One pointwise input.  ``index`` names the addressing scheme:
-    ``"flat"`` (same linear index as the output) or ``"row"`` / ``"col"``
-    broadcasts described by the owning ``Map``."""
+    ``"flat"`` (same linear index as the output), ``"col"`` (a vector along the
+    innermost axis), ``"row"`` (one value per output row) or ``"scalar"``."""
 
     name: str
     dtype: DType
@@ -265,7 +267,7 @@ class Map:
     def algo_bytes(self) -> int:
         b = self.numel * self.out_dtype.nbytes
         for o in self.operands:
-            b += (self.numel if o.index == "flat" else self.inner) * o.dtype.nbytes
+            b += {"flat": self.numel, "col": self.inner, "row": self.numel // max(self.inner, 1), "scalar": 1}[o.index] * o.dtype.nbytes
         return b
 
 

@@ -133,7 +133,7 @@ def _materialize(c: _Ctx, nid: str) -> None:
             c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
         c.done[nid] = nid
         return
-    for rec in (_rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_pointwise):
+    for rec in (_rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_pointwise):
         if rec(c, nid):
             return
     raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
@@ -482,6 +482,26 @@ def _rec_softmax(c: _Ctx, nid: str) -> bool:
     return True
 
 
+def _rec_row_sum(c: _Ctx, nid: str) -> bool:
+    """``sum`` / ``mean`` over the innermost axis as a row reduction with one value per row."""
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, (F.MeanOp, F.SumOp)):
+        return False
+    src = c.g.nodes[node.inputs[0]]
+    rank = len(src.output.shape)
+    if node.op.axis != rank - 1:
+        raise FusionError("sum / mean over a non-innermost axis is not supported")
+    xv = _need(c, node.inputs[0])
+    if xv.strides[-1] != 1:
+        raise FusionError("sum / mean: the reduced axis must be contiguous")
+    rows, x_addr = _row_addr(xv)
+    cols = int(src.output.shape[-1])
+    project = E.Var("s") / float(cols) if isinstance(node.op, F.MeanOp) else E.Var("s")
+    body = RowReduce(rows=rows, cols=cols, x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=node.output.dtype, stats=(Stat("s", "sum", E.Var("x")),), project=project, x_addr=x_addr, scalar_out=True)
+    _emit(c, nid, body, "mean_reduce" if isinstance(node.op, F.MeanOp) else "sum_reduce", [xv.base])
+    return True
+
+
 def _match_rope(c: _Ctx, nid: str):
     """``t*cos + cat(neg(t[..., h:]), t[..., :h]) * sin`` → ``(t, cos, sin)`` node ids."""
     g = c.g
@@ -750,47 +770,87 @@ _POINTWISE_FN = {"add": "add", "sub": "sub", "mul": "mul", "div": "div", "maximu
 _POINTWISE_UN = {"neg": "neg", "rsqrt": "rsqrt", "sqrt": "sqrt", "exp": "exp", "silu": "silu", "sigmoid": "sigmoid", "tanh": "tanh", "abs": "abs", "reciprocal": "rcp"}
 
 
+def _pointwise_node_expr(op, args: list[E.Expr]) -> E.Expr | None:
+    """The expression of one element-wise / cast / copy op over its argument expressions."""
+    if isinstance(op, (F.CastOp, F.ContiguousOp)):
+        return args[0]
+    if not isinstance(op, F.ElementwiseOp):
+        return None
+    if op.fn in _POINTWISE_UN and len(args) == 1:
+        return E.Un(_POINTWISE_UN[op.fn], args[0])
+    if op.fn == "pow" and op.scalar == 2.0:
+        return args[0] * args[0]
+    if op.fn in _POINTWISE_FN:
+        if op.scalar is not None:
+            a, b = (E.Const(op.scalar), args[0]) if op.scalar_first else (args[0], E.Const(op.scalar))
+        elif len(args) == 2:
+            a, b = args
+        else:
+            return None
+        return E.Bin(_POINTWISE_FN[op.fn], a, b)
+    raise FusionError(f"element-wise op {op.fn!r} is not supported")
+
+
+_MAX_FUSED_POINTWISE = 24  # ops folded into one map kernel
+
+
 def _rec_pointwise(c: _Ctx, nid: str) -> bool:
-    """Fallback: one element-wise op (or cast / copy) as a flat map over contiguous, same-shape operands."""
-    node = c.g.nodes[nid]
-    op = node.op
+    """Fallback: a tree of element-wise ops / casts as one flat map.  Producers
+    that are element-wise themselves, have this one reader and the same shape
+    are folded in with their own rounding point, so ``exp(neg(x)) * y`` is one
+    kernel; other inputs become operands (same shape, a vector along the last
+    axis, one value per row, or a scalar)."""
+    g = c.g
+    node = g.nodes[nid]
+    if not isinstance(node.op, (F.CastOp, F.ContiguousOp, F.ElementwiseOp)):
+        return False
     od = node.output.dtype
     shape = tuple(int(d) for d in node.output.shape)
-    if isinstance(op, (F.CastOp, F.ContiguousOp)):
-        views = [_need_logical(c, node.inputs[0])]
-        expr = E.Var("a0")
-    elif isinstance(op, F.ElementwiseOp):
-        views = [_need_logical(c, i) for i in node.inputs]
-        vars_ = [E.Var(f"a{i}") for i in range(len(views))]
-        if op.fn in _POINTWISE_UN and len(vars_) == 1:
-            expr = E.Un(_POINTWISE_UN[op.fn], vars_[0])
-        elif op.fn == "pow" and op.scalar == 2.0:
-            expr = vars_[0] * vars_[0]
-        elif op.fn in _POINTWISE_FN:
-            if op.scalar is not None:
-                a, b = (E.Const(op.scalar), vars_[0]) if op.scalar_first else (vars_[0], E.Const(op.scalar))
-            else:
-                a, b = vars_
-            expr = E.Bin(_POINTWISE_FN[op.fn], a, b)
-        else:
-            raise FusionError(f"element-wise op {op.fn!r} is not supported")
-    else:
-        return False
-    operands = []
-    for i, v in enumerate(views):
+    leaves: dict[str, E.Var] = {}  # frontend node id -> operand variable
+    folded = [0]
+
+    def build(cur: str, root: bool) -> E.Expr:
+        n = g.nodes[cur]
+        same_shape = tuple(int(d) for d in n.output.shape) == shape
+        foldable = isinstance(n.op, (F.CastOp, F.ContiguousOp, F.ElementwiseOp)) and same_shape and cur not in c.done and (root or (c.single_use(cur) and folded[0] < _MAX_FUSED_POINTWISE))
+        if not foldable:
+            if cur not in leaves:
+                leaves[cur] = E.Var(f"a{len(leaves)}")
+            return leaves[cur]
+        folded[0] += 1
+        args = [build(i, False) for i in n.inputs]
+        e = _pointwise_node_expr(n.op, args)
+        if e is None:
+            raise FusionError(f"no kernel recognizer for {type(n.op).__name__} at node {cur!r}")
+        return _round(n.output.dtype, e)
+
+    expr = build(nid, True)
+    inner = shape[-1] if shape else 1
+    operands, buffers, offsets = [], {}, {}
+    for leaf_id, var in leaves.items():
+        v = _need_logical(c, leaf_id)
+        lead_ones = len(v.shape) >= 1 and all(d == 1 for d in v.shape[:-1])
         if v.shape == shape and v.is_contiguous():
-            operands.append(MapOperand(f"a{i}", v.dtype, "flat"))
-        elif len(v.shape) >= 1 and v.shape[-1] == shape[-1] and all(d == 1 for d in v.shape[:-1]) and v.strides[-1] == 1:
-            operands.append(MapOperand(f"a{i}", v.dtype, "col"))
+            kind = "flat"
+        elif v.numel == 1:
+            kind = "scalar"
+        elif lead_ones and v.shape[-1] == inner and v.strides[-1] == 1:
+            kind = "col"
+        elif len(v.shape) == len(shape) and v.shape[:-1] == shape[:-1] and v.shape[-1] == 1 and View(v.base, v.offset, v.shape[:-1], v.strides[:-1], v.dtype).is_contiguous():
+            kind = "row"
         else:
-            raise FusionError(f"pointwise operand {i} of {nid!r} needs general broadcasting (shape {v.shape} strides {v.strides})")
+            raise FusionError(f"pointwise operand {leaf_id!r} of {nid!r} needs general broadcasting (shape {v.shape} strides {v.strides} into {shape})")
+        operands.append(MapOperand(var.name, v.dtype, kind))
+        buffers[var.name] = v.base
+        offsets[var.name] = v.offset
     numel = 1
     for d in shape:
         numel *= d
-    body = Map(numel=numel, operands=tuple(operands), expr=_round(od, expr) if od is not F32 else expr, out=nid, out_dtype=od, inner=shape[-1] if shape else 1)
-    body.operand_buffers = {f"a{i}": v.base for i, v in enumerate(views)}
-    body.operand_offsets = {f"a{i}": v.offset for i, v in enumerate(views)}
-    _emit(c, nid, body, f"pointwise_{type(op).__name__.lower().removesuffix('op')}", [v.base for v in views])
+    body = Map(numel=numel, operands=tuple(operands), expr=expr, out=nid, out_dtype=od, inner=inner)
+    body.operand_buffers = buffers
+    body.operand_offsets = offsets
+    label = "pointwise_" + (type(node.op).__name__.lower().removesuffix("op") if folded[0] == 1 else f"fused{folded[0]}")
+    _emit(c, nid, body, label, list(buffers.values()))
     return True
 
 

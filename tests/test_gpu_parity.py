@@ -416,3 +416,40 @@ def test_residual_linear_with_bias(device):
         eager.assert_close(prog.output_tensors()[compiled.outputs[0]].reshape(want.shape), want, 2e-2, 2e-2, "x + linear(x) with bias")
     finally:
         prog.close()
+
+
+def test_fused_pointwise_with_broadcasts_and_row_reductions(device):
+    class Mix(nn.Module):
+        def forward(self, x, y, w, s):
+            centred = x - x.mean(-1, keepdim=True)  # one value per row, broadcast back
+            return torch.exp(torch.neg(centred)) * y + w * s + x.sum(-1, keepdim=True) * 0.01  # vector, scalar
+
+    torch.manual_seed(8)
+    args = (torch.randn(96, 320), torch.randn(96, 320), torch.randn(320), torch.randn(1))
+    mod = Mix().eval()
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, args))
+    prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, args)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        want = mod(*[a.to(device) for a in args])
+        eager.assert_close(prog.output_tensors()[compiled.outputs[0]].reshape(want.shape), want, 1e-5, 1e-5, "fused pointwise + row reductions (fp32)")
+    finally:
+        prog.close()
+
+    class Bf16Chain(nn.Module):
+        def forward(self, x, y):
+            return torch.nn.functional.silu(x) * y + x  # every op rounds to bf16 in eager
+
+    xb, yb = torch.randn(64, 512).bfloat16(), torch.randn(64, 512).bfloat16()
+    compiled = be.compile(trace_module(Bf16Chain().eval(), (xb, yb)))
+    assert sum(isinstance(n_.op, HipOp) for n_ in compiled.nodes.values()) == 1
+    prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, (xb, yb))})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        want = Bf16Chain()(xb.to(device), yb.to(device))
+        eager.assert_close(prog.output_tensors()[compiled.outputs[0]].reshape(want.shape), want, 2e-2, 2e-2, "bf16 element-wise chain")
+    finally:
+        prog.close()

@@ -201,3 +201,34 @@ def test_dynamic_shapes_are_specialised_per_size(launcher_lib):
         be.variant(compiled, bad)
     with pytest.raises(NotImplementedError, match="not arguments"):
         trace_module(case.module, case.inputs, dynamic_shapes={"nope": {1: "s"}})
+
+
+def test_elementwise_trees_fold_into_one_map_kernel(launcher_lib):
+    class Tree(nn.Module):
+        def forward(self, x, y, w):
+            return torch.exp(torch.neg(x)) * y + w  # w: a vector along the last axis
+
+    g = trace_module(Tree(), (torch.randn(8, 64), torch.randn(8, 64), torch.randn(64)))
+    (k,) = kernels(HipBackend().compile(g))
+    assert k.kernel_name.startswith("k_pointwise_fused4") and k.kernel_source.count("expf(") >= 1
+    assert len(k.arg_order) == 4  # x, y, w, out
+
+    class Shared(nn.Module):
+        def forward(self, x):
+            t = torch.exp(x)  # two readers: stays a kernel of its own
+            return t * 2.0, t + 1.0
+
+    names = [k.kernel_name.rsplit("_", 1)[0] for k in kernels(HipBackend().compile(trace_module(Shared(), (torch.randn(4, 32),))))]
+    assert names == ["k_pointwise_elementwise"] * 3
+
+
+def test_row_sum_and_mean_are_row_reductions(launcher_lib):
+    class M(nn.Module):
+        def forward(self, x):
+            return x - x.mean(-1, keepdim=True)
+
+    ks = kernels(HipBackend().compile(trace_module(M(), (torch.randn(16, 256),))))
+    assert [k.kernel_name.rsplit("_", 1)[0] for k in ks] == ["k_mean_reduce", "k_pointwise_elementwise"]
+    assert "one value per row" in ks[0].comment and ks[0].algo_bytes == 16 * 256 * 4 + 16 * 4
+    with pytest.raises(NotImplementedError, match="non-innermost"):
+        HipBackend().compile(trace_module(type("S", (nn.Module,), {"forward": lambda self, x: x.sum(0)})(), (torch.randn(4, 8),)))
