@@ -453,3 +453,34 @@ def test_fused_pointwise_with_broadcasts_and_row_reductions(device):
         eager.assert_close(prog.output_tensors()[compiled.outputs[0]].reshape(want.shape), want, 2e-2, 2e-2, "bf16 element-wise chain")
     finally:
         prog.close()
+
+
+def test_staging_transports_are_bit_identical(device, monkeypatch):
+    """How operands reach LDS (through registers, or direct-to-LDS at any depth) must not change a
+    single output bit: same tile, same MFMA order (the reference pins the same property across its
+    staging transports, tests/compiler/e2e/test_matmul_coverage.py:298-328)."""
+    case = eager.linear_case(m=256, k=1024, n=512)
+    graph = trace_module(case.module, case.inputs)
+    x = case.inputs[0].to(device)
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x2/f1x2/k4")
+    outs = {}
+    for stage in ("d2/sync", "d2/dl", "d3/dl", "d4/dl"):
+        monkeypatch.setenv("EMMY_STAGE", stage)
+        be = HipBackend()
+        compiled = be.compile(graph)
+        (op,) = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+        assert op.knobs["STAGE"] == stage
+        prog = be.program(compiled, {compiled.inputs[0]: x})
+        try:
+            for _ in range(3):  # direct-to-LDS publication races would show as run-to-run differences
+                prog.run()
+                torch.cuda.synchronize()
+                y = prog.output_tensors()[compiled.outputs[0]].clone()
+                if stage in outs:
+                    assert torch.equal(y, outs[stage]), f"{stage}: outputs differ between launches"
+                outs[stage] = y
+        finally:
+            prog.close()
+    for stage, y in outs.items():
+        assert torch.equal(y, outs["d2/sync"]), f"{stage} differs from d2/sync"
+    eager.assert_close(outs["d2/sync"], eager.run_eager(case, device), case.rtol, case.atol, "pinned tile vs eager")
