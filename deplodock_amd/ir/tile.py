@@ -104,6 +104,7 @@ class RowReduce:
     reduce: ReducePlan = field(default_factory=ReducePlan)
     rows_per_block: int | None = None  # derived from the plan when None
     nontemporal: bool = False
+    stream: bool = False  # walk the row once per statistic level instead of keeping it in registers
     scalar_out: bool = False  # the output is one value per row: ``project`` over the statistics only
     # expression name -> buffer (graph node id) for col/row operands; identity when absent
     operand_buffers: dict = field(default_factory=dict)

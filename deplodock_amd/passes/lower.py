@@ -16,6 +16,7 @@ from deplodock_amd.emit.contraction import emit_contraction
 from deplodock_amd.emit.flash import emit_flash
 from deplodock_amd.emit.pointwise import emit_map
 from deplodock_amd.emit.reduce import emit_row_reduce
+from deplodock_amd.emit.reduce_stream import emit_row_reduce_streaming
 from deplodock_amd.graph import Graph
 from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.ir.tile import Contraction, Flash, Map, RowReduce, TileOp
@@ -26,7 +27,7 @@ _PLACEHOLDER = "EMH_KERNEL_NAME_"
 def lower_tile(op: TileOp, ctx: Context) -> HipOp:
     body = op.body
     if isinstance(body, RowReduce):
-        hip = emit_row_reduce(body, _PLACEHOLDER, ctx)
+        hip = (emit_row_reduce_streaming if body.stream else emit_row_reduce)(body, _PLACEHOLDER, ctx)
     elif isinstance(body, Contraction):
         hip = emit_contraction(body, _PLACEHOLDER, ctx)
     elif isinstance(body, Flash):

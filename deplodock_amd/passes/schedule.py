@@ -98,9 +98,19 @@ def _pow2_floor(v: int) -> int:
     return p
 
 
+#: fp32 row elements a lane keeps resident at most (the register-resident emitter's limit)
+_MAX_RESIDENT = 64
+
+
 def schedule_row_reduce(body: RowReduce, ctx: Context) -> dict:
     tuned = _tuned(body, ctx)
     pinned = _pin("REDUCE", tuned)
+    streamable = body.rotate is None and not body.row_operands
+    if streamable and ((pinned or "").endswith("/stream") or -(-body.cols // ctx.max_threads_per_block) > _MAX_RESIDENT):
+        # Too long to hold in registers (or pinned): one workgroup streams the row, one pass per statistic level.
+        body.stream = True
+        body.reduce = ReducePlan(coop=ctx.max_threads_per_block)
+        return {"REDUCE": f"b{ctx.max_threads_per_block}/stream", "NT": 0}
     plan = None
     if pinned is not None:
         try:

@@ -484,3 +484,51 @@ def test_staging_transports_are_bit_identical(device, monkeypatch):
     for stage, y in outs.items():
         assert torch.equal(y, outs["d2/sync"]), f"{stage} differs from d2/sync"
     eager.assert_close(outs["d2/sync"], eager.run_eager(case, device), case.rtol, case.atol, "pinned tile vs eager")
+
+
+@pytest.mark.parametrize("cols", [151936, 70000])
+def test_streamed_softmax_over_a_vocabulary(device, cols):
+    """Rows too long for registers are streamed; max and sum-of-exponentials share one pass (online carrier)."""
+    torch.manual_seed(12)
+    x = 3.0 * torch.randn(5, cols)
+    x[1, 1000:60000] = float("-inf")  # masked logits, including whole chunks of a lane
+    x[2, 7] = 80.0  # one dominant entry
+    be = HipBackend()
+    compiled = be.compile(trace_module(nn.Softmax(-1).eval(), (x,)))
+    (op,) = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+    assert op.knobs["REDUCE"] == "b1024/stream" and "2 reads of the row" in op.comment
+    prog = be.program(compiled, {compiled.inputs[0]: x.to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]]
+        want = torch.softmax(x.to(device), -1)
+        eager.assert_close(ours, want, 1e-5, 1e-9, f"streamed softmax over {cols} columns")
+        assert torch.allclose(ours.sum(-1), torch.ones(5, device=device), atol=1e-4)
+        ref = O.softmax(x[:1, :].double().numpy())
+        eager.assert_close(ours[:1].double().cpu(), torch.from_numpy(ref), 1e-5, 1e-9, "streamed softmax vs numpy restatement")
+    finally:
+        prog.close()
+
+
+def test_streamed_rms_norm_and_pinned_streaming(device, monkeypatch):
+    torch.manual_seed(13)
+    mod = nn.RMSNorm(100000, eps=1e-6).eval()
+    with torch.no_grad():
+        mod.weight.copy_(1.0 + 0.1 * torch.randn(100000))
+    x = torch.randn(3, 100000)
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, (x,)))
+    prog = be.program(compiled, {compiled.inputs[0]: x.to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        eager.assert_close(prog.output_tensors()[compiled.outputs[0]], mod.to(device)(x.to(device)), 1e-5, 1e-6, "streamed RMSNorm")
+    finally:
+        prog.close()
+    # the streaming form can be pinned on a row that would fit in registers; results agree with the resident form
+    case = eager.softmax_case(shape=(2, 3, 64, 2048))
+    monkeypatch.setenv("EMMY_REDUCE", "b1024/stream")
+    ours, want, compiled = run_case(case, device)
+    assert [n_.op.knobs["REDUCE"] for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)] == ["b1024/stream"]
+    eager.assert_close(ours, want, case.rtol, case.atol, "pinned streaming softmax")
