@@ -283,6 +283,14 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
             while body.waves > 1 and heads * -(-body.q_len // (32 * body.waves)) < ctx.compute_units:
                 body.waves //= 2
             body.kv_split = 2 if -(-body.kv_len // body.block_kv) >= 2 else 1
+        # wider heads: shrink the key block, then the key split, until the double-buffered K/V blocks fit the LDS
+        while 2 * body.kv_split * 2 * body.block_kv * body.head_dim * 2 > ctx.lds_bytes_per_cu:
+            if body.block_kv > 32:
+                body.block_kv //= 2
+            elif body.kv_split > 1:
+                body.kv_split //= 2
+            else:
+                break
     return {"FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "")}
 
 

@@ -190,6 +190,18 @@ def test_c4_sdpa_shapes_against_streaming_restatement(device, causal, dims):
     eager.assert_close(ours, torch.from_numpy(ref).float(), 2e-2, 2e-2, f"sdpa {dims} causal={causal} vs streaming restatement")
 
 
+@pytest.mark.parametrize("d,dtype,causal", [(256, torch.bfloat16, True), (256, torch.bfloat16, False), (128, torch.float16, True)])
+def test_c4_wide_heads_and_fp16(device, d, dtype, causal):
+    """head_dim 256 (two 128-wide accumulator groups; the schedule shrinks the key block to fit the LDS) and fp16 operands."""
+    torch.manual_seed(14)
+    q, k, v = (torch.randn(2, h, 192, d).to(dtype) for h in (4, 2, 2))
+    case = eager.Case("wide", eager.Sdpa(causal), (q, k, v), 2e-2, 2e-2)
+    ours, want, _ = run_case(case, device)
+    eager.assert_close(ours, want, 2e-2, 2e-2, f"sdpa d={d} {dtype} causal={causal} vs eager")
+    exact = nn.functional.scaled_dot_product_attention(q.to(device).float(), k.to(device).float(), v.to(device).float(), is_causal=causal, enable_gqa=True)
+    eager.assert_close(ours, exact, 2e-2, 2e-2, f"sdpa d={d} {dtype} causal={causal} vs fp32 eager")
+
+
 @pytest.mark.parametrize("pin", ["w4/kv64/s1", "w4/kv64/s2", "w2/kv64/s2", "w4/kv32/s2", "w1/kv32/s4", "w2/kv32/s4"])
 def test_c4_every_workgroup_shape(device, pin, monkeypatch):
     """Key-split groups, direct-to-LDS staging and the final (m, l, O) merge: the first
