@@ -52,11 +52,14 @@ from deplodock_amd.ir.tile import Flash
 # Each group keeps its own (m, l, O); they are merged through LDS at the end with
 # the same exp-family combine the streaming loop uses.  KVS = 1 is the plain form.
 _SRC = r"""
-EMH_DEV int emh_kswz(int row, int c) { return c ^ (row % CPR); }
+// K rows are XOR-swizzled per 256-byte bank line (KRPL rows of it), so the 16 rows
+// a fragment read touches at one k position land in 16 different bank groups.
+EMH_DEV int emh_kswz(int row, int c) { return c ^ ((row / KRPL) % CPR); }
 // V keeps [key][d] order; its 16-byte chunks are XOR-swizzled in groups of four
 // so the four consecutive key rows one transposing read touches sit in four
 // different bank quarters.
-EMH_DEV int emh_vswz(int row, int c) { return c ^ ((row % 4) << 2); }
+#define EMH_VROT(row) (D >= 128 ? ((row) % 4) : (((row) >> 1) & 1))  /* 128-byte rows: two rows share a bank line */
+EMH_DEV int emh_vswz(int row, int c) { return c ^ (EMH_VROT(row) << 2); }
 EMH_DEV float emh_xor32(float v) { return __shfl_xor(v, 32, 64); }
 typedef short emh_s16x4 __attribute__((ext_vector_type(4)));
 #define KBYTES (BKV * D * 2)
@@ -113,8 +116,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   constexpr int PER_T = KVS * CHUNKS / NT;     // chunks per thread, per operand
   // Chunk q = tid + i*NT of a step: block g = q / CHUNKS, row (q % CHUNKS) / CPR,
   // slot q % CPR = tid % CPR.  CHUNKS is a multiple of NT, so g and the row offset
-  // of iteration i are compile-time; with 256 or more threads the row offset is a
-  // multiple of 16 and the swizzled chunk choice is the same for every i.
+  // of iteration i are compile-time.
   const int st_row = tid / CPR, st_pos = tid % CPR;
   const ELT* gk_lane = kbase + (long)st_row * K_SS;
   const ELT* gv_lane = vbase + (long)st_row * V_SS;
@@ -125,7 +127,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       const int g_ = (i * NT) / CHUNKS, ro_ = ((i * NT) % CHUNKS) / CPR; \
       long krow_ = (long)((st) * KVS + g_) * BKV + ro_; \
       if (SKV % (KVS * BKV) != 0) { const long lim_ = SKV - 1 - st_row; if (krow_ > lim_) krow_ = lim_; } \
-      const int kc_ = emh_kswz(st_row + ro_ % CPR, st_pos), vc_ = emh_vswz(st_row + ro_ % 4, st_pos); \
+      const int kc_ = emh_kswz(st_row + ro_, st_pos), vc_ = emh_vswz(st_row + ro_, st_pos); \
       unsigned char* dk_ = sb_ + g_ * 2 * KBYTES + ((i * NT) % CHUNKS) * 16; \
       __builtin_amdgcn_global_load_lds((const void*)(gk_lane + krow_ * K_SS + kc_ * 8), (__attribute__((address_space(3))) void*)dk_, 16, 0, 0); \
       __builtin_amdgcn_global_load_lds((const void*)(gv_lane + krow_ * V_SS + vc_ * 8), (__attribute__((address_space(3))) void*)(dk_ + KBYTES), 16, 0, 0); } }
@@ -153,9 +155,9 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   // operand fragment of an MFMA step is two such reads and no shuffling.
   const int i16 = lane % 16, q4 = i16 / 4;
   const int v_lane = (4 * lh + q4) * (D * 2) + ((lane % 32) / 16) * 32 + (i16 % 4) * 8;
-  int v_tile[4];
+  int v_tile[TG];
   #pragma unroll
-  for (int T = 0; T < 4; ++T) v_tile[T] = v_lane + ((T ^ q4) * 64);
+  for (int T = 0; T < TG; ++T) v_tile[T] = v_lane + ((T ^ EMH_VROT(q4)) * 64);
 
   EMH_STAGE(0, 0);
   EMH_DMA_FENCE();
@@ -231,16 +233,14 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         #pragma unroll
         for (int t = 0; t < 8; ++t) pf[t] = (ELT)sacc[u][8 * s + t];
         #pragma unroll
-        for (int dg = 0; dg < D / 128; ++dg)
-        #pragma unroll
-        for (int T = 0; T < 4; ++T) {
-          const unsigned char* vp = sV + (32 * u + 16 * s) * (D * 2) + dg * 256 + v_tile[T];
+        for (int dt = 0; dt < D / 32; ++dt) {
+          const unsigned char* vp = sV + (32 * u + 16 * s) * (D * 2) + (dt / TG) * 256 + v_tile[dt % TG];
           const emh_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) emh_s16x4*)(vp));
           const emh_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) emh_s16x4*)(vp + 8 * (D * 2)));
           const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
           u32x4 av;
           av[0] = l2[0]; av[1] = l2[1]; av[2] = h2[0]; av[3] = h2[1];
-          oacc[dg * 4 + T] = MFMA(__builtin_bit_cast(FRAG, av), pf, oacc[dg * 4 + T], 0, 0, 0);
+          oacc[dt] = MFMA(__builtin_bit_cast(FRAG, av), pf, oacc[dt], 0, 0, 0);
         }
       }
     }
@@ -304,8 +304,8 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     D = body.head_dim
     if body.dtype.name not in ("bf16", "f16"):
         raise LoweringError("flash: MFMA tier needs 16-bit operands")
-    if D % 128 or D > 256:
-        raise LoweringError(f"flash: head_dim {D} must be 128 or 256 on this tier")
+    if D not in (64, 128, 256):
+        raise LoweringError(f"flash: head_dim {D} must be 64, 128 or 256 on this tier")
     if body.q_heads % body.kv_heads:
         raise LoweringError("flash: q heads must be a multiple of kv heads")
     waves = body.waves
@@ -341,6 +341,8 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "BKV": BKV,
         "KVS": kvs,
         "CPR": D // 8,
+        "KRPL": max(1, 16 // (D // 8)),
+        "TG": min(4, D // 32),
         "SQ": body.q_len,
         "SKV": body.kv_len,
         "HQ": body.q_heads,

@@ -190,9 +190,10 @@ def test_c4_sdpa_shapes_against_streaming_restatement(device, causal, dims):
     eager.assert_close(ours, torch.from_numpy(ref).float(), 2e-2, 2e-2, f"sdpa {dims} causal={causal} vs streaming restatement")
 
 
-@pytest.mark.parametrize("d,dtype,causal", [(256, torch.bfloat16, True), (256, torch.bfloat16, False), (128, torch.float16, True)])
+@pytest.mark.parametrize("d,dtype,causal", [(256, torch.bfloat16, True), (256, torch.bfloat16, False), (128, torch.float16, True), (64, torch.bfloat16, True), (64, torch.bfloat16, False), (64, torch.float16, True)])
 def test_c4_wide_heads_and_fp16(device, d, dtype, causal):
-    """head_dim 256 (two 128-wide accumulator groups; the schedule shrinks the key block to fit the LDS) and fp16 operands."""
+    """head_dim 256 (two 128-wide accumulator groups; the schedule shrinks the key block to fit the LDS),
+    head_dim 64 (128-byte K/V rows: two rows per bank line, their own swizzles) and fp16 operands."""
     torch.manual_seed(14)
     q, k, v = (torch.randn(2, h, 192, d).to(dtype) for h in (4, 2, 2))
     case = eager.Case("wide", eager.Sdpa(causal), (q, k, v), 2e-2, 2e-2)
@@ -200,6 +201,17 @@ def test_c4_wide_heads_and_fp16(device, d, dtype, causal):
     eager.assert_close(ours, want, 2e-2, 2e-2, f"sdpa d={d} {dtype} causal={causal} vs eager")
     exact = nn.functional.scaled_dot_product_attention(q.to(device).float(), k.to(device).float(), v.to(device).float(), is_causal=causal, enable_gqa=True)
     eager.assert_close(ours, exact, 2e-2, 2e-2, f"sdpa d={d} {dtype} causal={causal} vs fp32 eager")
+
+
+@pytest.mark.parametrize("pin", ["w4/kv64/s2", "w2/kv64/s1", "w1/kv64/s2", "w2/kv128/s2", "w2/kv64/s2/p"])
+def test_c4_head_dim_64_workgroup_shapes(device, pin, monkeypatch):
+    monkeypatch.setenv("EMMY_FLASH", pin)
+    torch.manual_seed(15)
+    q, k, v = (torch.randn(1, h, 512, 64).bfloat16() for h in (8, 2, 2))
+    case = eager.Case("d64", eager.Sdpa(True), (q, k, v), 2e-2, 2e-2)
+    ours, want, compiled = run_case(case, device)
+    assert [n_.op.knobs["FLASH"] for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)] == [pin]
+    eager.assert_close(ours, want, 2e-2, 2e-2, f"sdpa d=64 {pin} vs eager")
 
 
 @pytest.mark.parametrize("pin", ["w4/kv64/s1", "w4/kv64/s2", "w2/kv64/s2", "w4/kv32/s2", "w1/kv32/s4", "w2/kv32/s4"])
