@@ -393,6 +393,8 @@ class CompiledProgram:
         for zp, words in zero_packs:
             zgrid = (max(1, min(1024, -(-words // 256))), 1, 1)
             self.lib.launch(self.compiled.kernels[_ZERO_KERNEL_NAME].fn, zgrid, (256, 1, 1), 0, stream, zp)
+        if grid[0] * grid[1] * grid[2] == 0:
+            return  # an empty index space (zero rows): nothing to compute, and the driver rejects empty grids
         self.lib.launch(self.compiled.kernels[ln.kernel_name].fn, grid, block, ln.lds_bytes, stream, pack)
 
     def run(self, stream: int | None = None) -> None:

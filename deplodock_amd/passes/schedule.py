@@ -171,10 +171,10 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
         plan = TilePlan(atom=atom, units=(wm, wn), regs=(fm, fn), bk=bk)
         groups = -(-m // tm) * -(-n // tn)
         # penalise tiles that mostly hang over the edge of a small problem
-        waste = (-(-m // tm) * tm * -(-n // tn) * tn) / float(m * n)
+        waste = (-(-m // tm) * tm * -(-n // tn) * tn) / float(max(m * n, 1))
         if groups >= _FILL_FRACTION * ctx.compute_units and waste < 1.5:
             return plan
-        score = (min(groups, ctx.compute_units) / waste, tm * tn)
+        score = (min(groups, ctx.compute_units) / max(waste, 1e-9), tm * tn)
         if best is None or score > best[0]:
             best = (score, plan)
     if best is None:

@@ -8,6 +8,7 @@ import asyncio
 import numpy as np
 import pytest
 import torch
+from torch import nn
 
 from deplodock_amd import HipBackend, trace_module
 from deplodock_amd.backend.hip import launcher, program
@@ -131,3 +132,19 @@ def test_launch_errors_surface_as_exceptions(launcher_lib, device):
     torch.cuda.synchronize()
     assert float(buf.sum()) == 64.0
     np.testing.assert_equal(launcher_lib.func_attributes(k.fn)["private_bytes"], 0)
+
+
+@pytest.mark.parametrize("which", ["rms", "softmax", "linear"])
+def test_empty_inputs_run_and_return_empty_outputs(device, which):
+    """Zero rows: nothing is launched (the driver rejects empty grids) and the outputs are empty, as in eager."""
+    if which == "rms":
+        mod, x = nn.RMSNorm(64).eval(), torch.randn(0, 64)
+    elif which == "softmax":
+        mod, x = nn.Softmax(-1).eval(), torch.randn(3, 0, 16)
+    else:
+        mod, x = nn.Linear(32, 16, bias=False).bfloat16().eval(), torch.randn(0, 32).bfloat16()
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, (x,)))
+    res, _ = be.run(compiled, input_data={compiled.inputs[0]: x.to(device)})
+    out = res.outputs[compiled.outputs[0]]
+    assert out.size == 0 and tuple(out.shape) == tuple(mod(x).shape)
