@@ -65,6 +65,11 @@ typedef short emh_s16x4 __attribute__((ext_vector_type(4)));
 #define KBYTES (BKV * D * 2)
 #define WQ (NT / 64 / KVS)           /* waves (32-row groups) per key-split group */
 #define STEP_BYTES (KVS * 2 * KBYTES)  /* one step: K and V block of every group */
+#define QCHUNKS (BQ * CPR)             /* 16-byte chunks of a workgroup's Q (and O) tile */
+#define RPL (D / 32 * 16)              /* output registers per lane */
+#define RPG (RPL / KVS)                /* ... of which each key-split group finishes this many */
+#define OSW (D / 4 < 32 ? D / 4 : 32)  /* rows over which the O tile's 8-byte slots are XOR-swizzled */
+#define OACC(f) oacc[(f) / 16][(f) % 16]
 
 extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q, const ELT* __restrict__ Kp,
                                                       const ELT* __restrict__ Vp, ELT* __restrict__ Op) {
@@ -94,8 +99,22 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   const int qw0 = q0 + wq * 32;
   const int qrow = qw0 + lq;
 
+  // A lane's Q fragments are 16-byte pieces of one row: read straight from global
+  // memory a wave's load touches 32 rows per instruction.  With LDS to spare the
+  // tile comes in through the same swizzled direct-to-LDS path as a K block (whole
+  // rows per instruction) and the fragments are read from there.
   FRAG qf[D / 16];
-  {
+  if (Q_LDS) {
+    #pragma unroll
+    for (int c0 = 0; c0 < QCHUNKS; c0 += NT) {
+      if (QCHUNKS % NT == 0 || c0 + (tid - lane) < QCHUNKS) {  // whole waves: QCHUNKS is a multiple of 64
+        const int r_ = (c0 + tid) / CPR, p_ = (c0 + tid) % CPR;
+        const int qr_ = q0 + r_ < SQ ? q0 + r_ : SQ - 1;
+        __builtin_amdgcn_global_load_lds((const void*)(qbase + (long)qr_ * Q_SS + emh_kswz(r_, p_) * 8),
+                                         (__attribute__((address_space(3))) void*)(lds + Q_OFF_LDS + (c0 + tid - lane) * 16), 16, 0, 0);
+      }
+    }
+  } else {
     const int qr = qrow < SQ ? qrow : SQ - 1;
     const ELT* qp = qbase + (long)qr * Q_SS + 8 * lh;
     #pragma unroll
@@ -162,6 +181,11 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   EMH_STAGE(0, 0);
   EMH_DMA_FENCE();
   __syncthreads();
+  if (Q_LDS) {
+    const int qr_ = wq * 32 + lq;
+    #pragma unroll
+    for (int kk = 0; kk < D / 16; ++kk) qf[kk] = *(const FRAG*)(lds + Q_OFF_LDS + qr_ * (D * 2) + emh_kswz(qr_, kk * 2 + lh) * 16);
+  }
 
   for (int st = 0; st < nsteps; ++st) {
     if (st + 1 < nsteps) EMH_STAGE(st + 1, (st + 1) & 1);
@@ -248,56 +272,132 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
     __syncthreads();
   }
 
-  // ---- merge the key-split groups pairwise through LDS: in round r, group g with
-  // g % 2^(r+1) == 2^r parks (m, l, O) and group g - 2^r folds it in ----
-  float* park = (float*)lds;  // [slot][wq][66][64 lanes]; the staging buffers are free after the last barrier
-  #pragma unroll 1
-  for (int sft = 1; sft < KVS; sft *= 2) {
-    float* pw = park + ((grp / (2 * sft)) * WQ + wq) * (D / 32 * 16 + 2) * 64 + lane;
-    if (grp % (2 * sft) == sft) {
-      pw[0] = m_ref;
-      pw[64] = l_run;
-      #pragma unroll
-      for (int t = 0; t < D / 32; ++t)
-      #pragma unroll
-      for (int r = 0; r < 16; ++r) pw[(2 + t * 16 + r) * 64] = oacc[t][r];
-    }
-    __syncthreads();
-    if (grp % (2 * sft) == 0 && grp + sft < KVS) {
-      const float m_o = pw[0], l_o = pw[64];
-      const float m_new = fmaxf(m_ref, m_o);
-      const float a_s = EXP2(m_ref - m_new), a_o = EXP2(m_o - m_new);
-      m_ref = m_new;
-      l_run = l_run * a_s + l_o * a_o;
-      #pragma unroll
-      for (int t = 0; t < D / 32; ++t)
-      #pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[t][r] = oacc[t][r] * a_s + pw[(2 + t * 16 + r) * 64] * a_o;
+  // ---- close.  The key-split groups share the final combine: group g finishes
+  // registers [g*RPG, (g+1)*RPG) of its rows' RPL output registers.  Every group
+  // parks the registers the others own, and its (m, l); after one barrier each
+  // combines its share with the same exp-family merge the streaming loop uses,
+  // scales by 1/l and puts the 16-bit result into the O tile in LDS, which leaves
+  // through 16-byte stores of whole rows.  (The staging buffers are free after the
+  // loop's last barrier; the O tile sits behind the first of them, so the next
+  // pass may start staging without another barrier.)
+  if (KVS > 1) {
+    float* park = (float*)lds;
+    float* pml = (float*)(lds + PARK_ML) + ((grp * WQ + wq) * 2) * 64 + lane;
+    pml[0] = m_ref;
+    pml[64] = l_run;
+    #pragma unroll
+    for (int g = 0; g < KVS; ++g) {
+      if (g == grp) {
+        #pragma unroll
+        for (int h = 0; h < KVS; ++h) {
+          if (h != g) {
+            float* pw = park + (((h * (KVS - 1) + (g - (g > h ? 1 : 0))) * WQ + wq) * RPG) * 64 + lane * 4;
+            #pragma unroll
+            for (int r4 = 0; r4 < RPG / 4; ++r4) {
+              f32x4 t;
+              #pragma unroll
+              for (int j = 0; j < 4; ++j) t[j] = OACC(h * RPG + 4 * r4 + j);
+              *(f32x4*)(pw + r4 * 256) = t;
+            }
+          }
+        }
+      }
     }
     __syncthreads();
   }
-
-  if (grp == 0) {
-    const float l_tot = l_run + emh_xor32(l_run);
-    const float inv = 1.0f / l_tot;
-    if (qrow < SQ) {
-      ELT* op = Op + O_OFF + (long)batch * O_SB + (long)head * O_SH + (long)qrow * O_SS;
-      // Register r = 4*i + j of tile T is d = 32*T + 8*i + 4*lh + j.
+  #pragma unroll
+  for (int g = 0; g < KVS; ++g) {
+    if (g == grp) {
+      float a_own = 1.0f, l_tot = l_run;
+      float a_o[KVS];
+      if (KVS > 1) {
+        const float* pml = (const float*)(lds + PARK_ML) + lane;
+        float m_all = m_ref, m_o[KVS], l_o[KVS];
+        #pragma unroll
+        for (int h = 0; h < KVS; ++h) {
+          if (h != g) {
+            m_o[h] = pml[((h * WQ + wq) * 2) * 64];
+            l_o[h] = pml[((h * WQ + wq) * 2 + 1) * 64];
+            m_all = fmaxf(m_all, m_o[h]);
+          }
+        }
+        a_own = EXP2(m_ref - m_all);
+        l_tot = l_run * a_own;
+        #pragma unroll
+        for (int h = 0; h < KVS; ++h) {
+          if (h != g) {
+            a_o[h] = EXP2(m_o[h] - m_all);
+            l_tot += l_o[h] * a_o[h];
+          }
+        }
+      }
+      l_tot += emh_xor32(l_tot);
+      const float inv = 1.0f / l_tot;
+      const int orow = wq * 32 + lq;
       #pragma unroll
-      for (int T = 0; T < D / 32; ++T)
-      #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int r4 = 0; r4 < RPG / 4; ++r4) {
+        f32x4 acc;
+        #pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = OACC(g * RPG + 4 * r4 + j) * a_own;
+        if (KVS > 1) {
+          #pragma unroll
+          for (int h = 0; h < KVS; ++h) {
+            if (h != g) {
+              const f32x4 t = *(const f32x4*)((const float*)lds + (((g * (KVS - 1) + (h - (h > g ? 1 : 0))) * WQ + wq) * RPG) * 64 + lane * 4 + r4 * 256);
+              #pragma unroll
+              for (int j = 0; j < 4; ++j) acc[j] += t[j] * a_o[h];
+            }
+          }
+        }
         PACK4 y;
         #pragma unroll
-        for (int j = 0; j < 4; ++j) y[j] = (ELT)(oacc[T][4 * i + j] * inv);
-        *(PACK4*)(op + 32 * T + 8 * i + 4 * lh) = y;
+        for (int j = 0; j < 4; ++j) y[j] = (ELT)(acc[j] * inv);
+        // Registers 4i .. 4i+3 of tile T are d = 32*T + 8*i + 4*lh + (0..3): 8-byte slot 8*T + 2*i + lh of the row.
+        const int f = g * RPG + 4 * r4;
+        const int sl = 8 * (f / 16) + 2 * ((f % 16) / 4) + lh;
+        *(PACK4*)(lds + O_OFF_LDS + orow * (D * 2) + ((sl ^ (orow % OSW)) * 8)) = y;
       }
     }
   }
-  if (PAIR) __syncthreads();  // the staging buffers are rewritten by the next pass
+  __syncthreads();
+  {
+    ELT* obase = Op + O_OFF + (long)batch * O_SB + (long)head * O_SH;
+    #pragma unroll
+    for (int c0 = 0; c0 < QCHUNKS; c0 += NT) {
+      const int c = c0 + tid;
+      if (QCHUNKS % NT == 0 || c < QCHUNKS) {
+        const int r = c / CPR, pc = c % CPR, x = r % OSW;
+        // slots 2*pc and 2*pc + 1 of the row sit XOR x away: the same 16 bytes, halves swapped when x is odd
+        const u32x4 t = *(const u32x4*)(lds + O_OFF_LDS + r * (D * 2) + ((pc ^ (x >> 1)) * 16));
+        u32x4 y;
+        y[0] = (x & 1) ? t[2] : t[0]; y[1] = (x & 1) ? t[3] : t[1];
+        y[2] = (x & 1) ? t[0] : t[2]; y[3] = (x & 1) ? t[1] : t[3];
+        if (q0 + r < SQ) *(u32x4*)(obase + (long)(q0 + r) * O_SS + pc * 8) = y;
+      }
+    }
+  }
   }
 }
 """
+
+
+def lds_plan(waves: int, kvs: int, bkv: int, head_dim: int, limit: int) -> dict:
+    """LDS layout of a workgroup: ``[2 staging buffers | Q tile]``.
+
+    After the key loop the staging buffers hold the parked partial results of the
+    key-split groups (``(kvs-1) * waves * registers`` lane-vectors and an ``(m, l)``
+    table) and, behind both the parked data and the first staging buffer, the O
+    tile.  The Q tile is staged through LDS only when it fits behind all of that;
+    ``q_off`` is ``None`` when the fragments are read from global memory instead."""
+    step = kvs * 2 * bkv * head_dim * 2
+    regs = head_dim // 32 * 16
+    park_ml = (kvs - 1) * waves * regs * 256
+    park = park_ml + (kvs * waves * 512 if kvs > 1 else 0)
+    tile = 32 * waves * head_dim * 2
+    o_off = max(park, step)
+    end = max(2 * step, o_off + tile)
+    q_off = end if end + tile <= limit else None
+    return {"bytes": end + (tile if q_off is not None else 0), "q_off": q_off, "o_off": o_off, "park_ml": park_ml}
 
 
 def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
@@ -319,14 +419,20 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         raise LoweringError(f"flash: {waves} x {kvs} waves exceed {ctx.max_threads_per_block} threads")
     if (BKV * D // 8) % NT:
         raise LoweringError("flash: a key block's 16-byte chunks must be a multiple of the workgroup's threads")
-    lds = max(2 * kvs * 2 * BKV * D * 2, ((kvs + 1) // 2) * waves * (D // 32 * 16 + 2) * 64 * 4 if kvs > 1 else 0)
+    if (D // 32 * 16) % (4 * kvs):
+        raise LoweringError(f"flash: {kvs} key-split groups cannot share the {D // 32 * 16} output registers of a lane")
+    plan = lds_plan(waves, kvs, BKV, D, ctx.lds_bytes_per_cu)
+    lds = plan["bytes"]
     if lds > ctx.lds_bytes_per_cu:
         raise LoweringError(f"flash: {lds} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
     for st in (body.q_strides, body.k_strides, body.v_strides):
         if st[2] % 8:
             raise LoweringError("flash: sequence strides must keep 16-byte row alignment")
-    if body.o_strides[2] % 4 or any(o % 8 for o in (body.q_offset, body.k_offset, body.v_offset)) or body.o_offset % 4:
-        raise LoweringError("flash: offsets / output stride break vector alignment")
+    for st, heads in ((body.q_strides, body.q_heads), (body.k_strides, body.kv_heads), (body.v_strides, body.kv_heads), (body.o_strides, body.q_heads)):
+        if st[2] % 8 or (heads > 1 and st[1] % 8) or (body.batch > 1 and st[0] % 8):
+            raise LoweringError("flash: batch / head / sequence strides must keep 16-byte alignment")
+    if any(o % 8 for o in (body.q_offset, body.k_offset, body.v_offset, body.o_offset)):
+        raise LoweringError("flash: offsets break 16-byte alignment")
     qblocks = -(-body.q_len // BQ)
     pair = bool(body.pair)
     if pair and not (body.causal and qblocks % 2 == 0):
@@ -350,6 +456,10 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "QBLOCKS": qblocks,
         "QSLOTS": qslots,
         "PAIR": 1 if pair else 0,
+        "Q_LDS": 1 if plan["q_off"] is not None else 0,
+        "Q_OFF_LDS": plan["q_off"] or 0,
+        "O_OFF_LDS": plan["o_off"],
+        "PARK_ML": plan["park_ml"],
         "CAUSAL": 1 if body.causal else 0,
         "SCALE_LOG2": float_literal(body.scale * math.log2(math.e)),
         "Q_SB": body.q_strides[0], "Q_SH": body.q_strides[1], "Q_SS": body.q_strides[2], "Q_OFF": body.q_offset,

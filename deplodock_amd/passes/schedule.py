@@ -247,6 +247,12 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
     return {"TILE": plan.spell(), "STAGE": stage.spell()}
 
 
+def _flash_lds(body: Flash, ctx: Context) -> int:
+    from deplodock_amd.emit.flash import lds_plan
+
+    return lds_plan(body.waves, body.kv_split, body.block_kv, body.head_dim, ctx.lds_bytes_per_cu)["bytes"]
+
+
 def schedule_flash(body: Flash, ctx: Context) -> dict:
     """``EMMY_FLASH=w<row groups>/kv<keys per block>/s<key split>[/p]``.
 
@@ -275,8 +281,10 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
             chunks = body.block_kv * body.head_dim // 8
             if body.waves < 1 or body.kv_split < 1 or body.block_kv % 32 or chunks % (body.waves * body.kv_split * 64):
                 raise ScheduleError("unrealisable workgroup shape")
-            if 2 * body.kv_split * 2 * body.block_kv * body.head_dim * 2 > ctx.lds_bytes_per_cu:
+            if _flash_lds(body, ctx) > ctx.lds_bytes_per_cu:
                 raise ScheduleError("the double-buffered K/V blocks of all key-split groups exceed the LDS")
+            if (body.head_dim // 32 * 16) % (4 * body.kv_split):
+                raise ScheduleError("the key-split groups cannot share a lane's output registers")
             if body.pair and not (body.causal and -(-body.q_len // (32 * body.waves)) % 2 == 0):
                 raise ScheduleError("pairing mirrored query blocks needs a causal mask and an even block count")
         except (ValueError, ScheduleError) as exc:
@@ -293,7 +301,7 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 body.waves //= 2
             body.kv_split = 2 if -(-body.kv_len // body.block_kv) >= 2 else 1
         # wider heads: shrink the key block, then the key split, until the double-buffered K/V blocks fit the LDS
-        while 2 * body.kv_split * 2 * body.block_kv * body.head_dim * 2 > ctx.lds_bytes_per_cu:
+        while _flash_lds(body, ctx) > ctx.lds_bytes_per_cu:
             if body.block_kv > 32:
                 body.block_kv //= 2
             elif body.kv_split > 1:

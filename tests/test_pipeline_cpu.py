@@ -149,7 +149,8 @@ def test_flash_pin_grammar_and_degrade(launcher_lib, monkeypatch):
     assert kernels(compile_case(case))[0].knobs["FLASH"] == default
     monkeypatch.setenv("EMMY_FLASH", "w2/kv32/s4")
     k = kernels(compile_case(case))[0]
-    assert k.knobs["FLASH"] == "w2/kv32/s4" and k.block[0] == (512,) and k.lds_bytes == 2 * 4 * 2 * 32 * 128 * 2
+    assert k.knobs["FLASH"] == "w2/kv32/s4" and k.block[0] == (512,)
+    assert k.lds_bytes == 2 * 4 * 2 * 32 * 128 * 2 + 64 * 128 * 2  # double-buffered K/V blocks of four groups, then the Q tile
     monkeypatch.setenv("EMMY_FLASH", "w2/kv64/s4")  # 256 KiB of staging does not fit: degrade to the default pick
     assert kernels(compile_case(case))[0].knobs["FLASH"] == default
     monkeypatch.setenv("EMMY_FLASH", "w3/zz")
