@@ -140,16 +140,16 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   const ELT* gk_lane = kbase + (long)st_row * K_SS;
   const ELT* gv_lane = vbase + (long)st_row * V_SS;
   const int dst_lane = (tid - lane) * 16;
-  #define EMH_STAGE(st, buf) { \
-    unsigned char* sb_ = lds + (buf) * STEP_BYTES + dst_lane; \
-    _Pragma("unroll") for (int i = 0; i < PER_T; ++i) { \
-      const int g_ = (i * NT) / CHUNKS, ro_ = ((i * NT) % CHUNKS) / CPR; \
+  #define EMH_STAGE_PART(st, buf, i) { \
+      unsigned char* sb_ = lds + (buf) * STEP_BYTES + dst_lane; \
+      const int g_ = ((i) * NT) / CHUNKS, ro_ = (((i) * NT) % CHUNKS) / CPR; \
       long krow_ = (long)((st) * KVS + g_) * BKV + ro_; \
       if (SKV % (KVS * BKV) != 0) { const long lim_ = SKV - 1 - st_row; if (krow_ > lim_) krow_ = lim_; } \
       const int kc_ = emh_kswz(st_row + ro_, st_pos), vc_ = emh_vswz(st_row + ro_, st_pos); \
-      unsigned char* dk_ = sb_ + g_ * 2 * KBYTES + ((i * NT) % CHUNKS) * 16; \
+      unsigned char* dk_ = sb_ + g_ * 2 * KBYTES + (((i) * NT) % CHUNKS) * 16; \
       __builtin_amdgcn_global_load_lds((const void*)(gk_lane + krow_ * K_SS + kc_ * 8), (__attribute__((address_space(3))) void*)dk_, 16, 0, 0); \
-      __builtin_amdgcn_global_load_lds((const void*)(gv_lane + krow_ * V_SS + vc_ * 8), (__attribute__((address_space(3))) void*)(dk_ + KBYTES), 16, 0, 0); } }
+      __builtin_amdgcn_global_load_lds((const void*)(gv_lane + krow_ * V_SS + vc_ * 8), (__attribute__((address_space(3))) void*)(dk_ + KBYTES), 16, 0, 0); }
+  #define EMH_STAGE(st, buf) { _Pragma("unroll") for (int i = 0; i < PER_T; ++i) EMH_STAGE_PART(st, buf, i) }
 
   // Publishing direct-to-LDS data: vmcnt reaching zero does not yet mean the
   // data is visible to other waves' LDS reads (measured: stale reads right after
@@ -188,11 +188,15 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   }
 
   for (int st = 0; st < nsteps; ++st) {
-    if (st + 1 < nsteps) EMH_STAGE(st + 1, (st + 1) & 1);
+    // The next step's blocks are requested between this step's score MFMAs: the
+    // matrix pipe works through the chain while the wave issues the loads.
+    const bool more = st + 1 < nsteps;
     const int jt = st * KVS + grp;
     const int k0 = jt * BKV;
     const bool active = (jt < ntiles) && (!CAUSAL || (k0 <= qw0 + 31));
-    if (active) {
+    if (!active) {
+      if (more) EMH_STAGE(st + 1, (st + 1) & 1);
+    } else {
       const unsigned char* sK = lds + (st & 1) * STEP_BYTES + grp * 2 * KBYTES;
       const unsigned char* sV = sK + KBYTES;
       f32x16 sacc[BKV / 32];
@@ -208,8 +212,14 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         for (int kk = 0; kk < D / 16; ++kk) kf[kk] = *(const FRAG*)(sK + krow * (D * 2) + emh_kswz(krow, kk * 2 + lh) * 16);
         __builtin_amdgcn_sched_barrier(0);
         #pragma unroll
-        for (int kk = 0; kk < D / 16; ++kk) sacc[u] = MFMA(kf[kk], qf[kk], sacc[u], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int kk = 0; kk < D / 16; ++kk) {
+          sacc[u] = MFMA(kf[kk], qf[kk], sacc[u], 0, 0, 0);
+          if (more) {
+            #pragma unroll
+            for (int i = u * (D / 16) + kk; i < PER_T; i += (BKV / 32) * (D / 16)) EMH_STAGE_PART(st + 1, (st + 1) & 1, i);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
       float mx = -1.0e30f;
       if ((CAUSAL && (k0 + BKV - 1 > qw0)) || (k0 + BKV > SKV)) {
@@ -228,8 +238,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[u][r]);
       }
       mx *= SCALE_LOG2;
-      mx = fmaxf(mx, emh_xor32(mx));
-      if (__any(mx > m_ref + RESCALE_SLACK)) {
+      if (__any(mx > m_ref + RESCALE_SLACK)) {  // a vote over both halves of every row: the halves meet only when it passes
+        mx = fmaxf(mx, emh_xor32(mx));
         const float m_new = fmaxf(m_ref, mx);
         const float alpha = EXP2(m_ref - m_new);
         m_ref = m_new;
