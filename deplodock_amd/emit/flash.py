@@ -149,12 +149,12 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       unsigned char* dk_ = sb_ + g_ * 2 * KBYTES + (((i) * NT) % CHUNKS) * 16; \
       __builtin_amdgcn_global_load_lds((const void*)(gk_lane + krow_ * K_SS + kc_ * 8), (__attribute__((address_space(3))) void*)dk_, 16, 0, 0); \
       __builtin_amdgcn_global_load_lds((const void*)(gv_lane + krow_ * V_SS + vc_ * 8), (__attribute__((address_space(3))) void*)(dk_ + KBYTES), 16, 0, 0); }
-  // Request i of a step is issued behind MFMA number EMH_SLOT_OF(i) of the step
-  // (score MFMAs first, then the P V ones): the loads trickle into the memory
-  // pipeline instead of arriving as one burst from every wave.
+  // Request i of a step is issued behind score MFMA number EMH_SLOT_OF(i): spread
+  // evenly over the chain, so the loads trickle into the memory pipeline instead of
+  // arriving as one burst from every wave, and all of them are on their way before
+  // the softmax starts (requests issued later land after the step's fence).
   #define NQ_SLOTS ((BKV / 32) * (D / 16))
-  #define NP_SLOTS ((BKV / 32) * 2 * (D / 32))
-  #define EMH_SLOT_OF(i) (((i) * SPREAD) < NQ_SLOTS + NP_SLOTS ? ((i) * SPREAD) : ((i) % (NQ_SLOTS + NP_SLOTS)))
+  #define EMH_SLOT_OF(i) (((i) * NQ_SLOTS) / PER_T)
   #define EMH_STAGE(st, buf) { _Pragma("unroll") for (int i = 0; i < PER_T; ++i) EMH_STAGE_PART(st, buf, i) }
 
   // Publishing direct-to-LDS data: vmcnt reaching zero does not yet mean the
@@ -281,10 +281,6 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
           u32x4 av;
           av[0] = l2[0]; av[1] = l2[1]; av[2] = h2[0]; av[3] = h2[1];
           oacc[dt] = MFMA(__builtin_bit_cast(FRAG, av), pf, oacc[dt], 0, 0, 0);
-          if (more) {
-            #pragma unroll
-            for (int i = 0; i < PER_T; ++i) if (EMH_SLOT_OF(i) == NQ_SLOTS + (u * 2 + s) * (D / 32) + dt) EMH_STAGE_PART(st + 1, (st + 1) & 1, i);
-          }
         }
       }
     }
@@ -476,7 +472,6 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "QBLOCKS": qblocks,
         "QSLOTS": qslots,
         "PAIR": 1 if pair else 0,
-        "SPREAD": 2,  # every second MFMA; every fourth measured 10 % slower (the last requests land after the step's fence)
         "Q_LDS": 1 if plan["q_off"] is not None else 0,
         "Q_OFF_LDS": plan["q_off"] or 0,
         "O_OFF_LDS": plan["o_off"],

@@ -256,13 +256,18 @@ def _flash_lds(body: Flash, ctx: Context) -> int:
 def schedule_flash(body: Flash, ctx: Context) -> dict:
     """``EMMY_FLASH=w<row groups>/kv<keys per block>/s<key split>[/p]``.
 
-    Default: four 32-row groups x two key-split wave groups (8 waves, two per
-    SIMD; measured 41.5 us vs 62.7 us unsplit on the S=2048 causal shape), with the
-    row groups halved until the launch covers the CUs.  A causal self-attention
-    whose mirrored query-block pairs (``/p``: block b then block n-1-b in one
-    workgroup, equal key work for every workgroup) still cover the CUs takes
-    ``w2/kv32/s4/p`` instead: 36.6 us on the same shape, where unpaired
-    workgroups wait for the one that owns the last rows."""
+    Default: eight waves per workgroup, two per SIMD — four 32-row groups x two
+    key-split wave groups on 64-key blocks (``w4/kv64/s2``) when that many rows per
+    workgroup still cover the CUs, else two (or one) row groups x four key-split
+    groups on 32-key blocks.  A long causal self-attention whose mirrored
+    query-block pairs (``/p``: block b then block n-1-b in one workgroup, equal
+    key work for every workgroup) still cover the CUs is paired; below 2048 keys the
+    second prologue and close of a pair cost more than the balance gains.
+    Measured with 16 q / 8 kv heads of 128 (us, best three): S=512 ``w2/kv32/s4``
+    8.7, ``w1/kv32/s4`` 8.8, ``w2/kv64/s2`` 11.0; S=1024 ``w2/kv32/s4`` 13.5,
+    ``w1/kv32/s4/p`` 17.8; S=2048 ``w2/kv32/s4/p`` 27.8, ``w2/kv32/s4`` 28.5,
+    ``w4/kv64/s2`` 32.7; S=2048 unmasked ``w4/kv64/s2`` 36.5, ``w4/kv32/s2`` 41.3;
+    32 q heads S=4096 ``w4/kv64/s2/p`` 157, ``w2/kv32/s4/p`` 186."""
     pinned = _pin("FLASH", _tuned(body, ctx))
     if pinned:
         try:
@@ -292,14 +297,22 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
             pinned = None
     if not pinned:
         heads = body.batch * body.q_heads
-        blocks64 = -(-body.q_len // 64)
-        if body.causal and body.q_len == body.kv_len and blocks64 % 2 == 0 and heads * blocks64 // 2 >= _FILL_FRACTION * ctx.compute_units and body.head_dim == 128:
-            body.waves, body.block_kv, body.kv_split, body.pair = 2, 32, 4, True
-        else:
-            body.waves, body.block_kv, body.pair = 4, 64, False
-            while body.waves > 1 and heads * -(-body.q_len // (32 * body.waves)) < ctx.compute_units:
-                body.waves //= 2
-            body.kv_split = 2 if -(-body.kv_len // body.block_kv) >= 2 else 1
+        fill = _FILL_FRACTION * ctx.compute_units
+
+        def blocks(w: int) -> int:
+            return -(-body.q_len // (32 * w))
+
+        body.pair = False
+        if body.causal and body.q_len == body.kv_len and body.kv_len >= 2048:
+            for w in (4, 2):
+                if blocks(w) % 2 == 0 and heads * blocks(w) // 2 >= fill:
+                    body.waves, body.pair = w, True
+                    break
+        if not body.pair:
+            body.waves = next((w for w in (4, 2) if heads * blocks(w) >= fill), 1)
+        body.block_kv, body.kv_split = (64, 2) if body.waves == 4 else (32, 4)
+        while body.kv_split > 1 and -(-body.kv_len // body.block_kv) < body.kv_split:
+            body.kv_split //= 2  # fewer key blocks than key-split groups
         # wider heads: shrink the key block, then the key split, until the double-buffered K/V blocks fit the LDS
         while _flash_lds(body, ctx) > ctx.lds_bytes_per_cu:
             if body.block_kv > 32:

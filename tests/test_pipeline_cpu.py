@@ -141,7 +141,7 @@ def test_tile_and_stage_pins(launcher_lib, monkeypatch):
 def test_flash_pin_grammar_and_degrade(launcher_lib, monkeypatch):
     case = eager.sdpa_case(1, 8, 4, 320, 128)
     default = kernels(compile_case(case))[0].knobs["FLASH"]
-    assert default == "w1/kv64/s2"  # few heads, short sequence: one 32-row group per workgroup to cover the CUs
+    assert default == "w1/kv32/s4"  # few heads, short sequence: one 32-row group per workgroup, four key-split groups
     # long causal self-attention: mirrored query-block pairs, so every workgroup streams the same number of keys
     big = kernels(compile_case(eager.sdpa_case()))[0]
     assert big.knobs["FLASH"] == "w2/kv32/s4/p" and big.grid[0] == (16 * 32 // 2,) and "#define PAIR 1" in big.kernel_source
