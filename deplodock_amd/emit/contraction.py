@@ -60,6 +60,92 @@ def xcd_block(tiles_m: int, tiles_n: int, tile_m: int, tile_n: int, xcds: int) -
     return (best[0], best[1]) if best else (1, 1)
 
 
+def _emit_row_epilogue_tables(a, re, re_args: list[str], EPC: int, m_guard: bool) -> None:
+    """Fetch, at kernel start, the table chunks the row epilogue of this thread will
+    need (they depend on the output coordinates only): the k loop hides the latency."""
+    d = re.cols
+    vt_chunk = {2: None, 4: "f32x4"}.get(16 // EPC) or ("bf16x8" if re.row_operands and re.row_operands[0].dtype.name == "bf16" else "f16x8")
+    in_project = E.variables(re.project)
+    a(f"  constexpr int RE_IT = (TM * (TN / {EPC})) / T;")
+    for nm, ro in zip(re_args, re.row_operands):
+        a(f"  {vt_chunk} {nm}_v[RE_IT]" + (f", {nm}_p[RE_IT];" if re.rotate is not None and ro.name in in_project else ";"))
+    a(f"  if (n0 < {re.col_end}) {{")
+    a("    #pragma unroll")
+    a("    for (int it = 0; it < RE_IT; ++it) {")
+    a(f"      const int q = tid + it * T, row = q / (TN / {EPC}), cc = q % (TN / {EPC});")
+    a(f"      const int m = m0 + row, n = n0 + cc * {EPC}, gc = n % {d};")
+    mrow = "(m < M ? m : M - 1)" if m_guard else "m"
+    a(f"      const long rr = (long){mrow} * {re.col_end // d} + n / {d};  // the row number a separate row kernel would use")
+    for nm, ro in zip(re_args, re.row_operands):
+        a(f"      const {ro.dtype.c_name}* {nm}_row = {nm} + {ro.offset}L + ((rr / {ro.div}) % {ro.mod}) * {d};")
+        a(f"      {nm}_v[it] = *(const {vt_chunk}*)({nm}_row + gc);")
+        if re.rotate is not None and ro.name in in_project:
+            a(f"      {nm}_p[it] = *(const {vt_chunk}*)({nm}_row + (gc ^ {d // 2}));")
+    a("    }")
+    a("  }")
+
+
+def _emit_row_epilogue(a, body: Contraction, re, re_args: list[str], EPC: int, vt_chunk: str, out_c: str, m_guard: bool, n_guard: bool) -> None:
+    """The store loop of the tiles that hold row-epilogue columns: every thread
+    owns one 16-byte chunk of an output row at a time; the ``HC`` threads that
+    share a column group are consecutive lanes, so the group statistic is a
+    butterfly over them, and the half-rotated partner chunk is read from the tile
+    in LDS.  Leaves the ``else`` of the tile test open for the plain store loop."""
+    d = re.cols
+    HC = d // EPC
+    if HC & (HC - 1) or HC > 32 or HC < 2:
+        raise LoweringError(f"contraction: row-epilogue groups of {d} columns do not map onto lanes")
+    stat_names = [st.name for st in re.stats]
+    op_names = [ro.name for ro in re.row_operands]
+    for st in re.stats:
+        if E.variables(st.pre) - {"x"} or st.monoid not in ("sum", "max") or st.keep:
+            raise LoweringError(f"contraction: row-epilogue statistic {st.name!r} is not a plain sum/max over the group")
+    in_project = E.variables(re.project)
+    in_rotate = E.variables(re.rotate.expr) if re.rotate is not None else set()
+    unknown = (in_project - ({"x"} | set(stat_names) | set(op_names))) | (in_rotate - ({"y", "yr"} | set(stat_names) | set(op_names)))
+    if unknown:
+        raise LoweringError(f"contraction: row epilogue uses unknown names {sorted(unknown)}")
+    cast = "" if body.out_dtype is F32 else f"({out_c})"
+    a(f"  if (n0 < {re.col_end}) {{  // tiles of column groups that take the row epilogue")
+    a(r"""  #pragma unroll
+  for (int it = 0; it < (TM * CPRC) / T; ++it) {
+    const int q = tid + it * T;
+    const int row = q / CPRC, cc = q % CPRC;""")
+    a(f"    const int m = m0 + row, n = n0 + cc * {EPC};")
+    a(f"    const {vt_chunk} xv = *(const {vt_chunk}*)(emh_lds + row * CSTRIDE + cc * 16);")
+    for st in re.stats:
+        ident = "0.0f" if st.monoid == "sum" else "-__builtin_inff()"
+        a(f"    float {st.name} = {ident};")
+        a("    #pragma unroll")
+        a(f"    for (int r = 0; r < {EPC}; ++r) {{ const float x_ = (float)xv[r]; const float t_ = {E.render(st.pre, {'x': 'x_'})}; {st.name} = " + (f"{st.name} + t_" if st.monoid == "sum" else f"fmaxf({st.name}, t_)") + "; }")
+        a(f"    {st.name} = emh_wave_reduce<{prelude.MONOID_STRUCT[st.monoid]}, {HC}>({st.name});  // the group's chunks sit in {HC} consecutive lanes")
+    env_stats = {n_: n_ for n_ in stat_names}
+    if re.rotate is None:
+        a(f"    {vt_chunk} yo;")
+        a("    #pragma unroll")
+        a(f"    for (int r = 0; r < {EPC}; ++r) {{")
+        env = dict(env_stats, x="(float)xv[r]", **{ro.name: f"(float){nm}_v[it][r]" for nm, ro in zip(re_args, re.row_operands)})
+        a(f"      yo[r] = {cast}({E.render(re.project, env)});")
+        a("    }")
+    else:
+        a(f"    const {vt_chunk} pv = *(const {vt_chunk}*)(emh_lds + row * CSTRIDE + (cc ^ {HC // 2}) * 16);  // the half-rotated partner chunk")
+        a(f"    const float sgn = (cc % {HC}) < {HC // 2} ? -1.0f : 1.0f;")
+        a(f"    {vt_chunk} yo;")
+        a("    #pragma unroll")
+        a(f"    for (int r = 0; r < {EPC}; ++r) {{")
+        env_own = dict(env_stats, x="(float)xv[r]", **{ro.name: f"(float){nm}_v[it][r]" for nm, ro in zip(re_args, re.row_operands) if ro.name in in_project})
+        env_par = dict(env_stats, x="(float)pv[r]", **{ro.name: f"(float){nm}_p[it][r]" for nm, ro in zip(re_args, re.row_operands) if ro.name in in_project})
+        a(f"      const float y_ = {E.render(re.project, env_own)};")
+        a(f"      const float yr_ = sgn * ({E.render(re.project, env_par)});")
+        env_rot = dict(env_stats, y="y_", yr="yr_", **{ro.name: f"(float){nm}_v[it][r]" for nm, ro in zip(re_args, re.row_operands) if ro.name in in_rotate})
+        a(f"      yo[r] = {cast}({E.render(re.rotate.expr, env_rot)});")
+        a("    }")
+    conds = (["m < M"] if m_guard else []) + (["n < N"] if n_guard else [])
+    a(f"    if ({' && '.join(conds) if conds else 'true'}) *({vt_chunk}*)(O + {body.out_offset}L + (long)m * LDO + n) = yo;")
+    a("  }")
+    a("  } else {")
+
+
 def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> HipOp:
     plan = body.tile
     if plan is None:
@@ -146,6 +232,12 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     if body.bias is not None:
         params.append(f"const {body.bias_dtype.c_name}* __restrict__ BIAS")
     params += [f"const {dt.c_name}* __restrict__ e{i}" for i, (_, dt) in enumerate(body.epilogue_operands)]
+    rowepi = body.row_epilogue
+    re_args = [f"re{i}" for i in range(len(rowepi.row_operands))] if rowepi is not None else []
+    if rowepi is not None:
+        if body.post is not None or gate or TN % rowepi.cols or rowepi.col_end % TN or rowepi.col_end > N:
+            raise LoweringError("contraction: the row epilogue needs a plain result and output tiles of whole column groups")
+        params += [f"const {ro.dtype.c_name}* __restrict__ {nm}" for nm, ro in zip(re_args, rowepi.row_operands)]
     params.append(f"{out_c}* __restrict__ O")
 
     D = dict(
@@ -191,6 +283,8 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   const int wm = wave / WN, wn = wave % WN;
   const int lr = lane % AM, lk = lane / AM;  // fragment row, k-group
 """)
+    if body.row_epilogue is not None:
+        _emit_row_epilogue_tables(a, body.row_epilogue, [f"re{i}" for i in range(len(body.row_epilogue.row_operands))], 16 // body.out_dtype.nbytes, m_guard)
     # ---- staging ------------------------------------------------------------
     a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else ""))
     a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
@@ -430,6 +524,8 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         a("  __syncthreads();")
         vt_chunk = {("bf16"): "bf16x8", "f16": "f16x8", "f32": "f32x4"}[body.out_dtype.name]
         a(f"  constexpr int CPRC = TN / {EPC};  // 16-byte chunks per output-tile row")
+        if rowepi is not None:
+            _emit_row_epilogue(a, body, rowepi, re_args, EPC, vt_chunk, out_c, m_guard, n_guard)
         a(r"""  #pragma unroll
   for (int it = 0; it < (TM * CPRC) / T; ++it) {
     const int q = tid + it * T;
@@ -455,7 +551,11 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         a(f"      *({vt_chunk}*)(O + {body.out_offset}L + (long)m * LDO + n) = v;")
         a("    }")
         a("  }")
+        if rowepi is not None:
+            a("  }")
     else:
+        if rowepi is not None:
+            raise LoweringError("contraction: the row epilogue works on the staged output tile, which this tile shape does not have")
         a(r"""  #pragma unroll
   for (int i = 0; i < FM; ++i) {
     const int m = m0 + (wm * FM + i) * AM + lr;""")
@@ -498,7 +598,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
 // bits 3:0, vmcnt[5:4] in bits 15:14; expcnt left at its maximum, lgkmcnt = 0).
 #define EMH_WAIT_VM_LGKM0(n) ((((n) & 0xF) | ((((n) >> 4) & 0x3) << 14)) | 0x0070)
 """
-    source = prelude.header(vm_macro) + "\n".join(o) + "\n"
+    source = prelude.header(vm_macro, *((prelude.WAVE_REDUCE,) if rowepi is not None else ())) + "\n".join(o) + "\n"
     if N % 4 or TN % 4:
         raise LoweringError("contraction: N must be a multiple of 4 (8-byte output runs)")
     n_blocks = (tiles_m // gm) * (tiles_n // gn)
@@ -507,11 +607,14 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     return HipOp(
         kernel_source=source,
         kernel_name=name,
-        arg_order=(body.a, body.b, *((pro.weight,) if pro is not None and pro.weight is not None else ()), *((body.bias,) if body.bias is not None else ()), *(body.operand_buffers.get(n, n) for n in epi_names), body.out),
+        arg_order=(
+            body.a, body.b, *((pro.weight,) if pro is not None and pro.weight is not None else ()), *((body.bias,) if body.bias is not None else ()),
+            *(body.operand_buffers.get(n, n) for n in epi_names), *(rowepi.operand_buffers.get(ro.name, ro.name) for ro in (rowepi.row_operands if rowepi is not None else ())), body.out,
+        ),  # fmt: skip
         grid=((grid,), (1,), (1,)),
         block=((T,), (1,), (1,)),
         lds_bytes=lds_bytes,
-        comment=f"contraction M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()}" + (" a=row-normalised" if pro is not None else ""),
+        comment=f"contraction M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()}" + (" a=row-normalised" if pro is not None else "") + (f" row-epilogue={rowepi.col_end // rowepi.cols}x{rowepi.cols}" if rowepi is not None else ""),
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
         knobs={"TILE": plan.spell(), "STAGE": stage.spell()},

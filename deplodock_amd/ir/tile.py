@@ -135,6 +135,26 @@ class RowPrologue:
 
 
 @dataclass
+class RowEpilogue:
+    """A row kernel folded into the contraction's output stage.  Columns
+    ``[0, col_end)`` of the result are ``col_end / cols`` groups of ``cols``
+    columns (the heads of a merged q/k projection); on every (output row, group)
+    the statistics, projection and optional half-rotation of a ``RowReduce`` are
+    applied to the rounded contraction result while the output tile sits in LDS,
+    so ``linear -> head norm -> rotary embedding`` is one launch.  ``row_operands``
+    index their tables with the row number ``m * (col_end / cols) + group``, as the
+    separate kernel would; columns from ``col_end`` on are stored untouched."""
+
+    cols: int
+    col_end: int
+    stats: tuple[Stat, ...]
+    project: Expr
+    rotate: RotateHalf | None = None
+    row_operands: tuple[RowOperand, ...] = ()
+    operand_buffers: dict = field(default_factory=dict)  # row operand name -> buffer id
+
+
+@dataclass
 class Contraction:
     """``out[m, n] = epilogue(sum_k a[m, k] * b[n, k])`` — both operands
     K-contiguous (the reference's ``b_trans`` layout for ``nn.Linear`` weights,
@@ -175,6 +195,7 @@ class Contraction:
     a_prologue: RowPrologue | None = None
     bias: str | None = None  # length-n vector the epilogue may name ``bias`` (added to the fp32 accumulator)
     bias_dtype: DType | None = None
+    row_epilogue: RowEpilogue | None = None
 
     def algo_flops(self) -> int:
         return 2 * self.m * self.n * self.k * (2 if self.gate_pair else 1)
@@ -188,6 +209,9 @@ class Contraction:
             b += self.k * self.a_prologue.weight_dtype.nbytes
         if self.bias is not None:
             b += self.n * self.bias_dtype.nbytes
+        if self.row_epilogue is not None:
+            for ro in self.row_epilogue.row_operands:
+                b += ro.mod * self.row_epilogue.cols * ro.dtype.nbytes
         return b
 
 

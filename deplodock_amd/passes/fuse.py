@@ -33,7 +33,7 @@ from deplodock_amd.graph import Graph, Node, Tensor
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir import frontend as F
 from deplodock_amd.ir.base import ConstantOp, InputOp
-from deplodock_amd.ir.tile import Contraction, Flash, Map, MapOperand, RotateHalf, RowAddr, RowOperand, RowPrologue, RowReduce, Stat, TileOp
+from deplodock_amd.ir.tile import Contraction, Flash, Map, MapOperand, RotateHalf, RowAddr, RowEpilogue, RowOperand, RowPrologue, RowReduce, Stat, TileOp
 from deplodock_amd.passes.views import LAYOUT_OPS, NotViewable, View, apply_layout, contiguous_strides, resolve_view
 
 
@@ -680,10 +680,55 @@ def _rec_rope_pair(c: _Ctx, nid: str) -> bool:
     )  # fmt: skip
     body.rotate = RotateHalf(_rope_expr(od))
     body.operand_buffers = {"w": stacked, "cos": cos_v.base, "sin": sin_v.base}
+    raw_only_feeds_rope = all(_feeds_only(g, _peel_layout(g, rp.t_id), _rope_internal(g, rp.t_id, rid)) for rid, rp in ((id0, p0), (id1, p1)))
+    if raw_only_feeds_rope and _absorb_row_kernel(c, body, x0, a0, tokens, heads):
+        # the projection that produced the heads rotates them on its way out: the results are windows of its buffer
+        for rid, rp, first in ((id0, p0, 0), (id1, p1, h0)):
+            c.done[rid] = x0.base
+            c.windows[rid] = (a0.offset + first * d, rp.t_view_shape, _logical_strides(rp, (a0.stride_hi, d)))
+        return True
     c.out.add_node(TileOp(name=c.kname("rms_norm_rope"), body=body), list(dict.fromkeys([x0.base, stacked, cos_v.base, sin_v.base])), Tensor(fid, (tokens, heads, d), od), fid)
     for rid, rp, first in ((id0, p0, 0), (id1, p1, h0)):
         c.done[rid] = fid
         c.windows[rid] = (first * d, rp.t_view_shape, _logical_strides(rp, (heads * d, d)))
+    return True
+
+
+def _feeds_only(g: Graph, src_id: str, allowed: set[str]) -> bool:
+    """Does every path from ``src_id`` lead, through layout ops only, into ``allowed``?"""
+    if src_id in g.outputs:
+        return False
+    for cons in g.consumers(src_id):
+        if cons in allowed:
+            continue
+        if not isinstance(g.nodes[cons].op, LAYOUT_OPS) or not _feeds_only(g, cons, allowed):
+            return False
+    return True
+
+
+def _absorb_row_kernel(c: _Ctx, body: RowReduce, x: View, addr: RowAddr, tokens: int, groups: int) -> bool:
+    """Fold ``body`` (a row kernel over ``groups`` column groups per token, in place
+    on the leading columns of ``x``'s buffer) into the contraction that writes that
+    buffer.  Applies to a plain contraction whose result rows are the tokens."""
+    prod = c.out.nodes.get(x.base)
+    if prod is None or not isinstance(prod.op, TileOp) or not isinstance(prod.op.body, Contraction):
+        return False
+    con = prod.op.body
+    d = body.cols
+    if con.post is not None or con.gate_pair or con.row_epilogue is not None or con.reduce.cta != 1:
+        return False
+    if not (con.out == x.base and con.m == tokens and addr.stride_hi == (con.ldo or con.n) and addr.offset == con.out_offset and groups * d <= con.n):
+        return False
+    if not (con.out_dtype == body.x_dtype == body.out_dtype and all(ro.dtype == con.out_dtype for ro in body.row_operands)):
+        return False
+    if d % 16 or d & (d - 1) or body.col_operands:
+        return False
+    con.row_epilogue = RowEpilogue(cols=d, col_end=groups * d, stats=body.stats, project=body.project, rotate=body.rotate, row_operands=body.row_operands, operand_buffers=dict(body.operand_buffers))
+    for ro in body.row_operands:
+        buf = body.operand_buffers.get(ro.name, ro.name)
+        if buf not in prod.inputs:
+            prod.inputs.append(buf)
+    prod.op.name = prod.op.name.replace("linear", "linear_rope" if body.rotate is not None else "linear_rownorm", 1)
     return True
 
 

@@ -139,7 +139,7 @@ def schedule_row_reduce(body: RowReduce, ctx: Context) -> dict:
     return {"REDUCE": plan.spell(), "NT": int(body.nontemporal)}
 
 
-def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologue: bool = False) -> TilePlan:
+def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologue: bool = False, group_cols: tuple[int, int] | None = None) -> TilePlan:
     """First candidate (in measured-throughput order) whose launch covers the
     CUs, else the one that launches the most workgroups."""
     best = None
@@ -156,6 +156,8 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
         atom = ATOMS[atom_name]
         if tm % (wm * atom.m) or tn % (wn * atom.n):
             continue
+        if group_cols is not None and (tn % group_cols[0] or group_cols[1] % tn or (tm * tn // 8) % (wm * wn * 64)):
+            continue  # a row epilogue works on whole column groups of a staged output tile
         fm, fn = tm // (wm * atom.m), tn // (wn * atom.n)
         if fm * fn * atom.acc_per_lane * (2 if gate_pair else 1) > 256:
             continue
@@ -203,6 +205,9 @@ def _check_tile(plan: TilePlan, body: Contraction, ctx: Context, depth: int, dl:
         raise ScheduleError("accumulators exceed the register file")
     if threads > ctx.max_threads_per_block:
         raise ScheduleError(f"{threads} threads per workgroup is not launchable")
+    re = body.row_epilogue
+    if re is not None and (plan.tile_n % re.cols or re.col_end % plan.tile_n or (plan.tile_m * plan.tile_n // 8) % threads):
+        raise ScheduleError(f"the row epilogue needs output tiles of whole {re.cols}-column groups")
 
 
 def schedule_contraction(body: Contraction, ctx: Context) -> dict:
@@ -222,7 +227,8 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
             plan = None
     if plan is None:
         atom_dtype = body.in_dtype.name
-        plan = pick_tile(body.m, body.n, body.k, body.gate_pair, ctx, row_prologue=body.a_prologue is not None)
+        re = body.row_epilogue
+        plan = pick_tile(body.m, body.n, body.k, body.gate_pair, ctx, row_prologue=body.a_prologue is not None, group_cols=(re.cols, re.col_end) if re is not None else None)
         if plan.atom.dtype != atom_dtype:
             plan = TilePlan(atom=ATOMS[plan.atom.name.replace("bf16", atom_dtype)], units=plan.units, regs=plan.regs, bk=plan.bk)
     body.tile = plan

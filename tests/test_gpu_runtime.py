@@ -77,7 +77,7 @@ def test_benchmark_reports_event_times_and_e2e(device):
     compiled = be.compile(trace_module(case.module, case.inputs))
     calls = []
     res = asyncio.run(be.benchmark_async(compiled, warmup=2, num_iters=5, on_iter=lambda b: calls.append(b)))
-    assert res.num_launches == 6 and len(res.per_launch) == 6 and res.captured
+    assert res.num_launches == 5 and len(res.per_launch) == 5 and res.captured
     assert all(p.time_ms > 0 and len(p.samples) == 5 for p in res.per_launch)
     assert res.e2e_ms is not None and res.e2e_min_ms <= res.e2e_ms
     assert 0 < res.min_ms <= res.time_ms <= res.max_ms

@@ -75,7 +75,7 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
     compiled = compile_case(eager.qwen3_block_case(seq=64))
     names = [re.sub(r"_[0-9a-f]{6}$", "", k.kernel_name) for k in kernels(compiled)]
     assert names == [
-        "k_rms_norm_linear", "k_rms_norm_rope",
+        "k_rms_norm_linear_rope",
         "k_sdpa_reduce", "k_linear_add", "k_rms_norm_linear_silu_mul", "k_linear_add",
     ]  # fmt: skip
     # the two layer norms are prologues of the contractions that read them: the row
@@ -92,10 +92,11 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
         hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
     # layout ops produced no kernels and no buffers
     assert not any("transpose" in n or "view" in n or "slice" in n for n in compiled.nodes)
-    # the query and key head norms + rotary embeddings are one launch over the
-    # 16 + 8 heads of every token, with the two norm weights stacked per head
-    rope = kernels(compiled)[1]
-    assert "rows=1536 cols=128" in rope.comment and "(row / 24) * 4096L + (row % 24) * 128L" in rope.kernel_source
+    # the query and key head norms + rotary embeddings ride in the projection's
+    # output stage: its 128-column tiles are whole heads, the first 16 + 8 of which
+    # are normalised (two norm weights stacked per head) and rotated before the store
+    assert "row-epilogue=24x128" in qkv.comment and "if (n0 < 3072)" in qkv.kernel_source
+    assert qkv.arg_order[-3:-1] == ("cos", "sin") and "emh_wave_reduce<EmhSum, 16>(ss)" in qkv.kernel_source
     # q/k/v and gate/up weights are stacked into constants the runtime assembles
     stacked = sorted((n for n in compiled.nodes.values() if n.hints.get("stacked") and len(n.output.shape) == 2), key=lambda n: n.output.shape[0])
     assert [n.output.shape for n in stacked] == [(4096, 1024), (6144, 1024)]

@@ -33,10 +33,14 @@ def test_shape_keys_separate_what_the_schedule_depends_on(launcher_lib):
 
     block = fuse(trace_module(*(lambda c: (c.module, c.inputs))(eager.qwen3_block_case(seq=64))))
     keys = [shape_key(n.op.body) for n in block.nodes.values() if hasattr(n.op, "body")]
-    assert len(keys) == 6 and len(set(keys)) == 6
+    assert len(keys) == 5 and len(set(keys)) == 5
+    norm = fuse(trace_module(*(lambda c: (c.module, c.inputs))(eager.rms_norm_case())))
+    keys += [shape_key(n.op.body) for n in norm.nodes.values() if hasattr(n.op, "body")]
+    assert keys[-1] == "row_reduce/r32/c2048/f32>f32/s1/rot0"
     fams = {k.split("/")[0] for k in keys}
     assert fams == set(FAMILY_KNOBS)
-    assert "contraction/m64/n4096/k1024/bf16>bf16/g0/p0/a1" in keys and "contraction/m64/n3072/k1024/bf16>bf16/g1/p0/a1" in keys
+    # the merged q/k/v projection carries the head norm + rotary epilogue over 128-column groups: its own key
+    assert "contraction/m64/n4096/k1024/bf16>bf16/g0/p0/a1/e128" in keys and "contraction/m64/n3072/k1024/bf16>bf16/g1/p0/a1" in keys
     assert "contraction/m64/n1024/k2048/bf16>bf16/g0/p1/a0" in keys
     assert any(k.startswith("flash/b1/hq16/hkv8/sq64/skv64/d128/c1") for k in keys)
 
