@@ -563,7 +563,11 @@ def _plan_rope(c: _Ctx, nid: str) -> _RopePlan | None:
     node = g.nodes[nid]
     d = int(node.output.shape[-1])
     src_id = _peel_layout(g, t_id)
-    rms = _match_rms_chain(c, src_id)
+    src = g.nodes[src_id]
+    if isinstance(src.op, F.RmsNormOp):
+        rms = _RmsMatch(x=src.inputs[0], weight=src.inputs[1] if src.op.has_weight else None, eps=src.op.eps, inner=F32, cols=int(src.output.shape[-1]))
+    else:
+        rms = _match_rms_chain(c, src_id)
     fuse_norm = rms is not None and rms.cols == d and all(cons in _rope_internal(g, t_id, nid) or isinstance(g.nodes[cons].op, LAYOUT_OPS) for cons in g.consumers(src_id))
     # Address rows of the *output* in the memory order of the rotated operand
     # (so the kernel is a row map whatever transposes the trace applied).
@@ -675,7 +679,7 @@ def _rec_rope_pair(c: _Ctx, nid: str) -> bool:
     fid = f"{id0}__{id1}"
     body = RowReduce(
         rows=tokens * heads, cols=d, x=x0.base, x_dtype=x0.dtype, out=fid, out_dtype=od, stats=(Stat("ss", "sum", x * x),),
-        project=E.Var("w") * _round(p.rms.inner, norm), x_addr=RowAddr(offset=a0.offset, div=heads, stride_hi=a0.stride_hi, stride_lo=d),
+        project=_round(od, E.Var("w") * _round(p.rms.inner, norm)), x_addr=RowAddr(offset=a0.offset, div=heads, stride_hi=a0.stride_hi, stride_lo=d),
         row_operands=(RowOperand("w", w0.output.dtype, div=1, mod=heads, offset=0), *tables),
     )  # fmt: skip
     body.rotate = RotateHalf(_rope_expr(od))
@@ -745,6 +749,7 @@ def _rec_rope(c: _Ctx, nid: str) -> bool:
         body, inputs, xv = _rms_body(c, nid, p.rms, od)
         if (body.rows, body.cols) != (p.rows, d):
             raise FusionError("rope: norm rows do not match the rotated tensor")
+        body.project = _round(od, body.project)  # the norm's result is a tensor of the output dtype: keep its rounding point
     else:
         tv = resolve_view(g, p.t_id)
         xv = _need(c, p.t_id)

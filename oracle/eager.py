@@ -122,6 +122,54 @@ def qwen3_block_case(seq: int = 512, seed: int = 0, dtype=torch.bfloat16) -> Cas
     )  # fmt: skip
 
 
+class NormedRopeAttention(nn.Module):
+    """The front of a Qwen3-style attention layer with ``nn.RMSNorm`` head norms:
+    q/k/v projections, per-head norm of q and k, rotary embedding, causal GQA
+    attention.  Unlike the block case its norm weights are not all ones, so a
+    kernel that pairs a column with the wrong weight or table row shows."""
+
+    def __init__(self, hidden: int, q_heads: int, kv_heads: int, head_dim: int):
+        super().__init__()
+        self.hq, self.hkv, self.d = q_heads, kv_heads, head_dim
+        self.q_proj = nn.Linear(hidden, q_heads * head_dim, bias=False)
+        self.k_proj = nn.Linear(hidden, kv_heads * head_dim, bias=False)
+        self.v_proj = nn.Linear(hidden, kv_heads * head_dim, bias=False)
+        self.q_norm = nn.RMSNorm(head_dim, eps=1e-6)
+        self.k_norm = nn.RMSNorm(head_dim, eps=1e-6)
+
+    @staticmethod
+    def _rotate_half(x):
+        half = x.shape[-1] // 2
+        return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+
+    def forward(self, x, cos, sin):
+        b, s, _ = x.shape
+        q = self.q_norm(self.q_proj(x).view(b, s, self.hq, self.d)).transpose(1, 2)
+        k = self.k_norm(self.k_proj(x).view(b, s, self.hkv, self.d)).transpose(1, 2)
+        v = self.v_proj(x).view(b, s, self.hkv, self.d).transpose(1, 2)
+        c, sn = cos.unsqueeze(1), sin.unsqueeze(1)
+        q = q * c + self._rotate_half(q) * sn
+        k = k * c + self._rotate_half(k) * sn
+        o = nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+        return o.transpose(1, 2).reshape(b, s, self.hq * self.d)
+
+
+def normed_rope_attention_case(hidden: int = 256, q_heads: int = 4, kv_heads: int = 2, head_dim: int = 64, seq: int = 100, seed: int = 0) -> Case:
+    """bf16; projection weights ~N(0, 0.05), norm weights ~N(1, 0.2), x ~N(0,1), rotary base 1e4."""
+    torch.manual_seed(seed)
+    m = NormedRopeAttention(hidden, q_heads, kv_heads, head_dim)
+    with torch.no_grad():
+        for name, p in m.named_parameters():
+            p.copy_(1 + 0.2 * torch.randn_like(p) if "norm" in name else 0.05 * torch.randn_like(p))
+    x = torch.randn(1, seq, hidden)
+    ang = torch.arange(seq)[:, None] * (1e4 ** (-torch.arange(0, head_dim, 2) / head_dim))[None]
+    emb = torch.cat((ang, ang), -1)
+    return Case(
+        f"normed_rope_attention_h{hidden}_{q_heads}x{kv_heads}x{head_dim}_s{seq}", m.to(torch.bfloat16).eval(),
+        (x.to(torch.bfloat16), emb.cos()[None].to(torch.bfloat16), emb.sin()[None].to(torch.bfloat16)), BF16_RTOL, 2e-2,
+    )  # fmt: skip
+
+
 def block_weights(case: Case) -> dict:
     """Parameter arrays of a :func:`qwen3_block_case` keyed the way ``emmy_ops.qwen3_block`` wants."""
     sd = {k: v.float().numpy() for k, v in case.module.state_dict().items()}

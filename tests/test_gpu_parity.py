@@ -267,6 +267,18 @@ def test_c4_golden(device, golden):
 # -- C5 ---------------------------------------------------------------------------
 
 
+@pytest.mark.parametrize("dims", [(256, 4, 2, 64, 100), (512, 4, 2, 128, 72), (512, 8, 8, 64, 256)])
+def test_head_norm_and_rope_in_the_projection_epilogue(device, dims):
+    """q/k/v projection -> per-head RMSNorm (weights != 1) -> rotary embedding -> attention:
+    two launches, the norm and rotation applied to the projection's output tile.  Ragged
+    token counts exercise the row guards, 64-wide heads the eight-lane group reduce."""
+    case = eager.normed_rope_attention_case(*dims)
+    ours, want, compiled = run_case(case, device)
+    ks = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert len(ks) == 2 and "row-epilogue" in ks[0].comment
+    eager.assert_close(ours, want, case.rtol, case.atol, f"{case.name} vs eager (GPU)")
+
+
 @pytest.mark.parametrize("seq", [32, 64, 512])
 def test_c5_qwen3_block(device, seq, golden):
     case = eager.qwen3_block_case(seq=seq)

@@ -112,6 +112,18 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
     assert (data[stacked[0].id][2048:3072] == traced[parts[1]]).all()
 
 
+def test_head_norm_and_rope_fold_into_the_projection(launcher_lib, monkeypatch):
+    ks = kernels(compile_case(eager.normed_rope_attention_case()))
+    assert [re.sub(r"_[0-9a-f]{6}$", "", k.kernel_name) for k in ks] == ["k_linear_rope", "k_sdpa_reduce"]
+    k = ks[0]
+    assert "row-epilogue=6x64" in k.comment and "emh_wave_reduce<EmhSum, 8>(ss)" in k.kernel_source
+    assert "#define TN 64" in k.kernel_source  # output tiles are whole heads
+    hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+    # a pinned tile that splits a head degrades to the heuristic pick for this kernel
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_16x16x32_bf16/w1x2/f1x1/k4")
+    assert "#define TN 64" in kernels(compile_case(eager.normed_rope_attention_case()))[0].kernel_source
+
+
 def test_reduce_pin_is_authoritative_and_bad_pin_degrades(launcher_lib, monkeypatch):
     case = eager.rms_norm_case()
     monkeypatch.setenv("EMMY_REDUCE", "b64")
