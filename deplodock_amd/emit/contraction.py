@@ -187,6 +187,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     A_PER_T, B_PER_T = a_chunks // T, b_chunks // T
     slab_bytes = (TM + TN * NB) * BK * 2
     depth = max(2, stage.depth)
+    RS = 1 if stage.transport == "dl" else max(1, stage.reg_depth)  # register sets a slab travels through on the sync path
     lds_bytes = slab_bytes * depth
     if lds_bytes > ctx.lds_bytes_per_cu:
         raise LoweringError(f"contraction: {lds_bytes} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
@@ -243,7 +244,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     D = dict(
         name=name, T=T, M=M, N=N, K=K, LDA=lda, LDB=ldb, LDO=ldo, TM=TM, TN=TN, BK=BK, WM=WM, WN=WN, FM=FM, FN=FN,
         AM=AM, KG=KG, KSTEP=KSTEP, ACC=ACC, CPR=CPR, RPL=RPL, NB=NB, A_PER_T=A_PER_T, B_PER_T=B_PER_T,
-        SLAB=slab_bytes, DEPTH=depth, KT=KT, TILES_M=tiles_m, TILES_N=tiles_n, NTILES=n_tiles, GM=gm, GN=gn,
+        SLAB=slab_bytes, DEPTH=depth, RS=RS, KT=KT, TILES_M=tiles_m, TILES_N=tiles_n, NTILES=n_tiles, GM=gm, GN=gn,
         XCDS=ctx.xcds, frag_t=frag_t, in_c=in_c, out_c=out_c, params=", ".join(params), builtin=plan.atom.builtin,
         acc_t="f32x16" if ACC == 16 else "f32x4", G=ACC // 4,
     )  # fmt: skip
@@ -379,44 +380,52 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
             a("  for (int i = 0; i < A_PER_T; ++i)")
             a("  #pragma unroll")
             a("  for (int msk = 1; msk < CPR; msk *= 2) ss[i] += __shfl_xor(ss[i], msk, 64);")
-            wdecl = f" {frag_t} rw[A_PER_T];" if pro.weight is not None else ""
-            a(f"  u32x4 ra[A_PER_T], rb[B_PER_T];{wdecl}")
-            wload = " rw[i] = *(const FRAG_T*)(NW + (kt) * BK + ca[i]);".replace("FRAG_T", frag_t) if pro.weight is not None else ""
-            a("  #define EMH_GLOAD(kt) { \\")
-            a(f'    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) {{ ra[i] = *(const u32x4*)(ga[i] + (kt) * BK);{wload} }} \\')
-            a('    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[i] = *(const u32x4*)(gb[i] + (kt) * BK); }')
+            wdecl = f" {frag_t} rw[RS][A_PER_T];" if pro.weight is not None else ""
+            a(f"  u32x4 ra[RS][A_PER_T], rb[RS][B_PER_T];{wdecl}")
+            wload = " rw[S][i] = *(const FRAG_T*)(NW + (kt) * BK + ca[i]);".replace("FRAG_T", frag_t) if pro.weight is not None else ""
+            a("  #define EMH_GLOAD(kt, S) { \\")
+            a(f'    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) {{ ra[S][i] = *(const u32x4*)(ga[i] + (kt) * BK);{wload} }} \\')
+            a('    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[S][i] = *(const u32x4*)(gb[i] + (kt) * BK); }')
             env = {"x": "(float)xv_[e]", "ss": "ss[i]"}
             if pro.weight is not None:
-                env["w"] = "(float)rw[i][e]"
-            a("  #define EMH_LSTORE(buf) { \\")
+                env["w"] = "(float)rw[S][i][e]"
+            a("  #define EMH_LSTORE(buf, S) { \\")
             a("    unsigned char* s_ = emh_lds + (buf) * SLAB; \\")
             a('    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) { \\')
-            a(f"      {frag_t} xv_ = __builtin_bit_cast({frag_t}, ra[i]); \\")
+            a(f"      {frag_t} xv_ = __builtin_bit_cast({frag_t}, ra[S][i]); \\")
             a(f'      _Pragma("unroll") for (int e = 0; e < 8; ++e) xv_[e] = ({in_c})({E.render(pro.project, env)}); \\')
             a(f"      *({frag_t}*)(s_ + la[i]) = xv_; }} \\")
-            a('    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[i]; }')
+            a('    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[S][i]; }')
         else:
-            a(r"""  u32x4 ra[A_PER_T], rb[B_PER_T];
-  #define EMH_GLOAD(kt) { \
-    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) ra[i] = *(const u32x4*)(ga[i] + (kt) * BK); \
-    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[i] = *(const u32x4*)(gb[i] + (kt) * BK); }
-  #define EMH_LSTORE(buf) { \
+            a(r"""  u32x4 ra[RS][A_PER_T], rb[RS][B_PER_T];
+  #define EMH_GLOAD(kt, S) { \
+    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) ra[S][i] = *(const u32x4*)(ga[i] + (kt) * BK); \
+    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[S][i] = *(const u32x4*)(gb[i] + (kt) * BK); }
+  #define EMH_LSTORE(buf, S) { \
     unsigned char* s_ = emh_lds + (buf) * SLAB; \
-    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) *(u32x4*)(s_ + la[i]) = ra[i]; \
-    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[i]; }""")
-        a(r"""  EMH_GLOAD(0);
-  EMH_LSTORE(0);
+    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) *(u32x4*)(s_ + la[i]) = ra[S][i]; \
+    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[S][i]; }""")
+        # Slab j travels through register set j % RS: RS slabs are in flight from
+        # global memory while one is computed on, so a load has RS steps to arrive.
+        a(r"""  #pragma unroll
+  for (int p = 0; p < RS; ++p) if (p < KT) EMH_GLOAD(p, p);
+  EMH_LSTORE(0, 0);
   __syncthreads();
-  for (int kt = 0; kt < KT; ++kt) {
+  for (int kt0 = 0; kt0 < KT; kt0 += RS) {
+  #pragma unroll
+  for (int rs = 0; rs < RS; ++rs) {
+    const int kt = kt0 + rs;
+    if (KT % RS != 0 && kt >= KT) break;
     const int cur = kt % DEPTH;
-    if (kt + 1 < KT) EMH_GLOAD(kt + 1);
+    if (kt + RS < KT) EMH_GLOAD(kt + RS, rs);  // set rs held slab kt, which is in LDS by now
     EMH_READ(0, cur, 0);""")
         for kk in range(KS):
             if kk + 1 < KS:
                 a(f"    EMH_READ({(kk + 1) & 1}, cur, {kk + 1});")
             a(f"    EMH_MMA({kk & 1});")
-        a(r"""    if (kt + 1 < KT) EMH_LSTORE((kt + 1) % DEPTH);
+        a(r"""    if (kt + 1 < KT) EMH_LSTORE((kt + 1) % DEPTH, (rs + 1) % RS);
     __syncthreads();
+  }
   }""")
     else:
         if KS % 2:

@@ -500,7 +500,7 @@ def test_staging_transports_are_bit_identical(device, monkeypatch):
     x = case.inputs[0].to(device)
     monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x2/f1x2/k4")
     outs = {}
-    for stage in ("d2/sync", "d2/dl", "d3/dl", "d4/dl"):
+    for stage in ("d2/sync", "d2/sync/p2", "d2/sync/p3", "d2/dl", "d3/dl", "d4/dl"):  # 16 slabs: not a multiple of three register sets
         monkeypatch.setenv("EMMY_STAGE", stage)
         be = HipBackend()
         compiled = be.compile(graph)

@@ -57,6 +57,8 @@ def test_linear_is_one_mfma_kernel(launcher_lib, m):
     assert k.kernel_name.startswith("k_linear_")
     assert "__builtin_amdgcn_mfma_f32_" in k.kernel_source
     assert k.algo_flops == 2 * m * 3072 * 1024
+    # decode sizes stream the weight from HBM: two slabs in flight through two register sets
+    assert k.knobs["STAGE"] == ("d2/sync/p2" if m <= 128 else "d2/sync") and ("ra[RS][A_PER_T]" in k.kernel_source)
     hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
 
 
