@@ -47,7 +47,7 @@ TILE_SWEEP: tuple[str, ...] = (
     "a:mfma_16x16x32_bf16/w1x1/f1x1/k8",
     "a:mfma_16x16x32_bf16/w1x4/f1x1/k8",
 )
-STAGE_SWEEP: tuple[str, ...] = ("d2/sync", "d3/dl")
+STAGE_SWEEP: tuple[str, ...] = ("d2/sync", "d2/sync/p2", "d3/dl")
 REDUCE_SWEEP: tuple[str, ...] = ("b8", "b16", "b32", "b64", "b128", "b256", "b512", "b1024")
 NT_SWEEP: tuple[str, ...] = ("0", "1")
 FLASH_SWEEP: tuple[str, ...] = (
