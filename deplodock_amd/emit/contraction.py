@@ -438,9 +438,9 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   #define EMH_DLOAD(kt, buf) { \
     unsigned char* s_ = emh_lds + (buf) * SLAB; \
     _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) \
-      __builtin_amdgcn_global_load_lds((const void*)(ga[i] + (kt) * BK), (__attribute__((address_space(3))) void*)(s_ + la[i] - lane * 16), 16, 0, 0); \
+      emh_dma16(ga[i] + (kt) * BK, s_ + la[i] - lane * 16); \
     _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) \
-      __builtin_amdgcn_global_load_lds((const void*)(gb[i] + (kt) * BK), (__attribute__((address_space(3))) void*)(s_ + lb[i] - lane * 16), 16, 0, 0); }
+      emh_dma16(gb[i] + (kt) * BK, s_ + lb[i] - lane * 16); }
   // A plain s_barrier is used on purpose: a workgroup fence would drain every
   // outstanding direct-to-LDS load and serialise the pipeline.  Loads retire in
   // issue order, so "at most n outstanding" means the older slabs have landed.
@@ -450,7 +450,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   // them before the barrier.
   #define EMH_SLAB_SYNC(n) { \
     __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM_LGKM0(n)); \
-    { const unsigned d_ = *(volatile unsigned*)(emh_lds + tid * 4); asm volatile("s_waitcnt lgkmcnt(0)" :: "v"(d_) : "memory"); } \
+    emh_lds_publish(emh_lds + tid * 4); \
     asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
   #pragma unroll
   for (int p = 0; p < DEPTH; ++p) if (p < KT) EMH_DLOAD(p, p);""")

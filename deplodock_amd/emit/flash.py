@@ -110,8 +110,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       if (QCHUNKS % NT == 0 || c0 + (tid - lane) < QCHUNKS) {  // whole waves: QCHUNKS is a multiple of 64
         const int r_ = (c0 + tid) / CPR, p_ = (c0 + tid) % CPR;
         const int qr_ = q0 + r_ < SQ ? q0 + r_ : SQ - 1;
-        __builtin_amdgcn_global_load_lds((const void*)(qbase + (long)qr_ * Q_SS + emh_kswz(r_, p_) * 8),
-                                         (__attribute__((address_space(3))) void*)(lds + Q_OFF_LDS + (c0 + tid - lane) * 16), 16, 0, 0);
+        emh_dma16(qbase + (long)qr_ * Q_SS + emh_kswz(r_, p_) * 8, lds + Q_OFF_LDS + (c0 + tid - lane) * 16);
       }
     }
   } else {
@@ -147,8 +146,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       if (SKV % (KVS * BKV) != 0) { const long lim_ = SKV - 1 - st_row; if (krow_ > lim_) krow_ = lim_; } \
       const int kc_ = emh_kswz(st_row + ro_, st_pos), vc_ = emh_vswz(st_row + ro_, st_pos); \
       unsigned char* dk_ = sb_ + g_ * 2 * KBYTES + (((i) * NT) % CHUNKS) * 16; \
-      __builtin_amdgcn_global_load_lds((const void*)(gk_lane + krow_ * K_SS + kc_ * 8), (__attribute__((address_space(3))) void*)dk_, 16, 0, 0); \
-      __builtin_amdgcn_global_load_lds((const void*)(gv_lane + krow_ * V_SS + vc_ * 8), (__attribute__((address_space(3))) void*)(dk_ + KBYTES), 16, 0, 0); }
+      emh_dma16(gk_lane + krow_ * K_SS + kc_ * 8, dk_); \
+      emh_dma16(gv_lane + krow_ * V_SS + vc_ * 8, dk_ + KBYTES); }
   // Request i of a step is issued behind score MFMA number EMH_SLOT_OF(i): spread
   // evenly over the chain, so the loads trickle into the memory pipeline instead of
   // arriving as one burst from every wave, and all of them are on their way before
@@ -163,8 +162,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   // waiting for that read orders them before the barrier.
   #define EMH_DMA_FENCE() { \
     __builtin_amdgcn_s_waitcnt(0x0070); /* vmcnt(0) lgkmcnt(0) */ \
-    const unsigned d_ = *(volatile unsigned*)(lds + tid * 4); \
-    asm volatile("s_waitcnt lgkmcnt(0)" :: "v"(d_) : "memory"); }
+    emh_lds_publish(lds + tid * 4); }
 
   f32x16 oacc[D / 32];
   #pragma unroll

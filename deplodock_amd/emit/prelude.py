@@ -24,6 +24,26 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
 #define EMH_DEV __device__ __forceinline__
 EMH_DEV float emh_round_bf16(float v) { return (float)(__bf16)v; }
+// Direct-to-LDS load of 16 bytes per lane: lane l's bytes land at lds_base + 16*l
+// (lds_base: the wave-uniform LDS byte address, carried in M0).  Issued as inline
+// assembly on purpose: for the builtin the compiler assumes any later LDS read may
+// alias the load's LDS write and drains every outstanding load (vmcnt(0)) before
+// it, which turns a ring of slabs into one slab in flight.  The caller orders
+// reads after loads itself (vmcnt wait, LDS fence read, barrier).
+EMH_DEV unsigned emh_lds_addr(const void* p) { return (unsigned)(unsigned long)(__attribute__((address_space(3))) const void*)p; }
+// Publishing direct-to-LDS data to the other waves: the counter that tracks the
+// loads can reach its target before the LDS writes are visible.  A flat load from
+// LDS travels the same path as those writes and so queues behind them; waiting for
+// it (on the LDS counter alone: the vector-memory counter would also drain the
+// younger loads of the ring) orders them before the barrier that follows.
+EMH_DEV void emh_lds_publish(const void* lds_generic) {
+  unsigned d_;
+  asm volatile("flat_load_dword %0, %1 sc0 sc1\n\ts_waitcnt lgkmcnt(0)" : "=v"(d_) : "v"(lds_generic) : "memory");
+}
+EMH_DEV void emh_dma16(const void* g, const void* lds_wave_base) {
+  const unsigned m0_ = __builtin_amdgcn_readfirstlane(emh_lds_addr(lds_wave_base));
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(g), "s"(m0_) : "memory");
+}
 """
 
 # Wave64 butterflies.  Each step combines a lane with its partner at XOR

@@ -210,6 +210,39 @@ def _check_tile(plan: TilePlan, body: Contraction, ctx: Context, depth: int, dl:
         raise ScheduleError(f"the row epilogue needs output tiles of whole {re.cols}-column groups")
 
 
+def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
+    """Staging when nothing pins it.
+
+    * A row-normalised operand is transformed in registers on its way to LDS: ``sync``.
+    * Decode-size problems (M <= 128) stream the weight once, straight from HBM: ``sync``
+      through two register sets (measured with operands rotating through more memory
+      than the caches hold: 4.4 / 4.5 / 6.2 us at M = 1 / 16 / 128 on 1024x3072, against
+      5.2 / 5.4 / 6.9 through one set and 4.6 / 4.6 / 6.4 with a three-slab ``dl`` ring).
+    * Everything else: direct-to-LDS loads; a ring of three slabs where the LDS holds them
+      and a slab is less than ~600 cycles of MFMA work, else two (us, ``d2/sync`` -> ``d2/dl`` -> ``d3/dl``: 512x1024x3072 12.2 -> 9.5 ->
+      9.4; 512x1024x2048 7.4 -> 6.2 -> 6.2; 512x4096x1024 7.8 -> 6.8 -> 6.7; 2048x3072x1024
+      17.2 -> 15.9 -> 16.1; 4096^3 136 -> 122; the block as one graph 66.9 -> 65.2 -> 62.8)."""
+    steps = body.k // plan.bk_elems
+    if body.a_prologue is not None:
+        return Stage(depth=2, transport="sync")
+    if body.m <= 128:
+        return Stage(depth=2, transport="sync", reg_depth=2 if steps >= 3 else 1)
+    if (plan.bk_elems // plan.atom.k) % 2 == 0:
+        # a slab that keeps the matrix pipe busy for long hides the next one's latency by itself
+        mfma_cycles = plan.tile_m * plan.tile_n * (2 if body.gate_pair else 1) * plan.bk_elems * 2 // 4096
+        for depth in (3, 2):
+            if depth == 3 and (steps < 3 or mfma_cycles >= 600):
+                continue
+            try:
+                _check_tile(plan, body, ctx, depth=depth, dl=True)
+            except ScheduleError:
+                continue
+            loads = (plan.tile_m + plan.tile_n * (2 if body.gate_pair else 1)) * (plan.bk_elems // 8) // plan.block_threads
+            if (depth - 1) * loads <= 63:  # the vector-memory counter has six bits
+                return Stage(depth=depth, transport="dl")
+    return Stage(depth=2, transport="sync")
+
+
 def schedule_contraction(body: Contraction, ctx: Context) -> dict:
     tuned = _tuned(body, ctx)
     pinned = _pin("TILE", tuned)
@@ -248,11 +281,7 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
         logger.warning("STAGE=%s ignored: the row-normalised operand is transformed in registers (sync staging only)", stage.spell())
         stage = None
     if stage is None:
-        # Decode-size problems stream the weight once, straight from HBM: two register
-        # sets keep two slabs in flight per workgroup (measured with operands rotating
-        # through more memory than the caches hold: 5.2 -> 4.4 us at M=1, 6.9 -> 6.2 us
-        # at M=128 on 1024x3072; no change once the operands sit in the L2).
-        stage = Stage(depth=2, transport="sync", reg_depth=2 if body.m <= 128 and body.k // plan.bk_elems >= 3 else 1)
+        stage = _default_stage(plan, body, ctx)
     body.stage = stage
     return {"TILE": plan.spell(), "STAGE": stage.spell()}
 

@@ -58,7 +58,9 @@ def test_linear_is_one_mfma_kernel(launcher_lib, m):
     assert "__builtin_amdgcn_mfma_f32_" in k.kernel_source
     assert k.algo_flops == 2 * m * 3072 * 1024
     # decode sizes stream the weight from HBM: two slabs in flight through two register sets
-    assert k.knobs["STAGE"] == ("d2/sync/p2" if m <= 128 else "d2/sync") and ("ra[RS][A_PER_T]" in k.kernel_source)
+    # larger ones take direct-to-LDS loads (two slabs: a 128x192x64 slab is 768 cycles of MFMA work)
+    assert k.knobs["STAGE"] == ("d2/sync/p2" if m <= 128 else "d2/dl")
+    assert ("ra[RS][A_PER_T]" in k.kernel_source) == (m <= 128) and ("#define EMH_DLOAD" in k.kernel_source) == (m > 128)
     hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
 
 
@@ -144,13 +146,13 @@ def test_tile_and_stage_pins(launcher_lib, monkeypatch):
     monkeypatch.setenv("EMMY_STAGE", "d3/cp")
     k = kernels(compile_case(case))[0]
     assert k.knobs["TILE"] == "a:mfma_32x32x16_bf16/w2x2/f2x3/k4" and k.knobs["STAGE"] == "d3/dl"
-    assert "__builtin_amdgcn_global_load_lds" in k.kernel_source and k.lds_bytes == 3 * (128 + 192) * 64 * 2
+    assert "emh_dma16(" in k.kernel_source and "global_load_lds_dwordx4" in k.kernel_source and k.lds_bytes == 3 * (128 + 192) * 64 * 2
     assert k.grid[0] == (256,)
     hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
     monkeypatch.setenv("EMMY_TILE", "a:mma_m16n8k16_bf16/w2x2/f4x8/k2")  # an NVIDIA pin degrades to the gfx950 pick
     monkeypatch.setenv("EMMY_STAGE", "d2/tma")
     k = kernels(compile_case(case))[0]
-    assert "mfma" in k.knobs["TILE"] and k.knobs["STAGE"] == "d2/sync"
+    assert "mfma" in k.knobs["TILE"] and k.knobs["STAGE"] == "d2/dl"  # the default staging of this shape
 
 
 def test_flash_pin_grammar_and_degrade(launcher_lib, monkeypatch):
