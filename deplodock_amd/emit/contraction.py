@@ -186,8 +186,8 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
         raise LoweringError(f"contraction: tile {TM}x{TN}x{BK} does not divide over {T} threads")
     A_PER_T, B_PER_T = a_chunks // T, b_chunks // T
     slab_bytes = (TM + TN * NB) * BK * 2
-    depth = max(2, stage.depth)
-    RS = 1 if stage.transport == "dl" else max(1, stage.reg_depth)  # register sets a slab travels through on the sync path
+    depth = 2 if stage.transport == "mix" else max(2, stage.depth)
+    RS = 1 if stage.transport in ("dl", "mix") else max(1, stage.reg_depth)  # register sets a slab travels through on the sync path
     lds_bytes = slab_bytes * depth
     if lds_bytes > ctx.lds_bytes_per_cu:
         raise LoweringError(f"contraction: {lds_bytes} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
@@ -201,6 +201,9 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     m_guard = M % TM != 0
     n_guard = N % TN != 0
     dl = stage.transport == "dl"
+    mix = stage.transport == "mix"  # a through registers (it is transformed on the way), b direct to LDS
+    if mix and b_chunks % 64:
+        raise LoweringError("contraction: direct-to-LDS staging needs whole-wave chunk counts")
     if dl and (a_chunks % 64 or b_chunks % 64):
         raise LoweringError("contraction: direct-to-LDS staging needs whole-wave chunk counts")
 
@@ -306,7 +309,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     a(r"""  #pragma unroll
   for (int i = 0; i < B_PER_T; ++i) {
     const int q = tid + i * T;""")
-    if dl:
+    if dl or mix:
         a("    const int row = q / CPR, c = emh_swz(row, q % CPR);")
         a("    lb[i] = TM * BK * 2 + q * 16;")
     else:
@@ -358,7 +361,16 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
 """.replace("FRAG_T", frag_t).replace("BUILTIN", plan.atom.builtin))
     KS = BK // KSTEP
     if not dl:
-        # global -> VGPR -> LDS, one slab ahead, one barrier per slab.
+        # global -> VGPR -> LDS, one slab ahead, one barrier per slab.  With the
+        # mixed transport only the a operand takes that road (it may be transformed on
+        # the way); the b slab is requested direct-to-LDS at the same moment and is
+        # waited for, and published, where the a slab is written.
+        if mix:
+            b_gload = '{ unsigned char* sd_ = emh_lds + ((kt) % DEPTH) * SLAB; _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) emh_dma16(gb[i] + (kt) * BK, sd_ + lb[i] - lane * 16); }'
+            b_lstore = "__builtin_amdgcn_s_waitcnt(EMH_WAIT_VM_LGKM0(0)); emh_lds_publish(emh_lds + tid * 4);"
+        else:
+            b_gload = '_Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[S][i] = *(const u32x4*)(gb[i] + (kt) * BK);'
+            b_lstore = '_Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[S][i];'
         if pro is not None:
             # Row statistic over the full k extent of this thread's rows: the chunks of
             # a row's slab sit in CPR consecutive lanes, so a lane sums its own chunk
@@ -385,7 +397,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
             wload = " rw[S][i] = *(const FRAG_T*)(NW + (kt) * BK + ca[i]);".replace("FRAG_T", frag_t) if pro.weight is not None else ""
             a("  #define EMH_GLOAD(kt, S) { \\")
             a(f'    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) {{ ra[S][i] = *(const u32x4*)(ga[i] + (kt) * BK);{wload} }} \\')
-            a('    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[S][i] = *(const u32x4*)(gb[i] + (kt) * BK); }')
+            a("    " + b_gload + " }")
             env = {"x": "(float)xv_[e]", "ss": "ss[i]"}
             if pro.weight is not None:
                 env["w"] = "(float)rw[S][i][e]"
@@ -395,16 +407,16 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
             a(f"      {frag_t} xv_ = __builtin_bit_cast({frag_t}, ra[S][i]); \\")
             a(f'      _Pragma("unroll") for (int e = 0; e < 8; ++e) xv_[e] = ({in_c})({E.render(pro.project, env)}); \\')
             a(f"      *({frag_t}*)(s_ + la[i]) = xv_; }} \\")
-            a('    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[S][i]; }')
+            a("    " + b_lstore + " }")
         else:
             a(r"""  u32x4 ra[RS][A_PER_T], rb[RS][B_PER_T];
   #define EMH_GLOAD(kt, S) { \
     _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) ra[S][i] = *(const u32x4*)(ga[i] + (kt) * BK); \
-    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[S][i] = *(const u32x4*)(gb[i] + (kt) * BK); }
+    B_GLOAD }
   #define EMH_LSTORE(buf, S) { \
     unsigned char* s_ = emh_lds + (buf) * SLAB; \
     _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) *(u32x4*)(s_ + la[i]) = ra[S][i]; \
-    _Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[S][i]; }""")
+    B_LSTORE }""".replace("B_GLOAD", b_gload).replace("B_LSTORE", b_lstore))
         # Slab j travels through register set j % RS: RS slabs are in flight from
         # global memory while one is computed on, so a load has RS steps to arrive.
         a(r"""  #pragma unroll

@@ -223,7 +223,7 @@ class TilePlan:
 # STAGE
 # --------------------------------------------------------------------------
 
-_TRANSPORTS = {"sync": "sync", "dl": "dl", "cp": "dl"}
+_TRANSPORTS = {"sync": "sync", "dl": "dl", "cp": "dl", "mix": "mix"}
 
 
 @dataclass(frozen=True)
@@ -233,7 +233,8 @@ class Stage:
     ``depth``      LDS slabs in the ring (2 = double buffer).
     ``transport``  ``sync``: global → registers → ``ds_write`` (software
                    pipelined through ``reg_depth`` register sets);
-                   ``dl``: global loads that write LDS directly, no VGPR hop.
+                   ``dl``: global loads that write LDS directly, no VGPR hop;
+                   ``mix``: the a operand as ``sync``, the b operand as ``dl``.
     ``ring``       kept for grammar compatibility (a depth > 1 is a ring)."""
 
     depth: int = 2
@@ -261,7 +262,7 @@ class Stage:
             elif re.fullmatch(r"p\d+", tok):
                 kw["reg_depth"] = int(tok[1:])
             else:
-                raise ScheduleError(f"STAGE: cannot parse {tok!r} (expect d<depth> / sync|dl / ring / p<reg_depth>)")
+                raise ScheduleError(f"STAGE: cannot parse {tok!r} (expect d<depth> / sync|dl|mix / ring / p<reg_depth>)")
         st = cls(**kw)
         if not 1 <= st.depth <= 8:
             raise ScheduleError(f"STAGE: depth must be 1..8, got {st.depth}")

@@ -36,7 +36,7 @@ logger = logging.getLogger(__name__)
 # where a step of the k loop costs one L2-miss round trip whatever its size: deep
 # slabs (256 elements) and 4-8 waves per workgroup won every such shape.
 TILE_CANDIDATES: tuple[tuple[int, int, int, int, str, int], ...] = (
-    (256, 256, 2, 4, "mfma_32x32x16_bf16", 4),  # 962-977 TFLOP/s on 4096^3 and 8192x8192x4096
+    (256, 256, 2, 4, "mfma_16x16x32_bf16", 2),  # 4096^3 with a two-slab dl ring: 111.8 us = 1 230 TFLOP/s (32x32x16 atoms, same tile: 119.5 us)
     (128, 192, 4, 2, "mfma_16x16x32_bf16", 2),
     (128, 128, 2, 2, "mfma_32x32x16_bf16", 4),
     (128, 96, 4, 1, "mfma_32x32x16_bf16", 4),
@@ -213,7 +213,8 @@ def _check_tile(plan: TilePlan, body: Contraction, ctx: Context, depth: int, dl:
 def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
     """Staging when nothing pins it.
 
-    * A row-normalised operand is transformed in registers on its way to LDS: ``sync``.
+    * A row-normalised operand is transformed in registers on its way to LDS: ``sync``
+      (``mix`` sends the other operand direct to LDS; 12.7 / 15.8 us against 12.3 / 15.9 us).
     * Decode-size problems (M <= 128) stream the weight once, straight from HBM: ``sync``
       through two register sets (measured with operands rotating through more memory
       than the caches hold: 4.4 / 4.5 / 6.2 us at M = 1 / 16 / 128 on 1024x3072, against
@@ -224,7 +225,7 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
       17.2 -> 15.9 -> 16.1; 4096^3 136 -> 122; the block as one graph 66.9 -> 65.2 -> 62.8)."""
     steps = body.k // plan.bk_elems
     if body.a_prologue is not None:
-        return Stage(depth=2, transport="sync")
+        return Stage(depth=2, transport="sync")  # ``mix`` (b direct to LDS) measures the same on the block's two such kernels
     if body.m <= 128:
         return Stage(depth=2, transport="sync", reg_depth=2 if steps >= 3 else 1)
     if (plan.bk_elems // plan.atom.k) % 2 == 0:
@@ -277,8 +278,8 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
         except ScheduleError as exc:
             logger.warning("EMMY_STAGE=%r ignored: %s", pinned_stage, exc)
             stage = None
-    if stage is not None and body.a_prologue is not None and stage.transport != "sync":
-        logger.warning("STAGE=%s ignored: the row-normalised operand is transformed in registers (sync staging only)", stage.spell())
+    if stage is not None and body.a_prologue is not None and stage.transport == "dl":
+        logger.warning("STAGE=%s ignored: the row-normalised operand is transformed in registers (sync or mix staging only)", stage.spell())
         stage = None
     if stage is None:
         stage = _default_stage(plan, body, ctx)

@@ -491,6 +491,16 @@ def test_fused_pointwise_with_broadcasts_and_row_reductions(device):
         prog.close()
 
 
+def test_mixed_staging_with_a_normalised_operand(device, monkeypatch):
+    """``STAGE=d2/mix``: the normalised operand goes through registers, the weight slab direct to LDS."""
+    monkeypatch.setenv("EMMY_STAGE", "d2/mix")
+    case = eager.qwen3_block_case(seq=64)
+    ours, want, compiled = run_case(case, device)
+    stages = [n.op.knobs.get("STAGE") for n in compiled.nodes.values() if isinstance(n.op, HipOp) and "TILE" in n.op.knobs]
+    assert stages and all(s == "d2/mix" for s in stages)
+    eager.assert_close(ours, want, case.rtol, case.atol, "block with mixed staging vs eager (GPU)")
+
+
 def test_staging_transports_are_bit_identical(device, monkeypatch):
     """How operands reach LDS (through registers, or direct-to-LDS at any depth) must not change a
     single output bit: same tile, same MFMA order (the reference pins the same property across its
@@ -500,7 +510,7 @@ def test_staging_transports_are_bit_identical(device, monkeypatch):
     x = case.inputs[0].to(device)
     monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x2/f1x2/k4")
     outs = {}
-    for stage in ("d2/sync", "d2/sync/p2", "d2/sync/p3", "d2/dl", "d3/dl", "d4/dl"):  # 16 slabs: not a multiple of three register sets
+    for stage in ("d2/sync", "d2/sync/p2", "d2/sync/p3", "d2/mix", "d2/dl", "d3/dl", "d4/dl"):  # 16 slabs: not a multiple of three register sets
         monkeypatch.setenv("EMMY_STAGE", stage)
         be = HipBackend()
         compiled = be.compile(graph)
