@@ -65,10 +65,9 @@ def _emit_row_epilogue_tables(a, re, re_args: list[str], EPC: int, m_guard: bool
     need (they depend on the output coordinates only): the k loop hides the latency."""
     d = re.cols
     vt_chunk = {2: None, 4: "f32x4"}.get(16 // EPC) or ("bf16x8" if re.row_operands and re.row_operands[0].dtype.name == "bf16" else "f16x8")
-    in_project = E.variables(re.project)
     a(f"  constexpr int RE_IT = (TM * (TN / {EPC})) / T;")
     for nm, ro in zip(re_args, re.row_operands):
-        a(f"  {vt_chunk} {nm}_v[RE_IT]" + (f", {nm}_p[RE_IT];" if re.rotate is not None and ro.name in in_project else ";"))
+        a(f"  {vt_chunk} {nm}_v[RE_IT];")
     a(f"  if (n0 < {re.col_end}) {{")
     a("    #pragma unroll")
     a("    for (int it = 0; it < RE_IT; ++it) {")
@@ -79,8 +78,6 @@ def _emit_row_epilogue_tables(a, re, re_args: list[str], EPC: int, m_guard: bool
     for nm, ro in zip(re_args, re.row_operands):
         a(f"      const {ro.dtype.c_name}* {nm}_row = {nm} + {ro.offset}L + ((rr / {ro.div}) % {ro.mod}) * {d};")
         a(f"      {nm}_v[it] = *(const {vt_chunk}*)({nm}_row + gc);")
-        if re.rotate is not None and ro.name in in_project:
-            a(f"      {nm}_p[it] = *(const {vt_chunk}*)({nm}_row + (gc ^ {d // 2}));")
     a("    }")
     a("  }")
 
@@ -128,16 +125,19 @@ def _emit_row_epilogue(a, body: Contraction, re, re_args: list[str], EPC: int, v
         a(f"      yo[r] = {cast}({E.render(re.project, env)});")
         a("    }")
     else:
-        a(f"    const {vt_chunk} pv = *(const {vt_chunk}*)(emh_lds + row * CSTRIDE + (cc ^ {HC // 2}) * 16);  // the half-rotated partner chunk")
+        # The half-rotated partner of a chunk is the chunk HC/2 further on in the same group,
+        # i.e. the projected values of the lane HC/2 away: fetched across lanes, not recomputed.
+        fetch = "emh_dpp<0x128>(yv[r])" if HC == 16 else f"__shfl_xor(yv[r], {HC // 2}, 64)"  # row_ror:8 inside a 16-lane row
         a(f"    const float sgn = (cc % {HC}) < {HC // 2} ? -1.0f : 1.0f;")
+        a(f"    float yv[{EPC}];")
+        a("    #pragma unroll")
+        env_own = dict(env_stats, x="(float)xv[r]", **{ro.name: f"(float){nm}_v[it][r]" for nm, ro in zip(re_args, re.row_operands) if ro.name in in_project})
+        a(f"    for (int r = 0; r < {EPC}; ++r) yv[r] = {E.render(re.project, env_own)};")
         a(f"    {vt_chunk} yo;")
         a("    #pragma unroll")
         a(f"    for (int r = 0; r < {EPC}; ++r) {{")
-        env_own = dict(env_stats, x="(float)xv[r]", **{ro.name: f"(float){nm}_v[it][r]" for nm, ro in zip(re_args, re.row_operands) if ro.name in in_project})
-        env_par = dict(env_stats, x="(float)pv[r]", **{ro.name: f"(float){nm}_p[it][r]" for nm, ro in zip(re_args, re.row_operands) if ro.name in in_project})
-        a(f"      const float y_ = {E.render(re.project, env_own)};")
-        a(f"      const float yr_ = sgn * ({E.render(re.project, env_par)});")
-        env_rot = dict(env_stats, y="y_", yr="yr_", **{ro.name: f"(float){nm}_v[it][r]" for nm, ro in zip(re_args, re.row_operands) if ro.name in in_rotate})
+        a(f"      const float yr_ = sgn * {fetch};")
+        env_rot = dict(env_stats, y="yv[r]", yr="yr_", **{ro.name: f"(float){nm}_v[it][r]" for nm, ro in zip(re_args, re.row_operands) if ro.name in in_rotate})
         a(f"      yo[r] = {cast}({E.render(re.rotate.expr, env_rot)});")
         a("    }")
     conds = (["m < M"] if m_guard else []) + (["n < N"] if n_guard else [])
@@ -287,8 +287,6 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   const int wm = wave / WN, wn = wave % WN;
   const int lr = lane % AM, lk = lane / AM;  // fragment row, k-group
 """)
-    if body.row_epilogue is not None:
-        _emit_row_epilogue_tables(a, body.row_epilogue, [f"re{i}" for i in range(len(body.row_epilogue.row_operands))], 16 // body.out_dtype.nbytes, m_guard)
     # ---- staging ------------------------------------------------------------
     a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else ""))
     a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
@@ -423,6 +421,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   for (int p = 0; p < RS; ++p) if (p < KT) EMH_GLOAD(p, p);
   EMH_LSTORE(0, 0);
   __syncthreads();
+ROW_EPILOGUE_TABLES
   for (int kt0 = 0; kt0 < KT; kt0 += RS) {
   #pragma unroll
   for (int rs = 0; rs < RS; ++rs) {
@@ -469,6 +468,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         first_younger = min(depth - 1, KT - 1) * loads_per_slab
         a(f"  EMH_SLAB_SYNC({first_younger});")
         a("  EMH_READ(0, 0, 0);")
+        a("ROW_EPILOGUE_TABLES")
 
         def slab_steps(kt: str, static_kt: int | None) -> None:
             """MFMA steps of slab ``kt``.  With ``static_kt`` the hand-over to the
@@ -619,7 +619,13 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
 // bits 3:0, vmcnt[5:4] in bits 15:14; expcnt left at its maximum, lgkmcnt = 0).
 #define EMH_WAIT_VM_LGKM0(n) ((((n) & 0xF) | ((((n) >> 4) & 0x3) << 14)) | 0x0070)
 """
-    source = prelude.header(vm_macro, *((prelude.WAVE_REDUCE,) if rowepi is not None else ())) + "\n".join(o) + "\n"
+    # The row epilogue's table chunks are requested once the first slab is on its way (loads
+    # retire in order: requested earlier, the cold tables would hold up the operands behind them)
+    # and are not looked at before the k loop is over.
+    tables: list[str] = []
+    if rowepi is not None:
+        _emit_row_epilogue_tables(tables.append, rowepi, re_args, EPC, m_guard)
+    source = prelude.header(vm_macro, *((prelude.WAVE_REDUCE,) if rowepi is not None else ())) + "\n".join(o).replace("ROW_EPILOGUE_TABLES", "\n".join(tables)) + "\n"
     if N % 4 or TN % 4:
         raise LoweringError("contraction: N must be a multiple of 4 (8-byte output runs)")
     n_blocks = (tiles_m // gm) * (tiles_n // gn)
