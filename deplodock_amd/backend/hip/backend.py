@@ -115,7 +115,12 @@ class HipBackend(Backend):
                 import torch
 
                 parts = [data[p] if p in data else traced[p] for p in stacked.parts]
-                data[nid] = torch.cat([p if isinstance(p, torch.Tensor) else torch.as_tensor(p) for p in parts], dim=0).contiguous()
+                whole = torch.cat([p if isinstance(p, torch.Tensor) else torch.as_tensor(p) for p in parts], dim=0).contiguous()
+                if stacked.k_scale is not None:
+                    ks = data[stacked.k_scale] if stacked.k_scale in data else traced[stacked.k_scale]
+                    ks = ks if isinstance(ks, torch.Tensor) else torch.as_tensor(ks)
+                    whole = (whole.float() * ks.to(whole.device).float().reshape(1, -1)).to(whole.dtype)
+                data[nid] = whole
             elif nid in traced:
                 data[nid] = traced[nid]
         return data

@@ -220,12 +220,15 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
         raise LoweringError(f"contraction epilogue uses unknown names {sorted(unknown)} (operands belong in `post`)")
 
     pro = body.a_prologue
+    deferred = pro is not None and pro.scale is not None
+    if deferred and (pro.weight is not None or E.variables(pro.scale) - {"ss"}):
+        raise LoweringError("contraction: a deferred row scale is an expression over the row statistic; the column weight belongs in the b operand")
     if pro is not None:
         if dl:
             raise LoweringError("contraction: a row prologue transforms the operand in registers; it needs STAGE .../sync")
         if body.in_dtype.nbytes != 2 or (pro.weight is not None and pro.weight_dtype.nbytes != 2):
             raise LoweringError("contraction: the row prologue is written for 16-bit operands")
-        bad = (E.variables(pro.stat_pre) - {"x"}) | (E.variables(pro.project) - ({"x", "ss"} | ({"w"} if pro.weight else set())))
+        bad = (E.variables(pro.stat_pre) - {"x"}) | (set() if deferred else E.variables(pro.project) - ({"x", "ss"} | ({"w"} if pro.weight else set())))
         if bad:
             raise LoweringError(f"contraction: row prologue uses unknown names {sorted(bad)}")
         if CPR > 64:
@@ -377,19 +380,20 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
             a("  float ss[A_PER_T];")
             a("  #pragma unroll")
             a("  for (int i = 0; i < A_PER_T; ++i) ss[i] = 0.0f;")
-            a(f"  #pragma unroll {unroll}")
-            a("  for (int kt = 0; kt < KT; ++kt) {")
-            a("    #pragma unroll")
-            a("    for (int i = 0; i < A_PER_T; ++i) {")
-            a(f"      const {frag_t} xv = *(const {frag_t}*)(ga[i] + kt * BK);")
-            a("      #pragma unroll")
-            a("      for (int e = 0; e < 8; ++e) { const float x_ = (float)xv[e]; ss[i] += " + E.render(pro.stat_pre, {"x": "x_"}) + "; }")
-            a("    }")
-            a("  }")
-            a("  #pragma unroll")
-            a("  for (int i = 0; i < A_PER_T; ++i)")
-            a("  #pragma unroll")
-            a("  for (int msk = 1; msk < CPR; msk *= 2) ss[i] += __shfl_xor(ss[i], msk, 64);")
+            if not deferred:
+                a(f"  #pragma unroll {unroll}")
+                a("  for (int kt = 0; kt < KT; ++kt) {")
+                a("    #pragma unroll")
+                a("    for (int i = 0; i < A_PER_T; ++i) {")
+                a(f"      const {frag_t} xv = *(const {frag_t}*)(ga[i] + kt * BK);")
+                a("      #pragma unroll")
+                a("      for (int e = 0; e < 8; ++e) { const float x_ = (float)xv[e]; ss[i] += " + E.render(pro.stat_pre, {"x": "x_"}) + "; }")
+                a("    }")
+                a("  }")
+                a("  #pragma unroll")
+                a("  for (int i = 0; i < A_PER_T; ++i)")
+                a("  #pragma unroll")
+                a("  for (int msk = 1; msk < CPR; msk *= 2) ss[i] += __shfl_xor(ss[i], msk, 64);")
             wdecl = f" {frag_t} rw[RS][A_PER_T];" if pro.weight is not None else ""
             a(f"  u32x4 ra[RS][A_PER_T], rb[RS][B_PER_T];{wdecl}")
             wload = " rw[S][i] = *(const FRAG_T*)(NW + (kt) * BK + ca[i]);".replace("FRAG_T", frag_t) if pro.weight is not None else ""
@@ -403,7 +407,10 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
             a("    unsigned char* s_ = emh_lds + (buf) * SLAB; \\")
             a('    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) { \\')
             a(f"      {frag_t} xv_ = __builtin_bit_cast({frag_t}, ra[S][i]); \\")
-            a(f'      _Pragma("unroll") for (int e = 0; e < 8; ++e) xv_[e] = ({in_c})({E.render(pro.project, env)}); \\')
+            if deferred:  # the slab goes to LDS as it is; its share of the row statistic is taken on the way
+                a('      _Pragma("unroll") for (int e = 0; e < 8; ++e) { const float x_ = (float)xv_[e]; ss[i] += ' + E.render(pro.stat_pre, {"x": "x_"}) + "; } \\")
+            else:
+                a(f'      _Pragma("unroll") for (int e = 0; e < 8; ++e) xv_[e] = ({in_c})({E.render(pro.project, env)}); \\')
             a(f"      *({frag_t}*)(s_ + la[i]) = xv_; }} \\")
             a("    " + b_lstore + " }")
         else:
@@ -516,13 +523,31 @@ ROW_EPILOGUE_TABLES
   // of group g hold four consecutive n starting at g*4*KG + (l / AM)*4.""")
     if staged:
         lds_bytes = max(lds_bytes, TM * c_stride)
+    # The deferred row scales sit behind the output tile, inside the slab area: every step of the
+    # k loop ends with a barrier, so the slabs are dead when the scales are written.
+    rs_off = TM * c_stride if staged else 0
+    if deferred:
+        lds_bytes = max(lds_bytes, rs_off + TM * 4)
+        a("  // Row statistic: finish it over the lanes that hold a row's chunks, turn it into the row's")
+        a("  // scale factor and hand it to the lanes that own the row's accumulators.")
+        a("  #pragma unroll")
+        a("  for (int i = 0; i < A_PER_T; ++i) {")
+        a("    #pragma unroll")
+        a("    for (int msk = 1; msk < CPR; msk *= 2) ss[i] += __shfl_xor(ss[i], msk, 64);")
+        a(f"    if ((tid + i * T) % CPR == 0) ((float*)(emh_lds + {rs_off}))[(tid + i * T) / CPR] = {E.render(pro.scale, {'ss': 'ss[i]'})};")
+        a("  }")
+        if not staged:
+            a("  __syncthreads();")
+    if staged:
         a(f"  constexpr int CSTRIDE = {c_stride};")
         a("  __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM_LGKM0(0));" if dl else "")
         a("  __syncthreads();  // every wave is done with the operand slabs; reuse them for the output tile")
         a(r"""  #pragma unroll
   for (int i = 0; i < FM; ++i) {
-    const int ml = (wm * FM + i) * AM + lr;
-    #pragma unroll
+    const int ml = (wm * FM + i) * AM + lr;""")
+        if deferred:
+            a(f"    const float rs_ = ((const float*)(emh_lds + {rs_off}))[ml];")
+        a(r"""    #pragma unroll
     for (int j = 0; j < FN; ++j)
     #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -532,10 +557,11 @@ ROW_EPILOGUE_TABLES
             clamp = f"(n0 + nl < N ? n0 + nl : N - 4)" if n_guard else "(n0 + nl)"
             a(f"      const {bt4} bv = *(const {bt4}*)(BIAS + {clamp});")
         a(f"      {vt4} yo;")
+        sc = " * rs_" if deferred else ""
         for r in range(4):
-            env = {"acc": f"acc[0][i][j][g * 4 + {r}]"}
+            env = {"acc": f"(acc[0][i][j][g * 4 + {r}]{sc})"}
             if gate:
-                env["acc2"] = f"acc[1][i][j][g * 4 + {r}]"
+                env["acc2"] = f"(acc[1][i][j][g * 4 + {r}]{sc})"
             if body.bias is not None:
                 env["bias"] = f"(float)bv[{r}]"
             a(f"      yo[{r}] = {cast}({E.render(epi, env)});")
@@ -580,6 +606,8 @@ ROW_EPILOGUE_TABLES
         a(r"""  #pragma unroll
   for (int i = 0; i < FM; ++i) {
     const int m = m0 + (wm * FM + i) * AM + lr;""")
+        if deferred:
+            a(f"    const float rs_ = ((const float*)(emh_lds + {rs_off}))[(wm * FM + i) * AM + lr];")
         if m_guard:
             a("    if (m >= M) continue;")
         a(r"""    #pragma unroll
@@ -596,10 +624,11 @@ ROW_EPILOGUE_TABLES
             bt4 = _PACK4_T[body.bias_dtype.name]
             a(f"      const {bt4} bv = *(const {bt4}*)(BIAS + n);")
         a(f"      {vt4} yo;")
+        sc = " * rs_" if deferred else ""
         for r in range(4):
-            env = {"acc": f"acc[0][i][j][g * 4 + {r}]"}
+            env = {"acc": f"(acc[0][i][j][g * 4 + {r}]{sc})"}
             if gate:
-                env["acc2"] = f"acc[1][i][j][g * 4 + {r}]"
+                env["acc2"] = f"(acc[1][i][j][g * 4 + {r}]{sc})"
             if body.bias is not None:
                 env["bias"] = f"(float)bv[{r}]"
             pre = E.render(epi, env)
@@ -641,7 +670,7 @@ ROW_EPILOGUE_TABLES
         grid=((grid,), (1,), (1,)),
         block=((T,), (1,), (1,)),
         lds_bytes=lds_bytes,
-        comment=f"contraction M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()}" + (" a=row-normalised" if pro is not None else "") + (f" row-epilogue={rowepi.col_end // rowepi.cols}x{rowepi.cols}" if rowepi is not None else ""),
+        comment=f"contraction M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()}" + ((" a=row-scaled-after" if deferred else " a=row-normalised") if pro is not None else "") + (f" row-epilogue={rowepi.col_end // rowepi.cols}x{rowepi.cols}" if rowepi is not None else ""),
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
         knobs={"TILE": plan.spell(), "STAGE": stage.spell()},

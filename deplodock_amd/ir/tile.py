@@ -126,12 +126,24 @@ class RowPrologue:
     then maps each element with ``project`` (names ``x``, ``ss`` and, when
     ``weight`` is set, ``w`` — a length-``k`` vector) while staging the slab.
     ``project`` carries the producer's own rounding points, so the operand the
-    MFMAs see is bit-for-bit what the separate kernel would have written."""
+    MFMAs see is bit-for-bit what the separate kernel would have written.
+
+    With ``scale`` set the normalisation is *deferred*: when the projection is
+    ``x * f(ss) * w`` — a per-row factor and a per-column weight, as in RMSNorm —
+    then ``(x f(ss) w) @ W^T = f(ss) (x @ (W w)^T)``: the column weight is folded
+    into the constant ``b`` operand once, at bind time, the ``a`` operand is staged
+    untouched while its statistic is accumulated slab by slab, and the accumulators
+    are multiplied by ``scale`` (an expression over ``ss``) before the epilogue.
+    That drops the statistic pre-pass over the rows and the per-element transform
+    every workgroup of a row block would repeat; the normalised operand is then
+    never rounded to 16 bits, so the result is as close to the exact one as the
+    eager module's, not bit-equal to it."""
 
     stat_pre: Expr
     project: Expr
     weight: str | None = None
     weight_dtype: DType | None = None
+    scale: Expr | None = None
 
 
 @dataclass

@@ -53,6 +53,7 @@ class StackedConstant:
     emmy/compiler/ir/base.py:118-160)."""
 
     parts: tuple[str, ...]
+    k_scale: str | None = None  # a length-k constant multiplied into every row (a norm weight folded into the projection)
 
 
 @dataclass
@@ -157,13 +158,18 @@ def _matrix(view: View, what: str) -> tuple[int, int, int]:
     return rows, view.shape[-1], (ld if rows > 1 else view.shape[-1])
 
 
-def _a_operand(c: _Ctx, x_id: str, absorbers: set[str]) -> tuple[View, RowPrologue | None, list[str]]:
-    """The ``a`` operand of a contraction: ``(view, prologue, extra input buffers)``.
+def _a_operand(c: _Ctx, x_id: str, absorbers: set[str], fold: bool = False) -> tuple[View, RowPrologue | None, list[str], str | None]:
+    """The ``a`` operand of a contraction: ``(view, prologue, extra input buffers, weight to fold)``.
 
     When ``x_id`` is a row RMSNorm of 16-bit rows that nothing but the
     contractions in ``absorbers`` reads, the norm is not materialised: the view
     is the norm's *input* and the prologue carries its statistic and projection
-    (with the producer's rounding points), so ``norm -> linear`` is one launch."""
+    (with the producer's rounding points), so ``norm -> linear`` is one launch.
+
+    With ``fold`` the caller's ``b`` operand is a constant it assembles itself: the
+    normalisation is then deferred (``RowPrologue.scale``) and the fourth value names
+    the norm weight (a constant vector, or ``None``) the caller multiplies into the
+    columns of ``b``."""
     g = c.g
     node = g.nodes[x_id]
     if x_id not in c.done and x_id not in g.outputs and not (set(g.consumers(x_id)) - absorbers):
@@ -183,16 +189,18 @@ def _a_operand(c: _Ctx, x_id: str, absorbers: set[str]) -> tuple[View, RowProlog
                 wbuf = body.operand_buffers.get("w")
                 wdt = body.col_operands[0][1] if body.col_operands else None
                 if wbuf is None or wdt.nbytes == 2:
-                    shape = tuple(int(d) for d in node.output.shape)
                     view = View(xv.base, body.x_addr.offset, (body.rows, m.cols), (body.x_addr.stride_hi, 1), xv.dtype)
-                    del shape
-                    return view, RowPrologue(stat_pre=body.stats[0].pre, project=body.project, weight=wbuf, weight_dtype=wdt), ([wbuf] if wbuf else [])
-    return _need(c, x_id), None, []
+                    w_node = g.nodes[_peel_layout(g, m.weight)] if m.weight is not None else None
+                    if fold and (w_node is None or (isinstance(w_node.op, ConstantOp) and w_node.id == m.weight)):
+                        scale = E.Un("rsqrt", E.Var("ss") / float(m.cols) + m.eps)
+                        return view, RowPrologue(stat_pre=body.stats[0].pre, project=body.project, scale=scale), [], m.weight
+                    return view, RowPrologue(stat_pre=body.stats[0].pre, project=body.project, weight=wbuf, weight_dtype=wdt), ([wbuf] if wbuf else []), None
+    return _need(c, x_id), None, [], None
 
 
 def _linear_parts(c: _Ctx, nid: str):
     node = c.g.nodes[nid]
-    x, pro, extra = _a_operand(c, node.inputs[0], {nid})
+    x, pro, extra, _ = _a_operand(c, node.inputs[0], {nid})
     w = _need(c, node.inputs[1])
     m, k, lda = _matrix(x, "linear input")
     n, k2, ldb = _matrix(w, "linear weight")
@@ -258,19 +266,19 @@ def _rec_linear_siblings(c: _Ctx, nid: str) -> bool:
     ]
     if len(group) < 2:
         return False
-    x, pro, extra = _a_operand(c, x_id, set(group))
-    m, k, lda = _matrix(x, "linear input")
-    if k != int(w0.shape[1]):
-        raise FusionError("linear: inner dimensions differ")
     weights = [g.nodes[sid].inputs[1] for sid in group]
     widths = [int(g.nodes[w].output.shape[0]) for w in weights]
     if any(n % 8 for n in widths):
         return False  # column windows must stay 16-byte aligned for the consumers' vector loads
+    x, pro, extra, fold_w = _a_operand(c, x_id, set(group), fold=True)
+    m, k, lda = _matrix(x, "linear input")
+    if k != int(w0.shape[1]):
+        raise FusionError("linear: inner dimensions differ")
     n_total = sum(widths)
-    stacked = "__".join(weights)
+    stacked = "__".join(weights) + (f"__k*{fold_w}" if fold_w else "")
     if stacked not in c.out.nodes:
         c.out.add_constant(stacked, (n_total, k), w0.dtype)
-        c.out.nodes[stacked].hints["stacked"] = StackedConstant(tuple(weights))
+        c.out.nodes[stacked].hints["stacked"] = StackedConstant(tuple(weights), k_scale=fold_w)
     fid = "__".join(group)
     od = node.output.dtype
     body = Contraction(m=m, n=n_total, k=k, a=x.base, b=stacked, out=fid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset, a_prologue=pro)
@@ -328,13 +336,13 @@ def _rec_gate_up(c: _Ctx, nid: str) -> bool:
         wg, wu = c.g.nodes[gate.inputs[1]], c.g.nodes[up.inputs[1]]
         if not (isinstance(wg.op, ConstantOp) and isinstance(wu.op, ConstantOp)) or wg.output.shape != wu.output.shape:
             continue
-        x, pro, extra = _a_operand(c, gate.inputs[0], {gate.id, up.id})
+        x, pro, extra, fold_w = _a_operand(c, gate.inputs[0], {gate.id, up.id}, fold=True)
         m, k, lda = _matrix(x, "gate/up input")
         n = int(wg.output.shape[0])
-        stacked = f"{wg.id}__{wu.id}"
+        stacked = f"{wg.id}__{wu.id}" + (f"__k*{fold_w}" if fold_w else "")
         if stacked not in c.out.nodes:
             c.out.add_constant(stacked, (2 * n, k), wg.output.dtype)
-            c.out.nodes[stacked].hints["stacked"] = StackedConstant((wg.id, wu.id))
+            c.out.nodes[stacked].hints["stacked"] = StackedConstant((wg.id, wu.id), k_scale=fold_w)
         od = node.output.dtype
         epi = _round(od, E.Un("silu", _round(od, E.Var("acc")))) * _round(od, E.Var("acc2"))
         body = Contraction(m=m, n=n, k=k, a=x.base, b=stacked, out=nid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset, epilogue=epi, gate_pair=True, a_prologue=pro)

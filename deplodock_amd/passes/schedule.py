@@ -225,7 +225,9 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
       17.2 -> 15.9 -> 16.1; 4096^3 136 -> 122; the block as one graph 66.9 -> 65.2 -> 62.8)."""
     steps = body.k // plan.bk_elems
     if body.a_prologue is not None:
-        return Stage(depth=2, transport="sync")  # ``mix`` (b direct to LDS) measures the same on the block's two such kernels
+        # a goes through registers (transformed, or summed for the deferred scale); b may go direct to LDS
+        b_chunks = plan.tile_n * (2 if body.gate_pair else 1) * (plan.bk_elems // 8)
+        return Stage(depth=2, transport="mix" if body.a_prologue.scale is not None and b_chunks % 64 == 0 else "sync")
     if body.m <= 128:
         return Stage(depth=2, transport="sync", reg_depth=2 if steps >= 3 else 1)
     if (plan.bk_elems // plan.atom.k) % 2 == 0:

@@ -382,6 +382,51 @@ def test_row_norm_as_contraction_prologue(device, kind, m, k, n):
         prog.close()
 
 
+class _NormGateUp(nn.Module):
+    def __init__(self, k, n, norm):
+        super().__init__()
+        self.norm, self.gate, self.up = norm, nn.Linear(k, n, bias=False), nn.Linear(k, n, bias=False)
+
+    def forward(self, x):
+        h = self.norm(x)
+        return nn.functional.silu(self.gate(h)) * self.up(h)
+
+
+@pytest.mark.parametrize("kind,m,k,n", [("hf", 512, 1024, 768), ("torch", 100, 512, 256), ("hf", 64, 2048, 384)])
+def test_row_norm_deferred_into_a_stacked_projection(device, kind, m, k, n):
+    """``norm -> gate/up``: the norm weight (not all ones) is folded into the stacked weights when they are
+    bound, the rows are staged untouched and the accumulators take the row's ``rsqrt(mean x^2 + eps)``."""
+    torch.manual_seed(5)
+    norm = _HfRmsNorm(k) if kind == "hf" else nn.RMSNorm(k, eps=1e-6)
+    with torch.no_grad():
+        norm.weight.copy_(1.0 + 0.3 * torch.randn(k))
+    mod = _NormGateUp(k, n, norm).bfloat16().eval()
+    x = (2.0 * torch.randn(m, k)).bfloat16()
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, (x,)))
+    ops = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+    assert len(ops) == 1 and "a=row-scaled-after" in ops[0].comment and len(ops[0].arg_order) == 3
+    bound = be.bind(compiled, {})
+    (wname,) = [a for a in ops[0].arg_order if "__k*" in a]
+    want_w = (torch.cat([mod.gate.weight, mod.up.weight]).float() * mod.norm.weight.float()[None, :]).to(torch.bfloat16)
+    assert torch.equal(torch.as_tensor(bound[wname]).cpu(), want_w)
+    prog = be.program(compiled, {compiled.inputs[0]: x.to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]]
+        with torch.no_grad():
+            want = mod.to(device)(x.to(device))
+            exact = mod.float()(x.to(device).float())  # the same module without any 16-bit rounding inside
+        eager.assert_close(ours.reshape(want.shape), want, 2e-2, 2e-2, f"{kind} norm -> gate/up {m}x{k}x{n}")
+        # never rounding the normalised rows must not be *worse* than eager against the exact result
+        ours_err = (ours.reshape(exact.shape).float() - exact).abs().max().item()
+        eager_err = (want.float() - exact).abs().max().item()
+        assert ours_err <= 1.5 * eager_err + 1e-3, (ours_err, eager_err)
+    finally:
+        prog.close()
+
+
 def test_row_norm_with_a_second_reader_stays_a_kernel(device):
     torch.manual_seed(4)
     mod = _NormLinear(512, 256, _HfRmsNorm(512), share=True).bfloat16().eval()

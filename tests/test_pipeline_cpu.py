@@ -82,12 +82,13 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
         "k_rms_norm_linear_rope",
         "k_sdpa_reduce", "k_linear_add", "k_rms_norm_linear_silu_mul", "k_linear_add",
     ]  # fmt: skip
-    # the two layer norms are prologues of the contractions that read them: the row
-    # statistic is folded over the workgroup's rows before the k loop and the
-    # projection (with the norm's own rounding points) is applied while staging
+    # the two layer norms ride in the contractions that read them, deferred: the norm weight is
+    # folded into the stacked projection weights at bind time, the rows are staged as they are
+    # while their sum of squares is accumulated, and the accumulators take the row's scale factor
     first = kernels(compiled)[0]
-    assert "a=row-normalised" in first.comment and first.arg_order[0] == compiled.inputs[0]
-    assert "__shfl_xor(ss[i], msk, 64)" in first.kernel_source and "emh_round_bf16" in first.kernel_source
+    assert "a=row-scaled-after" in first.comment and first.arg_order[0] == compiled.inputs[0] and first.knobs["STAGE"] == "d2/mix"
+    assert "__shfl_xor(ss[i], msk, 64)" in first.kernel_source and "* rs_)" in first.kernel_source
+    assert "p_l_input_layernorm_weight" not in first.arg_order and first.arg_order[1].endswith("__k*p_l_input_layernorm_weight")
     # q, k and v projections are one contraction over the stacked weights; each
     # projection is a column window of its [tokens, 2048 + 1024 + 1024] result
     qkv = kernels(compiled)[0]
