@@ -224,7 +224,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     if deferred and (pro.weight is not None or E.variables(pro.scale) - {"ss"}):
         raise LoweringError("contraction: a deferred row scale is an expression over the row statistic; the column weight belongs in the b operand")
     if pro is not None:
-        if dl:
+        if dl and not deferred:
             raise LoweringError("contraction: a row prologue transforms the operand in registers; it needs STAGE .../sync")
         if body.in_dtype.nbytes != 2 or (pro.weight is not None and pro.weight_dtype.nbytes != 2):
             raise LoweringError("contraction: the row prologue is written for 16-bit operands")
@@ -472,6 +472,19 @@ ROW_EPILOGUE_TABLES
     asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
   #pragma unroll
   for (int p = 0; p < DEPTH; ++p) if (p < KT) EMH_DLOAD(p, p);""")
+        if deferred:
+            # the rows arrive in LDS untouched: every thread reads back the chunks it requested
+            # (any chunk of the row will do for a row sum) while the slab is resident
+            a("  float ss[A_PER_T];")
+            a("  #pragma unroll")
+            a("  for (int i = 0; i < A_PER_T; ++i) ss[i] = 0.0f;")
+            a(f"  {frag_t} sx[A_PER_T];")
+            a("  #define EMH_SUMSQ_READ(buf) { \\")
+            a(f'    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) sx[i] = *(const {frag_t}*)(emh_lds + (buf) * SLAB + la[i]); }}')
+            a("  #define EMH_SUMSQ_ADD() { \\")
+            a('    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) \\')
+            a('    _Pragma("unroll") for (int e = 0; e < 8; ++e) { const float x_ = (float)sx[i][e]; ss[i] += ' + E.render(pro.stat_pre, {"x": "x_"}) + "; } \\")
+            a("    __builtin_amdgcn_sched_barrier(0); }")
         first_younger = min(depth - 1, KT - 1) * loads_per_slab
         a(f"  EMH_SLAB_SYNC({first_younger});")
         a("  EMH_READ(0, 0, 0);")
@@ -483,6 +496,8 @@ ROW_EPILOGUE_TABLES
             steady state, where every condition holds and the body is branch-free
             (so the wait-count pass can see that only the newest reads are pending)."""
             a(f"    {{ const int cur = ({kt}) % DEPTH;")
+            if deferred:
+                a("    EMH_SUMSQ_READ(cur);  // queued with the fragment reads; summed behind the first MFMAs")
             for kk in range(KS):
                 P = kk & 1
                 if kk + 1 < KS:
@@ -498,6 +513,8 @@ ROW_EPILOGUE_TABLES
                         a(f"    EMH_DLOAD({static_kt + depth}, cur);")
                     a(f"    EMH_READ({P ^ 1}, {(static_kt + 1) % depth}, 0);")
                 a(f"    EMH_MMA({P});")
+                if deferred and kk == 0:
+                    a("    EMH_SUMSQ_ADD();")
             a("    }")
 
         steady = max(0, KT - depth)
@@ -530,6 +547,8 @@ ROW_EPILOGUE_TABLES
         lds_bytes = max(lds_bytes, rs_off + TM * 4)
         a("  // Row statistic: finish it over the lanes that hold a row's chunks, turn it into the row's")
         a("  // scale factor and hand it to the lanes that own the row's accumulators.")
+        if dl:
+            a("  __syncthreads();  // the last slab's fragments have been read by every wave")
         a("  #pragma unroll")
         a("  for (int i = 0; i < A_PER_T; ++i) {")
         a("    #pragma unroll")

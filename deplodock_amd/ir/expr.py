@@ -108,6 +108,14 @@ _UN_C = {
     "sigmoid": "(1.0f / (1.0f + expf(-({a}))))",
     "silu": "(({a}) / (1.0f + expf(-({a}))))",
 }
+# A transcendental whose result is rounded to a 16-bit type straight away takes the
+# hardware approximations (v_exp_f32 / v_rcp_f32, a couple of fp32 ulps): nothing of the
+# difference survives the rounding, and the precise forms cost ~25 instructions per element.
+_UN_C_ROUNDED = {
+    "exp": "__expf({a})",
+    "sigmoid": "__fdividef(1.0f, 1.0f + __expf(-({a})))",
+    "silu": "__fdividef(({a}), 1.0f + __expf(-({a})))",
+}
 _BIN_C = {
     "add": "(({a}) + ({b}))",
     "sub": "(({a}) - ({b}))",
@@ -130,6 +138,8 @@ def render(e: Expr, env: dict[str, str]) -> str:
     if isinstance(e, Bin):
         return _BIN_C[e.op].format(a=render(e.a, env), b=render(e.b, env))
     if isinstance(e, Round):
+        if isinstance(e.a, Un) and e.a.op in _UN_C_ROUNDED:
+            return _ROUND_C[e.dtype].format(a=_UN_C_ROUNDED[e.a.op].format(a=render(e.a.a, env)))
         return _ROUND_C[e.dtype].format(a=render(e.a, env))
     raise TypeError(f"cannot render {type(e).__name__}")
 

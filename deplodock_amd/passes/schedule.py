@@ -224,10 +224,8 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
       9.4; 512x1024x2048 7.4 -> 6.2 -> 6.2; 512x4096x1024 7.8 -> 6.8 -> 6.7; 2048x3072x1024
       17.2 -> 15.9 -> 16.1; 4096^3 136 -> 122; the block as one graph 66.9 -> 65.2 -> 62.8)."""
     steps = body.k // plan.bk_elems
-    if body.a_prologue is not None:
-        # a goes through registers (transformed, or summed for the deferred scale); b may go direct to LDS
-        b_chunks = plan.tile_n * (2 if body.gate_pair else 1) * (plan.bk_elems // 8)
-        return Stage(depth=2, transport="mix" if body.a_prologue.scale is not None and b_chunks % 64 == 0 else "sync")
+    if body.a_prologue is not None and body.a_prologue.scale is None:
+        return Stage(depth=2, transport="sync")  # transformed in registers on its way to LDS
     if body.m <= 128:
         return Stage(depth=2, transport="sync", reg_depth=2 if steps >= 3 else 1)
     if (plan.bk_elems // plan.atom.k) % 2 == 0:
@@ -280,7 +278,7 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
         except ScheduleError as exc:
             logger.warning("EMMY_STAGE=%r ignored: %s", pinned_stage, exc)
             stage = None
-    if stage is not None and body.a_prologue is not None and stage.transport == "dl":
+    if stage is not None and body.a_prologue is not None and body.a_prologue.scale is None and stage.transport == "dl":
         logger.warning("STAGE=%s ignored: the row-normalised operand is transformed in registers (sync or mix staging only)", stage.spell())
         stage = None
     if stage is None:

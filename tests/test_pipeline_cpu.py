@@ -86,7 +86,7 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
     # folded into the stacked projection weights at bind time, the rows are staged as they are
     # while their sum of squares is accumulated, and the accumulators take the row's scale factor
     first = kernels(compiled)[0]
-    assert "a=row-scaled-after" in first.comment and first.arg_order[0] == compiled.inputs[0] and first.knobs["STAGE"] == "d2/mix"
+    assert "a=row-scaled-after" in first.comment and first.arg_order[0] == compiled.inputs[0] and first.knobs["STAGE"] == "d2/sync/p2"  # 64 tokens: decode-size staging
     assert "__shfl_xor(ss[i], msk, 64)" in first.kernel_source and "* rs_)" in first.kernel_source
     assert "p_l_input_layernorm_weight" not in first.arg_order and first.arg_order[1].endswith("__k*p_l_input_layernorm_weight")
     # q, k and v projections are one contraction over the stacked weights; each
@@ -127,6 +127,15 @@ def test_head_norm_and_rope_fold_into_the_projection(launcher_lib, monkeypatch):
     # a pinned tile that splits a head degrades to the heuristic pick for this kernel
     monkeypatch.setenv("EMMY_TILE", "a:mfma_16x16x32_bf16/w1x2/f1x1/k4")
     assert "#define TN 64" in kernels(compile_case(eager.normed_rope_attention_case()))[0].kernel_source
+
+
+def test_deferred_norm_takes_the_direct_to_lds_ring_at_prefill_sizes(launcher_lib):
+    ks = kernels(compile_case(eager.qwen3_block_case(seq=512)))
+    qkv, gate_up = ks[0], ks[3]
+    assert qkv.knobs["STAGE"] == "d3/dl" and gate_up.knobs["STAGE"] == "d2/dl"  # three 48 KiB slabs fit, three 80 KiB ones do not
+    for k in (qkv, gate_up):
+        assert "a=row-scaled-after" in k.comment and "#define EMH_SUMSQ_READ(buf)" in k.kernel_source and "EMH_SUMSQ_ADD();" in k.kernel_source
+        hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
 
 
 def test_reduce_pin_is_authoritative_and_bad_pin_degrades(launcher_lib, monkeypatch):
