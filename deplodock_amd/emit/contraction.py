@@ -673,7 +673,7 @@ ROW_EPILOGUE_TABLES
     tables: list[str] = []
     if rowepi is not None:
         _emit_row_epilogue_tables(tables.append, rowepi, re_args, EPC, m_guard)
-    source = prelude.header(vm_macro, *((prelude.WAVE_REDUCE,) if rowepi is not None else ())) + "\n".join(o).replace("ROW_EPILOGUE_TABLES", "\n".join(tables)) + "\n"
+    source = prelude.header(prelude.DMA, vm_macro, *((prelude.WAVE_REDUCE,) if rowepi is not None else ())) + "\n".join(o).replace("ROW_EPILOGUE_TABLES", "\n".join(tables)) + "\n"
     if N % 4 or TN % 4:
         raise LoweringError("contraction: N must be a multiple of 4 (8-byte output runs)")
     n_blocks = (tiles_m // gm) * (tiles_n // gn)

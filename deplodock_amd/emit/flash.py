@@ -495,7 +495,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     head += "".join(f"#define {k} {v}\n" for k, v in defs.items())
     grid = qslots * body.q_heads * body.batch
     head += f"#define GRID {grid}\n#define XCDS {ctx.xcds}\n"
-    source = prelude.header() + head + _SRC
+    source = prelude.header(prelude.DMA) + head + _SRC
     return HipOp(
         kernel_source=source,
         kernel_name=name,

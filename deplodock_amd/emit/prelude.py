@@ -24,6 +24,10 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
 #define EMH_DEV __device__ __forceinline__
 EMH_DEV float emh_round_bf16(float v) { return (float)(__bf16)v; }
+"""
+
+# Direct-to-LDS loads and their publication; only the emitters that stage through LDS include it.
+DMA = r"""
 // Direct-to-LDS load of 16 bytes per lane: lane l's bytes land at lds_base + 16*l
 // (lds_base: the wave-uniform LDS byte address, carried in M0).  Issued as inline
 // assembly on purpose: for the builtin the compiler assumes any later LDS read may
