@@ -176,3 +176,19 @@ def test_qwen3_block_restatement_matches_eager_fp32(golden):
 def test_rotate_half():
     x = np.arange(8.0)[None]
     np.testing.assert_array_equal(O.rotate_half(x), np.array([[-4.0, -5, -6, -7, 0, 1, 2, 3]]))
+
+
+def test_deferred_rms_norm_identity():
+    """What the fused block relies on when it defers a layer norm into the projections that read it:
+    ``rms_norm(x, w) @ W^T == r * (x @ (W * w)^T)`` with ``r = rsqrt(mean x^2 + eps)`` per row, checked in
+    float64 against the restated norm and linear (a wrong axis for ``w``, a missing ``eps`` or a ``mean``
+    taken as a sum breaks it)."""
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((5, 96)) * 3.0
+    w = 1.0 + 0.3 * rng.standard_normal(96)
+    big_w = 0.05 * rng.standard_normal((40, 96))
+    eps = 1e-6
+    direct = O.linear(O.rms_norm(x, w, eps), big_w)
+    r = 1.0 / np.sqrt((x * x).mean(-1, keepdims=True) + eps)
+    deferred = r * O.linear(x, big_w * w[None, :])
+    np.testing.assert_allclose(deferred, direct, rtol=1e-5, atol=1e-6)
