@@ -144,20 +144,38 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
     CUs, else the one that launches the most workgroups."""
     best = None
     candidates = TILE_CANDIDATES
-    if gate_pair and not row_prologue:
-        # a gate/up pair stages two weight rows per output column, so the balanced
-        # slab is twice as tall as wide: 128x64 moves 20 % fewer bytes through the L1
-        # than 64x128 for the same workgroup count (10.96 vs 12.04 us on 512x1024x(2x3072)).
-        # Not with a row-normalised operand: its statistic pass re-reads the tile's rows,
-        # and twice the rows cost more than the slabs save (17.2 vs 15.9 us).
-        i = next(k for k, c in enumerate(TILE_CANDIDATES) if c[:2] == (64, 128))
-        candidates = (*TILE_CANDIDATES[:i], (128, 64, 4, 2, "mfma_16x16x32_bf16", 4), *TILE_CANDIDATES[i:])
-    for tm, tn, wm, wn, atom_name, bk in candidates:
+    exact_fit = None
+    if m >= 256:
+        # Prefill-sized rows: eight waves of one fragment each on the 32x64 tile (more
+        # loads in flight per CU than four waves of two): 6.20 vs 6.39 us on
+        # 512x1024x2048, 7.94 vs 9.16 us on 512x1024x3072, inside the decoder block.
+        candidates = tuple((32, 64, 2, 4, "mfma_16x16x32_bf16", 8) if c[:4] == (32, 64, 1, 4) else c for c in candidates)
+    if gate_pair:
+        i = next(k for k, c in enumerate(candidates) if c[:2] == (64, 128))
+        extra = []
+        # 64x96 is taken only where it makes (a multiple of) one workgroup per CU:
+        # 256 workgroups on 512x(2x3072)x1024 against 192 of 64x128, 10.4 vs 12.8 us.
+        exact_fit = (64, 96, 4, 2, "mfma_16x16x32_bf16", 2)
+        extra.append(exact_fit)
+        if not row_prologue:
+            # a gate/up pair stages two weight rows per output column, so the balanced
+            # slab is twice as tall as wide: 128x64 moves 20 % fewer bytes through the L1
+            # than 64x128 for the same workgroup count (10.96 vs 12.04 us on 512x1024x(2x3072)).
+            # Not with a row-normalised operand: its statistic pass re-reads the tile's rows,
+            # and twice the rows cost more than the slabs save (17.2 vs 15.9 us).
+            extra.append((128, 64, 4, 2, "mfma_16x16x32_bf16", 4))
+        candidates = (*candidates[:i], *extra, *candidates[i:])
+    for cand in candidates:
+        tm, tn, wm, wn, atom_name, bk = cand
         atom = ATOMS[atom_name]
         if tm % (wm * atom.m) or tn % (wn * atom.n):
             continue
         if group_cols is not None and (tn % group_cols[0] or group_cols[1] % tn or (tm * tn // 8) % (wm * wn * 64)):
             continue  # a row epilogue works on whole column groups of a staged output tile
+        if cand is exact_fit:
+            g = -(-m // tm) * -(-n // tn)
+            if m % tm or n % tn or g < ctx.compute_units or g / float(-(-g // ctx.compute_units) * ctx.compute_units) < 0.9:
+                continue
         fm, fn = tm // (wm * atom.m), tn // (wn * atom.n)
         if fm * fn * atom.acc_per_lane * (2 if gate_pair else 1) > 256:
             continue

@@ -132,7 +132,8 @@ def test_head_norm_and_rope_fold_into_the_projection(launcher_lib, monkeypatch):
 def test_deferred_norm_takes_the_direct_to_lds_ring_at_prefill_sizes(launcher_lib):
     ks = kernels(compile_case(eager.qwen3_block_case(seq=512)))
     qkv, gate_up = ks[0], ks[3]
-    assert qkv.knobs["STAGE"] == "d3/dl" and gate_up.knobs["STAGE"] == "d2/dl"  # three 48 KiB slabs fit, three 80 KiB ones do not
+    assert qkv.knobs["STAGE"] == "d3/dl" and gate_up.knobs["STAGE"] == "d3/dl"
+    assert gate_up.knobs["TILE"].endswith("/w4x2/f1x3/k2") and gate_up.grid[0][0] == 256  # 64x96 tiles: one workgroup per CU
     for k in (qkv, gate_up):
         assert "a=row-scaled-after" in k.comment and "#define EMH_SUMSQ_READ(buf)" in k.kernel_source and "EMH_SUMSQ_ADD();" in k.kernel_source
         hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
