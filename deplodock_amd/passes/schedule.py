@@ -145,8 +145,8 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
     best = None
     candidates = TILE_CANDIDATES
     exact_fit = None
-    if m >= 256:
-        # Prefill-sized rows: eight waves of one fragment each on the 32x64 tile (more
+    if m >= 128:
+        # From 128 rows on: eight waves of one fragment each on the 32x64 tile (more
         # loads in flight per CU than four waves of two): 6.20 vs 6.39 us on
         # 512x1024x2048, 7.94 vs 9.16 us on 512x1024x3072, inside the decoder block.
         candidates = tuple((32, 64, 2, 4, "mfma_16x16x32_bf16", 8) if c[:4] == (32, 64, 1, 4) else c for c in candidates)
@@ -233,10 +233,12 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
 
     * A row-normalised operand is transformed in registers on its way to LDS: ``sync``
       (``mix`` sends the other operand direct to LDS; 12.7 / 15.8 us against 12.3 / 15.9 us).
-    * Decode-size problems (M <= 128) stream the weight once, straight from HBM: ``sync``
+    * Decode-size problems (M < 128) stream the weight once, straight from HBM: ``sync``
       through two register sets (measured with operands rotating through more memory
       than the caches hold: 4.4 / 4.5 / 6.2 us at M = 1 / 16 / 128 on 1024x3072, against
       5.2 / 5.4 / 6.9 through one set and 4.6 / 4.6 / 6.4 with a three-slab ``dl`` ring).
+      At M = 128 the ring on the eight-wave 32x64 tile ties that when the weight comes from
+      HBM (6.25 vs 6.27 us) and wins when it sits in the caches (4.02 vs 4.64 us).
     * Everything else: direct-to-LDS loads; a ring of three slabs where the LDS holds them
       and a slab is less than ~600 cycles of MFMA work, else two (us, ``d2/sync`` -> ``d2/dl`` -> ``d3/dl``: 512x1024x3072 12.2 -> 9.5 ->
       9.4; 512x1024x2048 7.4 -> 6.2 -> 6.2; 512x4096x1024 7.8 -> 6.8 -> 6.7; 2048x3072x1024
@@ -244,7 +246,7 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
     steps = body.k // plan.bk_elems
     if body.a_prologue is not None and body.a_prologue.scale is None:
         return Stage(depth=2, transport="sync")  # transformed in registers on its way to LDS
-    if body.m <= 128:
+    if body.m < 128:
         return Stage(depth=2, transport="sync", reg_depth=2 if steps >= 3 else 1)
     if (plan.bk_elems // plan.atom.k) % 2 == 0:
         # a slab that keeps the matrix pipe busy for long hides the next one's latency by itself

@@ -58,9 +58,10 @@ def test_linear_is_one_mfma_kernel(launcher_lib, m):
     assert "__builtin_amdgcn_mfma_f32_" in k.kernel_source
     assert k.algo_flops == 2 * m * 3072 * 1024
     # decode sizes stream the weight from HBM: two slabs in flight through two register sets
-    # larger ones take direct-to-LDS loads (two slabs: a 128x192x64 slab is 768 cycles of MFMA work)
-    assert k.knobs["STAGE"] == ("d2/sync/p2" if m <= 128 else "d2/dl")
-    assert ("ra[RS][A_PER_T]" in k.kernel_source) == (m <= 128) and ("#define EMH_DLOAD" in k.kernel_source) == (m > 128)
+    # from 128 rows on direct-to-LDS loads (three 48 KiB slabs of the 32x64x256 tile; two where a slab is
+    # long enough by itself: a 128x192x64 slab is 768 cycles of MFMA work)
+    assert k.knobs["STAGE"] == {1: "d2/sync/p2", 16: "d2/sync/p2", 128: "d3/dl", 2048: "d2/dl"}[m]
+    assert ("ra[RS][A_PER_T]" in k.kernel_source) == (m < 128) and ("#define EMH_DLOAD" in k.kernel_source) == (m >= 128)
     hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
 
 
