@@ -327,7 +327,11 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
     8.7, ``w1/kv32/s4`` 8.8, ``w2/kv64/s2`` 11.0; S=1024 ``w2/kv32/s4`` 13.5,
     ``w1/kv32/s4/p`` 17.8; S=2048 ``w2/kv32/s4/p`` 27.8, ``w2/kv32/s4`` 28.5,
     ``w4/kv64/s2`` 32.7; S=2048 unmasked ``w4/kv64/s2`` 36.5, ``w4/kv32/s2`` 41.3;
-    32 q heads S=4096 ``w4/kv64/s2/p`` 157, ``w2/kv32/s4/p`` 186."""
+    32 q heads S=4096 ``w4/kv64/s2/p`` 157, ``w2/kv32/s4/p`` 186.
+    Where 256-row workgroups still cover the CUs they win (``w8/kv64/s1``: S=8192 unmasked
+    560 against 637 for ``w4/kv64/s2``, causal 303 against 351; S=16384 causal 1087 / 1239;
+    batch 4 S=2048 causal ``w8/kv64/s1/p`` 104 / 117; 16 heads S=4096 causal, 256 such
+    workgroups unpaired: 122 against 94, hence the 2x cover asked of an unpaired triangle)."""
     pinned = _pin("FLASH", _tuned(body, ctx))
     if pinned:
         try:
@@ -363,14 +367,27 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
             return -(-body.q_len // (32 * w))
 
         body.pair = False
-        if body.causal and body.q_len == body.kv_len and body.kv_len >= 2048:
+        body.waves = 0
+        if body.head_dim <= 128 and body.kv_len >= 2048:
+            # Enough rows to give every CU a 256-row workgroup: eight query waves share each
+            # K/V block (the blocks come out of the L2s at ~32 B/clk per CU whoever asks, so rows
+            # per block is what counts) and no key split is needed to put two waves on a SIMD.
+            cus = ctx.compute_units
+            if body.causal and body.q_len == body.kv_len:
+                if body.kv_len <= 4096 and blocks(8) % 2 == 0 and heads * blocks(8) // 2 >= cus:
+                    body.waves, body.pair = 8, True
+                elif heads * blocks(8) >= 2 * cus:
+                    body.waves = 8  # twice the CUs: the heaviest-first order balances the triangle
+            elif heads * blocks(8) >= cus:
+                body.waves = 8
+        if not body.waves and body.causal and body.q_len == body.kv_len and body.kv_len >= 2048:
             for w in (4, 2):
                 if blocks(w) % 2 == 0 and heads * blocks(w) // 2 >= fill:
                     body.waves, body.pair = w, True
                     break
-        if not body.pair:
+        if not body.waves:
             body.waves = next((w for w in (4, 2) if heads * blocks(w) >= fill), 1)
-        body.block_kv, body.kv_split = (64, 2) if body.waves == 4 else (32, 4)
+        body.block_kv, body.kv_split = {8: (64, 1), 4: (64, 2)}.get(body.waves, (32, 4))
         while body.kv_split > 1 and -(-body.kv_len // body.block_kv) < body.kv_split:
             body.kv_split //= 2  # fewer key blocks than key-split groups
         # wider heads: shrink the key block, then the key split, until the double-buffered K/V blocks fit the LDS

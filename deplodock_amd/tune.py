@@ -52,7 +52,7 @@ REDUCE_SWEEP: tuple[str, ...] = ("b8", "b16", "b32", "b64", "b128", "b256", "b51
 NT_SWEEP: tuple[str, ...] = ("0", "1")
 FLASH_SWEEP: tuple[str, ...] = (
     "w4/kv64/s2", "w2/kv64/s2", "w1/kv64/s2", "w2/kv32/s4", "w1/kv32/s4", "w4/kv32/s2", "w4/kv64/s1",
-    "w2/kv32/s4/p", "w2/kv64/s2/p", "w1/kv32/s4/p", "w4/kv64/s2/p",
+    "w2/kv32/s4/p", "w2/kv64/s2/p", "w1/kv32/s4/p", "w4/kv64/s2/p", "w8/kv64/s1", "w8/kv64/s1/p",
 )  # fmt: skip
 
 

@@ -214,7 +214,7 @@ def test_c4_head_dim_64_workgroup_shapes(device, pin, monkeypatch):
     eager.assert_close(ours, want, 2e-2, 2e-2, f"sdpa d=64 {pin} vs eager")
 
 
-@pytest.mark.parametrize("pin", ["w4/kv64/s1", "w4/kv64/s2", "w2/kv64/s2", "w4/kv32/s2", "w1/kv32/s4", "w2/kv32/s4"])
+@pytest.mark.parametrize("pin", ["w4/kv64/s1", "w4/kv64/s2", "w2/kv64/s2", "w4/kv32/s2", "w1/kv32/s4", "w2/kv32/s4", "w8/kv64/s1"])
 def test_c4_every_workgroup_shape(device, pin, monkeypatch):
     """Key-split groups, direct-to-LDS staging and the final (m, l, O) merge: the first
     key blocks are consumed right after they are staged, so every launch is checked."""
@@ -236,7 +236,7 @@ def test_c4_every_workgroup_shape(device, pin, monkeypatch):
         prog.close()
 
 
-@pytest.mark.parametrize("pin", ["w2/kv32/s4/p", "w1/kv64/s2/p", "w4/kv64/s2/p", "w2/kv64/s1/p"])
+@pytest.mark.parametrize("pin", ["w2/kv32/s4/p", "w1/kv64/s2/p", "w4/kv64/s2/p", "w2/kv64/s1/p", "w8/kv64/s1/p"])
 def test_c4_mirrored_query_block_pairs(device, pin, monkeypatch):
     """A workgroup that takes query block b and then block n-1-b reuses its LDS and
     registers for the second block: both halves of every pair are checked, on repeated launches."""
