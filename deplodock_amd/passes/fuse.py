@@ -806,7 +806,8 @@ def _rec_sdpa(c: _Ctx, nid: str) -> bool:
     # If the only consumer transposes to [B, S, H, D] (and flattens), write that layout directly.
     out_id, o_shape, o_strides = nid, (B, Hq, Sq, D), (Hq * Sq * D, Sq * D, D)
     cons = c.g.consumers(nid)
-    if len(cons) == 1 and nid not in c.g.outputs and _is(c.g.nodes[cons[0]], F.TransposeOp, dim0=1, dim1=2):
+    transposed = len(cons) == 1 and nid not in c.g.outputs and _is(c.g.nodes[cons[0]], F.TransposeOp, dim0=1, dim1=2)
+    if transposed:
         o_shape, o_strides = (B, Sq, Hq, D), (Sq * Hq * D, D, Hq * D)
     scale = node.op.scale if node.op.scale is not None else 1.0 / math.sqrt(D)
     body = Flash(
@@ -815,7 +816,7 @@ def _rec_sdpa(c: _Ctx, nid: str) -> bool:
         q_offset=q.offset, k_offset=k.offset, v_offset=v.offset,
     )  # fmt: skip
     _emit(c, nid, body, "sdpa_reduce", [q.base, k.base, v.base], shape=o_shape)
-    if o_shape != (B, Hq, Sq, D):
+    if transposed:  # (not a comparison of the shapes: they read the same when there are as many tokens as heads)
         c.out.nodes[nid].hints["logical_view"] = ((B, Hq, Sq, D), (o_strides[0], o_strides[1], o_strides[2], 1))
     return True
 

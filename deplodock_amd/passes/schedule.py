@@ -42,7 +42,15 @@ TILE_CANDIDATES: tuple[tuple[int, int, int, int, str, int], ...] = (
     (128, 96, 4, 1, "mfma_32x32x16_bf16", 4),
     (64, 128, 2, 4, "mfma_16x16x32_bf16", 4),
     (64, 64, 2, 2, "mfma_16x16x32_bf16", 4),
+    # Few-row problems (the decoder block at 64-256 tokens), ranked inside the block's graph: the tile that
+    # makes about one multi-wave workgroup per CU wins over more, smaller ones (256 rows: o / down
+    # projections 7.98 / 13.85 us on 1024 one-wave 16x16 tiles, 4.76 / 6.02 us on 256 four-wave 32x32 tiles;
+    # q/k/v projection 9.29 us on 64x128, 6.91 us on 32x128; 128 rows: 16x32 tiles 4.16 / 5.11 against 4.49 / 7.45 us).
+    (32, 128, 2, 4, "mfma_16x16x32_bf16", 4),
     (32, 64, 1, 4, "mfma_16x16x32_bf16", 8),
+    (32, 32, 2, 2, "mfma_16x16x32_bf16", 8),
+    (16, 128, 1, 4, "mfma_16x16x32_bf16", 8),
+    (16, 32, 1, 2, "mfma_16x16x32_bf16", 8),
     (16, 16, 1, 1, "mfma_16x16x32_bf16", 8),
 )
 
@@ -144,7 +152,7 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
     CUs, else the one that launches the most workgroups."""
     best = None
     candidates = TILE_CANDIDATES
-    exact_fit = None
+    exact_fit = ()
     if m >= 128:
         # From 128 rows on: eight waves of one fragment each on the 32x64 tile (more
         # loads in flight per CU than four waves of two): 6.20 vs 6.39 us on
@@ -155,8 +163,8 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
         extra = []
         # 64x96 is taken only where it makes (a multiple of) one workgroup per CU:
         # 256 workgroups on 512x(2x3072)x1024 against 192 of 64x128, 10.4 vs 12.8 us.
-        exact_fit = (64, 96, 4, 2, "mfma_16x16x32_bf16", 2)
-        extra.append(exact_fit)
+        exact_fit = ((64, 96, 4, 2, "mfma_16x16x32_bf16", 2), (32, 96, 2, 2, "mfma_16x16x32_bf16", 4))  # 256 rows: 32x96, 8.85 against 9.93 us on 64x64
+        extra.extend(exact_fit)
         if not row_prologue:
             # a gate/up pair stages two weight rows per output column, so the balanced
             # slab is twice as tall as wide: 128x64 moves 20 % fewer bytes through the L1
@@ -172,7 +180,7 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
             continue
         if group_cols is not None and (tn % group_cols[0] or group_cols[1] % tn or (tm * tn // 8) % (wm * wn * 64)):
             continue  # a row epilogue works on whole column groups of a staged output tile
-        if cand is exact_fit:
+        if cand in exact_fit:
             g = -(-m // tm) * -(-n // tn)
             if m % tm or n % tn or g < ctx.compute_units or g / float(-(-g // ctx.compute_units) * ctx.compute_units) < 0.9:
                 continue
@@ -192,7 +200,10 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
         groups = -(-m // tm) * -(-n // tn)
         # penalise tiles that mostly hang over the edge of a small problem
         waste = (-(-m // tm) * tm * -(-n // tn) * tn) / float(max(m * n, 1))
-        if groups >= _FILL_FRACTION * ctx.compute_units and waste < 1.5:
+        # two waves on a 16x32 tile beat one wave on each of twice as many 16x16 tiles down to half the CUs
+        # (64 rows x 1024 columns: 4.11 / 5.01 us on 128 workgroups against 4.84 / 6.43 us on 256)
+        fill = 0.5 if (tm, tn) == (16, 32) else _FILL_FRACTION
+        if groups >= fill * ctx.compute_units and waste < 1.5:
             return plan
         score = (min(groups, ctx.compute_units) / max(waste, 1e-9), tm * tn)
         if best is None or score > best[0]:
@@ -233,12 +244,13 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
 
     * A row-normalised operand is transformed in registers on its way to LDS: ``sync``
       (``mix`` sends the other operand direct to LDS; 12.7 / 15.8 us against 12.3 / 15.9 us).
-    * Decode-size problems (M < 128) stream the weight once, straight from HBM: ``sync``
+    * Decode-size problems (M <= 16) stream the weight once, straight from HBM: ``sync``
       through two register sets (measured with operands rotating through more memory
       than the caches hold: 4.4 / 4.5 / 6.2 us at M = 1 / 16 / 128 on 1024x3072, against
       5.2 / 5.4 / 6.9 through one set and 4.6 / 4.6 / 6.4 with a three-slab ``dl`` ring).
       At M = 128 the ring on the eight-wave 32x64 tile ties that when the weight comes from
-      HBM (6.25 vs 6.27 us) and wins when it sits in the caches (4.02 vs 4.64 us).
+      HBM (6.25 vs 6.27 us) and wins when it sits in the caches (4.02 vs 4.64 us); inside the
+      decoder block at 64 tokens the ring wins on every projection (o: 4.11 vs 5.00 us).
     * Everything else: direct-to-LDS loads; a ring of three slabs where the LDS holds them
       and a slab is less than ~600 cycles of MFMA work, else two (us, ``d2/sync`` -> ``d2/dl`` -> ``d3/dl``: 512x1024x3072 12.2 -> 9.5 ->
       9.4; 512x1024x2048 7.4 -> 6.2 -> 6.2; 512x4096x1024 7.8 -> 6.8 -> 6.7; 2048x3072x1024
@@ -246,7 +258,7 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
     steps = body.k // plan.bk_elems
     if body.a_prologue is not None and body.a_prologue.scale is None:
         return Stage(depth=2, transport="sync")  # transformed in registers on its way to LDS
-    if body.m < 128:
+    if body.m <= 16:
         return Stage(depth=2, transport="sync", reg_depth=2 if steps >= 3 else 1)
     if (plan.bk_elems // plan.atom.k) % 2 == 0:
         # a slab that keeps the matrix pipe busy for long hides the next one's latency by itself

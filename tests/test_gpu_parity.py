@@ -279,7 +279,7 @@ def test_head_norm_and_rope_in_the_projection_epilogue(device, dims):
     eager.assert_close(ours, want, case.rtol, case.atol, f"{case.name} vs eager (GPU)")
 
 
-@pytest.mark.parametrize("seq", [32, 64, 512])
+@pytest.mark.parametrize("seq", [8, 16, 32, 64, 128, 256, 512])  # 16 tokens = as many as query heads, 8 = as many as KV heads
 def test_c5_qwen3_block(device, seq, golden):
     case = eager.qwen3_block_case(seq=seq)
     ours, want, compiled = run_case(case, device)

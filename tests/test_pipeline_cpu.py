@@ -87,7 +87,10 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
     # folded into the stacked projection weights at bind time, the rows are staged as they are
     # while their sum of squares is accumulated, and the accumulators take the row's scale factor
     first = kernels(compiled)[0]
-    assert "a=row-scaled-after" in first.comment and first.arg_order[0] == compiled.inputs[0] and first.knobs["STAGE"] == "d2/sync/p2"  # 64 tokens: decode-size staging
+    assert "a=row-scaled-after" in first.comment and first.arg_order[0] == compiled.inputs[0] and first.knobs["STAGE"] == "d2/dl"
+    decode = kernels(compile_case(eager.qwen3_block_case(seq=16)))[0]  # 16 tokens (as many as heads): decode-size staging through registers
+    assert "a=row-scaled-after" in decode.comment and decode.knobs["STAGE"] == "d2/sync/p2" and "#define EMH_SUMSQ_READ" not in decode.kernel_source
+    hiprtc.compile_to_hsaco(decode.kernel_source, decode.kernel_name)
     assert "__shfl_xor(ss[i], msk, 64)" in first.kernel_source and "* rs_)" in first.kernel_source
     assert "p_l_input_layernorm_weight" not in first.arg_order and first.arg_order[1].endswith("__k*p_l_input_layernorm_weight")
     # q, k and v projections are one contraction over the stacked weights; each
