@@ -37,11 +37,13 @@ logger = logging.getLogger(__name__)
 # slabs (256 elements) and 4-8 waves per workgroup won every such shape.
 TILE_CANDIDATES: tuple[tuple[int, int, int, int, str, int], ...] = (
     (256, 256, 2, 4, "mfma_16x16x32_bf16", 2),  # 4096^3 with a two-slab dl ring: 111.8 us = 1 230 TFLOP/s (32x32x16 atoms, same tile: 119.5 us)
-    (128, 192, 4, 2, "mfma_16x16x32_bf16", 2),
-    (128, 128, 2, 2, "mfma_32x32x16_bf16", 4),
-    (128, 96, 4, 1, "mfma_32x32x16_bf16", 4),
+    (128, 256, 2, 4, "mfma_16x16x32_bf16", 2),
+    (128, 192, 2, 4, "mfma_16x16x32_bf16", 2),  # 2048x3072x1024: 16.9 us as 2x4 waves of 64x48, 17.2 as 4x2 of 32x96 (less LDS read traffic)
+    # eight waves on 16x16x32 atoms, 64-deep slabs: 1024 tokens q/k/v 16.3 us, gate/up 21.2 (four waves on 32x32x16 atoms: 18.2, 23.2)
+    (128, 128, 4, 2, "mfma_16x16x32_bf16", 2),
+    (128, 96, 4, 2, "mfma_16x16x32_bf16", 4),
     (64, 128, 2, 4, "mfma_16x16x32_bf16", 4),
-    (64, 64, 2, 2, "mfma_16x16x32_bf16", 4),
+    (64, 64, 2, 4, "mfma_16x16x32_bf16", 4),  # eight waves of 32x16: 1024x1024x2048 7.7 us (four of 32x32: 8.9)
     # Few-row problems (the decoder block at 64-256 tokens), ranked inside the block's graph: the tile that
     # makes about one multi-wave workgroup per CU wins over more, smaller ones (256 rows: o / down
     # projections 7.98 / 13.85 us on 1024 one-wave 16x16 tiles, 4.76 / 6.02 us on 256 four-wave 32x32 tiles;
@@ -148,31 +150,37 @@ def schedule_row_reduce(body: RowReduce, ctx: Context) -> dict:
 
 
 def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologue: bool = False, group_cols: tuple[int, int] | None = None) -> TilePlan:
-    """First candidate (in measured-throughput order) whose launch covers the
-    CUs, else the one that launches the most workgroups."""
+    """The largest candidate that makes one workgroup per CU (0.9-1.0 of the CUs, no ragged
+    edge), else the first (in measured-throughput order) whose launch covers 75 % of the CUs,
+    else the one that launches the most workgroups.
+
+    One round of workgroups, each as large as that allows, is what the decoder block's
+    projections prefer at every token count (in-graph times, us): 2048 tokens q/k/v 34.6 on
+    256 tiles of 128x128 with four waves, 28.2 on 256 tiles of 128x256; 1024 tokens gate/up
+    22.6 on 192 tiles of 128x128, 18.2 on 256 tiles of 128x96; 512 tokens gate/up 12.8 on 192
+    tiles of 64x128, 10.4 on 256 of 64x96; 256 tokens gate/up 9.93 on 64x64, 8.85 on 32x96."""
     best = None
     candidates = TILE_CANDIDATES
-    exact_fit = ()
+    one_round_only = {(128, 256)}  # offered only as an exact fit: as a 75 % cover it was not measured
     if m >= 128:
         # From 128 rows on: eight waves of one fragment each on the 32x64 tile (more
         # loads in flight per CU than four waves of two): 6.20 vs 6.39 us on
         # 512x1024x2048, 7.94 vs 9.16 us on 512x1024x3072, inside the decoder block.
         candidates = tuple((32, 64, 2, 4, "mfma_16x16x32_bf16", 8) if c[:4] == (32, 64, 1, 4) else c for c in candidates)
     if gate_pair:
-        i = next(k for k, c in enumerate(candidates) if c[:2] == (64, 128))
-        extra = []
-        # 64x96 is taken only where it makes (a multiple of) one workgroup per CU:
-        # 256 workgroups on 512x(2x3072)x1024 against 192 of 64x128, 10.4 vs 12.8 us.
-        exact_fit = ((64, 96, 4, 2, "mfma_16x16x32_bf16", 2), (32, 96, 2, 2, "mfma_16x16x32_bf16", 4))  # 256 rows: 32x96, 8.85 against 9.93 us on 64x64
-        extra.extend(exact_fit)
+        # two weight rows per output column: 96-column tiles make 32 column blocks of 2 x 3072 outputs
+        extra = ((128, 96, 4, 2, "mfma_16x16x32_bf16", 2), (64, 96, 4, 2, "mfma_16x16x32_bf16", 2), (32, 96, 2, 2, "mfma_16x16x32_bf16", 4))
+        one_round_only |= {c[:2] for c in extra}
         if not row_prologue:
             # a gate/up pair stages two weight rows per output column, so the balanced
             # slab is twice as tall as wide: 128x64 moves 20 % fewer bytes through the L1
             # than 64x128 for the same workgroup count (10.96 vs 12.04 us on 512x1024x(2x3072)).
             # Not with a row-normalised operand: its statistic pass re-reads the tile's rows,
             # and twice the rows cost more than the slabs save (17.2 vs 15.9 us).
-            extra.append((128, 64, 4, 2, "mfma_16x16x32_bf16", 4))
+            extra = (*extra, (128, 64, 4, 2, "mfma_16x16x32_bf16", 4))
+        i = next(k for k, c in enumerate(candidates) if c[:2] == (128, 96))
         candidates = (*candidates[:i], *extra, *candidates[i:])
+    plans = []
     for cand in candidates:
         tm, tn, wm, wn, atom_name, bk = cand
         atom = ATOMS[atom_name]
@@ -180,13 +188,9 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
             continue
         if group_cols is not None and (tn % group_cols[0] or group_cols[1] % tn or (tm * tn // 8) % (wm * wn * 64)):
             continue  # a row epilogue works on whole column groups of a staged output tile
-        if cand in exact_fit:
-            g = -(-m // tm) * -(-n // tn)
-            if m % tm or n % tn or g < ctx.compute_units or g / float(-(-g // ctx.compute_units) * ctx.compute_units) < 0.9:
-                continue
         fm, fn = tm // (wm * atom.m), tn // (wn * atom.n)
-        if fm * fn * atom.acc_per_lane * (2 if gate_pair else 1) > 256:
-            continue
+        if fm * fn * atom.acc_per_lane * (2 if gate_pair else 1) > 160:
+            continue  # two waves per SIMD leave 256 registers a lane: accumulators, fragments and addresses
         nb = 2 if gate_pair else 1
         while bk > 1 and (k % (bk * atom.k) or 2 * (tm + tn * nb) * bk * atom.k * 2 > ctx.lds_bytes_per_cu):
             bk //= 2
@@ -196,16 +200,24 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
         cpr = bk * atom.k // 8
         if (tm * cpr) % threads or (tn * cpr * (2 if gate_pair else 1)) % threads:
             continue
-        plan = TilePlan(atom=atom, units=(wm, wn), regs=(fm, fn), bk=bk)
+        plans.append((cand, TilePlan(atom=atom, units=(wm, wn), regs=(fm, fn), bk=bk)))
+    cus = ctx.compute_units
+    for (tm, tn, wm, wn, *_), plan in plans:
+        groups = -(-m // tm) * -(-n // tn)
+        if wm * wn > 1 and m % tm == 0 and n % tn == 0 and 0.9 * cus <= groups <= cus:
+            return plan  # (the one-wave tile is the last resort: two waves on half as many 16x32 tiles beat it)
+    for (tm, tn, *_), plan in plans:
+        if (tm, tn) in one_round_only:
+            continue
         groups = -(-m // tm) * -(-n // tn)
         # penalise tiles that mostly hang over the edge of a small problem
         waste = (-(-m // tm) * tm * -(-n // tn) * tn) / float(max(m * n, 1))
         # two waves on a 16x32 tile beat one wave on each of twice as many 16x16 tiles down to half the CUs
         # (64 rows x 1024 columns: 4.11 / 5.01 us on 128 workgroups against 4.84 / 6.43 us on 256)
         fill = 0.5 if (tm, tn) == (16, 32) else _FILL_FRACTION
-        if groups >= fill * ctx.compute_units and waste < 1.5:
+        if groups >= fill * cus and waste < 1.5:
             return plan
-        score = (min(groups, ctx.compute_units) / max(waste, 1e-9), tm * tn)
+        score = (min(groups, cus) / max(waste, 1e-9), tm * tn)
         if best is None or score > best[0]:
             best = (score, plan)
     if best is None:
