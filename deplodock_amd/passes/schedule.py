@@ -410,7 +410,8 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                     body.waves, body.pair = w, True
                     break
         if not body.waves:
-            body.waves = next((w for w in (4, 2) if heads * blocks(w) >= fill), 1)
+            # (two row groups pay down to half the CUs: 512 tokens x 16 heads, 128 workgroups of `w2` 8.81 us, 256 of `w1` 9.10)
+            body.waves = next((w for w in (4, 2) if heads * blocks(w) >= (fill if w == 4 else 0.5 * ctx.compute_units)), 1)
         body.block_kv, body.kv_split = {8: (64, 1), 4: (64, 2)}.get(body.waves, (32, 4))
         while body.kv_split > 1 and -(-body.kv_len // body.block_kv) < body.kv_split:
             body.kv_split //= 2  # fewer key blocks than key-split groups
