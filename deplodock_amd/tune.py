@@ -30,24 +30,28 @@ from deplodock_amd import config
 from deplodock_amd.ir.tile import Contraction, Flash, RowReduce
 
 TILE_SWEEP: tuple[str, ...] = (
-    "a:mfma_32x32x16_bf16/w2x4/f4x2/k4",
+    "a:mfma_16x16x32_bf16/w2x4/f8x4/k2",
+    "a:mfma_16x16x32_bf16/w2x4/f4x4/k2",
+    "a:mfma_16x16x32_bf16/w2x4/f4x3/k2",
     "a:mfma_16x16x32_bf16/w4x2/f2x6/k2",
-    "a:mfma_32x32x16_bf16/w2x2/f2x3/k4",
+    "a:mfma_16x16x32_bf16/w4x2/f2x4/k2",
     "a:mfma_32x32x16_bf16/w2x2/f2x2/k4",
-    "a:mfma_32x32x16_bf16/w4x1/f1x3/k4",
-    "a:mfma_32x32x16_bf16/w2x2/f1x2/k4",
+    "a:mfma_16x16x32_bf16/w4x2/f2x3/k2",
+    "a:mfma_16x16x32_bf16/w2x4/f2x4/k2",
     "a:mfma_16x16x32_bf16/w2x4/f2x2/k4",
+    "a:mfma_16x16x32_bf16/w4x2/f1x3/k2",
+    "a:mfma_16x16x32_bf16/w2x4/f2x1/k4",
     "a:mfma_16x16x32_bf16/w2x2/f2x2/k4",
-    "a:mfma_16x16x32_bf16/w2x2/f2x2/k8",
-    "a:mfma_16x16x32_bf16/w1x4/f2x1/k8",
-    "a:mfma_16x16x32_bf16/w2x2/f2x1/k8",
+    "a:mfma_16x16x32_bf16/w2x4/f1x2/k4",
+    "a:mfma_16x16x32_bf16/w2x2/f1x3/k4",
     "a:mfma_16x16x32_bf16/w2x4/f1x1/k8",
-    "a:mfma_16x16x32_bf16/w1x2/f2x2/k4",
+    "a:mfma_16x16x32_bf16/w1x4/f2x1/k8",
+    "a:mfma_16x16x32_bf16/w2x2/f1x1/k8",
+    "a:mfma_16x16x32_bf16/w1x4/f1x2/k8",
     "a:mfma_16x16x32_bf16/w1x2/f1x1/k8",
     "a:mfma_16x16x32_bf16/w1x1/f1x1/k8",
-    "a:mfma_16x16x32_bf16/w1x4/f1x1/k8",
-)
-STAGE_SWEEP: tuple[str, ...] = ("d2/sync", "d2/sync/p2", "d3/dl")
+)  # every tile that won an in-graph ranking of the decoder block's contractions at 64 ... 2048 tokens, and their neighbours
+STAGE_SWEEP: tuple[str, ...] = ("d2/dl", "d3/dl", "d2/sync/p2")
 REDUCE_SWEEP: tuple[str, ...] = ("b8", "b16", "b32", "b64", "b128", "b256", "b512", "b1024")
 NT_SWEEP: tuple[str, ...] = ("0", "1")
 FLASH_SWEEP: tuple[str, ...] = (
