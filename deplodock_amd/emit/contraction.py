@@ -168,8 +168,9 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     TM, TN = plan.tile_m, plan.tile_n
     BK = plan.bk_elems
     T = plan.block_threads
-    if K % BK:
-        raise LoweringError(f"contraction: K={K} is not a multiple of the slab depth {BK}")
+    k_guard = K % BK != 0  # the last slab is short: its missing chunks are staged as zeros (both operands)
+    if k_guard and (K % 8 or body.a_prologue is not None or stage.transport != "sync"):
+        raise LoweringError(f"contraction: K={K} is not a multiple of the slab depth {BK} (a short last slab needs whole 16-byte chunks, register staging and no row prologue)")
     if BK % 8 or BK > 256:
         raise LoweringError(f"contraction: slab depth {BK} must be a multiple of 8 and at most 256")
     if lda % 8 or ldb % 8 or ldo % 4 or body.a_offset % 8 or body.b_offset % 8 or body.out_offset % 8:
@@ -197,7 +198,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     tiles_m, tiles_n = -(-M // TM), -(-N // TN)
     n_tiles = tiles_m * tiles_n
     gm, gn = xcd_block(tiles_m, tiles_n, TM, TN, ctx.xcds)
-    KT = K // BK
+    KT = -(-K // BK)
     m_guard = M % TM != 0
     n_guard = N % TN != 0
     dl = stage.transport == "dl"
@@ -291,7 +292,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   const int lr = lane % AM, lk = lane / AM;  // fragment row, k-group
 """)
     # ---- staging ------------------------------------------------------------
-    a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else ""))
+    a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else "") + (" int ka[A_PER_T], kb[B_PER_T];" if k_guard else ""))
     a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
     a(r"""  #pragma unroll
   for (int i = 0; i < A_PER_T; ++i) {
@@ -306,6 +307,8 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     a(f"    ga[i] = A + {body.a_offset}L + (long)gr * LDA + c * 8;")
     if pro is not None:
         a("    ca[i] = c * 8;")
+    if k_guard:
+        a("    ka[i] = c * 8;")
     a("  }")
     a(r"""  #pragma unroll
   for (int i = 0; i < B_PER_T; ++i) {
@@ -323,6 +326,8 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     else:
         a(f"    int gr = n0 + row;{' if (gr > N - 1) gr = N - 1;' if n_guard else ''}")
     a(f"    gb[i] = B + {body.b_offset}L + (long)gr * LDB + c * 8;")
+    if k_guard:
+        a("    kb[i] = c * 8;")
     a("  }")
 
     a(f"  {D['acc_t']} acc[NB][FM][FN];")
@@ -371,6 +376,8 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
             b_lstore = "__builtin_amdgcn_s_waitcnt(EMH_WAIT_VM_LGKM0(0)); emh_lds_publish(emh_lds + tid * 4);"
         else:
             b_gload = '_Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) rb[S][i] = *(const u32x4*)(gb[i] + (kt) * BK);'
+            if k_guard:
+                b_gload = '_Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) { rb[S][i] = u32x4{0u, 0u, 0u, 0u}; if ((kt) * BK + kb[i] < K) rb[S][i] = *(const u32x4*)(gb[i] + (kt) * BK); }'
             b_lstore = '_Pragma("unroll") for (int i = 0; i < B_PER_T; ++i) *(u32x4*)(s_ + lb[i]) = rb[S][i];'
         if pro is not None:
             # Row statistic over the full k extent of this thread's rows: the chunks of
@@ -416,12 +423,15 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         else:
             a(r"""  u32x4 ra[RS][A_PER_T], rb[RS][B_PER_T];
   #define EMH_GLOAD(kt, S) { \
-    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) ra[S][i] = *(const u32x4*)(ga[i] + (kt) * BK); \
+    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) A_GLOAD \
     B_GLOAD }
   #define EMH_LSTORE(buf, S) { \
     unsigned char* s_ = emh_lds + (buf) * SLAB; \
     _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) *(u32x4*)(s_ + la[i]) = ra[S][i]; \
-    B_LSTORE }""".replace("B_GLOAD", b_gload).replace("B_LSTORE", b_lstore))
+    B_LSTORE }""".replace("B_GLOAD", b_gload).replace("B_LSTORE", b_lstore).replace(
+                "A_GLOAD",
+                "{ ra[S][i] = u32x4{0u, 0u, 0u, 0u}; if ((kt) * BK + ka[i] < K) ra[S][i] = *(const u32x4*)(ga[i] + (kt) * BK); }" if k_guard else "ra[S][i] = *(const u32x4*)(ga[i] + (kt) * BK);",
+            ))
         # Slab j travels through register set j % RS: RS slabs are in flight from
         # global memory while one is computed on, so a load has RS steps to arrive.
         a(r"""  #pragma unroll

@@ -178,7 +178,7 @@ def _a_operand(c: _Ctx, x_id: str, absorbers: set[str], fold: bool = False) -> t
             m = _RmsMatch(x=node.inputs[0], weight=node.inputs[1] if node.op.has_weight else None, eps=node.op.eps, inner=F32, cols=int(node.output.shape[-1]))
         elif len(node.output.shape) >= 2:
             m = _match_rms_chain(c, x_id)
-        if m is not None and node.output.dtype.nbytes == 2:
+        if m is not None and node.output.dtype.nbytes == 2 and m.cols % 32 == 0:  # (whole MFMA steps: a short last slab is not transformed)
             try:
                 body, inputs, xv = _rms_body(c, x_id, m, node.output.dtype)
             except FusionError:

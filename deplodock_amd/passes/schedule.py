@@ -192,10 +192,13 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
         if fm * fn * atom.acc_per_lane * (2 if gate_pair else 1) > 160:
             continue  # two waves per SIMD leave 256 registers a lane: accumulators, fragments and addresses
         nb = 2 if gate_pair else 1
-        while bk > 1 and (k % (bk * atom.k) or 2 * (tm + tn * nb) * bk * atom.k * 2 > ctx.lds_bytes_per_cu):
-            bk //= 2
-        if k % (bk * atom.k):
-            continue
+        if k % atom.k and k % 8 == 0 and not row_prologue:
+            bk = 2 if k > 2 * atom.k else 1  # a short last slab (zero-filled on the register-staged path)
+        else:
+            while bk > 1 and (k % (bk * atom.k) or 2 * (tm + tn * nb) * bk * atom.k * 2 > ctx.lds_bytes_per_cu):
+                bk //= 2
+            if k % (bk * atom.k):
+                continue
         threads = wm * wn * 64
         cpr = bk * atom.k // 8
         if (tm * cpr) % threads or (tn * cpr * (2 if gate_pair else 1)) % threads:
@@ -267,7 +270,9 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
       and a slab is less than ~600 cycles of MFMA work, else two (us, ``d2/sync`` -> ``d2/dl`` -> ``d3/dl``: 512x1024x3072 12.2 -> 9.5 ->
       9.4; 512x1024x2048 7.4 -> 6.2 -> 6.2; 512x4096x1024 7.8 -> 6.8 -> 6.7; 2048x3072x1024
       17.2 -> 15.9 -> 16.1; 4096^3 136 -> 122; the block as one graph 66.9 -> 65.2 -> 62.8)."""
-    steps = body.k // plan.bk_elems
+    steps = -(-body.k // plan.bk_elems)
+    if body.k % plan.bk_elems:
+        return Stage(depth=2, transport="sync")  # the short last slab is zero-filled in registers
     if body.a_prologue is not None and body.a_prologue.scale is None:
         return Stage(depth=2, transport="sync")  # transformed in registers on its way to LDS
     if body.m <= 16:
@@ -423,6 +428,15 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 body.kv_split //= 2
             else:
                 break
+        # narrower heads: a key block's 16-byte chunks are dealt over all threads of the workgroup, so it must
+        # hold at least one chunk per thread: grow the block while the LDS allows, else give up key-split groups
+        while (body.block_kv * body.head_dim // 8) % (body.waves * body.kv_split * 64):
+            body.block_kv *= 2
+            if _flash_lds(body, ctx) > ctx.lds_bytes_per_cu:
+                body.block_kv //= 2
+                if body.kv_split == 1:
+                    break
+                body.kv_split //= 2
     return {"FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "")}
 
 

@@ -129,10 +129,12 @@ def test_c3_linear(device, m):
     eager.assert_close(ours[: min(m, 8)], exact, 2 ** -7, 1e-3, f"linear M={m} vs float64")
 
 
-@pytest.mark.parametrize("m,k,n", [(17, 512, 200), (40, 1024, 1000), (70, 256, 136), (130, 2048, 1024), (260, 512, 96), (300, 1024, 4096), (1024, 1024, 3072), (2048, 512, 4096)])
+@pytest.mark.parametrize("m,k,n", [(17, 512, 200), (40, 1024, 1000), (70, 256, 136), (130, 2048, 1024), (260, 512, 96), (300, 1024, 4096), (1024, 1024, 3072), (2048, 512, 4096),
+                                   (30, 72, 192), (64, 200, 712), (4, 200, 4096), (300, 1000, 512), (128, 40, 64)])  # the last five: K is not a multiple of the MFMA depth
 def test_linear_heuristic_tiles_on_ragged_and_one_round_shapes(device, m, k, n):
     """What the tile picker chooses by itself — small multi-wave tiles with direct-to-LDS rings below 512 rows,
-    the largest tile that makes one workgroup per CU above — with rows and columns that do not fill the tiles."""
+    the largest tile that makes one workgroup per CU above — with rows and columns that do not fill the tiles,
+    and with a reduction extent whose last slab is short (zero-filled on its way through registers)."""
     case = eager.linear_case(m=m, k=k, n=n, seed=m)
     ours, want, compiled = run_case(case, device)
     eager.assert_close(ours, want, case.rtol, case.atol, f"linear {m}x{k}x{n} vs eager (GPU)")

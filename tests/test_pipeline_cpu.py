@@ -265,3 +265,13 @@ def test_row_sum_and_mean_are_row_reductions(launcher_lib):
     assert "one value per row" in ks[0].comment and ks[0].algo_bytes == 16 * 256 * 4 + 16 * 4
     with pytest.raises(NotImplementedError, match="non-innermost"):
         HipBackend().compile(trace_module(type("S", (nn.Module,), {"forward": lambda self, x: x.sum(0)})(), (torch.randn(4, 8),)))
+
+
+def test_short_last_slab_takes_the_register_staged_path(launcher_lib):
+    """K = 200 is 6 MFMA steps and 8 elements: the slabs are 64 deep, the fourth one is mostly zeros."""
+    k = kernels(compile_case(eager.linear_case(m=64, k=200, n=712)))[0]
+    assert k.knobs["STAGE"] == "d2/sync" and k.knobs["TILE"].endswith("/k2")
+    assert "if ((kt) * BK + ka[i] < K)" in k.kernel_source and "if ((kt) * BK + kb[i] < K)" in k.kernel_source
+    hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+    with pytest.raises(Exception):  # rows that are not whole 16-byte chunks stay unsupported
+        compile_case(eager.linear_case(m=64, k=100, n=712))
