@@ -60,6 +60,31 @@ def cache_key(source: str, name: str, arch: str) -> str:
     return h.hexdigest()
 
 
+# A kernel that defines this macro waits for part of its outstanding direct-to-LDS loads by count
+# (the contraction's slab ring): it must compile without vector-register spills, because spill
+# stores share the counter and complete out of order with loads.
+NO_SPILL_CONTRACT = "#define EMH_SLAB_SYNC(n)"
+
+
+def vgpr_spill_counts(code_object: bytes) -> list[int]:
+    """``.vgpr_spill_count`` of every kernel in a code object, read from the msgpack metadata note
+    (key string followed by a msgpack unsigned integer)."""
+    key = b".vgpr_spill_count"
+    out, pos = [], code_object.find(key)
+    while pos >= 0:
+        v = code_object[pos + len(key) : pos + len(key) + 5]
+        if v[:1] and v[0] <= 0x7F:
+            out.append(v[0])
+        elif v[:1] == b"\xcc":
+            out.append(v[1])
+        elif v[:1] == b"\xcd":
+            out.append(int.from_bytes(v[1:3], "big"))
+        elif v[:1] == b"\xce":
+            out.append(int.from_bytes(v[1:5], "big"))
+        pos = code_object.find(key, pos + 1)
+    return out
+
+
 def compile_to_hsaco(source: str, name: str, *, arch: str = "gfx950") -> Path:
     """Compile ``source`` into the cache and return the code-object path.
 
@@ -70,6 +95,16 @@ def compile_to_hsaco(source: str, name: str, *, arch: str = "gfx950") -> Path:
     if out.exists() and out.stat().st_size > 0:
         return out
     blob, _log = launcher.load().compile(source, name, arch, effective_flags())
+    if NO_SPILL_CONTRACT in source:
+        spilled = max(vgpr_spill_counts(blob), default=0)
+        if spilled:
+            raise launcher.CompileError(
+                f"{name}: the compiler spilled {spilled} vector registers, and this kernel waits for part of its outstanding "
+                "direct-to-LDS loads by count (spill stores complete out of order with loads and would satisfy the wait early): "
+                "pick a smaller tile or register staging",
+                0,
+                _log or "",
+            )
     fd, tmp = tempfile.mkstemp(dir=cache, suffix=".tmp")
     try:
         with os.fdopen(fd, "wb") as fh:

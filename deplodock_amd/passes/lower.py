@@ -10,6 +10,8 @@ Kernel names follow the reference's rule ``k_<label>_<hash[:6]>``
 from __future__ import annotations
 
 import hashlib
+import logging
+from dataclasses import replace
 
 from deplodock_amd.context import Context
 from deplodock_amd.emit.contraction import emit_contraction
@@ -24,18 +26,7 @@ from deplodock_amd.ir.tile import Contraction, Flash, Map, RowReduce, TileOp
 _PLACEHOLDER = "EMH_KERNEL_NAME_"
 
 
-def lower_tile(op: TileOp, ctx: Context) -> HipOp:
-    body = op.body
-    if isinstance(body, RowReduce):
-        hip = (emit_row_reduce_streaming if body.stream else emit_row_reduce)(body, _PLACEHOLDER, ctx)
-    elif isinstance(body, Contraction):
-        hip = emit_contraction(body, _PLACEHOLDER, ctx)
-    elif isinstance(body, Flash):
-        hip = emit_flash(body, _PLACEHOLDER, ctx)
-    elif isinstance(body, Map):
-        hip = emit_map(body, _PLACEHOLDER, ctx)
-    else:
-        raise TypeError(f"unknown tile body {type(body).__name__}")
+def _named(hip: HipOp, op: TileOp) -> HipOp:
     label = op.name.split("__")[0]
     digest = hashlib.sha1(hip.kernel_source.encode()).hexdigest()[:6]
     name = f"{label}_{digest}"
@@ -44,6 +35,48 @@ def lower_tile(op: TileOp, ctx: Context) -> HipOp:
     hip.source = op
     hip.knobs = {**op.knobs, **hip.knobs}
     return hip
+
+
+def _spills(hip: HipOp, ctx: Context) -> str | None:
+    """The compiler's complaint when ``hip`` is a direct-to-LDS ring kernel that only builds with
+    vector-register spills, else ``None``.  The code object lands in the cache the loader reads, so
+    the check costs no second compile."""
+    from deplodock_amd.backend.hip import hiprtc, launcher
+
+    if hiprtc.NO_SPILL_CONTRACT not in hip.kernel_source:
+        return None
+    try:
+        hiprtc.compile_to_hsaco(hip.kernel_source, hip.kernel_name, arch=ctx.arch)
+    except launcher.CompileError as exc:
+        if "spilled" in str(exc):
+            return str(exc)
+        raise
+    except launcher.LauncherError:
+        pass  # no launcher library here: the compile step at load time still refuses a spilling ring
+    return None
+
+
+def lower_tile(op: TileOp, ctx: Context) -> HipOp:
+    body = op.body
+    if isinstance(body, RowReduce):
+        hip = (emit_row_reduce_streaming if body.stream else emit_row_reduce)(body, _PLACEHOLDER, ctx)
+    elif isinstance(body, Contraction):
+        hip = _named(emit_contraction(body, _PLACEHOLDER, ctx), op)
+        complaint = _spills(hip, ctx)
+        if complaint is None:
+            return hip
+        # the schedule's register estimate cannot see every prologue / epilogue: render the kernel again
+        # with register staging, the same degrade path an unrealisable pin takes
+        logging.getLogger(__name__).warning("STAGE=%s degraded to register staging: %s", hip.knobs.get("STAGE"), complaint)
+        body.stage = replace(body.stage, transport="sync", depth=2)
+        hip = emit_contraction(body, _PLACEHOLDER, ctx)
+    elif isinstance(body, Flash):
+        hip = emit_flash(body, _PLACEHOLDER, ctx)
+    elif isinstance(body, Map):
+        hip = emit_map(body, _PLACEHOLDER, ctx)
+    else:
+        raise TypeError(f"unknown tile body {type(body).__name__}")
+    return _named(hip, op)
 
 
 def lower(graph: Graph, ctx: Context | None = None) -> Graph:

@@ -249,9 +249,17 @@ def _check_tile(plan: TilePlan, body: Contraction, ctx: Context, depth: int, dl:
         raise ScheduleError("accumulators exceed the register file")
     if threads > ctx.max_threads_per_block:
         raise ScheduleError(f"{threads} threads per workgroup is not launchable")
+    if dl and plan.regs[0] * plan.regs[1] * plan.atom.acc_per_lane * nb > (256 if threads <= 256 else 128 if threads <= 512 else 64):
+        # the ring waits for part of its outstanding loads by count; spill stores share that counter and
+        # complete out of order with loads, so a direct-to-LDS kernel must not spill
+        raise ScheduleError("accumulators take more than half the registers of a lane: direct-to-LDS staging must not spill")
+    if dl and (depth - 1) * ((a_chunks + b_chunks) // threads) > 63:
+        raise ScheduleError("too many direct-to-LDS loads in flight for the six-bit vector-memory counter")
     re = body.row_epilogue
     if re is not None and (plan.tile_n % re.cols or re.col_end % plan.tile_n or (plan.tile_m * plan.tile_n // 8) % threads):
         raise ScheduleError(f"the row epilogue needs output tiles of whole {re.cols}-column groups")
+    if re is not None and plan.tile_m * (plan.tile_n * body.out_dtype.nbytes + 16) > ctx.lds_bytes_per_cu:
+        raise ScheduleError("the row epilogue works on the output tile staged in LDS, which this tile does not fit")
 
 
 def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:

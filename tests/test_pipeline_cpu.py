@@ -275,3 +275,27 @@ def test_short_last_slab_takes_the_register_staged_path(launcher_lib):
     hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
     with pytest.raises(Exception):  # rows that are not whole 16-byte chunks stay unsupported
         compile_case(eager.linear_case(m=64, k=100, n=712))
+
+
+def test_direct_to_lds_ring_kernels_must_not_spill(launcher_lib, monkeypatch):
+    """The slab ring waits for part of its outstanding loads by count; spill stores share that counter and
+    complete out of order with loads.  A tile whose accumulators fill the registers degrades to register
+    staging at schedule time, and a ring kernel that spills anyway is refused by the compile step."""
+    from deplodock_amd.backend.hip import launcher as L
+    from deplodock_amd.dtype import BF16
+    from deplodock_amd.emit.contraction import emit_contraction
+    from deplodock_amd.ir.schedule import Stage, TilePlan
+    from deplodock_amd.ir.tile import Contraction
+
+    assert hiprtc.vgpr_spill_counts(b"xx.vgpr_spill_count\xcd\x01\xa1yy.vgpr_spill_count\x05") == [417, 5]
+    default = kernels(compile_case(eager.linear_case(m=2048)))[0]
+    assert default.knobs["STAGE"].endswith("/dl") and hiprtc.NO_SPILL_CONTRACT in default.kernel_source
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w1x1/f4x6/k2")
+    monkeypatch.setenv("EMMY_STAGE", "d2/dl")
+    k = kernels(compile_case(eager.linear_case(m=180, k=1024, n=1024)))[0]
+    assert k.knobs["TILE"].endswith("w1x1/f4x6/k2") and k.knobs["STAGE"] == "d2/sync"
+    body = Contraction(m=180, n=1024, k=1024, a="x", b="w", out="y", in_dtype=BF16, out_dtype=BF16,
+                       tile=TilePlan.parse("a:mfma_32x32x16_bf16/w1x1/f4x6/k2"), stage=Stage.parse("d2/dl"))  # fmt: skip
+    op = emit_contraction(body, "k_spilling_ring")
+    with pytest.raises(L.CompileError, match="spilled"):
+        hiprtc.compile_to_hsaco(op.kernel_source, op.kernel_name)
