@@ -12,6 +12,7 @@ from __future__ import annotations
 import functools
 import hashlib
 import os
+import re
 import shutil
 import tempfile
 from pathlib import Path
@@ -114,6 +115,19 @@ def compile_to_hsaco(source: str, name: str, *, arch: str = "gfx950") -> Path:
         Path(tmp).unlink(missing_ok=True)
         raise
     return out
+
+
+def spilled_vgprs(source: str, name: str, *, arch: str = "gfx950") -> int:
+    """Vector registers the compiler spills building ``source``.  The code object is cached as by
+    ``compile_to_hsaco`` (so the loader compiles nothing twice), except a spilling kernel under the
+    no-spill contract, which is never cached."""
+    try:
+        return max(vgpr_spill_counts(compile_to_hsaco(source, name, arch=arch).read_bytes()), default=0)
+    except launcher.CompileError as exc:
+        found = re.search(r"spilled (\d+) vector registers", str(exc))
+        if found is None:
+            raise
+        return int(found.group(1))
 
 
 class LoadedKernel:

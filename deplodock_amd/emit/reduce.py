@@ -184,6 +184,43 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
                 a(f"  ok[{i}] = true;")
             o.extend("  " + ln for ln in _load_vec("xr", idx, body.x_dtype, V, f"xv[{i}]", nontemporal))
 
+    if not body.scalar_out:
+        for ri, ro in enumerate(body.row_operands):
+            a(f"  const {ro.dtype.c_name}* rrow{ri} = r{ri} + {ro.offset}L + ((row / {ro.div}) % {ro.mod}) * {body.cols}L;")
+
+    def operand_loads(i: int, indent: str, tag: str = "") -> None:
+        idx = f"{i * L} + lane"
+        for ci, (_, dt) in enumerate(body.col_operands):
+            a(f"{indent}float cv{ci}{tag}[{V}];")
+            o.extend(indent + ln for ln in _load_vec(f"c{ci}", idx, dt, V, f"cv{ci}{tag}", False))
+        for ri, ro in enumerate(body.row_operands):
+            a(f"{indent}float rv{ri}{tag}[{V}];")
+            o.extend(indent + ln for ln in _load_vec(f"rrow{ri}", idx, ro.dtype, V, f"rv{ri}{tag}", False))
+
+    def operand_env(j: int, tag: str = "") -> dict[str, str]:
+        env = {n: f"cv{ci}{tag}[{j}]" for ci, (n, _) in enumerate(body.col_operands)}
+        env.update({ro.name: f"rv{ri}{tag}[{j}]" for ri, ro in enumerate(body.row_operands)})
+        return env
+
+    # The projection's other operands do not depend on the statistics: requested here, with the row, they
+    # arrive while the statistics are reduced instead of costing a second memory round trip after them.
+    n_operands = len(body.col_operands) + len(body.row_operands)
+    hoist = bool(body.stats) and not body.scalar_out and body.rotate is None and 0 < n_operands * NV * V <= 32
+    if hoist:
+        for i in range(NV):
+            if masked and (i + 1) * L > C:
+                for ci in range(len(body.col_operands)):
+                    a(f"  float cv{ci}_{i}[{V}] = {{}};")
+                for ri in range(len(body.row_operands)):
+                    a(f"  float rv{ri}_{i}[{V}] = {{}};")
+                a(f"  if (ok[{i}]) {{")
+                mark = len(o)
+                operand_loads(i, "    ", f"_{i}")
+                o[mark:] = [ln for ln in o[mark:] if not ln.strip().startswith("float ")]
+                a("  }")
+            else:
+                operand_loads(i, "  ", f"_{i}")
+
     if NW > 1 and body.stats:
         a(f"  __shared__ float emh_part[{len(body.stats)}][{R}][{NW}];")
         a(f"  const int wave_in_row = lane / {ctx.wave_size};")
@@ -239,22 +276,6 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
             knobs={"REDUCE": plan.spell(), "VEC": V, "NT": int(nontemporal)},
         )
     a(f"  {body.out_dtype.c_name}* orow = out + ({_row_offset(out_addr, 'row')});")
-    for ri, ro in enumerate(body.row_operands):
-        a(f"  const {ro.dtype.c_name}* rrow{ri} = r{ri} + {ro.offset}L + ((row / {ro.div}) % {ro.mod}) * {body.cols}L;")
-
-    def operand_loads(i: int, indent: str) -> None:
-        idx = f"{i * L} + lane"
-        for ci, (_, dt) in enumerate(body.col_operands):
-            a(f"{indent}float cv{ci}[{V}];")
-            o.extend(indent + ln for ln in _load_vec(f"c{ci}", idx, dt, V, f"cv{ci}", False))
-        for ri, ro in enumerate(body.row_operands):
-            a(f"{indent}float rv{ri}[{V}];")
-            o.extend(indent + ln for ln in _load_vec(f"rrow{ri}", idx, ro.dtype, V, f"rv{ri}", False))
-
-    def operand_env(j: int) -> dict[str, str]:
-        env = {n: f"cv{ci}[{j}]" for ci, (n, _) in enumerate(body.col_operands)}
-        env.update({ro.name: f"rv{ri}[{j}]" for ri, ro in enumerate(body.row_operands)})
-        return env
 
     if row_guard:
         a("  if (row_ok) {")
@@ -264,9 +285,10 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
             guard = f"if (ok[{i}]) " if masked and (i + 1) * L > C else ""
             a(f"  {guard}{{")
             a(f"    float y[{V}];")
-            operand_loads(i, "    ")
+            if not hoist:
+                operand_loads(i, "    ")
             for j in range(V):
-                env = dict(env_base, x=f"xv[{i}][{j}]", **operand_env(j))
+                env = dict(env_base, x=f"xv[{i}][{j}]", **operand_env(j, f"_{i}" if hoist else ""))
                 a(f"    y[{j}] = {E.render(body.project, env)};")
             o.extend("    " + ln for ln in _store_vec("orow", idx, body.out_dtype, V, "y", nontemporal))
             a("  }")

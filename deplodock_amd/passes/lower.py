@@ -24,6 +24,7 @@ from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.ir.tile import Contraction, Flash, Map, RowReduce, TileOp
 
 _PLACEHOLDER = "EMH_KERNEL_NAME_"
+logger = logging.getLogger(__name__)
 
 
 def _named(hip: HipOp, op: TileOp) -> HipOp:
@@ -37,39 +38,49 @@ def _named(hip: HipOp, op: TileOp) -> HipOp:
     return hip
 
 
-def _spills(hip: HipOp, ctx: Context) -> str | None:
-    """The compiler's complaint when ``hip`` is a direct-to-LDS ring kernel that only builds with
-    vector-register spills, else ``None``.  The code object lands in the cache the loader reads, so
-    the check costs no second compile."""
+def _spills(hip: HipOp, ctx: Context) -> int:
+    """Vector registers the compiler spilled building ``hip`` (0 without a launcher library: the compile
+    step at load time still refuses a spilling ring).  The code object lands in the cache the loader
+    reads, so the check costs no second compile."""
     from deplodock_amd.backend.hip import hiprtc, launcher
 
-    if hiprtc.NO_SPILL_CONTRACT not in hip.kernel_source:
-        return None
     try:
-        hiprtc.compile_to_hsaco(hip.kernel_source, hip.kernel_name, arch=ctx.arch)
-    except launcher.CompileError as exc:
-        if "spilled" in str(exc):
-            return str(exc)
+        return hiprtc.spilled_vgprs(hip.kernel_source, hip.kernel_name, arch=ctx.arch)
+    except launcher.CompileError:
         raise
     except launcher.LauncherError:
-        pass  # no launcher library here: the compile step at load time still refuses a spilling ring
-    return None
+        return 0
+
+
+def _lower_contraction(op: TileOp, ctx: Context) -> HipOp:
+    """Render a contraction whose kernel builds without vector-register spills.  A spilling MFMA kernel is
+    slow, and wrong where it waits for part of its outstanding loads by count (spill stores share that
+    counter).  The schedule's register estimate cannot see every prologue / epilogue, so the code object
+    decides: a spilling kernel is rendered again with register staging, then with the heuristic tile — the
+    same degrade path an unrealisable pin takes."""
+    from deplodock_amd.passes.schedule import default_contraction_schedule
+
+    body = op.body
+    hip = _named(emit_contraction(body, _PLACEHOLDER, ctx), op)
+    spilled = _spills(hip, ctx)
+    if spilled and (body.stage.transport != "sync" or body.stage.reg_depth > 1):
+        logger.warning("%s: STAGE=%s spills %d vector registers: plain register staging instead", hip.kernel_name, hip.knobs.get("STAGE"), spilled)
+        body.stage = replace(body.stage, transport="sync", depth=2, reg_depth=1)
+        hip = _named(emit_contraction(body, _PLACEHOLDER, ctx), op)
+        spilled = _spills(hip, ctx)
+    if spilled:
+        logger.warning("%s: TILE=%s spills %d vector registers: the heuristic tile instead", hip.kernel_name, hip.knobs.get("TILE"), spilled)
+        default_contraction_schedule(body, ctx)
+        hip = _named(emit_contraction(body, _PLACEHOLDER, ctx), op)
+    return hip
 
 
 def lower_tile(op: TileOp, ctx: Context) -> HipOp:
     body = op.body
+    if isinstance(body, Contraction):
+        return _lower_contraction(op, ctx)
     if isinstance(body, RowReduce):
         hip = (emit_row_reduce_streaming if body.stream else emit_row_reduce)(body, _PLACEHOLDER, ctx)
-    elif isinstance(body, Contraction):
-        hip = _named(emit_contraction(body, _PLACEHOLDER, ctx), op)
-        complaint = _spills(hip, ctx)
-        if complaint is None:
-            return hip
-        # the schedule's register estimate cannot see every prologue / epilogue: render the kernel again
-        # with register staging, the same degrade path an unrealisable pin takes
-        logging.getLogger(__name__).warning("STAGE=%s degraded to register staging: %s", hip.knobs.get("STAGE"), complaint)
-        body.stage = replace(body.stage, transport="sync", depth=2)
-        hip = emit_contraction(body, _PLACEHOLDER, ctx)
     elif isinstance(body, Flash):
         hip = emit_flash(body, _PLACEHOLDER, ctx)
     elif isinstance(body, Map):

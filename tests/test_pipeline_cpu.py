@@ -290,12 +290,26 @@ def test_direct_to_lds_ring_kernels_must_not_spill(launcher_lib, monkeypatch):
     assert hiprtc.vgpr_spill_counts(b"xx.vgpr_spill_count\xcd\x01\xa1yy.vgpr_spill_count\x05") == [417, 5]
     default = kernels(compile_case(eager.linear_case(m=2048)))[0]
     assert default.knobs["STAGE"].endswith("/dl") and hiprtc.NO_SPILL_CONTRACT in default.kernel_source
-    monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w1x1/f4x6/k2")
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w1x1/f3x4/k8")
     monkeypatch.setenv("EMMY_STAGE", "d2/dl")
-    k = kernels(compile_case(eager.linear_case(m=180, k=1024, n=1024)))[0]
-    assert k.knobs["TILE"].endswith("w1x1/f4x6/k2") and k.knobs["STAGE"] == "d2/sync"
-    body = Contraction(m=180, n=1024, k=1024, a="x", b="w", out="y", in_dtype=BF16, out_dtype=BF16,
-                       tile=TilePlan.parse("a:mfma_32x32x16_bf16/w1x1/f4x6/k2"), stage=Stage.parse("d2/dl"))  # fmt: skip
+    k = kernels(compile_case(eager.linear_case(m=2048, k=3072, n=3072)))[0]
+    assert hiprtc.spilled_vgprs(k.kernel_source, k.kernel_name) == 0
+    assert not (k.knobs["TILE"].endswith("w1x1/f3x4/k8") and k.knobs["STAGE"].endswith("/dl"))
+    body = Contraction(m=2048, n=3072, k=3072, a="x", b="w", out="y", in_dtype=BF16, out_dtype=BF16,
+                       tile=TilePlan.parse("a:mfma_32x32x16_bf16/w1x1/f3x4/k8"), stage=Stage.parse("d2/dl"))  # fmt: skip
     op = emit_contraction(body, "k_spilling_ring")
     with pytest.raises(L.CompileError, match="spilled"):
         hiprtc.compile_to_hsaco(op.kernel_source, op.kernel_name)
+
+
+def test_a_pinned_tile_that_only_builds_with_spills_degrades(launcher_lib, monkeypatch):
+    """The code object decides: register sets that overflow first give way to plain register staging, and a
+    tile that still spills to the heuristic one; the stamped knobs name what was built."""
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x1/f4x4/k4")
+    monkeypatch.setenv("EMMY_STAGE", "d2/sync/p3")
+    k = kernels(compile_case(eager.linear_case(m=256, k=1024, n=1024)))[0]
+    assert hiprtc.spilled_vgprs(k.kernel_source, k.kernel_name) == 0
+    assert k.knobs["STAGE"] != "d2/sync/p3"
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w1x1/f3x6/k2")  # 288 accumulators per lane
+    k = kernels(compile_case(eager.linear_case(m=256, k=1024, n=1024)))[0]
+    assert "f3x6" not in k.knobs["TILE"]
