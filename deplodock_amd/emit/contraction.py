@@ -153,6 +153,10 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     if body.in_dtype.name not in _FRAG_T or plan.atom.dtype != body.in_dtype.name:
         raise LoweringError(f"contraction: atom {plan.atom.name} does not take {body.in_dtype} operands")
     stage = body.stage or Stage(depth=2, transport="sync")
+    if stage.transport == "ks":
+        from deplodock_amd.emit.skinny import emit_contraction_skinny
+
+        return emit_contraction_skinny(body, name, ctx)
     if body.reduce.cta != 1:
         raise LoweringError("contraction: split-K is lowered by emit_contraction_splitk")
     M, N, K = body.m, body.n, body.k

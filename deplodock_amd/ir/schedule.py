@@ -223,7 +223,7 @@ class TilePlan:
 # STAGE
 # --------------------------------------------------------------------------
 
-_TRANSPORTS = {"sync": "sync", "dl": "dl", "cp": "dl", "mix": "mix"}
+_TRANSPORTS = {"sync": "sync", "dl": "dl", "cp": "dl", "mix": "mix", "ks": "ks"}
 
 
 @dataclass(frozen=True)
@@ -234,7 +234,10 @@ class Stage:
     ``transport``  ``sync``: global → registers → ``ds_write`` (software
                    pipelined through ``reg_depth`` register sets);
                    ``dl``: global loads that write LDS directly, no VGPR hop;
-                   ``mix``: the a operand as ``sync``, the b operand as ``dl``.
+                   ``mix``: the a operand as ``sync``, the b operand as ``dl``;
+                   ``ks``: no LDS staging — at most 16 rows, the reduction axis split
+                   over ``depth`` waves that load their fragments straight from global
+                   memory, all at once.
     ``ring``       kept for grammar compatibility (a depth > 1 is a ring)."""
 
     depth: int = 2

@@ -267,12 +267,18 @@ def _check_tile(plan: TilePlan, body: Contraction, ctx: Context, depth: int, dl:
         raise ScheduleError("the row epilogue works on the output tile staged in LDS, which this tile does not fit")
 
 
+from deplodock_amd.emit.skinny import skinny_waves  # noqa: E402
+
+
 def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
     """Staging when nothing pins it.
 
     * A row-normalised operand is transformed in registers on its way to LDS: ``sync``
       (``mix`` sends the other operand direct to LDS; 12.7 / 15.8 us against 12.3 / 15.9 us).
-    * Decode-size problems (M <= 16) stream the weight once, straight from HBM: ``sync``
+    * Decode-size problems (M <= 16) are one pass over the weight matrix and cost memory round trips:
+      where the shape allows, the k-split few-row form (``ks``: no slab loop, every wave requests all of
+      its fragments at once; us back to back / with the weight streamed from HBM, 1024x3072:
+      M = 1 3.03 / 4.40 -> 2.59 / 4.02, M = 16 3.10 / 4.56 -> 2.74 / 4.38).  Otherwise ``sync``
       through two register sets (measured with operands rotating through more memory
       than the caches hold: 4.4 / 4.5 / 6.2 us at M = 1 / 16 / 128 on 1024x3072, against
       5.2 / 5.4 / 6.9 through one set and 4.6 / 4.6 / 6.4 with a three-slab ``dl`` ring).
@@ -284,6 +290,8 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
       9.4; 512x1024x2048 7.4 -> 6.2 -> 6.2; 512x4096x1024 7.8 -> 6.8 -> 6.7; 2048x3072x1024
       17.2 -> 15.9 -> 16.1; 4096^3 136 -> 122; the block as one graph 66.9 -> 65.2 -> 62.8)."""
     steps = -(-body.k // plan.bk_elems)
+    if skinny_waves(body):
+        return Stage(depth=skinny_waves(body), transport="ks")
     if body.k % plan.bk_elems:
         return Stage(depth=2, transport="sync")  # the short last slab is zero-filled in registers
     if body.a_prologue is not None and body.a_prologue.scale is None:
@@ -347,7 +355,10 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
             stage = Stage.parse(pinned_stage)
             if stage is not None and stage.transport == "dl" and (plan.bk_elems // plan.atom.k) % 2:
                 raise ScheduleError("direct-to-LDS staging needs an even number of MFMA steps per slab")
-            if stage is not None:
+            if stage is not None and stage.transport == "ks":
+                if not skinny_waves(body) or stage.depth not in (1, 2, 4, 8, 16) or body.k % (32 * stage.depth):
+                    raise ScheduleError(f"the k-split few-row form does not fit M={body.m} N={body.n} K={body.k} with {stage.depth} waves")
+            elif stage is not None:
                 _check_tile(plan, body, ctx, depth=max(2, stage.depth), dl=stage.transport == "dl")
         except ScheduleError as exc:
             logger.warning("EMMY_STAGE=%r ignored: %s", pinned_stage, exc)

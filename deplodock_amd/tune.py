@@ -52,6 +52,7 @@ TILE_SWEEP: tuple[str, ...] = (
     "a:mfma_16x16x32_bf16/w1x1/f1x1/k8",
 )  # every tile that won an in-graph ranking of the decoder block's contractions at 64 ... 2048 tokens, and their neighbours
 STAGE_SWEEP: tuple[str, ...] = ("d2/dl", "d3/dl", "d2/sync/p2")
+FEW_ROW_SWEEP: tuple[str, ...] = ("d8/ks", "d4/ks")  # the k-split few-row form has no tile: one candidate each
 REDUCE_SWEEP: tuple[str, ...] = ("b8", "b16", "b32", "b64", "b128", "b256", "b512", "b1024")
 NT_SWEEP: tuple[str, ...] = ("0", "1")
 FLASH_SWEEP: tuple[str, ...] = (
@@ -167,7 +168,7 @@ def candidate_rounds(families: set[str]) -> list[dict[str, str]]:
     """One pin set per round; round r holds the r-th candidate of every family present."""
     per_family: dict[str, list[dict[str, str]]] = {}
     if "contraction" in families:
-        per_family["contraction"] = [{"TILE": t, "STAGE": s} for s in STAGE_SWEEP for t in TILE_SWEEP]
+        per_family["contraction"] = [{"TILE": t, "STAGE": s} for s in STAGE_SWEEP for t in TILE_SWEEP] + [{"TILE": TILE_SWEEP[-1], "STAGE": s} for s in FEW_ROW_SWEEP]
     if "row_reduce" in families:
         per_family["row_reduce"] = [{"REDUCE": r, "NT": n} for n in NT_SWEEP for r in REDUCE_SWEEP]
     if "flash" in families:

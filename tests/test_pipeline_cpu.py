@@ -57,11 +57,15 @@ def test_linear_is_one_mfma_kernel(launcher_lib, m):
     assert k.kernel_name.startswith("k_linear_")
     assert "__builtin_amdgcn_mfma_f32_" in k.kernel_source
     assert k.algo_flops == 2 * m * 3072 * 1024
-    # decode sizes stream the weight from HBM: two slabs in flight through two register sets
-    # from 128 rows on direct-to-LDS loads (three 48 KiB slabs of the 32x64x256 tile; two where a slab is
-    # long enough by itself: a 128x192x64 slab is 768 cycles of MFMA work)
-    assert k.knobs["STAGE"] == {1: "d2/sync/p2", 16: "d2/sync/p2", 128: "d3/dl", 2048: "d2/dl"}[m]
-    assert ("ra[RS][A_PER_T]" in k.kernel_source) == (m < 128) and ("#define EMH_DLOAD" in k.kernel_source) == (m >= 128)
+    # decode sizes are one pass over the weight: the reduction axis split over the eight waves of a workgroup,
+    # every fragment requested at once, no slab loop (a shape that does not fit that form goes through two
+    # register sets); from 128 rows on direct-to-LDS loads (three 48 KiB slabs of the 32x64x256 tile; two
+    # where a slab is long enough by itself: a 128x192x64 slab is 768 cycles of MFMA work)
+    assert k.knobs["STAGE"] == {1: "d8/ks", 16: "d8/ks", 128: "d3/dl", 2048: "d2/dl"}[m]
+    assert ("wave * 128 + lk * 8" in k.kernel_source) == (m < 128) and ("#define EMH_DLOAD" in k.kernel_source) == (m >= 128)
+    if m == 16:
+        odd = kernels(compile_case(eager.linear_case(m=16, k=1000, n=712)))[0]  # K is not a multiple of 32
+        assert odd.knobs["STAGE"].startswith("d2/sync") and "ra[RS][A_PER_T]" in odd.kernel_source
     hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
 
 

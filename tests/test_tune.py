@@ -81,7 +81,7 @@ def test_unrealisable_tile_pin_degrades_per_kernel(monkeypatch, launcher_lib):
 
 def test_candidate_rounds_cover_every_family_once():
     rounds = candidate_rounds({"contraction", "row_reduce", "flash"})
-    assert len(rounds) == 60  # the longest family: 20 tiles x 3 stagings
+    assert len(rounds) == 62  # the longest family: 20 tiles x 3 stagings + the two tile-less few-row forms
     assert {"TILE", "STAGE", "REDUCE", "NT", "FLASH"} <= set(rounds[0])
     assert "FLASH" not in rounds[-1] and "TILE" in rounds[-1]
     assert candidate_rounds({"row_reduce"}) and all(set(r) == {"REDUCE", "NT"} for r in candidate_rounds({"row_reduce"}))
