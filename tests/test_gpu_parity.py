@@ -129,6 +129,26 @@ def test_c3_linear(device, m):
     eager.assert_close(ours[: min(m, 8)], exact, 2 ** -7, 1e-3, f"linear M={m} vs float64")
 
 
+@pytest.mark.parametrize("waves", [None, 8, 4, 2, 1])
+@pytest.mark.parametrize("m,k,n", [(1, 1024, 3072), (16, 1024, 3072), (5, 512, 1960), (13, 3072, 1024), (16, 2048, 24), (3, 16384, 256), (2, 32, 40), (16, 8192, 64)])
+def test_few_row_linear_k_split_over_waves(device, m, k, n, waves, monkeypatch):
+    """At most 16 rows: the reduction axis is split over the waves of a workgroup, every weight fragment is
+    requested at once, the activation rows go through LDS where they fit (two rows of 16384 do, 16 of 8192
+    do not), long reduction extents loop over 16-step groups, and a column count that is no multiple of 16
+    re-reads the last row without storing it."""
+    if waves is not None:
+        monkeypatch.setenv("EMMY_STAGE", f"d{waves}/ks")
+    case = eager.linear_case(m=m, k=k, n=n, seed=m + k)
+    ours, want, compiled = run_case(case, device)
+    op = next(n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp))
+    assert op.knobs["STAGE"].endswith("/ks"), op.knobs  # a wave count that does not divide the extent degrades to the default one
+    if waves is not None and k % (32 * waves) == 0:
+        assert op.knobs["STAGE"] == f"d{waves}/ks"
+    eager.assert_close(ours, want, case.rtol, case.atol, f"few-row linear {m}x{k}x{n} vs eager (GPU)")
+    exact = case.inputs[0].double() @ case.module.weight.detach().double().cpu().T
+    eager.assert_close(ours, exact, 2 ** -7, 2e-3, f"few-row linear {m}x{k}x{n} vs float64")
+
+
 @pytest.mark.parametrize("m,k,n", [(17, 512, 200), (40, 1024, 1000), (70, 256, 136), (130, 2048, 1024), (260, 512, 96), (300, 1024, 4096), (1024, 1024, 3072), (2048, 512, 4096),
                                    (30, 72, 192), (64, 200, 712), (4, 200, 4096), (300, 1000, 512), (128, 40, 64)])  # the last five: K is not a multiple of the MFMA depth
 def test_linear_heuristic_tiles_on_ragged_and_one_round_shapes(device, m, k, n):
@@ -461,7 +481,8 @@ def test_row_norm_with_a_second_reader_stays_a_kernel(device):
         prog.close()
 
 
-@pytest.mark.parametrize("m,k,n,dtype", [(128, 512, 768, torch.bfloat16), (100, 512, 260, torch.bfloat16), (16, 1024, 3072, torch.float16), (2048, 1024, 3072, torch.bfloat16)])
+@pytest.mark.parametrize("m,k,n,dtype", [(128, 512, 768, torch.bfloat16), (100, 512, 260, torch.bfloat16), (16, 1024, 3072, torch.float16), (2048, 1024, 3072, torch.bfloat16),
+                                         (1, 1024, 3072, torch.bfloat16), (7, 512, 260, torch.float16)])
 def test_linear_with_bias(device, m, k, n, dtype):
     """``nn.Linear``'s default has a bias: it is added to the fp32 accumulator before the one rounding."""
     torch.manual_seed(5)
