@@ -128,12 +128,12 @@ def _cpu_baseline() -> dict:
 
 def _table(device, only: str | None = None, extended: bool = False) -> list[dict]:
     """Per-kernel µs / achieved rate / fraction of peak for every configuration.
-    The oracle package supplies each configuration's module + seeded inputs and
-    checks the kernels' outputs before they are timed; it is never what is timed."""
+    Each kernel's output is compared with PyTorch eager on the device before it is timed
+    (a wrong kernel's time means nothing); eager is never what is timed."""
     import torch
 
     from deplodock_amd import HipBackend, trace_module
-    from oracle import eager
+    from deplodock_amd import workloads as wl
 
     be = HipBackend(device_id=0)
     rows: list[dict] = []
@@ -190,8 +190,9 @@ def _table(device, only: str | None = None, extended: bool = False) -> list[dict
                 prog.run()
                 torch.cuda.synchronize()
                 ours = prog.output_tensors()[compiled.outputs[0]]
-                want = eager.run_eager(case, device)
-                eager.assert_close(ours.reshape(want.shape), want, case.rtol, case.atol, label)
+                with torch.no_grad():
+                    want = case.module.to(device)(*(t.to(device) for t in case.inputs))
+                torch.testing.assert_close(ours.reshape(want.shape).float(), want.float(), rtol=case.rtol, atol=case.atol, msg=lambda m: f"{label}: {m}")
             finally:
                 prog.close()
         res = be.benchmark(compiled, input_data=data, warmup=3, num_iters=20)
@@ -214,18 +215,18 @@ def _table(device, only: str | None = None, extended: bool = False) -> list[dict
                 row["achieved_cold"] = round(case.algo_bytes / (c_us * 1e-6) / 1e9, 1)
         rows.append(row)
 
-    bench(eager.rms_norm_case, "C1 rms_norm fp32 [1,32,2048]", "hbm", cold=True)
-    bench(lambda: eager.rms_norm_case(rows=32768), "C1x rms_norm fp32 [1,32768,2048]", "hbm")
-    bench(eager.softmax_case, "C2 softmax fp32 [1,28,2048,2048]", "hbm")
+    bench(wl.rms_norm_case, "C1 rms_norm fp32 [1,32,2048]", "hbm", cold=True)
+    bench(lambda: wl.rms_norm_case(rows=32768), "C1x rms_norm fp32 [1,32768,2048]", "hbm")
+    bench(wl.softmax_case, "C2 softmax fp32 [1,28,2048,2048]", "hbm")
     for m in (1, 16, 128):
-        bench(lambda m=m: eager.linear_case(m=m), f"C3 linear bf16 M={m} K=1024 N=3072", "hbm", cold=True)
-    bench(lambda: eager.linear_case(m=2048), "C3 linear bf16 M=2048 K=1024 N=3072", "mfma")
+        bench(lambda m=m: wl.linear_case(m=m), f"C3 linear bf16 M={m} K=1024 N=3072", "hbm", cold=True)
+    bench(lambda: wl.linear_case(m=2048), "C3 linear bf16 M=2048 K=1024 N=3072", "mfma")
     if extended:
-        bench(lambda: eager.linear_case(m=4096, k=4096, n=4096), "C3x linear bf16 M=4096 K=4096 N=4096", "mfma")
-    bench(eager.sdpa_case, "C4 causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
+        bench(lambda: wl.linear_case(m=4096, k=4096, n=4096), "C3x linear bf16 M=4096 K=4096 N=4096", "mfma")
+    bench(wl.sdpa_case, "C4 causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
     if extended:
-        bench(lambda: eager.sdpa_case(causal=False), "C4x non-causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
-    bench(lambda: eager.qwen3_block_case(seq=512), "C5 qwen3-0.6B block bf16 S=512", "mfma")
+        bench(lambda: wl.sdpa_case(causal=False), "C4x non-causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
+    bench(lambda: wl.qwen3_block_case(seq=512), "C5 qwen3-0.6B block bf16 S=512", "mfma")
     return rows
 
 

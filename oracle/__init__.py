@@ -10,8 +10,9 @@ Two layers:
                      and streaming carriers compute (each function cites the
                      reference file:line it follows).
 ``oracle.eager``     the oracle the task prescribes: PyTorch eager on the same
-                     ``nn.Module`` and seeded inputs, plus the seeded input
-                     recipes of the five benchmark configurations.
+                     ``nn.Module`` and seeded inputs (the workloads themselves —
+                     modules and input recipes — live in
+                     ``deplodock_amd.workloads`` and are re-exported here).
 
 Every function of ``emmy_ops`` is pinned in ``tests/test_oracle.py`` against
 PyTorch eager on the reference's own test recipes, against committed golden

@@ -1,9 +1,9 @@
 """The prescribed oracle: PyTorch eager on the same module and seeded inputs.
 
-TEST INFRASTRUCTURE ONLY (see ``oracle/__init__.py``).  Holds the seeded input
-recipes of the five benchmark configurations (generated on the CPU so every
-machine sees identical bits), the modules they run through, and the tolerance
-checker.
+TEST INFRASTRUCTURE ONLY (see ``oracle/__init__.py``).  Runs a workload
+(``deplodock_amd.workloads``: module + seeded inputs, re-exported here) through
+PyTorch eager, compares within the stated tolerance, and times eager on the host
+cores for the CPU baseline.
 """
 
 from __future__ import annotations
@@ -14,160 +14,20 @@ from dataclasses import dataclass
 import torch
 from torch import nn
 
-FP32_RTOL = 1e-5
-BF16_RTOL = 2e-2
-
-
-@dataclass
-class Case:
-    name: str
-    module: nn.Module
-    inputs: tuple
-    rtol: float
-    atol: float
-    algo_bytes: int = 0
-    algo_flops: int = 0
-
-
-class Sdpa(nn.Module):
-    def __init__(self, causal: bool = True):
-        super().__init__()
-        self.causal = causal
-
-    def forward(self, q, k, v):
-        return nn.functional.scaled_dot_product_attention(q, k, v, is_causal=self.causal, enable_gqa=True)
-
-
-def rms_norm_case(rows: int = 32, cols: int = 2048, seed: int = 0) -> Case:
-    """C1: ``nn.RMSNorm(2048, eps=1e-6)`` on fp32 ``[1, rows, cols]`` ~N(0,1), weight ~N(1, 0.1)."""
-    torch.manual_seed(seed)
-    x = torch.randn(1, rows, cols)
-    m = nn.RMSNorm(cols, eps=1e-6)
-    with torch.no_grad():
-        m.weight.copy_(1 + 0.1 * torch.randn(cols))
-    return Case(f"rms_norm_{rows}x{cols}", m.eval(), (x,), FP32_RTOL, 1e-6, algo_bytes=(2 * rows * cols + cols) * 4)
-
-
-def softmax_case(shape=(1, 28, 2048, 2048), seed: int = 0) -> Case:
-    """C2: ``nn.Softmax(-1)`` on fp32 ~N(0, 2).  The absolute floor covers outputs
-    near zero, where a pure relative bound is ill-posed."""
-    torch.manual_seed(seed)
-    x = 2 * torch.randn(*shape)
-    return Case("softmax_" + "x".join(map(str, shape)), nn.Softmax(dim=-1).eval(), (x,), FP32_RTOL, 1e-9, algo_bytes=2 * x.numel() * 4)
-
-
-def linear_case(m: int = 2048, k: int = 1024, n: int = 3072, seed: int = 0) -> Case:
-    """C3: ``nn.Linear(k, n, bias=False)`` bf16, x ~N(0,1), W ~N(0, 0.02)."""
-    torch.manual_seed(seed)
-    x = torch.randn(m, k).bfloat16()
-    lin = nn.Linear(k, n, bias=False)
-    with torch.no_grad():
-        lin.weight.copy_(0.02 * torch.randn(n, k))
-    return Case(f"linear_{m}x{k}x{n}", lin.bfloat16().eval(), (x,), BF16_RTOL, 2e-2, algo_bytes=(m * k + n * k + m * n) * 2, algo_flops=2 * m * n * k)
-
-
-def sdpa_case(b: int = 1, hq: int = 16, hkv: int = 8, s: int = 2048, d: int = 128, causal: bool = True, seed: int = 0) -> Case:
-    """C4: causal GQA attention, bf16 ~N(0,1), scale 1/sqrt(d)."""
-    torch.manual_seed(seed)
-    q = torch.randn(b, hq, s, d).bfloat16()
-    k = torch.randn(b, hkv, s, d).bfloat16()
-    v = torch.randn(b, hkv, s, d).bfloat16()
-    pairs = s * (s + 1) // 2 if causal else s * s
-    return Case(
-        f"sdpa_{b}x{hq}x{hkv}x{s}x{d}", Sdpa(causal).eval(), (q, k, v), BF16_RTOL, 2e-2,
-        algo_bytes=(2 * b * hq * s * d + 2 * b * hkv * s * d) * 2, algo_flops=4 * b * hq * d * pairs,
-    )  # fmt: skip
-
-
-class Qwen3Block(nn.Module):
-    """Wraps ``transformers``' ``Qwen3DecoderLayer`` (built from a local config,
-    no download) so it takes ``(x, cos, sin)`` and returns the hidden state."""
-
-    def __init__(self, layer):
-        super().__init__()
-        self.l = layer
-
-    def forward(self, x, cos, sin):
-        out = self.l(x, position_embeddings=(cos, sin), attention_mask=None)
-        return out[0] if isinstance(out, tuple) else out
-
-
-def qwen3_block_case(seq: int = 512, seed: int = 0, dtype=torch.bfloat16) -> Case:
-    """C5: one Qwen3-0.6B-architecture decoder block, weights ~N(0, 0.02), norm
-    weights 1, x ~N(0,1), positions 0..seq-1, RoPE theta 1e6."""
-    from transformers import Qwen3Config
-    from transformers.models.qwen3.modeling_qwen3 import Qwen3DecoderLayer, Qwen3RotaryEmbedding
-
-    cfg = Qwen3Config(
-        hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128, intermediate_size=3072,
-        rms_norm_eps=1e-6, rope_theta=1e6, num_hidden_layers=1, vocab_size=1024, max_position_embeddings=max(4096, seq),
-    )  # fmt: skip
-    cfg._attn_implementation = "sdpa"
-    torch.manual_seed(seed)
-    layer = Qwen3DecoderLayer(cfg, 0)
-    with torch.no_grad():
-        for name, p in layer.named_parameters():
-            if "norm" in name:
-                p.fill_(1.0)
-            else:
-                p.copy_(0.02 * torch.randn_like(p))
-    x = torch.randn(1, seq, 1024)
-    cos, sin = Qwen3RotaryEmbedding(cfg)(x, torch.arange(seq)[None])
-    h, hq, hkv, d, inter = 1024, 16, 8, 128, 3072
-    flops = 2 * seq * h * (hq * d + 2 * hkv * d) + 2 * seq * hq * d * h + 3 * 2 * seq * h * inter + 4 * hq * d * (seq * (seq + 1) // 2)
-    wbytes = (h * (hq * d + 2 * hkv * d) + hq * d * h + 3 * h * inter) * 2
-    return Case(
-        f"qwen3_block_s{seq}", Qwen3Block(layer).to(dtype).eval(), (x.to(dtype), cos.to(dtype), sin.to(dtype)),
-        BF16_RTOL if dtype is torch.bfloat16 else 1e-4, 4e-2 if dtype is torch.bfloat16 else 1e-4, algo_bytes=wbytes, algo_flops=flops,
-    )  # fmt: skip
-
-
-class NormedRopeAttention(nn.Module):
-    """The front of a Qwen3-style attention layer with ``nn.RMSNorm`` head norms:
-    q/k/v projections, per-head norm of q and k, rotary embedding, causal GQA
-    attention.  Unlike the block case its norm weights are not all ones, so a
-    kernel that pairs a column with the wrong weight or table row shows."""
-
-    def __init__(self, hidden: int, q_heads: int, kv_heads: int, head_dim: int):
-        super().__init__()
-        self.hq, self.hkv, self.d = q_heads, kv_heads, head_dim
-        self.q_proj = nn.Linear(hidden, q_heads * head_dim, bias=False)
-        self.k_proj = nn.Linear(hidden, kv_heads * head_dim, bias=False)
-        self.v_proj = nn.Linear(hidden, kv_heads * head_dim, bias=False)
-        self.q_norm = nn.RMSNorm(head_dim, eps=1e-6)
-        self.k_norm = nn.RMSNorm(head_dim, eps=1e-6)
-
-    @staticmethod
-    def _rotate_half(x):
-        half = x.shape[-1] // 2
-        return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
-
-    def forward(self, x, cos, sin):
-        b, s, _ = x.shape
-        q = self.q_norm(self.q_proj(x).view(b, s, self.hq, self.d)).transpose(1, 2)
-        k = self.k_norm(self.k_proj(x).view(b, s, self.hkv, self.d)).transpose(1, 2)
-        v = self.v_proj(x).view(b, s, self.hkv, self.d).transpose(1, 2)
-        c, sn = cos.unsqueeze(1), sin.unsqueeze(1)
-        q = q * c + self._rotate_half(q) * sn
-        k = k * c + self._rotate_half(k) * sn
-        o = nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
-        return o.transpose(1, 2).reshape(b, s, self.hq * self.d)
-
-
-def normed_rope_attention_case(hidden: int = 256, q_heads: int = 4, kv_heads: int = 2, head_dim: int = 64, seq: int = 100, seed: int = 0) -> Case:
-    """bf16; projection weights ~N(0, 0.05), norm weights ~N(1, 0.2), x ~N(0,1), rotary base 1e4."""
-    torch.manual_seed(seed)
-    m = NormedRopeAttention(hidden, q_heads, kv_heads, head_dim)
-    with torch.no_grad():
-        for name, p in m.named_parameters():
-            p.copy_(1 + 0.2 * torch.randn_like(p) if "norm" in name else 0.05 * torch.randn_like(p))
-    x = torch.randn(1, seq, hidden)
-    ang = torch.arange(seq)[:, None] * (1e4 ** (-torch.arange(0, head_dim, 2) / head_dim))[None]
-    emb = torch.cat((ang, ang), -1)
-    return Case(
-        f"normed_rope_attention_h{hidden}_{q_heads}x{kv_heads}x{head_dim}_s{seq}", m.to(torch.bfloat16).eval(),
-        (x.to(torch.bfloat16), emb.cos()[None].to(torch.bfloat16), emb.sin()[None].to(torch.bfloat16)), BF16_RTOL, 2e-2,
-    )  # fmt: skip
+from deplodock_amd.workloads import (  # noqa: F401  (the shapes are the product's; the checker re-exports them)
+    BF16_RTOL,
+    FP32_RTOL,
+    Case,
+    NormedRopeAttention,
+    Qwen3Block,
+    Sdpa,
+    linear_case,
+    normed_rope_attention_case,
+    qwen3_block_case,
+    rms_norm_case,
+    sdpa_case,
+    softmax_case,
+)
 
 
 def block_weights(case: Case) -> dict:
