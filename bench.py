@@ -13,8 +13,8 @@ JSON line printed carries:
 * ``roofline``     the dominant kernel against MI355X's 8 TB/s: algorithmic bytes
                    per launch / average launch duration from HIP events recorded
                    on the launch stream around the same K launches;
-* ``cpu_baseline`` PyTorch eager of the same module on the host cores, on a
-                   bounded sample of the same workload;
+* ``cpu_baseline`` PyTorch eager of the same module on the host cores, over the
+                   whole workload (20 passes of tens of milliseconds each);
 * ``kernels``      the per-kernel table the metric asks for: µs, achieved GB/s or
                    TFLOP/s and fraction of peak for RMSNorm, softmax, linear
                    (M in 1/16/128/2048), causal GQA attention, and the Qwen3 block.
@@ -109,20 +109,20 @@ def _headline(device, steps: int, warmup: int) -> dict:
 
 
 def _cpu_baseline() -> dict:
-    """PyTorch eager softmax on the host cores over 1/7 of the workload."""
+    """PyTorch eager softmax of the whole workload on the host cores (a pass takes tens of milliseconds)."""
     import torch
 
     from oracle import eager
 
     threads = min(os.cpu_count() or 1, 16)
-    case = eager.softmax_case(shape=(1, 4, 2048, 2048))
-    sec = eager.time_eager_cpu(case, threads=threads, warmup=1, iters=5)
+    case = eager.softmax_case()
+    sec = eager.time_eager_cpu(case, threads=threads, warmup=3, iters=20)
     return {
         "value": case.algo_bytes / sec / 1e9,
         "unit": "GB/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"PyTorch {torch.__version__} eager nn.Softmax(-1) on fp32 [1,4,2048,2048] (1/7 of the workload), median of 5 passes, {threads} threads",
+        "sample": f"PyTorch {torch.__version__} eager nn.Softmax(-1) on fp32 [1,28,2048,2048] (the whole workload), median of 20 passes after 3 warm-up passes, {threads} threads",
     }
 
 
