@@ -47,7 +47,7 @@ def _spills(hip: HipOp, ctx: Context) -> int:
     try:
         return hiprtc.spilled_vgprs(hip.kernel_source, hip.kernel_name, arch=ctx.arch)
     except launcher.CompileError:
-        raise
+        raise  # a real compile error (it is a LauncherError too, and must not be taken for a missing library)
     except launcher.LauncherError:
         return 0
 
@@ -63,6 +63,8 @@ def _lower_contraction(op: TileOp, ctx: Context) -> HipOp:
     body = op.body
     hip = _named(emit_contraction(body, _PLACEHOLDER, ctx), op)
     spilled = _spills(hip, ctx)
+    if body.stage is None:
+        return hip  # not scheduled (a hand-built body): nothing to degrade to
     if spilled and (body.stage.transport != "sync" or body.stage.reg_depth > 1):
         logger.warning("%s: STAGE=%s spills %d vector registers: plain register staging instead", hip.kernel_name, hip.knobs.get("STAGE"), spilled)
         body.stage = replace(body.stage, transport="sync", depth=2, reg_depth=1)
