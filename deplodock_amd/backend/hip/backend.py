@@ -38,6 +38,13 @@ class HipBackend(Backend):
         self.debug = config.debug_enabled() if debug is None else debug
         self.dump = dump
         self.bench_wall_timeout_s = bench_wall_timeout_s
+        self._worker = None
+        if bench_wall_timeout_s is not None:
+            # Benchmarks will run in a killable child forked from a clean server process: start that server
+            # now, while this process (if the backend is built first, as the tuner does) has not touched the GPU.
+            from deplodock_amd.backend.hip.bench_worker import start_server
+
+            start_server()
         self.bench_compile_timeout_s = bench_compile_timeout_s
         self.bench_run_timeout_s = bench_run_timeout_s
         self.device_id = device_id
@@ -161,7 +168,9 @@ class HipBackend(Backend):
     ) -> BenchmarkResult:
         """Event-timed benchmark (backend.py:179-237).  ``nvcc_flags`` keeps the
         reference's keyword; here it re-points ``EMMY_HIPRTC_FLAGS`` for this one
-        compile."""
+        compile.  With ``bench_wall_timeout_s`` set and no ``on_iter`` callback the
+        benchmark runs in an isolated worker process that is killed at the limit
+        (``RuntimeError``, the caller's bench_fail); otherwise in this process."""
         return self.benchmark(compiled, warmup=warmup, num_iters=num_iters, on_iter=on_iter, hiprtc_flags=nvcc_flags, capture_graphs=capture_graphs, input_data=input_data)
 
     def benchmark(self, compiled: Graph, *, warmup: int = 5, num_iters=20, on_iter=None, hiprtc_flags: str | None = None, capture_graphs: bool = True, input_data: dict | None = None) -> BenchmarkResult:
@@ -169,6 +178,23 @@ class HipBackend(Backend):
 
         self._select_device()
         compiled = self.variant(compiled, input_data)
+        if self.bench_wall_timeout_s is not None and on_iter is None:
+            from deplodock_amd.backend.hip.bench_worker import BenchWorker, benchmark_program_isolated
+
+            if self._worker is None:
+                self._worker = BenchWorker(device_id=self.device_id)
+            return benchmark_program_isolated(
+                compiled,
+                worker=self._worker,
+                wall_timeout_s=self.bench_wall_timeout_s,
+                input_data=self.bind(compiled, input_data),
+                hiprtc_flags=hiprtc_flags,
+                warmup=warmup,
+                num_iters=num_iters,
+                compile_timeout_s=self.bench_compile_timeout_s,
+                run_timeout_s=self.bench_run_timeout_s,
+                capture_graphs=capture_graphs,
+            )
         with config.hiprtc_flags_override(hiprtc_flags):
             return benchmark_program(
                 compiled,
@@ -180,6 +206,12 @@ class HipBackend(Backend):
                 run_timeout_s=self.bench_run_timeout_s,
                 capture_graphs=capture_graphs,
             )
+
+    def close(self) -> None:
+        """End the benchmark worker process, if one was started."""
+        if self._worker is not None:
+            self._worker.close()
+            self._worker = None
 
     def _select_device(self) -> None:
         if self.device_id is not None:

@@ -139,10 +139,50 @@ class LoadedKernel:
         self.name, self.module, self.fn, self.path = name, module, fn, path
 
 
-def load_function(source: str, name: str, *, arch: str = "gfx950") -> LoadedKernel:
-    """Compile (cached) and load ``name`` on the current device."""
+# (device, code-object file name, kernel name) -> the loaded kernel.  A code object is loaded onto a
+# device once per process and stays loaded: programs come and go (benchmark sweeps build hundreds, a
+# serving loop one per sequence length) and share the modules, whose number is bounded by the number of
+# distinct kernels, not by the number of programs.
+_loaded: dict[tuple[int, str, str], LoadedKernel] = {}
+
+
+def _current_device() -> int:
+    import torch
+
+    return torch.cuda.current_device() if torch.cuda.is_available() else -1
+
+
+def load_function(source: str, name: str, *, arch: str = "gfx950", cached: bool = True) -> LoadedKernel:
+    """Compile (cached on disk) and load ``name`` on the current device.  With ``cached`` (the default)
+    the module is shared by every caller in the process and must not be unloaded by them; with
+    ``cached=False`` the caller owns the module and unloads it (one-off probe kernels)."""
     path = compile_to_hsaco(source, name, arch=arch)
     lib = launcher.load()
+    key = (_current_device(), path.name, name)
+    if cached and key in _loaded:
+        return _loaded[key]
     module = lib.module_load(path.read_bytes())
-    fn = lib.get_function(module, name)
-    return LoadedKernel(name, module, fn, path)
+    try:
+        fn = lib.get_function(module, name)
+    except launcher.LauncherError:
+        lib.module_unload(module)
+        raise
+    kernel = LoadedKernel(name, module, fn, path)
+    if cached:
+        _loaded[key] = kernel
+    return kernel
+
+
+def unload_all() -> int:
+    """Unload every cached module (process teardown, or tests that count modules); returns how many."""
+    lib = launcher.load()
+    n = 0
+    for kernel in list(_loaded.values()):
+        lib.module_unload(kernel.module)
+        n += 1
+    _loaded.clear()
+    return n
+
+
+def loaded_module_count() -> int:
+    return len(_loaded)

@@ -321,6 +321,7 @@ class CompiledProgram:
         self._launch_graph_sizes: list[int] | None = None
         self._program_graph: int | None = None
         self._events: list[int] = []
+        self._hung = False  # set by the watchdog: the private stream may never drain
         self._build_packs()
 
     # -- construction ---------------------------------------------------------
@@ -426,6 +427,7 @@ class CompiledProgram:
         deadline = time.perf_counter() + _KERNEL_TIMEOUT_MS / 1000.0
         while not self.lib.event_query(event):
             if time.perf_counter() > deadline:
+                self._hung = True
                 raise HungKernelError(f"{what} did not finish within {_KERNEL_TIMEOUT_MS:.0f} ms")
             time.sleep(0)
 
@@ -472,9 +474,12 @@ class CompiledProgram:
                 try:
                     for _ in range(batch_sizes[i]):
                         self.launch_one(i, stream)
-                finally:
-                    g = self.lib.graph_end_capture(stream)
-                self._launch_graphs[i] = g
+                except BaseException:
+                    # the capture must still be ended, and the graph it hands back released
+                    with contextlib.suppress(launcher.LauncherError):
+                        self.lib.graph_destroy(self.lib.graph_end_capture(stream))
+                    raise
+                self._launch_graphs[i] = self.lib.graph_end_capture(stream)
         except launcher.LauncherError as exc:
             self._drop_launch_graphs()
             raise GraphCaptureError(f"graph capture failed: {exc}") from exc
@@ -496,8 +501,11 @@ class CompiledProgram:
             self.lib.graph_begin_capture(stream)
             try:
                 self.run(stream)
-            finally:
-                g = self.lib.graph_end_capture(stream)
+            except BaseException:
+                with contextlib.suppress(launcher.LauncherError):
+                    self.lib.graph_destroy(self.lib.graph_end_capture(stream))
+                raise
+            g = self.lib.graph_end_capture(stream)
         except launcher.LauncherError as exc:
             raise GraphCaptureError(f"whole-program graph capture failed: {exc}") from exc
         self._program_graph = g
@@ -521,6 +529,17 @@ class CompiledProgram:
         return self._elapsed(start, stop, "whole-program graph") / replays
 
     def close(self) -> None:
+        """Release graphs, events and the private stream.  The kernels' modules are shared through
+        ``hiprtc.load_function``'s per-device cache and stay loaded.  After the watchdog has fired the
+        stream may hold a kernel that never ends: waiting for it, or destroying it (which waits too),
+        would turn the ``HungKernelError`` into a stall, so the stream and what is queued on it are
+        abandoned to process teardown."""
+        if self._hung:
+            self._launch_graphs, self._launch_graph_sizes, self._program_graph = {}, None, None
+            self._events, self._stream = [], None
+            if hasattr(self, "_win"):
+                del self._win
+            return
         self._drop_launch_graphs()
         if self._program_graph is not None:
             self.lib.graph_destroy(self._program_graph)

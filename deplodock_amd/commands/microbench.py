@@ -1,9 +1,17 @@
-"""``microbench``: the two hardware figures the schedules are argued from.
+"""``microbench``: the hardware figures the schedules are argued from.
 
 * sustained MFMA rate (back-to-back ``mfma_f32_32x32x16_bf16``, one wave per SIMD);
 * MFMA / VALU co-issue: cycles for one MFMA followed by K independent vector
   instructions (``v_fma_f32`` or ``v_exp_f32``), for one and two waves per SIMD —
-  how much softmax arithmetic hides behind the matrix pipe.
+  how much softmax arithmetic hides behind the matrix pipe;
+* ``--l1fill``: the rate at which a compute unit can pull operand bytes in through
+  its vector L1 with nothing else going on — load-only kernels (plain
+  ``global_load_dwordx4`` into registers, and ``global_load_lds_dwordx4`` straight
+  into LDS) swept over waves per CU, loads in flight per wave, the address pattern
+  (contiguous 1 KiB per wave, or eight 128-byte pieces of rows a fixed stride apart,
+  which is what a GEMM slab fetch looks like) and L2-resident against streamed
+  operands.  That figure, not the MFMA peak, bounds a contraction whose tile needs
+  more bytes per MFMA cycle than it delivers.
 
 No counterpart in the reference (its constants are NVIDIA's); the kernels are
 emitted, compiled and launched through the same hipRTC / launcher path as
@@ -78,8 +86,160 @@ def coissue_seconds(k: int, kind: str, waves_per_simd: int, mfma: bool = True, i
     return ms * 1e-3 / (iters * 8) / waves_per_simd
 
 
+_L1FILL_SRC = r"""
+#define UNIT 1024  /* bytes one wave-level 16-byte-per-lane load moves */
+// Offsets stay 32-bit and every divisor is a power of two: the address arithmetic must not be
+// what the kernel measures.
+EMH_DEV unsigned emh_unit_offset(unsigned u, int lane) {
+  if (STRIDE == 0) return u * UNIT + lane * 16;  // contiguous: one wave reads 1 KiB in a run
+  // rows: a unit is the 128-byte piece kt of 8 consecutive rows; as in a GEMM slab fetch a
+  // workgroup walks all its ROWBLOCKS row blocks at one kt before it moves to the next piece
+  const unsigned rb = u % ROWBLOCKS, kt = (u / ROWBLOCKS) % KT, lap = u / (ROWBLOCKS * KT);
+  return ((lap * ROWBLOCKS + rb) * 8 + lane / 8) * (unsigned)STRIDE + kt * 128 + (lane % 8) * 16;
+}
+extern "C" __global__ __launch_bounds__(NT) void KNAME(const unsigned char* __restrict__ src, unsigned* __restrict__ out,
+                                                      int units_per_wave, int wg_units, int wg_kib, int share) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  // Workgroup ids rotate over the XCDs.  `share` workgroups of one XCD walk the same bytes
+  // (an L2-resident operand block shared by the tiles of a row, as in a GEMM); with share = 0
+  // every workgroup has bytes of its own.
+  const int xcd = blockIdx.x % XCDS, slot = blockIdx.x / XCDS;
+  const long base = (share ? (long)(xcd * share + slot % share) : (long)blockIdx.x) * wg_kib * 1024L;
+  const unsigned char* p = src + base;
+  u32x4 acc = {0u, 0u, 0u, 0u};
+  // wave w takes units w, w + waves, ...; workgroups sharing bytes start at different units
+  #define EMH_UNIT(i) emh_unit_offset(((unsigned)(i) * (NT / 64) + wave + slot * 7) & (unsigned)(wg_units - 1), lane)  /* wg_units is a power of two */
+#if TO_LDS
+  unsigned char* dst = lds + wave * (INFLIGHT * UNIT);
+  #pragma unroll
+  for (int i = 0; i < INFLIGHT; ++i) emh_dma16(p + EMH_UNIT(i), dst + i * UNIT);
+  for (int it = INFLIGHT; it < units_per_wave; it += INFLIGHT) {
+    #pragma unroll
+    for (int i = 0; i < INFLIGHT; ++i) {
+      __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(INFLIGHT - 1));  // the oldest load has landed: its slot is free again
+      emh_dma16(p + EMH_UNIT(it + i), dst + i * UNIT);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(0));
+  emh_lds_publish(lds + tid * 4);
+  acc[0] = *(const unsigned*)(dst + lane * 4);
+#else
+  u32x4 r[INFLIGHT];
+  #pragma unroll
+  for (int i = 0; i < INFLIGHT; ++i) r[i] = EMH_LD((const u32x4*)(p + EMH_UNIT(i)));
+  for (int it = INFLIGHT; it < units_per_wave; it += INFLIGHT) {
+    #pragma unroll
+    for (int i = 0; i < INFLIGHT; ++i) {
+      acc ^= r[i];
+      r[i] = EMH_LD((const u32x4*)(p + EMH_UNIT(it + i)));
+    }
+  }
+  #pragma unroll
+  for (int i = 0; i < INFLIGHT; ++i) acc ^= r[i];
+#endif
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) { out[blockIdx.x * NT + tid] = acc[0]; lds[tid] = 1; }  // keeps the loads (and the LDS that bounds occupancy) alive
+}
+"""
+
+_WAIT_VM = "#define EMH_WAIT_VM(n) ((((n) & 0xF) | ((((n) >> 4) & 0x3) << 14)) | 0x3F70)  /* vmcnt <= n, other counters left alone */\n"
+
+
+def l1fill_source(name: str, *, waves: int, inflight: int, stride: int, to_lds: bool, nontemporal: bool, row_blocks: int = 32, kt: int = 16, xcds: int = 8) -> str:
+    """Source of one load-only kernel.  ``stride`` = 0 reads contiguous 1 KiB runs; otherwise a wave
+    reads 128-byte pieces of 8 rows ``stride`` bytes apart."""
+    from deplodock_amd.emit import prelude
+
+    defs = {"KNAME": name, "NT": waves * 64, "INFLIGHT": inflight, "STRIDE": stride, "TO_LDS": int(to_lds), "ROWBLOCKS": row_blocks, "KT": kt, "XCDS": xcds,
+            "EMH_LD(p)": "__builtin_nontemporal_load(p)" if nontemporal else "(*(p))"}  # fmt: skip
+    return prelude.header(prelude.DMA) + _WAIT_VM + "".join(f"#define {k} {v}\n" for k, v in defs.items()) + _L1FILL_SRC
+
+
+def l1fill_bytes_per_second(*, waves: int, inflight: int, stride: int, to_lds: bool, resident: bool, wg_per_cu: int = 1, mib_per_wg: int = 16, lds_per_cu: int = 160 * 1024) -> float:
+    """Bytes per second the whole GPU pulls in with one load-only kernel (median of 5 launches).
+
+    ``resident``: the workgroups of an XCD loop over bytes that stay in its L2 (eight operand
+    blocks of 256 KiB, each walked by a quarter of the XCD's workgroups); otherwise every workgroup
+    streams 4 MiB of its own once, from a buffer larger than the last-level cache."""
+    import torch
+
+    from deplodock_amd.backend.hip import hiprtc, launcher
+    from deplodock_amd.backend.hip.launcher import PackedArgs
+
+    lib = launcher.load()
+    cus = lib.device_props(0)["compute_units"]
+    nt = waves * 64
+    name = f"k_l1fill_w{waves}_u{inflight}_s{stride}_{'lds' if to_lds else 'reg'}_{'l2' if resident else 'hbm'}"
+    fn = hiprtc.load_function(l1fill_source(name, waves=waves, inflight=inflight, stride=stride, to_lds=to_lds, nontemporal=not resident), name, cached=False)
+    lds_bytes = max(lds_per_cu // wg_per_cu - 4096, waves * inflight * 1024 if to_lds else 0)  # also pins the number of workgroups a CU holds
+    if lds_bytes > 64 * 1024:
+        try:
+            lib.func_set_dynamic_lds(fn.fn, lds_bytes)
+        except launcher.LauncherError as exc:
+            print(f"# {name}: {exc}; attributes {lib.func_attributes(fn.fn)}", flush=True)
+            if waves * inflight * 1024 > 64 * 1024:
+                raise
+            lds_bytes = 64 * 1024
+    grid = cus * wg_per_cu
+    wg_bytes = 256 * 1024 if resident else 4 * 1024 * 1024 * max(1, stride // 2048)  # streamed: 4 MiB actually read per workgroup
+    if stride:  # whole laps of (32 row blocks x 8 rows), of which 16 pieces of 128 bytes per row are read
+        laps = max(1, wg_bytes // (256 * stride))
+        wg_bytes, wg_units = laps * 256 * stride, laps * 512
+    else:
+        wg_units = wg_bytes // 1024
+    share = 8 if resident else 0
+    region = (8 * share * wg_bytes) if resident else grid * wg_bytes
+    buf = torch.empty(region + 4096, dtype=torch.uint8, device="cuda").random_(0, 255)
+    out = torch.zeros(grid * nt, dtype=torch.int32, device="cuda")
+    per_wave = (mib_per_wg * 1024 if resident else wg_units) // waves
+    units_per_wave = max(inflight, per_wave // inflight * inflight)
+    if wg_units & (wg_units - 1) or wg_bytes >= 2**31:
+        raise ValueError("l1fill: a workgroup's unit count must be a power of two and its bytes fit 31 bits")
+    args = PackedArgs([buf.data_ptr(), out.data_ptr()], [units_per_wave, wg_units, wg_bytes // 1024, share])
+    e0, e1 = lib.event_create(), lib.event_create()
+    times = []
+    for _ in range(6):
+        lib.event_record(e0, None)
+        lib.launch(fn.fn, (grid, 1, 1), (nt, 1, 1), lds_bytes, None, args)
+        lib.event_record(e1, None)
+        torch.cuda.synchronize()
+        times.append(lib.event_elapsed_ms(e0, e1) * 1e-3)
+    lib.event_destroy(e0)
+    lib.event_destroy(e1)
+    lib.module_unload(fn.module)
+    moved = grid * waves * units_per_wave * 1024
+    return moved / sorted(times[1:])[len(times[1:]) // 2]
+
+
+def handle_l1fill(args) -> None:
+    from deplodock_amd.backend.hip import launcher
+    from deplodock_amd.commands.table import render_table
+
+    props = launcher.load().device_props(0)
+    cus, clk = props["compute_units"], props["clock_khz"] * 1e3
+    print(f"load-only kernels on {cus} CUs; B/clk/CU at the {clk / 1e9:.2f} GHz engine clock the driver reports")
+    rows = []
+    quick = getattr(args, "quick", False)
+    for resident in (True, False):
+        for stride in (0, 2048, 2048 + 128, 8192) if not quick else (0, 2048):
+            for to_lds in (False, True):
+                for waves in (4, 8, 16) if not quick else (8,):
+                    for inflight in (2, 4, 8, 16) if not quick else (4,):
+                        if to_lds and waves * inflight > 128:
+                            continue
+                        bps = l1fill_bytes_per_second(waves=waves, inflight=inflight, stride=stride, to_lds=to_lds, resident=resident)
+                        rows.append(["L2" if resident else "HBM", "1 KiB runs" if stride == 0 else f"8 rows x 128 B, stride {stride}", "global_load_lds_dwordx4" if to_lds else "global_load_dwordx4",
+                                     str(waves), str(inflight), f"{waves * inflight}", f"{bps / 1e12:.2f}", f"{bps / clk / cus:.1f}"])  # fmt: skip
+                        print("  ".join(rows[-1]), flush=True)
+    print()
+    for line in render_table(["operands in", "pattern", "load", "waves/CU", "loads in flight/wave", "KiB in flight/CU", "TB/s", "B/clk/CU"], rows, "lllrrrrr"):
+        print(line)
+
+
 def register_microbench_command(subparsers) -> None:
-    p = subparsers.add_parser("microbench", help="Measure the MFMA rate and MFMA/VALU co-issue of the GPU")
+    p = subparsers.add_parser("microbench", help="Measure the MFMA rate, MFMA/VALU co-issue and the L1 fill rate of the GPU")
+    p.add_argument("--l1fill", action="store_true", help="sweep load-only kernels: bytes per clock a CU pulls through its vector L1")
+    p.add_argument("--quick", action="store_true", help="with --l1fill: a four-line sweep")
     p.set_defaults(func=handle_microbench)
 
 
@@ -89,6 +249,9 @@ def handle_microbench(args) -> None:
     if not torch.cuda.is_available():
         print("error: no HIP device visible", file=sys.stderr)
         sys.exit(1)
+    if getattr(args, "l1fill", False):
+        handle_l1fill(args)
+        return
     from deplodock_amd.backend.hip import launcher
     from deplodock_amd.commands.table import render_table
 

@@ -192,7 +192,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     A_PER_T, B_PER_T = a_chunks // T, b_chunks // T
     slab_bytes = (TM + TN * NB) * BK * 2
     depth = 2 if stage.transport == "mix" else max(2, stage.depth)
-    RS = 1 if stage.transport in ("dl", "mix") else max(1, stage.reg_depth)  # register sets a slab travels through on the sync path
+    RS = 1 if stage.transport in ("dl", "dli", "mix") else max(1, stage.reg_depth)  # register sets a slab travels through on the sync path
     lds_bytes = slab_bytes * depth
     if lds_bytes > ctx.lds_bytes_per_cu:
         raise LoweringError(f"contraction: {lds_bytes} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
@@ -205,7 +205,8 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     KT = -(-K // BK)
     m_guard = M % TM != 0
     n_guard = N % TN != 0
-    dl = stage.transport == "dl"
+    dli = stage.transport == "dli"  # direct to LDS, requests issued between the MFMAs of the slab before (see below)
+    dl = stage.transport in ("dl", "dli")
     mix = stage.transport == "mix"  # a through registers (it is transformed on the way), b direct to LDS
     if mix and b_chunks % 64:
         raise LoweringError("contraction: direct-to-LDS staging needs whole-wave chunk counts")
@@ -298,6 +299,12 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     # ---- staging ------------------------------------------------------------
     a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else "") + (" int ka[A_PER_T], kb[B_PER_T];" if k_guard else ""))
     a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
+    if dli:
+        if max(M * lda, N * NB * ldb) * 2 >= 2**32:
+            raise LoweringError("contraction: STAGE .../dli addresses operands with 32-bit byte offsets; this operand is larger than 4 GiB")
+        a("  unsigned va[A_PER_T], vb[B_PER_T];  // byte offset of each request's chunk from the operand base (the k position is added to the base, in scalar registers)")
+        a("  const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);  // wave-uniform by construction; says so to the compiler")
+        a("  const unsigned lds0 = emh_lds_addr(emh_lds);")
     a(r"""  #pragma unroll
   for (int i = 0; i < A_PER_T; ++i) {
     const int q = tid + i * T;""")
@@ -309,6 +316,8 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         a("    la[i] = row * (BK * 2) + emh_swz(row, c) * 16;")
     a(f"    int gr = m0 + row;{' if (gr > M - 1) gr = M - 1;' if m_guard else ''}")
     a(f"    ga[i] = A + {body.a_offset}L + (long)gr * LDA + c * 8;")
+    if dli:
+        a("    va[i] = ((unsigned)gr * LDA + c * 8) * 2u;")
     if pro is not None:
         a("    ca[i] = c * 8;")
     if k_guard:
@@ -330,6 +339,8 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     else:
         a(f"    int gr = n0 + row;{' if (gr > N - 1) gr = N - 1;' if n_guard else ''}")
     a(f"    gb[i] = B + {body.b_offset}L + (long)gr * LDB + c * 8;")
+    if dli:
+        a("    vb[i] = ((unsigned)gr * LDB + c * 8) * 2u;")
     if k_guard:
         a("    kb[i] = c * 8;")
     a("  }")
@@ -465,6 +476,8 @@ ROW_EPILOGUE_TABLES
         loads_per_slab = A_PER_T + B_PER_T
         if (depth - 1) * loads_per_slab > 63:
             raise LoweringError("contraction: too many loads in flight for the 6-bit vmcnt counter; lower STAGE depth")
+        if dli and depth < 3:
+            raise LoweringError("contraction: STAGE .../dli fills one slab while another is computed on and needs a ring of at least three")
         a(r"""  // Each wave-level direct-to-LDS load fills 64 consecutive 16-byte LDS slots
   // (slot = lane); the per-lane *global* address selects which chunk lands there.
   #define EMH_DLOAD(kt, buf) { \
@@ -485,7 +498,12 @@ ROW_EPILOGUE_TABLES
     emh_lds_publish(emh_lds + tid * 4); \
     asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
   #pragma unroll
-  for (int p = 0; p < DEPTH; ++p) if (p < KT) EMH_DLOAD(p, p);""")
+  for (int p = 0; p < DEPTH - DLI; ++p) if (p < KT) EMH_DLOAD(p, p);""".replace("DLI", "1" if dli else "0"))
+        if dli:
+            a(f"""  // One request of slab kt into ring buffer buf: the operand base moves along k in scalar registers, the
+  // lane's chunk offset is a loop-invariant 32-bit register, the LDS target a scalar: no vector arithmetic per request.
+  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L) + (long)(kt) * (BK * 2), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * T) * 16)
+  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L) + (long)(kt) * (BK * 2), vb[i], lds0 + (buf) * SLAB + TM * BK * 2 + (wave_u * 64 + (i) * T) * 16)""")
         if deferred:
             # the rows arrive in LDS untouched: every thread reads back the chunks it requested
             # (any chunk of the row will do for a row sum) while the slab is resident
@@ -499,7 +517,7 @@ ROW_EPILOGUE_TABLES
             a('    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) \\')
             a('    _Pragma("unroll") for (int e = 0; e < 8; ++e) { const float x_ = (float)sx[i][e]; ss[i] += ' + E.render(pro.stat_pre, {"x": "x_"}) + "; } \\")
             a("    __builtin_amdgcn_sched_barrier(0); }")
-        first_younger = min(depth - 1, KT - 1) * loads_per_slab
+        first_younger = min(depth - 1 - (1 if dli else 0), KT - 1) * loads_per_slab
         a(f"  EMH_SLAB_SYNC({first_younger});")
         a("  EMH_READ(0, 0, 0);")
         a("ROW_EPILOGUE_TABLES")
@@ -531,13 +549,65 @@ ROW_EPILOGUE_TABLES
                     a("    EMH_SUMSQ_ADD();")
             a("    }")
 
-        steady = max(0, KT - depth)
-        if steady:
-            a(f"  for (int kt = 0; kt < {steady}; ++kt) {{")
-            slab_steps("kt", None)
-            a("  }")
-        for kt_s in range(steady, KT):
-            slab_steps(str(kt_s), kt_s)
+        # ``dli``: the requests of slab kt + DEPTH - 1 are issued *between the MFMAs* of slab kt, into the buffer
+        # slab kt - 1 was read from (free since the barrier that ended it).  Issued as one burst behind the
+        # barrier, as ``dl`` does, every wave sits in the request queue at the same moment and the matrix pipe
+        # drains: load time and MFMA time add up instead of overlapping.
+        n_mma = NB * FM * FN
+        part_list = [("A", i) for i in range(A_PER_T)] + [("B", i) for i in range(B_PER_T)]
+        slot_of = [(q * KS * n_mma) // len(part_list) for q in range(len(part_list))]  # after which MFMA of the slab a request goes
+        n_pre = sum(1 for sl in slot_of if sl < (KS - 1) * n_mma)  # requests issued before the slab's closing barrier
+
+        def mma_with_parts(P: int, kk: int, kt: str | None) -> None:
+            idx = 0
+            for h in range(NB):
+                for i in range(FM):
+                    for j in range(FN):
+                        a(f"    acc[{h}][{i}][{j}] = {plan.atom.builtin}(fw[{P}][{h}][{j}], fx[{P}][{i}], acc[{h}][{i}][{j}], 0, 0, 0);")
+                        if kt is not None:
+                            for q, (which, pi) in enumerate(part_list):
+                                if slot_of[q] == kk * n_mma + idx:
+                                    a(f"    __builtin_amdgcn_sched_barrier(0); EMH_DPART_{which}(({kt}) + DEPTH - 1, (({kt}) + DEPTH - 1) % DEPTH, {pi}); __builtin_amdgcn_sched_barrier(0);")
+                        idx += 1
+            a("    __builtin_amdgcn_sched_barrier(0);")
+
+        def slab_steps_dli(kt: str, static_kt: int | None) -> None:
+            a(f"    {{ const int cur = ({kt}) % DEPTH;")
+            if deferred:
+                a("    EMH_SUMSQ_READ(cur);")
+            issuing = static_kt is None
+            for kk in range(KS):
+                P = kk & 1
+                if kk + 1 < KS:
+                    a(f"    EMH_READ({P ^ 1}, cur, {kk + 1});")
+                elif static_kt is None:
+                    # outstanding and younger than slab kt + 1: the whole slabs kt + 2 .. kt + DEPTH - 2 and what has been requested of slab kt + DEPTH - 1
+                    a(f"    EMH_SLAB_SYNC({(depth - 3) * loads_per_slab + n_pre});")
+                    a(f"    EMH_READ({P ^ 1}, (({kt}) + 1) % DEPTH, 0);")
+                elif static_kt + 1 < KT:
+                    a(f"    EMH_SLAB_SYNC({max(0, KT - 2 - static_kt) * loads_per_slab});")
+                    a(f"    EMH_READ({P ^ 1}, {(static_kt + 1) % depth}, 0);")
+                mma_with_parts(P, kk, kt if issuing else None)
+                if deferred and kk == 0:
+                    a("    EMH_SUMSQ_ADD();")
+            a("    }")
+
+        if dli:
+            steady = max(0, KT - depth + 1)
+            if steady:
+                a(f"  for (int kt = 0; kt < {steady}; ++kt) {{")
+                slab_steps_dli("kt", None)
+                a("  }")
+            for kt_s in range(steady, KT):
+                slab_steps_dli(str(kt_s), kt_s)
+        else:
+            steady = max(0, KT - depth)
+            if steady:
+                a(f"  for (int kt = 0; kt < {steady}; ++kt) {{")
+                slab_steps("kt", None)
+                a("  }")
+            for kt_s in range(steady, KT):
+                slab_steps(str(kt_s), kt_s)
 
     # ---- epilogue ------------------------------------------------------------------
     esz = body.out_dtype.nbytes

@@ -33,7 +33,8 @@ DMA = r"""
 // assembly on purpose: for the builtin the compiler assumes any later LDS read may
 // alias the load's LDS write and drains every outstanding load (vmcnt(0)) before
 // it, which turns a ring of slabs into one slab in flight.  The caller orders
-// reads after loads itself (vmcnt wait, LDS fence read, barrier).
+// reads after loads itself (vmcnt wait, LDS fence read, barrier).  M0 is named as
+// clobbered so the compiler never keeps a value of its own in it across the load.
 EMH_DEV unsigned emh_lds_addr(const void* p) { return (unsigned)(unsigned long)(__attribute__((address_space(3))) const void*)p; }
 // Publishing direct-to-LDS data to the other waves: the counter that tracks the
 // loads can reach its target before the LDS writes are visible.  A flat load from
@@ -46,7 +47,12 @@ EMH_DEV void emh_lds_publish(const void* lds_generic) {
 }
 EMH_DEV void emh_dma16(const void* g, const void* lds_wave_base) {
   const unsigned m0_ = __builtin_amdgcn_readfirstlane(emh_lds_addr(lds_wave_base));
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(g), "s"(m0_) : "memory");
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(g), "s"(m0_) : "memory", "m0");
+}
+// The same load with its address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit
+// per-lane byte offset: a loop that walks the base needs no vector arithmetic per request.
+EMH_DEV void emh_dma16s(const void* sbase, unsigned voff, unsigned lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(voff), "s"(sbase), "s"(lds_wave_base) : "memory", "m0");
 }
 """
 

@@ -223,7 +223,7 @@ class TilePlan:
 # STAGE
 # --------------------------------------------------------------------------
 
-_TRANSPORTS = {"sync": "sync", "dl": "dl", "cp": "dl", "mix": "mix", "ks": "ks"}
+_TRANSPORTS = {"sync": "sync", "dl": "dl", "dli": "dli", "cp": "dl", "mix": "mix", "ks": "ks"}
 
 
 @dataclass(frozen=True)
@@ -234,6 +234,8 @@ class Stage:
     ``transport``  ``sync``: global → registers → ``ds_write`` (software
                    pipelined through ``reg_depth`` register sets);
                    ``dl``: global loads that write LDS directly, no VGPR hop;
+                   ``dli``: the same loads, issued one at a time between the MFMAs of
+                   the slab before instead of as a burst behind its barrier;
                    ``mix``: the a operand as ``sync``, the b operand as ``dl``;
                    ``ks``: no LDS staging — at most 16 rows, the reduction axis split
                    over ``depth`` waves that load their fragments straight from global

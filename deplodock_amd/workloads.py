@@ -93,9 +93,10 @@ class Qwen3Block(nn.Module):
         return out[0] if isinstance(out, tuple) else out
 
 
-def qwen3_block_case(seq: int = 512, seed: int = 0, dtype=torch.bfloat16) -> Case:
+def qwen3_block_case(seq: int = 512, seed: int = 0, dtype=torch.bfloat16, norm_std: float = 0.0) -> Case:
     """C5: one Qwen3-0.6B-architecture decoder block, weights ~N(0, 0.02), norm
-    weights 1, x ~N(0,1), positions 0..seq-1, RoPE theta 1e6."""
+    weights 1 (``norm_std`` > 0: ~N(1, norm_std), so a norm weight paired with the
+    wrong column shows), x ~N(0,1), positions 0..seq-1, RoPE theta 1e6."""
     from transformers import Qwen3Config
     from transformers.models.qwen3.modeling_qwen3 import Qwen3DecoderLayer, Qwen3RotaryEmbedding
 
@@ -110,6 +111,8 @@ def qwen3_block_case(seq: int = 512, seed: int = 0, dtype=torch.bfloat16) -> Cas
         for name, p in layer.named_parameters():
             if "norm" in name:
                 p.fill_(1.0)
+                if norm_std:
+                    p.add_(norm_std * torch.randn_like(p))
             else:
                 p.copy_(0.02 * torch.randn_like(p))
     x = torch.randn(1, seq, 1024)
@@ -118,7 +121,7 @@ def qwen3_block_case(seq: int = 512, seed: int = 0, dtype=torch.bfloat16) -> Cas
     flops = 2 * seq * h * (hq * d + 2 * hkv * d) + 2 * seq * hq * d * h + 3 * 2 * seq * h * inter + 4 * hq * d * (seq * (seq + 1) // 2)
     wbytes = (h * (hq * d + 2 * hkv * d) + hq * d * h + 3 * h * inter) * 2
     return Case(
-        f"qwen3_block_s{seq}", Qwen3Block(layer).to(dtype).eval(), (x.to(dtype), cos.to(dtype), sin.to(dtype)),
+        f"qwen3_block_s{seq}" + (f"_nw{norm_std}" if norm_std else ""), Qwen3Block(layer).to(dtype).eval(), (x.to(dtype), cos.to(dtype), sin.to(dtype)),
         BF16_RTOL if dtype is torch.bfloat16 else 1e-4, 4e-2 if dtype is torch.bfloat16 else 1e-4, algo_bytes=wbytes, algo_flops=flops,
     )  # fmt: skip
 

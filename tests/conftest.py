@@ -16,6 +16,10 @@ if str(ROOT) not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a HIP device (run on an MI355X box)")
+    # The benchmark worker's fork server must be a process that never touched the GPU: start it before any test does.
+    from deplodock_amd.backend.hip.bench_worker import start_server
+
+    start_server()
 
 
 @pytest.fixture(scope="session")

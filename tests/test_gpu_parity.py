@@ -202,10 +202,22 @@ def test_c4_sdpa_full_size(device):
     q, k, v = (t.to(device).float() for t in case.inputs)
     exact = nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
     eager.assert_close(ours, exact, case.rtol, case.atol, "sdpa vs fp32 eager")
+    # Scale-aware: at S=2048 a late row is an average over ~2000 values and is only ~0.03 large, so the absolute
+    # floor above is most of the value.  Per row, relative L2 error against the fp32 run, bounded by 1.5 x what
+    # bf16 eager shows on the same inputs (worst row and mean).
+    eager.assert_rows_within_baseline(ours, want, exact, 1.5, "sdpa S=2048 rows vs fp32 eager")
     # size-independent property: attention rows sum to one, so V = 1 gives O = 1
     ones = eager.Case("ones", case.module, (case.inputs[0], case.inputs[1], torch.ones_like(case.inputs[2])), 2e-2, 2e-2)
     o1, _, _ = run_case(ones, device)
     assert float((o1.float() - 1).abs().max()) <= 2 ** -7
+    # V[j, :] = j / S: the output is each query's weighted mean key position; a key block that is skipped (it
+    # drops out of numerator and denominator alike, which V = 1 cannot see) or fetched from the wrong place
+    # shifts the row.  Same criterion, against fp32 eager on the same (bf16-valued) operands.
+    vpos = eager.position_coded_values(case.inputs[2])
+    coded = eager.Case("pos", case.module, (case.inputs[0], case.inputs[1], vpos), 2e-2, 2e-2)
+    op, wp, _ = run_case(coded, device)
+    exact_p = nn.functional.scaled_dot_product_attention(q, k, vpos.to(device).float(), is_causal=True, enable_gqa=True)
+    eager.assert_rows_within_baseline(op, wp, exact_p, 1.5, "sdpa S=2048 position-coded V vs fp32 eager")
 
 
 @pytest.mark.parametrize("causal", [True, False])
@@ -318,10 +330,32 @@ def test_c5_qwen3_block(device, seq, golden):
     ours, want, compiled = run_case(case, device)
     eager.assert_close(ours, want, case.rtol, case.atol, f"block S={seq} vs eager (GPU)")
     assert sum(isinstance(n.op, HipOp) for n in compiled.nodes.values()) == 5
+    # Scale-aware: the block's own contribution out - x has std ~0.3 and bf16 eager sits ~0.003 (mean) from the
+    # fp32 run, so the absolute floor above is loose.  On out - x: our mean distance from fp32 eager may be at
+    # most 1.5 x bf16 eager's, and no row may be further (relative L2) than 1.5 x bf16 eager's worst row.
+    exact = eager.run_eager_fp32(case, device)
+    x = case.inputs[0].to(device).float()
+    eager.assert_mean_error_within_baseline(ours.float() - x, want.float() - x, exact - x, 1.5, f"block S={seq} (out - x) vs fp32 eager")
+    eager.assert_rows_within_baseline(ours.float() - x, want.float() - x, exact - x, 1.5, f"block S={seq} rows of (out - x) vs fp32 eager")
     if seq == 32:
         gold = torch.from_numpy(golden["c5_y_bits"].view(np.int16).copy()).view(torch.bfloat16).float()
         eager.assert_close(ours, gold.reshape(ours.shape), case.rtol, case.atol, "block golden (CPU eager bf16)")
         eager.assert_close(ours, torch.from_numpy(golden["c5_y_f32"]).reshape(ours.shape), 2e-2, 6e-2, "block vs fp32 eager")
+        xc = case.inputs[0].float().reshape(ours.shape)
+        eager.assert_mean_error_within_baseline(ours.float().cpu() - xc, gold.reshape(ours.shape) - xc, torch.from_numpy(golden["c5_y_f32"]).reshape(ours.shape) - xc, 1.5, "block golden (out - x) vs fp32 eager")
+
+
+@pytest.mark.parametrize("seq", [512, 40])
+def test_c5_qwen3_block_with_random_norm_weights(device, seq):
+    """Layer-norm and head-norm weights ~N(1, 0.1) instead of ones: the fold of a norm weight into the stacked
+    projection weights and the pairing of head-norm weights with columns carry real values."""
+    case = eager.qwen3_block_case(seq=seq, norm_std=0.1, seed=3)
+    ours, want, _ = run_case(case, device)
+    eager.assert_close(ours, want, case.rtol, case.atol, f"block S={seq} random norm weights vs eager (GPU)")
+    exact = eager.run_eager_fp32(case, device)
+    x = case.inputs[0].to(device).float()
+    eager.assert_mean_error_within_baseline(ours.float() - x, want.float() - x, exact - x, 1.5, f"block S={seq} random norm weights (out - x) vs fp32 eager")
+    eager.assert_rows_within_baseline(ours.float() - x, want.float() - x, exact - x, 1.5, f"block S={seq} random norm weights rows vs fp32 eager")
 
 
 def test_run_api_returns_host_arrays_with_bf16_as_bits(device):

@@ -99,8 +99,42 @@ def test_watchdog_raises_instead_of_stalling(device, monkeypatch):
             prog.iter_once([64])
     finally:
         monkeypatch.undo()
-        prog.close()  # drains the stream: every wave exits normally
-    torch.cuda.synchronize()
+        assert prog._hung
+        prog.close()  # after the watchdog has fired close() must not wait on the stream (a real hang would never return)
+        assert prog._stream is None
+    torch.cuda.synchronize()  # the kernels here are healthy: every wave exits normally
+
+
+def test_isolated_benchmark_worker_is_killed_at_the_wall_limit_and_replaced(device):
+    """``bench_wall_timeout_s``: the benchmark runs in a worker process forked from a clean server; a limit
+    shorter than a healthy (but very long) run gets the worker killed and reported as a failed benchmark,
+    the next benchmark gets a fresh worker, and this process's own device state is untouched."""
+    case = eager.softmax_case(shape=(4096, 2048))
+    be = HipBackend(bench_wall_timeout_s=170.0)
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    data = {compiled.inputs[0]: case.inputs[0].to(device)}
+    try:
+        res = be.benchmark(compiled, warmup=2, num_iters=5, input_data=data)
+        assert res.num_launches == 1 and res.time_ms > 0 and res.captured
+        assert be._worker.spawned == 1 and be._worker.killed == 0
+        again = asyncio.run(be.benchmark_async(compiled, warmup=2, num_iters=5))  # same (kept) worker through the async entry point
+        assert again.time_ms > 0 and be._worker.spawned == 1
+        be.bench_wall_timeout_s = 0.5
+        be.bench_run_timeout_s = 3600.0
+        with pytest.raises(RuntimeError, match="wall budget"):
+            be.benchmark(compiled, warmup=2, num_iters=50_000_000)  # healthy kernels, far more windows than fit the limit
+        assert be._worker.killed == 1
+        be.bench_wall_timeout_s, be.bench_run_timeout_s = 170.0, 10.0
+        fresh = be.benchmark(compiled, warmup=2, num_iters=5)
+        assert fresh.time_ms > 0 and be._worker.spawned == 2
+        # an in-worker failure (run budget) comes back as the same RuntimeError the in-process path raises
+        be.bench_run_timeout_s = 1e-9
+        with pytest.raises(RuntimeError, match="bench_fail"):
+            be.benchmark(compiled, warmup=1, num_iters=3)
+    finally:
+        be.close()
+    ours, want = (lambda p: (p.run(), torch.cuda.synchronize(), p.output_tensors()[compiled.outputs[0]].clone(), p.close())[2])(HipBackend().program(compiled, data)), eager.run_eager(case, device)
+    eager.assert_close(ours.reshape(want.shape), want, case.rtol, case.atol, "in-process run after worker kills")
 
 
 def test_run_budget_marks_bench_fail(device):

@@ -5,6 +5,7 @@ from __future__ import annotations
 import numpy as np
 import pytest
 import torch
+from torch import nn
 
 from oracle import eager
 from oracle import emmy_ops as O
@@ -192,3 +193,74 @@ def test_deferred_rms_norm_identity():
     r = 1.0 / np.sqrt((x * x).mean(-1, keepdims=True) + eps)
     deferred = r * O.linear(x, big_w * w[None, :])
     np.testing.assert_allclose(deferred, direct, rtol=1e-5, atol=1e-6)
+
+
+# -- the scale-aware parity criteria themselves ----------------------------------------------------
+
+
+def _attention_with_dropped_block(q, k, v, row_from: int, key0: int, key1: int):
+    """fp32 causal attention in which rows >= ``row_from`` never see keys [key0, key1): what a flash loop
+    that skips one key block for late rows computes (the block is missing from numerator and denominator)."""
+    s = q.shape[-2]
+    mask = torch.ones(s, s, dtype=torch.bool).tril()
+    mask[row_from:, key0:key1] = False
+    return nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+
+
+def test_row_relative_criterion_sees_a_dropped_key_block():
+    """At S=2048 a late row's output is ~0.03 large, so the elementwise bound (rtol 2e-2 + atol 2e-2) hardly
+    sees an output with a whole 32-key block missing from its late rows: with random V it leaves 99 % of the
+    affected elements inside (only rows where the block held a dominant key stick out), and with
+    position-coded V it accepts the result outright.  The row-relative criterion against fp32 eager rejects
+    both, every affected row by a wide margin; V = 1 cannot see the omission at all (rows still sum to one)."""
+    torch.manual_seed(0)
+    s, d, row_from = 2048, 128, 1024
+    q, k, v = (torch.randn(1, 2, s, d).bfloat16() for _ in range(3))
+    qf, kf, vf = q.float(), k.float(), v.float()
+    exact = nn.functional.scaled_dot_product_attention(qf, kf, vf, is_causal=True)
+    bf16_eager = nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+    wrong = _attention_with_dropped_block(qf, kf, vf, row_from=row_from, key0=256, key1=288).bfloat16()
+    outside = (wrong.float() - exact).abs() > 2e-2 + 2e-2 * exact.abs()
+    assert float(outside[:, :, row_from:].float().mean()) < 0.02  # the loose bound passes 98 % of what is wrong
+    eager.assert_rows_within_baseline(bf16_eager, bf16_eager, exact, 1.5, "bf16 eager against itself")
+    with pytest.raises(AssertionError, match="row-relative L2"):
+        eager.assert_rows_within_baseline(wrong, bf16_eager, exact, 1.5, "dropped block")
+    limit = 1.5 * float(eager.row_rel_l2(bf16_eager, exact).max())
+    assert bool((eager.row_rel_l2(wrong, exact)[:, :, row_from:] > 5 * limit).all())  # every affected row, 5x over
+    # the same omission under V = 1 is invisible, under position-coded V it is not
+    ones = torch.ones_like(vf)
+    assert float((_attention_with_dropped_block(qf, kf, ones, row_from, 256, 288) - 1).abs().max()) < 1e-5
+    vpos = eager.position_coded_values(v)
+    np.testing.assert_array_equal(vpos[0, 0, :, 0].float().numpy(), (torch.arange(s) / s).bfloat16().float().numpy())
+    exact_p = nn.functional.scaled_dot_product_attention(qf, kf, vpos.float(), is_causal=True)
+    eager_p = nn.functional.scaled_dot_product_attention(q, k, vpos, is_causal=True)
+    wrong_p = _attention_with_dropped_block(qf, kf, vpos.float(), row_from, 256, 288).bfloat16()
+    eager.assert_close(wrong_p, exact_p, 2e-2, 2e-2, "the loose bound accepts the wrong result")  # does not raise
+    eager.assert_rows_within_baseline(eager_p, eager_p, exact_p, 1.5, "bf16 eager against itself, coded V")
+    with pytest.raises(AssertionError, match="row-relative L2"):
+        eager.assert_rows_within_baseline(wrong_p, eager_p, exact_p, 1.5, "dropped block, coded V")
+    limit_p = 1.5 * float(eager.row_rel_l2(eager_p, exact_p).max())
+    assert float((eager.row_rel_l2(wrong_p, exact_p)[:, :, row_from:] > limit_p).float().mean()) > 0.95
+
+
+def test_mean_error_criterion_sees_a_wrong_norm_weight_pairing():
+    """The block criterion: on out - x, our mean distance from the fp32 run may be at most 1.5 x bf16
+    eager's.  A block whose post-attention norm weights are applied to the wrong columns (rolled by one)
+    passes the elementwise bound atol 4e-2 on most elements and fails this one."""
+    c = eager.qwen3_block_case(seq=64, norm_std=0.1, seed=3)
+    exact = eager.run_eager_fp32(c)
+    bf16 = eager.run_eager(c).float()
+    x = c.inputs[0].float()
+    eager.assert_mean_error_within_baseline(bf16 - x, bf16 - x, exact - x, 1.5, "bf16 eager against itself")
+    import copy
+
+    broken = copy.deepcopy(c)
+    with torch.no_grad():
+        w = broken.module.l.post_attention_layernorm.weight
+        w.copy_(torch.roll(w, 1))
+    wrong = eager.run_eager(broken).float()
+    assert float(((wrong - bf16).abs() <= 4e-2 + 2e-2 * bf16.abs()).float().mean()) > 0.5  # the loose bound passes most of it
+    with pytest.raises(AssertionError, match="exceeds"):
+        eager.assert_mean_error_within_baseline(wrong - x, bf16 - x, exact - x, 1.5, "rolled norm weights")
+    with pytest.raises(AssertionError, match="row-relative L2"):
+        eager.assert_rows_within_baseline(wrong - x, bf16 - x, exact - x, 1.5, "rolled norm weights")

@@ -64,3 +64,39 @@ def test_no_device_means_a_loud_error_not_a_fallback():
 
     with pytest.raises(LauncherError, match="no CPU fallback"):
         program._device()
+
+
+def test_bench_worker_kills_at_the_wall_limit_reports_child_errors_and_respawns():
+    """Host-side behaviour of the isolated benchmark worker (no GPU involved): a request that is not
+    answered in time gets the child killed and a ``RuntimeError``; an exception inside the child comes
+    back as ``RuntimeError`` with its text and the child is replaced before the next job."""
+    from deplodock_amd.backend.hip.bench_worker import BenchWorker
+
+    w = BenchWorker()
+    try:
+        with pytest.raises(RuntimeError, match="wall budget"):
+            w.run_job({"graph": None, "input_data": {}, "kwargs": {}}, wall_timeout_s=0.0)
+        assert (w.spawned, w.killed) == (1, 1) and w._proc is None
+        with pytest.raises(RuntimeError, match="bench worker error: .*topological_order"):
+            w.run_job({"graph": "not a graph", "input_data": {}, "kwargs": {}}, wall_timeout_s=120.0)
+        assert w.spawned == 2
+        with pytest.raises(RuntimeError, match="bench worker error"):
+            w.run_job({"graph": "still not a graph", "input_data": {}, "kwargs": {}}, wall_timeout_s=120.0)
+        assert w.spawned == 3
+    finally:
+        w.close()
+
+
+def test_backend_routes_benchmarks_to_the_worker_only_with_a_wall_limit_and_no_callback(monkeypatch):
+    from deplodock_amd import HipBackend
+    from deplodock_amd.backend.hip import bench_worker, program
+
+    calls = []
+    monkeypatch.setattr(bench_worker, "benchmark_program_isolated", lambda g, **kw: calls.append(("worker", kw["wall_timeout_s"])) or "W")
+    monkeypatch.setattr(program, "benchmark_program", lambda g, **kw: calls.append(("inline", None)) or "I")
+    g = Graph()
+    assert HipBackend().benchmark(g) == "I"
+    be = HipBackend(bench_wall_timeout_s=7.0)
+    assert be.benchmark(g) == "W"
+    assert be.benchmark(g, on_iter=lambda n: None) == "I"  # a callback shares state with this process: in-process
+    assert calls == [("inline", None), ("worker", 7.0), ("inline", None)]
