@@ -14,20 +14,19 @@ import numpy as np
 
 @dataclass(frozen=True)
 class DType:
-    name: str  # "f32" | "bf16" | "f16" | "i32"
+    name: str  # "f32" | "bf16" | "f16" | "i32" — the canonical token a render target spells as a C type
     nbytes: int
-    c_name: str  # spelling in emitted HIP source
     np: np.dtype  # host carrier dtype
 
     def __repr__(self) -> str:
         return self.name
 
 
-F32 = DType("f32", 4, "float", np.dtype(np.float32))
-BF16 = DType("bf16", 2, "__bf16", np.dtype(np.uint16))
-F16 = DType("f16", 2, "_Float16", np.dtype(np.float16))
-I32 = DType("i32", 4, "int", np.dtype(np.int32))
-I64 = DType("i64", 8, "long long", np.dtype(np.int64))
+F32 = DType("f32", 4, np.dtype(np.float32))
+BF16 = DType("bf16", 2, np.dtype(np.uint16))
+F16 = DType("f16", 2, np.dtype(np.float16))
+I32 = DType("i32", 4, np.dtype(np.int32))
+I64 = DType("i64", 8, np.dtype(np.int64))
 
 _BY_NAME = {d.name: d for d in (F32, BF16, F16, I32, I64)}
 

@@ -30,14 +30,23 @@ from __future__ import annotations
 from deplodock_amd.context import Context
 from deplodock_amd.dtype import BF16, F16, F32
 from deplodock_amd.emit import prelude
+from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.ir.schedule import Stage
 from deplodock_amd.ir.tile import Contraction
 
-_FRAG_T = {"bf16": "bf16x8", "f16": "f16x8"}
-_PACK4_T = {"bf16": "bf16x4", "f16": "f16x4", "f32": "f32x4"}
+
+
+def _frag_t(dtype_name: str) -> str:
+    """The 16-byte MFMA operand fragment (eight 16-bit elements) of ``dtype_name``."""
+    return rt.vector_type(dtype_name, 8)[0]
+
+
+def _pack4_t(dtype_name: str) -> str:
+    """Four consecutive output elements, the run an accumulator group converts to."""
+    return rt.vector_type(dtype_name, 4)[0]
 
 
 def xcd_block(tiles_m: int, tiles_n: int, tile_m: int, tile_n: int, xcds: int) -> tuple[int, int]:
@@ -64,7 +73,7 @@ def _emit_row_epilogue_tables(a, re, re_args: list[str], EPC: int, m_guard: bool
     """Fetch, at kernel start, the table chunks the row epilogue of this thread will
     need (they depend on the output coordinates only): the k loop hides the latency."""
     d = re.cols
-    vt_chunk = {2: None, 4: "f32x4"}.get(16 // EPC) or ("bf16x8" if re.row_operands and re.row_operands[0].dtype.name == "bf16" else "f16x8")
+    vt_chunk = rt.vector_type(re.row_operands[0].dtype.name if re.row_operands else "bf16", EPC)[0]
     a(f"  constexpr int RE_IT = (TM * (TN / {EPC})) / T;")
     for nm, ro in zip(re_args, re.row_operands):
         a(f"  {vt_chunk} {nm}_v[RE_IT];")
@@ -76,7 +85,7 @@ def _emit_row_epilogue_tables(a, re, re_args: list[str], EPC: int, m_guard: bool
     mrow = "(m < M ? m : M - 1)" if m_guard else "m"
     a(f"      const long rr = (long){mrow} * {re.col_end // d} + n / {d};  // the row number a separate row kernel would use")
     for nm, ro in zip(re_args, re.row_operands):
-        a(f"      const {ro.dtype.c_name}* {nm}_row = {nm} + {ro.offset}L + ((rr / {ro.div}) % {ro.mod}) * {d};")
+        a(f"      const {rt.type_name(ro.dtype.name)}* {nm}_row = {nm} + {ro.offset}L + ((rr / {ro.div}) % {ro.mod}) * {d};")
         a(f"      {nm}_v[it] = *(const {vt_chunk}*)({nm}_row + gc);")
     a("    }")
     a("  }")
@@ -150,7 +159,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     plan = body.tile
     if plan is None:
         raise LoweringError("contraction: no TilePlan stamped")
-    if body.in_dtype.name not in _FRAG_T or plan.atom.dtype != body.in_dtype.name:
+    if body.in_dtype.name not in ("bf16", "f16") or plan.atom.dtype != body.in_dtype.name:
         raise LoweringError(f"contraction: atom {plan.atom.name} does not take {body.in_dtype} operands")
     stage = body.stage or Stage(depth=2, transport="sync")
     if stage.transport == "ks":
@@ -213,9 +222,9 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     if dl and (a_chunks % 64 or b_chunks % 64):
         raise LoweringError("contraction: direct-to-LDS staging needs whole-wave chunk counts")
 
-    frag_t = _FRAG_T[body.in_dtype.name]
-    in_c = body.in_dtype.c_name
-    out_c = body.out_dtype.c_name
+    frag_t = _frag_t(body.in_dtype.name)
+    in_c = rt.type_name(body.in_dtype.name)
+    out_c = rt.type_name(body.out_dtype.name)
     epi_names = [n for n, _ in body.epilogue_operands]
     epi = body.epilogue if body.epilogue is not None else E.Var("acc")
     allowed = {"acc"} | ({"acc2"} if gate else set()) | ({"bias"} if body.bias is not None else set())
@@ -241,16 +250,16 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
             raise LoweringError("contraction: a row's slab chunks must sit in one wave for the prologue's row sum")
     params = [f"const {in_c}* __restrict__ A", f"const {in_c}* __restrict__ B"]
     if pro is not None and pro.weight is not None:
-        params.append(f"const {pro.weight_dtype.c_name}* __restrict__ NW")
+        params.append(f"const {rt.type_name(pro.weight_dtype.name)}* __restrict__ NW")
     if body.bias is not None:
-        params.append(f"const {body.bias_dtype.c_name}* __restrict__ BIAS")
-    params += [f"const {dt.c_name}* __restrict__ e{i}" for i, (_, dt) in enumerate(body.epilogue_operands)]
+        params.append(f"const {rt.type_name(body.bias_dtype.name)}* __restrict__ BIAS")
+    params += [f"const {rt.type_name(dt.name)}* __restrict__ e{i}" for i, (_, dt) in enumerate(body.epilogue_operands)]
     rowepi = body.row_epilogue
     re_args = [f"re{i}" for i in range(len(rowepi.row_operands))] if rowepi is not None else []
     if rowepi is not None:
         if body.post is not None or gate or TN % rowepi.cols or rowepi.col_end % TN or rowepi.col_end > N:
             raise LoweringError("contraction: the row epilogue needs a plain result and output tiles of whole column groups")
-        params += [f"const {ro.dtype.c_name}* __restrict__ {nm}" for nm, ro in zip(re_args, rowepi.row_operands)]
+        params += [f"const {rt.type_name(ro.dtype.name)}* __restrict__ {nm}" for nm, ro in zip(re_args, rowepi.row_operands)]
     params.append(f"{out_c}* __restrict__ O")
 
     D = dict(
@@ -258,7 +267,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
         AM=AM, KG=KG, KSTEP=KSTEP, ACC=ACC, CPR=CPR, RPL=RPL, NB=NB, A_PER_T=A_PER_T, B_PER_T=B_PER_T,
         SLAB=slab_bytes, DEPTH=depth, RS=RS, KT=KT, TILES_M=tiles_m, TILES_N=tiles_n, NTILES=n_tiles, GM=gm, GN=gn,
         XCDS=ctx.xcds, frag_t=frag_t, in_c=in_c, out_c=out_c, params=", ".join(params), builtin=plan.atom.builtin,
-        acc_t="f32x16" if ACC == 16 else "f32x4", G=ACC // 4,
+        acc_t=rt.vector_type("f32", ACC)[0], G=ACC // 4,
     )  # fmt: skip
 
     o: list[str] = []
@@ -614,7 +623,7 @@ ROW_EPILOGUE_TABLES
     EPC = 16 // esz  # output elements per 16-byte chunk
     c_stride = TN * esz + 16
     staged = (N % EPC == 0) and (TN % EPC == 0) and (TM * c_stride <= ctx.lds_bytes_per_cu) and ((TM * (TN // EPC)) % T == 0)
-    vt4 = _PACK4_T[body.out_dtype.name]
+    vt4 = _pack4_t(body.out_dtype.name)
     cast = "" if body.out_dtype is F32 else f"({out_c})"
     post = body.post if body.post is not None else E.Var("y")
     unknown = E.variables(post) - ({"y"} | set(epi_names))
@@ -656,7 +665,7 @@ ROW_EPILOGUE_TABLES
     for (int g = 0; g < G; ++g) {
       const int nl = (wn * FN + j) * AM + g * 4 * KG + lk * 4;""")
         if body.bias is not None:
-            bt4 = _PACK4_T[body.bias_dtype.name]
+            bt4 = _pack4_t(body.bias_dtype.name)
             clamp = f"(n0 + nl < N ? n0 + nl : N - 4)" if n_guard else "(n0 + nl)"
             a(f"      const {bt4} bv = *(const {bt4}*)(BIAS + {clamp});")
         a(f"      {vt4} yo;")
@@ -672,7 +681,7 @@ ROW_EPILOGUE_TABLES
         a("    }")
         a("  }")
         a("  __syncthreads();")
-        vt_chunk = {("bf16"): "bf16x8", "f16": "f16x8", "f32": "f32x4"}[body.out_dtype.name]
+        vt_chunk = rt.vector_type(body.out_dtype.name, EPC)[0]
         a(f"  constexpr int CPRC = TN / {EPC};  // 16-byte chunks per output-tile row")
         if rowepi is not None:
             _emit_row_epilogue(a, body, rowepi, re_args, EPC, vt_chunk, out_c, m_guard, n_guard)
@@ -721,10 +730,10 @@ ROW_EPILOGUE_TABLES
         if n_guard:
             a("      if (n >= N) continue;  // N and tile widths are multiples of 4: a run is all in or all out")
         for i, (_, dt) in enumerate(body.epilogue_operands):
-            vt = _PACK4_T[dt.name]
+            vt = _pack4_t(dt.name)
             a(f"      const {vt} ev{i} = *(const {vt}*)(e{i} + (long)m * LDO + n);")
         if body.bias is not None:
-            bt4 = _PACK4_T[body.bias_dtype.name]
+            bt4 = _pack4_t(body.bias_dtype.name)
             a(f"      const {bt4} bv = *(const {bt4}*)(BIAS + n);")
         a(f"      {vt4} yo;")
         sc = " * rs_" if deferred else ""

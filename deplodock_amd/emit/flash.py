@@ -41,6 +41,7 @@ import math
 
 from deplodock_amd.context import Context
 from deplodock_amd.emit import prelude
+from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir.expr import float_literal
 from deplodock_amd.ir.hip import HipOp
@@ -480,13 +481,13 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "K_SB": body.k_strides[0], "K_SH": body.k_strides[1], "K_SS": body.k_strides[2], "K_OFF": body.k_offset,
         "V_SB": body.v_strides[0], "V_SH": body.v_strides[1], "V_SS": body.v_strides[2], "V_OFF": body.v_offset,
         "O_SB": body.o_strides[0], "O_SH": body.o_strides[1], "O_SS": body.o_strides[2], "O_OFF": body.o_offset,
-        "ELT": "__bf16" if bf16 else "_Float16",
-        "FRAG": "bf16x8" if bf16 else "f16x8",
-        "PACK4": "bf16x4" if bf16 else "f16x4",
+        "ELT": rt.type_name(body.dtype.name),
+        "FRAG": rt.vector_type(body.dtype.name, 8)[0],
+        "PACK4": rt.vector_type(body.dtype.name, 4)[0],
         "MFMA": "__builtin_amdgcn_mfma_f32_32x32x16_bf16" if bf16 else "__builtin_amdgcn_mfma_f32_32x32x16_f16",
         # 2^x straight on the transcendental unit; inputs are <= 0 and the result
         # feeds a 16-bit operand, so the fast form loses nothing that survives.
-        "EXP2": "__builtin_amdgcn_exp2f",
+        "EXP2": rt.intrinsic("fast_exp2", "f32"),
         # log2-domain slack before the accumulators are rescaled to a new maximum:
         # probabilities stay below 2^8, far inside fp32 / bf16 range.
         "RESCALE_SLACK": "8.0f",

@@ -10,6 +10,7 @@ from __future__ import annotations
 
 from deplodock_amd.context import Context
 from deplodock_amd.emit import prelude
+from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.emit.reduce import _load_vec, _store_vec
 from deplodock_amd.ir import expr as E
@@ -32,8 +33,8 @@ def emit_map(body: Map, name: str, ctx: Context = Context()) -> HipOp:
         V //= 2
     chunks = body.numel // V
     grid = max(1, -(-chunks // _T))
-    params = [f"const {o.dtype.c_name}* __restrict__ p{i}" for i, o in enumerate(body.operands)]
-    params.append(f"{body.out_dtype.c_name}* __restrict__ out")
+    params = [f"const {rt.type_name(o.dtype.name)}* __restrict__ p{i}" for i, o in enumerate(body.operands)]
+    params.append(f"{rt.type_name(body.out_dtype.name)}* __restrict__ out")
     o: list[str] = []
     a = o.append
     a(f"// {name}: numel={body.numel} vec={V}")

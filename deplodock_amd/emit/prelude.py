@@ -23,7 +23,6 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
 #define EMH_DEV __device__ __forceinline__
-EMH_DEV float emh_round_bf16(float v) { return (float)(__bf16)v; }
 """
 
 # Direct-to-LDS loads and their publication; only the emitters that stage through LDS include it.

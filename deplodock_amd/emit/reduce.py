@@ -23,6 +23,7 @@ from __future__ import annotations
 from deplodock_amd.context import Context
 from deplodock_amd.dtype import BF16, F16, F32, DType
 from deplodock_amd.emit import prelude
+from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
@@ -30,19 +31,12 @@ from deplodock_amd.ir.tile import RowAddr, RowReduce
 
 _MAX_RESIDENT = 64  # fp32 row elements a lane may keep in registers
 
-_VEC_T = {
-    ("f32", 4): "f32x4",
-    ("f32", 2): "f32x2",
-    ("f32", 1): "float",
-    ("bf16", 8): "bf16x8",
-    ("bf16", 4): "bf16x4",
-    ("bf16", 2): "bf16x2",
-    ("bf16", 1): "__bf16",
-    ("f16", 8): "f16x8",
-    ("f16", 4): "f16x4",
-    ("f16", 2): "f16x2",
-    ("f16", 1): "_Float16",
-}
+def _vec_t(dt: DType, v: int) -> str:
+    """C type of ``v`` elements of ``dt`` moved by one access."""
+    got = rt.vector_type(dt.name, v)
+    if got is None:
+        raise LoweringError(f"row kernel: no {v}-wide vector of {dt}")
+    return got[0]
 
 
 def pick_vec(cols: int, dtypes: list[DType], addrs: list[RowAddr]) -> int:
@@ -64,30 +58,27 @@ def _row_offset(addr: RowAddr, row: str) -> str:
 
 def _load_vec(ptr: str, idx: str, dt: DType, v: int, dst: str, nontemporal: bool) -> list[str]:
     """Lines that load ``v`` elements of ``dt`` at vector index ``idx`` into ``float dst[v]``."""
-    vt = _VEC_T[(dt.name, v)]
+    vt = _vec_t(dt, v)
     addr = f"((const {vt}*)({ptr}))[{idx}]" if v > 1 else f"({ptr})[{idx}]"
     if nontemporal:
         addr = f"__builtin_nontemporal_load(&{addr})"
     if v == 1:
-        return [f"{dst}[0] = (float){addr};"]
+        return [f"{dst}[0] = {rt.convert(addr, dt.name, 'f32')};"]
     lines = [f"{{ {vt} t_ = {addr};"]
-    if dt is F32:
-        lines += [f"  {dst}[{j}] = t_[{j}];" for j in range(v)]
-    else:
-        lines += [f"  {dst}[{j}] = (float)t_[{j}];" for j in range(v)]
+    lines += [f"  {dst}[{j}] = {rt.convert(f't_[{j}]', dt.name, 'f32')};" for j in range(v)]
     lines.append("}")
     return lines
 
 
 def _store_vec(ptr: str, idx: str, dt: DType, v: int, src: str, nontemporal: bool) -> list[str]:
-    vt = _VEC_T[(dt.name, v)]
-    cast = "" if dt is F32 else f"({dt.c_name})"
+    vt = _vec_t(dt, v)
+    cast = lambda x: rt.convert(x, "f32", dt.name)  # noqa: E731
     if v == 1:
         tgt = f"({ptr})[{idx}]"
-        val = f"{cast}{src}[0]"
+        val = cast(f"{src}[0]")
         return [f"__builtin_nontemporal_store({val}, &{tgt});" if nontemporal else f"{tgt} = {val};"]
     lines = [f"{{ {vt} t_;"]
-    lines += [f"  t_[{j}] = {cast}{src}[{j}];" for j in range(v)]
+    lines += [f"  t_[{j}] = {cast(f'{src}[{j}]')};" for j in range(v)]
     tgt = f"(({vt}*)({ptr}))[{idx}]"
     lines.append(f"  __builtin_nontemporal_store(t_, &{tgt});" if nontemporal else f"  {tgt} = t_;")
     lines.append("}")
@@ -151,10 +142,10 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
         if unknown:
             raise LoweringError(f"rotate-half expression uses unknown names {sorted(unknown)}")
 
-    params = [f"const {body.x_dtype.c_name}* __restrict__ x"]
-    params += [f"const {dt.c_name}* __restrict__ c{ci}" for ci, (_, dt) in enumerate(body.col_operands)]
-    params += [f"const {ro.dtype.c_name}* __restrict__ r{ri}" for ri, ro in enumerate(body.row_operands)]
-    params.append(f"{body.out_dtype.c_name}* __restrict__ out")
+    params = [f"const {rt.type_name(body.x_dtype.name)}* __restrict__ x"]
+    params += [f"const {rt.type_name(dt.name)}* __restrict__ c{ci}" for ci, (_, dt) in enumerate(body.col_operands)]
+    params += [f"const {rt.type_name(ro.dtype.name)}* __restrict__ r{ri}" for ri, ro in enumerate(body.row_operands)]
+    params.append(f"{rt.type_name(body.out_dtype.name)}* __restrict__ out")
 
     o: list[str] = []
     a = o.append
@@ -166,7 +157,7 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
     if row_guard:
         a(f"  const bool row_ok = row < {body.rows}L;")
         a(f"  if (!row_ok) row = {body.rows - 1}L;")
-    a(f"  const {body.x_dtype.c_name}* xr = x + ({_row_offset(x_addr, 'row')});")
+    a(f"  const {rt.type_name(body.x_dtype.name)}* xr = x + ({_row_offset(x_addr, 'row')});")
     a(f"  float xv[{NV}][{V}];")
     if masked:
         a(f"  bool ok[{NV}];")
@@ -186,7 +177,7 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
 
     if not body.scalar_out:
         for ri, ro in enumerate(body.row_operands):
-            a(f"  const {ro.dtype.c_name}* rrow{ri} = r{ri} + {ro.offset}L + ((row / {ro.div}) % {ro.mod}) * {body.cols}L;")
+            a(f"  const {rt.type_name(ro.dtype.name)}* rrow{ri} = r{ri} + {ro.offset}L + ((row / {ro.div}) % {ro.mod}) * {body.cols}L;")
 
     def operand_loads(i: int, indent: str, tag: str = "") -> None:
         idx = f"{i * L} + lane"
@@ -261,7 +252,7 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
         bad = E.variables(body.project) - set(stat_names)
         if bad or body.rotate is not None or body.col_operands or body.row_operands:
             raise LoweringError(f"row reduce: a one-value-per-row output maps the statistics only (got {sorted(bad)})")
-        cast_ = "" if body.out_dtype.name == "f32" else f"({body.out_dtype.c_name})"
+        cast_ = "" if body.out_dtype.name == "f32" else f"({rt.type_name(body.out_dtype.name)})"
         a(f"  if (lane == 0{' && row_ok' if row_guard else ''}) out[row] = {cast_}({E.render(body.project, env_base)});")
         a("}")
         return HipOp(
@@ -275,7 +266,7 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
             algo_bytes=body.algo_bytes(),
             knobs={"REDUCE": plan.spell(), "VEC": V, "NT": int(nontemporal)},
         )
-    a(f"  {body.out_dtype.c_name}* orow = out + ({_row_offset(out_addr, 'row')});")
+    a(f"  {rt.type_name(body.out_dtype.name)}* orow = out + ({_row_offset(out_addr, 'row')});")
 
     if row_guard:
         a("  if (row_ok) {")

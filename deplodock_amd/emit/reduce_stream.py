@@ -21,6 +21,7 @@ from __future__ import annotations
 
 from deplodock_amd.context import Context
 from deplodock_amd.emit import prelude
+from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.emit.reduce import _load_vec, _row_offset, _store_vec, pick_vec
 from deplodock_amd.ir import expr as E
@@ -79,9 +80,9 @@ def emit_row_reduce_streaming(body: RowReduce, name: str, ctx: Context = Context
         passes.append(group)
         i = j
 
-    params = [f"const {body.x_dtype.c_name}* __restrict__ x"]
-    params += [f"const {dt.c_name}* __restrict__ c{ci}" for ci, (_, dt) in enumerate(body.col_operands)]
-    params.append(f"{body.out_dtype.c_name}* __restrict__ out")
+    params = [f"const {rt.type_name(body.x_dtype.name)}* __restrict__ x"]
+    params += [f"const {rt.type_name(dt.name)}* __restrict__ c{ci}" for ci, (_, dt) in enumerate(body.col_operands)]
+    params.append(f"{rt.type_name(body.out_dtype.name)}* __restrict__ out")
     o: list[str] = []
     a = o.append
     a(f"// {name}: rows={body.rows} cols={body.cols} streamed by {T} lanes, vec={V}, {len(passes)} statistic pass(es)")
@@ -89,7 +90,7 @@ def emit_row_reduce_streaming(body: RowReduce, name: str, ctx: Context = Context
     a("  const int lane = threadIdx.x;")
     a(f"  const int wave = lane / {ctx.wave_size};")
     a("  const long row = blockIdx.x;")
-    a(f"  const {body.x_dtype.c_name}* xr = x + ({_row_offset(x_addr, 'row')});")
+    a(f"  const {rt.type_name(body.x_dtype.name)}* xr = x + ({_row_offset(x_addr, 'row')});")
     a(f"  __shared__ float emh_part[{NW}];")
     a("  float xv[%d];" % V)
 
@@ -144,10 +145,10 @@ def emit_row_reduce_streaming(body: RowReduce, name: str, ctx: Context = Context
             env_done[st.name] = f"s_{st.name}"
 
     if body.scalar_out:
-        cast = "" if body.out_dtype.name == "f32" else f"({body.out_dtype.c_name})"
+        cast = "" if body.out_dtype.name == "f32" else f"({rt.type_name(body.out_dtype.name)})"
         a(f"  if (lane == 0) out[{_row_offset(out_addr, 'row')}] = {cast}({E.render(body.project, env_done)});")
     else:
-        a(f"  {body.out_dtype.c_name}* orow = out + ({_row_offset(out_addr, 'row')});")
+        a(f"  {rt.type_name(body.out_dtype.name)}* orow = out + ({_row_offset(out_addr, 'row')});")
         a(f"  for (int c = lane; c < {C}; c += {T}) {{")
         o.extend("    " + ln for ln in _load_vec("xr", "c", body.x_dtype, V, "xv", False))
         for ci, (_, dt) in enumerate(body.col_operands):

@@ -25,13 +25,22 @@ from __future__ import annotations
 from deplodock_amd.context import Context
 from deplodock_amd.dtype import F32
 from deplodock_amd.emit import prelude
+from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.ir.tile import Contraction
 
-_FRAG_T = {"bf16": "bf16x8", "f16": "f16x8"}
-_PACK4_T = {"bf16": "bf16x4", "f16": "f16x4", "f32": "f32x4"}
+
+
+def _frag_t(dtype_name: str) -> str:
+    """The 16-byte MFMA operand fragment (eight 16-bit elements) of ``dtype_name``."""
+    return rt.vector_type(dtype_name, 8)[0]
+
+
+def _pack4_t(dtype_name: str) -> str:
+    """Four consecutive output elements, the run an accumulator group converts to."""
+    return rt.vector_type(dtype_name, 4)[0]
 _BUILTIN = {"bf16": "__builtin_amdgcn_mfma_f32_16x16x32_bf16", "f16": "__builtin_amdgcn_mfma_f32_16x16x32_f16"}
 
 #: MFMA steps whose fragments a wave requests in one go (2 x 4 registers each)
@@ -42,7 +51,7 @@ def skinny_waves(body: Contraction) -> int:
     """Waves that split the reduction axis (0: the shape does not take this form)."""
     if body.m > 16 or body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None or body.reduce.cta != 1:
         return 0
-    if body.in_dtype.name not in _FRAG_T or body.k % 32 or body.n % 4:
+    if body.in_dtype.name not in ("bf16", "f16") or body.k % 32 or body.n % 4:
         return 0
     for kw in (8, 4, 2, 1):
         if body.k % (32 * kw) == 0:
@@ -63,9 +72,9 @@ def emit_contraction_skinny(body: Contraction, name: str, ctx: Context = Context
     chunk = steps
     while chunk > MAX_STEPS_IN_FLIGHT:
         chunk = next(c for c in range(chunk - 1, 0, -1) if steps % c == 0)
-    frag_t = _FRAG_T[body.in_dtype.name]
-    in_c, out_c = body.in_dtype.c_name, body.out_dtype.c_name
-    vt4 = _PACK4_T[body.out_dtype.name]
+    frag_t = _frag_t(body.in_dtype.name)
+    in_c, out_c = rt.type_name(body.in_dtype.name), rt.type_name(body.out_dtype.name)
+    vt4 = _pack4_t(body.out_dtype.name)
     cast = "" if body.out_dtype is F32 else f"({out_c})"
     epi_names = [n for n, _ in body.epilogue_operands]
     epi = body.epilogue if body.epilogue is not None else E.Var("acc")
@@ -82,8 +91,8 @@ def emit_contraction_skinny(body: Contraction, name: str, ctx: Context = Context
 
     params = [f"const {in_c}* __restrict__ A", f"const {in_c}* __restrict__ B"]
     if body.bias is not None:
-        params.append(f"const {body.bias_dtype.c_name}* __restrict__ BIAS")
-    params += [f"const {dt.c_name}* __restrict__ e{i}" for i, (_, dt) in enumerate(body.epilogue_operands)]
+        params.append(f"const {rt.type_name(body.bias_dtype.name)}* __restrict__ BIAS")
+    params += [f"const {rt.type_name(dt.name)}* __restrict__ e{i}" for i, (_, dt) in enumerate(body.epilogue_operands)]
     params.append(f"{out_c}* __restrict__ O")
     T = 64 * KW
     o: list[str] = []
@@ -161,10 +170,10 @@ def emit_contraction_skinny(body: Contraction, name: str, ctx: Context = Context
     a("  const int m = lr, n = n0 + lk * 4;")
     a(f"  if (m >= {M} || n >= {N}) return;  // N is a multiple of 4: a run of four is all in or all out")
     for i, (_, dt) in enumerate(body.epilogue_operands):
-        vt = _PACK4_T[dt.name]
+        vt = _pack4_t(dt.name)
         a(f"  const {vt} ev{i} = *(const {vt}*)(e{i} + (long)m * {ldo} + n);")
     if body.bias is not None:
-        bt4 = _PACK4_T[body.bias_dtype.name]
+        bt4 = _pack4_t(body.bias_dtype.name)
         a(f"  const {bt4} bv = *(const {bt4}*)(BIAS + n);")
     a(f"  {vt4} yo;")
     for r in range(4):

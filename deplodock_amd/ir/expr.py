@@ -93,38 +93,53 @@ def float_literal(v: float) -> str:
     return f"{f.hex()}f"
 
 
-_UN_C = {
-    "neg": "(-({a}))",
-    "exp": "expf({a})",
-    "exp2": "exp2f({a})",
-    "fast_exp2": "__builtin_amdgcn_exp2f({a})",
-    "rsqrt": "rsqrtf({a})",
-    "sqrt": "sqrtf({a})",
-    "rcp": "(1.0f / ({a}))",
-    "abs": "fabsf({a})",
-    "tanh": "tanhf({a})",
-    # x * 1/(1+e^-x): the reference's SiLU decomposition
-    # (emmy/compiler/pipeline/passes/frontend/decomposition/020_silu.py).
-    "sigmoid": "(1.0f / (1.0f + expf(-({a}))))",
-    "silu": "(({a}) / (1.0f + expf(-({a}))))",
-}
-# A transcendental whose result is rounded to a 16-bit type straight away takes the
-# hardware approximations (v_exp_f32 / v_rcp_f32, a couple of fp32 ulps): nothing of the
-# difference survives the rounding, and the precise forms cost ~25 instructions per element.
-_UN_C_ROUNDED = {
-    "exp": "__expf({a})",
-    "sigmoid": "__fdividef(1.0f, 1.0f + __expf(-({a})))",
-    "silu": "__fdividef(({a}), 1.0f + __expf(-({a})))",
-}
-_BIN_C = {
-    "add": "(({a}) + ({b}))",
-    "sub": "(({a}) - ({b}))",
-    "mul": "(({a}) * ({b}))",
-    "div": "(({a}) / ({b}))",
-    "max": "fmaxf({a}, {b})",
-    "min": "fminf({a}, {b})",
-}
-_ROUND_C = {"bf16": "emh_round_bf16({a})", "f16": "((float)(_Float16)({a}))"}
+# Unary / binary ops as (template over {a}, {b}) built from the render target's intrinsic spellings:
+# this module decides the *shape* of an expression (what is a call, what an operator, where the
+# reference's SiLU decomposition x * 1/(1+e^-x) sits — emmy/compiler/pipeline/passes/frontend/
+# decomposition/020_silu.py), the target decides the names.
+def _call(op: str, *args: str) -> str:
+    from deplodock_amd.render_target import rt
+
+    return f"{rt.intrinsic(op, 'f32')}({', '.join(args)})"
+
+
+def _un_c(op: str, a: str, rounded: bool = False) -> str:
+    """fp32 text of unary ``op`` on ``a``.  ``rounded``: the result goes to a 16-bit type straight away,
+    so transcendentals take the hardware approximations (v_exp_f32 / v_rcp_f32, a couple of fp32 ulps):
+    nothing of the difference survives the rounding, and the precise forms cost ~25 instructions each."""
+    exp = (lambda x: _call("fast_exp", x)) if rounded else (lambda x: _call("exp", x))
+    div = (lambda x, y: _call("fast_div", x, y)) if rounded else (lambda x, y: f"(({x}) / ({y}))")
+    if op == "neg":
+        return f"(-({a}))"
+    if op == "exp":
+        return exp(a)
+    if op == "rcp":
+        return f"(1.0f / ({a}))"
+    if op == "sigmoid":
+        return div("1.0f", f"1.0f + {exp(f'-({a})')}") if rounded else f"(1.0f / (1.0f + {exp(f'-({a})')}))"
+    if op == "silu":
+        return div(f"({a})", f"1.0f + {exp(f'-({a})')}") if rounded else f"(({a}) / (1.0f + {exp(f'-({a})')}))"
+    if op in ("exp2", "fast_exp2", "rsqrt", "sqrt", "abs", "tanh"):
+        return _call(op, a)
+    raise KeyError(f"no rendering for unary op {op!r}")
+
+
+_ROUNDED_UN = ("exp", "sigmoid", "silu")
+_BIN_SYM = {"add": "+", "sub": "-", "mul": "*", "div": "/"}
+
+
+def _bin_c(op: str, a: str, b: str) -> str:
+    if op in _BIN_SYM:
+        return f"(({a}) {_BIN_SYM[op]} ({b}))"
+    if op in ("max", "min"):
+        return _call(op, a, b)
+    raise KeyError(f"no rendering for binary op {op!r}")
+
+
+def _round_c(dtype: str, a: str) -> str:
+    from deplodock_amd.render_target import rt
+
+    return rt.convert(rt.convert(a, "f32", dtype), dtype, "f32")
 
 
 def render(e: Expr, env: dict[str, str]) -> str:
@@ -134,13 +149,13 @@ def render(e: Expr, env: dict[str, str]) -> str:
     if isinstance(e, Const):
         return float_literal(e.value)
     if isinstance(e, Un):
-        return _UN_C[e.op].format(a=render(e.a, env))
+        return _un_c(e.op, render(e.a, env))
     if isinstance(e, Bin):
-        return _BIN_C[e.op].format(a=render(e.a, env), b=render(e.b, env))
+        return _bin_c(e.op, render(e.a, env), render(e.b, env))
     if isinstance(e, Round):
-        if isinstance(e.a, Un) and e.a.op in _UN_C_ROUNDED:
-            return _ROUND_C[e.dtype].format(a=_UN_C_ROUNDED[e.a.op].format(a=render(e.a.a, env)))
-        return _ROUND_C[e.dtype].format(a=render(e.a, env))
+        if isinstance(e.a, Un) and e.a.op in _ROUNDED_UN:
+            return _round_c(e.dtype, _un_c(e.a.op, render(e.a.a, env), rounded=True))
+        return _round_c(e.dtype, render(e.a, env))
     raise TypeError(f"cannot render {type(e).__name__}")
 
 

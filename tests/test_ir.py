@@ -61,7 +61,7 @@ def test_expr_render_and_evaluate_agree_on_rounding_points():
     want = (torch.tensor(1.5).bfloat16() * (t * torch.rsqrt((t * t).mean() + 1e-6)).bfloat16()).float().numpy()
     np.testing.assert_array_equal(got, want)
     text = E.render(e, {"x": "xv", "w": "wv", "ss": "acc"})
-    assert text.count("emh_round_bf16") == 2 and "rsqrtf" in text
+    assert text.count("((float)(((__bf16)(") == 2 and "rsqrtf" in text  # the render target's fp32 -> bf16 -> fp32 round trip
     assert E.variables(e) == {"x", "w", "ss"}
 
 
@@ -128,3 +128,63 @@ def test_knob_env_grammar(monkeypatch):
     monkeypatch.setenv("EMMY_KNOBS", "oops")
     with pytest.raises(ValueError):
         config.knobs_aggregate()
+
+
+# -- render target ----------------------------------------------------------------------------------
+
+
+def test_hip_render_target_implements_the_protocol_and_spells_gfx950_types():
+    from deplodock_amd.backend.hip.render_target import HipRenderTarget
+    from deplodock_amd.render_target import RenderTarget, current
+
+    t = HipRenderTarget()
+    assert isinstance(t, RenderTarget) and isinstance(current(), HipRenderTarget)
+    assert [t.type_name(d) for d in ("f32", "bf16", "f16", "i32")] == ["float", "__bf16", "_Float16", "int"]
+    assert t.literal("0.0f", "f32") == "0.0f" and t.literal("0.0f", "bf16") == "((__bf16)(0.0f))"
+    assert t.convert("v", "f32", "f32") == "v" and t.convert("v", "f32", "f16") == "((_Float16)(v))"
+    assert t.intrinsic("exp", "f32") == "expf" and t.intrinsic("fmax", "f32") == "fmaxf" and t.intrinsic("rsqrt", "f32") == "rsqrtf"
+    assert t.intrinsic("exp", "bf16") == "exp"  # no 16-bit forms: the renderer widens to fp32 and rounds back
+    assert t.has_native_op("exp", "f32") and t.has_native_op("add", "f32") and not t.has_native_op("add", "bf16")
+    assert t.vector_type("f32", 4) == ("f32x4", "float") and t.vector_type("bf16", 8) == ("bf16x8", "__bf16")
+    assert t.vector_type("f32", 1) == ("float", "float") and t.vector_type("bf16", 3) is None and t.vector_type("i32", 4) is None
+    with pytest.raises(KeyError):
+        t.type_name("f64")
+
+
+def test_emitters_take_their_spellings_from_the_installed_render_target():
+    """Another implementation of the protocol changes the emitted text without touching an emitter: every type,
+    vector, conversion and intrinsic spelling in a row kernel and a contraction comes from the target."""
+    from deplodock_amd import render_target
+    from deplodock_amd.backend.hip.render_target import HipRenderTarget
+    from deplodock_amd.dtype import BF16, F32
+    from deplodock_amd.emit.contraction import emit_contraction
+    from deplodock_amd.emit.reduce import emit_row_reduce
+    from deplodock_amd.ir.schedule import Stage, TilePlan
+    from deplodock_amd.ir.tile import Contraction, RowReduce, Stat
+
+    class Renamed(HipRenderTarget):
+        def type_name(self, dtype):
+            return {"f32": "my_f32", "bf16": "my_bf16"}.get(dtype, super().type_name(dtype))
+
+        def vector_type(self, dtype, n):
+            got = super().vector_type(dtype, n)
+            return None if got is None else ("my_" + got[0], self.type_name(dtype))
+
+        def intrinsic(self, op, dt):
+            return "my_" + super().intrinsic(op, dt)
+
+    x = E.Var("x")
+    row = RowReduce(rows=8, cols=256, x="X", x_dtype=F32, out="out", out_dtype=F32, stats=(Stat("ss", "sum", x * x),),
+                    project=x * E.Un("rsqrt", E.Var("ss") / 256.0 + 1e-6), reduce=ReducePlan(coop=64))  # fmt: skip
+    gemm = Contraction(m=64, n=64, k=64, a="x", b="w", out="y", in_dtype=BF16, out_dtype=BF16, tile=TilePlan.parse("a:mfma_16x16x32_bf16/w2x2/f2x2/k2"), stage=Stage.parse("d2/sync"))
+    plain = emit_row_reduce(row, "k_r").kernel_source, emit_contraction(gemm, "k_c").kernel_source
+    old = render_target.use(Renamed())
+    try:
+        renamed = emit_row_reduce(row, "k_r").kernel_source, emit_contraction(gemm, "k_c").kernel_source
+    finally:
+        render_target.use(old)
+    assert "const float* __restrict__ x" in plain[0] and "rsqrtf(" in plain[0] and "f32x4" in plain[0]
+    assert "const my_f32* __restrict__ x" in renamed[0] and "my_rsqrtf(" in renamed[0] and "my_f32x4" in renamed[0]
+    assert "const __bf16* __restrict__ A" in plain[1] and "bf16x8 fw[2]" in plain[1]
+    assert "const my_bf16* __restrict__ A" in renamed[1] and "my_bf16x8 fw[2]" in renamed[1] and "my_f32x4 acc" in renamed[1]
+    assert emit_row_reduce(row, "k_r").kernel_source == plain[0]  # and back
