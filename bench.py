@@ -14,14 +14,21 @@ JSON line printed carries:
                    per launch / average launch duration from HIP events recorded
                    on the launch stream around the same K launches;
 * ``cpu_baseline`` PyTorch eager of the same module on the host cores, over the
-                   whole workload (20 passes of tens of milliseconds each);
+                   whole workload (20 passes of tens of milliseconds each), with the
+                   host's core count, torch's thread count and the CPU model;
+* ``rooflines``    the dominant kernel of every configuration against the roofline
+                   that bounds it (HBM 8 TB/s or dense bf16 MFMA 2.5 PFLOP/s), same
+                   fields as ``roofline``: the MFMA kernels' fractions are part of
+                   the parsed record, not only of the table;
 * ``kernels``      the per-kernel table the metric asks for: µs, achieved GB/s or
                    TFLOP/s and fraction of peak for RMSNorm, softmax, linear
                    (M in 1/16/128/2048), causal GQA attention, and the Qwen3 block.
                    ``us`` replays one launch back to back (operands cache-resident
                    when they fit); the cache-sized configurations also carry
                    ``us_cold``: the same launch over rotating copies of its
-                   operands larger than the last-level cache.
+                   operands larger than the last-level cache.  ``cpu_us`` is PyTorch
+                   eager of the same module and inputs on the host cores (median of
+                   at least 3 passes, bounded to a few seconds per row).
 
 Every launch goes through ``libemmy_hip.so``; there is no fallback path.
 """
@@ -108,13 +115,28 @@ def _headline(device, steps: int, warmup: int) -> dict:
     }
 
 
+def _cpu_model() -> str:
+    try:
+        for line in Path("/proc/cpuinfo").read_text().splitlines():
+            if line.lower().startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _cpu_threads() -> int:
+    """Host threads the eager baseline runs on: the box gives one GPU's share of the host, 16 cores."""
+    return min(os.cpu_count() or 1, 16)
+
+
 def _cpu_baseline() -> dict:
     """PyTorch eager softmax of the whole workload on the host cores (a pass takes tens of milliseconds)."""
     import torch
 
     from oracle import eager
 
-    threads = min(os.cpu_count() or 1, 16)
+    threads = _cpu_threads()
     case = eager.softmax_case()
     sec = eager.time_eager_cpu(case, threads=threads, warmup=3, iters=20)
     return {
@@ -123,10 +145,25 @@ def _cpu_baseline() -> dict:
         "cores": threads,
         "kind": "port",
         "sample": f"PyTorch {torch.__version__} eager nn.Softmax(-1) on fp32 [1,28,2048,2048] (the whole workload), median of 20 passes after 3 warm-up passes, {threads} threads",
+        "os_cpu_count": os.cpu_count(),
+        "torch_num_threads": threads,
+        "torch_default_num_threads": torch.get_num_threads(),
+        "cpu_model": _cpu_model(),
     }
 
 
-def _table(device, only: str | None = None, extended: bool = False) -> list[dict]:
+def _cpu_us(case, budget_s: float = 4.0) -> float:
+    """µs per forward of PyTorch eager on the host cores: one warm-up pass, then passes until three are
+    timed and ``budget_s`` is used up (at most 20); the median."""
+    from oracle import eager
+
+    threads = _cpu_threads()
+    first = eager.time_eager_cpu(case, threads=threads, warmup=1, iters=1)
+    iters = max(3, min(20, int(budget_s / max(first, 1e-6))))
+    return eager.time_eager_cpu(case, threads=threads, warmup=0, iters=iters) * 1e6
+
+
+def _table(device, only: str | None = None, extended: bool = False, cpu: bool = True) -> list[dict]:
     """Per-kernel µs / achieved rate / fraction of peak for every configuration.
     Each kernel's output is compared with PyTorch eager on the device before it is timed
     (a wrong kernel's time means nothing); eager is never what is timed."""
@@ -213,6 +250,8 @@ def _table(device, only: str | None = None, extended: bool = False) -> list[dict
             row["cold_sets"] = sets
             if bound == "hbm":
                 row["achieved_cold"] = round(case.algo_bytes / (c_us * 1e-6) / 1e9, 1)
+        if cpu:
+            row["cpu_us"] = round(_cpu_us(case), 1)
         rows.append(row)
 
     bench(wl.rms_norm_case, "C1 rms_norm fp32 [1,32,2048]", "hbm", cold=True)
@@ -289,7 +328,14 @@ def main() -> int:
     }
     out["cpu_baseline"] = None if args.no_cpu else _cpu_baseline()
     if not args.no_table:
-        out["kernels"] = _table(device, args.only, args.extended)
+        out["kernels"] = _table(device, args.only, args.extended, cpu=not args.no_cpu)
+        # one roofline record per configuration, in the shape of `roofline` above (C1's 32 rows are launch-latency
+        # bound: its machine-filling variant C1x stands for the kernel; the decode-size linears are HBM bound)
+        peaks = {"hbm": (HBM_PEAK_GBPS, "GB/s"), "mfma": (MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")}
+        out["rooflines"] = [
+            {"config": r["config"], "bound": r["bound"], "achieved": r["achieved"], "peak": peaks[r["bound"]][0], "unit": peaks[r["bound"]][1], "frac": r["frac"], "kernel_us": r["us"]}
+            for r in out["kernels"]
+        ]
     print(json.dumps(out))
     return 0
 

@@ -39,6 +39,7 @@ _BATCH_TARGET_MS = 1.0  # launches per event window are sized to cover this
 _AUTO_BUDGET_MS = 100.0
 _AUTO_MAX_ITERS = 20000
 _SLAB_ALIGN = 256
+_E2E_MAX_COPIES = 64  # program copies one whole-program timing graph holds at most
 
 
 class HungKernelError(RuntimeError):
@@ -320,6 +321,7 @@ class CompiledProgram:
         self._launch_graphs: dict[int, int] = {}
         self._launch_graph_sizes: list[int] | None = None
         self._program_graph: int | None = None
+        self._program_graph_repeat = 1
         self._events: list[int] = []
         self._hung = False  # set by the watchdog: the private stream may never drain
         self._build_packs()
@@ -491,16 +493,24 @@ class CompiledProgram:
         self._launch_graphs = {}
         self._launch_graph_sizes = None
 
-    def capture_program_graph(self) -> None:
-        """One graph holding every launch in program order."""
-        if self._program_graph is not None:
+    def capture_program_graph(self, repeat: int = 1) -> None:
+        """One graph holding every launch in program order, ``repeat`` times back to back.  Timing windows use
+        ``repeat`` > 1 so that what they measure is device time: one graph launch per replay of a program of a
+        few short kernels would add the host's per-graph launch latency (several microseconds) to every replay,
+        which a caller that chains programs inside one graph — a model is many blocks — never pays."""
+        repeat = max(1, int(repeat))
+        if self._program_graph is not None and self._program_graph_repeat == repeat:
             return
+        if self._program_graph is not None:
+            self.lib.graph_destroy(self._program_graph)
+            self._program_graph = None
         stream = self._ensure_stream()
         self.lib.stream_synchronize(stream)
         try:
             self.lib.graph_begin_capture(stream)
             try:
-                self.run(stream)
+                for _ in range(repeat):
+                    self.run(stream)
             except BaseException:
                 with contextlib.suppress(launcher.LauncherError):
                     self.lib.graph_destroy(self.lib.graph_end_capture(stream))
@@ -508,15 +518,16 @@ class CompiledProgram:
             g = self.lib.graph_end_capture(stream)
         except launcher.LauncherError as exc:
             raise GraphCaptureError(f"whole-program graph capture failed: {exc}") from exc
-        self._program_graph = g
+        self._program_graph, self._program_graph_repeat = g, repeat
 
     def replay_program(self, stream: int | None = None) -> None:
-        if self._program_graph is None:
+        if self._program_graph is None or self._program_graph_repeat != 1:
             self.capture_program_graph()
         self.lib.graph_launch(self._program_graph, self._ensure_stream() if stream is None else stream)
 
     def time_program_window(self, replays: int) -> float:
-        """ms per whole-program replay over one event window of ``replays`` replays."""
+        """ms per whole-program run over one event window of ``replays`` launches of the program graph (each
+        holding the program ``repeat`` times)."""
         stream = self._ensure_stream()
         if not hasattr(self, "_win"):
             self._win = (self._event(), self._event())
@@ -526,7 +537,7 @@ class CompiledProgram:
             self.lib.graph_launch(self._program_graph, stream)
         self.lib.event_record(stop, stream)
         self._wait_for_event(stop, "whole-program graph")
-        return self._elapsed(start, stop, "whole-program graph") / replays
+        return self._elapsed(start, stop, "whole-program graph") / (replays * self._program_graph_repeat)
 
     def close(self) -> None:
         """Release graphs, events and the private stream.  The kernels' modules are shared through
@@ -676,18 +687,19 @@ def benchmark_program(
                 measured += 1
                 if measure_e2e and capture_graphs:
                     if e2e_replays == 0:
+                        it = sum(dts)
+                        e2e_replays = max(1, int(round(_BATCH_TARGET_MS / it))) if 0 < it < _BATCH_TARGET_MS else 1
                         try:
-                            prog.capture_program_graph()
+                            # the window's replays sit in one graph (up to 64 copies of the program): device time only
+                            prog.capture_program_graph(repeat=min(e2e_replays, _E2E_MAX_COPIES))
                         except GraphCaptureError as exc:
                             logger.warning("[hip] %s — skipping whole-program e2e timing", exc)
                             measure_e2e = False
-                        else:
-                            it = sum(dts)
-                            e2e_replays = max(1, int(round(_BATCH_TARGET_MS / it))) if 0 < it < _BATCH_TARGET_MS else 1
                     if measure_e2e:
-                        dt = prog.time_program_window(e2e_replays)
+                        launches = max(1, -(-e2e_replays // prog._program_graph_repeat))
+                        dt = prog.time_program_window(launches)
                         e2e_samples.append(dt)
-                        total_ms += dt * e2e_replays
+                        total_ms += dt * launches * prog._program_graph_repeat
                 if measured >= max_measured or (auto and cumulative_ms >= target_total_ms):
                     break
             return _samples_to_result(samples, prog.compiled.launches, captured=capture_graphs, e2e_samples=e2e_samples)

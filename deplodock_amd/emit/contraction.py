@@ -167,7 +167,13 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
 
         return emit_contraction_skinny(body, name, ctx)
     if body.reduce.cta != 1:
-        raise LoweringError("contraction: split-K is lowered by emit_contraction_splitk")
+        raise LoweringError("contraction: a cross-workgroup split (REDUCE=g<n>) is lowered as a partial kernel plus a combine (deplodock_amd.emit.splitk.lower_split_contraction), not by this emitter alone")
+    split = body.k_split
+    if split is not None:
+        if body.epilogue is not None or body.post is not None or body.bias is not None or body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None or body.out_dtype is not F32:
+            raise LoweringError("contraction: the partial kernel of a split stores bare fp32 accumulators; bias, epilogue and rounding belong to the combine")
+        if stage.transport not in ("sync", "dl", "dli"):
+            raise LoweringError(f"contraction: STAGE .../{stage.transport} does not combine with a cross-workgroup split")
     M, N, K = body.m, body.n, body.k
     lda = body.lda or K
     ldb = body.ldb or K
@@ -305,6 +311,12 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   const int wm = wave / WN, wn = wave % WN;
   const int lr = lane % AM, lk = lane / AM;  // fragment row, k-group
 """)
+    if split is not None:
+        a("  // cross-workgroup split of the reduction axis: workgroup row blockIdx.y owns slice blockIdx.y (K is the slice length)")
+        a("  const long KSL = (long)blockIdx.y * K;")
+        a("  const long OSL = " + ("(long)blockIdx.y * M * LDO;" if split[1] == "kernel" else "0;  // every slice adds into the one zeroed plane"))
+    else:
+        a("  constexpr long KSL = 0, OSL = 0;")
     # ---- staging ------------------------------------------------------------
     a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else "") + (" int ka[A_PER_T], kb[B_PER_T];" if k_guard else ""))
     a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
@@ -324,7 +336,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         a("    const int row = q / CPR, c = q % CPR;")
         a("    la[i] = row * (BK * 2) + emh_swz(row, c) * 16;")
     a(f"    int gr = m0 + row;{' if (gr > M - 1) gr = M - 1;' if m_guard else ''}")
-    a(f"    ga[i] = A + {body.a_offset}L + (long)gr * LDA + c * 8;")
+    a(f"    ga[i] = A + {body.a_offset}L + KSL + (long)gr * LDA + c * 8;")
     if dli:
         a("    va[i] = ((unsigned)gr * LDA + c * 8) * 2u;")
     if pro is not None:
@@ -347,7 +359,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
             a("    { const int lim = (row < TN) ? (N - 1) : (2 * N - 1); if (gr > lim) gr = lim; }")
     else:
         a(f"    int gr = n0 + row;{' if (gr > N - 1) gr = N - 1;' if n_guard else ''}")
-    a(f"    gb[i] = B + {body.b_offset}L + (long)gr * LDB + c * 8;")
+    a(f"    gb[i] = B + {body.b_offset}L + KSL + (long)gr * LDB + c * 8;")
     if dli:
         a("    vb[i] = ((unsigned)gr * LDB + c * 8) * 2u;")
     if k_guard:
@@ -511,8 +523,8 @@ ROW_EPILOGUE_TABLES
         if dli:
             a(f"""  // One request of slab kt into ring buffer buf: the operand base moves along k in scalar registers, the
   // lane's chunk offset is a loop-invariant 32-bit register, the LDS target a scalar: no vector arithmetic per request.
-  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L) + (long)(kt) * (BK * 2), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * T) * 16)
-  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L) + (long)(kt) * (BK * 2), vb[i], lds0 + (buf) * SLAB + TM * BK * 2 + (wave_u * 64 + (i) * T) * 16)""")
+  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L + KSL) + (long)(kt) * (BK * 2), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * T) * 16)
+  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L + KSL) + (long)(kt) * (BK * 2), vb[i], lds0 + (buf) * SLAB + TM * BK * 2 + (wave_u * 64 + (i) * T) * 16)""")
         if deferred:
             # the rows arrive in LDS untouched: every thread reads back the chunks it requested
             # (any chunk of the row will do for a row sum) while the slab is resident
@@ -707,7 +719,12 @@ ROW_EPILOGUE_TABLES
                 for i, (n_, _) in enumerate(body.epilogue_operands):
                     env[n_] = f"(float)ev{i}[{r}]"
                 a(f"      v[{r}] = {cast}({E.render(post, env)});")
-        a(f"      *({vt_chunk}*)(O + {body.out_offset}L + (long)m * LDO + n) = v;")
+        if split is not None and split[1] == "atomic":
+            a(f"      float* o_ = O + {body.out_offset}L + OSL + (long)m * LDO + n;")
+            a("      #pragma unroll")
+            a(f"      for (int r = 0; r < {EPC}; ++r) __builtin_amdgcn_global_atomic_fadd_f32((__attribute__((address_space(1))) float*)(o_ + r), v[r]);")
+        else:
+            a(f"      *({vt_chunk}*)(O + {body.out_offset}L + OSL + (long)m * LDO + n) = v;")
         a("    }")
         a("  }")
         if rowepi is not None:
@@ -750,7 +767,12 @@ ROW_EPILOGUE_TABLES
                     env2[n_] = f"(float)ev{i}[{r}]"
                 pre = E.render(post, env2)
             a(f"      yo[{r}] = {cast}({pre});")
-        a(f"      *({vt4}*)(O + {body.out_offset}L + (long)m * LDO + n) = yo;")
+        if split is not None and split[1] == "atomic":
+            a(f"      float* o_ = O + {body.out_offset}L + OSL + (long)m * LDO + n;")
+            a("      #pragma unroll")
+            a("      for (int r = 0; r < 4; ++r) __builtin_amdgcn_global_atomic_fadd_f32((__attribute__((address_space(1))) float*)(o_ + r), yo[r]);")
+        else:
+            a(f"      *({vt4}*)(O + {body.out_offset}L + OSL + (long)m * LDO + n) = yo;")
         a("    }")
         a("  }")
     a("}")
@@ -779,10 +801,11 @@ ROW_EPILOGUE_TABLES
             body.a, body.b, *((pro.weight,) if pro is not None and pro.weight is not None else ()), *((body.bias,) if body.bias is not None else ()),
             *(body.operand_buffers.get(n, n) for n in epi_names), *(rowepi.operand_buffers.get(ro.name, ro.name) for ro in (rowepi.row_operands if rowepi is not None else ())), body.out,
         ),  # fmt: skip
-        grid=((grid,), (1,), (1,)),
+        grid=((grid,), (split[0] if split is not None else 1,), (1,)),
         block=((T,), (1,), (1,)),
         lds_bytes=lds_bytes,
-        comment=f"contraction M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()}" + ((" a=row-scaled-after" if deferred else " a=row-normalised") if pro is not None else "") + (f" row-epilogue={rowepi.col_end // rowepi.cols}x{rowepi.cols}" if rowepi is not None else ""),
+        zero_outputs=(body.out,) if split is not None and split[1] == "atomic" else (),
+        comment=(f"partial of a {split[0]}-way split ({split[1]}) " if split is not None else "") + f"contraction M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()}" + ((" a=row-scaled-after" if deferred else " a=row-normalised") if pro is not None else "") + (f" row-epilogue={rowepi.col_end // rowepi.cols}x{rowepi.cols}" if rowepi is not None else ""),
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
         knobs={"TILE": plan.spell(), "STAGE": stage.spell()},

@@ -208,6 +208,11 @@ class Contraction:
     bias: str | None = None  # length-n vector the epilogue may name ``bias`` (added to the fp32 accumulator)
     bias_dtype: DType | None = None
     row_epilogue: RowEpilogue | None = None
+    # Set by the lowering on the *partial* kernel of a cross-workgroup split (``REDUCE=g<n>a|k``): ``(n, mode)``.
+    # ``k`` is then one slice of the reduction extent, workgroup ``blockIdx.y`` takes slice ``blockIdx.y`` of both
+    # operands, and the fp32 accumulators go to plane ``blockIdx.y`` of the workspace (``"kernel"``) or are added
+    # atomically into its single zeroed plane (``"atomic"``).
+    k_split: tuple[int, str] | None = None
 
     def algo_flops(self) -> int:
         return 2 * self.m * self.n * self.k * (2 if self.gate_pair else 1)

@@ -19,7 +19,10 @@ from deplodock_amd.emit.flash import emit_flash
 from deplodock_amd.emit.pointwise import emit_map
 from deplodock_amd.emit.reduce import emit_row_reduce
 from deplodock_amd.emit.reduce_stream import emit_row_reduce_streaming
-from deplodock_amd.graph import Graph
+from deplodock_amd.dtype import F32
+from deplodock_amd.emit.errors import LoweringError
+from deplodock_amd.emit.splitk import emit_splitk_combine, partial_body, split_planes
+from deplodock_amd.graph import Graph, Node, Tensor
 from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.ir.tile import Contraction, Flash, Map, RowReduce, TileOp
 
@@ -77,6 +80,30 @@ def _lower_contraction(op: TileOp, ctx: Context) -> HipOp:
     return hip
 
 
+def _lower_split_contraction(graph: Graph, node: Node, ctx: Context) -> None:
+    """``REDUCE=g<n>a|k`` on a contraction: the node becomes the combine kernel and gains a producer, the
+    partial kernel, whose output is the fp32 workspace (a scratch tensor of the graph) — the two-node form
+    of the reference's split rewrite (emmy/compiler/pipeline/passes/lowering/tile/030_split.py:135-334)."""
+    op: TileOp = node.op
+    body: Contraction = op.body
+    label, _, rest = op.name.partition("__")
+    ws_id = f"{node.id}__partial"
+    if ws_id in graph.nodes:
+        raise LoweringError(f"contraction: workspace id {ws_id!r} is taken")
+    part = partial_body(body, ws_id)
+    part_op = TileOp(name=f"{label}_partial__{rest}", body=part, knobs=dict(op.knobs))
+    part_hip = _named(emit_contraction(part, _PLACEHOLDER, ctx), part_op)
+    if _spills(part_hip, ctx):
+        raise LoweringError(f"{part_hip.kernel_name}: the partial kernel of the split spills vector registers; pin a smaller tile")
+    part_hip.knobs = {**part_hip.knobs, "REDUCE": body.reduce.spell()}
+    comb_op = TileOp(name=f"{label}_combine__{rest}", body=body, knobs=dict(op.knobs))
+    comb_hip = _named(emit_splitk_combine(body, ws_id, _PLACEHOLDER, ctx), comb_op)
+    comb_hip.knobs = {**part_hip.knobs}
+    graph.nodes[ws_id] = Node(ws_id, part_hip, [body.a, body.b], Tensor(ws_id, (split_planes(body), body.m, body.n), F32))
+    node.op = comb_hip
+    node.inputs = [ws_id, *node.inputs]
+
+
 def lower_tile(op: TileOp, ctx: Context) -> HipOp:
     body = op.body
     if isinstance(body, Contraction):
@@ -95,7 +122,10 @@ def lower_tile(op: TileOp, ctx: Context) -> HipOp:
 def lower(graph: Graph, ctx: Context | None = None) -> Graph:
     """Replace every ``TileOp`` by its ``HipOp`` (in place) and return the graph."""
     ctx = ctx or Context()
-    for node in graph.nodes.values():
+    for node in list(graph.nodes.values()):
         if isinstance(node.op, TileOp):
-            node.op = lower_tile(node.op, ctx)
+            if isinstance(node.op.body, Contraction) and node.op.body.reduce.cta > 1:
+                _lower_split_contraction(graph, node, ctx)
+            else:
+                node.op = lower_tile(node.op, ctx)
     return graph

@@ -79,8 +79,9 @@ def _tuned(body, ctx: Context) -> dict:
 
 
 def pick_coop(cols: int, elem_bytes: int, rows: int, ctx: Context, *, rotate: bool = False, stats: int = 2) -> int:
-    """Lanes that share one row.  A lane keeps at most 32 row elements resident;
-    up to 256 lanes are used as long as each still issues two 16-byte loads."""
+    """Lanes that share one row.  A lane keeps at most 32 row elements resident; beyond that the width
+    follows the number of 16-byte loads per lane that streams fastest (one with a single statistic, two
+    with more), on up to 512 lanes for machine-filling rows (1024 for rows of 2048 chunks and more)."""
     vec = max(1, 16 // elem_bytes)
     chunks = max(1, cols // vec) if cols % vec == 0 else cols
     if rotate:
@@ -91,18 +92,22 @@ def pick_coop(cols: int, elem_bytes: int, rows: int, ctx: Context, *, rotate: bo
     lanes = 1
     while lanes < 1024 and cols > lanes * 32:
         lanes *= 2
-    # Bandwidth-bound rows run fastest with two 16-byte loads per lane in flight
-    # and many waves per CU (measured on 2048-wide fp32 rows: b256 beats b64 by 10 %).
-    while lanes < 256 and chunks >= lanes * 4:
+    # Bandwidth-bound rows: what matters is how many 16-byte loads a lane keeps in flight and how many hand-off
+    # barriers the workgroup takes.  Swept over machine-filling fp32 rows of 1024 / 2048 / 4096 / 8192 columns
+    # (64 Mi elements in, as many out; us, best two widths):
+    #   one statistic (RMSNorm):  b256 81.6 / b128 82.9;  b512 82.1 / b128 84.9;  b256 86.3 / b512 86.3;  b1024 85.6 / b128 86.9
+    #   two statistics (softmax): b128 81.6 / b64 84.4;   b256 81.3 / b128 85.1;  b512 81.3 / b256 85.1;  b1024 86.7 / b128 88.6
+    # i.e. one load per lane with one statistic, two with more, on at most 512 lanes — 1024 once a lane of a
+    # 512-lane workgroup would hold four loads or more.  Rows that do not fill the machine stay at 256 lanes at
+    # most (wider workgroups only add hand-off latency there).
+    per_lane = 1 if stats == 1 else 2
+    filling = rows * 512 >= ctx.compute_units * 2048
+    limit = (1024 if chunks >= 4 * 512 else 512) if filling else 256
+    while lanes < limit and chunks >= lanes * 2 * per_lane:
         lanes *= 2
     # Few rows: spread each row over more lanes so more CUs take part.
     while lanes < 256 and rows * lanes < ctx.compute_units * 64 and chunks >= lanes * 2:
         lanes *= 2
-    # One statistic (one hand-off barrier) over machine-filling rows: one 16-byte load per lane on 512 lanes
-    # streams faster than two on 256 (32768 x 2048 fp32 RMSNorm: 85.7 -> 83.0 us); with two statistics the
-    # second barrier of the wider workgroup costs more than that (softmax 28 x 2048 x 2048: 145.5 -> 152.1 us).
-    if stats == 1 and lanes == 256 and chunks == 512 and rows * 512 >= ctx.compute_units * 2048:
-        lanes = 512
     return min(lanes, 1024)
 
 
@@ -369,7 +374,30 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
     if stage is None:
         stage = _default_stage(plan, body, ctx)
     body.stage = stage
-    return {"TILE": plan.spell(), "STAGE": stage.spell()}
+    knobs = {"TILE": plan.spell(), "STAGE": stage.spell()}
+    # Cross-workgroup split of the reduction axis (``REDUCE=g<n>k`` workspace + combine, ``g<n>a`` atomic adds
+    # into a zeroed workspace + combine).  Only a pin asks for it: on the measured shapes the second launch costs
+    # more than the idle CUs (see ``deplodock_amd.emit.splitk``).  A ``b<n>`` / ``r<n>`` pin is a row kernel's.
+    body.reduce = ReducePlan()
+    pinned_reduce = _pin("REDUCE", tuned)
+    if pinned_reduce:
+        try:
+            rp = ReducePlan.parse(pinned_reduce)
+            if rp.cta > 1:
+                if body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None:
+                    raise ScheduleError("a cross-workgroup split takes a plain contraction (no gate/up pair, row prologue or row epilogue)")
+                if body.k % rp.cta or (body.k // rp.cta) % plan.bk_elems:
+                    raise ScheduleError(f"K={body.k} does not split into {rp.cta} slices of whole {plan.bk_elems}-deep slabs")
+                if stage.transport in ("ks", "mix"):
+                    body.stage = stage = Stage(depth=2, transport="sync", reg_depth=2 if body.k // rp.cta // plan.bk_elems >= 3 else 1)
+                    knobs["STAGE"] = stage.spell()
+                if stage.transport in ("dl", "dli") and (plan.bk_elems // plan.atom.k) % 2:
+                    raise ScheduleError("direct-to-LDS staging needs an even number of MFMA steps per slab")
+                body.reduce = ReducePlan(cta=rp.cta, finalize=rp.finalize)
+                knobs["REDUCE"] = body.reduce.spell()
+        except ScheduleError as exc:
+            logger.warning("EMMY_REDUCE=%r ignored for the contraction: %s", pinned_reduce, exc)
+    return knobs
 
 
 def _flash_lds(body: Flash, ctx: Context) -> int:

@@ -234,6 +234,7 @@ def tune_graph(graph, backend, db: TuneDB | None = None, *, input_data: dict | N
                 progress(r, len(rounds), pins, f"failed: {exc}")
             continue
         us = {lt.idx: (min(lt.samples) if lt.samples else lt.time_ms) * 1e3 for lt in bench.per_launch}
+        timed: list[str] = []  # what the progress line reports: every kernel that kept its pin, with its time
         for idx, op, key in _kernels(compiled):
             res = results.get(key)
             if res is None:
@@ -244,13 +245,14 @@ def tune_graph(graph, backend, db: TuneDB | None = None, *, input_data: dict | N
             if not want_pins or not kept:
                 continue
             res.tried += 1
+            timed.append(f"{op.kernel_name} {us[idx]:.2f} us")
             if not ok:
                 res.rejected.append(",".join(f"{k}={v}" for k, v in want_pins.items()))
                 continue
             if us[idx] < res.best_us:
                 res.best_us, res.best_knobs = us[idx], dict(want_pins)
         if progress:
-            progress(r, len(rounds), pins, "ok" if ok else "outputs differ: rejected")
+            progress(r, len(rounds), pins, ("ok" if ok else "outputs differ: rejected") + (f" [{'; '.join(timed)}]" if timed else " [pin not kept]"))
     out = list(results.values())
     if db is not None:
         for res in out:

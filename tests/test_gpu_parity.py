@@ -567,6 +567,78 @@ def test_residual_linear_with_bias(device):
         prog.close()
 
 
+@pytest.mark.parametrize("reduce", ["g2k", "g4k", "g2a", "g4a"])
+@pytest.mark.parametrize("m,k,n", [(1, 1024, 3072), (16, 1024, 3072), (128, 1024, 3072), (40, 1536, 1000), (130, 4096, 264)])
+def test_split_k_linear(device, m, k, n, reduce, monkeypatch):
+    """Cross-workgroup split of the reduction axis, workspace + combine (``k``) and atomic adds into a cleared
+    workspace (``a``), on the decode / few-row shapes it is meant for, ragged rows and columns, a 1536-deep
+    reduction (three slabs of 512 for g2/g4... whole 64-deep slabs per slice): against eager and against float64.
+    The ``k`` arm adds its planes in a fixed order, so repeated launches are bit-identical."""
+    monkeypatch.setenv("EMMY_REDUCE", reduce)
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_16x16x32_bf16/w2x2/f1x2/k2")  # 64-deep slabs: every shape here splits into whole ones
+    case = eager.linear_case(m=m, k=k, n=n, seed=m + n)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    ops = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+    assert len(ops) == 2 and all(o.knobs["REDUCE"] == reduce for o in ops)
+    want = eager.run_eager(case, device)
+    exact = case.inputs[0].double() @ case.module.weight.detach().double().cpu().T
+    prog = be.program(compiled, {compiled.inputs[0]: case.inputs[0].to(device)})
+    try:
+        out = prog.output_tensors()[compiled.outputs[0]]
+        first = None
+        for rep in range(4):
+            out.zero_()
+            prog.run()
+            torch.cuda.synchronize()
+            eager.assert_close(out.reshape(want.shape), want, case.rtol, case.atol, f"split-K {reduce} {m}x{k}x{n} launch {rep} vs eager")
+            eager.assert_close(out.reshape(want.shape), exact, 2 ** -7, 2e-3, f"split-K {reduce} {m}x{k}x{n} launch {rep} vs float64")
+            if reduce.endswith("k"):
+                first = out.clone() if first is None else first
+                assert torch.equal(out, first), "workspace + combine must be bit-reproducible"
+    finally:
+        prog.close()
+
+
+def test_split_k_combine_owns_bias_and_residual(device, monkeypatch):
+    """The combine kernel applies what the unsplit kernel's output stage applies: bias into the fp32 sum, one
+    rounding, then the residual add and the second rounding — bit-identical to the unsplit kernel for the ``k`` arm."""
+
+    class Res(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = nn.Linear(512, 512)
+
+        def forward(self, x):
+            return x + self.lin(x)
+
+    torch.manual_seed(6)
+    mod = Res().bfloat16().eval()
+    with torch.no_grad():
+        mod.lin.bias.copy_(torch.randn(512))
+    x = torch.randn(96, 512).bfloat16()
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_16x16x32_bf16/w2x2/f1x2/k2")
+    outs = {}
+    for reduce in ("", "g2k", "g4a"):
+        monkeypatch.setenv("EMMY_REDUCE", reduce)
+        be = HipBackend()
+        compiled = be.compile(trace_module(mod, (x,)))
+        assert sum(isinstance(n_.op, HipOp) for n_ in compiled.nodes.values()) == (2 if reduce else 1)
+        prog = be.program(compiled, {compiled.inputs[0]: x.to(device)})
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            outs[reduce] = prog.output_tensors()[compiled.outputs[0]].clone()
+        finally:
+            prog.close()
+    with torch.no_grad():
+        want = mod.to(device)(x.to(device))
+    for reduce, y in outs.items():
+        eager.assert_close(y.reshape(want.shape), want, 2e-2, 2e-2, f"x + linear(x) with bias, REDUCE={reduce or '-'}")
+    # same fp32 terms, same rounding points; only the association of the k sum differs between split and unsplit
+    assert float((outs["g2k"].float() - outs[""].float()).abs().max()) <= 2 ** -6
+
+
 def test_fused_pointwise_with_broadcasts_and_row_reductions(device):
     class Mix(nn.Module):
         def forward(self, x, y, w, s):
@@ -623,7 +695,7 @@ def test_staging_transports_are_bit_identical(device, monkeypatch):
     x = case.inputs[0].to(device)
     monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x2/f1x2/k4")
     outs = {}
-    for stage in ("d2/sync", "d2/sync/p2", "d2/sync/p3", "d2/mix", "d2/dl", "d3/dl", "d4/dl"):  # 16 slabs: not a multiple of three register sets
+    for stage in ("d2/sync", "d2/sync/p2", "d2/sync/p3", "d2/mix", "d2/dl", "d3/dl", "d4/dl", "d3/dli", "d4/dli"):  # 16 slabs: not a multiple of three register sets
         monkeypatch.setenv("EMMY_STAGE", stage)
         be = HipBackend()
         compiled = be.compile(graph)
@@ -631,7 +703,7 @@ def test_staging_transports_are_bit_identical(device, monkeypatch):
         assert op.knobs["STAGE"] == stage
         prog = be.program(compiled, {compiled.inputs[0]: x})
         try:
-            for _ in range(3):  # direct-to-LDS publication races would show as run-to-run differences
+            for _ in range(40):  # direct-to-LDS publication races would show as run-to-run differences
                 prog.run()
                 torch.cuda.synchronize()
                 y = prog.output_tensors()[compiled.outputs[0]].clone()
@@ -643,6 +715,66 @@ def test_staging_transports_are_bit_identical(device, monkeypatch):
     for stage, y in outs.items():
         assert torch.equal(y, outs["d2/sync"]), f"{stage} differs from d2/sync"
     eager.assert_close(outs["d2/sync"], eager.run_eager(case, device), case.rtol, case.atol, "pinned tile vs eager")
+
+
+def _soak(prog, out_name: str, launches: int, what: str) -> None:
+    """``launches`` runs of a bound program on fixed inputs, every output compared bit for bit with the first
+    launch's; stops at the first mismatch."""
+    out = prog.output_tensors()[out_name]
+    prog.run()
+    torch.cuda.synchronize()
+    first = out.clone()
+    for i in range(1, launches):
+        out.zero_()
+        prog.run()
+        torch.cuda.synchronize()
+        if not torch.equal(out, first):
+            bad = int((out.view(torch.int16) != first.view(torch.int16)).sum())
+            pytest.fail(f"{what}: launch {i} of {launches} differs from the first launch in {bad} elements")
+
+
+@pytest.mark.parametrize("stage", ["d3/dl", "d3/dli"])
+def test_soak_direct_to_lds_contraction_is_bit_stable_over_thousands_of_launches(device, stage, monkeypatch):
+    """The publication fence of the direct-to-LDS rings (a flat LDS read of the issuing wave, waited for on the
+    LDS counter, before the barrier) as a test: a race that let one wave read a slab before another wave's loads
+    were visible showed as run-to-run differences in about a quarter of the launches without it.  3000 launches
+    of a machine-filling contraction on fixed inputs must reproduce the first launch bit for bit, and that
+    result must be the register-staged transport's."""
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_16x16x32_bf16/w2x4/f4x3/k2")
+    monkeypatch.setenv("EMMY_STAGE", stage)
+    case = eager.linear_case(m=2048, k=1024, n=3072, seed=21)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    (op,) = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+    assert op.knobs["STAGE"] == stage
+    prog = be.program(compiled, {compiled.inputs[0]: case.inputs[0].to(device)})
+    try:
+        _soak(prog, compiled.outputs[0], 3000, f"contraction {stage}")
+        got = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    monkeypatch.setenv("EMMY_STAGE", "d2/sync")
+    ref, _, _ = run_case(case, device)
+    assert torch.equal(got.reshape(ref.shape), ref), f"{stage} differs from register staging"
+
+
+@pytest.mark.parametrize("pin", ["w2/kv32/s4/p", "w4/kv64/s2", "w8/kv64/s1/p"])
+def test_soak_flash_staging_is_bit_stable_over_thousands_of_launches(device, pin, monkeypatch):
+    """The same for the attention kernel's K/V blocks (one family per workgroup shape: key-split pairs, key
+    split, eight query waves): 2000 launches on fixed inputs, bit-identical to the first, which matches eager."""
+    monkeypatch.setenv("EMMY_FLASH", pin)
+    case = eager.sdpa_case(b=1, hq=16, hkv=8, s=1024, d=128, seed=22)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    assert [n.op.knobs["FLASH"] for n in compiled.nodes.values() if isinstance(n.op, HipOp)] == [pin]
+    prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, case.inputs)})
+    try:
+        _soak(prog, compiled.outputs[0], 2000, f"flash {pin}")
+        got = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = eager.run_eager(case, device)
+    eager.assert_close(got.reshape(want.shape), want, case.rtol, case.atol, f"flash {pin} after the soak vs eager")
 
 
 @pytest.mark.parametrize("cols", [151936, 70000])

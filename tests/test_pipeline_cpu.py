@@ -159,6 +159,40 @@ def test_reduce_pin_is_authoritative_and_bad_pin_degrades(launcher_lib, monkeypa
     assert kernels(compile_case(case))[0].knobs["REDUCE"] == "b256"
 
 
+def test_split_k_pin_makes_a_partial_kernel_and_a_combine(launcher_lib, monkeypatch):
+    """``REDUCE=g<n>k``: a partial kernel over slices of k (grid y = the split) writing fp32 planes of a workspace,
+    and a combine kernel that folds them and owns bias / rounding; ``g<n>a``: one plane, cleared before the launch,
+    atomic adds.  A split that does not divide the reduction extent into whole slabs degrades to the unsplit kernel."""
+    from deplodock_amd.dtype import F32
+
+    case = eager.linear_case(m=128)
+    monkeypatch.setenv("EMMY_REDUCE", "g2k")
+    g = compile_case(case)
+    ks = {k.kernel_name.rsplit("_", 1)[0]: k for k in kernels(g)}
+    assert set(ks) == {"k_linear_partial", "k_linear_combine"}
+    part, comb = ks["k_linear_partial"], ks["k_linear_combine"]
+    assert part.grid[1] == (2,) and part.knobs["REDUCE"] == "g2k" and comb.knobs["REDUCE"] == "g2k" and part.zero_outputs == ()
+    ws = part.arg_order[-1]
+    assert comb.arg_order[0] == ws and g.nodes[ws].output.shape == (2, 128, 3072) and g.nodes[ws].output.dtype is F32 and g.node_role(ws) == "scratch"
+    assert "blockIdx.y * K" in part.kernel_source and "#define K 512" in part.kernel_source
+    order = g.topological_order()
+    assert order.index(ws) < order.index(g.outputs[0])
+    for k in (part, comb):
+        hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+    monkeypatch.setenv("EMMY_REDUCE", "g4a")
+    g = compile_case(case)
+    part = next(k for k in kernels(g) if "partial" in k.kernel_name)
+    assert part.grid[1] == (4,) and part.zero_outputs == (part.arg_order[-1],) and "global_atomic_fadd_f32" in part.kernel_source
+    assert g.nodes[part.arg_order[-1]].output.shape == (1, 128, 3072)
+    hiprtc.compile_to_hsaco(part.kernel_source, part.kernel_name)
+    monkeypatch.setenv("EMMY_REDUCE", "g3k")  # 1024 is not three slices of whole slabs
+    (k,) = kernels(compile_case(case))
+    assert "REDUCE" not in k.knobs and k.grid[1] == (1,)
+    monkeypatch.setenv("EMMY_REDUCE", "g2k")  # few rows: the k-split-over-waves form gives way to slab staging
+    part = next(k for k in kernels(compile_case(eager.linear_case(m=16))) if "partial" in k.kernel_name)
+    assert part.knobs["STAGE"].startswith("d2/sync")
+
+
 def test_tile_and_stage_pins(launcher_lib, monkeypatch):
     case = eager.linear_case()
     monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x2/f2x3/k4")
