@@ -146,13 +146,16 @@ class HipBackend(Backend):
                 outputs[alias] = vals.reshape(shape)
         return RunResult(outputs=outputs, time_ms=result.time_ms), pre
 
-    def program(self, compiled: Graph, input_data: dict | None = None):
-        """A persistent :class:`CompiledProgram` bound to device buffers (for serving loops)."""
+    def program(self, compiled: Graph, input_data: dict | None = None, *, library_scratch: bool = False):
+        """A persistent :class:`CompiledProgram` bound to device buffers (for serving loops).  With
+        ``library_scratch`` the program's intermediates live in the launcher library's own device scratch
+        array (``emh_launch_scratch``): nothing is allocated for them, at the price of a size limit and of
+        sharing that array with every other such program on the GPU."""
         from deplodock_amd.backend.hip.program import CompiledProgram
 
         self._select_device()
         compiled = self.variant(compiled, input_data)
-        return CompiledProgram.build(compiled, self.bind(compiled, input_data))
+        return CompiledProgram.build(compiled, self.bind(compiled, input_data), library_scratch=library_scratch)
 
     # -- benchmark --------------------------------------------------------------
     async def benchmark_async(

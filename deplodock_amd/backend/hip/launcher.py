@@ -17,6 +17,7 @@ from deplodock_amd import config
 
 EMH_RTC_ERROR_BASE = 100000
 EMH_ABI_VERSION = 1
+EMH_SCRATCH_MAX_BYTES = 16 * 1024 * 1024  # include/emmy_hip.h
 
 # name -> (restype, argtypes); mirrors include/emmy_hip.h declaration by declaration.
 _U3 = C.c_uint * 3
@@ -38,6 +39,7 @@ SIGNATURES: dict[str, tuple] = {
     "emh_func_set_dynamic_lds": (C.c_int, [C.c_void_p, C.c_int]),
     "emh_func_attributes": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "emh_launch": (C.c_int, [C.c_void_p, _U3, _U3, C.c_uint, C.c_void_p, C.POINTER(C.c_void_p), C.c_int]),
+    "emh_launch_scratch": (C.c_int, [C.c_void_p, _U3, _U3, C.c_uint, C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_int]),
     "emh_memset_async": (C.c_int, [C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]),
     "emh_stream_create": (C.c_int, [C.POINTER(C.c_void_p)]),
     "emh_stream_destroy": (C.c_int, [C.c_void_p]),
@@ -197,6 +199,12 @@ class Launcher:
         rc = self._dll.emh_launch(fn, _U3(*grid), _U3(*block), lds_bytes, stream, args.array, args.n)
         if rc != 0:
             raise LauncherError(f"emh_launch failed ({rc}): {self.last_error()}", rc)
+
+    def launch_scratch(self, fn: int, grid, block, lds_bytes: int, stream: int | None, args: PackedArgs, scratch_arg: int, scratch_offset: int, scratch_bytes: int, zero_first: bool) -> None:
+        """``launch`` with parameter ``scratch_arg`` pointed at the library's own device scratch array (no allocation anywhere)."""
+        rc = self._dll.emh_launch_scratch(fn, _U3(*grid), _U3(*block), lds_bytes, stream, args.array, args.n, scratch_arg, scratch_offset, scratch_bytes, int(zero_first))
+        if rc != 0:
+            raise LauncherError(f"emh_launch_scratch failed ({rc}): {self.last_error()}", rc)
 
     def memset_async(self, dptr: int, value: int, nbytes: int, stream: int | None) -> None:
         self._check(self._dll.emh_memset_async(dptr, value, nbytes, stream), "emh_memset_async")

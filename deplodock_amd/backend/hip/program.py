@@ -301,6 +301,15 @@ def _host(t, dtype: DType) -> np.ndarray:
 # ---------------------------------------------------------------------------
 
 
+@dataclass(frozen=True)
+class _LibraryScratch:
+    """A scratch buffer that lives in the launcher library's own device array (``emh_launch_scratch``)
+    instead of a tensor: the bytes ``[offset, offset + nbytes)`` of that array."""
+
+    offset: int
+    nbytes: int
+
+
 class CompiledProgram:
     """A compiled graph bound to device buffers, ready to launch repeatedly.
 
@@ -316,7 +325,7 @@ class CompiledProgram:
         self._slab = slab
         self.slab_bytes = slab_bytes
         self.naive_scratch_bytes = naive_bytes
-        self._packs: list[tuple[PackedArgs, tuple, tuple, list[tuple[PackedArgs, int]]]] = []
+        self._packs: list[tuple] = []  # (args, grid, block, fills of zeroed outputs, borrowed scratch range or None) per launch
         self._stream: int | None = None  # private stream for capture / timing
         self._launch_graphs: dict[int, int] = {}
         self._launch_graph_sizes: list[int] | None = None
@@ -328,7 +337,11 @@ class CompiledProgram:
 
     # -- construction ---------------------------------------------------------
     @classmethod
-    def build(cls, graph: Graph, input_data: dict | None = None, compile_timeout_s: float | None = None) -> CompiledProgram:
+    def build(cls, graph: Graph, input_data: dict | None = None, compile_timeout_s: float | None = None, library_scratch: bool = False) -> CompiledProgram:
+        """``library_scratch``: intermediates (the workspace of a split contraction) are not allocated at all;
+        each launch borrows the launcher library's device scratch array through ``emh_launch_scratch``, for
+        callers that must not allocate.  Limits: the planned scratch must fit that array, and a launch may name
+        one scratch buffer only."""
         t0 = time.perf_counter()
         compiled = _compile(graph)
         input_data = dict(input_data or {})
@@ -347,9 +360,16 @@ class CompiledProgram:
                 sizes[buf.name] = max(1, int(np.prod(shape))) * buf.dtype.nbytes
         intervals = compute_live_intervals(list(sizes), compiled.launches)
         offsets, total = plan_offsets(intervals, sizes)
-        slab = torch.zeros(max(total, _SLAB_ALIGN), dtype=torch.uint8, device=_device())
+        if library_scratch:
+            if total > launcher.EMH_SCRATCH_MAX_BYTES:
+                raise ValueError(f"the program's intermediates need {total} bytes; the library's scratch array holds {launcher.EMH_SCRATCH_MAX_BYTES}")
+            slab = None
+            for name, off in offsets.items():
+                arrays[name] = _LibraryScratch(off, -(-sizes[name] // 4) * 4)
+        else:
+            slab = torch.zeros(max(total, _SLAB_ALIGN), dtype=torch.uint8, device=_device())
         for buf in compiled.bufs:
-            if buf.role == "scratch":
+            if buf.role == "scratch" and not library_scratch:
                 shape = buf.resolve_shape(sym_values) or (1,)
                 off = offsets[buf.name]
                 arrays[buf.name] = slab[off : off + sizes[buf.name]].view(to_torch(buf.dtype)).view(shape)
@@ -365,8 +385,15 @@ class CompiledProgram:
         self._packs = []
         for ln in self.compiled.launches:
             ptrs = []
-            for name in ln.arg_names:
+            scratch = None  # (parameter index, offset, bytes, clear first) when the launch borrows the library's scratch array
+            for i, name in enumerate(ln.arg_names):
                 t = self.arrays[name]
+                if isinstance(t, _LibraryScratch):
+                    if scratch is not None and scratch[1] != t.offset:
+                        raise ValueError(f"kernel {ln.kernel_name!r} names two scratch buffers; a launch can borrow one range of the library's scratch array")
+                    scratch = (i, t.offset, t.nbytes, name in ln.zero_outputs)
+                    ptrs.append(0)
+                    continue
                 ptr = t.data_ptr()
                 if ptr % 16:
                     raise ValueError(f"buffer {name!r} is not 16-byte aligned (vector loads require it)")
@@ -378,13 +405,15 @@ class CompiledProgram:
             zero_packs = []
             for z in ln.zero_outputs:
                 t = self.arrays[z]
+                if isinstance(t, _LibraryScratch):
+                    continue  # cleared by emh_launch_scratch itself
                 nbytes = t.numel() * t.element_size()
                 if nbytes % 4:
                     raise ValueError(f"zero_outputs buffer {z!r} is not a whole number of 32-bit words")
                 zero_packs.append((PackedArgs([t.data_ptr()], [nbytes // 4]), nbytes // 4))
             if ln.lds_bytes > _STATIC_LDS_CAP:
                 self.lib.func_set_dynamic_lds(self.compiled.kernels[ln.kernel_name].fn, ln.lds_bytes)
-            self._packs.append((pack, grid, block, zero_packs))
+            self._packs.append((pack, grid, block, zero_packs, scratch))
 
     # -- launching ----------------------------------------------------------------
     def _torch_stream(self) -> int:
@@ -392,13 +421,16 @@ class CompiledProgram:
 
     def launch_one(self, i: int, stream: int | None) -> None:
         ln = self.compiled.launches[i]
-        pack, grid, block, zero_packs = self._packs[i]
+        pack, grid, block, zero_packs, scratch = self._packs[i]
         for zp, words in zero_packs:
             zgrid = (max(1, min(1024, -(-words // 256))), 1, 1)
             self.lib.launch(self.compiled.kernels[_ZERO_KERNEL_NAME].fn, zgrid, (256, 1, 1), 0, stream, zp)
         if grid[0] * grid[1] * grid[2] == 0:
             return  # an empty index space (zero rows): nothing to compute, and the driver rejects empty grids
-        self.lib.launch(self.compiled.kernels[ln.kernel_name].fn, grid, block, ln.lds_bytes, stream, pack)
+        if scratch is not None:
+            self.lib.launch_scratch(self.compiled.kernels[ln.kernel_name].fn, grid, block, ln.lds_bytes, stream, pack, *scratch)
+        else:
+            self.lib.launch(self.compiled.kernels[ln.kernel_name].fn, grid, block, ln.lds_bytes, stream, pack)
 
     def run(self, stream: int | None = None) -> None:
         """Issue every launch once, in program order, on ``stream`` (default: torch's current stream)."""

@@ -1,18 +1,30 @@
 // libemmy_hip.so — C-ABI kernel launcher for gfx950 (see include/emmy_hip.h).
 //
-// Host-only C++ over hipRTC and the HIP module API.  No device code lives
-// here: kernels arrive as source text from the Python emitter.  The library
-// allocates no device memory and starts no threads.
+// C++ over hipRTC and the HIP module API, built with hipcc for gfx950.  Kernels
+// arrive as source text from the Python emitter; the only device code here is
+// the scratch array emh_launch_scratch lends to kernels and the kernel that
+// clears it.  The library allocates no device memory and starts no threads.
 #include "emmy_hip.h"
 
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
+
+// Workspace lent to kernels by emh_launch_scratch.  In host code this name is a
+// stand-in, not a device address: the per-device address comes from
+// hipGetSymbolAddress (scratch_base below) and only that is ever handed on.
+static __device__ __align__(256) unsigned char emh_scratch[EMH_SCRATCH_MAX_BYTES];
+
+__global__ void __launch_bounds__(256) emh_scratch_zero_words(unsigned int* __restrict__ p, size_t words) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < words; i += (size_t)gridDim.x * 256) p[i] = 0u;
+}
 
 namespace {
 
@@ -40,6 +52,27 @@ int fail_arg(const char* what) {
     hipError_t e_ = (call);                         \
     if (e_ != hipSuccess) return fail_hip(e_, #call); \
   } while (0)
+
+// Address of emh_scratch on the current device, looked up once per device (each GPU holds its
+// own copy of the array at its own address).
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+unsigned char* g_scratch_base[kMaxDevices] = {};
+
+int scratch_base(unsigned char** out) {
+  int dev = -1;
+  EMH_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail_arg("emh_launch_scratch: device index out of range");
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_base[dev]) {
+    void* p = nullptr;
+    EMH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(emh_scratch)));
+    if (!p) return fail_arg("emh_launch_scratch: the scratch array has no address on this device");
+    g_scratch_base[dev] = static_cast<unsigned char*>(p);
+  }
+  *out = g_scratch_base[dev];
+  return 0;
+}
 
 }  // namespace
 
@@ -199,6 +232,37 @@ int emh_launch(void* fn, const unsigned grid[3], const unsigned block[3], unsign
                                 block[1], block[2], lds_bytes, static_cast<hipStream_t>(stream),
                                 args, nullptr));
   return 0;
+}
+
+int emh_launch_scratch(void* fn, const unsigned grid[3], const unsigned block[3],
+                       unsigned lds_bytes, void* stream, void** args, int nargs, int scratch_arg,
+                       size_t scratch_offset, size_t scratch_bytes, int zero_first) {
+  constexpr int kMaxArgs = 64;
+  if (!fn || !grid || !block) return fail_arg("emh_launch_scratch: NULL argument");
+  if (nargs <= 0 || nargs > kMaxArgs || !args) return fail_arg("emh_launch_scratch: bad argument list (1..64 parameters)");
+  if (scratch_arg < 0 || scratch_arg >= nargs) return fail_arg("emh_launch_scratch: scratch_arg is not a parameter of the kernel");
+  if (scratch_offset % 256 != 0 || scratch_bytes % 4 != 0)
+    return fail_arg("emh_launch_scratch: scratch_offset must be a multiple of 256 and scratch_bytes of 4");
+  if (scratch_bytes == 0 || scratch_offset > EMH_SCRATCH_MAX_BYTES || scratch_bytes > EMH_SCRATCH_MAX_BYTES - scratch_offset) {
+    g_last_error = "emh_launch_scratch: workspace of " + std::to_string(scratch_bytes) + " bytes at offset " +
+                   std::to_string(scratch_offset) + " does not fit the library's " + std::to_string(EMH_SCRATCH_MAX_BYTES) +
+                   "-byte scratch array (EMH_SCRATCH_MAX_BYTES)";
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  unsigned char* base = nullptr;
+  if (int rc = scratch_base(&base)) return rc;
+  void* ws = base + scratch_offset;  // the device address, never the array's name
+  void* local[kMaxArgs];
+  for (int i = 0; i < nargs; ++i) local[i] = args[i];
+  local[scratch_arg] = &ws;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (zero_first) {
+    const size_t words = scratch_bytes / 4;
+    const unsigned blocks = static_cast<unsigned>(std::min<size_t>(1024, (words + 255) / 256));
+    hipLaunchKernelGGL(emh_scratch_zero_words, dim3(blocks), dim3(256), 0, s, reinterpret_cast<unsigned int*>(ws), words);
+    EMH_HIP(hipGetLastError());
+  }
+  return emh_launch(fn, grid, block, lds_bytes, stream, local, nargs);
 }
 
 int emh_memset_async(void* dptr, int value, size_t bytes, void* stream) {

@@ -107,6 +107,34 @@ int emh_func_attributes(void* fn, int* num_regs, int* static_lds_bytes, int* pri
 int emh_launch(void* fn, const unsigned grid[3], const unsigned block[3], unsigned lds_bytes,
                void* stream, void** args, int nargs);
 
+/* Largest workspace (bytes) emh_launch_scratch can lend a kernel. */
+#define EMH_SCRATCH_MAX_BYTES (16u * 1024u * 1024u)
+
+/* emh_launch with the kernel's workspace lent by the library — an entry point
+ * that allocates nothing.  It has no counterpart in the reference (whose
+ * runtime allocates every buffer through cupy); it is for callers that cannot
+ * allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Kernels that need device memory beyond
+ * their inputs and outputs — the fp32 partial planes of a split contraction
+ * (partial kernel writes them, combine kernel folds them) — take that
+ * workspace as one pointer parameter; here parameter number `scratch_arg`
+ * (0-based, a device-pointer slot of `args`) is pointed at byte
+ * `scratch_offset` of a file-scope device array of EMH_SCRATCH_MAX_BYTES that
+ * every GPU the library runs on holds until the process ends; the value the
+ * caller stored in that slot is ignored and `args` is not modified.  With
+ * `zero_first` the `scratch_bytes` bytes from the offset are cleared on
+ * `stream` by a fill kernel first (never hipMemsetAsync: the call may be
+ * under capture).  Everything else is emh_launch.  Fails, launching nothing,
+ * when scratch_offset + scratch_bytes exceeds EMH_SCRATCH_MAX_BYTES, when
+ * the offset is not a multiple of 256 or the size not a multiple of 4, or
+ * when scratch_arg is not a slot of `args`.  Calls no hipMalloc / hipFree.
+ * All calls on one GPU share that GPU's array and it keeps the last call's
+ * contents: calls that overlap in time on one GPU (two streams, two threads)
+ * race on it, and a kernel that accumulates must ask for zero_first. */
+int emh_launch_scratch(void* fn, const unsigned grid[3], const unsigned block[3],
+                       unsigned lds_bytes, void* stream, void** args, int nargs, int scratch_arg,
+                       size_t scratch_offset, size_t scratch_bytes, int zero_first);
+
 /* Asynchronous byte fill of device memory on `stream`.  Replaces the
  * zero_outputs fill of emmy/compiler/backend/cuda/program.py:403-404.  Must
  * not be called while `stream` is being captured into a graph (use a fill

@@ -41,6 +41,9 @@ def test_every_header_entry_cites_the_reference():
             continue  # documented as a group with the entry above them
         head = text[: text.index(sym + "(")]
         comment = head[head.rindex("/*") :]
+        if sym == "emh_launch_scratch":  # the one entry point the reference has nothing like: its comment says so and names its callers
+            assert "no counterpart in the reference" in comment and "cannot\n * allocate" in comment
+            continue
         assert "emmy/" in comment, f"{sym}: no reference citation in its comment"
 
 
