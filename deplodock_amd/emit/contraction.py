@@ -159,8 +159,13 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     plan = body.tile
     if plan is None:
         raise LoweringError("contraction: no TilePlan stamped")
-    if body.in_dtype.name not in ("bf16", "f16") or plan.atom.dtype != body.in_dtype.name:
+    if body.in_dtype.name not in ("bf16", "f16", "f32") or plan.atom.dtype != body.in_dtype.name:
         raise LoweringError(f"contraction: atom {plan.atom.name} does not take {body.in_dtype} operands")
+    ES = body.in_dtype.nbytes  # operand element size
+    EPCK = 16 // ES  # operand elements per 16-byte chunk (what a lane's fragment read fetches: consecutive k of one row)
+    fp32_tier = body.in_dtype is F32
+    if fp32_tier and (body.a_prologue is not None or body.gate_pair or body.row_epilogue is not None):
+        raise LoweringError("contraction: row prologues, gate/up pairs and row epilogues are written for 16-bit operands")
     stage = body.stage or Stage(depth=2, transport="sync")
     if stage.transport == "ks":
         from deplodock_amd.emit.skinny import emit_contraction_skinny
@@ -180,7 +185,14 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     ldo = body.ldo or N
     AM = plan.atom.m  # 32 or 16 (square atoms)
     KG = 64 // AM  # lane groups along k
-    KSTEP = plan.atom.k  # k per MFMA
+    # k per fragment read: every lane fetches one 16-byte chunk, the KG lane groups of a row fetch neighbouring chunks.
+    # A 16-bit atom consumes that in one MFMA (atom.k = 8 * KG); an fp32 atom takes one element of the chunk per MFMA
+    # (atom.k = KG: lane group g feeds k = g), so a fragment feeds four MFMAs, element e of every lane's chunk in MFMA e —
+    # a contraction does not care in which order its k terms are paired, as long as both operands use the same one.
+    KSTEP = EPCK * KG
+    MPF = KSTEP // plan.atom.k  # MFMAs per fragment pair
+    if KSTEP % plan.atom.k or MPF not in (1, EPCK):
+        raise LoweringError(f"contraction: atom {plan.atom.name} does not consume 16-byte k chunks")
     ACC = plan.atom.acc_per_lane
     WM, WN = plan.units
     FM, FN = plan.regs
@@ -188,13 +200,13 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     BK = plan.bk_elems
     T = plan.block_threads
     k_guard = K % BK != 0  # the last slab is short: its missing chunks are staged as zeros (both operands)
-    if k_guard and (K % 8 or body.a_prologue is not None or stage.transport != "sync"):
+    if k_guard and (K % EPCK or body.a_prologue is not None or stage.transport != "sync"):
         raise LoweringError(f"contraction: K={K} is not a multiple of the slab depth {BK} (a short last slab needs whole 16-byte chunks, register staging and no row prologue)")
-    if BK % 8 or BK > 256:
-        raise LoweringError(f"contraction: slab depth {BK} must be a multiple of 8 and at most 256")
-    if lda % 8 or ldb % 8 or ldo % 4 or body.a_offset % 8 or body.b_offset % 8 or body.out_offset % 8:
+    if BK % EPCK or BK * ES > 512:
+        raise LoweringError(f"contraction: slab depth {BK} must be whole 16-byte chunks and at most 512 bytes a row")
+    if lda % EPCK or ldb % EPCK or ldo % 4 or body.a_offset % EPCK or body.b_offset % EPCK or body.out_offset % 8:
         raise LoweringError("contraction: leading dimensions must keep 16-byte operand / 8-byte output alignment")
-    CPR = BK // 8  # 16-byte chunks per slab row
+    CPR = BK // EPCK  # 16-byte chunks per slab row
     if CPR & (CPR - 1):
         raise LoweringError(f"contraction: slab depth {BK} must give a power-of-two chunk count")
     RPL = max(1, 16 // CPR)  # slab rows per 256-byte bank line
@@ -205,7 +217,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     if a_chunks % T or b_chunks % T:
         raise LoweringError(f"contraction: tile {TM}x{TN}x{BK} does not divide over {T} threads")
     A_PER_T, B_PER_T = a_chunks // T, b_chunks // T
-    slab_bytes = (TM + TN * NB) * BK * 2
+    slab_bytes = (TM + TN * NB) * BK * ES
     depth = 2 if stage.transport == "mix" else max(2, stage.depth)
     RS = 1 if stage.transport in ("dl", "dli", "mix") else max(1, stage.reg_depth)  # register sets a slab travels through on the sync path
     lds_bytes = slab_bytes * depth
@@ -228,7 +240,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     if dl and (a_chunks % 64 or b_chunks % 64):
         raise LoweringError("contraction: direct-to-LDS staging needs whole-wave chunk counts")
 
-    frag_t = _frag_t(body.in_dtype.name)
+    frag_t = rt.vector_type(body.in_dtype.name, EPCK)[0]
     in_c = rt.type_name(body.in_dtype.name)
     out_c = rt.type_name(body.out_dtype.name)
     epi_names = [n for n, _ in body.epilogue_operands]
@@ -270,7 +282,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
 
     D = dict(
         name=name, T=T, M=M, N=N, K=K, LDA=lda, LDB=ldb, LDO=ldo, TM=TM, TN=TN, BK=BK, WM=WM, WN=WN, FM=FM, FN=FN,
-        AM=AM, KG=KG, KSTEP=KSTEP, ACC=ACC, CPR=CPR, RPL=RPL, NB=NB, A_PER_T=A_PER_T, B_PER_T=B_PER_T,
+        AM=AM, KG=KG, KSTEP=KSTEP, ACC=ACC, ES=ES, EPCK=EPCK, MPF=MPF, CPR=CPR, RPL=RPL, NB=NB, A_PER_T=A_PER_T, B_PER_T=B_PER_T,
         SLAB=slab_bytes, DEPTH=depth, RS=RS, KT=KT, TILES_M=tiles_m, TILES_N=tiles_n, NTILES=n_tiles, GM=gm, GN=gn,
         XCDS=ctx.xcds, frag_t=frag_t, in_c=in_c, out_c=out_c, params=", ".join(params), builtin=plan.atom.builtin,
         acc_t=rt.vector_type("f32", ACC)[0], G=ACC // 4,
@@ -321,7 +333,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else "") + (" int ka[A_PER_T], kb[B_PER_T];" if k_guard else ""))
     a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
     if dli:
-        if max(M * lda, N * NB * ldb) * 2 >= 2**32:
+        if max(M * lda, N * NB * ldb) * ES >= 2**32:
             raise LoweringError("contraction: STAGE .../dli addresses operands with 32-bit byte offsets; this operand is larger than 4 GiB")
         a("  unsigned va[A_PER_T], vb[B_PER_T];  // byte offset of each request's chunk from the operand base (the k position is added to the base, in scalar registers)")
         a("  const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);  // wave-uniform by construction; says so to the compiler")
@@ -334,36 +346,36 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         a("    la[i] = q * 16;")
     else:
         a("    const int row = q / CPR, c = q % CPR;")
-        a("    la[i] = row * (BK * 2) + emh_swz(row, c) * 16;")
+        a("    la[i] = row * (BK * ES) + emh_swz(row, c) * 16;")
     a(f"    int gr = m0 + row;{' if (gr > M - 1) gr = M - 1;' if m_guard else ''}")
-    a(f"    ga[i] = A + {body.a_offset}L + KSL + (long)gr * LDA + c * 8;")
+    a(f"    ga[i] = A + {body.a_offset}L + KSL + (long)gr * LDA + c * EPCK;")
     if dli:
-        a("    va[i] = ((unsigned)gr * LDA + c * 8) * 2u;")
+        a("    va[i] = ((unsigned)gr * LDA + c * EPCK) * (unsigned)ES;")
     if pro is not None:
-        a("    ca[i] = c * 8;")
+        a("    ca[i] = c * EPCK;")
     if k_guard:
-        a("    ka[i] = c * 8;")
+        a("    ka[i] = c * EPCK;")
     a("  }")
     a(r"""  #pragma unroll
   for (int i = 0; i < B_PER_T; ++i) {
     const int q = tid + i * T;""")
     if dl or mix:
         a("    const int row = q / CPR, c = emh_swz(row, q % CPR);")
-        a("    lb[i] = TM * BK * 2 + q * 16;")
+        a("    lb[i] = TM * BK * ES + q * 16;")
     else:
         a("    const int row = q / CPR, c = q % CPR;")
-        a("    lb[i] = TM * BK * 2 + row * (BK * 2) + emh_swz(row, c) * 16;")
+        a("    lb[i] = TM * BK * ES + row * (BK * ES) + emh_swz(row, c) * 16;")
     if gate:
         a("    int gr = (row < TN) ? (n0 + row) : (N + n0 + row - TN);  // second half of the slab: the paired matrix")
         if n_guard:
             a("    { const int lim = (row < TN) ? (N - 1) : (2 * N - 1); if (gr > lim) gr = lim; }")
     else:
         a(f"    int gr = n0 + row;{' if (gr > N - 1) gr = N - 1;' if n_guard else ''}")
-    a(f"    gb[i] = B + {body.b_offset}L + KSL + (long)gr * LDB + c * 8;")
+    a(f"    gb[i] = B + {body.b_offset}L + KSL + (long)gr * LDB + c * EPCK;")
     if dli:
-        a("    vb[i] = ((unsigned)gr * LDB + c * 8) * 2u;")
+        a("    vb[i] = ((unsigned)gr * LDB + c * EPCK) * (unsigned)ES;")
     if k_guard:
-        a("    kb[i] = c * 8;")
+        a("    kb[i] = c * EPCK;")
     a("  }")
 
     a(f"  {D['acc_t']} acc[NB][FM][FN];")
@@ -376,6 +388,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   #pragma unroll
   for (int r = 0; r < ACC; ++r) acc[h][i][j][r] = 0.0f;
 """)
+    a("  #define EMH_OPND(f, e) " + ("((f)[e])  /* one element of the chunk per MFMA */" if MPF > 1 else "(f)"))
     frag_decl = f"  {frag_t} fw[2][NB][FN], fx[2][FM];"
     a(frag_decl)
     a(r"""  // Fragments are double-buffered in registers: the reads for step s+1 are
@@ -384,21 +397,22 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   // just before their use).
   #define EMH_READ(P, buf, kk) { \
     const unsigned char* sA_ = emh_lds + (buf) * SLAB; \
-    const unsigned char* sB_ = sA_ + TM * BK * 2; \
+    const unsigned char* sB_ = sA_ + TM * BK * ES; \
     const int c_ = (kk) * KG + lk; \
     _Pragma("unroll") for (int h = 0; h < NB; ++h) \
     _Pragma("unroll") for (int j = 0; j < FN; ++j) { \
       const int row_ = h * TN + (wn * FN + j) * AM + lr; \
-      fw[P][h][j] = *(const FRAG_T*)(sB_ + row_ * (BK * 2) + emh_swz(row_, c_) * 16); } \
+      fw[P][h][j] = *(const FRAG_T*)(sB_ + row_ * (BK * ES) + emh_swz(row_, c_) * 16); } \
     _Pragma("unroll") for (int i = 0; i < FM; ++i) { \
       const int row_ = (wm * FM + i) * AM + lr; \
-      fx[P][i] = *(const FRAG_T*)(sA_ + row_ * (BK * 2) + emh_swz(row_, c_) * 16); } \
+      fx[P][i] = *(const FRAG_T*)(sA_ + row_ * (BK * ES) + emh_swz(row_, c_) * 16); } \
     __builtin_amdgcn_sched_barrier(0); }
   #define EMH_MMA(P) { \
+    _Pragma("unroll") for (int e = 0; e < MPF; ++e) \
     _Pragma("unroll") for (int h = 0; h < NB; ++h) \
     _Pragma("unroll") for (int i = 0; i < FM; ++i) \
     _Pragma("unroll") for (int j = 0; j < FN; ++j) \
-      acc[h][i][j] = BUILTIN(fw[P][h][j], fx[P][i], acc[h][i][j], 0, 0, 0); \
+      acc[h][i][j] = BUILTIN(EMH_OPND(fw[P][h][j], e), EMH_OPND(fx[P][i], e), acc[h][i][j], 0, 0, 0); \
     __builtin_amdgcn_sched_barrier(0); }
 """.replace("FRAG_T", frag_t).replace("BUILTIN", plan.atom.builtin))
     KS = BK // KSTEP
@@ -523,8 +537,8 @@ ROW_EPILOGUE_TABLES
         if dli:
             a(f"""  // One request of slab kt into ring buffer buf: the operand base moves along k in scalar registers, the
   // lane's chunk offset is a loop-invariant 32-bit register, the LDS target a scalar: no vector arithmetic per request.
-  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L + KSL) + (long)(kt) * (BK * 2), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * T) * 16)
-  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L + KSL) + (long)(kt) * (BK * 2), vb[i], lds0 + (buf) * SLAB + TM * BK * 2 + (wave_u * 64 + (i) * T) * 16)""")
+  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L + KSL) + (long)(kt) * (BK * ES), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * T) * 16)
+  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L + KSL) + (long)(kt) * (BK * ES), vb[i], lds0 + (buf) * SLAB + TM * BK * ES + (wave_u * 64 + (i) * T) * 16)""")
         if deferred:
             # the rows arrive in LDS untouched: every thread reads back the chunks it requested
             # (any chunk of the row will do for a row sum) while the slab is resident
@@ -584,7 +598,8 @@ ROW_EPILOGUE_TABLES
             for h in range(NB):
                 for i in range(FM):
                     for j in range(FN):
-                        a(f"    acc[{h}][{i}][{j}] = {plan.atom.builtin}(fw[{P}][{h}][{j}], fx[{P}][{i}], acc[{h}][{i}][{j}], 0, 0, 0);")
+                        for e in range(MPF):
+                            a(f"    acc[{h}][{i}][{j}] = {plan.atom.builtin}(EMH_OPND(fw[{P}][{h}][{j}], {e}), EMH_OPND(fx[{P}][{i}], {e}), acc[{h}][{i}][{j}], 0, 0, 0);")
                         if kt is not None:
                             for q, (which, pi) in enumerate(part_list):
                                 if slot_of[q] == kk * n_mma + idx:

@@ -29,8 +29,11 @@ class ScheduleError(ValueError):
 @dataclass(frozen=True)
 class Atom:
     """One MFMA instruction shape: a wave64 computes an ``m x n`` fp32 tile
-    from ``m x k`` and ``n x k`` 16-bit operands; each lane feeds ``k_per_lane``
-    consecutive k-values of one row/column and owns ``m*n/64`` accumulators."""
+    from ``m x k`` and ``n x k`` operands; each lane feeds ``k_per_lane``
+    consecutive k-values of one row/column and owns ``m*n/64`` accumulators.
+    The fp32 atoms (``v_mfma_f32_32x32x2_f32`` / ``16x16x4``: full fp32 products,
+    no reduced-precision pass) stand where the reference's scalar fp32 tier does
+    (emmy/compiler/pipeline/passes/lowering/kernel/_atom.py:717-786)."""
 
     name: str
     m: int
@@ -48,6 +51,17 @@ class Atom:
     def acc_per_lane(self) -> int:
         return self.m * self.n // self.lanes
 
+    @property
+    def elem_bytes(self) -> int:
+        return 4 if self.dtype == "f32" else 2
+
+    @property
+    def frag_k(self) -> int:
+        """k-values one fragment read covers: every lane fetches a 16-byte chunk of its row, and the
+        ``64 / m`` lane groups of a row fetch neighbouring chunks.  A 16-bit atom consumes that in one
+        MFMA (``frag_k == k``), an fp32 atom in four."""
+        return (16 // self.elem_bytes) * (self.lanes // self.m)
+
 
 ATOMS: dict[str, Atom] = {
     a.name: a
@@ -56,6 +70,8 @@ ATOMS: dict[str, Atom] = {
         Atom("mfma_16x16x32_bf16", 16, 16, 32, "bf16", "__builtin_amdgcn_mfma_f32_16x16x32_bf16"),
         Atom("mfma_32x32x16_f16", 32, 32, 16, "f16", "__builtin_amdgcn_mfma_f32_32x32x16_f16"),
         Atom("mfma_16x16x32_f16", 16, 16, 32, "f16", "__builtin_amdgcn_mfma_f32_16x16x32_f16"),
+        Atom("mfma_32x32x2_f32", 32, 32, 2, "f32", "__builtin_amdgcn_mfma_f32_32x32x2f32"),
+        Atom("mfma_16x16x4_f32", 16, 16, 4, "f32", "__builtin_amdgcn_mfma_f32_16x16x4f32"),
     )
 }
 

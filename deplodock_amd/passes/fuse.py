@@ -560,6 +560,7 @@ class _RopePlan:
     div: int  # cos/sin table row of memory row r is (r // div) % mod
     mod: int
     rms: _RmsMatch | None  # the norm feeding the rotation when it can be fused in
+    pad: int = 0  # leading unit dims the traced result has more than the rotated tensor (``t_view_shape`` includes them, ``order`` does not)
 
 
 def _plan_rope(c: _Ctx, nid: str) -> _RopePlan | None:
@@ -593,8 +594,11 @@ def _plan_rope(c: _Ctx, nid: str) -> _RopePlan | None:
     pos_axes = [i for i in range(len(cos_shape) - 1) if cos_shape[i] > 1]
     if len(pos_axes) > 1 or cos_shape[-1] != d:
         raise FusionError("rope: cos/sin must vary over one position axis")
+    # The tables broadcast against the rotated tensor from the right, and the result takes the longer rank
+    # (a trace may carry a table with more leading unit dims than the tensor it rotates).
+    pad = max(0, len(node.output.shape) - len(tv.shape))
     if pos_axes:
-        pa = pos_axes[0]
+        pa = pos_axes[0] - (len(cos_shape) - len(tv.shape))
         if pa not in order:
             raise FusionError("rope: unsupported cos/sin layout")
         k = order.index(pa)
@@ -604,7 +608,8 @@ def _plan_rope(c: _Ctx, nid: str) -> _RopePlan | None:
         mod = mem_shape[k]
     else:
         div, mod = 1, 1
-    return _RopePlan(t_id, cos_id, sin_id, d, node.output.dtype, tuple(int(v) for v in g.nodes[t_id].output.shape), order, mem_shape, rows, div, mod, rms if fuse_norm else None)
+    t_shape = (1,) * pad + tuple(int(v) for v in g.nodes[t_id].output.shape)
+    return _RopePlan(t_id, cos_id, sin_id, d, node.output.dtype, t_shape, order, mem_shape, rows, div, mod, rms if fuse_norm else None, pad)
 
 
 def _rope_tables(c: _Ctx, p: _RopePlan, div: int) -> tuple[tuple[RowOperand, RowOperand], View, View]:
@@ -628,7 +633,7 @@ def _logical_strides(p: _RopePlan, mem_strides: tuple[int, ...]) -> tuple[int, .
     ``p.order``; ``mem_strides`` are the strides of those memory-order dims."""
     out = [0] * len(p.t_view_shape)
     for pos, i in enumerate(p.order):
-        out[i] = mem_strides[pos]
+        out[i + p.pad] = mem_strides[pos]
     out[-1] = 1
     return tuple(out)
 
@@ -761,7 +766,9 @@ def _rec_rope(c: _Ctx, nid: str) -> bool:
     else:
         tv = resolve_view(g, p.t_id)
         xv = _need(c, p.t_id)
-        rows2, x_addr = _row_addr(View(xv.base, xv.offset, tuple(tv.shape[i] for i in p.order) + (d,), tuple(tv.strides[i] for i in p.order) + (1,), xv.dtype))
+        # rows walk the rotated tensor in the planned order, addressed through the strides it really has
+        # (a window of a merged projection buffer is wider-strided than the traced tensor)
+        rows2, x_addr = _row_addr(View(xv.base, xv.offset, tuple(xv.shape[i] for i in p.order) + (d,), tuple(xv.strides[i] for i in p.order) + (1,), xv.dtype))
         body = RowReduce(rows=rows2, cols=d, x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=od, stats=(), project=E.Var("x"), x_addr=x_addr)
         body.operand_buffers = {}
         inputs = [xv.base]
@@ -794,30 +801,51 @@ def _rec_sdpa(c: _Ctx, nid: str) -> bool:
     if not isinstance(node.op, F.SdpaOp):
         return False
     q, k, v = (_need_logical(c, i) for i in node.inputs)
-    if len(q.shape) != 4:
-        raise FusionError("sdpa: expected [batch, heads, seq, head_dim] operands")
-    B, Hq, Sq, D = q.shape
-    _, Hkv, Skv, _ = k.shape
+    if min(len(q.shape), len(k.shape), len(v.shape)) < 3:
+        raise FusionError("sdpa: expected [batch..., heads, seq, head_dim] operands")
+
+    def batched(t: View) -> tuple[int, tuple[int, int, int]]:
+        """``(batch count, (batch, head, seq) strides)`` of an operand whose dims before the last three are
+        batch dims (the reference pads k / v with leading unit dims up to q's rank, frontend/ir.py:252-259)."""
+        lead = [(n, st) for n, st in zip(t.shape[:-3], t.strides[:-3]) if n != 1]
+        count, stride = 1, 0
+        for n, st in reversed(lead):
+            if count > 1 and st != stride * count:
+                raise FusionError("sdpa: batch dims must collapse into one uniformly strided axis")
+            stride = st if count == 1 else stride
+            count *= n
+        return count, (stride, t.strides[-3], t.strides[-2])
+
+    (B, q_str), (Bk, k_str), (Bv, v_str) = batched(q), batched(k), batched(v)
+    if Bk != B or Bv != B:
+        raise FusionError("sdpa: q, k and v must agree on the batch size")
+    Hq, Sq, D = q.shape[-3:]
+    Hkv, Skv = k.shape[-3], k.shape[-2]
     if Hq != Hkv and not node.op.enable_gqa:
         raise FusionError("sdpa: grouped heads need enable_gqa=True")
     for t in (q, k, v):
         if t.strides[-1] != 1:
             raise FusionError("sdpa: head_dim must be contiguous")
-    # If the only consumer transposes to [B, S, H, D] (and flattens), write that layout directly.
+    # If the only consumer swaps heads and sequence (to [B, S, H, D], then flattens), write that layout directly.
+    lead = len(node.output.shape) - 3
+    logical = tuple(int(d_) for d_ in node.output.shape)
     out_id, o_shape, o_strides = nid, (B, Hq, Sq, D), (Hq * Sq * D, Sq * D, D)
     cons = c.g.consumers(nid)
-    transposed = len(cons) == 1 and nid not in c.g.outputs and _is(c.g.nodes[cons[0]], F.TransposeOp, dim0=1, dim1=2)
+    transposed = len(cons) == 1 and nid not in c.g.outputs and _is(c.g.nodes[cons[0]], F.TransposeOp, dim0=lead, dim1=lead + 1)
     if transposed:
         o_shape, o_strides = (B, Sq, Hq, D), (Sq * Hq * D, D, Hq * D)
     scale = node.op.scale if node.op.scale is not None else 1.0 / math.sqrt(D)
     body = Flash(
         batch=B, q_heads=Hq, kv_heads=Hkv, q_len=Sq, kv_len=Skv, head_dim=D, q=q.base, k=k.base, v=v.base, out=out_id, dtype=q.dtype,
-        scale=float(scale), causal=node.op.is_causal, q_strides=q.strides[:3], k_strides=k.strides[:3], v_strides=v.strides[:3], o_strides=o_strides,
+        scale=float(scale), causal=node.op.is_causal, q_strides=q_str, k_strides=k_str, v_strides=v_str, o_strides=o_strides,
         q_offset=q.offset, k_offset=k.offset, v_offset=v.offset,
     )  # fmt: skip
     _emit(c, nid, body, "sdpa_reduce", [q.base, k.base, v.base], shape=o_shape)
-    if transposed:  # (not a comparison of the shapes: they read the same when there are as many tokens as heads)
-        c.out.nodes[nid].hints["logical_view"] = ((B, Hq, Sq, D), (o_strides[0], o_strides[1], o_strides[2], 1))
+    if transposed or len(logical) != 4:
+        # how the traced shape (with its batch dims as traced) maps onto the buffer (not a comparison of the shapes:
+        # they read the same when there are as many tokens as heads)
+        lead_strides = contiguous_strides(logical[:lead] + (1,))[:-1]
+        c.out.nodes[nid].hints["logical_view"] = (logical, (*(ls * o_strides[0] for ls in lead_strides), o_strides[1], o_strides[2], 1))
     return True
 
 

@@ -243,17 +243,19 @@ def _check_tile(plan: TilePlan, body: Contraction, ctx: Context, depth: int, dl:
     unrealisable pin degrades for the one kernel it does not fit instead of
     failing the whole lowering."""
     bk = plan.bk_elems
-    cpr = bk // 8
+    es = plan.atom.elem_bytes
+    epck = 16 // es
+    cpr = bk // epck
     nb = 2 if body.gate_pair else 1
     threads = plan.block_threads
-    if bk % 8 or bk > 256 or cpr & (cpr - 1):
-        raise ScheduleError(f"slab depth {bk} must be a power-of-two number of 16-byte chunks, at most 256 elements")
+    if bk % epck or bk * es > 512 or cpr & (cpr - 1) or bk % plan.atom.frag_k:
+        raise ScheduleError(f"slab depth {bk} must be a power-of-two number of 16-byte chunks, whole fragment reads, at most 512 bytes a row")
     a_chunks, b_chunks = plan.tile_m * cpr, plan.tile_n * cpr * nb
     if a_chunks % threads or b_chunks % threads:
         raise ScheduleError(f"tile {plan.tile_m}x{plan.tile_n}x{bk} does not divide over {threads} threads")
     if dl and (a_chunks % 64 or b_chunks % 64):
         raise ScheduleError("direct-to-LDS staging needs whole-wave chunk counts")
-    if (plan.tile_m + plan.tile_n * nb) * bk * 2 * depth > ctx.lds_bytes_per_cu:
+    if (plan.tile_m + plan.tile_n * nb) * bk * es * depth > ctx.lds_bytes_per_cu:
         raise ScheduleError("slabs exceed the LDS")
     if plan.regs[0] * plan.regs[1] * plan.atom.acc_per_lane * nb > 256:
         raise ScheduleError("accumulators exceed the 256 accumulation registers of a lane")
@@ -303,7 +305,7 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
         return Stage(depth=2, transport="sync")  # transformed in registers on its way to LDS
     if body.m <= 16:
         return Stage(depth=2, transport="sync", reg_depth=2 if steps >= 3 else 1)
-    if (plan.bk_elems // plan.atom.k) % 2 == 0:
+    if (plan.bk_elems // plan.atom.frag_k) % 2 == 0 and plan.bk_elems % plan.atom.frag_k == 0:
         # a slab that keeps the matrix pipe busy for long hides the next one's latency by itself
         mfma_cycles = plan.tile_m * plan.tile_n * (2 if body.gate_pair else 1) * plan.bk_elems * 2 // 4096
         for depth in (3, 2):
@@ -323,7 +325,14 @@ def _default_tile(body: Contraction, ctx: Context) -> TilePlan:
     atom_dtype = body.in_dtype.name
     re = body.row_epilogue
     plan = pick_tile(body.m, body.n, body.k, body.gate_pair, ctx, row_prologue=body.a_prologue is not None, group_cols=(re.cols, re.col_end) if re is not None else None)
-    if plan.atom.dtype != atom_dtype:
+    if atom_dtype == "f32":
+        # the fp32 tier keeps the candidate's tile and its slab's bytes per row: half the k-values, on the fp32 atom of the same m x n
+        atom = ATOMS[{16: "mfma_16x16x4_f32", 32: "mfma_32x32x2_f32"}[plan.atom.m]]
+        bk_elems = max(2 * atom.frag_k, plan.bk_elems // 2)
+        while bk_elems > 2 * atom.frag_k and body.k % bk_elems:
+            bk_elems //= 2
+        plan = TilePlan(atom=atom, units=plan.units, regs=plan.regs, bk=bk_elems // atom.k)
+    elif plan.atom.dtype != atom_dtype:
         plan = TilePlan(atom=ATOMS[plan.atom.name.replace("bf16", atom_dtype)], units=plan.units, regs=plan.regs, bk=plan.bk)
     return plan
 
@@ -346,6 +355,8 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
                 raise ScheduleError(f"atom {plan.atom.name} does not take {body.in_dtype} operands")
             if body.k % plan.bk_elems:
                 raise ScheduleError(f"K={body.k} is not a multiple of the slab depth {plan.bk_elems}")
+            if plan.atom.dtype == "f32" and (body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None):
+                raise ScheduleError("the fp32 tier takes a plain contraction")
             _check_tile(plan, body, ctx, depth=2)
         except ScheduleError as exc:
             logger.warning("EMMY_TILE=%r ignored: %s", pinned, exc)
@@ -358,7 +369,7 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
     if pinned_stage:
         try:
             stage = Stage.parse(pinned_stage)
-            if stage is not None and stage.transport == "dl" and (plan.bk_elems // plan.atom.k) % 2:
+            if stage is not None and stage.transport in ("dl", "dli") and ((plan.bk_elems // plan.atom.frag_k) % 2 or plan.bk_elems % plan.atom.frag_k):
                 raise ScheduleError("direct-to-LDS staging needs an even number of MFMA steps per slab")
             if stage is not None and stage.transport == "ks":
                 if not skinny_waves(body) or stage.depth not in (1, 2, 4, 8, 16) or body.k % (32 * stage.depth):
@@ -391,7 +402,7 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
                 if stage.transport in ("ks", "mix"):
                     body.stage = stage = Stage(depth=2, transport="sync", reg_depth=2 if body.k // rp.cta // plan.bk_elems >= 3 else 1)
                     knobs["STAGE"] = stage.spell()
-                if stage.transport in ("dl", "dli") and (plan.bk_elems // plan.atom.k) % 2:
+                if stage.transport in ("dl", "dli") and ((plan.bk_elems // plan.atom.frag_k) % 2 or plan.bk_elems % plan.atom.frag_k):
                     raise ScheduleError("direct-to-LDS staging needs an even number of MFMA steps per slab")
                 body.reduce = ReducePlan(cta=rp.cta, finalize=rp.finalize)
                 knobs["REDUCE"] = body.reduce.spell()

@@ -66,7 +66,14 @@ LAYOUT_OPS = (F.ViewOp, F.TransposeOp, F.PermuteOp, F.UnsqueezeOp, F.SqueezeOp, 
 
 def _reshape_strides(shape: tuple[int, ...], strides: tuple[int, ...], new_shape: tuple[int, ...]) -> tuple[int, ...] | None:
     """Strides that present the same elements in ``new_shape`` without a copy, or ``None``."""
-    old = [(n, s) for n, s in zip(shape, strides) if n != 1]
+    old: list[tuple[int, int]] = []
+    for n, s in zip(shape, strides):
+        if n == 1:
+            continue
+        if old and old[-1][1] == s * n:
+            old[-1] = (old[-1][0] * n, s)  # mutually contiguous neighbours are one run: any split of it is a view
+        else:
+            old.append((n, s))
     out: list[int] = []
     oi = 0
     ni = 0

@@ -567,6 +567,63 @@ def test_residual_linear_with_bias(device):
         prog.close()
 
 
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("m,k,n", [(2048, 1024, 3072), (512, 2048, 2048), (37, 200, 52), (1, 1024, 3072), (16, 512, 64), (300, 1000, 512), (130, 64, 1028)])
+def test_fp32_linear(device, m, k, n, bias):
+    """The fp32 contraction tier (fp32 MFMA, full-precision products): fp32 rtol 1e-5 against float64 and against
+    eager, with the absolute floor a sum of k products of unit-scale terms needs (1e-5; outputs are O(1))."""
+    torch.manual_seed(m + k)
+    lin = nn.Linear(k, n, bias=bias).eval()
+    x = torch.randn(m, k)
+    be = HipBackend()
+    compiled = be.compile(trace_module(lin, (x,)))
+    (op,) = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+    assert "_f32/" in op.knobs["TILE"]
+    prog = be.program(compiled, {compiled.inputs[0]: x.to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    exact = x.double() @ lin.weight.detach().double().T + (lin.bias.detach().double() if bias else 0.0)
+    eager.assert_close(ours.reshape(exact.shape), exact, 1e-5, 1e-5, f"fp32 linear {m}x{k}x{n} vs float64")
+    tf32 = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        with torch.no_grad():
+            want = lin.to(device)(x.to(device))
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = tf32
+    eager.assert_close(ours.reshape(want.shape), want, 1e-5, 2e-5, f"fp32 linear {m}x{k}x{n} vs eager")
+
+
+@pytest.mark.parametrize("stage", ["d2/sync", "d2/sync/p2", "d2/dl", "d3/dl", "d3/dli"])
+def test_fp32_linear_every_transport_is_bit_identical(device, stage, monkeypatch):
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_16x16x4_f32/w2x2/f2x2/k8")
+    torch.manual_seed(8)
+    lin = nn.Linear(512, 256, bias=False).eval()
+    x = torch.randn(192, 512)
+    outs = {}
+    for st in ("d2/sync", stage):
+        monkeypatch.setenv("EMMY_STAGE", st)
+        be = HipBackend()
+        compiled = be.compile(trace_module(lin, (x,)))
+        (op,) = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+        assert op.knobs["STAGE"] == st
+        prog = be.program(compiled, {compiled.inputs[0]: x.to(device)})
+        try:
+            for _ in range(5):
+                prog.run()
+                torch.cuda.synchronize()
+                y = prog.output_tensors()[compiled.outputs[0]].clone()
+                assert st not in outs or torch.equal(y, outs[st])
+                outs[st] = y
+        finally:
+            prog.close()
+    assert torch.equal(outs[stage], outs["d2/sync"])
+
+
 @pytest.mark.parametrize("reduce", ["g2k", "g4k", "g2a", "g4a"])
 @pytest.mark.parametrize("m,k,n", [(1, 1024, 3072), (16, 1024, 3072), (128, 1024, 3072), (40, 1536, 1000), (130, 4096, 264)])
 def test_split_k_linear(device, m, k, n, reduce, monkeypatch):

@@ -193,6 +193,26 @@ def test_split_k_pin_makes_a_partial_kernel_and_a_combine(launcher_lib, monkeypa
     assert part.knobs["STAGE"].startswith("d2/sync")
 
 
+def test_fp32_linear_takes_the_fp32_mfma_tier(launcher_lib, monkeypatch):
+    """An fp32 ``nn.Linear`` (what the reference's own perf suite runs, tests/perf/cases.py:20-23) lowers to the same
+    tiled kernel on ``v_mfma_f32_16x16x4_f32`` / ``32x32x2``: 16-byte chunks hold four k-values, one per MFMA."""
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(1024, 3072).eval()
+    x = torch.randn(2048, 1024)
+    (k,) = kernels(HipBackend().compile(trace_module(lin, (x,))))
+    assert k.knobs["TILE"].startswith("a:mfma_16x16x4_f32/") and "__builtin_amdgcn_mfma_f32_16x16x4f32" in k.kernel_source
+    assert "#define EPCK 4" in k.kernel_source and "#define MPF 4" in k.kernel_source and "f32x4 fw[2]" in k.kernel_source
+    assert k.algo_flops == 2 * 2048 * 1024 * 3072 and k.algo_bytes == (2048 * 1024 + 3072 * 1024 + 2048 * 3072 + 3072) * 4
+    assert hiprtc.vgpr_spill_counts(hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name).read_bytes()) == [0]
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x2_f32/w2x2/f2x2/k16")
+    monkeypatch.setenv("EMMY_STAGE", "d2/sync")
+    (k,) = kernels(HipBackend().compile(trace_module(lin, (x,))))
+    assert k.knobs["TILE"] == "a:mfma_32x32x2_f32/w2x2/f2x2/k16" and "mfma_f32_32x32x2f32" in k.kernel_source
+    monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x2/f2x2/k2")  # a 16-bit atom on fp32 operands degrades
+    (k,) = kernels(HipBackend().compile(trace_module(lin, (x,))))
+    assert "_f32/" in k.knobs["TILE"]
+
+
 def test_tile_and_stage_pins(launcher_lib, monkeypatch):
     case = eager.linear_case()
     monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x2/f2x3/k4")
