@@ -67,11 +67,52 @@ class HipBackend(Backend):
         result remembers how to re-trace (``compiled.dynamic``) and ``run`` /
         ``program`` / ``benchmark`` pick — building on first use — the variant that
         matches the shapes of the inputs they are given."""
-        compiled = Pipeline.build(HIP_PASSES, self.context).run(graph, dump_dir=self.dump)
         spec = getattr(graph, "dynamic", None)
+        if spec is not None and len(spec.hints) == 1 and self.symbolic_kernels:
+            symbolic = self._compile_symbolic(graph, spec)
+            if symbolic is not None:
+                return symbolic
+        compiled = Pipeline.build(HIP_PASSES, self.context).run(graph, dump_dir=self.dump)
         if spec is not None:
             compiled.dynamic = spec
             compiled.variants = OrderedDict({tuple(sorted(spec.hints.items())): compiled})
+        return compiled
+
+    #: lower a graph with one symbolic axis to kernels that take its extent as a runtime ``int`` (one code object per
+    #: kernel for every size); False: always specialise per size
+    symbolic_kernels = True
+
+    def _compile_symbolic(self, graph: Graph, spec) -> Graph | None:
+        """One lowering for every size of the symbolic axis: the module is fused at the traced size and at two
+        others, what changes must be affine in the size and must be something a kernel can take at run time
+        (``passes.symbolic``); the kernels are then scheduled at the traced size and emitted with a trailing
+        ``int`` parameter, run-time guards and launch-time grid factors.  ``None`` when the module does not
+        symbolise (the caller then lowers per size)."""
+        import logging
+
+        from deplodock_amd.emit.errors import LoweringError
+        from deplodock_amd.ir.sym import Affine
+        from deplodock_amd.passes.fuse import FusionError, fuse
+        from deplodock_amd.passes.symbolic import SymbolicError, symbolize
+
+        (name, s0), = spec.hints.items()
+        sizes = [s0, s0 + 7, s0 + 96]
+        try:
+            tiles = [fuse(graph)] + [fuse(spec.retrace({name: s})) for s in sizes[1:]]
+            base = symbolize(tiles, name, sizes)
+            compiled = base
+            for _pass_name, fn in HIP_PASSES[1:]:
+                compiled = fn(compiled, self.context)
+        except (SymbolicError, FusionError, LoweringError) as exc:
+            logging.getLogger(__name__).info("[hip] %s does not lower to runtime-int kernels (%s): specialising per size", name, exc)
+            return None
+        for node in compiled.nodes.values():
+            sym_shape = node.hints.get("sym_shape")
+            if sym_shape is not None:
+                # a dim that is the bare symbol is spelled by its name (how the runtime binds it to an input's shape)
+                node.output.shape = tuple(d.name if isinstance(d, Affine) and (d.a, d.b) == (1, 0) else d for d in sym_shape)
+        compiled.dynamic = spec
+        compiled.symbolic = name
         return compiled
 
     #: distinct size combinations kept per dynamically shaped graph
@@ -80,8 +121,8 @@ class HipBackend(Backend):
     def variant(self, compiled: Graph, input_data: dict | None) -> Graph:
         """The lowering of ``compiled``'s module at the sizes ``input_data`` has."""
         spec = getattr(compiled, "dynamic", None)
-        if spec is None or not input_data:
-            return compiled
+        if spec is None or not input_data or getattr(compiled, "symbolic", None) is not None:
+            return compiled  # static, or one lowering that takes the size at run time
         shapes = []
         for nid, axes in zip(compiled.inputs, spec.input_axes):
             if nid not in input_data:

@@ -80,7 +80,8 @@ class _Buffer:
     role: str  # input | constant | output | scratch
 
     def resolve_shape(self, sym_values: dict[str, int]) -> tuple[int, ...]:
-        return tuple(int(d) if not isinstance(d, str) else int(sym_values[d]) for d in self.shape)
+        """The shape at this launch's symbolic sizes: a ``str`` dim is a bare symbol, an ``Affine`` ``a * symbol + b``."""
+        return tuple(int(sym_values[d]) if isinstance(d, str) else int(d.at(sym_values)) if hasattr(d, "at") else int(d) for d in self.shape)
 
 
 @dataclass
@@ -105,6 +106,7 @@ class _Compiled:
     kernels: dict[str, hiprtc.LoadedKernel]
     launches: list[_Launch]
     symbolic_bindings: dict[str, tuple[str, int]] = field(default_factory=dict)
+    symbolic_hints: dict[str, int] = field(default_factory=dict)  # the sizes the graph was traced at (used when an input is not supplied)
 
 
 _ZERO_KERNEL_NAME = "emh_zero_words"
@@ -173,7 +175,8 @@ def _compile(graph: Graph) -> _Compiled:
     # Pass 2 — compile (cached) and load.
     kernels = {name: hiprtc.load_function(src, name) for name, src in sources.items()}
     constants = {nid: float(op.value) for nid, op in graph.constant_ops() if op.value is not None}
-    return _Compiled(bufs, {b.name: b for b in bufs}, constants, kernels, launches, _symbolic_bindings(graph))
+    hints = dict(getattr(getattr(graph, "dynamic", None), "hints", {}) or {})
+    return _Compiled(bufs, {b.name: b for b in bufs}, constants, kernels, launches, _symbolic_bindings(graph), hints)
 
 
 # ---------------------------------------------------------------------------
@@ -283,8 +286,18 @@ def _resolve_symbolic(compiled: _Compiled, input_data: dict) -> dict[str, int]:
     for name, (buf, dim) in compiled.symbolic_bindings.items():
         arr = input_data.get(buf)
         if arr is None:
+            if name in compiled.symbolic_hints:
+                env[name] = int(compiled.symbolic_hints[name])  # synthetic inputs: the traced size
+                continue
             raise ValueError(f"symbolic dim {name!r} reads from input {buf!r}.shape[{dim}] but no array was supplied")
         env[name] = int(arr.shape[dim])
+    for name, (buf, dim) in compiled.symbolic_bindings.items():
+        # every input that carries the symbol must agree on it
+        for b in compiled.bufs:
+            if b.role == "input" and b.name in input_data and b.name != buf:
+                for i, d in enumerate(b.shape):
+                    if d == name and int(input_data[b.name].shape[i]) != env[name]:
+                        raise ValueError(f"inputs disagree on {name!r}: {buf!r} gives {env[name]}, {b.name!r} gives {int(input_data[b.name].shape[i])}")
     return env
 
 

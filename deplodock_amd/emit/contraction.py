@@ -35,6 +35,7 @@ from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.ir.schedule import Stage
+from deplodock_amd.ir.sym import Affine, XcdRounds, c_value
 from deplodock_amd.ir.tile import Contraction
 
 
@@ -69,7 +70,7 @@ def xcd_block(tiles_m: int, tiles_n: int, tile_m: int, tile_n: int, xcds: int) -
     return (best[0], best[1]) if best else (1, 1)
 
 
-def _emit_row_epilogue_tables(a, re, re_args: list[str], EPC: int, m_guard: bool) -> None:
+def _emit_row_epilogue_tables(a, re, re_args: list[str], EPC: int, m_guard: bool, mods: list | None = None) -> None:
     """Fetch, at kernel start, the table chunks the row epilogue of this thread will
     need (they depend on the output coordinates only): the k loop hides the latency."""
     d = re.cols
@@ -84,8 +85,9 @@ def _emit_row_epilogue_tables(a, re, re_args: list[str], EPC: int, m_guard: bool
     a(f"      const int m = m0 + row, n = n0 + cc * {EPC}, gc = n % {d};")
     mrow = "(m < M ? m : M - 1)" if m_guard else "m"
     a(f"      const long rr = (long){mrow} * {re.col_end // d} + n / {d};  // the row number a separate row kernel would use")
-    for nm, ro in zip(re_args, re.row_operands):
-        a(f"      const {rt.type_name(ro.dtype.name)}* {nm}_row = {nm} + {ro.offset}L + ((rr / {ro.div}) % {ro.mod}) * {d};")
+    for i_, (nm, ro) in enumerate(zip(re_args, re.row_operands)):
+        mod = c_value(mods[i_]) if mods is not None else str(ro.mod)
+        a(f"      const {rt.type_name(ro.dtype.name)}* {nm}_row = {nm} + {ro.offset}L + ((rr / {ro.div}) % {mod}) * {d};")
         a(f"      {nm}_v[it] = *(const {vt_chunk}*)({nm}_row + gc);")
     a("    }")
     a("  }")
@@ -231,6 +233,18 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     gm, gn = xcd_block(tiles_m, tiles_n, TM, TN, ctx.xcds)
     KT = -(-K // BK)
     m_guard = M % TM != 0
+    # Symbolic row count (``body.sym`` marks ``m`` as ``a * seq_len + b``): M, the tile counts and the launch size
+    # become expressions over the kernel's trailing ``int`` parameter, rows are always guarded, and an XCD owns
+    # one-tile-row blocks (the compact block shape above is a function of the tile counts).
+    sym = getattr(body, "sym", None)
+    m_sym = sym.fields.get("m") if sym is not None else None
+    if m_sym is not None:
+        if split is not None or stage.transport == "ks":
+            raise LoweringError("contraction: a symbolic row count does not combine with a cross-workgroup split or the few-row form")
+        m_guard = True
+        gm = 1
+        while tiles_n % gn:
+            gn -= 1
     n_guard = N % TN != 0
     dli = stage.transport == "dli"  # direct to LDS, requests issued between the MFMAs of the slab before (see below)
     dl = stage.transport in ("dl", "dli")
@@ -279,6 +293,9 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
             raise LoweringError("contraction: the row epilogue needs a plain result and output tiles of whole column groups")
         params += [f"const {rt.type_name(ro.dtype.name)}* __restrict__ {nm}" for nm, ro in zip(re_args, rowepi.row_operands)]
     params.append(f"{out_c}* __restrict__ O")
+    sym_for_params = getattr(body, "sym", None)
+    if sym_for_params is not None and sym_for_params.fields:
+        params.append(f"int {sym_for_params.name}")
 
     D = dict(
         name=name, T=T, M=M, N=N, K=K, LDA=lda, LDB=ldb, LDO=ldo, TM=TM, TN=TN, BK=BK, WM=WM, WN=WN, FM=FM, FN=FN,
@@ -291,8 +308,10 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     o: list[str] = []
     a = o.append
     a(f"// {name}: M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()} xcd-block={gm}x{gn}")
+    if m_sym is not None:
+        D.update(M=m_sym.c(), TILES_M="((M + TM - 1) / TM)", NTILES="(TILES_M * TILES_N)")
     for k_, v_ in D.items():
-        if isinstance(v_, int):
+        if isinstance(v_, int) or (m_sym is not None and k_ in ("M", "TILES_M", "NTILES")):
             a(f"#define {k_} {v_}")
     a(r"""
 EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
@@ -305,7 +324,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   const int slot = bid / XCDS;
   constexpr int PER_BLOCK = GM * GN;
   constexpr int BLOCKS_N = TILES_N / GN;
-  constexpr int NBLOCKS = (TILES_M / GM) * BLOCKS_N;
+  const int NBLOCKS = (TILES_M / GM) * BLOCKS_N;
   int tm, tn;
   {
     // XCD x owns tile blocks x, x+XCDS, ...; `slot` walks the tiles of those blocks.
@@ -802,13 +821,16 @@ ROW_EPILOGUE_TABLES
     # and are not looked at before the k loop is over.
     tables: list[str] = []
     if rowepi is not None:
-        _emit_row_epilogue_tables(tables.append, rowepi, re_args, EPC, m_guard)
+        mods = [sym.fields.get(f"row_epilogue.row_operands.{i_}.mod", ro.mod) for i_, ro in enumerate(rowepi.row_operands)] if sym is not None else None
+        _emit_row_epilogue_tables(tables.append, rowepi, re_args, EPC, m_guard, mods)
     source = prelude.header(prelude.DMA, vm_macro, *((prelude.WAVE_REDUCE,) if rowepi is not None else ())) + "\n".join(o).replace("ROW_EPILOGUE_TABLES", "\n".join(tables)) + "\n"
     if N % 4 or TN % 4:
         raise LoweringError("contraction: N must be a multiple of 4 (8-byte output runs)")
     n_blocks = (tiles_m // gm) * (tiles_n // gn)
     rounds = -(-n_blocks // ctx.xcds)
     grid = rounds * ctx.xcds * gm * gn
+    if m_sym is not None:
+        grid = XcdRounds(m_sym, TM, tiles_n // gn, gn, ctx.xcds)
     return HipOp(
         kernel_source=source,
         kernel_name=name,
@@ -824,6 +846,7 @@ ROW_EPILOGUE_TABLES
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
         knobs={"TILE": plan.spell(), "STAGE": stage.spell()},
+        runtime_args=(sym.name,) if sym is not None and sym.fields else (),
     )
 
 

@@ -45,6 +45,7 @@ from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir.expr import float_literal
 from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.sym import Affine, CeilDiv, c_value
 from deplodock_amd.ir.tile import Flash
 
 # The key range of a workgroup's query rows is split over KVS wave groups.  Group g
@@ -73,7 +74,7 @@ typedef short emh_s16x4 __attribute__((ext_vector_type(4)));
 #define OACC(f) oacc[(f) / 16][(f) % 16]
 
 extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q, const ELT* __restrict__ Kp,
-                                                      const ELT* __restrict__ Vp, ELT* __restrict__ Op) {
+                                                      const ELT* __restrict__ Vp, ELT* __restrict__ Op SYM_PARAM) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // [2 buffers][group][K | V][key][d]
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int grp = wave / WQ, wq = wave % WQ;
@@ -450,6 +451,19 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         raise LoweringError("flash: offsets break 16-byte alignment")
     qblocks = -(-body.q_len // BQ)
     pair = bool(body.pair)
+    # Symbolic lengths (``body.sym``): SQ / SKV, the query-block count, the launch size and a [B, H, S, D] tensor's
+    # batch stride become expressions over the kernel's trailing ``int`` parameter; every guard the loop has for
+    # ragged lengths (row clamps, key masks, the causal block limit) already reads them at run time.
+    sym = getattr(body, "sym", None)
+    symf = sym.fields if sym is not None else {}
+    if symf:
+        if pair:
+            raise LoweringError("flash: mirrored query-block pairs need a block count known when the kernel is built")
+        for key in symf:
+            if key not in ("q_len", "kv_len") and not (key.split(".")[0] in ("q_strides", "k_strides", "v_strides", "o_strides") and key.split(".")[1] in ("0", "1", "2")):
+                raise LoweringError(f"flash: {key} cannot follow a symbolic axis")
+            if isinstance(symf[key], Affine) and "strides" in key and (symf[key].a % 8 or symf[key].b % 8):
+                raise LoweringError(f"flash: {key} = {symf[key]} does not keep 16-byte alignment at every size")
     if pair and not (body.causal and qblocks % 2 == 0):
         raise LoweringError("flash: pairing mirrored query blocks needs a causal mask and an even block count")
     qslots = qblocks // 2 if pair else qblocks
@@ -464,12 +478,13 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "CPR": D // 8,
         "KRPL": max(1, 16 // (D // 8)),
         "TG": min(4, D // 32),
-        "SQ": body.q_len,
-        "SKV": body.kv_len,
+        "SQ": c_value(symf.get("q_len", body.q_len)),
+        "SKV": c_value(symf.get("kv_len", body.kv_len)),
         "HQ": body.q_heads,
         "GROUP": body.q_heads // body.kv_heads,
-        "QBLOCKS": qblocks,
-        "QSLOTS": qslots,
+        "QBLOCKS": "((SQ + BQ - 1) / BQ)" if "q_len" in symf else qblocks,
+        "QSLOTS": "QBLOCKS" if "q_len" in symf else qslots,
+        "SYM_PARAM": f", int {sym.name}" if symf else "",
         "PAIR": 1 if pair else 0,
         "Q_LDS": 1 if plan["q_off"] is not None else 0,
         "Q_OFF_LDS": plan["q_off"] or 0,
@@ -477,10 +492,10 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "PARK_ML": plan["park_ml"],
         "CAUSAL": 1 if body.causal else 0,
         "SCALE_LOG2": float_literal(body.scale * math.log2(math.e)),
-        "Q_SB": body.q_strides[0], "Q_SH": body.q_strides[1], "Q_SS": body.q_strides[2], "Q_OFF": body.q_offset,
-        "K_SB": body.k_strides[0], "K_SH": body.k_strides[1], "K_SS": body.k_strides[2], "K_OFF": body.k_offset,
-        "V_SB": body.v_strides[0], "V_SH": body.v_strides[1], "V_SS": body.v_strides[2], "V_OFF": body.v_offset,
-        "O_SB": body.o_strides[0], "O_SH": body.o_strides[1], "O_SS": body.o_strides[2], "O_OFF": body.o_offset,
+        "Q_SB": c_value(symf.get("q_strides.0", body.q_strides[0])), "Q_SH": c_value(symf.get("q_strides.1", body.q_strides[1])), "Q_SS": c_value(symf.get("q_strides.2", body.q_strides[2])), "Q_OFF": body.q_offset,
+        "K_SB": c_value(symf.get("k_strides.0", body.k_strides[0])), "K_SH": c_value(symf.get("k_strides.1", body.k_strides[1])), "K_SS": c_value(symf.get("k_strides.2", body.k_strides[2])), "K_OFF": body.k_offset,
+        "V_SB": c_value(symf.get("v_strides.0", body.v_strides[0])), "V_SH": c_value(symf.get("v_strides.1", body.v_strides[1])), "V_SS": c_value(symf.get("v_strides.2", body.v_strides[2])), "V_OFF": body.v_offset,
+        "O_SB": c_value(symf.get("o_strides.0", body.o_strides[0])), "O_SH": c_value(symf.get("o_strides.1", body.o_strides[1])), "O_SS": c_value(symf.get("o_strides.2", body.o_strides[2])), "O_OFF": body.o_offset,
         "ELT": rt.type_name(body.dtype.name),
         "FRAG": rt.vector_type(body.dtype.name, 8)[0],
         "PACK4": rt.vector_type(body.dtype.name, 4)[0],
@@ -495,15 +510,16 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     head = f"// {name}: B={body.batch} Hq={body.q_heads} Hkv={body.kv_heads} Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal}\n"
     head += "".join(f"#define {k} {v}\n" for k, v in defs.items())
     grid = qslots * body.q_heads * body.batch
-    head += f"#define GRID {grid}\n#define XCDS {ctx.xcds}\n"
+    head += f"#define GRID {'((int)gridDim.x)' if 'q_len' in symf else grid}\n#define XCDS {ctx.xcds}\n"
     source = prelude.header(prelude.DMA) + head + _SRC
     return HipOp(
         kernel_source=source,
         kernel_name=name,
         arg_order=(body.q, body.k, body.v, body.out),
-        grid=((grid,), (1,), (1,)),
+        grid=((CeilDiv(symf["q_len"], BQ), body.q_heads * body.batch) if "q_len" in symf else (grid,), (1,), (1,)),
         block=((NT,), (1,), (1,)),
         lds_bytes=lds,
+        runtime_args=(sym.name,) if symf else (),
         comment=f"flash Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} bkv={BKV} split={kvs} pair={int(pair)}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),

@@ -15,6 +15,7 @@ from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.emit.reduce import _load_vec, _store_vec
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.sym import CeilDiv, c_value
 from deplodock_amd.ir.tile import Map
 
 _T = 256
@@ -33,14 +34,29 @@ def emit_map(body: Map, name: str, ctx: Context = Context()) -> HipOp:
         V //= 2
     chunks = body.numel // V
     grid = max(1, -(-chunks // _T))
+    # Symbolic extent (``body.sym``): the element count is an expression over the kernel's trailing ``int``
+    # parameter; the vector width must divide it at every size, i.e. divide both coefficients.
+    sym = getattr(body, "sym", None)
+    symf = sym.fields if sym is not None else {}
+    chunks_c = str(chunks) + "L"
+    if symf:
+        if set(symf) != {"numel"}:
+            raise LoweringError(f"map: {sorted(symf)} cannot follow a symbolic axis")
+        n_sym = symf["numel"]
+        while V > 1 and (n_sym.a % V or n_sym.b % V):
+            V //= 2
+        chunks_c = f"((long){c_value(n_sym)} / {V})"
+        grid = CeilDiv(n_sym, V * _T)
     params = [f"const {rt.type_name(o.dtype.name)}* __restrict__ p{i}" for i, o in enumerate(body.operands)]
     params.append(f"{rt.type_name(body.out_dtype.name)}* __restrict__ out")
+    if symf:
+        params.append(f"int {sym.name}")
     o: list[str] = []
     a = o.append
     a(f"// {name}: numel={body.numel} vec={V}")
     a(f'extern "C" __global__ __launch_bounds__({_T}) void {name}({", ".join(params)}) {{')
     a(f"  const long c = (long)blockIdx.x * {_T} + threadIdx.x;")
-    a(f"  if (c >= {chunks}L) return;")
+    a(f"  if (c >= {chunks_c}) return;")
     for i, op in enumerate(body.operands):
         a(f"  float v{i}[{V}];")
         if op.index == "flat":
@@ -67,5 +83,6 @@ def emit_map(body: Map, name: str, ctx: Context = Context()) -> HipOp:
         grid=((grid,), (1,), (1,)),
         block=((_T,), (1,), (1,)),
         comment=f"map numel={body.numel}",
+        runtime_args=(sym.name,) if symf else (),
         algo_bytes=body.algo_bytes(),
     )

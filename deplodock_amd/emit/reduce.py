@@ -27,6 +27,7 @@ from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.sym import CeilDiv, c_value
 from deplodock_amd.ir.tile import RowAddr, RowReduce
 
 _MAX_RESIDENT = 64  # fp32 row elements a lane may keep in registers
@@ -119,12 +120,20 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
     if T > ctx.max_threads_per_block or T % L:
         raise LoweringError(f"row reduce: {T} threads per workgroup is not launchable")
     R = T // L
+    # Symbolic row count (``body.sym``): rows and table extents become expressions over the kernel's trailing
+    # ``int`` parameter, the row guard is always there and the grid is sized at launch.
+    sym = getattr(body, "sym", None)
+    symf = sym.fields if sym is not None else {}
+    for key in symf:
+        if key != "rows" and not (key.startswith("row_operands.") and key.endswith(".mod")):
+            raise LoweringError(f"row reduce: {key} cannot follow a symbolic axis")
+    rows_c = c_value(symf.get("rows", body.rows))
     # Do not spread fewer rows than one workgroup holds over idle lanes.
-    while R > 1 and R > body.rows and T > ctx.wave_size:
+    while "rows" not in symf and R > 1 and R > body.rows and T > ctx.wave_size:
         R //= 2
         T = L * R
-    grid = -(-body.rows // R)
-    row_guard = body.rows % R != 0
+    grid = CeilDiv(symf["rows"], R) if "rows" in symf else -(-body.rows // R)
+    row_guard = "rows" in symf or body.rows % R != 0
     NW = max(1, L // ctx.wave_size)  # waves per row
     W = min(L, ctx.wave_size)  # butterfly width
 
@@ -146,6 +155,8 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
     params += [f"const {rt.type_name(dt.name)}* __restrict__ c{ci}" for ci, (_, dt) in enumerate(body.col_operands)]
     params += [f"const {rt.type_name(ro.dtype.name)}* __restrict__ r{ri}" for ri, ro in enumerate(body.row_operands)]
     params.append(f"{rt.type_name(body.out_dtype.name)}* __restrict__ out")
+    if symf:
+        params.append(f"int {sym.name}")
 
     o: list[str] = []
     a = o.append
@@ -155,8 +166,8 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
     a(f"  const int rib = threadIdx.x / {L};")
     a(f"  long row = (long)blockIdx.x * {R} + rib;")
     if row_guard:
-        a(f"  const bool row_ok = row < {body.rows}L;")
-        a(f"  if (!row_ok) row = {body.rows - 1}L;")
+        a(f"  const bool row_ok = row < (long){rows_c};")
+        a(f"  if (!row_ok) row = (long){rows_c} - 1;")
     a(f"  const {rt.type_name(body.x_dtype.name)}* xr = x + ({_row_offset(x_addr, 'row')});")
     a(f"  float xv[{NV}][{V}];")
     if masked:
@@ -177,7 +188,8 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
 
     if not body.scalar_out:
         for ri, ro in enumerate(body.row_operands):
-            a(f"  const {rt.type_name(ro.dtype.name)}* rrow{ri} = r{ri} + {ro.offset}L + ((row / {ro.div}) % {ro.mod}) * {body.cols}L;")
+            mod = c_value(symf.get(f"row_operands.{ri}.mod", ro.mod))
+            a(f"  const {rt.type_name(ro.dtype.name)}* rrow{ri} = r{ri} + {ro.offset}L + ((row / {ro.div}) % {mod}) * {body.cols}L;")
 
     def operand_loads(i: int, indent: str, tag: str = "") -> None:
         idx = f"{i * L} + lane"
@@ -265,6 +277,7 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
             comment=f"row_reduce rows={body.rows} cols={body.cols} REDUCE={plan.spell()} one value per row",
             algo_bytes=body.algo_bytes(),
             knobs={"REDUCE": plan.spell(), "VEC": V, "NT": int(nontemporal)},
+            runtime_args=(sym.name,) if symf else (),
         )
     a(f"  {rt.type_name(body.out_dtype.name)}* orow = out + ({_row_offset(out_addr, 'row')});")
 
@@ -341,6 +354,7 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
         comment=f"row_reduce rows={body.rows} cols={body.cols} REDUCE={plan.spell()}",
         algo_bytes=body.algo_bytes(),
         knobs={"REDUCE": plan.spell(), "VEC": V, "NT": int(nontemporal)},
+        runtime_args=(sym.name,) if symf else (),
     )
 
 

@@ -44,6 +44,22 @@ def _online_pair(stats: tuple[Stat, ...], i: int) -> bool:
 
 
 def emit_row_reduce_streaming(body: RowReduce, name: str, ctx: Context = Context()) -> HipOp:
+    if getattr(body, "sym", None) is not None and body.sym.fields:
+        return _emit_streaming_symbolic_rows(body, name, ctx)
+    return _emit_streaming(body, name, ctx)
+
+
+def _emit_streaming_symbolic_rows(body: RowReduce, name: str, ctx: Context) -> HipOp:
+    """One workgroup per row whatever the row count: the kernel never reads it, only the launch size follows it."""
+    sym = body.sym
+    if set(sym.fields) != {"rows"}:
+        raise LoweringError(f"streamed row reduce: {sorted(sym.fields)} cannot follow a symbolic axis")
+    op = _emit_streaming(body, name, ctx)
+    op.grid = ((sym.fields["rows"],), (1,), (1,))
+    return op
+
+
+def _emit_streaming(body: RowReduce, name: str, ctx: Context = Context()) -> HipOp:
     if body.rotate is not None or body.row_operands:
         raise LoweringError("row reduce: the streaming form has no rotate-half / per-row tables")
     x_addr = body.x_addr or RowAddr.uniform(body.cols)

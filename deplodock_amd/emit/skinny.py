@@ -51,6 +51,8 @@ def skinny_waves(body: Contraction) -> int:
     """Waves that split the reduction axis (0: the shape does not take this form)."""
     if body.m > 16 or body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None or body.reduce.cta != 1:
         return 0
+    if getattr(body, "sym", None) is not None and "m" in body.sym.fields:
+        return 0  # the few-row form holds every row in one MFMA tile: not with a row count known only at launch
     if body.in_dtype.name not in ("bf16", "f16") or body.k % 32 or body.n % 4:
         return 0
     for kw in (8, 4, 2, 1):

@@ -512,6 +512,8 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 if body.kv_split == 1:
                     break
                 body.kv_split //= 2
+    if getattr(body, "sym", None) is not None and body.sym.fields:
+        body.pair = False  # pairing mirrored query blocks needs the block count when the kernel is built
     return {"FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "")}
 
 

@@ -371,24 +371,121 @@ def test_run_api_returns_host_arrays_with_bf16_as_bits(device):
     eager.assert_close(torch.from_numpy(O.from_bf16_bits(out)), want, 2e-2, 2e-2, "run() output")
 
 
-def test_c5_block_dynamic_seq_len(device):
-    """One compile with a symbolic ``seq_len``; runs at other lengths go through the per-size variants."""
+def test_c5_block_dynamic_seq_len(device, monkeypatch):
+    """One compile with a symbolic ``seq_len``: every kernel takes the length as a runtime ``int``, so the same five
+    code objects run the block at every length — at most one hipRTC compile and one loaded module per kernel across
+    all of them — and each length matches eager (ragged lengths exercise the row / key-block guards)."""
+    from deplodock_amd.backend.hip import hiprtc, launcher
+
     case = eager.qwen3_block_case(seq=64)
     be = HipBackend()
     compiled = be.compile(trace_module(case.module, case.inputs, dynamic_shapes={"x": {1: "seq_len"}, "cos": {1: "seq_len"}, "sin": {1: "seq_len"}}))
-    for seq in (64, 96, 32):
+    assert compiled.symbolic == "seq_len"
+    ops = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert len(ops) == 5 and all(op.runtime_args == ("seq_len",) for op in ops)
+    compiles: list[str] = []
+    real = launcher.Launcher.compile
+    monkeypatch.setattr(launcher.Launcher, "compile", lambda self, source, name, arch, options: compiles.append(name) or real(self, source, name, arch, options))
+    before = hiprtc.loaded_module_count()
+    for seq in (64, 96, 32, 200, 7, 513):
         other = eager.qwen3_block_case(seq=seq)
         data = {n: t.to(device) for n, t in zip(compiled.inputs, other.inputs)}
         prog = be.program(compiled, data)
         try:
+            assert prog.sym_values == {"seq_len": seq}
             prog.run()
             torch.cuda.synchronize()
             ours = prog.output_tensors()[compiled.outputs[0]]
+            assert tuple(ours.shape) == (1, seq, 1024)
             want = eager.run_eager(other, device)
-            eager.assert_close(ours.reshape(want.shape), want, other.rtol, other.atol, f"block with seq_len={seq} through a seq_len=64 compile")
+            eager.assert_close(ours.reshape(want.shape), want, other.rtol, other.atol, f"block with seq_len={seq} through the runtime-int kernels")
+            exact = eager.run_eager_fp32(other, device)
+            x = other.inputs[0].to(device).float()
+            eager.assert_mean_error_within_baseline(ours.float() - x, want.float() - x, exact - x, 1.5, f"block seq_len={seq} (out - x) vs fp32 eager")
         finally:
             prog.close()
-    assert len(compiled.variants) == 3
+    assert len(compiles) <= 5 and len(set(compiles)) == len(compiles), compiles
+    assert hiprtc.loaded_module_count() - before <= 5
+    # a captured graph of one length replays correctly after programs of other lengths ran in between
+    data = {n: t.to(device) for n, t in zip(compiled.inputs, eager.qwen3_block_case(seq=96).inputs)}
+    prog = be.program(compiled, data)
+    try:
+        prog.capture_program_graph()
+        for _ in range(3):
+            prog.output_tensors()[compiled.outputs[0]].zero_()
+            prog.replay_program()
+            torch.cuda.synchronize()
+            want = eager.run_eager(eager.qwen3_block_case(seq=96), device)
+            eager.assert_close(prog.output_tensors()[compiled.outputs[0]].reshape(want.shape), want, 2e-2, 4e-2, "graph replay at seq_len=96")
+    finally:
+        prog.close()
+
+
+def test_dynamic_seq_len_per_size_variants_still_work(device):
+    """The fallback for modules that do not symbolise (forced here): a re-trace and re-lowering per size."""
+    case = eager.qwen3_block_case(seq=64)
+    be = HipBackend()
+    be.symbolic_kernels = False
+    compiled = be.compile(trace_module(case.module, case.inputs, dynamic_shapes={"x": {1: "seq_len"}, "cos": {1: "seq_len"}, "sin": {1: "seq_len"}}))
+    for seq in (64, 96):
+        other = eager.qwen3_block_case(seq=seq)
+        prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, other.inputs)})
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            want = eager.run_eager(other, device)
+            eager.assert_close(prog.output_tensors()[compiled.outputs[0]].reshape(want.shape), want, other.rtol, other.atol, f"block with seq_len={seq} through a per-size variant")
+        finally:
+            prog.close()
+    assert len(compiled.variants) == 2
+
+
+@pytest.mark.parametrize("which", ["rms_norm", "softmax", "silu_mul", "sdpa", "linear_bias"])
+def test_runtime_int_kernels_of_every_family(device, which):
+    """Row kernels (rows symbolic), a pointwise map (element count symbolic), attention on ``[B, H, S, D]`` operands
+    (lengths and the batch stride symbolic) and a biased linear (rows symbolic), each compiled once and run at
+    several sizes of the axis, including sizes below one tile and sizes that leave ragged tiles."""
+
+    class SiluMul(nn.Module):
+        def forward(self, x, y):
+            return nn.functional.silu(x) * y
+
+    torch.manual_seed(12)
+    if which == "rms_norm":
+        mod = nn.RMSNorm(1024, eps=1e-6).eval()
+        make = lambda s: (torch.randn(2, s, 1024),)  # noqa: E731
+        dyn, tol = {"x": {1: "s"}}, (1e-5, 1e-6)
+    elif which == "softmax":
+        mod = nn.Softmax(dim=-1).eval()
+        make = lambda s: (torch.randn(s, 777),)  # noqa: E731
+        dyn, tol = {"input": {0: "s"}}, (1e-5, 1e-9)
+    elif which == "silu_mul":
+        mod = SiluMul().eval()
+        make = lambda s: (torch.randn(s, 96).bfloat16(), torch.randn(s, 96).bfloat16())  # noqa: E731
+        dyn, tol = {"x": {0: "s"}, "y": {0: "s"}}, (2e-2, 2e-2)
+    elif which == "sdpa":
+        mod = eager.Sdpa(True).eval()
+        make = lambda s: (torch.randn(2, 4, s, 128).bfloat16(), torch.randn(2, 2, s, 128).bfloat16(), torch.randn(2, 2, s, 128).bfloat16())  # noqa: E731
+        dyn, tol = {"q": {2: "s"}, "k": {2: "s"}, "v": {2: "s"}}, (2e-2, 2e-2)
+    else:
+        mod = nn.Linear(256, 520).bfloat16().eval()
+        make = lambda s: (torch.randn(s, 256).bfloat16(),)  # noqa: E731
+        dyn, tol = {"input": {0: "s"}}, (2e-2, 2e-2)
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, make(48), dynamic_shapes=dyn))
+    assert compiled.symbolic == "s"
+    assert all(n.op.runtime_args == ("s",) for n in compiled.nodes.values() if isinstance(n.op, HipOp))
+    for size in (48, 1, 200, 33):
+        inputs = make(size)
+        prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, inputs)})
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            with torch.no_grad():
+                want = mod.to(device)(*(t.to(device) for t in inputs))
+            eager.assert_close(prog.output_tensors()[compiled.outputs[0]].reshape(want.shape), want, *tol, f"{which} at s={size}")
+        finally:
+            prog.close()
 
 
 class _HfRmsNorm(nn.Module):

@@ -10,8 +10,11 @@ import torch
 from torch import nn
 
 from deplodock_amd import HipBackend, trace_module
+from deplodock_amd.ir.sym import Affine as Affine_
 from deplodock_amd.backend.hip import hiprtc
 from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.dtype import F32
+from deplodock_amd.ir import expr as E
 from oracle import eager
 
 
@@ -266,14 +269,49 @@ def test_cache_is_content_addressed(launcher_lib, tmp_path, monkeypatch):
     assert not list(tmp_path.glob("*.tmp"))
 
 
-def test_dynamic_shapes_are_specialised_per_size(launcher_lib):
-    """``dynamic_shapes`` marks axes; the backend re-traces and re-lowers per distinct size and keeps an LRU."""
+def test_a_symbolic_axis_lowers_to_kernels_that_take_it_as_a_runtime_int(launcher_lib):
+    """``dynamic_shapes`` marks axes.  With one symbolic axis the module lowers once: every kernel whose work
+    follows the axis takes ``int seq_len`` as a trailing parameter, guards its rows / key blocks at run time and is
+    launched on a grid the runtime sizes per launch (the reference's form: ir/kernel/ir.py:258-276,
+    ir/cuda/ir.py:66-112).  One code object per kernel then serves every length."""
+    from deplodock_amd.ir.sym import Affine, CeilDiv, XcdRounds
+
     case = eager.qwen3_block_case(seq=64)
     g = trace_module(case.module, case.inputs, dynamic_shapes={"x": {1: "seq_len"}, "cos": {1: "seq_len"}, "sin": {1: "seq_len"}})
     assert g.dynamic.hints == {"seq_len": 64} and g.dynamic.input_axes == [{1: "seq_len"}] * 3
     be = HipBackend()
     compiled = be.compile(g)
-    assert be.variant(compiled, None) is compiled
+    assert compiled.symbolic == "seq_len" and not hasattr(compiled, "variants")
+    ks = kernels(compiled)
+    assert len(ks) == 5
+    for k in ks:
+        assert k.runtime_args == ("seq_len",) and k.kernel_source.count("int seq_len") == 1
+        hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+    flash = next(k for k in ks if k.kernel_name.startswith("k_sdpa"))
+    assert flash.grid[0] == (CeilDiv(Affine("seq_len", 1, 0), 32 * int(flash.knobs["FLASH"].split("/")[0][1:])), 16) and "/p" not in flash.knobs["FLASH"]
+    assert "#define SQ (seq_len)" in flash.kernel_source and "#define GRID ((int)gridDim.x)" in flash.kernel_source
+    lin = next(k for k in ks if k.kernel_name.startswith("k_linear_add"))
+    assert isinstance(lin.grid[0][0], XcdRounds) and "#define M (seq_len)" in lin.kernel_source and "/ks" not in lin.knobs["STAGE"]
+    assert lin.grid[0][0]({"seq_len": 200}) >= -(-200 // lin.grid[0][0].tile_m) * lin.grid[0][0].blocks_n * lin.grid[0][0].per_block
+    assert compiled.nodes["x"].output.shape == (1, "seq_len", 1024) and compiled.nodes[compiled.outputs[0]].output.shape == (1, "seq_len", 1024)
+
+    def inputs_at(s):
+        return {n: torch.zeros([s if i == 1 else d for i, d in enumerate(t.shape)], dtype=t.dtype) for n, t in zip(compiled.inputs, case.inputs)}
+
+    assert be.variant(compiled, inputs_at(96)) is compiled and be.variant(compiled, None) is compiled  # no per-size lowering
+    with pytest.raises(NotImplementedError, match="not arguments"):
+        trace_module(case.module, case.inputs, dynamic_shapes={"nope": {1: "s"}})
+
+
+def test_per_size_specialisation_remains_for_what_does_not_symbolise(launcher_lib):
+    """With runtime-int kernels switched off (or a module whose kernel boundaries change with the size) the backend
+    re-traces and re-lowers per distinct size and keeps an LRU of the results."""
+    case = eager.qwen3_block_case(seq=64)
+    g = trace_module(case.module, case.inputs, dynamic_shapes={"x": {1: "seq_len"}, "cos": {1: "seq_len"}, "sin": {1: "seq_len"}})
+    be = HipBackend()
+    be.symbolic_kernels = False
+    compiled = be.compile(g)
+    assert getattr(compiled, "symbolic", None) is None and be.variant(compiled, None) is compiled
 
     def inputs_at(s):
         return {n: torch.zeros([s if i == 1 else d for i, d in enumerate(t.shape)], dtype=t.dtype) for n, t in zip(compiled.inputs, case.inputs)}
@@ -281,8 +319,7 @@ def test_dynamic_shapes_are_specialised_per_size(launcher_lib):
     assert be.variant(compiled, inputs_at(64)) is compiled
     v96 = be.variant(compiled, inputs_at(96))
     assert v96 is not compiled and be.variant(compiled, inputs_at(96)) is v96
-    assert v96.nodes[v96.outputs[0]].output.shape[-2:] == (96, 1024) or 96 in v96.nodes[v96.outputs[0]].output.shape
-    assert v96.inputs == compiled.inputs and v96.outputs == compiled.outputs
+    assert 96 in v96.nodes[v96.outputs[0]].output.shape and v96.inputs == compiled.inputs and v96.outputs == compiled.outputs
     for s in range(1, 12):
         be.variant(compiled, inputs_at(32 * s + 32))
     assert len(compiled.variants) == HipBackend.VARIANT_CACHE
@@ -290,8 +327,27 @@ def test_dynamic_shapes_are_specialised_per_size(launcher_lib):
     bad[compiled.inputs[1]] = torch.zeros(1, 80, 128, dtype=torch.bfloat16)
     with pytest.raises(ValueError, match="disagree"):
         be.variant(compiled, bad)
-    with pytest.raises(NotImplementedError, match="not arguments"):
-        trace_module(case.module, case.inputs, dynamic_shapes={"nope": {1: "s"}})
+
+
+def test_symbolize_refuses_what_a_runtime_int_cannot_express():
+    from deplodock_amd.graph import Graph, Tensor
+    from deplodock_amd.ir.tile import RowReduce, Stat, TileOp
+    from deplodock_amd.passes.symbolic import SymbolicError, symbolize
+
+    def tile(rows, cols):
+        g = Graph()
+        g.add_input("X", (rows, cols))
+        body = RowReduce(rows=rows, cols=cols, x="X", x_dtype=F32, out="y", out_dtype=F32, stats=(Stat("s", "sum", E.Var("x")),), project=E.Var("x") / E.Var("s"))
+        g.add_node(TileOp(name="k_n", body=body), ["X"], Tensor("y", (rows, cols), F32))
+        g.outputs = ["y"]
+        return g
+
+    ok = symbolize([tile(8, 64), tile(15, 64), tile(104, 64)], "rows", [8, 15, 104])
+    assert ok.nodes["y"].op.body.sym.fields == {"rows": Affine_("rows", 1, 0)}
+    with pytest.raises(SymbolicError, match="cols"):  # the reduced extent is baked into the kernel
+        symbolize([tile(8, 64), tile(8, 71), tile(8, 160)], "cols", [64, 71, 160])
+    with pytest.raises(SymbolicError, match="not affine"):
+        symbolize([tile(8, 64), tile(16, 64), tile(100, 64)], "rows", [8, 15, 104])
 
 
 def test_elementwise_trees_fold_into_one_map_kernel(launcher_lib):
