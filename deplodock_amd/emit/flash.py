@@ -74,7 +74,7 @@ typedef short emh_s16x4 __attribute__((ext_vector_type(4)));
 #define OACC(f) oacc[(f) / 16][(f) % 16]
 
 extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q, const ELT* __restrict__ Kp,
-                                                      const ELT* __restrict__ Vp, ELT* __restrict__ Op SYM_PARAM) {
+                                                      const ELT* __restrict__ Vp MASK_PARAM, ELT* __restrict__ Op SYM_PARAM) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // [2 buffers][group][K | V][key][d]
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int grp = wave / WQ, wq = wave % WQ;
@@ -227,6 +227,27 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+#if HAS_MASK
+      {
+        // The additive mask: this lane's query row, the keys of its accumulator rows (runs of four consecutive
+        // keys).  Added before the scale is applied, divided by it, so the exponent's fma sees s * scale + mask.
+        const MELT* mrow_ = Mp + M_OFF + (long)batch * M_SB + (long)head * M_SH + (long)(qrow < SQ ? qrow : SQ - 1) * M_SS;
+        #pragma unroll
+        for (int u = 0; u < BKV / 32; ++u)
+        #pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int key0 = k0 + 32 * u + 8 * g4 + 4 * lh;
+          if (MASK_VEC && key0 + 3 < SKV) {
+            const MVEC4 mv_ = *(const MVEC4*)(mrow_ + key0);
+            #pragma unroll
+            for (int j = 0; j < 4; ++j) sacc[u][4 * g4 + j] += (float)mv_[j] * INV_SCALE;
+          } else {
+            #pragma unroll
+            for (int j = 0; j < 4; ++j) if (key0 + j < SKV) sacc[u][4 * g4 + j] += (float)mrow_[key0 + j] * INV_SCALE;
+          }
+        }
+      }
+#endif
       float mx = -1.0e30f;
       if ((CAUSAL && (k0 + BKV - 1 > qw0)) || (k0 + BKV > SKV)) {
         #pragma unroll
@@ -468,6 +489,16 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         raise LoweringError("flash: pairing mirrored query blocks needs a causal mask and an even block count")
     qslots = qblocks // 2 if pair else qblocks
     bf16 = body.dtype.name == "bf16"
+    has_mask = body.mask is not None
+    if has_mask:
+        if body.mask_dtype.name not in ("bf16", "f16", "f32"):
+            raise LoweringError("flash: the mask must be a floating-point tensor")
+        if symf:
+            raise LoweringError("flash: a mask operand does not combine with symbolic lengths")
+        if body.scale == 0.0:
+            raise LoweringError("flash: a mask with a zero scale is not supported")
+        # four keys per load (8 or 16 bytes) when every row of the mask starts on a four-element boundary
+        mask_vec = all(v % 4 == 0 for v in (*body.mask_strides, body.mask_offset))
     defs = {
         "KNAME": name,
         "NT": NT,
@@ -485,6 +516,11 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "QBLOCKS": "((SQ + BQ - 1) / BQ)" if "q_len" in symf else qblocks,
         "QSLOTS": "QBLOCKS" if "q_len" in symf else qslots,
         "SYM_PARAM": f", int {sym.name}" if symf else "",
+        "HAS_MASK": 1 if has_mask else 0,
+        "MASK_PARAM": f", const {rt.type_name(body.mask_dtype.name)}* __restrict__ Mp" if has_mask else "",
+        **({"MELT": rt.type_name(body.mask_dtype.name), "MVEC4": rt.vector_type(body.mask_dtype.name, 4)[0], "MASK_VEC": 1 if mask_vec else 0,
+            "M_SB": body.mask_strides[0], "M_SH": body.mask_strides[1], "M_SS": body.mask_strides[2], "M_OFF": body.mask_offset,
+            "INV_SCALE": float_literal(1.0 / body.scale)} if has_mask else {}),
         "PAIR": 1 if pair else 0,
         "Q_LDS": 1 if plan["q_off"] is not None else 0,
         "Q_OFF_LDS": plan["q_off"] or 0,
@@ -515,7 +551,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     return HipOp(
         kernel_source=source,
         kernel_name=name,
-        arg_order=(body.q, body.k, body.v, body.out),
+        arg_order=(body.q, body.k, body.v, *((body.mask,) if has_mask else ()), body.out),
         grid=((CeilDiv(symf["q_len"], BQ), body.q_heads * body.batch) if "q_len" in symf else (grid,), (1,), (1,)),
         block=((NT,), (1,), (1,)),
         lds_bytes=lds,

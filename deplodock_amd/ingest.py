@@ -126,10 +126,11 @@ def graph_from_reference_dict(data: dict, cast: DType | None = None) -> Graph:
         elif kind == "LinearOp":
             add(nid, F.LinearOp(has_bias=bool(fields.get("has_bias", False))), tensors)
         elif kind == "SdpaOp":
-            if len(tensors) != 3:
-                raise IngestError(f"node {nid!r}: attention with an explicit mask operand is not read")
+            if len(tensors) not in (3, 4):
+                raise IngestError(f"node {nid!r}: attention takes q, k, v and at most an additive mask")
             q, k = shape_of(tensors[0]), shape_of(tensors[1])
-            add(nid, F.SdpaOp(is_causal=bool(fields.get("is_causal", False)), scale=fields.get("scale"), enable_gqa=q[-3] != k[-3]), tensors)
+            masked = len(tensors) == 4  # an explicit mask replaces the causal term (decomposition/010_sdpa.py:91-101)
+            add(nid, F.SdpaOp(is_causal=not masked and bool(fields.get("is_causal", False)), scale=fields.get("scale"), enable_gqa=q[-3] != k[-3], has_mask=masked), tensors)
         elif kind in ("MeanOp", "SumOp"):
             rank = len(shape_of(tensors[0]))
             keep = len(shape_of(nid)) == rank

@@ -80,6 +80,7 @@ class SdpaOp(Op):
     is_causal: bool = False
     scale: float | None = None
     enable_gqa: bool = False
+    has_mask: bool = False  # a fourth input: an additive float bias on the scaled scores (emmy/compiler/trace/torch.py:559-583)
 
 
 @dataclass
@@ -103,6 +104,14 @@ class PermuteOp(Op):
 @dataclass
 class UnsqueezeOp(Op):
     dim: int = 0
+
+
+@dataclass
+class ExpandOp(Op):
+    """``expand``: size-1 dims (and new leading dims) repeated up to ``shape`` without moving data — every
+    repeated index reads element 0 (emmy/compiler/trace/torch.py:666-676: a broadcast, not a reshape)."""
+
+    shape: tuple = ()
 
 
 @dataclass

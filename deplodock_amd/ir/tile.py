@@ -267,6 +267,12 @@ class Flash:
     waves: int = 4  # 32-row query groups per workgroup
     kv_split: int = 1  # wave groups that split the key blocks of a query group between them
     pair: bool = False  # causal only: a workgroup takes query block b and its mirror QBLOCKS-1-b
+    # an additive bias on the scaled scores, ``[batch, head, query, key]`` addressed through (batch, head, query)
+    # strides (0 = broadcast) with keys contiguous; ``None``: no mask operand
+    mask: str | None = None
+    mask_dtype: DType | None = None
+    mask_strides: tuple[int, int, int] = (0, 0, 0)
+    mask_offset: int = 0
 
     def algo_flops(self) -> int:
         if self.causal and self.q_len == self.kv_len:
@@ -279,7 +285,11 @@ class Flash:
         e = self.dtype.nbytes
         q = self.batch * self.q_heads * self.q_len * self.head_dim
         kv = self.batch * self.kv_heads * self.kv_len * self.head_dim
-        return (2 * q + 2 * kv) * e
+        mask = 0
+        if self.mask is not None:
+            mb, mh, mq = self.mask_strides
+            mask = (self.batch if mb else 1) * (self.q_heads if mh else 1) * (self.q_len if mq else 1) * self.kv_len * self.mask_dtype.nbytes
+        return (2 * q + 2 * kv) * e + mask
 
 
 @dataclass

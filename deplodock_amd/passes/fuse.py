@@ -796,11 +796,33 @@ def _rope_internal(g: Graph, t_id: str, add_id: str) -> set[str]:
     return seen
 
 
+def _undo_repeat_kv(g: Graph, nid: str) -> tuple[str, int]:
+    """``(source, group)`` when ``nid`` is a KV tensor whose heads were repeated for grouped attention the
+    materialising way — ``x[:, :, None].expand(B, Hkv, group, S, D).reshape(B, Hkv * group, S, D)`` — so that
+    repeated head ``h`` reads source head ``h // group``: exactly what the kernel's grouped addressing does, with
+    no copy.  ``(nid, 1)`` otherwise."""
+    view, exp = g.nodes[nid], None
+    if isinstance(view.op, F.ContiguousOp):
+        view = g.nodes[view.inputs[0]]
+    if isinstance(view.op, F.ViewOp):
+        exp = g.nodes[view.inputs[0]]
+    if exp is None or not isinstance(exp.op, F.ExpandOp) or not _is(g.nodes[exp.inputs[0]], F.UnsqueezeOp, dim=2):
+        return nid, 1
+    src = g.nodes[exp.inputs[0]].inputs[0]
+    s_shape, e_shape, o_shape = (tuple(int(d) for d in g.nodes[n].output.shape) for n in (src, exp.id, view.id))
+    if len(s_shape) != 4 or e_shape != (*s_shape[:2], e_shape[2], *s_shape[2:]) or o_shape != (s_shape[0], s_shape[1] * e_shape[2], *s_shape[2:]):
+        return nid, 1
+    return src, e_shape[2]
+
+
 def _rec_sdpa(c: _Ctx, nid: str) -> bool:
     node = c.g.nodes[nid]
     if not isinstance(node.op, F.SdpaOp):
         return False
-    q, k, v = (_need_logical(c, i) for i in node.inputs)
+    (k_id, k_rep), (v_id, v_rep) = _undo_repeat_kv(c.g, node.inputs[1]), _undo_repeat_kv(c.g, node.inputs[2])
+    if k_rep != v_rep:
+        k_id, v_id, k_rep = node.inputs[1], node.inputs[2], 1
+    q, k, v = (_need_logical(c, i) for i in (node.inputs[0], k_id, v_id))
     if min(len(q.shape), len(k.shape), len(v.shape)) < 3:
         raise FusionError("sdpa: expected [batch..., heads, seq, head_dim] operands")
 
@@ -821,7 +843,7 @@ def _rec_sdpa(c: _Ctx, nid: str) -> bool:
         raise FusionError("sdpa: q, k and v must agree on the batch size")
     Hq, Sq, D = q.shape[-3:]
     Hkv, Skv = k.shape[-3], k.shape[-2]
-    if Hq != Hkv and not node.op.enable_gqa:
+    if Hq != Hkv and not (node.op.enable_gqa or k_rep > 1):
         raise FusionError("sdpa: grouped heads need enable_gqa=True")
     for t in (q, k, v):
         if t.strides[-1] != 1:
@@ -835,12 +857,21 @@ def _rec_sdpa(c: _Ctx, nid: str) -> bool:
     if transposed:
         o_shape, o_strides = (B, Sq, Hq, D), (Sq * Hq * D, D, Hq * D)
     scale = node.op.scale if node.op.scale is not None else 1.0 / math.sqrt(D)
+    mask_kw: dict = {}
+    inputs = [q.base, k.base, v.base]
+    if node.op.has_mask:
+        mv = _need_logical(c, node.inputs[3])
+        shp, st = (1,) * (4 - len(mv.shape)) + tuple(mv.shape), (0,) * (4 - len(mv.shape)) + tuple(mv.strides)
+        if len(shp) != 4 or shp[-1] != Skv or shp[-2] not in (1, Sq) or shp[0] not in (1, B) or shp[1] not in (1, Hq) or (shp[-1] > 1 and st[-1] != 1):
+            raise FusionError(f"sdpa: the mask must broadcast to [batch, heads, queries, keys] with contiguous keys, got {tuple(mv.shape)}")
+        mask_kw = dict(mask=mv.base, mask_dtype=mv.dtype, mask_offset=mv.offset, mask_strides=tuple(0 if n == 1 else s_ for n, s_ in zip(shp[:3], st[:3])))
+        inputs.append(mv.base)
     body = Flash(
         batch=B, q_heads=Hq, kv_heads=Hkv, q_len=Sq, kv_len=Skv, head_dim=D, q=q.base, k=k.base, v=v.base, out=out_id, dtype=q.dtype,
         scale=float(scale), causal=node.op.is_causal, q_strides=q_str, k_strides=k_str, v_strides=v_str, o_strides=o_strides,
-        q_offset=q.offset, k_offset=k.offset, v_offset=v.offset,
+        q_offset=q.offset, k_offset=k.offset, v_offset=v.offset, **mask_kw,
     )  # fmt: skip
-    _emit(c, nid, body, "sdpa_reduce", [q.base, k.base, v.base], shape=o_shape)
+    _emit(c, nid, body, "sdpa_reduce", inputs, shape=o_shape)
     if transposed or len(logical) != 4:
         # how the traced shape (with its batch dims as traced) maps onto the buffer (not a comparison of the shapes:
         # they read the same when there are as many tokens as heads)
@@ -916,6 +947,8 @@ def _rec_pointwise(c: _Ctx, nid: str) -> bool:
     operands, buffers, offsets = [], {}, {}
     for leaf_id, var in leaves.items():
         v = _need_logical(c, leaf_id)
+        if any(st == 0 and n > 1 for n, st in zip(v.shape, v.strides)):  # an expanded operand is its unit-size source, broadcast
+            v = View(v.base, v.offset, tuple(1 if st == 0 else n for n, st in zip(v.shape, v.strides)), v.strides, v.dtype)
         lead_ones = len(v.shape) >= 1 and all(d == 1 for d in v.shape[:-1])
         if v.shape == shape and v.is_contiguous():
             kind = "flat"

@@ -61,7 +61,7 @@ def contiguous_strides(shape: tuple[int, ...]) -> tuple[int, ...]:
     return tuple(reversed(out))
 
 
-LAYOUT_OPS = (F.ViewOp, F.TransposeOp, F.PermuteOp, F.UnsqueezeOp, F.SqueezeOp, F.SliceOp)
+LAYOUT_OPS = (F.ViewOp, F.TransposeOp, F.PermuteOp, F.UnsqueezeOp, F.SqueezeOp, F.SliceOp, F.ExpandOp)
 
 
 def _reshape_strides(shape: tuple[int, ...], strides: tuple[int, ...], new_shape: tuple[int, ...]) -> tuple[int, ...] | None:
@@ -139,6 +139,12 @@ def apply_layout(src: View, op, out_shape: tuple[int, ...], nid: str = "?") -> V
         sh.insert(op.dim, 1)
         st.insert(op.dim, 0)
         return View(src.base, src.offset, tuple(sh), tuple(st), src.dtype)
+    if isinstance(op, F.ExpandOp):
+        pad = len(out_shape) - len(src.shape)
+        if pad < 0 or any(n not in (1, o) for n, o in zip(src.shape, out_shape[pad:])):
+            raise NotViewable(nid)
+        st = [0] * pad + [0 if n == 1 and o != 1 else s for n, o, s in zip(src.shape, out_shape[pad:], src.strides)]
+        return View(src.base, src.offset, tuple(out_shape), tuple(st), src.dtype)
     if isinstance(op, F.SqueezeOp):
         sh, st = list(src.shape), list(src.strides)
         if sh[op.dim] == 1:

@@ -211,13 +211,16 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
         elif t == aten.scaled_dot_product_attention.default:
             mask = a[3] if len(a) > 3 else kw.get("attn_mask")
             if mask is not None:
-                raise TraceError("scaled_dot_product_attention with an explicit mask is not supported")
+                mval = mask.meta.get("val") if hasattr(mask, "meta") else None
+                if mval is None or not mval.dtype.is_floating_point:
+                    raise TraceError("scaled_dot_product_attention: only an additive floating-point mask is supported (a boolean mask is not)")
             dropout = a[4] if len(a) > 4 else kw.get("dropout_p", 0.0)
             if dropout:
                 raise TraceError("attention dropout is not supported")
             causal = bool(a[5] if len(a) > 5 else kw.get("is_causal", False))
             scale = kw.get("scale")
-            add(node, F.SdpaOp(is_causal=causal, scale=None if scale is None else float(scale), enable_gqa=bool(kw.get("enable_gqa", False))), [a[0], a[1], a[2]])
+            add(node, F.SdpaOp(is_causal=causal, scale=None if scale is None else float(scale), enable_gqa=bool(kw.get("enable_gqa", False)), has_mask=mask is not None),
+                [a[0], a[1], a[2]] + ([mask] if mask is not None else []))  # fmt: skip
         elif t in (aten.to.dtype, aten._to_copy.default, aten.to.dtype_layout):
             target = a[1] if len(a) > 1 and isinstance(a[1], torch.dtype) else kw.get("dtype")
             add(node, F.CastOp(dtype=dt.from_torch(target)), [a[0]])
@@ -238,6 +241,8 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
             add(node, F.PermuteOp(dims=tuple(_norm_dim(int(d), rank_in) for d in a[1])), [a[0]])
         elif t == aten.unsqueeze.default:
             add(node, F.UnsqueezeOp(dim=_norm_dim(int(a[1]), rank_in + 1)), [a[0]])
+        elif t == aten.expand.default:
+            add(node, F.ExpandOp(shape=tuple(int(d) for d in node.meta["val"].shape)), [a[0]])
         elif t == aten.squeeze.dim:
             add(node, F.SqueezeOp(dim=_norm_dim(int(a[1]), rank_in)), [a[0]])
         elif t == aten.slice.Tensor:

@@ -39,6 +39,14 @@ class Sdpa(nn.Module):
         return nn.functional.scaled_dot_product_attention(q, k, v, is_causal=self.causal, enable_gqa=True)
 
 
+class MaskedSdpa(nn.Module):
+    """Attention with an explicit additive mask, the way a whole-model trace of a HuggingFace decoder reaches it:
+    a float ``[1 | B, 1 | H, S, S_kv]`` bias of ``0`` / ``-inf`` (emmy/compiler/trace/torch.py:559-583)."""
+
+    def forward(self, q, k, v, mask):
+        return nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask, enable_gqa=True)
+
+
 def rms_norm_case(rows: int = 32, cols: int = 2048, seed: int = 0) -> Case:
     """C1: ``nn.RMSNorm(2048, eps=1e-6)`` on fp32 ``[1, rows, cols]`` ~N(0,1), weight ~N(1, 0.1)."""
     torch.manual_seed(seed)
@@ -91,6 +99,33 @@ class Qwen3Block(nn.Module):
     def forward(self, x, cos, sin):
         out = self.l(x, position_embeddings=(cos, sin), attention_mask=None)
         return out[0] if isinstance(out, tuple) else out
+
+
+class MaskedQwen3Block(nn.Module):
+    """The same layer called the way a whole-model trace calls it: with the model's ``[1, 1, S, S]`` float causal
+    bias as ``attention_mask``.  The layer then repeats the KV heads itself (unsqueeze / expand / reshape) and
+    passes the bias to attention as an explicit mask instead of ``is_causal``."""
+
+    def __init__(self, layer):
+        super().__init__()
+        self.l = layer
+
+    def forward(self, x, cos, sin, mask):
+        out = self.l(x, position_embeddings=(cos, sin), attention_mask=mask)
+        return out[0] if isinstance(out, tuple) else out
+
+
+def causal_bias(seq: int, dtype=torch.bfloat16) -> torch.Tensor:
+    """``[1, 1, seq, seq]``: 0 where key <= query, ``-inf`` above the diagonal."""
+    above = torch.arange(seq)[None, :] > torch.arange(seq)[:, None]
+    return torch.zeros(1, 1, seq, seq).masked_fill(above, -float("inf")).to(dtype)
+
+
+def masked_qwen3_block_case(seq: int = 512, seed: int = 0, norm_std: float = 0.0) -> Case:
+    """:func:`qwen3_block_case` with the causal structure carried by an explicit mask operand."""
+    base = qwen3_block_case(seq=seq, seed=seed, norm_std=norm_std)
+    return Case(base.name + "_masked", MaskedQwen3Block(base.module.l).eval(), (*base.inputs, causal_bias(seq)), base.rtol, base.atol,
+                algo_bytes=base.algo_bytes, algo_flops=base.algo_flops)  # fmt: skip
 
 
 def qwen3_block_case(seq: int = 512, seed: int = 0, dtype=torch.bfloat16, norm_std: float = 0.0) -> Case:

@@ -18,6 +18,10 @@ from deplodock_amd.workloads import (  # noqa: F401  (the shapes are the product
     BF16_RTOL,
     FP32_RTOL,
     Case,
+    MaskedQwen3Block,
+    MaskedSdpa,
+    causal_bias,
+    masked_qwen3_block_case,
     NormedRopeAttention,
     Qwen3Block,
     Sdpa,

@@ -94,8 +94,10 @@ def silu(x: np.ndarray) -> np.ndarray:
     return x * (1.0 / (1.0 + np.exp(-x)))
 
 
-def sdpa(q: np.ndarray, k: np.ndarray, v: np.ndarray, *, is_causal: bool, scale: float | None = None) -> np.ndarray:
-    """``softmax(q k^T * scale + causal) v`` with grouped KV heads.
+def sdpa(q: np.ndarray, k: np.ndarray, v: np.ndarray, *, is_causal: bool, scale: float | None = None, mask: np.ndarray | None = None) -> np.ndarray:
+    """``softmax(q k^T * scale + causal) v`` with grouped KV heads.  ``mask``: an additive bias broadcast onto
+    the scaled scores; it replaces the causal term (decomposition/010_sdpa.py:91-101: ``if inp_mask is not
+    None ... elif root.op.is_causal``).
 
     emmy/compiler/ir/frontend/ir.py:252-275 (``SdpaOp.forward``: K/V heads are
     repeated ``group = Hq // Hkv`` times, i.e. ``kv_head = q_head // group``;
@@ -110,7 +112,9 @@ def sdpa(q: np.ndarray, k: np.ndarray, v: np.ndarray, *, is_causal: bool, scale:
         v = np.repeat(v, group, axis=-3)
     d = q.shape[-1]
     s = (q @ np.swapaxes(k, -2, -1)) * (scale if scale is not None else 1.0 / np.sqrt(d))
-    if is_causal:
+    if mask is not None:
+        s = s + np.asarray(mask, dtype=np.float64)
+    elif is_causal:
         sq, sk = s.shape[-2], s.shape[-1]
         s = s - np.triu(np.ones((sq, sk)), k=1) * 1e9
     return softmax(s, -1) @ v
@@ -146,7 +150,7 @@ def online_softmax(x: np.ndarray, block: int) -> np.ndarray:
     return np.exp(x - m[..., None]) / d[..., None]
 
 
-def flash_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, *, is_causal: bool, scale: float, block_kv: int) -> np.ndarray:
+def flash_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, *, is_causal: bool, scale: float, block_kv: int, mask: np.ndarray | None = None) -> np.ndarray:
     """Streaming attention over key blocks with the ``(m, l, O)`` carrier:
     statistics start at ``m = -1e30, l = 0``; per block ``mn = max(m, rowmax)``,
     ``alpha = exp(m - mn)``, ``p = exp(s - mn)``, ``l = l*alpha + sum p``,
@@ -164,6 +168,7 @@ def flash_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, *, is_causal: b
     group = Hq // Hkv
     out = np.zeros((B, Hq, Sq, v.shape[-1]))
     rows = np.arange(Sq)[:, None]
+    bias = None if mask is None else np.broadcast_to(np.asarray(mask, dtype=np.float64), (B, Hq, Sq, Skv))
     for b in range(B):
         for h in range(Hq):
             kh, vh = k[b, h // group], v[b, h // group]
@@ -172,7 +177,9 @@ def flash_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, *, is_causal: b
             o = np.zeros((Sq, v.shape[-1]))
             for s0 in range(0, Skv, block_kv):
                 s = (q[b, h] @ kh[s0 : s0 + block_kv].T) * scale
-                if is_causal:
+                if bias is not None:  # the block's slice of the additive mask, in place of the causal term
+                    s = s + bias[b, h, :, s0 : s0 + block_kv]
+                elif is_causal:
                     cols = np.arange(s0, min(s0 + block_kv, Skv))[None, :]
                     s = np.where(cols > rows, -1e30, s)
                 mn = np.maximum(m, s.max(-1))

@@ -100,12 +100,12 @@ def evaluate_numpy(data: dict, values: dict[str, np.ndarray]) -> dict[str, np.nd
         elif kind == "LinearOp":
             env[nid] = O.linear(ts[0], ts[1], ts[2] if fields.get("has_bias") else None)
         elif kind == "SdpaOp":
-            q, k, v = ts
+            q, k, v = ts[:3]
             while k.ndim < q.ndim:
                 k = k[None]
             while v.ndim < q.ndim:
                 v = v[None]
-            env[nid] = O.sdpa(q, k, v, is_causal=bool(fields.get("is_causal", False)), scale=fields.get("scale"))
+            env[nid] = O.sdpa(q, k, v, is_causal=bool(fields.get("is_causal", False)), scale=fields.get("scale"), mask=ts[3] if len(ts) > 3 else None)
         elif kind == "MeanOp":
             env[nid] = np.mean(ts[0], axis=int(fields.get("axis", -1)), keepdims=len(nd["output"]["shape"]) == len(nodes[ins[0]]["output"]["shape"]))
         elif kind == "ReshapeOp":
@@ -156,14 +156,15 @@ def evaluate_torch(data: dict, values: dict, outputs_only: bool = True):
             elif kind == "LinearOp":
                 env[nid] = Fn.linear(ts[0], ts[1], ts[2] if fields.get("has_bias") else None)
             elif kind == "SdpaOp":
-                q, k, v = ts
+                q, k, v = ts[:3]
                 while k.ndim < q.ndim:
                     k = k[None]
                 while v.ndim < q.ndim:
                     v = v[None]
                 lead = q.shape[:-3]
-                o = Fn.scaled_dot_product_attention(q.reshape(-1, *q.shape[-3:]), k.reshape(-1, *k.shape[-3:]), v.reshape(-1, *v.shape[-3:]),
-                                                    is_causal=bool(fields.get("is_causal", False)), scale=fields.get("scale"), enable_gqa=q.shape[-3] != k.shape[-3])  # fmt: skip
+                mask = ts[3].expand(*lead, *ts[3].shape[-3:]).reshape(-1, *ts[3].shape[-3:]) if len(ts) > 3 else None
+                o = Fn.scaled_dot_product_attention(q.reshape(-1, *q.shape[-3:]), k.reshape(-1, *k.shape[-3:]), v.reshape(-1, *v.shape[-3:]), attn_mask=mask,
+                                                    is_causal=mask is None and bool(fields.get("is_causal", False)), scale=fields.get("scale"), enable_gqa=q.shape[-3] != k.shape[-3])  # fmt: skip
                 env[nid] = o.reshape(*lead, *o.shape[-3:])
             elif kind == "MeanOp":
                 env[nid] = torch.mean(ts[0], dim=int(fields.get("axis", -1)), keepdim=len(nd["output"]["shape"]) == len(nodes[ins[0]]["output"]["shape"]))

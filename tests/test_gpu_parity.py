@@ -235,6 +235,56 @@ def test_c4_sdpa_shapes_against_streaming_restatement(device, causal, dims):
     eager.assert_close(ours, torch.from_numpy(ref).float(), 2e-2, 2e-2, f"sdpa {dims} causal={causal} vs streaming restatement")
 
 
+@pytest.mark.parametrize("mask_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dims,mask_shape", [
+    ((1, 2, 1, 128, 128), (1, 1, 128, 128)), ((2, 4, 2, 200, 200), (2, 1, 200, 200)), ((2, 4, 2, 96, 160), (2, 4, 96, 160)),
+    ((1, 6, 2, 33, 33), (1, 1, 33, 33)), ((2, 4, 4, 70, 300), (2, 1, 1, 300)), ((1, 2, 2, 1, 70), (1, 2, 1, 70)),
+])  # fmt: skip
+def test_c4_sdpa_with_an_additive_mask(device, dims, mask_shape, mask_dtype):
+    """An explicit float mask (emmy/compiler/trace/torch.py:559-583) in every broadcast form, random finite
+    biases with ``-inf`` holes: key 0 stays open so no row is empty.  Against eager with the same mask and against
+    the streaming restatement in float64."""
+    b, hq, hkv, sq, skv = dims
+    torch.manual_seed(23)
+    q, k, v = torch.randn(b, hq, sq, 128).bfloat16(), torch.randn(b, hkv, skv, 128).bfloat16(), torch.randn(b, hkv, skv, 128).bfloat16()
+    mask = (2 * torch.randn(mask_shape)).to(mask_dtype)
+    mask[torch.rand(mask_shape) < 0.3] = -float("inf")
+    mask[..., 0] = 0.5
+    case = eager.Case("masked", eager.MaskedSdpa().eval(), (q, k, v, mask), 2e-2, 2e-2)
+    ours, want, compiled = run_case(case, device)
+    assert len([n for n in compiled.nodes.values() if isinstance(n.op, HipOp)]) == 1
+    eager.assert_close(ours, want, 2e-2, 2e-2, f"masked sdpa {dims} mask {mask_shape} {mask_dtype} vs eager")
+    ref = O.flash_attention(q.float().numpy(), k.float().numpy(), v.float().numpy(), is_causal=False, scale=128 ** -0.5, block_kv=64, mask=mask.float().numpy())
+    eager.assert_close(ours, torch.from_numpy(ref).float(), 2e-2, 2e-2, f"masked sdpa {dims} mask {mask_shape} vs streaming restatement")
+
+
+@pytest.mark.parametrize("seq", [64, 200, 512])
+def test_c5_block_called_with_an_attention_mask(device, seq):
+    """The block as a whole-model trace reaches it (mask operand, KV heads repeated by the layer): against eager on
+    the same call, and — the bias being the causal one — against the ``is_causal`` block's fp32 eager truth."""
+    case = eager.masked_qwen3_block_case(seq=seq, norm_std=0.1)
+    ours, want, compiled = run_case(case, device)
+    assert len([n for n in compiled.nodes.values() if isinstance(n.op, HipOp)]) == 5
+    plain = eager.qwen3_block_case(seq=seq, norm_std=0.1)
+    exact = eager.run_eager_fp32(plain, device)
+    eager.assert_mean_error_within_baseline(ours, want, exact, 1.5, f"masked block S={seq}")
+    eager.assert_rows_within_baseline(ours, want, exact, 1.5, f"masked block S={seq} rows")
+
+
+def test_c4_causal_bias_mask_equals_the_causal_kernel(device):
+    """HuggingFace's ``[1, 1, S, S]`` ``0 / -inf`` causal bias, at the benchmark's size: the masked kernel's rows
+    agree with the ``is_causal`` kernel's to the rounding of the output."""
+    case = eager.sdpa_case()
+    q, k, v = case.inputs
+    s = q.shape[-2]
+    tri = torch.zeros(1, 1, s, s).masked_fill(torch.arange(s)[None, :] > torch.arange(s)[:, None], -float("inf")).bfloat16()
+    ours, want, _ = run_case(eager.Case("tri", eager.MaskedSdpa().eval(), (q, k, v, tri), 2e-2, 2e-2), device)
+    causal, _, _ = run_case(case, device)
+    eager.assert_close(ours, want, 2e-2, 2e-2, "bias-masked sdpa S=2048 vs eager")
+    exact = nn.functional.scaled_dot_product_attention(q.to(device).float(), k.to(device).float(), v.to(device).float(), is_causal=True, enable_gqa=True)
+    eager.assert_rows_within_baseline(ours, causal, exact, 1.5, "bias-masked sdpa vs the causal kernel, fp32 eager as the truth")
+
+
 @pytest.mark.parametrize("d,dtype,causal", [(256, torch.bfloat16, True), (256, torch.bfloat16, False), (128, torch.float16, True), (64, torch.bfloat16, True), (64, torch.bfloat16, False), (64, torch.float16, True)])
 def test_c4_wide_heads_and_fp16(device, d, dtype, causal):
     """head_dim 256 (two 128-wide accumulator groups; the schedule shrinks the key block to fit the LDS),

@@ -67,6 +67,57 @@ def test_later_stage_or_foreign_json_is_refused():
         graph_from_reference_dict(data)
 
 
+def _masked_attention_json(b=1, hq=4, hkv=2, sq=24, skv=40, d=64) -> dict:
+    """A frontend graph in the reference's JSON form whose ``SdpaOp`` takes a fourth, additive-mask input
+    (emmy/compiler/trace/torch.py:559-583)."""
+    def t(name, shape):
+        return {"name": name, "shape": list(shape), "dtype": "f32"}
+
+    nodes = {n: {"op": "InputOp", "op_fields": {}, "inputs": [], "output": t(n, shp)}
+             for n, shp in (("q", (b, hq, sq, d)), ("k", (b, hkv, skv, d)), ("v", (b, hkv, skv, d)), ("mask", (1, 1, sq, skv)))}  # fmt: skip
+    nodes["attn"] = {"op": "SdpaOp", "op_fields": {"is_causal": True}, "inputs": ["q", "k", "v", "mask"], "output": t("attn", (b, hq, sq, d))}
+    return {"inputs": ["q", "k", "v", "mask"], "outputs": ["attn"], "nodes": nodes}
+
+
+def test_masked_attention_graph_reads_with_the_mask_as_an_operand(launcher_lib):
+    data = _masked_attention_json()
+    g = graph_from_reference_dict(data, cast=BF16)
+    op = g.nodes["attn"].op
+    assert isinstance(op, F.SdpaOp) and op.has_mask and not op.is_causal and g.nodes["attn"].inputs == ["q", "k", "v", "mask"]
+    compiled = HipBackend().compile(g)
+    ks = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert len(ks) == 1 and "#define HAS_MASK 1" in ks[0].kernel_source
+    # the two interpreters agree on the masked node, and the mask is what makes the difference
+    vals = ref_graph.random_values(data, seed=3)
+    vals["mask"] = torch.where(torch.rand(vals["mask"].shape, generator=torch.Generator().manual_seed(4)) < 0.3, -float("inf"), 1.0) * torch.ones_like(vals["mask"])
+    vals["mask"][..., 0] = 0.0
+    want = ref_graph.evaluate_torch(data, vals)["attn"].numpy()
+    got = ref_graph.evaluate_numpy(data, {k: v.numpy() for k, v in vals.items()})["attn"]
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5)
+    unmasked = ref_graph.evaluate_numpy(data, {**{k: v.numpy() for k, v in vals.items()}, "mask": np.zeros_like(vals["mask"].numpy())})["attn"]
+    assert np.abs(unmasked - got).max() > 1e-2
+
+
+@pytest.mark.gpu
+def test_masked_attention_graph_runs_on_the_gpu(device):
+    data = _masked_attention_json(b=2, hq=4, hkv=2, sq=100, skv=164, d=128)
+    vals = {k: v.bfloat16() for k, v in ref_graph.random_values(data, seed=5).items()}
+    hole = torch.rand(vals["mask"].shape, generator=torch.Generator().manual_seed(6)) < 0.4
+    vals["mask"] = vals["mask"].masked_fill(hole, -float("inf"))
+    vals["mask"][..., 0] = 0.0
+    be = HipBackend()
+    compiled = be.compile(graph_from_reference_dict(data, cast=BF16))
+    prog = be.program(compiled, {n: vals[n].to(device) for n in compiled.inputs})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()["attn"].clone()
+    finally:
+        prog.close()
+    want = ref_graph.evaluate_torch(data, {k: v.to(device) for k, v in vals.items()})["attn"]
+    eager.assert_close(ours.reshape(want.shape), want, 2e-2, 2e-2, "ingested masked attention vs eager")
+
+
 @pytest.mark.parametrize("path,launches", [(TINYLLAMA, 7), (QWEN25, 10)])
 def test_fixtures_lower_to_fused_kernels(launcher_lib, path, launches):
     """The ingested block compiles to the same kind of kernels a traced module does (norms folded into the

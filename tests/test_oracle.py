@@ -138,6 +138,32 @@ def test_flash_equals_sdpa(causal, block_kv):
     np.testing.assert_allclose(got, want, rtol=1e-10, atol=1e-12)
 
 
+@pytest.mark.parametrize("mask_shape", [(1, 1, 9, 13), (2, 1, 9, 13), (2, 4, 9, 13), (1, 4, 1, 13)])
+def test_sdpa_additive_mask_matches_torch(mask_shape):
+    """The mask is added to the *scaled* scores (a mask added before the scale, or multiplied in, fails), and
+    broadcasts over batch, heads and queries; ``-inf`` entries drop a key."""
+    torch.manual_seed(21)
+    q, k, v = torch.randn(2, 4, 9, 16, dtype=torch.float64), torch.randn(2, 2, 13, 16, dtype=torch.float64), torch.randn(2, 2, 13, 16, dtype=torch.float64)
+    mask = torch.randn(mask_shape, dtype=torch.float64) * 3
+    mask[..., 5] = -float("inf")
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask, enable_gqa=True).numpy()
+    np.testing.assert_allclose(O.sdpa(q.numpy(), k.numpy(), v.numpy(), is_causal=False, mask=mask.numpy()), ref, rtol=1e-9, atol=1e-12)
+    for block_kv in (1, 4, 64):
+        got = O.flash_attention(q.numpy(), k.numpy(), v.numpy(), is_causal=False, scale=0.25, block_kv=block_kv, mask=mask.numpy())
+        np.testing.assert_allclose(got, ref, rtol=1e-9, atol=1e-12)
+
+
+def test_sdpa_mask_replaces_the_causal_term():
+    """A ``0 / -inf`` lower-triangular bias is the causal attention (closed form), and with a mask present the
+    ``is_causal`` flag is not applied on top (decomposition/010_sdpa.py:91-101)."""
+    rng = np.random.default_rng(22)
+    q, k, v = rng.standard_normal((1, 2, 7, 8)), rng.standard_normal((1, 2, 7, 8)), rng.standard_normal((1, 2, 7, 8))
+    tri = np.where(np.arange(7)[None, :] > np.arange(7)[:, None], -np.inf, 0.0)[None, None]
+    np.testing.assert_allclose(O.sdpa(q, k, v, is_causal=False, mask=tri), O.sdpa(q, k, v, is_causal=True), rtol=1e-12)
+    zero = np.zeros((1, 1, 7, 7))
+    np.testing.assert_allclose(O.sdpa(q, k, v, is_causal=True, mask=zero), O.sdpa(q, k, v, is_causal=False), rtol=1e-12)
+
+
 # -- bf16 carrier ------------------------------------------------------------------------------
 
 

@@ -15,6 +15,8 @@ from deplodock_amd.backend.hip import hiprtc
 from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.dtype import F32
 from deplodock_amd.ir import expr as E
+from deplodock_amd.ir.tile import TileOp
+from deplodock_amd.passes.fuse import fuse
 from oracle import eager
 
 
@@ -81,6 +83,51 @@ def test_sdpa_is_one_flash_kernel(launcher_lib):
     assert "#define GROUP 2" in k.kernel_source and "#define CAUSAL 1" in k.kernel_source
     assert "flash_pv_smem" not in k.kernel_source  # P stays in registers
     hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+
+
+def test_sdpa_with_an_additive_mask_is_the_same_flash_kernel(launcher_lib):
+    """The mask is a fourth operand of the one attention kernel: added to the scores (over the scale, so the
+    exponent's fma sees ``s * scale + mask``) before the running maximum."""
+    torch.manual_seed(0)
+    q, k, v = torch.randn(2, 4, 96, 128).bfloat16(), torch.randn(2, 2, 160, 128).bfloat16(), torch.randn(2, 2, 160, 128).bfloat16()
+    for mask, strides, vec in ((torch.zeros(1, 1, 96, 160).bfloat16(), (0, 0, 160), 1), (torch.zeros(2, 4, 1, 160), (640, 160, 0), 1), (torch.zeros(2, 1, 96, 160)[..., 1:], None, 0)):
+        kk, vv = (k, v) if mask.shape[-1] == 160 else (k[:, :, 1:], v[:, :, 1:])
+        ks = kernels(compile_case(eager.Case("m", eager.MaskedSdpa().eval(), (q, kk, vv, mask), 2e-2, 2e-2)))
+        assert len(ks) == 1 and ks[0].kernel_name.startswith("k_sdpa_reduce_") and len(ks[0].arg_order) == 5
+        src = ks[0].kernel_source
+        assert "#define HAS_MASK 1" in src and "#define CAUSAL 0" in src and f"#define MASK_VEC {vec}" in src
+        if strides:
+            assert all(f"#define {n} {v_}" in src for n, v_ in zip(("M_SB", "M_SH", "M_SS"), strides))
+        hiprtc.compile_to_hsaco(src, ks[0].kernel_name)
+    with pytest.raises(Exception, match="bool"):
+        compile_case(eager.Case("m", eager.MaskedSdpa().eval(), (q, k, v, torch.ones(1, 1, 96, 160, dtype=torch.bool)), 2e-2, 2e-2))
+
+
+def test_masked_block_repeats_kv_heads_without_a_copy(launcher_lib):
+    """Called with an attention mask the layer repeats its KV heads itself (``x[:, :, None].expand(..).reshape(..)``,
+    not a view) and hands the bias to attention: still the five kernels of the unmasked block, the attention kernel
+    reading the projection's KV windows with grouped heads and the mask as a fourth operand."""
+    compiled = compile_case(eager.masked_qwen3_block_case(seq=64))
+    ks = kernels(compiled)
+    assert [re.sub(r"_[0-9a-f]{6}$", "", k.kernel_name) for k in ks] == ["k_rms_norm_linear_rope", "k_sdpa_reduce", "k_linear_add", "k_rms_norm_linear_silu_mul", "k_linear_add"]
+    flash = ks[1].kernel_source
+    assert "#define GROUP 2" in flash and "#define HAS_MASK 1" in flash and "#define CAUSAL 0" in flash and "#define M_SS 64" in flash
+    assert ks[1].arg_order[:3] == (ks[0].arg_order[-1],) * 3 and ks[1].arg_order[3] == compiled.inputs[3]
+
+
+def test_expanded_operands_are_broadcast_reads(launcher_lib):
+    class ColTimes(nn.Module):
+        def forward(self, x, b):
+            return x * b[None, :].expand(x.shape[0], -1)
+
+    class RowTimes(nn.Module):
+        def forward(self, x, b):
+            return x * b[:, None].expand(-1, x.shape[1])
+
+    for mod, b, kind in ((ColTimes(), torch.randn(2048), "col"), (RowTimes(), torch.randn(64), "row")):
+        g = trace_module(mod, (torch.randn(64, 2048), b))
+        tile = [n.op.body for n in fuse(g).nodes.values() if isinstance(n.op, TileOp)]
+        assert len(tile) == 1 and [o.index for o in tile[0].operands] == ["flat", kind]
 
 
 def test_qwen3_block_kernel_boundaries(launcher_lib):
