@@ -182,7 +182,14 @@ def _run_ir(args, device) -> None:
     graph = serialize.load(args.ir)
     be = HipBackend(dump=Path(args.dump_dir) if args.dump_dir else None, device_id=0, tune_db=getattr(args, "tune_db", None))
     compiled = graph if any(isinstance(n.op, HipOp) for n in graph.nodes.values()) else be.compile(graph)
-    data = serialize.random_inputs(compiled, seed=args.seed, device=device)
+    sizes = {}
+    for spec in args.at or []:  # a lowered graph whose kernels take a size at run time replays at any size
+        name, _, size = spec.partition("=")
+        if getattr(compiled, "symbolic", None) != name or not size.isdigit():
+            print(f"error: --at {spec}: expected NAME=SIZE with NAME the graph's runtime-int axis ({getattr(compiled, 'symbolic', None)!r})", file=sys.stderr)
+            sys.exit(2)
+        sizes[name] = int(size)
+    data = serialize.random_inputs(compiled, seed=args.seed, device=device, sizes=sizes)
     program = be.program(compiled, data)
     try:
         program.run()

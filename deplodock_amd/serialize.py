@@ -7,6 +7,12 @@ Two stages are serialisable here: the traced frontend graph (``stage:
 "torch"``) and the lowered ``Graph[HipOp]`` (``stage: "hip"``: kernel source,
 launch geometry, argument order, knobs).  Tensor *values* are never written —
 a reloaded graph runs on seeded random data, as the reference's ``--ir`` does.
+
+A lowered graph whose kernels take a size at run time keeps its symbolic parts: shapes
+with ``seq_len`` / ``a * seq_len + b`` dims, launch-time grid factors (``CeilDiv``,
+``XcdRounds``), the trailing ``int`` arguments, and the symbol's traced size (what a replay
+on synthetic inputs runs at) — the reference's JSON likewise keeps ``Dim`` expressions and
+symbolic grid factors (emmy/compiler/ir/cuda/ir.py:66-112).
 """
 
 from __future__ import annotations
@@ -20,6 +26,7 @@ from deplodock_amd.graph import Graph, Node, Tensor
 from deplodock_amd.ir import frontend as F
 from deplodock_amd.ir.base import ConstantOp, InputOp, Op
 from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.sym import Affine, CeilDiv, XcdRounds
 
 FORMAT = 1
 _SKIP_FIELDS = {"source"}
@@ -27,7 +34,15 @@ _OPS = {cls.__name__: cls for cls in (InputOp, ConstantOp, HipOp, *(v for v in v
 
 
 class SerializeError(TypeError):
-    """The graph holds something with no JSON form (a tile body, a symbolic launch factor)."""
+    """The graph holds something with no JSON form (a tile body, a python callable as a launch factor)."""
+
+
+@dataclasses.dataclass
+class TracedSizes:
+    """What a reloaded runtime-int graph remembers of its dynamic trace: the symbol's traced size.  (The module
+    itself is not in the file, so a reloaded graph cannot be re-traced at another size — it does not need to.)"""
+
+    hints: dict
 
 
 def _enc(v, where: str):
@@ -35,6 +50,12 @@ def _enc(v, where: str):
         return {"$dtype": v.name}
     if isinstance(v, (str, int, float, bool)) or v is None:
         return v
+    if isinstance(v, Affine):
+        return {"$affine": [v.name, v.a, v.b]}
+    if isinstance(v, CeilDiv):
+        return {"$ceildiv": [_enc(v.value, where), v.div]}
+    if isinstance(v, XcdRounds):
+        return {"$xcdrounds": [_enc(v.m, where), v.tile_m, v.blocks_n, v.per_block, v.xcds]}
     if isinstance(v, (tuple, list)):
         return {"$tuple": [_enc(x, where) for x in v]} if isinstance(v, tuple) else [_enc(x, where) for x in v]
     if isinstance(v, dict):
@@ -50,6 +71,14 @@ def _dec(v):
             return tuple(_dec(x) for x in v["$tuple"])
         if "$dict" in v:
             return {k: _dec(x) for k, x in v["$dict"].items()}
+        if "$affine" in v:
+            name, a, b = v["$affine"]
+            return Affine(str(name), int(a), int(b))
+        if "$ceildiv" in v:
+            return CeilDiv(_dec(v["$ceildiv"][0]), int(v["$ceildiv"][1]))
+        if "$xcdrounds" in v:
+            m, *rest = v["$xcdrounds"]
+            return XcdRounds(_dec(m), *(int(x) for x in rest))
         raise SerializeError(f"unknown encoded object {sorted(v)}")
     if isinstance(v, list):
         return [_dec(x) for x in v]
@@ -104,12 +133,15 @@ def graph_to_dict(g: Graph) -> dict:
                 "id": nid,
                 "op": op_to_dict(n.op, nid),
                 "inputs": list(n.inputs),
-                "shape": [int(d) for d in n.output.shape],
+                "shape": [d if isinstance(d, str) else _enc(d, nid) if isinstance(d, Affine) else int(d) for d in n.output.shape],
                 "dtype": n.output.dtype.name,
                 "hints": _hints_to_dict(n.hints, nid),
             }
         )
-    return {"format": FORMAT, "stage": stage, "arch": "gfx950", "inputs": list(g.inputs), "outputs": list(g.outputs), "nodes": nodes}
+    out = {"format": FORMAT, "stage": stage, "arch": "gfx950", "inputs": list(g.inputs), "outputs": list(g.outputs), "nodes": nodes}
+    if getattr(g, "symbolic", None) is not None:
+        out["symbolic"] = {"name": g.symbolic, "hints": {k: int(v) for k, v in (getattr(getattr(g, "dynamic", None), "hints", {}) or {}).items()}}
+    return out
 
 
 def graph_from_dict(d: dict) -> Graph:
@@ -118,7 +150,7 @@ def graph_from_dict(d: dict) -> Graph:
     g = Graph()
     for nd in d["nodes"]:
         op = op_from_dict(nd["op"])
-        t = Tensor(nd["id"], tuple(nd["shape"]), dt.by_name(nd["dtype"]), constant=isinstance(op, ConstantOp), value=getattr(op, "value", None))
+        t = Tensor(nd["id"], tuple(_dec(d_) for d_ in nd["shape"]), dt.by_name(nd["dtype"]), constant=isinstance(op, ConstantOp), value=getattr(op, "value", None))
         for i in nd["inputs"]:
             if i not in g.nodes:
                 raise SerializeError(f"node {nd['id']!r} references {i!r} before it is defined")
@@ -126,6 +158,9 @@ def graph_from_dict(d: dict) -> Graph:
     g.inputs = list(d["inputs"])
     g.outputs = list(d["outputs"])
     g.stage = d.get("stage", "torch")
+    if d.get("symbolic"):
+        g.symbolic = str(d["symbolic"]["name"])
+        g.dynamic = TracedSizes({str(k): int(v) for k, v in d["symbolic"].get("hints", {}).items()})
     return g
 
 
@@ -137,13 +172,17 @@ def load(path: str | Path) -> Graph:
     return graph_from_dict(json.loads(Path(path).read_text()))
 
 
-def random_inputs(g: Graph, seed: int = 0, device=None) -> dict:
+def random_inputs(g: Graph, seed: int = 0, device=None, sizes: dict | None = None) -> dict:
     """Seeded random tensors for every input and every constant without a static
-    value (stacked constants are left to the binder when their parts exist)."""
+    value (stacked constants are left to the binder when their parts exist).  A symbolic
+    dim takes its size from ``sizes``, else the size the graph was traced at."""
     import torch
+
+    from deplodock_amd.ir.sym import resolve
 
     gen = torch.Generator().manual_seed(seed)
     out = {}
+    env = {**(getattr(getattr(g, "dynamic", None), "hints", {}) or {}), **(sizes or {})}
     stacked_parts = {p for n in g.nodes.values() for p in getattr(n.hints.get("stacked"), "parts", ())}
     for nid, n in g.nodes.items():
         if not isinstance(n.op, (InputOp, ConstantOp)) or (isinstance(n.op, ConstantOp) and n.op.value is not None):
@@ -151,7 +190,7 @@ def random_inputs(g: Graph, seed: int = 0, device=None) -> dict:
         if n.hints.get("stacked") is not None and all(p in g.nodes for p in n.hints["stacked"].parts):
             continue
         scale = 0.05 if isinstance(n.op, ConstantOp) else 1.0
-        t = (scale * torch.randn(tuple(n.output.shape), generator=gen)).to({"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}.get(n.output.dtype.name, torch.float32))
+        t = (scale * torch.randn(tuple(resolve(d, env) for d in n.output.shape), generator=gen)).to({"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}.get(n.output.dtype.name, torch.float32))
         out[nid] = t.to(device) if device is not None else t
     del stacked_parts
     return out

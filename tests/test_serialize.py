@@ -46,6 +46,36 @@ def test_lowered_graph_round_trips_field_for_field(launcher_lib, tmp_path):
     assert all(torch.equal(data[k], again[k]) for k in data)
 
 
+def test_runtime_int_graph_round_trips_with_its_symbolic_parts(launcher_lib, tmp_path):
+    """A lowering with a symbolic axis keeps, through JSON: ``seq_len`` / affine dims in shapes, launch-time grid
+    factors, the trailing int arguments and the traced size."""
+    from deplodock_amd.ir.sym import resolve
+    from deplodock_amd.ir.hip import resolve_dim
+    from deplodock_amd.ir.sym import Affine, CeilDiv, XcdRounds
+
+    case = eager.qwen3_block_case(seq=64)
+    dyn = {"x": {1: "seq_len"}, "cos": {1: "seq_len"}, "sin": {1: "seq_len"}}
+    c = HipBackend().compile(trace_module(case.module, case.inputs, dynamic_shapes=dyn))
+    assert c.symbolic == "seq_len"
+    serialize.save(c, tmp_path / "sym.json")
+    c2 = serialize.load(tmp_path / "sym.json")
+    assert c2.symbolic == "seq_len" and c2.dynamic.hints == {"seq_len": 64}
+    kinds = set()
+    for x, y in zip(hip_ops(c), hip_ops(c2)):
+        assert x.grid == y.grid and x.runtime_args == y.runtime_args == ("seq_len",) and x.kernel_source == y.kernel_source
+        kinds |= {type(f) for dim in y.grid for f in (dim if isinstance(dim, tuple) else (dim,))}
+        for s_ in (7, 64, 513):
+            assert [resolve_dim(d, {"seq_len": s_}) for d in x.grid] == [resolve_dim(d, {"seq_len": s_}) for d in y.grid]
+    assert {CeilDiv, XcdRounds} <= kinds
+    for nid in c.nodes:
+        assert c.nodes[nid].output.shape == c2.nodes[nid].output.shape
+        assert [resolve(d, {"seq_len": 200}) for d in c2.nodes[nid].output.shape] == [resolve(d, {"seq_len": 200}) for d in c.nodes[nid].output.shape]
+    assert any(isinstance(d, (str, Affine)) for n in c2.nodes.values() for d in n.output.shape)
+    assert tuple(serialize.random_inputs(c2)["x"].shape) == (1, 64, 1024)
+    assert tuple(serialize.random_inputs(c2, sizes={"seq_len": 200})["cos"].shape)[1] == 200
+    assert HipBackend().variant(c2, {"x": torch.zeros(1, 200, 1024)}) is c2  # one lowering serves every size
+
+
 def test_tile_stage_has_no_json_form():
     case = eager.rms_norm_case()
     with pytest.raises(serialize.SerializeError, match="TileOp"):
@@ -76,6 +106,34 @@ def test_run_ir_replays_both_stages(tmp_path, capsys):
     assert out.startswith("RAN ") and "k_softmax_reduce" in out and "program:" in out
     main(["run", "--ir", str(traced)])
     assert capsys.readouterr().out.startswith("RAN ")
+
+
+@pytest.mark.gpu
+def test_reloaded_runtime_int_graph_runs_at_other_sizes(device, tmp_path, capsys):
+    """The reloaded symbolic lowering against eager at sizes it was not traced at, and ``run --ir --at``."""
+    case = eager.qwen3_block_case(seq=64)
+    dyn = {"x": {1: "seq_len"}, "cos": {1: "seq_len"}, "sin": {1: "seq_len"}}
+    be = HipBackend()
+    c = be.compile(trace_module(case.module, case.inputs, dynamic_shapes=dyn))
+    serialize.save(c, tmp_path / "sym.json")
+    c2 = serialize.load(tmp_path / "sym.json")
+    weights = {k: v.to(device) for k, v in be.bind(c, {}).items()}
+    for seq in (200, 33):
+        other = eager.qwen3_block_case(seq=seq)
+        data = {**weights, **{n: t.to(device) for n, t in zip(c2.inputs, other.inputs)}}
+        prog = be.program(c2, data)
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            ours = prog.output_tensors()[c2.outputs[0]].clone()
+        finally:
+            prog.close()
+        want = eager.run_eager(other, device)
+        exact = eager.run_eager_fp32(other, device)
+        eager.assert_mean_error_within_baseline(ours.reshape(want.shape), want, exact, 1.5, f"reloaded runtime-int block S={seq}")
+    main(["run", "--ir", str(tmp_path / "sym.json"), "--at", "seq_len=100"])
+    out = capsys.readouterr().out
+    assert out.startswith("RAN ") and "(1, 100, 1024)" in out
 
 
 @pytest.mark.gpu
