@@ -13,6 +13,11 @@
   operands.  That figure, not the MFMA peak, bounds a contraction whose tile needs
   more bytes per MFMA cycle than it delivers.
 
+* ``--lds``: the rate at which the waves of a CU read 16-byte MFMA operand fragments out of
+  LDS (``ds_read_b128``), for the lane-to-address patterns the emitters use — 16- and 32-row
+  fragment layouts over XOR-swizzled slabs of 64, 128 and 256 bytes a row — against a
+  conflict-free linear pattern, in bytes per clock per CU measured with the shader clock.
+
 No counterpart in the reference (its constants are NVIDIA's); the kernels are
 emitted, compiled and launched through the same hipRTC / launcher path as
 everything else.
@@ -236,10 +241,95 @@ def handle_l1fill(args) -> None:
         print(line)
 
 
+_LDS_SRC = r"""
+// Wave w reads fragments of rows (w * READS + r) * AM + lr, k chunk kk * KG + lk: the EMH_READ of a contraction.
+extern "C" __global__ __launch_bounds__(NT) void KNAME(unsigned long long* __restrict__ ticks, unsigned* __restrict__ out, int iters) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  for (int i = tid; i < LDS_BYTES / 4; i += NT) ((unsigned*)lds)[i] = i * 2654435761u;
+  __syncthreads();
+  const int lr = lane % AM, lk = lane / AM;
+  unsigned addr[KS][READS];
+  #pragma unroll
+  for (int kk = 0; kk < KS; ++kk)
+  #pragma unroll
+  for (int r = 0; r < READS; ++r) {
+    const int row = ((wave * READS + r) * AM + lr) % ROWS, c = kk * KG + lk;
+    addr[kk][r] = LINEAR ? (unsigned)((((wave * KS + kk) * READS + r) * 64 + lane) * 16) % LDS_BYTES
+                         : (unsigned)(row * ROWB + ((c ^ ((row / RPL) % CPR)) % CPR) * 16);
+  }
+  u32x4 acc = {0u, 0u, 0u, 0u};
+  const unsigned base = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned char*)lds;
+  const unsigned long long t0 = __builtin_amdgcn_s_memtime();
+  for (int it = 0; it < iters; ++it) {
+    #pragma unroll
+    for (int kk = 0; kk < KS; ++kk) {
+      u32x4 v[READS];
+      #pragma unroll
+      for (int r = 0; r < READS; ++r) asm volatile("ds_read_b128 %0, %1" : "=v"(v[r]) : "v"(base + addr[kk][r]));
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      #pragma unroll
+      for (int r = 0; r < READS; ++r) acc ^= v[r];
+    }
+  }
+  const unsigned long long t1 = __builtin_amdgcn_s_memtime();
+  if (lane == 0) ticks[blockIdx.x * (NT / 64) + wave] = t1 - t0;
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) out[tid] = acc[0];
+}
+"""
+
+
+def lds_read_bytes_per_clock(*, atom_rows: int, row_bytes: int, waves: int, reads: int = 8, linear: bool = False, iters: int = 2000) -> float:
+    """Bytes per shader clock one CU's waves read from LDS with the contraction emitter's fragment addressing:
+    ``atom_rows`` rows a fragment (16 or 32, the lane groups beyond them take neighbouring 16-byte k chunks),
+    ``row_bytes`` a slab row, chunks XOR-swizzled by ``(row / rows_per_256B) % chunks_per_row``."""
+    import torch
+
+    from deplodock_amd.backend.hip import hiprtc, launcher
+    from deplodock_amd.backend.hip.launcher import PackedArgs
+    from deplodock_amd.emit import prelude
+
+    lib = launcher.load()
+    cpr = row_bytes // 16
+    kg = 64 // atom_rows
+    ks = max(1, cpr // kg)
+    rows = 256
+    nt = waves * 64
+    name = f"k_ldsread_a{atom_rows}_r{row_bytes}_w{waves}_n{reads}_{int(linear)}"
+    defs = dict(NT=nt, AM=atom_rows, KG=kg, KS=ks, READS=reads, ROWS=rows, ROWB=row_bytes, CPR=cpr, RPL=max(1, 16 // cpr), LINEAR=int(linear), LDS_BYTES=rows * row_bytes)
+    src = prelude.header() + "".join(f"#define {k} {v}\n" for k, v in defs.items()) + _LDS_SRC.replace("KNAME", name)
+    fn = hiprtc.load_function(src, name, cached=False)
+    cus = lib.device_props(0)["compute_units"]
+    ticks = torch.zeros(cus * waves, dtype=torch.int64, device="cuda")
+    out = torch.zeros(nt, dtype=torch.int32, device="cuda")
+    args = PackedArgs([ticks.data_ptr(), out.data_ptr()], [iters])
+    for _ in range(2):
+        lib.launch(fn.fn, (cus, 1, 1), (nt, 1, 1), rows * row_bytes, None, args)
+    torch.cuda.synchronize()
+    lib.module_unload(fn.module)
+    per_cu = ticks.view(cus, waves).max(dim=1).values.double().median().item()  # a CU is done when its slowest wave is
+    return waves * iters * ks * reads * 1024 / per_cu
+
+
+def handle_lds(args) -> None:
+    from deplodock_amd.commands.table import render_table
+
+    rows = []
+    for waves in (4, 8, 16):
+        rows.append(["linear (lane * 16)", "-", str(waves), f"{lds_read_bytes_per_clock(atom_rows=16, row_bytes=128, waves=waves, linear=True):.1f}"])
+        for atom_rows in (16, 32):
+            for row_bytes in (64, 128, 256):
+                rows.append([f"{atom_rows}-row fragments", str(row_bytes), str(waves), f"{lds_read_bytes_per_clock(atom_rows=atom_rows, row_bytes=row_bytes, waves=waves):.1f}"])
+        print("  ".join(rows[-1]), flush=True)
+    for line in render_table(["ds_read_b128 pattern", "slab row bytes", "waves/CU", "B/clk/CU"], rows, "llrr"):
+        print(line)
+
+
 def register_microbench_command(subparsers) -> None:
     p = subparsers.add_parser("microbench", help="Measure the MFMA rate, MFMA/VALU co-issue and the L1 fill rate of the GPU")
     p.add_argument("--l1fill", action="store_true", help="sweep load-only kernels: bytes per clock a CU pulls through its vector L1")
     p.add_argument("--quick", action="store_true", help="with --l1fill: a four-line sweep")
+    p.add_argument("--lds", action="store_true", help="fragment-read rate out of LDS for the emitters' swizzled layouts")
     p.set_defaults(func=handle_microbench)
 
 
@@ -251,6 +341,9 @@ def handle_microbench(args) -> None:
         sys.exit(1)
     if getattr(args, "l1fill", False):
         handle_l1fill(args)
+        return
+    if getattr(args, "lds", False):
+        handle_lds(args)
         return
     from deplodock_amd.backend.hip import launcher
     from deplodock_amd.commands.table import render_table

@@ -157,6 +157,88 @@ def _emit_row_epilogue(a, body: Contraction, re, re_args: list[str], EPC: int, v
     a("  } else {")
 
 
+PP_PRODUCER_THREADS = 256  # the four request-issuing waves of STAGE .../pp (one per SIMD)
+
+
+def _emit_pingpong_loop(a, *, KT: int, KS: int, depth: int, parts: list[str]) -> None:
+    """The k loop of ``STAGE .../pp``: twelve waves, three on every SIMD, in three roles, one workgroup barrier a slab.
+
+    Waves 0-3 and 4-7 (one of each on every SIMD; every wave owns its own part of the output tile) are two
+    *consumer* groups that run half a slab apart.  In period j group 0 issues the MFMAs of slab j (at raised
+    priority) and then reads slab j + 1's fragments into registers; group 1 first reads slab j's fragments and
+    then issues its MFMAs.  So while one wave of a SIMD computes, the other reads, and LDS latency is paid by the
+    wave with nothing to compute.  Waves 8-11 are *producers*: they issue every direct-to-LDS request (``parts``:
+    the statements of one slab's requests of a producer thread, format strings over ``slab`` and ``buf``), wait
+    for them in issue order and publish them.  A request blocks its wave at issue while the memory pipeline is
+    full — which, with operands streaming from L2 at the rate this tile needs them, is most of the time; on a
+    producer wave that costs nothing, on a consumer it would stall the MFMAs queued behind it.
+
+        period j   group 0: MFMAs of slab j, read slab j + 1     group 1: read slab j, MFMAs of slab j
+                   producers: request slab j + DEPTH - 1 (into the buffer of slab j - 1, whose last reader, group 1
+                   in period j - 1, is done), then wait until slab j + 2 is complete and publish it;  barrier.
+
+    Slab j + 1 is read inside period j, so it has to be complete at the barrier that *starts* the period: a slab
+    requested in period q is waited for at the end of period q + DEPTH - 3, which needs DEPTH >= 4 to leave it
+    more than the rest of its own period.
+
+    (A wave gets about 32 bytes a clock out of LDS and issues in order, so group 1's MFMAs start some 400 clocks
+    into the period, when group 0 is about done with its own.  Moving part of the reads between the MFMAs, in
+    either group, measured slower: a read that blocks at issue holds back the MFMAs behind it.)"""
+    R = depth
+
+    def request(q: str) -> None:
+        for st in parts:
+            a("      " + st.format(slab=f"(({q}) + {R - 1})", buf=f"((({q}) + {R - 1}) % DEPTH)"))
+
+    def fetch(j: str) -> None:
+        for kk in range(KS):
+            a(f"      EMH_READ({kk}, ({j}) % DEPTH, {kk});")
+
+    def compute() -> None:
+        a("      __builtin_amdgcn_s_setprio(1);")
+        for kk in range(KS):
+            a(f"      EMH_MMA({kk});")
+        a("      __builtin_amdgcn_s_setprio(0);")
+
+    def allowed(q: int) -> int:
+        """Requests a producer thread may still have outstanding at the end of period q (-1: the period before
+        the first) with every slab up to q + 2 complete: what it issued after slab q + 2 (they retire in order)."""
+        last = min(q + R - 1, KT - 1) if q >= 0 else min(R - 2, KT - 1)
+        return max(0, last - (q + 2)) * len(parts)
+
+    a("  // a period ends when every wave is here")
+    a('  #define EMH_PHASE_END() { asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }')
+    steady = max(0, KT - R + 1)  # periods q for which slab q + R - 1 exists
+    a("  if (role == 2) {  // ---- producers")
+    a(f"    EMH_SLAB_SYNC({allowed(-1)});  // period -1")
+    if steady:
+        a(f"    for (int kt = 0; kt < {steady}; ++kt) {{")
+        request("kt")
+        a(f"      EMH_SLAB_SYNC({allowed(0)});")
+        a("    }")
+    for q in range(steady, KT):
+        a(f"    EMH_SLAB_SYNC({allowed(q)});")
+    a("  } else if (role == 0) {  // ---- consumer group 0")
+    a("    {")
+    fetch("0")
+    a("      EMH_PHASE_END(); }  // period -1")
+    a(f"    for (int kt = 0; kt < {KT}; ++kt) {{")
+    compute()
+    a(f"      if (kt + 1 < {KT}) {{")
+    fetch("kt + 1")
+    a("      }")
+    a("      EMH_PHASE_END();")
+    a("    }")
+    a("  } else {  // ---- consumer group 1")
+    a("    EMH_PHASE_END();  // period -1")
+    a(f"    for (int kt = 0; kt < {KT}; ++kt) {{")
+    fetch("kt")
+    compute()
+    a("      EMH_PHASE_END();")
+    a("    }")
+    a("  }")
+
+
 def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> HipOp:
     plan = body.tile
     if plan is None:
@@ -179,7 +261,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     if split is not None:
         if body.epilogue is not None or body.post is not None or body.bias is not None or body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None or body.out_dtype is not F32:
             raise LoweringError("contraction: the partial kernel of a split stores bare fp32 accumulators; bias, epilogue and rounding belong to the combine")
-        if stage.transport not in ("sync", "dl", "dli"):
+        if stage.transport not in ("sync", "dl", "dli", "pp"):
             raise LoweringError(f"contraction: STAGE .../{stage.transport} does not combine with a cross-workgroup split")
     M, N, K = body.m, body.n, body.k
     lda = body.lda or K
@@ -216,12 +298,15 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     NB = 2 if gate else 1  # weight matrices consumed per pass
     a_chunks = TM * CPR
     b_chunks = TN * CPR * NB
-    if a_chunks % T or b_chunks % T:
-        raise LoweringError(f"contraction: tile {TM}x{TN}x{BK} does not divide over {T} threads")
-    A_PER_T, B_PER_T = a_chunks // T, b_chunks // T
+    # STAGE .../pp: the tile's waves compute; four more waves (one per SIMD) do all the staging
+    ST = PP_PRODUCER_THREADS if stage.transport == "pp" else T  # threads that stage operands
+    TT = T + PP_PRODUCER_THREADS if stage.transport == "pp" else T  # threads launched
+    if a_chunks % ST or b_chunks % ST:
+        raise LoweringError(f"contraction: tile {TM}x{TN}x{BK} does not divide over {ST} threads")
+    A_PER_T, B_PER_T = a_chunks // ST, b_chunks // ST
     slab_bytes = (TM + TN * NB) * BK * ES
     depth = 2 if stage.transport == "mix" else max(2, stage.depth)
-    RS = 1 if stage.transport in ("dl", "dli", "mix") else max(1, stage.reg_depth)  # register sets a slab travels through on the sync path
+    RS = 1 if stage.transport in ("dl", "dli", "pp", "mix") else max(1, stage.reg_depth)  # register sets a slab travels through on the sync path
     lds_bytes = slab_bytes * depth
     if lds_bytes > ctx.lds_bytes_per_cu:
         raise LoweringError(f"contraction: {lds_bytes} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
@@ -247,7 +332,9 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
             gn -= 1
     n_guard = N % TN != 0
     dli = stage.transport == "dli"  # direct to LDS, requests issued between the MFMAs of the slab before (see below)
-    dl = stage.transport in ("dl", "dli")
+    pp = stage.transport == "pp"  # direct to LDS, the two waves of a SIMD in opposite phases (one computes, one fetches)
+    spec = pp  # specialised waves: the tile's own compute, four more stage
+    dl = stage.transport in ("dl", "dli", "pp")
     mix = stage.transport == "mix"  # a through registers (it is transformed on the way), b direct to LDS
     if mix and b_chunks % 64:
         raise LoweringError("contraction: direct-to-LDS staging needs whole-wave chunk counts")
@@ -298,7 +385,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
         params.append(f"int {sym_for_params.name}")
 
     D = dict(
-        name=name, T=T, M=M, N=N, K=K, LDA=lda, LDB=ldb, LDO=ldo, TM=TM, TN=TN, BK=BK, WM=WM, WN=WN, FM=FM, FN=FN,
+        name=name, T=T, ST=ST, TT=TT, M=M, N=N, K=K, LDA=lda, LDB=ldb, LDO=ldo, TM=TM, TN=TN, BK=BK, WM=WM, WN=WN, FM=FM, FN=FN,
         AM=AM, KG=KG, KSTEP=KSTEP, ACC=ACC, ES=ES, EPCK=EPCK, MPF=MPF, CPR=CPR, RPL=RPL, NB=NB, A_PER_T=A_PER_T, B_PER_T=B_PER_T,
         SLAB=slab_bytes, DEPTH=depth, RS=RS, KT=KT, TILES_M=tiles_m, TILES_N=tiles_n, NTILES=n_tiles, GM=gm, GN=gn,
         XCDS=ctx.xcds, frag_t=frag_t, in_c=in_c, out_c=out_c, params=", ".join(params), builtin=plan.atom.builtin,
@@ -316,7 +403,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     a(r"""
 EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
 """)
-    a(f'extern "C" __global__ __launch_bounds__({T}) void {name}({D["params"]}) {{')
+    a(f'extern "C" __global__ __launch_bounds__({TT}) void {name}({D["params"]}) {{')
     a(r"""  extern __shared__ __attribute__((aligned(16))) unsigned char emh_lds[];
   // ---- tile ownership: consecutive workgroup ids rotate over the XCDs ----
   const int bid = blockIdx.x;
@@ -339,7 +426,8 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   }
   const int m0 = tm * TM, n0 = tn * TN;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-  const int wm = wave / WN, wn = wave % WN;
+  const int stid = tid >= T ? tid - T : tid;  // staging thread id (the waves past the tile's own only stage)
+  const int wm = (wave / WN) % WM, wn = wave % WN;
   const int lr = lane % AM, lk = lane / AM;  // fragment row, k-group
 """)
     if split is not None:
@@ -351,15 +439,15 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     # ---- staging ------------------------------------------------------------
     a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else "") + (" int ka[A_PER_T], kb[B_PER_T];" if k_guard else ""))
     a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
-    if dli:
+    if dli or spec:
         if max(M * lda, N * NB * ldb) * ES >= 2**32:
             raise LoweringError("contraction: STAGE .../dli addresses operands with 32-bit byte offsets; this operand is larger than 4 GiB")
         a("  unsigned va[A_PER_T], vb[B_PER_T];  // byte offset of each request's chunk from the operand base (the k position is added to the base, in scalar registers)")
-        a("  const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);  // wave-uniform by construction; says so to the compiler")
+        a("  const int wave_u = __builtin_amdgcn_readfirstlane(stid / 64);  // wave-uniform by construction; says so to the compiler")
         a("  const unsigned lds0 = emh_lds_addr(emh_lds);")
     a(r"""  #pragma unroll
   for (int i = 0; i < A_PER_T; ++i) {
-    const int q = tid + i * T;""")
+    const int q = stid + i * ST;""")
     if dl:
         a("    const int row = q / CPR, c = emh_swz(row, q % CPR);  // lane order fixes the LDS slot; pick the chunk that belongs there")
         a("    la[i] = q * 16;")
@@ -368,7 +456,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         a("    la[i] = row * (BK * ES) + emh_swz(row, c) * 16;")
     a(f"    int gr = m0 + row;{' if (gr > M - 1) gr = M - 1;' if m_guard else ''}")
     a(f"    ga[i] = A + {body.a_offset}L + KSL + (long)gr * LDA + c * EPCK;")
-    if dli:
+    if dli or spec:
         a("    va[i] = ((unsigned)gr * LDA + c * EPCK) * (unsigned)ES;")
     if pro is not None:
         a("    ca[i] = c * EPCK;")
@@ -377,7 +465,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     a("  }")
     a(r"""  #pragma unroll
   for (int i = 0; i < B_PER_T; ++i) {
-    const int q = tid + i * T;""")
+    const int q = stid + i * ST;""")
     if dl or mix:
         a("    const int row = q / CPR, c = emh_swz(row, q % CPR);")
         a("    lb[i] = TM * BK * ES + q * 16;")
@@ -391,7 +479,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     else:
         a(f"    int gr = n0 + row;{' if (gr > N - 1) gr = N - 1;' if n_guard else ''}")
     a(f"    gb[i] = B + {body.b_offset}L + KSL + (long)gr * LDB + c * EPCK;")
-    if dli:
+    if dli or spec:
         a("    vb[i] = ((unsigned)gr * LDB + c * EPCK) * (unsigned)ES;")
     if k_guard:
         a("    kb[i] = c * EPCK;")
@@ -408,7 +496,8 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   for (int r = 0; r < ACC; ++r) acc[h][i][j][r] = 0.0f;
 """)
     a("  #define EMH_OPND(f, e) " + ("((f)[e])  /* one element of the chunk per MFMA */" if MPF > 1 else "(f)"))
-    frag_decl = f"  {frag_t} fw[2][NB][FN], fx[2][FM];"
+    KS = BK // KSTEP
+    frag_decl = f"  {frag_t} fw[{max(2, KS) if pp else 2}][NB][FN], fx[{max(2, KS) if pp else 2}][FM];"
     a(frag_decl)
     a(r"""  // Fragments are double-buffered in registers: the reads for step s+1 are
   // issued before the MFMAs of step s and complete in their shadow.  The
@@ -434,7 +523,6 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
       acc[h][i][j] = BUILTIN(EMH_OPND(fw[P][h][j], e), EMH_OPND(fx[P][i], e), acc[h][i][j], 0, 0, 0); \
     __builtin_amdgcn_sched_barrier(0); }
 """.replace("FRAG_T", frag_t).replace("BUILTIN", plan.atom.builtin))
-    KS = BK // KSTEP
     if not dl:
         # global -> VGPR -> LDS, one slab ahead, one barrier per slab.  With the
         # mixed transport only the a operand takes that road (it may be transformed on
@@ -525,8 +613,10 @@ ROW_EPILOGUE_TABLES
   }
   }""")
     else:
-        if KS % 2:
+        if KS % 2 and not pp:
             raise LoweringError(f"contraction: direct-to-LDS pipeline needs an even number of MFMA steps per slab (BK={BK}, step={KSTEP})")
+        if pp and (T != 512 or deferred or rowepi is not None or depth < 3):
+            raise LoweringError("contraction: STAGE .../pp takes a tile of eight waves (two groups of four alternate, four more waves stage), a ring of at least three, and no row prologue or row epilogue")
         loads_per_slab = A_PER_T + B_PER_T
         if (depth - 1) * loads_per_slab > 63:
             raise LoweringError("contraction: too many loads in flight for the 6-bit vmcnt counter; lower STAGE depth")
@@ -552,12 +642,12 @@ ROW_EPILOGUE_TABLES
     emh_lds_publish(emh_lds + tid * 4); \
     asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
   #pragma unroll
-  for (int p = 0; p < DEPTH - DLI; ++p) if (p < KT) EMH_DLOAD(p, p);""".replace("DLI", "1" if dli else "0"))
-        if dli:
+  for (int p = 0; p < DEPTH - DLI; ++p) if (p < KT STAGER) EMH_DLOAD(p, p);""".replace("DLI", "1" if dli or pp else "0").replace(" STAGER", " && tid >= T" if spec else ""))
+        if dli or spec:
             a(f"""  // One request of slab kt into ring buffer buf: the operand base moves along k in scalar registers, the
   // lane's chunk offset is a loop-invariant 32-bit register, the LDS target a scalar: no vector arithmetic per request.
-  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L + KSL) + (long)(kt) * (BK * ES), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * T) * 16)
-  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L + KSL) + (long)(kt) * (BK * ES), vb[i], lds0 + (buf) * SLAB + TM * BK * ES + (wave_u * 64 + (i) * T) * 16)""")
+  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L + KSL) + (long)(kt) * (BK * ES), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * ST) * 16)
+  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L + KSL) + (long)(kt) * (BK * ES), vb[i], lds0 + (buf) * SLAB + TM * BK * ES + (wave_u * 64 + (i) * ST) * 16)""")
         if deferred:
             # the rows arrive in LDS untouched: every thread reads back the chunks it requested
             # (any chunk of the row will do for a row sum) while the slab is resident
@@ -571,10 +661,15 @@ ROW_EPILOGUE_TABLES
             a('    _Pragma("unroll") for (int i = 0; i < A_PER_T; ++i) \\')
             a('    _Pragma("unroll") for (int e = 0; e < 8; ++e) { const float x_ = (float)sx[i][e]; ss[i] += ' + E.render(pro.stat_pre, {"x": "x_"}) + "; } \\")
             a("    __builtin_amdgcn_sched_barrier(0); }")
-        first_younger = min(depth - 1 - (1 if dli else 0), KT - 1) * loads_per_slab
+        first_younger = min(depth - 1 - (1 if dli or pp else 0), KT - 1) * loads_per_slab
         a(f"  EMH_SLAB_SYNC({first_younger});")
-        a("  EMH_READ(0, 0, 0);")
+        if not spec:
+            a("  EMH_READ(0, 0, 0);")
         a("ROW_EPILOGUE_TABLES")
+        if pp:
+            a("  const int role = __builtin_amdgcn_readfirstlane(tid / 256);  // 0, 1: the two consumer groups (waves 0-3, 4-7); 2: the producers")
+            part_fmt = [f"EMH_DPART_A({{slab}}, {{buf}}, {i});" for i in range(A_PER_T)] + [f"EMH_DPART_B({{slab}}, {{buf}}, {i});" for i in range(B_PER_T)]
+            _emit_pingpong_loop(a, KT=KT, KS=KS, depth=depth, parts=part_fmt)
 
         def slab_steps(kt: str, static_kt: int | None) -> None:
             """MFMA steps of slab ``kt``.  With ``static_kt`` the hand-over to the
@@ -647,7 +742,9 @@ ROW_EPILOGUE_TABLES
                     a("    EMH_SUMSQ_ADD();")
             a("    }")
 
-        if dli:
+        if spec:
+            pass
+        elif dli:
             steady = max(0, KT - depth + 1)
             if steady:
                 a(f"  for (int kt = 0; kt < {steady}; ++kt) {{")
@@ -700,6 +797,8 @@ ROW_EPILOGUE_TABLES
         a(f"  constexpr int CSTRIDE = {c_stride};")
         a("  __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM_LGKM0(0));" if dl else "")
         a("  __syncthreads();  // every wave is done with the operand slabs; reuse them for the output tile")
+        if spec:
+            a("  if (tid < T) {  // the staging waves hold no accumulators")
         a(r"""  #pragma unroll
   for (int i = 0; i < FM; ++i) {
     const int ml = (wm * FM + i) * AM + lr;""")
@@ -726,7 +825,11 @@ ROW_EPILOGUE_TABLES
         a(f"      *({vt4}*)(emh_lds + ml * CSTRIDE + nl * {esz}) = yo;")
         a("    }")
         a("  }")
+        if spec:
+            a("  }")
         a("  __syncthreads();")
+        if spec:
+            a("  if (tid >= T) return;  // no barrier follows")
         vt_chunk = rt.vector_type(body.out_dtype.name, EPC)[0]
         a(f"  constexpr int CPRC = TN / {EPC};  // 16-byte chunks per output-tile row")
         if rowepi is not None:
@@ -766,6 +869,8 @@ ROW_EPILOGUE_TABLES
     else:
         if rowepi is not None:
             raise LoweringError("contraction: the row epilogue works on the staged output tile, which this tile shape does not have")
+        if spec:
+            a("  if (tid >= T) return;  // the staging waves hold no accumulators, and no barrier follows")
         a(r"""  #pragma unroll
   for (int i = 0; i < FM; ++i) {
     const int m = m0 + (wm * FM + i) * AM + lr;""")
@@ -839,7 +944,7 @@ ROW_EPILOGUE_TABLES
             *(body.operand_buffers.get(n, n) for n in epi_names), *(rowepi.operand_buffers.get(ro.name, ro.name) for ro in (rowepi.row_operands if rowepi is not None else ())), body.out,
         ),  # fmt: skip
         grid=((grid,), (split[0] if split is not None else 1,), (1,)),
-        block=((T,), (1,), (1,)),
+        block=((TT,), (1,), (1,)),
         lds_bytes=lds_bytes,
         zero_outputs=(body.out,) if split is not None and split[1] == "atomic" else (),
         comment=(f"partial of a {split[0]}-way split ({split[1]}) " if split is not None else "") + f"contraction M={M} N={N} K={K} TILE={plan.spell()} STAGE={stage.spell()}" + ((" a=row-scaled-after" if deferred else " a=row-normalised") if pro is not None else "") + (f" row-epilogue={rowepi.col_end // rowepi.cols}x{rowepi.cols}" if rowepi is not None else ""),

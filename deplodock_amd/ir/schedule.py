@@ -239,7 +239,7 @@ class TilePlan:
 # STAGE
 # --------------------------------------------------------------------------
 
-_TRANSPORTS = {"sync": "sync", "dl": "dl", "dli": "dli", "cp": "dl", "mix": "mix", "ks": "ks"}
+_TRANSPORTS = {"sync": "sync", "dl": "dl", "dli": "dli", "pp": "pp", "cp": "dl", "mix": "mix", "ks": "ks"}
 
 
 @dataclass(frozen=True)
@@ -252,6 +252,9 @@ class Stage:
                    ``dl``: global loads that write LDS directly, no VGPR hop;
                    ``dli``: the same loads, issued one at a time between the MFMAs of
                    the slab before instead of as a burst behind its barrier;
+                   ``pp``: the same loads issued by four extra waves (one per SIMD) that
+                   do nothing else, while the tile's eight waves alternate in two groups
+                   half a slab apart (one computes while the other reads fragments);
                    ``mix``: the a operand as ``sync``, the b operand as ``dl``;
                    ``ks``: no LDS staging — at most 16 rows, the reduction axis split
                    over ``depth`` waves that load their fragments straight from global

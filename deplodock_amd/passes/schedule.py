@@ -277,6 +277,32 @@ def _check_tile(plan: TilePlan, body: Contraction, ctx: Context, depth: int, dl:
 from deplodock_amd.emit.skinny import skinny_waves  # noqa: E402
 
 
+def pingpong_fits(plan: TilePlan, body: Contraction, ctx: Context, depth: int = 4, worthwhile: bool = True) -> bool:
+    """Whether ``STAGE d<depth>/pp`` can be emitted for this tile, and (``worthwhile``) is worth it: eight waves own the tile (four
+    more stage), a wave holds a whole slab's fragments beside its accumulators in the 168 registers a lane has at
+    three waves a SIMD, the ring fits the LDS, the four staging waves' requests fit the six-bit counter, and a wave
+    has at least 256 clocks of MFMA work a slab (the period's barrier costs about 120).  Measured against the
+    default ``dl`` ring (us, same process): 2048x3072x1024 on the 128x192 tile 17.2 -> 13.6; 2048^3 on 128x128
+    21.3 -> 19.6; shorter steps lose (1024^3 on 64x64: 4.8 -> 5.0, 512x4096x1024 on 64x128: 7.0 -> 7.7)."""
+    if plan.block_threads != 512 or body.a_prologue is not None or body.row_epilogue is not None or body.k % plan.bk_elems:
+        return False
+    nb = 2 if body.gate_pair else 1
+    fm, fn = plan.regs
+    steps = plan.bk_elems // plan.atom.frag_k
+    if plan.bk_elems % plan.atom.frag_k or steps < 1:
+        return False
+    mfma_per_step = (plan.atom.frag_k // plan.atom.k) * fm * fn * nb
+    mfma_clocks = plan.atom.m * plan.atom.n * plan.atom.k * 2 // 1024  # 16 for a 16x16x32 16-bit atom, 32 for 32x32x16
+    regs = steps * (nb * fn + fm) * 4 + fm * fn * nb * plan.atom.acc_per_lane
+    chunks = (plan.tile_m + plan.tile_n * nb) * (plan.bk_elems * plan.atom.elem_bytes // 16)
+    slab = (plan.tile_m + plan.tile_n * nb) * plan.bk_elems * plan.atom.elem_bytes
+    return (
+        regs <= 136 and slab * depth <= ctx.lds_bytes_per_cu and chunks % 256 == 0 and (plan.tile_m * plan.bk_elems * plan.atom.elem_bytes // 16) % 256 == 0
+        and (depth - 1) * (chunks // 256) <= 63 and depth >= 3
+        and (not worthwhile or (steps * mfma_per_step * mfma_clocks >= 256 and -(-body.k // plan.bk_elems) >= depth))
+    )  # fmt: skip
+
+
 def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
     """Staging when nothing pins it.
 
@@ -292,6 +318,7 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
       At M = 128 the ring on the eight-wave 32x64 tile ties that when the weight comes from
       HBM (6.25 vs 6.27 us) and wins when it sits in the caches (4.02 vs 4.64 us); inside the
       decoder block at 64 tokens the ring wins on every projection (o: 4.11 vs 5.00 us).
+    * Where :func:`pingpong_fits`: the wave-specialised ring (``d4/pp``).
     * Everything else: direct-to-LDS loads; a ring of three slabs where the LDS holds them
       and a slab is less than ~600 cycles of MFMA work, else two (us, ``d2/sync`` -> ``d2/dl`` -> ``d3/dl``: 512x1024x3072 12.2 -> 9.5 ->
       9.4; 512x1024x2048 7.4 -> 6.2 -> 6.2; 512x4096x1024 7.8 -> 6.8 -> 6.7; 2048x3072x1024
@@ -305,6 +332,8 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
         return Stage(depth=2, transport="sync")  # transformed in registers on its way to LDS
     if body.m <= 16:
         return Stage(depth=2, transport="sync", reg_depth=2 if steps >= 3 else 1)
+    if body.k_split is None and body.in_dtype.nbytes == 2 and pingpong_fits(plan, body, ctx):
+        return Stage(depth=4, transport="pp")
     if (plan.bk_elems // plan.atom.frag_k) % 2 == 0 and plan.bk_elems % plan.atom.frag_k == 0:
         # a slab that keeps the matrix pipe busy for long hides the next one's latency by itself
         mfma_cycles = plan.tile_m * plan.tile_n * (2 if body.gate_pair else 1) * plan.bk_elems * 2 // 4096
@@ -374,6 +403,9 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
             if stage is not None and stage.transport == "ks":
                 if not skinny_waves(body) or stage.depth not in (1, 2, 4, 8, 16) or body.k % (32 * stage.depth):
                     raise ScheduleError(f"the k-split few-row form does not fit M={body.m} N={body.n} K={body.k} with {stage.depth} waves")
+            elif stage is not None and stage.transport == "pp":
+                if not pingpong_fits(plan, body, ctx, depth=stage.depth, worthwhile=False):
+                    raise ScheduleError("the wave-specialised ring takes a plain 16-bit contraction on an eight-wave tile whose slab fragments fit a lane's registers, and a ring of at least three that fits the LDS")
             elif stage is not None:
                 _check_tile(plan, body, ctx, depth=max(2, stage.depth), dl=stage.transport == "dl")
         except ScheduleError as exc:

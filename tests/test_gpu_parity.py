@@ -921,6 +921,44 @@ def test_staging_transports_are_bit_identical(device, monkeypatch):
     eager.assert_close(outs["d2/sync"], eager.run_eager(case, device), case.rtol, case.atol, "pinned tile vs eager")
 
 
+@pytest.mark.parametrize("dims,tile", [((256, 1024, 384), "a:mfma_16x16x32_bf16/w2x4/f4x3/k2"), ((200, 512, 388), "a:mfma_16x16x32_bf16/w2x4/f4x3/k2"),
+                                       ((512, 192, 512), "a:mfma_16x16x32_bf16/w4x2/f2x4/k2"), ((384, 64, 256), "a:mfma_32x32x16_bf16/w2x4/f1x1/k4")])  # fmt: skip
+def test_wave_specialised_ring_is_bit_identical_to_register_staging(device, dims, tile, monkeypatch):
+    """``STAGE d<n>/pp`` (four staging waves, the tile's eight waves alternating in two groups) at every ring depth
+    it takes, on whole and ragged tiles, long and short reduction axes (fewer slabs than the ring holds included):
+    the same bits as ``d2/sync`` on the same tile, launch after launch."""
+    m, k, n = dims
+    case = eager.linear_case(m=m, k=k, n=n, seed=31)
+    graph = trace_module(case.module, case.inputs)
+    x = case.inputs[0].to(device)
+    monkeypatch.setenv("EMMY_TILE", tile)
+    outs = {}
+    for stage in ("d2/sync", "d3/pp", "d4/pp", "d5/pp"):
+        monkeypatch.setenv("EMMY_STAGE", stage)
+        be = HipBackend()
+        compiled = be.compile(graph)
+        (op,) = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+        if op.knobs["STAGE"] != stage:
+            assert stage == "d5/pp"  # the deepest ring does not fit the LDS on the larger tiles
+            continue
+        assert stage.endswith("sync") or op.block[0] == (768,)
+        prog = be.program(compiled, {compiled.inputs[0]: x})
+        try:
+            for _ in range(30):
+                prog.run()
+                torch.cuda.synchronize()
+                y = prog.output_tensors()[compiled.outputs[0]].clone()
+                if stage in outs:
+                    assert torch.equal(y, outs[stage]), f"{stage}: outputs differ between launches"
+                outs[stage] = y
+        finally:
+            prog.close()
+    assert len(outs) >= 3
+    for stage, y in outs.items():
+        assert torch.equal(y, outs["d2/sync"]), f"{stage} differs from d2/sync"
+    eager.assert_close(outs["d2/sync"], eager.run_eager(case, device), case.rtol, case.atol, f"{tile} vs eager")
+
+
 def _soak(prog, out_name: str, launches: int, what: str) -> None:
     """``launches`` runs of a bound program on fixed inputs, every output compared bit for bit with the first
     launch's; stops at the first mismatch."""
@@ -937,7 +975,7 @@ def _soak(prog, out_name: str, launches: int, what: str) -> None:
             pytest.fail(f"{what}: launch {i} of {launches} differs from the first launch in {bad} elements")
 
 
-@pytest.mark.parametrize("stage", ["d3/dl", "d3/dli"])
+@pytest.mark.parametrize("stage", ["d3/dl", "d3/dli", "d4/pp", "d3/pp"])
 def test_soak_direct_to_lds_contraction_is_bit_stable_over_thousands_of_launches(device, stage, monkeypatch):
     """The publication fence of the direct-to-LDS rings (a flat LDS read of the issuing wave, waited for on the
     LDS counter, before the barrier) as a test: a race that let one wave read a slab before another wave's loads
