@@ -35,7 +35,7 @@ from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.ir.schedule import Stage
-from deplodock_amd.ir.sym import Affine, XcdRounds, c_value
+from deplodock_amd.ir.sym import Affine, XcdRounds, c_value, param_name
 from deplodock_amd.ir.tile import Contraction
 
 
@@ -382,7 +382,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     params.append(f"{out_c}* __restrict__ O")
     sym_for_params = getattr(body, "sym", None)
     if sym_for_params is not None and sym_for_params.fields:
-        params.append(f"int {sym_for_params.name}")
+        params.append(f"int {param_name(sym_for_params.name)}")
 
     D = dict(
         name=name, T=T, ST=ST, TT=TT, M=M, N=N, K=K, LDA=lda, LDB=ldb, LDO=ldo, TM=TM, TN=TN, BK=BK, WM=WM, WN=WN, FM=FM, FN=FN,

@@ -45,7 +45,7 @@ from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir.expr import float_literal
 from deplodock_amd.ir.hip import HipOp
-from deplodock_amd.ir.sym import Affine, CeilDiv, c_value
+from deplodock_amd.ir.sym import Affine, CeilDiv, c_value, param_name
 from deplodock_amd.ir.tile import Flash
 
 # The key range of a workgroup's query rows is split over KVS wave groups.  Group g
@@ -66,7 +66,8 @@ EMH_DEV float emh_xor32(float v) { return __shfl_xor(v, 32, 64); }
 typedef short emh_s16x4 __attribute__((ext_vector_type(4)));
 #define KBYTES (BKV * D * 2)
 #define WQ (NT / 64 / KVS)           /* waves (32-row groups) per key-split group */
-#define STEP_BYTES (KVS * 2 * KBYTES)  /* one step: K and V block of every group */
+#define SETB (KVS * KBYTES)          /* one ring slot: the K (or V) blocks of a step, one per key-split group */
+#define V_RING (RK * SETB)           /* LDS: [K ring: RK slots][V ring: RV slots] */
 #define QCHUNKS (BQ * CPR)             /* 16-byte chunks of a workgroup's Q (and O) tile */
 #define RPL (D / 32 * 16)              /* output registers per lane */
 #define RPG (RPL / KVS)                /* ... of which each key-split group finishes this many */
@@ -96,6 +97,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   const ELT* vbase = Vp + V_OFF + (long)batch * V_SB + (long)kvh * V_SH;
   #pragma unroll 1
   for (int pass = 0; pass < (PAIR ? 2 : 1); ++pass) {
+  if (PAIR && pass) __syncthreads();  // every thread is done copying the first block's O tile out of LDS
   const int qb = pass == 0 ? (QBLOCKS - 1) - slot : slot;
   const int q0 = qb * BQ;
   const int qw0 = q0 + wq * 32;
@@ -141,30 +143,57 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   const ELT* gk_lane = kbase + (long)st_row * K_SS;
   const ELT* gv_lane = vbase + (long)st_row * V_SS;
   const int dst_lane = (tid - lane) * 16;
-  #define EMH_STAGE_PART(st, buf, i) { \
-      unsigned char* sb_ = lds + (buf) * STEP_BYTES + dst_lane; \
+  const unsigned lds0 = emh_lds_addr(lds);
+  const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);  // wave-uniform by construction; says so to the compiler
+  // A request whose key block lies wholly inside the sequence is a scalar base (the head's K or V plane, moved
+  // along the keys per step in scalar registers), a loop-invariant 32-bit lane offset and a scalar LDS target:
+  // no vector arithmetic per request.  Only a block that hangs over the end clamps its rows per lane.
+  unsigned kvo[PER_T], vvo[PER_T];
+  #pragma unroll
+  for (int i = 0; i < PER_T; ++i) {
+    const int g_ = (i * NT) / CHUNKS, ro_ = ((i * NT) % CHUNKS) / CPR;
+    kvo[i] = (unsigned)((g_ * BKV + ro_ + st_row) * K_SS + emh_kswz(st_row + ro_, st_pos) * 8) * 2u;
+    vvo[i] = (unsigned)((g_ * BKV + ro_ + st_row) * V_SS + emh_vswz(st_row + ro_, st_pos) * 8) * 2u;
+  }
+  // EMH_STEP_BASES(st) names the scalar parts of the requests of step st once (K and V plane bases moved to the
+  // step's keys, the ring slots' LDS addresses); EMH_STAGE_K / _V(st, i) then issue request i against them.
+  #define EMH_STEP_BASES(tag, st) \
+      const unsigned char* kb##tag = emh_uniform((const unsigned char*)kbase + (long)(st) * (KVS * BKV) * K_SS * 2); \
+      const unsigned char* vb##tag = emh_uniform((const unsigned char*)vbase + (long)(st) * (KVS * BKV) * V_SS * 2); \
+      const unsigned kl##tag = emh_uniform(lds0 + ((st) % RK) * SETB + wave_u * 1024); \
+      const unsigned vl##tag = emh_uniform(lds0 + V_RING + ((st) % RV) * SETB + wave_u * 1024);
+  #define EMH_STAGE_ONE(st, i, sb_, lb_, base_, stride_, off_, swz_, ldo_) { \
       const int g_ = ((i) * NT) / CHUNKS, ro_ = (((i) * NT) % CHUNKS) / CPR; \
-      long krow_ = (long)((st) * KVS + g_) * BKV + ro_; \
-      if (SKV % (KVS * BKV) != 0) { const long lim_ = SKV - 1 - st_row; if (krow_ > lim_) krow_ = lim_; } \
-      const int kc_ = emh_kswz(st_row + ro_, st_pos), vc_ = emh_vswz(st_row + ro_, st_pos); \
-      unsigned char* dk_ = sb_ + g_ * 2 * KBYTES + (((i) * NT) % CHUNKS) * 16; \
-      emh_dma16(gk_lane + krow_ * K_SS + kc_ * 8, dk_); \
-      emh_dma16(gv_lane + krow_ * V_SS + vc_ * 8, dk_ + KBYTES); }
-  // Request i of a step is issued behind score MFMA number EMH_SLOT_OF(i): spread
-  // evenly over the chain, so the loads trickle into the memory pipeline instead of
-  // arriving as one burst from every wave, and all of them are on their way before
-  // the softmax starts (requests issued later land after the step's fence).
+      if (SKV % (KVS * BKV) == 0 || ((st) * KVS + g_ + 1) * BKV <= SKV) { \
+        emh_dma16s(sb_, off_[i], (lb_) + g_ * KBYTES + (((i) * NT) % CHUNKS) * 16); \
+      } else { \
+        long krow_ = (long)((st) * KVS + g_) * BKV + ro_ + st_row; \
+        if (krow_ > SKV - 1) krow_ = SKV - 1; \
+        emh_dma16((base_) + krow_ * (stride_) + swz_(st_row + ro_, st_pos) * 8, lds + (ldo_) + g_ * KBYTES + (((i) * NT) % CHUNKS) * 16 + dst_lane); } }
+  #define EMH_STAGE_K(tag, st, i) EMH_STAGE_ONE(st, i, kb##tag, kl##tag, kbase, K_SS, kvo, emh_kswz, ((st) % RK) * SETB)
+  #define EMH_STAGE_V(tag, st, i) EMH_STAGE_ONE(st, i, vb##tag, vl##tag, vbase, V_SS, vvo, emh_vswz, V_RING + ((st) % RV) * SETB)
+  // Requests are issued between MFMAs, spread evenly over a chain of NQ_SLOTS of them (request i behind MFMA
+  // number EMH_SLOT_OF(i)): they trickle into the memory pipeline instead of arriving as one burst from every wave.
   #define NQ_SLOTS ((BKV / 32) * (D / 16))
   #define EMH_SLOT_OF(i) (((i) * NQ_SLOTS) / PER_T)
-  #define EMH_STAGE(st, buf) { _Pragma("unroll") for (int i = 0; i < PER_T; ++i) EMH_STAGE_PART(st, buf, i) }
+  #define EMH_STAGE_ALL_K(st) { EMH_STEP_BASES(_a, st) _Pragma("unroll") for (int i = 0; i < PER_T; ++i) EMH_STAGE_K(_a, st, i) (void)vb_a; (void)vl_a; }
+  #define EMH_STAGE_ALL_V(st) { EMH_STEP_BASES(_a, st) _Pragma("unroll") for (int i = 0; i < PER_T; ++i) EMH_STAGE_V(_a, st, i) (void)kb_a; (void)kl_a; }
 
-  // Publishing direct-to-LDS data: vmcnt reaching zero does not yet mean the
+  // Publishing direct-to-LDS data: the request counter reaching its target does not yet mean the
   // data is visible to other waves' LDS reads (measured: stale reads right after
   // the barrier).  An LDS read of this wave queues behind its own DMA writes, so
-  // waiting for that read orders them before the barrier.
-  #define EMH_DMA_FENCE() { \
-    __builtin_amdgcn_s_waitcnt(0x0070); /* vmcnt(0) lgkmcnt(0) */ \
-    emh_lds_publish(lds + tid * 4); }
+  // waiting for that read orders them before the barrier.  Requests retire in issue order: "at most c * PER_T
+  // outstanding" means everything issued before the last c request groups has landed.
+  #define EMH_WAIT_VM(n) ((((n) & 0xF) | ((((n) >> 4) & 0x3) << 14)) | 0x0070)  /* vmcnt <= n, lgkmcnt = 0 */
+  #define EMH_LAND(c) { \
+    switch (c) { \
+      case 0: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(0)); break; \
+      case 1: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(PER_T)); break; \
+      case 2: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(2 * PER_T)); break; \
+      case 3: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(3 * PER_T)); break; \
+      default: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(4 * PER_T)); break; } \
+    emh_lds_publish(lds + tid * 4); \
+    __syncthreads(); }
 
   f32x16 oacc[D / 32];
   #pragma unroll
@@ -184,9 +213,21 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   #pragma unroll
   for (int T = 0; T < TG; ++T) v_tile[T] = v_lane + ((T ^ EMH_VROT(q4)) * 64);
 
-  EMH_STAGE(0, 0);
-  EMH_DMA_FENCE();
-  __syncthreads();
+  // DEEP: K runs through a ring of three slots, V through one of two.  K(j) is read by the score MFMAs of step j,
+  // V(j) by its output MFMAs; both are dead at the barrier that ends the step.  During step st the waves request
+  // V(st + 1) (between the score MFMAs) and then K(st + 2) (between the output MFMAs), and the step's end waits
+  // only for what is older than K(st + 2): the V block has the memory pipeline to itself for most of the step,
+  // and a K block has two steps to land.  Otherwise (two slots each): K(st + 1) and V(st + 1) are requested
+  // together during step st and both are waited for at its end.
+  // Issue order: K0 V0 [K1] | step 0: V1, K2 | step 1: V2, K3 | ...
+  EMH_STAGE_ALL_K(0);
+  EMH_STAGE_ALL_V(0);
+  if (DEEP) {
+    if (1 < nsteps) EMH_STAGE_ALL_K(1);
+    EMH_LAND((int)(1 < nsteps));
+  } else {
+    EMH_LAND(0);
+  }
   if (Q_LDS) {
     const int qr_ = wq * 32 + lq;
     #pragma unroll
@@ -200,11 +241,15 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
     const int jt = st * KVS + grp;
     const int k0 = jt * BKV;
     const bool active = (jt < ntiles) && (!CAUSAL || (k0 <= qw0 + 31));
+    EMH_STEP_BASES(1, st + 1)
+    EMH_STEP_BASES(2, st + 2)
+    (void)kb2; (void)kl2; (void)vb2; (void)vl2; (void)kb1; (void)kl1;
     if (!active) {
-      if (more) EMH_STAGE(st + 1, (st + 1) & 1);
+      if (more) { EMH_STAGE_ALL_V(st + 1); if (!DEEP) EMH_STAGE_ALL_K(st + 1); }
+      if (DEEP && st + 2 < nsteps) EMH_STAGE_ALL_K(st + 2);
     } else {
-      const unsigned char* sK = lds + (st & 1) * STEP_BYTES + grp * 2 * KBYTES;
-      const unsigned char* sV = sK + KBYTES;
+      const unsigned char* sK = lds + (st % RK) * SETB + grp * KBYTES;
+      const unsigned char* sV = lds + V_RING + (st % RV) * SETB + grp * KBYTES;
       f32x16 sacc[BKV / 32];
       #pragma unroll
       for (int u = 0; u < BKV / 32; ++u) {
@@ -222,7 +267,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
           sacc[u] = MFMA(kf[kk], qf[kk], sacc[u], 0, 0, 0);
           if (more) {
             #pragma unroll
-            for (int i = 0; i < PER_T; ++i) if (EMH_SLOT_OF(i) == u * (D / 16) + kk) EMH_STAGE_PART(st + 1, (st + 1) & 1, i);
+            for (int i = 0; i < PER_T; ++i) if (EMH_SLOT_OF(i) == u * (D / 16) + kk) { EMH_STAGE_V(1, st + 1, i); if (!DEEP) EMH_STAGE_K(1, st + 1, i); }
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -302,11 +347,15 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
           u32x4 av;
           av[0] = l2[0]; av[1] = l2[1]; av[2] = h2[0]; av[3] = h2[1];
           oacc[dt] = MFMA(__builtin_bit_cast(FRAG, av), pf, oacc[dt], 0, 0, 0);
+          if (DEEP && st + 2 < nsteps) {
+            #pragma unroll
+            for (int i = 0; i < PER_T; ++i) if ((i * ((BKV / 32) * 2 * (D / 32))) / PER_T == (u * 2 + s) * (D / 32) + dt) EMH_STAGE_K(2, st + 2, i);
+          }
         }
       }
     }
-    EMH_DMA_FENCE();  // the next step's blocks (they had this whole step to land)
-    __syncthreads();
+    // end of the step: everything but K(st + 2) has landed; every wave is done with K(st) and V(st)
+    EMH_LAND((int)(DEEP && st + 2 < nsteps));
   }
 
   // ---- close.  The key-split groups share the final combine: group g finishes
@@ -314,9 +363,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   // parks the registers the others own, and its (m, l); after one barrier each
   // combines its share with the same exp-family merge the streaming loop uses,
   // scales by 1/l and puts the 16-bit result into the O tile in LDS, which leaves
-  // through 16-byte stores of whole rows.  (The staging buffers are free after the
-  // loop's last barrier; the O tile sits behind the first of them, so the next
-  // pass may start staging without another barrier.)
+  // through 16-byte stores of whole rows.  (The rings are dead after the loop's last barrier.)
   if (KVS > 1) {
     float* park = (float*)lds;
     float* pml = (float*)(lds + PARK_ML) + ((grp * WQ + wq) * 2) * 64 + lane;
@@ -418,23 +465,28 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
 """
 
 
-def lds_plan(waves: int, kvs: int, bkv: int, head_dim: int, limit: int) -> dict:
-    """LDS layout of a workgroup: ``[2 staging buffers | Q tile]``.
+def lds_plan(waves: int, kvs: int, bkv: int, head_dim: int, limit: int, deep: bool = False) -> dict:
+    """LDS layout of a workgroup: ``[K ring | V ring | Q tile]``.
 
-    After the key loop the staging buffers hold the parked partial results of the
-    key-split groups (``(kvs-1) * waves * registers`` lane-vectors and an ``(m, l)``
-    table) and, behind both the parked data and the first staging buffer, the O
-    tile.  The Q tile is staged through LDS only when it fits behind all of that;
-    ``q_off`` is ``None`` when the fragments are read from global memory instead."""
-    step = kvs * 2 * bkv * head_dim * 2
+    A ring slot holds the K (or V) blocks of one step, one per key-split group.  ``deep``: three K slots and two V
+    slots (a K block is requested two steps ahead, and a step's end waits for the next V block only) instead of
+    two and two.
+
+    After the key loop the rings hold the parked partial results of the key-split groups (``(kvs-1) * waves *
+    registers`` lane-vectors and an ``(m, l)`` table) and, behind them, the O tile.  The Q tile is staged through
+    LDS only when it fits behind all of that; ``q_off`` is ``None`` when the fragments are read from global
+    memory instead."""
+    slot = kvs * bkv * head_dim * 2
+    rk, rv = (3, 2) if deep else (2, 2)
+    ring = (rk + rv) * slot
     regs = head_dim // 32 * 16
     park_ml = (kvs - 1) * waves * regs * 256
     park = park_ml + (kvs * waves * 512 if kvs > 1 else 0)
     tile = 32 * waves * head_dim * 2
-    o_off = max(park, step)
-    end = max(2 * step, o_off + tile)
+    o_off = park
+    end = max(ring, o_off + tile)
     q_off = end if end + tile <= limit else None
-    return {"bytes": end + (tile if q_off is not None else 0), "q_off": q_off, "o_off": o_off, "park_ml": park_ml}
+    return {"bytes": end + (tile if q_off is not None else 0), "q_off": q_off, "o_off": o_off, "park_ml": park_ml, "rk": rk, "rv": rv, "deep": deep}
 
 
 def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
@@ -458,7 +510,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         raise LoweringError("flash: a key block's 16-byte chunks must be a multiple of the workgroup's threads")
     if (D // 32 * 16) % (4 * kvs):
         raise LoweringError(f"flash: {kvs} key-split groups cannot share the {D // 32 * 16} output registers of a lane")
-    plan = lds_plan(waves, kvs, BKV, D, ctx.lds_bytes_per_cu)
+    plan = lds_plan(waves, kvs, BKV, D, ctx.lds_bytes_per_cu, deep=body.deep)
     lds = plan["bytes"]
     if lds > ctx.lds_bytes_per_cu:
         raise LoweringError(f"flash: {lds} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
@@ -515,13 +567,14 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "GROUP": body.q_heads // body.kv_heads,
         "QBLOCKS": "((SQ + BQ - 1) / BQ)" if "q_len" in symf else qblocks,
         "QSLOTS": "QBLOCKS" if "q_len" in symf else qslots,
-        "SYM_PARAM": f", int {sym.name}" if symf else "",
+        "SYM_PARAM": f", int {param_name(sym.name)}" if symf else "",
         "HAS_MASK": 1 if has_mask else 0,
         "MASK_PARAM": f", const {rt.type_name(body.mask_dtype.name)}* __restrict__ Mp" if has_mask else "",
         **({"MELT": rt.type_name(body.mask_dtype.name), "MVEC4": rt.vector_type(body.mask_dtype.name, 4)[0], "MASK_VEC": 1 if mask_vec else 0,
             "M_SB": body.mask_strides[0], "M_SH": body.mask_strides[1], "M_SS": body.mask_strides[2], "M_OFF": body.mask_offset,
             "INV_SCALE": float_literal(1.0 / body.scale)} if has_mask else {}),
         "PAIR": 1 if pair else 0,
+        "RK": plan["rk"], "RV": plan["rv"], "DEEP": 1 if plan["deep"] else 0,
         "Q_LDS": 1 if plan["q_off"] is not None else 0,
         "Q_OFF_LDS": plan["q_off"] or 0,
         "O_OFF_LDS": plan["o_off"],
@@ -559,5 +612,5 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         comment=f"flash Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} bkv={BKV} split={kvs} pair={int(pair)}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
-        knobs={"FLASH": f"w{waves}/kv{BKV}/s{kvs}" + ("/p" if pair else "")},
+        knobs={"FLASH": f"w{waves}/kv{BKV}/s{kvs}" + ("/p" if pair else "") + ("/k3" if plan["deep"] else "")},
     )

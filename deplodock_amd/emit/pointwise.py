@@ -15,7 +15,7 @@ from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.emit.reduce import _load_vec, _store_vec
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
-from deplodock_amd.ir.sym import CeilDiv, c_value
+from deplodock_amd.ir.sym import CeilDiv, c_value, param_name
 from deplodock_amd.ir.tile import Map
 
 _T = 256
@@ -50,7 +50,7 @@ def emit_map(body: Map, name: str, ctx: Context = Context()) -> HipOp:
     params = [f"const {rt.type_name(o.dtype.name)}* __restrict__ p{i}" for i, o in enumerate(body.operands)]
     params.append(f"{rt.type_name(body.out_dtype.name)}* __restrict__ out")
     if symf:
-        params.append(f"int {sym.name}")
+        params.append(f"int {param_name(sym.name)}")
     o: list[str] = []
     a = o.append
     a(f"// {name}: numel={body.numel} vec={V}")

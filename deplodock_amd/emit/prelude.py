@@ -53,6 +53,16 @@ EMH_DEV void emh_dma16(const void* g, const void* lds_wave_base) {
 EMH_DEV void emh_dma16s(const void* sbase, unsigned voff, unsigned lds_wave_base) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(voff), "s"(sbase), "s"(lds_wave_base) : "memory", "m0");
 }
+// Values that are wave-uniform by construction but that the compiler may keep in vector registers (they went
+// through a branch on the wave's role): these move them to scalar registers, once, where they are computed.
+EMH_DEV unsigned emh_uniform(unsigned x) { return (unsigned)__builtin_amdgcn_readfirstlane(x); }
+EMH_DEV const unsigned char* emh_uniform(const void* p) {
+  // the builtin returns a signed int: each half goes through unsigned, or a low half with bit 31 set would
+  // sign-extend over the high half
+  const unsigned long b_ = (unsigned long)p;
+  const unsigned lo_ = (unsigned)__builtin_amdgcn_readfirstlane((unsigned)b_), hi_ = (unsigned)__builtin_amdgcn_readfirstlane((unsigned)(b_ >> 32));
+  return (const unsigned char*)(((unsigned long)hi_ << 32) | (unsigned long)lo_);
+}
 """
 
 # Wave64 butterflies.  Each step combines a lane with its partner at XOR

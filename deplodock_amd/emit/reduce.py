@@ -27,7 +27,7 @@ from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
-from deplodock_amd.ir.sym import CeilDiv, c_value
+from deplodock_amd.ir.sym import CeilDiv, c_value, param_name
 from deplodock_amd.ir.tile import RowAddr, RowReduce
 
 _MAX_RESIDENT = 64  # fp32 row elements a lane may keep in registers
@@ -156,7 +156,7 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
     params += [f"const {rt.type_name(ro.dtype.name)}* __restrict__ r{ri}" for ri, ro in enumerate(body.row_operands)]
     params.append(f"{rt.type_name(body.out_dtype.name)}* __restrict__ out")
     if symf:
-        params.append(f"int {sym.name}")
+        params.append(f"int {param_name(sym.name)}")
 
     o: list[str] = []
     a = o.append

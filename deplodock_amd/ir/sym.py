@@ -15,6 +15,12 @@ from __future__ import annotations
 from dataclasses import dataclass
 
 
+def param_name(name: str) -> str:
+    """The C name of the kernel parameter that carries symbol ``name``.  The symbol's own name is the caller's
+    (``s``, ``n``, ``lane`` ...) and may be that of any local of an emitted kernel; the parameter's is reserved."""
+    return f"emh_n_{name}"
+
+
 @dataclass(frozen=True)
 class Affine:
     """``a * <name> + b``."""
@@ -27,8 +33,8 @@ class Affine:
         return self.a * int(env[self.name]) + self.b
 
     def c(self) -> str:
-        """C spelling over the kernel's ``int <name>`` parameter."""
-        core = self.name if self.a == 1 else f"{self.name} * {self.a}"
+        """C spelling over the kernel's ``int`` parameter of this symbol (:func:`param_name`)."""
+        core = param_name(self.name) if self.a == 1 else f"{param_name(self.name)} * {self.a}"
         return f"({core})" if self.b == 0 else f"({core} + {self.b})" if self.b > 0 else f"({core} - {-self.b})"
 
     def __call__(self, env: dict) -> int:  # usable as a launch-time grid factor
@@ -85,4 +91,4 @@ def resolve(v, env: dict) -> int:
     return v.at(env) if isinstance(v, Affine) else int(env[v]) if isinstance(v, str) else int(v)
 
 
-__all__ = ["Affine", "CeilDiv", "XcdRounds", "SymSpec", "c_value", "resolve"]
+__all__ = ["param_name", "Affine", "CeilDiv", "XcdRounds", "SymSpec", "c_value", "resolve"]

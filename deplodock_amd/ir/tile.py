@@ -267,6 +267,7 @@ class Flash:
     waves: int = 4  # 32-row query groups per workgroup
     kv_split: int = 1  # wave groups that split the key blocks of a query group between them
     pair: bool = False  # causal only: a workgroup takes query block b and its mirror QBLOCKS-1-b
+    deep: bool = False  # a K ring of three slots (K blocks requested two steps ahead) beside a V ring of two
     # an additive bias on the scaled scores, ``[batch, head, query, key]`` addressed through (batch, head, query)
     # strides (0 = broadcast) with keys contiguous; ``None``: no mask operand
     mask: str | None = None

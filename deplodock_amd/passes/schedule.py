@@ -446,11 +446,15 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
 def _flash_lds(body: Flash, ctx: Context) -> int:
     from deplodock_amd.emit.flash import lds_plan
 
-    return lds_plan(body.waves, body.kv_split, body.block_kv, body.head_dim, ctx.lds_bytes_per_cu)["bytes"]
+    return lds_plan(body.waves, body.kv_split, body.block_kv, body.head_dim, ctx.lds_bytes_per_cu, deep=body.deep)["bytes"]
 
 
 def schedule_flash(body: Flash, ctx: Context) -> dict:
-    """``EMMY_FLASH=w<row groups>/kv<keys per block>/s<key split>[/p]``.
+    """``EMMY_FLASH=w<row groups>/kv<keys per block>/s<key split>[/p][/k3]``.
+
+    ``/k3`` (a pin only): a K ring of three slots, K blocks requested two steps ahead and a step's end waiting for
+    the next V block alone.  Measured slower on the benchmark shape (S=2048, ``w2/kv32/s4/p``: 27.9 -> 31.8 us; the
+    ring takes the whole LDS, so the Q fragments come from global memory).
 
     Default: eight waves per workgroup, two per SIMD — four 32-row groups x two
     key-split wave groups on 64-key blocks (``w4/kv64/s2``) when that many rows per
@@ -471,10 +475,12 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
     pinned = _pin("FLASH", _tuned(body, ctx))
     if pinned:
         try:
-            body.pair = False
+            body.pair = body.deep = False
             for tok in pinned.split("/"):
                 if tok == "p":
                     body.pair = True
+                elif tok == "k3":
+                    body.deep = True
                 elif tok.startswith("w"):
                     body.waves = int(tok[1:])
                 elif tok.startswith("kv"):
@@ -482,7 +488,7 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 elif tok.startswith("s"):
                     body.kv_split = int(tok[1:])
                 else:
-                    raise ScheduleError(f"cannot parse {tok!r} (expect w<groups> / kv<keys> / s<split> / p)")
+                    raise ScheduleError(f"cannot parse {tok!r} (expect w<groups> / kv<keys> / s<split> / p / k3)")
             chunks = body.block_kv * body.head_dim // 8
             if body.waves < 1 or body.kv_split < 1 or body.block_kv % 32 or chunks % (body.waves * body.kv_split * 64):
                 raise ScheduleError("unrealisable workgroup shape")
@@ -502,7 +508,7 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
         def blocks(w: int) -> int:
             return -(-body.q_len // (32 * w))
 
-        body.pair = False
+        body.pair = body.deep = False
         body.waves = 0
         if body.head_dim <= 128 and body.kv_len >= 2048:
             # Enough rows to give every CU a 256-row workgroup: eight query waves share each
@@ -546,7 +552,7 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 body.kv_split //= 2
     if getattr(body, "sym", None) is not None and body.sym.fields:
         body.pair = False  # pairing mirrored query blocks needs the block count when the kernel is built
-    return {"FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "")}
+    return {"FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "") + ("/k3" if body.deep else "")}
 
 
 def schedule(graph: Graph, ctx: Context | None = None) -> Graph:

@@ -281,6 +281,27 @@ def test_tile_and_stage_pins(launcher_lib, monkeypatch):
     assert "mfma" in k.knobs["TILE"] and k.knobs["STAGE"] == "d4/pp"  # the default staging of this shape
 
 
+def test_uniform_pointer_halves_are_widened_unsigned(launcher_lib):
+    """``emh_uniform`` rebuilds a 64-bit pointer from two ``readfirstlane`` results, which the builtin returns as
+    signed ints: widened as they are, a low half with bit 31 set sign-extends over the high half and the requests
+    built on that base fault.  The flash kernel's code object must not hold the 32 -> 64 bit sign extension."""
+    import subprocess
+    import tempfile
+
+    from deplodock_amd.emit import prelude
+
+    assert prelude.DMA.count("(unsigned)__builtin_amdgcn_readfirstlane(") >= 3
+    k = kernels(compile_case(eager.sdpa_case()))[0]
+    assert "emh_uniform(" in k.kernel_source
+    blob = hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+    blob = blob if isinstance(blob, (bytes, bytearray)) else open(blob, "rb").read()
+    with tempfile.NamedTemporaryFile(suffix=".hsaco") as fh:
+        fh.write(blob)
+        fh.flush()
+        asm = subprocess.run(["/opt/rocm/llvm/bin/llvm-objdump", "-d", fh.name], capture_output=True, text=True, check=True).stdout
+    assert "global_load_lds_dwordx4" in asm and "s_bfe_i64" not in asm
+
+
 def test_flash_pin_grammar_and_degrade(launcher_lib, monkeypatch):
     case = eager.sdpa_case(1, 8, 4, 320, 128)
     default = kernels(compile_case(case))[0].knobs["FLASH"]
@@ -293,7 +314,11 @@ def test_flash_pin_grammar_and_degrade(launcher_lib, monkeypatch):
     monkeypatch.setenv("EMMY_FLASH", "w2/kv32/s4")
     k = kernels(compile_case(case))[0]
     assert k.knobs["FLASH"] == "w2/kv32/s4" and k.block[0] == (512,)
-    assert k.lds_bytes == 2 * 4 * 2 * 32 * 128 * 2 + 64 * 128 * 2  # double-buffered K/V blocks of four groups, then the Q tile
+    assert k.lds_bytes == 4 * 4 * 32 * 128 * 2 + 64 * 128 * 2  # four groups' blocks a slot, K and V rings of two slots, then the Q tile
+    monkeypatch.setenv("EMMY_FLASH", "w2/kv32/s4/k3")
+    k = kernels(compile_case(case))[0]
+    # a K ring of three slots beside the V ring of two fills the LDS (the Q fragments then come from global memory)
+    assert k.knobs["FLASH"] == "w2/kv32/s4/k3" and k.lds_bytes == 5 * 4 * 32 * 128 * 2 == 160 * 1024 and "#define DEEP 1" in k.kernel_source and "#define Q_LDS 0" in k.kernel_source
     monkeypatch.setenv("EMMY_FLASH", "w2/kv64/s4")  # 256 KiB of staging does not fit: degrade to the default pick
     assert kernels(compile_case(case))[0].knobs["FLASH"] == default
     monkeypatch.setenv("EMMY_FLASH", "w3/zz")
@@ -321,7 +346,7 @@ def test_cache_is_content_addressed(launcher_lib, tmp_path, monkeypatch):
 
 def test_a_symbolic_axis_lowers_to_kernels_that_take_it_as_a_runtime_int(launcher_lib):
     """``dynamic_shapes`` marks axes.  With one symbolic axis the module lowers once: every kernel whose work
-    follows the axis takes ``int seq_len`` as a trailing parameter, guards its rows / key blocks at run time and is
+    follows the axis takes the extent as a trailing ``int`` parameter (``emh_n_seq_len``: a name no local of a kernel has), guards its rows / key blocks at run time and is
     launched on a grid the runtime sizes per launch (the reference's form: ir/kernel/ir.py:258-276,
     ir/cuda/ir.py:66-112).  One code object per kernel then serves every length."""
     from deplodock_amd.ir.sym import Affine, CeilDiv, XcdRounds
@@ -335,13 +360,13 @@ def test_a_symbolic_axis_lowers_to_kernels_that_take_it_as_a_runtime_int(launche
     ks = kernels(compiled)
     assert len(ks) == 5
     for k in ks:
-        assert k.runtime_args == ("seq_len",) and k.kernel_source.count("int seq_len") == 1
+        assert k.runtime_args == ("seq_len",) and k.kernel_source.count("int emh_n_seq_len") == 1
         hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
     flash = next(k for k in ks if k.kernel_name.startswith("k_sdpa"))
     assert flash.grid[0] == (CeilDiv(Affine("seq_len", 1, 0), 32 * int(flash.knobs["FLASH"].split("/")[0][1:])), 16) and "/p" not in flash.knobs["FLASH"]
-    assert "#define SQ (seq_len)" in flash.kernel_source and "#define GRID ((int)gridDim.x)" in flash.kernel_source
+    assert "#define SQ (emh_n_seq_len)" in flash.kernel_source and "#define GRID ((int)gridDim.x)" in flash.kernel_source
     lin = next(k for k in ks if k.kernel_name.startswith("k_linear_add"))
-    assert isinstance(lin.grid[0][0], XcdRounds) and "#define M (seq_len)" in lin.kernel_source and "/ks" not in lin.knobs["STAGE"]
+    assert isinstance(lin.grid[0][0], XcdRounds) and "#define M (emh_n_seq_len)" in lin.kernel_source and "/ks" not in lin.knobs["STAGE"]
     assert lin.grid[0][0]({"seq_len": 200}) >= -(-200 // lin.grid[0][0].tile_m) * lin.grid[0][0].blocks_n * lin.grid[0][0].per_block
     assert compiled.nodes["x"].output.shape == (1, "seq_len", 1024) and compiled.nodes[compiled.outputs[0]].output.shape == (1, "seq_len", 1024)
 
