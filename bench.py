@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the emitted-kernel hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-table] [--no-cpu] [--only TEXT]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-table] [--no-cpu] [--only TEXT] [--live-traffic]
 
 A *step* is one pass of the headline kernel — the emitted ``nn.Softmax(-1)``
 row reduction over fp32 ``[1, 28, 2048, 2048]`` (the configuration the
@@ -12,7 +12,10 @@ JSON line printed carries:
                    (bracketed by device synchronisation on both sides);
 * ``roofline``     the dominant kernel against MI355X's 8 TB/s: algorithmic bytes
                    per launch / average launch duration from HIP events recorded
-                   on the launch stream around the same K launches;
+                   on the launch stream around the same K launches; ``traffic`` is the
+                   kernel's HBM bytes per launch from the hardware counters: the
+                   recorded figure for this exact kernel, or, with ``--live-traffic``,
+                   counted now by two ``rocprofv3 --pmc`` passes over this script;
 * ``cpu_baseline`` PyTorch eager of the same module on the host cores, over the
                    whole workload (20 passes of tens of milliseconds each), with the
                    host's core count, torch's thread count and the CPU model;
@@ -53,7 +56,62 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE (scaled by the same counters on a copy kernel of known size); keyed
 # by kernel name so a changed kernel reports null instead of a stale figure.
-MEASURED_TRAFFIC_BYTES: dict[str, int] = {"k_softmax_reduce_09dde4": 939580006}
+MEASURED_TRAFFIC_BYTES: dict[str, int] = {"k_softmax_reduce_0aa293": 939555721}
+COPY_PROBE_BYTES = 28 * 2048 * 2048 * 4  # read once and written once by the calibration copy
+
+
+def _counter_values(out_dir: Path, counter: str) -> dict[str, list[float]]:
+    """Per kernel name, the counter's value for every dispatch in rocprofv3's counter-collection CSVs under ``out_dir``."""
+    import csv
+
+    sums: dict[str, list[float]] = {}
+    for path in out_dir.rglob("*counter_collection.csv"):
+        with open(path, newline="") as fh:
+            for rec in csv.DictReader(fh):
+                if rec["Counter_Name"] == counter:
+                    sums.setdefault(rec["Kernel_Name"], []).append(float(rec["Counter_Value"]))
+    return sums
+
+
+def _calibrate(sums: dict[str, list[float]], kernel: str, counter: str) -> tuple[float, float]:
+    """``(bytes one count is worth, counts per launch of kernel)``.  Medians: the runtime's copy kernel also serves a
+    few small copies of torch's own, which a mean would fold into the calibration."""
+    copies, launches = sums.get("__amd_rocclr_copyBuffer"), sums.get(kernel)
+    if not copies or not launches:
+        raise RuntimeError(f"{counter} pass counted no {'copy' if not copies else kernel} dispatches")
+    return COPY_PROBE_BYTES / statistics.median(copies), statistics.median(launches)
+
+
+def _live_traffic(limit_s: int = 240) -> dict:
+    """HBM bytes per launch of the headline kernel, counted now.
+
+    Runs this script twice as a child under ``rocprofv3 --pmc`` (``FETCH_SIZE``, then ``WRITE_SIZE``, one
+    counter a pass, no trace domain beside it), each with ``--copy-probe`` so the same pass also counts a
+    plain device copy of known size; the copy fixes what one count of each counter is worth in bytes.
+    Called before this process touches the GPU.  Raises ``RuntimeError`` with the child's output when a
+    pass fails: a figure that was asked for is never silently replaced."""
+    import shutil
+    import subprocess
+    import tempfile
+
+    prof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    per_count: dict[str, float] = {}
+    counted: dict[str, float] = {}
+    kernel = None
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        out = tempfile.mkdtemp(prefix=f"emh_{counter.lower()}_", dir="/tmp")
+        cmd = ["timeout", "-s", "KILL", str(limit_s), prof, "--pmc", counter, "-d", out, "-o", "out", "--output-format", "csv", "--",
+               sys.executable, str(ROOT / "bench.py"), "--steps", "10", "--warmup", "2", "--no-table", "--no-cpu", "--copy-probe"]  # fmt: skip
+        run = subprocess.run(cmd, cwd="/tmp", env={**os.environ, "TMPDIR": "/tmp"}, capture_output=True, text=True)
+        if run.returncode != 0:
+            raise RuntimeError(f"{counter} pass failed ({run.returncode}): {run.stderr[-800:]}")
+        line = next(ln for ln in reversed(run.stdout.splitlines()) if ln.startswith("{"))
+        kernel = json.loads(line)["config"]["kernel"]
+        sums = _counter_values(Path(out), counter)
+        shutil.rmtree(out, ignore_errors=True)
+        per_count[counter], counted[counter] = _calibrate(sums, kernel, counter)
+    total = sum(counted[c] * per_count[c] for c in counted)
+    return {"kernel": kernel, "bytes": int(round(total)), "counts": counted, "bytes_per_count": {c: round(v, 3) for c, v in per_count.items()}}
 
 
 def _headline(device, steps: int, warmup: int) -> dict:
@@ -279,6 +337,7 @@ def main() -> int:
     ap.add_argument("--only", default=None, metavar="TEXT", help="restrict the kernel table to configurations whose label contains TEXT (e.g. 'M=2048', 'C4')")
     ap.add_argument("--extended", action="store_true", help="add machine-filling variants to the kernel table (4096^3 linear, non-causal attention)")
     ap.add_argument("--copy-probe", action="store_true", help="also run a plain 469762048-byte device copy 5 times (counter calibration under rocprofv3 --pmc)")
+    ap.add_argument("--live-traffic", action="store_true", help="count the headline kernel's HBM bytes now: two rocprofv3 --pmc passes over this script (adds about a minute)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(
@@ -287,6 +346,7 @@ def main() -> int:
             file=sys.stderr,
         )
         return 2
+    live = _live_traffic() if args.live_traffic else None
     import torch
 
     if not torch.cuda.is_available():
@@ -326,6 +386,11 @@ def main() -> int:
             "kernel_us": round(head["kernel_ms"] * 1e3, 2),
         },
     }
+    if live is not None:
+        if live["kernel"] != head["kernel"]:
+            raise RuntimeError(f"counter passes measured {live['kernel']}, this run launches {head['kernel']}")
+        out["roofline"]["traffic"] = live["bytes"]
+        out["roofline"]["traffic_counters"] = {"counts_per_launch": live["counts"], "bytes_per_count": live["bytes_per_count"]}
     out["cpu_baseline"] = None if args.no_cpu else _cpu_baseline()
     if not args.no_table:
         out["kernels"] = _table(device, args.only, args.extended, cpu=not args.no_cpu)

@@ -189,6 +189,7 @@ def l1fill_bytes_per_second(*, waves: int, inflight: int, stride: int, to_lds: b
     wg_bytes = 256 * 1024 if resident else 4 * 1024 * 1024 * max(1, stride // 2048)  # streamed: 4 MiB actually read per workgroup
     if stride:  # whole laps of (32 row blocks x 8 rows), of which 16 pieces of 128 bytes per row are read
         laps = max(1, wg_bytes // (256 * stride))
+        laps = 1 << (laps.bit_length() - 1)  # the kernel wraps a workgroup's unit index with a mask
         wg_bytes, wg_units = laps * 256 * stride, laps * 512
     else:
         wg_units = wg_bytes // 1024

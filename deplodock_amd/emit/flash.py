@@ -272,6 +272,27 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+      // The V operand fragments of the output MFMAs are requested here, behind the score MFMAs (where a lane
+      // has the registers for them): they land while the matrix pipe works through the scores and the softmax
+      // runs, instead of in front of each output MFMA.
+      u32x4 vfr[V_PRE ? (BKV / 32) * 2 * (D / 32) : 1];
+      if (V_PRE) {
+        #pragma unroll
+        for (int u = 0; u < BKV / 32; ++u)
+        #pragma unroll
+        for (int s = 0; s < 2; ++s)
+        #pragma unroll
+        for (int dt = 0; dt < D / 32; ++dt) {
+          const unsigned char* vp = sV + (32 * u + 16 * s) * (D * 2) + (dt / TG) * 256 + v_tile[dt % TG];
+          const emh_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) emh_s16x4*)(vp));
+          const emh_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) emh_s16x4*)(vp + 8 * (D * 2)));
+          const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+          u32x4 av;
+          av[0] = l2[0]; av[1] = l2[1]; av[2] = h2[0]; av[3] = h2[1];
+          vfr[(u * 2 + s) * (D / 32) + dt] = av;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #if HAS_MASK
       {
         // The additive mask: this lane's query row, the keys of its accumulator rows (runs of four consecutive
@@ -340,12 +361,16 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         for (int t = 0; t < 8; ++t) pf[t] = (ELT)sacc[u][8 * s + t];
         #pragma unroll
         for (int dt = 0; dt < D / 32; ++dt) {
-          const unsigned char* vp = sV + (32 * u + 16 * s) * (D * 2) + (dt / TG) * 256 + v_tile[dt % TG];
-          const emh_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) emh_s16x4*)(vp));
-          const emh_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) emh_s16x4*)(vp + 8 * (D * 2)));
-          const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
           u32x4 av;
-          av[0] = l2[0]; av[1] = l2[1]; av[2] = h2[0]; av[3] = h2[1];
+          if (V_PRE) {
+            av = vfr[(u * 2 + s) * (D / 32) + dt];
+          } else {
+            const unsigned char* vp = sV + (32 * u + 16 * s) * (D * 2) + (dt / TG) * 256 + v_tile[dt % TG];
+            const emh_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) emh_s16x4*)(vp));
+            const emh_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) emh_s16x4*)(vp + 8 * (D * 2)));
+            const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+            av[0] = l2[0]; av[1] = l2[1]; av[2] = h2[0]; av[3] = h2[1];
+          }
           oacc[dt] = MFMA(__builtin_bit_cast(FRAG, av), pf, oacc[dt], 0, 0, 0);
           if (DEEP && st + 2 < nsteps) {
             #pragma unroll
@@ -465,6 +490,9 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
 """
 
 
+_V_PRE = True
+
+
 def lds_plan(waves: int, kvs: int, bkv: int, head_dim: int, limit: int, deep: bool = False) -> dict:
     """LDS layout of a workgroup: ``[K ring | V ring | Q tile]``.
 
@@ -574,6 +602,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
             "M_SB": body.mask_strides[0], "M_SH": body.mask_strides[1], "M_SS": body.mask_strides[2], "M_OFF": body.mask_offset,
             "INV_SCALE": float_literal(1.0 / body.scale)} if has_mask else {}),
         "PAIR": 1 if pair else 0,
+        "V_PRE": 1 if _V_PRE and (BKV // 32) * 2 * (D // 32) * 4 <= 32 else 0,  # the prefetched V fragments take at most 32 registers
         "RK": plan["rk"], "RV": plan["rv"], "DEEP": 1 if plan["deep"] else 0,
         "Q_LDS": 1 if plan["q_off"] is not None else 0,
         "Q_OFF_LDS": plan["q_off"] or 0,
