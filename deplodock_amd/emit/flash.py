@@ -68,6 +68,7 @@ typedef short emh_s16x4 __attribute__((ext_vector_type(4)));
 #define WQ (NT / 64 / KVS)           /* waves (32-row groups) per key-split group */
 #define SETB (KVS * KBYTES)          /* one ring slot: the K (or V) blocks of a step, one per key-split group */
 #define V_RING (RK * SETB)           /* LDS: [K ring: RK slots][V ring: RV slots] */
+#define EMH_SLOT(st, R) ((R) == 2 ? ((st) & 1) : ((st) % (R)))  /* two slots: the step's parity, known when the loop runs in pairs */
 #define QCHUNKS (BQ * CPR)             /* 16-byte chunks of a workgroup's Q (and O) tile */
 #define RPL (D / 32 * 16)              /* output registers per lane */
 #define RPG (RPL / KVS)                /* ... of which each key-split group finishes this many */
@@ -160,8 +161,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   #define EMH_STEP_BASES(tag, st) \
       const unsigned char* kb##tag = emh_uniform((const unsigned char*)kbase + (long)(st) * (KVS * BKV) * K_SS * 2); \
       const unsigned char* vb##tag = emh_uniform((const unsigned char*)vbase + (long)(st) * (KVS * BKV) * V_SS * 2); \
-      const unsigned kl##tag = emh_uniform(lds0 + ((st) % RK) * SETB + wave_u * 1024); \
-      const unsigned vl##tag = emh_uniform(lds0 + V_RING + ((st) % RV) * SETB + wave_u * 1024);
+      const unsigned kl##tag = emh_uniform(lds0 + EMH_SLOT(st, RK) * SETB + wave_u * 1024); \
+      const unsigned vl##tag = emh_uniform(lds0 + V_RING + EMH_SLOT(st, RV) * SETB + wave_u * 1024);
   #define EMH_STAGE_ONE(st, i, sb_, lb_, base_, stride_, off_, swz_, ldo_) { \
       const int g_ = ((i) * NT) / CHUNKS, ro_ = (((i) * NT) % CHUNKS) / CPR; \
       if (SKV % (KVS * BKV) == 0 || ((st) * KVS + g_ + 1) * BKV <= SKV) { \
@@ -170,8 +171,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         long krow_ = (long)((st) * KVS + g_) * BKV + ro_ + st_row; \
         if (krow_ > SKV - 1) krow_ = SKV - 1; \
         emh_dma16((base_) + krow_ * (stride_) + swz_(st_row + ro_, st_pos) * 8, lds + (ldo_) + g_ * KBYTES + (((i) * NT) % CHUNKS) * 16 + dst_lane); } }
-  #define EMH_STAGE_K(tag, st, i) EMH_STAGE_ONE(st, i, kb##tag, kl##tag, kbase, K_SS, kvo, emh_kswz, ((st) % RK) * SETB)
-  #define EMH_STAGE_V(tag, st, i) EMH_STAGE_ONE(st, i, vb##tag, vl##tag, vbase, V_SS, vvo, emh_vswz, V_RING + ((st) % RV) * SETB)
+  #define EMH_STAGE_K(tag, st, i) EMH_STAGE_ONE(st, i, kb##tag, kl##tag, kbase, K_SS, kvo, emh_kswz, EMH_SLOT(st, RK) * SETB)
+  #define EMH_STAGE_V(tag, st, i) EMH_STAGE_ONE(st, i, vb##tag, vl##tag, vbase, V_SS, vvo, emh_vswz, V_RING + EMH_SLOT(st, RV) * SETB)
   // Requests are issued between MFMAs, spread evenly over a chain of NQ_SLOTS of them (request i behind MFMA
   // number EMH_SLOT_OF(i)): they trickle into the memory pipeline instead of arriving as one burst from every wave.
   #define NQ_SLOTS ((BKV / 32) * (D / 16))
@@ -234,7 +235,19 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
     for (int kk = 0; kk < D / 16; ++kk) qf[kk] = *(const FRAG*)(lds + Q_OFF_LDS + qr_ * (D * 2) + emh_kswz(qr_, kk * 2 + lh) * 16);
   }
 
+  // Steps run in pairs so that a step's ring slots (its parity) are known when the code is generated: the LDS
+  // addresses of the fragment reads are then a loop-invariant lane offset plus an immediate, with no vector
+  // arithmetic per step.
+#if PAIRSTEP
+  #pragma unroll 1
+  for (int st2 = 0; 2 * st2 < nsteps; ++st2)
+  #pragma unroll
+  for (int par = 0; par < 2; ++par) {
+    const int st = 2 * st2 + par;
+    if (st >= nsteps) break;
+#else
   for (int st = 0; st < nsteps; ++st) {
+#endif
     // The next step's blocks are requested between this step's score MFMAs: the
     // matrix pipe works through the chain while the wave issues the loads.
     const bool more = st + 1 < nsteps;
@@ -248,8 +261,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       if (more) { EMH_STAGE_ALL_V(st + 1); if (!DEEP) EMH_STAGE_ALL_K(st + 1); }
       if (DEEP && st + 2 < nsteps) EMH_STAGE_ALL_K(st + 2);
     } else {
-      const unsigned char* sK = lds + (st % RK) * SETB + grp * KBYTES;
-      const unsigned char* sV = lds + V_RING + (st % RV) * SETB + grp * KBYTES;
+      const unsigned char* sK = lds + EMH_SLOT(st, RK) * SETB + grp * KBYTES;
+      const unsigned char* sV = lds + V_RING + EMH_SLOT(st, RV) * SETB + grp * KBYTES;
       f32x16 sacc[BKV / 32];
       #pragma unroll
       for (int u = 0; u < BKV / 32; ++u) {
@@ -491,6 +504,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
 
 
 _V_PRE = True
+_PAIRSTEP = True
 
 
 def lds_plan(waves: int, kvs: int, bkv: int, head_dim: int, limit: int, deep: bool = False) -> dict:
@@ -602,6 +616,8 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
             "M_SB": body.mask_strides[0], "M_SH": body.mask_strides[1], "M_SS": body.mask_strides[2], "M_OFF": body.mask_offset,
             "INV_SCALE": float_literal(1.0 / body.scale)} if has_mask else {}),
         "PAIR": 1 if pair else 0,
+        # steps in parity pairs (static ring slots) unless the whole key range is one or two steps
+        "PAIRSTEP": 1 if _PAIRSTEP and (bool(symf) or -(-body.kv_len // (kvs * BKV)) > 2) else 0,
         "V_PRE": 1 if _V_PRE and (BKV // 32) * 2 * (D // 32) * 4 <= 32 else 0,  # the prefetched V fragments take at most 32 registers
         "RK": plan["rk"], "RV": plan["rv"], "DEEP": 1 if plan["deep"] else 0,
         "Q_LDS": 1 if plan["q_off"] is not None else 0,
