@@ -29,7 +29,7 @@ def register_run_command(subparsers) -> None:
     p.add_argument("--bench", "-b", action="store_true", help="Time eager PyTorch and the emitted kernels and print a comparison table.")
     p.add_argument("--warmup", type=int, default=10, help="Warmup iterations for --bench (default: 10).")
     p.add_argument("--iters", type=int, default=100, help="Measurement iterations for --bench (default: 100).")
-    p.add_argument("--ir", default=None, metavar="PATH", help="Replay a JSON graph written by `compile --json` (traced or lowered stage) on seeded random data; no eager check (there is no module to compare with).")
+    p.add_argument("--ir", default=None, metavar="PATH", help="Replay a JSON graph on seeded random data: one written by `compile --json` (traced or lowered stage), or one in the reference's own form (a traced block, or a Loop-IR kernel of its kernels/*.json corpus); no eager check (there is no module to compare with).")
     p.add_argument("--at", action="append", default=None, metavar="NAME=SIZE", help="With --dynamic: also run and check the expression with symbolic axis NAME at SIZE (repeatable).")
     p.add_argument("--ab", action="append", default=None, metavar="KNOBS", help="Also compile + bench a variant with these knobs pinned ('K1=V1,K2=V2'); repeatable; needs --bench.")
     p.set_defaults(func=handle_run)
@@ -179,7 +179,20 @@ def _run_ir(args, device) -> None:
     from deplodock_amd.backend.hip.backend import HipBackend
     from deplodock_amd.ir.hip import HipOp
 
-    graph = serialize.load(args.ir)
+    import json
+
+    doc = json.loads(Path(args.ir).read_text())
+    if isinstance(doc, dict) and isinstance(doc.get("nodes"), dict):
+        # the reference's own ``Graph.to_dict`` form (a traced block, or a Loop-IR kernel of its corpus)
+        from deplodock_amd.ingest import IngestError, graph_from_reference_dict
+
+        try:
+            graph = graph_from_reference_dict(doc)
+        except IngestError as exc:
+            print(f"error: {args.ir}: {exc}", file=sys.stderr)
+            sys.exit(2)
+    else:
+        graph = serialize.graph_from_dict(doc)
     be = HipBackend(dump=Path(args.dump_dir) if args.dump_dir else None, device_id=0, tune_db=getattr(args, "tune_db", None))
     compiled = graph if any(isinstance(n.op, HipOp) for n in graph.nodes.values()) else be.compile(graph)
     sizes = {}

@@ -8,8 +8,11 @@ The reference serialises every IR stage as ``{"inputs": [...], "outputs": [...],
 ``LinearOp``, ``SdpaOp``, ``MeanOp``, ``SumOp``, ``RmsNormOp``, ``SoftmaxOp`` and the layout ops
 ``ReshapeOp`` / ``TransposeOp`` / ``SliceOp`` / ``CatOp`` / ``UnsqueezeOp`` (emmy/compiler/ir/frontend/ir.py,
 emmy/compiler/ir/tensor/ir.py) — into this backend's traced-graph form, so a graph the reference wrote
-drives this backend.  Later stages (Loop IR, Tile IR, Kernel IR) hold the reference's own lowering and
-are refused.
+drives this backend.  Of the later stages the *Loop IR* is read too: a ``LoopOp`` node (a post-fusion, pre-tiling
+kernel, the form of the reference's on-disk kernel corpus ``kernels/*.json`` and
+``experiments/kernel_dataset/*/*.json``) keeps its statements (``ir/loopnest.py``: parsed, never evaluated) and
+lowers to a tiled kernel where it is a contraction or a row normalisation in disguise, else to the loop-nest
+emitter.  Tile IR and Kernel IR hold the reference's own lowering for another machine and are refused.
 
 Conventions of the format that are resolved here:
 
@@ -42,7 +45,7 @@ _ELEMENTWISE = {
     "add": "add", "subtract": "sub", "sub": "sub", "multiply": "mul", "mul": "mul", "divide": "div", "div": "div", "pow": "pow", "maximum": "maximum", "minimum": "minimum",
     "negative": "neg", "neg": "neg", "rsqrt": "rsqrt", "sqrt": "sqrt", "exp": "exp", "silu": "silu", "sigmoid": "sigmoid", "tanh": "tanh", "abs": "abs", "reciprocal": "reciprocal",
 }  # fmt: skip
-_LATER_STAGES = {"LoopOp", "TileOp", "KernelOp", "CudaOp", "ReduceOp", "IndexMapOp"}
+_LATER_STAGES = {"TileOp", "KernelOp", "CudaOp", "ReduceOp", "IndexMapOp"}
 _INT_MAX = 2**62
 
 
@@ -65,7 +68,7 @@ def graph_from_reference_dict(data: dict, cast: DType | None = None) -> Graph:
     scalars: dict[str, float] = {}
     for nid, nd in nodes.items():
         if nd["op"] in _LATER_STAGES:
-            raise IngestError(f"node {nid!r} is a {nd['op']}: only the frontend (traced) stage of the reference's JSON is read")
+            raise IngestError(f"node {nid!r} is a {nd['op']}: only the frontend (traced) and Loop-IR stages of the reference's JSON are read")
         if nd["op"] == "ConstantOp" and nd.get("op_fields", {}).get("value") is not None and list(nd["output"]["shape"]) in ([1], []):
             scalars[nid] = float(nd["op_fields"]["value"])
 
@@ -163,6 +166,14 @@ def graph_from_reference_dict(data: dict, cast: DType | None = None) -> Graph:
             src = shape_of(tensors[0])
             dim %= len(src)
             add(nid, F.SliceOp(dim=dim, start=start, end=start + shape_of(nid)[dim], step=1), tensors[:1])
+        elif kind == "LoopOp":
+            from deplodock_amd.ir import loopnest
+
+            try:
+                stmts = loopnest.parse_body(fields.get("body") or [])
+            except loopnest.LoopNestError as exc:
+                raise IngestError(f"node {nid!r}: {exc}") from exc
+            add(nid, F.LoopNestOp(stmts=stmts, loads=tuple(tensors), scalars={i: scalars[i] for i in ins if i in scalars}, out_name=nid), tensors)
         elif kind == "CatOp":
             dim = int(consts[-1]) if consts else int(fields.get("dim", -1))
             add(nid, F.CatOp(dim=dim % len(shape_of(tensors[0]))), tensors)

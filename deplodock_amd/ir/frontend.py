@@ -84,6 +84,18 @@ class SdpaOp(Op):
 
 
 @dataclass
+class LoopNestOp(Op):
+    """A kernel of the reference's Loop IR (a ``LoopOp``: post-fusion, pre-tiling; emmy/compiler/ir/loop/ir.py:89)
+    kept as its statements (``ir/loopnest.py``).  ``loads`` names, per graph input of the node, the name the body's
+    ``Load`` statements use for it; ``scalars`` are shape-[1] constants with a recorded value, folded into the body."""
+
+    stmts: tuple = ()
+    loads: tuple = ()
+    scalars: dict = None
+    out_name: str = ""
+
+
+@dataclass
 class ViewOp(Op):
     """``view`` / ``reshape`` / ``flatten`` to ``shape`` (row-major reinterpretation)."""
 

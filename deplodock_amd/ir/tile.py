@@ -325,6 +325,47 @@ class Map:
 
 
 @dataclass
+class LoopNest:
+    """A Loop-IR body rendered as it stands (``emit/loopnest.py``): the statements of a reference ``LoopOp``
+    (``ir/loopnest.py``), the tensors its ``Load`` statements name, and scalar constants folded into the text."""
+
+    stmts: tuple
+    operands: dict  # Load.input name -> (buffer id, shape, dtype)
+    scalars: dict  # Load.input name -> python float (a shape-[1] constant with a recorded value)
+    out: str  # buffer id of the result
+    out_name: str  # the name ``Write`` statements use for it
+    out_shape: tuple[int, ...]
+    out_dtype: DType
+
+    def _weights(self) -> tuple[int, int]:
+        """``(arithmetic statements executed, elements loaded)`` over the whole iteration space."""
+        from deplodock_amd.ir import loopnest as L
+
+        def run(body, times):
+            ops = loads = 0
+            for s in body:
+                if isinstance(s, L.Loop):
+                    o, l_ = run(s.body, times * s.extent)
+                    ops, loads = ops + o, loads + l_
+                elif isinstance(s, (L.Assign, L.Accum)):
+                    ops += times
+                elif isinstance(s, L.Load):
+                    loads += times
+            return ops, loads
+
+        return run(self.stmts, 1)
+
+    def algo_flops(self) -> int:
+        return self._weights()[0]
+
+    def algo_bytes(self) -> int:
+        import math
+
+        seen = {buf: math.prod(shape) * dt.nbytes for buf, shape, dt in self.operands.values()}
+        return int(sum(seen.values()) + math.prod(self.out_shape) * self.out_dtype.nbytes)
+
+
+@dataclass
 class TileOp(Op):
     """One kernel: a name plus a scheduled body."""
 

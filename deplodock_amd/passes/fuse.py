@@ -134,10 +134,35 @@ def _materialize(c: _Ctx, nid: str) -> None:
             c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
         c.done[nid] = nid
         return
-    for rec in (_rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_pointwise):
+    for rec in (_rec_loop_nest, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_pointwise):
         if rec(c, nid):
             return
     raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
+
+
+def _rec_loop_nest(c: _Ctx, nid: str) -> bool:
+    """A Loop-IR kernel of the reference: its operands are materialised as plain row-major tensors of their
+    recorded shapes and the statements go to the loop-nest emitter as they stand."""
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.LoopNestOp):
+        return False
+    from deplodock_amd.ir.tile import LoopNest
+
+    operands: dict = {}
+    inputs: list[str] = []
+    for load_name, src in zip(node.op.loads, node.inputs):
+        shape = tuple(int(d) for d in c.g.nodes[src].output.shape)
+        v = _need_logical(c, src)
+        if not ((v.offset == 0 and v.shape == shape and v.is_contiguous()) or _same_memory(v, shape)):
+            raise FusionError(f"loop nest {nid!r}: operand {src!r} is a strided view; a copy kernel is not implemented")
+        operands[load_name] = (v.base, shape, c.g.nodes[src].output.dtype)
+        inputs.append(v.base)
+    t = node.output
+    body = LoopNest(stmts=node.op.stmts, operands=operands, scalars=dict(node.op.scalars or {}), out=nid, out_name=node.op.out_name or nid,
+                    out_shape=tuple(int(d) for d in t.shape), out_dtype=t.dtype)  # fmt: skip
+    label = nid if nid.startswith("k_") else "k_" + "".join(ch if ch.isalnum() else "_" for ch in nid)[-40:]
+    _emit(c, nid, body, label.removeprefix("k_"), inputs)
+    return True
 
 
 def _emit(c: _Ctx, nid: str, body, label: str, inputs: list[str], shape=None, dtype=None) -> None:
