@@ -1006,6 +1006,9 @@ def _rec_pointwise(c: _Ctx, nid: str) -> bool:
 
 def fuse(g: Graph) -> Graph:
     """Lower a frontend ``Graph`` to ``Graph[TileOp + InputOp + ConstantOp]``."""
+    from deplodock_amd.passes.raise_loops import raise_loop_nests
+
+    g = raise_loop_nests(g)  # Loop-IR kernels that are a contraction / a row normalisation become frontend ops first
     out = Graph()
     out.constant_values = dict(getattr(g, "constant_values", {}))
     c = _Ctx(g=g, out=out)

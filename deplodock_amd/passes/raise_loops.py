@@ -1,0 +1,297 @@
+"""Loop-IR kernels that are a tiled kernel in disguise are raised back to frontend ops.
+
+A kernel of the reference's corpus is a fused loop nest (post-fusion, pre-tiling: the stage its own tile planner
+starts from, emmy/compiler/pipeline/passes/lowering/tile/).  Two shapes of nest have a tiled kernel here, and
+rendering them loop for loop would leave the matrix cores idle:
+
+* **a contraction with an element-wise output stage** — ``for m: for n: {pre; for k: acc += a[m,k] * b[n,k]; post;
+  write}`` — becomes ``LinearOp`` (``x @ W.T``, emmy/compiler/ir/frontend/ir.py:212-217; the reference decomposes
+  it into exactly this multiply + sum nest, decomposition/_helpers.py:87-110) followed by the ``ElementwiseOp``
+  nodes of its ``pre`` / ``post`` statements; the fusion pass then folds a residual add into the contraction's
+  output stage as it does for a traced module;
+* **a row RMS normalisation** — ``for r: {for c: acc += x*x; s = rsqrt(acc / count + eps); for c: write x*s*w}`` —
+  becomes ``RmsNormOp`` (frontend/ir.py:309-312; decomposition/080_rms_norm.py:25-57 + 090_mean.py:27-44).
+
+Anything else — attention scores with a rotary embedding folded into the operand reads, a softmax-weighted sum,
+operands read through a permuted index — stays a ``LoopNestOp`` and goes to the loop-nest emitter.  ``EMMY_NEST=loops``
+keeps every nest there (A/B, and the emitter's own tests).
+"""
+
+from __future__ import annotations
+
+from deplodock_amd import config
+from deplodock_amd.graph import Graph, Node, Tensor
+from deplodock_amd.ir import frontend as F
+from deplodock_amd.ir import loopnest as L
+
+_UNARY = {"negative": "neg", "reciprocal": "reciprocal", "rsqrt": "rsqrt", "sqrt": "sqrt", "exp": "exp", "tanh": "tanh", "sigmoid": "sigmoid", "silu": "silu", "abs": "abs"}
+_BINARY = {"add": "add", "subtract": "sub", "multiply": "mul", "divide": "div", "maximum": "maximum", "minimum": "minimum"}
+
+
+class _NoMatch(Exception):
+    pass
+
+
+def _simple_index(index: tuple, shape: tuple[int, ...], extents: dict[str, int]) -> list[str]:
+    """The loop axes a ``Load`` / ``Write`` index walks, in order, when every entry is a bare axis over its whole
+    dimension or a literal 0 on a dimension of extent 1."""
+    if len(index) != len(shape):
+        raise _NoMatch
+    axes = []
+    for e, dim in zip(index, shape):
+        if isinstance(e, L.Lit) and e.value == 0 and dim == 1:
+            continue
+        if isinstance(e, L.Var) and extents.get(e.name) == dim and e.name not in axes:
+            axes.append(e.name)
+            continue
+        raise _NoMatch
+    return axes
+
+
+class _Builder:
+    """New frontend nodes standing in for one ``LoopNestOp`` node."""
+
+    def __init__(self, g: Graph, node: Node):
+        self.g, self.node, self.new = g, node, []
+        self.dtype = node.output.dtype
+        self.n = 0
+
+    def add(self, op, inputs: list[str], shape: tuple[int, ...], final: bool = False) -> str:
+        nid = self.node.id if final else f"{self.node.id}__r{self.n}"
+        self.n += 1
+        self.new.append(Node(nid, op, list(inputs), Tensor(nid, tuple(shape), self.dtype)))
+        return nid
+
+    def shape_of(self, nid: str) -> tuple[int, ...]:
+        for n in self.new:
+            if n.id == nid:
+                return tuple(n.output.shape)
+        return tuple(int(d) for d in self.g.nodes[nid].output.shape)
+
+    def view(self, nid: str, shape: tuple[int, ...], final: bool = False) -> str:
+        if self.shape_of(nid) == tuple(shape) and not final:
+            return nid
+        return self.add(F.ViewOp(shape=tuple(shape)), [nid], shape, final)
+
+    def finish(self, res: str, out_shape: tuple[int, ...]) -> None:
+        """Make the new node ``res`` the stand-in for the raised node: under its id, in its recorded shape."""
+        if self.shape_of(res) != tuple(out_shape):
+            self.view(res, out_shape, final=True)
+            return
+        for n in self.new:
+            n.inputs = [self.node.id if i == res else i for i in n.inputs]
+            if n.id == res:
+                n.id = n.output.name = self.node.id
+        self.new.sort(key=lambda n: n.id == self.node.id)  # the stand-in last (stable: producers keep their order)
+
+
+def _source(node: Node, load: L.Load) -> str:
+    """The graph tensor a ``Load`` reads."""
+    try:
+        return node.inputs[node.op.loads.index(load.input)]
+    except ValueError as exc:
+        raise _NoMatch from exc
+
+
+def _elementwise(b: _Builder, stmts: list, env: dict, mn: tuple[str, str], extents: dict[str, int], full: tuple[int, ...]) -> None:
+    """Bind the value of every statement of an output stage in ``env``: a tensor node (broadcastable against
+    ``full``, the contraction's result shape) or a python float."""
+    node = b.node
+    m_ax, n_ax = mn
+    for s in stmts:
+        if isinstance(s, L.Load):
+            if s.input in (node.op.scalars or {}):
+                env[s.name] = float(node.op.scalars[s.input])
+                continue
+            src = _source(node, s)
+            axes = _simple_index(s.index, b.shape_of(src), extents)
+            if axes == [m_ax, n_ax]:
+                env[s.name] = b.view(src, full)
+            elif axes == [n_ax]:
+                env[s.name] = b.view(src, (extents[n_ax],))
+            elif axes == [m_ax]:
+                env[s.name] = b.view(src, full[:-1] + (1,))
+            elif axes == [] and b.shape_of(src) and all(d == 1 for d in b.shape_of(src)):
+                env[s.name] = b.view(src, (1,))
+            else:
+                raise _NoMatch
+        elif isinstance(s, L.Assign):
+            args = [env[a] for a in s.args if a in env]
+            if len(args) != len(s.args):
+                raise _NoMatch
+            tensors = [a for a in args if isinstance(a, str)]
+            if not tensors:
+                raise _NoMatch  # constant folding of scalars is not worth a case
+            if s.op in _UNARY:
+                env[s.name] = b.add(F.ElementwiseOp(fn=_UNARY[s.op]), tensors, _bshape(b, tensors, full))
+            elif s.op in _BINARY:
+                if len(tensors) == 2:
+                    env[s.name] = b.add(F.ElementwiseOp(fn=_BINARY[s.op]), tensors, _bshape(b, tensors, full))
+                else:
+                    scalar = next(a for a in args if not isinstance(a, str))
+                    env[s.name] = b.add(F.ElementwiseOp(fn=_BINARY[s.op], scalar=scalar, scalar_first=not isinstance(args[0], str)), tensors, _bshape(b, tensors, full))
+            else:
+                raise _NoMatch
+        else:
+            raise _NoMatch
+
+
+def _bshape(b: _Builder, tensors: list[str], full: tuple[int, ...]) -> tuple[int, ...]:
+    """Broadcast shape of ``tensors`` (each ``full``, a trailing vector, a column or a single value)."""
+    import numpy as np
+
+    return tuple(int(d) for d in np.broadcast_shapes(*(b.shape_of(t) for t in tensors)))
+
+
+def _try_contraction(g: Graph, node: Node) -> list[Node] | None:
+    op: F.LoopNestOp = node.op
+    stmts = list(op.stmts)
+    head = [s for s in stmts if not isinstance(s, L.Loop)]
+    loops = [s for s in stmts if isinstance(s, L.Loop)]
+    try:
+        if len(loops) != 1 or stmts[-1] is not loops[0] or not all(isinstance(s, L.Load) for s in head):
+            raise _NoMatch
+        lm = loops[0]
+        if len(lm.body) != 1 or not isinstance(lm.body[0], L.Loop):
+            raise _NoMatch
+        ln = lm.body[0]
+        inner = [s for s in ln.body if isinstance(s, L.Loop)]
+        if len(inner) != 1 or not isinstance(ln.body[-1], L.Write):
+            raise _NoMatch
+        lk = inner[0]
+        at = ln.body.index(lk)
+        pre, post, write = list(ln.body[:at]), list(ln.body[at + 1 : -1]), ln.body[-1]
+        extents = {lm.axis: lm.extent, ln.axis: ln.extent, lk.axis: lk.extent}
+        if len(extents) != 3:
+            raise _NoMatch
+        # the fold: acc += a * b over k, nothing else in the loop
+        kb = list(lk.body)
+        if len(kb) != 4 or not (isinstance(kb[-1], L.Accum) and kb[-1].op == "add" and isinstance(kb[-2], L.Assign) and kb[-2].op == "multiply" and kb[-1].value == kb[-2].name):
+            raise _NoMatch
+        loads = {s.name: s for s in kb[:2] if isinstance(s, L.Load)}
+        if len(loads) != 2 or set(kb[-2].args) != set(loads):
+            raise _NoMatch
+        b = _Builder(g, node)
+        a_load = b_load = None
+        for ld in loads.values():
+            if ld.input in (op.scalars or {}):
+                raise _NoMatch
+            axes = _simple_index(ld.index, b.shape_of(_source(node, ld)), extents)
+            if axes == [lm.axis, lk.axis]:
+                a_load = ld
+            elif axes == [ln.axis, lk.axis]:
+                b_load = ld
+        if a_load is None or b_load is None:
+            raise _NoMatch
+        x, w = _source(node, a_load), _source(node, b_load)
+        if g.nodes[x].output.dtype != b.dtype or g.nodes[w].output.dtype != b.dtype:
+            raise _NoMatch
+        if b.shape_of(w) != (ln.extent, lk.extent):
+            w = b.view(w, (ln.extent, lk.extent))  # unit dimensions around [N, K]
+        full = tuple(b.shape_of(x)[:-1]) + (ln.extent,)  # x is [1.., M, K] (checked above): the product is [1.., M, N]
+        out_shape = tuple(int(d) for d in node.output.shape)
+        if _simple_index(write.index, out_shape, extents) != [lm.axis, ln.axis]:
+            raise _NoMatch
+        env: dict = {}
+        _elementwise(b, head, env, (lm.axis, ln.axis), extents, full)
+        _elementwise(b, pre, env, (lm.axis, ln.axis), extents, full)
+        env[kb[-1].name] = b.add(F.LinearOp(has_bias=False), [x, w], full)
+        _elementwise(b, post, env, (lm.axis, ln.axis), extents, full)
+        res = env.get(write.value)
+        if not isinstance(res, str) or b.shape_of(res) != full or not any(n.id == res for n in b.new):
+            raise _NoMatch
+        b.finish(res, out_shape)
+        return b.new
+    except (_NoMatch, KeyError):
+        return None
+
+
+def _try_rms_norm(g: Graph, node: Node) -> list[Node] | None:
+    op: F.LoopNestOp = node.op
+    scalars = op.scalars or {}
+    try:
+        stmts = list(op.stmts)
+        head = {s.name: scalars[s.input] for s in stmts[:-1] if isinstance(s, L.Load) and s.input in scalars}
+        if len(head) != len(stmts) - 1 or not isinstance(stmts[-1], L.Loop):
+            raise _NoMatch
+        lr = stmts[-1]
+        body = list(lr.body)
+        if len(body) != 5 or not (isinstance(body[0], L.Loop) and isinstance(body[4], L.Loop) and all(isinstance(s, L.Assign) for s in body[1:4])):
+            raise _NoMatch
+        l1, (mean, plus, rs), l2 = body[0], body[1:4], body[4]
+        if l1.extent != l2.extent:
+            raise _NoMatch
+        # sum of squares
+        b1 = list(l1.body)
+        if len(b1) != 4 or not (isinstance(b1[0], L.Load) and isinstance(b1[1], L.Load) and isinstance(b1[2], L.Assign) and isinstance(b1[3], L.Accum)):
+            raise _NoMatch
+        if b1[0].input != b1[1].input or b1[0].index != b1[1].index or b1[2].op != "multiply" or set(b1[2].args) != {b1[0].name, b1[1].name} or b1[3].op != "add" or b1[3].value != b1[2].name:
+            raise _NoMatch
+        b = _Builder(g, node)
+        x = _source(node, b1[0])
+        ext1 = {lr.axis: lr.extent, l1.axis: l1.extent}
+        if _simple_index(b1[0].index, b.shape_of(x), ext1) != [lr.axis, l1.axis]:
+            raise _NoMatch
+        # mean, + eps, rsqrt
+        if not (mean.op == "divide" and mean.args[0] == b1[3].name and head.get(mean.args[1]) == float(l1.extent)):
+            raise _NoMatch
+        eps_name = [a for a in plus.args if a != mean.name]
+        if not (plus.op == "add" and mean.name in plus.args and len(eps_name) == 1 and eps_name[0] in head and rs.op == "rsqrt" and rs.args == (plus.name,)):
+            raise _NoMatch
+        # x * s * w
+        b2 = list(l2.body)
+        if len(b2) != 5 or not isinstance(b2[-1], L.Write):
+            raise _NoMatch
+        lds = {s.name: s for s in b2 if isinstance(s, L.Load)}
+        muls = [s for s in b2 if isinstance(s, L.Assign)]
+        if len(lds) != 2 or len(muls) != 2 or any(m.op != "multiply" for m in muls):
+            raise _NoMatch
+        ext2 = {lr.axis: lr.extent, l2.axis: l2.extent}
+        first, second = muls
+        if set(first.args) - {rs.name} == set() or rs.name not in first.args:
+            raise _NoMatch
+        (xn_name,) = set(first.args) - {rs.name}
+        (w_name,) = set(second.args) - {first.name}
+        if first.name not in second.args or xn_name not in lds or w_name not in lds or b2[-1].value != second.name:
+            raise _NoMatch
+        if _source(node, lds[xn_name]) != x or _simple_index(lds[xn_name].index, b.shape_of(x), ext2) != [lr.axis, l2.axis]:
+            raise _NoMatch
+        w = _source(node, lds[w_name])
+        if _simple_index(lds[w_name].index, b.shape_of(w), ext2) != [l2.axis] or b.shape_of(w) != (l2.extent,):
+            raise _NoMatch
+        out_shape = tuple(int(d) for d in node.output.shape)
+        if _simple_index(b2[-1].index, out_shape, ext2) != [lr.axis, l2.axis] or b.shape_of(x) != out_shape:
+            raise _NoMatch
+        if g.nodes[x].output.dtype != b.dtype or g.nodes[w].output.dtype != b.dtype:
+            raise _NoMatch
+        b.add(F.RmsNormOp(eps=float(head[eps_name[0]]), has_weight=True), [x, w], out_shape, final=True)
+        return b.new
+    except (_NoMatch, KeyError, ValueError):
+        return None
+
+
+def raise_loop_nests(g: Graph) -> Graph:
+    """``g`` with every ``LoopNestOp`` that has a tiled form replaced by frontend nodes (a new graph; ``g`` is left
+    as it was)."""
+    if not any(isinstance(n.op, F.LoopNestOp) for n in g.nodes.values()) or (config.knob_raw("NEST") or "").strip().lower() == "loops":
+        return g
+    out = Graph()
+    for attr, value in vars(g).items():
+        if attr != "nodes":
+            setattr(out, attr, value)
+    out.nodes = {}
+    for nid, node in g.nodes.items():
+        new = None
+        if isinstance(node.op, F.LoopNestOp):
+            new = _try_contraction(g, node) or _try_rms_norm(g, node)
+        if new is None:
+            out.nodes[nid] = node
+        else:
+            for n in new:
+                if n.id in out.nodes or (n.id in g.nodes and n.id != nid):
+                    raise ValueError(f"raised node id {n.id!r} is taken")
+                out.nodes[n.id] = n
+    return out
+
+
+__all__ = ["raise_loop_nests"]

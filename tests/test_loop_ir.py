@@ -201,17 +201,46 @@ def _kernels(compiled):
     return [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
 
 
-def test_every_reproducer_lowers_to_one_kernel_that_builds_for_gfx950(launcher_lib):
+RAISED = {  # what each reproducer becomes when nests with a tiled form are raised (kernel labels, in launch order)
+    "k_add_3_reduce": ["k_merged_merged_lift_add_3"],  # the attention output is read through a permuted index: stays a nest
+    "k_add_5_reduce": ["k_linear_add"],
+    "k_linear_1_reduce_reduce": ["k_linear"],
+    "k_linear_2_reduce_reduce": ["k_linear"],
+    "k_linear_4_reduce": ["k_linear"],
+    "k_linear_reduce_reduce": ["k_linear"],
+    "k_mul_1_reduce": ["k_rms_norm_reduce"],
+    "k_mul_7_reduce": ["k_rms_norm_reduce"],
+    "k_mul_8_reduce": ["k_linear", "k_pointwise_fused6"],
+    "k_scaled_dot_product_attention_masked_reduce": ["k_lift_scaled_dot_product_attention_masked"],  # rotary embedding in the operand reads
+    "k_scaled_dot_product_attention_reduce_reduce": ["k_lift_scaled_dot_product_attention_reduce"],  # softmax-weighted sum
+}
+
+
+@pytest.mark.parametrize("mode", ["raised", "loops"])
+def test_every_reproducer_lowers_to_kernels_that_build_for_gfx950(launcher_lib, monkeypatch, mode):
+    """By default a nest that is a contraction (+ element-wise output stage) or a row RMS normalisation is raised
+    to the tiled kernels (fp32 MFMA contraction, register-resident row kernel); ``EMMY_NEST=loops`` renders every
+    nest loop for loop."""
+    import re
+
     from deplodock_amd import HipBackend
     from deplodock_amd.backend.hip import hiprtc
     from deplodock_amd.ingest import load_reference_graph
 
+    if mode == "loops":
+        monkeypatch.setenv("EMMY_NEST", "loops")
     be = HipBackend()
     for path in sorted(CORPUS.glob("*.json")):
         ks = _kernels(be.compile(load_reference_graph(path)))
-        assert len(ks) == 1, path.name
-        hiprtc.compile_to_hsaco(ks[0].kernel_source, ks[0].kernel_name)
-        assert hiprtc.spilled_vgprs(ks[0].kernel_source, ks[0].kernel_name) == 0
+        labels = [re.sub(r"_[0-9a-f]{6}$", "", k.kernel_name) for k in ks]
+        if mode == "loops":
+            assert len(ks) == 1 and "NEST" in ks[0].knobs, (path.name, labels)
+        else:
+            assert labels == RAISED[path.stem], (path.name, labels)
+            assert [("NEST" in k.knobs) for k in ks] == [not lab.startswith(("k_linear", "k_rms_norm", "k_pointwise")) for lab in labels]
+        for k in ks:
+            hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+            assert hiprtc.spilled_vgprs(k.kernel_source, k.kernel_name) == 0
 
 
 def test_a_body_that_would_leave_its_operand_is_refused_on_the_host():
@@ -239,11 +268,18 @@ def _random_operands(doc: dict, seed: int) -> dict[str, np.ndarray]:
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["raised", "loops"])
 @pytest.mark.parametrize("kernel", sorted(p.stem for p in CORPUS.glob("*.json")))
-def test_reproducer_on_the_gpu_equals_the_interpreter(device, kernel):
-    """One kernel of the corpus, read from the reference's JSON, lowered and run through the launcher library,
-    against the float64 interpretation of the same statements on the same fp32 operands."""
+def test_reproducer_on_the_gpu_equals_the_interpreter(device, monkeypatch, kernel, mode):
+    """One kernel of the corpus, read from the reference's JSON, lowered (raised to the tiled kernels where it has
+    a tiled form, or loop for loop) and run through the launcher library, against the float64 interpretation of
+    the same statements on the same fp32 operands."""
     import torch
+
+    if mode == "loops":
+        if not RAISED[kernel][0].startswith(("k_linear", "k_rms_norm")):
+            pytest.skip("this reproducer is a loop nest in both modes")
+        monkeypatch.setenv("EMMY_NEST", "loops")
 
     from deplodock_amd import HipBackend
     from deplodock_amd.ingest import graph_from_reference_dict
@@ -273,10 +309,14 @@ def test_reproducer_on_the_gpu_equals_the_interpreter(device, kernel):
 
 
 @pytest.mark.gpu
-def test_the_corpus_chained_on_the_gpu_is_the_decoder_layer(device):
+@pytest.mark.parametrize("mode", ["raised", "loops"])
+def test_the_corpus_chained_on_the_gpu_is_the_decoder_layer(device, monkeypatch, mode):
     """The eleven kernels run in dependency order on the GPU, each feeding the next, reproduce the decoder layer
     they were cut from (PyTorch eager in float64 on the host)."""
     import torch
+
+    if mode == "loops":
+        monkeypatch.setenv("EMMY_NEST", "loops")
 
     from deplodock_amd import HipBackend
     from deplodock_amd.ingest import graph_from_reference_dict
