@@ -93,6 +93,7 @@ class LoopNestOp(Op):
     loads: tuple = ()
     scalars: dict = None
     out_name: str = ""
+    label: str = ""  # kernel label (default: from the node id)
 
 
 @dataclass

@@ -160,8 +160,8 @@ def _rec_loop_nest(c: _Ctx, nid: str) -> bool:
     t = node.output
     body = LoopNest(stmts=node.op.stmts, operands=operands, scalars=dict(node.op.scalars or {}), out=nid, out_name=node.op.out_name or nid,
                     out_shape=tuple(int(d) for d in t.shape), out_dtype=t.dtype)  # fmt: skip
-    label = nid if nid.startswith("k_") else "k_" + "".join(ch if ch.isalnum() else "_" for ch in nid)[-40:]
-    _emit(c, nid, body, label.removeprefix("k_"), inputs)
+    label = node.op.label or "".join(ch if ch.isalnum() else "_" for ch in nid)[-40:].lstrip("_")
+    _emit(c, nid, body, label, inputs)
     return True
 
 

@@ -12,8 +12,10 @@ rendering them loop for loop would leave the matrix cores idle:
 * **a row RMS normalisation** — ``for r: {for c: acc += x*x; s = rsqrt(acc / count + eps); for c: write x*s*w}`` —
   becomes ``RmsNormOp`` (frontend/ir.py:309-312; decomposition/080_rms_norm.py:25-57 + 090_mean.py:27-44).
 
-Anything else — attention scores with a rotary embedding folded into the operand reads, a softmax-weighted sum,
-operands read through a permuted index — stays a ``LoopNestOp`` and goes to the loop-nest emitter.  ``EMMY_NEST=loops``
+An operand of such a contraction that is read through a permuted or folded index (the o-projection reads the attention
+output ``[H, S, D]`` as ``[S, H*D]``) is first copied to a plain matrix by a small loop nest of its own.  Anything else
+— attention scores with a rotary embedding folded into the operand reads, a softmax-weighted sum — stays a
+``LoopNestOp`` and goes to the loop-nest emitter.  ``EMMY_NEST=loops``
 keeps every nest there (A/B, and the emitter's own tests).
 """
 
@@ -73,6 +75,14 @@ class _Builder:
             return nid
         return self.add(F.ViewOp(shape=tuple(shape)), [nid], shape, final)
 
+    def gather(self, load: L.Load, rows: L.Loop, cols: L.Loop) -> str:
+        """A plain row-major ``[rows, cols]`` copy of what ``load`` reads (its index any expression over the two
+        axes): a small loop nest of its own, so the contraction sees an ordinary matrix."""
+        nid = f"{self.node.id}__r{self.n}"
+        src = _source(self.node, load)
+        stmts = (L.Loop(rows.axis, rows.extent, (L.Loop(cols.axis, cols.extent, (L.Load("t", load.input, load.index), L.Write(nid, (L.Var(rows.axis), L.Var(cols.axis)), "t"))),)),)
+        return self.add(F.LoopNestOp(stmts=stmts, loads=(load.input,), scalars={}, out_name=nid, label="gather"), [src], (rows.extent, cols.extent))
+
     def finish(self, res: str, out_shape: tuple[int, ...]) -> None:
         """Make the new node ``res`` the stand-in for the raised node: under its id, in its recorded shape."""
         if self.shape_of(res) != tuple(out_shape):
@@ -93,7 +103,7 @@ def _source(node: Node, load: L.Load) -> str:
         raise _NoMatch from exc
 
 
-def _elementwise(b: _Builder, stmts: list, env: dict, mn: tuple[str, str], extents: dict[str, int], full: tuple[int, ...]) -> None:
+def _elementwise(b: _Builder, stmts: list, env: dict, mn: tuple[str, str], extents: dict[str, int], full: tuple[int, ...], loops=None) -> None:
     """Bind the value of every statement of an output stage in ``env``: a tensor node (broadcastable against
     ``full``, the contraction's result shape) or a python float."""
     node = b.node
@@ -104,7 +114,13 @@ def _elementwise(b: _Builder, stmts: list, env: dict, mn: tuple[str, str], exten
                 env[s.name] = float(node.op.scalars[s.input])
                 continue
             src = _source(node, s)
-            axes = _simple_index(s.index, b.shape_of(src), extents)
+            try:
+                axes = _simple_index(s.index, b.shape_of(src), extents)
+            except _NoMatch:
+                if set().union(*(L.expr_vars(e) for e in s.index)) != {m_ax, n_ax} or loops is None:
+                    raise
+                env[s.name] = b.view(b.gather(s, *loops), full)
+                continue
             if axes == [m_ax, n_ax]:
                 env[s.name] = b.view(src, full)
             elif axes == [n_ax]:
@@ -172,19 +188,29 @@ def _try_contraction(g: Graph, node: Node) -> list[Node] | None:
         if len(loads) != 2 or set(kb[-2].args) != set(loads):
             raise _NoMatch
         b = _Builder(g, node)
-        a_load = b_load = None
+        x = w = None
         for ld in loads.values():
             if ld.input in (op.scalars or {}):
                 raise _NoMatch
-            axes = _simple_index(ld.index, b.shape_of(_source(node, ld)), extents)
+            src = _source(node, ld)
+            if g.nodes[src].output.dtype != b.dtype:
+                raise _NoMatch
+            try:
+                axes = _simple_index(ld.index, b.shape_of(src), extents)
+            except _NoMatch:
+                axes = None
+            used = set().union(*(L.expr_vars(e) for e in ld.index))
             if axes == [lm.axis, lk.axis]:
-                a_load = ld
+                x = src
             elif axes == [ln.axis, lk.axis]:
-                b_load = ld
-        if a_load is None or b_load is None:
-            raise _NoMatch
-        x, w = _source(node, a_load), _source(node, b_load)
-        if g.nodes[x].output.dtype != b.dtype or g.nodes[w].output.dtype != b.dtype:
+                w = src
+            elif used == {lm.axis, lk.axis} and x is None:
+                x = b.gather(ld, lm, lk)  # read through a permuted / folded index: made a plain matrix first
+            elif used == {ln.axis, lk.axis} and w is None:
+                w = b.gather(ld, ln, lk)
+            else:
+                raise _NoMatch
+        if x is None or w is None:
             raise _NoMatch
         if b.shape_of(w) != (ln.extent, lk.extent):
             w = b.view(w, (ln.extent, lk.extent))  # unit dimensions around [N, K]
@@ -193,10 +219,10 @@ def _try_contraction(g: Graph, node: Node) -> list[Node] | None:
         if _simple_index(write.index, out_shape, extents) != [lm.axis, ln.axis]:
             raise _NoMatch
         env: dict = {}
-        _elementwise(b, head, env, (lm.axis, ln.axis), extents, full)
-        _elementwise(b, pre, env, (lm.axis, ln.axis), extents, full)
+        _elementwise(b, head, env, (lm.axis, ln.axis), extents, full, (lm, ln))
+        _elementwise(b, pre, env, (lm.axis, ln.axis), extents, full, (lm, ln))
         env[kb[-1].name] = b.add(F.LinearOp(has_bias=False), [x, w], full)
-        _elementwise(b, post, env, (lm.axis, ln.axis), extents, full)
+        _elementwise(b, post, env, (lm.axis, ln.axis), extents, full, (lm, ln))
         res = env.get(write.value)
         if not isinstance(res, str) or b.shape_of(res) != full or not any(n.id == res for n in b.new):
             raise _NoMatch

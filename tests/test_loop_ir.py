@@ -202,7 +202,7 @@ def _kernels(compiled):
 
 
 RAISED = {  # what each reproducer becomes when nests with a tiled form are raised (kernel labels, in launch order)
-    "k_add_3_reduce": ["k_merged_merged_lift_add_3"],  # the attention output is read through a permuted index: stays a nest
+    "k_add_3_reduce": ["k_gather", "k_linear_add"],  # the attention output is read through a permuted index: copied to a plain matrix first
     "k_add_5_reduce": ["k_linear_add"],
     "k_linear_1_reduce_reduce": ["k_linear"],
     "k_linear_2_reduce_reduce": ["k_linear"],
@@ -238,6 +238,7 @@ def test_every_reproducer_lowers_to_kernels_that_build_for_gfx950(launcher_lib, 
         else:
             assert labels == RAISED[path.stem], (path.name, labels)
             assert [("NEST" in k.knobs) for k in ks] == [not lab.startswith(("k_linear", "k_rms_norm", "k_pointwise")) for lab in labels]
+            assert sum("NEST" in k.knobs and lab != "k_gather" for k, lab in zip(ks, labels)) == (1 if "attention" in path.stem else 0)
         for k in ks:
             hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
             assert hiprtc.spilled_vgprs(k.kernel_source, k.kernel_name) == 0
@@ -277,7 +278,7 @@ def test_reproducer_on_the_gpu_equals_the_interpreter(device, monkeypatch, kerne
     import torch
 
     if mode == "loops":
-        if not RAISED[kernel][0].startswith(("k_linear", "k_rms_norm")):
+        if not RAISED[kernel][0].startswith(("k_linear", "k_rms_norm", "k_gather")):
             pytest.skip("this reproducer is a loop nest in both modes")
         monkeypatch.setenv("EMMY_NEST", "loops")
 
