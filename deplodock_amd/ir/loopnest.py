@@ -243,7 +243,10 @@ def parse_body(texts: list[str] | tuple[str, ...]) -> tuple:
             tree = ast.parse(text, mode="eval")
         except (SyntaxError, RecursionError, MemoryError) as exc:
             raise LoopNestError(f"LoopOp.body: not a statement expression ({type(exc).__name__})") from exc
-        out.append(_stmt(tree.body))
+        try:
+            out.append(_stmt(tree.body))
+        except RecursionError as exc:
+            raise LoopNestError("LoopOp.body: expression nested too deeply") from exc
     stmts = tuple(out)
     check_body(stmts)
     return stmts

@@ -341,3 +341,109 @@ def test_the_corpus_chained_on_the_gpu_is_the_decoder_layer(device, monkeypatch,
     want_t = torch.from_numpy(want).float()
     rms = float(want_t.pow(2).mean().sqrt())
     eager.assert_close(torch.from_numpy(got).float(), want_t, 1e-4, 2e-4 * rms, "corpus chain on the GPU vs the eager decoder layer")
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# hand-written nests: the branches of the raise (bias vector, row vector, scalar operands, a k-major weight) and
+# nests that must stay loop nests
+
+
+def _doc(body: list[str], tensors: dict[str, tuple], out: tuple[str, tuple], scalars: dict[str, float] | None = None) -> dict:
+    """A reference-format graph around one ``LoopOp``."""
+    name, shape = out
+    nodes = {}
+    for k, shp in tensors.items():
+        nodes[k] = {"op": "InputOp", "op_fields": {}, "inputs": [], "output": {"name": k, "shape": list(shp), "dtype": "float32"}}
+    for k, v in (scalars or {}).items():
+        nodes[k] = {"op": "ConstantOp", "op_fields": {"name": k, "value": v}, "inputs": [], "output": {"name": k, "shape": [1], "dtype": "float32"}}
+    nodes[name] = {"op": "LoopOp", "op_fields": {"body": body}, "inputs": [*tensors, *(scalars or {})], "output": {"name": name, "shape": list(shape), "dtype": "float32"}}
+    return {"inputs": list(tensors), "outputs": [name], "nodes": nodes}
+
+
+def _V(n):
+    return f"Var(name='{n}')"
+
+
+_ZERO = "Literal(value=0, dtype='int')"
+HAND = {
+    # y = max(x @ W.T + bias[n], 0.5) * rowscale[m] - 2.0 : bias vector, scalar operands on either side, row vector
+    "bias_clamp_rowscale": (
+        _doc(
+            ["Load(name='half', input='c_half', index=(" + _ZERO + ",))", "Load(name='two', input='c_two', index=(" + _ZERO + ",))",
+             f"Loop(axis=Axis(name='m', extent=70), body=(Loop(axis=Axis(name='n', extent=96), body=(Load(name='bb', input='bias', index=({_V('n')},)), "
+             f"Loop(axis=Axis(name='k', extent=200), body=(Load(name='a', input='X', index=({_ZERO}, {_V('m')}, {_V('k')})), Load(name='w', input='W', index=({_V('n')}, {_V('k')})), "
+             "Assign(name='p', op=ElementwiseImpl('multiply'), args=('w','a')), Accum(name='s', value='p'))), "
+             "Assign(name='t', op=ElementwiseImpl('add'), args=('s','bb')), Assign(name='u', op=ElementwiseImpl('maximum'), args=('half','t')), "
+             f"Load(name='r', input='rows', index=({_V('m')}, {_ZERO})), Assign(name='v', op=ElementwiseImpl('multiply'), args=('u','r')), "
+             f"Assign(name='y', op=ElementwiseImpl('subtract'), args=('v','two')), Write(output='Y', index=({_ZERO}, {_V('m')}, {_V('n')}), value='y'))),))"],
+            {"X": (1, 70, 200), "W": (96, 200), "bias": (96,), "rows": (70, 1)}, ("Y", (1, 70, 96)), {"c_half": 0.5, "c_two": 2.0}),
+        ["k_linear", "k_pointwise_fused4"],
+    ),
+    # the weight stored k-major ([K, N]): read through a transposing index, so it is copied to [N, K] first
+    "k_major_weight": (
+        _doc(
+            [f"Loop(axis=Axis(name='m', extent=64), body=(Loop(axis=Axis(name='n', extent=48), body=(Loop(axis=Axis(name='k', extent=128), body=("
+             f"Load(name='a', input='X', index=({_V('m')}, {_V('k')})), Load(name='w', input='Wt', index=({_V('k')}, {_V('n')})), "
+             "Assign(name='p', op=ElementwiseImpl('multiply'), args=('a','w')), Accum(name='s', value='p'))), "
+             f"Write(output='Y', index=({_V('m')}, {_V('n')}), value='s'))),))"],
+            {"X": (64, 128), "Wt": (128, 48)}, ("Y", (64, 48))),
+        ["k_gather", "k_linear"],
+    ),
+    # a normalisation without a weight and with a maximum instead of a sum: neither tiled form, stays a loop nest
+    "max_normalise": (
+        _doc(
+            [f"Loop(axis=Axis(name='r', extent=37), body=(Loop(axis=Axis(name='c', extent=300), body=(Load(name='x', input='X', index=({_V('r')}, {_V('c')})), "
+             "Assign(name='ab', op=ElementwiseImpl('abs'), args=('x',)), Accum(name='mx', value='ab', op=ElementwiseImpl('maximum')))), "
+             f"Loop(axis=Axis(name='c2', extent=300), body=(Load(name='x2', input='X', index=({_V('r')}, {_V('c2')})), Assign(name='y', op=ElementwiseImpl('divide'), args=('x2','mx')), "
+             f"Write(output='Y', index=({_V('r')}, {_V('c2')}), value='y')))))"],
+            {"X": (37, 300)}, ("Y", (37, 300))),
+        ["k_Y"],
+    ),
+}  # fmt: skip
+
+
+@pytest.mark.parametrize("case", sorted(HAND))
+def test_hand_written_nests_take_the_expected_route(launcher_lib, case):
+    import re
+
+    from deplodock_amd import HipBackend
+    from deplodock_amd.backend.hip import hiprtc
+    from deplodock_amd.ingest import graph_from_reference_dict
+
+    doc, labels = HAND[case]
+    ks = _kernels(HipBackend().compile(graph_from_reference_dict(doc)))
+    assert [re.sub(r"_[0-9a-f]{6}$", "", k.kernel_name) for k in ks] == labels
+    for k in ks:
+        hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["raised", "loops"])
+@pytest.mark.parametrize("case", sorted(HAND))
+def test_hand_written_nests_on_the_gpu_equal_the_interpreter(device, monkeypatch, case, mode):
+    import torch
+
+    from deplodock_amd import HipBackend
+    from deplodock_amd.ingest import graph_from_reference_dict
+    from oracle import eager
+
+    if mode == "loops":
+        monkeypatch.setenv("EMMY_NEST", "loops")
+    doc, _ = HAND[case]
+    nid, node = loop_node(doc)
+    rng = np.random.default_rng(5)
+    vals = {k: rng.standard_normal(tuple(nd["output"]["shape"])).astype(np.float32) for k, nd in doc["nodes"].items() if nd["op"] == "InputOp"}
+    operands = {**vals, **{k: np.full((1,), nd["op_fields"]["value"]) for k, nd in doc["nodes"].items() if nd["op"] == "ConstantOp"}}
+    stmts = L.parse_body(node["op_fields"]["body"])
+    want = loop_ir.run_vectorised(stmts, operands, tuple(node["output"]["shape"]))
+    be = HipBackend()
+    compiled = be.compile(graph_from_reference_dict(doc))
+    prog = be.program(compiled, {k: torch.from_numpy(v).to(device) for k, v in vals.items()})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want_t = torch.from_numpy(want).float()
+    eager.assert_close(ours.reshape(want_t.shape), want_t, 1e-4, 1e-4 * float(want_t.pow(2).mean().sqrt()), f"{case} ({mode}) vs the float64 interpretation")
