@@ -291,5 +291,5 @@ def emit_loop_nest(body: LoopNest, name: str, ctx: Context = Context()) -> HipOp
         comment=f"loop nest points={points} split={split}",
         algo_bytes=nbytes,
         algo_flops=body.algo_flops(),
-        knobs={"NEST": f"w{points}" + (f"/s{split}" if split > 1 else "")},
+        knobs={"NEST": f"loops/w{points}" + (f"/s{split}" if split > 1 else "")},  # the route, then how it was dealt (informational)
     )

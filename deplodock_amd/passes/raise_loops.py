@@ -228,7 +228,7 @@ def _try_contraction(g: Graph, node: Node) -> list[Node] | None:
             raise _NoMatch
         b.finish(res, out_shape)
         return b.new
-    except (_NoMatch, KeyError):
+    except (_NoMatch, KeyError, IndexError):
         return None
 
 
@@ -292,14 +292,14 @@ def _try_rms_norm(g: Graph, node: Node) -> list[Node] | None:
             raise _NoMatch
         b.add(F.RmsNormOp(eps=float(head[eps_name[0]]), has_weight=True), [x, w], out_shape, final=True)
         return b.new
-    except (_NoMatch, KeyError, ValueError):
+    except (_NoMatch, KeyError, ValueError, IndexError):
         return None
 
 
 def raise_loop_nests(g: Graph) -> Graph:
     """``g`` with every ``LoopNestOp`` that has a tiled form replaced by frontend nodes (a new graph; ``g`` is left
     as it was)."""
-    if not any(isinstance(n.op, F.LoopNestOp) for n in g.nodes.values()) or (config.knob_raw("NEST") or "").strip().lower() == "loops":
+    if not any(isinstance(n.op, F.LoopNestOp) for n in g.nodes.values()) or (config.knob_raw("NEST") or "").strip().lower().split("/")[0] == "loops":
         return g
     out = Graph()
     for attr, value in vars(g).items():
