@@ -258,6 +258,14 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     if body.reduce.cta != 1:
         raise LoweringError("contraction: a cross-workgroup split (REDUCE=g<n>) is lowered as a partial kernel plus a combine (deplodock_amd.emit.splitk.lower_split_contraction), not by this emitter alone")
     split = body.k_split
+    batch = int(getattr(body, "batch", 1) or 1)
+    if batch > 1:
+        if split is not None or body.bias is not None or body.a_prologue is not None or body.row_epilogue is not None or body.epilogue_operands or body.gate_pair:
+            raise LoweringError("contraction: a batch of products takes plain products only (no split, bias, prologue, row epilogue, epilogue operands or gate pair)")
+        if batch > 65535:
+            raise LoweringError(f"contraction: {batch} products exceed the launch's second dimension")
+        if (body.a_batch * ES) % 16 or (body.b_batch * ES) % 16 or (body.out_batch * body.out_dtype.nbytes) % 16:
+            raise LoweringError("contraction: batch strides must keep 16-byte alignment")
     if split is not None:
         if body.epilogue is not None or body.post is not None or body.bias is not None or body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None or body.out_dtype is not F32:
             raise LoweringError("contraction: the partial kernel of a split stores bare fp32 accumulators; bias, epilogue and rounding belong to the combine")
@@ -432,10 +440,13 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
 """)
     if split is not None:
         a("  // cross-workgroup split of the reduction axis: workgroup row blockIdx.y owns slice blockIdx.y (K is the slice length)")
-        a("  const long KSL = (long)blockIdx.y * K;")
+        a("  const long ASL = (long)blockIdx.y * K, BSL = ASL;")
         a("  const long OSL = " + ("(long)blockIdx.y * M * LDO;" if split[1] == "kernel" else "0;  // every slice adds into the one zeroed plane"))
+    elif batch > 1:
+        a("  // independent products: workgroup row blockIdx.y owns product blockIdx.y")
+        a(f"  const long ASL = (long)blockIdx.y * {body.a_batch}L, BSL = (long)blockIdx.y * {body.b_batch}L, OSL = (long)blockIdx.y * {body.out_batch}L;")
     else:
-        a("  constexpr long KSL = 0, OSL = 0;")
+        a("  constexpr long ASL = 0, BSL = 0, OSL = 0;")
     # ---- staging ------------------------------------------------------------
     a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else "") + (" int ka[A_PER_T], kb[B_PER_T];" if k_guard else ""))
     a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
@@ -455,7 +466,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         a("    const int row = q / CPR, c = q % CPR;")
         a("    la[i] = row * (BK * ES) + emh_swz(row, c) * 16;")
     a(f"    int gr = m0 + row;{' if (gr > M - 1) gr = M - 1;' if m_guard else ''}")
-    a(f"    ga[i] = A + {body.a_offset}L + KSL + (long)gr * LDA + c * EPCK;")
+    a(f"    ga[i] = A + {body.a_offset}L + ASL + (long)gr * LDA + c * EPCK;")
     if dli or spec:
         a("    va[i] = ((unsigned)gr * LDA + c * EPCK) * (unsigned)ES;")
     if pro is not None:
@@ -478,7 +489,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
             a("    { const int lim = (row < TN) ? (N - 1) : (2 * N - 1); if (gr > lim) gr = lim; }")
     else:
         a(f"    int gr = n0 + row;{' if (gr > N - 1) gr = N - 1;' if n_guard else ''}")
-    a(f"    gb[i] = B + {body.b_offset}L + KSL + (long)gr * LDB + c * EPCK;")
+    a(f"    gb[i] = B + {body.b_offset}L + BSL + (long)gr * LDB + c * EPCK;")
     if dli or spec:
         a("    vb[i] = ((unsigned)gr * LDB + c * EPCK) * (unsigned)ES;")
     if k_guard:
@@ -646,8 +657,8 @@ ROW_EPILOGUE_TABLES
         if dli or spec:
             a(f"""  // One request of slab kt into ring buffer buf: the operand base moves along k in scalar registers, the
   // lane's chunk offset is a loop-invariant 32-bit register, the LDS target a scalar: no vector arithmetic per request.
-  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L + KSL) + (long)(kt) * (BK * ES), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * ST) * 16)
-  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L + KSL) + (long)(kt) * (BK * ES), vb[i], lds0 + (buf) * SLAB + TM * BK * ES + (wave_u * 64 + (i) * ST) * 16)""")
+  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L + ASL) + (long)(kt) * (BK * ES), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * ST) * 16)
+  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L + BSL) + (long)(kt) * (BK * ES), vb[i], lds0 + (buf) * SLAB + TM * BK * ES + (wave_u * 64 + (i) * ST) * 16)""")
         if deferred:
             # the rows arrive in LDS untouched: every thread reads back the chunks it requested
             # (any chunk of the row will do for a row sum) while the slab is resident
@@ -943,7 +954,7 @@ ROW_EPILOGUE_TABLES
             body.a, body.b, *((pro.weight,) if pro is not None and pro.weight is not None else ()), *((body.bias,) if body.bias is not None else ()),
             *(body.operand_buffers.get(n, n) for n in epi_names), *(rowepi.operand_buffers.get(ro.name, ro.name) for ro in (rowepi.row_operands if rowepi is not None else ())), body.out,
         ),  # fmt: skip
-        grid=((grid,), (split[0] if split is not None else 1,), (1,)),
+        grid=((grid,), (split[0] if split is not None else batch,), (1,)),
         block=((TT,), (1,), (1,)),
         lds_bytes=lds_bytes,
         zero_outputs=(body.out,) if split is not None and split[1] == "atomic" else (),

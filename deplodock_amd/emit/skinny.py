@@ -49,7 +49,7 @@ MAX_STEPS_IN_FLIGHT = 16
 
 def skinny_waves(body: Contraction) -> int:
     """Waves that split the reduction axis (0: the shape does not take this form)."""
-    if body.m > 16 or body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None or body.reduce.cta != 1:
+    if body.m > 16 or body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None or body.reduce.cta != 1 or getattr(body, "batch", 1) > 1:
         return 0
     if getattr(body, "sym", None) is not None and "m" in body.sym.fields:
         return 0  # the few-row form holds every row in one MFMA tile: not with a row count known only at launch

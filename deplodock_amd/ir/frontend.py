@@ -57,6 +57,13 @@ class LinearOp(Op):
 
 
 @dataclass
+class BatchedLinearOp(Op):
+    """``x[p] @ w[p].T`` for every ``p`` of a leading batch axis: ``x`` is ``[P, M, K]``, ``w`` is ``[P, N, K]`` or
+    ``[1, N, K]`` (one weight for every product), the result ``[P, M, N]`` — the per-head products of attention
+    written as contractions (``LinearOp`` semantics, emmy/compiler/ir/frontend/ir.py:212-217, per batch entry)."""
+
+
+@dataclass
 class RmsNormOp(Op):
     """``x * rsqrt(mean(x^2, -1) + eps) * w`` (frontend/ir.py:309-312)."""
 

@@ -213,12 +213,22 @@ class Contraction:
     # operands, and the fp32 accumulators go to plane ``blockIdx.y`` of the workspace (``"kernel"``) or are added
     # atomically into its single zeroed plane (``"atomic"``).
     k_split: tuple[int, str] | None = None
+    # ``batch`` independent products in one launch (workgroup row ``blockIdx.y`` takes product ``blockIdx.y``): the
+    # operands and the result of product ``p`` start ``p * a_batch`` / ``p * b_batch`` / ``p * out_batch`` elements
+    # further on (``b_batch`` 0: every product reads the same ``b``).  Plain products only: no bias, prologue, row
+    # epilogue or epilogue operands, no split.
+    batch: int = 1
+    a_batch: int = 0
+    b_batch: int = 0
+    out_batch: int = 0
 
     def algo_flops(self) -> int:
-        return 2 * self.m * self.n * self.k * (2 if self.gate_pair else 1)
+        return 2 * self.m * self.n * self.k * (2 if self.gate_pair else 1) * self.batch
 
     def algo_bytes(self) -> int:
         nb = self.n * (2 if self.gate_pair else 1)
+        if self.batch > 1:
+            return self.batch * (self.m * self.k * self.in_dtype.nbytes + self.m * self.n * self.out_dtype.nbytes) + (self.batch if self.b_batch else 1) * nb * self.k * self.in_dtype.nbytes
         b = (self.m * self.k + nb * self.k) * self.in_dtype.nbytes + self.m * self.n * self.out_dtype.nbytes
         for _, dt in self.epilogue_operands:
             b += self.m * self.n * dt.nbytes

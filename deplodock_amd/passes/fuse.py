@@ -134,7 +134,7 @@ def _materialize(c: _Ctx, nid: str) -> None:
             c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
         c.done[nid] = nid
         return
-    for rec in (_rec_loop_nest, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_pointwise):
+    for rec in (_rec_loop_nest, _rec_batched_linear, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_pointwise):
         if rec(c, nid):
             return
     raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
@@ -254,6 +254,26 @@ def _rec_linear(c: _Ctx, nid: str) -> bool:
     bias = _bias_of(c, nid, n)
     body = Contraction(m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset, a_prologue=pro, **bias)
     _emit(c, nid, body, "rms_norm_linear" if pro else "linear", [x.base, w.base, *extra, *([bias["bias"]] if bias else [])])
+    return True
+
+
+def _rec_batched_linear(c: _Ctx, nid: str) -> bool:
+    """``[P, M, K] x [P | 1, N, K] -> [P, M, N]``: one launch, product ``p`` on workgroup row ``p``."""
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.BatchedLinearOp):
+        return False
+    x, w = _need(c, node.inputs[0]), _need(c, node.inputs[1])
+    if len(x.shape) != 3 or len(w.shape) != 3 or x.shape[2] != w.shape[2] or w.shape[0] not in (1, x.shape[0]):
+        raise FusionError(f"batched linear {nid!r}: operands {x.shape} x {w.shape} are not [P, M, K] x [P | 1, N, K]")
+    if x.strides[2] != 1 or w.strides[2] != 1:
+        raise FusionError(f"batched linear {nid!r}: the reduction axis must be contiguous in both operands")
+    p, m, k = (int(d) for d in x.shape)
+    n = int(w.shape[1])
+    body = Contraction(
+        m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=int(x.strides[1]) if m > 1 else k, ldb=int(w.strides[1]) if n > 1 else k,
+        a_offset=x.offset, b_offset=w.offset, batch=p, a_batch=int(x.strides[0]) if p > 1 else 0, b_batch=int(w.strides[0]) if w.shape[0] > 1 else 0, out_batch=m * n,
+    )  # fmt: skip
+    _emit(c, nid, body, "batched_linear", [x.base, w.base], shape=(p, m, n))
     return True
 
 

@@ -13,9 +13,13 @@ rendering them loop for loop would leave the matrix cores idle:
   becomes ``RmsNormOp`` (frontend/ir.py:309-312; decomposition/080_rms_norm.py:25-57 + 090_mean.py:27-44).
 
 An operand of such a contraction that is read through a permuted or folded index (the o-projection reads the attention
-output ``[H, S, D]`` as ``[S, H*D]``) is first copied to a plain matrix by a small loop nest of its own.  Anything else
-— attention scores with a rotary embedding folded into the operand reads, a softmax-weighted sum — stays a
-``LoopNestOp`` and goes to the loop-nest emitter.  ``EMMY_NEST=loops``
+output ``[H, S, D]`` as ``[S, H*D]``) is first copied to a plain matrix by a small loop nest of its own.
+
+* **the general form** (``_try_batched_contraction``) — a batch of outer loops, operands that are *computed* in the
+  reduction loop (a rotary embedding folded into the reads of q and k; softmax probabilities from two folds that
+  precede the loop), any output stage — becomes operand nests + one ``BatchedLinearOp`` + an output-stage nest.
+
+Anything else stays a ``LoopNestOp`` and goes to the loop-nest emitter.  ``EMMY_NEST=loops``
 keeps every nest there (A/B, and the emitter's own tests).
 """
 
@@ -232,6 +236,192 @@ def _try_contraction(g: Graph, node: Node) -> list[Node] | None:
         return None
 
 
+def _uses(stmt) -> tuple[str, ...]:
+    if isinstance(stmt, L.Assign):
+        return stmt.args
+    if isinstance(stmt, (L.Accum, L.Write)):
+        return (stmt.value,)
+    if isinstance(stmt, L.Select):
+        return tuple(v for v, _ in stmt.branches)
+    return ()
+
+
+def _index_vars(stmt) -> set[str]:
+    exprs = stmt.index if isinstance(stmt, (L.Load, L.Write)) else tuple(p for _, p in stmt.branches) if isinstance(stmt, L.Select) else ()
+    return set().union(*(L.expr_vars(e) for e in exprs)) if exprs else set()
+
+
+def _defined(body) -> set[str]:
+    """Names a statement list binds in its own scope (a loop contributes what it folds)."""
+    out: set[str] = set()
+    for s in body:
+        if isinstance(s, L.Loop):
+            out |= {t.name for t in s.body if isinstance(t, L.Accum)}
+        elif not isinstance(s, L.Write):
+            out.add(s.name)
+    return out
+
+
+def _all_uses(body) -> set[str]:
+    out: set[str] = set()
+    for s in L.walk(body):
+        out |= set(_uses(s))
+    return out
+
+
+def _nest_node(b: _Builder, stmts: tuple, shape: tuple[int, ...], label: str, extra: dict[str, str] | None = None) -> str:
+    """A ``LoopNestOp`` node over ``stmts`` (whose ``Write`` names the new node); its operands are the tensors of the
+    raised node that the statements load, plus ``extra`` (load name -> new node id)."""
+    node = b.node
+    nid = f"{node.id}__r{b.n}"
+    stmts = _retarget(stmts, nid)
+    names = list(dict.fromkeys(s.input for s in L.walk(stmts) if isinstance(s, L.Load)))
+    scalars = {k: v for k, v in (node.op.scalars or {}).items() if k in names}
+    loads, inputs = [], []
+    for name in names:
+        if name in scalars:
+            continue
+        if extra and name in extra:
+            loads.append(name)
+            inputs.append(extra[name])
+        elif name in node.op.loads:
+            loads.append(name)
+            inputs.append(node.inputs[node.op.loads.index(name)])
+        else:
+            raise _NoMatch
+    return b.add(F.LoopNestOp(stmts=stmts, loads=tuple(loads), scalars=scalars, out_name=nid, label=label), inputs, shape)
+
+
+def _retarget(stmts: tuple, out: str) -> tuple:
+    """``stmts`` with every ``Write`` pointed at ``out``."""
+    res = []
+    for s in stmts:
+        if isinstance(s, L.Loop):
+            res.append(L.Loop(s.axis, s.extent, _retarget(s.body, out)))
+        elif isinstance(s, L.Write):
+            res.append(L.Write(out, s.index, s.value))
+        else:
+            res.append(s)
+    return tuple(res)
+
+
+def _wrap(loops: list[L.Loop], body: tuple) -> tuple:
+    for lp in reversed(loops):
+        body = (L.Loop(lp.axis, lp.extent, tuple(body)),)
+    return tuple(body)
+
+
+def _try_batched_contraction(g: Graph, node: Node) -> list[Node] | None:
+    """The general form: outer loops that only wrap (a batch), then ``for m: {prefix; for n: {pre; for k: {...;
+    acc += u * v}; post; write}}`` where ``u`` is computed from values that do not vary with ``n`` and ``v`` from
+    values that do not vary with ``m``.  ``u`` and ``v`` are written out as ``[P, M, K]`` and ``[P | 1, N, K]`` by loop
+    nests of their own (with ``prefix`` — e.g. the two folds of a softmax — in the first), the products are one
+    batched contraction, and ``pre`` / ``post`` run in a third nest over its result."""
+    op: F.LoopNestOp = node.op
+    try:
+        stmts = list(op.stmts)
+        head = [s for s in stmts if not isinstance(s, L.Loop)]
+        if not stmts or not isinstance(stmts[-1], L.Loop) or len(head) != len(stmts) - 1 or not all(isinstance(s, L.Load) and not s.index or isinstance(s, L.Load) and not _index_vars(s) for s in head):
+            raise _NoMatch
+        batch: list[L.Loop] = []
+        cur = stmts[-1]
+        while len(cur.body) == 1 and isinstance(cur.body[0], L.Loop):
+            batch.append(cur)
+            cur = cur.body[0]
+        if cur.body and isinstance(cur.body[-1], L.Write) and batch:
+            lm, prefix, ln = batch.pop(), [], cur  # ``for m: for n: {...; write}``: nothing between the two loops
+        else:
+            lm = cur
+            if not lm.body or not isinstance(lm.body[-1], L.Loop) or any(isinstance(s, L.Write) for s in lm.body[:-1]):
+                raise _NoMatch
+            prefix, ln = list(lm.body[:-1]), lm.body[-1]
+        inner = [s for s in ln.body if isinstance(s, L.Loop)]
+        if len(inner) != 1 or not isinstance(ln.body[-1], L.Write) or any(isinstance(s, L.Write) for s in ln.body[:-1]):
+            raise _NoMatch
+        lk = inner[0]
+        at = ln.body.index(lk)
+        pre, post, write = list(ln.body[:at]), list(ln.body[at + 1 : -1]), ln.body[-1]
+        kb = list(lk.body)
+        if len(kb) < 3 or any(isinstance(s, (L.Loop, L.Write)) for s in kb) or sum(isinstance(s, L.Accum) for s in kb) != 1:
+            raise _NoMatch
+        acc, prod = kb[-1], kb[-2]
+        if not (isinstance(acc, L.Accum) and acc.op == "add" and isinstance(prod, L.Assign) and prod.op == "multiply" and acc.value == prod.name):
+            raise _NoMatch
+        axes = [lp.axis for lp in batch] + [lm.axis, ln.axis, lk.axis]
+        if len(set(axes)) != len(axes):
+            raise _NoMatch
+        bvars = {lp.axis for lp in batch}
+        # what every value of the k loop varies with
+        deps: dict[str, set[str]] = {s.name: set() for s in head}
+        for name in _defined(prefix):
+            deps[name] = bvars | {lm.axis}
+        for name in _defined(pre):
+            deps[name] = bvars | {lm.axis, ln.axis}
+        body_k = kb[:-2]
+        for s in body_k:
+            d = _index_vars(s)
+            for u in _uses(s):
+                if u not in deps:
+                    raise _NoMatch
+                d |= deps[u]
+            deps[s.name] = d
+        u_name, v_name = prod.args
+        if ln.axis in deps[u_name] or lm.axis in deps[v_name]:
+            u_name, v_name = v_name, u_name
+        if ln.axis in deps[u_name] or lm.axis in deps[v_name]:
+            raise _NoMatch
+
+        def side(target: str) -> list:
+            need, keep = {target}, []
+            for s in reversed(body_k):
+                if s.name in need:
+                    keep.append(s)
+                    need |= set(_uses(s))
+            return list(reversed(keep))
+
+        a_stmts, b_stmts = side(u_name), side(v_name)
+        if any(ln.axis in deps[s.name] for s in a_stmts) or any(lm.axis in deps[s.name] for s in b_stmts):
+            raise _NoMatch
+        b = _Builder(g, node)
+        pshape = tuple(lp.extent for lp in batch)
+        p = 1
+        for d in pshape:
+            p *= d
+        bidx = tuple(L.Var(lp.axis) for lp in batch)
+        a_head = [s for s in head if s.name in _all_uses(a_stmts) | _all_uses(prefix)]
+        a_body = _wrap(batch + [lm], (*prefix, L.Loop(lk.axis, lk.extent, (*a_stmts, L.Write("", (*bidx, L.Var(lm.axis), L.Var(lk.axis)), u_name)))))
+        a_id = _nest_node(b, (*a_head, *a_body), (*pshape, lm.extent, lk.extent), "operand_a")
+        b_batched = any(deps[s.name] & bvars for s in b_stmts)
+        b_loops = (batch if b_batched else []) + [ln]
+        b_head = [s for s in head if s.name in _all_uses(b_stmts)]
+        b_body = _wrap(b_loops, (L.Loop(lk.axis, lk.extent, (*b_stmts, L.Write("", (*(bidx if b_batched else ()), L.Var(ln.axis), L.Var(lk.axis)), v_name))),))
+        b_id = _nest_node(b, (*b_head, *b_body), (*(pshape if b_batched else ()), ln.extent, lk.extent), "operand_b")
+        x3 = b.view(a_id, (p, lm.extent, lk.extent))
+        w3 = b.view(b_id, (p if b_batched else 1, ln.extent, lk.extent))
+        t3 = b.add(F.BatchedLinearOp(), [x3, w3], (p, lm.extent, ln.extent))
+        t = b.view(t3, (*pshape, lm.extent, ln.extent))
+        # the output stage: pre / post over the products, as a nest of its own
+        out_shape = tuple(int(d) for d in node.output.shape)
+        stage = [*pre, *post]
+        if not stage and write.value == acc.name:
+            try:
+                if _simple_index(write.index, out_shape, {**{lp.axis: lp.extent for lp in batch}, lm.axis: lm.extent, ln.axis: ln.extent}) == [*(lp.axis for lp in batch), lm.axis, ln.axis]:
+                    b.finish(t3, out_shape)
+                    return b.new
+            except _NoMatch:
+                pass
+        used = _all_uses(stage) | {write.value}
+        e_prefix = prefix if used & _defined(prefix) else []
+        e_head = [s for s in head if s.name in used | _all_uses(e_prefix)]
+        load_t = L.Load(acc.name, t, (*bidx, L.Var(lm.axis), L.Var(ln.axis)))
+        e_body = _wrap(batch + [lm], (*e_prefix, L.Loop(ln.axis, ln.extent, (*pre, load_t, *post, write))))
+        res = _nest_node(b, (*e_head, *e_body), out_shape, "output_stage", extra={t: t})
+        b.finish(res, out_shape)
+        return b.new
+    except (_NoMatch, KeyError, IndexError, ValueError):
+        return None
+
+
 def _try_rms_norm(g: Graph, node: Node) -> list[Node] | None:
     op: F.LoopNestOp = node.op
     scalars = op.scalars or {}
@@ -309,7 +499,7 @@ def raise_loop_nests(g: Graph) -> Graph:
     for nid, node in g.nodes.items():
         new = None
         if isinstance(node.op, F.LoopNestOp):
-            new = _try_contraction(g, node) or _try_rms_norm(g, node)
+            new = _try_contraction(g, node) or _try_rms_norm(g, node) or _try_batched_contraction(g, node)
         if new is None:
             out.nodes[nid] = node
         else:

@@ -159,7 +159,7 @@ def schedule_row_reduce(body: RowReduce, ctx: Context) -> dict:
     return {"REDUCE": plan.spell(), "NT": int(body.nontemporal)}
 
 
-def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologue: bool = False, group_cols: tuple[int, int] | None = None) -> TilePlan:
+def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologue: bool = False, group_cols: tuple[int, int] | None = None, copies: int = 1) -> TilePlan:
     """The largest candidate that makes one workgroup per CU (0.9-1.0 of the CUs, no ragged
     edge), else the first (in measured-throughput order) whose launch covers 75 % of the CUs,
     else the one that launches the most workgroups.
@@ -168,7 +168,10 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
     projections prefer at every token count (in-graph times, us): 2048 tokens q/k/v 34.6 on
     256 tiles of 128x128 with four waves, 28.2 on 256 tiles of 128x256; 1024 tokens gate/up
     22.6 on 192 tiles of 128x128, 18.2 on 256 tiles of 128x96; 512 tokens gate/up 12.8 on 192
-    tiles of 64x128, 10.4 on 256 of 64x96; 256 tokens gate/up 9.93 on 64x64, 8.85 on 32x96."""
+    tiles of 64x128, 10.4 on 256 of 64x96; 256 tokens gate/up 9.93 on 64x64, 8.85 on 32x96.
+
+    ``copies``: independent products of this shape in the one launch (a batched contraction): each adds its own
+    workgroups."""
     best = None
     candidates = TILE_CANDIDATES
     one_round_only = {(128, 256)}  # offered only as an exact fit: as a 75 % cover it was not measured
@@ -216,13 +219,13 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
         plans.append((cand, TilePlan(atom=atom, units=(wm, wn), regs=(fm, fn), bk=bk)))
     cus = ctx.compute_units
     for (tm, tn, wm, wn, *_), plan in plans:
-        groups = -(-m // tm) * -(-n // tn)
+        groups = -(-m // tm) * -(-n // tn) * copies
         if wm * wn > 1 and m % tm == 0 and n % tn == 0 and 0.9 * cus <= groups <= cus:
             return plan  # (the one-wave tile is the last resort: two waves on half as many 16x32 tiles beat it)
     for (tm, tn, *_), plan in plans:
         if (tm, tn) in one_round_only:
             continue
-        groups = -(-m // tm) * -(-n // tn)
+        groups = -(-m // tm) * -(-n // tn) * copies
         # penalise tiles that mostly hang over the edge of a small problem
         waste = (-(-m // tm) * tm * -(-n // tn) * tn) / float(max(m * n, 1))
         # two waves on a 16x32 tile beat one wave on each of twice as many 16x16 tiles down to half the CUs
@@ -353,7 +356,8 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
 def _default_tile(body: Contraction, ctx: Context) -> TilePlan:
     atom_dtype = body.in_dtype.name
     re = body.row_epilogue
-    plan = pick_tile(body.m, body.n, body.k, body.gate_pair, ctx, row_prologue=body.a_prologue is not None, group_cols=(re.cols, re.col_end) if re is not None else None)
+    plan = pick_tile(body.m, body.n, body.k, body.gate_pair, ctx, row_prologue=body.a_prologue is not None, group_cols=(re.cols, re.col_end) if re is not None else None,
+                     copies=max(1, int(getattr(body, "batch", 1) or 1)))
     if atom_dtype == "f32":
         # the fp32 tier keeps the candidate's tile and its slab's bytes per row: half the k-values, on the fp32 atom of the same m x n
         atom = ATOMS[{16: "mfma_16x16x4_f32", 32: "mfma_32x32x2_f32"}[plan.atom.m]]
@@ -427,8 +431,8 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
         try:
             rp = ReducePlan.parse(pinned_reduce)
             if rp.cta > 1:
-                if body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None:
-                    raise ScheduleError("a cross-workgroup split takes a plain contraction (no gate/up pair, row prologue or row epilogue)")
+                if body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None or getattr(body, "batch", 1) > 1:
+                    raise ScheduleError("a cross-workgroup split takes a plain single contraction (no gate/up pair, row prologue, row epilogue or batch)")
                 if body.k % rp.cta or (body.k // rp.cta) % plan.bk_elems:
                     raise ScheduleError(f"K={body.k} does not split into {rp.cta} slices of whole {plan.bk_elems}-deep slabs")
                 if stage.transport in ("ks", "mix"):

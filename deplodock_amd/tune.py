@@ -65,7 +65,8 @@ def shape_key(body) -> str | None:
     """What a tuned pin is valid for: the kernel family and every size / dtype /
     structural flag its schedule depends on."""
     if isinstance(body, Contraction):
-        return f"contraction/m{body.m}/n{body.n}/k{body.k}/{body.in_dtype.name}>{body.out_dtype.name}/g{int(body.gate_pair)}/p{int(body.post is not None)}/a{int(body.a_prologue is not None)}" + (f"/e{body.row_epilogue.cols}" if body.row_epilogue is not None else "")
+        return f"contraction/m{body.m}/n{body.n}/k{body.k}/{body.in_dtype.name}>{body.out_dtype.name}/g{int(body.gate_pair)}/p{int(body.post is not None)}/a{int(body.a_prologue is not None)}" + (f"/e{body.row_epilogue.cols}" if body.row_epilogue is not None else "") + (
+            f"/x{body.batch}" if getattr(body, "batch", 1) > 1 else "")
     if isinstance(body, RowReduce):
         return f"row_reduce/r{body.rows}/c{body.cols}/{body.x_dtype.name}>{body.out_dtype.name}/s{len(body.stats)}/rot{int(body.rotate is not None)}"
     if isinstance(body, Flash):

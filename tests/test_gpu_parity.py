@@ -1065,3 +1065,40 @@ def test_streamed_rms_norm_and_pinned_streaming(device, monkeypatch):
     ours, want, compiled = run_case(case, device)
     assert [n_.op.knobs["REDUCE"] for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)] == ["b1024/stream"]
     eager.assert_close(ours, want, case.rtol, case.atol, "pinned streaming softmax")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize(
+    "dtype, p, m, n, k, shared",
+    [("bf16", 32, 128, 128, 64, False), ("bf16", 6, 100, 72, 96, True), ("f32", 32, 128, 64, 128, False), ("f32", 5, 37, 40, 72, True), ("bf16", 16, 512, 512, 64, False)],
+)
+def test_batched_linear(device, dtype, p, m, n, k, shared):
+    """``[P, M, K] x [P | 1, N, K] -> [P, M, N]``: the per-head products of attention as one launch of the MFMA
+    contraction (workgroup row ``p`` takes product ``p``), ragged tiles included, against a float64 product."""
+    from deplodock_amd.ir import frontend as F
+
+    dt, tdt = (BF16, torch.bfloat16) if dtype == "bf16" else (F32, torch.float32)
+    torch.manual_seed(21)
+    x = torch.randn(p, m, k).to(tdt)
+    w = (0.1 * torch.randn(1 if shared else p, n, k)).to(tdt)
+    g = Graph()
+    g.add_input("x", tuple(x.shape), dt)
+    g.add_input("w", tuple(w.shape), dt)
+    g.add_node(F.BatchedLinearOp(), ["x", "w"], Tensor("y", (p, m, n), dt), "y")
+    g.outputs = ["y"]
+    be = HipBackend()
+    compiled = be.compile(g)
+    ks = [nd.op for nd in compiled.nodes.values() if isinstance(nd.op, HipOp)]
+    assert len(ks) == 1 and ks[0].kernel_name.startswith("k_batched_linear_") and ks[0].grid[1] == (p,)
+    prog = be.program(compiled, {"x": x.to(device), "w": w.to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()["y"].clone()
+    finally:
+        prog.close()
+    want = torch.matmul(x.double(), w.double().transpose(-1, -2))
+    if dtype == "bf16":
+        eager.assert_close(ours.reshape(want.shape), want.float(), 2e-2, 2e-2, "batched linear bf16 vs float64")
+    else:
+        eager.assert_close(ours.reshape(want.shape), want.float(), 1e-4, 1e-4 * float(want.pow(2).mean().sqrt()), "batched linear fp32 vs float64")

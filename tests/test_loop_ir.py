@@ -211,8 +211,12 @@ RAISED = {  # what each reproducer becomes when nests with a tiled form are rais
     "k_mul_1_reduce": ["k_rms_norm_reduce"],
     "k_mul_7_reduce": ["k_rms_norm_reduce"],
     "k_mul_8_reduce": ["k_linear", "k_pointwise_fused6"],
-    "k_scaled_dot_product_attention_masked_reduce": ["k_lift_scaled_dot_product_attention_masked"],  # rotary embedding in the operand reads
-    "k_scaled_dot_product_attention_reduce_reduce": ["k_lift_scaled_dot_product_attention_reduce"],  # softmax-weighted sum
+    # scores: the rotary embedding is applied while each operand is written out, the per-head products are one batched
+    # contraction, scale and causal mask run over its result
+    "k_scaled_dot_product_attention_masked_reduce": ["k_operand_a", "k_operand_b", "k_batched_linear", "k_output_stage"],
+    # softmax-weighted sum: the probabilities (two folds and the division) and the transposed values are written out,
+    # then one batched contraction
+    "k_scaled_dot_product_attention_reduce_reduce": ["k_operand_a", "k_operand_b", "k_batched_linear"],
 }
 
 
@@ -237,8 +241,7 @@ def test_every_reproducer_lowers_to_kernels_that_build_for_gfx950(launcher_lib, 
             assert len(ks) == 1 and "NEST" in ks[0].knobs, (path.name, labels)
         else:
             assert labels == RAISED[path.stem], (path.name, labels)
-            assert [("NEST" in k.knobs) for k in ks] == [not lab.startswith(("k_linear", "k_rms_norm", "k_pointwise")) for lab in labels]
-            assert sum("NEST" in k.knobs and lab != "k_gather" for k, lab in zip(ks, labels)) == (1 if "attention" in path.stem else 0)
+            assert [("NEST" in k.knobs) for k in ks] == [lab in ("k_gather", "k_operand_a", "k_operand_b", "k_output_stage") for lab in labels]
         for k in ks:
             hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
             assert hiprtc.spilled_vgprs(k.kernel_source, k.kernel_name) == 0
@@ -278,8 +281,6 @@ def test_reproducer_on_the_gpu_equals_the_interpreter(device, monkeypatch, kerne
     import torch
 
     if mode == "loops":
-        if not RAISED[kernel][0].startswith(("k_linear", "k_rms_norm", "k_gather")):
-            pytest.skip("this reproducer is a loop nest in both modes")
         monkeypatch.setenv("EMMY_NEST", "loops")
 
     from deplodock_amd import HipBackend
