@@ -64,6 +64,13 @@ class BatchedLinearOp(Op):
 
 
 @dataclass
+class MatmulOp(Op):
+    """``a @ b`` with numpy semantics on the last two axes: ``a`` is ``[..., M, K]``, ``b`` is ``[K, N]`` or
+    ``[..., K, N]`` with the same leading axes (emmy/compiler/ir/frontend/ir.py ``MatmulOp``; the reference
+    decomposes it into a broadcast multiply and a sum, decomposition/070_matmul.py)."""
+
+
+@dataclass
 class RmsNormOp(Op):
     """``x * rsqrt(mean(x^2, -1) + eps) * w`` (frontend/ir.py:309-312)."""
 

@@ -134,7 +134,7 @@ def _materialize(c: _Ctx, nid: str) -> None:
             c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
         c.done[nid] = nid
         return
-    for rec in (_rec_loop_nest, _rec_batched_linear, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_pointwise):
+    for rec in (_rec_loop_nest, _rec_batched_linear, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_pointwise):
         if rec(c, nid):
             return
     raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
@@ -274,6 +274,71 @@ def _rec_batched_linear(c: _Ctx, nid: str) -> bool:
         a_offset=x.offset, b_offset=w.offset, batch=p, a_batch=int(x.strides[0]) if p > 1 else 0, b_batch=int(w.strides[0]) if w.shape[0] > 1 else 0, out_batch=m * n,
     )  # fmt: skip
     _emit(c, nid, body, "batched_linear", [x.base, w.base], shape=(p, m, n))
+    return True
+
+
+def _copy_of_view(c: _Ctx, v: View, order: tuple[int, ...], new_id: str) -> View:
+    """A dense row-major copy of ``v`` with its axes in ``order``, made by a loop nest of its own (``new_id``): what a
+    contraction needs when an operand's reduction axis is not the contiguous one, or its leading axes are not one
+    uniformly strided run."""
+    from deplodock_amd.ir import loopnest as L
+    from deplodock_amd.ir.tile import LoopNest
+
+    numel = c.out.nodes[v.base].output.numel
+    axes = [f"c{i}" for i in range(len(v.shape))]
+    flat: object = L.Lit(int(v.offset))
+    for ax, st in zip(axes, v.strides):
+        if st:
+            flat = L.Bin("+", flat, L.Bin("*", L.Var(ax), L.Lit(int(st))))
+    body: tuple = (L.Load("t", "src", (flat,)), L.Write(new_id, tuple(L.Var(axes[i]) for i in order), "t"))
+    for i in reversed(order):
+        body = (L.Loop(axes[i], int(v.shape[i]), body),)
+    shape = tuple(int(v.shape[i]) for i in order)
+    nest = LoopNest(stmts=body, operands={"src": (v.base, (int(numel),), v.dtype)}, scalars={}, out=new_id, out_name=new_id, out_shape=shape, out_dtype=v.dtype)
+    c.out.add_node(TileOp(name=c.kname("gather"), body=nest), [v.base], Tensor(new_id, shape, v.dtype), new_id)
+    return View(new_id, 0, shape, contiguous_strides(shape), v.dtype)
+
+
+def _rec_matmul(c: _Ctx, nid: str) -> bool:
+    """``[..., M, K] @ [..., K, N]``: one (batched) contraction.  The contraction reads both operands along their
+    reduction axis, so ``b`` is taken as ``[N, K]`` rows: a ``k.transpose(-1, -2)`` already is that in memory; a
+    plain ``[K, N]`` operand (``p @ v``) is transposed by a copy nest first."""
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.MatmulOp):
+        return False
+    a, b = _need(c, node.inputs[0]), _need(c, node.inputs[1])
+    if len(a.shape) < 2 or len(b.shape) < 2 or a.shape[-1] != b.shape[-2]:
+        raise FusionError(f"matmul {nid!r}: operands {a.shape} @ {b.shape}")
+    m, k, n = int(a.shape[-2]), int(a.shape[-1]), int(b.shape[-1])
+    lead = tuple(int(d) for d in a.shape[:-2])
+    p = 1
+    for d in lead:
+        p *= d
+    shared = len(b.shape) == 2 or all(int(d) == 1 for d in b.shape[:-2])
+    if not shared and tuple(int(d) for d in b.shape[:-2]) != lead:
+        raise FusionError(f"matmul {nid!r}: leading axes {a.shape[:-2]} and {b.shape[:-2]} differ")
+    if a.dtype != b.dtype:
+        raise FusionError(f"matmul {nid!r}: operand types differ")
+    if k % (16 // a.dtype.nbytes):
+        raise FusionError(f"matmul {nid!r}: the reduction extent {k} is not whole 16-byte chunks of {a.dtype} (the contraction reads its operands in such chunks)")
+    ra = len(a.shape)
+    if a.strides[-1] != 1 and k > 1 or a.collapse_leading(2) is None or (a.offset * a.dtype.nbytes) % 16 or (m > 1 and (a.strides[-2] * a.dtype.nbytes) % 16):
+        a = _copy_of_view(c, a, tuple(range(ra)), f"{nid}__a")
+    rb = len(b.shape)
+    order_b = (*range(rb - 2), rb - 1, rb - 2)  # [..., N, K]
+    if b.strides[-2] != 1 and k > 1 or b.collapse_leading(2) is None or (b.offset * b.dtype.nbytes) % 16 or (n > 1 and (b.strides[-1] * b.dtype.nbytes) % 16):
+        b = _copy_of_view(c, b, order_b, f"{nid}__bt")
+    else:
+        b = View(b.base, b.offset, tuple(b.shape[i] for i in order_b), tuple(b.strides[i] for i in order_b), b.dtype)
+    pa, sa = a.collapse_leading(2)
+    pb, sb = b.collapse_leading(2)
+    if (pa > 1 and (sa * a.dtype.nbytes) % 16) or (pb > 1 and (sb * b.dtype.nbytes) % 16) or (m * n * node.output.dtype.nbytes) % 16 and p > 1:
+        raise FusionError(f"matmul {nid!r}: batch strides break 16-byte alignment")
+    body = Contraction(
+        m=m, n=n, k=k, a=a.base, b=b.base, out=nid, in_dtype=a.dtype, out_dtype=node.output.dtype, lda=int(a.strides[-2]) if m > 1 else k, ldb=int(b.strides[-2]) if n > 1 else k,
+        a_offset=a.offset, b_offset=b.offset, batch=p, a_batch=int(sa) if p > 1 else 0, b_batch=0 if shared or p == 1 else int(sb), out_batch=m * n,
+    )  # fmt: skip
+    _emit(c, nid, body, "matmul", [a.base, b.base])
     return True
 
 

@@ -208,6 +208,11 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
         elif t == aten.linear.default:
             ins = [a[0], a[1]] + ([a[2]] if len(a) > 2 and a[2] is not None else [])
             add(node, F.LinearOp(has_bias=len(ins) == 3), ins)
+        elif t in (aten.matmul.default, aten.bmm.default, aten.mm.default):
+            ra, rb = len(a[0].meta["val"].shape), len(a[1].meta["val"].shape)
+            if ra < 2 or rb < 2 or (rb > 2 and tuple(a[0].meta["val"].shape[:-2]) != tuple(a[1].meta["val"].shape[:-2])):
+                raise TraceError(f"{t}: operands must be [..., M, K] and [K, N] or [..., K, N] with equal leading axes")
+            add(node, F.MatmulOp(), [a[0], a[1]])
         elif t == aten.scaled_dot_product_attention.default:
             mask = a[3] if len(a) > 3 else kw.get("attn_mask")
             if mask is not None:

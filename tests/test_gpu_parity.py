@@ -1102,3 +1102,59 @@ def test_batched_linear(device, dtype, p, m, n, k, shared):
         eager.assert_close(ours.reshape(want.shape), want.float(), 2e-2, 2e-2, "batched linear bf16 vs float64")
     else:
         eager.assert_close(ours.reshape(want.shape), want.float(), 1e-4, 1e-4 * float(want.pow(2).mean().sqrt()), "batched linear fp32 vs float64")
+
+
+class _EagerAttention(nn.Module):
+    """Attention spelled with matmuls, as a model without the fused op traces it."""
+
+    def forward(self, q, k, v):
+        s = torch.matmul(q, k.transpose(-1, -2)) * (1.0 / float(q.shape[-1]) ** 0.5)
+        return torch.softmax(s, -1) @ v
+
+
+class _Mm(nn.Module):
+    def forward(self, a, b):
+        return a @ b
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_matmul_spelled_attention(device, dtype):
+    """``q @ k.T`` reads ``k`` as it lies (the transpose is a view whose reduction axis is contiguous); ``p @ v`` needs
+    ``v`` transposed, which a copy nest does; both products are batched contractions over batch x heads."""
+    torch.manual_seed(31)
+    q, k, v = (torch.randn(2, 4, 104, 64).to(dtype) for _ in range(3))  # (the key count is the second product's reduction extent: whole 16-byte chunks)
+    mod = _EagerAttention().eval()
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, (q, k, v)))
+    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert names.count("k_matmul") == 2 and names.count("k_gather") == 1 and "k_softmax_reduce" in names
+    prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in (q, k, v)))))
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = mod(q.double(), k.double(), v.double()).float()
+    tol = (2e-2, 2e-2) if dtype is torch.bfloat16 else (1e-4, 1e-5)
+    eager.assert_close(ours.reshape(want.shape), want, *tol, f"matmul-spelled attention {dtype}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape_a, shape_b", [((70, 96), (96, 40)), ((3, 50, 64), (64, 72)), ((2, 3, 33, 32), (2, 3, 32, 48))])
+def test_plain_matmul(device, shape_a, shape_b):
+    """``a @ b`` with ``b`` stored ``[K, N]``: shared by every product or one per product."""
+    torch.manual_seed(32)
+    a, b = torch.randn(*shape_a), 0.2 * torch.randn(*shape_b)
+    be = HipBackend()
+    compiled = be.compile(trace_module(_Mm().eval(), (a, b)))
+    prog = be.program(compiled, dict(zip(compiled.inputs, (a.to(device), b.to(device)))))
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = (a.double() @ b.double()).float()
+    eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-4 * float(want.pow(2).mean().sqrt()), f"matmul {shape_a} @ {shape_b}")

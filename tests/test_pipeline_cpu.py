@@ -499,3 +499,34 @@ def test_a_pinned_tile_that_only_builds_with_spills_degrades(launcher_lib, monke
     monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w1x1/f3x6/k2")  # 288 accumulators per lane
     k = kernels(compile_case(eager.linear_case(m=256, k=1024, n=1024)))[0]
     assert "f3x6" not in k.knobs["TILE"]
+
+
+def test_matmul_spelled_attention_lowers_to_batched_contractions(launcher_lib):
+    """``torch.matmul`` / ``@`` trace to ``MatmulOp``: ``q @ k.T`` reads ``k`` in place (the transposed view's reduction
+    axis is the contiguous one), ``p @ v`` gets ``v`` transposed by a copy nest; each product is one launch whose
+    second grid dimension is batch x heads.  A reduction extent that is not whole 16-byte chunks is refused."""
+    import torch
+    from torch import nn
+
+    from deplodock_amd import HipBackend, trace_module
+    from deplodock_amd.backend.hip import hiprtc
+    from deplodock_amd.ir import frontend as F
+    from deplodock_amd.ir.hip import HipOp
+    from deplodock_amd.passes.fuse import FusionError
+
+    class Attn(nn.Module):
+        def forward(self, q, k, v):
+            return torch.softmax(torch.matmul(q, k.transpose(-1, -2)) * 0.125, -1) @ v
+
+    q = torch.randn(2, 4, 104, 64).bfloat16()
+    traced = trace_module(Attn().eval(), (q, q.clone(), q.clone()))
+    assert sum(isinstance(n.op, F.MatmulOp) for n in traced.nodes.values()) == 2
+    compiled = HipBackend().compile(traced)
+    ks = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert [k.kernel_name.rsplit("_", 1)[0] for k in ks] == ["k_matmul", "k_pointwise_elementwise", "k_softmax_reduce", "k_gather", "k_matmul"]
+    assert [k.grid[1] for k in ks if k.kernel_name.startswith("k_matmul")] == [(8,), (8,)]
+    for k in ks:
+        hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+    q = torch.randn(2, 4, 100, 64).bfloat16()
+    with pytest.raises(FusionError, match="whole 16-byte chunks"):
+        HipBackend().compile(trace_module(Attn().eval(), (q, q.clone(), q.clone())))
