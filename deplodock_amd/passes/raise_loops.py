@@ -439,9 +439,11 @@ def _try_rms_norm(g: Graph, node: Node) -> list[Node] | None:
             raise _NoMatch
         # sum of squares
         b1 = list(l1.body)
+        if len(b1) == 3:  # the row element loaded once and multiplied by itself
+            b1 = [b1[0], b1[0], *b1[1:]]
         if len(b1) != 4 or not (isinstance(b1[0], L.Load) and isinstance(b1[1], L.Load) and isinstance(b1[2], L.Assign) and isinstance(b1[3], L.Accum)):
             raise _NoMatch
-        if b1[0].input != b1[1].input or b1[0].index != b1[1].index or b1[2].op != "multiply" or set(b1[2].args) != {b1[0].name, b1[1].name} or b1[3].op != "add" or b1[3].value != b1[2].name:
+        if b1[0].input != b1[1].input or b1[0].index != b1[1].index or b1[2].op != "multiply" or len(b1[2].args) != 2 or set(b1[2].args) != {b1[0].name, b1[1].name} or b1[3].op != "add" or b1[3].value != b1[2].name:
             raise _NoMatch
         b = _Builder(g, node)
         x = _source(node, b1[0])

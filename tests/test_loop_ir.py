@@ -390,6 +390,31 @@ HAND = {
             {"X": (64, 128), "Wt": (128, 48)}, ("Y", (64, 48))),
         ["k_gather", "k_linear"],
     ),
+    # a batch of products whose first operand is computed in the reduction loop (scaled), whose second is shared by
+    # every product, with a bias in the output stage: operand nests + one batched contraction + an output-stage nest
+    "batched_computed_operand": (
+        _doc(
+            ["Load(name='two', input='c_two', index=(" + _ZERO + ",))",
+             f"Loop(axis=Axis(name='h', extent=3), body=(Loop(axis=Axis(name='m', extent=40), body=(Loop(axis=Axis(name='n', extent=24), body=("
+             f"Loop(axis=Axis(name='k', extent=32), body=(Load(name='a', input='X', index=({_V('h')}, {_V('m')}, {_V('k')})), Assign(name='u', op=ElementwiseImpl('multiply'), args=('a','two')), "
+             f"Load(name='w', input='W', index=({_V('n')}, {_V('k')})), Assign(name='p', op=ElementwiseImpl('multiply'), args=('u','w')), Accum(name='s', value='p'))), "
+             f"Load(name='bb', input='bias', index=({_V('n')},)), Assign(name='y', op=ElementwiseImpl('add'), args=('s','bb')), "
+             f"Write(output='Y', index=({_V('h')}, {_V('m')}, {_V('n')}), value='y'))),)),))"],
+            {"X": (3, 40, 32), "W": (24, 32), "bias": (24,)}, ("Y", (3, 40, 24)), {"c_two": 2.0}),
+        ["k_operand_a", "k_operand_b", "k_batched_linear", "k_output_stage"],
+    ),
+    # RMS normalisation with the row element loaded once and squared (the 512-token corpus spells it this way)
+    "rms_single_load": (
+        _doc(
+            ["Load(name='cnt', input='c_cnt', index=(" + _ZERO + ",))", "Load(name='eps', input='c_eps', index=(" + _ZERO + ",))",
+             f"Loop(axis=Axis(name='r', extent=50), body=(Loop(axis=Axis(name='c', extent=256), body=(Load(name='x', input='X', index=({_ZERO}, {_V('r')}, {_V('c')})), "
+             "Assign(name='sq', op=ElementwiseImpl('multiply'), args=('x','x')), Accum(name='ss', value='sq'))), "
+             "Assign(name='mean', op=ElementwiseImpl('divide'), args=('ss','cnt')), Assign(name='me', op=ElementwiseImpl('add'), args=('mean','eps')), Assign(name='rs', op=ElementwiseImpl('rsqrt'), args=('me',)), "
+             f"Loop(axis=Axis(name='c2', extent=256), body=(Load(name='x2', input='X', index=({_ZERO}, {_V('r')}, {_V('c2')})), Assign(name='xn', op=ElementwiseImpl('multiply'), args=('x2','rs')), "
+             f"Load(name='w', input='W', index=({_V('c2')},)), Assign(name='y', op=ElementwiseImpl('multiply'), args=('w','xn')), Write(output='Y', index=({_ZERO}, {_V('r')}, {_V('c2')}), value='y')))))"],
+            {"X": (1, 50, 256), "W": (256,)}, ("Y", (1, 50, 256)), {"c_cnt": 256.0, "c_eps": 1e-5}),
+        ["k_rms_norm_reduce"],
+    ),
     # a normalisation without a weight and with a maximum instead of a sum: neither tiled form, stays a loop nest
     "max_normalise": (
         _doc(
