@@ -264,8 +264,8 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
             raise LoweringError("contraction: a batch of products takes plain products only (no split, bias, prologue, row epilogue, epilogue operands or gate pair)")
         if batch > 65535:
             raise LoweringError(f"contraction: {batch} products exceed the launch's second dimension")
-        if (body.a_batch * ES) % 16 or (body.b_batch * ES) % 16 or (body.out_batch * body.out_dtype.nbytes) % 16:
-            raise LoweringError("contraction: batch strides must keep 16-byte alignment")
+        if (body.a_batch * ES) % 16 or (body.b_batch * ES) % 16 or body.out_batch % 4:
+            raise LoweringError("contraction: batch strides must keep 16-byte operand alignment and whole 4-element output runs")
     if split is not None:
         if body.epilogue is not None or body.post is not None or body.bias is not None or body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None or body.out_dtype is not F32:
             raise LoweringError("contraction: the partial kernel of a split stores bare fp32 accumulators; bias, epilogue and rounding belong to the combine")

@@ -277,7 +277,7 @@ def _rec_batched_linear(c: _Ctx, nid: str) -> bool:
     return True
 
 
-def _copy_of_view(c: _Ctx, v: View, order: tuple[int, ...], new_id: str) -> View:
+def _copy_of_view(c: _Ctx, v: View, order: tuple[int, ...], new_id: str, pad_last_to: int | None = None) -> View:
     """A dense row-major copy of ``v`` with its axes in ``order``, made by a loop nest of its own (``new_id``): what a
     contraction needs when an operand's reduction axis is not the contiguous one, or its leading axes are not one
     uniformly strided run."""
@@ -286,15 +286,29 @@ def _copy_of_view(c: _Ctx, v: View, order: tuple[int, ...], new_id: str) -> View
 
     numel = c.out.nodes[v.base].output.numel
     axes = [f"c{i}" for i in range(len(v.shape))]
+    last = order[-1]
+    extent = {i: int(v.shape[i]) for i in order}
+    padded = pad_last_to is not None and pad_last_to > extent[last]
+
+    def ax(i: int):
+        # a padded last axis runs past the source: its index is clamped (the value read there is replaced by zero)
+        return L.Ternary(L.Bin("<", L.Var(axes[i]), L.Lit(extent[i])), L.Var(axes[i]), L.Lit(0)) if padded and i == last else L.Var(axes[i])
+
     flat: object = L.Lit(int(v.offset))
-    for ax, st in zip(axes, v.strides):
+    for i, st in enumerate(v.strides):
         if st:
-            flat = L.Bin("+", flat, L.Bin("*", L.Var(ax), L.Lit(int(st))))
-    body: tuple = (L.Load("t", "src", (flat,)), L.Write(new_id, tuple(L.Var(axes[i]) for i in order), "t"))
+            flat = L.Bin("+", flat, L.Bin("*", ax(i), L.Lit(int(st))))
+    if padded:
+        body: tuple = (L.Load("t", "src", (flat,)), L.Load("z", "zero", (L.Lit(0),)),
+                       L.Select("u", (("t", L.Bin("<", L.Var(axes[last]), L.Lit(extent[last]))), ("z", L.Lit(1)))),
+                       L.Write(new_id, tuple(L.Var(axes[i]) for i in order), "u"))  # fmt: skip
+        extent[last] = int(pad_last_to)
+    else:
+        body = (L.Load("t", "src", (flat,)), L.Write(new_id, tuple(L.Var(axes[i]) for i in order), "t"))
     for i in reversed(order):
-        body = (L.Loop(axes[i], int(v.shape[i]), body),)
-    shape = tuple(int(v.shape[i]) for i in order)
-    nest = LoopNest(stmts=body, operands={"src": (v.base, (int(numel),), v.dtype)}, scalars={}, out=new_id, out_name=new_id, out_shape=shape, out_dtype=v.dtype)
+        body = (L.Loop(axes[i], extent[i], body),)
+    shape = tuple(extent[i] for i in order)
+    nest = LoopNest(stmts=body, operands={"src": (v.base, (int(numel),), v.dtype)}, scalars={"zero": 0.0} if padded else {}, out=new_id, out_name=new_id, out_shape=shape, out_dtype=v.dtype)
     c.out.add_node(TileOp(name=c.kname("gather"), body=nest), [v.base], Tensor(new_id, shape, v.dtype), new_id)
     return View(new_id, 0, shape, contiguous_strides(shape), v.dtype)
 
@@ -319,23 +333,24 @@ def _rec_matmul(c: _Ctx, nid: str) -> bool:
         raise FusionError(f"matmul {nid!r}: leading axes {a.shape[:-2]} and {b.shape[:-2]} differ")
     if a.dtype != b.dtype:
         raise FusionError(f"matmul {nid!r}: operand types differ")
-    if k % (16 // a.dtype.nbytes):
-        raise FusionError(f"matmul {nid!r}: the reduction extent {k} is not whole 16-byte chunks of {a.dtype} (the contraction reads its operands in such chunks)")
+    kp = -(-k // 8) * 8  # the contraction reads whole 16-byte chunks and MFMA steps: a ragged reduction extent is padded with zeros in both operands
     ra = len(a.shape)
-    if a.strides[-1] != 1 and k > 1 or a.collapse_leading(2) is None or (a.offset * a.dtype.nbytes) % 16 or (m > 1 and (a.strides[-2] * a.dtype.nbytes) % 16):
-        a = _copy_of_view(c, a, tuple(range(ra)), f"{nid}__a")
+    if kp != k or a.strides[-1] != 1 and k > 1 or a.collapse_leading(2) is None or (a.offset * a.dtype.nbytes) % 16 or (m > 1 and (a.strides[-2] * a.dtype.nbytes) % 16):
+        a = _copy_of_view(c, a, tuple(range(ra)), f"{nid}__a", pad_last_to=kp)
     rb = len(b.shape)
     order_b = (*range(rb - 2), rb - 1, rb - 2)  # [..., N, K]
-    if b.strides[-2] != 1 and k > 1 or b.collapse_leading(2) is None or (b.offset * b.dtype.nbytes) % 16 or (n > 1 and (b.strides[-1] * b.dtype.nbytes) % 16):
-        b = _copy_of_view(c, b, order_b, f"{nid}__bt")
+    if kp != k or b.strides[-2] != 1 and k > 1 or b.collapse_leading(2) is None or (b.offset * b.dtype.nbytes) % 16 or (n > 1 and (b.strides[-1] * b.dtype.nbytes) % 16):
+        b = _copy_of_view(c, b, order_b, f"{nid}__bt", pad_last_to=kp)
     else:
         b = View(b.base, b.offset, tuple(b.shape[i] for i in order_b), tuple(b.strides[i] for i in order_b), b.dtype)
     pa, sa = a.collapse_leading(2)
     pb, sb = b.collapse_leading(2)
-    if (pa > 1 and (sa * a.dtype.nbytes) % 16) or (pb > 1 and (sb * b.dtype.nbytes) % 16) or (m * n * node.output.dtype.nbytes) % 16 and p > 1:
+    if n % 4:
+        raise FusionError(f"matmul {nid!r}: {n} output columns are not whole runs of four (the contraction stores such runs)")
+    if (pa > 1 and (sa * a.dtype.nbytes) % 16) or (pb > 1 and (sb * b.dtype.nbytes) % 16):
         raise FusionError(f"matmul {nid!r}: batch strides break 16-byte alignment")
     body = Contraction(
-        m=m, n=n, k=k, a=a.base, b=b.base, out=nid, in_dtype=a.dtype, out_dtype=node.output.dtype, lda=int(a.strides[-2]) if m > 1 else k, ldb=int(b.strides[-2]) if n > 1 else k,
+        m=m, n=n, k=kp, a=a.base, b=b.base, out=nid, in_dtype=a.dtype, out_dtype=node.output.dtype, lda=int(a.strides[-2]) if m > 1 else kp, ldb=int(b.strides[-2]) if n > 1 else kp,
         a_offset=a.offset, b_offset=b.offset, batch=p, a_batch=int(sa) if p > 1 else 0, b_batch=0 if shared or p == 1 else int(sb), out_batch=m * n,
     )  # fmt: skip
     _emit(c, nid, body, "matmul", [a.base, b.base])
