@@ -24,6 +24,7 @@ from pathlib import Path
 from deplodock_amd import dtype as dt
 from deplodock_amd.graph import Graph, Node, Tensor
 from deplodock_amd.ir import frontend as F
+from deplodock_amd.ir import loopnest as _loopnest
 from deplodock_amd.ir.base import ConstantOp, InputOp, Op
 from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.ir.sym import Affine, CeilDiv, XcdRounds
@@ -45,6 +46,9 @@ class TracedSizes:
     hints: dict
 
 
+_LOOP_IR = ("Var", "Lit", "Bin", "Ternary", "Load", "Assign", "Accum", "Select", "Write", "Loop")  # statements of a LoopNestOp (ir/loopnest.py)
+
+
 def _enc(v, where: str):
     if isinstance(v, dt.DType):
         return {"$dtype": v.name}
@@ -60,6 +64,8 @@ def _enc(v, where: str):
         return {"$tuple": [_enc(x, where) for x in v]} if isinstance(v, tuple) else [_enc(x, where) for x in v]
     if isinstance(v, dict):
         return {"$dict": {str(k): _enc(x, where) for k, x in v.items()}}
+    if type(v).__name__ in _LOOP_IR and type(v) is getattr(_loopnest, type(v).__name__):
+        return {"$loop": [type(v).__name__, *(_enc(getattr(v, f.name), where) for f in dataclasses.fields(v))]}
     raise SerializeError(f"{where}: cannot serialise {type(v).__name__}")
 
 
@@ -79,6 +85,11 @@ def _dec(v):
         if "$xcdrounds" in v:
             m, *rest = v["$xcdrounds"]
             return XcdRounds(_dec(m), *(int(x) for x in rest))
+        if "$loop" in v:
+            kind, *fields = v["$loop"]
+            if kind not in _LOOP_IR:
+                raise SerializeError(f"unknown Loop-IR statement {kind!r}")
+            return getattr(_loopnest, kind)(*(_dec(x) for x in fields))
         raise SerializeError(f"unknown encoded object {sorted(v)}")
     if isinstance(v, list):
         return [_dec(x) for x in v]

@@ -154,3 +154,33 @@ def test_reloaded_lowered_graph_computes_what_the_original_does(device, tmp_path
         eager.assert_close(ours, eager.run_eager(case, device), case.rtol, case.atol, "reloaded linear vs eager")
     finally:
         prog.close()
+
+
+def test_loop_ir_and_matmul_graphs_round_trip(launcher_lib):
+    """A graph read from the reference's Loop-IR JSON (its statements are nested dataclasses) and a traced graph with
+    ``MatmulOp`` keep their JSON form: the reloaded graph lowers to the same kernels, name for name."""
+    import json
+    from pathlib import Path
+
+    import torch
+    from torch import nn
+
+    from deplodock_amd import HipBackend, serialize, trace_module
+    from deplodock_amd.ingest import load_reference_graph
+    from deplodock_amd.ir.hip import HipOp
+
+    class Mm(nn.Module):
+        def forward(self, a, b):
+            return a @ b
+
+    def kernels(g):
+        return [n.op.kernel_name for n in HipBackend().compile(g).nodes.values() if isinstance(n.op, HipOp)]
+
+    corpus = Path(__file__).parent / "golden" / "loop_ir"
+    graphs = [load_reference_graph(corpus / f"{k}.json") for k in ("k_mul_1_reduce", "k_scaled_dot_product_attention_masked_reduce", "k_add_3_reduce")]
+    graphs.append(trace_module(Mm().eval(), (torch.randn(4, 8, 16), torch.randn(16, 12))))
+    for g in graphs:
+        again = serialize.graph_from_dict(json.loads(json.dumps(serialize.graph_to_dict(g))))
+        assert kernels(again) == kernels(g)
+    with pytest.raises(serialize.SerializeError, match="unknown Loop-IR statement"):
+        serialize._dec({"$loop": ["Exec", "x"]})
