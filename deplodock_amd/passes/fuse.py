@@ -1084,7 +1084,14 @@ def _rec_pointwise(c: _Ctx, nid: str) -> bool:
         elif len(v.shape) == len(shape) and v.shape[:-1] == shape[:-1] and v.shape[-1] == 1 and View(v.base, v.offset, v.shape[:-1], v.strides[:-1], v.dtype).is_contiguous():
             kind = "row"
         else:
-            raise FusionError(f"pointwise operand {leaf_id!r} of {nid!r} needs general broadcasting (shape {v.shape} strides {v.strides} into {shape})")
+            # general broadcasting (e.g. a [1, 1, S, S] mask into [B, H, S, S]), or a strided operand: the operand is
+            # first written out densely in the result's shape by a copy nest (repeated axes read with stride 0)
+            pad = len(shape) - len(v.shape)
+            if pad < 0 or any(n not in (1, full) for n, full in zip(v.shape, shape[pad:])):
+                raise FusionError(f"pointwise operand {leaf_id!r} of {nid!r} does not broadcast (shape {v.shape} into {shape})")
+            wide = View(v.base, v.offset, shape, (0,) * pad + tuple(0 if n == 1 and full != 1 else st for n, st, full in zip(v.shape, v.strides, shape[pad:])), v.dtype)
+            v = _copy_of_view(c, wide, tuple(range(len(shape))), f"{nid}__b{len(operands)}")
+            kind = "flat"
         operands.append(MapOperand(var.name, v.dtype, kind))
         buffers[var.name] = v.base
         offsets[var.name] = v.offset
@@ -1108,7 +1115,10 @@ def fuse(g: Graph) -> Graph:
     """Lower a frontend ``Graph`` to ``Graph[TileOp + InputOp + ConstantOp]``."""
     from deplodock_amd.passes.raise_loops import raise_loop_nests
 
+    from deplodock_amd.passes.raise_attention import raise_attention
+
     g = raise_loop_nests(g)  # Loop-IR kernels that are a contraction / a row normalisation become frontend ops first
+    g = raise_attention(g)  # softmax(q @ k^T * scale [+ mask]) @ v spelled with matmuls becomes the fused op
     out = Graph()
     out.constant_values = dict(getattr(g, "constant_values", {}))
     c = _Ctx(g=g, out=out)

@@ -1129,7 +1129,10 @@ def test_matmul_spelled_attention(device, dtype, seq):
     be = HipBackend()
     compiled = be.compile(trace_module(mod, (q, k, v)))
     names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
-    assert names.count("k_matmul") == 2 and names.count("k_gather") == (1 if seq % 8 == 0 else 2) and "k_softmax_reduce" in names
+    if dtype is torch.bfloat16:
+        assert names == ["k_sdpa_reduce"]  # 16-bit: raised to the fused kernel
+    else:
+        assert names.count("k_matmul") == 2 and names.count("k_gather") == (1 if seq % 8 == 0 else 2) and "k_softmax_reduce" in names
     prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in (q, k, v)))))
     try:
         prog.run()
@@ -1159,3 +1162,43 @@ def test_plain_matmul(device, shape_a, shape_b):
         prog.close()
     want = (a.double() @ b.double()).float()
     eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-4 * float(want.pow(2).mean().sqrt()), f"matmul {shape_a} @ {shape_b}")
+
+
+class _EagerMaskedAttention(nn.Module):
+    def forward(self, q, k, v, mask):
+        s = torch.matmul(q, k.transpose(-1, -2)) / float(q.shape[-1]) ** 0.5 + mask
+        return torch.softmax(s, -1) @ v
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("masked", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_matmul_spelled_attention_is_raised_to_the_fused_kernel(device, dtype, masked):
+    """16-bit ``softmax(q @ k.T * scale [+ mask]) @ v`` becomes one attention kernel (what the reference reaches by
+    decomposing the fused op and finding the streaming form again); fp32 keeps its matmuls — and a ``[1, 1, S, S]``
+    mask broadcast into ``[B, H, S, S]`` goes through a dense copy."""
+    torch.manual_seed(33)
+    q, k, v = (torch.randn(2, 4, 200, 128).to(dtype) for _ in range(3))
+    args = [q, k, v]
+    mod = _EagerAttention().eval()
+    if masked:
+        args.append(causal_mask := torch.zeros(1, 1, 200, 200).masked_fill(torch.arange(200)[None, :] > torch.arange(200)[:, None], float("-inf")).to(dtype))
+        mod = _EagerMaskedAttention().eval()
+        assert causal_mask.shape == (1, 1, 200, 200)
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, tuple(args)))
+    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    if dtype is torch.bfloat16:
+        assert names == ["k_sdpa_reduce"]
+    else:
+        assert names.count("k_matmul") == 2 and "k_sdpa_reduce" not in names
+    prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in args))))
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = mod(*(t.double() for t in args)).float()
+    tol = (2e-2, 2e-2) if dtype is torch.bfloat16 else (1e-4, 1e-5)
+    eager.assert_close(ours.reshape(want.shape), want, *tol, f"matmul-spelled attention {dtype} masked={masked}")

@@ -516,7 +516,7 @@ def test_matmul_spelled_attention_lowers_to_batched_contractions(launcher_lib):
         def forward(self, q, k, v):
             return torch.softmax(torch.matmul(q, k.transpose(-1, -2)) * 0.125, -1) @ v
 
-    q = torch.randn(2, 4, 104, 64).bfloat16()
+    q = torch.randn(2, 4, 104, 64)  # (fp32: 16-bit operands are raised to the fused attention kernel instead)
     traced = trace_module(Attn().eval(), (q, q.clone(), q.clone()))
     assert sum(isinstance(n.op, F.MatmulOp) for n in traced.nodes.values()) == 2
     compiled = HipBackend().compile(traced)
@@ -525,9 +525,13 @@ def test_matmul_spelled_attention_lowers_to_batched_contractions(launcher_lib):
     assert [k.grid[1] for k in ks if k.kernel_name.startswith("k_matmul")] == [(8,), (8,)]
     for k in ks:
         hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+    # 16-bit operands: the same module is one attention kernel
+    qb = torch.randn(2, 4, 104, 64).bfloat16()
+    kb = [n.op.kernel_name.rsplit("_", 1)[0] for n in HipBackend().compile(trace_module(Attn().eval(), (qb, qb.clone(), qb.clone()))).nodes.values() if isinstance(n.op, HipOp)]
+    assert kb == ["k_sdpa_reduce"]
     # a key count that is not whole 16-byte chunks: the second product's operands are copied with their reduction axis
     # padded with zeros (both, so that nothing undefined meets a zero)
-    q = torch.randn(2, 4, 100, 64).bfloat16()
+    q = torch.randn(2, 4, 100, 64)
     ks = [n.op for n in HipBackend().compile(trace_module(Attn().eval(), (q, q.clone(), q.clone()))).nodes.values() if isinstance(n.op, HipOp)]
     assert [k.kernel_name.rsplit("_", 1)[0] for k in ks] == ["k_matmul", "k_pointwise_elementwise", "k_softmax_reduce", "k_gather", "k_gather", "k_matmul"]
     assert "K=104" in ks[-1].comment
