@@ -1,0 +1,170 @@
+"""Attention outside the flash kernel's reach is decomposed into loop nests before fusion.
+
+The flash kernel serves 16-bit operands with head_dim 64 / 128 / 256.  The reference compiles fp32 only and its
+perf cases call ``F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=...)`` on fp32 tensors
+(tests/perf/cases.py:64-69, 174-190); it lowers the fused op by decomposing it into ``q k^T -> * scale -> [+ mask] ->
+softmax -> @ v`` (emmy/compiler/pipeline/passes/frontend/decomposition/010_sdpa.py:53-138: grouped KV heads by
+``head // group`` indexing, a causal mask as ``+ (-1e9)`` where ``key > query``), which its loop fusion turns into
+two kernels: the masked scores, and softmax times ``v``.
+
+Here an ``SdpaOp`` the flash kernel does not take is rewritten into those same two kernels, written as Loop-IR
+statements (``LoopNestOp``): the loop-nest raiser then makes each a batched MFMA contraction with loop-nest operand
+and output stages, exactly as it does for the reference's own two attention kernels of its on-disk corpus.
+"""
+
+from __future__ import annotations
+
+import math
+
+from deplodock_amd.graph import Graph, Node, Tensor
+from deplodock_amd.ir import frontend as F
+from deplodock_amd.ir import loopnest as L
+
+FLASH_HEAD_DIMS = (64, 128, 256)
+
+
+class AttentionShapeError(ValueError):
+    pass
+
+
+def _static(shape) -> tuple[int, ...]:
+    if not all(isinstance(d, int) for d in shape):
+        raise AttentionShapeError("attention outside the flash kernel (fp32, or a head_dim other than 64 / 128 / 256) needs static shapes")
+    return tuple(int(d) for d in shape)
+
+
+def _wrap(axes: list[tuple[str, int]], body: tuple) -> tuple:
+    for name, extent in reversed(axes):
+        body = (L.Loop(name, extent, tuple(body)),)
+    return tuple(body)
+
+
+def _aligned_index(shape: tuple[int, ...], lead_vars: list[L.Var], lead_shape: tuple[int, ...], tail: tuple, what: str) -> tuple:
+    """Index of an operand whose dims before its last ``len(tail)`` line up, from the right, with q's leading dims
+    (each equal to q's, or 1 and then read at 0)."""
+    nlead = len(shape) - len(tail)
+    if nlead > len(lead_vars):
+        raise AttentionShapeError(f"sdpa: {what} has more leading dims than q")
+    idx = []
+    for d, var, full in zip(shape[:nlead], lead_vars[len(lead_vars) - nlead :], lead_shape[len(lead_shape) - nlead :]):
+        if d == full:
+            idx.append(var if full > 1 else L.Lit(0))
+        elif d == 1:
+            idx.append(L.Lit(0))
+        else:
+            raise AttentionShapeError(f"sdpa: {what} dim {d} does not match q's {full}")
+    return (*idx, *tail)
+
+
+def _decompose(g: Graph, node: Node, undo_repeat) -> list[Node]:
+    op: F.SdpaOp = node.op
+    nid = node.id
+    q_id, k_id, v_id = node.inputs[:3]
+    (k_src, k_rep), (v_src, v_rep) = undo_repeat(g, k_id), undo_repeat(g, v_id)
+    if k_rep == v_rep and k_rep > 1:
+        k_id, v_id = k_src, v_src  # the materialised repeat is the ``head // group`` indexing below
+    q, k, v = (_static(g.nodes[i].output.shape) for i in (q_id, k_id, v_id))
+    if min(len(q), len(k), len(v)) < 3:
+        raise AttentionShapeError("sdpa: expected [batch..., heads, seq, head_dim] operands")
+    hq, sq, d = q[-3:]
+    hkv, skv = k[-3], k[-2]
+    dv = v[-1]
+    if k[-1] != d or v[-3] != hkv or v[-2] != skv:
+        raise AttentionShapeError(f"sdpa: operands {q} / {k} / {v} do not fit together")
+    if hq != hkv and not (op.enable_gqa or k_rep > 1):
+        raise AttentionShapeError("sdpa: grouped heads need enable_gqa=True")
+    if hq % hkv:
+        raise AttentionShapeError("sdpa: q heads must be a multiple of kv heads")
+    group = hq // hkv
+    lead = q[:-3]
+    dtype = node.output.dtype
+    scale = float(op.scale) if op.scale is not None else 1.0 / math.sqrt(d)
+
+    lead_vars = [L.Var(f"b{i}") for i in range(len(lead))]
+    lead_axes = [(var.name, n) for var, n in zip(lead_vars, lead) if n > 1]  # unit dims are read at 0, with no loop
+    lead_idx = tuple(var if n > 1 else L.Lit(0) for var, n in zip(lead_vars, lead))
+    h, i, j, dd = L.Var("h"), L.Var("i"), L.Var("j"), L.Var("d")
+    kv_head = L.Bin("/", h, L.Lit(group)) if group > 1 else h
+
+    # kernel 1: scores[..., h, i, j] = sum_d q[..., h, i, d] * k[..., h / group, j, d] * scale (+ mask)
+    scores_id = f"{nid}__scores"
+    scores_shape = (*lead, hq, sq, skv)
+    head = [L.Load("c_scale", "scale", (L.Lit(0),))]
+    scalars = {"scale": scale}
+    loads, inputs = ["q", "k"], [q_id, k_id]
+    post = [L.Assign("scaled", "multiply", ("acc", "c_scale"))]
+    value = "scaled"
+    if op.has_mask:
+        m_id = node.inputs[3]
+        m = _static(g.nodes[m_id].output.shape)
+        if len(m) < 2 or m[-1] not in (1, skv) or m[-2] not in (1, sq):
+            raise AttentionShapeError(f"sdpa: the mask {m} must broadcast to [..., queries, keys]")
+        tail = (i if m[-2] > 1 else L.Lit(0), j if m[-1] > 1 else L.Lit(0))
+        m_idx = _aligned_index(m, [*lead_vars, h], (*lead, hq), tail, "the mask")
+        post = [L.Load("bias", "mask", m_idx), *post, L.Assign("masked", "add", ("scaled", "bias"))]
+        loads.append("mask")
+        inputs.append(m_id)
+        value = "masked"
+    elif op.is_causal:
+        head += [L.Load("c_zero", "mask_zero", (L.Lit(0),)), L.Load("c_fill", "mask_fill", (L.Lit(0),))]
+        scalars.update(mask_zero=0.0, mask_fill=-1e9)
+        post = [L.Select("bias", (("c_zero", L.Bin("<=", j, i)), ("c_fill", L.Bin(">", j, i)))), *post, L.Assign("masked", "add", ("scaled", "bias"))]
+        value = "masked"
+    k_loop = L.Loop("d", d, (
+        L.Load("qv", "q", (*lead_idx, h, i, dd)),
+        L.Load("kv", "k", _aligned_index(k, lead_vars, lead, (kv_head, j, dd), "k")),
+        L.Assign("prod", "multiply", ("qv", "kv")),
+        L.Accum("acc", "prod", "add"),
+    ))  # fmt: skip
+    body1 = _wrap([*lead_axes, ("h", hq), ("i", sq), ("j", skv)], (k_loop, *post, L.Write(scores_id, (*lead_idx, h, i, j), value)))
+    n1 = Node(scores_id, F.LoopNestOp(stmts=(*head, *body1), loads=tuple(loads), scalars=scalars, out_name=scores_id, label="sdpa_scores"),
+              inputs, Tensor(scores_id, scores_shape, dtype))  # fmt: skip
+
+    # kernel 2: out[..., h, i, e] = sum_j exp(s[j] - max_j s) / sum_j exp(s[j] - max_j s) * v[..., h / group, j, e]
+    s_idx = (*lead_idx, h, i, j)
+    e = L.Var("e")
+    fold_max = L.Loop("j", skv, (L.Load("s0", "scores", s_idx), L.Accum("row_max", "s0", "maximum")))
+    fold_sum = L.Loop("j", skv, (L.Load("s1", "scores", s_idx), L.Assign("c1", "subtract", ("s1", "row_max")), L.Assign("e1", "exp", ("c1",)), L.Accum("row_sum", "e1", "add")))
+    pv = L.Loop("j", skv, (
+        L.Load("s2", "scores", s_idx),
+        L.Assign("c2", "subtract", ("s2", "row_max")),
+        L.Assign("e2", "exp", ("c2",)),
+        L.Load("vv", "v", _aligned_index(v, lead_vars, lead, (kv_head, j, e), "v")),
+        L.Assign("p", "divide", ("e2", "row_sum")),
+        L.Assign("pv", "multiply", ("p", "vv")),
+        L.Accum("o", "pv", "add"),
+    ))  # fmt: skip
+    body2 = _wrap([*lead_axes, ("h", hq), ("i", sq)], (fold_max, fold_sum, L.Loop("e", dv, (pv, L.Write(nid, (*lead_idx, h, i, e), "o")))))
+    n2 = Node(nid, F.LoopNestOp(stmts=body2, loads=("scores", "v"), scalars={}, out_name=nid, label="sdpa_softmax_v"), [scores_id, v_id], node.output)
+    return [n1, n2]
+
+
+def decompose_attention(g: Graph, undo_repeat) -> Graph:
+    """``g`` with every ``SdpaOp`` the flash kernel does not take (operands wider than 16 bits, or a head_dim it has
+    no tiling for) replaced by the two loop nests of the decomposed form; a new graph when anything changed.
+    ``undo_repeat(g, node id) -> (source id, group)`` sees through a materialised head repeat."""
+
+    def flash_takes(node: Node) -> bool:
+        t = g.nodes[node.inputs[0]].output
+        return t.dtype.name in ("bf16", "f16") and t.shape[-1] in FLASH_HEAD_DIMS
+
+    hits = [nid for nid, n in g.nodes.items() if isinstance(n.op, F.SdpaOp) and not flash_takes(n)]
+    if not hits:
+        return g
+    out = Graph()
+    for attr, value in vars(g).items():
+        if attr != "nodes":
+            setattr(out, attr, value)
+    out.nodes = {}
+    for nid, node in g.nodes.items():
+        if nid not in hits:
+            out.nodes[nid] = node
+            continue
+        for n in _decompose(g, node, undo_repeat):
+            if n.id in out.nodes or (n.id in g.nodes and n.id != nid):
+                raise ValueError(f"decomposed node id {n.id!r} is taken")
+            out.nodes[n.id] = n
+    return out
+
+
+__all__ = ["decompose_attention", "AttentionShapeError"]

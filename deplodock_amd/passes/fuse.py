@@ -65,6 +65,7 @@ class _Ctx:
     # frontend node id -> (offset, shape, strides) of its value inside ``done[id]``
     # when it is a window of a wider buffer (column slice of a merged projection)
     windows: dict[str, tuple[int, tuple[int, ...], tuple[int, ...]]] = field(default_factory=dict)
+    dense: dict[str, View] = field(default_factory=dict)  # layout node id -> its value after a dense copy made it expressible
 
     def kname(self, label: str) -> str:
         """Kernel label; the lowering appends a hash of the rendered body, so
@@ -118,7 +119,18 @@ def _need(c: _Ctx, nid: str) -> View:
         shape = tuple(int(d) for d in g.nodes[cur].output.shape)
         v = View(base, 0, shape, contiguous_strides(shape), g.nodes[cur].output.dtype)
     for lid in reversed(chain):
-        v = apply_layout(v, g.nodes[lid].op, tuple(int(d) for d in g.nodes[lid].output.shape), lid)
+        if lid in c.dense:
+            v = c.dense[lid]
+            continue
+        try:
+            v = apply_layout(v, g.nodes[lid].op, tuple(int(d) for d in g.nodes[lid].output.shape), lid)
+        except NotViewable:
+            # e.g. ``x.transpose(1, 2).reshape(...)``: no strides express it, so the view so far is written out
+            # densely by a copy nest (what torch's reshape does) and the layout op applies to the copy
+            if not all(isinstance(d, int) for d in (*v.shape, *v.strides, v.offset)):
+                raise
+            dense = _copy_of_view(c, v, tuple(range(len(v.shape))), f"{lid}__dense")
+            v = c.dense[lid] = apply_layout(dense, g.nodes[lid].op, tuple(int(d) for d in g.nodes[lid].output.shape), lid)
     return v
 
 
@@ -148,17 +160,43 @@ def _rec_loop_nest(c: _Ctx, nid: str) -> bool:
         return False
     from deplodock_amd.ir.tile import LoopNest
 
+    from deplodock_amd.ir import loopnest as L
+
     operands: dict = {}
     inputs: list[str] = []
+    strided: dict[str, View] = {}
     for load_name, src in zip(node.op.loads, node.inputs):
         shape = tuple(int(d) for d in c.g.nodes[src].output.shape)
         v = _need_logical(c, src)
-        if not ((v.offset == 0 and v.shape == shape and v.is_contiguous()) or _same_memory(v, shape)):
-            raise FusionError(f"loop nest {nid!r}: operand {src!r} is a strided view; a copy kernel is not implemented")
-        operands[load_name] = (v.base, shape, c.g.nodes[src].output.dtype)
+        if (v.offset == 0 and v.shape == shape and v.is_contiguous()) or _same_memory(v, shape):
+            operands[load_name] = (v.base, shape, c.g.nodes[src].output.dtype)
+        else:
+            # a strided view: the buffer is indexed flat and every Load of it computes offset + sum(index * stride)
+            if tuple(int(d) for d in v.shape) != shape:
+                raise FusionError(f"loop nest {nid!r}: operand {src!r} is a view of shape {v.shape}, recorded as {shape}")
+            operands[load_name] = (v.base, (int(c.out.nodes[v.base].output.numel),), c.g.nodes[src].output.dtype)
+            strided[load_name] = v
         inputs.append(v.base)
+
+    def flat(stmts: tuple) -> tuple:
+        res = []
+        for s in stmts:
+            if isinstance(s, L.Loop):
+                s = L.Loop(s.axis, s.extent, flat(s.body))
+            elif isinstance(s, L.Load) and s.input in strided:
+                v = strided[s.input]
+                if len(s.index) != len(v.strides):
+                    raise FusionError(f"loop nest {nid!r}: load of {s.input!r} has {len(s.index)} indices for a rank-{len(v.strides)} operand")
+                at: object = L.Lit(int(v.offset))
+                for e, st in zip(s.index, v.strides):
+                    if st and not (isinstance(e, L.Lit) and e.value == 0):
+                        at = L.Bin("+", at, L.Bin("*", e, L.Lit(int(st))))
+                s = L.Load(s.name, s.input, (at,))
+            res.append(s)
+        return tuple(res)
+
     t = node.output
-    body = LoopNest(stmts=node.op.stmts, operands=operands, scalars=dict(node.op.scalars or {}), out=nid, out_name=node.op.out_name or nid,
+    body = LoopNest(stmts=flat(node.op.stmts) if strided else node.op.stmts, operands=operands, scalars=dict(node.op.scalars or {}), out=nid, out_name=node.op.out_name or nid,
                     out_shape=tuple(int(d) for d in t.shape), out_dtype=t.dtype)  # fmt: skip
     label = node.op.label or "".join(ch if ch.isalnum() else "_" for ch in nid)[-40:].lstrip("_")
     _emit(c, nid, body, label, inputs)
@@ -265,52 +303,90 @@ def _rec_batched_linear(c: _Ctx, nid: str) -> bool:
     x, w = _need(c, node.inputs[0]), _need(c, node.inputs[1])
     if len(x.shape) != 3 or len(w.shape) != 3 or x.shape[2] != w.shape[2] or w.shape[0] not in (1, x.shape[0]):
         raise FusionError(f"batched linear {nid!r}: operands {x.shape} x {w.shape} are not [P, M, K] x [P | 1, N, K]")
-    if x.strides[2] != 1 or w.strides[2] != 1:
-        raise FusionError(f"batched linear {nid!r}: the reduction axis must be contiguous in both operands")
-    p, m, k = (int(d) for d in x.shape)
-    n = int(w.shape[1])
-    body = Contraction(
-        m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=int(x.strides[1]) if m > 1 else k, ldb=int(w.strides[1]) if n > 1 else k,
-        a_offset=x.offset, b_offset=w.offset, batch=p, a_batch=int(x.strides[0]) if p > 1 else 0, b_batch=int(w.strides[0]) if w.shape[0] > 1 else 0, out_batch=m * n,
-    )  # fmt: skip
-    _emit(c, nid, body, "batched_linear", [x.base, w.base], shape=(p, m, n))
+    _emit_batched_contraction(c, nid, x, w, "batched_linear")
     return True
 
 
-def _copy_of_view(c: _Ctx, v: View, order: tuple[int, ...], new_id: str, pad_last_to: int | None = None) -> View:
+def _copy_of_view(c: _Ctx, v: View, order: tuple[int, ...], new_id: str, pad_last_to: int | None = None, pad_rows_to: int | None = None) -> View:
     """A dense row-major copy of ``v`` with its axes in ``order``, made by a loop nest of its own (``new_id``): what a
     contraction needs when an operand's reduction axis is not the contiguous one, or its leading axes are not one
-    uniformly strided run."""
+    uniformly strided run.  The last axis (``pad_last_to``) and the one before it (``pad_rows_to``) can be extended
+    with zeros."""
     from deplodock_amd.ir import loopnest as L
     from deplodock_amd.ir.tile import LoopNest
 
     numel = c.out.nodes[v.base].output.numel
     axes = [f"c{i}" for i in range(len(v.shape))]
-    last = order[-1]
     extent = {i: int(v.shape[i]) for i in order}
-    padded = pad_last_to is not None and pad_last_to > extent[last]
+    pads = {}  # source axis -> padded extent
+    if pad_last_to is not None and pad_last_to > extent[order[-1]]:
+        pads[order[-1]] = int(pad_last_to)
+    if pad_rows_to is not None and len(order) > 1 and pad_rows_to > extent[order[-2]]:
+        pads[order[-2]] = int(pad_rows_to)
 
     def ax(i: int):
-        # a padded last axis runs past the source: its index is clamped (the value read there is replaced by zero)
-        return L.Ternary(L.Bin("<", L.Var(axes[i]), L.Lit(extent[i])), L.Var(axes[i]), L.Lit(0)) if padded and i == last else L.Var(axes[i])
+        # a padded axis runs past the source: its index is clamped (the value read there is replaced by zero)
+        return L.Ternary(L.Bin("<", L.Var(axes[i]), L.Lit(extent[i])), L.Var(axes[i]), L.Lit(0)) if i in pads else L.Var(axes[i])
 
     flat: object = L.Lit(int(v.offset))
     for i, st in enumerate(v.strides):
         if st:
             flat = L.Bin("+", flat, L.Bin("*", ax(i), L.Lit(int(st))))
-    if padded:
-        body: tuple = (L.Load("t", "src", (flat,)), L.Load("z", "zero", (L.Lit(0),)),
-                       L.Select("u", (("t", L.Bin("<", L.Var(axes[last]), L.Lit(extent[last]))), ("z", L.Lit(1)))),
+    if pads:
+        inside: object = None
+        for i in pads:
+            here = L.Bin("<", L.Var(axes[i]), L.Lit(extent[i]))
+            inside = here if inside is None else L.Bin("&&", inside, here)
+        body: tuple = (L.Load("t", "src", (flat,)), L.Load("z", "zero", (L.Lit(0),)), L.Select("u", (("t", inside), ("z", L.Lit(1)))),
                        L.Write(new_id, tuple(L.Var(axes[i]) for i in order), "u"))  # fmt: skip
-        extent[last] = int(pad_last_to)
     else:
         body = (L.Load("t", "src", (flat,)), L.Write(new_id, tuple(L.Var(axes[i]) for i in order), "t"))
     for i in reversed(order):
-        body = (L.Loop(axes[i], extent[i], body),)
-    shape = tuple(extent[i] for i in order)
-    nest = LoopNest(stmts=body, operands={"src": (v.base, (int(numel),), v.dtype)}, scalars={"zero": 0.0} if padded else {}, out=new_id, out_name=new_id, out_shape=shape, out_dtype=v.dtype)
+        body = (L.Loop(axes[i], pads.get(i, extent[i]), body),)
+    shape = tuple(pads.get(i, extent[i]) for i in order)
+    nest = LoopNest(stmts=body, operands={"src": (v.base, (int(numel),), v.dtype)}, scalars={"zero": 0.0} if pads else {}, out=new_id, out_name=new_id, out_shape=shape, out_dtype=v.dtype)
     c.out.add_node(TileOp(name=c.kname("gather"), body=nest), [v.base], Tensor(new_id, shape, v.dtype), new_id)
     return View(new_id, 0, shape, contiguous_strides(shape), v.dtype)
+
+
+def _emit_batched_contraction(c: _Ctx, nid: str, a: View, b: View, label: str) -> None:
+    """``a [..., M, K] x b [... | 1..., N, K] -> [..., M, N]`` as one launch with a workgroup row per product.  The
+    kernel reads whole 16-byte chunks along ``K`` and stores runs of four columns: an operand that is not laid out
+    for that (reduction axis not contiguous, leading axes not one uniformly strided run, misaligned) is copied
+    first; a ragged ``K`` is padded with zeros in both operands; a ragged ``N`` is padded in ``b`` and the result
+    is a window of a wider buffer."""
+    node = c.g.nodes[nid]
+    m, k, n = int(a.shape[-2]), int(a.shape[-1]), int(b.shape[-2])
+    lead = tuple(int(d) for d in a.shape[:-2])
+    p = 1
+    for d in lead:
+        p *= d
+    shared = all(int(d) == 1 for d in b.shape[:-2])
+    if not shared and tuple(int(d) for d in b.shape[:-2]) != lead:
+        raise FusionError(f"{label} {nid!r}: leading axes {a.shape[:-2]} and {b.shape[:-2]} differ")
+    if a.dtype != b.dtype:
+        raise FusionError(f"{label} {nid!r}: operand types differ")
+    kp, n_pad = -(-k // 8) * 8, -(-n // 4) * 4
+    nb = a.dtype.nbytes
+
+    def unfit(v: View, rows: int) -> bool:
+        return v.strides[-1] != 1 and k > 1 or v.collapse_leading(2) is None or (v.offset * nb) % 16 != 0 or (rows > 1 and (v.strides[-2] * nb) % 16 != 0)
+
+    if kp != k or unfit(a, m):
+        a = _copy_of_view(c, a, tuple(range(len(a.shape))), f"{nid}__a", pad_last_to=kp)
+    if kp != k or n_pad != n or unfit(b, n):
+        b = _copy_of_view(c, b, tuple(range(len(b.shape))), f"{nid}__b", pad_last_to=kp, pad_rows_to=n_pad)
+    pa, sa = a.collapse_leading(2)
+    pb, sb = b.collapse_leading(2)
+    if (pa > 1 and (sa * nb) % 16) or (pb > 1 and (sb * nb) % 16):
+        raise FusionError(f"{label} {nid!r}: batch strides break 16-byte alignment")
+    body = Contraction(
+        m=m, n=n_pad, k=kp, a=a.base, b=b.base, out=nid, in_dtype=a.dtype, out_dtype=node.output.dtype, lda=int(a.strides[-2]) if m > 1 else kp, ldb=int(b.strides[-2]) if n_pad > 1 else kp,
+        a_offset=a.offset, b_offset=b.offset, batch=p, a_batch=int(sa) if p > 1 else 0, b_batch=0 if shared or p == 1 else int(sb), out_batch=m * n_pad,
+    )  # fmt: skip
+    _emit(c, nid, body, label, [a.base, b.base], shape=(*lead, m, n_pad))
+    if n_pad != n:
+        c.windows[nid] = (0, (*lead, m, n), contiguous_strides((*lead, m, n_pad)))
 
 
 def _rec_matmul(c: _Ctx, nid: str) -> bool:
@@ -323,37 +399,12 @@ def _rec_matmul(c: _Ctx, nid: str) -> bool:
     a, b = _need(c, node.inputs[0]), _need(c, node.inputs[1])
     if len(a.shape) < 2 or len(b.shape) < 2 or a.shape[-1] != b.shape[-2]:
         raise FusionError(f"matmul {nid!r}: operands {a.shape} @ {b.shape}")
-    m, k, n = int(a.shape[-2]), int(a.shape[-1]), int(b.shape[-1])
-    lead = tuple(int(d) for d in a.shape[:-2])
-    p = 1
-    for d in lead:
-        p *= d
-    shared = len(b.shape) == 2 or all(int(d) == 1 for d in b.shape[:-2])
-    if not shared and tuple(int(d) for d in b.shape[:-2]) != lead:
-        raise FusionError(f"matmul {nid!r}: leading axes {a.shape[:-2]} and {b.shape[:-2]} differ")
-    if a.dtype != b.dtype:
-        raise FusionError(f"matmul {nid!r}: operand types differ")
-    kp = -(-k // 8) * 8  # the contraction reads whole 16-byte chunks and MFMA steps: a ragged reduction extent is padded with zeros in both operands
-    ra = len(a.shape)
-    if kp != k or a.strides[-1] != 1 and k > 1 or a.collapse_leading(2) is None or (a.offset * a.dtype.nbytes) % 16 or (m > 1 and (a.strides[-2] * a.dtype.nbytes) % 16):
-        a = _copy_of_view(c, a, tuple(range(ra)), f"{nid}__a", pad_last_to=kp)
     rb = len(b.shape)
     order_b = (*range(rb - 2), rb - 1, rb - 2)  # [..., N, K]
-    if kp != k or b.strides[-2] != 1 and k > 1 or b.collapse_leading(2) is None or (b.offset * b.dtype.nbytes) % 16 or (n > 1 and (b.strides[-1] * b.dtype.nbytes) % 16):
-        b = _copy_of_view(c, b, order_b, f"{nid}__bt", pad_last_to=kp)
-    else:
-        b = View(b.base, b.offset, tuple(b.shape[i] for i in order_b), tuple(b.strides[i] for i in order_b), b.dtype)
-    pa, sa = a.collapse_leading(2)
-    pb, sb = b.collapse_leading(2)
-    if n % 4:
-        raise FusionError(f"matmul {nid!r}: {n} output columns are not whole runs of four (the contraction stores such runs)")
-    if (pa > 1 and (sa * a.dtype.nbytes) % 16) or (pb > 1 and (sb * b.dtype.nbytes) % 16):
-        raise FusionError(f"matmul {nid!r}: batch strides break 16-byte alignment")
-    body = Contraction(
-        m=m, n=n, k=kp, a=a.base, b=b.base, out=nid, in_dtype=a.dtype, out_dtype=node.output.dtype, lda=int(a.strides[-2]) if m > 1 else kp, ldb=int(b.strides[-2]) if n > 1 else kp,
-        a_offset=a.offset, b_offset=b.offset, batch=p, a_batch=int(sa) if p > 1 else 0, b_batch=0 if shared or p == 1 else int(sb), out_batch=m * n,
-    )  # fmt: skip
-    _emit(c, nid, body, "matmul", [a.base, b.base])
+    bt = View(b.base, b.offset, tuple(b.shape[i] for i in order_b), tuple(b.strides[i] for i in order_b), b.dtype)
+    if rb == 2 and len(a.shape) > 2:
+        bt = View(bt.base, bt.offset, (*(1,) * (len(a.shape) - 2), *bt.shape), (*(0,) * (len(a.shape) - 2), *bt.strides), bt.dtype)
+    _emit_batched_contraction(c, nid, a, bt, "matmul")
     return True
 
 
@@ -1113,10 +1164,14 @@ def _rec_pointwise(c: _Ctx, nid: str) -> bool:
 
 def fuse(g: Graph) -> Graph:
     """Lower a frontend ``Graph`` to ``Graph[TileOp + InputOp + ConstantOp]``."""
+    from deplodock_amd.passes.decompose_attention import AttentionShapeError, decompose_attention
+    from deplodock_amd.passes.raise_attention import raise_attention
     from deplodock_amd.passes.raise_loops import raise_loop_nests
 
-    from deplodock_amd.passes.raise_attention import raise_attention
-
+    try:
+        g = decompose_attention(g, _undo_repeat_kv)  # attention the flash kernel does not take (fp32, other head dims) becomes two loop nests
+    except AttentionShapeError as exc:
+        raise FusionError(str(exc)) from exc
     g = raise_loop_nests(g)  # Loop-IR kernels that are a contraction / a row normalisation become frontend ops first
     g = raise_attention(g)  # softmax(q @ k^T * scale [+ mask]) @ v spelled with matmuls becomes the fused op
     out = Graph()
@@ -1130,7 +1185,7 @@ def fuse(g: Graph) -> Graph:
         v = _need_logical(c, oid)
         shape = tuple(int(d) for d in g.nodes[oid].output.shape)
         if not (v.offset == 0 and v.shape == shape and v.is_contiguous()) and not _same_memory(v, shape):
-            raise FusionError(f"graph output {oid!r} is a strided view; a final copy kernel is not implemented")
+            v = _copy_of_view(c, v, tuple(range(len(v.shape))), f"{oid}__out")  # a strided view as a graph output: written out densely
         final_outputs.append(v.base)
         if v.base != oid:
             out.nodes[v.base].hints.setdefault("output_alias", []).append((oid, shape))

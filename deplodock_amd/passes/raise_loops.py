@@ -388,14 +388,31 @@ def _try_batched_contraction(g: Graph, node: Node) -> list[Node] | None:
         for d in pshape:
             p *= d
         bidx = tuple(L.Var(lp.axis) for lp in batch)
-        a_head = [s for s in head if s.name in _all_uses(a_stmts) | _all_uses(prefix)]
-        a_body = _wrap(batch + [lm], (*prefix, L.Loop(lk.axis, lk.extent, (*a_stmts, L.Write("", (*bidx, L.Var(lm.axis), L.Var(lk.axis)), u_name)))))
-        a_id = _nest_node(b, (*a_head, *a_body), (*pshape, lm.extent, lk.extent), "operand_a")
+        extents = {lp.axis: lp.extent for lp in (*batch, lm, ln, lk)}
+
+        def in_place(side_stmts: list, axes: list[str]) -> str | None:
+            """The graph tensor itself when the side is one plain load walking ``axes`` in order: no copy needed."""
+            if len(side_stmts) != 1 or not isinstance(side_stmts[0], L.Load) or side_stmts[0].input in (op.scalars or {}):
+                return None
+            try:
+                src = _source(node, side_stmts[0])
+                return src if _simple_index(side_stmts[0].index, b.shape_of(src), extents) == axes else None
+            except _NoMatch:
+                return None
+
+        baxes = [lp.axis for lp in batch]
+        a_id = in_place(a_stmts, [*baxes, lm.axis, lk.axis]) if not prefix else None
+        if a_id is None:
+            a_head = [s for s in head if s.name in _all_uses(a_stmts) | _all_uses(prefix)]
+            a_body = _wrap(batch + [lm], (*prefix, L.Loop(lk.axis, lk.extent, (*a_stmts, L.Write("", (*bidx, L.Var(lm.axis), L.Var(lk.axis)), u_name)))))
+            a_id = _nest_node(b, (*a_head, *a_body), (*pshape, lm.extent, lk.extent), "operand_a")
         b_batched = any(deps[s.name] & bvars for s in b_stmts)
-        b_loops = (batch if b_batched else []) + [ln]
-        b_head = [s for s in head if s.name in _all_uses(b_stmts)]
-        b_body = _wrap(b_loops, (L.Loop(lk.axis, lk.extent, (*b_stmts, L.Write("", (*(bidx if b_batched else ()), L.Var(ln.axis), L.Var(lk.axis)), v_name))),))
-        b_id = _nest_node(b, (*b_head, *b_body), (*(pshape if b_batched else ()), ln.extent, lk.extent), "operand_b")
+        b_id = in_place(b_stmts, [*(baxes if b_batched else []), ln.axis, lk.axis])
+        if b_id is None:
+            b_loops = (batch if b_batched else []) + [ln]
+            b_head = [s for s in head if s.name in _all_uses(b_stmts)]
+            b_body = _wrap(b_loops, (L.Loop(lk.axis, lk.extent, (*b_stmts, L.Write("", (*(bidx if b_batched else ()), L.Var(ln.axis), L.Var(lk.axis)), v_name))),))
+            b_id = _nest_node(b, (*b_head, *b_body), (*(pshape if b_batched else ()), ln.extent, lk.extent), "operand_b")
         x3 = b.view(a_id, (p, lm.extent, lk.extent))
         w3 = b.view(b_id, (p if b_batched else 1, ln.extent, lk.extent))
         t3 = b.add(F.BatchedLinearOp(), [x3, w3], (p, lm.extent, ln.extent))

@@ -1,0 +1,106 @@
+"""Attention the flash kernel does not take (fp32 operands, other head dims) is decomposed into the two loop nests
+the reference's own pipeline reaches (masked scores; softmax times v).  Pinned on the host: the two nests,
+evaluated by the Loop-IR restatement in float64, equal ``F.scaled_dot_product_attention`` in float64 — a wrong
+head-group index, mask predicate, scale or broadcast is an error of order one."""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as Fn
+from torch import nn
+
+from deplodock_amd import HipBackend, trace_module
+from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir import frontend as F
+from deplodock_amd.passes.decompose_attention import decompose_attention
+from deplodock_amd.passes.fuse import FusionError, _undo_repeat_kv
+from oracle import loop_ir
+
+
+class _Sdpa(nn.Module):
+    def __init__(self, **kw):
+        super().__init__()
+        self.kw = kw
+
+    def forward(self, q, k, v, mask=None):
+        return Fn.scaled_dot_product_attention(q, k, v, attn_mask=mask, **self.kw)
+
+
+class _RepeatedKv(nn.Module):
+    """Grouped heads the materialising way (``repeat_kv`` of the Llama family)."""
+
+    def forward(self, q, k, v):
+        b, h, s, d = k.shape
+        g = q.shape[1] // h
+        k = k[:, :, None].expand(b, h, g, s, d).reshape(b, h * g, s, d)
+        v = v[:, :, None].expand(b, h, g, s, d).reshape(b, h * g, s, d)
+        return Fn.scaled_dot_product_attention(q, k, v, is_causal=True)
+
+
+def _causal_bias(sq, skv):
+    return torch.zeros(sq, skv).masked_fill(torch.arange(skv)[None, :] > torch.arange(sq)[:, None], float("-inf"))
+
+
+CASES = {
+    "causal_gqa": (_Sdpa(is_causal=True, enable_gqa=True), [(1, 4, 12, 8), (1, 2, 12, 8), (1, 2, 12, 8)], None),
+    "plain_batch2": (_Sdpa(), [(2, 3, 9, 8), (2, 3, 9, 8), (2, 3, 9, 8)], None),
+    "cross_lengths_scale": (_Sdpa(scale=0.3), [(2, 2, 5, 4), (2, 2, 11, 4), (2, 2, 11, 6)], None),
+    "mask_1_1_s_s": (_Sdpa(), [(2, 3, 7, 4), (2, 3, 7, 4), (2, 3, 7, 4)], lambda: _causal_bias(7, 7)[None, None]),
+    "mask_b_1_1_s": (_Sdpa(enable_gqa=True), [(2, 4, 6, 4), (2, 2, 10, 4), (2, 2, 10, 4)], lambda: torch.randn(2, 1, 1, 10)),
+    "mask_s_s": (_Sdpa(), [(1, 2, 6, 4), (1, 2, 6, 4), (1, 2, 6, 4)], lambda: torch.randn(6, 6)),
+    "two_lead_dims": (_Sdpa(is_causal=True), [(2, 3, 2, 6, 4), (2, 3, 2, 6, 4), (2, 3, 2, 6, 4)], None),
+    "repeat_kv": (_RepeatedKv(), [(2, 6, 8, 4), (2, 2, 8, 4), (2, 2, 8, 4)], None),
+}
+
+
+@pytest.mark.parametrize("case", sorted(CASES))
+def test_decomposed_nests_equal_eager_attention(case):
+    mod, shapes, mask = CASES[case]
+    torch.manual_seed(5)
+    args = [torch.randn(*s) for s in shapes] + ([mask()] if mask else [])
+    g = trace_module(mod.eval(), tuple(args))
+    d = decompose_attention(g, _undo_repeat_kv)
+    assert not any(isinstance(n.op, F.SdpaOp) for n in d.nodes.values())
+    nests = [n for n in d.nodes.values() if isinstance(n.op, F.LoopNestOp)]
+    assert [n.op.label for n in nests] == ["sdpa_scores", "sdpa_softmax_v"]
+    if case == "repeat_kv":  # the repeat is the head // group index, not a copy
+        assert [d.nodes[i].output.shape[1] for i in nests[0].inputs] == [6, 2]
+    values = {nid: a.double().numpy() for nid, a in zip(g.inputs, args)}
+    for n in nests:
+        ins = {name: values[src] for name, src in zip(n.op.loads, n.inputs)}
+        ins.update({name: np.array([val]) for name, val in (n.op.scalars or {}).items()})
+        shape = tuple(int(x) for x in n.output.shape)
+        values[n.id] = loop_ir.run_vectorised(n.op.stmts, ins, shape)
+        if n.output.numel <= 2048:  # the literal python-loop reading of the same statements
+            np.testing.assert_allclose(loop_ir.run_loops(n.op.stmts, ins, shape), values[n.id], rtol=1e-12, atol=1e-12)
+    want = mod(*(a.double() for a in args)).numpy()
+    np.testing.assert_allclose(values[nests[1].id], want, rtol=1e-9, atol=1e-9)
+
+
+def _kernel_names(compiled):
+    return [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+
+
+def test_which_attention_is_decomposed():
+    """fp32, and 16-bit with a head_dim the flash kernel has no tiling for, become two batched contractions with
+    loop-nest operand / output stages; 16-bit head_dim 128 stays the one fused kernel."""
+    be = HipBackend()
+    q, k = torch.randn(1, 16, 128, 128), torch.randn(1, 8, 128, 128)
+    names = _kernel_names(be.compile(trace_module(_Sdpa(is_causal=True, enable_gqa=True).eval(), (q, k, k))))
+    assert names.count("k_batched_linear") == 2 and "k_sdpa_reduce" not in names
+    assert names.count("k_operand_a") == 1  # q is read in place; only the softmax is an operand stage of its own
+    names = _kernel_names(be.compile(trace_module(_Sdpa(is_causal=True, enable_gqa=True).eval(), (q.bfloat16(), k.bfloat16(), k.bfloat16()))))
+    assert names == ["k_sdpa_reduce"]
+    q32 = torch.randn(2, 4, 64, 32).bfloat16()
+    names = _kernel_names(be.compile(trace_module(_Sdpa().eval(), (q32, q32, q32))))
+    assert names.count("k_batched_linear") == 2 and "k_sdpa_reduce" not in names
+
+
+def test_grouped_heads_without_the_flag_are_refused():
+    q, k = torch.randn(1, 4, 8, 8), torch.randn(1, 2, 8, 8)
+    g = trace_module(_Sdpa(enable_gqa=True).eval(), (q, k, k))
+    for n in g.nodes.values():
+        if isinstance(n.op, F.SdpaOp):
+            n.op.enable_gqa = False
+    with pytest.raises(FusionError, match="enable_gqa"):
+        HipBackend().compile(g)

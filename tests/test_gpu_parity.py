@@ -1202,3 +1202,71 @@ def test_matmul_spelled_attention_is_raised_to_the_fused_kernel(device, dtype, m
     want = mod(*(t.double() for t in args)).float()
     tol = (2e-2, 2e-2) if dtype is torch.bfloat16 else (1e-4, 1e-5)
     eager.assert_close(ours.reshape(want.shape), want, *tol, f"matmul-spelled attention {dtype} masked={masked}")
+
+
+class _FusedAttention(nn.Module):
+    def __init__(self, **kw):
+        super().__init__()
+        self.kw = kw
+
+    def forward(self, q, k, v, mask=None):
+        return torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask, **self.kw)
+
+
+class _TokenMajorAttention(nn.Module):
+    """Heads split from token-major projections and merged back, as a decoder block does around the fused op."""
+
+    def forward(self, q, k, v):
+        o = torch.nn.functional.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True, enable_gqa=True)
+        return o.transpose(1, 2).reshape(q.shape[0], q.shape[1], -1)
+
+
+class _RepeatKvAttention(nn.Module):
+    def forward(self, q, k, v):
+        b, h, s, d = k.shape
+        g = q.shape[1] // h
+        k = k[:, :, None].expand(b, h, g, s, d).reshape(b, h * g, s, d)
+        v = v[:, :, None].expand(b, h, g, s, d).reshape(b, h * g, s, d)
+        return torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+
+
+_DECOMPOSED_ATTENTION = {
+    # the reference's fp32 perf cases: q [1, 16, S, 128], k / v [1, 8, S, 128], causal, grouped heads (tests/perf/cases.py:174-190)
+    "perf_s32": (_FusedAttention(is_causal=True, enable_gqa=True), torch.float32, [(1, 16, 32, 128), (1, 8, 32, 128), (1, 8, 32, 128)], None),
+    "perf_s128": (_FusedAttention(is_causal=True, enable_gqa=True), torch.float32, [(1, 16, 128, 128), (1, 8, 128, 128), (1, 8, 128, 128)], None),
+    "perf_s512": (_FusedAttention(is_causal=True, enable_gqa=True), torch.float32, [(1, 16, 512, 128), (1, 8, 512, 128), (1, 8, 512, 128)], None),
+    "ragged_keys": (_FusedAttention(), torch.float32, [(2, 4, 100, 64), (2, 4, 100, 64), (2, 4, 100, 64)], None),
+    "ragged_everything": (_FusedAttention(is_causal=True), torch.float32, [(1, 2, 33, 21), (1, 2, 33, 21), (1, 2, 33, 21)], None),
+    "cross_gqa": (_FusedAttention(enable_gqa=True, scale=0.2), torch.float32, [(1, 4, 50, 40), (1, 2, 70, 40), (1, 2, 70, 40)], None),
+    "mask_1_1_s_s": (_FusedAttention(), torch.float32, [(2, 3, 72, 64)] * 3, lambda: torch.zeros(72, 72).masked_fill(torch.arange(72)[None, :] > torch.arange(72)[:, None], float("-inf"))[None, None]),
+    "mask_per_batch_keys": (_FusedAttention(), torch.float32, [(2, 4, 40, 32)] * 3, lambda: torch.randn(2, 1, 1, 40)),
+    "token_major": (_TokenMajorAttention(), torch.float32, [(1, 128, 16, 128), (1, 128, 8, 128), (1, 128, 8, 128)], None),
+    "repeat_kv": (_RepeatKvAttention(), torch.float32, [(2, 8, 64, 64), (2, 2, 64, 64), (2, 2, 64, 64)], None),
+    "bf16_head_dim_32": (_FusedAttention(is_causal=True), torch.bfloat16, [(2, 4, 64, 32)] * 3, None),
+    "bf16_head_dim_96": (_FusedAttention(), torch.bfloat16, [(2, 4, 50, 96)] * 3, None),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", sorted(_DECOMPOSED_ATTENTION))
+def test_attention_outside_the_flash_kernel(device, case):
+    """The fused attention op on fp32 operands (what the reference's perf suite runs), or with a head_dim the flash
+    kernel has no tiling for: two batched MFMA contractions (fp32 atoms keep fp32 accuracy) around loop-nest stages,
+    against eager in float64."""
+    mod, dtype, shapes, mask = _DECOMPOSED_ATTENTION[case]
+    torch.manual_seed(41)
+    args = [torch.randn(*s).to(dtype) for s in shapes] + ([mask().to(dtype)] if mask else [])
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod.eval(), tuple(args)))
+    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert names.count("k_batched_linear") == 2 and "k_sdpa_reduce" not in names
+    prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in args))))
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = mod(*(t.double() for t in args)).float()
+    tol = (2e-2, 2e-2) if dtype is torch.bfloat16 else (1e-4, 1e-5)
+    eager.assert_close(ours.reshape(want.shape), want, *tol, f"decomposed attention {case}")

@@ -401,7 +401,7 @@ HAND = {
              f"Load(name='bb', input='bias', index=({_V('n')},)), Assign(name='y', op=ElementwiseImpl('add'), args=('s','bb')), "
              f"Write(output='Y', index=({_V('h')}, {_V('m')}, {_V('n')}), value='y'))),)),))"],
             {"X": (3, 40, 32), "W": (24, 32), "bias": (24,)}, ("Y", (3, 40, 24)), {"c_two": 2.0}),
-        ["k_operand_a", "k_operand_b", "k_batched_linear", "k_output_stage"],
+        ["k_operand_a", "k_batched_linear", "k_output_stage"],  # W is one plain load over (n, k): read in place
     ),
     # RMS normalisation with the row element loaded once and squared (the 512-token corpus spells it this way)
     "rms_single_load": (
