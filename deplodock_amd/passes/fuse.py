@@ -146,10 +146,22 @@ def _materialize(c: _Ctx, nid: str) -> None:
             c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
         c.done[nid] = nid
         return
-    for rec in (_rec_loop_nest, _rec_batched_linear, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_pointwise):
+    for rec in (_rec_same_type_cast, _rec_loop_nest, _rec_batched_linear, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_pointwise):
         if rec(c, nid):
             return
     raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
+
+
+def _rec_same_type_cast(c: _Ctx, nid: str) -> bool:
+    """``x.to(dtype)`` where ``x`` already has that type (an fp32 model's ``hidden_states.to(torch.float32)``): no
+    kernel, the node is another name for its operand's memory."""
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.CastOp) or c.g.nodes[node.inputs[0]].output.dtype != node.output.dtype:
+        return False
+    v = _need(c, node.inputs[0])
+    c.done[nid] = v.base
+    c.windows[nid] = (v.offset, tuple(v.shape), tuple(v.strides))
+    return True
 
 
 def _rec_loop_nest(c: _Ctx, nid: str) -> bool:
@@ -497,8 +509,8 @@ def _rec_linear_residual(c: _Ctx, nid: str) -> bool:
 
 def _rec_gate_up(c: _Ctx, nid: str) -> bool:
     node = c.g.nodes[nid]
-    if not (_is(node, F.ElementwiseOp, fn="mul") and len(node.inputs) == 2):
-        return False
+    if not (_is(node, F.ElementwiseOp, fn="mul") and len(node.inputs) == 2) or node.output.dtype.nbytes != 2:
+        return False  # (the paired tile is written for 16-bit operands: fp32 keeps two contractions and a map)
     for si, ui in ((0, 1), (1, 0)):
         silu = c.g.nodes[node.inputs[si]]
         up = c.g.nodes[node.inputs[ui]]
@@ -908,7 +920,7 @@ def _absorb_row_kernel(c: _Ctx, body: RowReduce, x: View, addr: RowAddr, tokens:
         return False
     con = prod.op.body
     d = body.cols
-    if con.post is not None or con.gate_pair or con.row_epilogue is not None or con.reduce.cta != 1:
+    if con.post is not None or con.gate_pair or con.row_epilogue is not None or con.reduce.cta != 1 or con.in_dtype.nbytes != 2:
         return False
     if not (con.out == x.base and con.m == tokens and addr.stride_hi == (con.ldo or con.n) and addr.offset == con.out_offset and groups * d <= con.n):
         return False

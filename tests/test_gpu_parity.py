@@ -1270,3 +1270,24 @@ def test_attention_outside_the_flash_kernel(device, case):
     want = mod(*(t.double() for t in args)).float()
     tol = (2e-2, 2e-2) if dtype is torch.bfloat16 else (1e-4, 1e-5)
     eager.assert_close(ours.reshape(want.shape), want, *tol, f"decomposed attention {case}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seq", [128, 40])
+def test_c5_qwen3_block_in_fp32(device, seq):
+    """The decoder block with fp32 parameters and activations — the only precision the reference compiles
+    (tests/perf/cases.py:20-23).  The fused forms written for 16-bit tiles (norm prologue, gate/up pair, head-norm +
+    rotary epilogue, flash attention) stand down: plain fp32-atom contractions, row kernels and the decomposed
+    attention; against the module in float64."""
+    import copy
+
+    case = eager.qwen3_block_case(seq=seq, dtype=torch.float32, norm_std=0.1, seed=5)
+    ours, want, compiled = run_case(case, device)
+    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert names.count("k_batched_linear") == 2 and "k_sdpa_reduce" not in names
+    with torch.no_grad():
+        exact = copy.deepcopy(case.module).cpu().double()(*(t.double() for t in case.inputs))
+    exact = (exact[0] if isinstance(exact, tuple) else exact).float()
+    scale = float(exact.pow(2).mean().sqrt())
+    eager.assert_close(ours.cpu(), exact.reshape(ours.shape), 1e-4, 1e-4 * scale, f"fp32 block S={seq} vs float64")
+    eager.assert_close(ours, want, 1e-4, 1e-4 * scale, f"fp32 block S={seq} vs eager fp32 (GPU)")
