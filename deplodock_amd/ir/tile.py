@@ -335,6 +335,27 @@ class Map:
 
 
 @dataclass
+class StridedCopy:
+    """A dense row-major tensor made from a strided view of ``src``: result axis ``i`` has ``axes[i] = (extent,
+    source extent, source stride)``; where the result extends past the source it is zero (``emit/copy.py``)."""
+
+    src: str
+    out: str
+    dtype: DType
+    src_offset: int
+    src_numel: int
+    axes: tuple  # ((result extent, source extent, source stride), ...) in result order
+
+    def algo_flops(self) -> int:
+        return 0
+
+    def algo_bytes(self) -> int:
+        import math
+
+        return int((math.prod(se for _, se, _ in self.axes) + math.prod(de for de, _, _ in self.axes)) * self.dtype.nbytes)
+
+
+@dataclass
 class LoopNest:
     """A Loop-IR body rendered as it stands (``emit/loopnest.py``): the statements of a reference ``LoopOp``
     (``ir/loopnest.py``), the tensors its ``Load`` statements name, and scalar constants folded into the text."""

@@ -320,44 +320,20 @@ def _rec_batched_linear(c: _Ctx, nid: str) -> bool:
 
 
 def _copy_of_view(c: _Ctx, v: View, order: tuple[int, ...], new_id: str, pad_last_to: int | None = None, pad_rows_to: int | None = None) -> View:
-    """A dense row-major copy of ``v`` with its axes in ``order``, made by a loop nest of its own (``new_id``): what a
-    contraction needs when an operand's reduction axis is not the contiguous one, or its leading axes are not one
+    """A dense row-major copy of ``v`` with its axes in ``order``, made by a copy kernel of its own (``new_id``): what
+    a contraction needs when an operand's reduction axis is not the contiguous one, or its leading axes are not one
     uniformly strided run.  The last axis (``pad_last_to``) and the one before it (``pad_rows_to``) can be extended
     with zeros."""
-    from deplodock_amd.ir import loopnest as L
-    from deplodock_amd.ir.tile import LoopNest
+    from deplodock_amd.ir.tile import StridedCopy
 
-    numel = c.out.nodes[v.base].output.numel
-    axes = [f"c{i}" for i in range(len(v.shape))]
-    extent = {i: int(v.shape[i]) for i in order}
-    pads = {}  # source axis -> padded extent
-    if pad_last_to is not None and pad_last_to > extent[order[-1]]:
-        pads[order[-1]] = int(pad_last_to)
-    if pad_rows_to is not None and len(order) > 1 and pad_rows_to > extent[order[-2]]:
-        pads[order[-2]] = int(pad_rows_to)
-
-    def ax(i: int):
-        # a padded axis runs past the source: its index is clamped (the value read there is replaced by zero)
-        return L.Ternary(L.Bin("<", L.Var(axes[i]), L.Lit(extent[i])), L.Var(axes[i]), L.Lit(0)) if i in pads else L.Var(axes[i])
-
-    flat: object = L.Lit(int(v.offset))
-    for i, st in enumerate(v.strides):
-        if st:
-            flat = L.Bin("+", flat, L.Bin("*", ax(i), L.Lit(int(st))))
-    if pads:
-        inside: object = None
-        for i in pads:
-            here = L.Bin("<", L.Var(axes[i]), L.Lit(extent[i]))
-            inside = here if inside is None else L.Bin("&&", inside, here)
-        body: tuple = (L.Load("t", "src", (flat,)), L.Load("z", "zero", (L.Lit(0),)), L.Select("u", (("t", inside), ("z", L.Lit(1)))),
-                       L.Write(new_id, tuple(L.Var(axes[i]) for i in order), "u"))  # fmt: skip
-    else:
-        body = (L.Load("t", "src", (flat,)), L.Write(new_id, tuple(L.Var(axes[i]) for i in order), "t"))
-    for i in reversed(order):
-        body = (L.Loop(axes[i], pads.get(i, extent[i]), body),)
-    shape = tuple(pads.get(i, extent[i]) for i in order)
-    nest = LoopNest(stmts=body, operands={"src": (v.base, (int(numel),), v.dtype)}, scalars={"zero": 0.0} if pads else {}, out=new_id, out_name=new_id, out_shape=shape, out_dtype=v.dtype)
-    c.out.add_node(TileOp(name=c.kname("gather"), body=nest), [v.base], Tensor(new_id, shape, v.dtype), new_id)
+    axes = [[int(v.shape[i]), int(v.shape[i]), int(v.strides[i])] for i in order]
+    if pad_last_to is not None and pad_last_to > axes[-1][0]:
+        axes[-1][0] = int(pad_last_to)
+    if pad_rows_to is not None and len(axes) > 1 and pad_rows_to > axes[-2][0]:
+        axes[-2][0] = int(pad_rows_to)
+    shape = tuple(a[0] for a in axes)
+    body = StridedCopy(src=v.base, out=new_id, dtype=v.dtype, src_offset=int(v.offset), src_numel=int(c.out.nodes[v.base].output.numel), axes=tuple(tuple(a) for a in axes))
+    c.out.add_node(TileOp(name=c.kname("gather"), body=body), [v.base], Tensor(new_id, shape, v.dtype), new_id)
     return View(new_id, 0, shape, contiguous_strides(shape), v.dtype)
 
 

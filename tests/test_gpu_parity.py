@@ -1291,3 +1291,54 @@ def test_c5_qwen3_block_in_fp32(device, seq):
     scale = float(exact.pow(2).mean().sqrt())
     eager.assert_close(ours.cpu(), exact.reshape(ours.shape), 1e-4, 1e-4 * scale, f"fp32 block S={seq} vs float64")
     eager.assert_close(ours, want, 1e-4, 1e-4 * scale, f"fp32 block S={seq} vs eager fp32 (GPU)")
+
+
+_COPIES = {
+    # name: (source shape, dtype, result-order of the source axes, pad rows to, pad last to)
+    "transpose_2d": ((1024, 2048), torch.float32, (1, 0), None, None),
+    "transpose_ragged_padded": ((100, 37), torch.float32, (1, 0), 40, 104),
+    "batched_transpose_bf16": ((6, 70, 130), torch.bfloat16, (0, 2, 1), 132, 72),
+    "heads_to_tokens": ((16, 128, 64), torch.float32, (1, 0, 2), None, None),
+    "rows_padded": ((5, 33, 50), torch.float32, (0, 1, 2), 36, 56),
+    "unit_axis_in_the_middle": ((7, 65, 3), torch.float32, (2, 0, 1), None, None),
+    "one_column": ((300, 1), torch.float32, (1, 0), None, None),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", sorted(_COPIES))
+def test_strided_copy(device, case):
+    """The layout-change kernel (rows written as they lie, or 64 x 64 tiles transposed through LDS) against torch's
+    ``permute`` + zero padding: bit-exact, it moves values."""
+    from deplodock_amd.dtype import from_torch
+    from deplodock_amd.ir.tile import StridedCopy
+
+    shape, dtype, order, pad_rows, pad_last = _COPIES[case]
+    torch.manual_seed(51)
+    # a window of a larger buffer, so offset and strides are not the dense ones
+    big = torch.randn(*(d + 3 for d in shape)).to(dtype)
+    view = big[tuple(slice(2, 2 + d) for d in shape)]
+    axes = [[shape[i], shape[i], view.stride(i)] for i in order]
+    if pad_last:
+        axes[-1][0] = pad_last
+    if pad_rows:
+        axes[-2][0] = pad_rows
+    out_shape = tuple(a[0] for a in axes)
+    dt = from_torch(dtype)
+    body = StridedCopy(src="X", out="out", dtype=dt, src_offset=view.storage_offset(), src_numel=big.numel(), axes=tuple(tuple(a) for a in axes))
+    g = Graph()
+    g.add_input("X", (big.numel(),), dt)
+    g.add_node(TileOp(name="k_gather", body=body), ["X"], Tensor("out", out_shape, dt))
+    g.outputs = ["out"]
+    be = HipBackend()
+    compiled = lower(g)
+    prog = be.program(compiled, {"X": big.reshape(-1).to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()["out"].clone().cpu()
+    finally:
+        prog.close()
+    want = torch.zeros(out_shape, dtype=dtype)
+    want[tuple(slice(0, shape[i]) for i in order)] = view.permute(*order)
+    assert torch.equal(ours.reshape(out_shape).view(torch.int16 if dtype is torch.bfloat16 else torch.int32), want.view(torch.int16 if dtype is torch.bfloat16 else torch.int32))
