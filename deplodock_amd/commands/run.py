@@ -19,6 +19,7 @@ from deplodock_amd.commands.table import render_table
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_F32_PEAK_TFLOPS = 157.3
 
 TOLERANCES = {"float32": (1e-5, 1e-5), "bfloat16": (2e-2, 2e-2), "float16": (2e-2, 2e-2)}
 
@@ -111,8 +112,9 @@ def kernel_rows(compiled, bench) -> list[list[str]]:
         if us:
             gbps = op.algo_bytes / (us * 1e-6) / 1e9
             tfs = op.algo_flops / (us * 1e-6) / 1e12
-            if op.algo_flops and tfs / MFMA_BF16_PEAK_TFLOPS > gbps / HBM_PEAK_GBPS:
-                rate, frac = f"{tfs:.1f} TFLOP/s", f"{100 * tfs / MFMA_BF16_PEAK_TFLOPS:.1f}% mfma"
+            peak = MFMA_F32_PEAK_TFLOPS if "_f32" in str(op.knobs.get("TILE", "")) else MFMA_BF16_PEAK_TFLOPS  # the atom names the matrix pipe's rate
+            if op.algo_flops and tfs / peak > gbps / HBM_PEAK_GBPS:
+                rate, frac = f"{tfs:.1f} TFLOP/s", f"{100 * tfs / peak:.1f}% mfma"
             else:
                 rate, frac = f"{gbps:.0f} GB/s", f"{100 * gbps / HBM_PEAK_GBPS:.1f}% hbm"
         knobs = " ".join(f"{k}={v}" for k, v in op.knobs.items())

@@ -370,6 +370,32 @@ def _default_tile(body: Contraction, ctx: Context) -> TilePlan:
     return plan
 
 
+def _fp32_underfilled(body: Contraction, plan: TilePlan, ctx: Context) -> tuple[TilePlan, int]:
+    """The fp32 matrix pipe runs at a sixteenth of the 16-bit rate, so an fp32 problem is bound by how evenly its
+    MFMA work spreads over the CUs long before memory matters: a 32 x 1024 x 3072 product on 128 one-wave tiles
+    leaves half the CUs idle and each wave walks all of K alone (22.7 us).  When 32x32 tiles would not cover the
+    CUs, the reduction axis is split across workgroups (partials workspace + combine kernel) until about two
+    workgroups per CU run, on four-wave 32x32 tiles with 32-deep slabs.  Measured (us, the unsplit default ->
+    this): 32x3072x1024 22.7 -> 5.8, 128x3072x1024 21.8 -> 10.7, 32x2048x1024 15.5 -> 4.9, 128x2048x1024 15.1 ->
+    8.5, 32x1024x2048 6.5 -> 4.8, 32x1024x1024 6.7 -> 4.1, 128x1024x1024 6.6 -> 6.2.  Problems whose 32x32 tiles
+    already cover the CUs keep the unsplit default (128x1024x2048: 6.8 unsplit, 8.4 split in two)."""
+    plain = not (body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None) and int(getattr(body, "batch", 1) or 1) == 1 and body.k_split is None
+    if body.in_dtype.name != "f32" or not plain or not all(isinstance(d, int) for d in (body.m, body.n, body.k)) or body.m <= 16 or body.k % 32 or body.k < 256:
+        return plan, 1
+    base = -(-body.m // 32) * -(-body.n // 32)
+    if base >= ctx.compute_units:
+        return plan, 1
+    split = 1
+    while split < 8 and base * split * 2 <= 2 * ctx.compute_units and (body.k // (split * 2)) % 32 == 0 and body.k // (split * 2) >= 128:
+        split *= 2
+    tile = TilePlan(atom=ATOMS["mfma_16x16x4_f32"], units=(2, 2), regs=(1, 1), bk=8)
+    try:
+        _check_tile(tile, body, ctx, depth=3, dl=True)
+    except ScheduleError:
+        return plan, 1
+    return tile, split
+
+
 def default_contraction_schedule(body: Contraction, ctx: Context) -> None:
     """Put the heuristic tile and staging on ``body``, whatever was pinned or tuned (the lowering's last
     resort for a pinned tile whose kernel only builds with register spills)."""
@@ -394,8 +420,11 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
         except ScheduleError as exc:
             logger.warning("EMMY_TILE=%r ignored: %s", pinned, exc)
             plan = None
+    auto_split = 1
     if plan is None:
         plan = _default_tile(body, ctx)
+        if not _pin("REDUCE", tuned):
+            plan, auto_split = _fp32_underfilled(body, plan, ctx)
     body.tile = plan
     stage = None
     pinned_stage = _pin("STAGE", tuned)
@@ -427,6 +456,9 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
     # more than the idle CUs (see ``deplodock_amd.emit.splitk``).  A ``b<n>`` / ``r<n>`` pin is a row kernel's.
     body.reduce = ReducePlan()
     pinned_reduce = _pin("REDUCE", tuned)
+    if auto_split > 1 and not pinned_reduce and stage.transport in ("dl", "sync"):
+        body.reduce = ReducePlan(cta=auto_split, finalize="kernel")
+        knobs["REDUCE"] = body.reduce.spell()
     if pinned_reduce:
         try:
             rp = ReducePlan.parse(pinned_reduce)
