@@ -358,6 +358,12 @@ def _default_tile(body: Contraction, ctx: Context) -> TilePlan:
     re = body.row_epilogue
     plan = pick_tile(body.m, body.n, body.k, body.gate_pair, ctx, row_prologue=body.a_prologue is not None, group_cols=(re.cols, re.col_end) if re is not None else None,
                      copies=max(1, int(getattr(body, "batch", 1) or 1)))
+    if atom_dtype == "f32" and all(isinstance(d, int) for d in (body.m, body.n, body.k)):
+        # One even round of workgroups matters most at the fp32 matrix rate: 64x96 tiles (eight waves of 16x48) when they
+        # make 0.9-1.0 workgroups per CU exactly (512x1024x3072: 30.6 us on 256 of them, 38.1 on 192 tiles of 64x128).
+        groups = (body.m // 64) * (body.n // 96) * max(1, int(getattr(body, "batch", 1) or 1))
+        if body.m % 64 == 0 and body.n % 96 == 0 and body.k % 64 == 0 and 0.9 * ctx.compute_units <= groups <= ctx.compute_units and not body.gate_pair and body.row_epilogue is None:
+            return TilePlan(atom=ATOMS["mfma_16x16x4_f32"], units=(4, 2), regs=(1, 3), bk=16)
     if atom_dtype == "f32":
         # the fp32 tier keeps the candidate's tile and its slab's bytes per row: half the k-values, on the fp32 atom of the same m x n
         atom = ATOMS[{16: "mfma_16x16x4_f32", 32: "mfma_32x32x2_f32"}[plan.atom.m]]
