@@ -104,3 +104,95 @@ def test_seeded_random_shapes(device, kind):
             prog.close()
         want = eager.run_eager(case, device)
         eager.assert_close(ours.reshape(want.shape), want, case.rtol, case.atol, f"{kind} #{i} {case.name}")
+
+
+class _MatMul(nn.Module):
+    def forward(self, a, b):
+        return a @ b
+
+
+class _MatMulT(nn.Module):
+    def forward(self, a, b):
+        return a @ b.transpose(-1, -2)
+
+
+class _Attention(nn.Module):
+    def __init__(self, causal: bool, gqa: bool, scale):
+        super().__init__()
+        self.kw = dict(is_causal=causal, enable_gqa=gqa, scale=scale)
+
+    def forward(self, q, k, v, mask=None):
+        return F.scaled_dot_product_attention(q, k, v, attn_mask=mask, **self.kw)
+
+
+class _BiasLinear(nn.Module):
+    def __init__(self, k: int, n: int, bias: bool, residual: bool):
+        super().__init__()
+        self.lin, self.residual = nn.Linear(k, n, bias=bias), residual
+
+    def forward(self, x, r):
+        y = self.lin(x)
+        return y + r if self.residual else y
+
+
+def _wide_case(kind: str, rnd: random.Random, seed: int):
+    """``(name, module, inputs, 16-bit?)`` for the families whose reference is the module in float64."""
+    torch.manual_seed(seed)
+    if kind == "matmul":
+        dt = rnd.choice([torch.float32, torch.float32, torch.bfloat16])
+        lead = rnd.choice([(), (rnd.randint(1, 5),), (2, rnd.randint(1, 3))])
+        m, k, n = rnd.choice([rnd.randint(1, 70), rnd.randint(1, 300), 128]), rnd.choice([rnd.randint(1, 40) * 8, rnd.randint(1, 300), 1024]), rnd.choice([rnd.randint(1, 60) * 4, rnd.randint(1, 200), 256])
+        transposed = rnd.random() < 0.4
+        shared = rnd.random() < 0.5 or not lead
+        b_shape = ((n, k) if transposed else (k, n)) if shared else (*lead, *((n, k) if transposed else (k, n)))
+        a, b = torch.randn(*lead, m, k).to(dt), (0.3 * torch.randn(*b_shape)).to(dt)
+        return f"matmul {tuple(a.shape)} @ {tuple(b.shape)}{'^T' if transposed else ''} {dt}", (_MatMulT() if transposed else _MatMul()).eval(), (a, b), dt is not torch.float32
+    if kind == "attention32":
+        hkv, group = rnd.choice([1, 2, 3]), rnd.choice([1, 2, 4])
+        sq = rnd.choice([rnd.randint(1, 40), rnd.randint(1, 200), 128])
+        causal = rnd.random() < 0.4
+        skv = sq if causal or rnd.random() < 0.5 else rnd.randint(1, 250)
+        d, dv = rnd.choice([16, 32, 40, 64, 128]), None
+        b = rnd.choice([1, 2])
+        q, k, v = torch.randn(b, hkv * group, sq, d), torch.randn(b, hkv, skv, d), torch.randn(b, hkv, skv, d)
+        mask = None
+        if not causal and rnd.random() < 0.5:
+            mask = torch.randn(*rnd.choice([(sq, skv), (1, 1, sq, skv), (b, 1, 1, skv), (b, hkv * group, sq, skv)]))
+        scale = rnd.choice([None, None, 0.25])
+        return f"attention fp32 {hkv * group}/{hkv} heads {sq}x{skv} d={d} causal={causal} mask={None if mask is None else tuple(mask.shape)}", _Attention(causal, group > 1, scale).eval(), (q, k, v) + ((mask,) if mask is not None else ()), False
+    # fp32 linear (+ bias, + residual): the underfilled-launch split and the exact-round tiles
+    m = rnd.choice([rnd.randint(17, 200), 32, 128, 512])
+    k, n = rnd.choice([256, 512, 1024, 2048, 3072, 96, 160]), rnd.choice([rnd.randint(1, 64) * 8, 256, 1024, 3072])
+    bias, residual = rnd.random() < 0.5, rnd.random() < 0.5
+    mod = _BiasLinear(k, n, bias, residual)
+    with torch.no_grad():
+        for p in mod.parameters():
+            p.copy_(0.05 * torch.randn_like(p))
+    return f"linear fp32 {m}x{k}x{n} bias={bias} residual={residual}", mod.eval(), (torch.randn(m, k), torch.randn(m, n)), False
+
+
+@pytest.mark.parametrize("kind", ["matmul", "attention32", "linear32"])
+def test_seeded_random_shapes_against_float64(device, kind):
+    """Families that reach the batched contraction, the layout-change copy, zero-padded ragged extents, the
+    decomposed attention and the fp32 tier's split of an underfilled launch: against the module in float64
+    (fp32: 1e-4 of the output's RMS; 16-bit: rtol 2e-2)."""
+    import copy
+
+    rnd = random.Random(f"emmy-wide-{kind}")
+    be = HipBackend()
+    for i in range(14):
+        name, mod, inputs, half = _wide_case(kind, rnd, seed=2000 + i)
+        print(f"{kind} #{i}: {name}", flush=True)  # names the case should the device fault
+        compiled = be.compile(trace_module(mod, inputs))
+        prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, inputs)})
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            ours = prog.output_tensors()[compiled.outputs[0]].clone().cpu()
+        finally:
+            prog.close()
+        with torch.no_grad():
+            want = copy.deepcopy(mod).double()(*(t.double() for t in inputs)).float()
+        rms = float(want.pow(2).mean().sqrt())
+        rtol, atol = (2e-2, 2e-2 * max(rms, 1.0)) if half else (1e-4, 1e-4 * max(rms, 1e-3))
+        eager.assert_close(ours.reshape(want.shape).float(), want, rtol, atol, f"{kind} #{i} {name}")
