@@ -8,6 +8,7 @@ result files can be joined on them.
 
 from __future__ import annotations
 
+import os
 from dataclasses import dataclass
 
 HIDDEN, INTERMEDIATE, HEADS, KV_HEADS, HEAD_DIM = 1024, 3072, 16, 8, 128
@@ -30,7 +31,8 @@ class Case:
     @property
     def code(self) -> str:
         s = self.shapes
-        rand = [f"torch.randn({tuple(x)})" for x in s]
+        kw = "" if self.dtype == "fp32" else f", dtype=torch.{TORCH_DTYPE[self.dtype]}"
+        rand = [f"torch.randn({tuple(x)}{kw})" for x in s]
         if self.op == "matmul":
             return f"a={rand[0]}; b={rand[1]}; torch.matmul(a,b)"
         if self.op == "rmsnorm":
@@ -54,7 +56,12 @@ class Case:
         return 20 if total > HEAVY_ELEMENTS else 100
 
 
-def _cases() -> list[Case]:
+TORCH_DTYPE = {"fp32": "float32", "bf16": "bfloat16", "fp16": "float16"}
+
+
+def _cases(dtype: str = "fp32") -> list[Case]:
+    if dtype not in TORCH_DTYPE:
+        raise ValueError(f"EMMY_PERF_DTYPE: expected one of {sorted(TORCH_DTYPE)}, got {dtype!r}")
     out: list[Case] = []
     q_dim, kv_dim = HEADS * HEAD_DIM, KV_HEADS * HEAD_DIM
     for s in SEQ_LENS:  # input / post-attention layer norm
@@ -72,7 +79,9 @@ def _cases() -> list[Case]:
             out.append(Case(f"matmul_add.{TAG}.{proj}.s{s}", "matmul_add", ((1, s, k), (k, HIDDEN), (1, s, HIDDEN))))
     for s in SEQ_LENS:
         out.append(Case(f"gated_mlp.{TAG}.s{s}", "gated_mlp", ((1, s, HIDDEN), (HIDDEN, INTERMEDIATE), (HIDDEN, INTERMEDIATE))))
-    return out
+    return [Case(c.name, c.op, c.shapes, dtype) for c in out]
 
 
-CASES = _cases()
+# The reference runs fp32 only and keeps ``dtype`` "so an FP16 column can be added later" (cases.py:20-23); here
+# ``EMMY_PERF_DTYPE=bf16`` (or ``fp16``) runs the same cases on this backend's 16-bit tier.
+CASES = _cases(os.environ.get("EMMY_PERF_DTYPE", "fp32"))
