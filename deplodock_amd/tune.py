@@ -51,6 +51,14 @@ TILE_SWEEP: tuple[str, ...] = (
     "a:mfma_16x16x32_bf16/w1x2/f1x1/k8",
     "a:mfma_16x16x32_bf16/w1x1/f1x1/k8",
 )  # every tile that won an in-graph ranking of the decoder block's contractions at 64 ... 2048 tokens, and their neighbours
+# The fp32 tier (fp32 MFMA atoms; slab depth in atom steps of 4): the tiles that ranked first somewhere in a sweep of the
+# decoder layer's projections at 32 / 128 / 512 tokens in fp32.
+TILE_SWEEP_F32: tuple[str, ...] = tuple(
+    f"a:mfma_16x16x4_f32/{units}/k{bk}"
+    for units in ("w4x2/f1x3", "w2x2/f2x3", "w2x4/f2x2", "w2x4/f2x1", "w4x2/f1x2", "w2x2/f2x2", "w2x4/f1x1", "w2x2/f1x2", "w2x2/f1x1", "w1x4/f1x1", "w1x2/f1x1")
+    for bk in (16, 32, 8)
+)
+STAGE_SWEEP_F32: tuple[str, ...] = ("d3/dl", "d2/dl")
 STAGE_SWEEP: tuple[str, ...] = ("d2/dl", "d3/dl", "d2/sync/p2")
 FEW_ROW_SWEEP: tuple[str, ...] = ("d8/ks", "d4/ks")  # the k-split few-row form has no tile: one candidate each
 REDUCE_SWEEP: tuple[str, ...] = ("b8", "b16", "b32", "b64", "b128", "b256", "b512", "b1024")
@@ -182,7 +190,16 @@ def candidate_rounds(families: set[str]) -> list[dict[str, str]]:
             if r < len(cands):
                 pins.update(cands[r])
         out.append(pins)
+    if "contraction_f32" in families:
+        # rounds of their own: TILE / STAGE name one atom type, and a 16-bit contraction of the same graph keeps its defaults meanwhile
+        out += [{"TILE": t, "STAGE": s} for s in STAGE_SWEEP_F32 for t in TILE_SWEEP_F32]
     return out
+
+
+def _family(key: str) -> str:
+    """Candidate family of a shape key: fp32 contractions sweep fp32 atoms."""
+    fam = key.split("/")[0]
+    return "contraction_f32" if fam == "contraction" and "/f32>" in key else fam
 
 
 def tune_graph(graph, backend, db: TuneDB | None = None, *, input_data: dict | None = None, warmup: int = 3, num_iters: int = 10,
@@ -215,7 +232,7 @@ def tune_graph(graph, backend, db: TuneDB | None = None, *, input_data: dict | N
         fam = key.split("/")[0]
         knobs = {k: str(op.knobs[k]) for k in FAMILY_KNOBS[fam] if k in op.knobs}
         results[key] = KernelTuning(key, op.kernel_name, knobs, base_us[idx], dict(knobs), base_us[idx])
-    rounds = candidate_rounds({k.split("/")[0] for k in results})
+    rounds = candidate_rounds({_family(k) for k in results})
     if max_rounds is not None:
         rounds = rounds[:max_rounds]
     for r, pins in enumerate(rounds):

@@ -87,6 +87,45 @@ def test_candidate_rounds_cover_every_family_once():
     assert candidate_rounds({"row_reduce"}) and all(set(r) == {"REDUCE", "NT"} for r in candidate_rounds({"row_reduce"}))
 
 
+def test_fp32_contractions_sweep_fp32_atoms_in_rounds_of_their_own():
+    from deplodock_amd.ir.schedule import TilePlan
+    from deplodock_amd.tune import STAGE_SWEEP_F32, TILE_SWEEP_F32, _family
+
+    assert _family("contraction/m512/n3072/k1024/f32>f32/g0/p0/a0") == "contraction_f32" and _family("contraction/m512/n3072/k1024/bf16>bf16/g0/p0/a0") == "contraction"
+    only = candidate_rounds({"contraction_f32"})
+    assert len(only) == len(TILE_SWEEP_F32) * len(STAGE_SWEEP_F32) and all(set(r) == {"TILE", "STAGE"} for r in only)
+    assert all(TilePlan.parse(r["TILE"]).atom.dtype == "f32" for r in only)
+    mixed = candidate_rounds({"contraction", "contraction_f32"})
+    assert len(mixed) == 62 + len(only) and mixed[62:] == only  # appended, never merged with the 16-bit pins of a round
+
+
+@pytest.mark.gpu
+def test_tuning_an_fp32_contraction_keeps_fp32_pins(device, tmp_path):
+    """The sweep over an fp32 matmul: candidates keep their pins (fp32 atoms), outputs stay equal, and whatever wins is
+    at least as fast as the default."""
+    import torch
+
+    from deplodock_amd.tune import tune_graph
+
+    class Mm(torch.nn.Module):
+        def forward(self, a, b):
+            return a @ b.transpose(-1, -2)
+
+    torch.manual_seed(3)
+    a, b = torch.randn(512, 512), torch.randn(768, 512)  # (enough 32x32 tiles to cover the CUs: the launch is not split)
+    be = HipBackend()
+    graph = trace_module(Mm().eval(), (a, b))
+    base = be.compile(graph)
+    data = dict(zip(base.inputs, (a.to(device), b.to(device))))
+    db = TuneDB(tmp_path / "tune.db")
+    try:
+        (res,) = tune_graph(graph, be, db, input_data=data, warmup=1, num_iters=3, max_rounds=12)
+    finally:
+        db.close()
+    assert res.tried >= 4 and not res.rejected and res.best_us <= res.baseline_us
+    assert "_f32/" in res.best_knobs["TILE"]
+
+
 def test_pinned_context_restores_the_environment(monkeypatch):
     monkeypatch.setenv("EMMY_TILE", "x")
     monkeypatch.setenv("EMMY_KNOBS", "REDUCE=b64")
