@@ -19,7 +19,7 @@ from deplodock_amd.context import Context
 from deplodock_amd.emit import prelude
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir.hip import HipOp
-from deplodock_amd.ir.tile import StridedCopy
+from deplodock_amd.ir.tile import IndexRows, StridedCopy
 from deplodock_amd.render_target import rt
 
 _TILE = 64
@@ -129,4 +129,39 @@ def emit_strided_copy(body: StridedCopy, name: str, ctx: Context = Context()) ->
     )
 
 
-__all__ = ["emit_strided_copy"]
+def emit_index_rows(body: IndexRows, name: str, ctx: Context = Context()) -> HipOp:
+    """One lane per result element, consecutive along ``inner``: the row index is read once per element (it sits in
+    cache for the whole row) and clamped into the table, so no value of ``idx`` can send a load outside ``src``."""
+    total = body.outer * body.count * body.inner
+    if min(body.outer, body.n, body.inner, body.count) < 1:
+        raise LoweringError("index rows: empty operand")
+    if total >= 1 << 31 or body.outer * body.n * body.inner >= 1 << 31:
+        raise LoweringError("index rows: index arithmetic is 32-bit; the tensor is too large")
+    if body.idx_dtype.name not in ("i32", "i64"):
+        raise LoweringError(f"index rows: indices must be int32 or int64, got {body.idx_dtype}")
+    T, IT = rt.type_name(body.dtype.name), rt.type_name(body.idx_dtype.name)
+    o: list[str] = []
+    a = o.append
+    a(f'extern "C" __global__ __launch_bounds__(256) void {name}(const {T}* __restrict__ src, const {IT}* __restrict__ idx, {T}* __restrict__ dst) {{')
+    a("  const unsigned lin = blockIdx.x * 256u + threadIdx.x;")
+    a(f"  if (lin >= {total}u) return;")
+    a(f"  const unsigned i = lin % {body.inner}u, j = (lin / {body.inner}u) % {body.count}u, o = lin / {body.inner * body.count}u;")
+    a("  long long r = (long long)idx[j];")
+    a(f"  r = r < 0 ? 0 : (r >= {body.n} ? {body.n - 1} : r);")
+    a(f"  dst[lin] = src[(o * {body.n}u + (unsigned)r) * {body.inner}u + i];")
+    a("}")
+    return HipOp(
+        kernel_source=prelude.header() + "\n".join(o) + "\n",
+        kernel_name=name,
+        arg_order=(body.src, body.idx, body.out),
+        grid=((-(-total // 256),), (1,), (1,)),
+        block=((256,), (1,), (1,)),
+        lds_bytes=0,
+        comment="index rows",
+        algo_bytes=body.algo_bytes(),
+        algo_flops=0,
+        knobs={"COPY": "index"},
+    )
+
+
+__all__ = ["emit_strided_copy", "emit_index_rows"]

@@ -13,6 +13,8 @@ reproduces the rounding points of an eager bf16 module.
 
 from __future__ import annotations
 
+import math
+
 from dataclasses import dataclass
 
 import numpy as np
@@ -58,13 +60,13 @@ class Const(Expr):
 
 @dataclass(frozen=True, eq=False)
 class Un(Expr):
-    op: str  # neg | exp | rsqrt | sqrt | rcp | sigmoid | silu | abs | tanh
+    op: str  # neg | exp | rsqrt | sqrt | rcp | sigmoid | silu | abs | tanh | relu | erf | gelu | gelu_tanh
     a: Expr
 
 
 @dataclass(frozen=True, eq=False)
 class Bin(Expr):
-    op: str  # add | sub | mul | div | max | min
+    op: str  # add | sub | mul | div | max | min | pow
     a: Expr
     b: Expr
 
@@ -119,8 +121,15 @@ def _un_c(op: str, a: str, rounded: bool = False) -> str:
         return div("1.0f", f"1.0f + {exp(f'-({a})')}") if rounded else f"(1.0f / (1.0f + {exp(f'-({a})')}))"
     if op == "silu":
         return div(f"({a})", f"1.0f + {exp(f'-({a})')}") if rounded else f"(({a}) / (1.0f + {exp(f'-({a})')}))"
-    if op in ("exp2", "fast_exp2", "rsqrt", "sqrt", "abs", "tanh"):
+    if op in ("exp2", "fast_exp2", "rsqrt", "sqrt", "abs", "tanh", "erf"):
         return _call(op, a)
+    if op == "relu":
+        return _call("max", a, "0.0f")
+    if op == "gelu":  # 0.5 x (1 + erf(x / sqrt 2)): emmy/compiler/pipeline/passes/frontend/decomposition/160_gelu.py
+        return f"(0.5f * ({a}) * (1.0f + {_call('erf', f'({a}) * {float_literal(1.0 / math.sqrt(2.0))}')}))"
+    if op == "gelu_tanh":  # 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))): decomposition/170_gelu_tanh.py
+        inner = f"{float_literal(math.sqrt(2.0 / math.pi))} * (({a}) + {float_literal(0.044715)} * ({a}) * ({a}) * ({a}))"
+        return f"(0.5f * ({a}) * (1.0f + {_call('tanh', inner)}))"
     raise KeyError(f"no rendering for unary op {op!r}")
 
 
@@ -131,7 +140,7 @@ _BIN_SYM = {"add": "+", "sub": "-", "mul": "*", "div": "/"}
 def _bin_c(op: str, a: str, b: str) -> str:
     if op in _BIN_SYM:
         return f"(({a}) {_BIN_SYM[op]} ({b}))"
-    if op in ("max", "min"):
+    if op in ("max", "min", "pow"):
         return _call(op, a, b)
     raise KeyError(f"no rendering for binary op {op!r}")
 
@@ -157,6 +166,10 @@ def render(e: Expr, env: dict[str, str]) -> str:
             return _round_c(e.dtype, _un_c(e.a.op, render(e.a.a, env), rounded=True))
         return _round_c(e.dtype, render(e.a, env))
     raise TypeError(f"cannot render {type(e).__name__}")
+
+
+def _erf(a: np.ndarray) -> np.ndarray:
+    return np.vectorize(math.erf, otypes=[np.float32])(np.asarray(a, dtype=np.float64)).astype(np.float32).reshape(np.shape(a))
 
 
 def evaluate(e: Expr, env: dict[str, np.ndarray]) -> np.ndarray:
@@ -186,6 +199,10 @@ def evaluate(e: Expr, env: dict[str, np.ndarray]) -> np.ndarray:
                 "tanh": lambda: np.tanh(a),
                 "sigmoid": lambda: (f32(1) / (f32(1) + np.exp(-a))).astype(f32),
                 "silu": lambda: (a / (f32(1) + np.exp(-a))).astype(f32),
+                "relu": lambda: np.maximum(a, f32(0)),
+                "erf": lambda: _erf(a),
+                "gelu": lambda: (f32(0.5) * a * (f32(1) + _erf(a * f32(1.0 / math.sqrt(2.0))))).astype(f32),
+                "gelu_tanh": lambda: (f32(0.5) * a * (f32(1) + np.tanh(f32(math.sqrt(2.0 / math.pi)) * (a + f32(0.044715) * a * a * a)))).astype(f32),
             }[e.op]().astype(f32)
     if isinstance(e, Bin):
         a = np.asarray(evaluate(e.a, env), dtype=f32)
@@ -198,6 +215,7 @@ def evaluate(e: Expr, env: dict[str, np.ndarray]) -> np.ndarray:
                 "div": lambda: a / b,
                 "max": lambda: np.maximum(a, b),
                 "min": lambda: np.minimum(a, b),
+                "pow": lambda: np.power(a, b),
             }[e.op]().astype(f32)
     raise TypeError(f"cannot evaluate {type(e).__name__}")
 

@@ -50,6 +50,24 @@ class SumOp(Op):
 
 
 @dataclass
+class AmaxOp(Op):
+    """``amax`` over one axis (the reference keeps torch's name for it, emmy/compiler/trace/torch.py:590-598)."""
+
+    axis: int = -1
+    keepdim: bool = False
+
+
+@dataclass
+class LayerNormOp(Op):
+    """``(x - mean) * rsqrt(var + eps) [* weight] [+ bias]`` over the last axis, biased variance
+    (frontend/ir.py:316-341, decomposition/085_layer_norm.py).  Inputs: ``x[, weight[, bias]]``."""
+
+    eps: float = 1e-5
+    has_weight: bool = False
+    has_bias: bool = False
+
+
+@dataclass
 class LinearOp(Op):
     """``x @ W.T (+ b)`` with ``W`` of shape ``[out, in]`` (frontend/ir.py:212-217)."""
 
@@ -157,6 +175,15 @@ class SliceOp(Op):
 @dataclass
 class CatOp(Op):
     dim: int = 0
+
+
+@dataclass
+class GatherOp(Op):
+    """Whole slices picked by an integer vector along ``axis``: ``embedding(table, idx)`` (axis 0, ``idx`` of any
+    shape) and ``index_select(x, axis, idx)`` (the reference's ``GatherOp``, emmy/compiler/trace/torch.py:738-756).
+    Inputs: ``x, idx``."""
+
+    axis: int = 0
 
 
 @dataclass

@@ -356,6 +356,28 @@ class StridedCopy:
 
 
 @dataclass
+class IndexRows:
+    """``out[o, j, i] = src[o, idx[j], i]`` over a dense ``src [outer, n, inner]`` and an integer vector ``idx [count]``
+    (an embedding lookup, ``index_select``); an index outside ``[0, n)`` is clamped (``emit/copy.py``)."""
+
+    src: str
+    idx: str
+    out: str
+    dtype: DType
+    idx_dtype: DType
+    outer: int
+    n: int
+    inner: int
+    count: int
+
+    def algo_flops(self) -> int:
+        return 0
+
+    def algo_bytes(self) -> int:
+        return int(2 * self.outer * self.count * self.inner * self.dtype.nbytes + self.count * self.idx_dtype.nbytes)
+
+
+@dataclass
 class LoopNest:
     """A Loop-IR body rendered as it stands (``emit/loopnest.py``): the statements of a reference ``LoopOp``
     (``ir/loopnest.py``), the tensors its ``Load`` statements name, and scalar constants folded into the text."""

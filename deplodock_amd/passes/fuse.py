@@ -146,7 +146,7 @@ def _materialize(c: _Ctx, nid: str) -> None:
             c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
         c.done[nid] = nid
         return
-    for rec in (_rec_same_type_cast, _rec_loop_nest, _rec_batched_linear, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_pointwise):
+    for rec in (_rec_same_type_cast, _rec_loop_nest, _rec_batched_linear, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_layer_norm, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_gather, _rec_cat, _rec_pointwise):
         if rec(c, nid):
             return
     raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
@@ -641,36 +641,159 @@ def _rec_softmax(c: _Ctx, nid: str) -> bool:
     node = c.g.nodes[nid]
     if not isinstance(node.op, F.SoftmaxOp):
         return False
-    if node.op.axis != len(node.output.shape) - 1:
-        raise FusionError("softmax over a non-innermost axis is not supported")
-    xv = _need(c, node.inputs[0])
-    if xv.strides[-1] != 1:
-        raise FusionError("softmax: the reduced axis must be contiguous")
+    xv, moved = _axis_last(c, nid, node.inputs[0], node.op.axis)
     rows, x_addr = _row_addr(xv)
     x = E.Var("x")
     stats = (Stat("m", "max", x), Stat("d", "sum", E.Un("exp", x - E.Var("m")), keep=True))
-    body = RowReduce(rows=rows, cols=int(node.output.shape[-1]), x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=node.output.dtype, stats=stats, project=x * E.Un("rcp", E.Var("d")), x_addr=x_addr)
-    _emit(c, nid, body, "softmax_reduce", [xv.base])
+    body = RowReduce(rows=rows, cols=int(xv.shape[-1]), x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=node.output.dtype, stats=stats, project=x * E.Un("rcp", E.Var("d")), x_addr=x_addr)
+    _emit(c, nid, body, "softmax_reduce", [xv.base], shape=tuple(xv.shape) if moved else None)
+    if moved:
+        # the result lies with the reduced axis last; readers address it in the traced order through these strides
+        logical = tuple(int(d) for d in node.output.shape)
+        dense = contiguous_strides(tuple(xv.shape))
+        axis = node.op.axis
+        strides = [0] * len(logical)
+        others = [i for i in range(len(logical)) if i != axis]
+        for pos, i in enumerate(others):
+            strides[i] = dense[pos]
+        strides[axis] = 1
+        c.out.nodes[nid].hints["logical_view"] = (logical, tuple(strides))
     return True
+
+
+def _axis_last(c: _Ctx, nid: str, src: str, axis: int) -> tuple[View, bool]:
+    """``src`` addressed with ``axis`` as its last, contiguous axis: as it lies when that is the case already, else
+    through a dense copy with the axis moved last.  Returns ``(view, moved)``."""
+    xv = _need(c, src)
+    rank = len(xv.shape)
+    if axis == rank - 1 and (xv.strides[-1] == 1 or xv.shape[-1] == 1):
+        return xv, False
+    order = (*(i for i in range(rank) if i != axis), axis)
+    if not all(isinstance(d, int) for d in (*xv.shape, *xv.strides, xv.offset)):
+        raise FusionError("a reduction over a non-innermost axis needs static shapes")
+    return _copy_of_view(c, xv, order, f"{nid}__axis_last"), axis != rank - 1
 
 
 def _rec_row_sum(c: _Ctx, nid: str) -> bool:
     """``sum`` / ``mean`` over the innermost axis as a row reduction with one value per row."""
     node = c.g.nodes[nid]
-    if not isinstance(node.op, (F.MeanOp, F.SumOp)):
+    if not isinstance(node.op, (F.MeanOp, F.SumOp, F.AmaxOp)):
         return False
-    src = c.g.nodes[node.inputs[0]]
-    rank = len(src.output.shape)
-    if node.op.axis != rank - 1:
-        raise FusionError("sum / mean over a non-innermost axis is not supported")
+    # any other axis is moved last by a dense copy; what is left of the shape keeps its order, so the result needs no view
+    xv, _ = _axis_last(c, nid, node.inputs[0], node.op.axis)
+    rows, x_addr = _row_addr(xv)
+    cols = int(xv.shape[-1])
+    project = E.Var("s") / float(cols) if isinstance(node.op, F.MeanOp) else E.Var("s")
+    monoid, label = ("max", "amax_reduce") if isinstance(node.op, F.AmaxOp) else ("sum", "mean_reduce" if isinstance(node.op, F.MeanOp) else "sum_reduce")
+    body = RowReduce(rows=rows, cols=cols, x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=node.output.dtype, stats=(Stat("s", monoid, E.Var("x")),), project=project, x_addr=x_addr, scalar_out=True)
+    _emit(c, nid, body, label, [xv.base])
+    return True
+
+
+def _dense(c: _Ctx, v: View, new_id: str) -> View:
+    """``v`` itself when it enumerates its memory in row-major order, else a dense copy."""
+    if v.strides == contiguous_strides(v.shape):
+        return v
+    return _copy_of_view(c, v, tuple(range(len(v.shape))), new_id)
+
+
+def _rec_gather(c: _Ctx, nid: str) -> bool:
+    """Embedding lookup / ``index_select``: one kernel that copies the picked slices."""
+    from deplodock_amd.ir.tile import IndexRows
+
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.GatherOp):
+        return False
+    xv = _dense(c, _need(c, node.inputs[0]), f"{nid}__table")
+    iv = _dense(c, _need(c, node.inputs[1]), f"{nid}__index")
+    axis = node.op.axis
+    shape = tuple(int(d) for d in xv.shape)
+    outer = math.prod(shape[:axis])
+    inner = math.prod(shape[axis + 1 :])
+    count = int(iv.numel)
+    if xv.offset or iv.offset:
+        raise FusionError(f"gather {nid!r}: operands must start at their buffers' first element")
+    body = IndexRows(src=xv.base, idx=iv.base, out=nid, dtype=xv.dtype, idx_dtype=iv.dtype, outer=outer, n=shape[axis], inner=inner, count=count)
+    _emit(c, nid, body, "index_rows", [xv.base, iv.base])
+    return True
+
+
+def _rec_cat(c: _Ctx, nid: str) -> bool:
+    """``cat`` along one axis as a loop nest over the result: every point loads (index clamped into range) from each
+    piece and keeps the one its position falls in — the reference lowers ``cat`` to the same index-mapped select
+    (decomposition/150_cat.py)."""
+    from deplodock_amd.ir import loopnest as L
+    from deplodock_amd.ir.tile import LoopNest
+
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.CatOp):
+        return False
+    out_shape = tuple(int(d) for d in node.output.shape)
+    dim = node.op.dim
+    axes = [L.Var(f"c{i}") for i in range(len(out_shape))]
+    stmts: list = []
+    branches: list = []
+    operands: dict = {}
+    inputs: list[str] = []
+    lo = 0
+    for k, src in enumerate(node.inputs):
+        v = _need(c, src)
+        if not all(isinstance(d, int) for d in (*v.shape, *v.strides, v.offset)):
+            raise FusionError("cat: static shapes only")
+        n = int(v.shape[dim])
+        hi = lo + n
+        inside = L.Bin("&&", L.Bin(">=", axes[dim], L.Lit(lo)), L.Bin("<", axes[dim], L.Lit(hi)))
+        at: object = L.Lit(int(v.offset))
+        for i, st in enumerate(v.strides):
+            if not st:
+                continue
+            e = L.Ternary(inside, L.Bin("-", axes[dim], L.Lit(lo)), L.Lit(0)) if i == dim else axes[i]
+            at = L.Bin("+", at, L.Bin("*", e, L.Lit(int(st))))
+        operands[f"s{k}"] = (v.base, (int(c.out.nodes[v.base].output.numel),), v.dtype)
+        inputs.append(v.base)
+        stmts.append(L.Load(f"t{k}", f"s{k}", (at,)))
+        branches.append((f"t{k}", L.Bin("<", axes[dim], L.Lit(hi)) if k < len(node.inputs) - 1 else L.Lit(1)))
+        lo = hi
+    if lo != out_shape[dim]:
+        raise FusionError(f"cat {nid!r}: the pieces add up to {lo}, the result has {out_shape[dim]}")
+    body: tuple = (*stmts, L.Select("u", tuple(branches)), L.Write(nid, tuple(axes), "u"))
+    for i in reversed(range(len(out_shape))):
+        body = (L.Loop(f"c{i}", out_shape[i], body),)
+    nest = LoopNest(stmts=body, operands=operands, scalars={}, out=nid, out_name=nid, out_shape=out_shape, out_dtype=node.output.dtype)
+    _emit(c, nid, nest, "cat", inputs)
+    return True
+
+
+def _rec_layer_norm(c: _Ctx, nid: str) -> bool:
+    """LayerNorm over the last axis as one register-resident row kernel: the mean, then the centred sum of squares
+    (a second statistic over the resident row, which is what keeps the variance free of cancellation), then the
+    projection; computed in fp32 and rounded once, as ``nn.LayerNorm`` does."""
+    node = c.g.nodes[nid]
+    if not isinstance(node.op, F.LayerNormOp):
+        return False
     xv = _need(c, node.inputs[0])
     if xv.strides[-1] != 1:
-        raise FusionError("sum / mean: the reduced axis must be contiguous")
+        xv = _copy_of_view(c, xv, tuple(range(len(xv.shape))), f"{nid}__rows")
     rows, x_addr = _row_addr(xv)
-    cols = int(src.output.shape[-1])
-    project = E.Var("s") / float(cols) if isinstance(node.op, F.MeanOp) else E.Var("s")
-    body = RowReduce(rows=rows, cols=cols, x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=node.output.dtype, stats=(Stat("s", "sum", E.Var("x")),), project=project, x_addr=x_addr, scalar_out=True)
-    _emit(c, nid, body, "mean_reduce" if isinstance(node.op, F.MeanOp) else "sum_reduce", [xv.base])
+    cols = int(xv.shape[-1])
+    x = E.Var("x")
+    mean = E.Var("s1") / float(cols)
+    stats = (Stat("s1", "sum", x), Stat("s2", "sum", (x - mean) * (x - mean)))
+    project = (x - mean) * E.Un("rsqrt", E.Var("s2") / float(cols) + node.op.eps)
+    col_ops, buffers, inputs = [], {}, [xv.base]
+    for name, src, on in (("w", 1, node.op.has_weight), ("b", 2, node.op.has_bias)):
+        if not on:
+            continue
+        pv = _need(c, node.inputs[src])
+        if not pv.is_contiguous() or pv.offset or pv.numel != cols:
+            raise FusionError(f"layer_norm: the {'weight' if name == 'w' else 'bias'} must be a plain vector of the normalised width")
+        col_ops.append((name, pv.dtype))
+        buffers[name] = pv.base
+        inputs.append(pv.base)
+        project = project * E.Var("w") if name == "w" else project + E.Var("b")
+    body = RowReduce(rows=rows, cols=cols, x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=node.output.dtype, stats=stats, project=project, col_operands=tuple(col_ops), x_addr=x_addr)
+    body.operand_buffers = buffers
+    _emit(c, nid, body, "layer_norm_reduce", inputs)
     return True
 
 
@@ -1049,7 +1172,8 @@ def _need_logical(c: _Ctx, nid: str) -> View:
 
 
 _POINTWISE_FN = {"add": "add", "sub": "sub", "mul": "mul", "div": "div", "maximum": "max", "minimum": "min"}
-_POINTWISE_UN = {"neg": "neg", "rsqrt": "rsqrt", "sqrt": "sqrt", "exp": "exp", "silu": "silu", "sigmoid": "sigmoid", "tanh": "tanh", "abs": "abs", "reciprocal": "rcp"}
+_POINTWISE_UN = {"neg": "neg", "rsqrt": "rsqrt", "sqrt": "sqrt", "exp": "exp", "silu": "silu", "sigmoid": "sigmoid", "tanh": "tanh", "abs": "abs", "reciprocal": "rcp",
+                 "relu": "relu", "erf": "erf", "gelu": "gelu", "gelu_tanh": "gelu_tanh"}  # fmt: skip
 
 
 def _pointwise_node_expr(op, args: list[E.Expr]) -> E.Expr | None:
@@ -1062,6 +1186,13 @@ def _pointwise_node_expr(op, args: list[E.Expr]) -> E.Expr | None:
         return E.Un(_POINTWISE_UN[op.fn], args[0])
     if op.fn == "pow" and op.scalar == 2.0:
         return args[0] * args[0]
+    if op.fn == "pow" and op.scalar is not None and not op.scalar_first and float(op.scalar) in (1.0, 3.0, 4.0):
+        out = args[0]  # small whole powers as products (the reference's decomposition/030_pow.py does the same)
+        for _ in range(int(op.scalar) - 1):
+            out = out * args[0]
+        return out
+    if op.fn == "pow" and len(args) == 1 and op.scalar is not None:
+        return E.Bin("pow", E.Const(op.scalar), args[0]) if op.scalar_first else E.Bin("pow", args[0], E.Const(op.scalar))
     if op.fn in _POINTWISE_FN:
         if op.scalar is not None:
             a, b = (E.Const(op.scalar), args[0]) if op.scalar_first else (args[0], E.Const(op.scalar))

@@ -15,7 +15,7 @@ from dataclasses import replace
 
 from deplodock_amd.context import Context
 from deplodock_amd.emit.contraction import emit_contraction
-from deplodock_amd.emit.copy import emit_strided_copy
+from deplodock_amd.emit.copy import emit_index_rows, emit_strided_copy
 from deplodock_amd.emit.flash import emit_flash
 from deplodock_amd.emit.loopnest import emit_loop_nest
 from deplodock_amd.emit.pointwise import emit_map
@@ -26,7 +26,7 @@ from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.emit.splitk import emit_splitk_combine, partial_body, split_planes
 from deplodock_amd.graph import Graph, Node, Tensor
 from deplodock_amd.ir.hip import HipOp
-from deplodock_amd.ir.tile import Contraction, Flash, LoopNest, Map, RowReduce, StridedCopy, TileOp
+from deplodock_amd.ir.tile import Contraction, Flash, IndexRows, LoopNest, Map, RowReduce, StridedCopy, TileOp
 
 _PLACEHOLDER = "EMH_KERNEL_NAME_"
 logger = logging.getLogger(__name__)
@@ -120,6 +120,8 @@ def lower_tile(op: TileOp, ctx: Context) -> HipOp:
         hip = emit_loop_nest(body, _PLACEHOLDER, ctx)
     elif isinstance(body, StridedCopy):
         hip = emit_strided_copy(body, _PLACEHOLDER, ctx)
+    elif isinstance(body, IndexRows):
+        hip = emit_index_rows(body, _PLACEHOLDER, ctx)
     else:
         raise TypeError(f"unknown tile body {type(body).__name__}")
     return _named(hip, op)

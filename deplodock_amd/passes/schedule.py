@@ -25,7 +25,7 @@ from deplodock_amd import config
 from deplodock_amd.context import Context
 from deplodock_amd.graph import Graph
 from deplodock_amd.ir.schedule import ATOMS, ReducePlan, ScheduleError, Stage, TilePlan
-from deplodock_amd.ir.tile import Contraction, Flash, LoopNest, Map, RowReduce, StridedCopy, TileOp
+from deplodock_amd.ir.tile import Contraction, Flash, IndexRows, LoopNest, Map, RowReduce, StridedCopy, TileOp
 
 logger = logging.getLogger(__name__)
 
@@ -611,7 +611,7 @@ def schedule(graph: Graph, ctx: Context | None = None) -> Graph:
             op.knobs.update(schedule_contraction(body, ctx))
         elif isinstance(body, Flash):
             op.knobs.update(schedule_flash(body, ctx))
-        elif isinstance(body, (Map, LoopNest, StridedCopy)):
+        elif isinstance(body, (Map, LoopNest, StridedCopy, IndexRows)):
             pass  # nothing to plan: a map is sized by its extent, a loop nest by its outer loops
         else:
             raise TypeError(f"unknown tile body {type(body).__name__}")

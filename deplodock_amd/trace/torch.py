@@ -203,6 +203,26 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
         if t == aten.rms_norm.default:
             x, _shape_arg, w, eps = (list(a) + [None, None])[:4]
             add(node, F.RmsNormOp(eps=float(eps if eps is not None else 1e-6), has_weight=w is not None), [x] + ([w] if w is not None else []))
+        elif t == aten.embedding.default:
+            add(node, F.GatherOp(axis=0), [a[0], a[1]])
+        elif t == aten.index_select.default:
+            if len(a[2].meta["val"].shape) != 1:
+                raise TraceError("index_select: the index must be a vector")
+            env[node.name] = g.add_node(F.GatherOp(axis=_norm_dim(int(a[1]), rank_in)), [env[a[0].name], env[a[2].name]], out_tensor(node), node.name)
+        elif t == aten.layer_norm.default:
+            x, nshape, w, b, eps = (list(a) + [None] * 5)[:5]
+            if len(nshape) != 1 or int(nshape[0]) != int(x.meta["val"].shape[-1]):
+                raise TraceError("layer_norm: only the last axis can be normalised")
+            if b is not None and w is None:
+                raise TraceError("layer_norm: a bias without a weight is not supported")
+            add(node, F.LayerNormOp(eps=float(eps if eps is not None else 1e-5), has_weight=w is not None, has_bias=b is not None), [x] + [p_ for p_ in (w, b) if p_ is not None])
+        elif t == aten.amax.default:
+            dims = a[1] if len(a) > 1 else []
+            dims = list(dims) if isinstance(dims, (list, tuple)) else [dims]
+            if len(dims) != 1:
+                raise TraceError("multi-axis reductions are not supported")
+            keep = bool(a[2]) if len(a) > 2 else bool(kw.get("keepdim", False))
+            add(node, F.AmaxOp(axis=_norm_dim(int(dims[0]), rank_in), keepdim=keep), [a[0]])
         elif t in (aten.softmax.int, aten._softmax.default):
             add(node, F.SoftmaxOp(axis=_norm_dim(int(a[1]), rank_in)), [a[0]])
         elif t == aten.linear.default:
@@ -265,6 +285,19 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
             add(node, F.CatOp(dim=dim), tensors)
         elif t in (aten.contiguous.default, aten.clone.default, aten.alias.default, aten.detach.default):
             add(node, F.ContiguousOp(), [a[0]])
+        elif t == aten.gelu.default:
+            # the tanh approximation is an op of its own, as in the reference (emmy/compiler/trace/torch.py:512-517)
+            add(node, F.ElementwiseOp(fn="gelu_tanh" if kw.get("approximate", "none") == "tanh" else "gelu"), [a[0]])
+        elif t == aten.t.default:
+            if rank_in != 2:
+                raise TraceError("aten.t: expected a matrix")
+            add(node, F.TransposeOp(dim0=0, dim1=1), [a[0]])
+        elif t == aten.addmm.default:
+            # bias + a @ b (GPT-2's Conv1D): a matmul node, then the broadcast add (emmy/compiler/trace/torch.py:548-557)
+            if kw.get("beta", 1) != 1 or kw.get("alpha", 1) != 1:
+                raise TraceError("aten.addmm: beta / alpha other than 1 are not supported")
+            mm_id = g.add_node(F.MatmulOp(), [env[a[1].name], env[a[2].name]], out_tensor(node).__class__(f"{node.name}__mm", out_tensor(node).shape, out_tensor(node).dtype), f"{node.name}__mm")
+            env[node.name] = g.add_node(F.ElementwiseOp(fn="add"), [mm_id, env[a[0].name]], out_tensor(node), node.name)
         elif t in _UNARY:
             add(node, F.ElementwiseOp(fn=_UNARY[t]), [a[0]])
         elif t in _BINARY:
@@ -298,6 +331,8 @@ def _tables():
         aten.tanh.default: "tanh",
         aten.abs.default: "abs",
         aten.reciprocal.default: "reciprocal",
+        aten.relu.default: "relu",
+        aten.erf.default: "erf",
     }
     binary = {
         aten.add.Tensor: "add",

