@@ -168,6 +168,8 @@ class HipBackend(Backend):
                     ks = data[stacked.k_scale] if stacked.k_scale in data else traced[stacked.k_scale]
                     ks = ks if isinstance(ks, torch.Tensor) else torch.as_tensor(ks)
                     whole = (whole.float() * ks.to(whole.device).float().reshape(1, -1)).to(whole.dtype)
+                if stacked.transpose:
+                    whole = whole.transpose(-1, -2).contiguous()
                 data[nid] = whole
             elif nid in traced:
                 data[nid] = traced[nid]

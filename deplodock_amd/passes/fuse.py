@@ -54,6 +54,7 @@ class StackedConstant:
 
     parts: tuple[str, ...]
     k_scale: str | None = None  # a length-k constant multiplied into every row (a norm weight folded into the projection)
+    transpose: bool = False  # the last two axes swapped afterwards (a ``[K, N]`` weight of ``x @ w`` stored as the ``[N, K]`` rows a contraction reads)
 
 
 @dataclass
@@ -273,10 +274,26 @@ def _a_operand(c: _Ctx, x_id: str, absorbers: set[str], fold: bool = False) -> t
     return _need(c, x_id), None, [], None
 
 
+def _transposed_parameter(c: _Ctx, w: View) -> View:
+    """``w`` as ``[N, K]`` rows when it is the transposed view of a dense ``[K, N]`` parameter: the transposition is
+    done once, when the program is bound (a constant assembled from the parameter), instead of by a copy per run."""
+    base = c.out.nodes.get(w.base)
+    if len(w.shape) != 2 or w.strides[-1] == 1 or base is None or not isinstance(base.op, ConstantOp) or base.op.value is not None:
+        return w
+    n, k = int(w.shape[0]), int(w.shape[1])
+    if w.offset != 0 or tuple(w.strides) != (1, n) or tuple(int(d) for d in base.output.shape) != (k, n):
+        return w
+    tid = f"{w.base}__t"
+    if tid not in c.out.nodes:
+        c.out.add_constant(tid, (n, k), w.dtype)
+        c.out.nodes[tid].hints["stacked"] = StackedConstant((w.base,), transpose=True)
+    return View(tid, 0, (n, k), (k, 1), w.dtype)
+
+
 def _linear_parts(c: _Ctx, nid: str):
     node = c.g.nodes[nid]
     x, pro, extra, _ = _a_operand(c, node.inputs[0], {nid})
-    w = _need(c, node.inputs[1])
+    w = _transposed_parameter(c, _need(c, node.inputs[1]))
     m, k, lda = _matrix(x, "linear input")
     n, k2, ldb = _matrix(w, "linear weight")
     if k != k2:
@@ -390,6 +407,8 @@ def _rec_matmul(c: _Ctx, nid: str) -> bool:
     rb = len(b.shape)
     order_b = (*range(rb - 2), rb - 1, rb - 2)  # [..., N, K]
     bt = View(b.base, b.offset, tuple(b.shape[i] for i in order_b), tuple(b.strides[i] for i in order_b), b.dtype)
+    if rb == 2:
+        bt = _transposed_parameter(c, bt)  # a parameter stored [K, N] (GPT-2's Conv1D): transposed once, when the program is bound
     if rb == 2 and len(a.shape) > 2:
         bt = View(bt.base, bt.offset, (*(1,) * (len(a.shape) - 2), *bt.shape), (*(0,) * (len(a.shape) - 2), *bt.strides), bt.dtype)
     _emit_batched_contraction(c, nid, a, bt, "matmul")
@@ -463,8 +482,11 @@ def _rec_linear_residual(c: _Ctx, nid: str) -> bool:
         return False
     for li, ri in ((0, 1), (1, 0)):
         lin_id, res_id = node.inputs[li], node.inputs[ri]
+        # a reshape of the projection's rows between it and the add (``y.view(batch, seq, n) + residual``) changes nothing in memory
+        while isinstance(c.g.nodes[lin_id].op, F.ViewOp) and c.single_use(lin_id) and lin_id not in c.done and c.g.nodes[lin_id].output.shape[-1] == c.g.nodes[c.g.nodes[lin_id].inputs[0]].output.shape[-1]:
+            lin_id = c.g.nodes[lin_id].inputs[0]
         lin = c.g.nodes[lin_id]
-        if not (isinstance(lin.op, F.LinearOp) and c.single_use(lin_id)):
+        if not (isinstance(lin.op, F.LinearOp) and c.single_use(lin_id)) or lin_id in c.done:
             continue
         if c.g.nodes[res_id].output.shape != node.output.shape or c.g.nodes[res_id].output.dtype != node.output.dtype:
             continue

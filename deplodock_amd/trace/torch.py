@@ -173,6 +173,7 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
         env[node.name] = g.add_node(op, [env[i.name] for i in inputs], out_tensor(node), node.name)
 
     aten = torch.ops.aten
+    tuples: dict[str, list[str]] = {}  # split / chunk node -> the node ids of its pieces
     for node in ep.graph.nodes:
         if node.op == "placeholder":
             spec = kinds[node.name]
@@ -199,7 +200,30 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
         if t in (aten._assert_tensor_metadata.default,):
             continue
         if t is operator.getitem:
-            raise TraceError("tuple-valued ops are not supported")
+            parts = tuples.get(getattr(a[0], "name", None))
+            if parts is None:
+                raise TraceError("tuple-valued ops other than split / chunk are not supported")
+            env[node.name] = parts[int(a[1])]
+            continue
+        if t in (aten.split.Tensor, aten.split_with_sizes.default, aten.chunk.default):
+            # the pieces are slices (views) of the operand, picked by the getitem nodes that follow
+            dim = _norm_dim(int(a[2]) if len(a) > 2 else int(kw.get("dim", 0)), rank_in)
+            size = int(a[0].meta["val"].shape[dim])
+            if t == aten.split_with_sizes.default:
+                sizes = [int(n) for n in a[1]]
+            else:
+                step = int(a[1]) if t == aten.split.Tensor else -(-size // int(a[1]))
+                sizes = [min(step, size - lo) for lo in range(0, size, step)]
+            parts, lo = [], 0
+            for i, (n, val) in enumerate(zip(sizes, node.meta["val"])):
+                pid = f"{node.name}__{i}"
+                parts.append(g.add_node(F.SliceOp(dim=dim, start=lo, end=lo + n, step=1), [env[a[0].name]], Tensor(pid, _shape(val), dt.from_torch(val.dtype)), pid))
+                lo += n
+            tuples[node.name] = parts
+            continue
+        if t in (aten.dropout.default, aten.native_dropout.default) and not (a[2] if len(a) > 2 else kw.get("train", False)):
+            env[node.name] = env[a[0].name]  # inference: the identity
+            continue
         if t == aten.rms_norm.default:
             x, _shape_arg, w, eps = (list(a) + [None, None])[:4]
             add(node, F.RmsNormOp(eps=float(eps if eps is not None else 1e-6), has_weight=w is not None), [x] + ([w] if w is not None else []))
@@ -296,8 +320,15 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
             # bias + a @ b (GPT-2's Conv1D): a matmul node, then the broadcast add (emmy/compiler/trace/torch.py:548-557)
             if kw.get("beta", 1) != 1 or kw.get("alpha", 1) != 1:
                 raise TraceError("aten.addmm: beta / alpha other than 1 are not supported")
-            mm_id = g.add_node(F.MatmulOp(), [env[a[1].name], env[a[2].name]], out_tensor(node).__class__(f"{node.name}__mm", out_tensor(node).shape, out_tensor(node).dtype), f"{node.name}__mm")
-            env[node.name] = g.add_node(F.ElementwiseOp(fn="add"), [mm_id, env[a[0].name]], out_tensor(node), node.name)
+            ot = out_tensor(node)
+            w_val, b_val = a[2].meta["val"], a[0].meta["val"]
+            if a[2].op == "placeholder" and kinds[a[2].name].kind.name != "USER_INPUT" and len(b_val.shape) == 1:
+                # a parameter: ``linear`` over its transposed view, so the bias rides in the contraction and the weight is transposed at bind time
+                wt = g.add_node(F.TransposeOp(dim0=0, dim1=1), [env[a[2].name]], Tensor(f"{node.name}__wt", (_shape(w_val)[1], _shape(w_val)[0]), ot.dtype), f"{node.name}__wt")
+                env[node.name] = g.add_node(F.LinearOp(has_bias=True), [env[a[1].name], wt, env[a[0].name]], ot, node.name)
+            else:
+                mm_id = g.add_node(F.MatmulOp(), [env[a[1].name], env[a[2].name]], Tensor(f"{node.name}__mm", ot.shape, ot.dtype), f"{node.name}__mm")
+                env[node.name] = g.add_node(F.ElementwiseOp(fn="add"), [mm_id, env[a[0].name]], ot, node.name)
         elif t in _UNARY:
             add(node, F.ElementwiseOp(fn=_UNARY[t]), [a[0]])
         elif t in _BINARY:

@@ -1418,3 +1418,73 @@ def test_frontend_op_coverage(device, case, dtype):
     if case in ("embedding", "index_select", "cat_last", "cat_first", "rotate_half") and dtype is torch.float32:
         assert torch.equal(ours.reshape(want.shape), want) or case == "cat_first"  # pure data movement is exact
     eager.assert_close(ours.reshape(want.shape).float(), want, rtol, atol, f"{case} {dtype}")
+
+
+class _FirstOutput(nn.Module):
+    def __init__(self, inner):
+        super().__init__()
+        self.inner = inner
+
+    def forward(self, x):
+        out = self.inner(x)
+        return out[0] if isinstance(out, tuple) else out
+
+
+def _gpt2_block():
+    from transformers import GPT2Config
+    from transformers.models.gpt2.modeling_gpt2 import GPT2Block
+
+    cfg = GPT2Config(n_embd=256, n_head=4, n_layer=1, n_positions=128)
+    cfg._attn_implementation = "sdpa"
+    return _FirstOutput(GPT2Block(cfg, 0))
+
+
+def _bert_layer():
+    from transformers import BertConfig
+    from transformers.models.bert.modeling_bert import BertLayer
+
+    cfg = BertConfig(hidden_size=256, num_attention_heads=4, intermediate_size=1024, num_hidden_layers=1)
+    cfg._attn_implementation = "sdpa"
+    return _FirstOutput(BertLayer(cfg))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("family", ["gpt2", "bert"])
+def test_layers_of_other_model_families(device, family, dtype):
+    """A GPT-2 block (LayerNorm, Conv1D = ``addmm`` over ``[K, N]`` parameters, ``split``, tanh-GELU spelled out,
+    causal attention) and a BERT layer (LayerNorm after the residual, erf-GELU, biased projections, inference
+    dropout) as ``transformers`` builds them: against the module in float64."""
+    import copy
+
+    torch.manual_seed(71)
+    mod = (_gpt2_block if family == "gpt2" else _bert_layer)()
+    with torch.no_grad():
+        for name, p in mod.named_parameters():
+            p.copy_(1 + 0.1 * torch.randn_like(p) if ("ln" in name.lower() or "norm" in name.lower()) and name.endswith("weight") else 0.05 * torch.randn_like(p))
+    mod = mod.to(dtype).eval()
+    x = torch.randn(2, 64, 256).to(dtype)
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, (x,)))
+    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert "k_layer_norm_reduce" in names
+    if family == "gpt2":
+        assert names[1].startswith("k_linear")  # the Conv1D weight is transposed at bind time: no copy kernel in front of the projection
+    if dtype is torch.bfloat16:
+        assert names.count("k_sdpa_reduce") == 1 and names.count("k_linear_add") == 2
+    prog = be.program(compiled, {compiled.inputs[0]: x.to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone().cpu()
+    finally:
+        prog.close()
+    with torch.no_grad():
+        want = copy.deepcopy(mod).double()(x.double()).float()
+        half = copy.deepcopy(mod)(x).float()  # what eager makes of it in the same precision
+    rms = float(want.pow(2).mean().sqrt())
+    if dtype is torch.float32:
+        eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-4 * rms, f"{family} fp32 vs float64")
+    else:
+        eager.assert_close(ours.reshape(want.shape).float(), want, 2e-2, 4e-2 * max(rms, 1.0), f"{family} bf16 vs float64")
+        eager.assert_mean_error_within_baseline(ours.reshape(want.shape).float(), half, want, 1.5, f"{family} bf16: mean error against eager bf16's")
