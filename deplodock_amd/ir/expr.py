@@ -232,6 +232,21 @@ def variables(e: Expr) -> set[str]:
     raise TypeError(type(e).__name__)
 
 
+def substitute(e: Expr, table: dict[str, Expr]) -> Expr:
+    """``e`` with every variable named in ``table`` replaced by its entry (other variables stay)."""
+    if isinstance(e, Var):
+        return table.get(e.name, e)
+    if isinstance(e, Const):
+        return e
+    if isinstance(e, Un):
+        return Un(e.op, substitute(e.a, table))
+    if isinstance(e, Round):
+        return Round(e.dtype, substitute(e.a, table))
+    if isinstance(e, Bin):
+        return Bin(e.op, substitute(e.a, table), substitute(e.b, table))
+    raise TypeError(type(e).__name__)
+
+
 def pretty(e: Expr) -> str:
     if isinstance(e, Var):
         return e.name

@@ -147,7 +147,7 @@ def _materialize(c: _Ctx, nid: str) -> None:
             c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
         c.done[nid] = nid
         return
-    for rec in (_rec_same_type_cast, _rec_loop_nest, _rec_batched_linear, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_layer_norm, _rec_softmax, _rec_sdpa, _rec_row_sum, _rec_gather, _rec_cat, _rec_pointwise):
+    for rec in (_rec_same_type_cast, _rec_loop_nest, _rec_batched_linear, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_layer_norm, _rec_softmax, _rec_sdpa, _rec_row_fused, _rec_row_sum, _rec_gather, _rec_cat, _rec_pointwise):
         if rec(c, nid):
             return
     raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
@@ -1227,6 +1227,114 @@ def _pointwise_node_expr(op, args: list[E.Expr]) -> E.Expr | None:
 
 
 _MAX_FUSED_POINTWISE = 24  # ops folded into one map kernel
+
+
+def _rec_row_fused(c: _Ctx, nid: str) -> bool:
+    """An element-wise tree whose leaves include ``keepdim`` reductions over the last axis of element-wise functions
+    of the *same* rows (a normalisation spelled out: Gemma's ``x * rsqrt(mean(x^2) + eps) * (1 + w)``, a hand-written
+    layer norm, ``x - x.amax(-1, keepdim=True)``) as one register-resident row kernel: each reduction is a row
+    statistic, the rest is the projection.  Casts are folded wherever they are read (recomputed, never stored);
+    anything the row kernel has no operand form for leaves the match to the one-op-per-kernel fallbacks."""
+    g = c.g
+    node = g.nodes[nid]
+    if not isinstance(node.op, (F.CastOp, F.ElementwiseOp)) or nid in c.done:
+        return False
+    shape = tuple(node.output.shape)
+    if len(shape) < 1 or not all(isinstance(d, int) for d in shape) or shape[-1] < 2:
+        return False
+    stat_shape = (*shape[:-1], 1)
+    cols = int(shape[-1])
+    leaves: dict[str, E.Var] = {}
+    stats: list[Stat] = []
+    stat_of: dict[str, E.Expr] = {}
+    folded = [0]
+
+    class _Decline(Exception):
+        pass
+
+    def build(cur: str, root: bool) -> E.Expr:
+        n = g.nodes[cur]
+        nshape = tuple(n.output.shape)
+        if cur in stat_of:
+            return stat_of[cur]
+        if isinstance(n.op, (F.MeanOp, F.SumOp, F.AmaxOp)) and cur not in c.done and n.op.keepdim and nshape == stat_shape and n.op.axis == len(shape) - 1 \
+                and tuple(g.nodes[n.inputs[0]].output.shape) == shape and c.single_use(cur):  # fmt: skip
+            pre = build(n.inputs[0], False)
+            name = f"s{len(stats)}"
+            stats.append(Stat(name, "max" if isinstance(n.op, F.AmaxOp) else "sum", pre))
+            stat_of[cur] = _round(n.output.dtype, E.Var(name) / float(cols) if isinstance(n.op, F.MeanOp) else E.Var(name))
+            return stat_of[cur]
+        elementwise = isinstance(n.op, (F.CastOp, F.ElementwiseOp)) and cur not in c.done and nshape in (shape, stat_shape)
+        foldable = elementwise and (root or isinstance(n.op, F.CastOp) or c.single_use(cur)) and folded[0] < _MAX_FUSED_POINTWISE
+        if not foldable:
+            if cur not in leaves:
+                leaves[cur] = E.Var(f"a{len(leaves)}")
+            return leaves[cur]
+        folded[0] += 1
+        args = [build(i, False) for i in n.inputs]
+        e = _pointwise_node_expr(n.op, args)
+        if e is None:
+            raise _Decline
+        return _round(n.output.dtype, e)
+
+    try:
+        project = build(nid, True)
+    except (_Decline, FusionError):
+        return False
+    if not stats:
+        return False
+    # operands: the resident row (the one tensor the statistics read), further tensors of the rows' shape (a residual),
+    # vectors along the row
+    in_stats = set().union(*(E.variables(st.pre) for st in stats))
+    x_leaf, col_ops, row_ops, buffers, inputs = None, [], [], {}, []
+    rename: dict[str, E.Expr] = {}
+    for leaf_id, var in leaves.items():
+        t = g.nodes[leaf_id].output
+        lshape = tuple(t.shape)
+        if lshape == shape and var.name in in_stats:
+            if x_leaf is not None:
+                return False
+            x_leaf = leaf_id
+            rename[var.name] = E.Var("x")
+        elif lshape == shape:
+            v = _need(c, leaf_id)
+            if v.strides != contiguous_strides(v.shape):
+                return False
+            name = f"r{len(row_ops)}"
+            row_ops.append((name, v))
+            rename[var.name] = E.Var(name)
+        elif len(lshape) >= 1 and lshape[-1] == cols and all(d == 1 for d in lshape[:-1]):
+            v = _need(c, leaf_id)
+            if v.strides[-1] != 1 or v.offset:
+                return False
+            name = f"w{len(col_ops)}"
+            col_ops.append((name, v.dtype))
+            buffers[name] = v.base
+            inputs.append(v.base)
+            rename[var.name] = E.Var(name)
+        elif isinstance(g.nodes[leaf_id].op, ConstantOp) and g.nodes[leaf_id].op.value is not None and t.numel == 1:
+            rename[var.name] = E.Const(float(g.nodes[leaf_id].op.value))
+        else:
+            return False
+    if x_leaf is None:
+        return False
+    xv = _need(c, x_leaf)
+    if xv.strides[-1] != 1:
+        return False
+    try:
+        rows, x_addr = _row_addr(xv)
+    except FusionError:
+        return False
+    sub = lambda e: E.substitute(e, rename)  # noqa: E731
+    for name, v in row_ops:
+        buffers[name] = v.base
+        inputs.append(v.base)
+    body = RowReduce(rows=rows, cols=cols, x=xv.base, x_dtype=xv.dtype, out=nid, out_dtype=node.output.dtype,
+                     stats=tuple(Stat(st.name, st.monoid, sub(st.pre)) for st in stats), project=sub(project), col_operands=tuple(col_ops),
+                     row_operands=tuple(RowOperand(name, v.dtype, div=1, mod=rows, offset=int(v.offset)) for name, v in row_ops), x_addr=x_addr)  # fmt: skip
+    body.operand_buffers = buffers
+    _emit(c, nid, body, "row_fused_reduce", [xv.base, *inputs])
+    return True
 
 
 def _rec_pointwise(c: _Ctx, nid: str) -> bool:

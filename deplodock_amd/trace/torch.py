@@ -270,6 +270,8 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
             scale = kw.get("scale")
             add(node, F.SdpaOp(is_causal=causal, scale=None if scale is None else float(scale), enable_gqa=bool(kw.get("enable_gqa", False)), has_mask=mask is not None),
                 [a[0], a[1], a[2]] + ([mask] if mask is not None else []))  # fmt: skip
+        elif t == aten.type_as.default:
+            add(node, F.CastOp(dtype=dt.from_torch(a[1].meta["val"].dtype)), [a[0]])
         elif t in (aten.to.dtype, aten._to_copy.default, aten.to.dtype_layout):
             target = a[1] if len(a) > 1 and isinstance(a[1], torch.dtype) else kw.get("dtype")
             add(node, F.CastOp(dtype=dt.from_torch(target)), [a[0]])

@@ -1353,6 +1353,19 @@ class _Fn(nn.Module):
         return self.fn(*args)
 
 
+class _GemmaNorm(nn.Module):
+    """Gemma's RMSNorm: computed in fp32, scaled by ``1 + weight``, cast back last."""
+
+    def __init__(self, dim: int):
+        super().__init__()
+        self.weight = nn.Parameter(0.1 * torch.randn(dim))
+
+    def forward(self, t):
+        f = t.float()
+        out = f * torch.rsqrt(f.pow(2).mean(-1, keepdim=True) + 1e-6)
+        return (out * (1.0 + self.weight.float())).type_as(t)
+
+
 def _op_cases():
     Fn = torch.nn.functional
     x = lambda *s: torch.randn(*s)  # noqa: E731
@@ -1384,6 +1397,11 @@ def _op_cases():
         "cat_first": (_Fn(lambda a, b: torch.cat([a, b * 2], 0)), lambda: (x(3, 8, 24), x(5, 8, 24))),
         "cat_three_slices": (_Fn(lambda a, b: torch.cat([a[..., :10], b, a[..., 5:9]], -1)), lambda: (x(4, 32, 24), x(4, 32, 7))),
         "rotate_half": (_Fn(lambda t: torch.cat((-t[..., 64:], t[..., :64]), -1)), lambda: (x(2, 8, 50, 128),)),
+        # normalisations spelled out with keepdim reductions: one fused row kernel each
+        "gemma_rms_norm": (_GemmaNorm(256), lambda: (x(4, 33, 256),)),
+        "manual_layer_norm": (_Fn(lambda t: (t - t.mean(-1, keepdim=True)) * torch.rsqrt((t - t.mean(-1, keepdim=True)).pow(2).mean(-1, keepdim=True) + 1e-5)), lambda: (2 + x(5, 40, 200),)),
+        "shift_by_row_max": (_Fn(lambda t: torch.exp(t - t.amax(-1, keepdim=True))), lambda: (3 * x(6, 300),)),
+        "residual_plus_norm": (_Fn(lambda t, r: r + t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + 1e-6)), lambda: (x(4, 33, 256), x(4, 33, 256))),
         # a transformer MLP of the GELU family, and a pre-norm projection
         "gelu_mlp": (nn.Sequential(nn.Linear(256, 512), nn.GELU(), nn.Linear(512, 256)), lambda: (x(2, 48, 256),)),
         "layer_norm_linear": (nn.Sequential(nn.LayerNorm(256), nn.Linear(256, 128)), lambda: (x(4, 33, 256),)),
@@ -1446,6 +1464,71 @@ def _bert_layer():
     cfg = BertConfig(hidden_size=256, num_attention_heads=4, intermediate_size=1024, num_hidden_layers=1)
     cfg._attn_implementation = "sdpa"
     return _FirstOutput(BertLayer(cfg))
+
+
+class _RotaryLayer(nn.Module):
+    def __init__(self, layer):
+        super().__init__()
+        self.layer = layer
+
+    def forward(self, x, cos, sin):
+        out = self.layer(x, position_embeddings=(cos, sin), attention_mask=None)
+        return out[0] if isinstance(out, tuple) else out
+
+
+_DECODER_FAMILIES = {
+    "llama": ("LlamaConfig", "LlamaDecoderLayer", "LlamaRotaryEmbedding", {}),
+    "mistral": ("MistralConfig", "MistralDecoderLayer", "MistralRotaryEmbedding", {}),
+    "qwen2": ("Qwen2Config", "Qwen2DecoderLayer", "Qwen2RotaryEmbedding", {}),
+    "gemma": ("GemmaConfig", "GemmaDecoderLayer", "GemmaRotaryEmbedding", {"head_dim": 64}),
+    "gemma2": ("Gemma2Config", "Gemma2DecoderLayer", "Gemma2RotaryEmbedding", {"head_dim": 64}),
+    "phi3": ("Phi3Config", "Phi3DecoderLayer", "Phi3RotaryEmbedding", {}),
+    "olmo2": ("Olmo2Config", "Olmo2DecoderLayer", "Olmo2RotaryEmbedding", {}),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("family", sorted(_DECODER_FAMILIES))
+def test_decoder_layers_of_other_families(device, family, dtype):
+    """One decoder layer of each family as ``transformers`` builds it (hidden 512, 8 query / 4 KV heads, 64 tokens,
+    random weights): the norm variants (Gemma's ``1 + w`` in fp32, OLMo-2's norm after the projection and on q / k),
+    fused qkv + ``chunk`` (Phi-3), biased projections (Qwen-2), GeGLU — against the module in float64."""
+    import copy
+    import importlib
+
+    cfg_name, layer_name, rotary_name, extra = _DECODER_FAMILIES[family]
+    modeling = importlib.import_module(f"transformers.models.{family}.modeling_{family}")
+    cfg = getattr(importlib.import_module(f"transformers.models.{family}.configuration_{family}"), cfg_name)(
+        hidden_size=512, num_attention_heads=8, num_key_value_heads=4, intermediate_size=1024, num_hidden_layers=1, vocab_size=1000, pad_token_id=0, eos_token_id=1, bos_token_id=2, **extra)  # fmt: skip
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(72)
+    layer = getattr(modeling, layer_name)(cfg, 0)
+    with torch.no_grad():
+        for name, p in layer.named_parameters():
+            p.copy_((0.1 if "gemma" in family else 1.0) + 0.1 * torch.randn_like(p) if "norm" in name else 0.04 * torch.randn_like(p))
+    x = torch.randn(1, 64, 512)
+    cos, sin = getattr(modeling, rotary_name)(cfg)(x, torch.arange(64)[None])
+    mod = _RotaryLayer(layer).to(dtype).eval()
+    args = tuple(t.to(dtype) for t in (x, cos, sin))
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, args))
+    prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in args))))
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone().cpu()
+    finally:
+        prog.close()
+    with torch.no_grad():
+        want = copy.deepcopy(mod).double()(*(t.double() for t in args)).float()
+        half = copy.deepcopy(mod)(*args).float()
+    rms = float(want.pow(2).mean().sqrt())
+    if dtype is torch.float32:
+        eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-4 * rms, f"{family} layer fp32 vs float64")
+    else:
+        eager.assert_close(ours.reshape(want.shape).float(), want, 2e-2, 4e-2 * max(rms, 1.0), f"{family} layer bf16 vs float64")
+        eager.assert_mean_error_within_baseline(ours.reshape(want.shape).float(), half, want, 1.5, f"{family} layer bf16: mean error against eager bf16's")
 
 
 @pytest.mark.gpu
