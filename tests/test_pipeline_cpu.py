@@ -449,8 +449,12 @@ def test_row_sum_and_mean_are_row_reductions(launcher_lib):
         def forward(self, x):
             return x - x.mean(-1, keepdim=True)
 
+    # centring rows is one row kernel (the mean a statistic of the resident row) ...
     ks = kernels(HipBackend().compile(trace_module(M(), (torch.randn(16, 256),))))
-    assert [k.kernel_name.rsplit("_", 1)[0] for k in ks] == ["k_mean_reduce", "k_pointwise_elementwise"]
+    assert [k.kernel_name.rsplit("_", 1)[0] for k in ks] == ["k_row_fused_reduce"] and ks[0].algo_bytes == 2 * 16 * 256 * 4
+    # ... and a mean that is a result of its own is a row reduction with one value per row
+    ks = kernels(HipBackend().compile(trace_module(type("Mean", (nn.Module,), {"forward": lambda self, x: x.mean(-1, keepdim=True)})(), (torch.randn(16, 256),))))
+    assert [k.kernel_name.rsplit("_", 1)[0] for k in ks] == ["k_mean_reduce"]
     assert "one value per row" in ks[0].comment and ks[0].algo_bytes == 16 * 256 * 4 + 16 * 4
     # any other axis is moved last by a dense copy first
     ks = kernels(HipBackend().compile(trace_module(type("S", (nn.Module,), {"forward": lambda self, x: x.sum(0)})(), (torch.randn(4, 8),))))
