@@ -1237,7 +1237,7 @@ def _rec_row_fused(c: _Ctx, nid: str) -> bool:
     anything the row kernel has no operand form for leaves the match to the one-op-per-kernel fallbacks."""
     g = c.g
     node = g.nodes[nid]
-    if not isinstance(node.op, (F.CastOp, F.ElementwiseOp)) or nid in c.done:
+    if not isinstance(node.op, (F.CastOp, F.ContiguousOp, F.ElementwiseOp)) or nid in c.done:
         return False
     shape = tuple(node.output.shape)
     if len(shape) < 1 or not all(isinstance(d, int) for d in shape) or shape[-1] < 2:
@@ -1252,33 +1252,58 @@ def _rec_row_fused(c: _Ctx, nid: str) -> bool:
     class _Decline(Exception):
         pass
 
-    def build(cur: str, root: bool) -> E.Expr:
+    def is_stat(cur: str) -> bool:
         n = g.nodes[cur]
-        nshape = tuple(n.output.shape)
+        return isinstance(n.op, (F.MeanOp, F.SumOp, F.AmaxOp)) and cur not in c.done and n.op.keepdim and tuple(n.output.shape) == stat_shape and n.op.axis == len(shape) - 1 \
+            and tuple(g.nodes[n.inputs[0]].output.shape) == shape and c.single_use(cur)  # fmt: skip
+
+    def foldable(cur: str, root: bool, strict: bool) -> bool:
+        n = g.nodes[cur]
+        if not isinstance(n.op, (F.CastOp, F.ContiguousOp, F.ElementwiseOp)) or cur in c.done or tuple(n.output.shape) not in (shape, stat_shape):
+            return False
+        if strict and sum(tuple(g.nodes[i].output.shape) == shape for i in n.inputs) > 1:
+            return False  # under a statistic the row has one source: an op that joins two tensors (a residual add) is that source, stored by its own kernel
+        return root or isinstance(n.op, (F.CastOp, F.ContiguousOp)) or c.single_use(cur)
+
+    def build(cur: str, root: bool, strict: bool) -> E.Expr:
+        n = g.nodes[cur]
         if cur in stat_of:
             return stat_of[cur]
-        if isinstance(n.op, (F.MeanOp, F.SumOp, F.AmaxOp)) and cur not in c.done and n.op.keepdim and nshape == stat_shape and n.op.axis == len(shape) - 1 \
-                and tuple(g.nodes[n.inputs[0]].output.shape) == shape and c.single_use(cur):  # fmt: skip
-            pre = build(n.inputs[0], False)
+        if cur in leaves:
+            return leaves[cur]  # once a tensor is read from memory it is read from memory everywhere
+        if is_stat(cur):
+            pre = build(n.inputs[0], False, True)
             name = f"s{len(stats)}"
             stats.append(Stat(name, "max" if isinstance(n.op, F.AmaxOp) else "sum", pre))
             stat_of[cur] = _round(n.output.dtype, E.Var(name) / float(cols) if isinstance(n.op, F.MeanOp) else E.Var(name))
             return stat_of[cur]
-        elementwise = isinstance(n.op, (F.CastOp, F.ElementwiseOp)) and cur not in c.done and nshape in (shape, stat_shape)
-        foldable = elementwise and (root or isinstance(n.op, F.CastOp) or c.single_use(cur)) and folded[0] < _MAX_FUSED_POINTWISE
-        if not foldable:
-            if cur not in leaves:
-                leaves[cur] = E.Var(f"a{len(leaves)}")
+        if not foldable(cur, root, strict) or folded[0] >= _MAX_FUSED_POINTWISE:
+            leaves[cur] = E.Var(f"a{len(leaves)}")
             return leaves[cur]
         folded[0] += 1
-        args = [build(i, False) for i in n.inputs]
+        args = [build(i, False, strict) for i in n.inputs]
         e = _pointwise_node_expr(n.op, args)
         if e is None:
             raise _Decline
         return _round(n.output.dtype, e)
 
+    def statistics_first(cur: str, root: bool, seen: set) -> None:
+        """The reductions the tree reaches, innermost first: their operand decides what the resident row is."""
+        if cur in seen:
+            return
+        seen.add(cur)
+        if is_stat(cur):
+            statistics_first(g.nodes[cur].inputs[0], False, seen)
+            build(cur, False, True)
+        elif foldable(cur, root, False):
+            for i in g.nodes[cur].inputs:
+                statistics_first(i, False, seen)
+
     try:
-        project = build(nid, True)
+        statistics_first(nid, True, set())
+        if not stats:
+            return False
+        project = build(nid, True, False)
     except (_Decline, FusionError):
         return False
     if not stats:

@@ -163,7 +163,6 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
 
     g = Graph()
     g.constant_values = {}
-    env: dict[str, str] = {}  # fx node name -> graph node id
 
     def out_tensor(node) -> Tensor:
         val = node.meta["val"]
@@ -174,6 +173,37 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
 
     aten = torch.ops.aten
     tuples: dict[str, list[str]] = {}  # split / chunk node -> the node ids of its pieces
+    # Values that depend on no input and no parameter (position ids, rotary tables built from a buffer, a causal bias
+    # built from ``arange``): computed here, once, and handed to the graph as constants where a kernel reads them —
+    # what the reference's constant folding does after the trace (decomposition/050_fold_into_constant.py).
+    folded: dict[str, object] = {}
+    FOLD_LIMIT = 1 << 26  # elements
+
+    class _Env(dict):
+        def __missing__(self, name: str) -> str:
+            if name not in folded:
+                raise KeyError(name)
+            value = folded[name]
+            if not isinstance(value, torch.Tensor):
+                raise TraceError(f"a value computed at trace time ({name}) is read where a tensor is needed")
+            value = value.detach().contiguous()
+            nid = g.add_constant(name, tuple(int(d) for d in value.shape) or (1,), dt.from_torch(value.dtype))
+            g.constant_values[nid] = value.reshape(tuple(int(d) for d in value.shape) or (1,))
+            self[name] = nid
+            return nid
+
+    env = _Env()  # fx node name -> graph node id
+
+    def concrete(x):
+        """``x`` with every fx node replaced by its folded value; raises ``KeyError`` when one has none."""
+        if isinstance(x, torch.fx.Node):
+            return folded[x.name]
+        if isinstance(x, (list, tuple)):
+            return type(x)(concrete(i) for i in x)
+        if isinstance(x, dict):
+            return {k: concrete(v) for k, v in x.items()}
+        return x
+
     for node in ep.graph.nodes:
         if node.op == "placeholder":
             spec = kinds[node.name]
@@ -181,10 +211,24 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
             if spec.kind.name == "USER_INPUT":
                 env[node.name] = g.add_input(node.name, _shape(val), dt.from_torch(val.dtype))
             else:
+                if spec.kind.name != "PARAMETER":
+                    folded[node.name] = state[spec.target].detach()  # a buffer (rotary inv_freq): foldable; a graph constant only if a kernel reads it
+                    continue
                 nid = g.add_constant(node.name, _shape(val), dt.from_torch(val.dtype), source_path=spec.target)
                 g.constant_values[nid] = state[spec.target].detach()
                 env[node.name] = nid
             continue
+        if node.op == "call_function" and node.target is not operator.getitem or (node.op == "call_function" and getattr(node.args[0], "name", None) in folded):
+            try:
+                with torch.no_grad():
+                    value = node.target(*concrete(node.args), **concrete(node.kwargs))
+                if not isinstance(value, torch.Tensor) or value.numel() <= FOLD_LIMIT:
+                    folded[node.name] = value
+                    continue
+            except KeyError:
+                pass  # depends on an input or a parameter: an op of the graph
+            except Exception as exc:  # noqa: BLE001 - an op that cannot run on its folded operands is reported by name
+                raise TraceError(f"constant folding of {node.target} (node {node.name}) failed: {exc}") from exc
         if node.op == "output":
             outs = node.args[0]
             outs = outs if isinstance(outs, (tuple, list)) else (outs,)
@@ -259,14 +303,26 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
             add(node, F.MatmulOp(), [a[0], a[1]])
         elif t == aten.scaled_dot_product_attention.default:
             mask = a[3] if len(a) > 3 else kw.get("attn_mask")
-            if mask is not None:
+            causal = bool(a[5] if len(a) > 5 else kw.get("is_causal", False))
+            if mask is not None and getattr(mask, "name", None) in folded and isinstance(folded[mask.name], torch.Tensor) and folded[mask.name].dtype == torch.bool:
+                # a boolean mask known at trace time (a whole-model trace builds its causal mask from ``arange``): the
+                # plain lower triangle is the kernel's own causal form; anything else becomes the additive bias it stands for
+                keep = folded[mask.name]
+                sq, skv = int(a[0].meta["val"].shape[-2]), int(a[1].meta["val"].shape[-2])
+                tri = torch.ones(sq, skv, dtype=torch.bool).tril()
+                if keep.shape[-2:] == (sq, skv) and sq == skv and not causal and bool((keep == tri).all()):
+                    mask, causal = None, True
+                else:
+                    bias = torch.zeros(keep.shape, dtype=a[0].meta["val"].dtype).masked_fill(~keep, float("-inf"))
+                    folded[f"{mask.name}__bias"] = bias
+                    mask = type("Folded", (), {"name": f"{mask.name}__bias"})()
+            elif mask is not None:
                 mval = mask.meta.get("val") if hasattr(mask, "meta") else None
                 if mval is None or not mval.dtype.is_floating_point:
-                    raise TraceError("scaled_dot_product_attention: only an additive floating-point mask is supported (a boolean mask is not)")
+                    raise TraceError("scaled_dot_product_attention: only an additive floating-point mask is supported (a boolean mask is not, unless it is known at trace time)")
             dropout = a[4] if len(a) > 4 else kw.get("dropout_p", 0.0)
             if dropout:
                 raise TraceError("attention dropout is not supported")
-            causal = bool(a[5] if len(a) > 5 else kw.get("is_causal", False))
             scale = kw.get("scale")
             add(node, F.SdpaOp(is_causal=causal, scale=None if scale is None else float(scale), enable_gqa=bool(kw.get("enable_gqa", False)), has_mask=mask is not None),
                 [a[0], a[1], a[2]] + ([mask] if mask is not None else []))  # fmt: skip

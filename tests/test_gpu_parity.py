@@ -1571,3 +1571,55 @@ def test_layers_of_other_model_families(device, family, dtype):
     else:
         eager.assert_close(ours.reshape(want.shape).float(), want, 2e-2, 4e-2 * max(rms, 1.0), f"{family} bf16 vs float64")
         eager.assert_mean_error_within_baseline(ours.reshape(want.shape).float(), half, want, 1.5, f"{family} bf16: mean error against eager bf16's")
+
+
+class _Logits(nn.Module):
+    def __init__(self, model):
+        super().__init__()
+        self.model = model
+
+    def forward(self, ids):
+        return self.model(input_ids=ids, use_cache=False).logits
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_whole_small_causal_lm(device, dtype):
+    """Token ids in, logits out: a two-layer ``LlamaForCausalLM`` as ``transformers`` builds it.  The embedding is a
+    gather kernel; position ids, the rotary tables and the causal mask depend on no input, so the trace computes
+    them once (the boolean lower-triangle mask becomes the attention kernel's own causal form); against the model in
+    float64, and the greedy next token of every position must agree wherever float64's top two are clearly apart."""
+    import copy
+
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    cfg = LlamaConfig(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, intermediate_size=512, num_hidden_layers=2, vocab_size=1000, pad_token_id=0, eos_token_id=1, bos_token_id=2)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(81)
+    model = LlamaForCausalLM(cfg).eval()
+    ids = torch.randint(3, 1000, (2, 48))
+    mod = _Logits(model).to(dtype).eval()
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod, (ids,)))
+    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert names[0] == "k_index_rows"
+    if dtype is torch.bfloat16:
+        assert names.count("k_sdpa_reduce") == 2 and "HAS_MASK 1" not in "".join(n.op.kernel_source for n in compiled.nodes.values() if isinstance(n.op, HipOp) and "sdpa" in n.op.kernel_name)
+    prog = be.program(compiled, {compiled.inputs[0]: ids.to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone().cpu().float()
+    finally:
+        prog.close()
+    with torch.no_grad():
+        want = copy.deepcopy(mod).double()(ids).float()
+    ours = ours.reshape(want.shape)
+    rms = float(want.pow(2).mean().sqrt())
+    if dtype is torch.float32:
+        eager.assert_close(ours, want, 1e-4, 1e-4 * rms, "causal LM logits fp32 vs float64")
+    else:
+        eager.assert_close(ours, want, 2e-2, 4e-2 * max(rms, 1.0), "causal LM logits bf16 vs float64")
+    top2 = want.topk(2, -1).values
+    clear = (top2[..., 0] - top2[..., 1]) > (1e-3 if dtype is torch.float32 else 0.1) * rms
+    assert bool(clear.any()) and bool((ours.argmax(-1) == want.argmax(-1))[clear].all())
