@@ -752,13 +752,20 @@ def _rec_cat(c: _Ctx, nid: str) -> bool:
         return False
     out_shape = tuple(int(d) for d in node.output.shape)
     dim = node.op.dim
+    # empty pieces (a key / value cache that holds nothing yet) contribute nothing
+    pieces = [src for src in node.inputs if all(int(d) > 0 for d in c.g.nodes[src].output.shape)]
+    if len(pieces) == 1:
+        v = _need(c, pieces[0])
+        c.done[nid] = v.base
+        c.windows[nid] = (v.offset, tuple(v.shape), tuple(v.strides))
+        return True
     axes = [L.Var(f"c{i}") for i in range(len(out_shape))]
     stmts: list = []
     branches: list = []
     operands: dict = {}
     inputs: list[str] = []
     lo = 0
-    for k, src in enumerate(node.inputs):
+    for k, src in enumerate(pieces):
         v = _need(c, src)
         if not all(isinstance(d, int) for d in (*v.shape, *v.strides, v.offset)):
             raise FusionError("cat: static shapes only")
@@ -774,7 +781,7 @@ def _rec_cat(c: _Ctx, nid: str) -> bool:
         operands[f"s{k}"] = (v.base, (int(c.out.nodes[v.base].output.numel),), v.dtype)
         inputs.append(v.base)
         stmts.append(L.Load(f"t{k}", f"s{k}", (at,)))
-        branches.append((f"t{k}", L.Bin("<", axes[dim], L.Lit(hi)) if k < len(node.inputs) - 1 else L.Lit(1)))
+        branches.append((f"t{k}", L.Bin("<", axes[dim], L.Lit(hi)) if k < len(pieces) - 1 else L.Lit(1)))
         lo = hi
     if lo != out_shape[dim]:
         raise FusionError(f"cat {nid!r}: the pieces add up to {lo}, the result has {out_shape[dim]}")

@@ -1579,32 +1579,51 @@ class _Logits(nn.Module):
         self.model = model
 
     def forward(self, ids):
-        return self.model(input_ids=ids, use_cache=False).logits
+        out = self.model(input_ids=ids)
+        return out.logits if hasattr(out, "logits") else out.last_hidden_state
+
+
+def _small_model(family: str):
+    import transformers as tf
+
+    common = dict(vocab_size=1000, pad_token_id=0, eos_token_id=1, bos_token_id=2)
+    if family == "llama":
+        cfg, cls = tf.LlamaConfig(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, intermediate_size=512, num_hidden_layers=2, **common), tf.LlamaForCausalLM
+    elif family == "qwen3":
+        cfg, cls = tf.Qwen3Config(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=64, intermediate_size=512, num_hidden_layers=2, **common), tf.Qwen3Model
+    elif family == "gpt2":
+        cfg, cls = tf.GPT2Config(n_embd=256, n_head=4, n_layer=2, n_positions=128, vocab_size=1000, bos_token_id=2, eos_token_id=1), tf.GPT2LMHeadModel
+    else:
+        cfg, cls = tf.BertConfig(hidden_size=256, num_attention_heads=4, intermediate_size=1024, num_hidden_layers=2, vocab_size=1000, pad_token_id=0), (lambda c_: tf.BertModel(c_, add_pooling_layer=False))
+    cfg._attn_implementation = "sdpa"
+    return cls(cfg)
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_whole_small_causal_lm(device, dtype):
-    """Token ids in, logits out: a two-layer ``LlamaForCausalLM`` as ``transformers`` builds it.  The embedding is a
-    gather kernel; position ids, the rotary tables and the causal mask depend on no input, so the trace computes
-    them once (the boolean lower-triangle mask becomes the attention kernel's own causal form); against the model in
-    float64, and the greedy next token of every position must agree wherever float64's top two are clearly apart."""
+@pytest.mark.parametrize("family", ["llama", "qwen3", "gpt2", "bert"])
+def test_whole_small_models(device, family, dtype):
+    """Token ids in, logits (or the last hidden state) out: two-layer models as ``transformers`` builds them — a Llama
+    and a GPT-2 causal LM, a Qwen-3 base model (the architecture of the reference's flagship embedding model), a BERT
+    encoder.  Embeddings are gather kernels; position ids, rotary tables, the causal mask and an empty key / value
+    cache depend on no input, so the trace computes them once (a boolean lower-triangle mask becomes the attention
+    kernel's own causal form); against the model in float64, and for the causal LMs the greedy next token of every
+    position must agree wherever float64's top two are clearly apart."""
     import copy
 
-    from transformers import LlamaConfig, LlamaForCausalLM
-
-    cfg = LlamaConfig(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, intermediate_size=512, num_hidden_layers=2, vocab_size=1000, pad_token_id=0, eos_token_id=1, bos_token_id=2)
-    cfg._attn_implementation = "sdpa"
     torch.manual_seed(81)
-    model = LlamaForCausalLM(cfg).eval()
+    model = _small_model(family).eval()
     ids = torch.randint(3, 1000, (2, 48))
     mod = _Logits(model).to(dtype).eval()
     be = HipBackend()
     compiled = be.compile(trace_module(mod, (ids,)))
-    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    ops = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    names = [op.kernel_name.rsplit("_", 1)[0] for op in ops]
     assert names[0] == "k_index_rows"
     if dtype is torch.bfloat16:
-        assert names.count("k_sdpa_reduce") == 2 and "HAS_MASK 1" not in "".join(n.op.kernel_source for n in compiled.nodes.values() if isinstance(n.op, HipOp) and "sdpa" in n.op.kernel_name)
+        assert names.count("k_sdpa_reduce") == 2
+        if family != "bert":
+            assert all("#define HAS_MASK 0" in op.kernel_source and "#define CAUSAL 1" in op.kernel_source for op in ops if "sdpa" in op.kernel_name)
     prog = be.program(compiled, {compiled.inputs[0]: ids.to(device)})
     try:
         prog.run()
@@ -1617,9 +1636,10 @@ def test_whole_small_causal_lm(device, dtype):
     ours = ours.reshape(want.shape)
     rms = float(want.pow(2).mean().sqrt())
     if dtype is torch.float32:
-        eager.assert_close(ours, want, 1e-4, 1e-4 * rms, "causal LM logits fp32 vs float64")
+        eager.assert_close(ours, want, 1e-4, 2e-4 * rms, f"{family} fp32 vs float64")
     else:
-        eager.assert_close(ours, want, 2e-2, 4e-2 * max(rms, 1.0), "causal LM logits bf16 vs float64")
-    top2 = want.topk(2, -1).values
-    clear = (top2[..., 0] - top2[..., 1]) > (1e-3 if dtype is torch.float32 else 0.1) * rms
-    assert bool(clear.any()) and bool((ours.argmax(-1) == want.argmax(-1))[clear].all())
+        eager.assert_close(ours, want, 2e-2, 4e-2 * max(rms, 1.0), f"{family} bf16 vs float64")
+    if family in ("llama", "gpt2"):
+        top2 = want.topk(2, -1).values
+        clear = (top2[..., 0] - top2[..., 1]) > (1e-3 if dtype is torch.float32 else 0.1) * rms
+        assert bool(clear.any()) and bool((ours.argmax(-1) == want.argmax(-1))[clear].all())
