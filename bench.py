@@ -273,12 +273,43 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
             for p in progs:
                 p.close()
 
-    def bench(make_case, label: str, bound: str, check: bool = True, cold: bool = False) -> None:
+    def bench(make_case, label: str, bound: str, check: bool = True, cold: bool = False, whole_model: bool = False) -> None:
         if only is not None and only not in label:
             return
         case = make_case()
         compiled = be.compile(trace_module(case.module, case.inputs))
         data = {n: t.to(device) for n, t in zip(compiled.inputs, case.inputs)}
+        eager_us = None
+        if whole_model:
+            # dozens of layers deep an element-wise bound says little: the mean distance from an fp32 run of the same
+            # model may be at most 1.5 x 16-bit eager's own; eager's latency is reported beside ours
+            check = False
+            prog = be.program(compiled, data)
+            try:
+                prog.run()
+                torch.cuda.synchronize()
+                ours = prog.output_tensors()[compiled.outputs[0]].float()
+                gm = case.module.to(device)
+                args = tuple(t.to(device) for t in case.inputs)
+                with torch.no_grad():
+                    half = gm(*args).float()
+                    exact = gm.float()(*args)
+                    gm.to(case.inputs[0].dtype if case.inputs[0].is_floating_point() else torch.bfloat16)
+                    err, base = float((ours.reshape(exact.shape) - exact).abs().mean()), float((half - exact).abs().mean())
+                    if not err <= 1.5 * base:
+                        raise AssertionError(f"{label}: mean |ours - fp32 eager| {err:.4g} exceeds 1.5 x mean |16-bit eager - fp32 eager| {base:.4g}")
+                    times = []
+                    for i in range(13):
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        e0.record()
+                        gm(*args)
+                        e1.record()
+                        torch.cuda.synchronize()
+                        if i >= 3:
+                            times.append(e0.elapsed_time(e1) * 1e3)
+                    eager_us = min(times)
+            finally:
+                prog.close()
         if check:
             prog = be.program(compiled, data)
             try:
@@ -308,7 +339,10 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
             row["cold_sets"] = sets
             if bound == "hbm":
                 row["achieved_cold"] = round(case.algo_bytes / (c_us * 1e-6) / 1e9, 1)
-        if cpu:
+        if eager_us is not None:
+            row["eager_gpu_us"] = round(eager_us, 1)
+            row.pop("per_kernel_us", None)  # (142 entries: the five kernels of a layer are the C5 row's)
+        if cpu and not whole_model:
             row["cpu_us"] = round(_cpu_us(case), 1)
         rows.append(row)
 
@@ -324,6 +358,8 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
     if extended:
         bench(lambda: wl.sdpa_case(causal=False), "C4x non-causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
     bench(lambda: wl.qwen3_block_case(seq=512), "C5 qwen3-0.6B block bf16 S=512", "mfma")
+    if extended:
+        bench(lambda: wl.qwen3_model_case(seq=512), "M qwen3-0.6B whole model (28 layers, random weights) bf16 S=512, token ids -> last hidden state", "mfma", whole_model=True)
     return rows
 
 
@@ -335,7 +371,7 @@ def main() -> int:
     ap.add_argument("--no-table", action="store_true", help="skip the per-configuration kernel table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default=None, metavar="TEXT", help="restrict the kernel table to configurations whose label contains TEXT (e.g. 'M=2048', 'C4')")
-    ap.add_argument("--extended", action="store_true", help="add machine-filling variants to the kernel table (4096^3 linear, non-causal attention)")
+    ap.add_argument("--extended", action="store_true", help="add machine-filling variants to the kernel table (4096^3 linear, non-causal attention) and the whole 28-layer model")
     ap.add_argument("--copy-probe", action="store_true", help="also run a plain 469762048-byte device copy 5 times (counter calibration under rocprofv3 --pmc)")
     ap.add_argument("--live-traffic", action="store_true", help="count the headline kernel's HBM bytes now: two rocprofv3 --pmc passes over this script (adds about a minute)")
     args = ap.parse_args()

@@ -161,6 +161,41 @@ def qwen3_block_case(seq: int = 512, seed: int = 0, dtype=torch.bfloat16, norm_s
     )  # fmt: skip
 
 
+class LastHiddenState(nn.Module):
+    """A ``transformers`` base model taking token ids and returning its last hidden state."""
+
+    def __init__(self, model):
+        super().__init__()
+        self.m = model
+
+    def forward(self, ids):
+        return self.m(input_ids=ids).last_hidden_state
+
+
+def qwen3_model_case(seq: int = 512, layers: int = 28, seed: int = 0, dtype=torch.bfloat16) -> Case:
+    """The whole Qwen3-0.6B-architecture base model (what Qwen3-Embedding-0.6B runs before pooling: hidden 1024,
+    16 query / 8 KV heads of 128, intermediate 3072, vocabulary 151 669), random weights scaled so activations keep
+    unit size through ``layers`` layers, random token ids: ids in, last hidden state out."""
+    from transformers import Qwen3Config, Qwen3Model
+
+    cfg = Qwen3Config(
+        hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128, intermediate_size=3072, num_hidden_layers=layers, vocab_size=151669,
+        rms_norm_eps=1e-6, rope_theta=1e6, max_position_embeddings=max(32768, seq), pad_token_id=0, eos_token_id=1, bos_token_id=2,
+    )  # fmt: skip
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(seed)
+    model = Qwen3Model(cfg).eval()
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if "norm" not in name:
+                p.mul_(0.5)
+    ids = torch.randint(3, 151000, (1, seq))
+    h, hq, hkv, d, inter = 1024, 16, 8, 128, 3072
+    flops = layers * (2 * seq * h * (hq * d + 2 * hkv * d) + 2 * seq * hq * d * h + 3 * 2 * seq * h * inter + 4 * hq * d * (seq * (seq + 1) // 2))
+    wbytes = layers * (h * (hq * d + 2 * hkv * d) + hq * d * h + 3 * h * inter) * 2
+    return Case(f"qwen3_model_l{layers}_s{seq}", LastHiddenState(model).to(dtype).eval(), (ids,), BF16_RTOL, 4e-2, algo_bytes=wbytes, algo_flops=flops)
+
+
 class NormedRopeAttention(nn.Module):
     """The front of a Qwen3-style attention layer with ``nn.RMSNorm`` head norms:
     q/k/v projections, per-head norm of q and k, rotary embedding, causal GQA

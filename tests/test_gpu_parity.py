@@ -1643,3 +1643,30 @@ def test_whole_small_models(device, family, dtype):
         top2 = want.topk(2, -1).values
         clear = (top2[..., 0] - top2[..., 1]) > (1e-3 if dtype is torch.float32 else 0.1) * rms
         assert bool(clear.any()) and bool((ours.argmax(-1) == want.argmax(-1))[clear].all())
+
+
+@pytest.mark.gpu
+def test_full_width_model_a_few_layers_deep(device):
+    """The bench's whole-model workload at four layers and 128 tokens (full width: hidden 1024, 16 / 8 heads of 128,
+    vocabulary 151 669): five launches per layer plus the embedding gather and the final norm, and a mean distance
+    from the fp32 run of the same model no larger than 1.5 x bf16 eager's own."""
+    from deplodock_amd import workloads as wl
+
+    case = wl.qwen3_model_case(seq=128, layers=4)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert len(names) == 1 + 4 * 5 + 1 and names[0] == "k_index_rows" and names.count("k_sdpa_reduce") == 4
+    prog = be.program(compiled, {compiled.inputs[0]: case.inputs[0].to(device)})
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone().float()
+    finally:
+        prog.close()
+    gm = case.module.to(device)
+    with torch.no_grad():
+        half = gm(case.inputs[0].to(device)).float()
+        exact = gm.float()(case.inputs[0].to(device))
+    eager.assert_mean_error_within_baseline(ours.reshape(exact.shape), half, exact, 1.5, "four-layer full-width model vs fp32 eager")
+    eager.assert_rows_within_baseline(ours.reshape(exact.shape), half, exact, 2.0, "four-layer full-width model rows vs fp32 eager")
