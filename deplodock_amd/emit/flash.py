@@ -617,7 +617,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
             "INV_SCALE": float_literal(1.0 / body.scale)} if has_mask else {}),
         "PAIR": 1 if pair else 0,
         # steps in parity pairs (static ring slots) unless the whole key range is one or two steps
-        "PAIRSTEP": 1 if _PAIRSTEP and (bool(symf) or -(-body.kv_len // (kvs * BKV)) > 2) else 0,
+        "PAIRSTEP": 1 if _PAIRSTEP and body.pair_steps and (bool(symf) or -(-body.kv_len // (kvs * BKV)) > 2) else 0,
         "V_PRE": 1 if _V_PRE and (BKV // 32) * 2 * (D // 32) * 4 <= 32 else 0,  # the prefetched V fragments take at most 32 registers
         "RK": plan["rk"], "RV": plan["rv"], "DEEP": 1 if plan["deep"] else 0,
         "Q_LDS": 1 if plan["q_off"] is not None else 0,

@@ -278,6 +278,7 @@ class Flash:
     kv_split: int = 1  # wave groups that split the key blocks of a query group between them
     pair: bool = False  # causal only: a workgroup takes query block b and its mirror QBLOCKS-1-b
     deep: bool = False  # a K ring of three slots (K blocks requested two steps ahead) beside a V ring of two
+    pair_steps: bool = True  # key steps unrolled in pairs so ring slots are compile-time (the lowering clears it if that build spills)
     # an additive bias on the scaled scores, ``[batch, head, query, key]`` addressed through (batch, head, query)
     # strides (0 = broadcast) with keys contiguous; ``None``: no mask operand
     mask: str | None = None

@@ -79,6 +79,36 @@ def _lower_contraction(op: TileOp, ctx: Context) -> HipOp:
         logger.warning("%s: TILE=%s spills %d vector registers: the heuristic tile instead", hip.kernel_name, hip.knobs.get("TILE"), spilled)
         default_contraction_schedule(body, ctx)
         hip = _named(emit_contraction(body, _PLACEHOLDER, ctx), op)
+        spilled = _spills(hip, ctx)
+    # The heuristic tile itself can spill under a heavy output stage (2048 tokens: the 128x256 tile of the q/k/v
+    # projection with head norms and rotary embedding in its epilogue): halve the fragments per wave, rows first (the
+    # output stage works on whole column groups), until the kernel builds clean.
+    from deplodock_amd.ir.schedule import ScheduleError, TilePlan
+    from deplodock_amd.passes.schedule import _check_tile, _default_stage
+
+    for _ in range(4):
+        if not spilled:
+            break
+        plan = body.tile
+        fm, fn = plan.regs
+        shrunk = None
+        for regs in ((fm // 2, fn), (fm, fn // 2)):
+            if min(regs) < 1 or regs == (fm, fn):
+                continue
+            cand = TilePlan(atom=plan.atom, units=plan.units, regs=regs, bk=plan.bk)
+            try:
+                _check_tile(cand, body, ctx, depth=2)
+            except ScheduleError:
+                continue
+            shrunk = cand
+            break
+        if shrunk is None:
+            break
+        logger.warning("%s: TILE=%s spills %d vector registers: %s instead", hip.kernel_name, plan.spell(), spilled, shrunk.spell())
+        body.tile = shrunk
+        body.stage = _default_stage(shrunk, body, ctx)
+        hip = _named(emit_contraction(body, _PLACEHOLDER, ctx), op)
+        spilled = _spills(hip, ctx)
     return hip
 
 
@@ -106,6 +136,34 @@ def _lower_split_contraction(graph: Graph, node: Node, ctx: Context) -> None:
     node.inputs = [ws_id, *node.inputs]
 
 
+def _lower_flash(op: TileOp, ctx: Context) -> HipOp:
+    """The attention kernel waits for part of its outstanding direct-to-LDS loads by count, as the contraction's
+    rings do, so it must build without vector-register spills too.  A schedule that spills gives up, in turn: the
+    pairwise unrolling of its key steps, the mirrored query-block pairing, and finally its shape for the smallest
+    one (two row groups x four key-split groups on 32-key blocks)."""
+    body = op.body
+    hip = _named(emit_flash(body, _PLACEHOLDER, ctx), op)
+    steps = (("pair_steps", False), ("pair", False), ("shape", None))
+    for what, value in steps:
+        spilled = _spills(hip, ctx)
+        if not spilled:
+            break
+        if what == "shape":
+            if (body.waves, body.block_kv, body.kv_split) == (2, 32, 4):
+                break
+            body.waves, body.block_kv, body.kv_split, body.deep = 2, 32, 4, False
+        elif getattr(body, what) == value:
+            continue
+        else:
+            setattr(body, what, value)
+        logger.warning("%s: FLASH=%s spills %d vector registers: rendered again without %s", hip.kernel_name, hip.knobs.get("FLASH"), spilled, {"pair_steps": "pairwise key steps", "pair": "query-block pairs", "shape": "its wave shape"}[what])
+        try:
+            hip = _named(emit_flash(body, _PLACEHOLDER, ctx), op)
+        except LoweringError:
+            break
+    return hip
+
+
 def lower_tile(op: TileOp, ctx: Context) -> HipOp:
     body = op.body
     if isinstance(body, Contraction):
@@ -113,7 +171,8 @@ def lower_tile(op: TileOp, ctx: Context) -> HipOp:
     if isinstance(body, RowReduce):
         hip = (emit_row_reduce_streaming if body.stream else emit_row_reduce)(body, _PLACEHOLDER, ctx)
     elif isinstance(body, Flash):
-        hip = emit_flash(body, _PLACEHOLDER, ctx)
+        hip = _lower_flash(op, ctx)
+        return hip
     elif isinstance(body, Map):
         hip = emit_map(body, _PLACEHOLDER, ctx)
     elif isinstance(body, LoopNest):

@@ -1670,3 +1670,32 @@ def test_full_width_model_a_few_layers_deep(device):
         exact = gm.float()(case.inputs[0].to(device))
     eager.assert_mean_error_within_baseline(ours.reshape(exact.shape), half, exact, 1.5, "four-layer full-width model vs fp32 eager")
     eager.assert_rows_within_baseline(ours.reshape(exact.shape), half, exact, 2.0, "four-layer full-width model rows vs fp32 eager")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seq", [2048, 4096])
+def test_c5_block_at_long_sequences(device, seq):
+    """At 2048 tokens the heuristic 128x256 tile of the q/k/v projection spills under its head-norm + rotary output
+    stage, and at 4096 the attention schedule spills with its key steps unrolled in pairs: both are rendered again
+    in a form that builds clean (a kernel that waits for loads by count must not spill), and the block still matches."""
+    from deplodock_amd.backend.hip import hiprtc
+
+    case = eager.qwen3_block_case(seq=seq, norm_std=0.1, seed=7)
+    ours, want, compiled = run_case(case, device)
+    for n in compiled.nodes.values():
+        if isinstance(n.op, HipOp):
+            assert hiprtc.spilled_vgprs(n.op.kernel_source, n.op.kernel_name) == 0, n.op.kernel_name
+    exact = eager.run_eager_fp32(case, device)
+    x = case.inputs[0].to(device).float()
+    eager.assert_mean_error_within_baseline(ours.float() - x, want.float() - x, exact - x, 1.5, f"block S={seq} (out - x) vs fp32 eager")
+    eager.assert_rows_within_baseline(ours.float() - x, want.float() - x, exact - x, 1.5, f"block S={seq} rows vs fp32 eager")
+
+
+@pytest.mark.gpu
+def test_c4_sdpa_at_4096_tokens(device):
+    case = eager.sdpa_case(s=4096)
+    ours, want, _ = run_case(case, device)
+    q, k, v = (t.to(device).float() for t in case.inputs)
+    exact = nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+    eager.assert_close(ours, want, 2e-2, 2e-2, "sdpa S=4096 vs eager")
+    eager.assert_rows_within_baseline(ours, want, exact, 1.5, "sdpa S=4096 rows vs fp32 eager")
