@@ -101,6 +101,9 @@ def emit_row_reduce(body: RowReduce, name: str, ctx: Context = Context()) -> Hip
     for ro in body.row_operands:
         while V > 1 and ro.offset % V:
             V //= 2
+    if body.rotate is not None:
+        while V > 1 and (body.cols // V) % 2:
+            V //= 2  # each half of the row is whole vectors (head_dim 40 in bf16: ten chunks of four, not five of eight)
     C = body.cols // V  # vector chunks per row
     if body.rotate is not None:
         if C % 2:

@@ -85,6 +85,9 @@ def pick_coop(cols: int, elem_bytes: int, rows: int, ctx: Context, *, rotate: bo
     vec = max(1, 16 // elem_bytes)
     chunks = max(1, cols // vec) if cols % vec == 0 else cols
     if rotate:
+        while vec > 1 and cols % vec == 0 and (cols // vec) % 2:
+            vec //= 2  # as the emitter: each half of the row is whole vectors
+        chunks = max(1, cols // vec) if cols % vec == 0 else cols
         lanes = 1
         while lanes * 2 <= 64 and (chunks // 2) % (lanes * 2) == 0 and chunks // (lanes * 2) >= 2:
             lanes *= 2

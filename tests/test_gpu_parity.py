@@ -1699,3 +1699,16 @@ def test_c4_sdpa_at_4096_tokens(device):
     exact = nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
     eager.assert_close(ours, want, 2e-2, 2e-2, "sdpa S=4096 vs eager")
     eager.assert_rows_within_baseline(ours, want, exact, 1.5, "sdpa S=4096 rows vs fp32 eager")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("head_dim", [40, 24])
+def test_rotary_embedding_on_heads_that_are_not_whole_16_byte_pairs(device, head_dim):
+    """head_dim 40 in bf16 is five 16-byte chunks: the rotate-half kernel keeps both halves of a row in one lane, so
+    it narrows its vectors until each half is whole vectors (ten chunks of four); attention at that head_dim takes the
+    decomposed route."""
+    case = eager.normed_rope_attention_case(hidden=256, q_heads=4, kv_heads=2, head_dim=head_dim, seq=50)
+    ours, want, compiled = run_case(case, device)
+    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert any("rope" in n for n in names) and names.count("k_batched_linear") == 2
+    eager.assert_close(ours, want, case.rtol, case.atol, f"rope + attention head_dim={head_dim} vs eager")
