@@ -1264,8 +1264,15 @@ def _rec_row_fused(c: _Ctx, nid: str) -> bool:
         return isinstance(n.op, (F.MeanOp, F.SumOp, F.AmaxOp)) and cur not in c.done and n.op.keepdim and tuple(n.output.shape) == stat_shape and n.op.axis == len(shape) - 1 \
             and tuple(g.nodes[n.inputs[0]].output.shape) == shape and c.single_use(cur)  # fmt: skip
 
+    def broadcast_of_stat(cur: str) -> bool:
+        """``stat.expand_as(x)``: a per-row value spelled at the rows' full shape."""
+        n = g.nodes[cur]
+        return isinstance(n.op, F.ExpandOp) and cur not in c.done and tuple(n.output.shape) == shape and tuple(g.nodes[n.inputs[0]].output.shape) == stat_shape
+
     def foldable(cur: str, root: bool, strict: bool) -> bool:
         n = g.nodes[cur]
+        if broadcast_of_stat(cur):
+            return True
         if not isinstance(n.op, (F.CastOp, F.ContiguousOp, F.ElementwiseOp)) or cur in c.done or tuple(n.output.shape) not in (shape, stat_shape):
             return False
         if strict and sum(tuple(g.nodes[i].output.shape) == shape for i in n.inputs) > 1:
@@ -1287,6 +1294,8 @@ def _rec_row_fused(c: _Ctx, nid: str) -> bool:
         if not foldable(cur, root, strict) or folded[0] >= _MAX_FUSED_POINTWISE:
             leaves[cur] = E.Var(f"a{len(leaves)}")
             return leaves[cur]
+        if broadcast_of_stat(cur):
+            return build(n.inputs[0], False, strict)
         folded[0] += 1
         args = [build(i, False, strict) for i in n.inputs]
         e = _pointwise_node_expr(n.op, args)

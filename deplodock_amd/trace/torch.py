@@ -326,6 +326,44 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
             scale = kw.get("scale")
             add(node, F.SdpaOp(is_causal=causal, scale=None if scale is None else float(scale), enable_gqa=bool(kw.get("enable_gqa", False)), has_mask=mask is not None),
                 [a[0], a[1], a[2]] + ([mask] if mask is not None else []))  # fmt: skip
+        elif t in (aten.clamp_min.default, aten.clamp_max.default, aten.clamp.default):
+            lo = a[1] if t != aten.clamp_max.default and len(a) > 1 else (kw.get("min") if t == aten.clamp.default else None)
+            hi = a[1] if t == aten.clamp_max.default else (a[2] if t == aten.clamp.default and len(a) > 2 else kw.get("max") if t == aten.clamp.default else None)
+            if any(hasattr(v, "meta") for v in (lo, hi)):
+                raise TraceError("clamp: tensor bounds are not supported")
+            cur, ot = env[a[0].name], out_tensor(node)
+            steps = [("maximum", lo)] * (lo is not None) + [("minimum", hi)] * (hi is not None)
+            if not steps:
+                raise TraceError("clamp: no bound")
+            for i, (fn, bound) in enumerate(steps):
+                last = i == len(steps) - 1
+                nid_ = node.name if last else f"{node.name}__lo"
+                cur = g.add_node(F.ElementwiseOp(fn=fn, scalar=float(bound)), [cur], Tensor(nid_, ot.shape, ot.dtype), nid_)
+            env[node.name] = cur
+        elif t == aten.linalg_vector_norm.default:
+            # the 2-norm over one axis: sqrt(sum(x^2)) (what F.normalize divides by)
+            ord_ = a[1] if len(a) > 1 else kw.get("ord", 2)
+            dims = a[2] if len(a) > 2 else kw.get("dim")
+            keep = bool(a[3]) if len(a) > 3 else bool(kw.get("keepdim", False))
+            dims = list(dims) if isinstance(dims, (list, tuple)) else [dims]
+            if float(ord_) != 2.0 or len(dims) != 1 or dims[0] is None:
+                raise TraceError("linalg_vector_norm: only the 2-norm over one axis is supported")
+            ot, xt = out_tensor(node), a[0].meta["val"]
+            sq = g.add_node(F.ElementwiseOp(fn="pow", scalar=2.0), [env[a[0].name]], Tensor(f"{node.name}__sq", _shape(xt), ot.dtype), f"{node.name}__sq")
+            sm = g.add_node(F.SumOp(axis=_norm_dim(int(dims[0]), rank_in), keepdim=keep), [sq], Tensor(f"{node.name}__sum", ot.shape, ot.dtype), f"{node.name}__sum")
+            env[node.name] = g.add_node(F.ElementwiseOp(fn="sqrt"), [sm], ot, node.name)
+        elif t == aten.select.int:
+            # x.select(dim, i): the one-wide slice, then that axis dropped (both views)
+            dim = _norm_dim(int(a[1]), rank_in)
+            size = int(a[0].meta["val"].shape[dim])
+            idx = int(a[2]) + (size if int(a[2]) < 0 else 0)
+            xs = list(_shape(a[0].meta["val"]))
+            xs[dim] = 1
+            ot = out_tensor(node)
+            sl = g.add_node(F.SliceOp(dim=dim, start=idx, end=idx + 1, step=1), [env[a[0].name]], Tensor(f"{node.name}__slice", tuple(xs), ot.dtype), f"{node.name}__slice")
+            env[node.name] = g.add_node(F.SqueezeOp(dim=dim), [sl], ot, node.name)
+        elif t == aten.expand_as.default:
+            add(node, F.ExpandOp(shape=tuple(int(d) for d in node.meta["val"].shape)), [a[0]])
         elif t == aten.type_as.default:
             add(node, F.CastOp(dtype=dt.from_torch(a[1].meta["val"].dtype)), [a[0]])
         elif t in (aten.to.dtype, aten._to_copy.default, aten.to.dtype_layout):

@@ -1402,6 +1402,13 @@ def _op_cases():
         "manual_layer_norm": (_Fn(lambda t: (t - t.mean(-1, keepdim=True)) * torch.rsqrt((t - t.mean(-1, keepdim=True)).pow(2).mean(-1, keepdim=True) + 1e-5)), lambda: (2 + x(5, 40, 200),)),
         "shift_by_row_max": (_Fn(lambda t: torch.exp(t - t.amax(-1, keepdim=True))), lambda: (3 * x(6, 300),)),
         "residual_plus_norm": (_Fn(lambda t, r: r + t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + 1e-6)), lambda: (x(4, 33, 256), x(4, 33, 256))),
+        # what an embedding model does after its last layer: pick the last token, normalise to unit length
+        "normalize": (_Fn(lambda t: Fn.normalize(t, p=2, dim=-1)), lambda: (x(4, 33, 256),)),
+        "last_token_normalize": (_Fn(lambda t: Fn.normalize(t[:, -1], p=2, dim=1)), lambda: (x(4, 33, 256),)),
+        "select": (_Fn(lambda t: t[:, 5] * 2), lambda: (x(4, 33, 40),)),
+        "clamp": (_Fn(lambda t: t.clamp(-0.5, 0.7)), lambda: (x(3, 100),)),
+        "clamp_min": (_Fn(lambda t: t.clamp_min(0.1) * 2), lambda: (x(3, 100),)),
+        "vector_norm_axis1": (_Fn(lambda t: torch.linalg.vector_norm(t, dim=1)), lambda: (x(4, 33, 40),)),
         # a transformer MLP of the GELU family, and a pre-norm projection
         "gelu_mlp": (nn.Sequential(nn.Linear(256, 512), nn.GELU(), nn.Linear(512, 256)), lambda: (x(2, 48, 256),)),
         "layer_norm_linear": (nn.Sequential(nn.LayerNorm(256), nn.Linear(256, 128)), lambda: (x(4, 33, 256),)),
