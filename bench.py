@@ -358,8 +358,7 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
     if extended:
         bench(lambda: wl.sdpa_case(causal=False), "C4x non-causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
     bench(lambda: wl.qwen3_block_case(seq=512), "C5 qwen3-0.6B block bf16 S=512", "mfma")
-    if extended:
-        bench(lambda: wl.qwen3_model_case(seq=512), "M qwen3-0.6B whole model (28 layers, random weights) bf16 S=512, token ids -> last hidden state", "mfma", whole_model=True)
+    bench(lambda: wl.qwen3_model_case(seq=512), "M qwen3-0.6B whole model (28 layers, random weights) bf16 S=512, token ids -> last hidden state", "mfma", whole_model=True)
     return rows
 
 
@@ -371,7 +370,7 @@ def main() -> int:
     ap.add_argument("--no-table", action="store_true", help="skip the per-configuration kernel table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default=None, metavar="TEXT", help="restrict the kernel table to configurations whose label contains TEXT (e.g. 'M=2048', 'C4')")
-    ap.add_argument("--extended", action="store_true", help="add machine-filling variants to the kernel table (4096^3 linear, non-causal attention) and the whole 28-layer model")
+    ap.add_argument("--extended", action="store_true", help="add machine-filling variants to the kernel table (4096^3 linear, non-causal attention)")
     ap.add_argument("--copy-probe", action="store_true", help="also run a plain 469762048-byte device copy 5 times (counter calibration under rocprofv3 --pmc)")
     ap.add_argument("--live-traffic", action="store_true", help="count the headline kernel's HBM bytes now: two rocprofv3 --pmc passes over this script (adds about a minute)")
     args = ap.parse_args()
