@@ -170,6 +170,8 @@ class HipBackend(Backend):
                     whole = (whole.float() * ks.to(whole.device).float().reshape(1, -1)).to(whole.dtype)
                 if stacked.transpose:
                     whole = whole.transpose(-1, -2).contiguous()
+                if stacked.pad_rows_to > whole.shape[0]:
+                    whole = torch.cat([whole, whole.new_zeros((stacked.pad_rows_to - whole.shape[0], *whole.shape[1:]))], dim=0)
                 data[nid] = whole
             elif nid in traced:
                 data[nid] = traced[nid]

@@ -17,7 +17,12 @@ from deplodock_amd import config
 
 
 def add_common_args(parser) -> None:
-    parser.add_argument("input", nargs="?", help="Unsupported here (model IDs and IR files): use --code.")
+    parser.add_argument("input", nargs="?", help="A model: a local directory with a transformers config.json (and weights, else random ones), or 'arch:<name>' for a built-in "
+                        "architecture with random weights (arch:qwen3-0.6b, arch:qwen3-tiny, arch:llama-tiny).  Hub model IDs need a download and are refused.  Mutually exclusive with --code.")  # fmt: skip
+    parser.add_argument("--layer", type=int, default=None, help="Decoder layer index of the model input (hidden states + rotary tables in); omit for the whole model (token ids in, logits out).")
+    parser.add_argument("--seq-len", type=int, default=32, help="Tokens of the example input for a model (default 32).")
+    parser.add_argument("--dtype", choices=["bf16", "fp16", "fp32"], default="bf16", help="Parameter / activation type for a model input (default bf16).")
+    parser.add_argument("--random-weights", action="store_true", help="Initialise the model from its config instead of loading weights from the directory.")
     parser.add_argument("--code", "-c", help="Inline Python whose last statement is the expression to compile, e.g. 'torch.nn.RMSNorm(2048)(torch.randn(1,32,2048))'.")
     parser.add_argument("--dump-dir", default=None, help="Directory for the graph after each pass and the final kernel sources.")
     parser.add_argument("--knobs", default=None, help="Pin scheduling knobs for this invocation, 'K1=V1,K2=V2' (the EMMY_KNOBS grammar), e.g. 'TILE=a:mfma_32x32x16_bf16/w2x2/f2x3/k4'.")
@@ -47,9 +52,11 @@ def trace_from_args(args):
     from deplodock_amd.commands.code import CodeError, parse_inline
     from deplodock_amd.trace.torch import trace_module
 
-    if args.input and not args.code:
-        print("error: model IDs and IR files are not handled by this backend; pass the module with --code", file=sys.stderr)
+    if args.input and args.code:
+        print("error: a model input and --code are mutually exclusive", file=sys.stderr)
         sys.exit(2)
+    if args.input:
+        return _trace_model(args)
     if not args.code:
         print("error: --code is required", file=sys.stderr)
         sys.exit(2)
@@ -62,6 +69,95 @@ def trace_from_args(args):
         print(f"error: {e}", file=sys.stderr)
         sys.exit(2)
     return trace_module(prog.module, prog.args, kwargs=prog.kwargs or None, dynamic_shapes=parse_dynamic(args.dynamic)), prog
+
+
+ARCHITECTURES = {
+    # name -> (transformers config class, its arguments): built from the config alone, random weights
+    "qwen3-0.6b": ("Qwen3Config", dict(hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128, intermediate_size=3072, num_hidden_layers=28, vocab_size=151669, rms_norm_eps=1e-6, rope_theta=1e6, max_position_embeddings=32768)),
+    "qwen3-tiny": ("Qwen3Config", dict(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=64, intermediate_size=512, num_hidden_layers=2, vocab_size=1000)),
+    "llama-tiny": ("LlamaConfig", dict(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, intermediate_size=512, num_hidden_layers=2, vocab_size=1000)),
+}  # fmt: skip
+
+
+def _trace_model(args):
+    """``(graph, program)`` for a model input, the way the reference's ``compile <model> [--layer N] [--seq-len S]`` traces
+    one (emmy/commands/trace.py:61-106): the whole causal LM on token ids, or one decoder layer on hidden states and
+    its rotary tables.  The model comes from a local directory or a built-in architecture; nothing is downloaded."""
+    import torch
+    from torch import nn
+
+    from deplodock_amd.commands.code import InlineProgram, slugify
+    from deplodock_amd.trace.torch import trace_module
+
+    try:
+        import transformers as tf
+    except ImportError:
+        print("error: a model input needs the transformers package", file=sys.stderr)
+        sys.exit(1)
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype]
+    torch.manual_seed(args.seed)
+    spec = args.input
+    if spec.startswith("arch:"):
+        name = spec[5:]
+        if name not in ARCHITECTURES:
+            print(f"error: unknown architecture {name!r}; known: {', '.join(sorted(ARCHITECTURES))}", file=sys.stderr)
+            sys.exit(2)
+        cfg_cls, kw = ARCHITECTURES[name]
+        cfg = getattr(tf, cfg_cls)(pad_token_id=0, eos_token_id=1, bos_token_id=2, **kw)
+        model = tf.AutoModelForCausalLM.from_config(cfg)
+    elif Path(spec).is_dir():
+        if spec.endswith(".json") or not (Path(spec) / "config.json").exists():
+            print(f"error: {spec} holds no config.json", file=sys.stderr)
+            sys.exit(2)
+        cfg = tf.AutoConfig.from_pretrained(spec, local_files_only=True)
+        model = None
+        if not args.random_weights:
+            try:
+                model = tf.AutoModelForCausalLM.from_pretrained(spec, local_files_only=True, torch_dtype=dtype)
+            except (OSError, ValueError) as exc:
+                print(f"note: no weights loaded from {spec} ({str(exc).splitlines()[0][:120]}); random weights instead", file=sys.stderr)
+        if model is None:
+            model = tf.AutoModelForCausalLM.from_config(cfg)
+    else:
+        print(f"error: {spec!r} is neither a local model directory nor 'arch:<name>'; hub model IDs need a download, which this environment does not do "
+              "(IR files go to `run --ir`)", file=sys.stderr)  # fmt: skip
+        sys.exit(2)
+    model.config._attn_implementation = "sdpa"
+    model = model.to(dtype).eval()
+    seq = int(args.seq_len)
+    if args.layer is None:
+
+        class Logits(nn.Module):
+            def __init__(self, m):
+                super().__init__()
+                self.m = m
+
+            def forward(self, input_ids):
+                return self.m(input_ids=input_ids).logits
+
+        module, inputs, kwargs = Logits(model).eval(), (torch.randint(0, int(model.config.vocab_size), (1, seq)),), {}
+        slug = f"{slugify(spec)}-full-s{seq}"
+    else:
+        layers = model.model.layers
+        if not 0 <= args.layer < len(layers):
+            print(f"error: layer {args.layer} not found (the model has {len(layers)})", file=sys.stderr)
+            sys.exit(1)
+
+        class Layer(nn.Module):
+            def __init__(self, layer):
+                super().__init__()
+                self.l = layer
+
+            def forward(self, x, cos, sin):
+                out = self.l(x, position_embeddings=(cos, sin), attention_mask=None)
+                return out[0] if isinstance(out, tuple) else out
+
+        x = torch.randn(1, seq, int(model.config.hidden_size))
+        cos, sin = model.model.rotary_emb(x.to(dtype), torch.arange(seq)[None])
+        module, inputs, kwargs = Layer(layers[args.layer]).eval(), (x.to(dtype), cos.to(dtype), sin.to(dtype)), {}
+        slug = f"{slugify(spec)}-layer{args.layer}-s{seq}"
+    graph = trace_module(module, inputs, dynamic_shapes=parse_dynamic(args.dynamic))
+    return graph, InlineProgram(module=module, args=inputs, kwargs=kwargs, slug=slug)
 
 
 def parse_dynamic(specs: list[str] | None) -> dict | None:

@@ -84,6 +84,19 @@ def _to_device(obj, device):
     return obj
 
 
+def _to_dtype(obj, dtype):
+    """Floating-point tensors of a nested argument structure cast to ``dtype`` (integer tensors stay)."""
+    import torch
+
+    if isinstance(obj, torch.Tensor):
+        return obj.to(dtype) if obj.is_floating_point() else obj
+    if isinstance(obj, (list, tuple)):
+        return type(obj)(_to_dtype(o, dtype) for o in obj)
+    if isinstance(obj, dict):
+        return {k: _to_dtype(v, dtype) for k, v in obj.items()}
+    return obj
+
+
 def _flatten_tensors(obj) -> list:
     import torch
 
@@ -264,7 +277,20 @@ def handle_run(args) -> None:
         torch.cuda.synchronize()
         outs = program.output_tensors()
         ok_all = True
-        for name, w in zip(compiled.outputs, want):
+        deep = bool(args.input) and want and want[0].dtype in (torch.bfloat16, torch.float16)
+        if deep:
+            # Layers deep in 16 bits an element-wise bound says little (eager's own result sits as far from the fp32
+            # run): the mean distance from the fp32 run of the same model may be at most 1.5 x 16-bit eager's.
+            with torch.no_grad():
+                exact = _flatten_tensors(module.float()(*_to_dtype(d_args, torch.float32), **_to_dtype(d_kwargs, torch.float32)))
+                module.to(want[0].dtype)
+            for name, w, e in zip(compiled.outputs, want, exact):
+                err = float((outs[name].reshape(e.shape).float() - e).abs().mean())
+                base = float((w.float() - e).abs().mean())
+                ok = err <= 1.5 * base or err == 0.0
+                ok_all &= ok
+                print(f"{'PASS' if ok else 'FAIL'}  {name}: mean |ours - fp32 eager| {err:.4g}, mean |{str(w.dtype).replace('torch.', '')} eager - fp32 eager| {base:.4g} (limit 1.5 x)")
+        for name, w in zip(compiled.outputs, want if not deep else []):
             ok, line = check_accuracy(outs[name], w)
             ok_all &= ok
             print(f"{'PASS' if ok else 'FAIL'}  {name}: {line}")

@@ -55,6 +55,7 @@ class StackedConstant:
     parts: tuple[str, ...]
     k_scale: str | None = None  # a length-k constant multiplied into every row (a norm weight folded into the projection)
     transpose: bool = False  # the last two axes swapped afterwards (a ``[K, N]`` weight of ``x @ w`` stored as the ``[N, K]`` rows a contraction reads)
+    pad_rows_to: int = 0  # zero rows appended up to this many (an output width that is not whole runs of four columns: a 151 669-word vocabulary)
 
 
 @dataclass
@@ -318,6 +319,24 @@ def _rec_linear(c: _Ctx, nid: str) -> bool:
     if not isinstance(node.op, F.LinearOp):
         return False
     x, w, m, n, k, lda, ldb, pro, extra = _linear_parts(c, nid)
+    if n % 4 and not node.op.has_bias:
+        # The contraction stores runs of four columns: the weight gets zero rows up to the next multiple of four (a
+        # parameter: once, at bind time; else by the copy kernel) and the result is a window of the wider buffer.
+        n_pad = -(-n // 4) * 4
+        base = c.out.nodes.get(w.base)
+        if isinstance(base.op, ConstantOp) and base.op.value is None and w.offset == 0 and tuple(w.strides) == (k, 1):
+            pid = f"{w.base}__rows{n_pad}"
+            if pid not in c.out.nodes:
+                c.out.add_constant(pid, (n_pad, k), w.dtype)
+                c.out.nodes[pid].hints["stacked"] = StackedConstant((w.base,), pad_rows_to=n_pad)
+            w = View(pid, 0, (n_pad, k), (k, 1), w.dtype)
+        else:
+            w = _copy_of_view(c, w, (0, 1), f"{nid}__w", pad_rows_to=n_pad)
+        lead = tuple(int(d) for d in node.output.shape[:-1])
+        body = Contraction(m=m, n=n_pad, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=lda, ldb=k, a_offset=x.offset, b_offset=0, a_prologue=pro)
+        _emit(c, nid, body, "rms_norm_linear" if pro else "linear", [x.base, w.base, *extra], shape=(*lead, n_pad))
+        c.windows[nid] = (0, (*lead, n), contiguous_strides((*lead, n_pad)))
+        return True
     bias = _bias_of(c, nid, n)
     body = Contraction(m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=node.output.dtype, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset, a_prologue=pro, **bias)
     _emit(c, nid, body, "rms_norm_linear" if pro else "linear", [x.base, w.base, *extra, *([bias["bias"]] if bias else [])])

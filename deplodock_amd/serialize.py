@@ -122,7 +122,7 @@ def _hints_to_dict(hints: dict, where: str) -> dict:
     out = {}
     for k, v in hints.items():
         if isinstance(v, StackedConstant):
-            out[k] = {"$stacked": list(v.parts), **({"k_scale": v.k_scale} if v.k_scale else {}), **({"transpose": True} if v.transpose else {})}
+            out[k] = {"$stacked": list(v.parts), **({"k_scale": v.k_scale} if v.k_scale else {}), **({"transpose": True} if v.transpose else {}), **({"pad_rows_to": v.pad_rows_to} if v.pad_rows_to else {})}
         else:
             out[k] = _enc(v, f"{where}.hints[{k}]")
     return out
@@ -131,7 +131,7 @@ def _hints_to_dict(hints: dict, where: str) -> dict:
 def _hints_from_dict(d: dict) -> dict:
     from deplodock_amd.passes.fuse import StackedConstant
 
-    return {k: StackedConstant(tuple(v["$stacked"]), k_scale=v.get("k_scale"), transpose=bool(v.get("transpose", False))) if isinstance(v, dict) and "$stacked" in v else _dec(v) for k, v in d.items()}
+    return {k: StackedConstant(tuple(v["$stacked"]), k_scale=v.get("k_scale"), transpose=bool(v.get("transpose", False)), pad_rows_to=int(v.get("pad_rows_to", 0))) if isinstance(v, dict) and "$stacked" in v else _dec(v) for k, v in d.items()}
 
 
 def graph_to_dict(g: Graph) -> dict:

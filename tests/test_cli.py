@@ -141,3 +141,40 @@ def test_tune_command_fills_a_database_run_then_uses(tmp_path, capsys):
     assert "row_reduce/r512/c1024" in out and f"database: {db}" in out
     main(["run", "--tune-db", str(db), "-c", "nn.RMSNorm(1024)(torch.randn(512, 1024))"])
     assert capsys.readouterr().out.startswith("PASS")
+
+
+def test_compile_a_built_in_architecture_whole_and_by_layer(capsys):
+    """``compile <model> [--layer N] [--seq-len S]`` as the reference's command takes a model
+    (emmy/commands/compile.py:66-97), from a built-in architecture with random weights: no download, no GPU."""
+    main(["compile", "arch:qwen3-tiny", "--seq-len", "16"])
+    out = capsys.readouterr().out
+    assert out.count("k_index_rows") >= 1 and out.count("// ---- k_sdpa_reduce") == 2  # embedding gather, two layers
+    main(["compile", "arch:qwen3-tiny", "--layer", "1", "--seq-len", "48", "--dtype", "fp32"])
+    out = capsys.readouterr().out
+    assert "k_index_rows" not in out and out.count("// ---- k_batched_linear") == 2  # one layer; fp32 attention is decomposed
+
+
+def test_compile_a_local_model_directory(tmp_path, capsys):
+    import transformers as tf
+
+    tf.LlamaConfig(hidden_size=128, num_attention_heads=2, num_key_value_heads=1, intermediate_size=256, num_hidden_layers=1, vocab_size=301, pad_token_id=0, eos_token_id=1, bos_token_id=2).save_pretrained(tmp_path)
+    main(["compile", str(tmp_path), "--seq-len", "8"])
+    captured = capsys.readouterr()
+    assert "random weights instead" in captured.err  # the directory holds a config and no weights
+    assert "N=304" in captured.out  # the 301-word vocabulary is padded to whole runs of four columns
+
+
+@pytest.mark.parametrize("argv, code", [(["compile", "Qwen/Qwen3-Embedding-0.6B"], 2), (["compile", "arch:nope"], 2), (["compile", "arch:qwen3-tiny", "--layer", "9"], 1), (["compile", "arch:qwen3-tiny", "-c", "torch.exp(torch.randn(4))"], 2)])
+def test_model_inputs_that_are_refused(argv, code, capsys):
+    with pytest.raises(SystemExit) as e:
+        main(argv)
+    assert e.value.code == code and "error:" in capsys.readouterr().err
+
+
+@pytest.mark.gpu
+def test_run_a_built_in_architecture(capsys):
+    main(["run", "--bench", "--iters", "5", "--warmup", "1", "arch:qwen3-tiny", "--seq-len", "40"])
+    out = capsys.readouterr().out
+    assert out.startswith("PASS") and "mean |ours - fp32 eager|" in out and "emmy (hip)" in out
+    main(["run", "arch:llama-tiny", "--dtype", "fp32", "--layer", "0", "--seq-len", "24"])
+    assert capsys.readouterr().out.startswith("PASS")

@@ -1409,6 +1409,9 @@ def _op_cases():
         "clamp": (_Fn(lambda t: t.clamp(-0.5, 0.7)), lambda: (x(3, 100),)),
         "clamp_min": (_Fn(lambda t: t.clamp_min(0.1) * 2), lambda: (x(3, 100),)),
         "vector_norm_axis1": (_Fn(lambda t: torch.linalg.vector_norm(t, dim=1)), lambda: (x(4, 33, 40),)),
+        # an output width that is not whole runs of four columns (a 151 669-word vocabulary in small): padded weight, windowed result
+        "linear_odd_width": (nn.Linear(64, 37, bias=False), lambda: (x(5, 9, 64),)),
+        "linear_odd_width_then_softmax": (nn.Sequential(nn.Linear(64, 37, bias=False), nn.Softmax(-1)), lambda: (x(21, 64),)),
         # a transformer MLP of the GELU family, and a pre-norm projection
         "gelu_mlp": (nn.Sequential(nn.Linear(256, 512), nn.GELU(), nn.Linear(512, 256)), lambda: (x(2, 48, 256),)),
         "layer_norm_linear": (nn.Sequential(nn.LayerNorm(256), nn.Linear(256, 128)), lambda: (x(4, 33, 256),)),
