@@ -156,7 +156,15 @@ def _run_at(be, compiled, module, d_args, d_kwargs, spec: str) -> bool:
         for axis, sym in axes.items():
             if sym == name:
                 shape[axis] = size
-        resized.append(torch.randn(shape, device=t.device).to(t.dtype) if tuple(shape) != tuple(t.shape) else t)
+        if tuple(shape) == tuple(t.shape):
+            resized.append(t)
+        elif t.is_floating_point():
+            resized.append(torch.randn(shape, device=t.device).to(t.dtype))
+        else:
+            # an index tensor (token ids): values drawn from the ones it already holds, so every index stays valid for
+            # eager too (an embedding lookup of an arbitrary integer reads outside its table)
+            pick = torch.randint(0, t.numel(), tuple(shape), device=t.device)
+            resized.append(t.reshape(-1)[pick.reshape(-1)].reshape(shape))
     it = iter(resized)
 
     def rebuild(obj):

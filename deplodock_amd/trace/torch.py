@@ -66,6 +66,9 @@ class DynamicSpec:
         from torch.utils import _pytree as pytree
 
         leaves, tree = pytree.tree_flatten((tuple(self.example_inputs), dict(self.kwargs)))
+        # the example tensors live where the module's parameters do by now (a caller may have moved it to the GPU since the first trace)
+        where = next((p.device for p in self.module.parameters()), None) if hasattr(self.module, "parameters") else None
+        where = where if where is not None else next((b.device for b in self.module.buffers()), None) if hasattr(self.module, "buffers") else where
         out = []
         t_i = 0
         for leaf in leaves:
@@ -75,12 +78,12 @@ class DynamicSpec:
             axes = self.input_axes[t_i]
             t_i += 1
             if not axes:
-                out.append(leaf)
+                out.append(leaf.to(where) if where is not None else leaf)
                 continue
             shape = list(leaf.shape)
             for axis, sym in axes.items():
                 shape[axis] = int(env[sym])
-            out.append(torch.zeros(shape, dtype=leaf.dtype))  # tracing reads shapes and dtypes only
+            out.append(torch.zeros(shape, dtype=leaf.dtype, device=where))  # tracing reads shapes and dtypes only
         args, kwargs = pytree.tree_unflatten(out, tree)
         g = trace_module(self.module, args, kwargs=kwargs or None)
         g.dynamic = DynamicSpec(self.module, self.example_inputs, self.kwargs, self.input_axes, self.hints)
@@ -309,11 +312,11 @@ def trace_module(module, example_inputs: tuple, kwargs: dict | None = None, dyna
                 # plain lower triangle is the kernel's own causal form; anything else becomes the additive bias it stands for
                 keep = folded[mask.name]
                 sq, skv = int(a[0].meta["val"].shape[-2]), int(a[1].meta["val"].shape[-2])
-                tri = torch.ones(sq, skv, dtype=torch.bool).tril()
+                tri = torch.ones(sq, skv, dtype=torch.bool, device=keep.device).tril()
                 if keep.shape[-2:] == (sq, skv) and sq == skv and not causal and bool((keep == tri).all()):
                     mask, causal = None, True
                 else:
-                    bias = torch.zeros(keep.shape, dtype=a[0].meta["val"].dtype).masked_fill(~keep, float("-inf"))
+                    bias = torch.zeros(keep.shape, dtype=a[0].meta["val"].dtype, device=keep.device).masked_fill(~keep, float("-inf"))
                     folded[f"{mask.name}__bias"] = bias
                     mask = type("Folded", (), {"name": f"{mask.name}__bias"})()
             elif mask is not None:
