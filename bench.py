@@ -341,6 +341,7 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
                 row["achieved_cold"] = round(case.algo_bytes / (c_us * 1e-6) / 1e9, 1)
         if eager_us is not None:
             row["eager_gpu_us"] = round(eager_us, 1)
+            row["tokens_per_s"] = round(int(case.inputs[0].numel()) / (us * 1e-6))
             row.pop("per_kernel_us", None)  # (142 entries: the five kernels of a layer are the C5 row's)
         if cpu and not whole_model:
             row["cpu_us"] = round(_cpu_us(case), 1)
