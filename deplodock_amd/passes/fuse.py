@@ -531,8 +531,8 @@ def _rec_gate_up(c: _Ctx, nid: str) -> bool:
     for si, ui in ((0, 1), (1, 0)):
         silu = c.g.nodes[node.inputs[si]]
         up = c.g.nodes[node.inputs[ui]]
-        if not (_is(silu, F.ElementwiseOp, fn="silu") and c.single_use(silu.id) and isinstance(up.op, F.LinearOp) and c.single_use(up.id)):
-            continue
+        if not (isinstance(silu.op, F.ElementwiseOp) and silu.op.fn in ("silu", "gelu_tanh", "gelu") and len(silu.inputs) == 1 and c.single_use(silu.id) and isinstance(up.op, F.LinearOp) and c.single_use(up.id)):
+            continue  # (SwiGLU, or GeGLU in either GELU form: the activation is a name in the tile's epilogue)
         gate = c.g.nodes[silu.inputs[0]]
         if not (isinstance(gate.op, F.LinearOp) and c.single_use(gate.id)) or gate.op.has_bias or up.op.has_bias:
             continue
@@ -549,9 +549,9 @@ def _rec_gate_up(c: _Ctx, nid: str) -> bool:
             c.out.add_constant(stacked, (2 * n, k), wg.output.dtype)
             c.out.nodes[stacked].hints["stacked"] = StackedConstant((wg.id, wu.id), k_scale=fold_w)
         od = node.output.dtype
-        epi = _round(od, E.Un("silu", _round(od, E.Var("acc")))) * _round(od, E.Var("acc2"))
+        epi = _round(od, E.Un(silu.op.fn, _round(od, E.Var("acc")))) * _round(od, E.Var("acc2"))
         body = Contraction(m=m, n=n, k=k, a=x.base, b=stacked, out=nid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset, epilogue=epi, gate_pair=True, a_prologue=pro)
-        _emit(c, nid, body, "rms_norm_linear_silu_mul" if pro else "linear_silu_mul", [x.base, stacked, *extra])
+        _emit(c, nid, body, ("rms_norm_" if pro else "") + f"linear_{silu.op.fn}_mul", [x.base, stacked, *extra])
         return True
     return False
 
