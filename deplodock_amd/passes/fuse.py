@@ -439,8 +439,10 @@ def _plain_projection(c: _Ctx, nid: str) -> bool:
     (so no other recognizer wants to absorb it) and is not a graph output."""
     g = c.g
     node = g.nodes[nid]
-    if not isinstance(node.op, F.LinearOp) or node.op.has_bias or nid in g.outputs or nid in c.done:
+    if not isinstance(node.op, F.LinearOp) or nid in g.outputs or nid in c.done:
         return False
+    if node.op.has_bias and not (isinstance(g.nodes[node.inputs[2]].op, ConstantOp) and len(g.nodes[node.inputs[2]].output.shape) == 1 and g.nodes[node.inputs[2]].op.value is None):
+        return False  # (a bias that is a plain parameter vector can be stacked like the weights)
     if not isinstance(g.nodes[node.inputs[1]].op, ConstantOp) or len(g.nodes[node.inputs[1]].output.shape) != 2:
         return False
     cons = g.consumers(nid)
@@ -465,6 +467,7 @@ def _rec_linear_siblings(c: _Ctx, nid: str) -> bool:
         and g.nodes[g.nodes[sid].inputs[1]].output.dtype == w0.dtype
         and g.nodes[g.nodes[sid].inputs[1]].output.shape[1] == w0.shape[1]
         and g.nodes[sid].output.shape[:-1] == node.output.shape[:-1]
+        and g.nodes[sid].op.has_bias == node.op.has_bias  # all biased (Qwen-2's q / k / v) or none
     ]
     if len(group) < 2:
         return False
@@ -483,8 +486,23 @@ def _rec_linear_siblings(c: _Ctx, nid: str) -> bool:
         c.out.nodes[stacked].hints["stacked"] = StackedConstant(tuple(weights), k_scale=fold_w)
     fid = "__".join(group)
     od = node.output.dtype
-    body = Contraction(m=m, n=n_total, k=k, a=x.base, b=stacked, out=fid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset, a_prologue=pro)
-    c.out.add_node(TileOp(name=c.kname("rms_norm_linear" if pro else "linear"), body=body), list(dict.fromkeys([x.base, stacked, *extra])), Tensor(fid, (m, n_total), od), fid)
+    bias_kw: dict = {}
+    bias_in: list[str] = []
+    if node.op.has_bias:
+        biases = [g.nodes[sid].inputs[2] for sid in group]
+        bdt = g.nodes[biases[0]].output.dtype
+        if any(g.nodes[b].output.dtype != bdt or int(g.nodes[b].output.shape[0]) != n for b, n in zip(biases, widths)):
+            return False
+        for b in biases:
+            _materialize(c, b)
+        sb = "__".join(biases)
+        if sb not in c.out.nodes:
+            c.out.add_constant(sb, (n_total,), bdt)
+            c.out.nodes[sb].hints["stacked"] = StackedConstant(tuple(biases))
+        bias_kw = {"bias": sb, "bias_dtype": bdt, "epilogue": E.Var("acc") + E.Var("bias")}
+        bias_in = [sb]
+    body = Contraction(m=m, n=n_total, k=k, a=x.base, b=stacked, out=fid, in_dtype=x.dtype, out_dtype=od, lda=lda, a_offset=x.offset, a_prologue=pro, **bias_kw)
+    c.out.add_node(TileOp(name=c.kname("rms_norm_linear" if pro else "linear"), body=body), list(dict.fromkeys([x.base, stacked, *extra, *bias_in])), Tensor(fid, (m, n_total), od), fid)
     col = 0
     for sid, n in zip(group, widths):
         shape = tuple(int(d) for d in g.nodes[sid].output.shape)
