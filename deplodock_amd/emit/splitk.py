@@ -48,6 +48,11 @@ def partial_body(body: Contraction, ws: str) -> Contraction:
     n = body.reduce.cta
     if n < 2:
         raise LoweringError("contraction: not a cross-workgroup split")
+    sym = getattr(body, "sym", None)
+    if sym is not None and sym.fields:
+        # ``sym`` is a plain attribute (``dataclasses.replace`` below would drop it) and the combine kernel bakes m in:
+        # a split kernel pair serves the traced size only, so the caller must lower per size instead.
+        raise LoweringError(f"contraction: a cross-workgroup split does not combine with a symbolic extent ({sorted(sym.fields)})")
     if body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None:
         raise LoweringError("contraction: a cross-workgroup split takes a plain contraction (no gate/up pair, row prologue or row epilogue)")
     if body.k % n or (body.tile is not None and (body.k // n) % body.tile.bk_elems):

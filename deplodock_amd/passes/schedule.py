@@ -389,6 +389,9 @@ def _fp32_underfilled(body: Contraction, plan: TilePlan, ctx: Context) -> tuple[
     8.5, 32x1024x2048 6.5 -> 4.8, 32x1024x1024 6.7 -> 4.1, 128x1024x1024 6.6 -> 6.2.  Problems whose 32x32 tiles
     already cover the CUs keep the unsplit default (128x1024x2048: 6.8 unsplit, 8.4 split in two)."""
     plain = not (body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None) and int(getattr(body, "batch", 1) or 1) == 1 and body.k_split is None
+    sym = getattr(body, "sym", None)
+    if sym is not None and sym.fields:
+        return plan, 1  # the split's kernel pair bakes the row count in: a runtime-int kernel stays unsplit
     if body.in_dtype.name != "f32" or not plain or not all(isinstance(d, int) for d in (body.m, body.n, body.k)) or body.m <= 16 or body.k % 32 or body.k < 256:
         return plan, 1
     base = -(-body.m // 32) * -(-body.n // 32)

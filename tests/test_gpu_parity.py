@@ -490,7 +490,7 @@ def test_dynamic_seq_len_per_size_variants_still_work(device):
     assert len(compiled.variants) == 2
 
 
-@pytest.mark.parametrize("which", ["rms_norm", "softmax", "silu_mul", "sdpa", "linear_bias"])
+@pytest.mark.parametrize("which", ["rms_norm", "softmax", "silu_mul", "sdpa", "linear_bias", "linear_f32"])
 def test_runtime_int_kernels_of_every_family(device, which):
     """Row kernels (rows symbolic), a pointwise map (element count symbolic), attention on ``[B, H, S, D]`` operands
     (lengths and the batch stride symbolic) and a biased linear (rows symbolic), each compiled once and run at
@@ -517,6 +517,12 @@ def test_runtime_int_kernels_of_every_family(device, which):
         mod = eager.Sdpa(True).eval()
         make = lambda s: (torch.randn(2, 4, s, 128).bfloat16(), torch.randn(2, 2, s, 128).bfloat16(), torch.randn(2, 2, s, 128).bfloat16())  # noqa: E731
         dyn, tol = {"q": {2: "s"}, "k": {2: "s"}, "v": {2: "s"}}, (2e-2, 2e-2)
+    elif which == "linear_f32":
+        # at the traced size the static fp32 lowering would split the reduction axis across workgroups (a kernel pair
+        # with the row count baked in): the runtime-int form must stay unsplit and serve every size
+        mod = nn.Linear(1024, 1024).eval()
+        make = lambda s: (torch.randn(s, 1024),)  # noqa: E731
+        dyn, tol = {"input": {0: "s"}}, (1e-5, 1e-5)
     else:
         mod = nn.Linear(256, 520).bfloat16().eval()
         make = lambda s: (torch.randn(s, 256).bfloat16(),)  # noqa: E731

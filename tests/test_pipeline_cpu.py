@@ -378,6 +378,29 @@ def test_a_symbolic_axis_lowers_to_kernels_that_take_it_as_a_runtime_int(launche
         trace_module(case.module, case.inputs, dynamic_shapes={"nope": {1: "s"}})
 
 
+def test_a_symbolic_fp32_linear_never_takes_the_cross_workgroup_split(launcher_lib, monkeypatch):
+    """A split contraction is a kernel pair with the row count baked in (partial grid, combine extent).  A module
+    traced with a symbolic row count must therefore either come out as runtime-int kernels on every launch (the
+    fp32 tier's automatic split stands down) or not be marked symbolic at all (a pinned split: per-size lowering)."""
+    import torch.nn as nn
+
+    mod = nn.Linear(1024, 1024).eval()
+    g = trace_module(mod, (torch.randn(64, 1024),), dynamic_shapes={"input": {0: "seq"}})
+    be = HipBackend()
+    compiled = be.compile(g)
+    assert compiled.symbolic == "seq"
+    ks = kernels(compiled)
+    assert ks and all(k.runtime_args == ("seq",) for k in ks), [(k.kernel_name, k.runtime_args) for k in ks]
+    assert not any("partial" in k.kernel_name or "combine" in k.kernel_name for k in ks)
+    # the static lowering of the same shape does split (so the case above is the one the guard is for)
+    static = be.compile(trace_module(mod, (torch.randn(64, 1024),)))
+    assert any("partial" in k.kernel_name for k in kernels(static))
+    # a pinned split cannot be symbolic: the backend falls back to lowering per size
+    monkeypatch.setenv("EMMY_REDUCE", "g4k")
+    pinned = HipBackend().compile(trace_module(mod, (torch.randn(64, 1024),), dynamic_shapes={"input": {0: "seq"}}))
+    assert getattr(pinned, "symbolic", None) is None and hasattr(pinned, "variants")
+
+
 def test_per_size_specialisation_remains_for_what_does_not_symbolise(launcher_lib):
     """With runtime-int kernels switched off (or a module whose kernel boundaries change with the size) the backend
     re-traces and re-lowers per distinct size and keeps an LRU of the results."""
