@@ -36,6 +36,9 @@ class HipBackend(Backend):
         context: Context | None = None,
     ) -> None:
         self.debug = config.debug_enabled() if debug is None else debug
+        #: what the last ``run`` under ``debug`` kept: per-launch host copies of every scratch / output buffer
+        #: (``DebugResult``); ``None`` after a plain run (emmy/compiler/backend/cuda/backend.py:158-161)
+        self.last_debug_result = None
         self.dump = dump
         self.bench_wall_timeout_s = bench_wall_timeout_s
         self._worker = None
@@ -179,11 +182,18 @@ class HipBackend(Backend):
 
     # -- run ------------------------------------------------------------------
     def run(self, compiled: Graph, *, input_data: dict | None = None, pre_run=None) -> tuple[RunResult, object]:
-        from deplodock_amd.backend.hip.program import run_program
+        from deplodock_amd.backend.hip.program import run_program, run_program_debug
 
         self._select_device()
         compiled = self.variant(compiled, input_data)
-        result, pre = run_program(compiled, input_data=self.bind(compiled, input_data), pre_run=pre_run)
+        if self.debug:
+            # launch by launch with a device synchronisation and a host copy of every written buffer after each
+            result, pre = run_program_debug(compiled, input_data=self.bind(compiled, input_data), pre_run=pre_run)
+            self.last_debug_result = result
+            result = RunResult(outputs=result.outputs, time_ms=None)
+        else:
+            self.last_debug_result = None
+            result, pre = run_program(compiled, input_data=self.bind(compiled, input_data), pre_run=pre_run)
         outputs = {}
         for name, vals in result.outputs.items():
             outputs[name] = vals
@@ -218,8 +228,20 @@ class HipBackend(Backend):
         reference's keyword; here it re-points ``EMMY_HIPRTC_FLAGS`` for this one
         compile.  With ``bench_wall_timeout_s`` set and no ``on_iter`` callback the
         benchmark runs in an isolated worker process that is killed at the limit
-        (``RuntimeError``, the caller's bench_fail); otherwise in this process."""
-        return self.benchmark(compiled, warmup=warmup, num_iters=num_iters, on_iter=on_iter, hiprtc_flags=nvcc_flags, capture_graphs=capture_graphs, input_data=input_data)
+        (``RuntimeError``, the caller's bench_fail); otherwise in this process.
+
+        The worker path waits for the worker's answer on a helper thread, so the event
+        loop keeps running other tasks while the benchmark is under way (the reference
+        awaits its subprocess, backend/cuda/program.py:1382-1533).  The in-process path
+        issues device work from the calling thread — torch's current device and stream
+        are per thread — and blocks for its (bounded) duration."""
+        kwargs = dict(warmup=warmup, num_iters=num_iters, on_iter=on_iter, hiprtc_flags=nvcc_flags, capture_graphs=capture_graphs, input_data=input_data)
+        if self.bench_wall_timeout_s is not None and on_iter is None:
+            import asyncio
+            import functools
+
+            return await asyncio.get_running_loop().run_in_executor(None, functools.partial(self.benchmark, compiled, **kwargs))
+        return self.benchmark(compiled, **kwargs)
 
     def benchmark(self, compiled: Graph, *, warmup: int = 5, num_iters=20, on_iter=None, hiprtc_flags: str | None = None, capture_graphs: bool = True, input_data: dict | None = None) -> BenchmarkResult:
         from deplodock_amd.backend.hip.program import benchmark_program

@@ -117,16 +117,14 @@ extern "C" __global__ __launch_bounds__(256) void emh_zero_words(unsigned int* _
 """
 
 
-def _launches(graph: Graph) -> list[Node]:
-    nodes = []
-    for nid in graph.topological_order():
-        node = graph.nodes[nid]
-        if isinstance(node.op, (InputOp, ConstantOp)):
-            continue
-        if not isinstance(node.op, HipOp):
-            raise TypeError(f"HipBackend: node {nid!r} has non-HipOp {type(node.op).__name__!r}; lowering must produce Graph[HipOp].")
-        nodes.append(node)
-    return nodes
+def _kernel_nodes(graph: Graph) -> list[Node]:
+    """The graph's launches in program order; anything that is neither a kernel nor an input / constant is a
+    lowering bug and is reported by node."""
+    order = [graph.nodes[nid] for nid in graph.topological_order()]
+    stray = next((n for n in order if not isinstance(n.op, (InputOp, ConstantOp, HipOp))), None)
+    if stray is not None:
+        raise TypeError(f"HipBackend: node {stray.id!r} has non-HipOp {type(stray.op).__name__!r}; lowering must produce Graph[HipOp].")
+    return [n for n in order if isinstance(n.op, HipOp)]
 
 
 def _buffers(graph: Graph) -> list[_Buffer]:
@@ -147,7 +145,7 @@ def _compile(graph: Graph) -> _Compiled:
     launches: list[_Launch] = []
     sources: dict[str, str] = {}
     # Pass 1 — validate the whole graph before anything touches the device.
-    for node in _launches(graph):
+    for node in _kernel_nodes(graph):
         op: HipOp = node.op
         kname = op.kernel_name
         if sources.setdefault(kname, op.kernel_source) != op.kernel_source:
@@ -374,8 +372,10 @@ class CompiledProgram:
         intervals = compute_live_intervals(list(sizes), compiled.launches)
         offsets, total = plan_offsets(intervals, sizes)
         if library_scratch:
-            if total > launcher.EMH_SCRATCH_MAX_BYTES:
-                raise ValueError(f"the program's intermediates need {total} bytes; the library's scratch array holds {launcher.EMH_SCRATCH_MAX_BYTES}")
+            # what the library checks per launch is offset + size rounded up to whole 32-bit words
+            need = max((off + -(-sizes[name] // 4) * 4 for name, off in offsets.items()), default=0)
+            if max(total, need) > launcher.EMH_SCRATCH_MAX_BYTES:
+                raise ValueError(f"the program's intermediates need {max(total, need)} bytes; the library's scratch array holds {launcher.EMH_SCRATCH_MAX_BYTES}")
             slab = None
             for name, off in offsets.items():
                 arrays[name] = _LibraryScratch(off, -(-sizes[name] // 4) * 4)
@@ -402,8 +402,9 @@ class CompiledProgram:
             for i, name in enumerate(ln.arg_names):
                 t = self.arrays[name]
                 if isinstance(t, _LibraryScratch):
-                    if scratch is not None and scratch[1] != t.offset:
-                        raise ValueError(f"kernel {ln.kernel_name!r} names two scratch buffers; a launch can borrow one range of the library's scratch array")
+                    if scratch is not None:
+                        # also for one buffer named in two parameter slots: the library repoints a single slot
+                        raise ValueError(f"kernel {ln.kernel_name!r} takes scratch memory in two parameter slots; a launch can borrow one range of the library's scratch array for one parameter")
                     scratch = (i, t.offset, t.nbytes, name in ln.zero_outputs)
                     ptrs.append(0)
                     continue
@@ -454,6 +455,11 @@ class CompiledProgram:
     def outputs(self) -> dict[str, np.ndarray]:
         _torch().cuda.synchronize()
         return {b.name: _host(self.arrays[b.name], b.dtype) for b in self.compiled.bufs if b.role == "output"}
+
+    def snapshot(self) -> dict[str, np.ndarray]:
+        """Host copies of every buffer the program writes (scratch and outputs), as they are now."""
+        _torch().cuda.synchronize()
+        return {b.name: _host(self.arrays[b.name], b.dtype) for b in self.compiled.bufs if b.role in ("scratch", "output") and b.name in self.arrays}
 
     def output_tensors(self) -> dict:
         return {b.name: self.arrays[b.name] for b in self.compiled.bufs if b.role == "output"}
@@ -634,16 +640,155 @@ def run_program(graph: Graph, input_data: dict | None = None, pre_run=None) -> t
     return RunResult(outputs=outputs, time_ms=elapsed), pre_result
 
 
-def _resolve_iter_budget(num_iters) -> tuple[float, int, bool]:
-    if isinstance(num_iters, str):
-        if num_iters != "auto":
-            raise ValueError(f"num_iters must be int or 'auto', got {num_iters!r}")
-        return (_AUTO_BUDGET_MS, _AUTO_MAX_ITERS, True)
-    return (float("inf"), int(num_iters), False)
+@dataclass
+class DebugResult:
+    """What a debug run keeps: the program's outputs and, per launch index, a host copy of every buffer that is
+    not an input or a constant, taken right after that launch finished (the reference's ``DebugResult``,
+    emmy/compiler/backend/cuda/program.py:1122-1125)."""
+
+    outputs: dict[str, np.ndarray]
+    per_launch: dict[int, dict[str, np.ndarray]] = field(default_factory=dict)
+    kernel_names: dict[int, str] = field(default_factory=dict)
 
 
-def _calibrate_batch_sizes(iter_dts: list[float]) -> list[int]:
-    return [max(1, int(round(_BATCH_TARGET_MS / dt))) if 0 < dt < _BATCH_TARGET_MS else 1 for dt in iter_dts]
+def run_program_debug(graph: Graph, input_data: dict | None = None, pre_run=None) -> tuple[DebugResult, object]:
+    """Run the program once, launch by launch, synchronising after each launch and copying every scratch and
+    output buffer to the host (program.py:1128-1149).  Scratch buffers share one slab planned by live interval:
+    a buffer read *after its last use* shows whatever took its place, a launch's own output is what that launch
+    wrote."""
+    shots: dict[int, dict[str, np.ndarray]] = {}
+    names: dict[int, str] = {}
+    with gpu_lock():
+        prog = CompiledProgram.build(graph, input_data)
+        try:
+            pre_result = pre_run() if pre_run is not None else None
+            torch = _torch()
+            stream = prog._torch_stream()
+            for i, ln in enumerate(prog.compiled.launches):
+                prog.launch_one(i, stream)
+                torch.cuda.synchronize()
+                shots[i] = prog.snapshot()
+                names[i] = ln.kernel_name
+            outputs = prog.outputs()
+        finally:
+            prog.close()
+    return DebugResult(outputs=outputs, per_launch=shots, kernel_names=names), pre_result
+
+
+@dataclass(frozen=True)
+class SampleBudget:
+    """When sampling stops: after ``max_samples`` measured passes, or — ``device_ms`` set, the ``"auto"`` mode — once
+    that much device time has been measured, whichever comes first."""
+
+    max_samples: int
+    device_ms: float | None = None
+
+    @classmethod
+    def parse(cls, num_iters) -> "SampleBudget":
+        if num_iters == "auto":
+            return cls(_AUTO_MAX_ITERS, _AUTO_BUDGET_MS)
+        if isinstance(num_iters, str):
+            raise ValueError(f"num_iters must be an int or 'auto', got {num_iters!r}")
+        return cls(int(num_iters))
+
+    def spent(self, samples: int, measured_ms: float) -> bool:
+        return samples >= self.max_samples or (self.device_ms is not None and measured_ms >= self.device_ms)
+
+
+def window_issues(per_issue_ms: float) -> int:
+    """Back-to-back issues of one launch that make an event window of about ``_BATCH_TARGET_MS``."""
+    if not 0.0 < per_issue_ms < _BATCH_TARGET_MS:
+        return 1
+    return max(1, round(_BATCH_TARGET_MS / per_issue_ms))
+
+
+class _BenchSession:
+    """The three phases of a benchmark over one built program: *probe* (single issues, to learn how long each
+    launch takes), *settle* (size the event windows from the probe, capture them into graphs, keep the device
+    busy until it has warmed up) and *sample*.  Every pass over the program goes through ``_pass``, which keeps
+    the device-time account the run budget is checked against."""
+
+    def __init__(self, prog: "CompiledProgram", *, on_iter, run_timeout_s: float | None, capture: bool) -> None:
+        self.prog = prog
+        self.on_iter = on_iter
+        self.limit_ms = None if run_timeout_s is None else run_timeout_s * 1000.0
+        self.capture = capture
+        self.n = len(prog.compiled.launches)
+        self.issues = [1] * self.n
+        self.device_ms = 0.0
+        self.last: list[float] = []
+
+    def _charge(self, ms: float) -> None:
+        self.device_ms += ms
+        if self.limit_ms is not None and self.device_ms > self.limit_ms:
+            raise RuntimeError(f"benchmark run stage exceeded {self.limit_ms / 1000.0:.1f}s of GPU time — variant marked bench_fail")
+
+    def _pass(self) -> float:
+        """One pass over the program's windows; returns the device time it took."""
+        self.last = self.prog.iter_once(self.issues, pre_iter=self.on_iter)
+        took = sum(dt * k for dt, k in zip(self.last, self.issues))
+        self._charge(took)
+        return took
+
+    def _capture_windows(self) -> None:
+        if not self.capture:
+            return
+        try:
+            self.prog.capture_launch_graphs(self.issues)
+        except GraphCaptureError as exc:
+            logger.warning("[hip] %s — continuing with uncaptured (dispatch-inclusive) timing", exc)
+            self.capture = False
+
+    def probe(self, passes: int) -> None:
+        for _ in range(passes):
+            self._pass()
+
+    def settle(self) -> None:
+        if self.last:
+            self.issues = [window_issues(dt) for dt in self.last]
+        self._capture_windows()
+        if not self.last:
+            return  # no warm-up asked for: sample from the first pass on
+        took = self._pass() if self.device_ms < _WARMUP_TARGET_MS else 0.0
+        while took > 0.0 and self.device_ms < _WARMUP_TARGET_MS:
+            took = self._pass()
+
+    def sample(self, budget: SampleBudget) -> tuple[list[list[float]], list[float]]:
+        per_launch: list[list[float]] = [[] for _ in range(self.n)]
+        whole: list[float] = []
+        whole_windows = self._whole_program_windows if self.n > 1 and self.capture else None
+        measured_ms, count = 0.0, 0
+        while not budget.spent(count, measured_ms):
+            measured_ms += self._pass()
+            count += 1
+            for column, dt in zip(per_launch, self.last):
+                column.append(dt)
+            if whole_windows is not None:
+                dt = whole_windows()
+                if dt is None:
+                    whole_windows = None
+                else:
+                    whole.append(dt)
+        return per_launch, whole
+
+    _whole_replays = 0
+
+    def _whole_program_windows(self) -> float | None:
+        """ms per run of the whole program from one window of graph launches; the graph (up to
+        ``_E2E_MAX_COPIES`` copies of the program, so the window holds device time only) is built on first use."""
+        prog = self.prog
+        if self._whole_replays == 0:
+            self._whole_replays = window_issues(sum(self.last))
+            try:
+                prog.capture_program_graph(repeat=min(self._whole_replays, _E2E_MAX_COPIES))
+            except GraphCaptureError as exc:
+                logger.warning("[hip] %s — skipping whole-program e2e timing", exc)
+                return None
+        copies = prog._program_graph_repeat
+        launches = max(1, -(-self._whole_replays // copies))
+        dt = prog.time_program_window(launches)
+        self._charge(dt * launches * copies)
+        return dt
 
 
 def _samples_to_result(samples: list[list[float]], launches: list[_Launch], *, captured: bool, e2e_samples: list[float]) -> BenchmarkResult:
@@ -676,77 +821,24 @@ def benchmark_program(
     run_timeout_s: float | None = None,
     capture_graphs: bool = True,
 ) -> BenchmarkResult:
-    """Time the program's launches with device events (program.py:1152-1325).
+    """Time the program's launches with device events (the contract of the reference's
+    ``benchmark_program``, program.py:1152-1325: ``BenchmarkResult`` with per-launch medians and samples,
+    ``captured``, whole-program ``e2e_ms`` for a multi-launch program).
 
-    One loop covers warm-up and measurement.  After ``warmup`` iterations the
-    per-launch batch sizes are calibrated so each event window spans about
-    ``_BATCH_TARGET_MS`` and, when ``capture_graphs`` holds, each batch is
-    captured into a graph so windows hold dense device work.  Warm-up is
-    extended until ``_WARMUP_TARGET_MS`` of device time has run.  Reported
-    per-launch time is the median of measured windows; a multi-launch program
-    also gets whole-program graph windows (``e2e_ms``).  Budgets: the per-window
-    watchdog (``HungKernelError``), ``run_timeout_s`` of accumulated device time,
-    and zero-elapsed windows raise ``RuntimeError`` (bench_fail)."""
-    target_total_ms, max_measured, auto = _resolve_iter_budget(num_iters)
+    Three phases (``_BenchSession``): ``warmup`` probe passes of single issues; then each launch's event window
+    is sized to about ``_BATCH_TARGET_MS`` of back-to-back issues, captured into a graph when ``capture_graphs``
+    holds, and passes go on until ``_WARMUP_TARGET_MS`` of device time has run; then ``num_iters`` measured passes
+    (``"auto"``: until ``_AUTO_BUDGET_MS`` of measured device time).  A multi-launch program also gets
+    whole-program graph windows per measured pass.  Budgets: the per-window watchdog (``HungKernelError``),
+    ``run_timeout_s`` of accumulated device time, and zero-elapsed windows raise ``RuntimeError`` (bench_fail)."""
+    budget = SampleBudget.parse(num_iters)
     with gpu_lock():
         prog = CompiledProgram.build(graph, input_data, compile_timeout_s=compile_timeout_s)
         try:
-            n = len(prog.compiled.launches)
-            batch_sizes = [1] * n
-            samples: list[list[float]] = [[] for _ in range(n)]
-            measure_e2e = n > 1
-            e2e_samples: list[float] = []
-            e2e_replays = 0
-            iters_run = measured = 0
-            cumulative_ms = total_ms = 0.0
-
-            def try_capture(sizes: list[int]) -> bool:
-                try:
-                    prog.capture_launch_graphs(sizes)
-                except GraphCaptureError as exc:
-                    logger.warning("[hip] %s — continuing with uncaptured (dispatch-inclusive) timing", exc)
-                    return False
-                return True
-
-            if capture_graphs and warmup == 0:
-                capture_graphs = try_capture(batch_sizes)
-            while True:
-                dts = prog.iter_once(batch_sizes, pre_iter=on_iter)
-                iters_run += 1
-                total_ms += sum(dts[i] * batch_sizes[i] for i in range(n))
-                if run_timeout_s is not None and total_ms > run_timeout_s * 1000.0:
-                    raise RuntimeError(f"benchmark run stage exceeded {run_timeout_s:.1f}s of GPU time — variant marked bench_fail")
-                if iters_run == warmup:
-                    batch_sizes = _calibrate_batch_sizes(dts)
-                    if capture_graphs:
-                        capture_graphs = try_capture(batch_sizes)
-                    if total_ms < _WARMUP_TARGET_MS:
-                        per_iter = sum(dts[i] * batch_sizes[i] for i in range(n))
-                        if per_iter > 0:
-                            warmup += int(math.ceil((_WARMUP_TARGET_MS - total_ms) / per_iter))
-                if iters_run <= warmup:
-                    continue
-                for i in range(n):
-                    samples[i].append(dts[i])
-                cumulative_ms += sum(dts[i] * batch_sizes[i] for i in range(n))
-                measured += 1
-                if measure_e2e and capture_graphs:
-                    if e2e_replays == 0:
-                        it = sum(dts)
-                        e2e_replays = max(1, int(round(_BATCH_TARGET_MS / it))) if 0 < it < _BATCH_TARGET_MS else 1
-                        try:
-                            # the window's replays sit in one graph (up to 64 copies of the program): device time only
-                            prog.capture_program_graph(repeat=min(e2e_replays, _E2E_MAX_COPIES))
-                        except GraphCaptureError as exc:
-                            logger.warning("[hip] %s — skipping whole-program e2e timing", exc)
-                            measure_e2e = False
-                    if measure_e2e:
-                        launches = max(1, -(-e2e_replays // prog._program_graph_repeat))
-                        dt = prog.time_program_window(launches)
-                        e2e_samples.append(dt)
-                        total_ms += dt * launches * prog._program_graph_repeat
-                if measured >= max_measured or (auto and cumulative_ms >= target_total_ms):
-                    break
-            return _samples_to_result(samples, prog.compiled.launches, captured=capture_graphs, e2e_samples=e2e_samples)
+            session = _BenchSession(prog, on_iter=on_iter, run_timeout_s=run_timeout_s, capture=capture_graphs)
+            session.probe(max(0, int(warmup)))
+            session.settle()
+            per_launch, whole = session.sample(budget)
+            return _samples_to_result(per_launch, prog.compiled.launches, captured=session.capture, e2e_samples=whole)
         finally:
             prog.close()

@@ -113,7 +113,8 @@ def _trace_model(args):
         model = None
         if not args.random_weights:
             try:
-                model = tf.AutoModelForCausalLM.from_pretrained(spec, local_files_only=True, torch_dtype=dtype)
+                # safetensors only: a pickled checkpoint would execute code from the file on load
+                model = tf.AutoModelForCausalLM.from_pretrained(spec, local_files_only=True, torch_dtype=dtype, use_safetensors=True, trust_remote_code=False)
             except (OSError, ValueError) as exc:
                 print(f"note: no weights loaded from {spec} ({str(exc).splitlines()[0][:120]}); random weights instead", file=sys.stderr)
         if model is None:

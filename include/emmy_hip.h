@@ -130,7 +130,10 @@ int emh_launch(void* fn, const unsigned grid[3], const unsigned block[3], unsign
  * when scratch_arg is not a slot of `args`.  Calls no hipMalloc / hipFree.
  * All calls on one GPU share that GPU's array and it keeps the last call's
  * contents: calls that overlap in time on one GPU (two streams, two threads)
- * race on it, and a kernel that accumulates must ask for zero_first. */
+ * race on it, and a kernel that accumulates must ask for zero_first.
+ * The array used is the one of the calling thread's *current* device
+ * (hipGetDevice), not of the device `stream` was created on: make the
+ * stream's device current before the call, as for emh_launch itself. */
 int emh_launch_scratch(void* fn, const unsigned grid[3], const unsigned block[3],
                        unsigned lds_bytes, void* stream, void** args, int nargs, int scratch_arg,
                        size_t scratch_offset, size_t scratch_bytes, int zero_first);

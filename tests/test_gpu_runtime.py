@@ -137,6 +137,68 @@ def test_isolated_benchmark_worker_is_killed_at_the_wall_limit_and_replaced(devi
     eager.assert_close(ours.reshape(want.shape), want, case.rtol, case.atol, "in-process run after worker kills")
 
 
+def test_debug_run_keeps_a_host_copy_of_every_written_buffer_per_launch(device):
+    """``HipBackend(debug=True)``: ``run`` goes launch by launch and ``last_debug_result`` holds, per launch index,
+    what every scratch / output buffer held right after it (emmy/compiler/backend/cuda/program.py:1128,
+    backend.py:158-161).  On the decoder block: five launches, each launch's own output differs from what it was
+    before the launch, the last launch's snapshot of the output is the run's output, and the outputs equal a plain
+    run's; a plain run afterwards clears ``last_debug_result``."""
+    case = eager.qwen3_block_case(seq=64)
+    be = HipBackend(debug=True)
+    compiled = be.compile(trace_module(case.module, case.inputs))
+    # inputs no other test uses: memory recycled from an earlier run of the same block cannot already hold these results
+    data = {n: (t * 0.37 if i == 0 else t).to(device) for i, (n, t) in enumerate(zip(compiled.inputs, case.inputs))}
+    res, _ = be.run(compiled, input_data=data)
+    dbg = be.last_debug_result
+    assert dbg is not None and res.time_ms is None
+    launches = [nid for nid in compiled.topological_order() if compiled.node_role(nid) in ("scratch", "output")]
+    assert sorted(dbg.per_launch) == list(range(len(launches))) == sorted(dbg.kernel_names) and len(launches) == 5
+    out = compiled.outputs[0]
+    for i, nid in enumerate(launches):
+        assert nid in dbg.per_launch[i] and out in dbg.per_launch[i]
+        if i:
+            assert not np.array_equal(dbg.per_launch[i][nid], dbg.per_launch[i - 1][nid]), f"launch {i} did not write {nid}"
+    assert np.array_equal(dbg.per_launch[len(launches) - 1][out], dbg.outputs[out]) and np.array_equal(res.outputs[out], dbg.outputs[out])
+    plain_be = HipBackend(debug=False)
+    plain, _ = plain_be.run(compiled, input_data=data)
+    assert plain_be.last_debug_result is None and plain.time_ms is not None
+    assert np.array_equal(plain.outputs[out], res.outputs[out])
+    be.debug = False
+    be.run(compiled, input_data=data)
+    assert be.last_debug_result is None
+
+
+def test_benchmark_async_leaves_the_event_loop_running_while_a_worker_benchmarks(device):
+    """With the isolated worker, ``benchmark_async`` waits for the worker's answer off the loop's thread: a task
+    scheduled beside it keeps ticking while the benchmark runs."""
+    case = eager.softmax_case(shape=(4096, 2048))
+    be = HipBackend(bench_wall_timeout_s=170.0)
+    compiled = be.compile(trace_module(case.module, case.inputs))
+
+    async def both():
+        ticks = 0
+        done = asyncio.Event()
+
+        async def ticker():
+            nonlocal ticks
+            while not done.is_set():
+                ticks += 1
+                await asyncio.sleep(0.005)
+
+        t = asyncio.ensure_future(ticker())
+        res = await be.benchmark_async(compiled, warmup=2, num_iters=20)
+        done.set()
+        await t
+        return res, ticks
+
+    try:
+        res, ticks = asyncio.run(both())
+    finally:
+        be.close()
+    assert res.time_ms > 0 and res.captured
+    assert ticks >= 5, f"the event loop ran {ticks} tick(s) during the benchmark"
+
+
 def test_run_budget_marks_bench_fail(device):
     case = eager.softmax_case(shape=(64, 2048))
     be = HipBackend(bench_run_timeout_s=1e-9)

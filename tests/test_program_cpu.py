@@ -48,11 +48,13 @@ def test_unknown_buffer_is_rejected():
 
 
 def test_batch_calibration_and_iter_budget():
-    assert program._calibrate_batch_sizes([0.002, 0.5, 3.0, 0.0]) == [500, 2, 1, 1]
-    assert program._resolve_iter_budget(20) == (float("inf"), 20, False)
-    assert program._resolve_iter_budget("auto")[2] is True
+    assert [program.window_issues(dt) for dt in (0.002, 0.5, 3.0, 0.0)] == [500, 2, 1, 1]
+    fixed = program.SampleBudget.parse(20)
+    assert not fixed.spent(19, 1e9) and fixed.spent(20, 0.0)
+    auto = program.SampleBudget.parse("auto")
+    assert auto.spent(1, program._AUTO_BUDGET_MS) and not auto.spent(1, 0.5 * program._AUTO_BUDGET_MS) and auto.spent(program._AUTO_MAX_ITERS, 0.0)
     with pytest.raises(ValueError):
-        program._resolve_iter_budget("many")
+        program.SampleBudget.parse("many")
 
 
 def test_no_device_means_a_loud_error_not_a_fallback():
