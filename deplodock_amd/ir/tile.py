@@ -279,6 +279,7 @@ class Flash:
     pair: bool = False  # causal only: a workgroup takes query block b and its mirror QBLOCKS-1-b
     deep: bool = False  # a K ring of three slots (K blocks requested two steps ahead) beside a V ring of two
     pair_steps: bool = True  # key steps unrolled in pairs so ring slots are compile-time (the lowering clears it if that build spills)
+    ws: bool = False  # wave-specialised form: four consumer waves (waves x kv_split = 4) and four staging waves
     # an additive bias on the scaled scores, ``[batch, head, query, key]`` addressed through (batch, head, query)
     # strides (0 = broadcast) with keys contiguous; ``None``: no mask operand
     mask: str | None = None
