@@ -532,7 +532,7 @@ def lds_plan(waves: int, kvs: int, bkv: int, head_dim: int, limit: int, deep: bo
 
 
 def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
-    if body.ws:
+    if body.ws or body.sp:
         from deplodock_amd.emit.flash_ws import emit_flash_ws
 
         return emit_flash_ws(body, name, ctx)

@@ -45,18 +45,18 @@ _PREFETCH = 3  # fragment reads are issued this many MFMAs ahead of their use
 _COST = {"max": 4, "misc": 4, "exp": 20, "cvt": 2, "add": 4}
 
 
-def ws_lds_plan(waves: int, kvs: int, head_dim: int, limit: int) -> dict:
+def ws_lds_plan(waves: int, kvs: int, head_dim: int, limit: int, rings: tuple[int, ...] = (4, 3)) -> dict:
     """``[K ring | V ring | Q tile]``; after the key loop the rings hold the parked partial results and the O
-    tile (the layout of ``flash.lds_plan``).  The ring depth is the largest of 4, 3 that fits."""
+    tile (the layout of ``flash.lds_plan``).  The ring depth is the largest of ``rings`` that fits."""
     slot = kvs * 32 * head_dim * 2
     tile = 32 * waves * head_dim * 2
     close = _close_plan(waves, kvs, 32, head_dim, 1 << 30)
     close_bytes = close["o_off"] + tile
-    for ring in (4, 3):
-        rings = 2 * ring * slot
-        if rings + tile <= limit and close_bytes <= rings:
-            return {"bytes": rings + tile, "ring": ring, "slot": slot, "q_off": rings, "o_off": close["o_off"], "park_ml": close["park_ml"]}
-    raise LoweringError(f"flash/ws: rings of three {slot}-byte sub-steps per operand and a {tile}-byte Q tile exceed {limit} B of LDS")
+    for ring in rings:
+        both = 2 * ring * slot
+        if both + tile <= limit and close_bytes <= both:
+            return {"bytes": both + tile, "ring": ring, "slot": slot, "q_off": both, "o_off": close["o_off"], "park_ml": close["park_ml"]}
+    raise LoweringError(f"flash: rings of {min(rings)} {slot}-byte sub-steps per operand and a {tile}-byte Q tile exceed {limit} B of LDS")
 
 
 class _Lines:
@@ -171,7 +171,13 @@ def _classic_softmax(a: _Lines, D: int, src: str, dst: str, *, masked: bool) -> 
 _LEAD_TICKS = 7  # ticks of vector work issued while the iteration's first fragment reads are in flight
 
 
-def _iteration(a: _Lines, D: int, *, par: int, has_pv: bool, kslot, vslot) -> None:
+def _request_statements(per_s: int) -> list[str]:
+    """The requests one staging thread issues in an iteration, in issue order: the V sub-step first, then the K one
+    (``EMH_SUB_BASES`` has named their scalar parts under the tags ``v`` and ``k``)."""
+    return [f"EMH_REQ_I(v, {i}, vvo0, vbase, V_SS, emh_vswz, V_RING)" for i in range(per_s)] + [f"EMH_REQ_I(k, {i}, kvo0, kbase, K_SS, emh_kswz, 0)" for i in range(per_s)]
+
+
+def _iteration(a: _Lines, D: int, *, par: int, has_pv: bool, kslot, vslot, t_expr: str | None = None, per_s: int = 0) -> None:
     """One steady consumer iteration on sub-block t (scores in ``sc<par>``): output MFMAs of sub-block t-1 (its
     probabilities in ``pq<par^1>``, V slot ``vslot``; none when ``has_pv`` is false: t = 0), the softmax of t
     (probabilities into ``pq<par>``), score MFMAs of sub-block t+1 (K slot ``kslot``) into ``sc<par^1>``.  Slots are ints
@@ -190,9 +196,15 @@ def _iteration(a: _Lines, D: int, *, par: int, has_pv: bool, kslot, vslot) -> No
     for i in range(max(len(pv), len(qk))):
         jobs += pv[i : i + 1] + qk[i : i + 1]
     body = _softmax_ticks(src, dst)
+    # self-staging waves: this iteration's requests, one behind each of the first MFMAs (a request that finds the memory
+    # pipeline full blocks its wave at issue; the other wave of the SIMD goes on)
+    reqs = _request_statements(per_s) if t_expr is not None else []
     a.open("")
     a("float psum;")
     a("EMH_STAMP_AT(3)  // since the end of the iteration before: the barrier")
+    if reqs:
+        a(f"EMH_SUB_BASES(v, ({t_expr}) + RING - 2, vbase, V_SS, V_RING)")
+        a(f"EMH_SUB_BASES(k, ({t_expr}) + RING, kbase, K_SS, 0)")
 
     def read(j: int) -> None:
         kind, arg = jobs[j]
@@ -240,12 +252,16 @@ def _iteration(a: _Lines, D: int, *, par: int, has_pv: bool, kslot, vslot) -> No
         if j + _PREFETCH < len(jobs):
             read(j + _PREFETCH)
         mfma(j)
+        if j < len(reqs):
+            a(reqs[j])
         target = lead_cost + total * (j + 1) / len(jobs)
         while idx < len(body) and (done + body[idx][1] / 2 <= target or j == len(jobs) - 1):
             ticks(1)
         if has_pv and j == len(jobs) // 2 - 1:
             a("EMH_STAMP_AT(1)  // the first half of the slices")
         a("__builtin_amdgcn_sched_barrier(0);")
+    for r in reqs[len(jobs):]:
+        a(r)
     a("EMH_STAMP_AT(2)  // the second half of the slices")
     a("l_run += psum; asm volatile(\"\" : \"+v\"(l_run));")
     if not has_pv:
@@ -253,16 +269,36 @@ def _iteration(a: _Lines, D: int, *, par: int, has_pv: bool, kslot, vslot) -> No
     a.close()
 
 
-def _consumer(a: _Lines, D: int, ring: int) -> None:
+def _consumer(a: _Lines, D: int, ring: int, per_s: int = 0) -> None:
     """The consumer role.  Naming is canonical at every loop boundary — the scores of the sub-block about to be
     reduced in ``sc0``, the probabilities of the one before it in ``pq1`` — so the unrolled loop has one entry, one
     back edge and one exit: ``lcm(2, ring)`` iterations per trip with ring slots and the double buffers' parity
     resolved in the text; what is left of a wave's full iterations runs in a loop with run-time slots that copies
-    the buffers back to their canonical names."""
+    the buffers back to their canonical names.
+
+    ``per_s`` > 0: the waves stage for themselves (no staging role): every iteration t, whatever the wave computes in
+    it, carries the wave's share of the requests of sub-steps V(t + ring - 2) and K(t + ring) and ends in ``EMH_LAND(t)``
+    (wait for what must have landed, publish, barrier) instead of a bare barrier."""
+    sp = per_s > 0
     L = ring * 2 // math.gcd(ring, 2)
     jobs = [(s, dt) for s in range(2) for dt in range(D // 32)]
-    a("// ---- consumers: one wave per SIMD, 32 query rows x the key blocks of one key-split group")
-    a("EMH_BARRIER();  // P: the Q tile and the first sub-steps of K have landed")
+
+    def end(t_expr: str) -> None:
+        a(f"EMH_LAND({t_expr})" if sp else "EMH_BARRIER();")
+
+    def requests_now(t_expr: str) -> None:
+        if sp:
+            a(f"{{ EMH_SUB_BASES(v, ({t_expr}) + RING - 2, vbase, V_SS, V_RING) EMH_SUB_BASES(k, ({t_expr}) + RING, kbase, K_SS, 0)")
+            for r in _request_statements(per_s):
+                a("  " + r)
+            a("}")
+
+    a("// ---- consumers: 32 query rows x the key blocks of one key-split group each")
+    if sp:
+        a("EMH_PROLOGUE_REQUESTS()")
+        a("EMH_LAND(-1)    // P: the Q tile and the first sub-steps of K have landed")
+    else:
+        a("EMH_BARRIER();  // P: the Q tile and the first sub-steps of K have landed")
     a("FRAG qf[D / 16];")
     a("{ const int qr_ = wq * 32 + lq;")
     a("  _Pragma(\"unroll\") for (int kk = 0; kk < D / 16; ++kk) qf[kk] = *(const FRAG*)(lds + Q_OFF_LDS + qr_ * (D * 2) + emh_kswz(qr_, kk * 2 + lh) * 16); }")
@@ -282,21 +318,21 @@ def _consumer(a: _Lines, D: int, ring: int) -> None:
     a("int t = 0;")
     a.open("if (nact >= 2)")
     a("// sub-block 0: softmax, and the scores of sub-block 1; no probabilities to multiply yet")
-    _iteration(a, D, par=1, has_pv=False, kslot=1 % ring, vslot=None)
-    a("EMH_BARRIER();")
+    _iteration(a, D, par=1, has_pv=False, kslot=1 % ring, vslot=None, t_expr="0" if sp else None, per_s=per_s)
+    end("0")
     a("t = 1;")
-    a(f"#pragma unroll 1")
+    a("#pragma unroll 1")
     a.open(f"for (; t + {L} < nact; t += {L})")
     for i in range(L):
-        _iteration(a, D, par=i & 1, has_pv=True, kslot=(i + 2) % ring, vslot=i % ring)
-        a("EMH_BARRIER();")
+        _iteration(a, D, par=i & 1, has_pv=True, kslot=(i + 2) % ring, vslot=i % ring, t_expr=f"t + {i}" if sp else None, per_s=per_s)
+        end(f"t + {i}")
     a.close()
     a("#pragma unroll 1")
     a.open("for (; t + 1 < nact; ++t)")
     a("const int kso = ((t + 1) % RING) * SLOT, vso = ((t + RING - 1) % RING) * SLOT;")
-    _iteration(a, D, par=0, has_pv=True, kslot="kso", vslot="vso")
+    _iteration(a, D, par=0, has_pv=True, kslot="kso", vslot="vso", t_expr="t" if sp else None, per_s=per_s)
     a("sc0 = sc1; pq1[0] = pq0[0]; pq1[1] = pq0[1];")
-    a("EMH_BARRIER();")
+    end("t")
     a.close()
     a.close(" else { sc0 = sc1; }")
     a("EMH_PHASE_AT(1)")
@@ -305,6 +341,7 @@ def _consumer(a: _Lines, D: int, ring: int) -> None:
     a("// slots; the output MFMAs of the sub-block before it, the masked softmax, and after the barrier its own output MFMAs.")
     a("const int k0t = t * SUBK + grp * 32;")
     a("const int vso_prev = ((t + RING - 1) % RING) * SLOT, vso = (t % RING) * SLOT;")
+    requests_now("t")
     a("if (resc) {  // left by the vote of the last steady iteration")
     for line in _RESCALE_IN_PLACE.split("\n"):
         a("  " + line)
@@ -320,13 +357,17 @@ def _consumer(a: _Lines, D: int, ring: int) -> None:
     a("float psum;")
     _classic_softmax(a, D, "sc0", "pq1", masked=True)
     a.close()
-    a("EMH_BARRIER();  // V(t) has landed")
+    end("t")  # V(t) has landed
     for j, (s, dt) in enumerate(jobs):
         _v_reads(a, f"vq{j}_", D, s, dt, "vso")
     for j, (s, dt) in enumerate(jobs):
         _v_mfma(a, f"vq{j}_", dt, f"pq1[{s}]")
     a.close()
-    a("for (int i_ = nact; i_ < nsub; ++i_) EMH_BARRIER();  // sub-steps the causal mask leaves this wave out of")
+    a("// sub-steps the causal mask leaves this wave out of")
+    a.open("for (int i_ = nact; i_ < nsub; ++i_)")
+    requests_now("i_")
+    end("i_")
+    a.close()
 
 
 _HEAD = r"""
@@ -345,14 +386,14 @@ typedef short emh_s16x4 __attribute__((ext_vector_type(4)));
 #define SLOT (KVS * KBYTES)            /* one ring slot: a sub-step, the 32-key blocks of all key-split groups */
 #define SUBK (KVS * 32)                /* keys per sub-step */
 #define V_RING (RING * SLOT)           /* LDS: [K ring][V ring][Q tile] */
-#define NC 256                         /* consumer threads (waves 0-3); the stagers are waves 4-7 */
+#define ST (SP ? NT : 256)             /* staging threads: every wave (SP), or waves 4-7 beside the consumer waves 0-3 */
 #define QCHUNKS (BQ * CPR)             /* 16-byte chunks of a workgroup's Q (and O) tile */
 #define RPL (D / 32 * 16)              /* output registers per lane */
 #define RPG (RPL / KVS)                /* ... of which each key-split group finishes this many */
 #define OSW (D / 4 < 32 ? D / 4 : 32)  /* rows over which the O tile's 8-byte slots are XOR-swizzled */
 #define OACC(f) oacc[(f) / 16][(f) % 16]
 #define CHUNKS (32 * D / 8)            /* 16-byte chunks of one 32-key block */
-#define PER_S (KVS * CHUNKS / NC)      /* requests per stager thread, per operand and sub-step */
+#define PER_S (KVS * CHUNKS / ST)      /* requests per staging thread, per operand and sub-step */
 #ifndef EMH_ABLATE
 #define EMH_ABLATE 0  /* -DEMH_ABLATE=1|2 through EMMY_HIPRTC_FLAGS: timing experiments whose results are not attention */
 #endif
@@ -369,8 +410,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
-  const bool consumer = wave < 4;
-  const int grp = (wave % 4) / WQ, wq = (wave % 4) % WQ;  // consumers: key-split group, row group
+  const bool consumer = SP || wave < 4;
+  const int grp = (wave % (WQ * KVS)) / WQ, wq = (wave % (WQ * KVS)) % WQ;  // consumers: key-split group, row group
   const int lq = lane % 32, lh = lane / 32;
   const f32x16 emh_zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
   // Workgroup ids go round-robin over the XCDs, each with its own L2: consecutive logical ids (the query
@@ -394,6 +435,59 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   const unsigned char* kb[D / 16];
   #pragma unroll
   for (int kk = 0; kk < D / 16; ++kk) kb[kk] = lds + grp * KBYTES + lq * (D * 2) + emh_kswz(lq, kk * 2 + lh) * 16;
+  // ---- staging.  A sub-step's K (or V) chunks are dealt over the ST staging threads; every wave-level load fills 64
+  // consecutive 16-byte LDS slots, so the swizzle is applied by choosing which global chunk each lane fetches.  A request
+  // is a scalar base (the operand plane moved along the keys to the sub-step, plus the request's row offset: whole
+  // multiples of 16 rows, which leave the swizzle of a lane's chunk unchanged), one loop-invariant 32-bit lane offset per
+  // operand and a scalar LDS target; only a sub-step that hangs over the end of the keys clamps its rows per lane.
+  const int stid = SP ? tid : tid - 256, sw = SP ? wave : wave - 4;
+  const int st_row = stid / CPR, st_pos = stid % CPR;
+  const unsigned kvo0 = (unsigned)(st_row * K_SS + emh_kswz(st_row, st_pos) * 8) * 2u;
+  const unsigned vvo0 = (unsigned)(st_row * V_SS + emh_vswz(st_row, st_pos) * 8) * 2u;
+  #define EMH_SUB_BASES(tag, s_, base_, stride_, ring0_) \
+    const int sub_##tag = (s_); \
+    const bool ok_##tag = sub_##tag >= 0 && sub_##tag < nsub; \
+    const bool whole_##tag = SKV % SUBK == 0 || (sub_##tag + 1) * SUBK <= SKV; \
+    const unsigned char* sb_##tag = emh_uniform((const unsigned char*)(base_) + (long)sub_##tag * SUBK * (stride_) * 2); \
+    const unsigned lb_##tag = emh_uniform(lds0 + (ring0_) + ((sub_##tag + RING) % RING) * SLOT + sw * 1024);
+  #define EMH_REQ_I(tag, i, voff_, base_, stride_, swz_, ring0_) { \
+    const int g_ = ((i) * ST) / CHUNKS, ro_ = (((i) * ST) % CHUNKS) / CPR; \
+    if (ok_##tag) { \
+      if (whole_##tag) { \
+        emh_dma16s(sb_##tag + (long)(g_ * 32 + ro_) * (stride_) * 2, voff_, lb_##tag + g_ * KBYTES + (((i) * ST) % CHUNKS) * 16); \
+      } else { \
+        long krow_ = (long)sub_##tag * SUBK + g_ * 32 + ro_ + st_row; \
+        if (krow_ > SKV - 1) krow_ = SKV - 1; \
+        emh_dma16((base_) + krow_ * (stride_) + swz_(st_row + ro_, st_pos) * 8, lds + (ring0_) + (sub_##tag % RING) * SLOT + g_ * KBYTES + (((i) * ST) % CHUNKS) * 16 + sw * 1024); } } }
+  // Requests retire in issue order.  In "iteration" tau (the prologue is iterations -RING .. -1) a staging thread issues
+  // V(tau + RING - 2) and then K(tau + RING), where they exist.  The barrier that ends iteration t_ needs K(t_ + 2) and
+  // V(t_): everything issued up to iteration t_ + 2 - RING.  What may still be outstanding is what iterations
+  // t_ + 3 - RING .. t_ issued.  Reaching the count does not yet make direct-to-LDS data visible to other waves: an LDS
+  // read of this wave queues behind its own writes, so waiting for it orders them before the barrier.
+  #define EMH_LAND(t_) { \
+    int cnt_ = 0; \
+    _Pragma("unroll") for (int d_ = 0; d_ < RING - 2; ++d_) { \
+      const int tau_ = (t_) - d_; \
+      cnt_ += (tau_ + RING - 2 >= 0 && tau_ + RING - 2 < nsub) + (tau_ + RING < nsub); } \
+    switch (cnt_) { \
+      case 0: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(0)); break; \
+      case 1: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(PER_S)); break; \
+      case 2: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(2 * PER_S)); break; \
+      case 3: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(3 * PER_S)); break; \
+      default: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(4 * PER_S)); break; } \
+    emh_lds_publish(lds + tid * 4); \
+    EMH_BARRIER(); }
+  // the Q tile (whole rows per instruction, swizzled like a K block) and the sub-steps that fill the rings before the loop
+  #define EMH_PROLOGUE_REQUESTS() { \
+    _Pragma("unroll") for (int c0 = 0; c0 < QCHUNKS; c0 += ST) { \
+      if (QCHUNKS % ST == 0 || c0 + (stid - lane) < QCHUNKS) {  /* whole waves: QCHUNKS is a multiple of 64 */ \
+        const int r_ = (c0 + stid) / CPR, p_ = (c0 + stid) % CPR; \
+        const int qr_ = q0 + r_ < SQ ? q0 + r_ : SQ - 1; \
+        emh_dma16(qbase + (long)qr_ * Q_SS + emh_kswz(r_, p_) * 8, lds + Q_OFF_LDS + (c0 + stid - lane) * 16); } } \
+    _Pragma("unroll") for (int tau = -RING; tau < 0; ++tau) { \
+      EMH_SUB_BASES(v, tau + RING - 2, vbase, V_SS, V_RING) EMH_SUB_BASES(k, tau + RING, kbase, K_SS, 0) \
+      _Pragma("unroll") for (int i = 0; i < PER_S; ++i) EMH_REQ_I(v, i, vvo0, vbase, V_SS, emh_vswz, V_RING) \
+      _Pragma("unroll") for (int i = 0; i < PER_S; ++i) EMH_REQ_I(k, i, kvo0, kbase, K_SS, emh_kswz, 0) } }
   unsigned st_acc[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
   unsigned long long st_last = EMH_STAMP ? __builtin_readcyclecounter() : 0ull;
   #pragma unroll 1
@@ -433,72 +527,18 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
 _STAGER = r"""
     __builtin_amdgcn_s_setprio(0);
   } else {
-    // ---- stagers: every direct-to-LDS request of the workgroup.  A sub-step's K (or V) chunks are dealt over the
-    // 256 stager threads; every wave-level load fills 64 consecutive 16-byte LDS slots, so the swizzle is applied
-    // by choosing which global chunk each lane fetches.
-    const int stid = tid - NC, sw = wave - 4;
-    const int st_row = stid / CPR, st_pos = stid % CPR;
-    unsigned kvo[PER_S], vvo[PER_S];
-    #pragma unroll
-    for (int i = 0; i < PER_S; ++i) {
-      const int g_ = (i * NC) / CHUNKS, ro_ = ((i * NC) % CHUNKS) / CPR;
-      kvo[i] = (unsigned)((g_ * 32 + ro_ + st_row) * K_SS + emh_kswz(st_row + ro_, st_pos) * 8) * 2u;
-      vvo[i] = (unsigned)((g_ * 32 + ro_ + st_row) * V_SS + emh_vswz(st_row + ro_, st_pos) * 8) * 2u;
-    }
-    // Requests of sub-step s_: the operand plane moved along the keys in scalar registers, a loop-invariant 32-bit
-    // lane offset and a scalar LDS target; only a sub-step that hangs over the end of the keys clamps rows per lane.
-    #define EMH_REQ(s_, base_, stride_, off_, swz_, ring0_) { \
-      const int sub_ = (s_); \
-      const unsigned char* sb_ = emh_uniform((const unsigned char*)(base_) + (long)sub_ * SUBK * (stride_) * 2); \
-      const unsigned lb_ = emh_uniform(lds0 + (ring0_) + (sub_ % RING) * SLOT + sw * 1024); \
-      _Pragma("unroll") for (int i = 0; i < PER_S; ++i) { \
-        const int g_ = (i * NC) / CHUNKS, ro_ = ((i * NC) % CHUNKS) / CPR; \
-        if (SKV % SUBK == 0 || (sub_ + 1) * SUBK <= SKV) { \
-          emh_dma16s(sb_, off_[i], lb_ + g_ * KBYTES + ((i * NC) % CHUNKS) * 16); \
-        } else { \
-          long krow_ = (long)sub_ * SUBK + g_ * 32 + ro_ + st_row; \
-          if (krow_ > SKV - 1) krow_ = SKV - 1; \
-          emh_dma16((base_) + krow_ * (stride_) + swz_(st_row + ro_, st_pos) * 8, lds + (ring0_) + (sub_ % RING) * SLOT + g_ * KBYTES + ((i * NC) % CHUNKS) * 16 + sw * 1024); } } }
-    #define EMH_REQ_K(s_) EMH_REQ(s_, kbase, K_SS, kvo, emh_kswz, 0)
-    #define EMH_REQ_V(s_) EMH_REQ(s_, vbase, V_SS, vvo, emh_vswz, V_RING)
-    // Requests retire in issue order.  In "iteration" tau (the prologue is iterations -RING .. -1) a stager issues
-    // V(tau + RING - 2) and then K(tau + RING), where they exist.  The barrier that ends iteration t_ needs K(t_ + 2)
-    // and V(t_): everything issued up to iteration t_ + 2 - RING.  What may still be outstanding is what iterations
-    // t_ + 3 - RING .. t_ issued.
-    #define EMH_LAND(t_) { \
-      int cnt_ = 0; \
-      _Pragma("unroll") for (int d_ = 0; d_ < RING - 2; ++d_) { \
-        const int tau_ = (t_) - d_; \
-        cnt_ += (tau_ + RING - 2 >= 0 && tau_ + RING - 2 < nsub) + (tau_ + RING < nsub); } \
-      switch (cnt_) { \
-        case 0: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(0)); break; \
-        case 1: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(PER_S)); break; \
-        case 2: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(2 * PER_S)); break; \
-        case 3: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(3 * PER_S)); break; \
-        default: __builtin_amdgcn_s_waitcnt(EMH_WAIT_VM(4 * PER_S)); break; } \
-      emh_lds_publish(lds + tid * 4); \
-      EMH_BARRIER(); }
-    // the Q tile: whole rows per instruction, swizzled like a K block
-    #pragma unroll
-    for (int c0 = 0; c0 < QCHUNKS; c0 += NC) {
-      if (QCHUNKS % NC == 0 || c0 + (stid - lane) < QCHUNKS) {  // whole waves: QCHUNKS is a multiple of 64
-        const int r_ = (c0 + stid) / CPR, p_ = (c0 + stid) % CPR;
-        const int qr_ = q0 + r_ < SQ ? q0 + r_ : SQ - 1;
-        emh_dma16(qbase + (long)qr_ * Q_SS + emh_kswz(r_, p_) * 8, lds + Q_OFF_LDS + (c0 + stid - lane) * 16);
-      }
-    }
-    #pragma unroll
-    for (int tau = -RING; tau < 0; ++tau) {
-      if (tau + RING - 2 >= 0 && tau + RING - 2 < nsub) EMH_REQ_V(tau + RING - 2)
-      if (tau + RING < nsub) EMH_REQ_K(tau + RING)
-    }
+    // ---- stagers: every direct-to-LDS request of the workgroup
+    EMH_PROLOGUE_REQUESTS()
     EMH_LAND(-1)     // P
     EMH_BARRIER();   // B0
     #pragma unroll 1
     for (int t = 0; t < nsub; ++t) {
       if (EMH_ABLATE != 1) {  // (1, measurement only: no requests inside the loop, the consumers work on what the prologue left)
-        if (t + RING - 2 < nsub) EMH_REQ_V(t + RING - 2)
-        if (t + RING < nsub) EMH_REQ_K(t + RING)
+        EMH_SUB_BASES(v, t + RING - 2, vbase, V_SS, V_RING) EMH_SUB_BASES(k, t + RING, kbase, K_SS, 0)
+        #pragma unroll
+        for (int i = 0; i < PER_S; ++i) EMH_REQ_I(v, i, vvo0, vbase, V_SS, emh_vswz, V_RING)
+        #pragma unroll
+        for (int i = 0; i < PER_S; ++i) EMH_REQ_I(k, i, kvo0, kbase, K_SS, emh_kswz, 0)
       }
       EMH_LAND(t)
     }
@@ -618,8 +658,16 @@ _STAGER = r"""
 """
 
 
+def _shape(body: Flash) -> tuple[bool, int, tuple[int, ...]]:
+    """``(self-staging, consumer waves, ring depths to try)`` of the form ``body`` asks for."""
+    sp = bool(getattr(body, "sp", False))
+    return sp, (8 if sp else CONSUMER_WAVES), ((4, 3, 2) if sp else (4, 3))
+
+
 def ws_supported(body: Flash, ctx: Context = Context()) -> str | None:
-    """``None`` when the wave-specialised form can take ``body`` with its current ``waves`` / ``kv_split``; else why not."""
+    """``None`` when the software-pipelined forms (``ws``: four consumer waves and four staging waves; ``sp``: eight
+    consumer waves that stage for themselves) can take ``body`` with its current ``waves`` / ``kv_split``; else why not."""
+    sp, consumers, rings = _shape(body)
     if body.dtype.name not in ("bf16", "f16"):
         return "16-bit operands only"
     if body.head_dim not in (64, 128):
@@ -628,14 +676,14 @@ def ws_supported(body: Flash, ctx: Context = Context()) -> str | None:
         return "no mask operand"
     if getattr(body, "sym", None) is not None and body.sym.fields:
         return "lengths known when the kernel is built"
-    if body.waves * body.kv_split != CONSUMER_WAVES:
-        return f"row groups x key-split groups must be {CONSUMER_WAVES} (one consumer wave per SIMD)"
+    if body.waves * body.kv_split != consumers:
+        return f"row groups x key-split groups must be {consumers} ({'two consumer waves' if sp else 'one consumer wave'} per SIMD)"
     if (body.head_dim // 32 * 16) % (4 * body.kv_split):
         return "the key-split groups cannot share a lane's output registers"
-    if (body.kv_split * 32 * body.head_dim // 8) % 256:
-        return "a sub-step's chunks must be a multiple of the 256 stager threads"
+    if (body.kv_split * 32 * body.head_dim // 8) % (512 if sp else 256):
+        return "a sub-step's chunks must be a multiple of the staging threads"
     try:
-        ws_lds_plan(body.waves, body.kv_split, body.head_dim, ctx.lds_bytes_per_cu)
+        ws_lds_plan(body.waves, body.kv_split, body.head_dim, ctx.lds_bytes_per_cu, rings)
     except LoweringError as exc:
         return str(exc)
     return None
@@ -644,14 +692,15 @@ def ws_supported(body: Flash, ctx: Context = Context()) -> str | None:
 def emit_flash_ws(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     why = ws_supported(body, ctx)
     if why is not None:
-        raise LoweringError(f"flash/ws: {why}")
+        raise LoweringError(f"flash/{'sp' if getattr(body, 'sp', False) else 'ws'}: {why}")
+    sp, consumers, rings = _shape(body)
     D = body.head_dim
     if body.q_heads % body.kv_heads:
         raise LoweringError("flash: q heads must be a multiple of kv heads")
     waves, kvs = body.waves, body.kv_split
     BQ = 32 * waves
-    NT = 64 * (CONSUMER_WAVES + STAGER_WAVES)
-    plan = ws_lds_plan(waves, kvs, D, ctx.lds_bytes_per_cu)
+    NT = 64 * (consumers if sp else CONSUMER_WAVES + STAGER_WAVES)
+    plan = ws_lds_plan(waves, kvs, D, ctx.lds_bytes_per_cu, rings)
     for st, heads in ((body.q_strides, body.q_heads), (body.k_strides, body.kv_heads), (body.v_strides, body.kv_heads), (body.o_strides, body.q_heads)):
         if st[2] % 8 or (heads > 1 and st[1] % 8) or (body.batch > 1 and st[0] % 8):
             raise LoweringError("flash: batch / head / sequence strides must keep 16-byte alignment")
@@ -664,8 +713,9 @@ def emit_flash_ws(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     qslots = qblocks // 2 if pair else qblocks
     bf16 = body.dtype.name == "bf16"
     grid = qslots * body.q_heads * body.batch
+    per_s = kvs * (32 * D // 8) // NT if sp else 0
     defs = {
-        "KNAME": name, "NT": NT, "D": D, "BQ": BQ, "KVS": kvs, "WQ": waves, "RING": plan["ring"],
+        "KNAME": name, "NT": NT, "SP": 1 if sp else 0, "D": D, "BQ": BQ, "KVS": kvs, "WQ": waves, "RING": plan["ring"],
         "CPR": D // 8, "KRPL": max(1, 16 // (D // 8)), "TG": min(4, D // 32),
         "SQ": body.q_len, "SKV": body.kv_len, "HQ": body.q_heads, "GROUP": body.q_heads // body.kv_heads,
         "QBLOCKS": qblocks, "QSLOTS": qslots, "PAIR": 1 if pair else 0, "CAUSAL": 1 if body.causal else 0,
@@ -680,14 +730,15 @@ def emit_flash_ws(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "MFMA": "__builtin_amdgcn_mfma_f32_32x32x16_bf16" if bf16 else "__builtin_amdgcn_mfma_f32_32x32x16_f16",
         "EXP2(x)": f"(EMH_ABLATE == 3 ? (x) : {rt.intrinsic('fast_exp2', 'f32')}(x))",
         "RESCALE_SLACK": "8.0f",
-        "CONSUMER_PRIO": 1,
+        "CONSUMER_PRIO": 0 if sp else 1,
         "GRID": grid, "XCDS": ctx.xcds,
     }  # fmt: skip
-    head = f"// {name}: B={body.batch} Hq={body.q_heads} Hkv={body.kv_heads} Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} (wave-specialised)\n"
+    form = "self-staging, software-pipelined" if sp else "wave-specialised"
+    head = f"// {name}: B={body.batch} Hq={body.q_heads} Hkv={body.kv_heads} Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} ({form})\n"
     head += "".join(f"#define {k} {v}\n" for k, v in defs.items())
     lines = _Lines()
     lines.depth = 2
-    _consumer(lines, D, plan["ring"])
+    _consumer(lines, D, plan["ring"], per_s)
     source = prelude.header(prelude.DMA) + head + _HEAD + "\n".join(lines.out) + _STAGER
     return HipOp(
         kernel_source=source,
@@ -696,10 +747,10 @@ def emit_flash_ws(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         grid=((grid,), (1,), (1,)),
         block=((NT,), (1,), (1,)),
         lds_bytes=plan["bytes"],
-        comment=f"flash/ws Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} split={kvs} pair={int(pair)} ring={plan['ring']}",
+        comment=f"flash/{'sp' if sp else 'ws'} Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} split={kvs} pair={int(pair)} ring={plan['ring']}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
-        knobs={"FLASH": f"w{waves}/kv32/s{kvs}" + ("/p" if pair else "") + "/ws"},
+        knobs={"FLASH": f"w{waves}/kv32/s{kvs}" + ("/p" if pair else "") + ("/sp" if sp else "/ws")},
     )
 
 

@@ -280,6 +280,7 @@ class Flash:
     deep: bool = False  # a K ring of three slots (K blocks requested two steps ahead) beside a V ring of two
     pair_steps: bool = True  # key steps unrolled in pairs so ring slots are compile-time (the lowering clears it if that build spills)
     ws: bool = False  # wave-specialised form: four consumer waves (waves x kv_split = 4) and four staging waves
+    sp: bool = False  # software-pipelined form without staging waves: eight consumer waves (waves x kv_split = 8) stage for themselves
     # an additive bias on the scaled scores, ``[batch, head, query, key]`` addressed through (batch, head, query)
     # strides (0 = broadcast) with keys contiguous; ``None``: no mask operand
     mask: str | None = None

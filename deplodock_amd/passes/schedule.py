@@ -523,12 +523,14 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
     pinned = _pin("FLASH", _tuned(body, ctx))
     if pinned:
         try:
-            body.pair = body.deep = body.ws = False
+            body.pair = body.deep = body.ws = body.sp = False
             for tok in pinned.split("/"):
                 if tok == "p":
                     body.pair = True
                 elif tok == "ws":
                     body.ws = True
+                elif tok == "sp":
+                    body.sp = True
                 elif tok == "k3":
                     body.deep = True
                 elif tok.startswith("w"):
@@ -539,17 +541,19 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                     body.kv_split = int(tok[1:])
                 else:
                     raise ScheduleError(f"cannot parse {tok!r} (expect w<groups> / kv<keys> / s<split> / p / k3)")
-            if body.ws:
+            if body.ws and body.sp:
+                raise ScheduleError("ws and sp are two forms: pin one")
+            if body.ws or body.sp:
                 from deplodock_amd.emit.flash_ws import ws_supported
 
                 body.block_kv = 32
                 why = ws_supported(body, ctx)
                 if why is not None:
-                    raise ScheduleError(f"the wave-specialised form needs {why}")
+                    raise ScheduleError(f"the software-pipelined forms need {why}")
             chunks = body.block_kv * body.head_dim // 8
-            if body.waves < 1 or body.kv_split < 1 or body.block_kv % 32 or chunks % (body.waves * body.kv_split * 64):
+            if body.waves < 1 or body.kv_split < 1 or body.block_kv % 32 or (not (body.ws or body.sp) and chunks % (body.waves * body.kv_split * 64)):
                 raise ScheduleError("unrealisable workgroup shape")
-            if not body.ws and _flash_lds(body, ctx) > ctx.lds_bytes_per_cu:
+            if not (body.ws or body.sp) and _flash_lds(body, ctx) > ctx.lds_bytes_per_cu:
                 raise ScheduleError("the double-buffered K/V blocks of all key-split groups exceed the LDS")
             if (body.head_dim // 32 * 16) % (4 * body.kv_split):
                 raise ScheduleError("the key-split groups cannot share a lane's output registers")
@@ -565,7 +569,7 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
         def blocks(w: int) -> int:
             return -(-body.q_len // (32 * w))
 
-        body.pair = body.deep = body.ws = False
+        body.pair = body.deep = body.ws = body.sp = False
         body.waves = 0
         if body.head_dim <= 128 and body.kv_len >= 2048:
             # Enough rows to give every CU a 256-row workgroup: eight query waves share each
@@ -609,7 +613,7 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 body.kv_split //= 2
     if getattr(body, "sym", None) is not None and body.sym.fields:
         body.pair = False  # pairing mirrored query blocks needs the block count when the kernel is built
-    return {"FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "") + ("/k3" if body.deep else "") + ("/ws" if body.ws else "")}
+    return {"FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "") + ("/k3" if body.deep else "") + ("/ws" if body.ws else "") + ("/sp" if body.sp else "")}
 
 
 def schedule(graph: Graph, ctx: Context | None = None) -> Graph:

@@ -1,5 +1,6 @@
-"""The wave-specialised attention kernel (``FLASH=.../ws``): its ring protocol replayed on the CPU, and parity
-on the GPU through the C-ABI for every shape of the form (row groups x key-split groups, mirrored pairs, ragged
+"""The software-pipelined attention kernels (``FLASH=.../ws``: four consumer waves and four staging waves;
+``.../sp``: eight consumer waves that stage for themselves): their ring protocol replayed on the CPU, and parity
+on the GPU through the C-ABI for every shape of the forms (row groups x key-split groups, mirrored pairs, ragged
 and unmasked lengths, head_dim 64, the full benchmark size)."""
 
 from __future__ import annotations
@@ -85,7 +86,7 @@ def _replay(ring: int, nsub: int, nacts: list[int], *, k_ahead: int | None = Non
                 assert start_of(tau) >= hi, f"{o}({s2}) is requested in iteration {tau} into the slot {o}({sub}) is still read from (until barrier {hi})"
 
 
-@pytest.mark.parametrize("ring", [3, 4])
+@pytest.mark.parametrize("ring", [2, 3, 4])
 def test_ring_protocol_never_overwrites_a_live_slot_and_never_reads_before_landing(ring):
     for nsub in range(1, 14):
         for nact in range(0, nsub + 1):
@@ -105,8 +106,10 @@ def test_replay_trips_on_schedules_that_are_wrong(mutant):
 def test_emitted_text_spells_the_replayed_schedule(launcher_lib):
     op = emit_flash_ws(_body(pair=True), "k_ws")
     src = op.kernel_source
-    assert "if (t + RING - 2 < nsub) EMH_REQ_V(t + RING - 2)" in src and "if (t + RING < nsub) EMH_REQ_K(t + RING)" in src
-    assert "for (int tau = -RING; tau < 0; ++tau)" in src and "const int tau_ = (t_) - d_;" in src and "d_ < RING - 2" in src
+    assert "EMH_SUB_BASES(v, t + RING - 2, vbase, V_SS, V_RING) EMH_SUB_BASES(k, t + RING, kbase, K_SS, 0)" in src  # what iteration t requests
+    assert "EMH_SUB_BASES(v, tau + RING - 2, vbase, V_SS, V_RING) EMH_SUB_BASES(k, tau + RING, kbase, K_SS, 0)" in src and "for (int tau = -RING; tau < 0; ++tau)" in src
+    assert "const bool ok_##tag = sub_##tag >= 0 && sub_##tag < nsub;" in src and "((sub_##tag + RING) % RING) * SLOT" in src  # existence, slot
+    assert "const int tau_ = (t_) - d_;" in src and "d_ < RING - 2" in src  # what a landing wait leaves outstanding
     assert src.count("EMH_BARRIER();") >= 8 and "#define RING 4" in src
     assert op.block[0] == (512,) and op.knobs["FLASH"] == "w2/kv32/s2/p/ws" and op.lds_bytes == 2 * 4 * 16384 + 16384
     from deplodock_amd.backend.hip import hiprtc
@@ -120,6 +123,25 @@ def test_what_the_form_takes_and_what_it_refuses():
     assert "head_dim" in ws_supported(_body(d=256))
     assert "LDS" in ws_supported(_body(waves=1, kvs=4))  # 32 KiB sub-steps: a ring of three per operand does not fit
     assert ws_lds_plan(2, 2, 128, 160 * 1024)["ring"] == 4 and ws_lds_plan(4, 1, 128, 160 * 1024)["ring"] == 4
+    # the self-staging form: eight consumer waves; 32 KiB sub-steps leave room for rings of two
+    sp = _body(waves=2, kvs=4)
+    sp.ws, sp.sp = False, True
+    assert ws_supported(sp) is None and ws_lds_plan(2, 4, 128, 160 * 1024, (4, 3, 2))["ring"] == 2
+    bad = _body(waves=2, kvs=2)
+    bad.ws, bad.sp = False, True
+    assert "must be 8" in ws_supported(bad)
+
+
+def test_self_staging_form_builds_without_spills_and_carries_its_requests_in_the_slices(launcher_lib):
+    from deplodock_amd.backend.hip import hiprtc
+
+    body = _body(waves=2, kvs=4, pair=True)
+    body.ws, body.sp = False, True
+    op = emit_flash_ws(body, "k_sp")
+    src = op.kernel_source
+    assert op.knobs["FLASH"] == "w2/kv32/s4/p/sp" and op.block[0] == (512,) and "#define SP 1" in src and "#define RING 2" in src
+    assert src.count("EMH_REQ_I(v, 0, vvo0") >= 4 and "EMH_LAND(t + 1)" in src and "EMH_PROLOGUE_REQUESTS()" in src
+    assert hiprtc.spilled_vgprs(src, "k_sp") == 0
 
 
 def test_pin_grammar_reaches_the_emitter(launcher_lib, monkeypatch):
@@ -144,6 +166,12 @@ CASES = [
     ("one key", dict(b=1, hq=2, hkv=2, s=1, d=128, seed=5), ["w2/kv32/s2/ws"]),
     ("unmasked ragged", dict(b=1, hq=4, hkv=2, s=333, d=128, seed=5, causal=False), ["w2/kv32/s2/ws", "w4/kv32/s1/ws"]),
     ("head_dim 64", dict(b=1, hq=8, hkv=2, s=512, d=64, seed=15), ["w2/kv32/s2/ws", "w4/kv32/s1/ws", "w1/kv32/s4/ws"]),
+    ("small causal", dict(b=1, hq=8, hkv=4, s=320, d=128, seed=9), ["w2/kv32/s4/sp", "w4/kv32/s2/sp", "w8/kv32/s1/sp"]),
+    ("pairs", dict(b=2, hq=4, hkv=2, s=512, d=128, seed=11), ["w2/kv32/s4/p/sp", "w4/kv32/s2/p/sp"]),
+    ("ragged causal", dict(b=1, hq=4, hkv=2, s=300, d=128, seed=3), ["w2/kv32/s4/sp", "w4/kv32/s2/sp"]),
+    ("shorter than a sub-step", dict(b=1, hq=2, hkv=1, s=40, d=128, seed=4), ["w2/kv32/s4/sp", "w8/kv32/s1/sp"]),
+    ("unmasked ragged", dict(b=1, hq=4, hkv=2, s=333, d=128, seed=5, causal=False), ["w2/kv32/s4/sp", "w4/kv32/s2/sp"]),
+    ("head_dim 64", dict(b=1, hq=8, hkv=2, s=512, d=64, seed=15), ["w4/kv32/s2/sp", "w2/kv32/s4/sp"]),
 ]
 
 
@@ -169,7 +197,7 @@ def test_ws_matches_eager_on_every_shape_of_the_form(device, label, kw, pin, mon
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("pin", ["w2/kv32/s2/p/ws", "w4/kv32/s1/ws"])
+@pytest.mark.parametrize("pin", ["w2/kv32/s2/p/ws", "w4/kv32/s1/ws", "w2/kv32/s4/p/sp"])
 def test_ws_full_size_rows_and_position_coded_values(device, pin, monkeypatch):
     """The benchmark shape with the scale-aware criteria of the default kernel's test: per-row relative error against
     an fp32 run bounded by 1.5 x 16-bit eager's, rows summing to one, and position-coded values (a skipped or
@@ -207,11 +235,12 @@ def test_ws_full_size_rows_and_position_coded_values(device, pin, monkeypatch):
 
 
 @pytest.mark.gpu
-def test_ws_large_score_jumps_raise_the_reference_maximum(device, monkeypatch):
+@pytest.mark.parametrize("pin", ["w2/kv32/s2/ws", "w2/kv32/s4/sp"])
+def test_ws_large_score_jumps_raise_the_reference_maximum(device, pin, monkeypatch):
     """Keys whose scores grow along the sequence (every sub-block outgrows the reference maximum of the one before by
     more than the slack) exercise the vote, the deferred rescale of the output accumulators and the merge of the
     key-split groups' statistics."""
-    monkeypatch.setenv("EMMY_FLASH", "w2/kv32/s2/ws")
+    monkeypatch.setenv("EMMY_FLASH", pin)
     torch.manual_seed(31)
     s, d = 384, 128
     q = torch.randn(1, 4, s, d)
@@ -235,10 +264,11 @@ def test_ws_large_score_jumps_raise_the_reference_maximum(device, monkeypatch):
 
 
 @pytest.mark.gpu
-def test_ws_soak_is_bit_stable(device, monkeypatch):
+@pytest.mark.parametrize("pin", ["w2/kv32/s2/p/ws", "w2/kv32/s4/p/sp"])
+def test_ws_soak_is_bit_stable(device, pin, monkeypatch):
     """2000 launches on fixed inputs reproduce the first bit for bit (the publication fence of the stagers' requests,
     the barrier protocol of the rings), and that result matches eager."""
-    monkeypatch.setenv("EMMY_FLASH", "w2/kv32/s2/p/ws")
+    monkeypatch.setenv("EMMY_FLASH", pin)
     case = eager.sdpa_case(b=1, hq=16, hkv=8, s=1024, d=128, seed=22)
     be = HipBackend()
     compiled = be.compile(trace_module(case.module, case.inputs))
