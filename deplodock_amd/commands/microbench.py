@@ -13,6 +13,11 @@
   operands.  That figure, not the MFMA peak, bounds a contraction whose tile needs
   more bytes per MFMA cycle than it delivers.
 
+* ``--flash``: where the software-pipelined attention kernels (``FLASH=.../ws``, ``.../sp``) spend their clocks on the
+  benchmark shape: per-iteration and per-pass phase stamps of wave 0 of workgroup 0 (``-DEMH_STAMP=1|2``, read with
+  the shader clock), and timings with one part of the kernel taken out (``-DEMH_ABLATE``: no requests inside the loop,
+  no consumer arithmetic, no exponentials, no fragment reads), next to the default kernel's time in the same process.
+
 * ``--lds``: the rate at which the waves of a CU read 16-byte MFMA operand fragments out of
   LDS (``ds_read_b128``), for the lane-to-address patterns the emitters use — 16- and 32-row
   fragment layouts over XOR-swizzled slabs of 64, 128 and 256 bytes a row — against a
@@ -326,11 +331,78 @@ def handle_lds(args) -> None:
         print(line)
 
 
+def handle_flash(args) -> None:
+    """Stamps and ablations of the software-pipelined attention forms (the switches are compile-time defines of
+    ``emit/flash_ws.py``; an ablated kernel's output is not attention, a stamped kernel's first output words hold the
+    stamps)."""
+    import os
+
+    import torch
+
+    from deplodock_amd import HipBackend, trace_module, workloads
+    from deplodock_amd.commands.table import render_table
+
+    dev = torch.device("cuda:0")
+    case = workloads.sdpa_case(s=int(args.seq))
+    pins = [p for p in (args.pins or "w2/kv32/s2/p/ws,w2/kv32/s4/p/sp").split(",") if p]
+    saved = {k: os.environ.get(k) for k in ("EMMY_FLASH", "EMMY_HIPRTC_FLAGS")}
+
+    def build(pin, flags):
+        for key, val in (("EMMY_FLASH", pin), ("EMMY_HIPRTC_FLAGS", flags)):
+            if val:
+                os.environ[key] = val
+            else:
+                os.environ.pop(key, None)
+        be = HipBackend()
+        compiled = be.compile(trace_module(case.module, case.inputs))
+        return be, compiled, {n: t.to(dev) for n, t in zip(compiled.inputs, case.inputs)}
+
+    def time_us(pin, flags):
+        be, compiled, data = build(pin, flags)
+        res = be.benchmark(compiled, warmup=3, num_iters=30, input_data=data)
+        return res.time_ms * 1e3
+
+    def stamps(pin, mode):
+        be, compiled, data = build(pin, f"-DEMH_STAMP={mode}")
+        prog = be.program(compiled, data)
+        try:
+            for _ in range(2):
+                prog.run()
+                torch.cuda.synchronize()
+            w = prog.output_tensors()[compiled.outputs[0]].reshape(-1)[:8].view(torch.float32)
+            return [w[i].item() for i in range(4)]
+        finally:
+            prog.close()
+
+    try:
+        rows = [["default", "-", f"{time_us(None, None):.2f}", "", "", "", ""]]
+        for pin in pins:
+            rows.append([pin, "-", f"{time_us(pin, None):.2f}", "", "", "", ""])
+            for what, flag in (("no requests in the loop", 1), ("no consumer arithmetic", 2), ("no exponentials", 3), ("no fragment reads", 4)):
+                rows.append([pin, what, f"{time_us(pin, f'-DEMH_ABLATE={flag}'):.2f}", "", "", "", ""])
+            it = stamps(pin, 1)
+            rows.append([pin, "clocks per iteration (wave 0): barrier / lead / first half / second half", "", f"{it[3]:.0f}", f"{it[0]:.0f}", f"{it[1]:.0f}", f"{it[2]:.0f}"])
+            ph = stamps(pin, 2)
+            rows.append([pin, "clocks per workgroup (wave 0): prologue / loops / tail / close + store", "", f"{ph[0]:.0f}", f"{ph[1]:.0f}", f"{ph[2]:.0f}", f"{ph[3]:.0f}"])
+            print("  ".join(rows[-1]), flush=True)
+    finally:
+        for key, val in saved.items():
+            if val is None:
+                os.environ.pop(key, None)
+            else:
+                os.environ[key] = val
+    for line in render_table(["FLASH", "variant", "us", "a", "b", "c", "d"], rows, "llrrrrr"):
+        print(line)
+
+
 def register_microbench_command(subparsers) -> None:
     p = subparsers.add_parser("microbench", help="Measure the MFMA rate, MFMA/VALU co-issue and the L1 fill rate of the GPU")
     p.add_argument("--l1fill", action="store_true", help="sweep load-only kernels: bytes per clock a CU pulls through its vector L1")
     p.add_argument("--quick", action="store_true", help="with --l1fill: a four-line sweep")
     p.add_argument("--lds", action="store_true", help="fragment-read rate out of LDS for the emitters' swizzled layouts")
+    p.add_argument("--flash", action="store_true", help="phase stamps and ablations of the software-pipelined attention kernels on the benchmark shape")
+    p.add_argument("--pins", default=None, help="with --flash: comma-separated EMMY_FLASH pins (default: the ws and sp forms of the benchmark shape)")
+    p.add_argument("--seq", default="2048", help="with --flash: sequence length")
     p.set_defaults(func=handle_microbench)
 
 
@@ -345,6 +417,9 @@ def handle_microbench(args) -> None:
         return
     if getattr(args, "lds", False):
         handle_lds(args)
+        return
+    if getattr(args, "flash", False):
+        handle_flash(args)
         return
     from deplodock_amd.backend.hip import launcher
     from deplodock_amd.commands.table import render_table
