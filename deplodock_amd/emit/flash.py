@@ -76,7 +76,7 @@ typedef short emh_s16x4 __attribute__((ext_vector_type(4)));
 #define OACC(f) oacc[(f) / 16][(f) % 16]
 
 extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q, const ELT* __restrict__ Kp,
-                                                      const ELT* __restrict__ Vp MASK_PARAM, ELT* __restrict__ Op SYM_PARAM) {
+                                                      const ELT* __restrict__ Vp MASK_PARAM, OUT_T* __restrict__ Op SYM_PARAM) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // [2 buffers][group][K | V][key][d]
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int grp = wave / WQ, wq = wave % WQ;
@@ -94,8 +94,18 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   const int batch = bid / (QSLOTS * HQ);
   const int kvh = head / GROUP;
   const ELT* qbase = Q + Q_OFF + (long)batch * Q_SB + (long)head * Q_SH;
-  const ELT* kbase = Kp + K_OFF + (long)batch * K_SB + (long)kvh * K_SH;
-  const ELT* vbase = Vp + V_OFF + (long)batch * V_SB + (long)kvh * V_SH;
+#if KV_CTAS > 1
+  // Cross-workgroup key split: slice blockIdx.y of the keys, [kv0, kv0 + SKV), is this workgroup's whole key range.
+  // Key indices below are relative to the slice; the causal comparison shifts the query index instead.
+  const int kv0 = (int)blockIdx.y * KV_CHUNK;
+  const int skv_slice = SKV_ALL - kv0 < KV_CHUNK ? SKV_ALL - kv0 : KV_CHUNK;
+  #define SKV skv_slice
+  #define QSHIFT kv0
+#else
+  #define QSHIFT 0
+#endif
+  const ELT* kbase = Kp + K_OFF + (long)batch * K_SB + (long)kvh * K_SH + (long)QSHIFT * K_SS;
+  const ELT* vbase = Vp + V_OFF + (long)batch * V_SB + (long)kvh * V_SH + (long)QSHIFT * V_SS;
   #pragma unroll 1
   for (int pass = 0; pass < (PAIR ? 2 : 1); ++pass) {
   if (PAIR && pass) __syncthreads();  // every thread is done copying the first block's O tile out of LDS
@@ -103,6 +113,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   const int q0 = qb * BQ;
   const int qw0 = q0 + wq * 32;
   const int qrow = qw0 + lq;
+  const int qw0_k = qw0 - QSHIFT, qrow_k = qrow - QSHIFT;  // the same rows as positions among this workgroup's keys
 
   // A lane's Q fragments are 16-byte pieces of one row: read straight from global
   // memory a wave's load touches 32 rows per instruction.  With LDS to spare the
@@ -126,7 +137,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   }
   int ntiles = (SKV + BKV - 1) / BKV;
   if (CAUSAL) {
-    const int lim = (q0 + BQ - 1 < SQ - 1 ? q0 + BQ - 1 : SQ - 1) / BKV + 1;
+    const int last_ = (q0 + BQ - 1 < SQ - 1 ? q0 + BQ - 1 : SQ - 1) - QSHIFT;  // the last key any row of the block may see
+    const int lim = last_ < 0 ? 0 : last_ / BKV + 1;
     if (lim < ntiles) ntiles = lim;
   }
   const int nsteps = (ntiles + KVS - 1) / KVS;
@@ -253,7 +265,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
     const bool more = st + 1 < nsteps;
     const int jt = st * KVS + grp;
     const int k0 = jt * BKV;
-    const bool active = (jt < ntiles) && (!CAUSAL || (k0 <= qw0 + 31));
+    const bool active = (jt < ntiles) && (!CAUSAL || (k0 <= qw0_k + 31));
     EMH_STEP_BASES(1, st + 1)
     EMH_STEP_BASES(2, st + 2)
     (void)kb2; (void)kl2; (void)vb2; (void)vl2; (void)kb1; (void)kl1;
@@ -328,13 +340,13 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       }
 #endif
       float mx = -1.0e30f;
-      if ((CAUSAL && (k0 + BKV - 1 > qw0)) || (k0 + BKV > SKV)) {
+      if ((CAUSAL && (k0 + BKV - 1 > qw0_k)) || (k0 + BKV > SKV)) {
         #pragma unroll
         for (int u = 0; u < BKV / 32; ++u)
         #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = k0 + 32 * u + 8 * (r / 4) + 4 * lh + (r % 4);
-          if ((CAUSAL && key > qrow) || key >= SKV) sacc[u][r] = -1.0e30f;
+          if ((CAUSAL && key > qrow_k) || key >= SKV) sacc[u][r] = -1.0e30f;
           mx = fmaxf(mx, sacc[u][r]);
         }
       } else {
@@ -430,7 +442,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   #pragma unroll
   for (int g = 0; g < KVS; ++g) {
     if (g == grp) {
-      float a_own = 1.0f, l_tot = l_run;
+      float a_own = 1.0f, l_tot = l_run, m_row = m_ref;
       float a_o[KVS];
       if (KVS > 1) {
         const float* pml = (const float*)(lds + PARK_ML) + lane;
@@ -444,6 +456,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
           }
         }
         a_own = EXP2(m_ref - m_all);
+        m_row = m_all;
         l_tot = l_run * a_own;
         #pragma unroll
         for (int h = 0; h < KVS; ++h) {
@@ -456,6 +469,12 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       l_tot += emh_xor32(l_tot);
       const float inv = 1.0f / l_tot;
       const int orow = wq * 32 + lq;
+#if KV_CTAS > 1
+      // The slice's state goes to the workspace as it is: per query row D unnormalised output values (at the scale of the
+      // row's reference maximum over the slice), then that maximum (log2 units, score scale folded in) and the row sum.
+      float* prow = Op + ((((long)blockIdx.y * BATCH + batch) * HQ + head) * SQ + (q0 + orow < SQ ? q0 + orow : SQ - 1)) * (D + 4);
+      if (q0 + orow < SQ && g == 0 && lh == 0) { prow[D] = m_row; prow[D + 1] = l_tot; }
+#endif
       #pragma unroll
       for (int r4 = 0; r4 < RPG / 4; ++r4) {
         f32x4 acc;
@@ -471,16 +490,22 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
             }
           }
         }
+        // Registers 4i .. 4i+3 of tile T are d = 32*T + 8*i + 4*lh + (0..3): 8-byte slot 8*T + 2*i + lh of the row.
+        const int f = g * RPG + 4 * r4;
+#if KV_CTAS > 1
+        (void)inv;
+        if (q0 + orow < SQ) *(f32x4*)(prow + 32 * (f / 16) + 8 * ((f % 16) / 4) + 4 * lh) = acc;
+#else
         PACK4 y;
         #pragma unroll
         for (int j = 0; j < 4; ++j) y[j] = (ELT)(acc[j] * inv);
-        // Registers 4i .. 4i+3 of tile T are d = 32*T + 8*i + 4*lh + (0..3): 8-byte slot 8*T + 2*i + lh of the row.
-        const int f = g * RPG + 4 * r4;
         const int sl = 8 * (f / 16) + 2 * ((f % 16) / 4) + lh;
         *(PACK4*)(lds + O_OFF_LDS + orow * (D * 2) + ((sl ^ (orow % OSW)) * 8)) = y;
+#endif
       }
     }
   }
+#if KV_CTAS == 1
   __syncthreads();
   {
     ELT* obase = Op + O_OFF + (long)batch * O_SB + (long)head * O_SH;
@@ -498,6 +523,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       }
     }
   }
+#endif
   }
 }
 """
@@ -570,6 +596,15 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         raise LoweringError("flash: offsets break 16-byte alignment")
     qblocks = -(-body.q_len // BQ)
     pair = bool(body.pair)
+    split = int(getattr(body, "kv_ctas", 1) or 1)
+    if split > 1:
+        if body.partials is None:
+            raise LoweringError("flash: a cross-workgroup key split (REDUCE=g<n>k) is lowered as a partial kernel plus a combine (passes.lower), not by this emitter alone")
+        if pair or body.mask is not None or (getattr(body, "sym", None) is not None and body.sym.fields):
+            raise LoweringError("flash: the cross-workgroup key split takes no mirrored pairs, mask operand or symbolic lengths")
+        step_keys = kvs * BKV
+        kv_chunk = -(-(-(-body.kv_len // split)) // step_keys) * step_keys  # whole key steps per slice
+        split = -(-body.kv_len // kv_chunk)  # slices that hold keys
     # Symbolic lengths (``body.sym``): SQ / SKV, the query-block count, the launch size and a [B, H, S, D] tensor's
     # batch stride become expressions over the kernel's trailing ``int`` parameter; every guard the loop has for
     # ragged lengths (row clamps, key masks, the causal block limit) already reads them at run time.
@@ -608,7 +643,9 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "KRPL": max(1, 16 // (D // 8)),
         "TG": min(4, D // 32),
         "SQ": c_value(symf.get("q_len", body.q_len)),
-        "SKV": c_value(symf.get("kv_len", body.kv_len)),
+        **({"SKV_ALL": body.kv_len, "KV_CHUNK": kv_chunk, "BATCH": body.batch} if split > 1 else {"SKV": c_value(symf.get("kv_len", body.kv_len))}),
+        "KV_CTAS": split,
+        "OUT_T": "float" if split > 1 else rt.type_name(body.dtype.name),
         "HQ": body.q_heads,
         "GROUP": body.q_heads // body.kv_heads,
         "QBLOCKS": "((SQ + BQ - 1) / BQ)" if "q_len" in symf else qblocks,
@@ -621,7 +658,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
             "INV_SCALE": float_literal(1.0 / body.scale)} if has_mask else {}),
         "PAIR": 1 if pair else 0,
         # steps in parity pairs (static ring slots) unless the whole key range is one or two steps
-        "PAIRSTEP": 1 if _PAIRSTEP and body.pair_steps and (bool(symf) or -(-body.kv_len // (kvs * BKV)) > 2) else 0,
+        "PAIRSTEP": 1 if _PAIRSTEP and body.pair_steps and (bool(symf) or -(-(kv_chunk if split > 1 else body.kv_len) // (kvs * BKV)) > 2) else 0,
         "V_PRE": 1 if _V_PRE and (BKV // 32) * 2 * (D // 32) * 4 <= 32 else 0,  # the prefetched V fragments take at most 32 registers
         "RK": plan["rk"], "RV": plan["rv"], "DEEP": 1 if plan["deep"] else 0,
         "Q_LDS": 1 if plan["q_off"] is not None else 0,
@@ -653,13 +690,62 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     return HipOp(
         kernel_source=source,
         kernel_name=name,
-        arg_order=(body.q, body.k, body.v, *((body.mask,) if has_mask else ()), body.out),
-        grid=((CeilDiv(symf["q_len"], BQ), body.q_heads * body.batch) if "q_len" in symf else (grid,), (1,), (1,)),
+        arg_order=(body.q, body.k, body.v, *((body.mask,) if has_mask else ()), body.partials if split > 1 else body.out),
+        grid=((CeilDiv(symf["q_len"], BQ), body.q_heads * body.batch) if "q_len" in symf else (grid,), (split,), (1,)),
         block=((NT,), (1,), (1,)),
         lds_bytes=lds,
         runtime_args=(sym.name,) if symf else (),
         comment=f"flash Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} bkv={BKV} split={kvs} pair={int(pair)}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
-        knobs={"FLASH": f"w{waves}/kv{BKV}/s{kvs}" + ("/p" if pair else "") + ("/k3" if plan["deep"] else "")},
+        knobs={"FLASH": f"w{waves}/kv{BKV}/s{kvs}" + ("/p" if pair else "") + ("/k3" if plan["deep"] else ""), **({"REDUCE": f"g{split}k"} if split > 1 else {})},
+    )
+
+
+def flash_partial_slices(body: Flash) -> int:
+    """Key slices the partial kernel of ``body``'s cross-workgroup split actually runs (slices are whole key steps, so
+    fewer than asked for can hold all the keys)."""
+    step_keys = body.kv_split * body.block_kv
+    chunk = -(-(-(-body.kv_len // body.kv_ctas)) // step_keys) * step_keys
+    return -(-body.kv_len // chunk)
+
+
+def emit_flash_combine(body: Flash, ws: str, name: str, ctx: Context = Context()) -> HipOp:
+    """Merge of the key slices' ``(m, l, O)``: per query row ``m = max m_s``, ``l = sum l_s 2^(m_s - m)``,
+    ``out = sum O_s 2^(m_s - m) / l`` — the exp-family combine the streaming loop uses, applied across workgroups (the
+    reference's kernel finalize of the twisted carrier, passes/lowering/tile/030_split.py:217-334).  One thread per four
+    consecutive output values; the workspace row is ``head_dim`` values, then ``m`` (log2 units) and ``l``."""
+    D, S = body.head_dim, flash_partial_slices(body)
+    rows = body.batch * body.q_heads * body.q_len
+    elt, pack4 = rt.type_name(body.dtype.name), rt.vector_type(body.dtype.name, 4)[0]
+    groups = rows * (D // 4)
+    o: list[str] = []
+    a = o.append
+    a(f"// {name}: combine of {S} key slices of attention B={body.batch} Hq={body.q_heads} Sq={body.q_len} D={D}")
+    a(f'extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ WS, {elt}* __restrict__ O) {{')
+    a("  const long q = (long)blockIdx.x * 256 + threadIdx.x;")
+    a(f"  if (q >= {groups}L) return;")
+    a(f"  const long row = q / {D // 4}; const int c = (int)(q % {D // 4}) * 4;")
+    a(f"  const long s_ = row % {body.q_len}, h_ = (row / {body.q_len}) % {body.q_heads}, b_ = row / {body.q_len * body.q_heads};")
+    a(f"  const float* w0 = WS + row * {D + 4};")
+    a("  float m = w0[" + str(D) + "];")
+    for s in range(1, S):
+        a(f"  m = fmaxf(m, w0[{s * rows * (D + 4) + D}L]);")
+    a("  float l = 0.0f; f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};")
+    for s in range(S):
+        a(f"  {{ const float* w = w0 + {s * rows * (D + 4)}L; const float e = exp2f(w[{D}] - m); l += w[{D + 1}] * e; const f32x4 t = *(const f32x4*)(w + c); acc[0] += t[0] * e; acc[1] += t[1] * e; acc[2] += t[2] * e; acc[3] += t[3] * e; }}")
+    a("  const float inv = 1.0f / l;")
+    a(f"  {pack4} y; y[0] = ({elt})(acc[0] * inv); y[1] = ({elt})(acc[1] * inv); y[2] = ({elt})(acc[2] * inv); y[3] = ({elt})(acc[3] * inv);")
+    a(f"  *({pack4}*)(O + {body.o_offset}L + b_ * {body.o_strides[0]}L + h_ * {body.o_strides[1]}L + s_ * {body.o_strides[2]}L + c) = y;")
+    a("}")
+    return HipOp(
+        kernel_source=prelude.header() + "\n".join(o) + "\n",
+        kernel_name=name,
+        arg_order=(ws, body.out),
+        grid=((-(-groups // 256),), (1,), (1,)),
+        block=((256,), (1,), (1,)),
+        comment=f"combine of {S} key slices of attention Sq={body.q_len} Skv={body.kv_len} D={D}",
+        algo_bytes=S * rows * (D + 4) * 4 + rows * D * body.dtype.nbytes,
+        algo_flops=0,
+        knobs={"REDUCE": f"g{S}k"},
     )

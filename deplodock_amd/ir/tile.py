@@ -281,6 +281,11 @@ class Flash:
     pair_steps: bool = True  # key steps unrolled in pairs so ring slots are compile-time (the lowering clears it if that build spills)
     ws: bool = False  # wave-specialised form: four consumer waves (waves x kv_split = 4) and four staging waves
     sp: bool = False  # software-pipelined form without staging waves: eight consumer waves (waves x kv_split = 8) stage for themselves
+    # cross-workgroup split of the keys (``REDUCE=g<n>k``): ``kv_ctas`` workgroups per query block each take a contiguous
+    # slice of the keys and leave their (m, l, O) in a workspace; a combine kernel merges the slices.  ``partials`` names
+    # the workspace when this body is the partial kernel of such a pair.
+    kv_ctas: int = 1
+    partials: str | None = None
     # an additive bias on the scaled scores, ``[batch, head, query, key]`` addressed through (batch, head, query)
     # strides (0 = broadcast) with keys contiguous; ``None``: no mask operand
     mask: str | None = None

@@ -26,6 +26,7 @@ from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.emit.splitk import emit_splitk_combine, partial_body, split_planes
 from deplodock_amd.graph import Graph, Node, Tensor
 from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.schedule import ReducePlan
 from deplodock_amd.ir.tile import Contraction, Flash, IndexRows, LoopNest, Map, RowReduce, StridedCopy, TileOp
 
 _PLACEHOLDER = "EMH_KERNEL_NAME_"
@@ -136,6 +137,74 @@ def _lower_split_contraction(graph: Graph, node: Node, ctx: Context) -> None:
     node.inputs = [ws_id, *node.inputs]
 
 
+def _lower_split_row_reduce(graph: Graph, node: Node, ctx: Context) -> None:
+    """``REDUCE=g<n>k`` on a row reduction with one value per row (``sum`` / ``mean`` / ``amax`` over the last axis, or
+    any single statistic followed by a projection of it): the columns of a row are split into ``n`` contiguous slices.
+    Slice j of row r is row ``r * n + j`` of the same buffer seen as ``[rows * n, cols / n]``, so the *partial* kernel is
+    the ordinary row kernel over that view with the bare statistic as its output (an fp32 ``[rows, n]`` workspace), and
+    the *combine* kernel is the ordinary row kernel over the workspace with the same monoid and the original projection —
+    applied once, after the cross-workgroup fold, so it need not distribute over it (the reference's deferred kernel
+    finalize, tests/compiler/e2e/test_reduce_coverage.py:280-345)."""
+    from deplodock_amd.ir import expr as E
+    from deplodock_amd.ir.tile import RowAddr, Stat
+    from deplodock_amd.passes.schedule import pick_coop
+
+    op: TileOp = node.op
+    body: RowReduce = op.body
+    n = body.reduce.cta
+    (stat,) = body.stats
+    label, _, rest = op.name.partition("__")
+    ws_id = f"{node.id}__partial"
+    if ws_id in graph.nodes:
+        raise LoweringError(f"row reduce: workspace id {ws_id!r} is taken")
+    addr = body.x_addr or RowAddr.uniform(body.cols)
+    width = body.cols // n
+    part = RowReduce(
+        rows=body.rows * n, cols=width, x=body.x, x_dtype=body.x_dtype, out=ws_id, out_dtype=F32, stats=(stat,), project=E.Var(stat.name),
+        x_addr=RowAddr(offset=addr.offset, div=n, stride_hi=addr.stride_hi, stride_lo=width), scalar_out=True, nontemporal=body.nontemporal,
+        reduce=ReducePlan(coop=pick_coop(width, body.x_dtype.nbytes, body.rows * n, ctx, rotate=False, stats=1)),
+    )  # fmt: skip
+    comb = RowReduce(
+        rows=body.rows, cols=n, x=ws_id, x_dtype=F32, out=body.out, out_dtype=body.out_dtype, stats=(Stat(stat.name, stat.monoid, E.Var("x")),), project=body.project,
+        out_addr=body.out_addr, scalar_out=True, reduce=ReducePlan(coop=pick_coop(n, 4, body.rows, ctx, rotate=False, stats=1)),
+    )  # fmt: skip
+    part_hip = _named(emit_row_reduce(part, _PLACEHOLDER, ctx), TileOp(name=f"{label}_partial__{rest}", body=part, knobs=dict(op.knobs)))
+    comb_hip = _named(emit_row_reduce(comb, _PLACEHOLDER, ctx), TileOp(name=f"{label}_combine__{rest}", body=comb, knobs=dict(op.knobs)))
+    part_hip.knobs = {**part_hip.knobs, "REDUCE": body.reduce.spell()}
+    comb_hip.knobs = {**comb_hip.knobs, "REDUCE": body.reduce.spell()}
+    graph.nodes[ws_id] = Node(ws_id, part_hip, list(node.inputs), Tensor(ws_id, (body.rows, n), F32))
+    node.op = comb_hip
+    node.inputs = [ws_id]
+
+
+def _lower_split_flash(graph: Graph, node: Node, ctx: Context) -> None:
+    """``REDUCE=g<n>k`` on attention: the node becomes the combine kernel and gains a producer, the partial kernel, whose
+    output is the fp32 workspace ``[slices, batch, heads, queries, head_dim + 4]`` (``head_dim`` unnormalised output
+    values, the slice's row maximum and row sum, padding to whole 16-byte rows) — the two-node form of the reference's
+    split rewrite (emmy/compiler/pipeline/passes/lowering/tile/030_split.py:217-334)."""
+    import dataclasses
+
+    from deplodock_amd.emit.flash import emit_flash_combine, flash_partial_slices
+
+    op: TileOp = node.op
+    body: Flash = op.body
+    label, _, rest = op.name.partition("__")
+    ws_id = f"{node.id}__partial"
+    if ws_id in graph.nodes:
+        raise LoweringError(f"flash: workspace id {ws_id!r} is taken")
+    part = dataclasses.replace(body, partials=ws_id, pair=False)
+    part_op = TileOp(name=f"{label}_partial__{rest}", body=part, knobs=dict(op.knobs))
+    part_hip = _lower_flash(part_op, ctx)
+    slices = flash_partial_slices(part)
+    comb_op = TileOp(name=f"{label}_combine__{rest}", body=body, knobs=dict(op.knobs))
+    comb_hip = _named(emit_flash_combine(part, ws_id, _PLACEHOLDER, ctx), comb_op)
+    comb_hip.knobs = {**part_hip.knobs}
+    inputs = [i for i in node.inputs]
+    graph.nodes[ws_id] = Node(ws_id, part_hip, inputs, Tensor(ws_id, (slices, body.batch, body.q_heads, body.q_len, body.head_dim + 4), F32))
+    node.op = comb_hip
+    node.inputs = [ws_id]
+
+
 def _lower_flash(op: TileOp, ctx: Context) -> HipOp:
     """The attention kernel waits for part of its outstanding direct-to-LDS loads by count, as the contraction's
     rings do, so it must build without vector-register spills too.  A schedule that spills gives up, in turn: the
@@ -193,6 +262,10 @@ def lower(graph: Graph, ctx: Context | None = None) -> Graph:
         if isinstance(node.op, TileOp):
             if isinstance(node.op.body, Contraction) and node.op.body.reduce.cta > 1:
                 _lower_split_contraction(graph, node, ctx)
+            elif isinstance(node.op.body, Flash) and node.op.body.kv_ctas > 1:
+                _lower_split_flash(graph, node, ctx)
+            elif isinstance(node.op.body, RowReduce) and node.op.body.reduce.cta > 1:
+                _lower_split_row_reduce(graph, node, ctx)
             else:
                 node.op = lower_tile(node.op, ctx)
     return graph

@@ -139,9 +139,25 @@ def schedule_row_reduce(body: RowReduce, ctx: Context) -> dict:
         try:
             plan = ReducePlan.parse(pinned)
             if plan.cta != 1:
-                raise ScheduleError("cross-workgroup split does not apply to a projected row")
-            if -(-body.cols // plan.coop) > 64:
-                raise ScheduleError(f"{body.cols} columns over {plan.coop} lanes do not fit the register-resident row")
+                # one value per row from a single statistic: the columns split across workgroups (partial row kernel into
+                # an fp32 workspace, combine row kernel with the projection); anything that writes the row back does not
+                addr = body.x_addr
+                if not (body.scalar_out and len(body.stats) == 1 and not body.col_operands and not body.row_operands and body.rotate is None):
+                    raise ScheduleError("cross-workgroup split does not apply to a projected row")
+                if addr is not None and addr.div != 1:
+                    raise ScheduleError("cross-workgroup split needs uniformly strided rows")
+                if getattr(body, "sym", None) is not None and body.sym.fields:
+                    raise ScheduleError("cross-workgroup split does not combine with a symbolic row count")
+                vec = max(1, 16 // body.x_dtype.nbytes)
+                if body.cols % plan.cta or (body.cols // plan.cta) % vec:
+                    raise ScheduleError(f"{body.cols} columns do not split into {plan.cta} slices of whole 16-byte chunks")
+                if plan.finalize == "atomic":
+                    logger.warning("EMMY_REDUCE=%r: a row's projection is applied once, after the fold: g%dk instead", pinned, plan.cta)
+                    plan = ReducePlan(cta=plan.cta, coop=plan.coop, reg=plan.reg, finalize="kernel")
+                if plan.coop == 1:
+                    plan = ReducePlan(cta=plan.cta, coop=pick_coop(body.cols // plan.cta, body.x_dtype.nbytes, body.rows * plan.cta, ctx, stats=1), reg=plan.reg, finalize="kernel")
+            if -(-(body.cols // plan.cta) // plan.coop) > 64:
+                raise ScheduleError(f"{body.cols // plan.cta} columns over {plan.coop} lanes do not fit the register-resident row")
             if body.rotate is not None:
                 vec = 16 // max(body.x_dtype.nbytes, body.out_dtype.nbytes)
                 if (body.cols // vec // 2) % plan.coop:
@@ -613,7 +629,45 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 body.kv_split //= 2
     if getattr(body, "sym", None) is not None and body.sym.fields:
         body.pair = False  # pairing mirrored query blocks needs the block count when the kernel is built
-    return {"FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "") + ("/k3" if body.deep else "") + ("/ws" if body.ws else "") + ("/sp" if body.sp else "")}
+    knobs = _schedule_flash_split(body, ctx, tuned if (tuned := _tuned(body, ctx)) else None)
+    return {**knobs, "FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "") + ("/k3" if body.deep else "") + ("/ws" if body.ws else "") + ("/sp" if body.sp else "")}
+
+
+def _schedule_flash_split(body: Flash, ctx: Context, tuned: dict | None) -> dict:
+    """``REDUCE=g<n>[k]`` on attention: ``n`` workgroups per query block split the keys and a combine kernel merges their
+    ``(m, l, O)`` (the reference's cross-CTA finalize of the twisted carrier is kernel-only, tests/compiler/e2e/
+    test_reduce_coverage.py:280-315; ``g<n>a`` is taken as ``g<n>k``).  Unpinned: where the query blocks cover less than
+    half the CUs and the keys are long — decode-size queries over a long cache — the keys are split until the launch covers
+    the CUs, in slices of at least 512 keys."""
+    body.kv_ctas = 1
+    plain = body.mask is None and not (getattr(body, "sym", None) is not None and body.sym.fields) and not (body.ws or body.sp)
+    pinned = _pin("REDUCE", tuned)
+    n = 1
+    if pinned:
+        try:
+            plan = ReducePlan.parse(pinned)
+            if plan.cta > 1:
+                if not plain:
+                    raise ScheduleError("the cross-workgroup key split takes no mask operand, symbolic lengths or software-pipelined form")
+                if plan.finalize == "atomic":
+                    logger.warning("EMMY_REDUCE=%r: the (m, l, O) carrier has no atomic finalize: g%dk instead", pinned, plan.cta)
+                n = plan.cta
+        except ScheduleError as exc:
+            logger.warning("EMMY_REDUCE=%r ignored for attention: %s", pinned, exc)
+    elif plain and not body.causal:
+        groups = body.batch * body.q_heads * -(-body.q_len // (32 * body.waves))
+        if 2 * groups <= ctx.compute_units and body.kv_len >= 2048:
+            n = 1
+            while n < 16 and groups * n * 2 <= ctx.compute_units and body.kv_len // (2 * n) >= 512:
+                n *= 2
+    if n > 1:
+        step = body.kv_split * body.block_kv
+        chunk = -(-(-(-body.kv_len // n)) // step) * step
+        n = -(-body.kv_len // chunk)
+    if n > 1:
+        body.kv_ctas, body.pair = n, False
+        return {"REDUCE": f"g{n}k"}
+    return {}
 
 
 def schedule(graph: Graph, ctx: Context | None = None) -> Graph:
