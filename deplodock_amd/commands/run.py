@@ -33,6 +33,9 @@ def register_run_command(subparsers) -> None:
     p.add_argument("--ir", default=None, metavar="PATH", help="Replay a JSON graph on seeded random data: one written by `compile --json` (traced or lowered stage), or one in the reference's own form (a traced block, or a Loop-IR kernel of its kernels/*.json corpus); no eager check (there is no module to compare with).")
     p.add_argument("--at", action="append", default=None, metavar="NAME=SIZE", help="With --dynamic: also run and check the expression with symbolic axis NAME at SIZE (repeatable).")
     p.add_argument("--ab", action="append", default=None, metavar="KNOBS", help="Also compile + bench a variant with these knobs pinned ('K1=V1,K2=V2'); repeatable; needs --bench.")
+    p.add_argument("--profile", action="store_true", help="Run the same command line again under rocprofv3 (a kernel trace, then one pass per counter set) and print a per-kernel table of launch time and hardware counters.")
+    p.add_argument("--pmc", action="append", default=None, metavar="COUNTERS", help="With --profile: one counter set per use, space separated (a set must fit one pass); default: 'SQ_INSTS_VALU SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES' and 'FETCH_SIZE' and 'WRITE_SIZE'.")
+    p.add_argument("--profile-dir", default=None, metavar="DIR", help="With --profile: keep rocprofv3's raw output here (default: a temporary directory).")
     p.set_defaults(func=handle_run)
 
 
@@ -247,7 +250,112 @@ def _run_ir(args, device) -> None:
             print(line)
 
 
+PROFILE_CHILD_ENV = "EMMY_PROFILE_CHILD"
+DEFAULT_COUNTER_SETS = ("SQ_INSTS_VALU SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES", "FETCH_SIZE", "WRITE_SIZE")
+
+
+def _child_command(argv: list[str]) -> list[str]:
+    """The command line of this invocation without the profiling options: what the profiler runs."""
+    out, skip = [], False
+    for tok in argv:
+        if skip:
+            skip = False
+            continue
+        if tok == "--profile":
+            continue
+        if tok in ("--pmc", "--profile-dir"):
+            skip = True
+            continue
+        if tok.startswith("--pmc=") or tok.startswith("--profile-dir="):
+            continue
+        out.append(tok)
+    return [sys.executable, "-m", "deplodock_amd", *out]
+
+
+def _read_csvs(root: Path, suffix: str) -> list[dict]:
+    import csv
+
+    rows: list[dict] = []
+    for path in sorted(root.rglob(f"*{suffix}")):
+        with open(path, newline="") as fh:
+            rows.extend(csv.DictReader(fh))
+    return rows
+
+
+def profile_tables(trace_dir: Path | None, counter_dirs: list[Path]) -> tuple[list[str], list[list[str]]]:
+    """Header and rows of the per-kernel table: launches and average / minimum duration from a kernel trace, the
+    per-launch average of every counter from the counter passes.  Only the emitted kernels (``k_*``) are listed."""
+    durations: dict[str, list[float]] = {}
+    if trace_dir is not None:
+        for rec in _read_csvs(trace_dir, "kernel_trace.csv"):
+            name = rec.get("Kernel_Name", "")
+            if name.startswith("k_"):
+                durations.setdefault(name, []).append((float(rec["End_Timestamp"]) - float(rec["Start_Timestamp"])) / 1e3)
+    counters: dict[str, dict[str, list[float]]] = {}
+    for d in counter_dirs:
+        for rec in _read_csvs(d, "counter_collection.csv"):
+            name = rec.get("Kernel_Name", "")
+            if name.startswith("k_"):
+                counters.setdefault(name, {}).setdefault(rec["Counter_Name"], []).append(float(rec["Counter_Value"]))
+    names = sorted(set(durations) | set(counters), key=lambda n: -sum(durations.get(n, [0.0])))
+    cols = sorted({c for per in counters.values() for c in per})
+    header = ["kernel", "launches", "avg us", "min us", *cols]
+    rows = []
+    for n in names:
+        ds = durations.get(n, [])
+        row = [n, str(len(ds) or len(next(iter(counters.get(n, {"": []}).values()), []))), f"{statistics.mean(ds):.2f}" if ds else "-", f"{min(ds):.2f}" if ds else "-"]
+        for c in cols:
+            vals = counters.get(n, {}).get(c)
+            row.append(f"{statistics.mean(vals):.4g}" if vals else "-")
+        rows.append(row)
+    return header, rows
+
+
+def run_profile(args, argv: list[str]) -> int:
+    """``run --profile``: the same command line again, as children of ``rocprofv3`` — the interpreter itself after ``--``,
+    one run for the kernel trace and one per counter set, none of them combined with a runtime trace — started before this
+    process has touched the GPU.  Prints the per-kernel table (the reference's ``--profile`` re-runs itself under its
+    vendor's profiler and prints a counter table, emmy/commands/run.py:691-928)."""
+    import os
+    import shutil
+    import subprocess
+    import tempfile
+
+    rocprof = shutil.which("rocprofv3")
+    if rocprof is None:
+        print("error: rocprofv3 is not on PATH", file=sys.stderr)
+        return 2
+    child = _child_command(argv)
+    keep = Path(args.profile_dir) if args.profile_dir else None
+    root = keep or Path(tempfile.mkdtemp(prefix="emmy_profile_"))
+    root.mkdir(parents=True, exist_ok=True)
+    env = {**os.environ, PROFILE_CHILD_ENV: "1", "TMPDIR": os.environ.get("TMPDIR", "/tmp")}
+    passes = [("trace", ["--kernel-trace", "--stats"])] + [(f"pmc{i}", ["--pmc", *cs.split()]) for i, cs in enumerate(args.pmc or DEFAULT_COUNTER_SETS)]
+    dirs: dict[str, Path] = {}
+    for tag, opts in passes:
+        out = root / tag
+        cmd = [rocprof, *opts, "--output-format", "csv", "-d", str(out), "--", *child]
+        print(f"[profile] {' '.join(cmd)}", flush=True)
+        res = subprocess.run(cmd, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=900)
+        if res.returncode != 0:
+            print(res.stdout[-2000:], file=sys.stderr)
+            print(f"error: the {tag} pass ended with status {res.returncode}", file=sys.stderr)
+            return 1
+        dirs[tag] = out
+    header, rows = profile_tables(dirs.get("trace"), [d for t, d in dirs.items() if t != "trace"])
+    print()
+    for line in render_table(header, rows, "l" + "r" * (len(header) - 1)):
+        print(line)
+    if keep is None:
+        shutil.rmtree(root, ignore_errors=True)
+    return 0
+
+
 def handle_run(args) -> None:
+    import os
+
+    if getattr(args, "profile", False) and not os.environ.get(PROFILE_CHILD_ENV):
+        sys.exit(run_profile(args, sys.argv[1:]))
     import torch
 
     from deplodock_amd.backend.hip.backend import HipBackend

@@ -178,3 +178,36 @@ def test_run_a_built_in_architecture(capsys):
     assert out.startswith("PASS") and "mean |ours - fp32 eager|" in out and "emmy (hip)" in out
     main(["run", "arch:llama-tiny", "--dtype", "fp32", "--layer", "0", "--seq-len", "24"])
     assert capsys.readouterr().out.startswith("PASS")
+
+
+def test_profile_child_command_drops_only_the_profiling_options():
+    """``run --profile`` runs the same command line again under the profiler: the interpreter itself, the module, and
+    every option except the ones that ask for the profile."""
+    import sys
+
+    from deplodock_amd.commands.run import _child_command
+
+    argv = ["run", "--profile", "--pmc", "SQ_INSTS_VALU SQ_INSTS_MFMA", "--bench", "-c", "nn.Softmax(-1)(torch.randn(4, 64))", "--pmc=FETCH_SIZE", "--profile-dir", "out", "--knobs", "REDUCE=b64"]
+    assert _child_command(argv) == [sys.executable, "-m", "deplodock_amd", "run", "--bench", "-c", "nn.Softmax(-1)(torch.randn(4, 64))", "--knobs", "REDUCE=b64"]
+
+
+def test_profile_table_joins_the_trace_with_the_counter_passes(tmp_path):
+    """Per emitted kernel: launches and average / minimum duration from the kernel trace, per-launch averages of every
+    counter from the counter passes; the runtime's own kernels are left out."""
+    from deplodock_amd.commands.run import profile_tables
+
+    trace, pmc0, pmc1 = tmp_path / "trace" / "vm", tmp_path / "pmc0" / "vm", tmp_path / "pmc1" / "vm"
+    for d in (trace, pmc0, pmc1):
+        d.mkdir(parents=True)
+    (trace / "1_kernel_trace.csv").write_text(
+        '"Kind","Agent_Id","Queue_Id","Stream_Id","Thread_Id","Dispatch_Id","Kernel_Id","Kernel_Name","Correlation_Id","Start_Timestamp","End_Timestamp"\n'
+        '"KERNEL_DISPATCH","Agent 1",1,1,1,1,1,"k_softmax_reduce_abc123",1,1000,3000\n'
+        '"KERNEL_DISPATCH","Agent 1",1,1,1,2,1,"k_softmax_reduce_abc123",2,5000,9000\n'
+        '"KERNEL_DISPATCH","Agent 1",1,1,1,3,2,"__amd_rocclr_copyBuffer",3,9000,9500\n'
+    )
+    head = '"Correlation_Id","Dispatch_Id","Agent_Id","Queue_Id","Process_Id","Thread_Id","Grid_Size","Kernel_Id","Kernel_Name","Workgroup_Size","LDS_Block_Size","Scratch_Size","VGPR_Count","Accum_VGPR_Count","SGPR_Count","Counter_Name","Counter_Value","Start_Timestamp","End_Timestamp"\n'
+    (pmc0 / "2_counter_collection.csv").write_text(head + '1,1,"Agent 1",1,1,1,256,1,"k_softmax_reduce_abc123",256,0,0,32,0,16,"SQ_INSTS_VALU",100,0,0\n1,2,"Agent 1",1,1,1,256,1,"k_softmax_reduce_abc123",256,0,0,32,0,16,"SQ_INSTS_VALU",300,0,0\n')
+    (pmc1 / "3_counter_collection.csv").write_text(head + '1,1,"Agent 1",1,1,1,256,1,"k_softmax_reduce_abc123",256,0,0,32,0,16,"FETCH_SIZE",64,0,0\n1,2,"Agent 1",1,1,1,256,2,"__amd_rocclr_copyBuffer",256,0,0,32,0,16,"FETCH_SIZE",999,0,0\n')
+    header, rows = profile_tables(tmp_path / "trace", [tmp_path / "pmc0", tmp_path / "pmc1"])
+    assert header == ["kernel", "launches", "avg us", "min us", "FETCH_SIZE", "SQ_INSTS_VALU"]
+    assert rows == [["k_softmax_reduce_abc123", "2", "3.00", "2.00", "64", "200"]]
