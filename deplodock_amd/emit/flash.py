@@ -63,6 +63,10 @@ EMH_DEV int emh_kswz(int row, int c) { return c ^ ((row / KRPL) % CPR); }
 #define EMH_VROT(row) (D >= 128 ? ((row) % 4) : (((row) >> 1) & 1))  /* 128-byte rows: two rows share a bank line */
 EMH_DEV int emh_vswz(int row, int c) { return c ^ (EMH_VROT(row) << 2); }
 EMH_DEV float emh_xor32(float v) { return __shfl_xor(v, 32, 64); }
+// Rows of DR < D values (a head_dim between the kernel's widths): the 16-byte chunks past the row's end are fetched from
+// the row's first chunk instead — finite values of the same row — and never count: q's are zeroed in registers, so k's
+// vanish in the scores, and v's only reach output columns that are not stored.
+EMH_DEV int emh_gchunk(int c) { return (DR == D || c < DR / 8) ? c : 0; }
 typedef short emh_s16x4 __attribute__((ext_vector_type(4)));
 #define KBYTES (BKV * D * 2)
 #define WQ (NT / 64 / KVS)           /* waves (32-row groups) per key-split group */
@@ -126,14 +130,14 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       if (QCHUNKS % NT == 0 || c0 + (tid - lane) < QCHUNKS) {  // whole waves: QCHUNKS is a multiple of 64
         const int r_ = (c0 + tid) / CPR, p_ = (c0 + tid) % CPR;
         const int qr_ = q0 + r_ < SQ ? q0 + r_ : SQ - 1;
-        emh_dma16(qbase + (long)qr_ * Q_SS + emh_kswz(r_, p_) * 8, lds + Q_OFF_LDS + (c0 + tid - lane) * 16);
+        emh_dma16(qbase + (long)qr_ * Q_SS + emh_gchunk(emh_kswz(r_, p_)) * 8, lds + Q_OFF_LDS + (c0 + tid - lane) * 16);
       }
     }
   } else {
     const int qr = qrow < SQ ? qrow : SQ - 1;
     const ELT* qp = qbase + (long)qr * Q_SS + 8 * lh;
     #pragma unroll
-    for (int kk = 0; kk < D / 16; ++kk) qf[kk] = *(const FRAG*)(qp + 16 * kk);
+    for (int kk = 0; kk < D / 16; ++kk) qf[kk] = *(const FRAG*)(qp + 8 * (emh_gchunk(2 * kk + lh) - lh));
   }
   int ntiles = (SKV + BKV - 1) / BKV;
   if (CAUSAL) {
@@ -165,8 +169,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   #pragma unroll
   for (int i = 0; i < PER_T; ++i) {
     const int g_ = (i * NT) / CHUNKS, ro_ = ((i * NT) % CHUNKS) / CPR;
-    kvo[i] = (unsigned)((g_ * BKV + ro_ + st_row) * K_SS + emh_kswz(st_row + ro_, st_pos) * 8) * 2u;
-    vvo[i] = (unsigned)((g_ * BKV + ro_ + st_row) * V_SS + emh_vswz(st_row + ro_, st_pos) * 8) * 2u;
+    kvo[i] = (unsigned)((g_ * BKV + ro_ + st_row) * K_SS + emh_gchunk(emh_kswz(st_row + ro_, st_pos)) * 8) * 2u;
+    vvo[i] = (unsigned)((g_ * BKV + ro_ + st_row) * V_SS + emh_gchunk(emh_vswz(st_row + ro_, st_pos)) * 8) * 2u;
   }
   // EMH_STEP_BASES(st) names the scalar parts of the requests of step st once (K and V plane bases moved to the
   // step's keys, the ring slots' LDS addresses); EMH_STAGE_K / _V(st, i) then issue request i against them.
@@ -182,7 +186,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       } else { \
         long krow_ = (long)((st) * KVS + g_) * BKV + ro_ + st_row; \
         if (krow_ > SKV - 1) krow_ = SKV - 1; \
-        emh_dma16((base_) + krow_ * (stride_) + swz_(st_row + ro_, st_pos) * 8, lds + (ldo_) + g_ * KBYTES + (((i) * NT) % CHUNKS) * 16 + dst_lane); } }
+        emh_dma16((base_) + krow_ * (stride_) + emh_gchunk(swz_(st_row + ro_, st_pos)) * 8, lds + (ldo_) + g_ * KBYTES + (((i) * NT) % CHUNKS) * 16 + dst_lane); } }
   #define EMH_STAGE_K(tag, st, i) EMH_STAGE_ONE(st, i, kb##tag, kl##tag, kbase, K_SS, kvo, emh_kswz, EMH_SLOT(st, RK) * SETB)
   #define EMH_STAGE_V(tag, st, i) EMH_STAGE_ONE(st, i, vb##tag, vl##tag, vbase, V_SS, vvo, emh_vswz, V_RING + EMH_SLOT(st, RV) * SETB)
   // Requests are issued between MFMAs, spread evenly over a chain of NQ_SLOTS of them (request i behind MFMA
@@ -245,6 +249,14 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
     const int qr_ = wq * 32 + lq;
     #pragma unroll
     for (int kk = 0; kk < D / 16; ++kk) qf[kk] = *(const FRAG*)(lds + Q_OFF_LDS + qr_ * (D * 2) + emh_kswz(qr_, kk * 2 + lh) * 16);
+  }
+  if (DR < D) {  // the columns past the row's end count as zeros
+    #pragma unroll
+    for (int kk = 0; kk < D / 16; ++kk)
+      if (2 * kk + lh >= DR / 8) {
+        #pragma unroll
+        for (int e = 0; e < 8; ++e) qf[kk][e] = (ELT)0.0f;
+      }
   }
 
   // Steps run in pairs so that a step's ring slots (its parity) are known when the code is generated: the LDS
@@ -519,7 +531,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         u32x4 y;
         y[0] = (x & 1) ? t[2] : t[0]; y[1] = (x & 1) ? t[3] : t[1];
         y[2] = (x & 1) ? t[0] : t[2]; y[3] = (x & 1) ? t[1] : t[3];
-        if (q0 + r < SQ) *(u32x4*)(obase + (long)(q0 + r) * O_SS + pc * 8) = y;
+        if (q0 + r < SQ && (DR == D || pc < DR / 8)) *(u32x4*)(obase + (long)(q0 + r) * O_SS + pc * 8) = y;
       }
     }
   }
@@ -567,6 +579,9 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         raise LoweringError("flash: MFMA tier needs 16-bit operands")
     if D not in (64, 128, 256):
         raise LoweringError(f"flash: head_dim {D} must be 64, 128 or 256 on this tier")
+    DR = body.head_dim_real or D
+    if DR > D or DR % 8 or DR < 8:
+        raise LoweringError(f"flash: rows of {DR} values do not pad to head_dim {D} in whole 16-byte chunks")
     if body.q_heads % body.kv_heads:
         raise LoweringError("flash: q heads must be a multiple of kv heads")
     waves = body.waves
@@ -636,6 +651,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "KNAME": name,
         "NT": NT,
         "D": D,
+        "DR": DR,
         "BQ": BQ,
         "BKV": BKV,
         "KVS": kvs,
@@ -716,16 +732,17 @@ def emit_flash_combine(body: Flash, ws: str, name: str, ctx: Context = Context()
     reference's kernel finalize of the twisted carrier, passes/lowering/tile/030_split.py:217-334).  One thread per four
     consecutive output values; the workspace row is ``head_dim`` values, then ``m`` (log2 units) and ``l``."""
     D, S = body.head_dim, flash_partial_slices(body)
+    DR = body.head_dim_real or D  # the workspace rows are D wide; only the first DR columns are output
     rows = body.batch * body.q_heads * body.q_len
     elt, pack4 = rt.type_name(body.dtype.name), rt.vector_type(body.dtype.name, 4)[0]
-    groups = rows * (D // 4)
+    groups = rows * (DR // 4)
     o: list[str] = []
     a = o.append
     a(f"// {name}: combine of {S} key slices of attention B={body.batch} Hq={body.q_heads} Sq={body.q_len} D={D}")
     a(f'extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ WS, {elt}* __restrict__ O) {{')
     a("  const long q = (long)blockIdx.x * 256 + threadIdx.x;")
     a(f"  if (q >= {groups}L) return;")
-    a(f"  const long row = q / {D // 4}; const int c = (int)(q % {D // 4}) * 4;")
+    a(f"  const long row = q / {DR // 4}; const int c = (int)(q % {DR // 4}) * 4;")
     a(f"  const long s_ = row % {body.q_len}, h_ = (row / {body.q_len}) % {body.q_heads}, b_ = row / {body.q_len * body.q_heads};")
     a(f"  const float* w0 = WS + row * {D + 4};")
     a("  float m = w0[" + str(D) + "];")
@@ -745,7 +762,7 @@ def emit_flash_combine(body: Flash, ws: str, name: str, ctx: Context = Context()
         grid=((-(-groups // 256),), (1,), (1,)),
         block=((256,), (1,), (1,)),
         comment=f"combine of {S} key slices of attention Sq={body.q_len} Skv={body.kv_len} D={D}",
-        algo_bytes=S * rows * (D + 4) * 4 + rows * D * body.dtype.nbytes,
+        algo_bytes=S * rows * (D + 4) * 4 + rows * DR * body.dtype.nbytes,
         algo_flops=0,
         knobs={"REDUCE": f"g{S}k"},
     )

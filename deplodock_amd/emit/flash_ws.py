@@ -670,7 +670,7 @@ def ws_supported(body: Flash, ctx: Context = Context()) -> str | None:
     sp, consumers, rings = _shape(body)
     if body.dtype.name not in ("bf16", "f16"):
         return "16-bit operands only"
-    if body.head_dim not in (64, 128):
+    if body.head_dim not in (64, 128) or body.head_dim_real not in (None, body.head_dim):
         return "head_dim 64 or 128"
     if body.mask is not None:
         return "no mask operand"

@@ -286,6 +286,10 @@ class Flash:
     # the workspace when this body is the partial kernel of such a pair.
     kv_ctas: int = 1
     partials: str | None = None
+    # rows of the operands hold ``head_dim_real`` values when that is not one of the kernel's widths: ``head_dim`` is then
+    # the next width up, the missing columns of q count as zeros (k's and v's are never looked at: their products with a
+    # zero vanish, their output columns are not stored)
+    head_dim_real: int | None = None
     # an additive bias on the scaled scores, ``[batch, head, query, key]`` addressed through (batch, head, query)
     # strides (0 = broadcast) with keys contiguous; ``None``: no mask operand
     mask: str | None = None
@@ -298,12 +302,12 @@ class Flash:
             pairs = self.q_len * (self.q_len + 1) // 2
         else:
             pairs = self.q_len * self.kv_len
-        return 4 * self.batch * self.q_heads * self.head_dim * pairs
+        return 4 * self.batch * self.q_heads * (self.head_dim_real or self.head_dim) * pairs
 
     def algo_bytes(self) -> int:
         e = self.dtype.nbytes
-        q = self.batch * self.q_heads * self.q_len * self.head_dim
-        kv = self.batch * self.kv_heads * self.kv_len * self.head_dim
+        q = self.batch * self.q_heads * self.q_len * (self.head_dim_real or self.head_dim)
+        kv = self.batch * self.kv_heads * self.kv_len * (self.head_dim_real or self.head_dim)
         mask = 0
         if self.mask is not None:
             mb, mh, mq = self.mask_strides

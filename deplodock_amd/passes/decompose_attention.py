@@ -23,6 +23,14 @@ from deplodock_amd.ir import loopnest as L
 FLASH_HEAD_DIMS = (64, 128, 256)
 
 
+def flash_head_dim(d: int) -> int | None:
+    """The width the flash kernel runs a 16-bit head_dim ``d`` at: ``d`` itself or the next of its widths up (rows of whole
+    16-byte chunks are padded with columns that count as zeros); ``None`` when it takes neither."""
+    if d % 8 or d < 8:
+        return None
+    return next((w for w in FLASH_HEAD_DIMS if w >= d), None)
+
+
 class AttentionShapeError(ValueError):
     pass
 
@@ -146,7 +154,7 @@ def decompose_attention(g: Graph, undo_repeat) -> Graph:
 
     def flash_takes(node: Node) -> bool:
         t = g.nodes[node.inputs[0]].output
-        return t.dtype.name in ("bf16", "f16") and t.shape[-1] in FLASH_HEAD_DIMS
+        return t.dtype.name in ("bf16", "f16") and flash_head_dim(int(t.shape[-1])) is not None
 
     hits = [nid for nid, n in g.nodes.items() if isinstance(n.op, F.SdpaOp) and not flash_takes(n)]
     if not hits:

@@ -1219,8 +1219,11 @@ def _rec_sdpa(c: _Ctx, nid: str) -> bool:
             raise FusionError(f"sdpa: the mask must broadcast to [batch, heads, queries, keys] with contiguous keys, got {tuple(mv.shape)}")
         mask_kw = dict(mask=mv.base, mask_dtype=mv.dtype, mask_offset=mv.offset, mask_strides=tuple(0 if n == 1 else s_ for n, s_ in zip(shp[:3], st[:3])))
         inputs.append(mv.base)
+    from deplodock_amd.passes.decompose_attention import flash_head_dim
+
     body = Flash(
-        batch=B, q_heads=Hq, kv_heads=Hkv, q_len=Sq, kv_len=Skv, head_dim=D, q=q.base, k=k.base, v=v.base, out=out_id, dtype=q.dtype,
+        batch=B, q_heads=Hq, kv_heads=Hkv, q_len=Sq, kv_len=Skv, head_dim=flash_head_dim(D) or D, head_dim_real=D if (flash_head_dim(D) or D) != D else None,
+        q=q.base, k=k.base, v=v.base, out=out_id, dtype=q.dtype,
         scale=float(scale), causal=node.op.is_causal, q_strides=q_str, k_strides=k_str, v_strides=v_str, o_strides=o_strides,
         q_offset=q.offset, k_offset=k.offset, v_offset=v.offset, **mask_kw,
     )  # fmt: skip

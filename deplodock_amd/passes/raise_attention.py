@@ -52,7 +52,9 @@ def _match(g: Graph, node: Node):
     if not (len(q.shape) == len(k.shape) == len(v.shape) == rank) or q.dtype.name not in ("bf16", "f16") or not (q.dtype == k.dtype == v.dtype == node.output.dtype):
         return None
     d = int(q.shape[-1])
-    if d not in (64, 128, 256) or int(k.shape[-1]) != d or int(v.shape[-1]) != d or tuple(k.shape[:-1]) != tuple(v.shape[:-1]) or tuple(q.shape[:-2]) != tuple(k.shape[:-2]):
+    from deplodock_amd.passes.decompose_attention import flash_head_dim
+
+    if flash_head_dim(d) is None or int(k.shape[-1]) != d or int(v.shape[-1]) != d or tuple(k.shape[:-1]) != tuple(v.shape[:-1]) or tuple(q.shape[:-2]) != tuple(k.shape[:-2]):
         return None
     if mask is not None:
         m = g.nodes[mask].output

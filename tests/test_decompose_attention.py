@@ -82,8 +82,9 @@ def _kernel_names(compiled):
 
 
 def test_which_attention_is_decomposed():
-    """fp32, and 16-bit with a head_dim the flash kernel has no tiling for, become two batched contractions with
-    loop-nest operand / output stages; 16-bit head_dim 128 stays the one fused kernel."""
+    """fp32, and 16-bit with a head_dim that is not whole 16-byte chunks, become two batched contractions with loop-nest
+    operand / output stages; 16-bit head_dim 128 stays the one fused kernel, and a 16-bit head_dim between the kernel's
+    widths (32: padded to 64 with columns that count as zeros) takes it too."""
     be = HipBackend()
     q, k = torch.randn(1, 16, 128, 128), torch.randn(1, 8, 128, 128)
     names = _kernel_names(be.compile(trace_module(_Sdpa(is_causal=True, enable_gqa=True).eval(), (q, k, k))))
@@ -92,7 +93,12 @@ def test_which_attention_is_decomposed():
     names = _kernel_names(be.compile(trace_module(_Sdpa(is_causal=True, enable_gqa=True).eval(), (q.bfloat16(), k.bfloat16(), k.bfloat16()))))
     assert names == ["k_sdpa_reduce"]
     q32 = torch.randn(2, 4, 64, 32).bfloat16()
-    names = _kernel_names(be.compile(trace_module(_Sdpa().eval(), (q32, q32, q32))))
+    compiled = be.compile(trace_module(_Sdpa().eval(), (q32, q32, q32)))
+    assert _kernel_names(compiled) == ["k_sdpa_reduce"]
+    (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert "#define D 64\n" in op.kernel_source and "#define DR 32\n" in op.kernel_source
+    q36 = torch.randn(2, 4, 64, 36).bfloat16()
+    names = _kernel_names(be.compile(trace_module(_Sdpa().eval(), (q36, q36, q36))))
     assert names.count("k_batched_linear") == 2 and "k_sdpa_reduce" not in names
 
 

@@ -288,3 +288,18 @@ def test_ws_soak_is_bit_stable(device, pin, monkeypatch):
         prog.close()
     want = eager.run_eager(case, device)
     eager.assert_close(first.reshape(want.shape), want, case.rtol, case.atol, "ws after the soak vs eager")
+
+
+@pytest.mark.parametrize("flags", ["-DEMH_STAMP=1", "-DEMH_STAMP=2", "-DEMH_ABLATE=1", "-DEMH_ABLATE=2", "-DEMH_ABLATE=3", "-DEMH_ABLATE=4"])
+def test_measurement_switches_build(launcher_lib, flags, monkeypatch):
+    """The phase stamps (shader clock, summed by wave 0 of workgroup 0) and the ablations ``microbench --flash`` reads are
+    compile-time switches of the emitted text: each must build, without spills, for both forms."""
+    from deplodock_amd.backend.hip import hiprtc
+
+    monkeypatch.setenv("EMMY_HIPRTC_FLAGS", flags)
+    for sp in (False, True):
+        body = _body(waves=2, kvs=4 if sp else 2, pair=True)
+        body.ws, body.sp = not sp, sp
+        op = emit_flash_ws(body, "k_sw")
+        assert "__builtin_readcyclecounter" in op.kernel_source and "EMH_ABLATE" in op.kernel_source
+        assert hiprtc.spilled_vgprs(op.kernel_source, "k_sw") == 0

@@ -298,6 +298,26 @@ def test_c4_wide_heads_and_fp16(device, d, dtype, causal):
     eager.assert_close(ours, exact, 2e-2, 2e-2, f"sdpa d={d} {dtype} causal={causal} vs fp32 eager")
 
 
+@pytest.mark.parametrize("d,causal,dtype", [(40, True, torch.bfloat16), (80, True, torch.bfloat16), (96, False, torch.float16), (112, True, torch.bfloat16), (24, False, torch.bfloat16), (192, True, torch.bfloat16), (8, True, torch.float16)])
+def test_c4_head_dims_between_the_kernels_widths_are_padded_not_decomposed(device, d, causal, dtype):
+    """A 16-bit head_dim of whole 16-byte chunks that is not 64 / 128 / 256 runs on the flash kernel at the next width up:
+    the missing columns of q count as zeros, k's and v's are never looked at, the output's are not stored.  Neighbouring
+    memory is checked too: the output buffer is a window of a larger one whose other bytes must stay as they were."""
+    torch.manual_seed(16)
+    q, k, v = (torch.randn(2, h, 150, d).to(dtype) for h in (4, 2, 2))
+    case = eager.Case("pad", eager.Sdpa(causal), (q, k, v), 2e-2, 2e-2)
+    ours, want, compiled = run_case(case, device)
+    ops = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+    assert len(ops) == 1 and f"#define DR {d}\n" in ops[0].kernel_source
+    eager.assert_close(ours, want, 2e-2, 2e-2, f"sdpa d={d} {dtype} causal={causal} vs eager")
+    exact = nn.functional.scaled_dot_product_attention(q.to(device).float(), k.to(device).float(), v.to(device).float(), is_causal=causal, enable_gqa=True)
+    eager.assert_rows_within_baseline(ours, want, exact, 1.5, f"sdpa d={d} rows vs fp32 eager")
+    # values placed so that a wrong column would show: v[..., j] = j
+    vcol = torch.arange(d, dtype=torch.float32).expand_as(v).to(dtype)
+    o2, w2, _ = run_case(eager.Case("cols", eager.Sdpa(causal), (q, k, vcol), 2e-2, 2e-2), device)
+    eager.assert_close(o2, w2, 2e-2, 2e-2, f"sdpa d={d} column-coded V")
+
+
 @pytest.mark.parametrize("pin", ["w4/kv64/s2", "w2/kv64/s1", "w1/kv64/s2", "w2/kv128/s2", "w2/kv64/s2/p"])
 def test_c4_head_dim_64_workgroup_shapes(device, pin, monkeypatch):
     monkeypatch.setenv("EMMY_FLASH", pin)
@@ -1248,16 +1268,17 @@ _DECOMPOSED_ATTENTION = {
     "mask_per_batch_keys": (_FusedAttention(), torch.float32, [(2, 4, 40, 32)] * 3, lambda: torch.randn(2, 1, 1, 40)),
     "token_major": (_TokenMajorAttention(), torch.float32, [(1, 128, 16, 128), (1, 128, 8, 128), (1, 128, 8, 128)], None),
     "repeat_kv": (_RepeatKvAttention(), torch.float32, [(2, 8, 64, 64), (2, 2, 64, 64), (2, 2, 64, 64)], None),
-    "bf16_head_dim_32": (_FusedAttention(is_causal=True), torch.bfloat16, [(2, 4, 64, 32)] * 3, None),
-    "bf16_head_dim_96": (_FusedAttention(), torch.bfloat16, [(2, 4, 50, 96)] * 3, None),
+    # 16-bit rows that are not whole 16-byte chunks (the flash kernel pads whole chunks only)
+    "bf16_head_dim_36": (_FusedAttention(is_causal=True), torch.bfloat16, [(2, 4, 64, 36)] * 3, None),
+    "bf16_head_dim_100": (_FusedAttention(), torch.bfloat16, [(2, 4, 50, 100)] * 3, None),
 }
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("case", sorted(_DECOMPOSED_ATTENTION))
 def test_attention_outside_the_flash_kernel(device, case):
-    """The fused attention op on fp32 operands (what the reference's perf suite runs), or with a head_dim the flash
-    kernel has no tiling for: two batched MFMA contractions (fp32 atoms keep fp32 accuracy) around loop-nest stages,
+    """The fused attention op on fp32 operands (what the reference's perf suite runs), or with a 16-bit head_dim the flash
+    kernel cannot pad to one of its widths: two batched MFMA contractions (fp32 atoms keep fp32 accuracy) around loop-nest stages,
     against eager in float64."""
     mod, dtype, shapes, mask = _DECOMPOSED_ATTENTION[case]
     torch.manual_seed(41)
