@@ -31,6 +31,10 @@ def flash_head_dim(d: int) -> int | None:
     return next((w for w in FLASH_HEAD_DIMS if w >= d), None)
 
 
+#: largest scores tensor ``[batch..., heads, queries, keys]`` the decomposed route writes to device memory
+SCORES_LIMIT_BYTES = 8 * 2**30
+
+
 class AttentionShapeError(ValueError):
     pass
 
@@ -97,6 +101,14 @@ def _decompose(g: Graph, node: Node, undo_repeat) -> list[Node]:
     # kernel 1: scores[..., h, i, j] = sum_d q[..., h, i, d] * k[..., h / group, j, d] * scale (+ mask)
     scores_id = f"{nid}__scores"
     scores_shape = (*lead, hq, sq, skv)
+    # This route materialises the scores (the flash kernel, which streams them, takes 16-bit operands only): bounded, so
+    # that a long fp32 sequence is refused with a message instead of asking the allocator for the memory.
+    scores_bytes = math.prod(scores_shape) * dtype.nbytes
+    if scores_bytes > SCORES_LIMIT_BYTES:
+        raise AttentionShapeError(
+            f"sdpa: the decomposed route (operands wider than 16 bits, or rows that are not whole 16-byte chunks) would materialise {scores_bytes / 2**30:.1f} GiB of scores "
+            f"{scores_shape}; the limit is {SCORES_LIMIT_BYTES / 2**30:.0f} GiB — run the module in bf16 / fp16 (streamed by the flash kernel) or on shorter sequences"
+        )
     head = [L.Load("c_scale", "scale", (L.Lit(0),))]
     scalars = {"scale": scale}
     loads, inputs = ["q", "k"], [q_id, k_id]

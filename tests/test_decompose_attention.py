@@ -110,3 +110,13 @@ def test_grouped_heads_without_the_flag_are_refused():
             n.op.enable_gqa = False
     with pytest.raises(FusionError, match="enable_gqa"):
         HipBackend().compile(g)
+
+
+def test_a_scores_tensor_beyond_the_limit_is_refused_with_a_message():
+    """The decomposed route writes the scores to device memory; a shape whose scores exceed the limit is refused when
+    the module is compiled, not when the runtime asks for the memory."""
+    from deplodock_amd.passes.fuse import FusionError
+
+    q = torch.zeros(1, 32, 16384, 8)
+    with pytest.raises(FusionError, match="32.0 GiB of scores"):
+        HipBackend().compile(trace_module(_Sdpa(is_causal=True).eval(), (q, q, q)))
