@@ -273,7 +273,27 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
             for p in progs:
                 p.close()
 
-    def bench(make_case, label: str, bound: str, check: bool = True, cold: bool = False, whole_model: bool = False) -> None:
+    def vendor_us(case) -> float:
+        """µs per call of PyTorch eager on the GPU for the same module and inputs — for a linear that is the vendor
+        library's GEMM (hipBLASLt through torch): back-to-back calls in one event window, best of five windows."""
+        gm = case.module.to(device)
+        args = tuple(t.to(device) for t in case.inputs)
+        with torch.no_grad():
+            for _ in range(5):
+                gm(*args)
+            torch.cuda.synchronize()
+            best = float("inf")
+            for _ in range(5):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(20):
+                    gm(*args)
+                e1.record()
+                torch.cuda.synchronize()
+                best = min(best, e0.elapsed_time(e1) * 1e3 / 20)
+        return best
+
+    def bench(make_case, label: str, bound: str, check: bool = True, cold: bool = False, whole_model: bool = False, vendor: bool = False) -> None:
         if only is not None and only not in label:
             return
         case = make_case()
@@ -298,6 +318,14 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
                     err, base = float((ours.reshape(exact.shape) - exact).abs().mean()), float((half - exact).abs().mean())
                     if not err <= 1.5 * base:
                         raise AssertionError(f"{label}: mean |ours - fp32 eager| {err:.4g} exceeds 1.5 x mean |16-bit eager - fp32 eager| {base:.4g}")
+                    # and per row (a single bad token row does not move the mean): relative L2 distance from the fp32
+                    # run, bounded by 1.5 x the worst row of 16-bit eager
+                    rows_ = exact.reshape(-1, exact.shape[-1])
+                    norm = rows_.norm(dim=-1).clamp_min(1e-12)
+                    ours_rows = (ours.reshape(rows_.shape) - rows_).norm(dim=-1) / norm
+                    half_rows = (half.reshape(rows_.shape) - rows_).norm(dim=-1) / norm
+                    if not float(ours_rows.max()) <= 1.5 * float(half_rows.max()):
+                        raise AssertionError(f"{label}: worst row {float(ours_rows.max()):.4g} from the fp32 run exceeds 1.5 x 16-bit eager's worst row {float(half_rows.max()):.4g}")
                     times = []
                     for i in range(13):
                         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -343,6 +371,11 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
             row["eager_gpu_us"] = round(eager_us, 1)
             row["tokens_per_s"] = round(int(case.inputs[0].numel()) / (us * 1e-6))
             row.pop("per_kernel_us", None)  # (142 entries: the five kernels of a layer are the C5 row's)
+        if vendor:
+            v_us = vendor_us(case)
+            row["vendor_us"] = round(v_us, 2)  # PyTorch eager on the same GPU: the vendor library's kernel for this problem
+            if bound == "mfma":
+                row["vendor_frac"] = round(case.algo_flops / (v_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
         if cpu and not whole_model:
             row["cpu_us"] = round(_cpu_us(case), 1)
         rows.append(row)
@@ -352,12 +385,13 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
     bench(wl.softmax_case, "C2 softmax fp32 [1,28,2048,2048]", "hbm")
     for m in (1, 16, 128):
         bench(lambda m=m: wl.linear_case(m=m), f"C3 linear bf16 M={m} K=1024 N=3072", "hbm", cold=True)
-    bench(lambda: wl.linear_case(m=2048), "C3 linear bf16 M=2048 K=1024 N=3072", "mfma")
-    if extended:
-        bench(lambda: wl.linear_case(m=4096, k=4096, n=4096), "C3x linear bf16 M=4096 K=4096 N=4096", "mfma")
-    bench(wl.sdpa_case, "C4 causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
+    bench(lambda: wl.linear_case(m=2048), "C3 linear bf16 M=2048 K=1024 N=3072", "mfma", vendor=True)
+    bench(lambda: wl.linear_case(m=4096, k=4096, n=4096), "C3x linear bf16 M=4096 K=4096 N=4096", "mfma", vendor=True)
+    bench(wl.sdpa_case, "C4 causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma", vendor=True)
+    bench(lambda: wl.sdpa_decode_case(q_len=1, kv_len=32768), "C4d decode GQA sdpa bf16 16q/8kv q=1 kv=32768 d=128 (key slices + combine)", "hbm", vendor=True)
     if extended:
         bench(lambda: wl.sdpa_case(causal=False), "C4x non-causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
+        bench(lambda: wl.sdpa_case(s=8192), "C4xx causal GQA sdpa bf16 16q/8kv S=8192 d=128", "mfma", vendor=True)
     bench(lambda: wl.qwen3_block_case(seq=512), "C5 qwen3-0.6B block bf16 S=512", "mfma")
     bench(lambda: wl.qwen3_model_case(seq=512), "M qwen3-0.6B whole model (28 layers, random weights) bf16 S=512, token ids -> last hidden state", "mfma", whole_model=True)
     return rows

@@ -88,6 +88,19 @@ def sdpa_case(b: int = 1, hq: int = 16, hkv: int = 8, s: int = 2048, d: int = 12
     )  # fmt: skip
 
 
+def sdpa_decode_case(q_len: int = 1, kv_len: int = 32768, b: int = 1, hq: int = 16, hkv: int = 8, d: int = 128, seed: int = 0) -> Case:
+    """Decode-size attention over a long cache: ``q_len`` new queries see all ``kv_len`` keys (no mask); bound by the K/V
+    stream (the algorithmic bytes are K, V, q and the output once)."""
+    torch.manual_seed(seed)
+    q = torch.randn(b, hq, q_len, d).bfloat16()
+    k = torch.randn(b, hkv, kv_len, d).bfloat16()
+    v = torch.randn(b, hkv, kv_len, d).bfloat16()
+    return Case(
+        f"sdpa_decode_{b}x{hq}x{hkv}x{q_len}x{kv_len}x{d}", Sdpa(False).eval(), (q, k, v), BF16_RTOL, 2e-2,
+        algo_bytes=(2 * b * hq * q_len * d + 2 * b * hkv * kv_len * d) * 2, algo_flops=4 * b * hq * d * q_len * kv_len,
+    )  # fmt: skip
+
+
 class Qwen3Block(nn.Module):
     """Wraps ``transformers``' ``Qwen3DecoderLayer`` (built from a local config,
     no download) so it takes ``(x, cos, sin)`` and returns the hidden state."""
@@ -245,4 +258,4 @@ def normed_rope_attention_case(hidden: int = 256, q_heads: int = 4, kv_heads: in
 
 
 __all__ = ["Case", "FP32_RTOL", "BF16_RTOL", "Sdpa", "Qwen3Block", "NormedRopeAttention", "rms_norm_case", "softmax_case", "linear_case",
-           "sdpa_case", "qwen3_block_case", "normed_rope_attention_case"]  # fmt: skip
+           "sdpa_case", "sdpa_decode_case", "qwen3_block_case", "normed_rope_attention_case"]  # fmt: skip
