@@ -157,21 +157,24 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   // slot q % CPR = tid % CPR.  CHUNKS is a multiple of NT, so g and the row offset
   // of iteration i are compile-time.
   const int st_row = tid / CPR, st_pos = tid % CPR;
-  const ELT* gk_lane = kbase + (long)st_row * K_SS;
-  const ELT* gv_lane = vbase + (long)st_row * V_SS;
-  const int dst_lane = (tid - lane) * 16;
   const unsigned lds0 = emh_lds_addr(lds);
   const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);  // wave-uniform by construction; says so to the compiler
-  // A request whose key block lies wholly inside the sequence is a scalar base (the head's K or V plane, moved
-  // along the keys per step in scalar registers), a loop-invariant 32-bit lane offset and a scalar LDS target:
-  // no vector arithmetic per request.  Only a block that hangs over the end clamps its rows per lane.
+  // A request is a scalar base (the head's K or V plane, moved along the keys per step in scalar registers), a
+  // 32-bit lane offset and a scalar LDS target: no vector arithmetic per request.  The lane offsets are the same
+  // for every step whose keys all lie inside the sequence.  Only the last step can hang over the end: before its
+  // requests are issued EMH_CLAMP_K / _V(st) recomputes the offsets once with each lane's row clamped to the last
+  // key (a duplicate row the score mask discards), so the requests themselves never branch on the length.
   unsigned kvo[PER_T], vvo[PER_T];
-  #pragma unroll
-  for (int i = 0; i < PER_T; ++i) {
-    const int g_ = (i * NT) / CHUNKS, ro_ = ((i * NT) % CHUNKS) / CPR;
-    kvo[i] = (unsigned)((g_ * BKV + ro_ + st_row) * K_SS + emh_gchunk(emh_kswz(st_row + ro_, st_pos)) * 8) * 2u;
-    vvo[i] = (unsigned)((g_ * BKV + ro_ + st_row) * V_SS + emh_gchunk(emh_vswz(st_row + ro_, st_pos)) * 8) * 2u;
-  }
+  #define EMH_LANE_OFFSETS(off_, stride_, swz_, lim_) \
+    _Pragma("unroll") for (int i = 0; i < PER_T; ++i) { \
+      const int g_ = (i * NT) / CHUNKS, ro_ = ((i * NT) % CHUNKS) / CPR; \
+      const int row_ = g_ * BKV + ro_ + st_row; \
+      off_[i] = (unsigned)((row_ < (lim_) ? row_ : (lim_)) * (stride_) + emh_gchunk(swz_(st_row + ro_, st_pos)) * 8) * 2u; }
+  EMH_LANE_OFFSETS(kvo, K_SS, emh_kswz, 0x7fffffff)
+  EMH_LANE_OFFSETS(vvo, V_SS, emh_vswz, 0x7fffffff)
+  #define EMH_RAGGED(st) (!WHOLE_STEPS && ((st) + 1) * (KVS * BKV) > SKV)
+  #define EMH_CLAMP_K(st) if (EMH_RAGGED(st)) { const int lim_ = SKV - 1 - (st) * (KVS * BKV); EMH_LANE_OFFSETS(kvo, K_SS, emh_kswz, (lim_ < 0 ? 0 : lim_)) }
+  #define EMH_CLAMP_V(st) if (EMH_RAGGED(st)) { const int lim_ = SKV - 1 - (st) * (KVS * BKV); EMH_LANE_OFFSETS(vvo, V_SS, emh_vswz, (lim_ < 0 ? 0 : lim_)) }
   // EMH_STEP_BASES(st) names the scalar parts of the requests of step st once (K and V plane bases moved to the
   // step's keys, the ring slots' LDS addresses); EMH_STAGE_K / _V(st, i) then issue request i against them.
   #define EMH_STEP_BASES(tag, st) \
@@ -179,16 +182,11 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       const unsigned char* vb##tag = emh_uniform((const unsigned char*)vbase + (long)(st) * (KVS * BKV) * V_SS * 2); \
       const unsigned kl##tag = emh_uniform(lds0 + EMH_SLOT(st, RK) * SETB + wave_u * 1024); \
       const unsigned vl##tag = emh_uniform(lds0 + V_RING + EMH_SLOT(st, RV) * SETB + wave_u * 1024);
-  #define EMH_STAGE_ONE(st, i, sb_, lb_, base_, stride_, off_, swz_, ldo_) { \
-      const int g_ = ((i) * NT) / CHUNKS, ro_ = (((i) * NT) % CHUNKS) / CPR; \
-      if (SKV % (KVS * BKV) == 0 || ((st) * KVS + g_ + 1) * BKV <= SKV) { \
-        emh_dma16s(sb_, off_[i], (lb_) + g_ * KBYTES + (((i) * NT) % CHUNKS) * 16); \
-      } else { \
-        long krow_ = (long)((st) * KVS + g_) * BKV + ro_ + st_row; \
-        if (krow_ > SKV - 1) krow_ = SKV - 1; \
-        emh_dma16((base_) + krow_ * (stride_) + emh_gchunk(swz_(st_row + ro_, st_pos)) * 8, lds + (ldo_) + g_ * KBYTES + (((i) * NT) % CHUNKS) * 16 + dst_lane); } }
-  #define EMH_STAGE_K(tag, st, i) EMH_STAGE_ONE(st, i, kb##tag, kl##tag, kbase, K_SS, kvo, emh_kswz, EMH_SLOT(st, RK) * SETB)
-  #define EMH_STAGE_V(tag, st, i) EMH_STAGE_ONE(st, i, vb##tag, vl##tag, vbase, V_SS, vvo, emh_vswz, V_RING + EMH_SLOT(st, RV) * SETB)
+  #define EMH_STAGE_ONE(st, i, sb_, lb_, off_) { \
+      const int g_ = ((i) * NT) / CHUNKS; \
+      emh_dma16s(sb_, off_[i], (lb_) + g_ * KBYTES + (((i) * NT) % CHUNKS) * 16); }
+  #define EMH_STAGE_K(tag, st, i) EMH_STAGE_ONE(st, i, kb##tag, kl##tag, kvo)
+  #define EMH_STAGE_V(tag, st, i) EMH_STAGE_ONE(st, i, vb##tag, vl##tag, vvo)
   // Requests are issued between MFMAs, spread evenly over a chain of NQ_SLOTS of them (request i behind MFMA
   // number EMH_SLOT_OF(i)): they trickle into the memory pipeline instead of arriving as one burst from every wave.
   #define NQ_SLOTS ((BKV / 32) * (D / 16))
@@ -237,10 +235,12 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   // and a K block has two steps to land.  Otherwise (two slots each): K(st + 1) and V(st + 1) are requested
   // together during step st and both are waited for at its end.
   // Issue order: K0 V0 [K1] | step 0: V1, K2 | step 1: V2, K3 | ...
+  EMH_CLAMP_K(0)
+  EMH_CLAMP_V(0)
   EMH_STAGE_ALL_K(0);
   EMH_STAGE_ALL_V(0);
   if (DEEP) {
-    if (1 < nsteps) EMH_STAGE_ALL_K(1);
+    if (1 < nsteps) { EMH_CLAMP_K(1) EMH_STAGE_ALL_K(1); }
     EMH_LAND((int)(1 < nsteps));
   } else {
     EMH_LAND(0);
@@ -280,6 +280,9 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
     const bool active = (jt < ntiles) && (!CAUSAL || (k0 <= qw0_k + 31));
     EMH_STEP_BASES(1, st + 1)
     EMH_STEP_BASES(2, st + 2)
+    // this step requests V(st + 1) and K(st + 1) (DEEP: K(st + 2)); a step past the sequence's last one is never requested
+    EMH_CLAMP_V(st + 1)
+    if (DEEP) { EMH_CLAMP_K(st + 2) } else { EMH_CLAMP_K(st + 1) }
     (void)kb2; (void)kl2; (void)vb2; (void)vl2; (void)kb1; (void)kl1;
     if (!active) {
       if (more) { EMH_STAGE_ALL_V(st + 1); if (!DEEP) EMH_STAGE_ALL_K(st + 1); }
@@ -661,6 +664,8 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "SQ": c_value(symf.get("q_len", body.q_len)),
         **({"SKV_ALL": body.kv_len, "KV_CHUNK": kv_chunk, "BATCH": body.batch} if split > 1 else {"SKV": c_value(symf.get("kv_len", body.kv_len))}),
         "KV_CTAS": split,
+        # every key step lies inside the sequence (or the slice of it), known when the kernel is built
+        "WHOLE_STEPS": 1 if "kv_len" not in symf and body.kv_len % (kvs * BKV) == 0 else 0,
         "OUT_T": "float" if split > 1 else rt.type_name(body.dtype.name),
         "HQ": body.q_heads,
         "GROUP": body.q_heads // body.kv_heads,
