@@ -151,6 +151,37 @@ class HipBackend(Backend):
 
     # -- binding ------------------------------------------------------------
     @staticmethod
+    def _bind_prefix_tables(compiled: Graph, data: dict, traced: dict) -> None:
+        """Constants of a runtime-int lowering whose rows follow the symbolic axis (position tables computed when the
+        module was traced; ``passes.symbolic._prefix_table``): bind the leading rows the inputs' size needs.  A size
+        beyond the largest table held re-traces the module once at (at least) twice that size and keeps the larger
+        tables for every later call."""
+        tables = [(nid, n.hints["prefix_table"], n.hints["sym_shape"]) for nid, n in compiled.nodes.items() if "prefix_table" in n.hints and nid not in data and nid in traced]
+        if not tables:
+            return
+        spec, name = compiled.dynamic, compiled.symbolic
+        size = None
+        for nid, axes in zip(compiled.inputs, spec.input_axes):
+            for dim, sym in (axes or {}).items():
+                if sym == name and nid in data:
+                    size = int(data[nid].shape[dim])
+        if size is None:
+            size = int(spec.hints[name])  # synthetic inputs: the traced size
+        if any(traced[nid].shape[d] < shape[d].at({name: size}) for nid, d, shape in tables):
+            from deplodock_amd.passes.fuse import fuse
+
+            if not hasattr(spec, "retrace"):
+                raise ValueError(f"{name} = {size} needs more rows of {[t[0] for t in tables]} than the graph holds and the module is not here to re-trace: pass the tables in input_data")
+            held = max(int(spec.hints[name]), getattr(compiled, "prefix_table_size", 0))
+            grown = max(size, 2 * held)
+            values = fuse(spec.retrace({name: grown})).constant_values
+            for nid, _d, _shape in tables:
+                traced[nid] = values[nid]
+            compiled.prefix_table_size = grown
+        for nid, d, shape in tables:
+            data[nid] = traced[nid].narrow(d, 0, shape[d].at({name: size})).contiguous()
+
+    @staticmethod
     def bind(compiled: Graph, input_data: dict | None) -> dict:
         """``input_data`` completed with the traced parameter values of every
         constant it does not override (stacked constants are assembled here)."""
@@ -158,6 +189,8 @@ class HipBackend(Backend):
 
         data = dict(input_data or {})
         traced = getattr(compiled, "constant_values", {})
+        if getattr(compiled, "symbolic", None) is not None:
+            HipBackend._bind_prefix_tables(compiled, data, traced)
         for nid, _op in compiled.constant_ops():
             if nid in data:
                 continue

@@ -15,10 +15,13 @@ against the buffer before anything is launched.
 
 from __future__ import annotations
 
+from dataclasses import dataclass
+
 from deplodock_amd.context import Context
 from deplodock_amd.emit import prelude
 from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir.hip import HipOp
+from deplodock_amd.ir.sym import Affine, c_value, param_name
 from deplodock_amd.ir.tile import IndexRows, StridedCopy
 from deplodock_amd.render_target import rt
 
@@ -131,7 +134,12 @@ def emit_strided_copy(body: StridedCopy, name: str, ctx: Context = Context()) ->
 
 def emit_index_rows(body: IndexRows, name: str, ctx: Context = Context()) -> HipOp:
     """One lane per result element, consecutive along ``inner``: the row index is read once per element (it sits in
-    cache for the whole row) and clamped into the table, so no value of ``idx`` can send a load outside ``src``."""
+    cache for the whole row) and clamped into the table, so no value of ``idx`` can send a load outside ``src``.
+
+    Symbolic form (``body.sym``): the number of looked-up rows ``count`` is an expression over the kernel's trailing
+    ``int`` parameter (token ids ``[batch, seq_len]`` into an embedding table); the table itself never follows the
+    axis.  The 32-bit index arithmetic then bounds the result at run time: a launch whose result would not fit is
+    refused by the grid factor (``_IndexRowsGrid``) before anything runs."""
     total = body.outer * body.count * body.inner
     if min(body.outer, body.n, body.inner, body.count) < 1:
         raise LoweringError("index rows: empty operand")
@@ -139,13 +147,19 @@ def emit_index_rows(body: IndexRows, name: str, ctx: Context = Context()) -> Hip
         raise LoweringError("index rows: index arithmetic is 32-bit; the tensor is too large")
     if body.idx_dtype.name not in ("i32", "i64"):
         raise LoweringError(f"index rows: indices must be int32 or int64, got {body.idx_dtype}")
+    sym = getattr(body, "sym", None)
+    symf = sym.fields if sym is not None else {}
+    if symf and set(symf) != {"count"}:
+        raise LoweringError(f"index rows: {sorted(symf)} cannot follow a symbolic axis (only the number of looked-up rows can)")
+    count_c = f"(unsigned){c_value(symf['count'])}" if symf else f"{body.count}u"
     T, IT = rt.type_name(body.dtype.name), rt.type_name(body.idx_dtype.name)
     o: list[str] = []
     a = o.append
-    a(f'extern "C" __global__ __launch_bounds__(256) void {name}(const {T}* __restrict__ src, const {IT}* __restrict__ idx, {T}* __restrict__ dst) {{')
+    a(f'extern "C" __global__ __launch_bounds__(256) void {name}(const {T}* __restrict__ src, const {IT}* __restrict__ idx, {T}* __restrict__ dst{f", int {param_name(sym.name)}" if symf else ""}) {{')
     a("  const unsigned lin = blockIdx.x * 256u + threadIdx.x;")
-    a(f"  if (lin >= {total}u) return;")
-    a(f"  const unsigned i = lin % {body.inner}u, j = (lin / {body.inner}u) % {body.count}u, o = lin / {body.inner * body.count}u;")
+    a(f"  const unsigned count = {count_c};")
+    a(f"  if (lin >= {body.outer * body.inner}u * count) return;")
+    a(f"  const unsigned i = lin % {body.inner}u, j = (lin / {body.inner}u) % count, o = lin / ({body.inner}u * count);")
     a("  long long r = (long long)idx[j];")
     a(f"  r = r < 0 ? 0 : (r >= {body.n} ? {body.n - 1} : r);")
     a(f"  dst[lin] = src[(o * {body.n}u + (unsigned)r) * {body.inner}u + i];")
@@ -154,14 +168,30 @@ def emit_index_rows(body: IndexRows, name: str, ctx: Context = Context()) -> Hip
         kernel_source=prelude.header() + "\n".join(o) + "\n",
         kernel_name=name,
         arg_order=(body.src, body.idx, body.out),
-        grid=((-(-total // 256),), (1,), (1,)),
+        grid=((_IndexRowsGrid(symf["count"], body.outer * body.inner) if symf else -(-total // 256),), (1,), (1,)),
         block=((256,), (1,), (1,)),
         lds_bytes=0,
+        runtime_args=(sym.name,) if symf else (),
         comment="index rows",
         algo_bytes=body.algo_bytes(),
         algo_flops=0,
         knobs={"COPY": "index"},
     )
+
+
+@dataclass(frozen=True)
+class _IndexRowsGrid:
+    """Launch-time grid of a symbolic lookup: one lane per result element, refused when the element count leaves the
+    kernel's 32-bit index arithmetic."""
+
+    count: Affine
+    per_row: int
+
+    def __call__(self, env: dict) -> int:
+        total = self.count.at(env) * self.per_row
+        if total >= 1 << 31:
+            raise ValueError(f"index rows: {total} result elements at {env} do not fit the kernel's 32-bit index arithmetic")
+        return -(-total // 256)
 
 
 __all__ = ["emit_strided_copy", "emit_index_rows"]

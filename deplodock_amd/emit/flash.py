@@ -632,9 +632,9 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         if pair:
             raise LoweringError("flash: mirrored query-block pairs need a block count known when the kernel is built")
         for key in symf:
-            if key not in ("q_len", "kv_len") and not (key.split(".")[0] in ("q_strides", "k_strides", "v_strides", "o_strides") and key.split(".")[1] in ("0", "1", "2")):
+            if key not in ("q_len", "kv_len") and not (key.split(".")[0] in ("q_strides", "k_strides", "v_strides", "o_strides", "mask_strides") and key.split(".")[1] in ("0", "1", "2")):
                 raise LoweringError(f"flash: {key} cannot follow a symbolic axis")
-            if isinstance(symf[key], Affine) and "strides" in key and (symf[key].a % 8 or symf[key].b % 8):
+            if isinstance(symf[key], Affine) and "strides" in key and not key.startswith("mask_") and (symf[key].a % 8 or symf[key].b % 8):
                 raise LoweringError(f"flash: {key} = {symf[key]} does not keep 16-byte alignment at every size")
     if pair and not (body.causal and qblocks % 2 == 0):
         raise LoweringError("flash: pairing mirrored query blocks needs a causal mask and an even block count")
@@ -644,12 +644,9 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     if has_mask:
         if body.mask_dtype.name not in ("bf16", "f16", "f32"):
             raise LoweringError("flash: the mask must be a floating-point tensor")
-        if symf:
-            raise LoweringError("flash: a mask operand does not combine with symbolic lengths")
         if body.scale == 0.0:
             raise LoweringError("flash: a mask with a zero scale is not supported")
-        # four keys per load (8 or 16 bytes) when every row of the mask starts on a four-element boundary
-        mask_vec = all(v % 4 == 0 for v in (*body.mask_strides, body.mask_offset))
+        m_strides = [symf.get(f"mask_strides.{i}", v) for i, v in enumerate(body.mask_strides)]
     defs = {
         "KNAME": name,
         "NT": NT,
@@ -674,8 +671,11 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         "SYM_PARAM": f", int {param_name(sym.name)}" if symf else "",
         "HAS_MASK": 1 if has_mask else 0,
         "MASK_PARAM": f", const {rt.type_name(body.mask_dtype.name)}* __restrict__ Mp" if has_mask else "",
-        **({"MELT": rt.type_name(body.mask_dtype.name), "MVEC4": rt.vector_type(body.mask_dtype.name, 4)[0], "MASK_VEC": 1 if mask_vec else 0,
-            "M_SB": body.mask_strides[0], "M_SH": body.mask_strides[1], "M_SS": body.mask_strides[2], "M_OFF": body.mask_offset,
+        **({"MELT": rt.type_name(body.mask_dtype.name), "MVEC4": rt.vector_type(body.mask_dtype.name, 4)[0],
+            # four keys per load (8 or 16 bytes) when every row of the mask starts on a four-element boundary: known when
+            # the kernel is built for static strides, one scalar test per launch when a stride follows a symbolic length
+            "MASK_VEC": "((((M_SB) | (M_SH) | (M_SS) | (M_OFF)) & 3) == 0)" if any(isinstance(v, Affine) for v in m_strides) else int(all(v % 4 == 0 for v in (*m_strides, body.mask_offset))),
+            "M_SB": c_value(m_strides[0]), "M_SH": c_value(m_strides[1]), "M_SS": c_value(m_strides[2]), "M_OFF": body.mask_offset,
             "INV_SCALE": float_literal(1.0 / body.scale)} if has_mask else {}),
         "PAIR": 1 if pair else 0,
         # steps in parity pairs (static ring slots) unless the whole key range is one or two steps

@@ -14,8 +14,9 @@ from __future__ import annotations
 import dataclasses
 
 from deplodock_amd.graph import Graph
+from deplodock_amd.ir.base import ConstantOp
 from deplodock_amd.ir.sym import Affine, SymSpec
-from deplodock_amd.ir.tile import Contraction, Flash, Map, RowReduce, TileOp
+from deplodock_amd.ir.tile import Contraction, Flash, IndexRows, Map, RowReduce, TileOp
 
 
 class SymbolicError(ValueError):
@@ -26,8 +27,11 @@ class SymbolicError(ValueError):
 _ALLOWED = {
     RowReduce: {"rows", "row_operands.*.mod"},
     Contraction: {"m", "row_epilogue.row_operands.*.mod"},
-    Flash: {"q_len", "kv_len", "q_strides.*", "k_strides.*", "v_strides.*", "o_strides.*"},  # the batch stride of a [B, H, S, D] tensor follows S
+    # the batch stride of a [B, H, S, D] tensor follows S; so does the row stride of a mask [.., S, S] (its head and batch
+    # strides are quadratic in S unless the mask is broadcast over them, and a quadratic field is refused by the fit)
+    Flash: {"q_len", "kv_len", "q_strides.*", "k_strides.*", "v_strides.*", "o_strides.*", "mask_strides.*"},
     Map: {"numel"},
+    IndexRows: {"count"},  # token ids [batch, seq_len] into a table that does not follow the axis
 }
 
 
@@ -72,6 +76,25 @@ def _walk(objs: list, path: str, pattern: str, allowed: set, name: str, sizes: l
     raise SymbolicError(f"{what}.{path} depends on {name} ({[o for o in objs]}), which a runtime int cannot express")
 
 
+def _prefix_table(nid: str, sym_shape: tuple, values: list, name: str) -> int:
+    """A constant whose shape follows the axis is a table computed from the positions when the module was traced (a
+    rotary embedding's cos / sin rows).  One compilation can serve every size only if the table at a smaller size is
+    the leading rows of the table at a larger one, laid out so that those rows are a prefix of the memory: exactly one
+    dim follows the axis, every dim before it is 1, and the traced values agree on their common rows.  Returns that
+    dim; the runtime then binds the leading rows of the largest table it has and re-traces for a larger one."""
+    dims = [i for i, d in enumerate(sym_shape) if isinstance(d, Affine)]
+    if len(dims) != 1 or any(d != 1 for d in sym_shape[: dims[0]]) or sym_shape[dims[0]].a < 1:
+        raise SymbolicError(f"constant {nid!r} of shape {sym_shape} follows {name} in more than its leading dim")
+    if any(v is None for v in values):
+        raise SymbolicError(f"constant {nid!r} follows {name} and has no traced value to compare across sizes")
+    d = dims[0]
+    for v in values[1:]:
+        small, large = (values[0], v) if values[0].shape[d] <= v.shape[d] else (v, values[0])
+        if small.dtype != large.dtype or not bool((large.narrow(d, 0, small.shape[d]) == small).all()):
+            raise SymbolicError(f"constant {nid!r} follows {name} and its rows at one size are not the leading rows at a larger size")
+    return d
+
+
 def symbolize(tiles: list[Graph], name: str, sizes: list[int]) -> Graph:
     """Annotate the tile graph of ``sizes[0]`` (the traced size): every ``TileOp`` body gets ``sym`` (a
     ``SymSpec``), every node ``hints['sym_shape']`` (its shape with ``Affine`` entries).  ``tiles`` are the fused,
@@ -90,6 +113,8 @@ def symbolize(tiles: list[Graph], name: str, sizes: list[int]) -> Graph:
         sym_shape = tuple(d[0] if len(set(d)) == 1 else _fit(name, sizes, list(d), f"{nid}.shape") for d in zip(*shapes))
         if any(isinstance(d, Affine) for d in sym_shape):
             node.hints["sym_shape"] = sym_shape
+            if isinstance(node.op, ConstantOp):
+                node.hints["prefix_table"] = _prefix_table(nid, sym_shape, [getattr(t, "constant_values", {}).get(nid) for t in tiles], name)
         # hints that carry views (logical shapes / strides over a buffer) must not depend on the axis either,
         # except through the shape entries the program resolves per launch
         if isinstance(node.op, TileOp):

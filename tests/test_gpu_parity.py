@@ -5,6 +5,8 @@ library.  Tolerances: fp32 rtol 1e-5 (plus a stated absolute floor), bf16 rtol
 
 from __future__ import annotations
 
+import copy
+
 import numpy as np
 import pytest
 import torch
@@ -510,7 +512,7 @@ def test_dynamic_seq_len_per_size_variants_still_work(device):
     assert len(compiled.variants) == 2
 
 
-@pytest.mark.parametrize("which", ["rms_norm", "softmax", "silu_mul", "sdpa", "linear_bias", "linear_f32"])
+@pytest.mark.parametrize("which", ["rms_norm", "softmax", "silu_mul", "sdpa", "sdpa_masked", "embedding", "linear_bias", "linear_f32"])
 def test_runtime_int_kernels_of_every_family(device, which):
     """Row kernels (rows symbolic), a pointwise map (element count symbolic), attention on ``[B, H, S, D]`` operands
     (lengths and the batch stride symbolic) and a biased linear (rows symbolic), each compiled once and run at
@@ -537,6 +539,21 @@ def test_runtime_int_kernels_of_every_family(device, which):
         mod = eager.Sdpa(True).eval()
         make = lambda s: (torch.randn(2, 4, s, 128).bfloat16(), torch.randn(2, 2, s, 128).bfloat16(), torch.randn(2, 2, s, 128).bfloat16())  # noqa: E731
         dyn, tol = {"q": {2: "s"}, "k": {2: "s"}, "v": {2: "s"}}, (2e-2, 2e-2)
+    elif which == "sdpa_masked":
+        # a float bias [1, 1, S, S] broadcast over batch and heads, the way a whole-model trace passes its mask: only the
+        # row stride follows the axis; rows start on a four-element boundary at some sizes (vector loads) and not at others
+        mod = eager.MaskedSdpa().eval()
+
+        def make(s):
+            bias = torch.zeros(1, 1, s, s).masked_fill(torch.ones(s, s, dtype=torch.bool).triu(1), float("-inf")).bfloat16()
+            return (torch.randn(2, 4, s, 128).bfloat16(), torch.randn(2, 2, s, 128).bfloat16(), torch.randn(2, 2, s, 128).bfloat16(), bias)
+
+        dyn, tol = {"q": {2: "s"}, "k": {2: "s"}, "v": {2: "s"}, "mask": {2: "s", 3: "s"}}, (2e-2, 2e-2)
+    elif which == "embedding":
+        # token ids [batch, s] into a table that does not follow the axis: the looked-up row count does
+        mod = nn.Embedding(300, 64).eval()
+        make = lambda s: (torch.randint(0, 300, (2, s)),)  # noqa: E731
+        dyn, tol = {"input": {1: "s"}}, (0.0, 0.0)
     elif which == "linear_f32":
         # at the traced size the static fp32 lowering would split the reduction axis across workgroups (a kernel pair
         # with the row count baked in): the runtime-int form must stay unsplit and serve every size
@@ -1721,6 +1738,36 @@ def test_full_width_model_a_few_layers_deep(device):
         exact = gm.float()(case.inputs[0].to(device))
     eager.assert_mean_error_within_baseline(ours.reshape(exact.shape), half, exact, 1.5, "four-layer full-width model vs fp32 eager")
     eager.assert_rows_within_baseline(ours.reshape(exact.shape), half, exact, 2.0, "four-layer full-width model rows vs fp32 eager")
+
+
+@pytest.mark.gpu
+def test_whole_model_is_one_set_of_runtime_int_kernels_over_the_sequence_length(device):
+    """Token ids in, last hidden state out, with the sequence length symbolic: the embedding gather takes its row count
+    at run time like every other kernel of the model, so one compilation serves every length (the rotary table rows
+    and the attention lengths follow the same ``int``)."""
+    from deplodock_amd import workloads as wl
+
+    case = wl.qwen3_model_case(seq=64, layers=2)
+    be = HipBackend()
+    compiled = be.compile(trace_module(case.module, case.inputs, dynamic_shapes={"ids": {1: "seq_len"}}))
+    assert compiled.symbolic == "seq_len"
+    ops = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert len(ops) == 1 + 2 * 5 + 1 and all(op.runtime_args == ("seq_len",) for op in ops)
+    gm = copy.deepcopy(case.module).to(device)
+    for seq in (64, 200, 5):
+        torch.manual_seed(seq)
+        ids = torch.randint(3, 151000, (1, seq))
+        prog = be.program(compiled, {compiled.inputs[0]: ids.to(device)})
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            ours = prog.output_tensors()[compiled.outputs[0]].clone().float()
+        finally:
+            prog.close()
+        with torch.no_grad():
+            half = gm(ids.to(device)).float()
+            exact = copy.deepcopy(gm).float()(ids.to(device))
+        eager.assert_mean_error_within_baseline(ours.reshape(exact.shape), half, exact, 1.5, f"two-layer model at {seq} tokens vs fp32 eager")
 
 
 @pytest.mark.gpu

@@ -401,6 +401,37 @@ def test_a_symbolic_fp32_linear_never_takes_the_cross_workgroup_split(launcher_l
     assert getattr(pinned, "symbolic", None) is None and hasattr(pinned, "variants")
 
 
+def test_position_tables_folded_at_trace_time_follow_a_symbolic_length_as_prefixes(launcher_lib):
+    """Token ids in: the rotary cos / sin tables are constants computed from the positions when the model is traced,
+    so their row count follows the symbolic length.  Rows at one length are the leading rows at any longer one: the
+    lowering stays one set of runtime-int kernels (embedding gather included), and binding hands out the leading rows
+    of the largest table held, re-tracing once for a length beyond it."""
+    from deplodock_amd import workloads as wl
+    from deplodock_amd.passes.symbolic import SymbolicError, _prefix_table
+
+    case = wl.qwen3_model_case(seq=64, layers=1)
+    g = trace_module(case.module, case.inputs, dynamic_shapes={"ids": {1: "seq_len"}})
+    be = HipBackend()
+    compiled = be.compile(g)
+    assert compiled.symbolic == "seq_len"
+    ks = kernels(compiled)
+    assert ks[0].kernel_name.startswith("k_index_rows_") and all(k.runtime_args == ("seq_len",) for k in ks)
+    tables = [nid for nid, n in compiled.nodes.items() if "prefix_table" in n.hints]
+    assert len(tables) == 2 and all(compiled.nodes[t].output.shape == (1, 1, "seq_len", 128) for t in tables)
+    for size, held in ((5, None), (64, None), (200, 200), (130, 200), (500, 500)):
+        data = be.bind(compiled, {compiled.inputs[0]: torch.randint(3, 1000, (1, size))})
+        want = fuse(g.dynamic.retrace({"seq_len": size})).constant_values
+        assert all(torch.equal(data[t], want[t]) for t in tables), size
+        assert getattr(compiled, "prefix_table_size", None) == held
+    # what is not such a table is refused: values that change on the common rows, or an inner dim that follows the axis
+    a = Affine_("s", 1, 0)
+    with pytest.raises(SymbolicError, match="leading rows"):
+        _prefix_table("c", (1, a, 4), [torch.zeros(1, 3, 4), torch.ones(1, 5, 4), torch.zeros(1, 9, 4)], "s")
+    with pytest.raises(SymbolicError, match="leading dim"):
+        _prefix_table("c", (2, a, 4), [torch.zeros(2, 3, 4), torch.zeros(2, 5, 4), torch.zeros(2, 9, 4)], "s")
+    assert _prefix_table("c", (1, a, 4), [torch.arange(12.0).reshape(1, 3, 4), torch.arange(20.0).reshape(1, 5, 4), torch.arange(36.0).reshape(1, 9, 4)], "s") == 1
+
+
 def test_per_size_specialisation_remains_for_what_does_not_symbolise(launcher_lib):
     """With runtime-int kernels switched off (or a module whose kernel boundaries change with the size) the backend
     re-traces and re-lowers per distinct size and keeps an LRU of the results."""
