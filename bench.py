@@ -293,11 +293,13 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
                 best = min(best, e0.elapsed_time(e1) * 1e3 / 20)
         return best
 
-    def bench(make_case, label: str, bound: str, check: bool = True, cold: bool = False, whole_model: bool = False, vendor: bool = False) -> None:
+    def bench(make_case, label: str, bound: str, check: bool = True, cold: bool = False, whole_model: bool = False, vendor: bool = False, dynamic: dict | None = None) -> None:
         if only is not None and only not in label:
             return
         case = make_case()
-        compiled = be.compile(trace_module(case.module, case.inputs))
+        compiled = be.compile(trace_module(case.module, case.inputs, **({"dynamic_shapes": dynamic} if dynamic else {})))
+        if dynamic and getattr(compiled, "symbolic", None) is None:
+            raise AssertionError(f"{label}: expected one set of runtime-int kernels, got a per-size lowering")
         data = {n: t.to(device) for n, t in zip(compiled.inputs, case.inputs)}
         eager_us = None
         if whole_model:
@@ -393,6 +395,9 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
         bench(lambda: wl.sdpa_case(causal=False), "C4x non-causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
         bench(lambda: wl.sdpa_case(s=8192), "C4xx causal GQA sdpa bf16 16q/8kv S=8192 d=128", "mfma", vendor=True)
     bench(lambda: wl.qwen3_block_case(seq=512), "C5 qwen3-0.6B block bf16 S=512", "mfma")
+    # the same block compiled once for every sequence length (kernels that take the length as a run-time int), run at 512
+    bench(lambda: wl.qwen3_block_case(seq=512), "C5s qwen3-0.6B block bf16, runtime-int kernels over seq_len, at S=512", "mfma",
+          dynamic={"x": {1: "seq_len"}, "cos": {1: "seq_len"}, "sin": {1: "seq_len"}})  # fmt: skip
     bench(lambda: wl.qwen3_model_case(seq=512), "M qwen3-0.6B whole model (28 layers, random weights) bf16 S=512, token ids -> last hidden state", "mfma", whole_model=True)
     return rows
 
