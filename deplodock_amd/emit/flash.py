@@ -216,6 +216,18 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   #pragma unroll
   for (int r = 0; r < 16; ++r) oacc[t][r] = 0.0f;
   float m_ref = -1.0e30f, l_run = 0.0f;
+  // MSUM: the row sums come out of the matrix pipe.  An all-ones A operand against the P fragments the output MFMAs
+  // already hold gives, in every row of a 32 x 32 tile, the sum over the 32 keys of each query column (both lane
+  // halves included): two MFMAs per 32-key sub-block replace 16 adds per lane, and the sum is of the rounded
+  // probabilities the output itself is made of.
+  f32x16 lacc;
+  FRAG ones_f;
+  if (MSUM) {
+    #pragma unroll
+    for (int r = 0; r < 16; ++r) lacc[r] = 0.0f;
+    #pragma unroll
+    for (int e = 0; e < 8; ++e) ones_f[e] = (ELT)1.0f;
+  }
 
   // ds_read_b64_tr_b16: within 16 lanes, lane i receives element (i % 4) of the
   // 8-byte chunks addressed by lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12.  Lane i
@@ -381,6 +393,10 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         for (int t = 0; t < D / 32; ++t)
         #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+        if (MSUM) {
+          #pragma unroll
+          for (int r = 0; r < 16; ++r) lacc[r] *= alpha;
+        }
       }
       float psum = 0.0f;
       #pragma unroll
@@ -389,7 +405,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       for (int r = 0; r < 16; ++r) {
         const float p = EXP2(__builtin_fmaf(sacc[u][r], SCALE_LOG2, -m_ref));
         sacc[u][r] = p;
-        psum += p;
+        if (!MSUM) psum += p;
       }
       l_run += psum;
       #pragma unroll
@@ -399,6 +415,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         FRAG pf;
         #pragma unroll
         for (int t = 0; t < 8; ++t) pf[t] = (ELT)sacc[u][8 * s + t];
+        if (MSUM) lacc = MFMA(ones_f, pf, lacc, 0, 0, 0);
         #pragma unroll
         for (int dt = 0; dt < D / 32; ++dt) {
           u32x4 av;
@@ -429,6 +446,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
   // combines its share with the same exp-family merge the streaming loop uses,
   // scales by 1/l and puts the 16-bit result into the O tile in LDS, which leaves
   // through 16-byte stores of whole rows.  (The rings are dead after the loop's last barrier.)
+  if (MSUM) l_run = 0.5f * lacc[0];  // every element of the tile's column is the whole sum: half each, as the two lane halves are added below
   if (KVS > 1) {
     float* park = (float*)lds;
     float* pml = (float*)(lds + PARK_ML) + ((grp * WQ + wq) * 2) * 64 + lane;
@@ -678,6 +696,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
             "M_SB": c_value(m_strides[0]), "M_SH": c_value(m_strides[1]), "M_SS": c_value(m_strides[2]), "M_OFF": body.mask_offset,
             "INV_SCALE": float_literal(1.0 / body.scale)} if has_mask else {}),
         "PAIR": 1 if pair else 0,
+        "MSUM": 1 if body.mfma_sum else 0,
         # steps in parity pairs (static ring slots) unless the whole key range is one or two steps
         "PAIRSTEP": 1 if _PAIRSTEP and body.pair_steps and (bool(symf) or -(-(kv_chunk if split > 1 else body.kv_len) // (kvs * BKV)) > 2) else 0,
         "V_PRE": 1 if _V_PRE and (BKV // 32) * 2 * (D // 32) * 4 <= 32 else 0,  # the prefetched V fragments take at most 32 registers
@@ -719,7 +738,7 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         comment=f"flash Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} bkv={BKV} split={kvs} pair={int(pair)}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
-        knobs={"FLASH": f"w{waves}/kv{BKV}/s{kvs}" + ("/p" if pair else "") + ("/k3" if plan["deep"] else ""), **({"REDUCE": f"g{split}k"} if split > 1 else {})},
+        knobs={"FLASH": f"w{waves}/kv{BKV}/s{kvs}" + ("/p" if pair else "") + ("/k3" if plan["deep"] else "") + ("/ms" if body.mfma_sum else ""), **({"REDUCE": f"g{split}k"} if split > 1 else {})},
     )
 
 

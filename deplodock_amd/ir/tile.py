@@ -279,6 +279,7 @@ class Flash:
     pair: bool = False  # causal only: a workgroup takes query block b and its mirror QBLOCKS-1-b
     deep: bool = False  # a K ring of three slots (K blocks requested two steps ahead) beside a V ring of two
     pair_steps: bool = True  # key steps unrolled in pairs so ring slots are compile-time (the lowering clears it if that build spills)
+    mfma_sum: bool = False  # the row sums come out of the matrix pipe (an all-ones operand against the P fragments) instead of one add per probability
     ws: bool = False  # wave-specialised form: four consumer waves (waves x kv_split = 4) and four staging waves
     sp: bool = False  # software-pipelined form without staging waves: eight consumer waves (waves x kv_split = 8) stage for themselves
     # cross-workgroup split of the keys (``REDUCE=g<n>k``): ``kv_ctas`` workgroups per query block each take a contiguous

@@ -539,10 +539,12 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
     pinned = _pin("FLASH", _tuned(body, ctx))
     if pinned:
         try:
-            body.pair = body.deep = body.ws = body.sp = False
+            body.pair = body.deep = body.ws = body.sp = body.mfma_sum = False
             for tok in pinned.split("/"):
                 if tok == "p":
                     body.pair = True
+                elif tok == "ms":
+                    body.mfma_sum = True
                 elif tok == "ws":
                     body.ws = True
                 elif tok == "sp":
@@ -556,7 +558,7 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 elif tok.startswith("s"):
                     body.kv_split = int(tok[1:])
                 else:
-                    raise ScheduleError(f"cannot parse {tok!r} (expect w<groups> / kv<keys> / s<split> / p / k3)")
+                    raise ScheduleError(f"cannot parse {tok!r} (expect w<groups> / kv<keys> / s<split> / p / k3 / ms / ws / sp)")
             if body.ws and body.sp:
                 raise ScheduleError("ws and sp are two forms: pin one")
             if body.ws or body.sp:

@@ -331,7 +331,7 @@ def test_c4_head_dim_64_workgroup_shapes(device, pin, monkeypatch):
     eager.assert_close(ours, want, 2e-2, 2e-2, f"sdpa d=64 {pin} vs eager")
 
 
-@pytest.mark.parametrize("pin", ["w4/kv64/s1", "w4/kv64/s2", "w2/kv64/s2", "w4/kv32/s2", "w1/kv32/s4", "w2/kv32/s4", "w8/kv64/s1"])
+@pytest.mark.parametrize("pin", ["w4/kv64/s1", "w4/kv64/s2", "w2/kv64/s2", "w4/kv32/s2", "w1/kv32/s4", "w2/kv32/s4", "w8/kv64/s1", "w2/kv32/s4/ms", "w4/kv64/s2/ms"])
 def test_c4_every_workgroup_shape(device, pin, monkeypatch):
     """Key-split groups, direct-to-LDS staging and the final (m, l, O) merge: the first
     key blocks are consumed right after they are staged, so every launch is checked."""
