@@ -256,15 +256,16 @@ class Stage:
                    do nothing else, while the tile's eight waves alternate in two groups
                    half a slab apart (one computes while the other reads fragments);
                    ``mix``: the a operand as ``sync``, the b operand as ``dl``;
-                   ``ks``: no LDS staging — at most 16 rows, the reduction axis split
+                   ``ks``: no LDS staging of the weights — a few rows, the reduction axis split
                    over ``depth`` waves that load their fragments straight from global
-                   memory, all at once.
+                   memory, all at once; ``c<n>`` output columns per workgroup.
     ``ring``       kept for grammar compatibility (a depth > 1 is a ring)."""
 
     depth: int = 2
     transport: str = "sync"
     ring: bool = False
     reg_depth: int = 1
+    cols: int = 0  # ``ks`` only: output columns per workgroup (``c4`` / ``c8`` / ``c12``; 0 = 16)
 
     @classmethod
     def parse(cls, spec: str | None) -> Stage | None:
@@ -285,6 +286,8 @@ class Stage:
                 kw["ring"] = True
             elif re.fullmatch(r"p\d+", tok):
                 kw["reg_depth"] = int(tok[1:])
+            elif re.fullmatch(r"c\d+", tok):
+                kw["cols"] = int(tok[1:]) % 16
             else:
                 raise ScheduleError(f"STAGE: cannot parse {tok!r} (expect d<depth> / sync|dl|mix / ring / p<reg_depth>)")
         st = cls(**kw)
@@ -298,4 +301,6 @@ class Stage:
             s += "/ring"
         if self.reg_depth > 1:
             s += f"/p{self.reg_depth}"
+        if self.cols:
+            s += f"/c{self.cols}"
         return s

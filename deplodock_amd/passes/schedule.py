@@ -296,7 +296,7 @@ def _check_tile(plan: TilePlan, body: Contraction, ctx: Context, depth: int, dl:
         raise ScheduleError("the row epilogue works on the output tile staged in LDS, which this tile does not fit")
 
 
-from deplodock_amd.emit.skinny import skinny_waves  # noqa: E402
+from deplodock_amd.emit.skinny import skinny_cols, skinny_waves  # noqa: E402
 
 
 def pingpong_fits(plan: TilePlan, body: Contraction, ctx: Context, depth: int = 4, worthwhile: bool = True) -> bool:
@@ -325,6 +325,15 @@ def pingpong_fits(plan: TilePlan, body: Contraction, ctx: Context, depth: int = 
     )  # fmt: skip
 
 
+#: The few-row form is the default up to this many rows and this many bytes of activation rows (it takes up to
+#: ``skinny.MAX_ROWS`` rows when pinned).  Every workgroup reads all the rows, so they bound what a CU moves whatever the
+#: column count: measured inside the decoder block (us, few-row form against the tiled ring), 16 rows: o_proj (K = 2048)
+#: 3.5 / 3.9, down_proj (K = 3072) 4.5 / 5.0; 32 rows: gate / up (K = 1024, 64 KiB of rows) 5.3 / 6.0, o_proj (128 KiB)
+#: 6.3 / 4.4, down_proj (192 KiB) 8.5 / 7.4.
+_FEW_ROWS = 32
+_FEW_ROWS_BYTES = 96 * 1024
+
+
 def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
     """Staging when nothing pins it.
 
@@ -346,8 +355,8 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
       9.4; 512x1024x2048 7.4 -> 6.2 -> 6.2; 512x4096x1024 7.8 -> 6.8 -> 6.7; 2048x3072x1024
       17.2 -> 15.9 -> 16.1; 4096^3 136 -> 122; the block as one graph 66.9 -> 65.2 -> 62.8)."""
     steps = -(-body.k // plan.bk_elems)
-    if skinny_waves(body):
-        return Stage(depth=skinny_waves(body), transport="ks")
+    if skinny_waves(body) and body.m <= _FEW_ROWS and body.m * body.k * body.in_dtype.nbytes <= _FEW_ROWS_BYTES:
+        return Stage(depth=skinny_waves(body), transport="ks", cols=skinny_cols(body, ctx) % 16)
     if body.k % plan.bk_elems:
         return Stage(depth=2, transport="sync")  # the short last slab is zero-filled in registers
     if body.a_prologue is not None and body.a_prologue.scale is None:
@@ -462,8 +471,8 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
             if stage is not None and stage.transport in ("dl", "dli") and ((plan.bk_elems // plan.atom.frag_k) % 2 or plan.bk_elems % plan.atom.frag_k):
                 raise ScheduleError("direct-to-LDS staging needs an even number of MFMA steps per slab")
             if stage is not None and stage.transport == "ks":
-                if not skinny_waves(body) or stage.depth not in (1, 2, 4, 8, 16) or body.k % (32 * stage.depth):
-                    raise ScheduleError(f"the k-split few-row form does not fit M={body.m} N={body.n} K={body.k} with {stage.depth} waves")
+                if not skinny_waves(body) or stage.depth not in (1, 2, 4, 8, 16) or body.k % (32 * stage.depth) or (stage.cols and (stage.cols % 4 or body.n % stage.cols)):
+                    raise ScheduleError(f"the k-split few-row form does not fit M={body.m} N={body.n} K={body.k} with {stage.depth} waves and {stage.cols or 16} columns a workgroup")
             elif stage is not None and stage.transport == "pp":
                 if not pingpong_fits(plan, body, ctx, depth=stage.depth, worthwhile=False):
                     raise ScheduleError("the wave-specialised ring takes a plain 16-bit contraction on an eight-wave tile whose slab fragments fit a lane's registers, and a ring of at least three that fits the LDS")

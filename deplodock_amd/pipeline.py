@@ -15,12 +15,14 @@ from deplodock_amd.context import Context
 from deplodock_amd.graph import Graph
 from deplodock_amd.passes.fuse import fuse
 from deplodock_amd.passes.lower import lower
+from deplodock_amd.passes.prefetch import add_weight_prefetch
 from deplodock_amd.passes.schedule import schedule
 
 HIP_PASSES: tuple[tuple[str, Callable], ...] = (
     ("fuse", lambda g, ctx: fuse(g)),
     ("lowering/tile", schedule),
     ("lowering/hip", lower),
+    ("lowering/prefetch", add_weight_prefetch),
 )
 
 
@@ -55,6 +57,6 @@ class Pipeline:
                 dump_dir.mkdir(parents=True, exist_ok=True)
                 tag = f"{(i + 1) * 10:02d}_{name.replace('/', '_')}"
                 (dump_dir / f"{tag}.txt").write_text(g.pretty_print() + "\n")
-                if i == len(self.passes) - 1:
+                if name == "lowering/hip":
                     (dump_dir / f"{tag}_kernels.hip").write_text(format_kernels(g))
         return g

@@ -67,7 +67,7 @@ def test_linear_is_one_mfma_kernel(launcher_lib, m):
     # register sets); from 128 rows on direct-to-LDS loads (three 48 KiB slabs
     # of the 32x64x256 tile); at 2048 rows the 128x192 tile's eight waves alternate in two groups behind four
     # staging waves (twelve waves, a ring of four 40 KiB slabs)
-    assert k.knobs["STAGE"] == {1: "d8/ks", 16: "d8/ks", 128: "d3/dl", 2048: "d4/pp"}[m]
+    assert k.knobs["STAGE"] == {1: "d8/ks/c12", 16: "d8/ks/c12", 128: "d3/dl", 2048: "d4/pp"}[m]
     assert ("wave * 128 + lk * 8" in k.kernel_source) == (m < 128) and ("#define EMH_DLOAD" in k.kernel_source) == (m >= 128)
     if m == 2048:
         assert k.block[0] == (768,) and k.lds_bytes == 4 * (128 + 192) * 64 * 2 and "role == 2" in k.kernel_source
