@@ -132,18 +132,21 @@ def test_c3_linear(device, m):
 
 
 @pytest.mark.parametrize("waves", [None, 8, 4, 2, 1])
-@pytest.mark.parametrize("m,k,n", [(1, 1024, 3072), (16, 1024, 3072), (5, 512, 1960), (13, 3072, 1024), (16, 2048, 24), (3, 16384, 256), (2, 32, 40), (16, 8192, 64)])
+@pytest.mark.parametrize("m,k,n", [(1, 1024, 3072), (16, 1024, 3072), (5, 512, 1960), (13, 3072, 1024), (16, 2048, 24), (3, 16384, 256), (2, 32, 40), (16, 8192, 64), (32, 1024, 3072), (24, 2048, 1000), (47, 1024, 520), (64, 512, 264)])
 def test_few_row_linear_k_split_over_waves(device, m, k, n, waves, monkeypatch):
-    """At most 16 rows: the reduction axis is split over the waves of a workgroup, every weight fragment is
-    requested at once, the activation rows go through LDS where they fit (two rows of 16384 do, 16 of 8192
-    do not), long reduction extents loop over 16-step groups, and a column count that is no multiple of 16
-    re-reads the last row without storing it."""
+    """A few rows (up to four 16-row MFMA tiles): the reduction axis is split over the waves of a workgroup, every
+    weight fragment is requested at once, the activation rows go through LDS where they fit (two rows of 16384 do,
+    16 of 8192 do not), long reduction extents loop over 16-step groups, and a column count that is no multiple of 16
+    re-reads the last row without storing it.  By default up to 32 rows of at most 96 KiB together take the form."""
     if waves is not None:
         monkeypatch.setenv("EMMY_STAGE", f"d{waves}/ks")
     case = eager.linear_case(m=m, k=k, n=n, seed=m + k)
     ours, want, compiled = run_case(case, device)
     op = next(n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp))
-    assert op.knobs["STAGE"].endswith("/ks"), op.knobs  # a wave count that does not divide the extent degrades to the default one
+    if waves is not None or (m <= 32 and m * k * 2 <= 96 * 1024):
+        assert "/ks" in op.knobs["STAGE"], op.knobs  # a wave count that does not divide the extent degrades to the default one
+    else:
+        assert "/ks" not in op.knobs["STAGE"], op.knobs
     if waves is not None and k % (32 * waves) == 0:
         assert op.knobs["STAGE"] == f"d{waves}/ks"
     eager.assert_close(ours, want, case.rtol, case.atol, f"few-row linear {m}x{k}x{n} vs eager (GPU)")
@@ -192,6 +195,56 @@ def test_c3_golden(device, golden):
     ours, _, _ = run_case(case, device)
     want = torch.from_numpy(golden["c3_y_bits"].view(np.int16).copy()).view(torch.bfloat16).float()
     eager.assert_close(ours, want, 2e-2, 2e-2, "linear golden")
+
+
+@pytest.mark.parametrize("cols", [4, 8, 12, 16])
+@pytest.mark.parametrize("m,k,n", [(1, 1024, 3072), (16, 3072, 1032), (32, 1024, 1536), (40, 512, 24)])
+def test_few_row_columns_per_workgroup(device, m, k, n, cols, monkeypatch):
+    """4, 8, 12 or 16 output columns a workgroup: the spare weight rows of the MFMA tile request nothing and count as
+    zeros, and only the workgroup's own columns are stored.  A column count that does not divide N is refused (the
+    default form runs instead)."""
+    monkeypatch.setenv("EMMY_STAGE", f"d8/ks/c{cols}" if cols != 16 else "d8/ks")
+    case = eager.linear_case(m=m, k=k, n=n, seed=cols + m)
+    ours, want, compiled = run_case(case, device)
+    op = next(n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp))
+    if cols == 16 or n % cols == 0:
+        assert op.knobs["STAGE"] == (f"d8/ks/c{cols}" if cols != 16 else "d8/ks") and op.grid[0] == (-(-n // cols),)
+    eager.assert_close(ours, want, case.rtol, case.atol, f"few-row linear {m}x{k}x{n} c{cols} vs eager (GPU)")
+    exact = case.inputs[0].double() @ case.module.weight.detach().double().cpu().T
+    eager.assert_close(ours, exact, 2 ** -7, 2e-3, f"few-row linear {m}x{k}x{n} c{cols} vs float64")
+
+
+class _GateUp(nn.Module):
+    """``down(silu(gate(norm(x))) * up(norm(x)))`` without the down projection: a gate / up pair behind an RMSNorm."""
+
+    def __init__(self, k, n):
+        super().__init__()
+        self.norm = nn.RMSNorm(k, eps=1e-6)
+        self.gate = nn.Linear(k, n, bias=False)
+        self.up = nn.Linear(k, n, bias=False)
+        with torch.no_grad():
+            self.norm.weight.copy_(1.0 + 0.1 * torch.randn(k))
+
+    def forward(self, x):
+        h = self.norm(x)
+        return nn.functional.silu(self.gate(h)) * self.up(h)
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 1024, 3072), (16, 1024, 3072), (32, 1024, 768), (7, 512, 264)])
+def test_few_row_gate_up_pair_behind_a_deferred_norm(device, m, k, n):
+    """One launch: the norm's column weight is folded into both weight matrices, the row statistic is accumulated from
+    the fragments each lane holds (lanes of a row through a butterfly, waves through LDS) and scales both accumulators
+    before ``silu(gate) * up``."""
+    torch.manual_seed(m + n)
+    mod = _GateUp(k, n).bfloat16().eval()
+    case = eager.Case("gate_up", mod, (torch.randn(m, k).bfloat16(),), 2e-2, 2e-2)
+    ours, want, compiled = run_case(case, device)
+    ops = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+    assert len(ops) == 1 and "/ks" in ops[0].knobs["STAGE"] and "silu" in ops[0].kernel_name, [o.knobs for o in ops]
+    with torch.no_grad():
+        exact = copy.deepcopy(mod).cpu().double()(case.inputs[0].cpu().double())
+    eager.assert_close(ours, want, 2e-2, 2e-2, f"gate/up {m}x{k}x{n} vs eager")
+    eager.assert_mean_error_within_baseline(ours, want, exact.float(), 1.5, f"gate/up {m}x{k}x{n} vs float64")
 
 
 # -- C4 ---------------------------------------------------------------------------
