@@ -26,8 +26,9 @@ The pass runs after lowering and is on by default only where it can pay: a progr
 last-level cache, and in it a consumer between ``MIN_INTENSITY`` and ``MAX_INTENSITY`` flop per byte (``EMMY_PREFETCH=1`` /
 ``0`` force it on for every consumer / off).  Measured on the 28-layer Qwen3-0.6B-architecture model (880 MB of weights;
 us per forward as one graph replay, without / with): 1 token 735 / 776, 16 tokens 842 / 846, 32 tokens 959 / 929,
-128 tokens 1090 / 1019 — below about 32 rows a launch is too short to hide its successor's lines behind, and the extra
-wave or workgroups cost more than the warm start gains.
+128 tokens 1090 / 1019, 256 tokens 1283 / 1166, 512 tokens 1544 / 1531 — below about 32 rows a launch is too short to hide
+its successor's lines behind and the extra wave or workgroups cost more than the warm start gains; at 512 rows the
+consumers are busy with arithmetic and the gain is within the spread of two runs.
 """
 
 from __future__ import annotations
