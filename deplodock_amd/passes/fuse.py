@@ -991,6 +991,10 @@ def _logical_strides(p: _RopePlan, mem_strides: tuple[int, ...]) -> tuple[int, .
     return tuple(out)
 
 
+#: tokens up to which the q / k head norm + rotary embedding stays a launch of its own behind the few-row projection
+_ROW_EPILOGUE_MIN_TOKENS = 16
+
+
 def _rec_rope_pair(c: _Ctx, nid: str) -> bool:
     """Query and key head-norm + rotary embedding as one launch.  Applies when
     both read adjacent head ranges of one merged projection buffer
@@ -999,7 +1003,11 @@ def _rec_rope_pair(c: _Ctx, nid: str) -> bool:
     result is a window of the ``[tokens, q heads + k heads, d]`` output."""
     g = c.g
     p = _plan_rope(c, nid)
-    if p is None or p.rms is None or p.rms.weight is None or len(p.mem_shape) != 2 or p.mod != p.mem_shape[0]:
+    if p is None or p.rms is None or p.rms.weight is None:
+        return False
+    # one token: the token dim is a unit dim the plan drops; the heads alone are the rows
+    single = len(p.mem_shape) == 1 and p.mod == 1
+    if not single and (len(p.mem_shape) != 2 or p.mod != p.mem_shape[0]):
         return False
     partner = None
     for oid in g.topological_order():
@@ -1008,7 +1016,7 @@ def _rec_rope_pair(c: _Ctx, nid: str) -> bool:
         q = _plan_rope(c, oid)
         if q is None or q.rms is None or q.rms.weight is None:
             continue
-        if (q.cos_id, q.sin_id, q.d, q.od, q.mod, q.order, q.rms.eps, q.rms.inner) == (p.cos_id, p.sin_id, p.d, p.od, p.mod, p.order, p.rms.eps, p.rms.inner) and len(q.mem_shape) == 2:
+        if (q.cos_id, q.sin_id, q.d, q.od, q.mod, q.order, q.rms.eps, q.rms.inner) == (p.cos_id, p.sin_id, p.d, p.od, p.mod, p.order, p.rms.eps, p.rms.inner) and len(q.mem_shape) == len(p.mem_shape):
             partner = (oid, q)
             break
     if partner is None:
@@ -1024,16 +1032,25 @@ def _rec_rope_pair(c: _Ctx, nid: str) -> bool:
         (rows0, a0), (rows1, a1) = _row_addr(x0), _row_addr(x1)
     except FusionError:
         return False
-    h0, h1 = p0.mem_shape[1], p1.mem_shape[1]
+    h0, h1 = p0.mem_shape[-1], p1.mem_shape[-1]
     d = p.d
-    if not (a0.div == h0 and a1.div == h1 and a0.stride_lo == d and a1.stride_lo == d and a0.stride_hi == a1.stride_hi and a1.offset == a0.offset + h0 * d and (h0 + h1) * d <= a0.stride_hi):
+    if single:
+        # [heads, d] windows of one row of the merged projection: rows d apart, the key heads right behind the query heads
+        if not (a0.div == 1 and a1.div == 1 and rows0 == h0 and rows1 == h1 and (h0 == 1 or a0.stride_hi == d) and (h1 == 1 or a1.stride_hi == d) and a1.offset == a0.offset + h0 * d):
+            return False
+        prod = c.out.nodes.get(x0.base)
+        pitch = (h0 + h1) * d
+        if prod is not None and isinstance(prod.op, TileOp) and isinstance(prod.op.body, Contraction):
+            pitch = prod.op.body.ldo or prod.op.body.n
+        a0 = RowAddr(offset=a0.offset, div=h0 + h1, stride_hi=pitch, stride_lo=d)
+    elif not (a0.div == h0 and a1.div == h1 and a0.stride_lo == d and a1.stride_lo == d and a0.stride_hi == a1.stride_hi and a1.offset == a0.offset + h0 * d and (h0 + h1) * d <= a0.stride_hi):
         return False
     # the two weights are only read through their stacked copy: they get no buffers of their own
     w0, w1 = g.nodes[p0.rms.weight], g.nodes[p1.rms.weight]
     if not (isinstance(w0.op, ConstantOp) and isinstance(w1.op, ConstantOp) and w0.output.dtype == w1.output.dtype and tuple(w0.output.shape) == tuple(w1.output.shape) == (d,)):
         return False
     heads = h0 + h1
-    tokens = p0.mem_shape[0]
+    tokens = 1 if single else p0.mem_shape[0]
     stacked = f"{p0.rms.weight}__x{h0}__{p1.rms.weight}__x{h1}"
     if stacked not in c.out.nodes:
         c.out.add_constant(stacked, (heads * d,), w0.output.dtype)
@@ -1050,17 +1067,21 @@ def _rec_rope_pair(c: _Ctx, nid: str) -> bool:
     )  # fmt: skip
     body.rotate = RotateHalf(_rope_expr(od))
     body.operand_buffers = {"w": stacked, "cos": cos_v.base, "sin": sin_v.base}
+    mem = (lambda hi: (d,)) if single else (lambda hi: (hi, d))  # strides of the plan's memory-order dims (heads [, tokens])
     raw_only_feeds_rope = all(_feeds_only(g, _peel_layout(g, rp.t_id), _rope_internal(g, rp.t_id, rid)) for rid, rp in ((id0, p0), (id1, p1)))
-    if raw_only_feeds_rope and _absorb_row_kernel(c, body, x0, a0, tokens, heads):
+    # With a few tokens the projection is one pass over its weights in the few-row form, which has no output tile to
+    # run a row kernel on: a second small launch costs less than giving that form up (us in the decoder block, fused
+    # against few-row projection + this kernel: 16 tokens 7.3 against 3.0 + 1.9).
+    if tokens > _ROW_EPILOGUE_MIN_TOKENS and raw_only_feeds_rope and _absorb_row_kernel(c, body, x0, a0, tokens, heads):
         # the projection that produced the heads rotates them on its way out: the results are windows of its buffer
         for rid, rp, first in ((id0, p0, 0), (id1, p1, h0)):
             c.done[rid] = x0.base
-            c.windows[rid] = (a0.offset + first * d, rp.t_view_shape, _logical_strides(rp, (a0.stride_hi, d)))
+            c.windows[rid] = (a0.offset + first * d, rp.t_view_shape, _logical_strides(rp, mem(a0.stride_hi)))
         return True
     c.out.add_node(TileOp(name=c.kname("rms_norm_rope"), body=body), list(dict.fromkeys([x0.base, stacked, cos_v.base, sin_v.base])), Tensor(fid, (tokens, heads, d), od), fid)
     for rid, rp, first in ((id0, p0, 0), (id1, p1, h0)):
         c.done[rid] = fid
-        c.windows[rid] = (first * d, rp.t_view_shape, _logical_strides(rp, (heads * d, d)))
+        c.windows[rid] = (first * d, rp.t_view_shape, _logical_strides(rp, mem(heads * d)))
     return True
 
 

@@ -145,9 +145,17 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
     # while their sum of squares is accumulated, and the accumulators take the row's scale factor
     first = kernels(compiled)[0]
     assert "a=row-scaled-after" in first.comment and first.arg_order[0] == compiled.inputs[0] and first.knobs["STAGE"] == "d2/dl"
-    decode = kernels(compile_case(eager.qwen3_block_case(seq=16)))[0]  # 16 tokens (as many as heads): decode-size staging through registers
-    assert "a=row-scaled-after" in decode.comment and decode.knobs["STAGE"] == "d2/sync/p2" and "#define EMH_SUMSQ_READ" not in decode.kernel_source
-    hiprtc.compile_to_hsaco(decode.kernel_source, decode.kernel_name)
+    # 16 tokens (as many as heads) and fewer: the projection takes the few-row form with the deferred norm (the row
+    # statistic from the fragments a lane holds, the accumulators scaled), and the head norms + rotary embedding of q
+    # and k are one small row kernel behind it; one token, whose token dim is a unit dim, pairs q and k the same way
+    for seq in (16, 1):
+        few = kernels(compile_case(eager.qwen3_block_case(seq=seq)))
+        assert [re.sub(r"_[0-9a-f]{6}$", "", k.kernel_name) for k in few] == ["k_rms_norm_linear", "k_rms_norm_rope", "k_sdpa_reduce", "k_linear_add", "k_rms_norm_linear_silu_mul", "k_linear_add"]
+        decode, rope = few[0], few[1]
+        assert decode.knobs["STAGE"] == "d8/ks" and "ss[t] += emh_xor16(ss[t])" in decode.kernel_source and "* rs_)" in decode.kernel_source
+        assert decode.arg_order[1].endswith("__k*p_l_input_layernorm_weight") and rope.arg_order[0] == decode.arg_order[-1]
+        for k in few[:2]:
+            hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
     assert "__shfl_xor(ss[i], msk, 64)" in first.kernel_source and "* rs_)" in first.kernel_source
     assert "p_l_input_layernorm_weight" not in first.arg_order and first.arg_order[1].endswith("__k*p_l_input_layernorm_weight")
     # q, k and v projections are one contraction over the stacked weights; each
