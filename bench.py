@@ -357,6 +357,19 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
         if res.num_launches > 1:
             row["sum_of_kernels_us"] = round(res.time_ms * 1e3, 2)
             row["per_kernel_us"] = {f"{i}:{p.kernel_name}": round(p.time_ms * 1e3, 2) for i, p in enumerate(res.per_launch)}
+            # every launch against both rooflines; the one that bounds it is the one its algorithmic work takes longer on
+            # (more than 312 flop per byte, the ratio of the two peaks: the matrix pipe; else HBM)
+            ops = {n.op.kernel_name: n.op for n in compiled.nodes.values() if hasattr(n.op, "kernel_name")}
+            per = []
+            for i, p in enumerate(res.per_launch):
+                op, t = ops[p.kernel_name], p.time_ms * 1e-3
+                if t <= 0 or not op.algo_bytes:
+                    continue
+                tf, gb = op.algo_flops / t / 1e12, op.algo_bytes / t / 1e9
+                f_mfma, f_hbm = tf / MFMA_BF16_PEAK_TFLOPS, gb / HBM_PEAK_GBPS
+                per.append({"kernel": f"{i}:{p.kernel_name}", "us": round(t * 1e6, 2), "bound": "mfma" if f_mfma >= f_hbm else "hbm", "tflops": round(tf, 1), "gbps": round(gb, 1),
+                            "frac_mfma": round(f_mfma, 4), "frac_hbm": round(f_hbm, 4), "frac": round(max(f_mfma, f_hbm), 4)})  # fmt: skip
+            row["per_kernel"] = per
         if bound == "hbm":
             gbps = case.algo_bytes / (us * 1e-6) / 1e9
             row.update(bound="hbm", achieved=round(gbps, 1), unit="GB/s", frac=round(gbps / HBM_PEAK_GBPS, 4))
@@ -373,6 +386,7 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
             row["eager_gpu_us"] = round(eager_us, 1)
             row["tokens_per_s"] = round(int(case.inputs[0].numel()) / (us * 1e-6))
             row.pop("per_kernel_us", None)  # (142 entries: the five kernels of a layer are the C5 row's)
+            row.pop("per_kernel", None)
         if vendor:
             v_us = vendor_us(case)
             row["vendor_us"] = round(v_us, 2)  # PyTorch eager on the same GPU: the vendor library's kernel for this problem
@@ -473,7 +487,8 @@ def main() -> int:
         # bound: its machine-filling variant C1x stands for the kernel; the decode-size linears are HBM bound)
         peaks = {"hbm": (HBM_PEAK_GBPS, "GB/s"), "mfma": (MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")}
         out["rooflines"] = [
-            {"config": r["config"], "bound": r["bound"], "achieved": r["achieved"], "peak": peaks[r["bound"]][0], "unit": peaks[r["bound"]][1], "frac": r["frac"], "kernel_us": r["us"]}
+            {"config": r["config"], "bound": r["bound"], "achieved": r["achieved"], "peak": peaks[r["bound"]][0], "unit": peaks[r["bound"]][1], "frac": r["frac"], "kernel_us": r["us"],
+             **({"per_kernel": r["per_kernel"]} if "per_kernel" in r else {})}
             for r in out["kernels"]
         ]
     print(json.dumps(out))
