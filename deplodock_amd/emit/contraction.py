@@ -269,7 +269,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     if split is not None:
         if body.epilogue is not None or body.post is not None or body.bias is not None or body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None or body.out_dtype is not F32:
             raise LoweringError("contraction: the partial kernel of a split stores bare fp32 accumulators; bias, epilogue and rounding belong to the combine")
-        if stage.transport not in ("sync", "dl", "dli", "pp"):
+        if stage.transport not in ("sync", "dl", "dli", "dlm", "pp"):
             raise LoweringError(f"contraction: STAGE .../{stage.transport} does not combine with a cross-workgroup split")
     M, N, K = body.m, body.n, body.k
     lda = body.lda or K
@@ -314,7 +314,7 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
     A_PER_T, B_PER_T = a_chunks // ST, b_chunks // ST
     slab_bytes = (TM + TN * NB) * BK * ES
     depth = 2 if stage.transport == "mix" else max(2, stage.depth)
-    RS = 1 if stage.transport in ("dl", "dli", "pp", "mix") else max(1, stage.reg_depth)  # register sets a slab travels through on the sync path
+    RS = 1 if stage.transport in ("dl", "dli", "dlm", "pp", "mix") else max(1, stage.reg_depth)  # register sets a slab travels through on the sync path
     lds_bytes = slab_bytes * depth
     if lds_bytes > ctx.lds_bytes_per_cu:
         raise LoweringError(f"contraction: {lds_bytes} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
@@ -340,9 +340,10 @@ def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> 
             gn -= 1
     n_guard = N % TN != 0
     dli = stage.transport == "dli"  # direct to LDS, requests issued between the MFMAs of the slab before (see below)
+    dlm = stage.transport == "dlm"  # direct to LDS as ``dl``, the steady-state requests spread among the MFMAs of the slab's last step
     pp = stage.transport == "pp"  # direct to LDS, the two waves of a SIMD in opposite phases (one computes, one fetches)
     spec = pp  # specialised waves: the tile's own compute, four more stage
-    dl = stage.transport in ("dl", "dli", "pp")
+    dl = stage.transport in ("dl", "dli", "dlm", "pp")
     mix = stage.transport == "mix"  # a through registers (it is transformed on the way), b direct to LDS
     if mix and b_chunks % 64:
         raise LoweringError("contraction: direct-to-LDS staging needs whole-wave chunk counts")
@@ -450,7 +451,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     # ---- staging ------------------------------------------------------------
     a(f"  const {in_c}* ga[A_PER_T]; int la[A_PER_T];" + (" int ca[A_PER_T];" if pro is not None else "") + (" int ka[A_PER_T], kb[B_PER_T];" if k_guard else ""))
     a(f"  const {in_c}* gb[B_PER_T]; int lb[B_PER_T];")
-    if dli or spec:
+    if dli or dlm or spec:
         if max(M * lda, N * NB * ldb) * ES >= 2**32:
             raise LoweringError("contraction: STAGE .../dli addresses operands with 32-bit byte offsets; this operand is larger than 4 GiB")
         a("  unsigned va[A_PER_T], vb[B_PER_T];  // byte offset of each request's chunk from the operand base (the k position is added to the base, in scalar registers)")
@@ -467,7 +468,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         a("    la[i] = row * (BK * ES) + emh_swz(row, c) * 16;")
     a(f"    int gr = m0 + row;{' if (gr > M - 1) gr = M - 1;' if m_guard else ''}")
     a(f"    ga[i] = A + {body.a_offset}L + ASL + (long)gr * LDA + c * EPCK;")
-    if dli or spec:
+    if dli or dlm or spec:
         a("    va[i] = ((unsigned)gr * LDA + c * EPCK) * (unsigned)ES;")
     if pro is not None:
         a("    ca[i] = c * EPCK;")
@@ -490,7 +491,7 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
     else:
         a(f"    int gr = n0 + row;{' if (gr > N - 1) gr = N - 1;' if n_guard else ''}")
     a(f"    gb[i] = B + {body.b_offset}L + BSL + (long)gr * LDB + c * EPCK;")
-    if dli or spec:
+    if dli or dlm or spec:
         a("    vb[i] = ((unsigned)gr * LDB + c * EPCK) * (unsigned)ES;")
     if k_guard:
         a("    kb[i] = c * EPCK;")
@@ -654,7 +655,7 @@ ROW_EPILOGUE_TABLES
     asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
   #pragma unroll
   for (int p = 0; p < DEPTH - DLI; ++p) if (p < KT STAGER) EMH_DLOAD(p, p);""".replace("DLI", "1" if dli or pp else "0").replace(" STAGER", " && tid >= T" if spec else ""))
-        if dli or spec:
+        if dli or dlm or spec:
             a(f"""  // One request of slab kt into ring buffer buf: the operand base moves along k in scalar registers, the
   // lane's chunk offset is a loop-invariant 32-bit register, the LDS target a scalar: no vector arithmetic per request.
   #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L + ASL) + (long)(kt) * (BK * ES), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * ST) * 16)
@@ -682,6 +683,24 @@ ROW_EPILOGUE_TABLES
             part_fmt = [f"EMH_DPART_A({{slab}}, {{buf}}, {i});" for i in range(A_PER_T)] + [f"EMH_DPART_B({{slab}}, {{buf}}, {i});" for i in range(B_PER_T)]
             _emit_pingpong_loop(a, KT=KT, KS=KS, depth=depth, parts=part_fmt)
 
+        def mma_spread(P: int, kt: str) -> None:
+            """The MFMAs of a slab's last step with the requests of slab ``kt + DEPTH`` (into the buffer this slab leaves)
+            spread evenly among them."""
+            parts = [("A", i) for i in range(A_PER_T)] + [("B", i) for i in range(B_PER_T)]
+            n = NB * FM * FN
+            after = [(q * n) // len(parts) for q in range(len(parts))]
+            idx = 0
+            for h in range(NB):
+                for i in range(FM):
+                    for j in range(FN):
+                        for e in range(MPF):
+                            a(f"    acc[{h}][{i}][{j}] = {plan.atom.builtin}(EMH_OPND(fw[{P}][{h}][{j}], {e}), EMH_OPND(fx[{P}][{i}], {e}), acc[{h}][{i}][{j}], 0, 0, 0);")
+                        for q, (which, pi) in enumerate(parts):
+                            if after[q] == idx:
+                                a(f"    __builtin_amdgcn_sched_barrier(0); EMH_DPART_{which}(({kt}) + DEPTH, cur, {pi}); __builtin_amdgcn_sched_barrier(0);")
+                        idx += 1
+            a("    __builtin_amdgcn_sched_barrier(0);")
+
         def slab_steps(kt: str, static_kt: int | None) -> None:
             """MFMA steps of slab ``kt``.  With ``static_kt`` the hand-over to the
             next slab is resolved at emit time (tail); otherwise it is the
@@ -696,6 +715,12 @@ ROW_EPILOGUE_TABLES
                     a(f"    EMH_READ({P ^ 1}, cur, {kk + 1});")
                 elif static_kt is None:
                     a(f"    EMH_SLAB_SYNC({(depth - 2) * loads_per_slab});")
+                    if dlm:
+                        # the buffer is free from here on (the last step's fragments are in registers): its next slab is
+                        # requested one request at a time between this step's MFMAs instead of as a burst in front of them
+                        a(f"    EMH_READ({P ^ 1}, (({kt}) + 1) % DEPTH, 0);")
+                        mma_spread(P, kt)
+                        continue
                     a(f"    EMH_DLOAD(({kt}) + DEPTH, cur);")
                     a(f"    EMH_READ({P ^ 1}, (({kt}) + 1) % DEPTH, 0);")
                 elif static_kt + 1 < KT:

@@ -239,7 +239,7 @@ class TilePlan:
 # STAGE
 # --------------------------------------------------------------------------
 
-_TRANSPORTS = {"sync": "sync", "dl": "dl", "dli": "dli", "pp": "pp", "cp": "dl", "mix": "mix", "ks": "ks"}
+_TRANSPORTS = {"sync": "sync", "dl": "dl", "dli": "dli", "dlm": "dlm", "pp": "pp", "cp": "dl", "mix": "mix", "ks": "ks"}
 
 
 @dataclass(frozen=True)
@@ -252,6 +252,8 @@ class Stage:
                    ``dl``: global loads that write LDS directly, no VGPR hop;
                    ``dli``: the same loads, issued one at a time between the MFMAs of
                    the slab before instead of as a burst behind its barrier;
+                   ``dlm``: as ``dl`` (any ring depth), the requests of the steady state
+                   spread among the MFMAs of the slab's last step;
                    ``pp``: the same loads issued by four extra waves (one per SIMD) that
                    do nothing else, while the tile's eight waves alternate in two groups
                    half a slab apart (one computes while the other reads fragments);

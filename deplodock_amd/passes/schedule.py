@@ -377,7 +377,13 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
                 continue
             loads = (plan.tile_m + plan.tile_n * (2 if body.gate_pair else 1)) * (plan.bk_elems // 8) // plan.block_threads
             if (depth - 1) * loads <= 63:  # the vector-memory counter has six bits
-                return Stage(depth=depth, transport="dl")
+                # With four and more MFMAs a step per wave the next slab's requests go out one at a time between the MFMAs
+                # of the slab's last step (``dlm``) instead of as a burst in front of them: 4096^3 on the 256x256 tile
+                # 111 -> 103 us; in the decoder block at 2 048 tokens gate/up 29.9 -> 27.9, o_proj 13.3 -> 12.8, down_proj
+                # 18.4 -> 17.5 us, at 512 tokens q/k/v 9.6 -> 9.4 and gate/up 10.4 -> 10.1.  One-fragment waves (a single MFMA a
+                # step) have nothing to spread over and lose (down_proj at 512 tokens 8.0 -> 8.7 us): they keep the burst.
+                spread = plan.regs[0] * plan.regs[1] * (2 if body.gate_pair else 1) >= 4
+                return Stage(depth=depth, transport="dlm" if spread else "dl")
     return Stage(depth=2, transport="sync")
 
 
@@ -468,7 +474,7 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
     if pinned_stage:
         try:
             stage = Stage.parse(pinned_stage)
-            if stage is not None and stage.transport in ("dl", "dli") and ((plan.bk_elems // plan.atom.frag_k) % 2 or plan.bk_elems % plan.atom.frag_k):
+            if stage is not None and stage.transport in ("dl", "dli", "dlm") and ((plan.bk_elems // plan.atom.frag_k) % 2 or plan.bk_elems % plan.atom.frag_k):
                 raise ScheduleError("direct-to-LDS staging needs an even number of MFMA steps per slab")
             if stage is not None and stage.transport == "ks":
                 if not skinny_waves(body) or stage.depth not in (1, 2, 4, 8, 16) or body.k % (32 * stage.depth) or (stage.cols and (stage.cols % 4 or body.n % stage.cols)):
@@ -477,11 +483,11 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
                 if not pingpong_fits(plan, body, ctx, depth=stage.depth, worthwhile=False):
                     raise ScheduleError("the wave-specialised ring takes a plain 16-bit contraction on an eight-wave tile whose slab fragments fit a lane's registers, and a ring of at least three that fits the LDS")
             elif stage is not None:
-                _check_tile(plan, body, ctx, depth=max(2, stage.depth), dl=stage.transport == "dl")
+                _check_tile(plan, body, ctx, depth=max(2, stage.depth), dl=stage.transport in ("dl", "dlm"))
         except ScheduleError as exc:
             logger.warning("EMMY_STAGE=%r ignored: %s", pinned_stage, exc)
             stage = None
-    if stage is not None and body.a_prologue is not None and body.a_prologue.scale is None and stage.transport == "dl":
+    if stage is not None and body.a_prologue is not None and body.a_prologue.scale is None and stage.transport in ("dl", "dlm"):
         logger.warning("STAGE=%s ignored: the row-normalised operand is transformed in registers (sync or mix staging only)", stage.spell())
         stage = None
     if stage is None:
@@ -493,7 +499,7 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
     # more than the idle CUs (see ``deplodock_amd.emit.splitk``).  A ``b<n>`` / ``r<n>`` pin is a row kernel's.
     body.reduce = ReducePlan()
     pinned_reduce = _pin("REDUCE", tuned)
-    if auto_split > 1 and not pinned_reduce and stage.transport in ("dl", "sync"):
+    if auto_split > 1 and not pinned_reduce and stage.transport in ("dl", "dlm", "sync"):
         body.reduce = ReducePlan(cta=auto_split, finalize="kernel")
         knobs["REDUCE"] = body.reduce.spell()
     if pinned_reduce:
@@ -507,7 +513,7 @@ def schedule_contraction(body: Contraction, ctx: Context) -> dict:
                 if stage.transport in ("ks", "mix"):
                     body.stage = stage = Stage(depth=2, transport="sync", reg_depth=2 if body.k // rp.cta // plan.bk_elems >= 3 else 1)
                     knobs["STAGE"] = stage.spell()
-                if stage.transport in ("dl", "dli") and ((plan.bk_elems // plan.atom.frag_k) % 2 or plan.bk_elems % plan.atom.frag_k):
+                if stage.transport in ("dl", "dli", "dlm") and ((plan.bk_elems // plan.atom.frag_k) % 2 or plan.bk_elems % plan.atom.frag_k):
                     raise ScheduleError("direct-to-LDS staging needs an even number of MFMA steps per slab")
                 body.reduce = ReducePlan(cta=rp.cta, finalize=rp.finalize)
                 knobs["REDUCE"] = body.reduce.spell()

@@ -847,7 +847,7 @@ def test_fp32_linear(device, m, k, n, bias):
     eager.assert_close(ours.reshape(want.shape), want, 1e-5, 2e-5, f"fp32 linear {m}x{k}x{n} vs eager")
 
 
-@pytest.mark.parametrize("stage", ["d2/sync", "d2/sync/p2", "d2/dl", "d3/dl", "d3/dli"])
+@pytest.mark.parametrize("stage", ["d2/sync", "d2/sync/p2", "d2/dl", "d3/dl", "d3/dli", "d2/dlm", "d3/dlm"])
 def test_fp32_linear_every_transport_is_bit_identical(device, stage, monkeypatch):
     monkeypatch.setenv("EMMY_TILE", "a:mfma_16x16x4_f32/w2x2/f2x2/k8")
     torch.manual_seed(8)
@@ -1001,7 +1001,7 @@ def test_staging_transports_are_bit_identical(device, monkeypatch):
     x = case.inputs[0].to(device)
     monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x2/f1x2/k4")
     outs = {}
-    for stage in ("d2/sync", "d2/sync/p2", "d2/sync/p3", "d2/mix", "d2/dl", "d3/dl", "d4/dl", "d3/dli", "d4/dli"):  # 16 slabs: not a multiple of three register sets
+    for stage in ("d2/sync", "d2/sync/p2", "d2/sync/p3", "d2/mix", "d2/dl", "d3/dl", "d4/dl", "d3/dli", "d4/dli", "d2/dlm", "d3/dlm", "d4/dlm"):  # 16 slabs: not a multiple of three register sets
         monkeypatch.setenv("EMMY_STAGE", stage)
         be = HipBackend()
         compiled = be.compile(graph)
@@ -1077,7 +1077,7 @@ def _soak(prog, out_name: str, launches: int, what: str) -> None:
             pytest.fail(f"{what}: launch {i} of {launches} differs from the first launch in {bad} elements")
 
 
-@pytest.mark.parametrize("stage", ["d3/dl", "d3/dli", "d4/pp", "d3/pp"])
+@pytest.mark.parametrize("stage", ["d3/dl", "d3/dli", "d2/dlm", "d3/dlm", "d4/pp", "d3/pp"])
 def test_soak_direct_to_lds_contraction_is_bit_stable_over_thousands_of_launches(device, stage, monkeypatch):
     """The publication fence of the direct-to-LDS rings (a flat LDS read of the issuing wave, waited for on the
     LDS counter, before the barrier) as a test: a race that let one wave read a slab before another wave's loads

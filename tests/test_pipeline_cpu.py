@@ -201,7 +201,9 @@ def test_head_norm_and_rope_fold_into_the_projection(launcher_lib, monkeypatch):
 def test_deferred_norm_takes_the_direct_to_lds_ring_at_prefill_sizes(launcher_lib):
     ks = kernels(compile_case(eager.qwen3_block_case(seq=512)))
     qkv, gate_up = ks[0], ks[3]
-    assert qkv.knobs["STAGE"] == "d3/dl" and gate_up.knobs["STAGE"] == "d3/dl"
+    # four and more MFMAs a step per wave: the next slab's requests are spread among the MFMAs of the slab's last step
+    assert qkv.knobs["STAGE"] == "d3/dlm" and gate_up.knobs["STAGE"] == "d3/dlm" and ks[2].knobs["STAGE"] == ks[4].knobs["STAGE"] == "d3/dl"
+    assert qkv.kernel_source.count("EMH_DPART_A((kt) + DEPTH, cur,") >= 1 and "EMH_DLOAD((kt) + DEPTH, cur);" not in qkv.kernel_source
     assert gate_up.knobs["TILE"].endswith("/w4x2/f1x3/k2") and gate_up.grid[0][0] == 256  # 64x96 tiles: one workgroup per CU
     for k in (qkv, gate_up):
         assert "a=row-scaled-after" in k.comment and "#define EMH_SUMSQ_READ(buf)" in k.kernel_source and "EMH_SUMSQ_ADD();" in k.kernel_source

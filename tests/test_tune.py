@@ -76,7 +76,7 @@ def test_unrealisable_tile_pin_degrades_per_kernel(monkeypatch, launcher_lib):
     monkeypatch.setenv("EMMY_TILE", "a:mfma_32x32x16_bf16/w2x4/f4x2/k4")  # 256x256 tile, 8 waves, 64-deep slabs
     monkeypatch.setenv("EMMY_STAGE", "d4/dl")  # 4 x 64 KiB of slabs: does not fit
     k = kernels(HipBackend().compile(trace_module(*(lambda c: (c.module, c.inputs))(eager.linear_case(m=2048)))))[0]
-    assert k.knobs["TILE"] == "a:mfma_32x32x16_bf16/w2x4/f4x2/k4" and k.knobs["STAGE"] == "d2/dl"  # two slabs of it do
+    assert k.knobs["TILE"] == "a:mfma_32x32x16_bf16/w2x4/f4x2/k4" and k.knobs["STAGE"] == "d2/dlm"  # two slabs of it do (eight MFMAs a step: requests spread among the last step's)
 
 
 def test_candidate_rounds_cover_every_family_once():
