@@ -455,6 +455,14 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
         if max(M * lda, N * NB * ldb) * ES >= 2**32:
             raise LoweringError("contraction: STAGE .../dli addresses operands with 32-bit byte offsets; this operand is larger than 4 GiB")
         a("  unsigned va[A_PER_T], vb[B_PER_T];  // byte offset of each request's chunk from the operand base (the k position is added to the base, in scalar registers)")
+        # Request i of a thread is request 0 moved down ST / CPR rows (the chunk column is the same): where no row is
+        # clamped that is a constant added to the scalar base, and one lane offset serves every request of an operand.
+        lin_a = not m_guard and not dli
+        lin_b = not n_guard and not gate and not dli
+        # (... and the same swizzled chunk: the swizzle repeats every RPL * CPR rows)
+        lin = "(ST % CPR == 0 && (ST / CPR) % (RPL * CPR) == 0)"
+        a(f"  constexpr bool LIN_A = {lin if lin_a else 'false'}, LIN_B = {lin if lin_b else 'false'};")
+        a("  constexpr long STEP_A = LIN_A ? (long)(ST / CPR) * LDA * ES : 0, STEP_B = LIN_B ? (long)(ST / CPR) * LDB * ES : 0;")
         a("  const int wave_u = __builtin_amdgcn_readfirstlane(stid / 64);  // wave-uniform by construction; says so to the compiler")
         a("  const unsigned lds0 = emh_lds_addr(emh_lds);")
     a(r"""  #pragma unroll
@@ -658,8 +666,8 @@ ROW_EPILOGUE_TABLES
         if dli or dlm or spec:
             a(f"""  // One request of slab kt into ring buffer buf: the operand base moves along k in scalar registers, the
   // lane's chunk offset is a loop-invariant 32-bit register, the LDS target a scalar: no vector arithmetic per request.
-  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L + ASL) + (long)(kt) * (BK * ES), va[i], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * ST) * 16)
-  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L + BSL) + (long)(kt) * (BK * ES), vb[i], lds0 + (buf) * SLAB + TM * BK * ES + (wave_u * 64 + (i) * ST) * 16)""")
+  #define EMH_DPART_A(kt, buf, i) emh_dma16s((const unsigned char*)(A + {body.a_offset}L + ASL) + (long)(kt) * (BK * ES) + (long)(i) * STEP_A, va[LIN_A ? 0 : (i)], lds0 + (buf) * SLAB + (wave_u * 64 + (i) * ST) * 16)
+  #define EMH_DPART_B(kt, buf, i) emh_dma16s((const unsigned char*)(B + {body.b_offset}L + BSL) + (long)(kt) * (BK * ES) + (long)(i) * STEP_B, vb[LIN_B ? 0 : (i)], lds0 + (buf) * SLAB + TM * BK * ES + (wave_u * 64 + (i) * ST) * 16)""")
         if deferred:
             # the rows arrive in LDS untouched: every thread reads back the chunks it requested
             # (any chunk of the row will do for a row sum) while the slab is resident
@@ -683,9 +691,10 @@ ROW_EPILOGUE_TABLES
             part_fmt = [f"EMH_DPART_A({{slab}}, {{buf}}, {i});" for i in range(A_PER_T)] + [f"EMH_DPART_B({{slab}}, {{buf}}, {i});" for i in range(B_PER_T)]
             _emit_pingpong_loop(a, KT=KT, KS=KS, depth=depth, parts=part_fmt)
 
-        def mma_spread(P: int, kt: str) -> None:
+        def mma_spread(P: int, kt: str, read_next: str) -> None:
             """The MFMAs of a slab's last step with the requests of slab ``kt + DEPTH`` (into the buffer this slab leaves)
-            spread evenly among them."""
+            spread evenly among them.  The step's operands are in registers when the barrier opens, so the matrix pipe
+            gets its first MFMAs at once and the next slab's first fragment reads (``read_next``) follow them."""
             parts = [("A", i) for i in range(A_PER_T)] + [("B", i) for i in range(B_PER_T)]
             n = NB * FM * FN
             after = [(q * n) // len(parts) for q in range(len(parts))]
@@ -695,6 +704,8 @@ ROW_EPILOGUE_TABLES
                     for j in range(FN):
                         for e in range(MPF):
                             a(f"    acc[{h}][{i}][{j}] = {plan.atom.builtin}(EMH_OPND(fw[{P}][{h}][{j}], {e}), EMH_OPND(fx[{P}][{i}], {e}), acc[{h}][{i}][{j}], 0, 0, 0);")
+                        if idx == min(1, n - 1):
+                            a(f"    __builtin_amdgcn_sched_barrier(0); {read_next} __builtin_amdgcn_sched_barrier(0);")
                         for q, (which, pi) in enumerate(parts):
                             if after[q] == idx:
                                 a(f"    __builtin_amdgcn_sched_barrier(0); EMH_DPART_{which}(({kt}) + DEPTH, cur, {pi}); __builtin_amdgcn_sched_barrier(0);")
@@ -718,8 +729,7 @@ ROW_EPILOGUE_TABLES
                     if dlm:
                         # the buffer is free from here on (the last step's fragments are in registers): its next slab is
                         # requested one request at a time between this step's MFMAs instead of as a burst in front of them
-                        a(f"    EMH_READ({P ^ 1}, (({kt}) + 1) % DEPTH, 0);")
-                        mma_spread(P, kt)
+                        mma_spread(P, kt, read_next=f"EMH_READ({P ^ 1}, (({kt}) + 1) % DEPTH, 0);")
                         continue
                     a(f"    EMH_DLOAD(({kt}) + DEPTH, cur);")
                     a(f"    EMH_READ({P ^ 1}, (({kt}) + 1) % DEPTH, 0);")
