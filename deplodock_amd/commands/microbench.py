@@ -395,12 +395,82 @@ def handle_flash(args) -> None:
         print(line)
 
 
+def handle_stamps(args) -> None:
+    """Phase stamps of the default attention kernel and of the ring contractions (``-DEMH_STAMP=1`` / ``2`` builds of
+    ``emit/flash.py`` and ``emit/contraction.py``): the first thread of workgroup 0 leaves four floats over the first
+    16 bytes it stored — clocks per key step / slab by phase, and clocks per part of the kernel."""
+    import os
+
+    import torch
+
+    from deplodock_amd import HipBackend, trace_module, workloads
+    from deplodock_amd.commands.table import render_table
+    from deplodock_amd.ir.hip import HipOp
+
+    dev = torch.device("cuda:0")
+    saved = os.environ.get("EMMY_HIPRTC_FLAGS")
+
+    def run(case, mode, where):
+        if mode:
+            os.environ["EMMY_HIPRTC_FLAGS"] = f"-DEMH_STAMP={mode}"
+        else:
+            os.environ.pop("EMMY_HIPRTC_FLAGS", None)
+        be = HipBackend()
+        compiled = be.compile(trace_module(case.module, case.inputs))
+        (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+        data = {n: t.to(dev) for n, t in zip(compiled.inputs, case.inputs)}
+        if not mode:
+            res = be.benchmark(compiled, warmup=3, num_iters=30, input_data=data)
+            return op, res.time_ms * 1e3
+        prog = be.program(compiled, data)
+        try:
+            for _ in range(3):
+                prog.run()
+                torch.cuda.synchronize()
+            flat = prog.output_tensors()[compiled.outputs[0]].reshape(-1)
+            w = flat[where(op) : where(op) + 8].view(torch.float32)
+            return op, [w[i].item() for i in range(4)]
+        finally:
+            prog.close()
+
+    rows = []
+    try:
+        for seq in (2048, 512):
+            case = workloads.sdpa_case(s=seq)
+
+            def first_row(op, seq=seq):  # the first row workgroup 0 stores in its last pass: row 0 of a mirrored pair, else the last query block's
+                rows_wg = 32 * int(op.knobs["FLASH"].split("/")[0][1:])
+                return 0 if "/p" in op.knobs["FLASH"] else (seq - rows_wg) * 128
+
+            op, us = run(case, 0, first_row)
+            _, st = run(case, 1, first_row)
+            _, ph = run(case, 2, first_row)
+            rows.append([f"attention S={seq} {op.knobs['FLASH']}", f"{us:.2f}", "step: scores / softmax / output MFMAs / hand-over", *(f"{v:.0f}" for v in st)])
+            rows.append(["", "", "pass: prologue / key loop / close / store", *(f"{v:.0f}" for v in ph)])
+        for m, k, n in ((4096, 4096, 4096), (2048, 1024, 3072), (512, 1024, 3072)):
+            case = workloads.linear_case(m=m, k=k, n=n)
+            op, us = run(case, 0, lambda op: 0)
+            _, st = run(case, 1, lambda op: 0)
+            _, ph = run(case, 2, lambda op: 0)
+            what = "period: MFMAs / fragment reads / barrier / -" if op.knobs["STAGE"].endswith("/pp") else "slab: steps before / hand-over / last step / -"
+            rows.append([f"linear {m}x{k}x{n} {op.knobs['TILE'].split('/', 1)[1]} {op.knobs['STAGE']}", f"{us:.2f}", what, *(f"{v:.0f}" for v in st)])
+            rows.append(["", "", "kernel: prologue / k loop / epilogue arithmetic / stores", *(f"{v:.0f}" for v in ph)])
+    finally:
+        if saved is None:
+            os.environ.pop("EMMY_HIPRTC_FLAGS", None)
+        else:
+            os.environ["EMMY_HIPRTC_FLAGS"] = saved
+    for line in render_table(["kernel", "us", "clocks of workgroup 0's first wave", "a", "b", "c", "d"], rows, "lrlrrrr"):
+        print(line)
+
+
 def register_microbench_command(subparsers) -> None:
     p = subparsers.add_parser("microbench", help="Measure the MFMA rate, MFMA/VALU co-issue and the L1 fill rate of the GPU")
     p.add_argument("--l1fill", action="store_true", help="sweep load-only kernels: bytes per clock a CU pulls through its vector L1")
     p.add_argument("--quick", action="store_true", help="with --l1fill: a four-line sweep")
     p.add_argument("--lds", action="store_true", help="fragment-read rate out of LDS for the emitters' swizzled layouts")
     p.add_argument("--flash", action="store_true", help="phase stamps and ablations of the software-pipelined attention kernels on the benchmark shape")
+    p.add_argument("--stamps", action="store_true", help="phase stamps (shader clocks) of the default attention kernel and of the ring contractions on the benchmark shapes")
     p.add_argument("--pins", default=None, help="with --flash: comma-separated EMMY_FLASH pins (default: the ws and sp forms of the benchmark shape)")
     p.add_argument("--seq", default="2048", help="with --flash: sequence length")
     p.set_defaults(func=handle_microbench)
@@ -420,6 +490,9 @@ def handle_microbench(args) -> None:
         return
     if getattr(args, "flash", False):
         handle_flash(args)
+        return
+    if getattr(args, "stamps", False):
+        handle_stamps(args)
         return
     from deplodock_amd.backend.hip import launcher
     from deplodock_amd.commands.table import render_table

@@ -224,10 +224,13 @@ def _emit_pingpong_loop(a, *, KT: int, KS: int, depth: int, parts: list[str]) ->
     a("      EMH_PHASE_END(); }  // period -1")
     a(f"    for (int kt = 0; kt < {KT}; ++kt) {{")
     compute()
+    a("      EMH_STAMP_AT(0)  // this group's MFMAs issued")
     a(f"      if (kt + 1 < {KT}) {{")
     fetch("kt + 1")
     a("      }")
+    a("      EMH_STAMP_AT(1)  // the next slab's fragment reads issued")
     a("      EMH_PHASE_END();")
+    a("      EMH_STAMP_AT(2)  // the period's barrier")
     a("    }")
     a("  } else {  // ---- consumer group 1")
     a("    EMH_PHASE_END();  // period -1")
@@ -237,6 +240,11 @@ def _emit_pingpong_loop(a, *, KT: int, KS: int, depth: int, parts: list[str]) ->
     a("      EMH_PHASE_END();")
     a("    }")
     a("  }")
+
+
+#: fraction of the last step's MFMAs the ``dlm`` requests are spread over, and of a step's MFMAs the next step's fragment reads are
+_SPREAD = 1.0
+_READ_SPREAD = 0.5
 
 
 def emit_contraction(body: Contraction, name: str, ctx: Context = Context()) -> HipOp:
@@ -435,6 +443,17 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
   }
   const int m0 = tm * TM, n0 = tn * TN;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  // Measurement build (-DEMH_STAMP=1 or 2 among the compiler options): the first thread of workgroup 0 sums the clocks
+  // its slabs spend per phase of the k loop (1, averaged per slab) or the kernel spends per part (2: prologue / k loop /
+  // epilogue arithmetic / stores) and leaves four floats over the first 16 bytes of its output tile; the rest of the
+  // output is the product as usual.
+#ifndef EMH_STAMP
+#define EMH_STAMP 0
+#endif
+#define EMH_STAMP_AT(i) if (EMH_STAMP == 1) { const unsigned long long now_ = __builtin_readcyclecounter(); st_acc[i] += (unsigned)(now_ - st_last); st_last = now_; st_acc[4 + (i)] += 1u; }
+#define EMH_PHASE_AT(i) if (EMH_STAMP == 2) { const unsigned long long now_ = __builtin_readcyclecounter(); st_acc[i] += (unsigned)(now_ - st_last); st_last = now_; st_acc[4 + (i)] = 1u; }
+  unsigned st_acc[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+  unsigned long long st_last = EMH_STAMP ? __builtin_readcyclecounter() : 0ull;
   const int stid = tid >= T ? tid - T : tid;  // staging thread id (the waves past the tile's own only stage)
   const int wm = (wave / WN) % WM, wn = wave % WN;
   const int lr = lane % AM, lk = lane / AM;  // fragment row, k-group
@@ -535,6 +554,10 @@ EMH_DEV int emh_swz(int row, int c) { return c ^ ((row / RPL) % CPR); }
       const int row_ = (wm * FM + i) * AM + lr; \
       fx[P][i] = *(const FRAG_T*)(sA_ + row_ * (BK * ES) + emh_swz(row_, c_) * 16); } \
     __builtin_amdgcn_sched_barrier(0); }
+  #define EMH_READ_W(P, buf, kk, h, j) { const int row_ = (h) * TN + (wn * FN + (j)) * AM + lr; \
+    fw[P][h][j] = *(const FRAG_T*)(emh_lds + (buf) * SLAB + TM * BK * ES + row_ * (BK * ES) + emh_swz(row_, (kk) * KG + lk) * 16); }
+  #define EMH_READ_X(P, buf, kk, i) { const int row_ = (wm * FM + (i)) * AM + lr; \
+    fx[P][i] = *(const FRAG_T*)(emh_lds + (buf) * SLAB + row_ * (BK * ES) + emh_swz(row_, (kk) * KG + lk) * 16); }
   #define EMH_MMA(P) { \
     _Pragma("unroll") for (int e = 0; e < MPF; ++e) \
     _Pragma("unroll") for (int h = 0; h < NB; ++h) \
@@ -686,30 +709,40 @@ ROW_EPILOGUE_TABLES
         if not spec:
             a("  EMH_READ(0, 0, 0);")
         a("ROW_EPILOGUE_TABLES")
+        a("  EMH_PHASE_AT(0)  // tile decode, first requests, first slab landed")
+        a("  if (EMH_STAMP == 1) st_last = __builtin_readcyclecounter();")
         if pp:
             a("  const int role = __builtin_amdgcn_readfirstlane(tid / 256);  // 0, 1: the two consumer groups (waves 0-3, 4-7); 2: the producers")
             part_fmt = [f"EMH_DPART_A({{slab}}, {{buf}}, {i});" for i in range(A_PER_T)] + [f"EMH_DPART_B({{slab}}, {{buf}}, {i});" for i in range(B_PER_T)]
             _emit_pingpong_loop(a, KT=KT, KS=KS, depth=depth, parts=part_fmt)
 
-        def mma_spread(P: int, kt: str, read_next: str) -> None:
-            """The MFMAs of a slab's last step with the requests of slab ``kt + DEPTH`` (into the buffer this slab leaves)
-            spread evenly among them.  The step's operands are in registers when the barrier opens, so the matrix pipe
-            gets its first MFMAs at once and the next slab's first fragment reads (``read_next``) follow them."""
-            parts = [("A", i) for i in range(A_PER_T)] + [("B", i) for i in range(B_PER_T)]
+        def frag_reads(P: int, buf: str, kk: int) -> list[str]:
+            """One statement per fragment of step ``kk`` of the slab in ring buffer ``buf`` into register set ``P``."""
+            return [f"EMH_READ_W({P}, {buf}, {kk}, {h}, {j});" for h in range(NB) for j in range(FN)] + [f"EMH_READ_X({P}, {buf}, {kk}, {i});" for i in range(FM)]
+
+        def mma_interleaved(P: int, reads: list[str], requests: list[str]) -> None:
+            """The MFMAs of a step with the next step's fragment reads (over the first ``_READ_SPREAD`` of them: the data
+            has the rest of the step to arrive) and, in a slab's last step, the requests of slab ``kt + DEPTH`` (over the
+            first ``_SPREAD`` of them) issued one at a time in between: the matrix pipe always has an MFMA of this wave
+            queued behind whatever else the wave issues."""
             n = NB * FM * FN
-            after = [(q * n) // len(parts) for q in range(len(parts))]
-            idx = 0
-            for h in range(NB):
-                for i in range(FM):
-                    for j in range(FN):
-                        for e in range(MPF):
+            if 4 * n < 5 * len(reads):
+                # about as many reads as MFMAs: spread out, the last ones would land after the step that needs them has
+                # begun (512-token gate/up, six MFMAs and seven reads a step: 10.1 -> 11.2 us); they go out together
+                a("    " + " ".join(reads) + " __builtin_amdgcn_sched_barrier(0);")
+                reads = []
+            r_after = [int(q * n * _READ_SPREAD) // max(len(reads), 1) for q in range(len(reads))]
+            q_after = [int(q * n * _SPREAD) // max(len(requests), 1) for q in range(len(requests))]
+            for e in range(MPF):  # (the MFMAs a fragment feeds are a pass over all accumulators each, as in EMH_MMA)
+                idx = 0
+                for h in range(NB):
+                    for i in range(FM):
+                        for j in range(FN):
                             a(f"    acc[{h}][{i}][{j}] = {plan.atom.builtin}(EMH_OPND(fw[{P}][{h}][{j}], {e}), EMH_OPND(fx[{P}][{i}], {e}), acc[{h}][{i}][{j}], 0, 0, 0);")
-                        if idx == min(1, n - 1):
-                            a(f"    __builtin_amdgcn_sched_barrier(0); {read_next} __builtin_amdgcn_sched_barrier(0);")
-                        for q, (which, pi) in enumerate(parts):
-                            if after[q] == idx:
-                                a(f"    __builtin_amdgcn_sched_barrier(0); EMH_DPART_{which}(({kt}) + DEPTH, cur, {pi}); __builtin_amdgcn_sched_barrier(0);")
-                        idx += 1
+                            extra = [st for st, at in zip(reads, r_after) if at == idx] + [st for st, at in zip(requests, q_after) if at == idx] if e == 0 else []
+                            if extra:
+                                a("    __builtin_amdgcn_sched_barrier(0); " + " ".join(extra) + " __builtin_amdgcn_sched_barrier(0);")
+                            idx += 1
             a("    __builtin_amdgcn_sched_barrier(0);")
 
         def slab_steps(kt: str, static_kt: int | None) -> None:
@@ -723,13 +756,22 @@ ROW_EPILOGUE_TABLES
             for kk in range(KS):
                 P = kk & 1
                 if kk + 1 < KS:
+                    if dlm and static_kt is None:
+                        mma_interleaved(P, frag_reads(P ^ 1, "cur", kk + 1), [])
+                        if deferred and kk == 0:
+                            a("    EMH_SUMSQ_ADD();")
+                        continue
                     a(f"    EMH_READ({P ^ 1}, cur, {kk + 1});")
                 elif static_kt is None:
+                    a("    EMH_STAMP_AT(0)  // the steps before the hand-over issued")
                     a(f"    EMH_SLAB_SYNC({(depth - 2) * loads_per_slab});")
+                    a("    EMH_STAMP_AT(1)  // requests waited for, published, barrier")
                     if dlm:
                         # the buffer is free from here on (the last step's fragments are in registers): its next slab is
                         # requested one request at a time between this step's MFMAs instead of as a burst in front of them
-                        mma_spread(P, kt, read_next=f"EMH_READ({P ^ 1}, (({kt}) + 1) % DEPTH, 0);")
+                        parts = [f"EMH_DPART_A(({kt}) + DEPTH, cur, {i});" for i in range(A_PER_T)] + [f"EMH_DPART_B(({kt}) + DEPTH, cur, {i});" for i in range(B_PER_T)]
+                        mma_interleaved(P, frag_reads(P ^ 1, f"((({kt}) + 1) % DEPTH)", 0), parts)
+                        a("    EMH_STAMP_AT(2)  // the last step and the next slab's requests issued")
                         continue
                     a(f"    EMH_DLOAD(({kt}) + DEPTH, cur);")
                     a(f"    EMH_READ({P ^ 1}, (({kt}) + 1) % DEPTH, 0);")
@@ -740,6 +782,8 @@ ROW_EPILOGUE_TABLES
                         a(f"    EMH_DLOAD({static_kt + depth}, cur);")
                     a(f"    EMH_READ({P ^ 1}, {(static_kt + 1) % depth}, 0);")
                 a(f"    EMH_MMA({P});")
+                if static_kt is None and kk + 1 == KS:
+                    a("    EMH_STAMP_AT(2)  // the last step issued")
                 if deferred and kk == 0:
                     a("    EMH_SUMSQ_ADD();")
             a("    }")
@@ -807,6 +851,7 @@ ROW_EPILOGUE_TABLES
             for kt_s in range(steady, KT):
                 slab_steps(str(kt_s), kt_s)
 
+    a("  EMH_PHASE_AT(1)  // the k loop")
     # ---- epilogue ------------------------------------------------------------------
     esz = body.out_dtype.nbytes
     EPC = 16 // esz  # output elements per 16-byte chunk
@@ -876,6 +921,7 @@ ROW_EPILOGUE_TABLES
         a("  __syncthreads();")
         if spec:
             a("  if (tid >= T) return;  // no barrier follows")
+        a("  EMH_PHASE_AT(2)  // accumulators mapped, rounded and staged")
         vt_chunk = rt.vector_type(body.out_dtype.name, EPC)[0]
         a(f"  constexpr int CPRC = TN / {EPC};  // 16-byte chunks per output-tile row")
         if rowepi is not None:
@@ -912,6 +958,11 @@ ROW_EPILOGUE_TABLES
         a("  }")
         if rowepi is not None:
             a("  }")
+        a("  EMH_PHASE_AT(3)  // the tile stored")
+        a("  if (EMH_STAMP && bid == 0 && tid == 0) {  // over the 16 bytes this thread stored first: the start of its tile's first row")
+        a("    #pragma unroll")
+        a(f"    for (int i = 0; i < 4; ++i) ((float*)(O + {body.out_offset}L + OSL + (long)m0 * LDO + n0))[i] = (float)st_acc[i] / (float)(st_acc[4 + i] ? st_acc[4 + i] : 1u);")
+        a("  }")
     else:
         if rowepi is not None:
             raise LoweringError("contraction: the row epilogue works on the staged output tile, which this tile shape does not have")

@@ -110,6 +110,17 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
 #endif
   const ELT* kbase = Kp + K_OFF + (long)batch * K_SB + (long)kvh * K_SH + (long)QSHIFT * K_SS;
   const ELT* vbase = Vp + V_OFF + (long)batch * V_SB + (long)kvh * V_SH + (long)QSHIFT * V_SS;
+  // Measurement build (-DEMH_STAMP=1 or 2 among the compiler options): the first thread of workgroup 0 sums the clocks
+  // its key steps spend per phase (1: score phase / softmax / output MFMAs / end-of-step hand-over, averaged per step) or
+  // its passes spend per part (2: prologue / key loop / close / store) and leaves four floats in the first 16 bytes it
+  // stored itself; the rest of the output is the attention result as usual.
+#ifndef EMH_STAMP
+#define EMH_STAMP 0
+#endif
+#define EMH_STAMP_AT(i) if (EMH_STAMP == 1) { const unsigned long long now_ = __builtin_readcyclecounter(); st_acc[i] += (unsigned)(now_ - st_last); st_last = now_; st_acc[4 + (i)] += 1u; }
+#define EMH_PHASE_AT(i) if (EMH_STAMP == 2) { const unsigned long long now_ = __builtin_readcyclecounter(); st_acc[i] += (unsigned)(now_ - st_last); st_last = now_; st_acc[4 + (i)] = 1u; }
+  unsigned st_acc[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+  unsigned long long st_last = EMH_STAMP ? __builtin_readcyclecounter() : 0ull;
   #pragma unroll 1
   for (int pass = 0; pass < (PAIR ? 2 : 1); ++pass) {
   if (PAIR && pass) __syncthreads();  // every thread is done copying the first block's O tile out of LDS
@@ -271,6 +282,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       }
   }
 
+  EMH_PHASE_AT(0)
   // Steps run in pairs so that a step's ring slots (its parity) are known when the code is generated: the LDS
   // addresses of the fragment reads are then a loop-invariant lane offset plus an immediate, with no vector
   // arithmetic per step.
@@ -324,6 +336,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+      EMH_STAMP_AT(0)
       // The V operand fragments of the output MFMAs are requested here, behind the score MFMAs (where a lane
       // has the registers for them): they land while the matrix pipe works through the scores and the softmax
       // runs, instead of in front of each output MFMA.
@@ -408,6 +421,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         if (!MSUM) psum += p;
       }
       l_run += psum;
+      EMH_STAMP_AT(1)
       #pragma unroll
       for (int u = 0; u < BKV / 32; ++u)
       #pragma unroll
@@ -436,9 +450,12 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         }
       }
     }
+    EMH_STAMP_AT(2)
     // end of the step: everything but K(st + 2) has landed; every wave is done with K(st) and V(st)
     EMH_LAND((int)(DEEP && st + 2 < nsteps));
+    EMH_STAMP_AT(3)
   }
+  EMH_PHASE_AT(1)
 
   // ---- close.  The key-split groups share the final combine: group g finishes
   // registers [g*RPG, (g+1)*RPG) of its rows' RPL output registers.  Every group
@@ -538,6 +555,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
       }
     }
   }
+  EMH_PHASE_AT(2)
 #if KV_CTAS == 1
   __syncthreads();
   {
@@ -554,6 +572,11 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q
         y[2] = (x & 1) ? t[0] : t[2]; y[3] = (x & 1) ? t[1] : t[3];
         if (q0 + r < SQ && (DR == D || pc < DR / 8)) *(u32x4*)(obase + (long)(q0 + r) * O_SS + pc * 8) = y;
       }
+    }
+    EMH_PHASE_AT(3)
+    if (EMH_STAMP && bid == 0 && tid == 0 && pass == (PAIR ? 1 : 0)) {  // over the 16 bytes this thread has just stored: the first of row q0
+      #pragma unroll
+      for (int i = 0; i < 4; ++i) ((float*)(obase + (long)q0 * O_SS))[i] = (float)st_acc[i] / (float)(st_acc[4 + i] ? st_acc[4 + i] : 1u);
     }
   }
 #endif

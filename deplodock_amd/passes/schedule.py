@@ -377,12 +377,13 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
                 continue
             loads = (plan.tile_m + plan.tile_n * (2 if body.gate_pair else 1)) * (plan.bk_elems // 8) // plan.block_threads
             if (depth - 1) * loads <= 63:  # the vector-memory counter has six bits
-                # With four and more MFMAs a step per wave the next slab's requests go out one at a time between the MFMAs
-                # of the slab's last step (``dlm``) instead of as a burst in front of them: 4096^3 on the 256x256 tile
-                # 111 -> 103 us; in the decoder block at 2 048 tokens gate/up 29.9 -> 27.9, o_proj 13.3 -> 12.8, down_proj
-                # 18.4 -> 17.5 us, at 512 tokens q/k/v 9.6 -> 9.4 and gate/up 10.4 -> 10.1.  One-fragment waves (a single MFMA a
-                # step) have nothing to spread over and lose (down_proj at 512 tokens 8.0 -> 8.7 us): they keep the burst.
-                spread = plan.regs[0] * plan.regs[1] * (2 if body.gate_pair else 1) >= 4
+                # With eight and more MFMAs a step per wave the next slab's requests and the next step's fragment reads go
+                # out one at a time between the MFMAs (``dlm``) instead of as a burst in front of them: 4096^3 on the 256x256
+                # tile 111 -> 98.5 us; in the decoder block at 2 048 tokens q/k/v 31.4 -> 26.2, gate/up 29.9 -> 28.4 us.  Tiles
+                # with fewer MFMAs a step have too little to spread over: four to six a step measured within +-4 % either
+                # way depending on the box (gate/up at 512 tokens 10.4 -> 10.1 on one, 10.9 -> 11.4 on another), one a step
+                # loses (down_proj at 512 tokens 8.0 -> 8.7 us): they keep the burst.
+                spread = plan.regs[0] * plan.regs[1] * (2 if body.gate_pair else 1) >= 8
                 return Stage(depth=depth, transport="dlm" if spread else "dl")
     return Stage(depth=2, transport="sync")
 

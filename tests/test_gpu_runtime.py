@@ -244,3 +244,40 @@ def test_empty_inputs_run_and_return_empty_outputs(device, which):
     res, _ = be.run(compiled, input_data={compiled.inputs[0]: x.to(device)})
     out = res.outputs[compiled.outputs[0]]
     assert out.size == 0 and tuple(out.shape) == tuple(mod(x).shape)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("what", ["attention", "linear_dlm", "linear_pp"])
+def test_a_stamped_build_computes_the_same_result_and_leaves_its_clocks_in_the_first_words(device, what, monkeypatch):
+    """The measurement build (``-DEMH_STAMP=1``) is the product kernel plus clock reads: apart from the 16 bytes the
+    stamps are left in, its output is bit for bit the plain build's, and the four stamps are positive clock counts."""
+    from deplodock_amd import workloads as wl
+
+    case = {"attention": lambda: wl.sdpa_case(s=512), "linear_dlm": lambda: wl.linear_case(m=1024, k=1024, n=4096), "linear_pp": lambda: wl.linear_case(m=2048)}[what]()
+    if what == "linear_dlm":
+        monkeypatch.setenv("EMMY_TILE", "a:mfma_16x16x32_bf16/w2x4/f8x4/k2")
+    outs = []
+    for flags in (None, "-DEMH_STAMP=1"):
+        if flags:
+            monkeypatch.setenv("EMMY_HIPRTC_FLAGS", flags)
+        be = HipBackend()
+        compiled = be.compile(trace_module(case.module, case.inputs))
+        (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+        if what != "attention":
+            assert op.knobs["STAGE"].endswith("/dlm" if what == "linear_dlm" else "/pp"), op.knobs
+        prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, case.inputs)})
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            outs.append((prog.output_tensors()[compiled.outputs[0]].reshape(-1).clone(), op))
+        finally:
+            prog.close()
+    (plain, _), (stamped, op) = outs
+    # workgroup 0 leaves the stamps over the first 16 bytes it stored: the start of the output for the contractions, of
+    # its query block's first row for attention (the last block of head 0: 512 tokens run unpaired)
+    at = 0 if what != "attention" else (512 - 32 * int(op.knobs["FLASH"].split("/")[0][1:])) * 128
+    stamps = stamped[at : at + 8].view(torch.float32)
+    assert bool((stamps[:3] > 0).all()) and bool((stamps < 1e7).all()), stamps
+    keep = torch.ones_like(plain, dtype=torch.bool)
+    keep[at : at + 8] = False
+    assert torch.equal(plain[keep], stamped[keep])

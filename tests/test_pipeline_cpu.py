@@ -201,9 +201,12 @@ def test_head_norm_and_rope_fold_into_the_projection(launcher_lib, monkeypatch):
 def test_deferred_norm_takes_the_direct_to_lds_ring_at_prefill_sizes(launcher_lib):
     ks = kernels(compile_case(eager.qwen3_block_case(seq=512)))
     qkv, gate_up = ks[0], ks[3]
-    # four and more MFMAs a step per wave: the next slab's requests are spread among the MFMAs of the slab's last step
-    assert qkv.knobs["STAGE"] == "d3/dlm" and gate_up.knobs["STAGE"] == "d3/dlm" and ks[2].knobs["STAGE"] == ks[4].knobs["STAGE"] == "d3/dl"
-    assert qkv.kernel_source.count("EMH_DPART_A((kt) + DEPTH, cur,") >= 1 and "EMH_DLOAD((kt) + DEPTH, cur);" not in qkv.kernel_source
+    assert all(k.knobs["STAGE"] == "d3/dl" for k in (ks[0], ks[2], ks[3], ks[4]))  # four to six MFMAs a step: the request burst stays
+    # eight and more MFMAs a step per wave (2 048 tokens: the q/k/v projection's 128x256 tile): the next slab's requests and the
+    # next step's fragment reads go out one at a time between the MFMAs
+    big = kernels(compile_case(eager.qwen3_block_case(seq=2048)))[0]
+    assert big.knobs["STAGE"].endswith("/dlm") and "EMH_DPART_A((kt) + DEPTH, cur," in big.kernel_source and "EMH_DLOAD((kt) + DEPTH, cur);" not in big.kernel_source
+    assert "EMH_READ_W(" in big.kernel_source and "EMH_READ_X(" in big.kernel_source
     assert gate_up.knobs["TILE"].endswith("/w4x2/f1x3/k2") and gate_up.grid[0][0] == 256  # 64x96 tiles: one workgroup per CU
     for k in (qkv, gate_up):
         assert "a=row-scaled-after" in k.comment and "#define EMH_SUMSQ_READ(buf)" in k.kernel_source and "EMH_SUMSQ_ADD();" in k.kernel_source
@@ -606,3 +609,20 @@ def test_matmul_spelled_attention_lowers_to_batched_contractions(launcher_lib):
     assert "K=104" in ks[-1].comment
     for k in ks:
         hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)
+
+
+@pytest.mark.parametrize("mode", [1, 2])
+def test_stamped_measurement_builds_of_the_attention_and_ring_contraction_kernels_compile(launcher_lib, mode, monkeypatch):
+    """``-DEMH_STAMP=1|2`` among the compiler options builds the same kernels with shader-clock stamps at their phase
+    boundaries (``microbench --stamps`` reads them): the stamped sources of the default attention kernel, the burst and
+    spread direct-to-LDS rings and the wave-specialised ring build without spills; without the define the statements are
+    compiled out (same source text, the define decides)."""
+    monkeypatch.setenv("EMMY_HIPRTC_FLAGS", f"-DEMH_STAMP={mode}")
+    cases = [eager.sdpa_case(), eager.sdpa_case(s=512), eager.linear_case(m=4096, k=4096, n=4096), eager.linear_case(m=2048), eager.linear_case(m=512)]
+    stages = []
+    for case in cases:
+        (k,) = kernels(compile_case(case))
+        assert "EMH_STAMP_AT(" in k.kernel_source and "EMH_PHASE_AT(" in k.kernel_source and "#ifndef EMH_STAMP" in k.kernel_source
+        assert hiprtc.spilled_vgprs(k.kernel_source, k.kernel_name) == 0, k.kernel_name
+        stages.append(k.knobs.get("STAGE"))
+    assert stages[2:] == ["d2/dlm", "d4/pp", "d3/dl"]
