@@ -618,6 +618,10 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         from deplodock_amd.emit.flash_ws import emit_flash_ws
 
         return emit_flash_ws(body, name, ctx)
+    if body.dtype.name == "f32":
+        from deplodock_amd.emit.flash_f32 import emit_flash_f32
+
+        return emit_flash_f32(body, name, ctx)
     D = body.head_dim
     if body.dtype.name not in ("bf16", "f16"):
         raise LoweringError("flash: MFMA tier needs 16-bit operands")

@@ -1,6 +1,7 @@
-"""Attention outside the flash kernel's reach is decomposed into loop nests before fusion.
+"""Attention outside the streaming kernels' reach is decomposed into loop nests before fusion.
 
-The flash kernel serves 16-bit operands with head_dim 64 / 128 / 256.  The reference compiles fp32 only and its
+The flash kernels serve 16-bit operands whose rows are whole 16-byte chunks up to head_dim 256, and fp32 operands of any
+head_dim up to 256; what is left is 16-bit rows of other lengths, wider head dims, and mixed operand types.  The reference compiles fp32 only and its
 perf cases call ``F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=...)`` on fp32 tensors
 (tests/perf/cases.py:64-69, 174-190); it lowers the fused op by decomposing it into ``q k^T -> * scale -> [+ mask] ->
 softmax -> @ v`` (emmy/compiler/pipeline/passes/frontend/decomposition/010_sdpa.py:53-138: grouped KV heads by
@@ -31,6 +32,13 @@ def flash_head_dim(d: int) -> int | None:
     return next((w for w in FLASH_HEAD_DIMS if w >= d), None)
 
 
+def f32_head_dim(d) -> bool:
+    """Whether the fp32 streaming kernel takes rows of ``d`` values (``emit/flash_f32.py``: up to 256, any alignment)."""
+    from deplodock_amd.emit.flash_f32 import f32_supported
+
+    return isinstance(d, int) and f32_supported(d)
+
+
 #: largest scores tensor ``[batch..., heads, queries, keys]`` the decomposed route writes to device memory
 SCORES_LIMIT_BYTES = 8 * 2**30
 
@@ -41,7 +49,7 @@ class AttentionShapeError(ValueError):
 
 def _static(shape) -> tuple[int, ...]:
     if not all(isinstance(d, int) for d in shape):
-        raise AttentionShapeError("attention outside the flash kernel (fp32, or a head_dim other than 64 / 128 / 256) needs static shapes")
+        raise AttentionShapeError("attention outside the streaming kernels (16-bit rows that are not whole 16-byte chunks, head dims beyond 256) needs static shapes")
     return tuple(int(d) for d in shape)
 
 
@@ -106,8 +114,8 @@ def _decompose(g: Graph, node: Node, undo_repeat) -> list[Node]:
     scores_bytes = math.prod(scores_shape) * dtype.nbytes
     if scores_bytes > SCORES_LIMIT_BYTES:
         raise AttentionShapeError(
-            f"sdpa: the decomposed route (operands wider than 16 bits, or rows that are not whole 16-byte chunks) would materialise {scores_bytes / 2**30:.1f} GiB of scores "
-            f"{scores_shape}; the limit is {SCORES_LIMIT_BYTES / 2**30:.0f} GiB — run the module in bf16 / fp16 (streamed by the flash kernel) or on shorter sequences"
+            f"sdpa: the decomposed route (16-bit rows that are not whole 16-byte chunks, head dims beyond 256) would materialise {scores_bytes / 2**30:.1f} GiB of scores "
+            f"{scores_shape}; the limit is {SCORES_LIMIT_BYTES / 2**30:.0f} GiB — pad the head_dim to whole 16-byte chunks (streamed by the flash kernel) or run shorter sequences"
         )
     head = [L.Load("c_scale", "scale", (L.Lit(0),))]
     scalars = {"scale": scale}
@@ -159,16 +167,26 @@ def _decompose(g: Graph, node: Node, undo_repeat) -> list[Node]:
     return [n1, n2]
 
 
-def decompose_attention(g: Graph, undo_repeat) -> Graph:
-    """``g`` with every ``SdpaOp`` the flash kernel does not take (operands wider than 16 bits, or a head_dim it has
-    no tiling for) replaced by the two loop nests of the decomposed form; a new graph when anything changed.
-    ``undo_repeat(g, node id) -> (source id, group)`` sees through a materialised head repeat."""
+def decompose_attention(g: Graph, undo_repeat, streamed=None) -> Graph:
+    """``g`` with every ``SdpaOp`` no streaming kernel takes (16-bit rows that are not whole 16-byte chunks, head dims
+    beyond 256, value rows of another length than the keys') replaced by the two loop nests of the decomposed form; a new
+    graph when anything changed.  ``undo_repeat(g, node id) -> (source id, group)`` sees through a materialised head
+    repeat; ``streamed(node) -> bool`` replaces the rule for which ops stay fused."""
 
     def flash_takes(node: Node) -> bool:
-        t = g.nodes[node.inputs[0]].output
-        return t.dtype.name in ("bf16", "f16") and flash_head_dim(int(t.shape[-1])) is not None
+        q, k, v = (g.nodes[i].output for i in node.inputs[:3])
+        if q.dtype.name == "f32":
+            # the fp32 streaming kernel: any row length it has registers for, q / k / v rows alike
+            if not (k.dtype.name == v.dtype.name == "f32" and f32_head_dim(q.shape[-1]) and k.shape[-1] == v.shape[-1] == q.shape[-1]):
+                return False
+            if node.op.has_mask:  # the kernel reads a mask with the keys along its last axis; a column mask is left to the decomposed form
+                m = g.nodes[node.inputs[3]].output
+                if len(m.shape) > 4 or len(m.shape) < 1 or m.shape[-1] != k.shape[-2] or (k.shape[-2] == 1 and len(m.shape) > 1):
+                    return False
+            return True
+        return q.dtype.name in ("bf16", "f16") and flash_head_dim(int(q.shape[-1])) is not None
 
-    hits = [nid for nid, n in g.nodes.items() if isinstance(n.op, F.SdpaOp) and not flash_takes(n)]
+    hits = [nid for nid, n in g.nodes.items() if isinstance(n.op, F.SdpaOp) and not (streamed or flash_takes)(n)]
     if not hits:
         return g
     out = Graph()

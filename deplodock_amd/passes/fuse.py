@@ -1242,8 +1242,9 @@ def _rec_sdpa(c: _Ctx, nid: str) -> bool:
         inputs.append(mv.base)
     from deplodock_amd.passes.decompose_attention import flash_head_dim
 
+    width = D if q.dtype == F32 else (flash_head_dim(D) or D)  # (the fp32 kernel pads its tiles itself)
     body = Flash(
-        batch=B, q_heads=Hq, kv_heads=Hkv, q_len=Sq, kv_len=Skv, head_dim=flash_head_dim(D) or D, head_dim_real=D if (flash_head_dim(D) or D) != D else None,
+        batch=B, q_heads=Hq, kv_heads=Hkv, q_len=Sq, kv_len=Skv, head_dim=width, head_dim_real=D if width != D else None,
         q=q.base, k=k.base, v=v.base, out=out_id, dtype=q.dtype,
         scale=float(scale), causal=node.op.is_causal, q_strides=q_str, k_strides=k_str, v_strides=v_str, o_strides=o_strides,
         q_offset=q.offset, k_offset=k.offset, v_offset=v.offset, **mask_kw,

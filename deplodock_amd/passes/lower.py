@@ -212,6 +212,8 @@ def _lower_flash(op: TileOp, ctx: Context) -> HipOp:
     one (two row groups x four key-split groups on 32-key blocks)."""
     body = op.body
     hip = _named(emit_flash(body, _PLACEHOLDER, ctx), op)
+    if body.dtype.name == "f32":
+        return hip  # one shape, sized to a wave's registers for every head_dim it takes
     steps = (("pair_steps", False), ("pair", False), ("shape", None))
     for what, value in steps:
         spilled = _spills(hip, ctx)

@@ -552,6 +552,8 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
     560 against 637 for ``w4/kv64/s2``, causal 303 against 351; S=16384 causal 1087 / 1239;
     batch 4 S=2048 causal ``w8/kv64/s1/p`` 104 / 117; 16 heads S=4096 causal, 256 such
     workgroups unpaired: 122 against 94, hence the 2x cover asked of an unpaired triangle)."""
+    if body.dtype.name == "f32":
+        return _schedule_flash_f32(body, ctx)
     pinned = _pin("FLASH", _tuned(body, ctx))
     if pinned:
         try:
@@ -649,6 +651,44 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
         body.pair = False  # pairing mirrored query blocks needs the block count when the kernel is built
     knobs = _schedule_flash_split(body, ctx, tuned if (tuned := _tuned(body, ctx)) else None)
     return {**knobs, "FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "") + ("/k3" if body.deep else "") + ("/ws" if body.ws else "") + ("/sp" if body.sp else "")}
+
+
+def _schedule_flash_f32(body: Flash, ctx: Context) -> dict:
+    """``EMMY_FLASH=f32/w<row groups>`` or ``f32/s<key-split waves>``.
+
+    ``w<n>``: 1, 2 or 4 groups of 32 query rows per 256-thread workgroup share each K / V block (the other waves only stage).
+    ``s<k>``: one group of 32 rows per workgroup whose 2, 4 or 8 waves split the key blocks and stage for themselves.
+    Default: the key-split form wherever rows are whole aligned 16-byte chunks of at most 128 values — four waves, two
+    from four workgroups per CU on (measured, 16 / 8 heads of 128, causal, us, ``w4`` / ``s2`` / ``s4``: S=128 25.7 / 15.6 /
+    10.9, 512: 86.5 / 47.4 / 27.3, 1024: 166 / 90.9 / 58.9, 2048: 325 / 196 / 209, 4096: 761 / 766 / 800) — except for a
+    single key block, where there is nothing to split (S=32: 7.4 against 9.9); else the most row groups that still give
+    every CU a workgroup."""
+    from deplodock_amd.emit.flash_f32 import max_key_split, whole_chunk_rows
+
+    body.pair = body.deep = body.ws = body.sp = body.mfma_sum = False
+    body.kv_ctas, body.block_kv = 1, 32
+    heads = body.batch * body.q_heads
+    can_split = all(whole_chunk_rows(body))
+    most = min(4, max_key_split(body.head_dim, ctx.lds_bytes_per_cu)) if can_split else 1
+    symbolic = getattr(body, "sym", None) is not None and bool(body.sym.fields)
+    if most > 1 and (body.kv_len > 32 or symbolic):
+        body.waves, body.kv_split = 1, (2 if heads * -(-body.q_len // 32) >= 4 * ctx.compute_units else most)
+    else:
+        body.waves, body.kv_split = next((w for w in (4, 2) if heads * -(-body.q_len // (32 * w)) >= ctx.compute_units), 1), 1
+    pinned = _pin("FLASH", _tuned(body, ctx))
+    if pinned and pinned.split("/")[0] == "f32":
+        try:
+            (tok,) = pinned.split("/")[1:]
+            n = int(tok[1:])
+            if tok[0] == "w" and n in (1, 2, 4):
+                body.waves, body.kv_split = n, 1
+            elif tok[0] == "s" and n in (2, 4, 8) and can_split and n <= max_key_split(body.head_dim, ctx.lds_bytes_per_cu):
+                body.waves, body.kv_split = 1, n
+            else:
+                raise ValueError(tok)
+        except ValueError:
+            logger.warning("EMMY_FLASH=%r ignored: expect f32/w1, f32/w2, f32/w4 or f32/s2, f32/s4, f32/s8 (rows of whole 16-byte chunks, regions within the LDS)", pinned)
+    return {"FLASH": f"f32/s{body.kv_split}" if body.kv_split > 1 else f"f32/w{body.waves}"}
 
 
 def _schedule_flash_split(body: Flash, ctx: Context, tuned: dict | None) -> dict:

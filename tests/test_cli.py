@@ -151,7 +151,7 @@ def test_compile_a_built_in_architecture_whole_and_by_layer(capsys):
     assert out.count("k_index_rows") >= 1 and out.count("// ---- k_sdpa_reduce") == 2  # embedding gather, two layers
     main(["compile", "arch:qwen3-tiny", "--layer", "1", "--seq-len", "48", "--dtype", "fp32"])
     out = capsys.readouterr().out
-    assert "k_index_rows" not in out and out.count("// ---- k_batched_linear") == 2  # one layer; fp32 attention is decomposed
+    assert "k_index_rows" not in out and out.count("// ---- k_sdpa_reduce") == 1 and "mfma_f32_32x32x2f32" in out  # one layer; fp32 attention streams on fp32 atoms
 
 
 def test_compile_a_local_model_directory(tmp_path, capsys):

@@ -1,4 +1,4 @@
-"""Attention the flash kernel does not take (fp32 operands, other head dims) is decomposed into the two loop nests
+"""Attention no streaming kernel takes (16-bit rows that are not whole 16-byte chunks, head dims beyond 256) is decomposed into the two loop nests
 the reference's own pipeline reaches (masked scores; softmax times v).  Pinned on the host: the two nests,
 evaluated by the Loop-IR restatement in float64, equal ``F.scaled_dot_product_attention`` in float64 — a wrong
 head-group index, mask predicate, scale or broadcast is an error of order one."""
@@ -59,7 +59,7 @@ def test_decomposed_nests_equal_eager_attention(case):
     torch.manual_seed(5)
     args = [torch.randn(*s) for s in shapes] + ([mask()] if mask else [])
     g = trace_module(mod.eval(), tuple(args))
-    d = decompose_attention(g, _undo_repeat_kv)
+    d = decompose_attention(g, _undo_repeat_kv, streamed=lambda node: False)  # (fp32 operands of these sizes would stay fused)
     assert not any(isinstance(n.op, F.SdpaOp) for n in d.nodes.values())
     nests = [n for n in d.nodes.values() if isinstance(n.op, F.LoopNestOp)]
     assert [n.op.label for n in nests] == ["sdpa_scores", "sdpa_softmax_v"]
@@ -82,14 +82,20 @@ def _kernel_names(compiled):
 
 
 def test_which_attention_is_decomposed():
-    """fp32, and 16-bit with a head_dim that is not whole 16-byte chunks, become two batched contractions with loop-nest
-    operand / output stages; 16-bit head_dim 128 stays the one fused kernel, and a 16-bit head_dim between the kernel's
-    widths (32: padded to 64 with columns that count as zeros) takes it too."""
+    """16-bit rows that are not whole 16-byte chunks, fp32 head dims beyond 256 and value rows of another length than the
+    keys' become two batched contractions with loop-nest operand / output stages; fp32 up to head_dim 256 is one streaming
+    kernel on fp32 atoms, 16-bit head_dim 128 the one fused kernel, and a 16-bit head_dim between the kernel's widths
+    (32: padded to 64 with columns that count as zeros) takes it too."""
     be = HipBackend()
     q, k = torch.randn(1, 16, 128, 128), torch.randn(1, 8, 128, 128)
-    names = _kernel_names(be.compile(trace_module(_Sdpa(is_causal=True, enable_gqa=True).eval(), (q, k, k))))
-    assert names.count("k_batched_linear") == 2 and "k_sdpa_reduce" not in names
-    assert names.count("k_operand_a") == 1  # q is read in place; only the softmax is an operand stage of its own
+    compiled = be.compile(trace_module(_Sdpa(is_causal=True, enable_gqa=True).eval(), (q, k, k)))
+    assert _kernel_names(compiled) == ["k_sdpa_reduce"]
+    (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert "mfma_f32_32x32x2f32" in op.kernel_source and op.knobs["FLASH"].startswith("f32/")
+    for shapes in ([(1, 2, 40, 320)] * 3, [(1, 2, 40, 16), (1, 2, 40, 16), (1, 2, 40, 24)]):
+        names = _kernel_names(be.compile(trace_module(_Sdpa().eval(), tuple(torch.randn(*s) for s in shapes))))
+        assert names.count("k_batched_linear") == 2 and "k_sdpa_reduce" not in names
+        assert names.count("k_operand_a") == 1  # q is read in place; only the softmax is an operand stage of its own
     names = _kernel_names(be.compile(trace_module(_Sdpa(is_causal=True, enable_gqa=True).eval(), (q.bfloat16(), k.bfloat16(), k.bfloat16()))))
     assert names == ["k_sdpa_reduce"]
     q32 = torch.randn(2, 4, 64, 32).bfloat16()
@@ -117,6 +123,46 @@ def test_a_scores_tensor_beyond_the_limit_is_refused_with_a_message():
     the module is compiled, not when the runtime asks for the memory."""
     from deplodock_amd.passes.fuse import FusionError
 
-    q = torch.zeros(1, 32, 16384, 8)
-    with pytest.raises(FusionError, match="32.0 GiB of scores"):
+    q = torch.zeros(1, 32, 16384, 12).bfloat16()
+    with pytest.raises(FusionError, match="16.0 GiB of scores"):
         HipBackend().compile(trace_module(_Sdpa(is_causal=True).eval(), (q, q, q)))
+
+
+@pytest.mark.parametrize("head_dim, form", [(3, "w1"), (21, "w4"), (40, "s4"), (64, "s8"), (128, "s4"), (128, "s2"), (128, "w4"), (200, "w2"), (256, "w1")])
+def test_fp32_streaming_attention_builds_without_spills(head_dim, form, monkeypatch):
+    """Every head_dim up to 256 and both forms of the fp32 streaming kernel build within a wave's registers (the
+    key-split form counts its outstanding direct-to-LDS requests, which spill traffic would disturb); the key-split
+    form is refused — and the shared form taken — for rows that are not whole 16-byte chunks or wider than 128 values."""
+    from deplodock_amd.backend.hip import hiprtc, launcher
+
+    monkeypatch.setenv("EMMY_FLASH", f"f32/{form}")
+    q = torch.randn(1, 4, 70, head_dim)
+    k = torch.randn(1, 2, 90, head_dim)
+    compiled = HipBackend().compile(trace_module(_Sdpa(enable_gqa=True).eval(), (q, k, k, torch.randn(70, 90))))
+    (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert op.knobs["FLASH"] == f"f32/{form}" and "mfma_f32_32x32x2f32" in op.kernel_source
+    assert op.block[0] == ((64 * int(form[1:]),) if form[0] == "s" else (256,))
+    try:
+        assert hiprtc.spilled_vgprs(op.kernel_source, op.kernel_name) == 0
+    except launcher.CompileError:
+        raise
+    except launcher.LauncherError:
+        pytest.skip("no launcher library: the code object is not built here")
+
+
+def test_fp32_streaming_attention_default_forms(monkeypatch):
+    monkeypatch.delenv("EMMY_FLASH", raising=False)
+
+    def form(q_shape, kv_shape):
+        q, k = torch.randn(*q_shape), torch.randn(*kv_shape)
+        (op,) = [n.op for n in HipBackend().compile(trace_module(_Sdpa(is_causal=True, enable_gqa=True).eval(), (q, k, k))).nodes.values() if isinstance(n.op, HipOp)]
+        return op.knobs["FLASH"]
+
+    assert form((1, 16, 32, 128), (1, 8, 32, 128)) == "f32/w1"  # one key block: nothing to split
+    assert form((1, 16, 512, 128), (1, 8, 512, 128)) == "f32/s4"
+    assert form((1, 16, 2048, 128), (1, 8, 2048, 128)) == "f32/s2"  # four workgroups per CU and more
+    assert form((1, 2, 40, 21), (1, 2, 40, 21)) == "f32/w1"  # rows that are not whole 16-byte chunks
+    assert form((1, 2, 40, 256), (1, 2, 40, 256)) == "f32/w1"  # beyond 128 columns
+    # a pin the shape cannot take is ignored
+    monkeypatch.setenv("EMMY_FLASH", "f32/s4")
+    assert form((1, 2, 40, 21), (1, 2, 40, 21)) == "f32/w1"

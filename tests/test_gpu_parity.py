@@ -1332,29 +1332,120 @@ class _RepeatKvAttention(nn.Module):
         return torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
 
 
-_DECOMPOSED_ATTENTION = {
+_FP32_ATTENTION = {
     # the reference's fp32 perf cases: q [1, 16, S, 128], k / v [1, 8, S, 128], causal, grouped heads (tests/perf/cases.py:174-190)
-    "perf_s32": (_FusedAttention(is_causal=True, enable_gqa=True), torch.float32, [(1, 16, 32, 128), (1, 8, 32, 128), (1, 8, 32, 128)], None),
-    "perf_s128": (_FusedAttention(is_causal=True, enable_gqa=True), torch.float32, [(1, 16, 128, 128), (1, 8, 128, 128), (1, 8, 128, 128)], None),
-    "perf_s512": (_FusedAttention(is_causal=True, enable_gqa=True), torch.float32, [(1, 16, 512, 128), (1, 8, 512, 128), (1, 8, 512, 128)], None),
-    "ragged_keys": (_FusedAttention(), torch.float32, [(2, 4, 100, 64), (2, 4, 100, 64), (2, 4, 100, 64)], None),
-    "ragged_everything": (_FusedAttention(is_causal=True), torch.float32, [(1, 2, 33, 21), (1, 2, 33, 21), (1, 2, 33, 21)], None),
-    "cross_gqa": (_FusedAttention(enable_gqa=True, scale=0.2), torch.float32, [(1, 4, 50, 40), (1, 2, 70, 40), (1, 2, 70, 40)], None),
-    "mask_1_1_s_s": (_FusedAttention(), torch.float32, [(2, 3, 72, 64)] * 3, lambda: torch.zeros(72, 72).masked_fill(torch.arange(72)[None, :] > torch.arange(72)[:, None], float("-inf"))[None, None]),
-    "mask_per_batch_keys": (_FusedAttention(), torch.float32, [(2, 4, 40, 32)] * 3, lambda: torch.randn(2, 1, 1, 40)),
-    "token_major": (_TokenMajorAttention(), torch.float32, [(1, 128, 16, 128), (1, 128, 8, 128), (1, 128, 8, 128)], None),
-    "repeat_kv": (_RepeatKvAttention(), torch.float32, [(2, 8, 64, 64), (2, 2, 64, 64), (2, 2, 64, 64)], None),
+    "perf_s32": (_FusedAttention(is_causal=True, enable_gqa=True), [(1, 16, 32, 128), (1, 8, 32, 128), (1, 8, 32, 128)], None),
+    "perf_s128": (_FusedAttention(is_causal=True, enable_gqa=True), [(1, 16, 128, 128), (1, 8, 128, 128), (1, 8, 128, 128)], None),
+    "perf_s512": (_FusedAttention(is_causal=True, enable_gqa=True), [(1, 16, 512, 128), (1, 8, 512, 128), (1, 8, 512, 128)], None),
+    "perf_s2048": (_FusedAttention(is_causal=True, enable_gqa=True), [(1, 16, 2048, 128), (1, 8, 2048, 128), (1, 8, 2048, 128)], None),
+    "ragged_keys": (_FusedAttention(), [(2, 4, 100, 64), (2, 4, 100, 64), (2, 4, 100, 64)], None),
+    "ragged_everything": (_FusedAttention(is_causal=True), [(1, 2, 33, 21), (1, 2, 33, 21), (1, 2, 33, 21)], None),
+    "cross_gqa": (_FusedAttention(enable_gqa=True, scale=0.2), [(1, 4, 50, 40), (1, 2, 70, 40), (1, 2, 70, 40)], None),
+    "cross_causal_more_keys": (_FusedAttention(is_causal=True), [(2, 3, 45, 32), (2, 3, 150, 32), (2, 3, 150, 32)], None),
+    "cross_causal_more_queries": (_FusedAttention(is_causal=True), [(1, 3, 150, 32), (1, 3, 45, 32), (1, 3, 45, 32)], None),
+    "one_query_long_cache": (_FusedAttention(enable_gqa=True), [(2, 8, 1, 128), (2, 2, 1000, 128), (2, 2, 1000, 128)], None),
+    "head_dim_256": (_FusedAttention(is_causal=True), [(1, 3, 200, 256)] * 3, None),
+    "head_dim_3": (_FusedAttention(), [(1, 2, 70, 3)] * 3, None),
+    "mask_1_1_s_s": (_FusedAttention(), [(2, 3, 72, 64)] * 3, lambda: torch.zeros(72, 72).masked_fill(torch.arange(72)[None, :] > torch.arange(72)[:, None], float("-inf"))[None, None]),
+    "mask_per_batch_keys": (_FusedAttention(), [(2, 4, 40, 32)] * 3, lambda: torch.randn(2, 1, 1, 40)),
+    "mask_full_odd_keys": (_FusedAttention(), [(2, 2, 37, 20), (2, 2, 51, 20), (2, 2, 51, 20)], lambda: torch.randn(2, 2, 37, 51)),
+    "mask_s_s": (_FusedAttention(), [(1, 2, 64, 16)] * 3, lambda: torch.randn(64, 64)),
+    "token_major": (_TokenMajorAttention(), [(1, 128, 16, 128), (1, 128, 8, 128), (1, 128, 8, 128)], None),
+    "repeat_kv": (_RepeatKvAttention(), [(2, 8, 64, 64), (2, 2, 64, 64), (2, 2, 64, 64)], None),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", sorted(_FP32_ATTENTION))
+def test_fp32_attention_streams_on_fp32_atoms(device, case):
+    """The fused attention op on fp32 operands (what the reference's perf suite runs) is one streaming kernel on fp32 MFMA
+    atoms — no scores in device memory — for every head_dim up to 256, ragged lengths, grouped heads, causal masks with
+    unequal lengths (top-left aligned, as eager's) and additive masks of every broadcast form; against eager in float64."""
+    mod, shapes, mask = _FP32_ATTENTION[case]
+    torch.manual_seed(41)
+    args = [torch.randn(*s) for s in shapes] + ([mask()] if mask else [])
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod.eval(), tuple(args)))
+    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert names.count("k_sdpa_reduce") == 1 and "k_batched_linear" not in names, names
+    prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in args))))
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = mod(*(t.double() for t in args)).float()
+    eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-5, f"fp32 attention {case}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("form", ["w1", "w2", "w4", "s2", "s4", "s8"])
+def test_fp32_attention_forms(device, form, monkeypatch):
+    """``EMMY_FLASH=f32/w<n>``: 1, 2 or 4 of a workgroup's four waves own query rows and share the staged K / V blocks;
+    ``f32/s<k>``: the k waves of a workgroup split the key blocks of one row group and stage for themselves.  Here with a
+    last query block that is partly empty, keys that end inside a block, grouped heads and an additive mask."""
+    monkeypatch.setenv("EMMY_FLASH", f"f32/{form}")
+    torch.manual_seed(43)
+    for mod, args in (
+        (_FusedAttention(is_causal=True, enable_gqa=True), [torch.randn(2, 4, 300, 64), torch.randn(2, 2, 300, 64), torch.randn(2, 2, 300, 64)]),
+        (_FusedAttention(enable_gqa=True), [torch.randn(1, 4, 70, 64), torch.randn(1, 2, 333, 64), torch.randn(1, 2, 333, 64), torch.randn(1, 4, 70, 333)]),
+    ):
+        be = HipBackend()
+        compiled = be.compile(trace_module(mod.eval(), tuple(args)))
+        (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+        assert op.knobs["FLASH"] == f"f32/{form}"
+        prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in args))))
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            ours = prog.output_tensors()[compiled.outputs[0]].clone()
+        finally:
+            prog.close()
+        want = mod(*(t.double() for t in args)).float()
+        eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-5, f"fp32 attention {form}")
+
+
+@pytest.mark.gpu
+def test_fp32_attention_with_a_runtime_sequence_length(device):
+    """One compilation of fp32 causal attention with the sequence length as the kernel's trailing ``int``, bound at
+    several lengths (ragged blocks, one key block, more blocks than waves), against eager in float64."""
+    mod = _FusedAttention(is_causal=True, enable_gqa=True)
+    torch.manual_seed(47)
+    mk = lambda s: [torch.randn(1, 4, s, 128), torch.randn(1, 2, s, 128), torch.randn(1, 2, s, 128)]  # noqa: E731
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod.eval(), tuple(mk(64)), dynamic_shapes={"q": {2: "s"}, "k": {2: "s"}, "v": {2: "s"}}))
+    (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert op.runtime_args and op.knobs["FLASH"].startswith("f32/s")
+    for s in (64, 1, 31, 200, 513):
+        args = mk(s)
+        prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in args))))
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            ours = prog.output_tensors()[compiled.outputs[0]].clone()
+        finally:
+            prog.close()
+        want = mod(*(t.double() for t in args)).float()
+        eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-5, f"fp32 attention, runtime length {s}")
+
+
+_DECOMPOSED_ATTENTION = {
     # 16-bit rows that are not whole 16-byte chunks (the flash kernel pads whole chunks only)
     "bf16_head_dim_36": (_FusedAttention(is_causal=True), torch.bfloat16, [(2, 4, 64, 36)] * 3, None),
     "bf16_head_dim_100": (_FusedAttention(), torch.bfloat16, [(2, 4, 50, 100)] * 3, None),
+    # fp32: head dims beyond the streaming kernel's registers, value rows of another length than the keys'
+    "fp32_head_dim_320": (_FusedAttention(is_causal=True), torch.float32, [(1, 2, 48, 320)] * 3, None),
+    "fp32_value_rows_24": (_FusedAttention(), torch.float32, [(1, 2, 40, 16), (1, 2, 56, 16), (1, 2, 56, 24)], None),
+    "fp32_column_mask": (_FusedAttention(), torch.float32, [(2, 2, 40, 32)] * 3, lambda: torch.randn(2, 1, 40, 1)),
 }
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("case", sorted(_DECOMPOSED_ATTENTION))
 def test_attention_outside_the_flash_kernel(device, case):
-    """The fused attention op on fp32 operands (what the reference's perf suite runs), or with a 16-bit head_dim the flash
-    kernel cannot pad to one of its widths: two batched MFMA contractions (fp32 atoms keep fp32 accuracy) around loop-nest stages,
+    """The fused attention op with 16-bit rows the flash kernel cannot pad to one of its widths, or fp32 shapes outside
+    the streaming kernel's: two batched MFMA contractions (fp32 atoms keep fp32 accuracy) around loop-nest stages,
     against eager in float64."""
     mod, dtype, shapes, mask = _DECOMPOSED_ATTENTION[case]
     torch.manual_seed(41)
@@ -1380,14 +1471,14 @@ def test_attention_outside_the_flash_kernel(device, case):
 def test_c5_qwen3_block_in_fp32(device, seq):
     """The decoder block with fp32 parameters and activations — the only precision the reference compiles
     (tests/perf/cases.py:20-23).  The fused forms written for 16-bit tiles (norm prologue, gate/up pair, head-norm +
-    rotary epilogue, flash attention) stand down: plain fp32-atom contractions, row kernels and the decomposed
-    attention; against the module in float64."""
+    rotary epilogue) stand down: plain fp32-atom contractions, row kernels and the fp32 streaming attention kernel;
+    against the module in float64."""
     import copy
 
     case = eager.qwen3_block_case(seq=seq, dtype=torch.float32, norm_std=0.1, seed=5)
     ours, want, compiled = run_case(case, device)
     names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
-    assert names.count("k_batched_linear") == 2 and "k_sdpa_reduce" not in names
+    assert names.count("k_sdpa_reduce") == 1 and "k_batched_linear" not in names
     with torch.no_grad():
         exact = copy.deepcopy(case.module).cpu().double()(*(t.double() for t in case.inputs))
     exact = (exact[0] if isinstance(exact, tuple) else exact).float()
