@@ -52,6 +52,7 @@ if str(ROOT) not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_FP32_PEAK_TFLOPS = 157.3
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE (scaled by the same counters on a copy kernel of known size); keyed
@@ -375,7 +376,9 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
             row.update(bound="hbm", achieved=round(gbps, 1), unit="GB/s", frac=round(gbps / HBM_PEAK_GBPS, 4))
         else:
             tf = case.algo_flops / (us * 1e-6) / 1e12
-            row.update(bound="mfma", achieved=round(tf, 1), unit="TFLOP/s", frac=round(tf / MFMA_BF16_PEAK_TFLOPS, 4))
+            row.update(bound="mfma", achieved=round(tf, 1), unit="TFLOP/s", frac=round(tf / (MFMA_FP32_PEAK_TFLOPS if bound == "mfma_f32" else MFMA_BF16_PEAK_TFLOPS), 4))
+            if bound == "mfma_f32":
+                row["peak"] = MFMA_FP32_PEAK_TFLOPS
         if cold:
             c_us, sets = cold_us(compiled, data, case.algo_bytes)
             row["us_cold"] = round(c_us, 2)
@@ -390,8 +393,8 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
         if vendor:
             v_us = vendor_us(case)
             row["vendor_us"] = round(v_us, 2)  # PyTorch eager on the same GPU: the vendor library's kernel for this problem
-            if bound == "mfma":
-                row["vendor_frac"] = round(case.algo_flops / (v_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
+            if bound in ("mfma", "mfma_f32"):
+                row["vendor_frac"] = round(case.algo_flops / (v_us * 1e-6) / 1e12 / (MFMA_FP32_PEAK_TFLOPS if bound == "mfma_f32" else MFMA_BF16_PEAK_TFLOPS), 4)
         if cpu and not whole_model:
             row["cpu_us"] = round(_cpu_us(case), 1)
         rows.append(row)
@@ -405,6 +408,9 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
     bench(lambda: wl.linear_case(m=4096, k=4096, n=4096), "C3x linear bf16 M=4096 K=4096 N=4096", "mfma", vendor=True)
     bench(wl.sdpa_case, "C4 causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma", vendor=True)
     bench(lambda: wl.sdpa_decode_case(q_len=1, kv_len=32768), "C4d decode GQA sdpa bf16 16q/8kv q=1 kv=32768 d=128 (key slices + combine)", "hbm", vendor=True)
+    # the reference's own precision: the same shape in fp32 (its sdpa perf cases run S = 32 / 128 / 512), on fp32 MFMA atoms
+    bench(lambda: wl.sdpa_case(s=512, fp32=True), "C4f causal GQA sdpa fp32 16q/8kv S=512 d=128", "mfma_f32", vendor=True)
+    bench(lambda: wl.sdpa_case(fp32=True), "C4f causal GQA sdpa fp32 16q/8kv S=2048 d=128", "mfma_f32", vendor=True)
     if extended:
         bench(lambda: wl.sdpa_case(causal=False), "C4x non-causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
         bench(lambda: wl.sdpa_case(s=8192), "C4xx causal GQA sdpa bf16 16q/8kv S=8192 d=128", "mfma", vendor=True)
@@ -487,7 +493,7 @@ def main() -> int:
         # bound: its machine-filling variant C1x stands for the kernel; the decode-size linears are HBM bound)
         peaks = {"hbm": (HBM_PEAK_GBPS, "GB/s"), "mfma": (MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")}
         out["rooflines"] = [
-            {"config": r["config"], "bound": r["bound"], "achieved": r["achieved"], "peak": peaks[r["bound"]][0], "unit": peaks[r["bound"]][1], "frac": r["frac"], "kernel_us": r["us"],
+            {"config": r["config"], "bound": r["bound"], "achieved": r["achieved"], "peak": r.get("peak", peaks[r["bound"]][0]), "unit": peaks[r["bound"]][1], "frac": r["frac"], "kernel_us": r["us"],
              **({"per_kernel": r["per_kernel"]} if "per_kernel" in r else {})}
             for r in out["kernels"]
         ]

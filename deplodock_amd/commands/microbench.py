@@ -395,6 +395,66 @@ def handle_flash(args) -> None:
         print(line)
 
 
+def handle_fp32_attention(args) -> None:
+    """fp32 causal attention with grouped heads (the reference's ``sdpa`` perf shape, tests/perf/cases.py:174-190, and
+    longer sequences): the streaming kernel's forms against the decomposed route and eager."""
+    import os
+
+    import torch
+
+    from deplodock_amd import HipBackend, trace_module, workloads
+    from deplodock_amd.commands.table import render_table
+    from deplodock_amd.ir.hip import HipOp
+
+    dev = torch.device("cuda:0")
+    saved = os.environ.get("EMMY_FLASH")
+    rows = []
+    try:
+        for seq in (int(x) for x in args.seq.split(",")):
+            case = workloads.sdpa_case(s=seq)
+            inputs = tuple(t.float() for t in case.inputs)
+            on_dev = [t.to(dev) for t in inputs]
+            for _ in range(3):
+                case.module(*on_dev)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                case.module(*on_dev)
+            e1.record()
+            torch.cuda.synchronize()
+            row = [str(seq), f"{case.algo_flops / 1e9:.2f}"]
+            best = None
+            for pin in (None, "f32/w4", "f32/s2", "f32/s4", "decompose"):
+                if pin == "decompose" and seq > 2048:
+                    row.append("")
+                    continue
+                if pin:
+                    os.environ["EMMY_FLASH"] = pin
+                else:
+                    os.environ.pop("EMMY_FLASH", None)
+                be = HipBackend()
+                compiled = be.compile(trace_module(case.module, inputs))
+                res = be.benchmark(compiled, warmup=3, num_iters=10 if seq >= 2048 else 30, input_data=dict(zip(compiled.inputs, on_dev)))
+                us = sum(p.time_ms for p in res.per_launch) * 1e3
+                if pin is None:
+                    (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+                    row.append(f"{op.knobs['FLASH']} {us:.1f}")
+                    best = us
+                else:
+                    row.append(f"{us:.1f}")
+            row += [f"{e0.elapsed_time(e1) * 100:.1f}", f"{case.algo_flops / best / 1e6:.1f}", f"{case.algo_flops / best / 1e6 / 157.3:.2f}"]
+            rows.append(row)
+    finally:
+        if saved is None:
+            os.environ.pop("EMMY_FLASH", None)
+        else:
+            os.environ["EMMY_FLASH"] = saved
+    print("fp32 causal attention, 16 query / 8 key-value heads of 128, us per call (the decomposed route: sum of its kernels)")
+    for line in render_table(["S", "GFLOP", "default", "w4", "s2", "s4", "decomposed", "eager fp32", "TFLOP/s", "of fp32 MFMA peak"], rows, "rrlrrrrrrr"):
+        print(line)
+
+
 def handle_stamps(args) -> None:
     """Phase stamps of the default attention kernel and of the ring contractions (``-DEMH_STAMP=1`` / ``2`` builds of
     ``emit/flash.py`` and ``emit/contraction.py``): the first thread of workgroup 0 leaves four floats over the first
@@ -471,8 +531,9 @@ def register_microbench_command(subparsers) -> None:
     p.add_argument("--lds", action="store_true", help="fragment-read rate out of LDS for the emitters' swizzled layouts")
     p.add_argument("--flash", action="store_true", help="phase stamps and ablations of the software-pipelined attention kernels on the benchmark shape")
     p.add_argument("--stamps", action="store_true", help="phase stamps (shader clocks) of the default attention kernel and of the ring contractions on the benchmark shapes")
+    p.add_argument("--fp32-attention", action="store_true", help="fp32 attention: the streaming kernel's forms against the decomposed route and eager (--seq: comma-separated lengths)")
     p.add_argument("--pins", default=None, help="with --flash: comma-separated EMMY_FLASH pins (default: the ws and sp forms of the benchmark shape)")
-    p.add_argument("--seq", default="2048", help="with --flash: sequence length")
+    p.add_argument("--seq", default="2048", help="with --flash: sequence length; with --fp32-attention: comma-separated lengths")
     p.set_defaults(func=handle_microbench)
 
 
@@ -493,6 +554,9 @@ def handle_microbench(args) -> None:
         return
     if getattr(args, "stamps", False):
         handle_stamps(args)
+        return
+    if getattr(args, "fp32_attention", False):
+        handle_fp32_attention(args)
         return
     from deplodock_amd.backend.hip import launcher
     from deplodock_amd.commands.table import render_table

@@ -173,7 +173,13 @@ def decompose_attention(g: Graph, undo_repeat, streamed=None) -> Graph:
     graph when anything changed.  ``undo_repeat(g, node id) -> (source id, group)`` sees through a materialised head
     repeat; ``streamed(node) -> bool`` replaces the rule for which ops stay fused."""
 
+    from deplodock_amd import config
+
+    pinned_apart = config.knob_raw("FLASH") == "decompose"  # ``EMMY_FLASH=decompose``: the reference's two-kernel route everywhere
+
     def flash_takes(node: Node) -> bool:
+        if pinned_apart:
+            return False
         q, k, v = (g.nodes[i].output for i in node.inputs[:3])
         if q.dtype.name == "f32":
             # the fp32 streaming kernel: any row length it has registers for, q / k / v rows alike

@@ -75,13 +75,19 @@ def linear_case(m: int = 2048, k: int = 1024, n: int = 3072, seed: int = 0) -> C
     return Case(f"linear_{m}x{k}x{n}", lin.bfloat16().eval(), (x,), BF16_RTOL, 2e-2, algo_bytes=(m * k + n * k + m * n) * 2, algo_flops=2 * m * n * k)
 
 
-def sdpa_case(b: int = 1, hq: int = 16, hkv: int = 8, s: int = 2048, d: int = 128, causal: bool = True, seed: int = 0) -> Case:
-    """C4: causal GQA attention, bf16 ~N(0,1), scale 1/sqrt(d)."""
+def sdpa_case(b: int = 1, hq: int = 16, hkv: int = 8, s: int = 2048, d: int = 128, causal: bool = True, seed: int = 0, fp32: bool = False) -> Case:
+    """C4: causal GQA attention, bf16 ~N(0,1), scale 1/sqrt(d); ``fp32``: the same values (rounded to bf16) held as fp32,
+    the precision of the reference's ``sdpa`` perf cases (tests/perf/cases.py:174-190)."""
     torch.manual_seed(seed)
     q = torch.randn(b, hq, s, d).bfloat16()
     k = torch.randn(b, hkv, s, d).bfloat16()
     v = torch.randn(b, hkv, s, d).bfloat16()
     pairs = s * (s + 1) // 2 if causal else s * s
+    if fp32:
+        return Case(
+            f"sdpa_fp32_{b}x{hq}x{hkv}x{s}x{d}", Sdpa(causal).eval(), (q.float(), k.float(), v.float()), 1e-4, 1e-5,
+            algo_bytes=(2 * b * hq * s * d + 2 * b * hkv * s * d) * 4, algo_flops=4 * b * hq * d * pairs,
+        )  # fmt: skip
     return Case(
         f"sdpa_{b}x{hq}x{hkv}x{s}x{d}", Sdpa(causal).eval(), (q, k, v), BF16_RTOL, 2e-2,
         algo_bytes=(2 * b * hq * s * d + 2 * b * hkv * s * d) * 2, algo_flops=4 * b * hq * d * pairs,
