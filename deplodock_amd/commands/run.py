@@ -128,7 +128,7 @@ def kernel_rows(compiled, bench) -> list[list[str]]:
         if us:
             gbps = op.algo_bytes / (us * 1e-6) / 1e9
             tfs = op.algo_flops / (us * 1e-6) / 1e12
-            peak = MFMA_F32_PEAK_TFLOPS if "_f32" in str(op.knobs.get("TILE", "")) else MFMA_BF16_PEAK_TFLOPS  # the atom names the matrix pipe's rate
+            peak = MFMA_F32_PEAK_TFLOPS if "_f32" in str(op.knobs.get("TILE", "")) or str(op.knobs.get("FLASH", "")).startswith("f32/") else MFMA_BF16_PEAK_TFLOPS  # the atom names the matrix pipe's rate
             if op.algo_flops and tfs / peak > gbps / HBM_PEAK_GBPS:
                 rate, frac = f"{tfs:.1f} TFLOP/s", f"{100 * tfs / peak:.1f}% mfma"
             else:

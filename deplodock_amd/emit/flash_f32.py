@@ -64,20 +64,23 @@ _SOFTMAX = r"""      // register r: key k0 + 8 (r / 4) + 4 h + r % 4 of query qr
         mx = fmaxf(mx, v);
       }
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run, mx);
-      const float m_use = m_new == -__builtin_inff() ? 0.0f : m_new;  // nothing but masked keys so far: every term is 0
-      const float alpha = exp2f(m_run - m_use);
-      float lsum = 0.0f;
-      #pragma unroll
-      for (int r = 0; r < 16; ++r) { s[r] = exp2f(s[r] - m_use); lsum += s[r]; }
-      l_run = l_run * alpha + lsum;
-      m_run = m_new;
-      if (__any(alpha != 1.0f)) {
+      // The reference maximum is raised only when a row outgrows it by 2^8 (probabilities stay below 2^8, far inside
+      // fp32 range), so the rescale of the accumulators is rare.
+      const bool raise = mx > m_run + 8.0f;  // (from -inf any finite maximum raises; a block of masked keys never does)
+      if (__any(raise)) {
+        const float alpha = raise ? exp2f(m_run - mx) : 1.0f;
+        m_run = raise ? mx : m_run;
+        l_run *= alpha;
         #pragma unroll
         for (int b = 0; b < NDB; ++b)
           #pragma unroll
           for (int r = 0; r < 16; ++r) oacc[b][r] *= alpha;
       }
+      const float m_use = m_run == -__builtin_inff() ? 0.0f : m_run;  // nothing but masked keys so far: every term is 0
+      float lsum = 0.0f;
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) { s[r] = exp2f(s[r] - m_use); lsum += s[r]; }
+      l_run += lsum;
 """
 
 _SRC = r"""
@@ -227,15 +230,17 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
 # the softmax and the output atoms, the next V block is requested after the output atoms and lands under the next
 # scores.  The (m, l, O) of the waves are merged through LDS with the exp-family combine.
 _SRC_PRIVATE = r"""
-#define CPRL (DPL / 4)                 /* 16-byte chunks per LDS row (DPL: the padded row length, a power of two) */
-#define NI (32 * CPRL / 64)            /* direct-to-LDS requests of a wave per block */
+#define CPRL (DPL / 4)                 /* 16-byte chunks per V row in LDS (DPL: the padded row length, a power of two) */
+#define RPR (64 / CPRL)                /* V rows per direct-to-LDS request */
+#define NIK (DP / 8)                   /* requests of a wave per K block: 32 rows x two chunks each */
+#define NIV (32 / RPR)                 /* requests of a wave per V block: whole rows */
 #define NDB (DP / 32)                  /* 32-column blocks of the output */
-#define REGION (2 * 32 * DPL)          /* floats of LDS per wave: its K block, then its V block */
+#define REGION (32 * DP + 32 * DPL)    /* floats of LDS per wave: its K block, then its V block */
 #define PS (DPL + 4)                   /* floats per row of a wave's partial output at the close */
-// K rows are XOR-swizzled per 256-byte bank line so that the 16-byte reads of 16 consecutive keys at one column hit
-// 16 different bank groups; V chunks swap 128-byte halves between rows r and r + 4, the two rows a 4-byte read touches.
-#define KRPL (CPRL >= 16 ? 1 : 16 / CPRL)
-EMH_DEV int emh_kswz(int row) { return (row / KRPL) % (CPRL < 16 ? CPRL : 16); }
+// K lies in LDS as [pair of chunks u][row][8 floats]: the 16-byte fragment reads of a wave at one u (row n, half h) are
+// 1 KiB in a row, conflict-free, and request u of a block is one lane offset plus 32 bytes x u.  V keeps [row][d] with its
+// 128-byte halves swapped between rows r and r + 4, the two rows a 4-byte read touches; the rows of one request share
+// that swap, so a request is one of two lane offsets plus a row step.
 EMH_DEV int emh_vswz(int row) { return CPRL >= 16 ? ((row >> 2) & 1) << 3 : 0; }
 // chunks past the row's end (a head_dim below the tile's width) are fetched from the row's first chunk: finite values
 // that never count — q's columns there are zero, and v's only reach output columns that are not stored
@@ -243,7 +248,7 @@ EMH_DEV int emh_gchunk(int c) { return c < DR / 4 ? c : 0; }
 
 extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__ Q, const float* __restrict__ Kp,
                                                       const float* __restrict__ Vp MASK_PARAM, float* __restrict__ Op SYM_PARAM) {
-  extern __shared__ __attribute__((aligned(16))) float lds[];  // [KVS waves][K: 32 x DPL | V: 32 x DPL]
+  extern __shared__ __attribute__((aligned(16))) float lds[];  // [KVS waves][K: DP / 8 x 32 x 8 | V: 32 x DPL]
   const int tid = threadIdx.x, lane = tid % 64, grp = __builtin_amdgcn_readfirstlane(tid / 64);
   const int n = lane % 32, h = lane / 32;
   const int grid = (int)gridDim.x;
@@ -267,14 +272,34 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
   const int nblocks = (kend + 31) / 32;
 
   float* kl = lds + grp * REGION;
-  float* vl = kl + 32 * DPL;
-  // request i of a block: LDS chunk i * 64 + lane of the region, i.e. row (i * 64 + lane) / CPRL at position
-  // (i * 64 + lane) % CPRL, which holds the row's chunk position ^ swizzle(row)
-  #define EMH_REQUEST(base_, stride_, swz_, dst_, j_) { \
-    _Pragma("unroll") for (int i = 0; i < NI; ++i) { \
-      const int p_ = i * 64 + lane, row_ = p_ / CPRL, c_ = (p_ % CPRL) ^ swz_(row_); \
-      int key_ = (j_) * 32 + row_; key_ = key_ < SKV ? key_ : SKV - 1;  /* rows past the end repeat the last key: masked, finite */ \
-      emh_dma16((base_) + (long)key_ * (stride_) + emh_gchunk(c_) * 4, (dst_) + i * 256); \
+  float* vl = kl + 32 * DP;
+  const unsigned kl_s = emh_uniform(emh_lds_addr(kl)), vl_s = emh_uniform(emh_lds_addr(vl));
+  // Lane offsets of the requests of a block that lies wholly inside the sequence: K request u is rows lane / 2, chunk
+  // 2 u + lane % 2; V request i is rows i RPR + lane / CPRL, chunk position lane % CPRL, which holds chunk position ^ swap.
+  const unsigned koff = (unsigned)(lane / 2) * (unsigned)(K_SS * 4) + (unsigned)(lane % 2) * 16u;
+  const unsigned voff0 = (unsigned)(lane / CPRL) * (unsigned)(V_SS * 4) + (unsigned)emh_gchunk(lane % CPRL) * 16u;
+  const unsigned voff1 = (unsigned)(lane / CPRL) * (unsigned)(V_SS * 4) + (unsigned)emh_gchunk((lane % CPRL) ^ 8) * 16u;
+  // A block that hangs over the sequence's end repeats the last key in the rows past it (masked below, finite here): per-lane addresses.
+  #define EMH_REQUEST_K(j_) { \
+    if ((j_) * 32 + 32 <= SKV) { \
+      const unsigned char* b_ = emh_uniform(kbase + (long)(j_) * 32 * K_SS); \
+      _Pragma("unroll") for (int i = 0; i < NIK; ++i) emh_dma16s(b_ + (2 * i < DR / 4 ? i * 32 : 0), koff, kl_s + i * 1024); \
+    } else { \
+      _Pragma("unroll") for (int i = 0; i < NIK; ++i) { \
+        int key_ = (j_) * 32 + lane / 2; key_ = key_ < SKV ? key_ : SKV - 1; \
+        emh_dma16(kbase + (long)key_ * K_SS + (2 * i < DR / 4 ? i * 8 : 0) + (lane % 2) * 4, kl + i * 256); \
+      } \
+    } }
+  #define EMH_REQUEST_V(j_) { \
+    if ((j_) * 32 + 32 <= SKV) { \
+      const unsigned char* b_ = emh_uniform(vbase + (long)(j_) * 32 * V_SS); \
+      _Pragma("unroll") for (int i = 0; i < NIV; ++i) emh_dma16s(b_ + (long)i * RPR * V_SS * 4, emh_vswz(i * RPR) ? voff1 : voff0, vl_s + i * 1024); \
+    } else { \
+      _Pragma("unroll") for (int i = 0; i < NIV; ++i) { \
+        const int row_ = i * RPR + lane / CPRL; \
+        int key_ = (j_) * 32 + row_; key_ = key_ < SKV ? key_ : SKV - 1; \
+        emh_dma16(vbase + (long)key_ * V_SS + emh_gchunk((lane % CPRL) ^ emh_vswz(row_)) * 4, vl + i * 256); \
+      } \
     } }
 
   f32x16 oacc[NDB];
@@ -285,8 +310,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
   float m_run = -__builtin_inff(), l_run = 0.0f;
 
   if (grp < nblocks) {
-    EMH_REQUEST(kbase, K_SS, emh_kswz, kl, grp)
-    EMH_REQUEST(vbase, V_SS, emh_vswz, vl, grp)
+    EMH_REQUEST_K(grp)
+    EMH_REQUEST_V(grp)
   }
   // The query's values, requested behind the first blocks and waited for here, before the loop: a load of the
   // compiler's own still outstanding at the loop's head would make it wait inside the loop, by a count that knows
@@ -310,26 +335,25 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
   for (int j = grp; j < nblocks; j += KVS) {
     const bool more = j + KVS < nblocks;
     const int k0 = j * 32;
-    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NI) : "memory");  // this block's K has landed (its V may still be on its way)
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NIV) : "memory");  // this block's K has landed (its V may still be on its way)
     emh_lds_publish(kl);
     f32x16 s;
     #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.0f;
     {
-      const float* krow = kl + n * DPL;
-      const int ksw = emh_kswz(n);
+      const float* kfrag = kl + n * 8 + h * 4;
       #pragma unroll
       for (int u = 0; u < DP / 8; ++u) {
-        const f32x4 kf = *(const f32x4*)(krow + ((2 * u + h) ^ ksw) * 4);
+        const f32x4 kf = *(const f32x4*)(kfrag + u * 256);
         #pragma unroll
         for (int i = 0; i < 4; ++i) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[i], qf[u][i], s, 0, 0, 0);
       }
     }
     // the K fragments are in registers (the atoms above consumed them): the region takes the next block
     asm volatile("" :: "v"(s[0]) : "memory");
-    if (more) EMH_REQUEST(kbase, K_SS, emh_kswz, kl, j + KVS)
+    if (more) EMH_REQUEST_K(j + KVS)
 @SOFTMAX@
-    if (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NI) : "memory");  // V of this block (the next K block may be on its way)
+    if (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NIK) : "memory");  // V of this block (the next K block may be on its way)
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     emh_lds_publish(vl);
     #pragma unroll
@@ -341,7 +365,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
     }
     #pragma unroll
     for (int b = 0; b < NDB; ++b) asm volatile("" :: "v"(oacc[b][0]) : "memory");  // every V fragment has been consumed
-    if (more) EMH_REQUEST(vbase, V_SS, emh_vswz, vl, j + KVS)
+    if (more) EMH_REQUEST_V(j + KVS)
   }
 
   // Close: every wave leaves its unnormalised output rows, maximum and sum in its own region; after the barrier the
@@ -413,8 +437,8 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         if key not in ("q_len", "kv_len") and not (key.split(".")[0] in ("q_strides", "k_strides", "v_strides", "o_strides", "mask_strides") and key.split(".")[1] in ("0", "1", "2")):
             raise LoweringError(f"flash: {key} cannot follow a symbolic axis")
     vec_in, vec_out = whole_chunk_rows(body)
-    if private and not (vec_in and vec_out):
-        raise LoweringError("flash (fp32 form): the key-split form needs rows of whole, aligned 16-byte chunks")
+    if private and not (vec_in and vec_out and D % 8 == 0):
+        raise LoweringError("flash (fp32 form): the key-split form needs rows of whole, aligned pairs of 16-byte chunks")
 
     def stride(field: str, i: int):
         return symf.get(f"{field}.{i}", getattr(body, field)[i])
@@ -478,7 +502,7 @@ def whole_chunk_rows(body: Flash) -> tuple[bool, bool]:
 
 def private_lds_bytes(head_dim: int, kvs: int) -> int:
     dp = padded_head_dim(head_dim)
-    return kvs * 2 * 32 * (1 << (dp - 1).bit_length()) * 4
+    return kvs * 32 * (dp + (1 << (dp - 1).bit_length())) * 4
 
 
 def max_key_split(head_dim: int, lds_limit: int) -> int:

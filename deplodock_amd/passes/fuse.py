@@ -148,7 +148,7 @@ def _materialize(c: _Ctx, nid: str) -> None:
             c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
         c.done[nid] = nid
         return
-    for rec in (_rec_same_type_cast, _rec_loop_nest, _rec_batched_linear, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_layer_norm, _rec_softmax, _rec_sdpa, _rec_row_fused, _rec_row_sum, _rec_gather, _rec_cat, _rec_pointwise):
+    for rec in (_rec_same_type_cast, _rec_loop_nest, _rec_batched_linear, _rec_matmul_residual, _rec_matmul_gated, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_layer_norm, _rec_softmax, _rec_sdpa, _rec_row_fused, _rec_row_sum, _rec_gather, _rec_cat, _rec_pointwise):
         if rec(c, nid):
             return
     raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
@@ -373,7 +373,7 @@ def _copy_of_view(c: _Ctx, v: View, order: tuple[int, ...], new_id: str, pad_las
     return View(new_id, 0, shape, contiguous_strides(shape), v.dtype)
 
 
-def _emit_batched_contraction(c: _Ctx, nid: str, a: View, b: View, label: str) -> None:
+def _emit_batched_contraction(c: _Ctx, nid: str, a: View, b: View, label: str, residual: View | None = None, post: E.Expr | None = None) -> None:
     """``a [..., M, K] x b [... | 1..., N, K] -> [..., M, N]`` as one launch with a workgroup row per product.  The
     kernel reads whole 16-byte chunks along ``K`` and stores runs of four columns: an operand that is not laid out
     for that (reduction axis not contiguous, leading axes not one uniformly strided run, misaligned) is copied
@@ -407,10 +407,82 @@ def _emit_batched_contraction(c: _Ctx, nid: str, a: View, b: View, label: str) -
     body = Contraction(
         m=m, n=n_pad, k=kp, a=a.base, b=b.base, out=nid, in_dtype=a.dtype, out_dtype=node.output.dtype, lda=int(a.strides[-2]) if m > 1 else kp, ldb=int(b.strides[-2]) if n_pad > 1 else kp,
         a_offset=a.offset, b_offset=b.offset, batch=p, a_batch=int(sa) if p > 1 else 0, b_batch=0 if shared or p == 1 else int(sb), out_batch=m * n_pad,
+        # ``residual``: a tensor of the result's shape read in the output stage as ``res``; ``post`` says what it does there (default: added)
+        **({"post": post if post is not None else E.Var("y") + E.Var("res"), "epilogue_operands": (("res", node.output.dtype),)} if residual is not None else {}),
     )  # fmt: skip
-    _emit(c, nid, body, label, [a.base, b.base], shape=(*lead, m, n_pad))
+    if residual is not None:
+        if p != 1 or n_pad != n:
+            raise FusionError(f"{label} {nid!r}: a residual rides on a single unpadded product")
+        body.operand_buffers = {"res": residual.base}
+    _emit(c, nid, body, label, [a.base, b.base, *([residual.base] if residual is not None else [])], shape=(*lead, m, n_pad))
     if n_pad != n:
         c.windows[nid] = (0, (*lead, m, n), contiguous_strides((*lead, m, n_pad)))
+
+
+def _rec_matmul_residual(c: _Ctx, nid: str) -> bool:
+    """``a @ w + residual`` with a single product (the reference's ``matmul_add`` perf cases, tests/perf/cases.py:193-210:
+    o_proj / down_proj + residual as one launch): the residual is added to the accumulator in the contraction's output
+    stage, as ``_rec_linear_residual`` does for ``F.linear``."""
+    node = c.g.nodes[nid]
+    if not (_is(node, F.ElementwiseOp, fn="add") and len(node.inputs) == 2):
+        return False
+    for mi, ri in ((0, 1), (1, 0)):
+        mm_id, res_id = node.inputs[mi], node.inputs[ri]
+        mm = c.g.nodes[mm_id]
+        if not (isinstance(mm.op, F.MatmulOp) and c.single_use(mm_id)) or mm_id in c.done or mm_id in c.g.outputs:
+            continue
+        ta, tb = c.g.nodes[mm.inputs[0]].output, c.g.nodes[mm.inputs[1]].output
+        if len(tb.shape) != 2 or len(ta.shape) < 2 or not all(isinstance(d, int) for d in (*ta.shape, *tb.shape)):
+            continue
+        if math.prod(int(d) for d in ta.shape[:-2]) != 1 or int(tb.shape[1]) % 4 or int(tb.shape[0]) % 8:
+            continue
+        rt_ = c.g.nodes[res_id].output
+        if tuple(rt_.shape) != tuple(node.output.shape) or tuple(mm.output.shape) != tuple(node.output.shape) or rt_.dtype != node.output.dtype or mm.output.dtype != node.output.dtype:
+            continue
+        res = _need(c, res_id)
+        if not res.is_contiguous() or res.offset:
+            continue
+        a, b = _need(c, mm.inputs[0]), _need(c, mm.inputs[1])
+        bt = _transposed_parameter(c, View(b.base, b.offset, (b.shape[1], b.shape[0]), (b.strides[1], b.strides[0]), b.dtype))
+        if len(a.shape) > 2:
+            bt = View(bt.base, bt.offset, (*(1,) * (len(a.shape) - 2), *bt.shape), (*(0,) * (len(a.shape) - 2), *bt.strides), bt.dtype)
+        _emit_batched_contraction(c, nid, a, bt, "matmul_add", residual=res)
+        return True
+    return False
+
+
+def _rec_matmul_gated(c: _Ctx, nid: str) -> bool:
+    """``act(x @ wg) * (x @ wu)`` on fp32 operands (the reference's ``gated_mlp`` perf cases, tests/perf/cases.py:213-232):
+    the gate product is a contraction of its own and the activation and the product with it ride in the output stage of
+    the up contraction — two launches instead of two contractions and a map.  (16-bit operands with constant weights
+    take the paired tile of ``_rec_gate_up``.)"""
+    node = c.g.nodes[nid]
+    if not (_is(node, F.ElementwiseOp, fn="mul") and len(node.inputs) == 2) or node.output.dtype is not F32:
+        return False
+    for si, ui in ((0, 1), (1, 0)):
+        act, up = c.g.nodes[node.inputs[si]], c.g.nodes[node.inputs[ui]]
+        if not (isinstance(act.op, F.ElementwiseOp) and act.op.fn in ("silu", "gelu_tanh", "gelu") and len(act.inputs) == 1 and c.single_use(act.id) and act.id not in c.g.outputs):
+            continue
+        gate = c.g.nodes[act.inputs[0]]
+        if not (isinstance(gate.op, F.MatmulOp) and isinstance(up.op, F.MatmulOp) and c.single_use(gate.id) and c.single_use(up.id)) or up.id in c.done or up.id in c.g.outputs or gate.id in c.g.outputs:
+            continue
+        ta, tb = c.g.nodes[up.inputs[0]].output, c.g.nodes[up.inputs[1]].output
+        if len(tb.shape) != 2 or len(ta.shape) < 2 or not all(isinstance(d, int) for d in (*ta.shape, *tb.shape)):
+            continue
+        if math.prod(int(d) for d in ta.shape[:-2]) != 1 or int(tb.shape[1]) % 4 or int(tb.shape[0]) % 8:
+            continue
+        if tuple(gate.output.shape) != tuple(node.output.shape) or tuple(up.output.shape) != tuple(node.output.shape) or gate.output.dtype is not F32 or up.output.dtype is not F32:
+            continue
+        g_view = _need(c, gate.id)
+        if not g_view.is_contiguous() or g_view.offset:
+            continue
+        a, b = _need(c, up.inputs[0]), _need(c, up.inputs[1])
+        bt = _transposed_parameter(c, View(b.base, b.offset, (b.shape[1], b.shape[0]), (b.strides[1], b.strides[0]), b.dtype))
+        if len(a.shape) > 2:
+            bt = View(bt.base, bt.offset, (*(1,) * (len(a.shape) - 2), *bt.shape), (*(0,) * (len(a.shape) - 2), *bt.strides), bt.dtype)
+        _emit_batched_contraction(c, nid, a, bt, f"matmul_{act.op.fn}_mul", residual=g_view, post=E.Un(act.op.fn, E.Var("res")) * E.Var("y"))
+        return True
+    return False
 
 
 def _rec_matmul(c: _Ctx, nid: str) -> bool:

@@ -668,7 +668,7 @@ def _schedule_flash_f32(body: Flash, ctx: Context) -> dict:
     body.pair = body.deep = body.ws = body.sp = body.mfma_sum = False
     body.kv_ctas, body.block_kv = 1, 32
     heads = body.batch * body.q_heads
-    can_split = all(whole_chunk_rows(body))
+    can_split = all(whole_chunk_rows(body)) and body.head_dim % 8 == 0
     most = min(4, max_key_split(body.head_dim, ctx.lds_bytes_per_cu)) if can_split else 1
     symbolic = getattr(body, "sym", None) is not None and bool(body.sym.fields)
     if most > 1 and (body.kv_len > 32 or symbolic):

@@ -1266,6 +1266,71 @@ def test_plain_matmul(device, shape_a, shape_b):
     eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-4 * float(want.pow(2).mean().sqrt()), f"matmul {shape_a} @ {shape_b}")
 
 
+class _MmAdd(nn.Module):
+    def forward(self, a, b, r):
+        return torch.matmul(a, b) + r
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows, k, n", [(512, 2048, 1024), (32, 3072, 1024), (100, 64, 72), (7, 50, 20)])
+def test_matmul_plus_residual_is_one_contraction(device, dtype, rows, k, n):
+    """``a @ w + residual`` (the reference's ``matmul_add`` perf cases, tests/perf/cases.py:193-210): the residual is added in
+    the contraction's output stage where the product is a single unpadded one (``k`` whole 8s, ``n`` whole 4s); other
+    shapes keep the separate add.  Against float64."""
+    torch.manual_seed(36)
+    a, b, r = torch.randn(1, rows, k).to(dtype), (0.05 * torch.randn(k, n)).to(dtype), torch.randn(1, rows, n).to(dtype)
+    be = HipBackend()
+    compiled = be.compile(trace_module(_MmAdd().eval(), (a, b, r)))
+    names = [nd.op.kernel_name.rsplit("_", 1)[0] for nd in compiled.nodes.values() if isinstance(nd.op, HipOp)]
+    fused = k % 8 == 0 and n % 4 == 0
+    assert ("k_pointwise_elementwise" not in names) == fused, names
+    prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in (a, b, r)))))
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = a.double() @ b.double() + r.double()
+    tol = (2e-2, 2e-2) if dtype is torch.bfloat16 else (1e-4, 1e-4 * float(want.pow(2).mean().sqrt()))
+    eager.assert_close(ours.reshape(want.shape).double(), want, *tol, f"matmul + residual {rows}x{k}x{n} {dtype}")
+
+
+class _GatedMm(nn.Module):
+    def __init__(self, act):
+        super().__init__()
+        self.act = act
+
+    def forward(self, x, g, u):
+        return self.act(torch.matmul(x, g)) * torch.matmul(x, u)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows", [512, 32, 50])
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
+def test_fp32_gated_matmul_pair_is_two_contractions(device, rows, act):
+    """``act(x @ wg) * (x @ wu)`` on fp32 run-time operands (the reference's ``gated_mlp`` perf cases,
+    tests/perf/cases.py:213-232): the activation of the gate product and the product with it ride in the up contraction's
+    output stage — no element-wise launch; also where the contractions are split over workgroups (few rows).  Against float64."""
+    fn = {"silu": torch.nn.functional.silu, "gelu_tanh": lambda t: torch.nn.functional.gelu(t, approximate="tanh")}[act]
+    torch.manual_seed(37)
+    x, g, u = torch.randn(1, rows, 1024), 0.03 * torch.randn(1024, 768), 0.03 * torch.randn(1024, 768)
+    be = HipBackend()
+    compiled = be.compile(trace_module(_GatedMm(fn).eval(), (x, g, u)))
+    names = [nd.op.kernel_name.rsplit("_", 1)[0] for nd in compiled.nodes.values() if isinstance(nd.op, HipOp)]
+    assert not any(nm.startswith("k_pointwise") for nm in names) and any(nm.startswith(f"k_matmul_{act}_mul") for nm in names), names
+    prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in (x, g, u)))))
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = fn(x.double() @ g.double()) * (x.double() @ u.double())
+    eager.assert_close(ours.reshape(want.shape).double(), want, 1e-4, 1e-4 * float(want.pow(2).mean().sqrt()), f"gated matmul pair, {rows} rows, {act}")
+
+
 class _EagerMaskedAttention(nn.Module):
     def forward(self, q, k, v, mask):
         s = torch.matmul(q, k.transpose(-1, -2)) / float(q.shape[-1]) ** 0.5 + mask
