@@ -618,9 +618,9 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         from deplodock_amd.emit.flash_ws import emit_flash_ws
 
         return emit_flash_ws(body, name, ctx)
-    if body.dtype.name == "f32":
-        from deplodock_amd.emit.flash_f32 import emit_flash_f32
+    from deplodock_amd.emit.flash_f32 import emit_flash_f32, on_f32_atoms
 
+    if on_f32_atoms(body):
         return emit_flash_f32(body, name, ctx)
     D = body.head_dim
     if body.dtype.name not in ("bf16", "f16"):

@@ -1,4 +1,5 @@
-"""Streaming attention on fp32 operands: ``softmax(q k^T * scale + mask) v`` with fp32 MFMA atoms.
+"""Streaming attention on fp32 MFMA atoms: ``softmax(q k^T * scale + mask) v`` for fp32 operands, and for 16-bit
+operands whose rows are not whole 16-byte chunks (converted to fp32 as they are staged).
 
 fp32 is the precision the reference compiles (tests/perf/cases.py:20-23, its ``sdpa`` cases ``:174-190``); it reaches a
 streaming kernel by decomposing the fused op and finding the online ``(m, l, O)`` carrier again
@@ -93,19 +94,19 @@ _SRC = r"""
 
 // Four values of a row starting at column c (a multiple of 4): one 16-byte load where rows are whole aligned chunks,
 // else value by value; columns at or past the row's end read as zero.
-EMH_DEV f32x4 emh_row4(const float* __restrict__ row, int c) {
+EMH_DEV f32x4 emh_row4(const ELT* __restrict__ row, int c) {
   f32x4 r = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (VEC4) {
-    if (c < DR) r = *(const f32x4*)(row + c);
-  } else {
-    #pragma unroll
-    for (int i = 0; i < 4; ++i) if (c + i < DR) r[i] = row[c + i];
-  }
+#if VEC4
+  if (c < DR) r = *(const f32x4*)(row + c);
+#else
+  #pragma unroll
+  for (int i = 0; i < 4; ++i) if (c + i < DR) r[i] = (float)row[c + i];
+#endif
   return r;
 }
 
-extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__ Q, const float* __restrict__ Kp,
-                                                      const float* __restrict__ Vp MASK_PARAM, float* __restrict__ Op SYM_PARAM) {
+extern "C" __global__ __launch_bounds__(NT) void KNAME(const ELT* __restrict__ Q, const ELT* __restrict__ Kp,
+                                                      const ELT* __restrict__ Vp MASK_PARAM, ELT* __restrict__ Op SYM_PARAM) {
   extern __shared__ __attribute__((aligned(16))) float lds[];  // [2 buffers][K: BKV x KS | V: BKV x VS]
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int n = lane % 32, h = lane / 32;
@@ -126,7 +127,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
   // A lane's query, in the order the score atoms walk d: atoms 4u .. 4u+3 contract d = 8u + 4h + 0..3.
   float qf[DP / 8][4];
   if (owns_rows) {
-    const float* qp = Q + Q_OFF + (long)batch * Q_SB + (long)head * Q_SH + (long)qrow_c * Q_SS;
+    const ELT* qp = Q + Q_OFF + (long)batch * Q_SB + (long)head * Q_SH + (long)qrow_c * Q_SS;
     #pragma unroll
     for (int u = 0; u < DP / 8; ++u) {
       const f32x4 t = emh_row4(qp, 8 * u + 4 * h);
@@ -134,8 +135,8 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
       for (int i = 0; i < 4; ++i) qf[u][i] = t[i];
     }
   }
-  const float* kbase = Kp + K_OFF + (long)batch * K_SB + (long)kvh * K_SH;
-  const float* vbase = Vp + V_OFF + (long)batch * V_SB + (long)kvh * V_SH;
+  const ELT* kbase = Kp + K_OFF + (long)batch * K_SB + (long)kvh * K_SH;
+  const ELT* vbase = Vp + V_OFF + (long)batch * V_SB + (long)kvh * V_SH;
 #if HAS_MASK
   const MELT* mrow = Mp + M_OFF + (long)batch * M_SB + (long)head * M_SH + (long)qrow_c * M_SS;
 #endif
@@ -206,18 +207,18 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
   if (owns_rows && qrow < SQ) {  // lanes n and n + 32 hold the same query: both halves of an exchange are in or out together
     const float l = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = 1.0f / l;
-    float* op = Op + O_OFF + (long)batch * O_SB + (long)head * O_SH + (long)qrow * O_SS;
+    ELT* op = Op + O_OFF + (long)batch * O_SB + (long)head * O_SH + (long)qrow * O_SS;
     #pragma unroll
     for (int b = 0; b < NDB; ++b)
       #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int d = 32 * b + 8 * g + 4 * h;  // registers 4g .. 4g+3: output columns d .. d+3 of this lane's query
-        if (OVEC4) {
-          if (d < DR) { f32x4 y; y[0] = oacc[b][4 * g] * inv; y[1] = oacc[b][4 * g + 1] * inv; y[2] = oacc[b][4 * g + 2] * inv; y[3] = oacc[b][4 * g + 3] * inv; *(f32x4*)(op + d) = y; }
-        } else {
-          #pragma unroll
-          for (int i = 0; i < 4; ++i) if (d + i < DR) op[d + i] = oacc[b][4 * g + i] * inv;
-        }
+#if OVEC4
+        if (d < DR) { f32x4 y; y[0] = oacc[b][4 * g] * inv; y[1] = oacc[b][4 * g + 1] * inv; y[2] = oacc[b][4 * g + 2] * inv; y[3] = oacc[b][4 * g + 3] * inv; *(f32x4*)(op + d) = y; }
+#else
+        #pragma unroll
+        for (int i = 0; i < 4; ++i) if (d + i < DR) op[d + i] = (ELT)(oacc[b][4 * g + i] * inv);
+#endif
       }
   }
 }
@@ -412,10 +413,17 @@ def f32_supported(head_dim: int) -> bool:
     return 1 <= head_dim <= MAX_HEAD_DIM
 
 
+def on_f32_atoms(body: Flash) -> bool:
+    """Whether ``body`` is this emitter's: fp32 operands, or 16-bit rows that are not whole 16-byte chunks (the 16-bit
+    kernel pads whole chunks only), which are converted to fp32 as they are staged."""
+    return body.dtype.name == "f32" or (body.dtype.name in ("bf16", "f16") and body.head_dim % 8 != 0 and body.head_dim_real is None)
+
+
 def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     D = body.head_dim
-    if body.dtype.name != "f32":
-        raise LoweringError("flash (fp32 form): fp32 operands only")
+    if body.dtype.name not in ("f32", "bf16", "f16"):
+        raise LoweringError("flash (fp32 atoms): fp32, bf16 or fp16 operands")
+    narrow = body.dtype.name != "f32"  # 16-bit operands (rows the 16-bit kernel has no chunks for): converted as they are staged
     if not f32_supported(D) or body.head_dim_real not in (None, D):
         raise LoweringError(f"flash (fp32 form): head_dim {D} outside 1..{MAX_HEAD_DIM}")
     if body.q_heads % body.kv_heads:
@@ -436,7 +444,7 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     for key in symf:
         if key not in ("q_len", "kv_len") and not (key.split(".")[0] in ("q_strides", "k_strides", "v_strides", "o_strides", "mask_strides") and key.split(".")[1] in ("0", "1", "2")):
             raise LoweringError(f"flash: {key} cannot follow a symbolic axis")
-    vec_in, vec_out = whole_chunk_rows(body)
+    vec_in, vec_out = (False, False) if narrow else whole_chunk_rows(body)
     if private and not (vec_in and vec_out and D % 8 == 0):
         raise LoweringError("flash (fp32 form): the key-split form needs rows of whole, aligned pairs of 16-byte chunks")
 
@@ -449,7 +457,7 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     BQ = 32 * waves
     NT = 64 * kvs if private else THREADS
     defs = {
-        "KNAME": name, "NT": NT, "WAVES": waves, "KVS": kvs, "BQ": BQ, "BKV": BLOCK_KV, "D": D, "DR": D, "DP": DP, "DPL": DPL,
+        "KNAME": name, "ELT": rt.type_name(body.dtype.name), "NT": NT, "WAVES": waves, "KVS": kvs, "BQ": BQ, "BKV": BLOCK_KV, "D": D, "DR": D, "DP": DP, "DPL": DPL,
         "VEC4": int(vec_in), "OVEC4": int(vec_out), "PRE": int(DP <= 128),
         "SQ": c_value(symf.get("q_len", body.q_len)), "SKV": c_value(symf.get("kv_len", body.kv_len)),
         "HQ": body.q_heads, "GROUP": body.q_heads // body.kv_heads, "CAUSAL": int(bool(body.causal)), "XCDS": ctx.xcds,
@@ -513,4 +521,4 @@ def max_key_split(head_dim: int, lds_limit: int) -> int:
     return next((k for k in (8, 4, 2) if private_lds_bytes(head_dim, k) <= lds_limit), 1)
 
 
-__all__ = ["emit_flash_f32", "f32_supported", "lds_bytes", "padded_head_dim", "whole_chunk_rows", "max_key_split", "MAX_HEAD_DIM"]
+__all__ = ["emit_flash_f32", "f32_supported", "on_f32_atoms", "lds_bytes", "padded_head_dim", "whole_chunk_rows", "max_key_split", "MAX_HEAD_DIM"]

@@ -1,7 +1,8 @@
 """Attention outside the streaming kernels' reach is decomposed into loop nests before fusion.
 
-The flash kernels serve 16-bit operands whose rows are whole 16-byte chunks up to head_dim 256, and fp32 operands of any
-head_dim up to 256; what is left is 16-bit rows of other lengths, wider head dims, and mixed operand types.  The reference compiles fp32 only and its
+The flash kernels serve 16-bit operands whose rows are whole 16-byte chunks up to head_dim 256 and, on fp32 atoms, fp32
+operands and other 16-bit rows of any head_dim up to 256; what is left is wider head dims, value rows of another length
+than the keys', masks without a key axis and mixed operand types.  The reference compiles fp32 only and its
 perf cases call ``F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=...)`` on fp32 tensors
 (tests/perf/cases.py:64-69, 174-190); it lowers the fused op by decomposing it into ``q k^T -> * scale -> [+ mask] ->
 softmax -> @ v`` (emmy/compiler/pipeline/passes/frontend/decomposition/010_sdpa.py:53-138: grouped KV heads by
@@ -181,16 +182,19 @@ def decompose_attention(g: Graph, undo_repeat, streamed=None) -> Graph:
         if pinned_apart:
             return False
         q, k, v = (g.nodes[i].output for i in node.inputs[:3])
-        if q.dtype.name == "f32":
-            # the fp32 streaming kernel: any row length it has registers for, q / k / v rows alike
-            if not (k.dtype.name == v.dtype.name == "f32" and f32_head_dim(q.shape[-1]) and k.shape[-1] == v.shape[-1] == q.shape[-1]):
-                return False
-            if node.op.has_mask:  # the kernel reads a mask with the keys along its last axis; a column mask is left to the decomposed form
-                m = g.nodes[node.inputs[3]].output
-                if len(m.shape) > 4 or len(m.shape) < 1 or m.shape[-1] != k.shape[-2] or (k.shape[-2] == 1 and len(m.shape) > 1):
-                    return False
+        if q.dtype.name in ("bf16", "f16") and flash_head_dim(int(q.shape[-1])) is not None:
             return True
-        return q.dtype.name in ("bf16", "f16") and flash_head_dim(int(q.shape[-1])) is not None
+        # the kernel on fp32 atoms: fp32 operands, or 16-bit rows that are not whole 16-byte chunks — any row length it
+        # has registers for, q / k / v rows alike
+        if q.dtype.name not in ("f32", "bf16", "f16") or not (k.dtype.name == v.dtype.name == q.dtype.name):
+            return False
+        if not (f32_head_dim(q.shape[-1]) and k.shape[-1] == v.shape[-1] == q.shape[-1]):
+            return False
+        if node.op.has_mask:  # the kernel reads a mask with the keys along its last axis; a column mask is left to the decomposed form
+            m = g.nodes[node.inputs[3]].output
+            if len(m.shape) > 4 or len(m.shape) < 1 or m.shape[-1] != k.shape[-2] or (k.shape[-2] == 1 and len(m.shape) > 1):
+                return False
+        return True
 
     hits = [nid for nid, n in g.nodes.items() if isinstance(n.op, F.SdpaOp) and not (streamed or flash_takes)(n)]
     if not hits:

@@ -212,7 +212,9 @@ def _lower_flash(op: TileOp, ctx: Context) -> HipOp:
     one (two row groups x four key-split groups on 32-key blocks)."""
     body = op.body
     hip = _named(emit_flash(body, _PLACEHOLDER, ctx), op)
-    if body.dtype.name == "f32":
+    from deplodock_amd.emit.flash_f32 import on_f32_atoms
+
+    if on_f32_atoms(body):
         return hip  # one shape, sized to a wave's registers for every head_dim it takes
     steps = (("pair_steps", False), ("pair", False), ("shape", None))
     for what, value in steps:

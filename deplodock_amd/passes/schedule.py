@@ -552,7 +552,9 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
     560 against 637 for ``w4/kv64/s2``, causal 303 against 351; S=16384 causal 1087 / 1239;
     batch 4 S=2048 causal ``w8/kv64/s1/p`` 104 / 117; 16 heads S=4096 causal, 256 such
     workgroups unpaired: 122 against 94, hence the 2x cover asked of an unpaired triangle)."""
-    if body.dtype.name == "f32":
+    from deplodock_amd.emit.flash_f32 import on_f32_atoms
+
+    if on_f32_atoms(body):
         return _schedule_flash_f32(body, ctx)
     pinned = _pin("FLASH", _tuned(body, ctx))
     if pinned:
@@ -668,7 +670,7 @@ def _schedule_flash_f32(body: Flash, ctx: Context) -> dict:
     body.pair = body.deep = body.ws = body.sp = body.mfma_sum = False
     body.kv_ctas, body.block_kv = 1, 32
     heads = body.batch * body.q_heads
-    can_split = all(whole_chunk_rows(body)) and body.head_dim % 8 == 0
+    can_split = body.dtype.name == "f32" and all(whole_chunk_rows(body)) and body.head_dim % 8 == 0
     most = min(4, max_key_split(body.head_dim, ctx.lds_bytes_per_cu)) if can_split else 1
     symbolic = getattr(body, "sym", None) is not None and bool(body.sym.fields)
     if most > 1 and (body.kv_len > 32 or symbolic):

@@ -103,8 +103,13 @@ def test_which_attention_is_decomposed():
     assert _kernel_names(compiled) == ["k_sdpa_reduce"]
     (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
     assert "#define D 64\n" in op.kernel_source and "#define DR 32\n" in op.kernel_source
-    q36 = torch.randn(2, 4, 64, 36).bfloat16()
-    names = _kernel_names(be.compile(trace_module(_Sdpa().eval(), (q36, q36, q36))))
+    q36 = torch.randn(2, 4, 64, 36).bfloat16()  # rows that are not whole 16-byte chunks: the kernel on fp32 atoms, converting as it stages
+    compiled = be.compile(trace_module(_Sdpa().eval(), (q36, q36, q36)))
+    assert _kernel_names(compiled) == ["k_sdpa_reduce"]
+    (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert "mfma_f32_32x32x2f32" in op.kernel_source and "#define ELT __bf16\n" in op.kernel_source
+    q320 = torch.randn(1, 2, 40, 320).bfloat16()
+    names = _kernel_names(be.compile(trace_module(_Sdpa().eval(), (q320, q320, q320))))
     assert names.count("k_batched_linear") == 2 and "k_sdpa_reduce" not in names
 
 
@@ -123,7 +128,7 @@ def test_a_scores_tensor_beyond_the_limit_is_refused_with_a_message():
     the module is compiled, not when the runtime asks for the memory."""
     from deplodock_amd.passes.fuse import FusionError
 
-    q = torch.zeros(1, 32, 16384, 12).bfloat16()
+    q = torch.zeros(1, 32, 16384, 264).bfloat16()
     with pytest.raises(FusionError, match="16.0 GiB of scores"):
         HipBackend().compile(trace_module(_Sdpa(is_causal=True).eval(), (q, q, q)))
 

@@ -1495,11 +1495,41 @@ def test_fp32_attention_with_a_runtime_sequence_length(device):
         eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-5, f"fp32 attention, runtime length {s}")
 
 
-_DECOMPOSED_ATTENTION = {
-    # 16-bit rows that are not whole 16-byte chunks (the flash kernel pads whole chunks only)
+_NARROW_ON_FP32_ATOMS = {
+    # 16-bit rows that are not whole 16-byte chunks (the 16-bit flash kernel pads whole chunks only)
     "bf16_head_dim_36": (_FusedAttention(is_causal=True), torch.bfloat16, [(2, 4, 64, 36)] * 3, None),
     "bf16_head_dim_100": (_FusedAttention(), torch.bfloat16, [(2, 4, 50, 100)] * 3, None),
-    # fp32: head dims beyond the streaming kernel's registers, value rows of another length than the keys'
+    "fp16_head_dim_20_gqa_mask": (_FusedAttention(enable_gqa=True), torch.float16, [(2, 4, 70, 20), (2, 2, 90, 20), (2, 2, 90, 20)], lambda: torch.randn(2, 1, 70, 90)),
+    "bf16_head_dim_250_causal": (_FusedAttention(is_causal=True), torch.bfloat16, [(1, 2, 130, 250)] * 3, None),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", sorted(_NARROW_ON_FP32_ATOMS))
+def test_16_bit_attention_with_rows_that_are_not_whole_chunks_streams_on_fp32_atoms(device, case):
+    """16-bit attention whose head_dim is not a multiple of 8 takes the streaming kernel on fp32 atoms (operands converted
+    as they are staged, probabilities kept in fp32): one launch, no scores in device memory; against eager in float64."""
+    mod, dtype, shapes, mask = _NARROW_ON_FP32_ATOMS[case]
+    torch.manual_seed(41)
+    args = [torch.randn(*s).to(dtype) for s in shapes] + ([mask().to(dtype)] if mask else [])
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod.eval(), tuple(args)))
+    (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert op.kernel_name.startswith("k_sdpa_reduce") and op.knobs["FLASH"].startswith("f32/w")
+    prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in args))))
+    try:
+        prog.run()
+        torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = mod(*(t.double() for t in args)).float()
+    eager.assert_close(ours.float().reshape(want.shape), want, 2e-2, 2e-2, f"16-bit attention on fp32 atoms {case}")
+
+
+_DECOMPOSED_ATTENTION = {
+    # head dims beyond the streaming kernels' registers, value rows of another length than the keys', a mask without a key axis
+    "bf16_head_dim_320": (_FusedAttention(is_causal=True), torch.bfloat16, [(1, 2, 48, 320)] * 3, None),
     "fp32_head_dim_320": (_FusedAttention(is_causal=True), torch.float32, [(1, 2, 48, 320)] * 3, None),
     "fp32_value_rows_24": (_FusedAttention(), torch.float32, [(1, 2, 40, 16), (1, 2, 56, 16), (1, 2, 56, 24)], None),
     "fp32_column_mask": (_FusedAttention(), torch.float32, [(2, 2, 40, 32)] * 3, lambda: torch.randn(2, 1, 40, 1)),
@@ -1509,9 +1539,8 @@ _DECOMPOSED_ATTENTION = {
 @pytest.mark.gpu
 @pytest.mark.parametrize("case", sorted(_DECOMPOSED_ATTENTION))
 def test_attention_outside_the_flash_kernel(device, case):
-    """The fused attention op with 16-bit rows the flash kernel cannot pad to one of its widths, or fp32 shapes outside
-    the streaming kernel's: two batched MFMA contractions (fp32 atoms keep fp32 accuracy) around loop-nest stages,
-    against eager in float64."""
+    """The fused attention op in shapes no streaming kernel takes: two batched MFMA contractions (fp32 atoms keep fp32
+    accuracy) around loop-nest stages, against eager in float64."""
     mod, dtype, shapes, mask = _DECOMPOSED_ATTENTION[case]
     torch.manual_seed(41)
     args = [torch.randn(*s).to(dtype) for s in shapes] + ([mask().to(dtype)] if mask else [])
