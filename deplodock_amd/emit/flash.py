@@ -614,14 +614,14 @@ def lds_plan(waves: int, kvs: int, bkv: int, head_dim: int, limit: int, deep: bo
 
 
 def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
-    if body.ws or body.sp:
-        from deplodock_amd.emit.flash_ws import emit_flash_ws
-
-        return emit_flash_ws(body, name, ctx)
     from deplodock_amd.emit.flash_f32 import emit_flash_f32, on_f32_atoms
 
     if on_f32_atoms(body):
         return emit_flash_f32(body, name, ctx)
+    if body.ws or body.sp:
+        from deplodock_amd.emit.flash_ws import emit_flash_ws
+
+        return emit_flash_ws(body, name, ctx)
     D = body.head_dim
     if body.dtype.name not in ("bf16", "f16"):
         raise LoweringError("flash: MFMA tier needs 16-bit operands")

@@ -332,43 +332,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
       #pragma unroll
       for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(qf[u][i]));
   }
-  #pragma unroll 1
-  for (int j = grp; j < nblocks; j += KVS) {
-    const bool more = j + KVS < nblocks;
-    const int k0 = j * 32;
-    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NIV) : "memory");  // this block's K has landed (its V may still be on its way)
-    emh_lds_publish(kl);
-    f32x16 s;
-    #pragma unroll
-    for (int r = 0; r < 16; ++r) s[r] = 0.0f;
-    {
-      const float* kfrag = kl + n * 8 + h * 4;
-      #pragma unroll
-      for (int u = 0; u < DP / 8; ++u) {
-        const f32x4 kf = *(const f32x4*)(kfrag + u * 256);
-        #pragma unroll
-        for (int i = 0; i < 4; ++i) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[i], qf[u][i], s, 0, 0, 0);
-      }
-    }
-    // the K fragments are in registers (the atoms above consumed them): the region takes the next block
-    asm volatile("" :: "v"(s[0]) : "memory");
-    if (more) EMH_REQUEST_K(j + KVS)
-@SOFTMAX@
-    if (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NIK) : "memory");  // V of this block (the next K block may be on its way)
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    emh_lds_publish(vl);
-    #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = 8 * (r / 4) + 4 * h + (r % 4);
-      const float* vr = vl + row * DPL + (n % 4);
-      #pragma unroll
-      for (int b = 0; b < NDB; ++b) oacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[((8 * b + n / 4) ^ emh_vswz(row)) * 4], s[r], oacc[b], 0, 0, 0);
-    }
-    #pragma unroll
-    for (int b = 0; b < NDB; ++b) asm volatile("" :: "v"(oacc[b][0]) : "memory");  // every V fragment has been consumed
-    if (more) EMH_REQUEST_V(j + KVS)
-  }
-
+@LOOP@
   // Close: every wave leaves its unnormalised output rows, maximum and sum in its own region; after the barrier the
   // threads of the workgroup each finish 16-byte pieces of the output rows (consecutive threads, consecutive pieces).
   {
@@ -408,6 +372,156 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
 }
 """
 
+_LOOP_PLAIN = r"""  #pragma unroll 1
+  for (int j = grp; j < nblocks; j += KVS) {
+    const bool more = j + KVS < nblocks;
+    const int k0 = j * 32;
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NIV) : "memory");  // this block's K has landed (its V may still be on its way)
+    emh_lds_publish(kl);
+    f32x16 s;
+    #pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+    {
+      const float* kfrag = kl + n * 8 + h * 4;
+      #pragma unroll
+      for (int u = 0; u < DP / 8; ++u) {
+        const f32x4 kf = *(const f32x4*)(kfrag + u * 256);
+        #pragma unroll
+        for (int i = 0; i < 4; ++i) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[i], qf[u][i], s, 0, 0, 0);
+      }
+    }
+    // the K fragments are in registers (the atoms above consumed them): the region takes the next block
+    asm volatile("" :: "v"(s[0]) : "memory");
+    if (more) EMH_REQUEST_K(j + KVS)
+@SOFTMAX@
+    if (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NIK) : "memory");  // V of this block (the next K block may be on its way)
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    emh_lds_publish(vl);
+    #pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = 8 * (r / 4) + 4 * h + (r % 4);
+      const float* vr = vl + row * DPL + (n % 4);
+      #pragma unroll
+      for (int b = 0; b < NDB; ++b) oacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[((8 * b + n / 4) ^ emh_vswz(row)) * 4], s[r], oacc[b], 0, 0, 0);
+    }
+    #pragma unroll
+    for (int b = 0; b < NDB; ++b) asm volatile("" :: "v"(oacc[b][0]) : "memory");  // every V fragment has been consumed
+    if (more) EMH_REQUEST_V(j + KVS)
+  }
+
+"""
+
+# The software-pipelined order of the key-split form: the output atoms of block t-1 run under the softmax of block t
+# (one wave per SIMD: nothing else would fill the matrix pipe while the vector pipe takes exponentials).  Per step:
+# scores of block t -> request K(t+1) -> { P(t-1) V(t-1) atoms, interleaved with scale / mask / maximum of block t in
+# the first half and its exponentials in the second } -> request V(t) -> rescale (rare) -> P(t) becomes P(t-1).
+_PIPE_DEFS = r"""
+  #define EMH_SCORES(s_) { \
+    _Pragma("unroll") for (int r = 0; r < 16; ++r) s_[r] = 0.0f; \
+    const float* kfrag = kl + n * 8 + h * 4; \
+    _Pragma("unroll") for (int u = 0; u < DP / 8; ++u) { \
+      const f32x4 kf = *(const f32x4*)(kfrag + u * 256); \
+      _Pragma("unroll") for (int i = 0; i < 4; ++i) s_ = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[i], qf[u][i], s_, 0, 0, 0); \
+    } \
+    asm volatile("" :: "v"(s_[0]) : "memory");  /* the K fragments are in registers: the region takes the next block */ }
+  #if HAS_MASK
+  #define EMH_MASK_TERM(key_) + (float)mrow[(key_) < SKV ? (key_) : SKV - 1] * 1.4426950408889634f
+  #else
+  #define EMH_MASK_TERM(key_)
+  #endif
+  // element r of a block's scores: key k0 + 8 (r / 4) + 4 h + r % 4 of query qrow, in log2 units from here on
+  #define EMH_SCALE_ONE(s_, r, k0_) { \
+    const int key_ = (k0_) + 8 * ((r) / 4) + 4 * h + ((r) % 4); \
+    float v_ = s_[r] * SCALE_LOG2 EMH_MASK_TERM(key_); \
+    if (key_ >= SKV || (CAUSAL && key_ > qrow)) v_ = -__builtin_inff(); \
+    s_[r] = v_; mx = fmaxf(mx, v_); }
+  // The reference maximum is raised only when a row outgrows it by 2^8 (probabilities stay below 2^8, far inside fp32
+  // range), so the rescale of the accumulators is rare.
+  #define EMH_MAX_DONE() { \
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64)); \
+    raise = mx > m_run + 8.0f;  /* (from -inf any finite maximum raises; a block of masked keys never does) */ \
+    alpha = raise ? exp2f(m_run - mx) : 1.0f; \
+    m_run = raise ? mx : m_run; \
+    l_run *= alpha; \
+    m_use = m_run == -__builtin_inff() ? 0.0f : m_run;  /* nothing but masked keys so far: every term is 0 */ }
+  // (the empty asm keeps the exponential where it is written: its result is not needed before the next step's atoms, and
+  // the compiler would otherwise sink it out of the atoms' shadow)
+  #define EMH_EXP_ONE(s_, r) { s_[r] = exp2f(s_[r] - m_use); asm volatile("" : "+v"(s_[r])); l_run += s_[r]; }
+  #define EMH_RESCALE() if (__any(raise)) { \
+    _Pragma("unroll") for (int b = 0; b < NDB; ++b) _Pragma("unroll") for (int r = 0; r < 16; ++r) oacc[b][r] *= alpha; }
+  #define EMH_V_READ(P, r) { \
+    const int row_ = 8 * ((r) / 4) + 4 * h + ((r) % 4); \
+    const float* vr_ = vl + row_ * DPL + (n % 4); \
+    _Pragma("unroll") for (int b = 0; b < NDB; ++b) vf[P][b] = vr_[((8 * b + n / 4) ^ emh_vswz(row_)) * 4]; }
+  #define EMH_PV_MMA(P, p_, r) { \
+    _Pragma("unroll") for (int b = 0; b < NDB; ++b) oacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[P][b], p_[r], oacc[b], 0, 0, 0); }
+  #define EMH_V_CONSUMED() { _Pragma("unroll") for (int b = 0; b < NDB; ++b) asm volatile("" :: "v"(oacc[b][0]) : "memory"); }
+"""
+
+
+def _pipelined_loop() -> str:
+    o: list[str] = [_PIPE_DEFS]
+    a = o.append
+    a("  if (grp < nblocks) {")
+    a("    f32x16 p, s;")
+    a("    float vf[2][NDB];")
+    a("    float mx, alpha, m_use; bool raise;")
+    a("    // first block: scores and softmax, nothing to overlap yet")
+    a('    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NIV) : "memory");')
+    a("    emh_lds_publish(kl);")
+    a("    EMH_SCORES(p)")
+    a("    if (grp + KVS < nblocks) EMH_REQUEST_K(grp + KVS)")
+    a("    mx = -__builtin_inff();")
+    for r in range(16):
+        a(f"    EMH_SCALE_ONE(p, {r}, grp * 32)")
+    a("    EMH_MAX_DONE()")
+    for r in range(16):
+        a(f"    EMH_EXP_ONE(p, {r})")
+    a("    // the accumulators are still zero: a raise from -inf needs no rescale")
+    a("    #pragma unroll 1")
+    a("    for (int j = grp + KVS; j < nblocks; j += KVS) {")
+    a("      const bool more = j + KVS < nblocks;")
+    a("      const int k0 = j * 32;")
+    a("      // this block's K has landed; the first time round the V block before it is older than it and lands with it")
+    a('      if (j == grp + KVS) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");')
+    a('      else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NIV) : "memory");')
+    a("      emh_lds_publish(kl);")
+    a("      EMH_SCORES(s)")
+    a("      if (more) EMH_REQUEST_K(j + KVS)")
+    a('      if (more) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NIK) : "memory");  // V of the block before (the next K block may be on its way)')
+    a('      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");')
+    a("      emh_lds_publish(vl);")
+    a("      mx = -__builtin_inff();")
+    a("      EMH_V_READ(0, 0)")
+    for r in range(16):
+        # the V fragments of the next key are read before this key's atoms; a step's vector work stays behind its atoms
+        if r < 15:
+            a(f"      EMH_V_READ({(r + 1) % 2}, {r + 1})")
+        a(f"      EMH_PV_MMA({r % 2}, p, {r})")
+        if r < 8:
+            a(f"      EMH_SCALE_ONE(s, {2 * r}, k0) EMH_SCALE_ONE(s, {2 * r + 1}, k0)")
+        if r == 8:
+            a("      EMH_MAX_DONE()")
+        if r >= 8:
+            a(f"      EMH_EXP_ONE(s, {2 * (r - 8)}) EMH_EXP_ONE(s, {2 * (r - 8) + 1})")
+        a("      __builtin_amdgcn_sched_barrier(0);")
+    a("      EMH_V_CONSUMED()")
+    a("      EMH_REQUEST_V(j)")
+    a("      EMH_RESCALE()  // the atoms above added P(t-1) V(t-1) relative to the old reference maximum")
+    a("      p = s;")
+    a("    }")
+    a("    // last block: its output atoms")
+    a('    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");')
+    a("    emh_lds_publish(vl);")
+    a("    EMH_V_READ(0, 0)")
+    for r in range(16):
+        if r < 15:
+            a(f"    EMH_V_READ({(r + 1) % 2}, {r + 1})")
+        a(f"    EMH_PV_MMA({r % 2}, p, {r})")
+    a("  }")
+    return "\n".join(o) + "\n"
+
+
 
 def f32_supported(head_dim: int) -> bool:
     return 1 <= head_dim <= MAX_HEAD_DIM
@@ -428,8 +542,8 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         raise LoweringError(f"flash (fp32 form): head_dim {D} outside 1..{MAX_HEAD_DIM}")
     if body.q_heads % body.kv_heads:
         raise LoweringError("flash: q heads must be a multiple of kv heads")
-    if body.kv_ctas > 1 or body.pair or body.ws or body.sp or body.mfma_sum:
-        raise LoweringError("flash (fp32 form): no key split across workgroups, mirrored pairs or software-pipelined forms")
+    if body.kv_ctas > 1 or body.pair or body.ws or body.mfma_sum or (body.sp and body.kv_split < 2):
+        raise LoweringError("flash (fp32 form): no key split across workgroups or mirrored pairs; the software-pipelined order is the key-split form's")
     waves, kvs = body.waves, body.kv_split
     private = kvs > 1
     if (not private and waves not in (1, 2, 4)) or (private and (waves != 1 or kvs not in (2, 4, 8))):
@@ -475,7 +589,8 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     head = f"// {name}: fp32 B={body.batch} Hq={body.q_heads} Hkv={body.kv_heads} Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal}\n"
     head += "".join(f"#define {k} {v}\n" for k, v in defs.items())
     qblocks = -(-body.q_len // BQ)
-    src = (_SRC_PRIVATE if private else _SRC).replace("@SOFTMAX@", _SOFTMAX)
+    piped = private and bool(body.sp)
+    src = (_SRC_PRIVATE.replace("@LOOP@", _pipelined_loop() if piped else _LOOP_PLAIN) if private else _SRC).replace("@SOFTMAX@", _SOFTMAX)
     return HipOp(
         kernel_source=(prelude.header(prelude.DMA) if private else prelude.header()) + head + src,
         kernel_name=name,
@@ -487,7 +602,7 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         comment=f"flash fp32 Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} split={kvs}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
-        knobs={"FLASH": f"f32/s{kvs}" if private else f"f32/w{waves}"},
+        knobs={"FLASH": (f"f32/s{kvs}" + ("/sp" if piped else "")) if private else f"f32/w{waves}"},
     )
 
 

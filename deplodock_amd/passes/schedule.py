@@ -655,6 +655,10 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
     return {**knobs, "FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "") + ("/k3" if body.deep else "") + ("/ws" if body.ws else "") + ("/sp" if body.sp else "")}
 
 
+#: the key-split fp32 attention form runs its software-pipelined order unless pinned ``/np``
+_F32_PIPELINED = False
+
+
 def _schedule_flash_f32(body: Flash, ctx: Context) -> dict:
     """``EMMY_FLASH=f32/w<row groups>`` or ``f32/s<key-split waves>``.
 
@@ -678,19 +682,23 @@ def _schedule_flash_f32(body: Flash, ctx: Context) -> dict:
     else:
         body.waves, body.kv_split = next((w for w in (4, 2) if heads * -(-body.q_len // (32 * w)) >= ctx.compute_units), 1), 1
     pinned = _pin("FLASH", _tuned(body, ctx))
+    body.sp = body.kv_split > 1 and _F32_PIPELINED
     if pinned and pinned.split("/")[0] == "f32":
         try:
-            (tok,) = pinned.split("/")[1:]
+            tok, *rest = pinned.split("/")[1:]
             n = int(tok[1:])
-            if tok[0] == "w" and n in (1, 2, 4):
-                body.waves, body.kv_split = n, 1
+            if rest not in ([], ["sp"], ["np"]):
+                raise ValueError(rest)
+            if tok[0] == "w" and n in (1, 2, 4) and not rest:
+                body.waves, body.kv_split, body.sp = n, 1, False
             elif tok[0] == "s" and n in (2, 4, 8) and can_split and n <= max_key_split(body.head_dim, ctx.lds_bytes_per_cu):
                 body.waves, body.kv_split = 1, n
+                body.sp = rest == ["sp"] or (not rest and _F32_PIPELINED)
             else:
                 raise ValueError(tok)
         except ValueError:
             logger.warning("EMMY_FLASH=%r ignored: expect f32/w1, f32/w2, f32/w4 or f32/s2, f32/s4, f32/s8 (rows of whole 16-byte chunks, regions within the LDS)", pinned)
-    return {"FLASH": f"f32/s{body.kv_split}" if body.kv_split > 1 else f"f32/w{body.waves}"}
+    return {"FLASH": (f"f32/s{body.kv_split}" + ("/sp" if body.sp else "")) if body.kv_split > 1 else f"f32/w{body.waves}"}
 
 
 def _schedule_flash_split(body: Flash, ctx: Context, tuned: dict | None) -> dict:
