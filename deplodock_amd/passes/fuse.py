@@ -452,13 +452,14 @@ def _rec_matmul_residual(c: _Ctx, nid: str) -> bool:
 
 
 def _rec_matmul_gated(c: _Ctx, nid: str) -> bool:
-    """``act(x @ wg) * (x @ wu)`` on fp32 operands (the reference's ``gated_mlp`` perf cases, tests/perf/cases.py:213-232):
-    the gate product is a contraction of its own and the activation and the product with it ride in the output stage of
-    the up contraction — two launches instead of two contractions and a map.  (16-bit operands with constant weights
-    take the paired tile of ``_rec_gate_up``.)"""
+    """``act(x @ wg) * (x @ wu)`` with run-time weights (the reference's ``gated_mlp`` perf cases,
+    tests/perf/cases.py:213-232): the gate product is a contraction of its own and the activation (rounded where the
+    module rounds it) and the product with it ride in the output stage of the up contraction — two launches instead of
+    two contractions and a map.  (``F.linear`` over constant 16-bit weights takes the paired tile of ``_rec_gate_up``.)"""
     node = c.g.nodes[nid]
-    if not (_is(node, F.ElementwiseOp, fn="mul") and len(node.inputs) == 2) or node.output.dtype is not F32:
+    if not (_is(node, F.ElementwiseOp, fn="mul") and len(node.inputs) == 2):
         return False
+    od = node.output.dtype
     for si, ui in ((0, 1), (1, 0)):
         act, up = c.g.nodes[node.inputs[si]], c.g.nodes[node.inputs[ui]]
         if not (isinstance(act.op, F.ElementwiseOp) and act.op.fn in ("silu", "gelu_tanh", "gelu") and len(act.inputs) == 1 and c.single_use(act.id) and act.id not in c.g.outputs):
@@ -471,7 +472,7 @@ def _rec_matmul_gated(c: _Ctx, nid: str) -> bool:
             continue
         if math.prod(int(d) for d in ta.shape[:-2]) != 1 or int(tb.shape[1]) % 4 or int(tb.shape[0]) % 8:
             continue
-        if tuple(gate.output.shape) != tuple(node.output.shape) or tuple(up.output.shape) != tuple(node.output.shape) or gate.output.dtype is not F32 or up.output.dtype is not F32:
+        if tuple(gate.output.shape) != tuple(node.output.shape) or tuple(up.output.shape) != tuple(node.output.shape) or gate.output.dtype != od or up.output.dtype != od or act.output.dtype != od:
             continue
         g_view = _need(c, gate.id)
         if not g_view.is_contiguous() or g_view.offset:
@@ -480,7 +481,7 @@ def _rec_matmul_gated(c: _Ctx, nid: str) -> bool:
         bt = _transposed_parameter(c, View(b.base, b.offset, (b.shape[1], b.shape[0]), (b.strides[1], b.strides[0]), b.dtype))
         if len(a.shape) > 2:
             bt = View(bt.base, bt.offset, (*(1,) * (len(a.shape) - 2), *bt.shape), (*(0,) * (len(a.shape) - 2), *bt.strides), bt.dtype)
-        _emit_batched_contraction(c, nid, a, bt, f"matmul_{act.op.fn}_mul", residual=g_view, post=E.Un(act.op.fn, E.Var("res")) * E.Var("y"))
+        _emit_batched_contraction(c, nid, a, bt, f"matmul_{act.op.fn}_mul", residual=g_view, post=_round(od, E.Un(act.op.fn, E.Var("res"))) * E.Var("y"))
         return True
     return False
 
