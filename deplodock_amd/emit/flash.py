@@ -618,6 +618,10 @@ def emit_flash(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
 
     if on_f32_atoms(body):
         return emit_flash_f32(body, name, ctx)
+    if body.private:
+        from deplodock_amd.emit.flash_pv import emit_flash_pv
+
+        return emit_flash_pv(body, name, ctx)
     if body.ws or body.sp:
         from deplodock_amd.emit.flash_ws import emit_flash_ws
 

@@ -216,6 +216,10 @@ def _lower_flash(op: TileOp, ctx: Context) -> HipOp:
 
     if on_f32_atoms(body):
         return hip  # one shape, sized to a wave's registers for every head_dim it takes
+    if body.private:
+        if _spills(hip, ctx):
+            raise LoweringError(f"{hip.kernel_name}: the key-split-waves form spills vector registers")
+        return hip
     steps = (("pair_steps", False), ("pair", False), ("shape", None))
     for what, value in steps:
         spilled = _spills(hip, ctx)

@@ -559,9 +559,11 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
     pinned = _pin("FLASH", _tuned(body, ctx))
     if pinned:
         try:
-            body.pair = body.deep = body.ws = body.sp = body.mfma_sum = False
+            body.pair = body.deep = body.ws = body.sp = body.mfma_sum = body.private = False
             for tok in pinned.split("/"):
-                if tok == "p":
+                if tok == "pv":
+                    body.private = True
+                elif tok == "p":
                     body.pair = True
                 elif tok == "ms":
                     body.mfma_sum = True
@@ -578,9 +580,18 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 elif tok.startswith("s"):
                     body.kv_split = int(tok[1:])
                 else:
-                    raise ScheduleError(f"cannot parse {tok!r} (expect w<groups> / kv<keys> / s<split> / p / k3 / ms / ws / sp)")
+                    raise ScheduleError(f"cannot parse {tok!r} (expect w<groups> / kv<keys> / s<split> / p / k3 / ms / ws / sp / pv)")
             if body.ws and body.sp:
                 raise ScheduleError("ws and sp are two forms: pin one")
+            if body.private:
+                from deplodock_amd.emit.flash_pv import max_key_split as pv_max_split
+                from deplodock_amd.emit.flash_pv import pv_supported
+
+                why = pv_supported(body)
+                if why is not None:
+                    raise ScheduleError(f"the key-split-waves form needs {why}")
+                if body.waves != 1 or body.block_kv != 32 or body.kv_split not in (2, 4, 8) or body.kv_split > pv_max_split(body.head_dim, ctx.lds_bytes_per_cu) or body.pair or body.deep or body.ws or body.sp or body.mfma_sum:
+                    raise ScheduleError("the key-split-waves form is w1/kv32/s<2|4|8>/pv within the LDS")
             if body.ws or body.sp:
                 from deplodock_amd.emit.flash_ws import ws_supported
 
@@ -589,9 +600,9 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 if why is not None:
                     raise ScheduleError(f"the software-pipelined forms need {why}")
             chunks = body.block_kv * body.head_dim // 8
-            if body.waves < 1 or body.kv_split < 1 or body.block_kv % 32 or (not (body.ws or body.sp) and chunks % (body.waves * body.kv_split * 64)):
+            if body.waves < 1 or body.kv_split < 1 or body.block_kv % 32 or (not (body.ws or body.sp or body.private) and chunks % (body.waves * body.kv_split * 64)):
                 raise ScheduleError("unrealisable workgroup shape")
-            if not (body.ws or body.sp) and _flash_lds(body, ctx) > ctx.lds_bytes_per_cu:
+            if not (body.ws or body.sp or body.private) and _flash_lds(body, ctx) > ctx.lds_bytes_per_cu:
                 raise ScheduleError("the double-buffered K/V blocks of all key-split groups exceed the LDS")
             if (body.head_dim // 32 * 16) % (4 * body.kv_split):
                 raise ScheduleError("the key-split groups cannot share a lane's output registers")
@@ -607,7 +618,7 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
         def blocks(w: int) -> int:
             return -(-body.q_len // (32 * w))
 
-        body.pair = body.deep = body.ws = body.sp = False
+        body.pair = body.deep = body.ws = body.sp = body.private = False
         body.waves = 0
         if body.head_dim <= 128 and body.kv_len >= 2048:
             # Enough rows to give every CU a 256-row workgroup: eight query waves share each
@@ -651,6 +662,9 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                 body.kv_split //= 2
     if getattr(body, "sym", None) is not None and body.sym.fields:
         body.pair = False  # pairing mirrored query blocks needs the block count when the kernel is built
+    if body.private:
+        body.kv_ctas = 1
+        return {"FLASH": f"w1/kv32/s{body.kv_split}/pv"}
     knobs = _schedule_flash_split(body, ctx, tuned if (tuned := _tuned(body, ctx)) else None)
     return {**knobs, "FLASH": f"w{body.waves}/kv{body.block_kv}/s{body.kv_split}" + ("/p" if body.pair else "") + ("/k3" if body.deep else "") + ("/ws" if body.ws else "") + ("/sp" if body.sp else "")}
 

@@ -406,6 +406,46 @@ def test_c4_every_workgroup_shape(device, pin, monkeypatch):
         prog.close()
 
 
+@pytest.mark.parametrize("split", [2, 4, 8])
+@pytest.mark.parametrize("d", [128, 64])
+def test_c4_key_split_waves(device, split, d, monkeypatch):
+    """``FLASH=w1/kv32/s<k>/pv``: one 32-row group per workgroup whose k waves take every k-th key block and stage for
+    themselves, merged once at the close.  Causal and not, grouped heads, ragged lengths (a last query block that is
+    partly empty, keys that end inside a block, fewer blocks than waves), unequal lengths, an additive mask with holes;
+    ten launches of the first shape (the first blocks are consumed right after they land); against eager and the
+    streaming restatement in float64."""
+    monkeypatch.setenv("EMMY_FLASH", f"w1/kv32/s{split}/pv")
+    torch.manual_seed(61)
+    shapes = [(1, 8, 4, 320, 320, True), (2, 4, 2, 200, 200, True), (1, 4, 4, 96, 160, False), (1, 6, 2, 33, 33, True), (1, 2, 2, 1, 70, False), (1, 4, 2, 70, 45, True)]
+    for n_case, (b, hq, hkv, sq, skv, causal) in enumerate(shapes):
+        q, k, v = torch.randn(b, hq, sq, d).bfloat16(), torch.randn(b, hkv, skv, d).bfloat16(), torch.randn(b, hkv, skv, d).bfloat16()
+        case = eager.Case("pv", eager.Sdpa(causal), (q, k, v), 2e-2, 2e-2)
+        be = HipBackend()
+        compiled = be.compile(trace_module(case.module, case.inputs))
+        assert [n.op.knobs["FLASH"] for n in compiled.nodes.values() if isinstance(n.op, HipOp)] == [f"w1/kv32/s{split}/pv"]
+        want = eager.run_eager(case, device)
+        prog = be.program(compiled, {n: t.to(device) for n, t in zip(compiled.inputs, case.inputs)})
+        try:
+            out = prog.output_tensors()[compiled.outputs[0]]
+            for rep in range(10 if n_case == 0 else 1):
+                out.zero_()
+                prog.run()
+                torch.cuda.synchronize()
+                eager.assert_close(out.reshape(want.shape), want, 2e-2, 2e-2, f"sdpa pv s{split} d={d} {(b, hq, hkv, sq, skv, causal)} launch {rep}")
+            ref = O.flash_attention(q.float().numpy(), k.float().numpy(), v.float().numpy(), is_causal=causal, scale=d ** -0.5, block_kv=64)
+            eager.assert_close(out.reshape(want.shape), torch.from_numpy(ref).float(), 2e-2, 2e-2, f"sdpa pv s{split} d={d} vs streaming restatement")
+        finally:
+            prog.close()
+    q, k, v = torch.randn(2, 4, 70, d).bfloat16(), torch.randn(2, 2, 300, d).bfloat16(), torch.randn(2, 2, 300, d).bfloat16()
+    mask = (2 * torch.randn(2, 1, 70, 300)).bfloat16()
+    mask[torch.rand(2, 1, 70, 300) < 0.3] = -float("inf")
+    mask[..., 0] = 0.5
+    case = eager.Case("pv masked", eager.MaskedSdpa().eval(), (q, k, v, mask), 2e-2, 2e-2)
+    ours, want, compiled = run_case(case, device)
+    assert [n.op.knobs["FLASH"] for n in compiled.nodes.values() if isinstance(n.op, HipOp)] == [f"w1/kv32/s{split}/pv"]
+    eager.assert_close(ours, want, 2e-2, 2e-2, f"masked sdpa pv s{split} d={d} vs eager")
+
+
 @pytest.mark.parametrize("pin", ["w2/kv32/s4/p", "w1/kv64/s2/p", "w4/kv64/s2/p", "w2/kv64/s1/p", "w8/kv64/s1/p"])
 def test_c4_mirrored_query_block_pairs(device, pin, monkeypatch):
     """A workgroup that takes query block b and then block n-1-b reuses its LDS and
