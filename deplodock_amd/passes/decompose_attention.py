@@ -192,7 +192,7 @@ def decompose_attention(g: Graph, undo_repeat, streamed=None) -> Graph:
             return False
         if node.op.has_mask:  # the kernel reads a mask with the keys along its last axis; a column mask is left to the decomposed form
             m = g.nodes[node.inputs[3]].output
-            if len(m.shape) > 4 or len(m.shape) < 1 or m.shape[-1] != k.shape[-2] or (k.shape[-2] == 1 and len(m.shape) > 1):
+            if len(m.shape) > 4 or len(m.shape) < 1 or m.shape[-1] != k.shape[-2]:
                 return False
         return True
 

@@ -174,7 +174,7 @@ def _wide_case(kind: str, rnd: random.Random, seed: int):
 @pytest.mark.parametrize("kind", ["matmul", "attention32", "linear32"])
 def test_seeded_random_shapes_against_float64(device, kind):
     """Families that reach the batched contraction, the layout-change copy, zero-padded ragged extents, the
-    decomposed attention and the fp32 tier's split of an underfilled launch: against the module in float64
+    fp32 streaming attention kernel and the fp32 tier's split of an underfilled launch: against the module in float64
     (fp32: 1e-4 of the output's RMS; 16-bit: rtol 2e-2)."""
     import copy
 
