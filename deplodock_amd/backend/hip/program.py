@@ -36,6 +36,7 @@ _STATIC_LDS_CAP = 64 * 1024  # per-workgroup LDS available without opting in
 _KERNEL_TIMEOUT_MS = 1000.0  # per-window watchdog
 _WARMUP_TARGET_MS = 10.0  # keep warming until this much device time has run
 _BATCH_TARGET_MS = 1.0  # launches per event window are sized to cover this
+_PASS_TARGET_MS = 100.0  # ... but a pass over all of a program's windows to no more than this (a program of hundreds of launches)
 _AUTO_BUDGET_MS = 100.0
 _AUTO_MAX_ITERS = 20000
 _SLAB_ALIGN = 256
@@ -695,11 +696,11 @@ class SampleBudget:
         return samples >= self.max_samples or (self.device_ms is not None and measured_ms >= self.device_ms)
 
 
-def window_issues(per_issue_ms: float) -> int:
-    """Back-to-back issues of one launch that make an event window of about ``_BATCH_TARGET_MS``."""
-    if not 0.0 < per_issue_ms < _BATCH_TARGET_MS:
+def window_issues(per_issue_ms: float, target_ms: float = _BATCH_TARGET_MS) -> int:
+    """Back-to-back issues of one launch that make an event window of about ``target_ms``."""
+    if not 0.0 < per_issue_ms < target_ms:
         return 1
-    return max(1, round(_BATCH_TARGET_MS / per_issue_ms))
+    return max(1, round(target_ms / per_issue_ms))
 
 
 class _BenchSession:
@@ -745,7 +746,8 @@ class _BenchSession:
 
     def settle(self) -> None:
         if self.last:
-            self.issues = [window_issues(dt) for dt in self.last]
+            target = min(_BATCH_TARGET_MS, _PASS_TARGET_MS / max(1, self.n))
+            self.issues = [window_issues(dt, target) for dt in self.last]
         self._capture_windows()
         if not self.last:
             return  # no warm-up asked for: sample from the first pass on

@@ -49,6 +49,7 @@ def test_unknown_buffer_is_rejected():
 
 def test_batch_calibration_and_iter_budget():
     assert [program.window_issues(dt) for dt in (0.002, 0.5, 3.0, 0.0)] == [500, 2, 1, 1]
+    assert [program.window_issues(dt, 0.25) for dt in (0.002, 0.5)] == [125, 1]  # (a program of 400 launches: windows of a quarter millisecond)
     fixed = program.SampleBudget.parse(20)
     assert not fixed.spent(19, 1e9) and fixed.spent(20, 0.0)
     auto = program.SampleBudget.parse("auto")
