@@ -148,7 +148,7 @@ def _materialize(c: _Ctx, nid: str) -> None:
             c.out.add_constant(nid, t.shape, t.dtype, value=node.op.value, source_path=node.op.source_path)
         c.done[nid] = nid
         return
-    for rec in (_rec_same_type_cast, _rec_loop_nest, _rec_batched_linear, _rec_matmul_residual, _rec_matmul_gated, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_layer_norm, _rec_softmax, _rec_sdpa, _rec_row_fused, _rec_row_sum, _rec_gather, _rec_cat, _rec_pointwise):
+    for rec in (_rec_same_type_cast, _rec_loop_nest, _rec_batched_linear, _rec_matmul_residual, _rec_matmul_gated, _rec_matmul, _rec_linear_residual, _rec_gate_up, _rec_gate_up_f32, _rec_linear_siblings, _rec_linear, _rec_rope_pair, _rec_rope, _rec_rms_chain, _rec_rms_op, _rec_layer_norm, _rec_softmax, _rec_sdpa, _rec_row_fused, _rec_row_sum, _rec_gather, _rec_cat, _rec_pointwise):
         if rec(c, nid):
             return
     raise FusionError(f"no kernel recognizer for {type(node.op).__name__} at node {nid!r}")
@@ -615,10 +615,40 @@ def _rec_linear_residual(c: _Ctx, nid: str) -> bool:
     return False
 
 
+def _rec_gate_up_f32(c: _Ctx, nid: str) -> bool:
+    """``act(gate(x)) * up(x)`` on fp32 operands: the paired tile of ``_rec_gate_up`` is written for 16-bit operands, so
+    the gate projection stays a contraction of its own and its activation and the product ride in the output stage of
+    the up projection (two launches instead of two contractions and a map)."""
+    node = c.g.nodes[nid]
+    if not (_is(node, F.ElementwiseOp, fn="mul") and len(node.inputs) == 2) or node.output.dtype is not F32:
+        return False
+    for si, ui in ((0, 1), (1, 0)):
+        act, up = c.g.nodes[node.inputs[si]], c.g.nodes[node.inputs[ui]]
+        if not (isinstance(act.op, F.ElementwiseOp) and act.op.fn in ("silu", "gelu_tanh", "gelu") and len(act.inputs) == 1 and c.single_use(act.id) and act.id not in c.g.outputs):
+            continue
+        gate = c.g.nodes[act.inputs[0]]
+        if not (isinstance(gate.op, F.LinearOp) and isinstance(up.op, F.LinearOp) and c.single_use(gate.id) and c.single_use(up.id)) or up.id in c.done or up.id in c.g.outputs or gate.id in c.g.outputs:
+            continue
+        if tuple(gate.output.shape) != tuple(node.output.shape) or tuple(up.output.shape) != tuple(node.output.shape) or gate.output.dtype is not F32 or up.output.dtype is not F32:
+            continue
+        g_view = _need(c, gate.id)
+        if not g_view.is_contiguous() or g_view.offset:
+            continue
+        x, w, m, n, k, lda, ldb, pro, extra = _linear_parts(c, up.id)
+        body = Contraction(
+            m=m, n=n, k=k, a=x.base, b=w.base, out=nid, in_dtype=x.dtype, out_dtype=F32, lda=lda, ldb=ldb, a_offset=x.offset, b_offset=w.offset,
+            post=E.Un(act.op.fn, E.Var("res")) * E.Var("y"), epilogue_operands=(("res", F32),), a_prologue=pro, **(bias := _bias_of(c, up.id, n)),
+        )  # fmt: skip
+        body.operand_buffers = {"res": g_view.base}
+        _emit(c, nid, body, f"linear_{act.op.fn}_mul", [x.base, w.base, *extra, *([bias["bias"]] if bias else []), g_view.base])
+        return True
+    return False
+
+
 def _rec_gate_up(c: _Ctx, nid: str) -> bool:
     node = c.g.nodes[nid]
     if not (_is(node, F.ElementwiseOp, fn="mul") and len(node.inputs) == 2) or node.output.dtype.nbytes != 2:
-        return False  # (the paired tile is written for 16-bit operands: fp32 keeps two contractions and a map)
+        return False  # (the paired tile is written for 16-bit operands: fp32 takes ``_rec_gate_up_f32``)
     for si, ui in ((0, 1), (1, 0)):
         silu = c.g.nodes[node.inputs[si]]
         up = c.g.nodes[node.inputs[ui]]
