@@ -14,7 +14,6 @@ from __future__ import annotations
 import contextlib
 import fcntl
 import logging
-import math
 import statistics
 import time
 from dataclasses import dataclass, field

@@ -35,7 +35,7 @@ from deplodock_amd.emit.errors import LoweringError
 from deplodock_amd.ir import expr as E
 from deplodock_amd.ir.hip import HipOp
 from deplodock_amd.ir.schedule import Stage
-from deplodock_amd.ir.sym import Affine, XcdRounds, c_value, param_name
+from deplodock_amd.ir.sym import XcdRounds, c_value, param_name
 from deplodock_amd.ir.tile import Contraction
 
 

@@ -21,7 +21,7 @@ designed for wave64 instead of translated:
 from __future__ import annotations
 
 from deplodock_amd.context import Context
-from deplodock_amd.dtype import BF16, F16, F32, DType
+from deplodock_amd.dtype import BF16, F16, DType
 from deplodock_amd.emit import prelude
 from deplodock_amd.render_target import rt
 from deplodock_amd.emit.errors import LoweringError

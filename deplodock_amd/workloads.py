@@ -9,7 +9,6 @@ PyTorch eager is the business of the test-side oracle, not of this module.
 
 from __future__ import annotations
 
-import math
 from dataclasses import dataclass
 
 import torch
