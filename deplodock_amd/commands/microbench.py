@@ -425,7 +425,7 @@ def handle_fp32_attention(args) -> None:
             torch.cuda.synchronize()
             row = [str(seq), f"{case.algo_flops / 1e9:.2f}"]
             best = None
-            for pin in (None, "f32/w4", "f32/s2", "f32/s2/sp", "f32/s4", "f32/s4/sp", "decompose"):
+            for pin in (None, "f32/w4", "f32/s2", "f32/s2/sp", "f32/s4", "f32/s4/sp", "f32/s4/o", "f32/s8/o", "decompose"):
                 if pin == "decompose" and seq > 2048:
                     row.append("")
                     continue
@@ -451,7 +451,7 @@ def handle_fp32_attention(args) -> None:
         else:
             os.environ["EMMY_FLASH"] = saved
     print("fp32 causal attention, 16 query / 8 key-value heads of 128, us per call (the decomposed route: sum of its kernels)")
-    for line in render_table(["S", "GFLOP", "default", "w4", "s2", "s2/sp", "s4", "s4/sp", "decomposed", "eager fp32", "TFLOP/s", "of fp32 MFMA peak"], rows, "rrlrrrrrrrrr"):
+    for line in render_table(["S", "GFLOP", "default", "w4", "s2", "s2/sp", "s4", "s4/sp", "s4/o", "s8/o", "decomposed", "eager fp32", "TFLOP/s", "of fp32 MFMA peak"], rows, "rrlrrrrrrrrrrr"):
         print(line)
 
 

@@ -236,8 +236,13 @@ _SRC_PRIVATE = r"""
 #define NIK (DP / 8)                   /* requests of a wave per K block: 32 rows x two chunks each */
 #define NIV (32 / RPR)                 /* requests of a wave per V block: whole rows */
 #define NDB (DP / 32)                  /* 32-column blocks of the output */
+#if ONE_REGION
+#define REGION (32 * DPL)             /* floats of LDS per wave in the loop: its K block and its V block take turns */
+#else
 #define REGION (32 * DP + 32 * DPL)    /* floats of LDS per wave: its K block, then its V block */
+#endif
 #define PS (DPL + 4)                   /* floats per row of a wave's partial output at the close */
+#define PART (ONE_REGION ? 32 * PS + 64 : REGION)  /* floats between the waves' partials at the close */
 // K lies in LDS as [pair of chunks u][row][8 floats]: the 16-byte fragment reads of a wave at one u (row n, half h) are
 // 1 KiB in a row, conflict-free, and request u of a block is one lane offset plus 32 bytes x u.  V keeps [row][d] with its
 // 128-byte halves swapped between rows r and r + 4, the two rows a 4-byte read touches; the rows of one request share
@@ -247,7 +252,13 @@ EMH_DEV int emh_vswz(int row) { return CPRL >= 16 ? ((row >> 2) & 1) << 3 : 0; }
 // that never count — q's columns there are zero, and v's only reach output columns that are not stored
 EMH_DEV int emh_gchunk(int c) { return c < DR / 4 ? c : 0; }
 
-extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__ Q, const float* __restrict__ Kp,
+// (one region a wave: two waves a SIMD is the point, so the register budget is half the file)
+#if ONE_REGION
+#define EMH_OCCUPANCY __attribute__((amdgpu_waves_per_eu(2)))
+#else
+#define EMH_OCCUPANCY
+#endif
+extern "C" __global__ __launch_bounds__(NT) EMH_OCCUPANCY void KNAME(const float* __restrict__ Q, const float* __restrict__ Kp,
                                                       const float* __restrict__ Vp MASK_PARAM, float* __restrict__ Op SYM_PARAM) {
   extern __shared__ __attribute__((aligned(16))) float lds[];  // [KVS waves][K: DP / 8 x 32 x 8 | V: 32 x DPL]
   const int tid = threadIdx.x, lane = tid % 64, grp = __builtin_amdgcn_readfirstlane(tid / 64);
@@ -273,7 +284,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
   const int nblocks = (kend + 31) / 32;
 
   float* kl = lds + grp * REGION;
-  float* vl = kl + 32 * DP;
+  float* vl = ONE_REGION ? kl : kl + 32 * DP;
   const unsigned kl_s = emh_uniform(emh_lds_addr(kl)), vl_s = emh_uniform(emh_lds_addr(vl));
   // Lane offsets of the requests of a block that lies wholly inside the sequence: K request u is rows lane / 2, chunk
   // 2 u + lane % 2; V request i is rows i RPR + lane / CPRL, chunk position lane % CPRL, which holds chunk position ^ swap.
@@ -312,7 +323,7 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
 
   if (grp < nblocks) {
     EMH_REQUEST_K(grp)
-    EMH_REQUEST_V(grp)
+    if (!ONE_REGION) EMH_REQUEST_V(grp)
   }
   // The query's values, requested behind the first blocks and waited for here, before the loop: a load of the
   // compiler's own still outstanding at the loop's head would make it wait inside the loop, by a count that knows
@@ -333,11 +344,13 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
       for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(qf[u][i]));
   }
 @LOOP@
-  // Close: every wave leaves its unnormalised output rows, maximum and sum in its own region; after the barrier the
-  // threads of the workgroup each finish 16-byte pieces of the output rows (consecutive threads, consecutive pieces).
+  // Close: every wave leaves its unnormalised output rows, maximum and sum in LDS; after the barrier the threads of
+  // the workgroup each finish 16-byte pieces of the output rows (consecutive threads, consecutive pieces).  Where the
+  // partials are wider than the loop's regions they overlap a neighbour's blocks: every wave is done with those first.
+  if (ONE_REGION) __syncthreads();
   {
     const float l = l_run + __shfl_xor(l_run, 32, 64);
-    float* part = lds + grp * REGION;
+    float* part = lds + grp * PART;
     #pragma unroll
     for (int b = 0; b < NDB; ++b)
       #pragma unroll
@@ -353,13 +366,13 @@ extern "C" __global__ __launch_bounds__(NT) void KNAME(const float* __restrict__
     if (q0 + row >= SQ) continue;
     float m = -__builtin_inff();
     #pragma unroll
-    for (int g = 0; g < KVS; ++g) m = fmaxf(m, lds[g * REGION + 32 * PS + 2 * row]);
+    for (int g = 0; g < KVS; ++g) m = fmaxf(m, lds[g * PART + 32 * PS + 2 * row]);
     const float m_use = m == -__builtin_inff() ? 0.0f : m;
     float l = 0.0f;
     f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
     #pragma unroll
     for (int g = 0; g < KVS; ++g) {
-      const float* part = lds + g * REGION;
+      const float* part = lds + g * PART;
       const float w = exp2f(part[32 * PS + 2 * row] - m_use);
       l += part[32 * PS + 2 * row + 1] * w;
       const f32x4 t = *(const f32x4*)(part + row * PS + c4);
@@ -407,6 +420,48 @@ _LOOP_PLAIN = r"""  #pragma unroll 1
     #pragma unroll
     for (int b = 0; b < NDB; ++b) asm volatile("" :: "v"(oacc[b][0]) : "memory");  // every V fragment has been consumed
     if (more) EMH_REQUEST_V(j + KVS)
+  }
+
+"""
+
+# One region a wave: its K block and its V block take turns in it.  A wave then waits for each landing in the open —
+# the V block is requested when the scores are done and has only the softmax to land under, the next K block is
+# requested after the output atoms — but a wave needs half the LDS, so a SIMD holds two of them and one's atoms fill
+# the other's waits.
+_LOOP_ONE = r"""  #pragma unroll 1
+  for (int j = grp; j < nblocks; j += KVS) {
+    const bool more = j + KVS < nblocks;
+    const int k0 = j * 32;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this block's K has landed: nothing else is on its way
+    emh_lds_publish(kl);
+    f32x16 s;
+    #pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+    {
+      const float* kfrag = kl + n * 8 + h * 4;
+      #pragma unroll
+      for (int u = 0; u < DP / 8; ++u) {
+        const f32x4 kf = *(const f32x4*)(kfrag + u * 256);
+        #pragma unroll
+        for (int i = 0; i < 4; ++i) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[i], qf[u][i], s, 0, 0, 0);
+      }
+    }
+    // the K fragments are in registers (the atoms above consumed them): the region takes this block's V
+    asm volatile("" :: "v"(s[0]) : "memory");
+    EMH_REQUEST_V(j)
+@SOFTMAX@
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    emh_lds_publish(vl);
+    #pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = 8 * (r / 4) + 4 * h + (r % 4);
+      const float* vr = vl + row * DPL + (n % 4);
+      #pragma unroll
+      for (int b = 0; b < NDB; ++b) oacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[((8 * b + n / 4) ^ emh_vswz(row)) * 4], s[r], oacc[b], 0, 0, 0);
+    }
+    #pragma unroll
+    for (int b = 0; b < NDB; ++b) asm volatile("" :: "v"(oacc[b][0]) : "memory");  // every V fragment has been consumed
+    if (more) EMH_REQUEST_K(j + KVS)
   }
 
 """
@@ -550,7 +605,7 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         raise LoweringError(f"flash (fp32 form): w{waves}/s{kvs} is neither 1, 2 or 4 row groups nor one row group of 2, 4 or 8 key-split waves")
     DP = padded_head_dim(D)
     DPL = 1 << (DP - 1).bit_length()
-    lds = private_lds_bytes(D, kvs) if private else lds_bytes(D)
+    lds = private_lds_bytes(D, kvs, bool(body.one_region)) if private else lds_bytes(D)
     if lds > ctx.lds_bytes_per_cu:
         raise LoweringError(f"flash (fp32 form): {lds} B of LDS exceeds {ctx.lds_bytes_per_cu} B per CU")
     sym = getattr(body, "sym", None)
@@ -572,7 +627,7 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     NT = 64 * kvs if private else THREADS
     defs = {
         "KNAME": name, "ELT": rt.type_name(body.dtype.name), "NT": NT, "WAVES": waves, "KVS": kvs, "BQ": BQ, "BKV": BLOCK_KV, "D": D, "DR": D, "DP": DP, "DPL": DPL,
-        "VEC4": int(vec_in), "OVEC4": int(vec_out), "PRE": int(DP <= 128),
+        "VEC4": int(vec_in), "OVEC4": int(vec_out), "PRE": int(DP <= 128), "ONE_REGION": int(bool(body.one_region) and private),
         "SQ": c_value(symf.get("q_len", body.q_len)), "SKV": c_value(symf.get("kv_len", body.kv_len)),
         "HQ": body.q_heads, "GROUP": body.q_heads // body.kv_heads, "CAUSAL": int(bool(body.causal)), "XCDS": ctx.xcds,
         "SCALE_LOG2": float_literal(body.scale * math.log2(math.e)),
@@ -590,7 +645,10 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     head += "".join(f"#define {k} {v}\n" for k, v in defs.items())
     qblocks = -(-body.q_len // BQ)
     piped = private and bool(body.sp)
-    src = (_SRC_PRIVATE.replace("@LOOP@", _pipelined_loop() if piped else _LOOP_PLAIN) if private else _SRC).replace("@SOFTMAX@", _SOFTMAX)
+    one = private and bool(body.one_region)
+    if piped and one:
+        raise LoweringError("flash (fp32 form): the software-pipelined order keeps a K and a V block at once")
+    src = (_SRC_PRIVATE.replace("@LOOP@", _pipelined_loop() if piped else (_LOOP_ONE if one else _LOOP_PLAIN)) if private else _SRC).replace("@SOFTMAX@", _SOFTMAX)
     return HipOp(
         kernel_source=(prelude.header(prelude.DMA) if private else prelude.header()) + head + src,
         kernel_name=name,
@@ -602,7 +660,7 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         comment=f"flash fp32 Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} split={kvs}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
-        knobs={"FLASH": (f"f32/s{kvs}" + ("/sp" if piped else "")) if private else f"f32/w{waves}"},
+        knobs={"FLASH": (f"f32/s{kvs}" + ("/sp" if piped else "") + ("/o" if one else "")) if private else f"f32/w{waves}"},
     )
 
 
@@ -623,17 +681,20 @@ def whole_chunk_rows(body: Flash) -> tuple[bool, bool]:
             whole and ok("o_strides", body.o_offset, body.q_heads))  # fmt: skip
 
 
-def private_lds_bytes(head_dim: int, kvs: int) -> int:
+def private_lds_bytes(head_dim: int, kvs: int, one_region: bool = False) -> int:
     dp = padded_head_dim(head_dim)
-    return kvs * 32 * (dp + (1 << (dp - 1).bit_length())) * 4
+    dpl = 1 << (dp - 1).bit_length()
+    if one_region:  # (the partials of the close are a little wider than a block)
+        return kvs * (32 * (dpl + 4) + 64) * 4
+    return kvs * 32 * (dp + dpl) * 4
 
 
-def max_key_split(head_dim: int, lds_limit: int) -> int:
+def max_key_split(head_dim: int, lds_limit: int, one_region: bool = False) -> int:
     """Most key-split waves (8, 4, 2, or 1 = none) whose private K / V regions fit the LDS; none beyond 128 columns, where
     a wave's query and output registers leave no room for the form's fragments."""
     if padded_head_dim(head_dim) > 128:
         return 1
-    return next((k for k in (8, 4, 2) if private_lds_bytes(head_dim, k) <= lds_limit), 1)
+    return next((k for k in (8, 4, 2) if private_lds_bytes(head_dim, k, one_region) <= lds_limit), 1)
 
 
 __all__ = ["emit_flash_f32", "f32_supported", "on_f32_atoms", "lds_bytes", "padded_head_dim", "whole_chunk_rows", "max_key_split", "MAX_HEAD_DIM"]

@@ -282,6 +282,7 @@ class Flash:
     mfma_sum: bool = False  # the row sums come out of the matrix pipe (an all-ones operand against the P fragments) instead of one add per probability
     ws: bool = False  # wave-specialised form: four consumer waves (waves x kv_split = 4) and four staging waves
     sp: bool = False  # software-pipelined form without staging waves: eight consumer waves (waves x kv_split = 8) stage for themselves
+    one_region: bool = False  # fp32 key-split form: a wave's K and V blocks take turns in one LDS region (half the LDS a wave, two waves a SIMD)
     private: bool = False  # short sequences: one row group whose kv_split waves each stage and stream their own key blocks (no barrier in the loop)
     # cross-workgroup split of the keys (``REDUCE=g<n>k``): ``kv_ctas`` workgroups per query block each take a contiguous
     # slice of the keys and leave their (m, l, O) in a workspace; a combine kernel merges the slices.  ``partials`` names

@@ -678,41 +678,48 @@ def _schedule_flash_f32(body: Flash, ctx: Context) -> dict:
 
     ``w<n>``: 1, 2 or 4 groups of 32 query rows per 256-thread workgroup share each K / V block (the other waves only stage).
     ``s<k>``: one group of 32 rows per workgroup whose 2, 4 or 8 waves split the key blocks and stage for themselves.
-    Default: the key-split form wherever rows are whole aligned 16-byte chunks of at most 128 values — four waves, two
-    from four workgroups per CU on (measured, 16 / 8 heads of 128, causal, us, ``w4`` / ``s2`` / ``s4``: S=128 25.7 / 15.6 /
-    10.9, 512: 86.5 / 47.4 / 27.3, 1024: 166 / 90.9 / 58.9, 2048: 325 / 196 / 209, 4096: 761 / 766 / 800) — except for a
-    single key block, where there is nothing to split (S=32: 7.4 against 9.9); else the most row groups that still give
-    every CU a workgroup."""
+    ``s<k>/o``: the same with a wave's K and V blocks taking turns in one LDS region — half the LDS a wave, two waves a SIMD.
+    ``s<k>/sp``: the software-pipelined order (a tie, kept as a pin).
+    Default: the one-region key-split form wherever rows are whole aligned pairs of 16-byte chunks of at most 128 values —
+    eight waves where a row group has eight key blocks and more and the launch is under four workgroups per CU, else four
+    (measured, 16 / 8 heads of 128, causal, us, ``w4`` / ``s2`` / ``s4`` / ``s4/o`` / ``s8/o``: S=128 25.1 / 15.1 / 11.2 /
+    10.6 / 12.1, 512: 82.5 / 44.2 / 26.4 / 24.9 / 24.7, 1024: 159 / 84.7 / 56.3 / 74.8 / 52.8, 2048: 313 / 180 / 193 / 179 /
+    182, 4096: 713 / 699 / 711 / 621 / 664, 8192: 2625 / 2562 / 2641 / 2255 / 2351) — except for a single key block,
+    where there is nothing to split (S=32: 7.4 against 9.9); else the most row groups that still give every CU a
+    workgroup."""
     from deplodock_amd.emit.flash_f32 import max_key_split, whole_chunk_rows
 
     body.pair = body.deep = body.ws = body.sp = body.mfma_sum = False
     body.kv_ctas, body.block_kv = 1, 32
     heads = body.batch * body.q_heads
     can_split = body.dtype.name == "f32" and all(whole_chunk_rows(body)) and body.head_dim % 8 == 0
-    most = min(4, max_key_split(body.head_dim, ctx.lds_bytes_per_cu)) if can_split else 1
+    most = max_key_split(body.head_dim, ctx.lds_bytes_per_cu, one_region=True) if can_split else 1
     symbolic = getattr(body, "sym", None) is not None and bool(body.sym.fields)
+    body.one_region = False
     if most > 1 and (body.kv_len > 32 or symbolic):
-        body.waves, body.kv_split = 1, (2 if heads * -(-body.q_len // 32) >= 4 * ctx.compute_units else most)
+        wide = most >= 8 and (symbolic or body.kv_len >= 8 * 32) and heads * -(-body.q_len // 32) < 4 * ctx.compute_units
+        body.waves, body.kv_split, body.one_region = 1, (8 if wide else min(4, most)), True
     else:
         body.waves, body.kv_split = next((w for w in (4, 2) if heads * -(-body.q_len // (32 * w)) >= ctx.compute_units), 1), 1
     pinned = _pin("FLASH", _tuned(body, ctx))
-    body.sp = body.kv_split > 1 and _F32_PIPELINED
+    body.sp = body.kv_split > 1 and _F32_PIPELINED and not body.one_region
     if pinned and pinned.split("/")[0] == "f32":
         try:
             tok, *rest = pinned.split("/")[1:]
             n = int(tok[1:])
-            if rest not in ([], ["sp"], ["np"]):
+            if rest not in ([], ["sp"], ["np"], ["o"]):
                 raise ValueError(rest)
             if tok[0] == "w" and n in (1, 2, 4) and not rest:
-                body.waves, body.kv_split, body.sp = n, 1, False
-            elif tok[0] == "s" and n in (2, 4, 8) and can_split and n <= max_key_split(body.head_dim, ctx.lds_bytes_per_cu):
+                body.waves, body.kv_split, body.sp, body.one_region = n, 1, False, False
+            elif tok[0] == "s" and n in (2, 4, 8) and can_split and n <= max_key_split(body.head_dim, ctx.lds_bytes_per_cu, rest == ["o"]):
                 body.waves, body.kv_split = 1, n
                 body.sp = rest == ["sp"] or (not rest and _F32_PIPELINED)
+                body.one_region = rest == ["o"]
             else:
                 raise ValueError(tok)
         except ValueError:
-            logger.warning("EMMY_FLASH=%r ignored: expect f32/w1, f32/w2, f32/w4 or f32/s2, f32/s4, f32/s8 (rows of whole 16-byte chunks, regions within the LDS)", pinned)
-    return {"FLASH": (f"f32/s{body.kv_split}" + ("/sp" if body.sp else "")) if body.kv_split > 1 else f"f32/w{body.waves}"}
+            logger.warning("EMMY_FLASH=%r ignored: expect f32/w1, f32/w2, f32/w4 or f32/s2, f32/s4, f32/s8[/sp|/o] (rows of whole 16-byte chunks, regions within the LDS)", pinned)
+    return {"FLASH": (f"f32/s{body.kv_split}" + ("/sp" if body.sp else "") + ("/o" if body.one_region else "")) if body.kv_split > 1 else f"f32/w{body.waves}"}
 
 
 def _schedule_flash_split(body: Flash, ctx: Context, tuned: dict | None) -> dict:

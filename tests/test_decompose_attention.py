@@ -133,7 +133,7 @@ def test_a_scores_tensor_beyond_the_limit_is_refused_with_a_message():
         HipBackend().compile(trace_module(_Sdpa(is_causal=True).eval(), (q, q, q)))
 
 
-@pytest.mark.parametrize("head_dim, form", [(3, "w1"), (21, "w4"), (40, "s4"), (64, "s8"), (128, "s4"), (128, "s2"), (128, "w4"), (200, "w2"), (256, "w1")])
+@pytest.mark.parametrize("head_dim, form", [(3, "w1"), (21, "w4"), (40, "s4"), (64, "s8"), (128, "s4"), (128, "s2"), (128, "s8/o"), (128, "s4/o"), (64, "s2/o"), (128, "s4/sp"), (128, "w4"), (200, "w2"), (256, "w1")])
 def test_fp32_streaming_attention_builds_without_spills(head_dim, form, monkeypatch):
     """Every head_dim up to 256 and both forms of the fp32 streaming kernel build within a wave's registers (the
     key-split form counts its outstanding direct-to-LDS requests, which spill traffic would disturb); the key-split
@@ -146,7 +146,7 @@ def test_fp32_streaming_attention_builds_without_spills(head_dim, form, monkeypa
     compiled = HipBackend().compile(trace_module(_Sdpa(enable_gqa=True).eval(), (q, k, k, torch.randn(70, 90))))
     (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
     assert op.knobs["FLASH"] == f"f32/{form}" and "mfma_f32_32x32x2f32" in op.kernel_source
-    assert op.block[0] == ((64 * int(form[1:]),) if form[0] == "s" else (256,))
+    assert op.block[0] == ((64 * int(form.split("/")[0][1:]),) if form[0] == "s" else (256,))
     try:
         assert hiprtc.spilled_vgprs(op.kernel_source, op.kernel_name) == 0
     except launcher.CompileError:
@@ -164,8 +164,9 @@ def test_fp32_streaming_attention_default_forms(monkeypatch):
         return op.knobs["FLASH"]
 
     assert form((1, 16, 32, 128), (1, 8, 32, 128)) == "f32/w1"  # one key block: nothing to split
-    assert form((1, 16, 512, 128), (1, 8, 512, 128)) == "f32/s4"
-    assert form((1, 16, 2048, 128), (1, 8, 2048, 128)) == "f32/s2"  # four workgroups per CU and more
+    assert form((1, 16, 128, 128), (1, 8, 128, 128)) == "f32/s4/o"  # four key blocks: four waves
+    assert form((1, 16, 512, 128), (1, 8, 512, 128)) == "f32/s8/o"
+    assert form((1, 16, 2048, 128), (1, 8, 2048, 128)) == "f32/s4/o"  # four workgroups per CU and more
     assert form((1, 2, 40, 21), (1, 2, 40, 21)) == "f32/w1"  # rows that are not whole 16-byte chunks
     assert form((1, 2, 40, 256), (1, 2, 40, 256)) == "f32/w1"  # beyond 128 columns
     # a pin the shape cannot take is ignored

@@ -1487,7 +1487,7 @@ def test_fp32_attention_streams_on_fp32_atoms(device, case):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("form", ["w1", "w2", "w4", "s2", "s4", "s8", "s2/sp", "s4/sp", "s8/sp"])
+@pytest.mark.parametrize("form", ["w1", "w2", "w4", "s2", "s4", "s8", "s2/sp", "s4/sp", "s8/sp", "s2/o", "s4/o", "s8/o"])
 def test_fp32_attention_forms(device, form, monkeypatch):
     """``EMMY_FLASH=f32/w<n>``: 1, 2 or 4 of a workgroup's four waves own query rows and share the staged K / V blocks;
     ``f32/s<k>``: the k waves of a workgroup split the key blocks of one row group and stage for themselves.  Here with a
