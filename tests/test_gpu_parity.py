@@ -1514,14 +1514,26 @@ def test_fp32_attention_forms(device, form, monkeypatch):
 
 
 @pytest.mark.gpu
-def test_fp32_attention_with_a_runtime_sequence_length(device):
-    """One compilation of fp32 causal attention with the sequence length as the kernel's trailing ``int``, bound at
-    several lengths (ragged blocks, one key block, more blocks than waves), against eager in float64."""
-    mod = _FusedAttention(is_causal=True, enable_gqa=True)
+@pytest.mark.parametrize("masked", [False, True])
+def test_fp32_attention_with_a_runtime_sequence_length(device, masked):
+    """One compilation of fp32 attention (causal, or with a ``[1, 1, S, S]`` additive mask whose row stride follows the
+    length) with the sequence length as the kernel's trailing ``int``, bound at several lengths (ragged blocks, one key
+    block, more blocks than waves), against eager in float64."""
+    mod = _FusedAttention(enable_gqa=True) if masked else _FusedAttention(is_causal=True, enable_gqa=True)
     torch.manual_seed(47)
-    mk = lambda s: [torch.randn(1, 4, s, 128), torch.randn(1, 2, s, 128), torch.randn(1, 2, s, 128)]  # noqa: E731
+
+    def mk(s):
+        qkv = [torch.randn(1, 4, s, 128), torch.randn(1, 2, s, 128), torch.randn(1, 2, s, 128)]
+        if masked:
+            m = torch.randn(1, 1, s, s)
+            m[torch.rand(1, 1, s, s) < 0.3] = -float("inf")
+            m[..., 0] = 0.5
+            qkv.append(m)
+        return qkv
+
+    dyn = {"q": {2: "s"}, "k": {2: "s"}, "v": {2: "s"}, **({"mask": {2: "s", 3: "s"}} if masked else {})}
     be = HipBackend()
-    compiled = be.compile(trace_module(mod.eval(), tuple(mk(64)), dynamic_shapes={"q": {2: "s"}, "k": {2: "s"}, "v": {2: "s"}}))
+    compiled = be.compile(trace_module(mod.eval(), tuple(mk(64)), dynamic_shapes=dyn))
     (op,) = [n.op for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
     assert op.runtime_args and op.knobs["FLASH"].startswith("f32/s")
     for s in (64, 1, 31, 200, 513):
@@ -1534,7 +1546,7 @@ def test_fp32_attention_with_a_runtime_sequence_length(device):
         finally:
             prog.close()
         want = mod(*(t.double() for t in args)).float()
-        eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-5, f"fp32 attention, runtime length {s}")
+        eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-5, f"fp32 attention, runtime length {s}, masked={masked}")
 
 
 _NARROW_ON_FP32_ATOMS = {
