@@ -16,10 +16,15 @@ never reach device memory, and lays it out the way the 16-bit kernel is:
   columns walk the block's keys in that order, and the V operand is read from LDS in the same order.
 * The contraction over ``d`` in the scores is order-free as well: a lane reads 16 bytes of its key's row per four atoms
   (``d = 8 u + 4 h + 0..3``) and holds its query's values in the same order.
-* 256 threads per workgroup: ``waves`` of them (1, 2 or 4) own 32 query rows each, all of them stage the 32-key K / V
-  blocks (global -> registers -> LDS, two buffers, one barrier a step; up to 128 columns the loads are issued a step
-  ahead of the arithmetic).  K rows are padded by 4 floats and V
-  rows by 8, which makes the 16-byte K reads and the 4-byte V reads of a wave conflict-free.
+* Two forms.  *Key-split* (``kv_split`` = 2, 4 or 8; rows of whole aligned pairs of 16-byte chunks, up to 128 columns):
+  a workgroup is one group of 32 query rows whose waves each take every k-th 32-key block and stage it themselves with
+  direct-to-LDS loads — no barrier in the loop, one merge of the waves' ``(m, l, O)`` through LDS at the close.  By
+  default a wave's K block and V block take turns in one LDS region (``one_region``: they are never needed at the same
+  time), which halves a wave's LDS so that a SIMD holds two waves and one's atoms fill the other's waits.  *Shared*
+  (everything else): 256 threads per workgroup, ``waves`` of them (1, 2 or 4) own 32 query rows each, all of them stage
+  the 32-key K / V blocks (global -> registers -> LDS, two buffers, one barrier a step; up to 128 columns the loads are
+  issued a step ahead of the arithmetic); K rows are padded by 4 floats and V rows by 8, which makes the 16-byte K
+  reads and the 4-byte V reads of a wave conflict-free.
 * Rows of any length up to 256 values: the tiles are ``DP`` = the next multiple of 32 wide, columns past the row's end are
   staged as zeros and not stored; rows that are not whole aligned 16-byte chunks are read value by value.
 """
