@@ -371,7 +371,7 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
                 if t <= 0 or not op.algo_bytes:
                     continue
                 tf, gb = op.algo_flops / t / 1e12, op.algo_bytes / t / 1e9
-                f_mfma, f_hbm = tf / MFMA_BF16_PEAK_TFLOPS, gb / HBM_PEAK_GBPS
+                f_mfma, f_hbm = tf / (MFMA_FP32_PEAK_TFLOPS if bound == "mfma_f32" else MFMA_BF16_PEAK_TFLOPS), gb / HBM_PEAK_GBPS
                 per.append({"kernel": f"{i}:{p.kernel_name}", "us": round(t * 1e6, 2), "bound": "mfma" if f_mfma >= f_hbm else "hbm", "tflops": round(tf, 1), "gbps": round(gb, 1),
                             "frac_mfma": round(f_mfma, 4), "frac_hbm": round(f_hbm, 4), "frac": round(max(f_mfma, f_hbm), 4)})  # fmt: skip
             row["per_kernel"] = per
@@ -423,6 +423,8 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
     # the same block compiled once for every sequence length (kernels that take the length as a run-time int), run at 512
     bench(lambda: wl.qwen3_block_case(seq=512), "C5s qwen3-0.6B block bf16, runtime-int kernels over seq_len, at S=512", "mfma",
           dynamic={"x": {1: "seq_len"}, "cos": {1: "seq_len"}, "sin": {1: "seq_len"}})  # fmt: skip
+    # the reference's own precision: the same block with fp32 parameters and activations (fp32 MFMA atoms throughout)
+    bench(lambda: wl.qwen3_block_case(seq=512, dtype=torch.float32), "C5f qwen3-0.6B block fp32 S=512", "mfma_f32", vendor=True)
     bench(lambda: wl.qwen3_model_case(seq=512), "M qwen3-0.6B whole model (28 layers, random weights) bf16 S=512, token ids -> last hidden state", "mfma", whole_model=True)
     return rows
 
