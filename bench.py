@@ -416,6 +416,7 @@ def _table(device, only: str | None = None, extended: bool = False, cpu: bool = 
     # the reference's own precision: the same shape in fp32 (its sdpa perf cases run S = 32 / 128 / 512), on fp32 MFMA atoms
     bench(lambda: wl.sdpa_case(s=512, fp32=True), "C4f causal GQA sdpa fp32 16q/8kv S=512 d=128", "mfma_f32", vendor=True)
     bench(lambda: wl.sdpa_case(fp32=True), "C4f causal GQA sdpa fp32 16q/8kv S=2048 d=128", "mfma_f32", vendor=True)
+    bench(lambda: wl.sdpa_decode_case(q_len=1, kv_len=32768, fp32=True), "C4df decode GQA sdpa fp32 16q/8kv q=1 kv=32768 d=128 (key slices + combine)", "hbm", vendor=True)
     if extended:
         bench(lambda: wl.sdpa_case(causal=False), "C4x non-causal GQA sdpa bf16 16q/8kv S=2048 d=128", "mfma")
         bench(lambda: wl.sdpa_case(s=8192), "C4xx causal GQA sdpa bf16 16q/8kv S=8192 d=128", "mfma", vendor=True)

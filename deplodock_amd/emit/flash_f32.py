@@ -279,8 +279,18 @@ extern "C" __global__ __launch_bounds__(NT) EMH_OCCUPANCY void KNAME(const float
   const int qrow = q0 + n;
   const int qrow_c = qrow < SQ ? qrow : SQ - 1;
 
-  const float* kbase = Kp + K_OFF + (long)batch * K_SB + (long)kvh * K_SH;
-  const float* vbase = Vp + V_OFF + (long)batch * V_SB + (long)kvh * V_SH;
+#if KV_CTAS > 1
+  // Key split across workgroups: slice blockIdx.y of the keys, [kv0, kv0 + SKV), is this workgroup's whole key range (no
+  // mask of either kind in this form, so key indices below are simply relative to the slice); the close leaves the
+  // slice's unnormalised output rows, maximum and sum in the workspace for the combine kernel.
+  const int kv0 = (int)blockIdx.y * KV_CHUNK;
+  const int skv_slice = SKV_ALL - kv0 < KV_CHUNK ? SKV_ALL - kv0 : KV_CHUNK;
+  #define SKV skv_slice
+#else
+  const int kv0 = 0;
+#endif
+  const float* kbase = Kp + K_OFF + (long)batch * K_SB + (long)kvh * K_SH + (long)kv0 * K_SS;
+  const float* vbase = Vp + V_OFF + (long)batch * V_SB + (long)kvh * V_SH + (long)kv0 * V_SS;
 #if HAS_MASK
   const MELT* mrow = Mp + M_OFF + (long)batch * M_SB + (long)head * M_SH + (long)qrow_c * M_SS;
 #endif
@@ -383,9 +393,15 @@ extern "C" __global__ __launch_bounds__(NT) EMH_OCCUPANCY void KNAME(const float
       const f32x4 t = *(const f32x4*)(part + row * PS + c4);
       acc[0] += t[0] * w; acc[1] += t[1] * w; acc[2] += t[2] * w; acc[3] += t[3] * w;
     }
+#if KV_CTAS > 1
+    float* prow = Op + ((((long)blockIdx.y * BATCH + batch) * HQ + head) * SQ + (q0 + row)) * (D + 4);
+    *(f32x4*)(prow + c4) = acc;
+    if (c4 == 0) { prow[D] = m; prow[D + 1] = l; }
+#else
     const float inv = 1.0f / l;
     f32x4 y; y[0] = acc[0] * inv; y[1] = acc[1] * inv; y[2] = acc[2] * inv; y[3] = acc[3] * inv;
     *(f32x4*)(Op + O_OFF + (long)batch * O_SB + (long)head * O_SH + (long)(q0 + row) * O_SS + c4) = y;
+#endif
   }
 }
 """
@@ -602,8 +618,18 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
         raise LoweringError(f"flash (fp32 form): head_dim {D} outside 1..{MAX_HEAD_DIM}")
     if body.q_heads % body.kv_heads:
         raise LoweringError("flash: q heads must be a multiple of kv heads")
-    if body.kv_ctas > 1 or body.pair or body.ws or body.mfma_sum or (body.sp and body.kv_split < 2):
-        raise LoweringError("flash (fp32 form): no key split across workgroups or mirrored pairs; the software-pipelined order is the key-split form's")
+    if body.pair or body.ws or body.mfma_sum or (body.sp and body.kv_split < 2):
+        raise LoweringError("flash (fp32 form): no mirrored pairs; the software-pipelined order is the key-split form's")
+    split = int(body.kv_ctas or 1)
+    if split > 1:
+        sym_ = getattr(body, "sym", None)
+        if body.partials is None:
+            raise LoweringError("flash: a cross-workgroup key split (REDUCE=g<n>k) is lowered as a partial kernel plus a combine (passes.lower), not by this emitter alone")
+        if body.kv_split < 2 or body.causal or body.mask is not None or (sym_ is not None and sym_.fields) or body.dtype.name != "f32" or D % 4:
+            raise LoweringError("flash (fp32 form): the cross-workgroup key split is the key-split form's, without masks or symbolic lengths")
+        step_keys = body.kv_split * body.block_kv
+        kv_chunk = -(-(-(-body.kv_len // split)) // step_keys) * step_keys  # whole key steps per slice
+        split = -(-body.kv_len // kv_chunk)  # slices that hold keys
     waves, kvs = body.waves, body.kv_split
     private = kvs > 1
     if (not private and waves not in (1, 2, 4)) or (private and (waves != 1 or kvs not in (2, 4, 8))):
@@ -633,7 +659,9 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     defs = {
         "KNAME": name, "ELT": rt.type_name(body.dtype.name), "NT": NT, "WAVES": waves, "KVS": kvs, "BQ": BQ, "BKV": BLOCK_KV, "D": D, "DR": D, "DP": DP, "DPL": DPL,
         "VEC4": int(vec_in), "OVEC4": int(vec_out), "PRE": int(DP <= 128), "ONE_REGION": int(bool(body.one_region) and private),
-        "SQ": c_value(symf.get("q_len", body.q_len)), "SKV": c_value(symf.get("kv_len", body.kv_len)),
+        "SQ": c_value(symf.get("q_len", body.q_len)),
+        **({"SKV_ALL": body.kv_len, "KV_CHUNK": kv_chunk, "BATCH": body.batch} if split > 1 else {"SKV": c_value(symf.get("kv_len", body.kv_len))}),
+        "KV_CTAS": split,
         "HQ": body.q_heads, "GROUP": body.q_heads // body.kv_heads, "CAUSAL": int(bool(body.causal)), "XCDS": ctx.xcds,
         "SCALE_LOG2": float_literal(body.scale * math.log2(math.e)),
         "SYM_PARAM": f", int {param_name(sym.name)}" if symf else "",
@@ -657,15 +685,15 @@ def emit_flash_f32(body: Flash, name: str, ctx: Context = Context()) -> HipOp:
     return HipOp(
         kernel_source=(prelude.header(prelude.DMA) if private else prelude.header()) + head + src,
         kernel_name=name,
-        arg_order=(body.q, body.k, body.v, *((body.mask,) if has_mask else ()), body.out),
-        grid=((CeilDiv(symf["q_len"], BQ), body.q_heads * body.batch) if "q_len" in symf else (qblocks * body.q_heads * body.batch,), (1,), (1,)),
+        arg_order=(body.q, body.k, body.v, *((body.mask,) if has_mask else ()), body.partials if split > 1 else body.out),
+        grid=((CeilDiv(symf["q_len"], BQ), body.q_heads * body.batch) if "q_len" in symf else (qblocks * body.q_heads * body.batch,), (split,), (1,)),
         block=((NT,), (1,), (1,)),
         lds_bytes=lds,
         runtime_args=(sym.name,) if symf else (),
         comment=f"flash fp32 Sq={body.q_len} Skv={body.kv_len} D={D} causal={body.causal} waves={waves} split={kvs}",
         algo_bytes=body.algo_bytes(),
         algo_flops=body.algo_flops(),
-        knobs={"FLASH": (f"f32/s{kvs}" + ("/sp" if piped else "") + ("/o" if one else "")) if private else f"f32/w{waves}"},
+        knobs={"FLASH": (f"f32/s{kvs}" + ("/sp" if piped else "") + ("/o" if one else "")) if private else f"f32/w{waves}", **({"REDUCE": f"g{split}k"} if split > 1 else {})},
     )
 
 

@@ -719,7 +719,14 @@ def _schedule_flash_f32(body: Flash, ctx: Context) -> dict:
                 raise ValueError(tok)
         except ValueError:
             logger.warning("EMMY_FLASH=%r ignored: expect f32/w1, f32/w2, f32/w4 or f32/s2, f32/s4, f32/s8[/sp|/o] (rows of whole 16-byte chunks, regions within the LDS)", pinned)
-    return {"FLASH": (f"f32/s{body.kv_split}" + ("/sp" if body.sp else "") + ("/o" if body.one_region else "")) if body.kv_split > 1 else f"f32/w{body.waves}"}
+    flash = (f"f32/s{body.kv_split}" + ("/sp" if body.sp else "") + ("/o" if body.one_region else "")) if body.kv_split > 1 else f"f32/w{body.waves}"
+    knobs: dict = {}
+    if body.kv_split > 1 and body.dtype.name == "f32" and not body.causal and body.mask is None and not symbolic and body.head_dim % 4 == 0:
+        # decode-size queries over a long cache: the keys are also split across workgroups (partial kernel + combine)
+        knobs = _schedule_flash_split(body, ctx, tuned if (tuned := _tuned(body, ctx)) else None)
+    elif _pin("REDUCE", _tuned(body, ctx)):
+        logger.warning("EMMY_REDUCE ignored for this fp32 attention: the cross-workgroup key split takes the key-split form without masks or symbolic lengths")
+    return {**knobs, "FLASH": flash}
 
 
 def _schedule_flash_split(body: Flash, ctx: Context, tuned: dict | None) -> dict:

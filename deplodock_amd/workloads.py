@@ -93,16 +93,19 @@ def sdpa_case(b: int = 1, hq: int = 16, hkv: int = 8, s: int = 2048, d: int = 12
     )  # fmt: skip
 
 
-def sdpa_decode_case(q_len: int = 1, kv_len: int = 32768, b: int = 1, hq: int = 16, hkv: int = 8, d: int = 128, seed: int = 0) -> Case:
+def sdpa_decode_case(q_len: int = 1, kv_len: int = 32768, b: int = 1, hq: int = 16, hkv: int = 8, d: int = 128, seed: int = 0, fp32: bool = False) -> Case:
     """Decode-size attention over a long cache: ``q_len`` new queries see all ``kv_len`` keys (no mask); bound by the K/V
-    stream (the algorithmic bytes are K, V, q and the output once)."""
+    stream (the algorithmic bytes are K, V, q and the output once).  ``fp32``: the same bf16-valued operands held as fp32."""
     torch.manual_seed(seed)
     q = torch.randn(b, hq, q_len, d).bfloat16()
     k = torch.randn(b, hkv, kv_len, d).bfloat16()
     v = torch.randn(b, hkv, kv_len, d).bfloat16()
+    nb = 4 if fp32 else 2
+    if fp32:
+        q, k, v = q.float(), k.float(), v.float()
     return Case(
-        f"sdpa_decode_{b}x{hq}x{hkv}x{q_len}x{kv_len}x{d}", Sdpa(False).eval(), (q, k, v), BF16_RTOL, 2e-2,
-        algo_bytes=(2 * b * hq * q_len * d + 2 * b * hkv * kv_len * d) * 2, algo_flops=4 * b * hq * d * q_len * kv_len,
+        f"sdpa_decode_{'fp32_' if fp32 else ''}{b}x{hq}x{hkv}x{q_len}x{kv_len}x{d}", Sdpa(False).eval(), (q, k, v), 1e-4 if fp32 else BF16_RTOL, 1e-5 if fp32 else 2e-2,
+        algo_bytes=(2 * b * hq * q_len * d + 2 * b * hkv * kv_len * d) * nb, algo_flops=4 * b * hq * d * q_len * kv_len,
     )  # fmt: skip
 
 

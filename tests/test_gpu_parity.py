@@ -1549,6 +1549,55 @@ def test_fp32_attention_with_a_runtime_sequence_length(device, masked):
         eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-5, f"fp32 attention, runtime length {s}, masked={masked}")
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("q_len, kv_len", [(1, 32768), (16, 4096), (7, 5000), (40, 2100)])
+def test_fp32_decode_attention_splits_the_keys_across_workgroups(device, q_len, kv_len):
+    """Decode-size fp32 queries over a long cache (no mask): the keys are split over workgroups as well — the partial
+    kernel leaves each slice's ``(O, m, l)`` in a workspace and the combine kernel merges them (``REDUCE=g<n>k``, the
+    form the 16-bit kernel has) — ragged last slices and grouped heads included; against eager in float64."""
+    mod = _FusedAttention(enable_gqa=True)
+    torch.manual_seed(53)
+    args = [torch.randn(1, 16, q_len, 128), torch.randn(1, 8, kv_len, 128), torch.randn(1, 8, kv_len, 128)]
+    be = HipBackend()
+    compiled = be.compile(trace_module(mod.eval(), tuple(args)))
+    names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+    assert sorted(names) == ["k_sdpa_reduce_combine", "k_sdpa_reduce_partial"], names
+    prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in args))))
+    try:
+        for _ in range(2):
+            prog.run()
+            torch.cuda.synchronize()
+        ours = prog.output_tensors()[compiled.outputs[0]].clone()
+    finally:
+        prog.close()
+    want = mod(*(t.double() for t in args)).float()
+    eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-5, f"fp32 decode attention q={q_len} kv={kv_len}")
+
+
+@pytest.mark.gpu
+def test_fp32_attention_key_split_across_workgroups_by_pin(device, monkeypatch):
+    """``EMMY_REDUCE=g4k`` on a non-causal fp32 attention that would not split by itself, with a batch and a ragged length;
+    a causal one ignores the pin."""
+    monkeypatch.setenv("EMMY_REDUCE", "g4k")
+    torch.manual_seed(54)
+    for causal in (False, True):
+        mod = _FusedAttention(is_causal=causal, enable_gqa=True)
+        args = [torch.randn(2, 4, 100, 64), torch.randn(2, 2, 1100, 64), torch.randn(2, 2, 1100, 64)]
+        be = HipBackend()
+        compiled = be.compile(trace_module(mod.eval(), tuple(args)))
+        names = [n.op.kernel_name.rsplit("_", 1)[0] for n in compiled.nodes.values() if isinstance(n.op, HipOp)]
+        assert (sorted(names) == ["k_sdpa_reduce_combine", "k_sdpa_reduce_partial"]) == (not causal), names
+        prog = be.program(compiled, dict(zip(compiled.inputs, (t.to(device) for t in args))))
+        try:
+            prog.run()
+            torch.cuda.synchronize()
+            ours = prog.output_tensors()[compiled.outputs[0]].clone()
+        finally:
+            prog.close()
+        want = mod(*(t.double() for t in args)).float()
+        eager.assert_close(ours.reshape(want.shape), want, 1e-4, 1e-5, f"fp32 attention g4k causal={causal}")
+
+
 _NARROW_ON_FP32_ATOMS = {
     # 16-bit rows that are not whole 16-byte chunks (the 16-bit flash kernel pads whole chunks only)
     "bf16_head_dim_36": (_FusedAttention(is_causal=True), torch.bfloat16, [(2, 4, 64, 36)] * 3, None),
