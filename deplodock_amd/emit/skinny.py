@@ -70,8 +70,10 @@ def skinny_waves(body: Contraction) -> int:
         return 0  # the few-row form holds every row in a fixed number of MFMA tiles: not with a row count known only at launch
     if body.in_dtype.name not in ("bf16", "f16") or body.k % 32 or body.n % 4:
         return 0
+    # at least 256 values of the reduction axis a wave (eight MFMA steps): in the decoder block at 1-32 rows, K = 1024
+    # takes 2.74-2.96 us on two or four waves against 2.89-3.12 on eight; K = 3072 is 3.72 on eight, 4.39 on four
     for kw in (8, 4, 2, 1):
-        if body.k % (32 * kw) == 0:
+        if body.k % (32 * kw) == 0 and (body.k // kw >= 256 or kw == 1):
             return kw
     return 0
 
@@ -86,6 +88,10 @@ def skinny_cols(body: Contraction, ctx: Context = Context()) -> int:
         rounds = -(-(-(-body.n // c)) // ctx.compute_units)
         return rounds * (x_bytes + c * body.k * body.in_dtype.nbytes * nb)
 
+    if -(-body.n // 16) >= 0.75 * ctx.compute_units:
+        # whole 16-wide MFMA tiles already cover the machine: fewer, fuller workgroups ask the L2s for the rows less often
+        # (gate / up pair, N = 3072, 8-32 rows: 3.93 / 3.98 / 4.65 us on 192 workgroups of 16 against 4.21 / 4.24 / 5.13 on 256 of 12)
+        return 16
     return min((c for c in (16, 12, 8, 4) if body.n % c == 0 or c == 16), key=lambda c: (per_cu(c), -c))
 
 

@@ -1095,7 +1095,9 @@ def _logical_strides(p: _RopePlan, mem_strides: tuple[int, ...]) -> tuple[int, .
 
 
 #: tokens up to which the q / k head norm + rotary embedding stays a launch of its own behind the few-row projection
-_ROW_EPILOGUE_MIN_TOKENS = 16
+#: (the decoder block as one graph, two launches against the fused one: 24 tokens 25.3 / 26.0 us, 32 tokens 26.1 / 26.7;
+#: 64 tokens 30.0 / 28.8)
+_ROW_EPILOGUE_MIN_TOKENS = 32
 
 
 def _rec_rope_pair(c: _Ctx, nid: str) -> bool:

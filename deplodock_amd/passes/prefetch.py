@@ -52,8 +52,8 @@ LAST_LEVEL_CACHE_BYTES = 256 * 1024 * 1024
 #: flop per byte of the consumer (about its row count, for a weight-streaming contraction) between which a prefetch pays
 MIN_INTENSITY = 24.0
 MAX_INTENSITY = 200.0
-#: LDS up to which extra workgroups run beside the kernel's own on a CU
-_SMALL_LDS = 48 * 1024
+#: LDS up to which extra workgroups run beside the kernel's own on a CU (two of them fit a CU's 160 KiB)
+_SMALL_LDS = 76 * 1024
 LINE = 128
 
 

@@ -194,11 +194,14 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
     best = None
     candidates = TILE_CANDIDATES
     one_round_only = {(128, 256)}  # offered only as an exact fit: as a 75 % cover it was not measured
-    if m >= 128:
-        # From 128 rows on: eight waves of one fragment each on the 32x64 tile (more
+    if m > 64:
+        # Beyond 64 rows: eight waves of one fragment each on the 32x64 tile (more
         # loads in flight per CU than four waves of two): 6.20 vs 6.39 us on
-        # 512x1024x2048, 7.94 vs 9.16 us on 512x1024x3072, inside the decoder block.
-        candidates = tuple((32, 64, 2, 4, "mfma_16x16x32_bf16", 8) if c[:4] == (32, 64, 1, 4) else c for c in candidates)
+        # 512x1024x2048, 7.94 vs 9.16 us on 512x1024x3072, inside the decoder block; the
+        # gate / up pair at 80 / 96 / 112 rows 6.53 / 6.60 / 6.58 against 7.75 / 7.61 / 7.69.
+        # (below 128 rows the four-wave form stays behind it, for the shapes the eight-wave one does not divide)
+        eight = (32, 64, 2, 4, "mfma_16x16x32_bf16", 8)
+        candidates = tuple(x for c in candidates for x in ((eight,) if c[:4] == (32, 64, 1, 4) and m >= 128 else (eight, c) if c[:4] == (32, 64, 1, 4) else (c,)))
     if gate_pair:
         # two weight rows per output column: 96-column tiles make 32 column blocks of 2 x 3072 outputs
         extra = ((128, 96, 4, 2, "mfma_16x16x32_bf16", 2), (64, 96, 4, 2, "mfma_16x16x32_bf16", 2), (32, 96, 2, 2, "mfma_16x16x32_bf16", 4))
@@ -241,18 +244,27 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
         groups = -(-m // tm) * -(-n // tn) * copies
         if wm * wn > 1 and m % tm == 0 and n % tn == 0 and 0.9 * cus <= groups <= cus:
             return plan  # (the one-wave tile is the last resort: two waves on half as many 16x32 tiles beat it)
+    half_round = None  # the first (largest) tile that covers at least half the CUs
     for (tm, tn, *_), plan in plans:
         if (tm, tn) in one_round_only:
             continue
         groups = -(-m // tm) * -(-n // tn) * copies
         # penalise tiles that mostly hang over the edge of a small problem
         waste = (-(-m // tm) * tm * -(-n // tn) * tn) / float(max(m * n, 1))
-        # two waves on a 16x32 tile beat one wave on each of twice as many 16x16 tiles down to half the CUs
-        # (64 rows x 1024 columns: 4.11 / 5.01 us on 128 workgroups against 4.84 / 6.43 us on 256)
-        fill = 0.5 if (tm, tn) == (16, 32) else _FILL_FRACTION
+        if half_round is None and 0.5 * cus <= groups <= cus and waste < 1.5:
+            half_round = plan
+        if half_round is not None and cus < groups < 1.5 * cus and waste < 1.5:
+            # a second round of workgroups for a few stragglers: the tile twice the size does the same work in one round
+            # (96 rows, gate / up pair of 3072 columns: 288 workgroups of 32x32 11.07 us, 144 of 32x64 6.60)
+            return half_round
+        # two waves on a 16x32 tile beat one wave on each of twice as many 16x16 tiles down to a quarter of the CUs
+        # (64 rows x 1024 columns: 4.11 / 5.01 us on 128 workgroups against 4.84 / 6.43 us on 256; 32 rows x 1024
+        # columns, K = 3072: 4.70 us on 64 workgroups against 7.04 us on 128)
+        fill = 0.25 if (tm, tn) == (16, 32) else _FILL_FRACTION
         if groups >= fill * cus and waste < 1.5:
             return plan
-        score = (min(groups, cus) / max(waste, 1e-9), tm * tn)
+        one_wave = (tm, tn) == (16, 16)  # a lone wave walks the whole reduction axis: worth half a multi-wave workgroup
+        score = (min(groups, cus) * (0.5 if one_wave else 1.0) / max(waste, 1e-9), tm * tn)
         if best is None or score > best[0]:
             best = (score, plan)
     if best is None:
@@ -329,8 +341,8 @@ def pingpong_fits(plan: TilePlan, body: Contraction, ctx: Context, depth: int = 
 #: ``skinny.MAX_ROWS`` rows when pinned).  Every workgroup reads all the rows, so they bound what a CU moves whatever the
 #: column count: measured inside the decoder block (us, few-row form against the tiled ring), 16 rows: o_proj (K = 2048)
 #: 3.5 / 3.9, down_proj (K = 3072) 4.5 / 5.0; 32 rows: gate / up (K = 1024, 64 KiB of rows) 5.3 / 6.0, o_proj (128 KiB)
-#: 6.3 / 4.4, down_proj (192 KiB) 8.5 / 7.4.
-_FEW_ROWS = 32
+#: 6.3 / 4.4, down_proj (192 KiB) 8.5 / 7.4; 48 rows: gate / up (96 KiB) 5.45 / 6.18; 64 rows: gate / up 7.7 / 6.0.
+_FEW_ROWS = 48
 _FEW_ROWS_BYTES = 96 * 1024
 
 
@@ -355,7 +367,8 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
       9.4; 512x1024x2048 7.4 -> 6.2 -> 6.2; 512x4096x1024 7.8 -> 6.8 -> 6.7; 2048x3072x1024
       17.2 -> 15.9 -> 16.1; 4096^3 136 -> 122; the block as one graph 66.9 -> 65.2 -> 62.8)."""
     steps = -(-body.k // plan.bk_elems)
-    if skinny_waves(body) and body.m <= _FEW_ROWS and body.m * body.k * body.in_dtype.nbytes <= _FEW_ROWS_BYTES:
+    if skinny_waves(body) and body.m <= _FEW_ROWS and body.m * body.k * body.in_dtype.nbytes <= _FEW_ROWS_BYTES and (body.m <= 16 or body.k <= 1024):
+        # (17-24 rows of K = 2048 fit the byte bound too, but two waves on 16x32 tiles are ahead there: 4.08 against 4.31 us)
         return Stage(depth=skinny_waves(body), transport="ks", cols=skinny_cols(body, ctx) % 16)
     if body.k % plan.bk_elems:
         return Stage(depth=2, transport="sync")  # the short last slab is zero-filled in registers
@@ -641,8 +654,8 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
             # (two row groups pay down to half the CUs: 512 tokens x 16 heads, 128 workgroups of `w2` 8.81 us, 256 of `w1` 9.10)
             body.waves = next((w for w in (4, 2) if heads * blocks(w) >= (fill if w == 4 else 0.5 * ctx.compute_units)), 1)
         body.block_kv, body.kv_split = {8: (64, 1), 4: (64, 2)}.get(body.waves, (32, 4))
-        while body.kv_split > 1 and -(-body.kv_len // body.block_kv) < body.kv_split:
-            body.kv_split //= 2  # fewer key blocks than key-split groups
+        while body.kv_split > 1 and -(-body.kv_len // body.block_kv) <= body.kv_split // 2:
+            body.kv_split //= 2  # half the key-split groups would have no block (three blocks keep four groups: 96 keys 4.71 us, two groups 6.05)
         # wider heads: shrink the key block, then the key split, until the double-buffered K/V blocks fit the LDS
         while _flash_lds(body, ctx) > ctx.lds_bytes_per_cu:
             if body.block_kv > 32:

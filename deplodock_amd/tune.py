@@ -64,7 +64,8 @@ TILE_SWEEP_F32: tuple[str, ...] = tuple(
 )  # (the 32x32x2 atoms never ranked first at these sizes: kept so that a sweep says so)
 STAGE_SWEEP_F32: tuple[str, ...] = ("d3/dl", "d2/dl")
 STAGE_SWEEP: tuple[str, ...] = ("d2/dl", "d3/dl", "d2/sync/p2")
-FEW_ROW_SWEEP: tuple[str, ...] = ("d8/ks", "d4/ks")  # the k-split few-row form has no tile: one candidate each
+# the k-split few-row form has no tile: waves that split the reduction axis x output columns a workgroup (16 unless named)
+FEW_ROW_SWEEP: tuple[str, ...] = ("d8/ks", "d4/ks", "d2/ks", "d8/ks/c12", "d4/ks/c12", "d8/ks/c8", "d4/ks/c8", "d2/ks/c8", "d8/ks/c4", "d4/ks/c4")
 REDUCE_SWEEP: tuple[str, ...] = ("b8", "b16", "b32", "b64", "b128", "b256", "b512", "b1024")
 NT_SWEEP: tuple[str, ...] = ("0", "1")
 FLASH_SWEEP: tuple[str, ...] = (

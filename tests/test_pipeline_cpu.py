@@ -62,13 +62,13 @@ def test_linear_is_one_mfma_kernel(launcher_lib, m):
     assert k.kernel_name.startswith("k_linear_")
     assert "__builtin_amdgcn_mfma_f32_" in k.kernel_source
     assert k.algo_flops == 2 * m * 3072 * 1024
-    # decode sizes are one pass over the weight: the reduction axis split over the eight waves of a workgroup,
+    # decode sizes are one pass over the weight: the reduction axis split over the four waves of a workgroup (256 values each),
     # every fragment requested at once, no slab loop (a shape that does not fit that form goes through two
     # register sets); from 128 rows on direct-to-LDS loads (three 48 KiB slabs
     # of the 32x64x256 tile); at 2048 rows the 128x192 tile's eight waves alternate in two groups behind four
     # staging waves (twelve waves, a ring of four 40 KiB slabs)
-    assert k.knobs["STAGE"] == {1: "d8/ks/c12", 16: "d8/ks/c12", 128: "d3/dl", 2048: "d4/pp"}[m]
-    assert ("wave * 128 + lk * 8" in k.kernel_source) == (m < 128) and ("#define EMH_DLOAD" in k.kernel_source) == (m >= 128)
+    assert k.knobs["STAGE"] == {1: "d4/ks", 16: "d4/ks", 128: "d3/dl", 2048: "d4/pp"}[m]
+    assert ("wave * 256 + lk * 8" in k.kernel_source) == (m < 128) and ("#define EMH_DLOAD" in k.kernel_source) == (m >= 128)
     if m == 2048:
         assert k.block[0] == (768,) and k.lds_bytes == 4 * (128 + 192) * 64 * 2 and "role == 2" in k.kernel_source
     if m == 16:
@@ -152,7 +152,7 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
         few = kernels(compile_case(eager.qwen3_block_case(seq=seq)))
         assert [re.sub(r"_[0-9a-f]{6}$", "", k.kernel_name) for k in few] == ["k_rms_norm_linear", "k_rms_norm_rope", "k_sdpa_reduce", "k_linear_add", "k_rms_norm_linear_silu_mul", "k_linear_add"]
         decode, rope = few[0], few[1]
-        assert decode.knobs["STAGE"] == "d8/ks" and "ss[t] += emh_xor16(ss[t])" in decode.kernel_source and "* rs_)" in decode.kernel_source
+        assert decode.knobs["STAGE"] == "d4/ks" and "ss[t] += emh_xor16(ss[t])" in decode.kernel_source and "* rs_)" in decode.kernel_source
         assert decode.arg_order[1].endswith("__k*p_l_input_layernorm_weight") and rope.arg_order[0] == decode.arg_order[-1]
         for k in few[:2]:
             hiprtc.compile_to_hsaco(k.kernel_source, k.kernel_name)

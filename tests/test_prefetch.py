@@ -30,9 +30,10 @@ def test_only_programs_beyond_the_last_level_cache_prefetch_by_default(launcher_
     forced = kernels(HipBackend().compile(trace_module(case.module, case.inputs)))
     assert len(forced) == len(plain)
     forms = [k.knobs.get("PREFETCH") for k in forced]
-    # embedding -> q/k/v weights; q/k/v projection -> attention (no weights); attention -> o_proj; o_proj -> gate/up;
-    # gate/up -> down; down -> the next layer's q/k/v (the last one: the final norm, no large constant)
-    assert forms == ["workgroups", None, "workgroups", "workgroups", "wave", "workgroups", None, "workgroups", "workgroups", "wave", None, None]
+    # embedding -> q/k/v weights; q/k/v projection -> head norms + rotary embedding -> attention (no weights); attention
+    # -> o_proj; o_proj -> gate/up; gate/up -> down; down -> the next layer's q/k/v (the last one: the final norm, no
+    # large constant)
+    assert forms == ["workgroups", None, None, "workgroups", "workgroups", "wave", "workgroups", None, None, "workgroups", "workgroups", "wave", None, None]
     for before, after in zip(plain, forced):
         if "PREFETCH" not in after.knobs:
             assert after.kernel_name == before.kernel_name
@@ -73,7 +74,7 @@ def test_a_consumer_whose_rows_to_workgroups_mapping_is_known_is_prefetched_per_
     case = wl.qwen3_model_case(seq=32, layers=1)
     ks = kernels(HipBackend().compile(trace_module(case.module, case.inputs)))
     gate_up = next(k for k in ks if "silu_mul" in k.kernel_name)
-    assert gate_up.knobs["STAGE"].startswith("d8/ks") and gate_up.weight_slices[1] * gate_up.weight_slices[2] == 2 * 3072 * 1024 * 2
+    assert gate_up.knobs["STAGE"].startswith("d4/ks") and gate_up.weight_slices[1] * gate_up.weight_slices[2] == 2 * 3072 * 1024 * 2
     before = ks[ks.index(gate_up) - 1]
     assert before.arg_order[-1] == gate_up.weight_slices[0]
     assert "const unsigned xcd_ = blockIdx.x % 8u" in before.kernel_source and "slices xcd_, xcd_ + 8" in before.kernel_source
