@@ -242,7 +242,10 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
     cus = ctx.compute_units
     for (tm, tn, wm, wn, *_), plan in plans:
         groups = -(-m // tm) * -(-n // tn) * copies
-        if wm * wn > 1 and m % tm == 0 and n % tn == 0 and 0.9 * cus <= groups <= cus:
+        # (the gate / up pair's 64x96 tile also as a three-quarter cover: 384 rows, 192 workgroups 10.23 us against 11.80
+        # on 144 of 64x128 and more on 288 of 64x64)
+        floor = 0.75 if gate_pair and (tm, tn) == (64, 96) else 0.9
+        if wm * wn > 1 and m % tm == 0 and n % tn == 0 and floor * cus <= groups <= cus:
             return plan  # (the one-wave tile is the last resort: two waves on half as many 16x32 tiles beat it)
     half_round = None  # the first (largest) tile that covers at least half the CUs
     for (tm, tn, *_), plan in plans:
@@ -431,14 +434,18 @@ def _fp32_underfilled(body: Contraction, plan: TilePlan, ctx: Context) -> tuple[
     CUs, the reduction axis is split across workgroups (partials workspace + combine kernel) until about two
     workgroups per CU run, on four-wave 32x32 tiles with 32-deep slabs.  Measured (us, the unsplit default ->
     this): 32x3072x1024 22.7 -> 5.8, 128x3072x1024 21.8 -> 10.7, 32x2048x1024 15.5 -> 4.9, 128x2048x1024 15.1 ->
-    8.5, 32x1024x2048 6.5 -> 4.8, 32x1024x1024 6.7 -> 4.1, 128x1024x1024 6.6 -> 6.2.  Problems whose 32x32 tiles
-    already cover the CUs keep the unsplit default (128x1024x2048: 6.8 unsplit, 8.4 split in two)."""
+    8.5, 32x1024x2048 6.5 -> 4.8, 32x1024x1024 6.7 -> 4.1, 128x1024x1024 6.6 -> 6.2; 16 rows and fewer likewise
+    (16x1024x3072 19.9 -> 4.5 + 1.9, 16x4096x1024 7.7 -> 4.8 + 1.9; the fp32 decoder block at 1 / 16 tokens 71.1 / 72.5
+    -> 46.8 / 49.1).  Problems whose 32x32 tiles already cover the CUs keep the unsplit default (128x1024x2048: 6.8
+    unsplit, 8.4 split in two)."""
     plain = not (body.gate_pair or body.a_prologue is not None or body.row_epilogue is not None) and int(getattr(body, "batch", 1) or 1) == 1 and body.k_split is None
     sym = getattr(body, "sym", None)
     if sym is not None and sym.fields:
         return plan, 1  # the split's kernel pair bakes the row count in: a runtime-int kernel stays unsplit
-    if body.in_dtype.name != "f32" or not plain or not all(isinstance(d, int) for d in (body.m, body.n, body.k)) or body.m <= 16 or body.k % 32 or body.k < 256:
+    if body.in_dtype.name != "f32" or not plain or not all(isinstance(d, int) for d in (body.m, body.n, body.k)) or body.k % 32 or body.k < 256:
         return plan, 1
+    if body.m <= 16 and body.k * body.n < (1 << 20):
+        return plan, 1  # a small weight at decode sizes is one short launch: a second one would cost more than the idle CUs
     base = -(-body.m // 32) * -(-body.n // 32)
     if base >= ctx.compute_units:
         return plan, 1
@@ -651,8 +658,10 @@ def schedule_flash(body: Flash, ctx: Context) -> dict:
                     body.waves, body.pair = w, True
                     break
         if not body.waves:
-            # (two row groups pay down to half the CUs: 512 tokens x 16 heads, 128 workgroups of `w2` 8.81 us, 256 of `w1` 9.10)
-            body.waves = next((w for w in (4, 2) if heads * blocks(w) >= (fill if w == 4 else 0.5 * ctx.compute_units)), 1)
+            # (two row groups pay down to half the CUs: 512 tokens x 16 heads, 128 workgroups of `w2` 8.81 us, 256 of `w1` 9.10;
+            # and wherever there are more than two of their 64-row blocks, however few the workgroups: they share each K / V
+            # block's way into the LDS: 160 / 192 / 384 tokens x 16 heads 6.15 / 6.16 / 7.32 us against 6.42 / 6.45 / 7.48)
+            body.waves = next((w for w in (4, 2) if heads * blocks(w) >= (fill if w == 4 else 0.5 * ctx.compute_units) or (w == 2 and blocks(2) > 2)), 1)
         body.block_kv, body.kv_split = {8: (64, 1), 4: (64, 2)}.get(body.waves, (32, 4))
         while body.kv_split > 1 and -(-body.kv_len // body.block_kv) <= body.kv_split // 2:
             body.kv_split //= 2  # half the key-split groups would have no block (three blocks keep four groups: 96 keys 4.71 us, two groups 6.05)

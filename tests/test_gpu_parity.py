@@ -867,8 +867,11 @@ def test_fp32_linear(device, m, k, n, bias):
     x = torch.randn(m, k)
     be = HipBackend()
     compiled = be.compile(trace_module(lin, (x,)))
-    (op,) = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
-    assert "_f32/" in op.knobs["TILE"]
+    ops = [n_.op for n_ in compiled.nodes.values() if isinstance(n_.op, HipOp)]
+    assert all("_f32/" in op.knobs["TILE"] for op in ops)
+    # one row over a 12 MiB weight leaves most CUs idle on 32-column tiles: the reduction axis is split across workgroups
+    # (partials + combine); every other case here is one launch
+    assert sorted(op.kernel_name.rsplit("_", 1)[0] for op in ops) == (["k_linear_combine", "k_linear_partial"] if (m, k, n) == (1, 1024, 3072) else ["k_linear"])
     prog = be.program(compiled, {compiled.inputs[0]: x.to(device)})
     try:
         prog.run()

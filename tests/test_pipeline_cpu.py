@@ -318,7 +318,7 @@ def test_uniform_pointer_halves_are_widened_unsigned(launcher_lib):
 def test_flash_pin_grammar_and_degrade(launcher_lib, monkeypatch):
     case = eager.sdpa_case(1, 8, 4, 320, 128)
     default = kernels(compile_case(case))[0].knobs["FLASH"]
-    assert default == "w1/kv32/s4"  # few heads, short sequence: one 32-row group per workgroup, four key-split groups
+    assert default == "w2/kv32/s4"  # few heads, short sequence: two 32-row groups share each K / V block, four key-split groups
     # long causal self-attention: mirrored query-block pairs, so every workgroup streams the same number of keys
     big = kernels(compile_case(eager.sdpa_case()))[0]
     assert big.knobs["FLASH"] == "w2/kv32/s4/p" and big.grid[0] == (16 * 32 // 2,) and "#define PAIR 1" in big.kernel_source
