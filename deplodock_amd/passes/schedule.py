@@ -387,6 +387,8 @@ def _default_stage(plan: TilePlan, body: Contraction, ctx: Context) -> Stage:
         for depth in (3, 2):
             if depth == 3 and (steps < 3 or mfma_cycles >= 600):
                 continue
+            if depth == 3 and body.in_dtype.name == "f32" and plan.block_threads <= 256 and plan.bk_elems >= 64:
+                continue  # four-wave fp32 tiles: two slots leave the LDS to more workgroups a CU (see _fp32_even_rounds)
             try:
                 _check_tile(plan, body, ctx, depth=depth, dl=True)
             except ScheduleError:
@@ -422,9 +424,39 @@ def _default_tile(body: Contraction, ctx: Context) -> TilePlan:
         while bk_elems > 2 * atom.frag_k and body.k % bk_elems:
             bk_elems //= 2
         plan = TilePlan(atom=atom, units=plan.units, regs=plan.regs, bk=bk_elems // atom.k)
+        plan = _fp32_even_rounds(body, plan, ctx)
     elif plan.atom.dtype != atom_dtype:
         plan = TilePlan(atom=ATOMS[plan.atom.name.replace("bf16", atom_dtype)], units=plan.units, regs=plan.regs, bk=plan.bk)
     return plan
+
+
+def _fp32_even_rounds(body: Contraction, plan: TilePlan, ctx: Context) -> TilePlan:
+    """At the fp32 matrix rate a launch is as long as its fullest CU's MFMA work.  A tile whose workgroups fill the last
+    round of CUs to less than 85 % gives way to four-wave 32x32 tiles when those make at least two rounds that come out
+    more even (256 x 3072 x 1024: 192 tiles of 64x64 21.9 us, 768 of 32x32 17.6; 384 x 3072 x 1024: 144 tiles of 64x128
+    1.4 times the 1 152 of 32x32).  That tile streams 64-deep slabs (128-deep
+    beyond K = 2048) through two ring slots, which leaves the LDS for several workgroups a CU, one wave each a SIMD
+    (256 x 1024 x 2048: 13.1 us against 15.0 with three 128-deep slabs; 256 x 1024 x 3072: 20.8 against 21.9)."""
+    if not all(isinstance(d, int) for d in (body.m, body.n, body.k)) or body.gate_pair or body.row_epilogue is not None or body.a_prologue is not None:
+        return plan
+    cus = ctx.compute_units
+    copies = max(1, int(getattr(body, "batch", 1) or 1))
+
+    def evenness(tm: int, tn: int) -> tuple[int, float]:
+        groups = -(-body.m // tm) * -(-body.n // tn) * copies
+        return groups, groups / float(-(-groups // cus) * cus)
+
+    small = (plan.units, plan.regs, plan.atom.name) == ((2, 2), (1, 1), "mfma_16x16x4_f32")
+    if not small:
+        _, even = evenness(plan.tile_m, plan.tile_n)
+        groups32, even32 = evenness(32, 32)
+        small = even < 0.85 and groups32 >= 2 * cus and even32 >= even + 0.1
+    if not small:
+        return plan
+    bk = 16 if body.k <= 2048 else 32
+    while bk > 8 and body.k % (bk * 4):
+        bk //= 2
+    return TilePlan(atom=ATOMS["mfma_16x16x4_f32"], units=(2, 2), regs=(1, 1), bk=bk)
 
 
 def _fp32_underfilled(body: Contraction, plan: TilePlan, ctx: Context) -> tuple[TilePlan, int]:
