@@ -26,9 +26,10 @@ The pass runs after lowering and is on by default only where it can pay: a progr
 last-level cache, and in it a consumer between ``MIN_INTENSITY`` and ``MAX_INTENSITY`` flop per byte (``EMMY_PREFETCH=1`` /
 ``0`` force it on for every consumer / off).  Measured on the 28-layer Qwen3-0.6B-architecture model (880 MB of weights;
 us per forward as one graph replay, without / with): 1 token 735 / 776, 16 tokens 842 / 846, 32 tokens 959 / 929,
-128 tokens 1090 / 1019, 256 tokens 1283 / 1166, 512 tokens 1544 / 1531 — below about 32 rows a launch is too short to hide
-its successor's lines behind and the extra wave or workgroups cost more than the warm start gains; at 512 rows the
-consumers are busy with arithmetic and the gain is within the spread of two runs.
+128 tokens 1090 / 1019, 256 tokens 1284 / 1180, 384 tokens 1477 / 1459, 512 tokens 1519 / 1489 — below about 32 rows a launch
+is too short to hide its successor's lines behind and the extra wave or workgroups cost more than the warm start gains; from
+512 rows on the consumers are busy with arithmetic and the gain is down to 1-2 % (an upper bound of 200 flop per byte left the
+256-token gate / up projection, at 219, without its prefetch: 1234).
 """
 
 from __future__ import annotations
@@ -51,7 +52,7 @@ MAX_BYTES = 64 * 1024 * 1024
 LAST_LEVEL_CACHE_BYTES = 256 * 1024 * 1024
 #: flop per byte of the consumer (about its row count, for a weight-streaming contraction) between which a prefetch pays
 MIN_INTENSITY = 24.0
-MAX_INTENSITY = 200.0
+MAX_INTENSITY = 400.0
 #: LDS up to which extra workgroups run beside the kernel's own on a CU (two of them fit a CU's 160 KiB)
 _SMALL_LDS = 76 * 1024
 LINE = 128
