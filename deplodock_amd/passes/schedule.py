@@ -777,19 +777,19 @@ def _schedule_flash_f32(body: Flash, ctx: Context) -> dict:
     knobs: dict = {}
     if body.kv_split > 1 and body.dtype.name == "f32" and not body.causal and body.mask is None and not symbolic and body.head_dim % 4 == 0:
         # decode-size queries over a long cache: the keys are also split across workgroups (partial kernel + combine)
-        knobs = _schedule_flash_split(body, ctx, tuned if (tuned := _tuned(body, ctx)) else None, min_keys=256)
+        knobs = _schedule_flash_split(body, ctx, tuned if (tuned := _tuned(body, ctx)) else None)
     elif _pin("REDUCE", _tuned(body, ctx)):
         logger.warning("EMMY_REDUCE ignored for this fp32 attention: the cross-workgroup key split takes the key-split form without masks or symbolic lengths")
     return {**knobs, "FLASH": flash}
 
 
-def _schedule_flash_split(body: Flash, ctx: Context, tuned: dict | None, min_keys: int = 512) -> dict:
+def _schedule_flash_split(body: Flash, ctx: Context, tuned: dict | None, min_keys: int = 256) -> dict:
     """``REDUCE=g<n>[k]`` on attention: ``n`` workgroups per query block split the keys and a combine kernel merges their
     ``(m, l, O)`` (the reference's cross-CTA finalize of the twisted carrier is kernel-only, tests/compiler/e2e/
     test_reduce_coverage.py:280-315; ``g<n>a`` is taken as ``g<n>k``).  Unpinned: where the query blocks cover less than
     half the CUs and the keys are long — decode-size queries over a long cache — the keys are split until the launch covers
-    the CUs, in slices of at least ``min_keys`` keys (512; 256 on fp32 atoms, where a key block is sixteen times the matrix
-    work: 16 queries over 4 096 keys in fp32, 16 slices 19.1 us against 26.5 on 8)."""
+    the CUs, in slices of at least ``min_keys`` keys (us, slices of 256 against 512 keys: one bf16 query over 2 048 / 4 096 keys
+    7.98 / 9.16 against 9.92 / 10.20, 16 queries over 4 096 keys 9.94 against 10.44; in fp32 19.1 against 26.5)."""
     body.kv_ctas = 1
     plain = body.mask is None and not (getattr(body, "sym", None) is not None and body.sym.fields) and not (body.ws or body.sp)
     pinned = _pin("REDUCE", tuned)
