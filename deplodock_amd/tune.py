@@ -72,6 +72,9 @@ FLASH_SWEEP: tuple[str, ...] = (
     "w4/kv64/s2", "w2/kv64/s2", "w1/kv64/s2", "w2/kv32/s4", "w1/kv32/s4", "w4/kv32/s2", "w4/kv64/s1",
     "w2/kv32/s4/p", "w2/kv64/s2/p", "w1/kv32/s4/p", "w4/kv64/s2/p", "w8/kv64/s1", "w8/kv64/s1/p",
 )  # fmt: skip
+#: attention on fp32 MFMA atoms: row groups that share each staged block, or waves that split a row group's key blocks
+#: (``/o``: a wave's K and V blocks take turns in one LDS region; ``/sp``: the software-pipelined order)
+FLASH_SWEEP_F32: tuple[str, ...] = ("f32/w1", "f32/w2", "f32/w4", "f32/s2", "f32/s4", "f32/s8", "f32/s2/o", "f32/s4/o", "f32/s8/o", "f32/s4/sp")
 
 
 def shape_key(body) -> str | None:
@@ -198,12 +201,16 @@ def candidate_rounds(families: set[str]) -> list[dict[str, str]]:
     if "contraction_f32" in families:
         # rounds of their own: TILE / STAGE name one atom type, and a 16-bit contraction of the same graph keeps its defaults meanwhile
         out += [{"TILE": t, "STAGE": s} for s in STAGE_SWEEP_F32 for t in TILE_SWEEP_F32]
+    if "flash_f32" in families:
+        out += [{"FLASH": f} for f in FLASH_SWEEP_F32]  # (rounds of their own for the same reason)
     return out
 
 
 def _family(key: str) -> str:
     """Candidate family of a shape key: fp32 contractions sweep fp32 atoms."""
     fam = key.split("/")[0]
+    if fam == "flash" and key.endswith("/f32"):
+        return "flash_f32"
     return "contraction_f32" if fam == "contraction" and "/f32>" in key else fam
 
 

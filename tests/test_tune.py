@@ -97,6 +97,10 @@ def test_fp32_contractions_sweep_fp32_atoms_in_rounds_of_their_own():
     assert all(TilePlan.parse(r["TILE"]).atom.dtype == "f32" for r in only)
     mixed = candidate_rounds({"contraction", "contraction_f32"})
     assert len(mixed) == 70 + len(only) and mixed[70:] == only  # appended, never merged with the 16-bit pins of a round
+    # attention on fp32 atoms likewise sweeps its own forms
+    assert _family("flash/b1/hq16/hkv8/sq512/skv512/d128/c1/f32") == "flash_f32" and _family("flash/b1/hq16/hkv8/sq512/skv512/d128/c1/bf16") == "flash"
+    f32_flash = candidate_rounds({"flash_f32"})
+    assert f32_flash and all(set(r) == {"FLASH"} and r["FLASH"].startswith("f32/") for r in f32_flash)
 
 
 @pytest.mark.gpu
