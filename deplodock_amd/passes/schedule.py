@@ -51,7 +51,7 @@ TILE_CANDIDATES: tuple[tuple[int, int, int, int, str, int], ...] = (
     (32, 128, 2, 4, "mfma_16x16x32_bf16", 4),
     (32, 64, 1, 4, "mfma_16x16x32_bf16", 8),
     (32, 32, 2, 2, "mfma_16x16x32_bf16", 8),
-    (16, 128, 1, 4, "mfma_16x16x32_bf16", 8),
+    (16, 128, 1, 4, "mfma_16x16x32_bf16", 4),  # 128-deep slabs leave the LDS for a third ring slot: the q/k/v projection at 64 / 128 tokens 5.95 / 6.11 us (256-deep, two slots: 6.35 / 6.49)
     (16, 32, 1, 2, "mfma_16x16x32_bf16", 8),
     (16, 16, 1, 1, "mfma_16x16x32_bf16", 8),
 )

@@ -144,7 +144,7 @@ def test_qwen3_block_kernel_boundaries(launcher_lib):
     # folded into the stacked projection weights at bind time, the rows are staged as they are
     # while their sum of squares is accumulated, and the accumulators take the row's scale factor
     first = kernels(compiled)[0]
-    assert "a=row-scaled-after" in first.comment and first.arg_order[0] == compiled.inputs[0] and first.knobs["STAGE"] == "d2/dl"
+    assert "a=row-scaled-after" in first.comment and first.arg_order[0] == compiled.inputs[0] and first.knobs["STAGE"] == "d3/dl"
     # 16 tokens (as many as heads) and fewer: the projection takes the few-row form with the deferred norm (the row
     # statistic from the fragments a lane holds, the accumulators scaled), and the head norms + rotary embedding of q
     # and k are one small row kernel behind it; one token, whose token dim is a unit dim, pairs q and k the same way
