@@ -234,6 +234,10 @@ def pick_tile(m: int, n: int, k: int, gate_pair: bool, ctx: Context, row_prologu
                 bk //= 2
             if k % (bk * atom.k):
                 continue
+            if bk == 8 and 3 * (tm + tn * nb) * bk * atom.k * 2 > ctx.lds_bytes_per_cu and k % (4 * atom.k) == 0:
+                # the few-row tiles' 256-deep slabs give way to 128-deep ones where only those leave the LDS for a third ring
+                # slot (the gate / up pair on the eight-wave 32x64 tile at 96 / 128 rows: 6.18 / 6.21 us against 6.60 / 6.62)
+                bk = 4
         threads = wm * wn * 64
         cpr = bk * atom.k // 8
         if (tm * cpr) % threads or (tn * cpr * (2 if gate_pair else 1)) % threads:
