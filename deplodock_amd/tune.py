@@ -49,6 +49,10 @@ TILE_SWEEP: tuple[str, ...] = (
     "a:mfma_16x16x32_bf16/w2x2/f1x1/k8",
     "a:mfma_16x16x32_bf16/w1x4/f1x2/k8",
     "a:mfma_16x16x32_bf16/w1x2/f1x1/k8",
+    # the few-row tiles on 128-deep slabs (room for a third ring slot where 256-deep ones leave none)
+    "a:mfma_16x16x32_bf16/w2x4/f1x1/k4",
+    "a:mfma_16x16x32_bf16/w1x4/f1x2/k4",
+    "a:mfma_16x16x32_bf16/w1x2/f1x1/k4",
     "a:mfma_16x16x32_bf16/w1x1/f1x1/k8",
 )  # every tile that won an in-graph ranking of the decoder block's contractions at 64 ... 2048 tokens, and their neighbours
 # The fp32 tier (fp32 MFMA atoms; slab depth in atom steps of 4): the tiles that ranked first somewhere in a sweep of the
